@@ -1,0 +1,260 @@
+"""ctypes binding of ``libadh.so``.  There is no fallback: if the library is missing, or a
+call is made without a GPU, an exception is raised."""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libadh.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+ADH_F32 = 0
+ADH_BF16 = 1
+ADH_OK, ADH_EINVAL, ADH_EUNIMPL, ADH_ENULL, ADH_EALIGN, ADH_EWORKSPACE = 0, -1, -2, -3, -4, -5
+ADH_CONV_FWD, ADH_CONV_BWD_DATA, ADH_CONV_BWD_FILTER = 0, 1, 2
+ADH_MAX_TILES = 16
+
+u32, u64, i32, f32, vp, sz = (ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int, ctypes.c_float,
+                              ctypes.c_void_p, ctypes.c_size_t)
+vpp = ctypes.POINTER(ctypes.c_void_p)
+
+# name -> (restype, argtypes); every symbol include/adh_capi.h declares
+SIGNATURES = {
+    "adh_version": (i32, []),
+    "adh_error_string": (ctypes.c_char_p, [i32]),
+    "adh_fill_f32": (i32, [u64, f32, vp, vp]),
+    "adh_add_f32": (i32, [u64, vp, vp, vp]),
+    "adh_halo_exchange_nchw": (i32, [i32, u32, u32, u32, u32, u32, u32, u32, vpp, vp]),
+    "adh_halo_reduce_nchw": (i32, [i32, u32, u32, u32, u32, u32, u32, u32, vpp, vp]),
+    "adh_halo_exchange_nchw_rank": (i32, [i32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vp]),
+    "adh_halo_reduce_nchw_rank": (i32, [i32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vp]),
+    "adh_halo_pad_nchw": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp]),
+    "adh_halo_pad_add_nchw": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp]),
+    "adh_halo_unpad_nchw": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp]),
+    "adh_halo_unpad_add_nchw": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp]),
+    "adh_halo_repad_nchw": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vp, vp]),
+    "adh_slice_copy_nchw": (i32, [i32, u32, u32, u32, u32, vp, u32, u32, u32, u32, u32, u32,
+                                  vp, u32, u32, u32, u32, u32, u32, vp]),
+    "adh_slice_add_nchw": (i32, [i32, u32, u32, u32, u32, vp, u32, u32, u32, u32, u32, u32,
+                                 vp, u32, u32, u32, u32, u32, u32, vp]),
+    "adh_tiles_pack_nchw": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vp]),
+    "adh_tiles_unpack_nchw": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vp]),
+    "adh_conv3x3_workspace_bytes": (sz, [i32, i32, u32, u32, u32, u32, u32, u32]),
+    "adh_conv3x3_slab_fwd": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
+    "adh_conv3x3_slab_fwd_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp, sz, vp]),
+    "adh_conv3x3_slab_bwd_data": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
+    "adh_conv3x3_slab_bwd_data_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
+    "adh_conv3x3_slab_bwd_filter": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
+    "adh_conv3x3_slab_bwd_filter_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp, f32, vp, sz, vp]),
+    "adh_softmax_fwd": (i32, [u32, u32, vp, vp, vp]),
+    "adh_softmax_nll_loss_fwd": (i32, [u32, u32, vp, vp, vp, vp]),
+    "adh_softmax_nll_loss_bwd": (i32, [u32, u32, vp, vp, vp, vp, vp]),
+    "adh_softmax_xent_fwd": (i32, [u32, u32, vp, vp, vp, vp, vp]),
+}
+
+
+def build(force=True):
+    """Compile libadh.so for gfx950 with hipcc (cross-compiles without a GPU)."""
+    args = ["make", "-s", "-C", CSRC, "-j8"]
+    if force:
+        args.append("-B")
+    subprocess.check_call(args)
+    return LIB_PATH
+
+
+class AdhError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        super().__init__("%s failed: %d (%s)" % (what, code, lib().adh_error_string(code).decode()))
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built: there is no CPU fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libadh.so is not built (%s); run __graft_entry__.build() or "
+                               "`make -C arraydiff_cuda_amd/csrc`" % LIB_PATH)
+        l = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(l, name)  # AttributeError if a declared symbol is not exported
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def check(code, what="adh call"):
+    if code != 0:
+        raise AdhError(code, what)
+    return code
+
+
+def ptr_table(ptrs):
+    """Host array of device pointers from ints / None."""
+    arr = (ctypes.c_void_p * len(ptrs))(*[p if p else None for p in ptrs])
+    return ctypes.cast(arr, vpp), arr
+
+
+# ---------------------------------------------------------------------------
+# torch-tensor convenience wrappers (tests / bench).  Tensors must live on the GPU.
+# ---------------------------------------------------------------------------
+def _dt(t):
+    import torch
+    if t.dtype == torch.float32:
+        return ADH_F32
+    if t.dtype == torch.bfloat16:
+        return ADH_BF16
+    raise TypeError("dtype %s not supported" % t.dtype)
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is not None and (not t.is_cuda or not t.is_contiguous()):
+            raise ValueError("tensors must be contiguous GPU tensors")
+
+
+def _stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _tbl(ts):
+    return ptr_table([t.data_ptr() for t in ts])
+
+
+def fill_f32(x, v):
+    _dev(x)
+    return lib().adh_fill_f32(x.numel(), v, x.data_ptr(), _stream())
+
+
+def add_f32(x, y):
+    _dev(x, y)
+    return lib().adh_add_f32(x.numel(), x.data_ptr(), y.data_ptr(), _stream())
+
+
+def halo_exchange(tiles, grid_w, grid_h, p, W, H, C, N, rank=None):
+    _dev(*tiles)
+    tb, keep = _tbl(tiles)
+    if rank is None:
+        return lib().adh_halo_exchange_nchw(_dt(tiles[0]), grid_w, grid_h, p, W, H, C, N, tb, _stream())
+    return lib().adh_halo_exchange_nchw_rank(_dt(tiles[0]), grid_w, grid_h, rank, p, W, H, C, N, tb, _stream())
+
+
+def halo_reduce(tiles, grid_w, grid_h, p, W, H, C, N, rank=None):
+    _dev(*tiles)
+    tb, keep = _tbl(tiles)
+    if rank is None:
+        return lib().adh_halo_reduce_nchw(_dt(tiles[0]), grid_w, grid_h, p, W, H, C, N, tb, _stream())
+    return lib().adh_halo_reduce_nchw_rank(_dt(tiles[0]), grid_w, grid_h, rank, p, W, H, C, N, tb, _stream())
+
+
+def _padlike(name, p, W, H, C, N, a, b):
+    _dev(a, b)
+    return getattr(lib(), name)(_dt(a), p, W, H, C, N, a.data_ptr(), b.data_ptr(), _stream())
+
+
+def halo_pad(p, W, H, C, N, x, y):
+    return _padlike("adh_halo_pad_nchw", p, W, H, C, N, x, y)
+
+
+def halo_pad_add(p, W, H, C, N, x, y):
+    return _padlike("adh_halo_pad_add_nchw", p, W, H, C, N, x, y)
+
+
+def halo_unpad(p, W, H, C, N, x, y):
+    return _padlike("adh_halo_unpad_nchw", p, W, H, C, N, x, y)
+
+
+def halo_unpad_add(p, W, H, C, N, x, y):
+    return _padlike("adh_halo_unpad_add_nchw", p, W, H, C, N, x, y)
+
+
+def halo_repad(ps, pd, W, H, C, N, x, y):
+    _dev(x, y)
+    return lib().adh_halo_repad_nchw(_dt(x), ps, pd, W, H, C, N, x.data_ptr(), y.data_ptr(), _stream())
+
+
+def slice_nchw(add, count, N, src, src_dims, src_off, dst, dst_dims, dst_off):
+    _dev(src, dst)
+    fn = lib().adh_slice_add_nchw if add else lib().adh_slice_copy_nchw
+    return fn(_dt(src), count[0], count[1], count[2], N, src.data_ptr(), src_dims[0], src_dims[1], src_dims[2],
+              src_off[0], src_off[1], src_off[2], dst.data_ptr(), dst_dims[0], dst_dims[1], dst_dims[2],
+              dst_off[0], dst_off[1], dst_off[2], _stream())
+
+
+def tiles_pack(K, p, W, H, C, N, x, tiles):
+    _dev(x, *tiles)
+    tb, keep = _tbl(tiles)
+    return lib().adh_tiles_pack_nchw(_dt(x), K, p, W, H, C, N, x.data_ptr(), tb, _stream())
+
+
+def tiles_unpack(K, p, W, H, C, N, tiles, y):
+    _dev(y, *tiles)
+    tb, keep = _tbl(tiles)
+    return lib().adh_tiles_unpack_nchw(_dt(y), K, p, W, H, C, N, tb, y.data_ptr(), _stream())
+
+
+def conv_workspace_bytes(which, dtype, K, N, Cin, Cout, H, W):
+    return lib().adh_conv3x3_workspace_bytes(which, dtype, K, N, Cin, Cout, H, W)
+
+
+def _ws(ws):
+    if ws is None:
+        return None, 0
+    return ws.data_ptr(), ws.numel() * ws.element_size()
+
+
+def conv_fwd_tiles(xs, w, ys, N, Cin, Cout, H, W, beta=0.0, ws=None):
+    _dev(w, *xs, *ys)
+    xt, k1 = _tbl(xs)
+    yt, k2 = _tbl(ys)
+    wp, wb = _ws(ws)
+    return lib().adh_conv3x3_slab_fwd_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, xt, w.data_ptr(), yt, beta,
+                                            wp, wb, _stream())
+
+
+def conv_bwd_data_tiles(w, dys, dxs, N, Cin, Cout, H, W, beta=0.0, ws=None):
+    _dev(w, *dys, *dxs)
+    dt, k1 = _tbl(dys)
+    xt, k2 = _tbl(dxs)
+    wp, wb = _ws(ws)
+    return lib().adh_conv3x3_slab_bwd_data_tiles(_dt(dys[0]), len(dys), N, Cin, Cout, H, W, w.data_ptr(), dt, xt,
+                                                 beta, wp, wb, _stream())
+
+
+def conv_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, H, W, beta=0.0, ws=None):
+    _dev(dw, *xs, *dys)
+    xt, k1 = _tbl(xs)
+    dt, k2 = _tbl(dys)
+    wp, wb = _ws(ws)
+    return lib().adh_conv3x3_slab_bwd_filter_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, xt, dt, dw.data_ptr(),
+                                                   beta, wp, wb, _stream())
+
+
+def softmax_fwd(x, y):
+    _dev(x, y)
+    N, C = x.shape
+    return lib().adh_softmax_fwd(C, N, x.data_ptr(), y.data_ptr(), _stream())
+
+
+def softmax_xent_fwd(x, label, y, loss):
+    _dev(x, label, y, loss)
+    N, C = x.shape
+    return lib().adh_softmax_xent_fwd(C, N, x.data_ptr(), label.data_ptr(), y.data_ptr(), loss.data_ptr(), _stream())
+
+
+def softmax_nll_loss_fwd(y, label, loss):
+    _dev(y, label, loss)
+    N, C = y.shape
+    return lib().adh_softmax_nll_loss_fwd(C, N, y.data_ptr(), label.data_ptr(), loss.data_ptr(), _stream())
+
+
+def softmax_nll_loss_bwd(y, label, dloss, dx):
+    _dev(y, label, dloss, dx)
+    N, C = y.shape
+    return lib().adh_softmax_nll_loss_bwd(C, N, y.data_ptr(), label.data_ptr(), dloss.data_ptr(), dx.data_ptr(),
+                                          _stream())

@@ -1,0 +1,361 @@
+// 3x3 convolution over the halo-padded slab on the gfx950 matrix cores (fp32 MFMA).
+//
+// One kernel serves forward and backward-data, both written as
+//   out[o][oh][ow] = beta*out + sum_{k,a,b} Wt(o,k,a,b) * in[k][oh + a - pad][ow + b - pad]
+// (zero outside the input plane):
+//   forward       : in = padded slab x (H+2, W+2), out = y (H, W),        pad = 0,
+//                   Wt(o=co,k=ci,a,b) = w[co][ci][a][b]
+//   backward-data : in = dy (H, W),  out = WHOLE padded slab dx (H+2, W+2), pad = 2,
+//                   Wt(o=ci,k=co,a,b) = w[co][ci][2-a][2-b]
+//
+// Mapping to the hardware (wave64, v_mfma_f32_16x16x4_f32):
+//   * implicit GEMM D[o][pixel] += A[o][k] * B[k][pixel]; the MFMA "column" dimension is
+//     the pixel, so lane%16 walks consecutive output pixels and stores are contiguous runs.
+//   * a workgroup (4 waves) owns R output rows x TW columns of one image for 64 output
+//     channels; wave v owns output channels [16v, 16v+16) and ALL NT = ceil(R*TW/16) pixel
+//     tiles, so the four matrix pipes of a CU carry identical work (NT accumulators of 4
+//     VGPRs each per wave).
+//   * the reduction runs over chunks of 8 input channels.  The (R+2) x (TW+2) input patch of
+//     a chunk is staged once in LDS (pitch 64 floats, channel stride = 16 mod 64 banks so the
+//     four k-groups of an MFMA read disjoint banks) and reused by all 9 taps, all 4 waves and
+//     all 64 output channels: each input element is fetched from HBM once per workgroup.
+//     Every B operand is one ds_read_b32 at lane_base + compile-time immediate.
+//   * weights never touch LDS: each lane keeps the 18 A values of the current chunk in
+//     registers and prefetches the next chunk's 18 from L2 while the current chunk computes.
+//   * global->LDS staging of chunk c+1 is issued before the MFMAs of chunk c and written to
+//     the other LDS buffer after them: one barrier per chunk.
+#include "adh_common.h"
+
+namespace adh {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+static constexpr int kConvThreads = 256;
+static constexpr int kChunk = 8;        // reduction channels per LDS stage
+static constexpr int kLdsPitch = 64;    // floats per staged patch row
+static constexpr int kMaxTW = kLdsPitch - 2;
+
+struct ConvParams {
+  const float *in[ADH_MAX_TILES];
+  float *out[ADH_MAX_TILES];
+  const float *w;
+  uint32_t num_tiles, N;
+  uint32_t Cred, Cout;      // reduction channels / output channels of this pass
+  uint32_t IH, IW, OH, OW;  // input and output plane extents
+  int32_t pad;              // input row = oh + a - pad
+  uint32_t R, TW;           // workgroup tile: R output rows x TW output columns
+  uint32_t tiles_x;         // ceil(OW / TW); grid.x = tiles_x * ceil(OH / R)
+  uint32_t w_out_stride, w_red_stride;  // weight address = o*w_out_stride + k*w_red_stride + tap'
+  int32_t w_flip;           // tap' = w_flip ? 8 - tap : tap
+  float beta;
+  FastDiv div_tiles_x, div_TW;
+};
+
+template <int RROWS>
+struct ConvLds {
+  static constexpr int kRows = 4 * RROWS;                      // staged patch rows (>= R + 2)
+  static constexpr int kChanStride = kRows * kLdsPitch + 16;   // == 16 (mod 64)
+  static constexpr int kBufFloats = kChunk * kChanStride;
+  static constexpr int kBytes = 2 * kBufFloats * 4;
+};
+
+template <int NT, int RROWS>
+__global__ __launch_bounds__(kConvThreads, 1) void conv3x3_f32_kernel(const ConvParams P) {
+  typedef ConvLds<RROWS> L;
+  __shared__ float lds[2 * L::kBufFloats];
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & 63u, wv = tid >> 6, g = lane >> 4, l16 = lane & 15u;
+
+  const uint32_t ty = P.div_tiles_x.div(blockIdx.x);
+  const uint32_t tx = blockIdx.x - ty * P.tiles_x;
+  const uint32_t n = blockIdx.z / P.num_tiles;
+  const uint32_t t = blockIdx.z - n * P.num_tiles;
+  const uint32_t oh0 = ty * P.R, ow0 = tx * P.TW;
+  const uint32_t o_blk = blockIdx.y * 64u;
+  const uint64_t in_plane = (uint64_t)P.IH * P.IW;
+  const uint64_t out_plane = (uint64_t)P.OH * P.OW;
+  const float *__restrict__ in = P.in[t] + (uint64_t)n * P.Cred * in_plane;
+  float *__restrict__ out = P.out[t] + (uint64_t)n * P.Cout * out_plane;
+
+  const uint32_t rows_here = min(P.R, P.OH - oh0);
+  const uint32_t cols_here = min(P.TW, P.OW - ow0);
+  const uint32_t npix = P.R * P.TW;
+
+  // LDS float offset of this lane's pixel in each pixel tile (+ the lane's k-group plane)
+  uint32_t pix[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    uint32_t q = 16u * j + l16;
+    if (q >= npix) q = 0;
+    uint32_t r_, c_;
+    P.div_TW.divmod(q, r_, c_);
+    pix[j] = g * L::kChanStride + r_ * kLdsPitch + c_;
+  }
+
+  // ---- staging of the input patch: lane = patch column, wave = patch row (mod 4) ----
+  const int32_t iw = (int32_t)(ow0 + lane) - P.pad;
+  const bool col_ok = lane < P.TW + 2u && iw >= 0 && iw < (int32_t)P.IW;
+  const uint32_t patch_rows = P.R + 2u;
+  float stage[kChunk * RROWS];
+
+  // Staging loads are unconditional (addresses clamped into the tensor); out-of-range
+  // elements are replaced by zero only when the registers are written to LDS, after the
+  // MFMAs of the current chunk, so no load is waited for before the matrix work starts.
+  uint32_t row_off[RROWS];
+  bool row_ok[RROWS];
+#pragma unroll
+  for (int rr = 0; rr < RROWS; ++rr) {
+    const uint32_t prow = wv + 4u * rr;
+    const int32_t ih = (int32_t)(oh0 + prow) - P.pad;
+    row_ok[rr] = col_ok && prow < patch_rows && ih >= 0 && ih < (int32_t)P.IH;
+    row_off[rr] = row_ok[rr] ? (uint32_t)ih * P.IW + (uint32_t)iw : 0u;
+  }
+  auto load_patch = [&](uint32_t k0) {
+#pragma unroll
+    for (int kl = 0; kl < kChunk; ++kl) {
+      const float *src = in + (uint64_t)min(k0 + kl, P.Cred - 1u) * in_plane;
+#pragma unroll
+      for (int rr = 0; rr < RROWS; ++rr) stage[kl * RROWS + rr] = src[row_off[rr]];
+    }
+  };
+  auto store_patch = [&](float *buf, uint32_t k0) {
+#pragma unroll
+    for (int kl = 0; kl < kChunk; ++kl) {
+      const bool k_ok = k0 + kl < P.Cred;
+#pragma unroll
+      for (int rr = 0; rr < RROWS; ++rr) {
+        const uint32_t prow = wv + 4u * rr;
+        buf[kl * L::kChanStride + prow * kLdsPitch + lane] = (k_ok && row_ok[rr]) ? stage[kl * RROWS + rr] : 0.f;
+      }
+    }
+  };
+
+  // ---- weights: A[o = o_blk + 16*wv + l16][k = k0 + 4*kk + g][tap], 18 values per chunk ----
+  const uint32_t o_a = o_blk + 16u * wv + l16;
+  const bool o_ok = o_a < P.Cout;
+  const float *__restrict__ w_o = P.w + (uint64_t)min(o_a, P.Cout - 1u) * P.w_out_stride;
+  auto load_weights = [&](uint32_t k0, float (&a)[18]) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const float *wk = w_o + (uint64_t)min(k0 + 4u * kk + g, P.Cred - 1u) * P.w_red_stride;
+#pragma unroll
+      for (int tap = 0; tap < 9; ++tap) a[kk * 9 + tap] = wk[P.w_flip ? 8 - tap : tap];
+    }
+  };
+  auto mask_weights = [&](uint32_t k0, const float (&src)[18], float (&dst)[18]) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const bool ok = o_ok && k0 + 4u * kk + g < P.Cred;
+#pragma unroll
+      for (int tap = 0; tap < 9; ++tap) dst[kk * 9 + tap] = ok ? src[kk * 9 + tap] : 0.f;
+    }
+  };
+
+  floatx4 acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  float a_cur[18], a_nxt[18];
+  const uint32_t nchunks = (P.Cred + kChunk - 1) / kChunk;
+
+  auto compute = [&](const float *cur) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+      for (int kh = 0; kh < 3; ++kh) {
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw) {
+          const float a = a_cur[kk * 9 + kh * 3 + kw];
+          const int off = kk * 4 * L::kChanStride + kh * kLdsPitch + kw;
+#pragma unroll
+          for (int j = 0; j < NT; ++j) {
+            const float b = cur[pix[j] + off];
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[j], 0, 0, 0);
+          }
+        }
+      }
+    }
+  };
+
+  load_patch(0);
+  load_weights(0, a_nxt);
+  store_patch(lds, 0);
+  mask_weights(0, a_nxt, a_cur);
+  __syncthreads();
+
+  for (uint32_t c = 0; c + 1 < nchunks; ++c) {
+    const float *cur = lds + (c & 1u) * L::kBufFloats;
+    float *nxt = lds + ((c + 1u) & 1u) * L::kBufFloats;
+    load_patch((c + 1) * kChunk);
+    load_weights((c + 1) * kChunk, a_nxt);
+    compute(cur);
+    store_patch(nxt, (c + 1) * kChunk);
+    mask_weights((c + 1) * kChunk, a_nxt, a_cur);
+    __syncthreads();
+  }
+  compute(lds + ((nchunks - 1u) & 1u) * L::kBufFloats);
+
+  // ---- epilogue: lane holds D[o = 4*g + i][pixel = l16] of each tile ----
+  const uint32_t o_d = o_blk + 16u * wv + 4u * g;
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const uint32_t q = 16u * j + l16;
+    uint32_t r_, c_;
+    P.div_TW.divmod(q, r_, c_);
+    if (q < npix && r_ < rows_here && c_ < cols_here) {
+      float *dst = out + (uint64_t)o_d * out_plane + (uint64_t)(oh0 + r_) * P.OW + ow0 + c_;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (o_d + i < P.Cout) {
+          float v = acc[j][i];
+          if (P.beta != 0.f) v += P.beta * dst[(uint64_t)i * out_plane];
+          dst[(uint64_t)i * out_plane] = v;
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side: tile selection and launch
+// ---------------------------------------------------------------------------
+struct ConvTile {
+  int nt;          // pixel tiles per workgroup (template instance)
+  uint32_t R, TW;  // output rows / columns per workgroup
+  uint64_t blocks;
+};
+
+static const int kNtVariants[] = {8, 16, 25, 29};
+static constexpr int kRRows = 3;  // staged patch rows = 12 -> R <= 10
+
+// Picks (NT, R, TW) minimising the modelled time ceil(blocks / 256) * NT: a workgroup's
+// time is proportional to NT and 256 CUs run one workgroup each per round.
+static ConvTile choose_tile(uint32_t OH, uint32_t OW, uint64_t planes, uint32_t o_groups) {
+  ConvTile best = {0, 0, 0, 0};
+  double best_cost = 1e300;
+  for (int nt : kNtVariants) {
+    const uint32_t cap = 16u * nt;
+    const uint32_t max_cols = OW < (uint32_t)kMaxTW ? OW : (uint32_t)kMaxTW;
+    for (uint32_t ncol = (OW + max_cols - 1) / max_cols; ncol <= OW && ncol <= (OW + max_cols - 1) / max_cols + 2; ++ncol) {
+      const uint32_t TW = (OW + ncol - 1) / ncol;
+      if (TW == 0 || TW > (uint32_t)kMaxTW || TW > cap) continue;
+      uint32_t Rmax = cap / TW;
+      if (Rmax > 4u * kRRows - 2u) Rmax = 4u * kRRows - 2u;
+      if (Rmax > OH) Rmax = OH;
+      for (uint32_t R = 1; R <= Rmax; ++R) {
+        const uint64_t tiles_y = (OH + R - 1) / R;
+        const uint64_t blocks = tiles_y * ncol * planes * o_groups;
+        const uint64_t rounds = (blocks + 255) / 256;
+        // second-order term prefers fewer, fuller workgroups when rounds tie
+        const double cost = (double)rounds * nt + 1e-6 * (double)blocks * nt;
+        if (cost < best_cost) {
+          best_cost = cost;
+          best.nt = nt; best.R = R; best.TW = TW; best.blocks = blocks;
+        }
+      }
+    }
+  }
+  return best;
+}
+
+template <int NT>
+static void launch_conv(const ConvParams &P, dim3 grid, hipStream_t st) {
+  hipLaunchKernelGGL((conv3x3_f32_kernel<NT, kRRows>), grid, dim3(kConvThreads), 0, st, P);
+}
+
+// which: ADH_CONV_FWD or ADH_CONV_BWD_DATA.  H, W are the interior extents.
+static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                       uint32_t W, const void *const *in_tiles, const void *w, void *const *out_tiles, float beta,
+                       hipStream_t st) {
+  if (!dtype_ok(dtype)) return ADH_EINVAL;
+  if (dtype != ADH_F32) return ADH_EUNIMPL;
+  if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
+  if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
+  if (N == 0 || Cin == 0 || Cout == 0 || H == 0 || W == 0) return ADH_OK;
+  if (!in_tiles || !out_tiles || !w) return ADH_ENULL;
+  if (!aligned_to(w, 4)) return ADH_EALIGN;
+  const uint64_t HP = (uint64_t)H + 2, WP = (uint64_t)W + 2;
+  if (HP * WP >= (1ull << 31) || (uint64_t)N * num_tiles > 65535ull) return ADH_EINVAL;
+  ConvParams P = {};
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!in_tiles[t] || !out_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(in_tiles[t], 4) || !aligned_to(out_tiles[t], 4)) return ADH_EALIGN;
+    P.in[t] = reinterpret_cast<const float *>(in_tiles[t]);
+    P.out[t] = reinterpret_cast<float *>(out_tiles[t]);
+  }
+  P.w = reinterpret_cast<const float *>(w);
+  P.num_tiles = num_tiles;
+  P.N = N;
+  P.beta = beta;
+  if (which == ADH_CONV_FWD) {
+    P.Cred = Cin; P.Cout = Cout;
+    P.IH = (uint32_t)HP; P.IW = (uint32_t)WP; P.OH = H; P.OW = W;
+    P.pad = 0;
+    P.w_out_stride = Cin * 9u; P.w_red_stride = 9u; P.w_flip = 0;
+  } else {
+    P.Cred = Cout; P.Cout = Cin;
+    P.IH = H; P.IW = W; P.OH = (uint32_t)HP; P.OW = (uint32_t)WP;
+    P.pad = 2;
+    P.w_out_stride = 9u; P.w_red_stride = Cin * 9u; P.w_flip = 1;
+  }
+  const uint32_t o_groups = (P.Cout + 63u) / 64u;
+  const ConvTile tile = choose_tile(P.OH, P.OW, (uint64_t)N * num_tiles, o_groups);
+  if (tile.nt == 0) return ADH_EINVAL;
+  P.R = tile.R; P.TW = tile.TW;
+  P.tiles_x = (P.OW + P.TW - 1) / P.TW;
+  const uint32_t tiles_y = (P.OH + P.R - 1) / P.R;
+  P.div_tiles_x = FastDiv(P.tiles_x);
+  P.div_TW = FastDiv(P.TW);
+  dim3 grid(P.tiles_x * tiles_y, o_groups, N * num_tiles);
+  switch (tile.nt) {
+    case 8: launch_conv<8>(P, grid, st); break;
+    case 16: launch_conv<16>(P, grid, st); break;
+    case 25: launch_conv<25>(P, grid, st); break;
+    case 29: launch_conv<29>(P, grid, st); break;
+    default: return ADH_EINVAL;
+  }
+  return launch_status();
+}
+
+}  // namespace adh
+
+using namespace adh;
+
+extern "C" {
+
+int adh_conv3x3_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                               uint32_t W, const void *const *x_pad_tiles, const void *w, void *const *y_tiles,
+                               float beta, void *workspace, size_t workspace_bytes, void *stream) {
+  (void)workspace; (void)workspace_bytes;
+  return conv_direct(ADH_CONV_FWD, dtype, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, w, y_tiles, beta,
+                     as_stream(stream));
+}
+
+int adh_conv3x3_slab_fwd(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                         const void *x_pad, const void *w, void *y, float beta, void *workspace,
+                         size_t workspace_bytes, void *stream) {
+  const void *xs[1] = {x_pad};
+  void *ys[1] = {y};
+  return adh_conv3x3_slab_fwd_tiles(dtype, 1, N, Cin, Cout, H, W, xs, w, ys, beta, workspace, workspace_bytes, stream);
+}
+
+int adh_conv3x3_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                    uint32_t H, uint32_t W, const void *w, const void *const *dy_tiles,
+                                    void *const *dx_pad_tiles, float beta, void *workspace, size_t workspace_bytes,
+                                    void *stream) {
+  (void)workspace; (void)workspace_bytes;
+  return conv_direct(ADH_CONV_BWD_DATA, dtype, num_tiles, N, Cin, Cout, H, W, dy_tiles, w, dx_pad_tiles, beta,
+                     as_stream(stream));
+}
+
+int adh_conv3x3_slab_bwd_data(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                              const void *w, const void *dy, void *dx_pad, float beta, void *workspace,
+                              size_t workspace_bytes, void *stream) {
+  const void *dys[1] = {dy};
+  void *dxs[1] = {dx_pad};
+  return adh_conv3x3_slab_bwd_data_tiles(dtype, 1, N, Cin, Cout, H, W, w, dys, dxs, beta, workspace, workspace_bytes,
+                                         stream);
+}
+
+}  // extern "C"

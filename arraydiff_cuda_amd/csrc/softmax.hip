@@ -1,0 +1,162 @@
+// Row-wise softmax and negative log likelihood for gfx950.
+//
+// One 64-lane wavefront owns one row: the row is read once into registers (up to 1024
+// classes; longer rows are re-read from cache), the max and the sum are reduced across
+// the wavefront with cross-lane shuffles (no LDS, no barrier), and y is written once.
+// A row of 1000 fp32 logits is 4 KB, so the kernel is HBM/latency bound; N rows give N
+// single-wave workgroups, which spreads 256 rows over all 256 CUs.
+#include <math.h>
+
+#include "adh_common.h"
+
+namespace adh {
+
+static constexpr int kWave = 64;
+static constexpr int kCached = 16;  // register-cached elements per lane -> rows up to 1024
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+
+// y = softmax(x) per row; if LOSS, also loss[row] = -logf(y[row, label[row]]) computed
+// from the rounded fp32 y, i.e. exactly what a separate nll pass over y would produce.
+template <bool LOSS>
+__global__ __launch_bounds__(kWave) void softmax_row_kernel(uint32_t C, uint32_t N, const float *__restrict__ x,
+                                                           const uint32_t *__restrict__ label,
+                                                           float *__restrict__ y, float *__restrict__ loss) {
+  const uint32_t row = blockIdx.x;
+  const uint32_t lane = threadIdx.x;
+  if (row >= N) return;
+  const float *xr = x + (uint64_t)row * C;
+  float *yr = y + (uint64_t)row * C;
+  const bool cached = C <= (uint32_t)(kWave * kCached);
+  float v[kCached];
+  float m = -INFINITY;
+  if (cached) {
+#pragma unroll
+    for (int k = 0; k < kCached; ++k) {
+      const uint32_t j = lane + k * kWave;
+      v[k] = j < C ? xr[j] : -INFINITY;
+      m = fmaxf(m, v[k]);
+    }
+  } else {
+    for (uint32_t j = lane; j < C; j += kWave) m = fmaxf(m, xr[j]);
+  }
+  m = wave_max(m);
+  float s = 0.f;
+  if (cached) {
+#pragma unroll
+    for (int k = 0; k < kCached; ++k) {
+      v[k] = expf(v[k] - m);  // exp(-inf) = 0 for the padding lanes
+      s += v[k];
+    }
+  } else {
+    for (uint32_t j = lane; j < C; j += kWave) s += expf(xr[j] - m);
+  }
+  s = wave_sum(s);
+  const uint32_t lab = LOSS ? label[row] : 0u;
+  if (cached) {
+#pragma unroll
+    for (int k = 0; k < kCached; ++k) {
+      const uint32_t j = lane + k * kWave;
+      if (j < C) {
+        const float yv = v[k] / s;
+        yr[j] = yv;
+        if (LOSS && j == lab) loss[row] = -logf(yv);
+      }
+    }
+  } else {
+    for (uint32_t j = lane; j < C; j += kWave) {
+      const float yv = expf(xr[j] - m) / s;
+      yr[j] = yv;
+      if (LOSS && j == lab) loss[row] = -logf(yv);
+    }
+  }
+  if (LOSS && lab >= C && lane == 0) loss[row] = NAN;  // label outside [0, C)
+}
+
+__global__ __launch_bounds__(256) void nll_loss_fwd_kernel(uint32_t C, uint32_t N, const float *__restrict__ y,
+                                                          const uint32_t *__restrict__ label,
+                                                          float *__restrict__ loss) {
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= N) return;
+  const uint32_t lab = label[i];
+  loss[i] = lab < C ? -logf(y[lab + (uint64_t)C * i]) : NAN;
+}
+
+// dx[i,j] += dloss[i] * (y[i,j] - [j == label[i]]); grid = (chunks of a row, rows)
+__global__ __launch_bounds__(256) void nll_loss_bwd_kernel(uint32_t C, uint32_t N, const float *__restrict__ y,
+                                                          const uint32_t *__restrict__ label,
+                                                          const float *__restrict__ dloss, float *__restrict__ dx) {
+  const uint32_t j = blockIdx.x * 256 + threadIdx.x;
+  const uint32_t i = blockIdx.y;
+  if (j >= C || i >= N) return;
+  const uint64_t idx = (uint64_t)i * C + j;
+  const float yv = y[idx];
+  const float dl = dloss[i];
+  const float g = (label[i] == j) ? dl * (yv - 1.0f) : dl * yv;
+  dx[idx] += g;
+}
+
+}  // namespace adh
+
+using namespace adh;
+
+extern "C" {
+
+int adh_softmax_fwd(uint32_t C, uint32_t N, const float *x, float *y, void *stream) {
+  if (C == 0 || N == 0) return ADH_OK;
+  if (!x || !y) return ADH_ENULL;
+  if (!aligned_to(x, 4) || !aligned_to(y, 4)) return ADH_EALIGN;
+  hipLaunchKernelGGL((softmax_row_kernel<false>), dim3(N), dim3(kWave), 0, as_stream(stream), C, N, x,
+                     (const uint32_t *)nullptr, y, (float *)nullptr);
+  return launch_status();
+}
+
+int adh_softmax_xent_fwd(uint32_t C, uint32_t N, const float *x, const uint32_t *label, float *y, float *loss,
+                         void *stream) {
+  if (C == 0 || N == 0) return ADH_OK;
+  if (!x || !y || !label || !loss) return ADH_ENULL;
+  if (!aligned_to(x, 4) || !aligned_to(y, 4) || !aligned_to(label, 4) || !aligned_to(loss, 4)) return ADH_EALIGN;
+  hipLaunchKernelGGL((softmax_row_kernel<true>), dim3(N), dim3(kWave), 0, as_stream(stream), C, N, x, label, y, loss);
+  return launch_status();
+}
+
+int adh_softmax_nll_loss_fwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label, float *loss,
+                             void *stream) {
+  if (C == 0 || N == 0) return ADH_OK;
+  if (!y || !label || !loss) return ADH_ENULL;
+  if (!aligned_to(y, 4) || !aligned_to(label, 4) || !aligned_to(loss, 4)) return ADH_EALIGN;
+  hipLaunchKernelGGL(nll_loss_fwd_kernel, dim3((N + 255) / 256), dim3(256), 0, as_stream(stream), C, N, y, label,
+                     loss);
+  return launch_status();
+}
+
+int adh_softmax_nll_loss_bwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label, const float *dloss,
+                             float *dx, void *stream) {
+  if (C == 0 || N == 0) return ADH_OK;
+  if (!y || !label || !dloss || !dx) return ADH_ENULL;
+  if (!aligned_to(y, 4) || !aligned_to(label, 4) || !aligned_to(dloss, 4) || !aligned_to(dx, 4)) return ADH_EALIGN;
+  if (N > 65535u) {
+    // rows beyond the grid.y limit: split the launch
+    for (uint32_t i0 = 0; i0 < N; i0 += 65535u) {
+      const uint32_t rows = (N - i0) < 65535u ? (N - i0) : 65535u;
+      hipLaunchKernelGGL(nll_loss_bwd_kernel, dim3((C + 255) / 256, rows), dim3(256), 0, as_stream(stream), C, rows,
+                         y + (uint64_t)i0 * C, label + i0, dloss + i0, dx + (uint64_t)i0 * C);
+    }
+    return launch_status();
+  }
+  hipLaunchKernelGGL(nll_loss_bwd_kernel, dim3((C + 255) / 256, N), dim3(256), 0, as_stream(stream), C, N, y, label,
+                     dloss, dx);
+  return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,188 @@
+/*
+ * adh_capi.h -- C ABI of the MI355X (gfx950) spatially-parallel convolution path.
+ *
+ * This is the launcher-level seam of the reference
+ * (include/arraydiff/kernels.hh:72-262 plus the cuDNN calls in src/op.cc):
+ * free functions taking raw device pointers, uint32 extents and a stream, which
+ * enqueue work asynchronously and own nothing.  Differences, on purpose:
+ *   - every function returns int: 0 = ok, <0 = ADH_E* argument error (nothing was
+ *     enqueued), >0 = a hipError_t from the launch.  Nothing aborts.
+ *   - one launch serves all K tiles that live in this GPU's memory, where the
+ *     reference launched one kernel per rank; `*_rank` variants do one rank's share
+ *     so that a per-rank caller (Spatial2DComm::group_end) keeps its call shape.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *
+ * Layout: NCHW with W fastest, idx = w + W*(h + H*(c + C*n))
+ * (src/kernels/spatial.cu:22-36).  A halo-padded tile of interior (W,H) and halo p
+ * is a packed (W+2p, H+2p, C, N) buffer; "tile pointers" are BASE pointers of such
+ * buffers (what GPUBatchArray::base_as_view().dptr() returns,
+ * include/arraydiff/array_gpu.hh:544-548).  Pointer tables (`void* const*`) are
+ * HOST arrays of DEVICE pointers; they are read before the call returns.
+ *
+ * Re-entrant, no global state, callable from any host thread.
+ */
+#ifndef ADH_CAPI_H
+#define ADH_CAPI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ADH_VERSION 1
+
+/* element types (Spatial2DDataType in include/arraydiff/spatial.hh:25-29 has
+ * FLOAT/DOUBLE/HALF and only FLOAT is implemented, src/spatial.cc:76-78) */
+#define ADH_F32 0
+#define ADH_BF16 1
+
+/* error codes */
+#define ADH_OK 0
+#define ADH_EINVAL (-1)  /* bad extent, window out of bounds, H % K != 0, too many tiles */
+#define ADH_EUNIMPL (-2) /* combination the reference asserts "unimplemented" on, e.g. 2x2 grid */
+#define ADH_ENULL (-3)   /* a required pointer is NULL (src/spatial.cc:71-73) */
+#define ADH_EALIGN (-4)  /* pointer not aligned to its element size */
+#define ADH_EWORKSPACE (-5) /* workspace too small; see *_workspace_bytes */
+
+#define ADH_MAX_TILES 16 /* ARRAYDIFF_MAX_PEERS is 8, include/arraydiff/spatial.hh:11 */
+
+int adh_version(void);
+const char *adh_error_string(int code);
+
+/* ---- Z1: whole-buffer fill / accumulate ---------------------------------- */
+/* array_set_constant_packed<float>, src/kernels/array.cu:58-68,155-164 */
+int adh_fill_f32(uint64_t n, float value, float *x, void *stream);
+/* array_add_packed<float> (y += x), src/kernels/array.cu:83-94,199-208 */
+int adh_add_f32(uint64_t n, const float *x, float *y, void *stream);
+
+/* ---- H1/H2/H3: halo exchange / reduce ------------------------------------- */
+/* spatial2d_1x{2,4}_halo_exch_nchw, src/kernels/spatial.cu:455-485,596-623 (rows),
+ * spatial2d_2x1_halo_exch_nchw :708-731 (columns), for any K <= ADH_MAX_TILES.
+ * grid_w x grid_h follows Spatial2DComm::group_end, src/spatial.cc:76-135:
+ * 1x1 no-op, 1xK rows, Kx1 columns, both > 1 -> ADH_EUNIMPL.
+ * W,H are one tile's interior extents; tile_bufs[r], r = r_w + grid_w*r_h. */
+int adh_halo_exchange_nchw(int dtype, uint32_t grid_w, uint32_t grid_h, uint32_t halo_pad,
+                           uint32_t W, uint32_t H, uint32_t C, uint32_t N,
+                           void *const *tile_bufs, void *stream);
+/* spatial2d_1x{2,4}_halo_reduce_nchw, src/kernels/spatial.cu:487-510,625-652.
+ * Plain (non-atomic) adds: needs H >= 2*halo_pad (W >= 2*halo_pad for columns) so each
+ * destination has one contributor, else ADH_EINVAL.  Column reduce (declared but never
+ * linked in the reference, src/spatial.cc:166-178) is the W mirror of the row reduce. */
+int adh_halo_reduce_nchw(int dtype, uint32_t grid_w, uint32_t grid_h, uint32_t halo_pad,
+                         uint32_t W, uint32_t H, uint32_t C, uint32_t N,
+                         void *const *tile_bufs, void *stream);
+/* one rank's share of the above (what one reference kernel launch did) */
+int adh_halo_exchange_nchw_rank(int dtype, uint32_t grid_w, uint32_t grid_h, uint32_t rank,
+                                uint32_t halo_pad, uint32_t W, uint32_t H, uint32_t C, uint32_t N,
+                                void *const *tile_bufs, void *stream);
+int adh_halo_reduce_nchw_rank(int dtype, uint32_t grid_w, uint32_t grid_h, uint32_t rank,
+                              uint32_t halo_pad, uint32_t W, uint32_t H, uint32_t C, uint32_t N,
+                              void *const *tile_bufs, void *stream);
+
+/* ---- P1/P2/P3: pad / unpad (the strided cudnnAddTensor uses) -------------- */
+/* HaloPad2DOp::_forward, src/op.cc:2574-2641: whole padded buffer zeroed, interior = x.
+ * One pass instead of memset + AddTensor. */
+int adh_halo_pad_nchw(int dtype, uint32_t halo_pad, uint32_t W, uint32_t H, uint32_t C, uint32_t N,
+                      const void *x_packed, void *y_padded, void *stream);
+/* HaloUnpad2DOp::_backward, src/op.cc:2798-2870: interior(y_padded) += x_packed */
+int adh_halo_pad_add_nchw(int dtype, uint32_t halo_pad, uint32_t W, uint32_t H, uint32_t C, uint32_t N,
+                          const void *x_packed, void *y_padded, void *stream);
+/* HaloUnpad2DOp::_forward, src/op.cc:2715-2793: y_packed = interior(x_padded) */
+int adh_halo_unpad_nchw(int dtype, uint32_t halo_pad, uint32_t W, uint32_t H, uint32_t C, uint32_t N,
+                        const void *x_padded, void *y_packed, void *stream);
+/* HaloPad2DOp::_backward, src/op.cc:2644-2712: y_packed += interior(x_padded) */
+int adh_halo_unpad_add_nchw(int dtype, uint32_t halo_pad, uint32_t W, uint32_t H, uint32_t C, uint32_t N,
+                            const void *x_padded, void *y_packed, void *stream);
+/* HaloRepad2DOp::_forward, src/op.cc:2873-2960: interior of a p_src buffer -> interior of a
+ * p_dst buffer whose border is zeroed */
+int adh_halo_repad_nchw(int dtype, uint32_t pad_src, uint32_t pad_dst, uint32_t W, uint32_t H,
+                        uint32_t C, uint32_t N, const void *x_padded, void *y_padded, void *stream);
+
+/* ---- S1/S2: box copy / add between packed NCHW tensors -------------------- */
+/* slice2d_copy_hw_nchw_packed / slice2d_add_hw_nchw_packed, src/kernels/slice.cu:43-105,
+ * extended by a channel range (the reference's call is count_c == src_C == dst_C, c offsets 0).
+ * Window bounds are checked like slice.cu:61-64 but reported as ADH_EINVAL. */
+int adh_slice_copy_nchw(int dtype, uint32_t count_w, uint32_t count_h, uint32_t count_c, uint32_t N,
+                        const void *src, uint32_t src_W, uint32_t src_H, uint32_t src_C,
+                        uint32_t src_w_off, uint32_t src_h_off, uint32_t src_c_off,
+                        void *dst, uint32_t dst_W, uint32_t dst_H, uint32_t dst_C,
+                        uint32_t dst_w_off, uint32_t dst_h_off, uint32_t dst_c_off, void *stream);
+int adh_slice_add_nchw(int dtype, uint32_t count_w, uint32_t count_h, uint32_t count_c, uint32_t N,
+                       const void *src, uint32_t src_W, uint32_t src_H, uint32_t src_C,
+                       uint32_t src_w_off, uint32_t src_h_off, uint32_t src_c_off,
+                       void *dst, uint32_t dst_W, uint32_t dst_H, uint32_t dst_C,
+                       uint32_t dst_w_off, uint32_t dst_h_off, uint32_t dst_c_off, void *stream);
+
+/* ---- fused pack / unpack --------------------------------------------------- */
+/* pack = SpatialScatter2DOp::_forward (src/op.cc:2396-2429) + HaloPad2DOp::_forward +
+ * HaloExch2DOp::_forward (src/op.cc:2963-3003) in one pass: unsplit (W,H,C,N) -> K padded
+ * tiles of (W+2p, H/K+2p, C, N), halo rows filled from the neighbouring rows, border zero.
+ * H is the UNSPLIT height, H % K == 0 (src/op.cc:2385-2387), H/K >= halo_pad. */
+int adh_tiles_pack_nchw(int dtype, uint32_t K, uint32_t halo_pad, uint32_t W, uint32_t H, uint32_t C,
+                        uint32_t N, const void *x_unsplit, void *const *tile_bufs, void *stream);
+/* unpack = HaloUnpad2DOp::_forward + SpatialGather2DOp::_forward (src/op.cc:2480-2514):
+ * interiors of K padded tiles -> unsplit tensor; halo contents are ignored. */
+int adh_tiles_unpack_nchw(int dtype, uint32_t K, uint32_t halo_pad, uint32_t W, uint32_t H, uint32_t C,
+                          uint32_t N, const void *const *tile_bufs, void *y_unsplit, void *stream);
+
+/* ---- C2/C3/C4: 3x3 convolution over the halo-padded slab ------------------ */
+/* All three: cross-correlation, stride 1, dilation 1, conv pad 0 over a slab padded by 1
+ * (Conv2DShape.halo_padded_input, src/op.cc:1354-1410), filter KCRS (Cout,Cin,3,3),
+ * no bias.  beta is 0 (overwrite) or 1 (accumulate), the two values the reference passes.
+ * `*_tiles` variants run K slabs of identical shape in one launch.  Workspace may be NULL
+ * when the matching *_workspace_bytes query returns 0. */
+#define ADH_CONV_FWD 0
+#define ADH_CONV_BWD_DATA 1
+#define ADH_CONV_BWD_FILTER 2
+size_t adh_conv3x3_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,
+                                   uint32_t Cout, uint32_t H, uint32_t W);
+/* cudnnConvolutionForward at src/op.cc:1576-1587:
+ * y[n,co,h,w] = beta*y + sum_{ci,kh,kw} w[co,ci,kh,kw] * x_pad[n,ci,h+kh,w+kw] */
+int adh_conv3x3_slab_fwd(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                         const void *x_pad, const void *w, void *y, float beta,
+                         void *workspace, size_t workspace_bytes, void *stream);
+int adh_conv3x3_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                               uint32_t H, uint32_t W, const void *const *x_pad_tiles, const void *w,
+                               void *const *y_tiles, float beta, void *workspace,
+                               size_t workspace_bytes, void *stream);
+/* cudnnConvolutionBackwardData at src/op.cc:1701-1712: writes the WHOLE padded slab
+ * dx_pad[n,ci,h',w'] = beta*dx_pad + sum_{co,kh,kw} w[co,ci,kh,kw] * dy[n,co,h'-kh,w'-kw] */
+int adh_conv3x3_slab_bwd_data(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                              const void *w, const void *dy, void *dx_pad, float beta,
+                              void *workspace, size_t workspace_bytes, void *stream);
+int adh_conv3x3_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                    uint32_t H, uint32_t W, const void *w, const void *const *dy_tiles,
+                                    void *const *dx_pad_tiles, float beta, void *workspace,
+                                    size_t workspace_bytes, void *stream);
+/* cudnnConvolutionBackwardFilter at src/op.cc:1660-1671:
+ * dw[co,ci,kh,kw] = beta*dw + sum_{tiles,n,h,w} dy[n,co,h,w] * x_pad[n,ci,h+kh,w+kw]
+ * (the sum over tiles is what ParallelSGDOptimizer's ncclReduce did across ranks,
+ * include/arraydiff/optimize.hh:443-451).  dw is always fp32.  Deterministic. */
+int adh_conv3x3_slab_bwd_filter(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                                const void *x_pad, const void *dy, float *dw, float beta,
+                                void *workspace, size_t workspace_bytes, void *stream);
+int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,
+                                      uint32_t Cout, uint32_t H, uint32_t W,
+                                      const void *const *x_pad_tiles, const void *const *dy_tiles,
+                                      float *dw, float beta, void *workspace, size_t workspace_bytes,
+                                      void *stream);
+
+/* ---- L1/L2/L3: softmax + negative log likelihood (fp32) ------------------- */
+/* cudnnSoftmaxForward(ACCURATE, MODE_INSTANCE) on (N,C,1,1), src/op.cc:4129-4152 */
+int adh_softmax_fwd(uint32_t C, uint32_t N, const float *x, float *y, void *stream);
+/* softmax_nll_loss_fwd<float>, src/kernels/softmax.cu:36-54,86-89 */
+int adh_softmax_nll_loss_fwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label,
+                             float *loss, void *stream);
+/* softmax_nll_loss_bwd<float>, src/kernels/softmax.cu:56-78,92-95: dx += dloss*(y - onehot) */
+int adh_softmax_nll_loss_bwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label,
+                             const float *dloss, float *dx, void *stream);
+/* CudnnSoftmaxNLLLossOp::_forward, src/op.cc:4118-4163, in one kernel: y and loss together */
+int adh_softmax_xent_fwd(uint32_t C, uint32_t N, const float *x, const uint32_t *label, float *y,
+                         float *loss, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ADH_CAPI_H */
