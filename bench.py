@@ -1,0 +1,240 @@
+#!/usr/bin/env python3
+"""Benchmark of the spatially-parallel convolution path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one pass of the hot path's dominant stage over one batch of synthetic input:
+the 3x3 slab convolution forward over the 4 halo-padded row-tiles of a ResNet-50
+conv2_x-shaped activation (fp32 NCHW N=32, Cin=Cout=64, 4 tiles of 14(+2) x 56(+2)), one launch
+through the C ABI, inputs resident in HBM.  One JSON line is printed: `value` is the conv
+throughput in TFLOP/s (algorithmic flops 2*N*Cout*Cin*H*W*9 per tile), `roofline` is that
+kernel against the fp32 MFMA peak, `cpu_baseline` is the scalar CPU port timed on this host,
+and `secondary` carries the HBM-bound kernels of the path (halo pack / unpack / exchange /
+reduce, channel slice, softmax-NLL) and the two backward convolutions with their own roofline
+figures.  Everything is timed with device events on the stream the kernels are launched on.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F32_PEAK_TFLOPS = 157.3
+METRIC = "halo pack/unpack GB/s (% HBM peak); 3x3 slab-conv TFLOP/s (% MFMA peak)"
+
+
+def time_gpu(fn, reps, warmup):
+    """Average milliseconds per call of fn(), device events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-secondary", action="store_true", help="time only the headline kernel")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU (the K row-tiles live in one HBM, there are no "
+              "inter-GPU collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from arraydiff_cuda_amd import capi
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; there is no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+    lib = capi.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    # ---- workload: BASELINE configs[1] (conv) on the tensors of configs[0] (halo) ----
+    K, p, N, C, H, W = 4, 1, 32, 64, 56, 56
+    Ht = H // K
+    g = torch.Generator(device="cuda").manual_seed(0x5EED)
+    X = torch.rand((N, C, H, W), device="cuda", generator=g) * 2 - 1
+    wt = torch.randn((C, C, 3, 3), device="cuda", generator=g) * (2.0 / (C * 9)) ** 0.5
+    dY = torch.randn((N, C, H, W), device="cuda", generator=g)
+    tiles = [torch.empty((N, C, Ht + 2, W + 2), device="cuda") for _ in range(K)]
+    ys = [torch.empty((N, C, Ht, W), device="cuda") for _ in range(K)]
+    dys = [dY[:, :, r * Ht:(r + 1) * Ht].contiguous() for r in range(K)]
+    gs = [torch.zeros((N, C, Ht + 2, W + 2), device="cuda") for _ in range(K)]
+    gw = torch.zeros_like(wt)
+    Y = torch.empty_like(X)
+    capi.check(capi.tiles_pack(K, p, W, H, C, N, X, tiles), "pack")
+
+    tile_tbl, _k1 = capi.ptr_table([t.data_ptr() for t in tiles])
+    y_tbl, _k2 = capi.ptr_table([t.data_ptr() for t in ys])
+    dy_tbl, _k3 = capi.ptr_table([t.data_ptr() for t in dys])
+    g_tbl, _k4 = capi.ptr_table([t.data_ptr() for t in gs])
+    ws_bytes = capi.conv_workspace_bytes(capi.ADH_CONV_BWD_FILTER, capi.ADH_F32, K, N, C, C, Ht, W)
+    ws = torch.empty(max(ws_bytes // 4, 1), device="cuda")
+
+    def conv_fwd():
+        lib.adh_conv3x3_slab_fwd_tiles(capi.ADH_F32, K, N, C, C, Ht, W, tile_tbl, wt.data_ptr(), y_tbl, 0.0,
+                                       None, 0, stream)
+
+    capi.check(lib.adh_conv3x3_slab_fwd_tiles(capi.ADH_F32, K, N, C, C, Ht, W, tile_tbl, wt.data_ptr(), y_tbl, 0.0,
+                                              None, 0, stream), "conv fwd")
+
+    # ---- the timed region: W warmup steps, then exactly K steps between two synchronisations ----
+    for _ in range(args.warmup):
+        conv_fwd()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        conv_fwd()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    kernel_ms = e0.elapsed_time(e1) / args.steps
+    flops_step = 2.0 * N * C * C * Ht * W * 9 * K
+    value = flops_step / (ms_per_step * 1e-3) / 1e12
+    achieved = flops_step / (kernel_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": METRIC, "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: 3x3 slab conv fwd, fp32 NCHW N=32 Cin=Cout=64, 4 row-tiles of "
+                               "14(+2)x56(+2), one launch over all tiles",
+                   "flops_per_step": flops_step, "tiles": K, "halo": p},
+        "roofline": {"kernel": "conv3x3_f32_kernel<25,3> (fwd)", "bound": "mfma", "achieved": round(achieved, 3),
+                     "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / MFMA_F32_PEAK_TFLOPS, 4),
+                     "traffic": None, "launch_ms": round(kernel_ms, 5)},
+    }
+
+    # ---- secondary kernels of the path ----
+    if not args.no_secondary:
+        es = 4
+        strip = p * W * C * N * es
+        reps, wu = 200, 20
+        sec = []
+
+        def add(name, fn, bound, work, peak, unit, note=None):
+            ms = time_gpu(fn, reps, wu)
+            ach = work / (ms * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
+            e = {"name": name, "ms": round(ms, 5), "bound": bound, "achieved": round(ach, 3), "peak": peak,
+                 "unit": unit, "frac": round(ach / peak, 4), "work": work}
+            if note:
+                e["note"] = note
+            sec.append(e)
+
+        unsplit_b = N * C * H * W * es
+        padded_b = K * N * C * (Ht + 2 * p) * (W + 2 * p) * es
+        add("halo pack cfg1 (unsplit -> 4 padded tiles)",
+            lambda: lib.adh_tiles_pack_nchw(0, K, p, W, H, C, N, X.data_ptr(), tile_tbl, stream),
+            "hbm", unsplit_b + padded_b, HBM_PEAK_GBS, "GB/s")
+        add("halo unpack cfg1 (4 padded tiles -> unsplit)",
+            lambda: lib.adh_tiles_unpack_nchw(0, K, p, W, H, C, N, tile_tbl, Y.data_ptr(), stream),
+            "hbm", 2 * unsplit_b, HBM_PEAK_GBS, "GB/s")
+        add("halo exchange cfg1 (6 strips)",
+            lambda: lib.adh_halo_exchange_nchw(0, 1, K, p, W, Ht, C, N, tile_tbl, stream),
+            "hbm", 2 * 2 * (K - 1) * strip, HBM_PEAK_GBS, "GB/s",
+            note="reference figure of merit p*W*C*N*4/t = %d B / t" % strip)
+        add("halo reduce cfg1 (6 strips)",
+            lambda: lib.adh_halo_reduce_nchw(0, 1, K, p, W, Ht, C, N, g_tbl, stream),
+            "hbm", 3 * 2 * (K - 1) * strip, HBM_PEAK_GBS, "GB/s")
+        sl = torch.empty((N, 32, H, W), device="cuda")
+        add("channel slice [16,48) cfg4",
+            lambda: lib.adh_slice_copy_nchw(0, W, H, 32, N, X.data_ptr(), W, H, C, 0, 0, 16, sl.data_ptr(), W, H, 32,
+                                            0, 0, 0, stream),
+            "hbm", 2 * N * 32 * H * W * es, HBM_PEAK_GBS, "GB/s")
+        Ns, Cs = 256, 1000
+        logits = torch.randn((Ns, Cs), device="cuda", generator=g) * 2
+        labels = torch.randint(0, Cs, (Ns,), device="cuda", dtype=torch.int32)
+        sy = torch.empty_like(logits)
+        sloss = torch.empty(Ns, device="cuda")
+        sdx = torch.zeros_like(logits)
+        dl = torch.full((Ns,), 1.0 / Ns, device="cuda")
+        add("softmax + nll fwd cfg4 (256x1000)",
+            lambda: lib.adh_softmax_xent_fwd(Cs, Ns, logits.data_ptr(), labels.data_ptr(), sy.data_ptr(),
+                                             sloss.data_ptr(), stream),
+            "hbm", 2 * Ns * Cs * 4 + 8 * Ns, HBM_PEAK_GBS, "GB/s")
+        add("softmax-nll bwd cfg4 (256x1000)",
+            lambda: lib.adh_softmax_nll_loss_bwd(Cs, Ns, sy.data_ptr(), labels.data_ptr(), dl.data_ptr(),
+                                                 sdx.data_ptr(), stream),
+            "hbm", 3 * Ns * Cs * 4 + 8 * Ns, HBM_PEAK_GBS, "GB/s")
+        add("conv bwd-data cfg3 (4 tiles)",
+            lambda: lib.adh_conv3x3_slab_bwd_data_tiles(0, K, N, C, C, Ht, W, wt.data_ptr(), dy_tbl, g_tbl, 0.0, None,
+                                                        0, stream),
+            "mfma", flops_step, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+        add("conv bwd-filter cfg3 (4 tiles, two kernels)",
+            lambda: lib.adh_conv3x3_slab_bwd_filter_tiles(0, K, N, C, C, Ht, W, tile_tbl, dy_tbl, gw.data_ptr(), 0.0,
+                                                          ws.data_ptr(), ws_bytes, stream),
+            "mfma", flops_step, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+
+        # config 5 sized pack / unpack: 0.5 GB, larger than the on-package cache
+        K5, N5, H5, W5 = 8, 2, 1024, 2048
+        X5 = (torch.rand((N5, C, H5, W5), device="cuda", generator=g) * 2 - 1).to(torch.bfloat16)
+        t5 = [torch.empty((N5, C, H5 // K5 + 2, W5 + 2), device="cuda", dtype=torch.bfloat16) for _ in range(K5)]
+        t5_tbl, _k5 = capi.ptr_table([t.data_ptr() for t in t5])
+        Y5 = torch.empty_like(X5)
+        b5 = N5 * C * H5 * W5 * 2
+        reps, wu = 50, 5
+        add("halo pack cfg5 (bf16, 8 tiles of 128 rows)",
+            lambda: lib.adh_tiles_pack_nchw(1, K5, 1, W5, H5, C, N5, X5.data_ptr(), t5_tbl, stream),
+            "hbm", b5 + K5 * N5 * C * (H5 // K5 + 2) * (W5 + 2) * 2, HBM_PEAK_GBS, "GB/s")
+        add("halo unpack cfg5 (bf16)",
+            lambda: lib.adh_tiles_unpack_nchw(1, K5, 1, W5, H5, C, N5, t5_tbl, Y5.data_ptr(), stream),
+            "hbm", 2 * b5, HBM_PEAK_GBS, "GB/s")
+        del X5, t5, Y5
+        out["secondary"] = sec
+
+    # ---- CPU baseline: the scalar port, single thread, on a bounded sample ----
+    if not args.no_cpu:
+        import oracle
+        wn = wt.cpu().numpy()
+        host_x = [t.cpu().numpy() for t in tiles]
+        yc = np.empty((N, C, Ht, W), np.float32)
+        cpu_reps = 2  # 2 passes over all 4 tiles = 14.8 GFLOP of scalar work
+        t0 = time.perf_counter()
+        for _ in range(cpu_reps):
+            for r in range(K):
+                oracle.conv_slab_fwd_f32(host_x[r], wn, yc)
+        dt = (time.perf_counter() - t0) / cpu_reps
+        err = float(np.abs(yc - ys[K - 1].cpu().numpy()).max() / np.abs(yc).max())
+        out["cpu_baseline"] = {
+            "value": round(flops_step / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": "%d passes over the same 4 tiles (N=32, C=64, 14x56 outputs each, 7.4 GFLOP per pass), scalar "
+                      "fp32 direct conv, gcc -O2, one thread, %.2f s per pass; GPU result agrees to rel-err %.1e"
+                      % (cpu_reps, dt, err)}
+        # the reference kernels' own loop structure for the halo exchange (idx -> (w,c,n) by div/mod)
+        host_tiles = [t.cpu().numpy() for t in tiles]
+        t0 = time.perf_counter()
+        reps_cpu = 20
+        for _ in range(reps_cpu):
+            oracle.halo_op(oracle.EXCH, 1, K, p, W, Ht, C, N, host_tiles)
+        dt = (time.perf_counter() - t0) / reps_cpu
+        out["cpu_baseline"]["halo_exchange_GBs"] = round(2 * 2 * (K - 1) * p * W * C * N * 4 / dt / 1e9, 3)
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
