@@ -4,12 +4,14 @@
 //
 // All of these are HBM-bound copies with at most one add per element.  The two rules
 // that shape them:
-//   * every destination buffer that is contiguous is written with 16-byte stores by
-//     consecutive lanes (a wavefront writes 1 KiB contiguous), the shifted source rows
-//     are gathered with element loads that stay inside the same cache lines;
-//   * one launch covers all K tiles and all planes: grid = (chunks of one plane, C,
-//     N * tiles), so a launch has thousands of workgroups and only one division by a
-//     launch-time constant (a mul_hi) per thread.
+//   * every destination buffer that is contiguous is written with aligned 16-byte stores by
+//     consecutive lanes (a wavefront writes 1 KiB contiguous); the matching source run is
+//     fetched with ONE 16-byte load at the source's own element alignment (padded rows are
+//     shifted by 2p elements per row, so source and destination can never both be 16-byte
+//     aligned); only vectors that straddle a row end fall back to element loads;
+//   * one launch covers all K tiles and all planes, so a launch has thousands of
+//     workgroups; index arithmetic is two or three divisions by launch-time constants
+//     (mul_hi + shift) per 16 bytes.
 #include "adh_common.h"
 
 namespace adh {
@@ -17,149 +19,166 @@ namespace adh {
 static constexpr int kBlock = 256;
 
 // ---------------------------------------------------------------------------
-// plane_gather: dst planes are contiguous (DW x DH elements each); every dst element is
-// either a source element at a shifted position or zero.  Serves pack, pad, repad,
-// unpack, unpad and full-row slices.
+// row_copy: the one copy kernel behind pack, unpack, pad, unpad, repad and all slices.
+//
+// For every destination row (hp, c, n) of every destination buffer r:
+//   source row gs = hp - off_h + r*row_step; if 0 <= gs < valid_h the W elements
+//   dst[hp][off_w .. off_w+W) are copied from (or, ADD, incremented by) the source row,
+//   else they are zeroed (never when ADD);
+//   with ZERO_BORDER the dst columns left and right of the copied run are zeroed too.
+// A thread moves one vector of EPT consecutive elements of a row with ONE 16-byte load and
+// ONE 16-byte store, both at element alignment (padded rows are shifted by 2p elements per
+// row, so source and destination can never both be 16-byte aligned; the hardware takes
+// unaligned vector accesses, and a wavefront still touches one contiguous run per row).
+// Each thread handles VPT vectors, all loads issued before the first store.
 // ---------------------------------------------------------------------------
-struct GatherParams {
-  void *dst[ADH_MAX_TILES];
+struct RowCopyParams {
+  void *dst[ADH_MAX_TILES];        // per launch-row r = blockIdx.y
   const void *src[ADH_MAX_TILES];
-  uint32_t n_dst;          // number of dst tiles; blockIdx.z = n * n_dst + r
-  uint32_t DW, DH;         // dst plane dims; plane_elems = DW * DH
-  uint32_t plane_elems;
-  uint64_t dst_off;        // element offset of plane (c=0,n=0) in each dst buffer
-  uint64_t dst_c_stride, dst_n_stride;
-  int32_t off_w, off_h;    // src coords: ws = wp - off_w, gs = hp - off_h + r * row_step
-  uint32_t row_step;
-  uint32_t valid_w, valid_h;  // src element exists iff 0 <= ws < valid_w && 0 <= gs < valid_h
-  uint32_t src_rows_per_tile; // ROW_TILED: source tile = gs / src_rows_per_tile
-  uint64_t src_off;           // element offset of (ws=0, gs=0, c=0, n=0) in each src buffer
-  uint64_t src_c_stride, src_n_stride;
+  uint32_t W;                // elements moved per row
+  uint32_t VR;               // vectors per row = ceil(W / EPT)
+  uint32_t DH;               // destination rows per plane
+  uint32_t C;                // planes per image (plane = c + C*n)
+  uint32_t total_vectors;    // VR * DH * C * N  (per destination buffer)
+  uint32_t dst_pitch, off_w; // dst row pitch and first written column
+  uint32_t border_l, border_r;  // ZERO_BORDER: columns zeroed left / right of the run
+  uint64_t dst_off, dst_c_stride, dst_n_stride;
+  int32_t off_h;
+  uint32_t row_step, valid_h;
   uint32_t src_pitch;
-  FastDiv div_DW, div_rows;
+  uint64_t src_off, src_c_stride, src_n_stride;
+  FastDiv div_VR, div_DH, div_C;
 };
 
-template <typename T, int EPT>
-struct VecOf;
-template <>
-struct VecOf<float, 4> { typedef float4 type; };
-template <>
-struct VecOf<float, 1> { typedef float type; };
-template <>
-struct VecOf<uint16_t, 8> { typedef uint4 type; };
-template <>
-struct VecOf<uint16_t, 1> { typedef uint16_t type; };
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// 16 bytes at 2-byte alignment: valid for both element types (fp32 rows are 4-byte aligned)
+typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
 
-template <typename T, int EPT, bool ROW_TILED>
-__global__ __launch_bounds__(kBlock) void plane_gather_kernel(const GatherParams P) {
-  const uint32_t c = blockIdx.y;
-  const uint32_t z = blockIdx.z;
-  const uint32_t n = z / P.n_dst;
-  const uint32_t r = z - n * P.n_dst;
-  const uint32_t e0 = (blockIdx.x * kBlock + threadIdx.x) * EPT;
-  if (e0 >= P.plane_elems) return;
-  uint32_t hp, wp;
-  P.div_DW.divmod(e0, hp, wp);
-  const int32_t row_base = (int32_t)(r * P.row_step) - P.off_h;
-  const uint64_t src_plane = P.src_off + c * P.src_c_stride + n * P.src_n_stride;
-  union {
-    typename VecOf<T, EPT>::type v;
+// TAIL = (W % EPT != 0): the last vector of a row is partial and is moved element-wise.
+template <typename T, bool ADD, bool ZERO_BORDER, bool TAIL, int VPT>
+__global__ __launch_bounds__(kBlock) void row_copy_kernel(const RowCopyParams P) {
+  constexpr int EPT = 16 / sizeof(T);
+  typedef u32x4_unaligned VU;
+  union Pack {
+    u32x4 v;
     T e[EPT];
-  } out;
+  };
+  const uint32_t r = blockIdx.y;
+  const T *__restrict__ sbase = reinterpret_cast<const T *>(P.src[r]) + P.src_off;
+  T *__restrict__ dbase = reinterpret_cast<T *>(P.dst[r]) + P.dst_off;
+  const int32_t row_base = (int32_t)(r * P.row_step) - P.off_h;
+
+  uint64_t so[VPT], dof[VPT];
+  uint32_t cnt[VPT];   // elements of this vector inside the row (0 = no work)
+  bool have_src[VPT], first[VPT];
+  u32x4 in[VPT], old[VPT];
+
 #pragma unroll
-  for (int i = 0; i < EPT; ++i) {
-    const int32_t ws = (int32_t)wp - P.off_w;
-    int32_t gs = (int32_t)hp + row_base;
-    T val = (T)0;
-    if ((uint32_t)ws < P.valid_w && (uint32_t)gs < P.valid_h) {
-      uint32_t t = 0;
-      if (ROW_TILED) {
-        t = P.div_rows.div((uint32_t)gs);
-        gs -= (int32_t)(t * P.src_rows_per_tile);
+  for (int k = 0; k < VPT; ++k) {
+    const uint32_t v = (blockIdx.x * VPT + k) * kBlock + threadIdx.x;
+    const bool live = v < P.total_vectors;
+    uint32_t row, vr, pl, hp, n, c;
+    P.div_VR.divmod(live ? v : 0u, row, vr);
+    P.div_DH.divmod(row, pl, hp);
+    P.div_C.divmod(pl, n, c);
+    const uint32_t w0 = vr * EPT;
+    cnt[k] = live ? (TAIL ? min((uint32_t)EPT, P.W - w0) : (uint32_t)EPT) : 0u;
+    first[k] = vr == 0;
+    const int32_t gs = (int32_t)hp + row_base;
+    have_src[k] = (uint32_t)gs < P.valid_h;
+    so[k] = c * P.src_c_stride + n * P.src_n_stride + (uint64_t)(have_src[k] ? (uint32_t)gs : 0u) * P.src_pitch + w0;
+    dof[k] = c * P.dst_c_stride + n * P.dst_n_stride + (uint64_t)hp * P.dst_pitch + P.off_w + w0;
+    in[k] = u32x4{0u, 0u, 0u, 0u};
+    old[k] = u32x4{0u, 0u, 0u, 0u};
+  }
+  // all loads first
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    // addresses are valid even for idle threads and zero rows (clamped above), so the
+    // vector loads need no branch when rows have no tail
+    if (!TAIL || cnt[k] == (uint32_t)EPT) {
+      in[k] = *reinterpret_cast<const VU *>(sbase + so[k]);
+      if (ADD) old[k] = *reinterpret_cast<const VU *>(dbase + dof[k]);
+    } else if (TAIL && cnt[k] > 0) {
+      Pack pi, po;
+      pi.v = in[k];
+      po.v = old[k];
+#pragma unroll
+      for (int i = 0; i < EPT - 1; ++i) {
+        if ((uint32_t)i < cnt[k]) {
+          pi.e[i] = sbase[so[k] + i];
+          if (ADD) po.e[i] = dbase[dof[k] + i];
+        }
       }
-      const T *s = reinterpret_cast<const T *>(P.src[t]);
-      val = s[src_plane + (uint64_t)gs * P.src_pitch + (uint32_t)ws];
-    }
-    out.e[i] = val;
-    if (++wp == P.DW) {
-      wp = 0;
-      ++hp;
+      in[k] = pi.v;
+      old[k] = po.v;
     }
   }
-  T *d = reinterpret_cast<T *>(P.dst[r]) + P.dst_off + c * P.dst_c_stride + n * P.dst_n_stride + e0;
-  *reinterpret_cast<typename VecOf<T, EPT>::type *>(d) = out.v;
-}
-
-template <typename T, int EPT>
-static int launch_gather_t(const GatherParams &P, uint32_t C, uint32_t N, bool row_tiled, hipStream_t st) {
-  const uint32_t per_block = kBlock * EPT;
-  dim3 grid((P.plane_elems + per_block - 1) / per_block, C, N * P.n_dst);
-  if (grid.z > 65535u || grid.y > 65535u) return ADH_EINVAL;
-  if (row_tiled)
-    hipLaunchKernelGGL((plane_gather_kernel<T, EPT, true>), grid, dim3(kBlock), 0, st, P);
-  else
-    hipLaunchKernelGGL((plane_gather_kernel<T, EPT, false>), grid, dim3(kBlock), 0, st, P);
-  return launch_status();
-}
-
-// Picks the 16-byte-store variant when every dst plane start is 16-byte aligned.
-static int launch_gather(int dtype, GatherParams &P, uint32_t C, uint32_t N, bool row_tiled, hipStream_t st) {
-  if (P.plane_elems == 0 || C == 0 || N == 0) return ADH_OK;
-  P.div_DW = FastDiv(P.DW);
-  P.div_rows = FastDiv(P.src_rows_per_tile);
-  const size_t es = dtype_size(dtype);
-  const uint32_t ept = (uint32_t)(16 / es);
-  bool vec = (P.plane_elems % ept == 0) && (P.dst_off % ept == 0) && (P.dst_c_stride % ept == 0) &&
-             (P.dst_n_stride % ept == 0);
-  for (uint32_t r = 0; r < P.n_dst; ++r) vec = vec && aligned_to(P.dst[r], 16);
-  if (dtype == ADH_F32)
-    return vec ? launch_gather_t<float, 4>(P, C, N, row_tiled, st) : launch_gather_t<float, 1>(P, C, N, row_tiled, st);
-  return vec ? launch_gather_t<uint16_t, 8>(P, C, N, row_tiled, st)
-             : launch_gather_t<uint16_t, 1>(P, C, N, row_tiled, st);
-}
-
-// ---------------------------------------------------------------------------
-// box_map: general window copy / add, one element per thread.
-// ---------------------------------------------------------------------------
-struct BoxParams {
-  const void *src;
-  void *dst;
-  uint32_t cw, ch;  // window extents inside a plane
-  uint32_t src_pitch, dst_pitch;
-  uint64_t src_off, dst_off;  // element offset of window origin at (c=0, n=0)
-  uint64_t src_c_stride, src_n_stride, dst_c_stride, dst_n_stride;
-  FastDiv div_cw;
-};
-
-template <typename T, bool ADD>
-__global__ __launch_bounds__(kBlock) void box_map_kernel(const BoxParams P) {
-  const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
-  if (e >= P.cw * P.ch) return;
-  uint32_t h, w;
-  P.div_cw.divmod(e, h, w);
-  const uint32_t c = blockIdx.y, n = blockIdx.z;
-  const T *s = reinterpret_cast<const T *>(P.src) + P.src_off + c * P.src_c_stride + n * P.src_n_stride +
-               (uint64_t)h * P.src_pitch + w;
-  T *d = reinterpret_cast<T *>(P.dst) + P.dst_off + c * P.dst_c_stride + n * P.dst_n_stride +
-         (uint64_t)h * P.dst_pitch + w;
-  if (ADD)
-    *d = elem_add(*d, *s);
-  else
-    *d = *s;
-}
-
-static int launch_box(int dtype, bool add, BoxParams &P, uint32_t cc, uint32_t N, hipStream_t st) {
-  if (P.cw == 0 || P.ch == 0 || cc == 0 || N == 0) return ADH_OK;
-  if ((uint64_t)P.cw * P.ch >= (1ull << 31) || cc > 65535u || N > 65535u) return ADH_EINVAL;
-  P.div_cw = FastDiv(P.cw);
-  dim3 grid((P.cw * P.ch + kBlock - 1) / kBlock, cc, N);
-  if (dtype == ADH_F32) {
-    if (add) hipLaunchKernelGGL((box_map_kernel<float, true>), grid, dim3(kBlock), 0, st, P);
-    else hipLaunchKernelGGL((box_map_kernel<float, false>), grid, dim3(kBlock), 0, st, P);
-  } else {
-    if (add) hipLaunchKernelGGL((box_map_kernel<uint16_t, true>), grid, dim3(kBlock), 0, st, P);
-    else hipLaunchKernelGGL((box_map_kernel<uint16_t, false>), grid, dim3(kBlock), 0, st, P);
+  // Keep every load above this point (the empty asm consumes the loaded registers), so the
+  // compiler cannot sink a load into its store's branch and serialise load -> wait -> store.
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    asm volatile("" : "+v"(in[k]));
+    if (ADD) asm volatile("" : "+v"(old[k]));
   }
+  // then all stores
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    if (cnt[k] == 0) continue;
+    if (ADD && !have_src[k]) continue;
+    Pack out;
+    if (ADD) {
+      Pack pi, po;
+      pi.v = in[k];
+      po.v = old[k];
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) out.e[i] = elem_add(po.e[i], pi.e[i]);
+    } else {
+      out.v = have_src[k] ? in[k] : u32x4{0u, 0u, 0u, 0u};
+    }
+    T *d = dbase + dof[k];
+    if (!TAIL || cnt[k] == (uint32_t)EPT) {
+      *reinterpret_cast<VU *>(d) = out.v;
+    } else {
+#pragma unroll
+      for (int i = 0; i < EPT - 1; ++i)
+        if ((uint32_t)i < cnt[k]) d[i] = out.e[i];
+    }
+    if (ZERO_BORDER && first[k]) {
+      T *row = d - P.off_w;
+      for (uint32_t i = 0; i < P.border_l; ++i) row[i] = (T)0;
+      for (uint32_t i = 0; i < P.border_r; ++i) row[P.off_w + P.W + i] = (T)0;
+    }
+  }
+}
+
+template <typename T>
+static void launch_row_copy_t(bool add, bool zero_border, bool tail, const RowCopyParams &P, dim3 grid,
+                              hipStream_t st) {
+  constexpr int VPT = 2;
+#define ADH_RC(A, Z, TL) hipLaunchKernelGGL((row_copy_kernel<T, A, Z, TL, VPT>), grid, dim3(kBlock), 0, st, P)
+  if (add) { if (tail) ADH_RC(true, false, true); else ADH_RC(true, false, false); }
+  else if (zero_border) { if (tail) ADH_RC(false, true, true); else ADH_RC(false, true, false); }
+  else { if (tail) ADH_RC(false, false, true); else ADH_RC(false, false, false); }
+#undef ADH_RC
+}
+
+// N is the image count; P.C must be set.  All extents validated by the callers.
+static int launch_row_copy(int dtype, bool add, bool zero_border, RowCopyParams &P, uint32_t n_dst, uint32_t N,
+                           hipStream_t st) {
+  if (P.W == 0 || P.DH == 0 || P.C == 0 || N == 0 || n_dst == 0) return ADH_OK;
+  const uint32_t ept = (uint32_t)(16 / dtype_size(dtype));
+  P.VR = (P.W + ept - 1) / ept;
+  const uint64_t total = (uint64_t)P.VR * P.DH * P.C * N;
+  if (total >= (1ull << 31)) return ADH_EINVAL;
+  P.total_vectors = (uint32_t)total;
+  P.div_VR = FastDiv(P.VR);
+  P.div_DH = FastDiv(P.DH);
+  P.div_C = FastDiv(P.C);
+  const bool tail = P.W % ept != 0;
+  dim3 grid((P.total_vectors + kBlock * 2 - 1) / (kBlock * 2), n_dst, 1);
+  if (dtype == ADH_F32) launch_row_copy_t<float>(add, zero_border, tail, P, grid, st);
+  else launch_row_copy_t<uint16_t>(add, zero_border, tail, P, grid, st);
   return launch_status();
 }
 
@@ -390,17 +409,16 @@ static int pad_like(int dtype, uint32_t ps, uint32_t q, uint32_t W, uint32_t H, 
   const uint64_t DW = (uint64_t)W + 2 * q, DH = (uint64_t)H + 2 * q;
   const uint64_t SW = (uint64_t)W + 2 * ps, SH = (uint64_t)H + 2 * ps;
   if (!plane_limits_ok(DW * DH, DW * DH * C * N) || !plane_limits_ok(SW * SH, SW * SH * C * N)) return ADH_EINVAL;
-  GatherParams P = {};
+  RowCopyParams P = {};
   P.dst[0] = y;
   P.src[0] = x;
-  P.n_dst = 1;
-  P.DW = (uint32_t)DW; P.DH = (uint32_t)DH; P.plane_elems = (uint32_t)(DW * DH);
+  P.W = W; P.DH = (uint32_t)DH; P.C = C;
+  P.dst_pitch = (uint32_t)DW; P.off_w = q; P.border_l = q; P.border_r = q;
   P.dst_off = 0; P.dst_c_stride = DW * DH; P.dst_n_stride = DW * DH * C;
-  P.off_w = (int32_t)q; P.off_h = (int32_t)q; P.row_step = 0;
-  P.valid_w = W; P.valid_h = H; P.src_rows_per_tile = 1;
-  P.src_off = (uint64_t)ps * SW + ps; P.src_c_stride = SW * SH; P.src_n_stride = SW * SH * C;
+  P.off_h = (int32_t)q; P.row_step = 0; P.valid_h = H;
   P.src_pitch = (uint32_t)SW;
-  return launch_gather(dtype, P, C, N, false, as_stream(stream));
+  P.src_off = (uint64_t)ps * SW + ps; P.src_c_stride = SW * SH; P.src_n_stride = SW * SH * C;
+  return launch_row_copy(dtype, false, q > 0, P, 1, N, as_stream(stream));
 }
 
 int adh_halo_pad_nchw(int dtype, uint32_t halo_pad, uint32_t W, uint32_t H, uint32_t C, uint32_t N,
@@ -431,29 +449,16 @@ static int slice_op(bool add, int dtype, uint32_t cw, uint32_t ch, uint32_t cc, 
   if (!aligned_to(src, es) || !aligned_to(dst, es)) return ADH_EALIGN;
   const uint64_t splane = (uint64_t)sW * sH, dplane = (uint64_t)dW * dH;
   if (!plane_limits_ok(splane, splane * sC * N) || !plane_limits_ok(dplane, dplane * dC * N)) return ADH_EINVAL;
-  if (!add && cw == dW && ch == dH) {
-    // dst window = whole planes: contiguous destination, 16-byte stores
-    GatherParams P = {};
-    P.dst[0] = dst;
-    P.src[0] = src;
-    P.n_dst = 1;
-    P.DW = dW; P.DH = dH; P.plane_elems = (uint32_t)dplane;
-    P.dst_off = (uint64_t)dc * dplane; P.dst_c_stride = dplane; P.dst_n_stride = dplane * dC;
-    P.off_w = 0; P.off_h = 0; P.row_step = 0;
-    P.valid_w = cw; P.valid_h = ch; P.src_rows_per_tile = 1;
-    P.src_off = (uint64_t)sc * splane + (uint64_t)sh * sW + sw;
-    P.src_c_stride = splane; P.src_n_stride = splane * sC; P.src_pitch = sW;
-    return launch_gather(dtype, P, cc, N, false, as_stream(stream));
-  }
-  BoxParams B = {};
-  B.src = src; B.dst = dst;
-  B.cw = cw; B.ch = ch;
-  B.src_pitch = sW; B.dst_pitch = dW;
-  B.src_off = (uint64_t)sc * splane + (uint64_t)sh * sW + sw;
-  B.dst_off = (uint64_t)dc * dplane + (uint64_t)dh * dW + dw;
-  B.src_c_stride = splane; B.src_n_stride = splane * sC;
-  B.dst_c_stride = dplane; B.dst_n_stride = dplane * dC;
-  return launch_box(dtype, add, B, cc, N, as_stream(stream));
+  RowCopyParams P = {};
+  P.dst[0] = dst;
+  P.src[0] = src;
+  P.W = cw; P.DH = ch; P.C = cc;
+  P.dst_pitch = dW; P.off_w = 0;
+  P.dst_off = (uint64_t)dc * dplane + (uint64_t)dh * dW + dw; P.dst_c_stride = dplane; P.dst_n_stride = dplane * dC;
+  P.off_h = 0; P.row_step = 0; P.valid_h = ch;
+  P.src_pitch = sW;
+  P.src_off = (uint64_t)sc * splane + (uint64_t)sh * sW + sw; P.src_c_stride = splane; P.src_n_stride = splane * sC;
+  return launch_row_copy(dtype, add, false, P, 1, N, as_stream(stream));
 }
 
 int adh_slice_copy_nchw(int dtype, uint32_t count_w, uint32_t count_h, uint32_t count_c, uint32_t N,
@@ -496,20 +501,20 @@ int adh_tiles_pack_nchw(int dtype, uint32_t K, uint32_t p, uint32_t W, uint32_t 
   const uint64_t DW = (uint64_t)W + 2 * p, DH = (uint64_t)Ht + 2 * p;
   if (!plane_limits_ok(DW * DH, DW * DH * C * N) || !plane_limits_ok((uint64_t)W * H, (uint64_t)W * H * C * N))
     return ADH_EINVAL;
-  GatherParams P = {};
+  RowCopyParams P = {};
   for (uint32_t r = 0; r < K; ++r) {
     if (!tile_bufs[r]) return ADH_ENULL;
     if (!aligned_to(tile_bufs[r], es)) return ADH_EALIGN;
     P.dst[r] = tile_bufs[r];
+    P.src[r] = x_unsplit;
   }
-  P.src[0] = x_unsplit;
-  P.n_dst = K;
-  P.DW = (uint32_t)DW; P.DH = (uint32_t)DH; P.plane_elems = (uint32_t)(DW * DH);
+  P.W = W; P.DH = (uint32_t)DH; P.C = C;
+  P.dst_pitch = (uint32_t)DW; P.off_w = p; P.border_l = p; P.border_r = p;
   P.dst_off = 0; P.dst_c_stride = DW * DH; P.dst_n_stride = DW * DH * C;
-  P.off_w = (int32_t)p; P.off_h = (int32_t)p; P.row_step = Ht;
-  P.valid_w = W; P.valid_h = H; P.src_rows_per_tile = 1;
-  P.src_off = 0; P.src_c_stride = (uint64_t)W * H; P.src_n_stride = (uint64_t)W * H * C; P.src_pitch = W;
-  return launch_gather(dtype, P, C, N, false, as_stream(stream));
+  P.off_h = (int32_t)p; P.row_step = Ht; P.valid_h = H;
+  P.src_pitch = W;
+  P.src_off = 0; P.src_c_stride = (uint64_t)W * H; P.src_n_stride = (uint64_t)W * H * C;
+  return launch_row_copy(dtype, false, p > 0, P, K, N, as_stream(stream));
 }
 
 int adh_tiles_unpack_nchw(int dtype, uint32_t K, uint32_t p, uint32_t W, uint32_t H, uint32_t C, uint32_t N,
@@ -523,21 +528,20 @@ int adh_tiles_unpack_nchw(int dtype, uint32_t K, uint32_t p, uint32_t W, uint32_
   const uint64_t SW = (uint64_t)W + 2 * p, SH = (uint64_t)Ht + 2 * p;
   if (!plane_limits_ok(SW * SH, SW * SH * C * N) || !plane_limits_ok((uint64_t)W * H, (uint64_t)W * H * C * N))
     return ADH_EINVAL;
-  GatherParams P = {};
+  RowCopyParams P = {};
   for (uint32_t r = 0; r < K; ++r) {
     if (!tile_bufs[r]) return ADH_ENULL;
     if (!aligned_to(tile_bufs[r], es)) return ADH_EALIGN;
     P.src[r] = tile_bufs[r];
+    P.dst[r] = reinterpret_cast<char *>(y_unsplit) + (size_t)r * Ht * W * es;  // rows [r*Ht, (r+1)*Ht)
   }
-  P.dst[0] = y_unsplit;
-  P.n_dst = 1;
-  P.DW = W; P.DH = H; P.plane_elems = (uint32_t)((uint64_t)W * H);
+  P.W = W; P.DH = Ht; P.C = C;
+  P.dst_pitch = W; P.off_w = 0;
   P.dst_off = 0; P.dst_c_stride = (uint64_t)W * H; P.dst_n_stride = (uint64_t)W * H * C;
-  P.off_w = 0; P.off_h = 0; P.row_step = 0;
-  P.valid_w = W; P.valid_h = H; P.src_rows_per_tile = Ht;
-  P.src_off = (uint64_t)p * SW + p; P.src_c_stride = SW * SH; P.src_n_stride = SW * SH * C;
+  P.off_h = 0; P.row_step = 0; P.valid_h = Ht;
   P.src_pitch = (uint32_t)SW;
-  return launch_gather(dtype, P, C, N, true, as_stream(stream));
+  P.src_off = (uint64_t)p * SW + p; P.src_c_stride = SW * SH; P.src_n_stride = SW * SH * C;
+  return launch_row_copy(dtype, false, false, P, K, N, as_stream(stream));
 }
 
 }  // extern "C"
