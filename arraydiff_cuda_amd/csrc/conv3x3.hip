@@ -20,10 +20,11 @@
 //     four k-groups of an MFMA read disjoint banks) and reused by all 9 taps, all 4 waves and
 //     all 64 output channels: each input element is fetched from HBM once per workgroup.
 //     Every B operand is one ds_read_b32 at lane_base + compile-time immediate.
-//   * weights never touch LDS: each lane keeps the 18 A values of the current chunk in
-//     registers and prefetches the next chunk's 18 from L2 while the current chunk computes.
-//   * global->LDS staging of chunk c+1 is issued before the MFMAs of chunk c and written to
-//     the other LDS buffer after them: one barrier per chunk.
+//   * the 64 x 8 x 9 weights of a chunk are staged in LDS too (read from global in memory
+//     order, coalesced); an A operand is one ds_read_b32 per NT MFMAs.
+//   * staging is asynchronous and register-free: global_load_lds writes each lane's dword
+//     straight into LDS.  The loads of chunk c+1 are issued before the MFMAs of chunk c into
+//     the other buffer pair; one barrier per chunk.
 #include "adh_common.h"
 
 namespace adh {
@@ -34,6 +35,9 @@ static constexpr int kConvThreads = 256;
 static constexpr int kChunk = 8;        // reduction channels per LDS stage
 static constexpr int kLdsPitch = 64;    // floats per staged patch row
 static constexpr int kMaxTW = kLdsPitch - 2;
+static constexpr int kWBufFloats = 64 * kChunk * 9;  // weights of one chunk in LDS
+// word 3 of a gfx9-family buffer resource: 32-bit data format, raw (unstructured) addressing
+static constexpr int kBufferFlags = 0x00020000;
 
 struct ConvParams {
   const float *in[ADH_MAX_TILES];
@@ -56,13 +60,19 @@ struct ConvLds {
   static constexpr int kRows = 4 * RROWS;                      // staged patch rows (>= R + 2)
   static constexpr int kChanStride = kRows * kLdsPitch + 16;   // == 16 (mod 64)
   static constexpr int kBufFloats = kChunk * kChanStride;
-  static constexpr int kBytes = 2 * kBufFloats * 4;
 };
 
-template <int NT, int RROWS>
+// FLIP = false: forward (weights walked as w[o][k][tap]); FLIP = true: backward-data
+// (weights walked as w[k][o][8-tap]).
+template <int NT, int RROWS, bool FLIP>
 __global__ __launch_bounds__(kConvThreads, 1) void conv3x3_f32_kernel(const ConvParams P) {
   typedef ConvLds<RROWS> L;
-  __shared__ float lds[2 * L::kBufFloats];
+  // two patch buffers and two weight buffers as separate arrays: the compiler can then tell
+  // that the LDS reads of one buffer never alias the asynchronous writes into the other
+  __shared__ float patch0[L::kBufFloats];
+  __shared__ float patch1[L::kBufFloats];
+  __shared__ float wbuf0[kWBufFloats];
+  __shared__ float wbuf1[kWBufFloats];
 
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63u, wv = tid >> 6, g = lane >> 4, l16 = lane & 15u;
@@ -81,6 +91,8 @@ __global__ __launch_bounds__(kConvThreads, 1) void conv3x3_f32_kernel(const Conv
   const uint32_t rows_here = min(P.R, P.OH - oh0);
   const uint32_t cols_here = min(P.TW, P.OW - ow0);
   const uint32_t npix = P.R * P.TW;
+  const uint32_t nchunks = (P.Cred + kChunk - 1) / kChunk;
+  const bool ragged_k = (P.Cred % kChunk) != 0;
 
   // LDS float offset of this lane's pixel in each pixel tile (+ the lane's k-group plane)
   uint32_t pix[NT];
@@ -93,15 +105,11 @@ __global__ __launch_bounds__(kConvThreads, 1) void conv3x3_f32_kernel(const Conv
     pix[j] = g * L::kChanStride + r_ * kLdsPitch + c_;
   }
 
-  // ---- staging of the input patch: lane = patch column, wave = patch row (mod 4) ----
+  // ---- patch staging: lane = patch column, wave = patch row (mod 4); global -> LDS without
+  // passing through registers (buffer_load ... lds: each lane's dword lands at base + 4*lane) ----
   const int32_t iw = (int32_t)(ow0 + lane) - P.pad;
   const bool col_ok = lane < P.TW + 2u && iw >= 0 && iw < (int32_t)P.IW;
   const uint32_t patch_rows = P.R + 2u;
-  float stage[kChunk * RROWS];
-
-  // Staging loads are unconditional (addresses clamped into the tensor); out-of-range
-  // elements are replaced by zero only when the registers are written to LDS, after the
-  // MFMAs of the current chunk, so no load is waited for before the matrix work starts.
   uint32_t row_off[RROWS];
   bool row_ok[RROWS];
 #pragma unroll
@@ -111,90 +119,148 @@ __global__ __launch_bounds__(kConvThreads, 1) void conv3x3_f32_kernel(const Conv
     row_ok[rr] = col_ok && prow < patch_rows && ih >= 0 && ih < (int32_t)P.IH;
     row_off[rr] = row_ok[rr] ? (uint32_t)ih * P.IW + (uint32_t)iw : 0u;
   }
-  auto load_patch = [&](uint32_t k0) {
+  // Elements outside the input plane must read as zero and are never written by the masked
+  // loads: clear both patch buffers once.
+  for (uint32_t i = tid; i < (uint32_t)L::kBufFloats; i += kConvThreads) {
+    patch0[i] = 0.f;
+    patch1[i] = 0.f;
+  }
+  __syncthreads();
+
+  // Buffer addressing: a 128-bit resource (SGPRs) for this image, one 32-bit VGPR offset per
+  // lane that never changes, and the channel offset in an SGPR - no per-load address math.
+  const __amdgpu_buffer_rsrc_t rsrc_in = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(in), 0, (int)min((uint64_t)P.Cred * in_plane * 4u, (uint64_t)0xffffffffu), kBufferFlags);
+  auto stage_patch = [&](float *buf, uint32_t k0) {
 #pragma unroll
     for (int kl = 0; kl < kChunk; ++kl) {
-      const float *src = in + (uint64_t)min(k0 + kl, P.Cred - 1u) * in_plane;
-#pragma unroll
-      for (int rr = 0; rr < RROWS; ++rr) stage[kl * RROWS + rr] = src[row_off[rr]];
-    }
-  };
-  auto store_patch = [&](float *buf, uint32_t k0) {
-#pragma unroll
-    for (int kl = 0; kl < kChunk; ++kl) {
-      const bool k_ok = k0 + kl < P.Cred;
+      const bool k_ok = k0 + kl < P.Cred;  // uniform
+      const uint32_t soff = min(k0 + kl, P.Cred - 1u) * (uint32_t)in_plane * 4u;
 #pragma unroll
       for (int rr = 0; rr < RROWS; ++rr) {
-        const uint32_t prow = wv + 4u * rr;
-        buf[kl * L::kChanStride + prow * kLdsPitch + lane] = (k_ok && row_ok[rr]) ? stage[kl * RROWS + rr] : 0.f;
-      }
-    }
-  };
-
-  // ---- weights: A[o = o_blk + 16*wv + l16][k = k0 + 4*kk + g][tap], 18 values per chunk ----
-  const uint32_t o_a = o_blk + 16u * wv + l16;
-  const bool o_ok = o_a < P.Cout;
-  const float *__restrict__ w_o = P.w + (uint64_t)min(o_a, P.Cout - 1u) * P.w_out_stride;
-  auto load_weights = [&](uint32_t k0, float (&a)[18]) {
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      const float *wk = w_o + (uint64_t)min(k0 + 4u * kk + g, P.Cred - 1u) * P.w_red_stride;
-#pragma unroll
-      for (int tap = 0; tap < 9; ++tap) a[kk * 9 + tap] = wk[P.w_flip ? 8 - tap : tap];
-    }
-  };
-  auto mask_weights = [&](uint32_t k0, const float (&src)[18], float (&dst)[18]) {
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      const bool ok = o_ok && k0 + 4u * kk + g < P.Cred;
-#pragma unroll
-      for (int tap = 0; tap < 9; ++tap) dst[kk * 9 + tap] = ok ? src[kk * 9 + tap] : 0.f;
-    }
-  };
-
-  floatx4 acc[NT];
-#pragma unroll
-  for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  float a_cur[18], a_nxt[18];
-  const uint32_t nchunks = (P.Cred + kChunk - 1) / kChunk;
-
-  auto compute = [&](const float *cur) {
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-      for (int kh = 0; kh < 3; ++kh) {
-#pragma unroll
-        for (int kw = 0; kw < 3; ++kw) {
-          const float a = a_cur[kk * 9 + kh * 3 + kw];
-          const int off = kk * 4 * L::kChanStride + kh * kLdsPitch + kw;
-#pragma unroll
-          for (int j = 0; j < NT; ++j) {
-            const float b = cur[pix[j] + off];
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[j], 0, 0, 0);
-          }
+        float *dst = buf + kl * L::kChanStride + (wv + 4u * rr) * kLdsPitch;  // wave-uniform
+        if (k_ok) {
+          if (row_ok[rr]) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, dst, 4, row_off[rr] * 4u, soff, 0, 0);
+        } else {
+          dst[lane] = 0.f;  // ragged last chunk: channels past Cred contribute zero
         }
       }
     }
   };
 
-  load_patch(0);
-  load_weights(0, a_nxt);
-  store_patch(lds, 0);
-  mask_weights(0, a_nxt, a_cur);
-  __syncthreads();
+  // ---- weight staging: the 4608 floats of a chunk in memory order, 18 per thread, also
+  // global -> LDS directly.  forward: wl[o][72] (72 contiguous floats per output channel);
+  // backward-data: wl[k][576] (576 contiguous floats per reduction channel). ----
+  uint32_t w_goff[18];
+  uint32_t w_omask = 0;  // bit i: the output channel of element i exists
+#pragma unroll
+  for (int i = 0; i < 18; ++i) {
+    const uint32_t f = tid + 256u * i;
+    uint32_t o_l, goff;
+    if (FLIP) {
+      const uint32_t k_l = f / 576u;
+      const uint32_t rem = f - k_l * 576u;
+      o_l = rem / 9u;
+      goff = k_l * P.w_red_stride + rem;
+    } else {
+      o_l = f / 72u;
+      goff = o_l * P.w_out_stride + (f - o_l * 72u);
+    }
+    const bool ok = o_blk + o_l < P.Cout;
+    w_goff[i] = ok ? goff : 0u;
+    w_omask |= ok ? (1u << i) : 0u;
+  }
+  const uint32_t w_blk = FLIP ? o_blk * 9u : o_blk * P.w_out_stride;
+  const uint32_t w_chunk_stride = FLIP ? kChunk * P.w_red_stride : kChunk * 9u;
+  const bool ragged_w = ragged_k || (P.Cout % 64u) != 0;
 
-  for (uint32_t c = 0; c + 1 < nchunks; ++c) {
-    const float *cur = lds + (c & 1u) * L::kBufFloats;
-    float *nxt = lds + ((c + 1u) & 1u) * L::kBufFloats;
-    load_patch((c + 1) * kChunk);
-    load_weights((c + 1) * kChunk, a_nxt);
-    compute(cur);
-    store_patch(nxt, (c + 1) * kChunk);
-    mask_weights((c + 1) * kChunk, a_nxt, a_cur);
+  const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(P.w), 0, (int)min((uint64_t)P.Cout * P.Cred * 36u, (uint64_t)0xffffffffu), kBufferFlags);
+  auto stage_weights = [&](float *wl, uint32_t c) {
+    const uint32_t soff = (w_blk + c * w_chunk_stride) * 4u;
+    if (!ragged_w) {
+#pragma unroll
+      for (int i = 0; i < 18; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, wl + 256 * i + 64u * wv, 4, w_goff[i] * 4u, soff, 0, 0);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 18; ++i) {
+        const uint32_t f = tid + 256u * i;
+        const uint32_t k_l = FLIP ? f / 576u : (f % 72u) / 9u;
+        const bool ok = ((w_omask >> i) & 1u) && c * kChunk + k_l < P.Cred;
+        if (ok) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, wl + 256 * i + 64u * wv, 4, w_goff[i] * 4u, soff, 0, 0);
+        else wl[f] = 0.f;
+      }
+    }
+  };
+  // A[o = 16*wv + l16][k = 4*kk + g][tap]
+  const uint32_t a_lane = FLIP ? (16u * wv + l16) * 9u + g * 576u : (16u * wv + l16) * 72u + g * 9u;
+
+  floatx4 acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // One chunk = 18 k-steps (2 groups of 4 channels x 9 taps), NT MFMAs each.  The operands of
+  // k-step s+1 are read from LDS while the MFMAs of k-step s issue, one ds_read per MFMA, into
+  // the other half of a two-deep register buffer; the scheduling-group barriers pin that
+  // interleaving (left alone, the scheduler hoists hundreds of reads and spills).
+  auto a_off = [](int s_) {
+    const int kk = s_ / 9, tap = s_ % 9;
+    return FLIP ? kk * 4 * 576 + (8 - tap) : kk * 36 + tap;
+  };
+  auto b_off = [](int s_) {
+    const int kk = s_ / 9, tap = s_ % 9;
+    return kk * 4 * L::kChanStride + (tap / 3) * kLdsPitch + (tap % 3);
+  };
+  auto compute = [&](const float *cur, const float *wcur) {
+    float a[2], b[2][NT];
+    a[0] = wcur[a_lane + a_off(0)];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) b[0][j] = cur[pix[j] + b_off(0)];
+#pragma unroll
+    for (int s_ = 0; s_ < 18; ++s_) {
+      const int cb = s_ & 1, nb = cb ^ 1;
+      if (s_ + 1 < 18) a[nb] = wcur[a_lane + a_off(s_ + 1)];
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        if (s_ + 1 < 18) b[nb][j] = cur[pix[j] + b_off(s_ + 1)];
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[cb], b[cb][j], acc[j], 0, 0, 0);
+      }
+      if (s_ + 1 < 18) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // the A read
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  stage_patch(patch0, 0);
+  stage_weights(wbuf0, 0);
+  __syncthreads();  // the compiler waits for the outstanding LDS-bound loads before the barrier
+
+  for (uint32_t c = 0; c < nchunks; ++c) {
+    const bool more = c + 1 < nchunks;
+    if ((c & 1u) == 0) {
+      if (more) {
+        stage_patch(patch1, (c + 1) * kChunk);
+        stage_weights(wbuf1, c + 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep the async loads ahead of the matrix work
+      compute(patch0, wbuf0);
+    } else {
+      if (more) {
+        stage_patch(patch0, (c + 1) * kChunk);
+        stage_weights(wbuf0, c + 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      compute(patch1, wbuf1);
+    }
     __syncthreads();
   }
-  compute(lds + ((nchunks - 1u) & 1u) * L::kBufFloats);
 
   // ---- epilogue: lane holds D[o = 4*g + i][pixel = l16] of each tile ----
   const uint32_t o_d = o_blk + 16u * wv + 4u * g;
@@ -261,7 +327,10 @@ static ConvTile choose_tile(uint32_t OH, uint32_t OW, uint64_t planes, uint32_t 
 
 template <int NT>
 static void launch_conv(const ConvParams &P, dim3 grid, hipStream_t st) {
-  hipLaunchKernelGGL((conv3x3_f32_kernel<NT, kRRows>), grid, dim3(kConvThreads), 0, st, P);
+  if (P.w_flip)
+    hipLaunchKernelGGL((conv3x3_f32_kernel<NT, kRRows, true>), grid, dim3(kConvThreads), 0, st, P);
+  else
+    hipLaunchKernelGGL((conv3x3_f32_kernel<NT, kRRows, false>), grid, dim3(kConvThreads), 0, st, P);
 }
 
 // which: ADH_CONV_FWD or ADH_CONV_BWD_DATA.  H, W are the interior extents.
