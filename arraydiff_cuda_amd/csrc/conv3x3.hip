@@ -31,13 +31,14 @@ namespace adh {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-static constexpr int kConvThreads = 256;
 static constexpr int kChunk = 8;        // reduction channels per LDS stage
 static constexpr int kLdsPitch = 64;    // floats per staged patch row
 static constexpr int kMaxTW = kLdsPitch - 2;
 static constexpr int kWBufFloats = 64 * kChunk * 9;  // weights of one chunk in LDS
 // word 3 of a gfx9-family buffer resource: 32-bit data format, raw (unstructured) addressing
 static constexpr int kBufferFlags = 0x00020000;
+// a byte offset no resource of at most 2 GiB contains: such a lane loads zero
+static constexpr uint32_t kOutOfRange = 0x80000000u;
 
 struct ConvParams {
   const float *in[ADH_MAX_TILES];
@@ -55,27 +56,45 @@ struct ConvParams {
   FastDiv div_tiles_x, div_TW;
 };
 
-template <int RROWS>
-struct ConvLds {
-  static constexpr int kRows = 4 * RROWS;                      // staged patch rows (>= R + 2)
-  static constexpr int kChanStride = kRows * kLdsPitch + 16;   // == 16 (mod 64)
-  static constexpr int kBufFloats = kChunk * kChanStride;
+static constexpr int kPatchRows = 12;                                  // staged patch rows (>= R + 2)
+static constexpr int kChanStride = kPatchRows * kLdsPitch + 16;        // == 16 (mod 64)
+static constexpr int kPatchFloats = kChunk * kChanStride;
+static constexpr int kMaxR = kPatchRows - 2;
+
+template <int V>
+struct IntTag {
+  static constexpr int value = V;
 };
 
-// FLIP = false: forward (weights walked as w[o][k][tap]); FLIP = true: backward-data
-// (weights walked as w[k][o][8-tap]).
-template <int NT, int RROWS, bool FLIP>
-__global__ __launch_bounds__(kConvThreads, 1) void conv3x3_f32_kernel(const ConvParams P) {
-  typedef ConvLds<RROWS> L;
+// NT    = pixel tiles of 16 per workgroup (R*TW <= 16*NT)
+// WAVES = 4: wave v owns output channels [16v,16v+16) and all NT tiles;
+//         8: two waves per SIMD, waves v and v+4 share the channels and split the tiles
+//            (ceil(NT/2) and the rest), which hides LDS latency and barrier skew behind the
+//            other wave's MFMAs while every SIMD still carries exactly NT tile-MFMAs per k-step
+// FLIP  = false: forward (weights walked as w[o][k][tap]); true: backward-data
+//         (weights walked as w[k][o][8-tap]).
+template <int NT, int WAVES, bool FLIP>
+__global__ __launch_bounds__(64 * WAVES, 1) void conv3x3_f32_kernel(const ConvParams P) {
+  constexpr int kThreads = 64 * WAVES;
+  constexpr int G = WAVES / 4;                 // pixel groups
+  constexpr int NTA = (NT + G - 1) / G;        // tiles of every group but the last
+  constexpr int NTL = NT - (G - 1) * NTA;      // tiles of the last group
+  constexpr int RROWS = (kPatchRows + WAVES - 1) / WAVES;
+  constexpr int WLOADS = kWBufFloats / kThreads;
+  static_assert(kWBufFloats % kThreads == 0 && NTL > 0, "bad configuration");
   // two patch buffers and two weight buffers as separate arrays: the compiler can then tell
   // that the LDS reads of one buffer never alias the asynchronous writes into the other
-  __shared__ float patch0[L::kBufFloats];
-  __shared__ float patch1[L::kBufFloats];
+  __shared__ float patch0[kPatchFloats];
+  __shared__ float patch1[kPatchFloats];
   __shared__ float wbuf0[kWBufFloats];
   __shared__ float wbuf1[kWBufFloats];
 
   const uint32_t tid = threadIdx.x;
-  const uint32_t lane = tid & 63u, wv = tid >> 6, g = lane >> 4, l16 = lane & 15u;
+  const uint32_t lane = tid & 63u, g = lane >> 4, l16 = lane & 15u;
+  // the wave index is uniform; saying so keeps LDS destinations of the async loads in SGPRs
+  const uint32_t wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t ot = wv & 3u;   // output-channel tile of this wave
+  const uint32_t pg = wv >> 2;   // pixel group of this wave
 
   const uint32_t ty = P.div_tiles_x.div(blockIdx.x);
   const uint32_t tx = blockIdx.x - ty * P.tiles_x;
@@ -94,68 +113,53 @@ __global__ __launch_bounds__(kConvThreads, 1) void conv3x3_f32_kernel(const Conv
   const uint32_t nchunks = (P.Cred + kChunk - 1) / kChunk;
   const bool ragged_k = (P.Cred % kChunk) != 0;
 
-  // LDS float offset of this lane's pixel in each pixel tile (+ the lane's k-group plane)
-  uint32_t pix[NT];
-#pragma unroll
-  for (int j = 0; j < NT; ++j) {
-    uint32_t q = 16u * j + l16;
-    if (q >= npix) q = 0;
-    uint32_t r_, c_;
-    P.div_TW.divmod(q, r_, c_);
-    pix[j] = g * L::kChanStride + r_ * kLdsPitch + c_;
-  }
-
-  // ---- patch staging: lane = patch column, wave = patch row (mod 4); global -> LDS without
-  // passing through registers (buffer_load ... lds: each lane's dword lands at base + 4*lane) ----
+  // ---- patch staging: lane = patch column, wave = patch row (mod WAVES); global -> LDS
+  // without passing through registers (buffer_load ... lds: each lane's dword lands at
+  // base + 4*lane).  Buffer addressing: a 128-bit resource (SGPRs) for this image, one 32-bit
+  // VGPR offset per lane that never changes, and the channel offset in an SGPR - no per-load
+  // address math and no branches: a lane whose element lies outside the input plane carries
+  // an offset beyond the resource's size, for which the hardware writes ZERO into LDS. ----
   const int32_t iw = (int32_t)(ow0 + lane) - P.pad;
   const bool col_ok = lane < P.TW + 2u && iw >= 0 && iw < (int32_t)P.IW;
   const uint32_t patch_rows = P.R + 2u;
-  uint32_t row_off[RROWS];
-  bool row_ok[RROWS];
+  uint32_t row_voff[RROWS];
 #pragma unroll
   for (int rr = 0; rr < RROWS; ++rr) {
-    const uint32_t prow = wv + 4u * rr;
+    const uint32_t prow = wv + (uint32_t)WAVES * rr;
     const int32_t ih = (int32_t)(oh0 + prow) - P.pad;
-    row_ok[rr] = col_ok && prow < patch_rows && ih >= 0 && ih < (int32_t)P.IH;
-    row_off[rr] = row_ok[rr] ? (uint32_t)ih * P.IW + (uint32_t)iw : 0u;
+    const bool ok = col_ok && prow < patch_rows && ih >= 0 && ih < (int32_t)P.IH;
+    row_voff[rr] = ok ? ((uint32_t)ih * P.IW + (uint32_t)iw) * 4u : kOutOfRange;
   }
-  // Elements outside the input plane must read as zero and are never written by the masked
-  // loads: clear both patch buffers once.
-  for (uint32_t i = tid; i < (uint32_t)L::kBufFloats; i += kConvThreads) {
-    patch0[i] = 0.f;
-    patch1[i] = 0.f;
-  }
-  __syncthreads();
-
-  // Buffer addressing: a 128-bit resource (SGPRs) for this image, one 32-bit VGPR offset per
-  // lane that never changes, and the channel offset in an SGPR - no per-load address math.
-  const __amdgpu_buffer_rsrc_t rsrc_in = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float *>(in), 0, (int)min((uint64_t)P.Cred * in_plane * 4u, (uint64_t)0xffffffffu), kBufferFlags);
+  const __amdgpu_buffer_rsrc_t rsrc_in =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), 0, (int)(P.Cred * (uint32_t)in_plane * 4u), kBufferFlags);
   auto stage_patch = [&](float *buf, uint32_t k0) {
+    const bool ragged = ragged_k && k0 + kChunk > P.Cred;  // uniform: a ragged last chunk
 #pragma unroll
-    for (int kl = 0; kl < kChunk; ++kl) {
-      const bool k_ok = k0 + kl < P.Cred;  // uniform
-      const uint32_t soff = min(k0 + kl, P.Cred - 1u) * (uint32_t)in_plane * 4u;
+    for (int rr = 0; rr < RROWS; ++rr) {
+      const uint32_t prow = wv + (uint32_t)WAVES * rr;
+      if (kPatchRows % WAVES != 0 && prow >= (uint32_t)kPatchRows) continue;  // wave-uniform
 #pragma unroll
-      for (int rr = 0; rr < RROWS; ++rr) {
-        float *dst = buf + kl * L::kChanStride + (wv + 4u * rr) * kLdsPitch;  // wave-uniform
-        if (k_ok) {
-          if (row_ok[rr]) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, dst, 4, row_off[rr] * 4u, soff, 0, 0);
-        } else {
-          dst[lane] = 0.f;  // ragged last chunk: channels past Cred contribute zero
+      for (int kl = 0; kl < kChunk; ++kl) {
+        float *dst = buf + kl * kChanStride + prow * kLdsPitch;
+        if (!ragged) {
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, dst, 4, row_voff[rr], (k0 + kl) * (uint32_t)in_plane * 4u, 0, 0);
+        } else {  // channels past Cred are loaded as zero
+          const bool k_ok = k0 + kl < P.Cred;
+          const uint32_t soff = __builtin_amdgcn_readfirstlane(min(k0 + kl, P.Cred - 1u) * (uint32_t)in_plane * 4u);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, dst, 4, k_ok ? row_voff[rr] : kOutOfRange, soff, 0, 0);
         }
       }
     }
   };
 
-  // ---- weight staging: the 4608 floats of a chunk in memory order, 18 per thread, also
-  // global -> LDS directly.  forward: wl[o][72] (72 contiguous floats per output channel);
+  // ---- weight staging: the 4608 floats of a chunk in memory order, also global -> LDS
+  // directly.  forward: wl[o][72] (72 contiguous floats per output channel);
   // backward-data: wl[k][576] (576 contiguous floats per reduction channel). ----
-  uint32_t w_goff[18];
-  uint32_t w_omask = 0;  // bit i: the output channel of element i exists
+  uint32_t w_voff[WLOADS];  // byte offset inside the chunk's weight block, out of range if the
+                            // element's output channel does not exist
 #pragma unroll
-  for (int i = 0; i < 18; ++i) {
-    const uint32_t f = tid + 256u * i;
+  for (int i = 0; i < WLOADS; ++i) {
+    const uint32_t f = tid + (uint32_t)kThreads * i;
     uint32_t o_l, goff;
     if (FLIP) {
       const uint32_t k_l = f / 576u;
@@ -166,75 +170,125 @@ __global__ __launch_bounds__(kConvThreads, 1) void conv3x3_f32_kernel(const Conv
       o_l = f / 72u;
       goff = o_l * P.w_out_stride + (f - o_l * 72u);
     }
-    const bool ok = o_blk + o_l < P.Cout;
-    w_goff[i] = ok ? goff : 0u;
-    w_omask |= ok ? (1u << i) : 0u;
+    w_voff[i] = (o_blk + o_l < P.Cout) ? goff * 4u : kOutOfRange;
   }
   const uint32_t w_blk = FLIP ? o_blk * 9u : o_blk * P.w_out_stride;
   const uint32_t w_chunk_stride = FLIP ? kChunk * P.w_red_stride : kChunk * 9u;
-  const bool ragged_w = ragged_k || (P.Cout % 64u) != 0;
-
-  const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float *>(P.w), 0, (int)min((uint64_t)P.Cout * P.Cred * 36u, (uint64_t)0xffffffffu), kBufferFlags);
+  const __amdgpu_buffer_rsrc_t rsrc_w =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.w), 0, (int)(P.Cout * P.Cred * 36u), kBufferFlags);
   auto stage_weights = [&](float *wl, uint32_t c) {
     const uint32_t soff = (w_blk + c * w_chunk_stride) * 4u;
-    if (!ragged_w) {
+    const bool ragged = ragged_k && (c + 1u) * kChunk > P.Cred;  // uniform
 #pragma unroll
-      for (int i = 0; i < 18; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, wl + 256 * i + 64u * wv, 4, w_goff[i] * 4u, soff, 0, 0);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 18; ++i) {
-        const uint32_t f = tid + 256u * i;
+    for (int i = 0; i < WLOADS; ++i) {
+      uint32_t voff = w_voff[i];
+      if (ragged) {
+        const uint32_t f = tid + (uint32_t)kThreads * i;
         const uint32_t k_l = FLIP ? f / 576u : (f % 72u) / 9u;
-        const bool ok = ((w_omask >> i) & 1u) && c * kChunk + k_l < P.Cred;
-        if (ok) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, wl + 256 * i + 64u * wv, 4, w_goff[i] * 4u, soff, 0, 0);
-        else wl[f] = 0.f;
+        if (c * kChunk + k_l >= P.Cred) voff = kOutOfRange;
       }
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, wl + kThreads * i + 64u * wv, 4, voff, soff, 0, 0);
     }
   };
-  // A[o = 16*wv + l16][k = 4*kk + g][tap]
-  const uint32_t a_lane = FLIP ? (16u * wv + l16) * 9u + g * 576u : (16u * wv + l16) * 72u + g * 9u;
+  // A[o = 16*ot + l16][k = 4*kk + g][tap]
+  const uint32_t a_lane = FLIP ? (16u * ot + l16) * 9u + g * 576u : (16u * ot + l16) * 72u + g * 9u;
 
-  floatx4 acc[NT];
-#pragma unroll
-  for (int j = 0; j < NT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  // One chunk = 18 k-steps (2 groups of 4 channels x 9 taps), NT MFMAs each.  The operands of
-  // k-step s+1 are read from LDS while the MFMAs of k-step s issue, one ds_read per MFMA, into
-  // the other half of a two-deep register buffer; the scheduling-group barriers pin that
-  // interleaving (left alone, the scheduler hoists hundreds of reads and spills).
   auto a_off = [](int s_) {
     const int kk = s_ / 9, tap = s_ % 9;
     return FLIP ? kk * 4 * 576 + (8 - tap) : kk * 36 + tap;
   };
   auto b_off = [](int s_) {
     const int kk = s_ / 9, tap = s_ % 9;
-    return kk * 4 * L::kChanStride + (tap / 3) * kLdsPitch + (tap % 3);
+    return kk * 4 * kChanStride + (tap / 3) * kLdsPitch + (tap % 3);
   };
-  auto compute = [&](const float *cur, const float *wcur) {
-    float a[2], b[2][NT];
-    a[0] = wcur[a_lane + a_off(0)];
+
+  // Everything that depends on the number of pixel tiles this wave owns.
+  auto run = [&](auto cnt_tag, uint32_t tile0) {
+    constexpr int CNT = decltype(cnt_tag)::value;
+
+    // LDS float offset of this lane's pixel in each pixel tile (+ the lane's k-group plane)
+    uint32_t pix[CNT];
 #pragma unroll
-    for (int j = 0; j < NT; ++j) b[0][j] = cur[pix[j] + b_off(0)];
+    for (int j = 0; j < CNT; ++j) {
+      uint32_t q = 16u * (tile0 + j) + l16;
+      if (q >= npix) q = 0;
+      uint32_t r_, c_;
+      P.div_TW.divmod(q, r_, c_);
+      pix[j] = g * kChanStride + r_ * kLdsPitch + c_;
+    }
+
+    floatx4 acc[CNT];
 #pragma unroll
-    for (int s_ = 0; s_ < 18; ++s_) {
-      const int cb = s_ & 1, nb = cb ^ 1;
-      if (s_ + 1 < 18) a[nb] = wcur[a_lane + a_off(s_ + 1)];
+    for (int j = 0; j < CNT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // One chunk = 18 k-steps (2 groups of 4 channels x 9 taps), CNT MFMAs each.  The operands
+    // of k-step s+1 are read from LDS while the MFMAs of k-step s issue, one ds_read per MFMA,
+    // into the other half of a two-deep register buffer; the scheduling-group barriers pin
+    // that interleaving (left alone, the scheduler hoists hundreds of reads and spills).
+    auto compute = [&](const float *cur, const float *wcur) {
+      float a[2], b[2][CNT];
+      a[0] = wcur[a_lane + a_off(0)];
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        if (s_ + 1 < 18) b[nb][j] = cur[pix[j] + b_off(s_ + 1)];
-        acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[cb], b[cb][j], acc[j], 0, 0, 0);
-      }
-      if (s_ + 1 < 18) {
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // the A read
+      for (int j = 0; j < CNT; ++j) b[0][j] = cur[pix[j] + b_off(0)];
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+      for (int s_ = 0; s_ < 18; ++s_) {
+        const int cb = s_ & 1, nb = cb ^ 1;
+        if (s_ + 1 < 18) a[nb] = wcur[a_lane + a_off(s_ + 1)];
+#pragma unroll
+        for (int j = 0; j < CNT; ++j) {
+          if (s_ + 1 < 18) b[nb][j] = cur[pix[j] + b_off(s_ + 1)];
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[cb], b[cb][j], acc[j], 0, 0, 0);
         }
+        if (s_ + 1 < 18) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // the A read
+#pragma unroll
+          for (int j = 0; j < CNT; ++j) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+
+    // two chunks per trip so that each phase names its buffers statically
+    for (uint32_t c = 0;;) {
+      if (c + 1 < nchunks) {
+        stage_patch(patch1, (c + 1) * kChunk);
+        stage_weights(wbuf1, c + 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep the async loads ahead of the matrix work
+      compute(patch0, wbuf0);
+      __syncthreads();
+      if (++c == nchunks) break;
+      if (c + 1 < nchunks) {
+        stage_patch(patch0, (c + 1) * kChunk);
+        stage_weights(wbuf0, c + 1);
       }
       __builtin_amdgcn_sched_barrier(0);
+      compute(patch1, wbuf1);
+      __syncthreads();
+      if (++c == nchunks) break;
+    }
+
+    // ---- epilogue: lane holds D[o = 4*g + i][pixel = l16] of each tile ----
+    const uint32_t o_d = o_blk + 16u * ot + 4u * g;
+#pragma unroll
+    for (int j = 0; j < CNT; ++j) {
+      const uint32_t q = 16u * (tile0 + j) + l16;
+      uint32_t r_, c_;
+      P.div_TW.divmod(q, r_, c_);
+      if (q < npix && r_ < rows_here && c_ < cols_here) {
+        float *dst = out + (uint64_t)o_d * out_plane + (uint64_t)(oh0 + r_) * P.OW + ow0 + c_;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (o_d + i < P.Cout) {
+            float v = acc[j][i];
+            if (P.beta != 0.f) v += P.beta * dst[(uint64_t)i * out_plane];
+            dst[(uint64_t)i * out_plane] = v;
+          }
+        }
+      }
     }
   };
 
@@ -242,44 +296,12 @@ __global__ __launch_bounds__(kConvThreads, 1) void conv3x3_f32_kernel(const Conv
   stage_weights(wbuf0, 0);
   __syncthreads();  // the compiler waits for the outstanding LDS-bound loads before the barrier
 
-  for (uint32_t c = 0; c < nchunks; ++c) {
-    const bool more = c + 1 < nchunks;
-    if ((c & 1u) == 0) {
-      if (more) {
-        stage_patch(patch1, (c + 1) * kChunk);
-        stage_weights(wbuf1, c + 1);
-      }
-      __builtin_amdgcn_sched_barrier(0);  // keep the async loads ahead of the matrix work
-      compute(patch0, wbuf0);
-    } else {
-      if (more) {
-        stage_patch(patch0, (c + 1) * kChunk);
-        stage_weights(wbuf0, c + 1);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      compute(patch1, wbuf1);
-    }
-    __syncthreads();
-  }
-
-  // ---- epilogue: lane holds D[o = 4*g + i][pixel = l16] of each tile ----
-  const uint32_t o_d = o_blk + 16u * wv + 4u * g;
-#pragma unroll
-  for (int j = 0; j < NT; ++j) {
-    const uint32_t q = 16u * j + l16;
-    uint32_t r_, c_;
-    P.div_TW.divmod(q, r_, c_);
-    if (q < npix && r_ < rows_here && c_ < cols_here) {
-      float *dst = out + (uint64_t)o_d * out_plane + (uint64_t)(oh0 + r_) * P.OW + ow0 + c_;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (o_d + i < P.Cout) {
-          float v = acc[j][i];
-          if (P.beta != 0.f) v += P.beta * dst[(uint64_t)i * out_plane];
-          dst[(uint64_t)i * out_plane] = v;
-        }
-      }
-    }
+  if (G == 1 || NTL == NTA) {
+    run(IntTag<NTA>(), pg * NTA);
+  } else if (pg < (uint32_t)(G - 1)) {   // wave-uniform
+    run(IntTag<NTA>(), pg * NTA);
+  } else {
+    run(IntTag<NTL>(), pg * NTA);
   }
 }
 
@@ -293,7 +315,6 @@ struct ConvTile {
 };
 
 static const int kNtVariants[] = {8, 16, 25, 29};
-static constexpr int kRRows = 3;  // staged patch rows = 12 -> R <= 10
 
 // Picks (NT, R, TW) minimising the modelled time ceil(blocks / 256) * NT: a workgroup's
 // time is proportional to NT and 256 CUs run one workgroup each per round.
@@ -307,7 +328,7 @@ static ConvTile choose_tile(uint32_t OH, uint32_t OW, uint64_t planes, uint32_t 
       const uint32_t TW = (OW + ncol - 1) / ncol;
       if (TW == 0 || TW > (uint32_t)kMaxTW || TW > cap) continue;
       uint32_t Rmax = cap / TW;
-      if (Rmax > 4u * kRRows - 2u) Rmax = 4u * kRRows - 2u;
+      if (Rmax > (uint32_t)kMaxR) Rmax = (uint32_t)kMaxR;
       if (Rmax > OH) Rmax = OH;
       for (uint32_t R = 1; R <= Rmax; ++R) {
         const uint64_t tiles_y = (OH + R - 1) / R;
@@ -325,12 +346,12 @@ static ConvTile choose_tile(uint32_t OH, uint32_t OW, uint64_t planes, uint32_t 
   return best;
 }
 
-template <int NT>
+template <int NT, int WAVES>
 static void launch_conv(const ConvParams &P, dim3 grid, hipStream_t st) {
   if (P.w_flip)
-    hipLaunchKernelGGL((conv3x3_f32_kernel<NT, kRRows, true>), grid, dim3(kConvThreads), 0, st, P);
+    hipLaunchKernelGGL((conv3x3_f32_kernel<NT, WAVES, true>), grid, dim3(64 * WAVES), 0, st, P);
   else
-    hipLaunchKernelGGL((conv3x3_f32_kernel<NT, kRRows, false>), grid, dim3(kConvThreads), 0, st, P);
+    hipLaunchKernelGGL((conv3x3_f32_kernel<NT, WAVES, false>), grid, dim3(64 * WAVES), 0, st, P);
 }
 
 // which: ADH_CONV_FWD or ADH_CONV_BWD_DATA.  H, W are the interior extents.
@@ -346,6 +367,9 @@ static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uin
   if (!aligned_to(w, 4)) return ADH_EALIGN;
   const uint64_t HP = (uint64_t)H + 2, WP = (uint64_t)W + 2;
   if (HP * WP >= (1ull << 31) || (uint64_t)N * num_tiles > 65535ull) return ADH_EINVAL;
+  // one image and the filter are each addressed through a 32-bit buffer resource
+  const uint64_t cmax = Cin > Cout ? Cin : Cout;
+  if (cmax * HP * WP * 4u >= (1ull << 31) || (uint64_t)Cin * Cout * 36u >= (1ull << 31)) return ADH_EINVAL;
   ConvParams P = {};
   for (uint32_t t = 0; t < num_tiles; ++t) {
     if (!in_tiles[t] || !out_tiles[t]) return ADH_ENULL;
@@ -378,10 +402,10 @@ static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uin
   P.div_TW = FastDiv(P.TW);
   dim3 grid(P.tiles_x * tiles_y, o_groups, N * num_tiles);
   switch (tile.nt) {
-    case 8: launch_conv<8>(P, grid, st); break;
-    case 16: launch_conv<16>(P, grid, st); break;
-    case 25: launch_conv<25>(P, grid, st); break;
-    case 29: launch_conv<29>(P, grid, st); break;
+    case 8: launch_conv<8, 4>(P, grid, st); break;
+    case 16: launch_conv<16, 8>(P, grid, st); break;
+    case 25: launch_conv<25, 8>(P, grid, st); break;
+    case 29: launch_conv<29, 8>(P, grid, st); break;
     default: return ADH_EINVAL;
   }
   return launch_status();
