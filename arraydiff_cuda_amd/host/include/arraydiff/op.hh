@@ -1,0 +1,846 @@
+// Operator layer of the spatial path: the graph core the ops plug into, and the eight ops of
+// the path with the reference's names, factories and _forward/_backward entry points.
+//
+// Mirrors include/arraydiff/op.hh + src/op.cc of the reference for this path only:
+//   ids and traversal        op.hh:40-169, 593-683   (NodeId/TxnId/EpochId, OperatorStack, Op)
+//   TxnVar / VarData / Var   op.hh:171-591, 685-697  (first-touch-per-transaction buffers)
+//   SpatialScatter2DOp       op.hh:2175-2263, op.cc:2383-2468
+//   SpatialGather2DOp        op.hh:2265-2353, op.cc:2470-2553
+//   HaloPad2DOp              op.hh:2355-2453, op.cc:2555-2712
+//   HaloUnpad2DOp            op.hh:2455-2545, op.cc:2714-2870
+//   HaloRepad2DOp            op.hh:2547-2643, op.cc:2872-2960  (forward only, as in the reference)
+//   HaloExch2DOp             op.hh:2645-2709, op.cc:2962-3052
+//   CudnnConv2DOp            op.hh:1799-1940, op.cc:1343-1727  (here SlabConv2DOp; the old name is an alias)
+//   CudnnSoftmaxNLLLossOp    op.hh:3380-3459, op.cc:4112-4188  (here SoftmaxNLLLossOp; alias kept)
+// The write protocol is the reference's: overwrite() = one exclusive writer per transaction;
+// accumulate(init_fn) = the first toucher in a transaction runs init_fn (zeroing), every node
+// adds once.  Buffers are allocated on first write and shared by clones of a VarData.
+// All arithmetic is behind the C ABI (adh_capi.h); nothing here launches a kernel itself.
+#ifndef ARRAYDIFF_OP_HH
+#define ARRAYDIFF_OP_HH
+
+#include "arraydiff/array_gpu.hh"
+#include "arraydiff/context.hh"
+#include "arraydiff/spatial.hh"
+
+#include <array>
+#include <cassert>
+#include <functional>
+#include <map>
+#include <memory>
+#include <set>
+#include <type_traits>
+#include <vector>
+
+namespace arraydiff {
+
+using std::array;
+using std::function;
+using std::make_shared;
+using std::shared_ptr;
+using std::vector;
+
+// ---------------------------------------------------------------------------
+// ids (thread-local counters, op.cc:77-110)
+// ---------------------------------------------------------------------------
+uint64_t next_raw_id(int kind);
+
+template <int Kind>
+class RawId {
+public:
+  RawId() : id_(next_raw_id(Kind)) {}
+  uint64_t raw_id() const { return id_; }
+  bool operator==(const RawId &o) const { return id_ == o.id_; }
+
+private:
+  uint64_t id_;
+};
+typedef RawId<0> NodeId;
+typedef RawId<1> EpochId;
+typedef RawId<2> TxnId;
+typedef RawId<3> VarId;
+
+// A read/write hazard the reference would assert on (op.hh:249-478).
+class HazardError : public std::logic_error {
+public:
+  explicit HazardError(const std::string &w) : std::logic_error(w) {}
+};
+
+// ---------------------------------------------------------------------------
+// TxnVar: one buffer, (re)initialised per transaction
+// ---------------------------------------------------------------------------
+template <typename V>
+struct IsBatchArray : std::false_type {};
+template <typename Dim, typename T>
+struct IsBatchArray<GPUBatchArray<Dim, T>> : std::true_type {};
+
+template <typename V>
+class TxnVar {
+public:
+  typedef typename V::Shape VShape;
+  typedef typename V::Ctx Ctx;
+
+  TxnVar() {}
+  explicit TxnVar(VShape shape, size_t batch_shape = 0)
+      : shape_(shape), offset_(VShape::Zero()), stride_(shape.packed_stride()), batch_shape_(batch_shape),
+        buf_(make_shared<Buf>()) {}
+  TxnVar(VShape shape, VShape offset, VShape stride, size_t batch_shape)
+      : shape_(shape), offset_(offset), stride_(stride), batch_shape_(batch_shape), buf_(make_shared<Buf>()) {}
+
+  TxnVar clone() const { return *this; }  // shares the buffer
+  VarId var() const { return buf_->var; }
+  VShape shape() const { return shape_; }
+  VShape offset() const { return offset_; }
+  VShape stride() const { return stride_; }
+  size_t batch_shape() const { return batch_shape_; }
+
+  // Exclusive write.  true: the caller is (or becomes) the only writer of this transaction
+  // and must produce the value; false: another node already produced it.
+  bool overwrite(TxnId txn, NodeId node, Ctx *ctx) {
+    begin(txn, ctx);
+    Buf &b = *buf_;
+    if (b.readers.count(node.raw_id())) throw HazardError("overwrite after read by the same node");
+    if (!b.writers.empty() && !b.writers.count(node.raw_id())) return false;
+    b.writers.insert(node.raw_id());
+    return true;
+  }
+  // Accumulating write.  The first toucher of a transaction runs init_fn on the buffer; the
+  // return value says whether THIS node still has to add its contribution.
+  bool accumulate(TxnId txn, NodeId node, Ctx *ctx, function<void(V *)> init_fn) {
+    const bool fresh = begin(txn, ctx);
+    Buf &b = *buf_;
+    if (fresh) init_fn(b.buffer.get());
+    if (b.writers.count(node.raw_id())) return false;
+    b.writers.insert(node.raw_id());
+    return true;
+  }
+  // Read access: the value must have been written in this transaction.
+  V &get(TxnId txn, NodeId node) {
+    Buf &b = *buf_;
+    if (!b.buffer || !b.has_txn || !(b.txn == txn.raw_id())) throw HazardError("read of a variable not written in this transaction");
+    b.readers.insert(node.raw_id());
+    return *b.buffer;
+  }
+  V &get_mut(TxnId txn, NodeId node) {
+    Buf &b = *buf_;
+    if (!b.buffer || !b.has_txn || !(b.txn == txn.raw_id()) || !b.writers.count(node.raw_id()))
+      throw HazardError("get_mut by a node that is not a writer of this transaction");
+    return *b.buffer;
+  }
+  V &get_excl(TxnId txn, NodeId node) {
+    V &v = get_mut(txn, node);
+    if (buf_->writers.size() != 1) throw HazardError("get_excl with more than one writer");
+    return v;
+  }
+  bool written(TxnId txn) const { return buf_->has_txn && buf_->txn == txn.raw_id() && !buf_->writers.empty(); }
+
+private:
+  struct Buf {
+    VarId var;
+    bool has_txn = false;
+    uint64_t txn = 0;
+    std::set<uint64_t> writers, readers;
+    std::unique_ptr<V> buffer;
+  };
+  bool begin(TxnId txn, Ctx *ctx) {
+    Buf &b = *buf_;
+    if (b.has_txn && b.txn == txn.raw_id()) return false;
+    b.has_txn = true;
+    b.txn = txn.raw_id();
+    b.writers.clear();
+    b.readers.clear();
+    if (!b.buffer) allocate(ctx);
+    return true;
+  }
+  void allocate(Ctx *ctx) {
+    if constexpr (IsBatchArray<V>::value)
+      buf_->buffer.reset(new V(V::ZerosPadded(shape_, offset_, stride_, batch_shape_, ctx)));
+    else
+      buf_->buffer.reset(new V(V::Zeros(shape_, ctx)));
+  }
+  VShape shape_, offset_, stride_;
+  size_t batch_shape_ = 0;
+  shared_ptr<Buf> buf_;
+};
+
+template <typename V>
+class VarData {
+public:
+  typedef typename V::Shape VShape;
+  VarData() {}
+  explicit VarData(VShape shape, size_t batch_shape = 0) : val_(shape, batch_shape), grad_(shape, batch_shape) {}
+  VarData(VShape shape, VShape offset, VShape stride, size_t batch_shape)
+      : val_(shape, offset, stride, batch_shape), grad_(shape, offset, stride, batch_shape) {}
+  VarData clone() const { return *this; }
+  TxnVar<V> &val() { return val_; }
+  TxnVar<V> &grad() { return grad_; }
+  VShape shape() const { return val_.shape(); }
+  VShape offset() const { return val_.offset(); }
+  VShape stride() const { return val_.stride(); }
+  size_t batch_shape() const { return val_.batch_shape(); }
+
+private:
+  TxnVar<V> val_, grad_;
+};
+
+// ---------------------------------------------------------------------------
+// traversal
+// ---------------------------------------------------------------------------
+// Counts visits per epoch so that a node with several consumers runs once on the way in
+// (first push) and once on the way out (when every consumer has popped), op.hh:593-668.
+class OperatorStack {
+public:
+  size_t push(EpochId e) { return sync(e), ++pushes_; }
+  size_t degree(EpochId e) { return sync(e), pushes_; }
+  size_t pop(EpochId e) { return sync(e), ++pops_; }
+
+private:
+  void sync(EpochId e) {
+    if (!has_ || !(epoch_ == e.raw_id())) {
+      has_ = true;
+      epoch_ = e.raw_id();
+      pushes_ = pops_ = 0;
+    }
+  }
+  bool has_ = false;
+  uint64_t epoch_ = 0;
+  size_t pushes_ = 0, pops_ = 0;
+};
+
+class Op {
+public:
+  Op() {}
+  virtual ~Op() {}
+  NodeId id() const { return node_id_; }
+
+  virtual void _push(EpochId epoch, function<void(Op *)> apply) = 0;
+  virtual void _pop(EpochId epoch, function<void(Op *)> apply) = 0;
+  virtual void _forward(TxnId txn) = 0;
+  virtual void _backward(TxnId txn) = 0;
+  virtual void _set_grad_sink(TxnId txn) { (void)txn; }
+
+  // forward pass of everything this node depends on, in dependency order (op.cc:196-221)
+  void eval(TxnId txn) {
+    EpochId e;
+    _push(e, [txn](Op *op) { op->_forward(txn); });
+    _pop(e, [](Op *) {});
+  }
+  // forward, seed this node's gradient, then backward in reverse order (op.cc:223-234)
+  void gradient(TxnId txn) {
+    EpochId e;
+    _push(e, [txn](Op *op) { op->_forward(txn); });
+    _set_grad_sink(txn);
+    _pop(e, [txn](Op *op) { op->_backward(txn); });
+  }
+
+protected:
+  OperatorStack stack_;
+
+private:
+  NodeId node_id_;
+};
+
+template <typename V>
+class Var : public virtual Op {
+public:
+  virtual ~Var() {}
+  virtual typename V::Shape shape() = 0;
+  virtual typename V::Shape offset() = 0;
+  virtual typename V::Shape stride() = 0;
+  virtual size_t batch_shape() = 0;
+  virtual VarData<V> data() = 0;
+  virtual vector<VarId> vars() {
+    VarData<V> d = data();
+    return {d.val().var(), d.grad().var()};
+  }
+};
+
+// boilerplate shared by ops that own one output VarData `y_`
+#define ARRAYDIFF_VAR_ACCESSORS(V)                                   \
+  virtual typename V::Shape shape() { return y_.shape(); }           \
+  virtual typename V::Shape offset() { return y_.offset(); }         \
+  virtual typename V::Shape stride() { return y_.stride(); }         \
+  virtual size_t batch_shape() { return y_.batch_shape(); }          \
+  virtual VarData<V> data() { return y_.clone(); }
+
+inline GPUContext *gpu_ctx_of(const shared_ptr<Context> &ctx) {
+  GPUContext *c = dynamic_cast<GPUContext *>(ctx.get());
+  if (!c) throw std::invalid_argument("operator needs a GPUContext");
+  return c;
+}
+inline MultiGPUContext *mgpu_ctx_of(const shared_ptr<Context> &ctx) {
+  MultiGPUContext *c = dynamic_cast<MultiGPUContext *>(ctx.get());
+  if (!c) throw std::invalid_argument("operator needs a MultiGPUContext");
+  return c;
+}
+
+// ---------------------------------------------------------------------------
+// sources
+// ---------------------------------------------------------------------------
+// A batch-array input fed from host memory (the role of the reference's SrcOp / IOOp,
+// op.hh:699-1087, reduced to what the path's tests and tools need).
+template <typename V>
+class SrcOp : public virtual Op, public virtual Var<V> {
+public:
+  static shared_ptr<SrcOp<V>> Make(typename V::Shape shape, size_t batch_shape, shared_ptr<Context> ctx) {
+    return make_shared<SrcOp<V>>(shape, batch_shape, ctx);
+  }
+  SrcOp(typename V::Shape shape, size_t batch_shape, shared_ptr<Context> ctx) : ctx_(ctx), y_(shape, batch_shape) {}
+
+  // dense host data of shape (shape, batch_shape), copied in synchronously
+  template <typename T>
+  void load(TxnId txn, const T *host) {
+    GPUContext *c = gpu_ctx_of(ctx_);
+    if (y_.val().overwrite(txn, id(), c)) {
+      GPUConn conn = c->conn();
+      y_.val().get_excl(txn, id()).load_sync(host, conn);
+    }
+  }
+  template <typename T>
+  void store_grad(TxnId txn, T *host) {
+    GPUConn conn = gpu_ctx_of(ctx_)->conn();
+    y_.grad().get(txn, id()).store_sync(host, conn);
+  }
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) apply(this);
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) apply(this);
+  }
+  virtual void _forward(TxnId) {}
+  virtual void _backward(TxnId) {}
+  ARRAYDIFF_VAR_ACCESSORS(V)
+
+private:
+  shared_ptr<Context> ctx_;
+  VarData<V> y_;
+};
+
+// A parameter (dense, no batch dimension), e.g. the conv filter GPUArray4D<float>.
+template <typename A>
+class ParamOp : public virtual Op, public virtual Var<A> {
+public:
+  static shared_ptr<ParamOp<A>> Make(typename A::Shape shape, shared_ptr<Context> ctx) {
+    return make_shared<ParamOp<A>>(shape, ctx);
+  }
+  ParamOp(typename A::Shape shape, shared_ptr<Context> ctx) : ctx_(ctx), y_(shape) {}
+  template <typename T>
+  void load(TxnId txn, const T *host) {
+    GPUContext *c = gpu_ctx_of(ctx_);
+    if (y_.val().overwrite(txn, id(), c)) {
+      GPUConn conn = c->conn();
+      y_.val().get_excl(txn, id()).load_sync(host, conn);
+    }
+  }
+  template <typename T>
+  void store_grad(TxnId txn, T *host) {
+    GPUConn conn = gpu_ctx_of(ctx_)->conn();
+    y_.grad().get(txn, id()).store_sync(host, conn);
+  }
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) apply(this);
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) apply(this);
+  }
+  virtual void _forward(TxnId) {}
+  virtual void _backward(TxnId) {}
+  virtual typename A::Shape shape() { return y_.shape(); }
+  virtual typename A::Shape offset() { return y_.offset(); }
+  virtual typename A::Shape stride() { return y_.stride(); }
+  virtual size_t batch_shape() { return 0; }
+  virtual VarData<A> data() { return y_.clone(); }
+
+private:
+  shared_ptr<Context> ctx_;
+  VarData<A> y_;
+};
+
+// A variable that is a view of another op's data (outputs of HaloExch2DOp, op.hh:2653-2659).
+template <typename V>
+class NoOp : public virtual Op, public virtual Var<V> {
+public:
+  NoOp(shared_ptr<Op> op, VarData<V> y) : op_(op), y_(y) {}
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) op_->_push(e, apply);
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) op_->_pop(e, apply);
+  }
+  virtual void _forward(TxnId) {}
+  virtual void _backward(TxnId) {}
+  ARRAYDIFF_VAR_ACCESSORS(V)
+
+private:
+  shared_ptr<Op> op_;
+  VarData<V> y_;
+};
+
+// Test / tool sink: identity on the value, seeds the input's gradient from host memory.
+template <typename V>
+class HostGradSinkOp : public virtual Op, public virtual Var<V> {
+public:
+  static shared_ptr<HostGradSinkOp<V>> Make(shared_ptr<Var<V>> input, shared_ptr<Context> ctx) {
+    return make_shared<HostGradSinkOp<V>>(input, ctx);
+  }
+  HostGradSinkOp(shared_ptr<Var<V>> input, shared_ptr<Context> ctx) : ctx_(ctx), input_(input), y_(input->data()) {}
+  void set_host_grad(const float *g) { host_grad_ = g; }
+  template <typename T>
+  void store_val(TxnId txn, T *host) {
+    GPUConn conn = gpu_ctx_of(ctx_)->conn();
+    y_.val().get(txn, id()).store_sync(host, conn);
+  }
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) {
+      input_->_push(e, apply);
+      apply(this);
+    }
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) {
+      apply(this);
+      input_->_pop(e, apply);
+    }
+  }
+  virtual void _forward(TxnId) {}
+  virtual void _backward(TxnId) {}
+  virtual void _set_grad_sink(TxnId txn) {
+    GPUContext *c = gpu_ctx_of(ctx_);
+    const float *g = host_grad_;
+    y_.grad().accumulate(txn, id(), c, [c, g](V *grad) {
+      GPUConn conn = c->conn();
+      grad->load_sync(g, conn);
+    });
+  }
+  ARRAYDIFF_VAR_ACCESSORS(V)
+
+private:
+  shared_ptr<Context> ctx_;
+  shared_ptr<Var<V>> input_;
+  VarData<V> y_;
+  const float *host_grad_ = nullptr;
+};
+
+// ---------------------------------------------------------------------------
+// single-input ops share their traversal
+// ---------------------------------------------------------------------------
+template <typename V>
+class UnaryVarOp : public virtual Op, public virtual Var<V> {
+public:
+  UnaryVarOp(shared_ptr<Var<V>> input, shared_ptr<Context> ctx) : ctx_(ctx), input_(input), x_(input->data()) {}
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) {
+      input_->_push(e, apply);
+      apply(this);
+    }
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) {
+      apply(this);
+      input_->_pop(e, apply);
+    }
+  }
+  ARRAYDIFF_VAR_ACCESSORS(V)
+
+protected:
+  shared_ptr<Context> ctx_;
+  shared_ptr<Var<V>> input_;
+  VarData<V> x_;
+  VarData<V> y_;
+};
+
+template <typename V>
+static vector<shared_ptr<Var<V>>> make_per_rank(
+    shared_ptr<Context> ctx, function<shared_ptr<Var<V>>(size_t rank, shared_ptr<Context> dev_ctx)> make) {
+  MultiGPUContext *m = mgpu_ctx_of(ctx);
+  vector<shared_ptr<Var<V>>> out;
+  for (size_t r = 0; r < m->num_ranks(); ++r) out.push_back(make(r, m->device_context(r)));
+  return out;
+}
+
+// SpatialScatter2DOp: rows [rank*H/K, (rank+1)*H/K) of the full input -> this rank's tile.
+template <typename V>
+class SpatialScatter2DOp : public UnaryVarOp<V> {
+public:
+  static shared_ptr<Var<V>> Make(size_t rank, size_t num_ranks, shared_ptr<Var<V>> input, shared_ptr<Context> ctx) {
+    return make_shared<SpatialScatter2DOp<V>>(rank, num_ranks, input, ctx);
+  }
+  // inputs.at(rank) is the (replicated) full tensor seen by that rank
+  static vector<shared_ptr<Var<V>>> MakeParallel(vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+    const size_t k = mgpu_ctx_of(ctx)->num_ranks();
+    return make_per_rank<V>(ctx, [&](size_t r, shared_ptr<Context> dc) { return Make(r, k, inputs.at(r), dc); });
+  }
+  SpatialScatter2DOp(size_t rank, size_t num_ranks, shared_ptr<Var<V>> input, shared_ptr<Context> ctx)
+      : UnaryVarOp<V>(input, ctx), rank_(rank), num_ranks_(num_ranks) {
+    this->y_ = VarData<V>(_get_output_shape(input->shape()), input->batch_shape());
+  }
+  typename V::Shape _get_output_shape(typename V::Shape in_shape) {
+    if (in_shape.shape[1] % num_ranks_ != 0) throw std::invalid_argument("SpatialScatter2DOp: H % num_ranks != 0");
+    return typename V::Shape(in_shape.shape[0], in_shape.shape[1] / num_ranks_, in_shape.shape[2]);
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+
+private:
+  size_t rank_, num_ranks_;
+};
+
+// SpatialGather2DOp: this rank's tile -> rows [rank*H/K, ...) of a zeroed full-size tensor.
+// In the reference every rank produces a partially filled full tensor and an AllreduceOp sums
+// them (src/zoo.cc:1841-1842); MakeJoined is the one-memory form: all ranks write their rows
+// into ONE output.
+template <typename V>
+class SpatialGather2DOp : public UnaryVarOp<V> {
+public:
+  static shared_ptr<Var<V>> Make(size_t rank, size_t num_ranks, shared_ptr<Var<V>> input, shared_ptr<Context> ctx) {
+    return make_shared<SpatialGather2DOp<V>>(rank, num_ranks, input, ctx);
+  }
+  static vector<shared_ptr<Var<V>>> MakeParallel(vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+    const size_t k = mgpu_ctx_of(ctx)->num_ranks();
+    return make_per_rank<V>(ctx, [&](size_t r, shared_ptr<Context> dc) { return Make(r, k, inputs.at(r), dc); });
+  }
+  SpatialGather2DOp(size_t rank, size_t num_ranks, shared_ptr<Var<V>> input, shared_ptr<Context> ctx)
+      : UnaryVarOp<V>(input, ctx), rank_(rank), num_ranks_(num_ranks) {
+    auto s = input->shape();
+    this->y_ = VarData<V>(typename V::Shape(s.shape[0], s.shape[1] * num_ranks, s.shape[2]), input->batch_shape());
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+
+private:
+  size_t rank_, num_ranks_;
+};
+
+// The one-memory form of gather: K unpadded tiles -> ONE full tensor in a single launch (an
+// all-gather along H); backward hands each rank its rows of the gradient.
+template <typename V>
+class SpatialJoinedGather2DOp : public virtual Op, public virtual Var<V> {
+public:
+  static shared_ptr<SpatialJoinedGather2DOp<V>> Make(vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+    return make_shared<SpatialJoinedGather2DOp<V>>(inputs, ctx);
+  }
+  SpatialJoinedGather2DOp(vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) : ctx_(ctx), inputs_(inputs) {
+    if (inputs.empty() || inputs.size() > ADH_MAX_TILES) throw std::invalid_argument("SpatialJoinedGather2DOp: 1..16 tiles");
+    for (auto &in : inputs) {
+      if (in->shape() != inputs[0]->shape()) throw std::invalid_argument("SpatialJoinedGather2DOp: tile shapes differ");
+      xs_.push_back(in->data());
+    }
+    auto s = inputs[0]->shape();
+    y_ = VarData<V>(typename V::Shape(s.shape[0], s.shape[1] * inputs.size(), s.shape[2]), inputs[0]->batch_shape());
+  }
+  template <typename T>
+  void store_val(TxnId txn, T *host) {
+    GPUConn conn = mgpu_ctx_of(ctx_)->device_context(0)->conn();
+    y_.val().get(txn, id()).store_sync(host, conn);
+  }
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) {
+      for (auto &in : inputs_) in->_push(e, apply);
+      apply(this);
+    }
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) {
+      apply(this);
+      for (size_t r = inputs_.size(); r-- > 0;) inputs_.at(r)->_pop(e, apply);
+    }
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+  ARRAYDIFF_VAR_ACCESSORS(V)
+
+private:
+  shared_ptr<Context> ctx_;
+  vector<shared_ptr<Var<V>>> inputs_;
+  vector<VarData<V>> xs_;
+  VarData<V> y_;
+};
+
+template <typename V>
+class HaloPad2DOp : public UnaryVarOp<V> {
+public:
+  static shared_ptr<Var<V>> Make(size_t halo_pad, shared_ptr<Var<V>> input, shared_ptr<Context> ctx) {
+    return make_shared<HaloPad2DOp<V>>(halo_pad, input, ctx);
+  }
+  static vector<shared_ptr<Var<V>>> MakeParallel(size_t halo_pad, vector<shared_ptr<Var<V>>> inputs,
+                                                 shared_ptr<Context> ctx) {
+    return make_per_rank<V>(ctx, [&](size_t r, shared_ptr<Context> dc) { return Make(halo_pad, inputs.at(r), dc); });
+  }
+  HaloPad2DOp(size_t halo_pad, shared_ptr<Var<V>> input, shared_ptr<Context> ctx)
+      : UnaryVarOp<V>(input, ctx), halo_pad_(halo_pad) {
+    this->y_ = VarData<V>(input->shape(), _get_output_offset(input->shape()), _get_output_stride(input->shape()),
+                          input->batch_shape());
+  }
+  typename V::Shape _get_output_offset(typename V::Shape) { return typename V::Shape(halo_pad_, halo_pad_, 0); }
+  typename V::Shape _get_output_stride(typename V::Shape s) {
+    return typename V::Shape(s.shape[0] + 2 * halo_pad_, s.shape[1] + 2 * halo_pad_, s.shape[2]).packed_stride();
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+
+private:
+  size_t halo_pad_;
+};
+
+template <typename V>
+class HaloUnpad2DOp : public UnaryVarOp<V> {
+public:
+  static shared_ptr<Var<V>> Make(size_t halo_pad, shared_ptr<Var<V>> input, shared_ptr<Context> ctx) {
+    return make_shared<HaloUnpad2DOp<V>>(halo_pad, input, ctx);
+  }
+  static vector<shared_ptr<Var<V>>> MakeParallel(size_t halo_pad, vector<shared_ptr<Var<V>>> inputs,
+                                                 shared_ptr<Context> ctx) {
+    return make_per_rank<V>(ctx, [&](size_t r, shared_ptr<Context> dc) { return Make(halo_pad, inputs.at(r), dc); });
+  }
+  HaloUnpad2DOp(size_t halo_pad, shared_ptr<Var<V>> input, shared_ptr<Context> ctx)
+      : UnaryVarOp<V>(input, ctx), halo_pad_(halo_pad) {
+    this->y_ = VarData<V>(input->shape(), input->batch_shape());
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+
+private:
+  size_t halo_pad_;
+};
+
+template <typename V>
+class HaloRepad2DOp : public UnaryVarOp<V> {
+public:
+  static shared_ptr<Var<V>> Make(size_t src_halo_pad, size_t dst_halo_pad, shared_ptr<Var<V>> input,
+                                 shared_ptr<Context> ctx) {
+    return make_shared<HaloRepad2DOp<V>>(src_halo_pad, dst_halo_pad, input, ctx);
+  }
+  static vector<shared_ptr<Var<V>>> MakeParallel(size_t src_halo_pad, size_t dst_halo_pad,
+                                                 vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+    return make_per_rank<V>(
+        ctx, [&](size_t r, shared_ptr<Context> dc) { return Make(src_halo_pad, dst_halo_pad, inputs.at(r), dc); });
+  }
+  HaloRepad2DOp(size_t src_halo_pad, size_t dst_halo_pad, shared_ptr<Var<V>> input, shared_ptr<Context> ctx)
+      : UnaryVarOp<V>(input, ctx), src_pad_(src_halo_pad), dst_pad_(dst_halo_pad) {
+    auto s = input->shape();
+    this->y_ = VarData<V>(s, typename V::Shape(dst_pad_, dst_pad_, 0),
+                          typename V::Shape(s.shape[0] + 2 * dst_pad_, s.shape[1] + 2 * dst_pad_, s.shape[2]).packed_stride(),
+                          input->batch_shape());
+  }
+  virtual void _forward(TxnId txn);
+  // the reference defines no backward for this op (SURVEY: op.cc:2872-2960 only)
+  virtual void _backward(TxnId) { throw std::logic_error("HaloRepad2DOp has no backward"); }
+
+private:
+  size_t src_pad_, dst_pad_;
+};
+
+// One node spanning all ranks, in place on the K pad outputs; the outputs are NoOp views of
+// the same VarData.
+template <typename V>
+class HaloExch2DOp : public virtual Op {
+public:
+  static vector<shared_ptr<Var<V>>> MakeParallel(size_t halo_pad, vector<shared_ptr<Var<V>>> inputs,
+                                                 shared_ptr<Context> ctx) {
+    auto op = make_shared<HaloExch2DOp<V>>(halo_pad, inputs, ctx);
+    vector<shared_ptr<Var<V>>> outputs;
+    for (size_t r = 0; r < inputs.size(); ++r) outputs.push_back(make_shared<NoOp<V>>(op, op->xs_.at(r).clone()));
+    return outputs;
+  }
+  HaloExch2DOp(size_t halo_pad, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx)
+      : ctx_(ctx), halo_pad_(halo_pad), inputs_(inputs) {
+    if (inputs.size() != mgpu_ctx_of(ctx)->num_ranks()) throw std::invalid_argument("HaloExch2DOp: one input per rank");
+    for (auto &in : inputs) xs_.push_back(in->data());
+  }
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) {
+      for (auto &in : inputs_) in->_push(e, apply);
+      apply(this);
+    }
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) {
+      apply(this);
+      for (size_t r = inputs_.size(); r-- > 0;) inputs_.at(r)->_pop(e, apply);
+    }
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+
+private:
+  shared_ptr<Context> ctx_;
+  size_t halo_pad_;
+  vector<shared_ptr<Var<V>>> inputs_;
+  vector<VarData<V>> xs_;
+};
+
+// ---------------------------------------------------------------------------
+// convolution over the halo-padded slab
+// ---------------------------------------------------------------------------
+class Conv2DShape {
+public:
+  size_t filters;
+  array<size_t, 2> axes;
+  array<size_t, 2> kernel;
+  array<size_t, 2> dilate;
+  array<size_t, 2> stride;
+  array<size_t, 2> pad;
+  bool halo_padded_input;
+  bool enable_hmma;
+};
+
+// V = GPUBatchArray3D<float>, A = GPUArray4D<float> (filter, Shape4D(kw,kh,Cin,Cout) = KCRS).
+// Supported: 3x3, stride 1, dilation 1, pad 1, halo_padded_input, no bias - the configuration of
+// the spatially-parallel blocks (src/zoo.cc:577-652); anything else throws at construction.
+// One node serves all ranks it was made for: the K slabs go to the device in ONE launch per
+// pass (the reference ran one cuDNN call per rank on K GPUs).  Make() is the one-rank form and
+// is itself the output variable; MakeParallel() returns per-rank views of one node.
+template <typename V, typename A>
+class SlabConv2DOp : public virtual Op, public virtual Var<V> {
+public:
+  static shared_ptr<Var<V>> Make(Conv2DShape shape, shared_ptr<Var<V>> input, shared_ptr<Var<A>> kernel,
+                                 shared_ptr<Context> ctx) {
+    return make_shared<SlabConv2DOp<V, A>>(shape, vector<shared_ptr<Var<V>>>{input},
+                                           vector<shared_ptr<Var<A>>>{kernel}, ctx);
+  }
+  // each rank holds its own copy of the filter in the reference; here kernels.at(r) may all be
+  // the same variable, its gradient then accumulates over the tiles
+  static vector<shared_ptr<Var<V>>> MakeParallel(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs,
+                                                 vector<shared_ptr<Var<A>>> kernels, shared_ptr<Context> ctx) {
+    auto op = make_shared<SlabConv2DOp<V, A>>(shape, inputs, kernels, ctx);
+    vector<shared_ptr<Var<V>>> outputs;
+    for (size_t r = 0; r < inputs.size(); ++r) outputs.push_back(make_shared<NoOp<V>>(op, op->ys_.at(r).clone()));
+    return outputs;
+  }
+  SlabConv2DOp(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs, vector<shared_ptr<Var<A>>> kernels,
+               shared_ptr<Context> ctx)
+      : ctx_(ctx), shape_(shape), x_vars_(inputs), kernel_vars_(kernels) {
+    if (shape.kernel[0] != 3 || shape.kernel[1] != 3 || shape.stride[0] != 1 || shape.stride[1] != 1 ||
+        shape.dilate[0] != 1 || shape.dilate[1] != 1 || shape.pad[0] != 1 || shape.pad[1] != 1 ||
+        !shape.halo_padded_input)
+      throw std::invalid_argument("SlabConv2DOp: only 3x3 / stride 1 / dilation 1 / pad 1 over a halo-padded input");
+    if (inputs.empty() || inputs.size() != kernels.size() || inputs.size() > ADH_MAX_TILES)
+      throw std::invalid_argument("SlabConv2DOp: one kernel variable per input");
+    for (size_t r = 0; r < inputs.size(); ++r) {
+      auto off = inputs[r]->offset();
+      if (off.shape[0] != 1 || off.shape[1] != 1 || off.shape[2] != 0)
+        throw std::invalid_argument("SlabConv2DOp: input halo must equal the conv pad");
+      if (inputs[r]->shape() != inputs[0]->shape() || inputs[r]->batch_shape() != inputs[0]->batch_shape())
+        throw std::invalid_argument("SlabConv2DOp: all slabs must have one shape");
+      xs_.push_back(inputs[r]->data());
+      kernels_.push_back(kernels[r]->data());
+      ys_.push_back(VarData<V>(_get_output_shape(inputs[r]->shape(), inputs[r]->batch_shape()), inputs[r]->batch_shape()));
+    }
+  }
+  // out = floor((H + 2p - ((k-1)d+1)) / s) + 1 = H for 3x3/s1/p1 (op.cc:1512-1523)
+  Shape3D _get_output_shape(Shape3D in_shape, size_t) {
+    return Shape3D(in_shape.shape[0], in_shape.shape[1], shape_.filters);
+  }
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) {
+      for (size_t r = 0; r < x_vars_.size(); ++r) {
+        x_vars_[r]->_push(e, apply);
+        kernel_vars_[r]->_push(e, apply);
+      }
+      apply(this);
+    }
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) {
+      apply(this);
+      for (size_t r = x_vars_.size(); r-- > 0;) {
+        kernel_vars_[r]->_pop(e, apply);
+        x_vars_[r]->_pop(e, apply);
+      }
+    }
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+  virtual typename V::Shape shape() { return ys_[0].shape(); }
+  virtual typename V::Shape offset() { return ys_[0].offset(); }
+  virtual typename V::Shape stride() { return ys_[0].stride(); }
+  virtual size_t batch_shape() { return ys_[0].batch_shape(); }
+  virtual VarData<V> data() { return ys_[0].clone(); }
+
+private:
+  shared_ptr<Context> ctx_;
+  Conv2DShape shape_;
+  vector<shared_ptr<Var<V>>> x_vars_;
+  vector<shared_ptr<Var<A>>> kernel_vars_;
+  vector<VarData<V>> xs_;
+  vector<VarData<A>> kernels_;
+  vector<VarData<V>> ys_;
+};
+template <typename V, typename A, typename B = A>
+using CudnnConv2DOp = SlabConv2DOp<V, A>;
+
+// ---------------------------------------------------------------------------
+// softmax + negative log likelihood (1-D logits)
+// ---------------------------------------------------------------------------
+template <typename V, typename Label, typename Loss>
+class SoftmaxNLLLossOp : public virtual Op, public virtual Var<Loss> {
+public:
+  SoftmaxNLLLossOp(shared_ptr<Var<V>> input, shared_ptr<Var<Label>> label, shared_ptr<Context> ctx)
+      : ctx_(ctx), input_(input), label_var_(label), x_(input->data()), y_(input->shape(), input->batch_shape()),
+        label_(label->data()), loss_(typename Loss::Shape(), input->batch_shape()) {}
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) {
+      input_->_push(e, apply);
+      label_var_->_push(e, apply);
+      apply(this);
+    }
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) {
+      apply(this);
+      label_var_->_pop(e, apply);
+      input_->_pop(e, apply);
+    }
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+  // per-example losses: the sink gradient is 1 for every example (the reference reaches the
+  // same through batch_sum + ScaleOp, src/zoo.cc:1877-1878)
+  virtual void _set_grad_sink(TxnId txn) {
+    GPUContext *c = gpu_ctx_of(ctx_);
+    loss_.grad().accumulate(txn, id(), c, [c](Loss *g) {
+      GPUConn conn = c->conn();
+      g->as_view().set_constant(1.0f, conn);
+    });
+  }
+  template <typename T>
+  void store_loss(TxnId txn, T *host) {
+    GPUConn conn = gpu_ctx_of(ctx_)->conn();
+    loss_.val().get(txn, id()).store_sync(host, conn);
+  }
+  template <typename T>
+  void store_prob(TxnId txn, T *host) {
+    GPUConn conn = gpu_ctx_of(ctx_)->conn();
+    y_.val().get(txn, id()).store_sync(host, conn);
+  }
+  virtual typename Loss::Shape shape() { return loss_.shape(); }
+  virtual typename Loss::Shape offset() { return loss_.offset(); }
+  virtual typename Loss::Shape stride() { return loss_.stride(); }
+  virtual size_t batch_shape() { return loss_.batch_shape(); }
+  virtual VarData<Loss> data() { return loss_.clone(); }
+
+private:
+  shared_ptr<Context> ctx_;
+  shared_ptr<Var<V>> input_;
+  shared_ptr<Var<Label>> label_var_;
+  VarData<V> x_;
+  VarData<V> y_;  // softmax output, kept for backward
+  VarData<Label> label_;
+  VarData<Loss> loss_;
+};
+template <typename V, typename Label, typename Loss>
+using CudnnSoftmaxNLLLossOp = SoftmaxNLLLossOp<V, Label, Loss>;
+
+template <typename V, typename Label, typename Loss>
+shared_ptr<SoftmaxNLLLossOp<V, Label, Loss>> softmax_nll_loss(shared_ptr<Var<V>> input, shared_ptr<Var<Label>> label,
+                                                              shared_ptr<Context> ctx) {
+  return make_shared<SoftmaxNLLLossOp<V, Label, Loss>>(input, label, ctx);
+}
+
+// the float instantiations live in src/op.cc
+typedef GPUBatchArray3D<float> Tile3f;
+typedef GPUArray4D<float> Filter4f;
+
+}  // namespace arraydiff
+
+#endif

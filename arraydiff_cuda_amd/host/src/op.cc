@@ -1,0 +1,491 @@
+// _forward / _backward of the spatial-path ops for float tiles: argument checks as in the
+// reference's src/op.cc (cited per op), arithmetic behind the C ABI.
+#include "arraydiff/op.hh"
+
+#include "adh_capi.h"
+
+namespace arraydiff {
+
+uint64_t next_raw_id(int kind) {
+  static thread_local uint64_t counters[4] = {0, 0, 0, 0};
+  return ++counters[kind & 3];
+}
+
+typedef GPUBatchArray3D<float> V3;
+typedef GPUArray4D<float> A4;
+
+namespace {
+
+struct TileDims {
+  uint32_t W, H, C, N;
+};
+TileDims dims_of(V3 &a) {
+  auto d = a.dim();
+  return TileDims{(uint32_t)d.shape[0], (uint32_t)d.shape[1], (uint32_t)d.shape[2], (uint32_t)a.batch_size()};
+}
+
+// offset == (p,p,0) and stride == packed stride of the padded extents (op.cc:2587-2609)
+void check_padded(V3 &a, size_t p, const char *who) {
+  auto d = a.dim();
+  auto want = Shape3D(d.shape[0] + 2 * p, d.shape[1] + 2 * p, d.shape[2]).packed_stride();
+  if (a.offset() != Shape3D(p, p, 0) || a.stride() != want)
+    throw std::invalid_argument(std::string(who) + ": array is not halo-padded by the expected width");
+}
+void check_packed(V3 &a, const char *who) {
+  if (!a.offset().is_zero() || !a.dim().is_packed(a.stride()))
+    throw std::invalid_argument(std::string(who) + ": array is not packed");
+}
+
+}  // namespace
+
+// ---- SpatialScatter2DOp (op.cc:2396-2468) ----
+template <>
+void SpatialScatter2DOp<V3>::_forward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &x = x_.val().get(txn, id());
+  const TileDims xd = dims_of(x);
+  if (y_.val().overwrite(txn, id(), ctx)) {
+    GPUConn conn = ctx->conn();
+    V3 &y = y_.val().get_excl(txn, id());
+    y.set_batch_size(xd.N);
+    check_packed(x, "SpatialScatter2DOp");
+    const uint32_t Ht = xd.H / (uint32_t)num_ranks_;
+    slice2d_copy_hw_nchw_packed<float>(xd.W, Ht, xd.W, xd.H, xd.W, Ht, xd.C, xd.N, x.as_view().dptr(), 0,
+                                       (uint32_t)rank_ * Ht, y.as_view().dptr(), 0, 0, conn.stream());
+  }
+}
+template <>
+void SpatialScatter2DOp<V3>::_backward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &dy = y_.grad().get(txn, id());
+  const TileDims yd = dims_of(dy);
+  const size_t batch = yd.N;
+  if (x_.grad().accumulate(txn, id(), ctx, [ctx, batch](V3 *g) {
+        GPUConn conn = ctx->conn();
+        g->set_batch_size(batch);
+        g->as_view().set_constant(0.0f, conn);
+      })) {
+    GPUConn conn = ctx->conn();
+    V3 &dx = x_.grad().get_mut(txn, id());
+    const TileDims xd = dims_of(dx);
+    slice2d_add_hw_nchw_packed<float>(xd.W, yd.H, xd.W, yd.H, xd.W, xd.H, xd.C, xd.N, dy.as_view().dptr(), 0, 0,
+                                      dx.as_view().dptr(), 0, (uint32_t)rank_ * yd.H, conn.stream());
+  }
+}
+
+// ---- SpatialGather2DOp (op.cc:2480-2553) ----
+template <>
+void SpatialGather2DOp<V3>::_forward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &x = x_.val().get(txn, id());
+  const TileDims xd = dims_of(x);
+  const size_t batch = xd.N;
+  if (y_.val().accumulate(txn, id(), ctx, [ctx, batch](V3 *v) {
+        GPUConn conn = ctx->conn();
+        v->set_batch_size(batch);
+        v->as_view().set_constant(0.0f, conn);
+      })) {
+    GPUConn conn = ctx->conn();
+    V3 &y = y_.val().get_mut(txn, id());
+    const TileDims yd = dims_of(y);
+    slice2d_copy_hw_nchw_packed<float>(xd.W, xd.H, xd.W, xd.H, yd.W, yd.H, xd.C, xd.N, x.as_view().dptr(), 0, 0,
+                                       y.as_view().dptr(), 0, (uint32_t)rank_ * xd.H, conn.stream());
+  }
+}
+template <>
+void SpatialGather2DOp<V3>::_backward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &dy = y_.grad().get(txn, id());
+  const TileDims yd = dims_of(dy);
+  const size_t batch = yd.N;
+  if (x_.grad().accumulate(txn, id(), ctx, [ctx, batch](V3 *g) {
+        GPUConn conn = ctx->conn();
+        g->set_batch_size(batch);
+        g->as_view().set_constant(0.0f, conn);
+      })) {
+    GPUConn conn = ctx->conn();
+    V3 &dx = x_.grad().get_mut(txn, id());
+    const TileDims xd = dims_of(dx);
+    slice2d_add_hw_nchw_packed<float>(xd.W, xd.H, yd.W, yd.H, xd.W, xd.H, xd.C, xd.N, dy.as_view().dptr(), 0,
+                                      (uint32_t)rank_ * xd.H, dx.as_view().dptr(), 0, 0, conn.stream());
+  }
+}
+
+// ---- SpatialJoinedGather2DOp: gather of src/zoo.cc:1841-1842 without the zero-fill + allreduce ----
+template <>
+void SpatialJoinedGather2DOp<V3>::_forward(TxnId txn) {
+  MultiGPUContext *ctx = mgpu_ctx_of(ctx_);
+  GPUContext *dc = ctx->device_context(0).get();
+  if (y_.val().overwrite(txn, id(), dc)) {
+    const void *tiles[ADH_MAX_TILES];
+    TileDims d{};
+    for (size_t r = 0; r < xs_.size(); ++r) {
+      V3 &x = xs_[r].val().get(txn, id());
+      check_packed(x, "SpatialJoinedGather2DOp");
+      d = dims_of(x);
+      tiles[r] = x.as_view().dptr();
+    }
+    V3 &y = y_.val().get_excl(txn, id());
+    y.set_batch_size(d.N);
+    GPUConn conn = dc->conn();
+    adh_check(adh_tiles_unpack_nchw(ADH_F32, (uint32_t)xs_.size(), 0, d.W, d.H * (uint32_t)xs_.size(), d.C, d.N, tiles,
+                                    y.as_view().dptr(), conn.stream()),
+              "SpatialJoinedGather2DOp::_forward");
+  }
+}
+template <>
+void SpatialJoinedGather2DOp<V3>::_backward(TxnId txn) {
+  MultiGPUContext *ctx = mgpu_ctx_of(ctx_);
+  V3 &dy = y_.grad().get(txn, id());
+  const TileDims yd = dims_of(dy);
+  const size_t batch = yd.N;
+  for (size_t r = 0; r < xs_.size(); ++r) {
+    GPUContext *dc = ctx->device_context(r).get();
+    if (xs_[r].grad().accumulate(txn, id(), dc, [dc, batch](V3 *g) {
+          GPUConn conn = dc->conn();
+          g->set_batch_size(batch);
+          g->as_view().set_constant(0.0f, conn);
+        })) {
+      GPUConn conn = dc->conn();
+      V3 &dx = xs_[r].grad().get_mut(txn, id());
+      const TileDims xd = dims_of(dx);
+      slice2d_add_hw_nchw_packed<float>(xd.W, xd.H, yd.W, yd.H, xd.W, xd.H, xd.C, xd.N, dy.as_view().dptr(), 0,
+                                        (uint32_t)r * xd.H, dx.as_view().dptr(), 0, 0, conn.stream());
+    }
+  }
+}
+
+// ---- HaloPad2DOp (op.cc:2574-2712) ----
+template <>
+void HaloPad2DOp<V3>::_forward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &x = x_.val().get(txn, id());
+  const TileDims xd = dims_of(x);
+  const size_t batch = xd.N;
+  // the pad kernel writes border and interior in one pass, so the first-touch step only has
+  // to size the batch (the reference zero-fills here and then copies, op.cc:2581-2585,2634)
+  if (y_.val().accumulate(txn, id(), ctx, [batch](V3 *v) { v->set_batch_size(batch); })) {
+    GPUConn conn = ctx->conn();
+    V3 &y = y_.val().get_mut(txn, id());
+    check_packed(x, "HaloPad2DOp");
+    check_padded(y, halo_pad_, "HaloPad2DOp");
+    if (y.dim() != x.dim() || y.batch_size() != batch) throw std::invalid_argument("HaloPad2DOp: shape mismatch");
+    adh_check(adh_halo_pad_nchw(ADH_F32, (uint32_t)halo_pad_, xd.W, xd.H, xd.C, xd.N, x.as_view().dptr(),
+                                y.base_as_view().dptr(), conn.stream()),
+              "HaloPad2DOp::_forward");
+  }
+}
+template <>
+void HaloPad2DOp<V3>::_backward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &dy = y_.grad().get(txn, id());
+  const TileDims d = dims_of(dy);
+  const size_t batch = d.N;
+  if (x_.grad().accumulate(txn, id(), ctx, [ctx, batch](V3 *g) {
+        GPUConn conn = ctx->conn();
+        g->set_batch_size(batch);
+        g->as_view().set_constant(0.0f, conn);
+      })) {
+    GPUConn conn = ctx->conn();
+    V3 &dx = x_.grad().get_mut(txn, id());
+    check_padded(dy, halo_pad_, "HaloPad2DOp");
+    adh_check(adh_halo_unpad_add_nchw(ADH_F32, (uint32_t)halo_pad_, d.W, d.H, d.C, d.N, dy.base_as_view().dptr(),
+                                      dx.as_view().dptr(), conn.stream()),
+              "HaloPad2DOp::_backward");
+  }
+}
+
+// ---- HaloUnpad2DOp (op.cc:2715-2870) ----
+template <>
+void HaloUnpad2DOp<V3>::_forward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &x = x_.val().get(txn, id());
+  const TileDims d = dims_of(x);
+  if (y_.val().overwrite(txn, id(), ctx)) {
+    GPUConn conn = ctx->conn();
+    V3 &y = y_.val().get_excl(txn, id());
+    y.set_batch_size(d.N);
+    check_padded(x, halo_pad_, "HaloUnpad2DOp");  // op.cc:2746-2748
+    adh_check(adh_halo_unpad_nchw(ADH_F32, (uint32_t)halo_pad_, d.W, d.H, d.C, d.N, x.base_as_view().dptr(),
+                                  y.as_view().dptr(), conn.stream()),
+              "HaloUnpad2DOp::_forward");
+  }
+}
+template <>
+void HaloUnpad2DOp<V3>::_backward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &dy = y_.grad().get(txn, id());
+  const TileDims d = dims_of(dy);
+  const size_t batch = d.N;
+  if (x_.grad().accumulate(txn, id(), ctx, [ctx, batch](V3 *g) {
+        GPUConn conn = ctx->conn();
+        g->set_batch_size(batch);
+        g->base_as_view().set_constant(0.0f, conn);
+      })) {
+    GPUConn conn = ctx->conn();
+    V3 &dx = x_.grad().get_mut(txn, id());
+    check_padded(dx, halo_pad_, "HaloUnpad2DOp");
+    adh_check(adh_halo_pad_add_nchw(ADH_F32, (uint32_t)halo_pad_, d.W, d.H, d.C, d.N, dy.as_view().dptr(),
+                                    dx.base_as_view().dptr(), conn.stream()),
+              "HaloUnpad2DOp::_backward");
+  }
+}
+
+// ---- HaloRepad2DOp (op.cc:2873-2960) ----
+template <>
+void HaloRepad2DOp<V3>::_forward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &x = x_.val().get(txn, id());
+  const TileDims d = dims_of(x);
+  const size_t batch = d.N;
+  if (y_.val().accumulate(txn, id(), ctx, [batch](V3 *v) { v->set_batch_size(batch); })) {
+    GPUConn conn = ctx->conn();
+    V3 &y = y_.val().get_mut(txn, id());
+    check_padded(x, src_pad_, "HaloRepad2DOp");
+    check_padded(y, dst_pad_, "HaloRepad2DOp");
+    adh_check(adh_halo_repad_nchw(ADH_F32, (uint32_t)src_pad_, (uint32_t)dst_pad_, d.W, d.H, d.C, d.N,
+                                  x.base_as_view().dptr(), y.base_as_view().dptr(), conn.stream()),
+              "HaloRepad2DOp::_forward");
+  }
+}
+
+// ---- HaloExch2DOp (op.cc:2963-3052) ----
+// All ranks or none take part (op.cc:2973,3021).  The reference brackets the exchange with two
+// host-side syncs of every device (op.cc:2976,3001); with all tiles on one in-order stream the
+// producers' kernels are already ordered before it, so there is nothing to wait for.
+template <>
+void HaloExch2DOp<V3>::_forward(TxnId txn) {
+  MultiGPUContext *ctx = mgpu_ctx_of(ctx_);
+  size_t num_writes = 0;
+  for (size_t r = 0; r < ctx->num_ranks(); ++r)
+    if (xs_.at(r).val().accumulate(txn, id(), ctx->device_context(r).get(), [](V3 *) {})) ++num_writes;
+  if (num_writes != 0 && num_writes != ctx->num_ranks()) throw HazardError("HaloExch2DOp: some ranks already exchanged");
+  if (num_writes == 0) return;
+  for (size_t r = 0; r < ctx->num_ranks(); ++r) {
+    V3 &x = xs_.at(r).val().get_mut(txn, id());
+    check_padded(x, halo_pad_, "HaloExch2DOp");  // op.cc:2981-2982
+    const TileDims d = dims_of(x);
+    ctx->spatial_comm(r)->group_start();
+    ctx->spatial_comm(r)->halo_exchange(x.base_as_view().dptr(), (uint32_t)halo_pad_, d.W, d.H, d.C, d.N,
+                                        SPATIAL2D_TENSOR_NCHW, SPATIAL2D_DATA_FLOAT);
+  }
+  GPUConn conn = ctx->device_context(0)->conn();
+  adh_check(Spatial2DComm::group_end_all(ctx->spatial_comm(0), conn), "HaloExch2DOp::_forward");
+}
+template <>
+void HaloExch2DOp<V3>::_backward(TxnId txn) {
+  MultiGPUContext *ctx = mgpu_ctx_of(ctx_);
+  size_t num_writes = 0;
+  for (size_t r = 0; r < ctx->num_ranks(); ++r) {
+    GPUContext *dc = ctx->device_context(r).get();
+    const size_t batch = xs_.at(r).val().get(txn, id()).batch_size();
+    if (xs_.at(r).grad().accumulate(txn, id(), dc, [dc, batch](V3 *g) {
+          GPUConn conn = dc->conn();
+          g->set_batch_size(batch);
+          g->base_as_view().set_constant(0.0f, conn);
+        }))
+      ++num_writes;
+  }
+  if (num_writes != 0 && num_writes != ctx->num_ranks()) throw HazardError("HaloExch2DOp: some ranks already reduced");
+  if (num_writes == 0) return;
+  for (size_t r = 0; r < ctx->num_ranks(); ++r) {
+    V3 &g = xs_.at(r).grad().get_mut(txn, id());
+    check_padded(g, halo_pad_, "HaloExch2DOp");
+    const TileDims d = dims_of(g);
+    ctx->spatial_comm(r)->group_start();
+    ctx->spatial_comm(r)->halo_reduce(g.base_as_view().dptr(), (uint32_t)halo_pad_, d.W, d.H, d.C, d.N,
+                                      SPATIAL2D_TENSOR_NCHW, SPATIAL2D_DATA_FLOAT);
+  }
+  GPUConn conn = ctx->device_context(0)->conn();
+  adh_check(Spatial2DComm::group_end_all(ctx->spatial_comm(0), conn), "HaloExch2DOp::_backward");
+}
+
+// ---- SlabConv2DOp (op.cc:1547-1727) ----
+namespace {
+GPUContext *rank_ctx(const shared_ptr<Context> &ctx, size_t r) {
+  if (MultiGPUContext *m = dynamic_cast<MultiGPUContext *>(ctx.get())) return m->device_context(r).get();
+  return gpu_ctx_of(ctx);
+}
+void check_filter(A4 &w, size_t cin, size_t cout) {
+  if (w.dim() != Shape4D(3, 3, cin, cout) || !w.is_packed())
+    throw std::invalid_argument("SlabConv2DOp: filter must be a packed Shape4D(3,3,Cin,Cout)");
+}
+}  // namespace
+
+template <>
+void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
+  const size_t K = xs_.size();
+  vector<size_t> todo;
+  for (size_t r = 0; r < K; ++r)
+    if (ys_[r].val().overwrite(txn, id(), rank_ctx(ctx_, r))) todo.push_back(r);
+  // group the ranks by filter buffer: one launch per distinct filter
+  while (!todo.empty()) {
+    const float *w0 = kernels_[todo[0]].val().get(txn, id()).dptr();
+    const void *xt[ADH_MAX_TILES];
+    void *yt[ADH_MAX_TILES];
+    uint32_t n = 0;
+    TileDims d{};
+    vector<size_t> rest;
+    for (size_t r : todo) {
+      A4 &w = kernels_[r].val().get(txn, id());
+      if (w.dptr() != w0) {
+        rest.push_back(r);
+        continue;
+      }
+      V3 &x = xs_[r].val().get(txn, id());
+      V3 &y = ys_[r].val().get_excl(txn, id());
+      d = dims_of(x);
+      y.set_batch_size(d.N);
+      check_padded(x, 1, "SlabConv2DOp");
+      check_filter(w, d.C, shape_.filters);
+      xt[n] = x.base_as_view().dptr();
+      yt[n] = y.as_view().dptr();
+      ++n;
+    }
+    GPUConn conn = rank_ctx(ctx_, todo[0])->conn();
+    adh_check(adh_conv3x3_slab_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt, 0.0f,
+                                         nullptr, 0, conn.stream()),
+              "SlabConv2DOp::_forward");
+    todo.swap(rest);
+  }
+}
+
+template <>
+void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
+  const size_t K = xs_.size();
+  // filter gradient: dw += sum over the tiles that share the filter (zeroed on first touch,
+  // op.cc:1651-1654; beta = 1, op.cc:1660-1671)
+  vector<size_t> todo;
+  for (size_t r = 0; r < K; ++r) {
+    GPUContext *dc = rank_ctx(ctx_, r);
+    if (kernels_[r].grad().accumulate(txn, id(), dc, [dc](A4 *g) {
+          GPUConn conn = dc->conn();
+          g->set_constant(0.0f, conn);
+        }))
+      todo.push_back(r);
+  }
+  // ranks whose kernel variable was already counted through a shared VarData still contribute
+  for (size_t r = 0; r < K; ++r) {
+    bool listed = false;
+    for (size_t q : todo) listed = listed || q == r;
+    if (!listed) {
+      for (size_t q : todo)
+        if (kernels_[q].grad().var() == kernels_[r].grad().var()) {
+          todo.push_back(r);
+          break;
+        }
+    }
+  }
+  while (!todo.empty()) {
+    float *dw = kernels_[todo[0]].grad().get_mut(txn, id()).dptr();
+    const void *xt[ADH_MAX_TILES];
+    const void *dyt[ADH_MAX_TILES];
+    uint32_t n = 0;
+    TileDims d{};
+    vector<size_t> rest;
+    for (size_t r : todo) {
+      if (kernels_[r].grad().get(txn, id()).dptr() != dw) {
+        rest.push_back(r);
+        continue;
+      }
+      V3 &x = xs_[r].val().get(txn, id());
+      V3 &dy = ys_[r].grad().get(txn, id());
+      d = dims_of(x);
+      xt[n] = x.base_as_view().dptr();
+      dyt[n] = dy.as_view().dptr();
+      ++n;
+    }
+    GPUContext *dc = rank_ctx(ctx_, todo[0]);
+    const size_t ws = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
+                                                  d.H, d.W);
+    dc->reserve_scratch(ws);
+    auto scratch = dc->get_scratch();
+    GPUConn conn = dc->conn();
+    adh_check(adh_conv3x3_slab_bwd_filter_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, dyt, dw,
+                                                1.0f, scratch->dptr(), scratch->size(), conn.stream()),
+              "SlabConv2DOp::_backward (filter)");
+    todo.swap(rest);
+  }
+  // input gradient over the WHOLE padded slab, zeroed on first touch (op.cc:1687-1691), beta = 1
+  todo.clear();
+  for (size_t r = 0; r < K; ++r) {
+    GPUContext *dc = rank_ctx(ctx_, r);
+    const size_t batch = xs_[r].val().get(txn, id()).batch_size();
+    if (xs_[r].grad().accumulate(txn, id(), dc, [dc, batch](V3 *g) {
+          GPUConn conn = dc->conn();
+          g->set_batch_size(batch);
+          g->base_as_view().set_constant(0.0f, conn);
+        }))
+      todo.push_back(r);
+  }
+  while (!todo.empty()) {
+    const float *w0 = kernels_[todo[0]].val().get(txn, id()).dptr();
+    const void *dyt[ADH_MAX_TILES];
+    void *dxt[ADH_MAX_TILES];
+    uint32_t n = 0;
+    TileDims d{};
+    vector<size_t> rest;
+    for (size_t r : todo) {
+      if (kernels_[r].val().get(txn, id()).dptr() != w0) {
+        rest.push_back(r);
+        continue;
+      }
+      V3 &dx = xs_[r].grad().get_mut(txn, id());
+      V3 &dy = ys_[r].grad().get(txn, id());
+      check_padded(dx, 1, "SlabConv2DOp");
+      d = dims_of(dx);
+      dyt[n] = dy.as_view().dptr();
+      dxt[n] = dx.base_as_view().dptr();
+      ++n;
+    }
+    GPUConn conn = rank_ctx(ctx_, todo[0])->conn();
+    adh_check(adh_conv3x3_slab_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, w0, dyt, dxt,
+                                              1.0f, nullptr, 0, conn.stream()),
+              "SlabConv2DOp::_backward (data)");
+    todo.swap(rest);
+  }
+}
+
+// ---- SoftmaxNLLLossOp, 1-D logits (op.cc:4118-4188) ----
+typedef GPUBatchArray1D<float> V1;
+typedef GPUBatchArray0D<uint32_t> L0;
+typedef GPUBatchArray0D<float> F0;
+
+template <>
+void SoftmaxNLLLossOp<V1, L0, F0>::_forward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V1 &x = x_.val().get(txn, id());
+  const uint32_t C = (uint32_t)x.dim().shape[0], N = (uint32_t)x.batch_size();
+  const bool wy = y_.val().overwrite(txn, id(), ctx);
+  const bool wl = loss_.val().overwrite(txn, id(), ctx);
+  if (wy || wl) {
+    GPUConn conn = ctx->conn();
+    V1 &y = y_.val().get_excl(txn, id());
+    F0 &loss = loss_.val().get_excl(txn, id());
+    L0 &label = label_.val().get(txn, id());
+    y.set_batch_size(N);
+    loss.set_batch_size(N);
+    if (label.batch_size() != N) throw std::invalid_argument("SoftmaxNLLLossOp: one label per example");
+    softmax_fwd<float>(C, N, x.as_view().dptr(), y.as_view().dptr(), conn.stream());
+    softmax_nll_loss_fwd<float>(C, N, y.as_view().dptr(), label.as_view().dptr(), loss.as_view().dptr(), conn.stream());
+  }
+}
+template <>
+void SoftmaxNLLLossOp<V1, L0, F0>::_backward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V1 &y = y_.val().get(txn, id());
+  const uint32_t C = (uint32_t)y.dim().shape[0], N = (uint32_t)y.batch_size();
+  const size_t batch = N;
+  if (x_.grad().accumulate(txn, id(), ctx, [ctx, batch](V1 *g) {
+        GPUConn conn = ctx->conn();
+        g->set_batch_size(batch);
+        g->as_view().set_constant(0.0f, conn);
+      })) {
+    GPUConn conn = ctx->conn();
+    softmax_nll_loss_bwd<float>(C, N, y.as_view().dptr(), label_.val().get(txn, id()).as_view().dptr(),
+                                loss_.grad().get(txn, id()).as_view().dptr(),
+                                x_.grad().get_mut(txn, id()).as_view().dptr(), conn.stream());
+  }
+}
+
+}  // namespace arraydiff

@@ -1,0 +1,345 @@
+// Tests of the C++ host layer (arraydiff_cuda_amd/host) written the way a user of the
+// reference's op API would write them.  `test_host cpu` runs the parts that need no GPU
+// (shape algebra, Spatial2DComm protocol and error codes); `test_host gpu` builds the
+// spatially-parallel conv graph with the reference's factories and checks values, input
+// gradient and filter gradient against the CPU oracle's UNSPLIT convolution.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "arraydiff/op.hh"
+
+extern "C" {
+// CPU oracle (oracle/adh_oracle.c): the checker
+void orc_conv_slab_fwd(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, uint32_t k, const float *x_pad,
+                       const float *wt, float beta, float *y);
+void orc_conv_slab_bwd_data(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, uint32_t k,
+                            const float *wt, const float *dy, float beta, float *dx_pad);
+void orc_conv_slab_bwd_filter(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, uint32_t k,
+                              const float *x_pad, const float *dy, float beta, float *dw);
+void orc_halo_pad(int dtype, uint32_t p, uint32_t W, uint32_t H, uint32_t C, uint32_t N, const void *x, void *y);
+void orc_halo_unpad(int dtype, uint32_t p, uint32_t W, uint32_t H, uint32_t C, uint32_t N, const void *x, void *y);
+int orc_halo_op(int which, int dtype, uint32_t gw, uint32_t gh, uint32_t p, uint32_t W, uint32_t H, uint32_t C,
+                uint32_t N, void *const *tiles);
+void orc_softmax_fwd(uint32_t C, uint32_t N, const float *x, float *y);
+void orc_softmax_nll_loss_fwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label, float *loss);
+void orc_softmax_nll_loss_bwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label, const float *dloss,
+                              float *dx);
+}
+
+using namespace arraydiff;
+
+static int failures = 0;
+#define CHECK(cond)                                                       \
+  do {                                                                    \
+    if (!(cond)) {                                                        \
+      std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);         \
+      ++failures;                                                         \
+    }                                                                     \
+  } while (0)
+
+static double rel_err(const std::vector<float> &a, const std::vector<float> &b) {
+  double num = 0, den = 0;
+  for (size_t i = 0; i < a.size(); ++i) {
+    num = std::fmax(num, std::fabs((double)a[i] - b[i]));
+    den = std::fmax(den, std::fabs((double)b[i]));
+  }
+  return num / (den > 0 ? den : 1);
+}
+
+static void test_shapes() {
+  Shape3D padded(58, 16, 64);
+  CHECK(padded.packed_stride().shape[2] == 928);
+  Shape3D dim(56, 14, 64), off(1, 1, 0), stride = padded.packed_stride();
+  CHECK(stride.packed_dim(dim.minor()) == padded);
+  CHECK(!dim.is_packed(stride) && dim.is_packed(dim.packed_stride()));
+  CHECK(off.to_index(stride) == 59);
+  CHECK(dim.append(32) == Shape4D(56, 14, 64, 32));
+  CHECK(Shape3D::Zero().is_zero() && dim.flat_size() == 56u * 14 * 64);
+  // brute force: to_index of (w,h,c,n) against nested loops over a padded buffer
+  size_t p = 2, W = 5, H = 4, C = 3, N = 2, lin = 0;
+  Shape4D st = Shape3D(W + 2 * p, H + 2 * p, C).packed_stride().append((W + 2 * p) * (H + 2 * p) * C);
+  for (size_t n = 0; n < N; ++n)
+    for (size_t c = 0; c < C; ++c)
+      for (size_t h = 0; h < H + 2 * p; ++h)
+        for (size_t w = 0; w < W + 2 * p; ++w, ++lin) CHECK(Shape4D(w, h, c, n).to_index(st) == lin);
+  CHECK(Shape0D().flat_size() == 1 && Shape0D().append(7) == Shape1D(7));
+}
+
+static void test_comm_protocol() {
+  Spatial2DComm comms[4];
+  CHECK(Spatial2DComm::InitAll(comms, 2, 2) == ADH_OK);
+  // rank = r_w + num_w * r_h
+  CHECK(comms[3].rank == 3 && comms[3].rank_w == 1 && comms[3].rank_h == 1 && comms[2].rank_w == 0);
+  CHECK(Spatial2DComm::InitAll(comms, 0, 2) == ADH_EINVAL);
+  CHECK(Spatial2DComm::InitAll(nullptr, 1, 2) == ADH_ENULL);
+  GPUConn conn(0, nullptr);
+  float dummy[4];
+  // 2x2 grid: every rank recorded, but the combination is unimplemented
+  CHECK(Spatial2DComm::InitAll(comms, 2, 2) == ADH_OK);
+  for (int r = 0; r < 4; ++r) {
+    comms[r].group_start();
+    comms[r].halo_exchange(dummy, 1, 2, 2, 1, 1, SPATIAL2D_TENSOR_NCHW, SPATIAL2D_DATA_FLOAT);
+  }
+  CHECK(comms[0].group_end(conn) == ADH_EUNIMPL);
+  // 1x4: a peer that has not recorded for this epoch -> protocol error instead of a hang
+  CHECK(Spatial2DComm::InitAll(comms, 1, 4) == ADH_OK);
+  for (int r = 0; r < 3; ++r) {
+    comms[r].group_start();
+    comms[r].halo_exchange(dummy, 1, 2, 2, 1, 1, SPATIAL2D_TENSOR_NCHW, SPATIAL2D_DATA_FLOAT);
+  }
+  CHECK(comms[0].group_end(conn) == ADH_EPROTOCOL);
+  comms[3].group_start();
+  comms[3].halo_exchange(nullptr, 1, 2, 2, 1, 1, SPATIAL2D_TENSOR_NCHW, SPATIAL2D_DATA_FLOAT);
+  CHECK(comms[0].group_end(conn) == ADH_ENULL);  // NULL buffer (src/spatial.cc:71-73)
+  // unsupported format / type
+  for (int r = 0; r < 4; ++r) {
+    comms[r].group_start();
+    comms[r].halo_exchange(dummy, 1, 2, 2, 1, 1, SPATIAL2D_TENSOR_NHWC, SPATIAL2D_DATA_FLOAT);
+  }
+  CHECK(comms[1].group_end(conn) == ADH_EUNIMPL);
+  for (int r = 0; r < 4; ++r) {
+    comms[r].group_start();
+    comms[r].halo_reduce(dummy, 1, 2, 2, 1, 1, SPATIAL2D_TENSOR_NCHW, SPATIAL2D_DATA_DOUBLE);
+  }
+  CHECK(comms[1].group_end(conn) == ADH_EUNIMPL);
+  CHECK(Spatial2DComm::group_end_all(comms, conn) == ADH_EUNIMPL);
+  // mismatched arguments between ranks
+  for (int r = 0; r < 4; ++r) {
+    comms[r].group_start();
+    comms[r].halo_exchange(dummy, 1, 2 + (r == 2), 2, 1, 1, SPATIAL2D_TENSOR_NCHW, SPATIAL2D_DATA_FLOAT);
+  }
+  CHECK(Spatial2DComm::group_end_all(comms, conn) == ADH_EINVAL);
+  // reduce with H < 2*halo: rejected by the C ABI before any launch
+  for (int r = 0; r < 4; ++r) {
+    comms[r].group_start();
+    comms[r].halo_reduce(dummy, 2, 4, 3, 1, 1, SPATIAL2D_TENSOR_NCHW, SPATIAL2D_DATA_FLOAT);
+  }
+  CHECK(comms[2].group_end(conn) == ADH_EINVAL);
+  // 1x1: nothing to do
+  Spatial2DComm one[1];
+  CHECK(Spatial2DComm::InitAll(one, 1, 1) == ADH_OK);
+  one[0].group_start();
+  one[0].halo_exchange(dummy, 1, 2, 2, 1, 1, SPATIAL2D_TENSOR_NCHW, SPATIAL2D_DATA_FLOAT);
+  CHECK(one[0].group_end(conn) == ADH_OK);
+  CHECK(comms[0].epoch == comms[1].epoch);
+}
+
+static std::vector<float> uniform(std::mt19937 &g, size_t n, float lo, float hi) {
+  std::uniform_real_distribution<float> d(lo, hi);
+  std::vector<float> v(n);
+  for (auto &x : v) x = d(g);
+  return v;
+}
+static std::vector<float> normal(std::mt19937 &g, size_t n, float s) {
+  std::normal_distribution<float> d(0.f, s);
+  std::vector<float> v(n);
+  for (auto &x : v) x = d(g);
+  return v;
+}
+
+// Broadcast(X) -> Scatter -> HaloPad -> HaloExch -> Conv(halo_padded_input) -> gather, the block
+// of src/zoo.cc:577-652 and :1522-1526, on K row-tiles of one GPU.
+static void test_spatial_conv_graph(size_t K, size_t N, size_t C, size_t Co, size_t H, size_t W) {
+  std::mt19937 gen(1234 + (unsigned)K);
+  auto ctx = MultiGPUContext::Make(K);
+  std::vector<float> X = uniform(gen, N * C * H * W, -1, 1);
+  std::vector<float> Wt = normal(gen, Co * C * 9, std::sqrt(2.0f / (C * 9)));
+  std::vector<float> dY = normal(gen, N * Co * H * W, 1.0f);
+
+  typedef GPUBatchArray3D<float> V;
+  typedef GPUArray4D<float> A;
+  auto x_src = SrcOp<V>::Make(Shape3D(W, H, C), N, ctx->device_context(0));
+  auto w_src = ParamOp<A>::Make(Shape4D(3, 3, C, Co), ctx->device_context(0));
+  vector<shared_ptr<Var<V>>> xs(K, x_src);
+  vector<shared_ptr<Var<A>>> ws(K, w_src);
+  auto tiles = SpatialScatter2DOp<V>::MakeParallel(xs, ctx);
+  auto padded = HaloPad2DOp<V>::MakeParallel(1, tiles, ctx);
+  auto exch = HaloExch2DOp<V>::MakeParallel(1, padded, ctx);
+  Conv2DShape cs;
+  cs.filters = Co;
+  cs.axes = {0, 1};
+  cs.kernel = {3, 3};
+  cs.dilate = {1, 1};
+  cs.stride = {1, 1};
+  cs.pad = {1, 1};
+  cs.halo_padded_input = true;
+  cs.enable_hmma = false;
+  auto ys = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch, ws, ctx);
+  auto y_full = SpatialJoinedGather2DOp<V>::Make(ys, ctx);
+  auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
+  sink->set_host_grad(dY.data());
+
+  CHECK(padded[0]->offset() == Shape3D(1, 1, 0));
+  CHECK(padded[0]->stride() == Shape3D(W + 2, H / K + 2, C).packed_stride());
+  CHECK(ys[0]->shape() == Shape3D(W, H / K, Co));
+
+  for (int rep = 0; rep < 2; ++rep) {  // two transactions: buffers are reused, first touch re-zeroes
+    TxnId txn;
+    x_src->load(txn, X.data());
+    w_src->load(txn, Wt.data());
+    sink->gradient(txn);
+    ctx->sync();
+    std::vector<float> Y(N * Co * H * W), dX(X.size()), dW(Wt.size());
+    sink->store_val(txn, Y.data());
+    x_src->store_grad(txn, dX.data());
+    w_src->store_grad(txn, dW.data());
+
+    // oracle: the UNSPLIT convolution over the zero-padded full tensor
+    std::vector<float> Xp(N * C * (H + 2) * (W + 2));
+    orc_halo_pad(0, 1, W, H, C, N, X.data(), Xp.data());
+    std::vector<float> Yr(Y.size()), dXp(Xp.size()), dXr(X.size()), dWr(Wt.size());
+    orc_conv_slab_fwd(N, C, Co, H, W, 3, Xp.data(), Wt.data(), 0.f, Yr.data());
+    orc_conv_slab_bwd_data(N, C, Co, H, W, 3, Wt.data(), dY.data(), 0.f, dXp.data());
+    orc_halo_unpad(0, 1, W, H, C, N, dXp.data(), dXr.data());
+    orc_conv_slab_bwd_filter(N, C, Co, H, W, 3, Xp.data(), dY.data(), 0.f, dWr.data());
+    const double ey = rel_err(Y, Yr), ex = rel_err(dX, dXr), ew = rel_err(dW, dWr);
+    std::printf("graph K=%zu N=%zu C=%zu->%zu %zux%zu rep %d: rel-err y %.2e dx %.2e dw %.2e\n", K, N, C, Co, H, W, rep,
+                ey, ex, ew);
+    CHECK(ey <= 1e-5 && ex <= 1e-5 && ew <= 1e-5);
+  }
+}
+
+// The call sequence of tools/microbench_spatial_conv.cc:227-263: raw buffers, per-rank
+// group_start / halo_exchange / group_end, no Op machinery.
+static void test_microbench_sequence() {
+  const uint32_t K = 4, p = 1, W = 9, H = 5, C = 3, N = 2;
+  auto ctx = MultiGPUContext::Make(K);
+  std::mt19937 gen(7);
+  const size_t elems = (size_t)(W + 2 * p) * (H + 2 * p) * C * N;
+  std::vector<std::vector<float>> host(K);
+  std::vector<GPUMemory<float>> dev;
+  void *want_ptrs[K];
+  std::vector<std::vector<float>> want(K);
+  for (uint32_t r = 0; r < K; ++r) {
+    host[r] = uniform(gen, elems, -1, 1);
+    want[r] = host[r];
+    want_ptrs[r] = want[r].data();
+    dev.emplace_back(elems, ctx->device_context(r).get());
+    GPUConn conn = ctx->device_context(r)->conn();
+    dev[r].load_sync(host[r].data(), 0, elems, conn);
+  }
+  for (int which = 0; which < 2; ++which) {
+    CHECK(orc_halo_op(which, 0, 1, K, p, W, H, C, N, want_ptrs) == 0);
+    for (uint32_t r = 0; r < K; ++r) {
+      ctx->spatial_comm(r)->group_start();
+      if (which == 0)
+        ctx->spatial_comm(r)->halo_exchange(dev[r].dptr(), p, W, H, C, N, SPATIAL2D_TENSOR_NCHW, SPATIAL2D_DATA_FLOAT);
+      else
+        ctx->spatial_comm(r)->halo_reduce(dev[r].dptr(), p, W, H, C, N, SPATIAL2D_TENSOR_NCHW, SPATIAL2D_DATA_FLOAT);
+    }
+    for (uint32_t r = 0; r < K; ++r) {
+      GPUConn conn = ctx->device_context(r)->conn();
+      CHECK(ctx->spatial_comm(r)->group_end(conn) == ADH_OK);
+    }
+    ctx->sync();
+    for (uint32_t r = 0; r < K; ++r) {
+      std::vector<float> got(elems);
+      GPUConn conn = ctx->device_context(r)->conn();
+      dev[r].store_sync(got.data(), 0, elems, conn);
+      CHECK(std::memcmp(got.data(), want[r].data(), elems * 4) == 0);
+    }
+  }
+  // the reference's launcher names work on the same buffers
+  float *b[4] = {dev[0].dptr(), dev[1].dptr(), dev[2].dptr(), dev[3].dptr()};
+  CHECK(orc_halo_op(0, 0, 1, K, p, W, H, C, N, want_ptrs) == 0);
+  for (uint32_t r = 0; r < K; ++r)
+    spatial2d_1x4_halo_exch_nchw<float>(r, p, W, H, C, N, b[0], b[1], b[2], b[3], ctx->stream());
+  ctx->sync();
+  for (uint32_t r = 0; r < K; ++r) {
+    std::vector<float> got(elems);
+    GPUConn conn = ctx->device_context(r)->conn();
+    dev[r].store_sync(got.data(), 0, elems, conn);
+    CHECK(std::memcmp(got.data(), want[r].data(), elems * 4) == 0);
+  }
+}
+
+static void test_softmax_loss_op() {
+  const size_t N = 64, C = 1000;
+  auto ctx = GPUContext::Make(0);
+  std::mt19937 gen(99);
+  std::vector<float> x = normal(gen, N * C, 2.0f);
+  std::vector<uint32_t> label(N);
+  for (size_t i = 0; i < N; ++i) label[i] = gen() % C;
+  typedef GPUBatchArray1D<float> V1;
+  typedef GPUBatchArray0D<uint32_t> L0;
+  typedef GPUBatchArray0D<float> F0;
+  auto x_src = SrcOp<V1>::Make(Shape1D(C), N, ctx);
+  auto l_src = SrcOp<L0>::Make(Shape0D(), N, ctx);
+  auto loss = softmax_nll_loss<V1, L0, F0>(x_src, l_src, ctx);
+  TxnId txn;
+  x_src->load(txn, x.data());
+  l_src->load(txn, label.data());
+  loss->gradient(txn);
+  ctx->sync();
+  std::vector<float> got_loss(N), got_dx(N * C), got_y(N * C);
+  loss->store_loss(txn, got_loss.data());
+  loss->store_prob(txn, got_y.data());
+  x_src->store_grad(txn, got_dx.data());
+  std::vector<float> y(N * C), l(N), dx(N * C, 0.f), ones(N, 1.0f);
+  orc_softmax_fwd(C, N, x.data(), y.data());
+  orc_softmax_nll_loss_fwd(C, N, y.data(), label.data(), l.data());
+  orc_softmax_nll_loss_bwd(C, N, y.data(), label.data(), ones.data(), dx.data());
+  const double ey = rel_err(got_y, y), el = rel_err(got_loss, l), ed = rel_err(got_dx, dx);
+  std::printf("softmax-nll op: rel-err y %.2e loss %.2e dx %.2e\n", ey, el, ed);
+  CHECK(ey <= 1e-5 && el <= 1e-5 && ed <= 1e-5);
+}
+
+static void test_txn_hazards() {
+  auto ctx = GPUContext::Make(0);
+  typedef GPUBatchArray3D<float> V;
+  auto src = SrcOp<V>::Make(Shape3D(4, 4, 2), 1, ctx);
+  auto pad = HaloPad2DOp<V>::Make(1, src, ctx);
+  TxnId txn;
+  bool threw = false;
+  try {
+    pad->eval(txn);  // the source was never loaded in this transaction
+  } catch (const HazardError &) {
+    threw = true;
+  }
+  CHECK(threw);
+  // pad -> unpad round trip through the ops, and HaloRepad forward
+  std::vector<float> x(32), y(32);
+  for (size_t i = 0; i < x.size(); ++i) x[i] = (float)i + 1;
+  auto unpad = HaloUnpad2DOp<V>::Make(1, pad, ctx);
+  auto sink = HostGradSinkOp<V>::Make(unpad, ctx);
+  std::vector<float> g(32, 2.0f), dx(32);
+  sink->set_host_grad(g.data());
+  TxnId t2;
+  src->load(t2, x.data());
+  sink->gradient(t2);
+  sink->store_val(t2, y.data());
+  src->store_grad(t2, dx.data());
+  CHECK(x == y && dx == g);
+  bool bad = false;
+  try {
+    Conv2DShape cs{};
+    cs.filters = 2; cs.kernel = {5, 5}; cs.stride = {1, 1}; cs.dilate = {1, 1}; cs.pad = {2, 2}; cs.halo_padded_input = true;
+    auto w = ParamOp<GPUArray4D<float>>::Make(Shape4D(5, 5, 2, 2), ctx);
+    auto c = CudnnConv2DOp<V, GPUArray4D<float>>::Make(cs, pad, w, ctx);
+  } catch (const std::invalid_argument &) {
+    bad = true;
+  }
+  CHECK(bad);
+}
+
+int main(int argc, char **argv) {
+  const std::string mode = argc > 1 ? argv[1] : "cpu";
+  test_shapes();
+  test_comm_protocol();
+  if (mode == "gpu") {
+    test_txn_hazards();
+    test_microbench_sequence();
+    test_spatial_conv_graph(4, 2, 8, 16, 8, 12);
+    test_spatial_conv_graph(2, 3, 5, 7, 6, 9);
+    test_spatial_conv_graph(1, 1, 16, 16, 5, 5);
+    test_spatial_conv_graph(4, 4, 64, 64, 56, 56);
+    test_softmax_loss_op();
+  }
+  std::printf("%s: %d failure(s)\n", mode.c_str(), failures);
+  return failures ? 1 : 0;
+}

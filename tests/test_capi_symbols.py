@@ -1,0 +1,52 @@
+"""The C-ABI library loads and exports every symbol include/adh_capi.h declares; argument
+validation that returns before any device work is exercised without a GPU."""
+import ctypes
+import os
+import re
+
+from arraydiff_cuda_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    hdr = open(os.path.join(ROOT, "include", "adh_capi.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    return sorted(set(re.findall(r"\b(adh_[a-z0-9_]+)\s*\(", hdr)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    names = declared_symbols()
+    assert len(names) >= 28
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), "libadh.so does not export %s" % n
+    assert set(names) == set(capi.SIGNATURES), "capi.SIGNATURES out of sync with the header"
+    assert capi.lib().adh_version() == 1
+    assert b"NULL" in capi.lib().adh_error_string(capi.ADH_ENULL)
+
+
+def test_argument_errors_need_no_gpu():
+    l = capi.lib()
+    bogus = ctypes.c_void_p(0x1000)
+    tb, keep = capi.ptr_table([0x1000, None])
+    assert l.adh_halo_exchange_nchw(0, 1, 2, 1, 4, 4, 1, 1, tb, None) == capi.ADH_ENULL
+    tb4, keep4 = capi.ptr_table([0x1000] * 4)
+    assert l.adh_halo_exchange_nchw(0, 2, 2, 1, 4, 4, 1, 1, tb4, None) == capi.ADH_EUNIMPL
+    assert l.adh_halo_exchange_nchw(7, 1, 2, 1, 4, 4, 1, 1, tb4, None) == capi.ADH_EINVAL          # dtype
+    assert l.adh_halo_reduce_nchw(0, 1, 4, 3, 4, 4, 1, 1, tb4, None) == capi.ADH_EINVAL            # H < 2p
+    assert l.adh_halo_exchange_nchw(0, 1, 1, 1, 4, 4, 1, 1, tb4, None) == capi.ADH_OK              # 1x1 no-op
+    odd, keepo = capi.ptr_table([0x1001, 0x1000])
+    assert l.adh_halo_exchange_nchw(0, 1, 2, 1, 4, 4, 1, 1, odd, None) == capi.ADH_EALIGN
+    assert l.adh_tiles_pack_nchw(0, 3, 1, 4, 8, 1, 1, bogus, tb4, None) == capi.ADH_EINVAL          # H % K
+    assert l.adh_tiles_pack_nchw(0, 17, 1, 4, 34, 1, 1, bogus, tb4, None) == capi.ADH_EINVAL        # > 16 tiles
+    assert l.adh_slice_copy_nchw(0, 5, 1, 1, 1, bogus, 4, 4, 1, 0, 0, 0, bogus, 8, 8, 1, 0, 0, 0, None) == capi.ADH_EINVAL
+    assert l.adh_conv3x3_slab_fwd(0, 1, 4, 4, 3, 3, bogus, bogus, bogus, 0.5, None, 0, None) == capi.ADH_EINVAL  # beta
+    assert l.adh_conv3x3_slab_fwd(1, 1, 4, 4, 3, 3, bogus, bogus, bogus, 0.0, None, 0, None) == capi.ADH_EUNIMPL  # bf16
+    assert l.adh_conv3x3_slab_fwd(0, 1, 4, 4, 3, 3, None, bogus, bogus, 0.0, None, 0, None) == capi.ADH_ENULL
+    assert l.adh_conv3x3_slab_bwd_filter(0, 1, 4, 4, 3, 3, bogus, bogus, bogus, 0.0, bogus, 16, None) == capi.ADH_EWORKSPACE
+    assert l.adh_conv3x3_workspace_bytes(capi.ADH_CONV_BWD_FILTER, 0, 4, 32, 64, 64, 14, 56) > 0
+    assert l.adh_conv3x3_workspace_bytes(capi.ADH_CONV_FWD, 0, 4, 32, 64, 64, 14, 56) == 0
+    assert l.adh_softmax_fwd(10, 2, None, bogus, None) == capi.ADH_ENULL
+    assert l.adh_fill_f32(0, 1.0, None, None) == capi.ADH_OK                                       # empty
+    assert l.adh_softmax_fwd(0, 0, None, None, None) == capi.ADH_OK
