@@ -3,15 +3,18 @@
 //
 // GEMM view: D[co][ci] (one 16x16 tile per tap) += A[co][pixel] * B[pixel][ci], the reduction
 // runs over pixels, 4 consecutive pixels of one row per v_mfma_f32_16x16x4_f32.
-//   * a workgroup (4 waves) owns a run of output rows of one image and ALL 64 x 64 x 9
-//     filter taps: wave v owns output channels [16v,16v+16) x 4 ci-tiles x 9 taps = 36
-//     accumulator tiles (144 accumulator registers), so dy is read once per workgroup and
-//     every A operand feeds 36 MFMAs.
-//   * rows stream through LDS: the slab rows live in a 4-slot ring (row y in slot y%4), so
-//     each new output row loads exactly one new slab row and one dy row while the previous
-//     row is being multiplied; channel strides are 4 (mod 64) so the 16 channels x 4 pixels
-//     of one operand read hit 64 different banks.
-//   * every workgroup writes its partial 64x64x9 block to the workspace and a second kernel
+//   * a workgroup (8 waves, two per SIMD) owns a run of output rows of one image, 32 output
+//     channels, 64 input channels and all 9 taps: wave = (co tile, ci tile), 9 accumulator tiles.
+//     Halving the output channels per workgroup halves the partial block it has to write.
+//   * rows stream through LDS: the slab rows live in a 4-slot ring (4 separate arrays so that
+//     every phase of the 4x unrolled row loop names its slots statically), each new output row
+//     loads exactly one new slab row and one dy row, asynchronously and register-free with
+//     buffer_load ... lds, while the previous row is being multiplied; lanes past the row end
+//     carry an out-of-range offset and the hardware writes zero.  Channel pitch 68 floats
+//     (== 4 mod 64): the 16 channels x 4 pixels of one operand read hit 64 different banks.
+//   * LDS reads of k-step s+1 are interleaved 1:1 with the MFMAs of k-step s (two-deep register
+//     buffer, pinned with scheduling-group barriers).
+//   * every workgroup writes its partial 32x64x9 block to the workspace and a second kernel
 //     sums the partials in a fixed order: the result is deterministic (no float atomics).
 #include "adh_common.h"
 
@@ -19,179 +22,228 @@ namespace adh {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-static constexpr int kWgThreads = 256;
-static constexpr int kPitch = 64;                 // floats per staged row
-static constexpr int kXStride = 4 * kPitch + 4;   // slab ring: 4 rows per channel, == 4 (mod 64)
-static constexpr int kDStride = 2 * kPitch + 4;   // dy double buffer: 2 rows per channel
-// the last k-step reads columns up to 4*ceil(W/4)+1, which must stay inside the row
-static constexpr int kMaxW = kPitch - 4;
+static constexpr int kWgWaves = 8;
+static constexpr int kWgThreads = 64 * kWgWaves;
+static constexpr int kRowPitch = 68;              // floats per staged channel row, == 4 (mod 64)
+static constexpr int kXSlotFloats = 64 * kRowPitch;
+static constexpr int kDSlotFloats = 32 * kRowPitch;
+// the last k-step reads columns up to 4*ceil(W/4)+5 < kRowPitch, and a row is one 64-lane load
+static constexpr int kMaxW = 60;
+static constexpr int kPartialFloats = 32 * 64 * 9;
+static constexpr int kWgBufferFlags = 0x00020000;
+static constexpr uint32_t kWgOutOfRange = 0x80000000u;
 
 struct WgradParams {
   const float *x[ADH_MAX_TILES];
   const float *dy[ADH_MAX_TILES];
-  float *partial;            // [num_blocks][64*64*9] in (co, ci, tap) order, co/ci local to the group
+  float *partial;            // [grid.y][grid.x][32*64*9] in (co, ci, tap) order, local to the group
   uint32_t num_tiles, N, Cin, Cout, H, W;
   uint32_t rows_per_block, chunks_per_plane;  // grid.x = chunks_per_plane * N * num_tiles
-  uint32_t ci_groups;        // grid.y = ci_groups * co_groups
+  uint32_t ci_groups;        // grid.y = co_halves * ci_groups, co_halves = ceil(Cout/32)
   FastDiv div_chunks, div_tiles, div_ci_groups;
 };
 
 __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const WgradParams P) {
-  __shared__ float xs[64 * kXStride];
-  __shared__ float dys[64 * kDStride];
+  __shared__ float xs0[kXSlotFloats];
+  __shared__ float xs1[kXSlotFloats];
+  __shared__ float xs2[kXSlotFloats];
+  __shared__ float xs3[kXSlotFloats];
+  __shared__ float dys0[kDSlotFloats];
+  __shared__ float dys1[kDSlotFloats];
 
   const uint32_t tid = threadIdx.x;
-  const uint32_t lane = tid & 63u, wv = tid >> 6, g = lane >> 4, l16 = lane & 15u;
+  const uint32_t lane = tid & 63u, g = lane >> 4, l16 = lane & 15u;
+  const uint32_t wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t ot = wv & 1u;   // co tile inside the 32-channel half
+  const uint32_t ct = wv >> 1;   // ci tile
 
   uint32_t plane, chunk;
   P.div_chunks.divmod(blockIdx.x, plane, chunk);
   uint32_t n, t;
   P.div_tiles.divmod(plane, n, t);
-  uint32_t cog, cig;
-  P.div_ci_groups.divmod(blockIdx.y, cog, cig);
+  uint32_t coh, cig;
+  P.div_ci_groups.divmod(blockIdx.y, coh, cig);
   const uint32_t r0 = chunk * P.rows_per_block;
   const uint32_t r1 = min(r0 + P.rows_per_block, P.H);
   const uint32_t WP = P.W + 2u, HP = P.H + 2u;
-  const uint32_t ci0 = cig * 64u, co0 = cog * 64u;
+  const uint32_t ci0 = cig * 64u, co0 = coh * 32u;
   const float *__restrict__ x = P.x[t] + ((uint64_t)n * P.Cin) * HP * WP;
   const float *__restrict__ dy = P.dy[t] + ((uint64_t)n * P.Cout) * P.H * P.W;
 
-  // ---- staging: lane = column, wave v loads channels v, v+4, ... (16 per row) ----
-  const bool xcol_ok = lane < WP;
-  const bool dcol_ok = lane < P.W;
-  float xst[16], dst_[16];
-  auto load_x_row = [&](uint32_t y) {  // slab row y (clamped; masked at store)
-    const uint32_t off = min(y, HP - 1u) * WP + (xcol_ok ? lane : 0u);
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const uint32_t ci = min(ci0 + wv + 4u * i, P.Cin - 1u);
-      xst[i] = x[(uint64_t)ci * HP * WP + off];
-    }
-  };
-  auto store_x_row = [&](uint32_t y) {
-    const bool row_ok = xcol_ok && y < HP;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const uint32_t cl = wv + 4u * i;
-      xs[cl * kXStride + (y & 3u) * kPitch + lane] = (row_ok && ci0 + cl < P.Cin) ? xst[i] : 0.f;
-    }
-  };
-  auto load_dy_row = [&](uint32_t r) {
-    const uint32_t off = min(r, P.H - 1u) * P.W + (dcol_ok ? lane : 0u);
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const uint32_t co = min(co0 + wv + 4u * i, P.Cout - 1u);
-      dst_[i] = dy[(uint64_t)co * P.H * P.W + off];
-    }
-  };
-  auto store_dy_row = [&](uint32_t r) {
-    const bool row_ok = dcol_ok && r < r1;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const uint32_t cl = wv + 4u * i;
-      dys[cl * kDStride + (r & 1u) * kPitch + lane] = (row_ok && co0 + cl < P.Cout) ? dst_[i] : 0.f;
-    }
-  };
-
-  floatx4 acc[4][9];
-#pragma unroll
-  for (int ct = 0; ct < 4; ++ct)
-#pragma unroll
-    for (int tap = 0; tap < 9; ++tap) acc[ct][tap] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  // prologue: slab rows r0, r0+1, r0+2 and dy row r0
-  load_x_row(r0);
-  store_x_row(r0);
-  load_x_row(r0 + 1);
-  store_x_row(r0 + 1);
-  load_x_row(r0 + 2);
-  load_dy_row(r0);
-  store_x_row(r0 + 2);
-  store_dy_row(r0);
-  __syncthreads();
-
-  const uint32_t ksteps = (P.W + 3u) / 4u;
-  const uint32_t a_lane = (16u * wv + l16) * kDStride + g;
-  const uint32_t b_lane = l16 * kXStride + g;
-
-  for (uint32_t r = r0; r < r1; ++r) {
-    const bool more = r + 1 < r1;  // uniform
-    if (more) {
-      load_x_row(r + 3);
-      load_dy_row(r + 1);
-    }
-    const float *arow = dys + a_lane + (r & 1u) * kPitch;
-    const float *brow0 = xs + b_lane + ((r + 0u) & 3u) * kPitch;
-    const float *brow1 = xs + b_lane + ((r + 1u) & 3u) * kPitch;
-    const float *brow2 = xs + b_lane + ((r + 2u) & 3u) * kPitch;
-#pragma unroll 2
-    for (uint32_t ks = 0; ks < ksteps; ++ks) {
-      const float a = arow[4u * ks];
-#pragma unroll
-      for (int ct = 0; ct < 4; ++ct) {
-#pragma unroll
-        for (int kw = 0; kw < 3; ++kw) {
-          const float b0 = brow0[ct * 16 * kXStride + 4u * ks + kw];
-          const float b1 = brow1[ct * 16 * kXStride + 4u * ks + kw];
-          const float b2 = brow2[ct * 16 * kXStride + 4u * ks + kw];
-          acc[ct][0 + kw] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b0, acc[ct][0 + kw], 0, 0, 0);
-          acc[ct][3 + kw] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b1, acc[ct][3 + kw], 0, 0, 0);
-          acc[ct][6 + kw] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b2, acc[ct][6 + kw], 0, 0, 0);
-        }
-      }
-    }
-    if (more) {
-      store_x_row(r + 3);   // slot (r+3)%4 held row r-1, last read one barrier ago
-      store_dy_row(r + 1);
-    }
-    __syncthreads();
+  // columns 64..67 of every staged row are read by the last k-steps of wide rows but never
+  // written by the 64-lane loads: clear them once
+  for (uint32_t i = tid; i < 64u * 4u; i += kWgThreads) {
+    const uint32_t o = (i >> 2) * kRowPitch + 64u + (i & 3u);
+    xs0[o] = 0.f; xs1[o] = 0.f; xs2[o] = 0.f; xs3[o] = 0.f;
   }
 
-  // ---- epilogue: lane holds D[co = 4g+i][ci = l16] of each (ct, tap) tile ----
-  const uint32_t block_lin = blockIdx.y * gridDim.x + blockIdx.x;
-  float *__restrict__ part = P.partial + (uint64_t)block_lin * (64u * 64u * 9u);
+  // ---- staging: one 64-lane load = one channel row; wave v loads slab channels [8v,8v+8) and
+  // dy channels [4v,4v+4) ----
+  const __amdgpu_buffer_rsrc_t rsrc_x =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(x), 0, (int)(P.Cin * HP * WP * 4u), kWgBufferFlags);
+  const __amdgpu_buffer_rsrc_t rsrc_dy =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(dy), 0, (int)(P.Cout * P.H * P.W * 4u), kWgBufferFlags);
+  const uint32_t x_voff = lane < WP ? lane * 4u : kWgOutOfRange;
+  const uint32_t d_voff = lane < P.W ? lane * 4u : kWgOutOfRange;
+  const bool ragged_c = (ci0 + 64u > P.Cin) || (co0 + 32u > P.Cout);  // uniform
+  auto stage_x_row = [&](float *slot, uint32_t y) {  // slab row y of the 64 input channels
 #pragma unroll
-  for (int ct = 0; ct < 4; ++ct)
-#pragma unroll
-    for (int tap = 0; tap < 9; ++tap)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t co_l = 16u * wv + 4u * g + i, ci_l = 16u * ct + l16;
-        part[(co_l * 64u + ci_l) * 9u + tap] = acc[ct][tap][i];
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t cl = wv * 8u + i;
+      uint32_t voff = x_voff;
+      uint32_t ci = ci0 + cl;
+      if (ragged_c && ci >= P.Cin) {
+        voff = kWgOutOfRange;
+        ci = 0;
       }
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, slot + cl * kRowPitch, 4, voff,
+                                               __builtin_amdgcn_readfirstlane((ci * HP + y) * WP * 4u), 0, 0);
+    }
+  };
+  auto stage_dy_row = [&](float *slot, uint32_t r) {  // output row r of the 32 output channels
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t cl = wv * 4u + i;
+      uint32_t voff = d_voff;
+      uint32_t co = co0 + cl;
+      if (ragged_c && co >= P.Cout) {
+        voff = kWgOutOfRange;
+        co = 0;
+      }
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_dy, slot + cl * kRowPitch, 4, voff,
+                                               __builtin_amdgcn_readfirstlane((co * P.H + r) * P.W * 4u), 0, 0);
+    }
+  };
+
+  floatx4 acc[9];
+#pragma unroll
+  for (int tap = 0; tap < 9; ++tap) acc[tap] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const uint32_t ksteps = (P.W + 3u) / 4u;
+  const uint32_t npairs = (ksteps + 1u) / 2u;   // an odd tail k-step multiplies the zero columns
+  const uint32_t a_lane = (16u * ot + l16) * kRowPitch + g;
+  const uint32_t b_lane = (16u * ct + l16) * kRowPitch + g;
+
+  // one output row: dyr = its dy slot, b0/b1/b2 = the slab rows r, r+1, r+2
+  auto compute_row = [&](const float *dyr, const float *b0, const float *b1, const float *b2) {
+    float a[2], b[2][9];
+    auto read_operands = [&](int buf, uint32_t ks) {
+      const uint32_t col = 4u * ks;
+      a[buf] = dyr[a_lane + col];
+#pragma unroll
+      for (int kw = 0; kw < 3; ++kw) {
+        b[buf][0 + kw] = b0[b_lane + col + kw];
+        b[buf][3 + kw] = b1[b_lane + col + kw];
+        b[buf][6 + kw] = b2[b_lane + col + kw];
+      }
+    };
+    auto step = [&](int cur, uint32_t next_ks) {
+      read_operands(cur ^ 1, next_ks);
+#pragma unroll
+      for (int tap = 0; tap < 9; ++tap)
+        acc[tap] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[cur], b[cur][tap], acc[tap], 0, 0, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // the A read
+#pragma unroll
+      for (int tap = 0; tap < 9; ++tap) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    read_operands(0, 0);
+    const uint32_t last = 2u * npairs - 1u;
+    for (uint32_t kp = 0; kp < npairs; ++kp) {
+      step(0, 2u * kp + 1u);
+      step(1, min(2u * kp + 2u, last));  // the final prefetch is not used; keep it in range
+    }
+  };
+
+  // prologue: slab rows r0, r0+1, r0+2 -> slots 0,1,2 and dy row r0 -> slot 0
+  stage_x_row(xs0, r0);
+  stage_x_row(xs1, r0 + 1u);
+  stage_x_row(xs2, r0 + 2u);
+  stage_dy_row(dys0, r0);
+  __syncthreads();
+
+  // four rows per trip: each phase names its ring slots statically
+  for (uint32_t r = r0;;) {
+    if (r + 1u < r1) { stage_x_row(xs3, r + 3u); stage_dy_row(dys1, r + 1u); }
+    __builtin_amdgcn_sched_barrier(0);
+    compute_row(dys0, xs0, xs1, xs2);
+    __syncthreads();
+    if (++r == r1) break;
+    if (r + 1u < r1) { stage_x_row(xs0, r + 3u); stage_dy_row(dys0, r + 1u); }
+    __builtin_amdgcn_sched_barrier(0);
+    compute_row(dys1, xs1, xs2, xs3);
+    __syncthreads();
+    if (++r == r1) break;
+    if (r + 1u < r1) { stage_x_row(xs1, r + 3u); stage_dy_row(dys1, r + 1u); }
+    __builtin_amdgcn_sched_barrier(0);
+    compute_row(dys0, xs2, xs3, xs0);
+    __syncthreads();
+    if (++r == r1) break;
+    if (r + 1u < r1) { stage_x_row(xs2, r + 3u); stage_dy_row(dys0, r + 1u); }
+    __builtin_amdgcn_sched_barrier(0);
+    compute_row(dys1, xs3, xs0, xs1);
+    __syncthreads();
+    if (++r == r1) break;
+  }
+
+  // ---- epilogue: lane holds D[co = 4g+i][ci = l16] of each tap tile ----
+  const uint32_t block_lin = blockIdx.y * gridDim.x + blockIdx.x;
+  float *__restrict__ part = P.partial + (uint64_t)block_lin * kPartialFloats;
+#pragma unroll
+  for (int tap = 0; tap < 9; ++tap)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t co_l = 16u * ot + 4u * g + i, ci_l = 16u * ct + l16;
+      part[(co_l * 64u + ci_l) * 9u + tap] = acc[tap][i];
+    }
 }
 
-// dw[co][ci][tap] = beta*dw + sum over the pixel-chunk partials of its (co,ci) group, in
-// block order (deterministic).
+// dw[co][ci][tap] = beta*dw + sum over the pixel-chunk partials of its (co half, ci group), in
+// a fixed order (deterministic): 4 lanes-groups each sum a quarter of the partials, then the
+// quarters are combined through LDS in index order.
 struct WgradReduceParams {
   const float *partial;
   float *dw;
-  uint32_t Cin, Cout, blocks_x, ci_groups;
+  uint32_t Cin, Cout, blocks_x, ci_groups, total;
   float beta;
   FastDiv div9, div_cin;
 };
 
 __global__ __launch_bounds__(256) void conv3x3_wgrad_reduce_kernel(const WgradReduceParams P) {
-  const uint32_t e = blockIdx.x * 256u + threadIdx.x;
-  if (e >= P.Cout * P.Cin * 9u) return;
-  uint32_t cc, tap, co, ci;
-  P.div9.divmod(e, cc, tap);
-  P.div_cin.divmod(cc, co, ci);
-  const uint32_t grp = (co >> 6) * P.ci_groups + (ci >> 6);
-  const uint32_t local = (((co & 63u) * 64u) + (ci & 63u)) * 9u + tap;
-  const float *p = P.partial + ((uint64_t)grp * P.blocks_x) * (64u * 64u * 9u) + local;
-  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-  uint32_t b = 0;
-  for (; b + 4 <= P.blocks_x; b += 4) {
-    s0 += p[(uint64_t)(b + 0) * 36864u];
-    s1 += p[(uint64_t)(b + 1) * 36864u];
-    s2 += p[(uint64_t)(b + 2) * 36864u];
-    s3 += p[(uint64_t)(b + 3) * 36864u];
+  __shared__ float part[4][64];
+  const uint32_t q = threadIdx.x >> 6, j = threadIdx.x & 63u;
+  const uint32_t e = blockIdx.x * 64u + j;
+  float s = 0.f;
+  if (e < P.total) {
+    uint32_t cc, tap, co, ci;
+    P.div9.divmod(e, cc, tap);
+    P.div_cin.divmod(cc, co, ci);
+    const uint32_t grp = (co >> 5) * P.ci_groups + (ci >> 6);
+    const uint32_t local = (((co & 31u) * 64u) + (ci & 63u)) * 9u + tap;
+    const float *p = P.partial + ((uint64_t)grp * P.blocks_x) * kPartialFloats + local;
+    const uint32_t per = (P.blocks_x + 3u) / 4u;
+    const uint32_t b0 = q * per, b1 = min(b0 + per, P.blocks_x);
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    uint32_t b = b0;
+    for (; b + 4u <= b1; b += 4u) {
+      s0 += p[(uint64_t)(b + 0u) * kPartialFloats];
+      s1 += p[(uint64_t)(b + 1u) * kPartialFloats];
+      s2 += p[(uint64_t)(b + 2u) * kPartialFloats];
+      s3 += p[(uint64_t)(b + 3u) * kPartialFloats];
+    }
+    for (; b < b1; ++b) s0 += p[(uint64_t)b * kPartialFloats];
+    s = (s0 + s1) + (s2 + s3);
   }
-  for (; b < P.blocks_x; ++b) s0 += p[(uint64_t)b * 36864u];
-  float s = (s0 + s1) + (s2 + s3);
-  if (P.beta != 0.f) s += P.beta * P.dw[e];
-  P.dw[e] = s;
+  part[q][j] = s;
+  __syncthreads();
+  if (q == 0 && e < P.total) {
+    float r = (part[0][j] + part[1][j]) + (part[2][j] + part[3][j]);
+    if (P.beta != 0.f) r += P.beta * P.dw[e];
+    P.dw[e] = r;
+  }
 }
 
 struct WgradPlan {
@@ -203,18 +255,20 @@ static bool wgrad_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Co
                        WgradPlan *plan) {
   if (W > (uint32_t)kMaxW) return false;
   const uint64_t planes = (uint64_t)num_tiles * N;
-  const uint32_t groups = ((Cin + 63u) / 64u) * ((Cout + 63u) / 64u);
+  const uint32_t groups = ((Cin + 63u) / 64u) * ((Cout + 31u) / 32u);
   // aim at >= 256 workgroups (one per CU) with as few partial blocks as that allows
   uint32_t chunks = 1;
   while (planes * chunks * groups < 256 && chunks < H) ++chunks;
   uint32_t rows = (H + chunks - 1) / chunks;
   chunks = (H + rows - 1) / rows;
   if (planes * chunks > 0x7fffffffull) return false;
+  // one image of x / dy is addressed through a 32-bit buffer resource
+  if ((uint64_t)Cin * (H + 2) * (W + 2) * 4u >= (1ull << 31) || (uint64_t)Cout * H * W * 4u >= (1ull << 31)) return false;
   plan->rows_per_block = rows;
   plan->chunks_per_plane = chunks;
   plan->blocks_x = (uint32_t)(planes * chunks);
   plan->groups = groups;
-  plan->workspace_bytes = (size_t)plan->blocks_x * groups * 36864u * sizeof(float);
+  plan->workspace_bytes = (size_t)plan->blocks_x * groups * kPartialFloats * sizeof(float);
   return true;
 }
 
@@ -251,6 +305,7 @@ int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N,
     return ADH_OK;
   }
   if (!x_pad_tiles || !dy_tiles) return ADH_ENULL;
+  if ((uint64_t)Cin * Cout * 9u >= (1ull << 31)) return ADH_EINVAL;
   WgradPlan plan;
   if (!wgrad_plan(num_tiles, N, Cin, Cout, H, W, &plan)) return ADH_EUNIMPL;
   if (!workspace) return ADH_ENULL;
@@ -279,9 +334,9 @@ int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N,
   WgradReduceParams R = {};
   R.partial = P.partial; R.dw = dw; R.Cin = Cin; R.Cout = Cout;
   R.blocks_x = plan.blocks_x; R.ci_groups = P.ci_groups; R.beta = beta;
+  R.total = Cin * Cout * 9u;
   R.div9 = FastDiv(9); R.div_cin = FastDiv(Cin);
-  const uint32_t total = Cin * Cout * 9u;
-  hipLaunchKernelGGL(conv3x3_wgrad_reduce_kernel, dim3((total + 255u) / 256u), dim3(256), 0, st, R);
+  hipLaunchKernelGGL(conv3x3_wgrad_reduce_kernel, dim3((R.total + 63u) / 64u), dim3(256), 0, st, R);
   return launch_status();
 }
 
