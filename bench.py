@@ -24,6 +24,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# HBM bytes per conv-forward launch on cfg2 measured with rocprofv3 PMC (FETCH_SIZE x 2.000 +
+# WRITE_SIZE x 1.000, factors from a 1 GiB plain copy); the summary with the commands is
+# profiles/conv3x3_fwd_cfg2_hbm_traffic.txt.  Not re-measured by this script.
+CONV_FWD_CFG2_TRAFFIC_BYTES = 64.07e6
 HBM_PEAK_GBS = 8000.0
 MFMA_F32_PEAK_TFLOPS = 157.3
 METRIC = "halo pack/unpack GB/s (% HBM peak); 3x3 slab-conv TFLOP/s (% MFMA peak)"
@@ -53,6 +57,9 @@ def main():
                     help="untimed steps; a few hundred so that the GPU clocks have ramped up")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-secondary", action="store_true", help="time only the headline kernel")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain copy of known size (1 GiB read + 1 GiB written) 10 times: the kernel "
+                         "whose FETCH_SIZE / WRITE_SIZE readings calibrate the HBM traffic counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (the K row-tiles live in one HBM, there are no "
@@ -127,8 +134,19 @@ def main():
                    "flops_per_step": flops_step, "tiles": K, "halo": p},
         "roofline": {"kernel": "conv3x3_f32_kernel<25,8,false> (fwd)", "bound": "mfma", "achieved": round(achieved, 3),
                      "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / MFMA_F32_PEAK_TFLOPS, 4),
-                     "traffic": None, "launch_ms": round(kernel_ms, 5)},
+                     "traffic": CONV_FWD_CFG2_TRAFFIC_BYTES, "launch_ms": round(kernel_ms, 5)},
     }
+
+    if args.copy_calibration:
+        cw, chh, cc, cn = 1024, 1024, 64, 4  # 2^28 floats = 1 GiB each way, rows contiguous
+        src = torch.ones((cn, cc, chh, cw), device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            capi.check(lib.adh_slice_copy_nchw(0, cw, chh, cc, cn, src.data_ptr(), cw, chh, cc, 0, 0, 0, dst.data_ptr(),
+                                               cw, chh, cc, 0, 0, 0, stream), "copy calibration")
+        torch.cuda.synchronize()
+        out["copy_calibration_bytes_each_way"] = cw * chh * cc * cn * 4
+        del src, dst
 
     # ---- secondary kernels of the path ----
     if not args.no_secondary:
