@@ -55,7 +55,10 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
 
 // TAIL = (W % EPT != 0): the last vector of a row is partial and is moved element-wise.
-template <typename T, bool ADD, bool ZERO_BORDER, bool TAIL, int VPT>
+// STREAM = the transfer is larger than the on-package cache: loads and stores are marked
+// non-temporal so that lines are not kept (a few percent more bandwidth from HBM, but a loss
+// when the data would have stayed cache-resident, so the host decides by size).
+template <typename T, bool ADD, bool ZERO_BORDER, bool TAIL, bool STREAM, int VPT>
 __global__ __launch_bounds__(kBlock) void row_copy_kernel(const RowCopyParams P) {
   constexpr int EPT = 16 / sizeof(T);
   typedef u32x4_unaligned VU;
@@ -97,7 +100,8 @@ __global__ __launch_bounds__(kBlock) void row_copy_kernel(const RowCopyParams P)
     // addresses are valid even for idle threads and zero rows (clamped above), so the
     // vector loads need no branch when rows have no tail
     if (!TAIL || cnt[k] == (uint32_t)EPT) {
-      in[k] = *reinterpret_cast<const VU *>(sbase + so[k]);
+      in[k] = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const VU *>(sbase + so[k]))
+                     : *reinterpret_cast<const VU *>(sbase + so[k]);
       if (ADD) old[k] = *reinterpret_cast<const VU *>(dbase + dof[k]);
     } else if (TAIL && cnt[k] > 0) {
       Pack pi, po;
@@ -138,7 +142,8 @@ __global__ __launch_bounds__(kBlock) void row_copy_kernel(const RowCopyParams P)
     }
     T *d = dbase + dof[k];
     if (!TAIL || cnt[k] == (uint32_t)EPT) {
-      *reinterpret_cast<VU *>(d) = out.v;
+      if (STREAM) __builtin_nontemporal_store(out.v, reinterpret_cast<VU *>(d));
+      else *reinterpret_cast<VU *>(d) = out.v;
     } else {
 #pragma unroll
       for (int i = 0; i < EPT - 1; ++i)
@@ -152,11 +157,11 @@ __global__ __launch_bounds__(kBlock) void row_copy_kernel(const RowCopyParams P)
   }
 }
 
-template <typename T>
+template <typename T, bool STREAM>
 static void launch_row_copy_t(bool add, bool zero_border, bool tail, const RowCopyParams &P, dim3 grid,
                               hipStream_t st) {
   constexpr int VPT = 2;
-#define ADH_RC(A, Z, TL) hipLaunchKernelGGL((row_copy_kernel<T, A, Z, TL, VPT>), grid, dim3(kBlock), 0, st, P)
+#define ADH_RC(A, Z, TL) hipLaunchKernelGGL((row_copy_kernel<T, A, Z, TL, STREAM, VPT>), grid, dim3(kBlock), 0, st, P)
   if (add) { if (tail) ADH_RC(true, false, true); else ADH_RC(true, false, false); }
   else if (zero_border) { if (tail) ADH_RC(false, true, true); else ADH_RC(false, true, false); }
   else { if (tail) ADH_RC(false, false, true); else ADH_RC(false, false, false); }
@@ -177,8 +182,17 @@ static int launch_row_copy(int dtype, bool add, bool zero_border, RowCopyParams 
   P.div_C = FastDiv(P.C);
   const bool tail = P.W % ept != 0;
   dim3 grid((P.total_vectors + kBlock * 2 - 1) / (kBlock * 2), n_dst, 1);
-  if (dtype == ADH_F32) launch_row_copy_t<float>(add, zero_border, tail, P, grid, st);
-  else launch_row_copy_t<uint16_t>(add, zero_border, tail, P, grid, st);
+  // bytes read + written by the launch; above half of the 256 MB on-package cache nothing
+  // would stay resident anyway
+  const uint64_t moved = 2ull * P.W * P.DH * P.C * N * n_dst * dtype_size(dtype);
+  const bool stream = moved > (128ull << 20);
+  if (dtype == ADH_F32) {
+    if (stream) launch_row_copy_t<float, true>(add, zero_border, tail, P, grid, st);
+    else launch_row_copy_t<float, false>(add, zero_border, tail, P, grid, st);
+  } else {
+    if (stream) launch_row_copy_t<uint16_t, true>(add, zero_border, tail, P, grid, st);
+    else launch_row_copy_t<uint16_t, false>(add, zero_border, tail, P, grid, st);
+  }
   return launch_status();
 }
 
