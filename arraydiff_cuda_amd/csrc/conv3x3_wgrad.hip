@@ -38,9 +38,11 @@ struct WgradParams {
   const float *dy[ADH_MAX_TILES];
   float *partial;            // [grid.y][grid.x][32*64*9] in (co, ci, tap) order, local to the group
   uint32_t num_tiles, N, Cin, Cout, H, W;
-  uint32_t rows_per_block, chunks_per_plane;  // grid.x = chunks_per_plane * N * num_tiles
+  uint32_t rows_per_block, chunks_per_plane;  // row chunks of a plane
+  uint32_t cols_per_block, col_tiles;         // column tiles of a plane (<= kMaxW columns each)
+  // grid.x = col_tiles * chunks_per_plane * N * num_tiles
   uint32_t ci_groups;        // grid.y = co_halves * ci_groups, co_halves = ceil(Cout/32)
-  FastDiv div_chunks, div_tiles, div_ci_groups;
+  FastDiv div_chunks, div_tiles, div_ci_groups, div_cols;
 };
 
 __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const WgradParams P) {
@@ -57,8 +59,9 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
   const uint32_t ot = wv & 1u;   // co tile inside the 32-channel half
   const uint32_t ct = wv >> 1;   // ci tile
 
-  uint32_t plane, chunk;
-  P.div_chunks.divmod(blockIdx.x, plane, chunk);
+  uint32_t rest, ctile, plane, chunk;
+  P.div_cols.divmod(blockIdx.x, rest, ctile);
+  P.div_chunks.divmod(rest, plane, chunk);
   uint32_t n, t;
   P.div_tiles.divmod(plane, n, t);
   uint32_t coh, cig;
@@ -83,8 +86,10 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(x), 0, (int)(P.Cin * HP * WP * 4u), kWgBufferFlags);
   const __amdgpu_buffer_rsrc_t rsrc_dy =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(dy), 0, (int)(P.Cout * P.H * P.W * 4u), kWgBufferFlags);
-  const uint32_t x_voff = lane < WP ? lane * 4u : kWgOutOfRange;
-  const uint32_t d_voff = lane < P.W ? lane * 4u : kWgOutOfRange;
+  const uint32_t w0 = ctile * P.cols_per_block;
+  const uint32_t tw = min(P.cols_per_block, P.W - w0);  // columns of this workgroup
+  const uint32_t x_voff = lane < tw + 2u ? (w0 + lane) * 4u : kWgOutOfRange;
+  const uint32_t d_voff = lane < tw ? (w0 + lane) * 4u : kWgOutOfRange;
   const bool ragged_c = (ci0 + 64u > P.Cin) || (co0 + 32u > P.Cout);  // uniform
   auto stage_x_row = [&](float *slot, uint32_t y) {  // slab row y of the 64 input channels
 #pragma unroll
@@ -119,7 +124,7 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
 #pragma unroll
   for (int tap = 0; tap < 9; ++tap) acc[tap] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const uint32_t ksteps = (P.W + 3u) / 4u;
+  const uint32_t ksteps = (tw + 3u) / 4u;
   const uint32_t npairs = (ksteps + 1u) / 2u;   // an odd tail k-step multiplies the zero columns
   const uint32_t a_lane = (16u * ot + l16) * kRowPitch + g;
   const uint32_t b_lane = (16u * ct + l16) * kRowPitch + g;
@@ -247,26 +252,43 @@ __global__ __launch_bounds__(256) void conv3x3_wgrad_reduce_kernel(const WgradRe
 }
 
 struct WgradPlan {
-  uint32_t rows_per_block, chunks_per_plane, blocks_x, groups;
+  uint32_t rows_per_block, chunks_per_plane, cols_per_block, col_tiles, blocks_x, groups;
   size_t workspace_bytes;
 };
 
 static bool wgrad_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
                        WgradPlan *plan) {
-  if (W > (uint32_t)kMaxW) return false;
   const uint64_t planes = (uint64_t)num_tiles * N;
   const uint32_t groups = ((Cin + 63u) / 64u) * ((Cout + 31u) / 32u);
-  // aim at >= 256 workgroups (one per CU) with as few partial blocks as that allows
-  uint32_t chunks = 1;
-  while (planes * chunks * groups < 256 && chunks < H) ++chunks;
-  uint32_t rows = (H + chunks - 1) / chunks;
-  chunks = (H + rows - 1) / rows;
-  if (planes * chunks > 0x7fffffffull) return false;
+  const uint32_t col_tiles = (W + kMaxW - 1) / kMaxW;
+  const uint32_t cols = (W + col_tiles - 1) / col_tiles;
+  // Row chunks per plane: a workgroup's time grows with its rows, 256 CUs run one workgroup each
+  // per round, and every workgroup costs one partial block to write and reduce (priced here as
+  // two rows of work).  Pick the chunk count with the least modelled time.
+  const uint64_t per_chunk = planes * col_tiles * groups;
+  uint32_t best_chunks = 1;
+  double best_cost = 1e300;
+  for (uint32_t chunks = 1; chunks <= H; ++chunks) {
+    const uint32_t rows = (H + chunks - 1) / chunks;
+    if ((H + rows - 1) / rows != chunks) continue;  // same row count as a smaller chunk number
+    const uint64_t blocks = per_chunk * chunks;
+    const double cost = (double)((blocks + 255) / 256) * (rows + 2.0);
+    if (cost < best_cost) {
+      best_cost = cost;
+      best_chunks = chunks;
+    }
+    if (blocks >= 4096) break;
+  }
+  const uint32_t rows = (H + best_chunks - 1) / best_chunks;
+  const uint64_t blocks_x = planes * best_chunks * col_tiles;
+  if (blocks_x > 0x7fffffffull) return false;
   // one image of x / dy is addressed through a 32-bit buffer resource
   if ((uint64_t)Cin * (H + 2) * (W + 2) * 4u >= (1ull << 31) || (uint64_t)Cout * H * W * 4u >= (1ull << 31)) return false;
   plan->rows_per_block = rows;
-  plan->chunks_per_plane = chunks;
-  plan->blocks_x = (uint32_t)(planes * chunks);
+  plan->chunks_per_plane = best_chunks;
+  plan->cols_per_block = cols;
+  plan->col_tiles = col_tiles;
+  plan->blocks_x = (uint32_t)blocks_x;
   plan->groups = groups;
   plan->workspace_bytes = (size_t)plan->blocks_x * groups * kPartialFloats * sizeof(float);
   return true;
@@ -322,6 +344,9 @@ int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N,
   P.num_tiles = num_tiles; P.N = N; P.Cin = Cin; P.Cout = Cout; P.H = H; P.W = W;
   P.rows_per_block = plan.rows_per_block;
   P.chunks_per_plane = plan.chunks_per_plane;
+  P.cols_per_block = plan.cols_per_block;
+  P.col_tiles = plan.col_tiles;
+  P.div_cols = FastDiv(plan.col_tiles);
   P.ci_groups = (Cin + 63u) / 64u;
   P.div_chunks = FastDiv(plan.chunks_per_plane);
   P.div_tiles = FastDiv(num_tiles);
