@@ -354,6 +354,10 @@ static void launch_conv(const ConvParams &P, dim3 grid, hipStream_t st) {
     hipLaunchKernelGGL((conv3x3_f32_kernel<NT, WAVES, false>), grid, dim3(64 * WAVES), 0, st, P);
 }
 
+int conv_bf16_via_f32(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                      const void *const *in_tiles, const void *w, void *const *out_tiles, float beta, void *workspace,
+                      size_t workspace_bytes, hipStream_t st);
+
 // which: ADH_CONV_FWD or ADH_CONV_BWD_DATA.  H, W are the interior extents.
 static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                        uint32_t W, const void *const *in_tiles, const void *w, void *const *out_tiles, float beta,
@@ -420,7 +424,9 @@ extern "C" {
 int adh_conv3x3_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                                uint32_t W, const void *const *x_pad_tiles, const void *w, void *const *y_tiles,
                                float beta, void *workspace, size_t workspace_bytes, void *stream) {
-  (void)workspace; (void)workspace_bytes;
+  if (dtype == ADH_BF16)
+    return conv_bf16_via_f32(ADH_CONV_FWD, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, w, y_tiles, beta, workspace,
+                             workspace_bytes, as_stream(stream));
   return conv_direct(ADH_CONV_FWD, dtype, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, w, y_tiles, beta,
                      as_stream(stream));
 }
@@ -437,7 +443,9 @@ int adh_conv3x3_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, u
                                     uint32_t H, uint32_t W, const void *w, const void *const *dy_tiles,
                                     void *const *dx_pad_tiles, float beta, void *workspace, size_t workspace_bytes,
                                     void *stream) {
-  (void)workspace; (void)workspace_bytes;
+  if (dtype == ADH_BF16)
+    return conv_bf16_via_f32(ADH_CONV_BWD_DATA, num_tiles, N, Cin, Cout, H, W, dy_tiles, w, dx_pad_tiles, beta,
+                             workspace, workspace_bytes, as_stream(stream));
   return conv_direct(ADH_CONV_BWD_DATA, dtype, num_tiles, N, Cin, Cout, H, W, dy_tiles, w, dx_pad_tiles, beta,
                      as_stream(stream));
 }

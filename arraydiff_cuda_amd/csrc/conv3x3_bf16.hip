@@ -1,0 +1,176 @@
+// bf16 entry of the 3x3 slab convolution: bf16 tensors in HBM, fp32 accumulation.
+//
+// Current implementation: the bf16 slabs, filter and (for beta = 1) outputs are widened to fp32
+// in the caller's workspace, the fp32 MFMA kernels run on the copies, and the result is rounded
+// back to bf16 (round to nearest even).  Every product is therefore exact and every sum is in
+// fp32, i.e. the arithmetic of a bf16-input / fp32-accumulate matrix core, at the speed of the
+// fp32 path plus three streaming passes.  The filter gradient stays fp32.
+#include "adh_common.h"
+
+namespace adh {
+
+__global__ __launch_bounds__(256) void widen_bf16_kernel(uint64_t n, const uint16_t *__restrict__ src,
+                                                        float *__restrict__ dst) {
+  const uint64_t stride = (uint64_t)gridDim.x * 256u * 8u;
+  for (uint64_t i = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * 8u; i < n; i += stride) {
+    if (i + 8u <= n) {
+      typedef uint4 U4 __attribute__((aligned(2)));
+      const uint4 v = *reinterpret_cast<const U4 *>(src + i);
+      float4 lo, hi;
+      lo.x = __uint_as_float(v.x << 16); lo.y = __uint_as_float(v.x & 0xffff0000u);
+      lo.z = __uint_as_float(v.y << 16); lo.w = __uint_as_float(v.y & 0xffff0000u);
+      hi.x = __uint_as_float(v.z << 16); hi.y = __uint_as_float(v.z & 0xffff0000u);
+      hi.z = __uint_as_float(v.w << 16); hi.w = __uint_as_float(v.w & 0xffff0000u);
+      *reinterpret_cast<float4 *>(dst + i) = lo;
+      *reinterpret_cast<float4 *>(dst + i + 4) = hi;
+    } else {
+      for (uint64_t j = i; j < n; ++j) dst[j] = bf16_bits_to_f32(src[j]);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void narrow_bf16_kernel(uint64_t n, const float *__restrict__ src,
+                                                         uint16_t *__restrict__ dst) {
+  const uint64_t stride = (uint64_t)gridDim.x * 256u * 8u;
+  for (uint64_t i = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * 8u; i < n; i += stride) {
+    if (i + 8u <= n) {
+      const float4 lo = *reinterpret_cast<const float4 *>(src + i);
+      const float4 hi = *reinterpret_cast<const float4 *>(src + i + 4);
+      uint4 v;
+      v.x = (uint32_t)f32_to_bf16_bits(lo.x) | ((uint32_t)f32_to_bf16_bits(lo.y) << 16);
+      v.y = (uint32_t)f32_to_bf16_bits(lo.z) | ((uint32_t)f32_to_bf16_bits(lo.w) << 16);
+      v.z = (uint32_t)f32_to_bf16_bits(hi.x) | ((uint32_t)f32_to_bf16_bits(hi.y) << 16);
+      v.w = (uint32_t)f32_to_bf16_bits(hi.z) | ((uint32_t)f32_to_bf16_bits(hi.w) << 16);
+      typedef uint4 U4 __attribute__((aligned(2)));
+      *reinterpret_cast<U4 *>(dst + i) = v;
+    } else {
+      for (uint64_t j = i; j < n; ++j) dst[j] = f32_to_bf16_bits(src[j]);
+    }
+  }
+}
+
+static uint32_t cvt_grid(uint64_t n) {
+  uint64_t b = (n + 2047) / 2048;
+  if (b > 256ull * 32) b = 256ull * 32;
+  return (uint32_t)(b ? b : 1);
+}
+
+// fp32 scratch copies live in 256-byte aligned consecutive regions of the workspace
+static size_t region(uint64_t elems) { return (size_t)((elems * 4u + 255u) / 256u * 256u); }
+
+size_t bf16_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                            uint32_t W, size_t fp32_path_bytes) {
+  const uint64_t slab = (uint64_t)N * Cin * (H + 2) * (W + 2), out = (uint64_t)N * Cout * H * W;
+  const uint64_t filt = (uint64_t)Cin * Cout * 9u;
+  size_t total = 0;
+  if (which == ADH_CONV_BWD_FILTER) total = num_tiles * (region(slab) + region(out));
+  else total = num_tiles * (region(slab) + region(out)) + region(filt);
+  return total + (fp32_path_bytes + 255u) / 256u * 256u;
+}
+
+}  // namespace adh
+
+using namespace adh;
+
+// fp32 kernels of the other translation units
+extern "C" size_t adh_conv3x3_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,
+                                              uint32_t Cout, uint32_t H, uint32_t W);
+
+namespace adh {
+
+static int widen(uint64_t n, const void *src, float *dst, hipStream_t st) {
+  hipLaunchKernelGGL(widen_bf16_kernel, dim3(cvt_grid(n)), dim3(256), 0, st, n, reinterpret_cast<const uint16_t *>(src), dst);
+  return launch_status();
+}
+static int narrow(uint64_t n, const float *src, void *dst, hipStream_t st) {
+  hipLaunchKernelGGL(narrow_bf16_kernel, dim3(cvt_grid(n)), dim3(256), 0, st, n, src, reinterpret_cast<uint16_t *>(dst));
+  return launch_status();
+}
+
+// which = ADH_CONV_FWD: in = x_pad tiles (slab sized), out = y tiles; ADH_CONV_BWD_DATA: in = dy
+// tiles, out = dx_pad tiles.  Called by the dispatchers in conv3x3.hip for dtype == ADH_BF16.
+int conv_bf16_via_f32(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                      const void *const *in_tiles, const void *w, void *const *out_tiles, float beta, void *workspace,
+                      size_t workspace_bytes, hipStream_t st) {
+  if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
+  if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
+  if (N == 0 || Cin == 0 || Cout == 0 || H == 0 || W == 0) return ADH_OK;
+  if (!in_tiles || !out_tiles || !w) return ADH_ENULL;
+  if (!aligned_to(w, 2)) return ADH_EALIGN;
+  const size_t need = bf16_workspace_bytes(which, num_tiles, N, Cin, Cout, H, W, 0);
+  if (!workspace) return ADH_ENULL;
+  if (!aligned_to(workspace, 256)) return ADH_EALIGN;
+  if (workspace_bytes < need) return ADH_EWORKSPACE;
+  const uint64_t slab = (uint64_t)N * Cin * (H + 2) * (W + 2), outn = (uint64_t)N * Cout * H * W;
+  const uint64_t in_elems = which == ADH_CONV_FWD ? slab : outn;
+  const uint64_t out_elems = which == ADH_CONV_FWD ? outn : slab;
+  char *ws = reinterpret_cast<char *>(workspace);
+  const void *in32[ADH_MAX_TILES];
+  void *out32[ADH_MAX_TILES];
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!in_tiles[t] || !out_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(in_tiles[t], 2) || !aligned_to(out_tiles[t], 2)) return ADH_EALIGN;
+  }
+  float *w32 = reinterpret_cast<float *>(ws);
+  ws += region((uint64_t)Cin * Cout * 9u);
+  int e = widen((uint64_t)Cin * Cout * 9u, w, w32, st);
+  if (e) return e;
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    float *i32 = reinterpret_cast<float *>(ws);
+    ws += region(in_elems);
+    float *o32 = reinterpret_cast<float *>(ws);
+    ws += region(out_elems);
+    if ((e = widen(in_elems, in_tiles[t], i32, st))) return e;
+    if (beta != 0.f && (e = widen(out_elems, out_tiles[t], o32, st))) return e;
+    in32[t] = i32;
+    out32[t] = o32;
+  }
+  if (which == ADH_CONV_FWD)
+    e = adh_conv3x3_slab_fwd_tiles(ADH_F32, num_tiles, N, Cin, Cout, H, W, in32, w32, out32, beta, nullptr, 0, st);
+  else
+    e = adh_conv3x3_slab_bwd_data_tiles(ADH_F32, num_tiles, N, Cin, Cout, H, W, w32, in32, out32, beta, nullptr, 0, st);
+  if (e) return e;
+  for (uint32_t t = 0; t < num_tiles; ++t)
+    if ((e = narrow(out_elems, reinterpret_cast<const float *>(out32[t]), out_tiles[t], st))) return e;
+  return ADH_OK;
+}
+
+int conv_bf16_filter_via_f32(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                             const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta,
+                             void *workspace, size_t workspace_bytes, hipStream_t st) {
+  if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
+  if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
+  if (Cin == 0 || Cout == 0) return ADH_OK;
+  if (!dw) return ADH_ENULL;
+  if (N == 0 || H == 0 || W == 0)
+    return adh_conv3x3_slab_bwd_filter_tiles(ADH_F32, num_tiles, N, Cin, Cout, H, W, x_tiles, dy_tiles, dw, beta,
+                                             workspace, workspace_bytes, st);
+  if (!x_tiles || !dy_tiles) return ADH_ENULL;
+  const size_t f32_bytes = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, num_tiles, N, Cin, Cout, H, W);
+  if (f32_bytes == 0) return ADH_EUNIMPL;
+  const size_t need = bf16_workspace_bytes(ADH_CONV_BWD_FILTER, num_tiles, N, Cin, Cout, H, W, f32_bytes);
+  if (!workspace) return ADH_ENULL;
+  if (!aligned_to(workspace, 256)) return ADH_EALIGN;
+  if (workspace_bytes < need) return ADH_EWORKSPACE;
+  const uint64_t slab = (uint64_t)N * Cin * (H + 2) * (W + 2), outn = (uint64_t)N * Cout * H * W;
+  char *ws = reinterpret_cast<char *>(workspace);
+  const void *x32[ADH_MAX_TILES];
+  const void *dy32[ADH_MAX_TILES];
+  int e;
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!x_tiles[t] || !dy_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(x_tiles[t], 2) || !aligned_to(dy_tiles[t], 2)) return ADH_EALIGN;
+    float *a = reinterpret_cast<float *>(ws);
+    ws += region(slab);
+    float *b = reinterpret_cast<float *>(ws);
+    ws += region(outn);
+    if ((e = widen(slab, x_tiles[t], a, st))) return e;
+    if ((e = widen(outn, dy_tiles[t], b, st))) return e;
+    x32[t] = a;
+    dy32[t] = b;
+  }
+  return adh_conv3x3_slab_bwd_filter_tiles(ADH_F32, num_tiles, N, Cin, Cout, H, W, x32, dy32, dw, beta, ws,
+                                           workspace_bytes - (size_t)(ws - reinterpret_cast<char *>(workspace)), st);
+}
+
+}  // namespace adh

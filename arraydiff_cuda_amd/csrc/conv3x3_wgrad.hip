@@ -294,6 +294,12 @@ static bool wgrad_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Co
   return true;
 }
 
+size_t bf16_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                            uint32_t W, size_t fp32_path_bytes);
+int conv_bf16_filter_via_f32(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                             const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta,
+                             void *workspace, size_t workspace_bytes, hipStream_t st);
+
 }  // namespace adh
 
 using namespace adh;
@@ -302,11 +308,15 @@ extern "C" {
 
 size_t adh_conv3x3_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
                                    uint32_t H, uint32_t W) {
-  if (which != ADH_CONV_BWD_FILTER || dtype != ADH_F32) return 0;
   if (num_tiles == 0 || N == 0 || Cin == 0 || Cout == 0 || H == 0 || W == 0) return 0;
-  WgradPlan plan;
-  if (!wgrad_plan(num_tiles, N, Cin, Cout, H, W, &plan)) return 0;
-  return plan.workspace_bytes;
+  size_t f32_bytes = 0;
+  if (which == ADH_CONV_BWD_FILTER) {
+    WgradPlan plan;
+    if (!wgrad_plan(num_tiles, N, Cin, Cout, H, W, &plan)) return 0;
+    f32_bytes = plan.workspace_bytes;
+  }
+  if (dtype == ADH_BF16) return bf16_workspace_bytes(which, num_tiles, N, Cin, Cout, H, W, f32_bytes);
+  return dtype == ADH_F32 ? f32_bytes : 0;
 }
 
 int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
@@ -314,7 +324,9 @@ int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N,
                                       const void *const *dy_tiles, float *dw, float beta, void *workspace,
                                       size_t workspace_bytes, void *stream) {
   if (!dtype_ok(dtype)) return ADH_EINVAL;
-  if (dtype != ADH_F32) return ADH_EUNIMPL;
+  if (dtype == ADH_BF16)
+    return conv_bf16_filter_via_f32(num_tiles, N, Cin, Cout, H, W, x_pad_tiles, dy_tiles, dw, beta, workspace,
+                                    workspace_bytes, as_stream(stream));
   if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
   if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
   if (Cin == 0 || Cout == 0) return ADH_OK;

@@ -132,7 +132,9 @@ int adh_tiles_unpack_nchw(int dtype, uint32_t K, uint32_t halo_pad, uint32_t W, 
  * (Conv2DShape.halo_padded_input, src/op.cc:1354-1410), filter KCRS (Cout,Cin,3,3),
  * no bias.  beta is 0 (overwrite) or 1 (accumulate), the two values the reference passes.
  * `*_tiles` variants run K slabs of identical shape in one launch.  Workspace may be NULL
- * when the matching *_workspace_bytes query returns 0. */
+ * when the matching *_workspace_bytes query returns 0; otherwise it must be 256-byte aligned.
+ * ADH_BF16: x, w, y, dy, dx are bf16 in memory, sums are fp32, results rounded to nearest even;
+ * dw stays fp32.  The bf16 entry needs a workspace for all three passes. */
 #define ADH_CONV_FWD 0
 #define ADH_CONV_BWD_DATA 1
 #define ADH_CONV_BWD_FILTER 2

@@ -42,7 +42,8 @@ def test_argument_errors_need_no_gpu():
     assert l.adh_tiles_pack_nchw(0, 17, 1, 4, 34, 1, 1, bogus, tb4, None) == capi.ADH_EINVAL        # > 16 tiles
     assert l.adh_slice_copy_nchw(0, 5, 1, 1, 1, bogus, 4, 4, 1, 0, 0, 0, bogus, 8, 8, 1, 0, 0, 0, None) == capi.ADH_EINVAL
     assert l.adh_conv3x3_slab_fwd(0, 1, 4, 4, 3, 3, bogus, bogus, bogus, 0.5, None, 0, None) == capi.ADH_EINVAL  # beta
-    assert l.adh_conv3x3_slab_fwd(1, 1, 4, 4, 3, 3, bogus, bogus, bogus, 0.0, None, 0, None) == capi.ADH_EUNIMPL  # bf16
+    assert l.adh_conv3x3_slab_fwd(1, 1, 4, 4, 3, 3, bogus, bogus, bogus, 0.0, None, 0, None) == capi.ADH_ENULL  # bf16 needs a workspace
+    assert l.adh_conv3x3_workspace_bytes(capi.ADH_CONV_FWD, 1, 1, 1, 4, 4, 3, 3) > 0
     assert l.adh_conv3x3_slab_fwd(0, 1, 4, 4, 3, 3, None, bogus, bogus, 0.0, None, 0, None) == capi.ADH_ENULL
     assert l.adh_conv3x3_slab_bwd_filter(0, 1, 4, 4, 3, 3, bogus, bogus, bogus, 0.0, bogus, 16, None) == capi.ADH_EWORKSPACE
     assert l.adh_conv3x3_workspace_bytes(capi.ADH_CONV_BWD_FILTER, 0, 4, 32, 64, 64, 14, 56) > 0

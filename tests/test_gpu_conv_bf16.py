@@ -1,0 +1,138 @@
+"""GPU parity of the bf16 slab convolution (bf16 in HBM, fp32 accumulate): rel-err
+max|a-b| / max|b| <= 2e-2 against the oracle fed with the same bf16 values, on small shapes in
+full and at the full high-resolution configuration (N=2, C=64, 1024x2048, 8 row-tiles of 128
+rows, halo 1) by sampling: every tile-boundary row for some channels plus >= 1e5 random outputs,
+each recomputed in float64 from the UNSPLIT tensors.  Every call goes through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from arraydiff_cuda_amd import capi
+from gpu_util import dev, host, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def ws_for(which, K, N, Cin, Cout, H, W):
+    nbytes = capi.conv_workspace_bytes(which, capi.ADH_BF16, K, N, Cin, Cout, H, W)
+    assert nbytes > 0
+    return torch.empty(nbytes // 4 + 64, device="cuda")
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,H,W", [(1, 2, 8, 16, 5, 9), (2, 1, 19, 7, 6, 33), (3, 2, 64, 64, 7, 56)])
+def test_bf16_conv_small_vs_oracle(oracle, K, N, Cin, Cout, H, W):
+    rng = np.random.default_rng(77 + Cin)
+    bf = lambda a: oracle.f32_to_bf16(a.astype(np.float32))
+    xs = [bf(rng.uniform(-1, 1, size=(N, Cin, H + 2, W + 2))) for _ in range(K)]
+    w = bf(rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9)))
+    dys = [bf(rng.standard_normal((N, Cout, H, W))) for _ in range(K)]
+    wf = oracle.bf16_to_f32(w)
+    dw_want = np.zeros((Cout, Cin, 3, 3), np.float32)
+    d_xs, d_dys, d_w = [dev(x) for x in xs], [dev(d) for d in dys], dev(w)
+    ys = [torch.empty((N, Cout, H, W), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
+    gs = [torch.empty((N, Cin, H + 2, W + 2), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
+    capi.check(capi.conv_fwd_tiles(d_xs, d_w, ys, N, Cin, Cout, H, W, ws=ws_for(capi.ADH_CONV_FWD, K, N, Cin, Cout, H, W)))
+    capi.check(capi.conv_bwd_data_tiles(d_w, d_dys, gs, N, Cin, Cout, H, W,
+                                        ws=ws_for(capi.ADH_CONV_BWD_DATA, K, N, Cin, Cout, H, W)))
+    dw = torch.zeros((Cout, Cin, 3, 3), device="cuda")
+    capi.check(capi.conv_bwd_filter_tiles(d_xs, d_dys, dw, N, Cin, Cout, H, W, beta=1.0,
+                                          ws=ws_for(capi.ADH_CONV_BWD_FILTER, K, N, Cin, Cout, H, W)))
+    for r in range(K):
+        xf, dyf = oracle.bf16_to_f32(xs[r]), oracle.bf16_to_f32(dys[r])
+        y = np.empty((N, Cout, H, W), np.float32)
+        oracle.conv_slab_fwd(xf, wf, y)
+        assert rel_err(oracle.bf16_to_f32(host(ys[r])), y) <= TOL
+        g = np.empty((N, Cin, H + 2, W + 2), np.float32)
+        oracle.conv_slab_bwd_data(wf, dyf, g)
+        assert rel_err(oracle.bf16_to_f32(host(gs[r])), g) <= TOL
+        oracle.conv_slab_bwd_filter(xf, dyf, dw_want, beta=1.0)
+    assert rel_err(host(dw), dw_want) <= 1e-4  # fp32 output, exact bf16 products
+    # beta = 1 accumulates onto a bf16 output
+    y2 = [y.clone() for y in ys]
+    capi.check(capi.conv_fwd_tiles(d_xs, d_w, y2, N, Cin, Cout, H, W, beta=1.0,
+                                   ws=ws_for(capi.ADH_CONV_FWD, K, N, Cin, Cout, H, W)))
+    assert rel_err(y2[0].float().cpu().numpy(), 2 * ys[0].float().cpu().numpy()) <= TOL
+    small = torch.empty(16, device="cuda")
+    assert capi.conv_fwd_tiles(d_xs, d_w, ys, N, Cin, Cout, H, W, ws=small) == capi.ADH_EWORKSPACE
+
+
+def test_config5_highres_bf16_fwd_bwd_sampled(oracle):
+    """bf16 N=2, C=64, 1024x2048 in 8 row-tiles of 128 rows + halo 1: pack, conv fwd, bwd-data +
+    halo reduce + unpack, bwd-filter, each checked against the UNSPLIT convolution on samples."""
+    K, N, C, H, W, p = 8, 2, 64, 1024, 2048, 1
+    Ht = H // K
+    g = torch.Generator(device="cuda").manual_seed(0x5EED)
+    X = (torch.rand((N, C, H, W), device="cuda", generator=g) * 2 - 1).to(torch.bfloat16)
+    wt = (torch.randn((C, C, 3, 3), device="cuda", generator=g) * (2.0 / (C * 9)) ** 0.5).to(torch.bfloat16)
+    dY = torch.randn((N, C, H, W), device="cuda", generator=g).to(torch.bfloat16)
+    tiles = [torch.empty((N, C, Ht + 2, W + 2), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
+    capi.check(capi.tiles_pack(K, p, W, H, C, N, X, tiles))
+    ys = [torch.empty((N, C, Ht, W), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
+    ws = ws_for(capi.ADH_CONV_BWD_FILTER, K, N, C, C, Ht, W)
+    assert ws.numel() * 4 >= capi.conv_workspace_bytes(capi.ADH_CONV_FWD, capi.ADH_BF16, K, N, C, C, Ht, W)
+    capi.check(capi.conv_fwd_tiles(tiles, wt, ys, N, C, C, Ht, W, ws=ws))
+    Y = torch.cat(ys, dim=2)
+    dys = [dY[:, :, r * Ht:(r + 1) * Ht].contiguous() for r in range(K)]
+    gs = [torch.empty((N, C, Ht + 2, W + 2), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
+    capi.check(capi.conv_bwd_data_tiles(wt, dys, gs, N, C, C, Ht, W, ws=ws))
+    capi.check(capi.halo_reduce(gs, 1, K, p, W, Ht, C, N))
+    gX = torch.empty_like(X)
+    capi.check(capi.tiles_unpack(K, p, W, H, C, N, gs, gX))
+    gw = torch.zeros((C, C, 3, 3), device="cuda")
+    capi.check(capi.conv_bwd_filter_tiles(tiles, dys, gw, N, C, C, Ht, W, beta=1.0, ws=ws))
+    torch.cuda.synchronize()
+    del ws, tiles, gs
+
+    Xh = np.pad(X.float().cpu().numpy(), ((0, 0), (0, 0), (1, 1), (1, 1)))
+    dYh = np.pad(dY.float().cpu().numpy(), ((0, 0), (0, 0), (1, 1), (1, 1)))
+    wh = wt.float().cpu().numpy().astype(np.float64)
+    Yh = Y.float().cpu().numpy()
+    gXh = gX.float().cpu().numpy()
+    rng = np.random.default_rng(5)
+
+    def sample_coords(count):
+        n = rng.integers(0, N, count)
+        c = rng.integers(0, C, count)
+        h = rng.integers(0, H, count)
+        w_ = rng.integers(0, W, count)
+        # all tile-boundary rows (+-2) for two (n, c) pairs, every column
+        rows = np.array([r * Ht + d for r in range(1, K) for d in (-2, -1, 0, 1)] + [0, 1, H - 2, H - 1])
+        for (nn, cc) in ((0, 3), (1, 40)):
+            hh, ww = np.meshgrid(rows, np.arange(W), indexing="ij")
+            n = np.concatenate([n, np.full(hh.size, nn)])
+            c = np.concatenate([c, np.full(hh.size, cc)])
+            h = np.concatenate([h, hh.ravel()])
+            w_ = np.concatenate([w_, ww.ravel()])
+        return n, c, h, w_
+
+    # forward: y[n,co,h,w] = sum_{ci,a,b} w[co,ci,a,b] * Xp[n,ci,h+a,w+b]
+    n, co, h, w_ = sample_coords(100000)
+    ref = np.zeros(n.size, np.float64)
+    for a in range(3):
+        for b in range(3):
+            patch = Xh[n, :, h + a, w_ + b].astype(np.float64)      # (samples, C)
+            ref += np.einsum("sc,sc->s", patch, wh[co, :, a, b])
+    got = Yh[n, co, h, w_]
+    assert np.max(np.abs(got - ref)) / np.max(np.abs(ref)) <= TOL
+    # backward-data of the unsplit conv: dx[n,ci,h,w] = sum_{co,a,b} w[co,ci,a,b] * dYp[n,co,h+2-a,w+2-b]
+    n, ci, h, w_ = sample_coords(100000)
+    ref = np.zeros(n.size, np.float64)
+    for a in range(3):
+        for b in range(3):
+            patch = dYh[n, :, h + 2 - a, w_ + 2 - b].astype(np.float64)
+            ref += np.einsum("sc,sc->s", patch, wh[:, ci, a, b].T)
+    got = gXh[n, ci, h, w_]
+    assert np.max(np.abs(got - ref)) / np.max(np.abs(ref)) <= TOL
+    # backward-filter on 48 (co, ci) pairs, all 9 taps, summed over every pixel
+    gwh = gw.cpu().numpy()
+    dYc = dYh[:, :, 1:-1, 1:-1]
+    errs, mags = [], []
+    for _ in range(48):
+        co_, ci_ = int(rng.integers(0, C)), int(rng.integers(0, C))
+        for a in range(3):
+            for b in range(3):
+                ref1 = float(np.sum(dYc[:, co_].astype(np.float64) * Xh[:, ci_, a:a + H, b:b + W]))
+                errs.append(abs(gwh[co_, ci_, a, b] - ref1))
+                mags.append(abs(ref1))
+    assert max(errs) / max(mags) <= 1e-3
