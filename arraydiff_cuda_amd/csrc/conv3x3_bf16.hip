@@ -1,6 +1,8 @@
 // bf16 entry of the 3x3 slab convolution: bf16 tensors in HBM, fp32 accumulation.
 //
-// Current implementation: the bf16 slabs, filter and (for beta = 1) outputs are widened to fp32
+// Forward and backward-data with at most 64 reduction channels run on the bf16 matrix-core
+// kernel of conv3x3_bf16_mfma.hip.  Everything else (wider reductions, the filter gradient) takes
+// the route below: the bf16 slabs, filter and (for beta = 1) outputs are widened to fp32
 // in the caller's workspace, the fp32 MFMA kernels run on the copies, and the result is rounded
 // back to bf16 (round to nearest even).  Every product is therefore exact and every sum is in
 // fp32, i.e. the arithmetic of a bf16-input / fp32-accumulate matrix core, at the speed of the
@@ -58,8 +60,16 @@ static uint32_t cvt_grid(uint64_t n) {
 // fp32 scratch copies live in 256-byte aligned consecutive regions of the workspace
 static size_t region(uint64_t elems) { return (size_t)((elems * 4u + 255u) / 256u * 256u); }
 
+bool conv_bf16_mfma_supported(int which, uint32_t Cin, uint32_t Cout);
+size_t conv_bf16_mfma_workspace_bytes(int which, uint32_t Cin, uint32_t Cout);
+int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                   const void *const *in_tiles, const void *w, void *const *out_tiles, float beta, void *workspace,
+                   hipStream_t st);
+
 size_t bf16_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                             uint32_t W, size_t fp32_path_bytes) {
+  if (which != ADH_CONV_BWD_FILTER && conv_bf16_mfma_supported(which, Cin, Cout))
+    return conv_bf16_mfma_workspace_bytes(which, Cin, Cout);
   const uint64_t slab = (uint64_t)N * Cin * (H + 2) * (W + 2), out = (uint64_t)N * Cout * H * W;
   const uint64_t filt = (uint64_t)Cin * Cout * 9u;
   size_t total = 0;
@@ -101,16 +111,23 @@ int conv_bf16_via_f32(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, u
   if (!workspace) return ADH_ENULL;
   if (!aligned_to(workspace, 256)) return ADH_EALIGN;
   if (workspace_bytes < need) return ADH_EWORKSPACE;
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!in_tiles[t] || !out_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(in_tiles[t], 2) || !aligned_to(out_tiles[t], 2)) return ADH_EALIGN;
+  }
+  if (conv_bf16_mfma_supported(which, Cin, Cout)) {
+    // one image is addressed through a 32-bit buffer resource
+    const uint64_t cmax = Cin > Cout ? Cin : Cout;
+    if (cmax * (H + 2ull) * (W + 2ull) * 2u >= (1ull << 31) || (uint64_t)Cin * Cout * 18u >= (1ull << 31))
+      return ADH_EINVAL;
+    return conv_bf16_mfma(which, num_tiles, N, Cin, Cout, H, W, in_tiles, w, out_tiles, beta, workspace, st);
+  }
   const uint64_t slab = (uint64_t)N * Cin * (H + 2) * (W + 2), outn = (uint64_t)N * Cout * H * W;
   const uint64_t in_elems = which == ADH_CONV_FWD ? slab : outn;
   const uint64_t out_elems = which == ADH_CONV_FWD ? outn : slab;
   char *ws = reinterpret_cast<char *>(workspace);
   const void *in32[ADH_MAX_TILES];
   void *out32[ADH_MAX_TILES];
-  for (uint32_t t = 0; t < num_tiles; ++t) {
-    if (!in_tiles[t] || !out_tiles[t]) return ADH_ENULL;
-    if (!aligned_to(in_tiles[t], 2) || !aligned_to(out_tiles[t], 2)) return ADH_EALIGN;
-  }
   float *w32 = reinterpret_cast<float *>(ws);
   ws += region((uint64_t)Cin * Cout * 9u);
   int e = widen((uint64_t)Cin * Cout * 9u, w, w32, st);

@@ -20,7 +20,12 @@ def ws_for(which, K, N, Cin, Cout, H, W):
     return torch.empty(nbytes // 4 + 64, device="cuda")
 
 
-@pytest.mark.parametrize("K,N,Cin,Cout,H,W", [(1, 2, 8, 16, 5, 9), (2, 1, 19, 7, 6, 33), (3, 2, 64, 64, 7, 56)])
+# shapes cover: channel counts off the 8/32/64 steps, two output-channel groups, odd widths,
+# widths off the 32-column strip, row counts off the 8-row step and split into row segments,
+# and reductions wider than 64 channels (the widening route)
+@pytest.mark.parametrize("K,N,Cin,Cout,H,W", [(1, 2, 8, 16, 5, 9), (2, 1, 19, 7, 6, 33), (3, 2, 64, 64, 7, 56),
+                                              (1, 1, 20, 70, 9, 61), (2, 2, 64, 64, 40, 70), (1, 1, 64, 64, 3, 130),
+                                              (1, 1, 72, 64, 6, 20), (1, 1, 64, 72, 6, 20), (1, 3, 33, 40, 17, 31)])
 def test_bf16_conv_small_vs_oracle(oracle, K, N, Cin, Cout, H, W):
     rng = np.random.default_rng(77 + Cin)
     bf = lambda a: oracle.f32_to_bf16(a.astype(np.float32))
@@ -43,9 +48,11 @@ def test_bf16_conv_small_vs_oracle(oracle, K, N, Cin, Cout, H, W):
         y = np.empty((N, Cout, H, W), np.float32)
         oracle.conv_slab_fwd(xf, wf, y)
         assert rel_err(oracle.bf16_to_f32(host(ys[r])), y) <= TOL
+        # exact products and fp32 sums: only the final rounding to bf16 (2^-9 relative) remains
+        assert rel_err(oracle.bf16_to_f32(host(ys[r])), y) <= 5e-3
         g = np.empty((N, Cin, H + 2, W + 2), np.float32)
         oracle.conv_slab_bwd_data(wf, dyf, g)
-        assert rel_err(oracle.bf16_to_f32(host(gs[r])), g) <= TOL
+        assert rel_err(oracle.bf16_to_f32(host(gs[r])), g) <= 5e-3
         oracle.conv_slab_bwd_filter(xf, dyf, dw_want, beta=1.0)
     assert rel_err(host(dw), dw_want) <= 1e-4  # fp32 output, exact bf16 products
     # beta = 1 accumulates onto a bf16 output
