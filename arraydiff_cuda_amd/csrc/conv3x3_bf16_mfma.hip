@@ -19,6 +19,8 @@
 //
 // Out-of-range rows, channels and buffer ends are handled by the buffer resource's range check
 // (out-of-range dwords read as zero); out-of-range columns by per-dword masks.
+#include <utility>
+
 #include "adh_common.h"
 
 namespace adh {
@@ -31,9 +33,12 @@ typedef u32x2 u32x2_unaligned __attribute__((aligned(2)));
 
 constexpr int kStripCols = 32;                        // output columns per work item
 constexpr int kStepRows = 8;                          // output rows per step
-constexpr int kRingRows = 18;                         // 10 rows in use + 8 rows in flight
+constexpr int kRingRows = 18;                         // 10 rows in use + 8 rows being written
 constexpr int kPatchCols = kStripCols + 2;            // 34
-constexpr int kPxPitch = 144;                         // bytes per pixel in LDS
+#ifndef EXP_PITCH
+#define EXP_PITCH 144
+#endif
+constexpr int kPxPitch = EXP_PITCH;                   // bytes per pixel in LDS
 constexpr int kRowPitch = kPatchCols * kPxPitch;      // 4896
 constexpr int kRingBytes = kRingRows * kRowPitch;     // 88128
 constexpr uint32_t kOutOfRange = 0x80000000u;
@@ -71,10 +76,23 @@ __global__ __launch_bounds__(256) void conv3x3_bf16_filter_kernel(const uint16_t
   wt[i] = v;
 }
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+template <int V>
+struct IntTag { static constexpr int value = V; };
+template <int... T, typename F>
+__device__ __forceinline__ void for_each_int(std::integer_sequence<int, T...>, F &&f) {
+  (f(IntTag<T>()), ...);
 }
 
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// two floats -> two bf16 (round to nearest even) in one dword: one v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  const floatx2 f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+
+template <bool BETA>
 __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) {
   __shared__ __attribute__((aligned(16))) uint8_t ring[kRingBytes];
 
@@ -107,7 +125,15 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
 
   const uint32_t read_lane_base = (16u * cb + l16) * kPxPitch + g * 16u;
 
-  for (uint32_t item = blockIdx.x; item < P.items; item += gridDim.x) {
+  // Workgroups are dealt to the eight XCDs (each with its own L2) in turn.  Renumber them so
+  // that an XCD works on neighbouring strips: those share the 128-byte lines at strip borders.
+  uint32_t vblock = blockIdx.x;
+  if ((gridDim.x & 7u) == 0u) vblock = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+#ifdef EXP_TIMING
+  uint64_t tacc[4] = {0, 0, 0, 0};
+  const uint64_t tstart = __builtin_readcyclecounter();
+#endif
+  for (uint32_t item = vblock; item < P.items; item += gridDim.x) {
     uint32_t strip, t1, seg, plane, tile, n;
     P.div_strips.divmod(item, t1, strip);
     P.div_segs.divmod(t1, plane, seg);
@@ -137,34 +163,49 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
     const int32_t vbase = (int32_t)((chg * 8u * P.IH) * P.IW * 2u) + ((arow0 + (int32_t)lrow) * (int32_t)P.IW + icol0) * 2;
     const int32_t tbase = vbase + (tcol0 - icol0) * 2;
 
-    u32x4 ld[8];
-    uint32_t lt[8];
+    // per-channel load offsets and keep-masks (all ones for a channel that exists)
+    uint32_t vch[8], vkeep[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      vch[j] = (uint32_t)vbase + (uint32_t)j * plane_bytes;
+      vkeep[j] = ((chvalid >> j) & 1u) ? 0xffffffffu : 0u;
+    }
+    // column-halo tail (patch pixels 32, 33): this thread fetches channels 2*pxb, 2*pxb+1 of its group
+    uint32_t tch[2], tkeep[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      tch[j] = (uint32_t)tbase + (2u * pxb + j) * plane_bytes;
+      tkeep[j] = ((chvalid >> (2u * pxb + j)) & 1u) ? 0xffffffffu : 0u;
+    }
 
-    auto issue = [&](int32_t row0) {
+    // registers of the load round in flight
+    struct LoadRegs {
+      u32x4 ld[8];
+      uint32_t lt[2];
+    };
+    LoadRegs L0, L1;
+
+    // offsets of absent rows and channels are replaced by one that is always out of range
+    auto issue = [&](int32_t row0, LoadRegs &L) {
       const int32_t i = row0 + (int32_t)lrow;
       const int32_t arow = arow0 + i;
-      const bool ok = i >= 0 && arow >= 0 && arow < (int32_t)P.IH;
-      const uint32_t v = (uint32_t)(vbase + row0 * (int32_t)P.IW * 2);
-      const uint32_t t = (uint32_t)(tbase + row0 * (int32_t)P.IW * 2);
+      const uint32_t rowkeep = (i >= 0 && arow >= 0 && arow < (int32_t)P.IH) ? 0xffffffffu : 0u;
+      const uint32_t step_off = (uint32_t)(row0 * (int32_t)P.IW * 2);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const bool okj = ok && ((chvalid >> j) & 1u);
-        ld[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, okj ? v + (uint32_t)j * plane_bytes : kOutOfRange, 0, 0);
+        const uint32_t keep = vkeep[j] & rowkeep;
+        L.ld[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ((vch[j] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
       }
-      if (pxb == 0) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const bool okj = ok && ((chvalid >> j) & 1u);
-          lt[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, okj ? t + (uint32_t)j * plane_bytes : kOutOfRange, 0, 0);
-        }
+      for (int j = 0; j < 2; ++j) {
+        const uint32_t keep = tkeep[j] & rowkeep;
+        L.lt[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ((tch[j] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
       }
     };
 
-    auto commit = [&](int32_t row0) {
+    auto commit = [&](int32_t row0, LoadRegs &L) {
       const int32_t i = row0 + (int32_t)lrow;
       if (i < 0) return;
-      // The range check drops a dword that straddles the end of the image even though its low
-      // half is the image's last element: fetch that element on its own.
       {
         const int32_t arow = arow0 + i;
         // A load that starts left of the image's first element (first row of channel 0, left
@@ -174,8 +215,10 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
           const int32_t v = vbase + row0 * (int32_t)P.IW * 2;
 #pragma unroll
           for (int d = 0; d < 4; ++d)
-            ld[0][d] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, v + 4 * d >= 0 ? (uint32_t)(v + 4 * d) : kOutOfRange, 0, 0);
+            L.ld[0][d] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, v + 4 * d >= 0 ? (uint32_t)(v + 4 * d) : kOutOfRange, 0, 0);
         }
+        // The range check drops a dword that straddles the end of the image even though its low
+        // half is the image's last element: fetch that element on its own.
         if (arow == (int32_t)P.IH - 1 && chg == (P.Cred - 1u) >> 3) {
           const uint32_t j = (P.Cred - 1u) & 7u;
           const uint32_t v = (uint32_t)(vbase + row0 * (int32_t)P.IW * 2) + j * plane_bytes;
@@ -186,16 +229,14 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
 #pragma unroll
             for (int jj = 0; jj < 8; ++jj)
 #pragma unroll
-              for (int dd = 0; dd < 4; ++dd)
-                if ((uint32_t)jj == j && (uint32_t)dd == d) ld[jj][dd] |= e;
+              for (int dd = 0; dd < 4; ++dd) L.ld[jj][dd] |= ((uint32_t)jj == j && (uint32_t)dd == d) ? e : 0u;
           }
-          if (pxb == 0) {
+          if (pxb == (j >> 1)) {
             const uint32_t t = (uint32_t)(tbase + row0 * (int32_t)P.IW * 2) + j * plane_bytes;
             if (t == image_bytes - 2u) {
               const uint32_t e = __builtin_amdgcn_raw_buffer_load_b16(rsrc, image_bytes - 2u, 0, 0) & 0xffffu;
-#pragma unroll
-              for (int jj = 0; jj < 8; ++jj)
-                if ((uint32_t)jj == j) lt[jj] |= e;
+              L.lt[0] |= (j & 1u) ? 0u : e;
+              L.lt[1] |= (j & 1u) ? e : 0u;
             }
           }
         }
@@ -207,118 +248,265 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
         u32x4 even, odd;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const uint32_t lo = ld[2 * q][d] & md[d], hi = ld[2 * q + 1][d] & md[d];
+          const uint32_t lo = L.ld[2 * q][d] & md[d], hi = L.ld[2 * q + 1][d] & md[d];
           even[q] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
           odd[q] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
         }
         *reinterpret_cast<u32x4 *>(dst + (2 * d) * kPxPitch) = even;
         *reinterpret_cast<u32x4 *>(dst + (2 * d + 1) * kPxPitch) = odd;
       }
-      if (pxb == 0) {
-        u32x4 even, odd;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const uint32_t lo = lt[2 * q] & mt, hi = lt[2 * q + 1] & mt;
-          even[q] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-          odd[q] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
-        }
-        uint8_t *td = ring + slot * kRowPitch + kStripCols * kPxPitch + chg * 16u;
-        *reinterpret_cast<u32x4 *>(td) = even;
-        *reinterpret_cast<u32x4 *>(td + kPxPitch) = odd;
+      {
+        const uint32_t lo = L.lt[0] & mt, hi = L.lt[1] & mt;
+        uint8_t *td = ring + slot * kRowPitch + kStripCols * kPxPitch + chg * 16u + pxb * 4u;
+        *reinterpret_cast<uint32_t *>(td) = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        *reinterpret_cast<uint32_t *>(td + kPxPitch) = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
       }
     };
 
     // ring-relative rows 0..9 of the first step
-    issue(2 - kStepRows);
-    commit(2 - kStepRows);
-    issue(2);
-    commit(2);
+    issue(2 - kStepRows, L0);
+    issue(2, L1);
+    commit(2 - kStepRows, L0);
+    commit(2, L1);
+    if (nsteps > 1) issue(kStepRows + 2, L0);  // rows of step 1, committed at the start of step 0
     __syncthreads();
 
-    uint32_t sb = 0;  // ring slot of this step's first input row
-    for (uint32_t s = 0; s < nsteps; ++s) {
-      const bool more = s + 1 < nsteps;
-      const int32_t next_row0 = (int32_t)((s + 1) * kStepRows) + 2;
-      if (more) issue(next_row0);
+    // Output of a step is kept packed in registers and stored at the start of the next step, so
+    // that the stores drain behind that step's MFMAs; for beta = 1 the old values are fetched at
+    // the start of their own step for the same reason.
+    const uint32_t ocol = (uint32_t)c0 + 16u * cb + 4u * g;
+    const uint32_t co0 = grp * 64u + 32u * h + l16;
+    const bool ok_ct[2] = {co0 < P.Cout, co0 + 16u < P.Cout};
+    const bool full_cols = ocol + 3u < P.OW;
+    const size_t ct_stride = (size_t)16u * P.OH * P.OW;
+    uint16_t *const olane = out_img + (size_t)co0 * P.OH * P.OW + ocol;
+    u32x2 pk[2][kStepRows], old[2][kStepRows];
 
+    // common case, decided per wave: all eight rows, both channel tiles, four whole columns
+    const bool lanes_whole = __builtin_amdgcn_ballot_w64(!(full_cols && ok_ct[0] && ok_ct[1])) == 0ull;
+
+    auto store_packed = [&](uint32_t row0, uint32_t nrows) {
+      uint16_t *obase = olane + (size_t)row0 * P.OW;
+      if (lanes_whole && nrows >= (uint32_t)kStepRows) {
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+          for (int r = 0; r < kStepRows; ++r)
+            *reinterpret_cast<u32x2_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW) = pk[ct][r];
+      } else if (full_cols) {
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+          for (int r = 0; r < kStepRows; ++r)
+            if ((uint32_t)r < nrows && ok_ct[ct])
+              *reinterpret_cast<u32x2_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW) = pk[ct][r];
+      } else if (ocol < P.OW) {
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+          for (int r = 0; r < kStepRows; ++r)
+            if ((uint32_t)r < nrows && ok_ct[ct]) {
+              uint16_t *p = obase + ct * ct_stride + (size_t)r * P.OW;
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (ocol + e < P.OW) p[e] = (uint16_t)(pk[ct][r][e >> 1] >> ((e & 1) * 16));
+            }
+      }
+    };
+    auto load_old = [&](uint32_t row0, uint32_t nrows) {
+      if (!BETA) return;
+      const uint16_t *obase = olane + (size_t)row0 * P.OW;
+      if (lanes_whole && nrows >= (uint32_t)kStepRows) {
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+          for (int r = 0; r < kStepRows; ++r)
+            old[ct][r] = *reinterpret_cast<const u32x2_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW);
+      } else if (full_cols) {
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+          for (int r = 0; r < kStepRows; ++r)
+            if ((uint32_t)r < nrows && ok_ct[ct])
+              old[ct][r] = *reinterpret_cast<const u32x2_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW);
+      } else if (ocol < P.OW) {
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+          for (int r = 0; r < kStepRows; ++r)
+            if ((uint32_t)r < nrows && ok_ct[ct]) {
+              const uint16_t *p = obase + ct * ct_stride + (size_t)r * P.OW;
+              uint32_t e4[4];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) e4[e] = ocol + e < P.OW ? (uint32_t)p[e] : 0u;
+              old[ct][r][0] = e4[0] | (e4[1] << 16);
+              old[ct][r][1] = e4[2] | (e4[3] << 16);
+            }
+      }
+    };
+
+    uint32_t sb = 0;  // ring slot of this step's first input row
+    uint32_t prev_row0 = 0, prev_nrows = 0;
+
+    // The matrix part of a step: 60 operand reads (input row, column shift, channel half), each
+    // fetched kAhead reads before its MFMAs so that the LDS latency hides behind the matrix pipe,
+    // then the results are packed to bf16.  kVm global-memory instructions issued just before
+    // are spread over the first rounds, one per round: issued in a burst they would fill the
+    // memory pipeline's queue and hold every wave of the workgroup at the same point.
+    auto compute = [&](auto vm_tag, auto &&vm_op) {
+      constexpr int kVm = decltype(vm_tag)::value;
       floatx4 acc[kStepRows][2];
 #pragma unroll
       for (int r = 0; r < kStepRows; ++r)
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) acc[r][ct] = (floatx4){0.f, 0.f, 0.f, 0.f};
-
+      #ifndef EXP_AHEAD
+#define EXP_AHEAD 3
+#endif
+      constexpr int kReads = (kStepRows + 2) * 6, kAhead = EXP_AHEAD;
+      uint32_t row_addr[kStepRows + 2];
 #pragma unroll
       for (int ir = 0; ir < kStepRows + 2; ++ir) {
         uint32_t slot = sb + (uint32_t)ir;
         slot = slot >= (uint32_t)kRingRows ? slot - (uint32_t)kRingRows : slot;
-        const uint8_t *src = ring + slot * kRowPitch + read_lane_base;
+        row_addr[ir] = slot * kRowPitch;
+      }
+      u32x4 abuf[kAhead + 1];
+      auto fetch = [&](int t) {
+        const int ir = t / 6, kw = (t % 6) >> 1, half = t & 1;
+        abuf[t % (kAhead + 1)] =
+            *reinterpret_cast<const u32x4 *>(ring + row_addr[ir] + read_lane_base + kw * kPxPitch + half * 64);
+      };
 #pragma unroll
-        for (int kw = 0; kw < 3; ++kw) {
+      for (int t = 0; t < kAhead; ++t) fetch(t);
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+      auto round = [&](auto tag) {
+        constexpr int t = decltype(tag)::value;
+        if constexpr (t + kAhead < kReads) {
+          fetch(t + kAhead);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        constexpr int ir = t / 6, kw = (t % 6) >> 1, half = t & 1;
+        const bf16x8 a = __builtin_bit_cast(bf16x8, abuf[t % (kAhead + 1)]);
+        constexpr int kh_lo = ir - (kStepRows - 1) > 0 ? ir - (kStepRows - 1) : 0;
+        constexpr int kh_hi = ir < 2 ? ir : 2;
 #pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const u32x4 a = *reinterpret_cast<const u32x4 *>(src + kw * kPxPitch + half * 64);
+        for (int kh = kh_lo; kh <= kh_hi; ++kh) {
 #pragma unroll
-            for (int kh = 0; kh < 3; ++kh) {
-              const int orow = ir - kh;
-              if (orow < 0 || orow >= kStepRows) continue;
-#pragma unroll
-              for (int ct = 0; ct < 2; ++ct)
-                acc[orow][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, wreg[kh * 3 + kw][half][ct]),
-                    acc[orow][ct], 0, 0, 0);
-            }
+          for (int ct = 0; ct < 2; ++ct)
+            acc[ir - kh][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                a, __builtin_bit_cast(bf16x8, wreg[kh * 3 + kw][half][ct]), acc[ir - kh][ct], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * (kh_hi - kh_lo + 1), 0);
+        // memory instruction i goes after round floor(i * kReads / kVm)
+        if constexpr (kVm > 0) {
+          constexpr int i = (t * kVm + kReads - 1) / kReads;  // first i with i * kReads >= t * kVm
+          if constexpr (i < kVm && (i * kReads) / kVm == t) {
+            vm_op(IntTag<i>());
+            __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
           }
         }
-      }
+      };
+#ifndef EXP_NO_MFMA
+      for_each_int(std::make_integer_sequence<int, kReads>(), round);
+#endif
+      __builtin_amdgcn_sched_barrier(0);
 
-      // results: lane (l16, g) holds output channel l16 of its tile, columns 4g..4g+3
-      {
-        const uint32_t col = (uint32_t)c0 + 16u * cb + 4u * g;
-        const uint32_t row0 = r_begin + s * kStepRows;
+      // lane (l16, g) holds output channel l16 of its tile, columns 4g..4g+3
 #pragma unroll
-        for (int ct = 0; ct < 2; ++ct) {
-          const uint32_t co = grp * 64u + 32u * h + 16u * ct + l16;
-          if (co < P.Cout && col < P.OW) {
-            uint16_t *orow_ptr = out_img + ((size_t)co * P.OH + row0) * P.OW + col;
-            const bool full = col + 3u < P.OW;
+      for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
-            for (int r = 0; r < kStepRows; ++r) {
-              if (row0 + r < r_end) {
-                uint16_t *p = orow_ptr + (size_t)r * P.OW;
-                floatx4 v = acc[r][ct];
-                if (full) {
-                  if (P.beta != 0.f) {
-                    const u32x2 old = *reinterpret_cast<const u32x2_unaligned *>(p);
-                    v[0] += __uint_as_float(old[0] << 16);
-                    v[1] += __uint_as_float(old[0] & 0xffff0000u);
-                    v[2] += __uint_as_float(old[1] << 16);
-                    v[3] += __uint_as_float(old[1] & 0xffff0000u);
-                  }
-                  u32x2 o;
-                  o[0] = pack_bf16x2(v[0], v[1]);
-                  o[1] = pack_bf16x2(v[2], v[3]);
-                  *reinterpret_cast<u32x2_unaligned *>(p) = o;
-                } else {
-#pragma unroll
-                  for (int e = 0; e < 4; ++e)
-                    if (col + e < P.OW) {
-                      float f = v[e];
-                      if (P.beta != 0.f) f += bf16_bits_to_f32(p[e]);
-                      p[e] = f32_to_bf16_bits(f);
-                    }
-                }
-              }
-            }
+        for (int r = 0; r < kStepRows; ++r) {
+          floatx4 v = acc[r][ct];
+          if (BETA) {
+            v[0] += __uint_as_float(old[ct][r][0] << 16);
+            v[1] += __uint_as_float(old[ct][r][0] & 0xffff0000u);
+            v[2] += __uint_as_float(old[ct][r][1] << 16);
+            v[3] += __uint_as_float(old[ct][r][1] & 0xffff0000u);
           }
+          pk[ct][r][0] = pack_bf16x2(v[0], v[1]);
+          pk[ct][r][1] = pack_bf16x2(v[2], v[3]);
         }
-      }
+    };
 
-      if (more) commit(next_row0);
+    // One step.  The rows of step s + 1, requested a whole step ago, go into the ring first (they
+    // land in slots this step does not read); then the rows of step s + 2 are requested.  Every
+    // wait on memory therefore only covers requests that are at least one step old.
+    for (uint32_t s = 0; s < nsteps; ++s) {
+      const bool more = s + 1 < nsteps, more2 = s + 2 < nsteps;
+      const int32_t next_row0 = (int32_t)((s + 1) * kStepRows) + 2;
+#ifdef EXP_TIMING
+      const uint64_t tq0 = __builtin_readcyclecounter();
+#endif
+      if (more) commit(next_row0, L0);
+      // Everything still in flight here (the previous step's stores) is a step old.  Draining it
+      // explicitly keeps the compiler from guarding register reuse further down with waits that
+      // would also cover the requests this step is about to issue.
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+#ifdef EXP_TIMING
+      const uint64_t tq1 = __builtin_readcyclecounter();
+#endif
+      const uint32_t row0 = r_begin + s * kStepRows;
+      const uint32_t nrows = r_end - row0;  // rows >= nrows of this step do not exist
+      if (lanes_whole && s > 0 && nrows >= (uint32_t)kStepRows) {
+        // straight-line variant: every memory instruction is unconditional (rows requested
+        // past the end of the segment are never used)
+        const int32_t irow0 = next_row0 + kStepRows;
+        const int32_t li = irow0 + (int32_t)lrow, larow = arow0 + li;
+        const uint32_t rowkeep = (larow >= 0 && larow < (int32_t)P.IH) ? 0xffffffffu : 0u;
+        const uint32_t step_off = (uint32_t)(irow0 * (int32_t)P.IW * 2);
+        uint16_t *const sbase = olane + (size_t)prev_row0 * P.OW;
+        const uint16_t *const obase = olane + (size_t)row0 * P.OW;
+        compute(IntTag<BETA ? 42 : 26>(), [&](auto tag) {
+          constexpr int t = decltype(tag)::value;
+#ifdef EXP_VM_NOLOAD
+          if constexpr (t < 10) return;
+#endif
+#ifdef EXP_VM_NOSTORE
+          if constexpr (t >= 10 && t < 26) return;
+#endif
+          if constexpr (t < 8) {
+            const uint32_t keep = vkeep[t] & rowkeep;
+            L0.ld[t] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ((vch[t] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
+          } else if constexpr (t < 10) {
+            const uint32_t keep = tkeep[t - 8] & rowkeep;
+            L0.lt[t - 8] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ((tch[t - 8] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
+          } else if constexpr (t < 26) {
+            constexpr int ct = (t - 10) / kStepRows, r = (t - 10) % kStepRows;
+            *reinterpret_cast<u32x2_unaligned *>(sbase + ct * ct_stride + (size_t)r * P.OW) = pk[ct][r];
+          } else {
+            constexpr int ct = (t - 26) / kStepRows, r = (t - 26) % kStepRows;
+            old[ct][r] = *reinterpret_cast<const u32x2_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW);
+          }
+        });
+      } else {
+        if (more2) issue(next_row0 + kStepRows, L0);
+        if (s > 0) store_packed(prev_row0, prev_nrows);
+        if (BETA) load_old(row0, nrows);
+        compute(IntTag<0>(), [](auto) {});
+      }
+      prev_row0 = row0;
+      prev_nrows = nrows;
+#ifdef EXP_TIMING
+      const uint64_t tq2 = __builtin_readcyclecounter();
+#endif
       __syncthreads();
+#ifdef EXP_TIMING
+      const uint64_t tq3 = __builtin_readcyclecounter();
+      tacc[0] += tq1 - tq0; tacc[1] += tq2 - tq1; tacc[2] += tq3 - tq2; tacc[3] += 1;
+#endif
       sb += kStepRows;
       sb = sb >= (uint32_t)kRingRows ? sb - (uint32_t)kRingRows : sb;
     }
+    store_packed(prev_row0, prev_nrows);
   }
+#ifdef EXP_TIMING
+  if (lane == 0) {
+    uint64_t *dbg = reinterpret_cast<uint64_t *>(const_cast<uint16_t *>(P.wt) + kWtGroupElems) + (blockIdx.x * 4 + wv) * 8;
+    dbg[0] = tacc[0]; dbg[1] = tacc[1]; dbg[2] = tacc[2]; dbg[3] = tacc[3];
+    dbg[4] = __builtin_readcyclecounter() - tstart;
+  }
+#endif
 }
 
 static int g_num_cus = 0;
@@ -396,7 +584,10 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
   P.div_N = FastDiv(N);
   uint32_t gx = cus / groups ? cus / groups : 1u;
   if (gx > P.items) gx = P.items;
-  hipLaunchKernelGGL(conv3x3_bf16_kernel, dim3(gx, groups), dim3(256), 0, st, P);
+  if (beta != 0.f)
+    hipLaunchKernelGGL(conv3x3_bf16_kernel<true>, dim3(gx, groups), dim3(256), 0, st, P);
+  else
+    hipLaunchKernelGGL(conv3x3_bf16_kernel<false>, dim3(gx, groups), dim3(256), 0, st, P);
   return launch_status();
 }
 
