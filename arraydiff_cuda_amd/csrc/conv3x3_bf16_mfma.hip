@@ -185,6 +185,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
     };
     LoadRegs L0, L1;
 
+    bool tails_loaded = false;  // L0.lt holds the tails of the rows in L0.ld (uniform)
     // offsets of absent rows and channels are replaced by one that is always out of range
     auto issue = [&](int32_t row0, LoadRegs &L) {
       const int32_t i = row0 + (int32_t)lrow;
@@ -201,11 +202,20 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
         const uint32_t keep = tkeep[j] & rowkeep;
         L.lt[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ((tch[j] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
       }
+      tails_loaded = true;
     };
 
-    auto commit = [&](int32_t row0, LoadRegs &L) {
+    // the pieces of a row in ring order: eight pixels of eight channels each, plus this thread's
+    // share of the two tail pixels
+    struct Transposed {
+      u32x4 px[8];
+      uint32_t tail[2];
+      uint32_t dst, tdst;
+    };
+    // patches up what the range check dropped, then turns the loaded channel-major registers
+    // into pixel-major pieces; the caller makes sure that ring row row0 + lrow is not negative
+    auto transpose = [&](int32_t row0, LoadRegs &L, Transposed &T) {
       const int32_t i = row0 + (int32_t)lrow;
-      if (i < 0) return;
       {
         const int32_t arow = arow0 + i;
         // A load that starts left of the image's first element (first row of channel 0, left
@@ -231,36 +241,65 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
 #pragma unroll
               for (int dd = 0; dd < 4; ++dd) L.ld[jj][dd] |= ((uint32_t)jj == j && (uint32_t)dd == d) ? e : 0u;
           }
-          if (pxb == (j >> 1)) {
-            const uint32_t t = (uint32_t)(tbase + row0 * (int32_t)P.IW * 2) + j * plane_bytes;
-            if (t == image_bytes - 2u) {
-              const uint32_t e = __builtin_amdgcn_raw_buffer_load_b16(rsrc, image_bytes - 2u, 0, 0) & 0xffffu;
-              L.lt[0] |= (j & 1u) ? 0u : e;
-              L.lt[1] |= (j & 1u) ? e : 0u;
-            }
+        }
+      }
+      const uint32_t slot = (uint32_t)i % (uint32_t)kRingRows;
+      T.dst = slot * kRowPitch + (pxb * 8u) * kPxPitch + chg * 16u;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t lo = L.ld[2 * q][d] & md[d], hi = L.ld[2 * q + 1][d] & md[d];
+          T.px[2 * d][q] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+          T.px[2 * d + 1][q] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+        }
+      }
+    };
+    // the same for this thread's two channels of the tail pixels, loaded into lt0 / lt1
+    auto transpose_tail = [&](int32_t row0, uint32_t lt0, uint32_t lt1, Transposed &T) {
+      const int32_t i = row0 + (int32_t)lrow;
+      if (arow0 + i == (int32_t)P.IH - 1 && chg == (P.Cred - 1u) >> 3) {
+        const uint32_t j = (P.Cred - 1u) & 7u;
+        if (pxb == (j >> 1)) {
+          const uint32_t t = (uint32_t)(tbase + row0 * (int32_t)P.IW * 2) + j * plane_bytes;
+          if (t == image_bytes - 2u) {
+            const uint32_t e = __builtin_amdgcn_raw_buffer_load_b16(rsrc, image_bytes - 2u, 0, 0) & 0xffffu;
+            lt0 |= (j & 1u) ? 0u : e;
+            lt1 |= (j & 1u) ? e : 0u;
           }
         }
       }
       const uint32_t slot = (uint32_t)i % (uint32_t)kRingRows;
-      uint8_t *dst = ring + slot * kRowPitch + (pxb * 8u) * kPxPitch + chg * 16u;
+      T.tdst = slot * kRowPitch + kStripCols * kPxPitch + chg * 16u + pxb * 4u;
+      const uint32_t lo = lt0 & mt, hi = lt1 & mt;
+      T.tail[0] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+      T.tail[1] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+    };
+    // LDS write number w of a transposed row piece: 0..7 the pixels of the block, 8 and 9 the tail
+    auto ring_write = [&](auto tag, const Transposed &T) {
+      constexpr int w = decltype(tag)::value;
+      if constexpr (w < 8)
+        *reinterpret_cast<u32x4 *>(ring + T.dst + w * kPxPitch) = T.px[w];
+      else
+        *reinterpret_cast<uint32_t *>(ring + T.tdst + (w - 8) * kPxPitch) = T.tail[w - 8];
+    };
+    auto commit = [&](int32_t row0, LoadRegs &L) {
+      if (!tails_loaded) {
+        // the step before ran the straight-line variant, which leaves the tails to its successor
+        const int32_t tarow = arow0 + row0 + (int32_t)lrow;
+        const uint32_t rowkeep = (tarow >= 0 && tarow < (int32_t)P.IH) ? 0xffffffffu : 0u;
+        const uint32_t step_off = (uint32_t)(row0 * (int32_t)P.IW * 2);
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        u32x4 even, odd;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const uint32_t lo = L.ld[2 * q][d] & md[d], hi = L.ld[2 * q + 1][d] & md[d];
-          even[q] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-          odd[q] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+        for (int j = 0; j < 2; ++j) {
+          const uint32_t keep = tkeep[j] & rowkeep;
+          L.lt[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ((tch[j] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
         }
-        *reinterpret_cast<u32x4 *>(dst + (2 * d) * kPxPitch) = even;
-        *reinterpret_cast<u32x4 *>(dst + (2 * d + 1) * kPxPitch) = odd;
       }
-      {
-        const uint32_t lo = L.lt[0] & mt, hi = L.lt[1] & mt;
-        uint8_t *td = ring + slot * kRowPitch + kStripCols * kPxPitch + chg * 16u + pxb * 4u;
-        *reinterpret_cast<uint32_t *>(td) = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-        *reinterpret_cast<uint32_t *>(td + kPxPitch) = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
-      }
+      if (row0 + (int32_t)lrow < 0) return;
+      Transposed T;
+      transpose(row0, L, T);
+      transpose_tail(row0, L.lt[0], L.lt[1], T);
+      for_each_int(std::make_integer_sequence<int, 10>(), [&](auto tag) { ring_write(tag, T); });
     };
 
     // ring-relative rows 0..9 of the first step
@@ -353,8 +392,9 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
     // then the results are packed to bf16.  kVm global-memory instructions issued just before
     // are spread over the first rounds, one per round: issued in a burst they would fill the
     // memory pipeline's queue and hold every wave of the workgroup at the same point.
-    auto compute = [&](auto vm_tag, auto &&vm_op) {
+    auto compute = [&](auto vm_tag, auto &&vm_op, auto lds_tag, auto &&lds_op) {
       constexpr int kVm = decltype(vm_tag)::value;
+      constexpr int kLds = decltype(lds_tag)::value;
       floatx4 acc[kStepRows][2];
 #pragma unroll
       for (int r = 0; r < kStepRows; ++r)
@@ -382,14 +422,17 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
       __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
       auto round = [&](auto tag) {
         constexpr int t = decltype(tag)::value;
+#ifndef EXP_NO_MFMA
         if constexpr (t + kAhead < kReads) {
           fetch(t + kAhead);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
+#endif
         constexpr int ir = t / 6, kw = (t % 6) >> 1, half = t & 1;
         const bf16x8 a = __builtin_bit_cast(bf16x8, abuf[t % (kAhead + 1)]);
         constexpr int kh_lo = ir - (kStepRows - 1) > 0 ? ir - (kStepRows - 1) : 0;
         constexpr int kh_hi = ir < 2 ? ir : 2;
+#ifndef EXP_NO_MFMA
 #pragma unroll
         for (int kh = kh_lo; kh <= kh_hi; ++kh) {
 #pragma unroll
@@ -398,18 +441,24 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
                 a, __builtin_bit_cast(bf16x8, wreg[kh * 3 + kw][half][ct]), acc[ir - kh][ct], 0, 0, 0);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 2 * (kh_hi - kh_lo + 1), 0);
-        // memory instruction i goes after round floor(i * kReads / kVm)
-        if constexpr (kVm > 0) {
-          constexpr int i = (t * kVm + kReads - 1) / kReads;  // first i with i * kReads >= t * kVm
-          if constexpr (i < kVm && (i * kReads) / kVm == t) {
-            vm_op(IntTag<i>());
-            __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
-          }
+#else
+        if constexpr (t == 0) acc[0][0] += __builtin_bit_cast(floatx4, a);
+#endif
+        // LDS write w goes after round 5 w + 2
+        if constexpr (t % 5 == 2 && t / 5 < kLds) {
+          lds_op(IntTag<t / 5>());
+          __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
+        // Memory instructions, one per round from the start of the step: first the stores of
+        // the previous step's results, then the loads.  At the start of a step no load of this
+        // workgroup is in flight, and the L1 takes stores quickly only then: a store behind
+        // pending loads waits for them.
+        if constexpr (t < kVm) {
+          vm_op(IntTag<t>());
+          __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
         }
       };
-#ifndef EXP_NO_MFMA
       for_each_int(std::make_integer_sequence<int, kReads>(), round);
-#endif
       __builtin_amdgcn_sched_barrier(0);
 
       // lane (l16, g) holds output channel l16 of its tile, columns 4g..4g+3
@@ -438,7 +487,14 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
 #ifdef EXP_TIMING
       const uint64_t tq0 = __builtin_readcyclecounter();
 #endif
-      if (more) commit(next_row0, L0);
+      const uint32_t row0 = r_begin + s * kStepRows;
+      const uint32_t nrows = r_end - row0;  // rows >= nrows of this step do not exist
+      const bool fast = lanes_whole && s > 0 && nrows >= (uint32_t)kStepRows;
+      Transposed T;
+      if (fast)
+        transpose(next_row0, L0, T);  // written to the ring between the MFMAs below
+      else if (more)
+        commit(next_row0, L0);
       // Everything still in flight here (the previous step's stores) is a step old.  Draining it
       // explicitly keeps the compiler from guarding register reuse further down with waits that
       // would also cover the requests this step is about to issue.
@@ -446,44 +502,56 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
 #ifdef EXP_TIMING
       const uint64_t tq1 = __builtin_readcyclecounter();
 #endif
-      const uint32_t row0 = r_begin + s * kStepRows;
-      const uint32_t nrows = r_end - row0;  // rows >= nrows of this step do not exist
-      if (lanes_whole && s > 0 && nrows >= (uint32_t)kStepRows) {
+      if (fast) {
         // straight-line variant: every memory instruction is unconditional (rows requested
         // past the end of the segment are never used)
+        // A tail pixel shares its 128-byte line with the row's main pieces.  Requested right
+        // behind them it would find that line still on its way and hold up the whole L1 queue,
+        // so the tails of the rows of step s + 1 are requested now, a step after their main
+        // pieces, and written at the end of this step.
         const int32_t irow0 = next_row0 + kStepRows;
         const int32_t li = irow0 + (int32_t)lrow, larow = arow0 + li;
         const uint32_t rowkeep = (larow >= 0 && larow < (int32_t)P.IH) ? 0xffffffffu : 0u;
         const uint32_t step_off = (uint32_t)(irow0 * (int32_t)P.IW * 2);
+        const int32_t tarow = arow0 + next_row0 + (int32_t)lrow;
+        const uint32_t trowkeep = (tarow >= 0 && tarow < (int32_t)P.IH) ? 0xffffffffu : 0u;
+        const uint32_t tstep_off = (uint32_t)(next_row0 * (int32_t)P.IW * 2);
+        uint32_t lt_now[2];
         uint16_t *const sbase = olane + (size_t)prev_row0 * P.OW;
         const uint16_t *const obase = olane + (size_t)row0 * P.OW;
         compute(IntTag<BETA ? 42 : 26>(), [&](auto tag) {
           constexpr int t = decltype(tag)::value;
-#ifdef EXP_VM_NOLOAD
-          if constexpr (t < 10) return;
-#endif
 #ifdef EXP_VM_NOSTORE
-          if constexpr (t >= 10 && t < 26) return;
+          if constexpr (t < 16) return;
 #endif
-          if constexpr (t < 8) {
-            const uint32_t keep = vkeep[t] & rowkeep;
-            L0.ld[t] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ((vch[t] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
-          } else if constexpr (t < 10) {
-            const uint32_t keep = tkeep[t - 8] & rowkeep;
-            L0.lt[t - 8] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ((tch[t - 8] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
-          } else if constexpr (t < 26) {
-            constexpr int ct = (t - 10) / kStepRows, r = (t - 10) % kStepRows;
+#ifdef EXP_VM_NOLOAD
+          if constexpr (t >= 16) return;
+#endif
+          if constexpr (t < 16) {
+            constexpr int ct = t / kStepRows, r = t % kStepRows;
             *reinterpret_cast<u32x2_unaligned *>(sbase + ct * ct_stride + (size_t)r * P.OW) = pk[ct][r];
+          } else if constexpr (t < 18) {
+            constexpr int j = t - 16;
+            const uint32_t keep = tkeep[j] & trowkeep;
+            lt_now[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ((tch[j] + tstep_off) & keep) | (kOutOfRange & ~keep), 0, 0);
+          } else if constexpr (t < 26) {
+            constexpr int j = t - 18;
+            const uint32_t keep = vkeep[j] & rowkeep;
+            L0.ld[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ((vch[j] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
           } else {
             constexpr int ct = (t - 26) / kStepRows, r = (t - 26) % kStepRows;
             old[ct][r] = *reinterpret_cast<const u32x2_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW);
           }
-        });
+        }, IntTag<8>(), [&](auto tag) { ring_write(tag, T); });
+        transpose_tail(next_row0, lt_now[0], lt_now[1], T);
+        ring_write(IntTag<8>(), T);
+        ring_write(IntTag<9>(), T);
+        tails_loaded = false;
       } else {
         if (more2) issue(next_row0 + kStepRows, L0);
         if (s > 0) store_packed(prev_row0, prev_nrows);
         if (BETA) load_old(row0, nrows);
-        compute(IntTag<0>(), [](auto) {});
+        compute(IntTag<0>(), [](auto) {}, IntTag<0>(), [](auto) {});
       }
       prev_row0 = row0;
       prev_nrows = nrows;
