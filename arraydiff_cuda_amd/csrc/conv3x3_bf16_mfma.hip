@@ -29,18 +29,15 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef u32x2 u32x2_unaligned __attribute__((aligned(2)));
+typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
 
-constexpr int kStripCols = 32;                        // output columns per work item
-constexpr int kStepRows = 8;                          // output rows per step
-constexpr int kRingRows = 18;                         // 10 rows in use + 8 rows being written
-constexpr int kPatchCols = kStripCols + 2;            // 34
-#ifndef EXP_PITCH
-#define EXP_PITCH 144
-#endif
-constexpr int kPxPitch = EXP_PITCH;                   // bytes per pixel in LDS
-constexpr int kRowPitch = kPatchCols * kPxPitch;      // 4896
-constexpr int kRingBytes = kRingRows * kRowPitch;     // 88128
+constexpr int kStripCols = 64;                        // output columns per work item
+constexpr int kStepRows = 4;                          // output rows per step
+constexpr int kRingRows = 10;                         // 6 rows in use + 4 rows being written
+constexpr int kPatchCols = kStripCols + 2;            // 66
+constexpr int kPxPitch = 144;                         // bytes per pixel in LDS
+constexpr int kRowPitch = kPatchCols * kPxPitch;      // 9504
+constexpr int kRingBytes = kRingRows * kRowPitch;     // 95040
 constexpr uint32_t kOutOfRange = 0x80000000u;
 constexpr uint32_t kWtGroupElems = 9u * 2u * 64u * 32u;  // transformed filter elements per group of 64 outputs
 
@@ -99,7 +96,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
   const uint32_t wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const uint32_t h = wv & 1u, cb = wv >> 1;
+  const uint32_t h = wv & 1u, cw = wv >> 1;  // output-channel half, column half of the strip
   const uint32_t grp = blockIdx.y;
 
   // this wave's filter share, in B-operand order: lane (n = l16, k-block = g)
@@ -115,15 +112,18 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
           wreg[tap][half][ct] = wt[((tap * 2 + half) * 64 + (int)(32u * h + 16u * ct + l16)) * 4 + (int)g];
   }
 
-  // loader role of this thread: one input row, eight channels, eight pixels
-  const uint32_t lrow = tid >> 5, chg = (tid >> 2) & 7u, pxb = tid & 3u;
+  // loader role of this thread: one input row, eight channels, eight pixels; and for the two
+  // tail pixels of a row (patch columns 64, 65) one channel
+  const uint32_t lrow = tid >> 6, chg = (tid >> 3) & 7u, pxb = tid & 7u, tch = tid & 63u;
   const uint32_t plane_bytes = P.IH * P.IW * 2u;
   const uint32_t image_bytes = P.Cred * plane_bytes;
   uint32_t chvalid = 0;
 #pragma unroll
   for (int j = 0; j < 8; ++j) chvalid |= (chg * 8u + j < P.Cred ? 1u : 0u) << j;
+  const uint32_t tkeep = tch < P.Cred ? 0xffffffffu : 0u;
 
-  const uint32_t read_lane_base = (16u * cb + l16) * kPxPitch + g * 16u;
+  // operand reads: pixel (32 cw + l16) of a ring row, channels 8 g .. 8 g + 7 of a half
+  const uint32_t read_lane_base = (32u * cw + l16) * kPxPitch + g * 16u;
 
   // Workgroups are dealt to the eight XCDs (each with its own L2) in turn.  Renumber them so
   // that an XCD works on neighbouring strips: those share the 128-byte lines at strip borders.
@@ -155,13 +155,13 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
       const int32_t ca = icol0 + 2 * d, cb2 = ca + 1;
       md[d] = ((ca >= 0 && ca < (int32_t)P.IW) ? 0x0000ffffu : 0u) | ((cb2 >= 0 && cb2 < (int32_t)P.IW) ? 0xffff0000u : 0u);
     }
-    const int32_t tcol0 = c0 - P.pad + kStripCols;  // tail pixels 32, 33
+    const int32_t tcol0 = c0 - P.pad + kStripCols;  // tail pixels
     const uint32_t mt = ((tcol0 >= 0 && tcol0 < (int32_t)P.IW) ? 0x0000ffffu : 0u) |
                         ((tcol0 + 1 >= 0 && tcol0 + 1 < (int32_t)P.IW) ? 0xffff0000u : 0u);
     const int32_t arow0 = (int32_t)r_begin - P.pad;  // input row of ring-relative row 0
     // byte offset of (channel chg*8, input row arow0 + lrow, column icol0); may be negative
     const int32_t vbase = (int32_t)((chg * 8u * P.IH) * P.IW * 2u) + ((arow0 + (int32_t)lrow) * (int32_t)P.IW + icol0) * 2;
-    const int32_t tbase = vbase + (tcol0 - icol0) * 2;
+    const int32_t tbase = (int32_t)((tch * P.IH) * P.IW * 2u) + ((arow0 + (int32_t)lrow) * (int32_t)P.IW + tcol0) * 2;
 
     // per-channel load offsets and keep-masks (all ones for a channel that exists)
     uint32_t vch[8], vkeep[8];
@@ -170,46 +170,39 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
       vch[j] = (uint32_t)vbase + (uint32_t)j * plane_bytes;
       vkeep[j] = ((chvalid >> j) & 1u) ? 0xffffffffu : 0u;
     }
-    // column-halo tail (patch pixels 32, 33): this thread fetches channels 2*pxb, 2*pxb+1 of its group
-    uint32_t tch[2], tkeep[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      tch[j] = (uint32_t)tbase + (2u * pxb + j) * plane_bytes;
-      tkeep[j] = ((chvalid >> (2u * pxb + j)) & 1u) ? 0xffffffffu : 0u;
-    }
 
-    // registers of the load round in flight
+    // registers of a load round
     struct LoadRegs {
       u32x4 ld[8];
-      uint32_t lt[2];
+      uint32_t lt;
     };
     LoadRegs L0, L1;
 
-    bool tails_loaded = false;  // L0.lt holds the tails of the rows in L0.ld (uniform)
-    // offsets of absent rows and channels are replaced by one that is always out of range
-    auto issue = [&](int32_t row0, LoadRegs &L) {
+    // one load of a round: k < 8 the k-th channel of the pixel block, k = 8 the tail; offsets
+    // of absent rows and channels are replaced by one that is always out of range
+    auto load_one = [&](auto tag, int32_t row0, LoadRegs &L) {
+      constexpr int k = decltype(tag)::value;
       const int32_t i = row0 + (int32_t)lrow;
       const int32_t arow = arow0 + i;
       const uint32_t rowkeep = (i >= 0 && arow >= 0 && arow < (int32_t)P.IH) ? 0xffffffffu : 0u;
       const uint32_t step_off = (uint32_t)(row0 * (int32_t)P.IW * 2);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t keep = vkeep[j] & rowkeep;
-        L.ld[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ((vch[j] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
+      if constexpr (k < 8) {
+        const uint32_t keep = vkeep[k] & rowkeep;
+        L.ld[k] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ((vch[k] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
+      } else {
+        const uint32_t keep = tkeep & rowkeep;
+        L.lt = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (((uint32_t)tbase + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
       }
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const uint32_t keep = tkeep[j] & rowkeep;
-        L.lt[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ((tch[j] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
-      }
-      tails_loaded = true;
+    };
+    auto issue = [&](int32_t row0, LoadRegs &L) {
+      for_each_int(std::make_integer_sequence<int, 9>(), [&](auto tag) { load_one(tag, row0, L); });
     };
 
     // the pieces of a row in ring order: eight pixels of eight channels each, plus this thread's
-    // share of the two tail pixels
+    // channel of the two tail pixels
     struct Transposed {
       u32x4 px[8];
-      uint32_t tail[2];
+      uint32_t tail;
       uint32_t dst, tdst;
     };
     // patches up what the range check dropped, then turns the loaded channel-major registers
@@ -229,22 +222,27 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
         }
         // The range check drops a dword that straddles the end of the image even though its low
         // half is the image's last element: fetch that element on its own.
-        if (arow == (int32_t)P.IH - 1 && chg == (P.Cred - 1u) >> 3) {
-          const uint32_t j = (P.Cred - 1u) & 7u;
-          const uint32_t v = (uint32_t)(vbase + row0 * (int32_t)P.IW * 2) + j * plane_bytes;
-          const uint32_t gap = image_bytes - 2u - v;  // distance of the last element from the load start
-          if (gap < 16u && (gap & 3u) == 0u) {
-            const uint32_t e = __builtin_amdgcn_raw_buffer_load_b16(rsrc, image_bytes - 2u, 0, 0) & 0xffffu;
-            const uint32_t d = gap >> 2;
+        if (arow == (int32_t)P.IH - 1) {
+          if (chg == (P.Cred - 1u) >> 3) {
+            const uint32_t j = (P.Cred - 1u) & 7u;
+            const uint32_t v = (uint32_t)(vbase + row0 * (int32_t)P.IW * 2) + j * plane_bytes;
+            const uint32_t gap = image_bytes - 2u - v;  // distance of the last element from the load start
+            if (gap < 16u && (gap & 3u) == 0u) {
+              const uint32_t e = __builtin_amdgcn_raw_buffer_load_b16(rsrc, image_bytes - 2u, 0, 0) & 0xffffu;
+              const uint32_t d = gap >> 2;
 #pragma unroll
-            for (int jj = 0; jj < 8; ++jj)
+              for (int jj = 0; jj < 8; ++jj)
 #pragma unroll
-              for (int dd = 0; dd < 4; ++dd) L.ld[jj][dd] |= ((uint32_t)jj == j && (uint32_t)dd == d) ? e : 0u;
+                for (int dd = 0; dd < 4; ++dd) L.ld[jj][dd] |= ((uint32_t)jj == j && (uint32_t)dd == d) ? e : 0u;
+            }
           }
+          if (tch == P.Cred - 1u && (uint32_t)(tbase + row0 * (int32_t)P.IW * 2) == image_bytes - 2u)
+            L.lt |= __builtin_amdgcn_raw_buffer_load_b16(rsrc, image_bytes - 2u, 0, 0) & 0xffffu;
         }
       }
       const uint32_t slot = (uint32_t)i % (uint32_t)kRingRows;
       T.dst = slot * kRowPitch + (pxb * 8u) * kPxPitch + chg * 16u;
+      T.tdst = slot * kRowPitch + kStripCols * kPxPitch + tch * 2u;
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
 #pragma unroll
@@ -254,26 +252,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
           T.px[2 * d + 1][q] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
         }
       }
-    };
-    // the same for this thread's two channels of the tail pixels, loaded into lt0 / lt1
-    auto transpose_tail = [&](int32_t row0, uint32_t lt0, uint32_t lt1, Transposed &T) {
-      const int32_t i = row0 + (int32_t)lrow;
-      if (arow0 + i == (int32_t)P.IH - 1 && chg == (P.Cred - 1u) >> 3) {
-        const uint32_t j = (P.Cred - 1u) & 7u;
-        if (pxb == (j >> 1)) {
-          const uint32_t t = (uint32_t)(tbase + row0 * (int32_t)P.IW * 2) + j * plane_bytes;
-          if (t == image_bytes - 2u) {
-            const uint32_t e = __builtin_amdgcn_raw_buffer_load_b16(rsrc, image_bytes - 2u, 0, 0) & 0xffffu;
-            lt0 |= (j & 1u) ? 0u : e;
-            lt1 |= (j & 1u) ? e : 0u;
-          }
-        }
-      }
-      const uint32_t slot = (uint32_t)i % (uint32_t)kRingRows;
-      T.tdst = slot * kRowPitch + kStripCols * kPxPitch + chg * 16u + pxb * 4u;
-      const uint32_t lo = lt0 & mt, hi = lt1 & mt;
-      T.tail[0] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-      T.tail[1] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+      T.tail = L.lt & mt;
     };
     // LDS write number w of a transposed row piece: 0..7 the pixels of the block, 8 and 9 the tail
     auto ring_write = [&](auto tag, const Transposed &T) {
@@ -281,28 +260,16 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
       if constexpr (w < 8)
         *reinterpret_cast<u32x4 *>(ring + T.dst + w * kPxPitch) = T.px[w];
       else
-        *reinterpret_cast<uint32_t *>(ring + T.tdst + (w - 8) * kPxPitch) = T.tail[w - 8];
+        *reinterpret_cast<uint16_t *>(ring + T.tdst + (w - 8) * kPxPitch) = (uint16_t)(T.tail >> ((w - 8) * 16));
     };
     auto commit = [&](int32_t row0, LoadRegs &L) {
-      if (!tails_loaded) {
-        // the step before ran the straight-line variant, which leaves the tails to its successor
-        const int32_t tarow = arow0 + row0 + (int32_t)lrow;
-        const uint32_t rowkeep = (tarow >= 0 && tarow < (int32_t)P.IH) ? 0xffffffffu : 0u;
-        const uint32_t step_off = (uint32_t)(row0 * (int32_t)P.IW * 2);
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const uint32_t keep = tkeep[j] & rowkeep;
-          L.lt[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ((tch[j] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
-        }
-      }
       if (row0 + (int32_t)lrow < 0) return;
       Transposed T;
       transpose(row0, L, T);
-      transpose_tail(row0, L.lt[0], L.lt[1], T);
       for_each_int(std::make_integer_sequence<int, 10>(), [&](auto tag) { ring_write(tag, T); });
     };
 
-    // ring-relative rows 0..9 of the first step
+    // ring-relative rows 0 .. kStepRows + 1 of the first step
     issue(2 - kStepRows, L0);
     issue(2, L1);
     commit(2 - kStepRows, L0);
@@ -310,35 +277,30 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
     if (nsteps > 1) issue(kStepRows + 2, L0);  // rows of step 1, committed at the start of step 0
     __syncthreads();
 
-    // Output of a step is kept packed in registers and stored at the start of the next step, so
-    // that the stores drain behind that step's MFMAs; for beta = 1 the old values are fetched at
-    // the start of their own step for the same reason.
-    const uint32_t ocol = (uint32_t)c0 + 16u * cb + 4u * g;
+    // Output.  The MFMA leaves a lane with four neighbouring columns of one output channel in
+    // each of its two column tiles; a swap between lane rows (v_permlane16_swap) turns that into
+    // eight neighbouring columns, so a store moves 16 bytes per lane and four lanes fill a
+    // 64-byte run.  The packed result of a step is stored during the next step.
+    const uint32_t ocol = (uint32_t)c0 + 32u * cw + ((g & 1u) ? 16u : 0u) + (g >> 1) * 8u;
     const uint32_t co0 = grp * 64u + 32u * h + l16;
     const bool ok_ct[2] = {co0 < P.Cout, co0 + 16u < P.Cout};
-    const bool full_cols = ocol + 3u < P.OW;
+    const bool full_cols = ocol + 7u < P.OW;
     const size_t ct_stride = (size_t)16u * P.OH * P.OW;
     uint16_t *const olane = out_img + (size_t)co0 * P.OH * P.OW + ocol;
-    u32x2 pk[2][kStepRows], old[2][kStepRows];
+    u32x4 pk[2][kStepRows], old[2][kStepRows];
 
-    // common case, decided per wave: all eight rows, both channel tiles, four whole columns
+    // common case, decided per wave: all rows of a step, both channel tiles, eight whole columns
     const bool lanes_whole = __builtin_amdgcn_ballot_w64(!(full_cols && ok_ct[0] && ok_ct[1])) == 0ull;
 
     auto store_packed = [&](uint32_t row0, uint32_t nrows) {
       uint16_t *obase = olane + (size_t)row0 * P.OW;
-      if (lanes_whole && nrows >= (uint32_t)kStepRows) {
-#pragma unroll
-        for (int ct = 0; ct < 2; ++ct)
-#pragma unroll
-          for (int r = 0; r < kStepRows; ++r)
-            *reinterpret_cast<u32x2_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW) = pk[ct][r];
-      } else if (full_cols) {
+      if (full_cols) {
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
           for (int r = 0; r < kStepRows; ++r)
             if ((uint32_t)r < nrows && ok_ct[ct])
-              *reinterpret_cast<u32x2_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW) = pk[ct][r];
+              *reinterpret_cast<u32x4_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW) = pk[ct][r];
       } else if (ocol < P.OW) {
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct)
@@ -347,7 +309,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
             if ((uint32_t)r < nrows && ok_ct[ct]) {
               uint16_t *p = obase + ct * ct_stride + (size_t)r * P.OW;
 #pragma unroll
-              for (int e = 0; e < 4; ++e)
+              for (int e = 0; e < 8; ++e)
                 if (ocol + e < P.OW) p[e] = (uint16_t)(pk[ct][r][e >> 1] >> ((e & 1) * 16));
             }
       }
@@ -355,55 +317,43 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
     auto load_old = [&](uint32_t row0, uint32_t nrows) {
       if (!BETA) return;
       const uint16_t *obase = olane + (size_t)row0 * P.OW;
-      if (lanes_whole && nrows >= (uint32_t)kStepRows) {
 #pragma unroll
-        for (int ct = 0; ct < 2; ++ct)
+      for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
-          for (int r = 0; r < kStepRows; ++r)
-            old[ct][r] = *reinterpret_cast<const u32x2_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW);
-      } else if (full_cols) {
+        for (int r = 0; r < kStepRows; ++r) {
+          old[ct][r] = (u32x4){0u, 0u, 0u, 0u};
+          if ((uint32_t)r < nrows && ok_ct[ct]) {
+            const uint16_t *p = obase + ct * ct_stride + (size_t)r * P.OW;
+            if (full_cols) {
+              old[ct][r] = *reinterpret_cast<const u32x4_unaligned *>(p);
+            } else if (ocol < P.OW) {
 #pragma unroll
-        for (int ct = 0; ct < 2; ++ct)
-#pragma unroll
-          for (int r = 0; r < kStepRows; ++r)
-            if ((uint32_t)r < nrows && ok_ct[ct])
-              old[ct][r] = *reinterpret_cast<const u32x2_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW);
-      } else if (ocol < P.OW) {
-#pragma unroll
-        for (int ct = 0; ct < 2; ++ct)
-#pragma unroll
-          for (int r = 0; r < kStepRows; ++r)
-            if ((uint32_t)r < nrows && ok_ct[ct]) {
-              const uint16_t *p = obase + ct * ct_stride + (size_t)r * P.OW;
-              uint32_t e4[4];
-#pragma unroll
-              for (int e = 0; e < 4; ++e) e4[e] = ocol + e < P.OW ? (uint32_t)p[e] : 0u;
-              old[ct][r][0] = e4[0] | (e4[1] << 16);
-              old[ct][r][1] = e4[2] | (e4[3] << 16);
+              for (int e = 0; e < 8; ++e)
+                if (ocol + e < P.OW) old[ct][r][e >> 1] |= (uint32_t)p[e] << ((e & 1) * 16);
             }
-      }
+          }
+        }
     };
 
     uint32_t sb = 0;  // ring slot of this step's first input row
     uint32_t prev_row0 = 0, prev_nrows = 0;
 
-    // The matrix part of a step: 60 operand reads (input row, column shift, channel half), each
-    // fetched kAhead reads before its MFMAs so that the LDS latency hides behind the matrix pipe,
-    // then the results are packed to bf16.  kVm global-memory instructions issued just before
-    // are spread over the first rounds, one per round: issued in a burst they would fill the
-    // memory pipeline's queue and hold every wave of the workgroup at the same point.
+    // The matrix part of a step: 72 operand reads (input row, column shift, channel half, column
+    // tile), each fetched kAhead reads before its MFMAs so that the LDS latency hides behind the
+    // matrix pipe; then the results are packed to bf16.  kVm global-memory instructions and kLds
+    // ring writes are spread over the rounds: issued in a burst they would fill the memory
+    // pipeline's queue and hold every wave of the workgroup at the same point.
     auto compute = [&](auto vm_tag, auto &&vm_op, auto lds_tag, auto &&lds_op) {
       constexpr int kVm = decltype(vm_tag)::value;
       constexpr int kLds = decltype(lds_tag)::value;
-      floatx4 acc[kStepRows][2];
+      floatx4 acc[kStepRows][2][2];
 #pragma unroll
       for (int r = 0; r < kStepRows; ++r)
 #pragma unroll
-        for (int ct = 0; ct < 2; ++ct) acc[r][ct] = (floatx4){0.f, 0.f, 0.f, 0.f};
-      #ifndef EXP_AHEAD
-#define EXP_AHEAD 3
-#endif
-      constexpr int kReads = (kStepRows + 2) * 6, kAhead = EXP_AHEAD;
+        for (int cti = 0; cti < 2; ++cti)
+#pragma unroll
+          for (int ct = 0; ct < 2; ++ct) acc[r][cti][ct] = (floatx4){0.f, 0.f, 0.f, 0.f};
+      constexpr int kReads = (kStepRows + 2) * 12, kAhead = 3;
       uint32_t row_addr[kStepRows + 2];
 #pragma unroll
       for (int ir = 0; ir < kStepRows + 2; ++ir) {
@@ -413,74 +363,75 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
       }
       u32x4 abuf[kAhead + 1];
       auto fetch = [&](int t) {
-        const int ir = t / 6, kw = (t % 6) >> 1, half = t & 1;
-        abuf[t % (kAhead + 1)] =
-            *reinterpret_cast<const u32x4 *>(ring + row_addr[ir] + read_lane_base + kw * kPxPitch + half * 64);
+        const int ir = t / 12, kw = (t % 12) >> 2, half = (t >> 1) & 1, cti = t & 1;
+        abuf[t % (kAhead + 1)] = *reinterpret_cast<const u32x4 *>(ring + row_addr[ir] + read_lane_base +
+                                                                  (cti * 16 + kw) * kPxPitch + half * 64);
       };
 #pragma unroll
       for (int t = 0; t < kAhead; ++t) fetch(t);
       __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
       auto round = [&](auto tag) {
         constexpr int t = decltype(tag)::value;
-#ifndef EXP_NO_MFMA
         if constexpr (t + kAhead < kReads) {
           fetch(t + kAhead);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
-#endif
-        constexpr int ir = t / 6, kw = (t % 6) >> 1, half = t & 1;
+        constexpr int ir = t / 12, kw = (t % 12) >> 2, half = (t >> 1) & 1, cti = t & 1;
         const bf16x8 a = __builtin_bit_cast(bf16x8, abuf[t % (kAhead + 1)]);
         constexpr int kh_lo = ir - (kStepRows - 1) > 0 ? ir - (kStepRows - 1) : 0;
         constexpr int kh_hi = ir < 2 ? ir : 2;
-#ifndef EXP_NO_MFMA
 #pragma unroll
         for (int kh = kh_lo; kh <= kh_hi; ++kh) {
 #pragma unroll
           for (int ct = 0; ct < 2; ++ct)
-            acc[ir - kh][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                a, __builtin_bit_cast(bf16x8, wreg[kh * 3 + kw][half][ct]), acc[ir - kh][ct], 0, 0, 0);
+            acc[ir - kh][cti][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                a, __builtin_bit_cast(bf16x8, wreg[kh * 3 + kw][half][ct]), acc[ir - kh][cti][ct], 0, 0, 0);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 2 * (kh_hi - kh_lo + 1), 0);
-#else
-        if constexpr (t == 0) acc[0][0] += __builtin_bit_cast(floatx4, a);
-#endif
-        // LDS write w goes after round 5 w + 2
-        if constexpr (t % 5 == 2 && t / 5 < kLds) {
-          lds_op(IntTag<t / 5>());
+        // ring write w goes after round 7 w + 3
+        if constexpr (t % 7 == 3 && t / 7 < kLds) {
+          lds_op(IntTag<t / 7>());
           __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
-        // Memory instructions, one per round from the start of the step: first the stores of
-        // the previous step's results, then the loads.  At the start of a step no load of this
-        // workgroup is in flight, and the L1 takes stores quickly only then: a store behind
-        // pending loads waits for them.
-        if constexpr (t < kVm) {
-          vm_op(IntTag<t>());
-          __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        // memory instruction i goes after round floor(i * kReads / kVm)
+        if constexpr (kVm > 0) {
+          constexpr int i = (t * kVm + kReads - 1) / kReads;  // first i with i * kReads >= t * kVm
+          if constexpr (i < kVm && (i * kReads) / kVm == t) {
+            vm_op(IntTag<i>());
+            __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+          }
         }
       };
       for_each_int(std::make_integer_sequence<int, kReads>(), round);
       __builtin_amdgcn_sched_barrier(0);
 
-      // lane (l16, g) holds output channel l16 of its tile, columns 4g..4g+3
 #pragma unroll
       for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
         for (int r = 0; r < kStepRows; ++r) {
-          floatx4 v = acc[r][ct];
+          floatx4 v0 = acc[r][0][ct], v1 = acc[r][1][ct];
           if (BETA) {
-            v[0] += __uint_as_float(old[ct][r][0] << 16);
-            v[1] += __uint_as_float(old[ct][r][0] & 0xffff0000u);
-            v[2] += __uint_as_float(old[ct][r][1] << 16);
-            v[3] += __uint_as_float(old[ct][r][1] & 0xffff0000u);
+            // back to the MFMA's arrangement: the swap is its own inverse
+            const u32x2 s0 = __builtin_amdgcn_permlane16_swap(old[ct][r][0], old[ct][r][2], false, false);
+            const u32x2 s1 = __builtin_amdgcn_permlane16_swap(old[ct][r][1], old[ct][r][3], false, false);
+            v0[0] += __uint_as_float(s0[0] << 16);
+            v0[1] += __uint_as_float(s0[0] & 0xffff0000u);
+            v0[2] += __uint_as_float(s1[0] << 16);
+            v0[3] += __uint_as_float(s1[0] & 0xffff0000u);
+            v1[0] += __uint_as_float(s0[1] << 16);
+            v1[1] += __uint_as_float(s0[1] & 0xffff0000u);
+            v1[2] += __uint_as_float(s1[1] << 16);
+            v1[3] += __uint_as_float(s1[1] & 0xffff0000u);
           }
-          pk[ct][r][0] = pack_bf16x2(v[0], v[1]);
-          pk[ct][r][1] = pack_bf16x2(v[2], v[3]);
+          const u32x2 q0 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[0], v0[1]), pack_bf16x2(v1[0], v1[1]), false, false);
+          const u32x2 q1 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[2], v0[3]), pack_bf16x2(v1[2], v1[3]), false, false);
+          pk[ct][r] = (u32x4){q0[0], q1[0], q0[1], q1[1]};
         }
     };
 
-    // One step.  The rows of step s + 1, requested a whole step ago, go into the ring first (they
-    // land in slots this step does not read); then the rows of step s + 2 are requested.  Every
-    // wait on memory therefore only covers requests that are at least one step old.
+    // One step.  The rows of step s + 1, requested a whole step ago, are turned into ring order
+    // first (they go to slots this step does not read); then the rows of step s + 2 are
+    // requested.  Every wait on memory therefore only covers requests that are a step old.
     for (uint32_t s = 0; s < nsteps; ++s) {
       const bool more = s + 1 < nsteps, more2 = s + 2 < nsteps;
       const int32_t next_row0 = (int32_t)((s + 1) * kStepRows) + 2;
@@ -505,52 +456,25 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
       if (fast) {
         // straight-line variant: every memory instruction is unconditional (rows requested
         // past the end of the segment are never used)
-        // A tail pixel shares its 128-byte line with the row's main pieces.  Requested right
-        // behind them it would find that line still on its way and hold up the whole L1 queue,
-        // so the tails of the rows of step s + 1 are requested now, a step after their main
-        // pieces, and written at the end of this step.
-        const int32_t irow0 = next_row0 + kStepRows;
-        const int32_t li = irow0 + (int32_t)lrow, larow = arow0 + li;
-        const uint32_t rowkeep = (larow >= 0 && larow < (int32_t)P.IH) ? 0xffffffffu : 0u;
-        const uint32_t step_off = (uint32_t)(irow0 * (int32_t)P.IW * 2);
-        const int32_t tarow = arow0 + next_row0 + (int32_t)lrow;
-        const uint32_t trowkeep = (tarow >= 0 && tarow < (int32_t)P.IH) ? 0xffffffffu : 0u;
-        const uint32_t tstep_off = (uint32_t)(next_row0 * (int32_t)P.IW * 2);
-        uint32_t lt_now[2];
         uint16_t *const sbase = olane + (size_t)prev_row0 * P.OW;
         const uint16_t *const obase = olane + (size_t)row0 * P.OW;
-        compute(IntTag<BETA ? 42 : 26>(), [&](auto tag) {
+        compute(IntTag<BETA ? 25 : 17>(), [&](auto tag) {
           constexpr int t = decltype(tag)::value;
-#ifdef EXP_VM_NOSTORE
-          if constexpr (t < 16) return;
-#endif
-#ifdef EXP_VM_NOLOAD
-          if constexpr (t >= 16) return;
-#endif
-          if constexpr (t < 16) {
-            constexpr int ct = t / kStepRows, r = t % kStepRows;
-            *reinterpret_cast<u32x2_unaligned *>(sbase + ct * ct_stride + (size_t)r * P.OW) = pk[ct][r];
-          } else if constexpr (t < 18) {
-            constexpr int j = t - 16;
-            const uint32_t keep = tkeep[j] & trowkeep;
-            lt_now[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ((tch[j] + tstep_off) & keep) | (kOutOfRange & ~keep), 0, 0);
-          } else if constexpr (t < 26) {
-            constexpr int j = t - 18;
-            const uint32_t keep = vkeep[j] & rowkeep;
-            L0.ld[j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ((vch[j] + step_off) & keep) | (kOutOfRange & ~keep), 0, 0);
+          if constexpr (t < 9) {
+            load_one(tag, next_row0 + kStepRows, L0);
+          } else if constexpr (BETA && t < 17) {
+            constexpr int ct = (t - 9) / kStepRows, r = (t - 9) % kStepRows;
+            old[ct][r] = *reinterpret_cast<const u32x4_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW);
           } else {
-            constexpr int ct = (t - 26) / kStepRows, r = (t - 26) % kStepRows;
-            old[ct][r] = *reinterpret_cast<const u32x2_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW);
+            constexpr int u = t - (BETA ? 17 : 9);
+            constexpr int ct = u / kStepRows, r = u % kStepRows;
+            *reinterpret_cast<u32x4_unaligned *>(sbase + ct * ct_stride + (size_t)r * P.OW) = pk[ct][r];
           }
-        }, IntTag<8>(), [&](auto tag) { ring_write(tag, T); });
-        transpose_tail(next_row0, lt_now[0], lt_now[1], T);
-        ring_write(IntTag<8>(), T);
-        ring_write(IntTag<9>(), T);
-        tails_loaded = false;
+        }, IntTag<10>(), [&](auto tag) { ring_write(tag, T); });
       } else {
         if (more2) issue(next_row0 + kStepRows, L0);
         if (s > 0) store_packed(prev_row0, prev_nrows);
-        if (BETA) load_old(row0, nrows);
+        load_old(row0, nrows);
         compute(IntTag<0>(), [](auto) {}, IntTag<0>(), [](auto) {});
       }
       prev_row0 = row0;
