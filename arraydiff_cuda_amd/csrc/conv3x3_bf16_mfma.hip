@@ -1,21 +1,26 @@
 // 3x3 slab convolution on the bf16 matrix cores (v_mfma_f32_16x16x32_bf16), forward and
 // backward-data, for up to 64 reduction channels.
 //
-// Shape of the computation.  A workgroup of four waves is persistent: it walks work items
-// (image, 32-column strip, row segment) and, inside an item, steps down the strip eight output
-// rows at a time.  The input rows of the strip live in LDS as a ring of 18 rows in
-// [pixel][channel] order (144 bytes per pixel: 64 channels + 16 bytes of padding, which makes the
-// 16-byte operand reads of 16 neighbouring pixels hit 64 distinct banks), so each input row is
-// fetched from HBM exactly once per strip; only the one-pixel column halo of a strip is read twice.
-// NCHW rows are turned into that order on the way in: a thread loads eight channels x eight
-// pixels (eight 16-byte buffer loads), transposes the 8x8 block of 16-bit values with byte
-// permutes and writes eight 16-byte LDS rows.
+// Shape of the computation.  A workgroup of four waves (one per SIMD, which leaves each wave the
+// whole register file) is persistent: it walks work items (image, 64-column strip, row segment)
+// and, inside an item, steps down the strip four output rows at a time.  The input rows of the
+// strip live in LDS as a ring of ten rows in [pixel][channel] order, so each input row is fetched
+// from HBM once per strip; only the one-pixel column halo of a strip is read twice.  NCHW rows
+// are turned into that order on the way in: a thread loads eight channels x eight pixels (eight
+// 16-byte buffer loads), transposes the 8x8 block of 16-bit values with byte permutes and writes
+// eight 16-byte LDS pieces.
 //
-// A wave owns 32 output channels x 16 columns x 8 rows.  Its share of the filter, 9 taps x 64
+// A wave owns 32 output channels x 32 columns x 4 rows.  Its share of the filter, 9 taps x 64
 // reduction channels x 32 output channels, is loaded once per kernel into 144 registers in matrix
-// operand order and never touches LDS.  Per step a wave reads 10 input rows x 3 column shifts x
-// 2 channel halves = 60 pixel operands and issues 288 MFMAs: an operand read for input row r
-// serves the output rows r, r-1, r-2 (taps kh = 0, 1, 2).
+// operand order and never touches LDS.  Per step a wave reads 6 input rows x 3 column shifts x
+// 2 channel halves x 2 column tiles = 72 pixel operands and issues 288 MFMAs: an operand read
+// for input row r serves the output rows r, r-1, r-2 (taps kh = 0, 1, 2).
+//
+// What bounds the kernel is the number of global-memory instructions, not their bytes: an
+// instruction that touches 16 separate short runs costs the memory pipeline the same whatever
+// the run length.  Hence 64-column strips (128-byte runs per channel row on the way in) and, on
+// the way out, a swap between lane rows that turns the MFMA's four columns per lane into eight,
+// so that four lanes fill a 64-byte run per store.
 //
 // Out-of-range rows, channels and buffer ends are handled by the buffer resource's range check
 // (out-of-range dwords read as zero); out-of-range columns by per-dword masks.
@@ -35,9 +40,16 @@ constexpr int kStripCols = 64;                        // output columns per work
 constexpr int kStepRows = 4;                          // output rows per step
 constexpr int kRingRows = 10;                         // 6 rows in use + 4 rows being written
 constexpr int kPatchCols = kStripCols + 2;            // 66
-constexpr int kPxPitch = 144;                         // bytes per pixel in LDS
-constexpr int kRowPitch = kPatchCols * kPxPitch;      // 9504
-constexpr int kRingBytes = kRingRows * kRowPitch;     // 95040
+// LDS layout of a ring row: pixel px sits in slot px + px / 8 (one empty slot after every eight
+// pixels), 160 bytes per slot (64 channels + 32 bytes of padding).  Measured on gfx950 with four
+// waves: the 16-byte operand reads of 16 neighbouring pixels run at the rate of a linear read,
+// and the loader's writes (eight lanes eight pixels apart) at 64 cycles instead of the 256 of a
+// dense 144-byte layout.
+constexpr int kPxPitch = 160;
+constexpr int kRowSlots = kPatchCols + kPatchCols / 8;   // 74
+constexpr int kRowPitch = kRowSlots * kPxPitch;       // 11840
+constexpr int kRingBytes = kRingRows * kRowPitch;     // 118400
+__host__ __device__ constexpr int px_slot(int px) { return px + (px >> 3); }
 constexpr uint32_t kOutOfRange = 0x80000000u;
 constexpr uint32_t kWtGroupElems = 9u * 2u * 64u * 32u;  // transformed filter elements per group of 64 outputs
 
@@ -122,17 +134,18 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
   for (int j = 0; j < 8; ++j) chvalid |= (chg * 8u + j < P.Cred ? 1u : 0u) << j;
   const uint32_t tkeep = tch < P.Cred ? 0xffffffffu : 0u;
 
-  // operand reads: pixel (32 cw + l16) of a ring row, channels 8 g .. 8 g + 7 of a half
-  const uint32_t read_lane_base = (32u * cw + l16) * kPxPitch + g * 16u;
+  // operand reads: pixel (32 cw + 16 cti + l16 + kw) of a ring row, channels 8 g .. 8 g + 7 of a half
+  uint32_t read_lane_off[2][3];
+#pragma unroll
+  for (int cti = 0; cti < 2; ++cti)
+#pragma unroll
+    for (int kw = 0; kw < 3; ++kw)
+      read_lane_off[cti][kw] = (uint32_t)px_slot((int)(32u * cw + 16u * cti + l16) + kw) * kPxPitch + g * 16u;
 
   // Workgroups are dealt to the eight XCDs (each with its own L2) in turn.  Renumber them so
   // that an XCD works on neighbouring strips: those share the 128-byte lines at strip borders.
   uint32_t vblock = blockIdx.x;
   if ((gridDim.x & 7u) == 0u) vblock = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-#ifdef EXP_TIMING
-  uint64_t tacc[4] = {0, 0, 0, 0};
-  const uint64_t tstart = __builtin_readcyclecounter();
-#endif
   for (uint32_t item = vblock; item < P.items; item += gridDim.x) {
     uint32_t strip, t1, seg, plane, tile, n;
     P.div_strips.divmod(item, t1, strip);
@@ -205,9 +218,9 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
       uint32_t tail;
       uint32_t dst, tdst;
     };
-    // patches up what the range check dropped, then turns the loaded channel-major registers
-    // into pixel-major pieces; the caller makes sure that ring row row0 + lrow is not negative
-    auto transpose = [&](int32_t row0, LoadRegs &L, Transposed &T) {
+    // patches up what the range check dropped and works out where the row goes in the ring; the
+    // caller makes sure that ring row row0 + lrow is not negative
+    auto transpose_prepare = [&](int32_t row0, LoadRegs &L, Transposed &T) {
       const int32_t i = row0 + (int32_t)lrow;
       {
         const int32_t arow = arow0 + i;
@@ -241,18 +254,20 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
         }
       }
       const uint32_t slot = (uint32_t)i % (uint32_t)kRingRows;
-      T.dst = slot * kRowPitch + (pxb * 8u) * kPxPitch + chg * 16u;
-      T.tdst = slot * kRowPitch + kStripCols * kPxPitch + tch * 2u;
+      T.dst = slot * kRowPitch + (uint32_t)px_slot((int)(pxb * 8u)) * kPxPitch + chg * 16u;
+      T.tdst = slot * kRowPitch + px_slot(kStripCols) * kPxPitch + tch * 2u;
+    };
+    // piece d of the transposition: dword d of the eight channel registers -> pixels 2d, 2d + 1
+    // (d = 0 also takes the tail along)
+    auto transpose_piece = [&](auto tag, const LoadRegs &L, Transposed &T) {
+      constexpr int d = decltype(tag)::value;
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const uint32_t lo = L.ld[2 * q][d] & md[d], hi = L.ld[2 * q + 1][d] & md[d];
-          T.px[2 * d][q] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-          T.px[2 * d + 1][q] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
-        }
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t lo = L.ld[2 * q][d] & md[d], hi = L.ld[2 * q + 1][d] & md[d];
+        T.px[2 * d][q] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        T.px[2 * d + 1][q] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
       }
-      T.tail = L.lt & mt;
+      if constexpr (d == 0) T.tail = L.lt & mt;
     };
     // LDS write number w of a transposed row piece: 0..7 the pixels of the block, 8 and 9 the tail
     auto ring_write = [&](auto tag, const Transposed &T) {
@@ -265,7 +280,8 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
     auto commit = [&](int32_t row0, LoadRegs &L) {
       if (row0 + (int32_t)lrow < 0) return;
       Transposed T;
-      transpose(row0, L, T);
+      transpose_prepare(row0, L, T);
+      for_each_int(std::make_integer_sequence<int, 4>(), [&](auto tag) { transpose_piece(tag, L, T); });
       for_each_int(std::make_integer_sequence<int, 10>(), [&](auto tag) { ring_write(tag, T); });
     };
 
@@ -343,7 +359,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
     // matrix pipe; then the results are packed to bf16.  kVm global-memory instructions and kLds
     // ring writes are spread over the rounds: issued in a burst they would fill the memory
     // pipeline's queue and hold every wave of the workgroup at the same point.
-    auto compute = [&](auto vm_tag, auto &&vm_op, auto lds_tag, auto &&lds_op) {
+    auto compute = [&](auto vm_tag, auto &&vm_op, auto lds_tag, auto &&lds_op, auto &&valu_op) {
       constexpr int kVm = decltype(vm_tag)::value;
       constexpr int kLds = decltype(lds_tag)::value;
       floatx4 acc[kStepRows][2][2];
@@ -361,11 +377,36 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
         slot = slot >= (uint32_t)kRingRows ? slot - (uint32_t)kRingRows : slot;
         row_addr[ir] = slot * kRowPitch;
       }
+      u32x4 pk_next[2][kStepRows];
+      // packs output row r of this step to bf16 in store order
+      auto pack_row = [&](auto rtag) {
+        constexpr int r = decltype(rtag)::value;
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) {
+          floatx4 v0 = acc[r][0][ct], v1 = acc[r][1][ct];
+          if (BETA) {
+            // back to the MFMA's arrangement: the swap is its own inverse
+            const u32x2 s0 = __builtin_amdgcn_permlane16_swap(old[ct][r][0], old[ct][r][2], false, false);
+            const u32x2 s1 = __builtin_amdgcn_permlane16_swap(old[ct][r][1], old[ct][r][3], false, false);
+            v0[0] += __uint_as_float(s0[0] << 16);
+            v0[1] += __uint_as_float(s0[0] & 0xffff0000u);
+            v0[2] += __uint_as_float(s1[0] << 16);
+            v0[3] += __uint_as_float(s1[0] & 0xffff0000u);
+            v1[0] += __uint_as_float(s0[1] << 16);
+            v1[1] += __uint_as_float(s0[1] & 0xffff0000u);
+            v1[2] += __uint_as_float(s1[1] << 16);
+            v1[3] += __uint_as_float(s1[1] & 0xffff0000u);
+          }
+          const u32x2 q0 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[0], v0[1]), pack_bf16x2(v1[0], v1[1]), false, false);
+          const u32x2 q1 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[2], v0[3]), pack_bf16x2(v1[2], v1[3]), false, false);
+          pk_next[ct][r] = (u32x4){q0[0], q1[0], q0[1], q1[1]};
+        }
+      };
       u32x4 abuf[kAhead + 1];
       auto fetch = [&](int t) {
         const int ir = t / 12, kw = (t % 12) >> 2, half = (t >> 1) & 1, cti = t & 1;
-        abuf[t % (kAhead + 1)] = *reinterpret_cast<const u32x4 *>(ring + row_addr[ir] + read_lane_base +
-                                                                  (cti * 16 + kw) * kPxPitch + half * 64);
+        abuf[t % (kAhead + 1)] =
+            *reinterpret_cast<const u32x4 *>(ring + row_addr[ir] + read_lane_off[cti][kw] + half * 64);
       };
 #pragma unroll
       for (int t = 0; t < kAhead; ++t) fetch(t);
@@ -388,45 +429,33 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
                 a, __builtin_bit_cast(bf16x8, wreg[kh * 3 + kw][half][ct]), acc[ir - kh][cti][ct], 0, 0, 0);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 2 * (kh_hi - kh_lo + 1), 0);
-        // ring write w goes after round 7 w + 3
-        if constexpr (t % 7 == 3 && t / 7 < kLds) {
-          lds_op(IntTag<t / 7>());
+        // Rounds 0..3: the four pieces of the transposition of the rows loaded a step ago (they
+        // read the registers the loads below refill).  Ring write w goes after round 6 w + 4,
+        // memory instruction i after round 4 + floor(i * (kReads - 4) / kVm).
+        if constexpr (kLds > 0 && t < 4) valu_op(IntTag<t>());
+        if constexpr (t >= 4 && (t - 4) % 6 == 0 && (t - 4) / 6 < kLds) {
+          lds_op(IntTag<(t - 4) / 6>());
           __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
-        // memory instruction i goes after round floor(i * kReads / kVm)
-        if constexpr (kVm > 0) {
-          constexpr int i = (t * kVm + kReads - 1) / kReads;  // first i with i * kReads >= t * kVm
-          if constexpr (i < kVm && (i * kReads) / kVm == t) {
+        if constexpr (kVm > 0 && t >= 4) {
+          constexpr int span = kReads - 4, u = t - 4;
+          constexpr int i = (u * kVm + span - 1) / span;  // first i with i * span >= u * kVm
+          if constexpr (i < kVm && (i * span) / kVm == u) {
             vm_op(IntTag<i>());
             __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
           }
         }
+        // an output row is complete once the input row two below it has been through; its
+        // packing is dealt out over the next rounds
       };
       for_each_int(std::make_integer_sequence<int, kReads>(), round);
       __builtin_amdgcn_sched_barrier(0);
-
+      for_each_int(std::make_integer_sequence<int, kStepRows>(), pack_row);
+      // pk itself is still being stored while the rounds run
 #pragma unroll
       for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
-        for (int r = 0; r < kStepRows; ++r) {
-          floatx4 v0 = acc[r][0][ct], v1 = acc[r][1][ct];
-          if (BETA) {
-            // back to the MFMA's arrangement: the swap is its own inverse
-            const u32x2 s0 = __builtin_amdgcn_permlane16_swap(old[ct][r][0], old[ct][r][2], false, false);
-            const u32x2 s1 = __builtin_amdgcn_permlane16_swap(old[ct][r][1], old[ct][r][3], false, false);
-            v0[0] += __uint_as_float(s0[0] << 16);
-            v0[1] += __uint_as_float(s0[0] & 0xffff0000u);
-            v0[2] += __uint_as_float(s1[0] << 16);
-            v0[3] += __uint_as_float(s1[0] & 0xffff0000u);
-            v1[0] += __uint_as_float(s0[1] << 16);
-            v1[1] += __uint_as_float(s0[1] & 0xffff0000u);
-            v1[2] += __uint_as_float(s1[1] << 16);
-            v1[3] += __uint_as_float(s1[1] & 0xffff0000u);
-          }
-          const u32x2 q0 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[0], v0[1]), pack_bf16x2(v1[0], v1[1]), false, false);
-          const u32x2 q1 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[2], v0[3]), pack_bf16x2(v1[2], v1[3]), false, false);
-          pk[ct][r] = (u32x4){q0[0], q1[0], q0[1], q1[1]};
-        }
+        for (int r = 0; r < kStepRows; ++r) pk[ct][r] = pk_next[ct][r];
     };
 
     // One step.  The rows of step s + 1, requested a whole step ago, are turned into ring order
@@ -435,24 +464,18 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
     for (uint32_t s = 0; s < nsteps; ++s) {
       const bool more = s + 1 < nsteps, more2 = s + 2 < nsteps;
       const int32_t next_row0 = (int32_t)((s + 1) * kStepRows) + 2;
-#ifdef EXP_TIMING
-      const uint64_t tq0 = __builtin_readcyclecounter();
-#endif
       const uint32_t row0 = r_begin + s * kStepRows;
       const uint32_t nrows = r_end - row0;  // rows >= nrows of this step do not exist
       const bool fast = lanes_whole && s > 0 && nrows >= (uint32_t)kStepRows;
       Transposed T;
       if (fast)
-        transpose(next_row0, L0, T);  // written to the ring between the MFMAs below
+        transpose_prepare(next_row0, L0, T);  // transposed and written to the ring between the MFMAs below
       else if (more)
         commit(next_row0, L0);
       // Everything still in flight here (the previous step's stores) is a step old.  Draining it
       // explicitly keeps the compiler from guarding register reuse further down with waits that
       // would also cover the requests this step is about to issue.
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-#ifdef EXP_TIMING
-      const uint64_t tq1 = __builtin_readcyclecounter();
-#endif
       if (fast) {
         // straight-line variant: every memory instruction is unconditional (rows requested
         // past the end of the segment are never used)
@@ -460,45 +483,32 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
         const uint16_t *const obase = olane + (size_t)row0 * P.OW;
         compute(IntTag<BETA ? 25 : 17>(), [&](auto tag) {
           constexpr int t = decltype(tag)::value;
-          if constexpr (t < 9) {
-            load_one(tag, next_row0 + kStepRows, L0);
-          } else if constexpr (BETA && t < 17) {
-            constexpr int ct = (t - 9) / kStepRows, r = (t - 9) % kStepRows;
+          // beta = 1: the old values first, in the order the rows are packed
+          if constexpr (BETA && t < 8) {
+            constexpr int ct = t & 1, r = t >> 1;
             old[ct][r] = *reinterpret_cast<const u32x4_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW);
+          } else if constexpr (t < (BETA ? 17 : 9)) {
+            load_one(IntTag<t - (BETA ? 8 : 0)>(), next_row0 + kStepRows, L0);
           } else {
             constexpr int u = t - (BETA ? 17 : 9);
             constexpr int ct = u / kStepRows, r = u % kStepRows;
             *reinterpret_cast<u32x4_unaligned *>(sbase + ct * ct_stride + (size_t)r * P.OW) = pk[ct][r];
           }
-        }, IntTag<10>(), [&](auto tag) { ring_write(tag, T); });
+        }, IntTag<10>(), [&](auto tag) { ring_write(tag, T); }, [&](auto tag) { transpose_piece(tag, L0, T); });
       } else {
         if (more2) issue(next_row0 + kStepRows, L0);
         if (s > 0) store_packed(prev_row0, prev_nrows);
         load_old(row0, nrows);
-        compute(IntTag<0>(), [](auto) {}, IntTag<0>(), [](auto) {});
+        compute(IntTag<0>(), [](auto) {}, IntTag<0>(), [](auto) {}, [](auto) {});
       }
       prev_row0 = row0;
       prev_nrows = nrows;
-#ifdef EXP_TIMING
-      const uint64_t tq2 = __builtin_readcyclecounter();
-#endif
       __syncthreads();
-#ifdef EXP_TIMING
-      const uint64_t tq3 = __builtin_readcyclecounter();
-      tacc[0] += tq1 - tq0; tacc[1] += tq2 - tq1; tacc[2] += tq3 - tq2; tacc[3] += 1;
-#endif
       sb += kStepRows;
       sb = sb >= (uint32_t)kRingRows ? sb - (uint32_t)kRingRows : sb;
     }
     store_packed(prev_row0, prev_nrows);
   }
-#ifdef EXP_TIMING
-  if (lane == 0) {
-    uint64_t *dbg = reinterpret_cast<uint64_t *>(const_cast<uint16_t *>(P.wt) + kWtGroupElems) + (blockIdx.x * 4 + wv) * 8;
-    dbg[0] = tacc[0]; dbg[1] = tacc[1]; dbg[2] = tacc[2]; dbg[3] = tacc[3];
-    dbg[4] = __builtin_readcyclecounter() - tstart;
-  }
-#endif
 }
 
 static int g_num_cus = 0;
