@@ -30,6 +30,7 @@ if ROOT not in sys.path:
 CONV_FWD_CFG2_TRAFFIC_BYTES = 64.07e6
 HBM_PEAK_GBS = 8000.0
 MFMA_F32_PEAK_TFLOPS = 157.3
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 METRIC = "halo pack/unpack GB/s (% HBM peak); 3x3 slab-conv TFLOP/s (% MFMA peak)"
 
 
@@ -222,7 +223,31 @@ def main():
         add("halo unpack cfg5 (bf16)",
             lambda: lib.adh_tiles_unpack_nchw(1, K5, 1, W5, H5, C, N5, t5_tbl, Y5.data_ptr(), stream),
             "hbm", 2 * b5, HBM_PEAK_GBS, "GB/s")
-        del X5, t5, Y5
+        # config 5 slab conv on the bf16 matrix cores: fwd, bwd-data (beta = 1, as the reference
+        # accumulates input gradients), bwd-filter (bf16 widened to fp32, fp32 MFMA)
+        Ht5 = H5 // K5
+        w5 = (torch.randn((C, C, 3, 3), device="cuda", generator=g) * (2.0 / (C * 9)) ** 0.5).to(torch.bfloat16)
+        y5 = [torch.empty((N5, C, Ht5, W5), device="cuda", dtype=torch.bfloat16) for _ in range(K5)]
+        y5_tbl, _ky = capi.ptr_table([t.data_ptr() for t in y5])
+        gw5 = torch.zeros((C, C, 3, 3), device="cuda")
+        ws5_bytes = max(lib.adh_conv3x3_workspace_bytes(wh, 1, K5, N5, C, C, Ht5, W5) for wh in (0, 1, 2))
+        ws5 = torch.empty(ws5_bytes // 4 + 64, device="cuda")
+        flops5 = 2.0 * K5 * N5 * C * C * 9 * Ht5 * W5
+        reps, wu = 20, 3
+        add("conv fwd cfg5 (bf16, 8 tiles)",
+            lambda: lib.adh_conv3x3_slab_fwd_tiles(1, K5, N5, C, C, Ht5, W5, t5_tbl, w5.data_ptr(), y5_tbl, 0.0,
+                                                   ws5.data_ptr(), ws5_bytes, stream),
+            "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
+        add("conv bwd-data cfg5 (bf16, beta=1)",
+            lambda: lib.adh_conv3x3_slab_bwd_data_tiles(1, K5, N5, C, C, Ht5, W5, w5.data_ptr(), y5_tbl, t5_tbl, 1.0,
+                                                        ws5.data_ptr(), ws5_bytes, stream),
+            "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
+        reps, wu = 5, 1
+        add("conv bwd-filter cfg5 (bf16 in, widened, fp32 MFMA)",
+            lambda: lib.adh_conv3x3_slab_bwd_filter_tiles(1, K5, N5, C, C, Ht5, W5, t5_tbl, y5_tbl, gw5.data_ptr(), 0.0,
+                                                          ws5.data_ptr(), ws5_bytes, stream),
+            "mfma", flops5, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+        del X5, t5, Y5, y5, ws5
         out["secondary"] = sec
 
     # ---- CPU baseline: the scalar port, single thread, on a bounded sample ----
