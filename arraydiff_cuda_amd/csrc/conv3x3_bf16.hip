@@ -66,8 +66,16 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
                    const void *const *in_tiles, const void *w, void *const *out_tiles, float beta, void *workspace,
                    hipStream_t st);
 
+bool conv_bf16_wgrad_mfma_supported(uint32_t Cin, uint32_t Cout, uint32_t W);
+size_t conv_bf16_wgrad_mfma_workspace_bytes(uint32_t num_tiles, uint32_t N, uint32_t W);
+int conv_bf16_wgrad_mfma(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                         const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta,
+                         void *workspace, hipStream_t st);
+
 size_t bf16_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                             uint32_t W, size_t fp32_path_bytes) {
+  if (which == ADH_CONV_BWD_FILTER && conv_bf16_wgrad_mfma_supported(Cin, Cout, W))
+    return conv_bf16_wgrad_mfma_workspace_bytes(num_tiles, N, W);
   if (which != ADH_CONV_BWD_FILTER && conv_bf16_mfma_supported(which, Cin, Cout))
     return conv_bf16_mfma_workspace_bytes(which, Cin, Cout);
   const uint64_t slab = (uint64_t)N * Cin * (H + 2) * (W + 2), out = (uint64_t)N * Cout * H * W;
@@ -163,6 +171,18 @@ int conv_bf16_filter_via_f32(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint3
     return adh_conv3x3_slab_bwd_filter_tiles(ADH_F32, num_tiles, N, Cin, Cout, H, W, x_tiles, dy_tiles, dw, beta,
                                              workspace, workspace_bytes, st);
   if (!x_tiles || !dy_tiles) return ADH_ENULL;
+  if (conv_bf16_wgrad_mfma_supported(Cin, Cout, W)) {
+    if (!workspace) return ADH_ENULL;
+    if (!aligned_to(workspace, 256) || !aligned_to(dw, 4)) return ADH_EALIGN;
+    if (workspace_bytes < conv_bf16_wgrad_mfma_workspace_bytes(num_tiles, N, W)) return ADH_EWORKSPACE;
+    // one image is addressed through a 32-bit buffer resource
+    if (64ull * (H + 2ull) * (W + 2ull) * 2u >= (1ull << 31)) return ADH_EINVAL;
+    for (uint32_t t = 0; t < num_tiles; ++t) {
+      if (!x_tiles[t] || !dy_tiles[t]) return ADH_ENULL;
+      if (!aligned_to(x_tiles[t], 2) || !aligned_to(dy_tiles[t], 2)) return ADH_EALIGN;
+    }
+    return conv_bf16_wgrad_mfma(num_tiles, N, Cin, Cout, H, W, x_tiles, dy_tiles, dw, beta, workspace, st);
+  }
   const size_t f32_bytes = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, num_tiles, N, Cin, Cout, H, W);
   if (f32_bytes == 0) return ADH_EUNIMPL;
   const size_t need = bf16_workspace_bytes(ADH_CONV_BWD_FILTER, num_tiles, N, Cin, Cout, H, W, f32_bytes);

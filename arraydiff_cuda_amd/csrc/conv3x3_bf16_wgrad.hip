@@ -1,0 +1,286 @@
+// Filter gradient of the 3x3 slab convolution on the bf16 matrix cores, for up to 64 input and
+// 64 output channels and image widths that are a multiple of eight:
+//   dw[co][ci][kh][kw] = sum over images, rows h, columns w of dy[co][h][w] * x_pad[ci][h+kh][w+kw]
+//
+// The reduction runs over pixels, and eight neighbouring pixels of a channel row are 16
+// contiguous bytes in NCHW, so both MFMA operands come straight from rows as they lie in memory:
+// A = dy (m = output channel, k = 32 columns), B = x_pad (k = 32 columns, n = input channel).
+// Rows are copied into LDS by `buffer_load ... lds` with 16 bytes per lane (asynchronous, no
+// registers), one row of x_pad and one of dy per stage, three stages.
+//
+// A workgroup of eight waves (two per SIMD) walks down a 64-column strip of one image.  A wave
+// owns one tile of 16 input channels, one half of the output channels (two tiles of 16) and all
+// nine taps: 18 accumulator tiles, fed by both 32-column halves of the strip.  x_pad row r meets
+// the dy rows r, r-1, r-2 (taps kh = 0, 1, 2); the three dy rows are kept in registers, so each
+// row step reads four dy operands and two x operands from LDS for 36 MFMAs.  The x operand for
+// column shift kw = 1 is made from the aligned 16 bytes and the next dword with four funnel
+// shifts, kw = 2 is the same five dwords taken one further: 16-byte LDS reads that are not
+// 16-byte aligned run nine times slower.
+//
+// Every wave keeps its sums over all the strips it visits and writes them once, its part of the
+// workgroup's partial filter; a second kernel adds the partials in a fixed order.
+#include <utility>
+
+#include "adh_common.h"
+
+namespace adh {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWgCols = 64;                       // dy columns per strip
+constexpr int kWgLanes = 9;                       // 16-byte lanes per channel row in LDS
+constexpr int kWgPitch = kWgLanes * 16;           // 144 bytes: 66 x_pad columns, or 64 dy columns + pad
+constexpr int kWgRegion = 64 * kWgPitch;          // 9216 bytes: 64 channel rows
+constexpr int kWgStageBytes = 2 * kWgRegion;      // x_pad row, then dy row
+constexpr int kWgDmaPerStage = kWgStageBytes / 1024;  // 18 wave-wide copies
+constexpr uint32_t kWgOutOfRange = 0x80000000u;
+constexpr uint32_t kWgPartialFloats = 64u * 64u * 9u;
+
+struct WgradBf16Params {
+  const uint16_t *x[ADH_MAX_TILES];
+  const uint16_t *dy[ADH_MAX_TILES];
+  float *partial;  // [gridDim.x][64 co][64 ci][9]
+  uint32_t N, Cin, Cout, H, W;
+  uint32_t strips, items;
+  FastDiv div_strips, div_N;
+};
+
+template <int V>
+struct WgTag { static constexpr int value = V; };
+
+__global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Params P) {
+  // one array per stage: the compiler can then tell the asynchronous writes of one stage from
+  // the reads of another
+  __shared__ __attribute__((aligned(16))) uint8_t stage0[kWgStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t stage1[kWgStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t stage2[kWgStageBytes];
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
+  const uint32_t wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t cit = wv & 3u, coh = wv >> 2;  // input-channel tile, output-channel half
+
+  floatx4 acc[3][3][2];
+#pragma unroll
+  for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+    for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+      for (int cot = 0; cot < 2; ++cot) acc[kh][kw][cot] = (floatx4){0.f, 0.f, 0.f, 0.f};
+
+  // operand addresses inside a stage, for the left 32 columns (+ 64 bytes for the right ones)
+  const uint32_t b_off = (16u * cit + l16) * kWgPitch + g * 16u;
+  const uint32_t a_off = kWgRegion + (32u * coh + l16) * kWgPitch + g * 16u;  // + cot * 16 * kWgPitch
+
+  // copies this wave issues per stage: numbers wv, wv + 8, wv + 16 of the 18
+  const uint32_t HP = P.H + 2u, WP = P.W + 2u;
+  const uint32_t last_row = P.H + 1u;
+
+  for (uint32_t item = blockIdx.x; item < P.items; item += gridDim.x) {
+    uint32_t strip, plane, tile, n;
+    P.div_strips.divmod(item, plane, strip);
+    P.div_N.divmod(plane, tile, n);
+    const uint32_t c0 = strip * kWgCols;
+    const uint16_t *x_img = P.x[tile] + (size_t)n * P.Cin * HP * WP;
+    const uint16_t *dy_img = P.dy[tile] + (size_t)n * P.Cout * P.H * P.W;
+    const __amdgpu_buffer_rsrc_t rsrc_x =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(x_img), 0, P.Cin * HP * WP * 2u, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_dy =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(dy_img), 0, P.Cout * P.H * P.W * 2u, 0x00020000);
+
+    // per-lane source offsets of row 0 for the (up to) three copies; out of range where the
+    // channel, the piece or the column does not exist
+    uint32_t voff[3];
+#pragma unroll
+    for (int q = 0; q < 3; ++q) {
+      const uint32_t k = wv + 8u * q;
+      const uint32_t j = (k % 9u) * 64u + lane;  // lane slot within the x_pad or dy region
+      const uint32_t ch = j / kWgLanes, piece = j - ch * kWgLanes;
+      if (k < 9u) {
+        voff[q] = ch < P.Cin ? (ch * HP * WP + c0 + piece * 8u) * 2u : kWgOutOfRange;
+      } else {
+        const uint32_t col = c0 + piece * 8u;
+        voff[q] = (ch < P.Cout && piece < 8u && col < P.W) ? (ch * P.H * P.W + col) * 2u : kWgOutOfRange;
+      }
+    }
+
+    auto dma_row = [&](uint32_t r, uint8_t *stage) {
+#pragma unroll
+      for (int q = 0; q < 3; ++q) {
+        const uint32_t k = wv + 8u * q;  // uniform
+        if (k >= (uint32_t)kWgDmaPerStage) continue;
+        uint8_t *dst = stage + k * 1024u;
+        if (k < 9u) {
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (__attribute__((address_space(3))) void *)dst, 16, voff[q],
+                                                   __builtin_amdgcn_readfirstlane(r * WP * 2u), 0, 0);
+        } else {
+          const uint32_t v = r < P.H ? voff[q] : kWgOutOfRange;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_dy, (__attribute__((address_space(3))) void *)dst, 16, v,
+                                                   __builtin_amdgcn_readfirstlane(r * P.W * 2u), 0, 0);
+        }
+      }
+    };
+
+    // dy rows r, r-1, r-2 as A operands: two column halves x two output-channel tiles each
+    u32x4 win[3][2][2];
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int cot = 0; cot < 2; ++cot) win[a][kb][cot] = (u32x4){0u, 0u, 0u, 0u};
+
+    __syncthreads();  // the previous item's last rows have been read
+    dma_row(0, stage0);
+    if (last_row >= 1u) dma_row(1, stage1);
+
+    // one row; PH = r mod 3 picks the stage and the window slot that takes the new dy row
+    auto step = [&](auto ph, uint32_t r, uint8_t *cur, uint8_t *nxt2) {
+      constexpr int PH = decltype(ph)::value;
+      // wait for this wave's copies of row r; those of row r + 1 may stay in flight
+      if (r + 1u <= last_row) {
+        if (wv < 2u) __builtin_amdgcn_s_waitcnt(0x0F70 | 3);
+        else __builtin_amdgcn_s_waitcnt(0x0F70 | 2);
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+      }
+      __syncthreads();  // row r is complete in LDS; everybody is done with row r - 1
+      if (r + 2u <= last_row) dma_row(r + 2u, nxt2);
+
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int cot = 0; cot < 2; ++cot)
+          win[PH][kb][cot] = *reinterpret_cast<const u32x4 *>(cur + a_off + cot * 16 * kWgPitch + kb * 64);
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const u32x4 b0 = *reinterpret_cast<const u32x4 *>(cur + b_off + kb * 64);
+        const uint32_t b4 = *reinterpret_cast<const uint32_t *>(cur + b_off + kb * 64 + 16);
+        u32x4 b1;
+        b1[0] = __builtin_amdgcn_alignbit(b0[1], b0[0], 16);
+        b1[1] = __builtin_amdgcn_alignbit(b0[2], b0[1], 16);
+        b1[2] = __builtin_amdgcn_alignbit(b0[3], b0[2], 16);
+        b1[3] = __builtin_amdgcn_alignbit(b4, b0[3], 16);
+        const u32x4 b2 = (u32x4){b0[1], b0[2], b0[3], b4};
+        const u32x4 bs[3] = {b0, b1, b2};
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh) {
+          const int slot = (PH + 3 - kh) % 3;  // dy row r - kh
+#pragma unroll
+          for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+            for (int cot = 0; cot < 2; ++cot)
+              acc[kh][kw][cot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  __builtin_bit_cast(bf16x8, win[slot][kb][cot]), __builtin_bit_cast(bf16x8, bs[kw]),
+                  acc[kh][kw][cot], 0, 0, 0);
+        }
+      }
+    };
+
+    for (uint32_t r = 0; r <= last_row; r += 3u) {
+      step(WgTag<0>(), r, stage0, stage2);
+      if (r + 1u <= last_row) step(WgTag<1>(), r + 1u, stage1, stage0);
+      if (r + 2u <= last_row) step(WgTag<2>(), r + 2u, stage2, stage1);
+    }
+  }
+
+  // D[m = 4 g + i][n = l16]: output channel 32 coh + 16 cot + 4 g + i, input channel 16 cit + l16
+  float *part = P.partial + (size_t)blockIdx.x * kWgPartialFloats;
+#pragma unroll
+  for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+    for (int kw = 0; kw < 3; ++kw)
+#pragma unroll
+      for (int cot = 0; cot < 2; ++cot)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t co = 32u * coh + 16u * cot + 4u * g + i, ci = 16u * cit + l16;
+          part[(co * 64u + ci) * 9u + kh * 3 + kw] = acc[kh][kw][cot][i];
+        }
+}
+
+// dw[co][ci][tap] = beta * dw + sum over partials, in a fixed order: 64 elements per workgroup,
+// four quarters of the partials in parallel
+__global__ __launch_bounds__(256) void conv3x3_bf16_wgrad_reduce_kernel(const float *__restrict__ partial,
+                                                                        uint32_t num_partials, float *dw, uint32_t Cin,
+                                                                        uint32_t Cout, float beta) {
+  __shared__ float part[4][64];
+  const uint32_t q = threadIdx.x >> 6, j = threadIdx.x & 63u;
+  const uint32_t e = blockIdx.x * 64u + j;
+  const uint32_t total = Cout * Cin * 9u;
+  float s = 0.f;
+  if (e < total) {
+    const uint32_t tap = e % 9u, cc = e / 9u, ci = cc % Cin, co = cc / Cin;
+    const float *p = partial + (co * 64u + ci) * 9u + tap;
+    const uint32_t per = (num_partials + 3u) / 4u;
+    const uint32_t b0 = q * per, b1 = min(b0 + per, num_partials);
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    uint32_t b = b0;
+    for (; b + 4u <= b1; b += 4u) {
+      s0 += p[(size_t)(b + 0u) * kWgPartialFloats];
+      s1 += p[(size_t)(b + 1u) * kWgPartialFloats];
+      s2 += p[(size_t)(b + 2u) * kWgPartialFloats];
+      s3 += p[(size_t)(b + 3u) * kWgPartialFloats];
+    }
+    for (; b < b1; ++b) s0 += p[(size_t)b * kWgPartialFloats];
+    s = (s0 + s1) + (s2 + s3);
+  }
+  part[q][j] = s;
+  __syncthreads();
+  if (q == 0 && e < total) {
+    float r = (part[0][j] + part[1][j]) + (part[2][j] + part[3][j]);
+    if (beta != 0.f) r += beta * dw[e];
+    dw[e] = r;
+  }
+}
+
+static uint32_t wgrad_bf16_blocks(uint64_t items) {
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+    n = 256;
+  return (uint32_t)(items < (uint64_t)n ? items : (uint64_t)n);
+}
+
+bool conv_bf16_wgrad_mfma_supported(uint32_t Cin, uint32_t Cout, uint32_t W) {
+  return Cin <= 64u && Cout <= 64u && (W % 8u) == 0u;
+}
+
+static uint64_t wgrad_bf16_items(uint32_t num_tiles, uint32_t N, uint32_t W) {
+  return (uint64_t)num_tiles * N * ((W + kWgCols - 1) / kWgCols);
+}
+
+size_t conv_bf16_wgrad_mfma_workspace_bytes(uint32_t num_tiles, uint32_t N, uint32_t W) {
+  return (size_t)wgrad_bf16_blocks(wgrad_bf16_items(num_tiles, N, W)) * kWgPartialFloats * sizeof(float);
+}
+
+// Arguments are validated by the caller (pointers, alignment, workspace size, extents > 0).
+int conv_bf16_wgrad_mfma(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                         const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta,
+                         void *workspace, hipStream_t st) {
+  WgradBf16Params P = {};
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    P.x[t] = reinterpret_cast<const uint16_t *>(x_tiles[t]);
+    P.dy[t] = reinterpret_cast<const uint16_t *>(dy_tiles[t]);
+  }
+  P.partial = reinterpret_cast<float *>(workspace);
+  P.N = N; P.Cin = Cin; P.Cout = Cout; P.H = H; P.W = W;
+  P.strips = (W + kWgCols - 1) / kWgCols;
+  const uint64_t items = wgrad_bf16_items(num_tiles, N, W);
+  if (items >= (1ull << 31)) return ADH_EINVAL;
+  P.items = (uint32_t)items;
+  P.div_strips = FastDiv(P.strips);
+  P.div_N = FastDiv(N);
+  const uint32_t blocks = wgrad_bf16_blocks(items);
+  hipLaunchKernelGGL(conv3x3_bf16_wgrad_kernel, dim3(blocks), dim3(512), 0, st, P);
+  int e = launch_status();
+  if (e) return e;
+  const uint32_t total = Cout * Cin * 9u;
+  hipLaunchKernelGGL(conv3x3_bf16_wgrad_reduce_kernel, dim3((total + 63u) / 64u), dim3(256), 0, st,
+                     reinterpret_cast<const float *>(workspace), blocks, dw, Cin, Cout, beta);
+  return launch_status();
+}
+
+}  // namespace adh

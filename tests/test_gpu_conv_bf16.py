@@ -25,7 +25,10 @@ def ws_for(which, K, N, Cin, Cout, H, W):
 # and reductions wider than 64 channels (the widening route)
 @pytest.mark.parametrize("K,N,Cin,Cout,H,W", [(1, 2, 8, 16, 5, 9), (2, 1, 19, 7, 6, 33), (3, 2, 64, 64, 7, 56),
                                               (1, 1, 20, 70, 9, 61), (2, 2, 64, 64, 40, 70), (1, 1, 64, 64, 3, 130),
-                                              (1, 1, 72, 64, 6, 20), (1, 1, 64, 72, 6, 20), (1, 3, 33, 40, 17, 31)])
+                                              (1, 1, 72, 64, 6, 20), (1, 1, 64, 72, 6, 20), (1, 3, 33, 40, 17, 31),
+                                              # widths that are multiples of eight: the bf16 filter-gradient kernel
+                                              (1, 2, 16, 24, 5, 8), (2, 1, 64, 64, 9, 72), (1, 1, 40, 48, 3, 136),
+                                              (3, 2, 7, 5, 1, 64), (1, 1, 64, 64, 2, 200)])
 def test_bf16_conv_small_vs_oracle(oracle, K, N, Cin, Cout, H, W):
     rng = np.random.default_rng(77 + Cin)
     bf = lambda a: oracle.f32_to_bf16(a.astype(np.float32))
