@@ -6,7 +6,7 @@
 // contiguous bytes in NCHW, so both MFMA operands come straight from rows as they lie in memory:
 // A = dy (m = output channel, k = 32 columns), B = x_pad (k = 32 columns, n = input channel).
 // Rows are copied into LDS by `buffer_load ... lds` with 16 bytes per lane (asynchronous, no
-// registers), one row of x_pad and one of dy per stage, three stages.
+// registers), one row of x_pad and one of dy per stage, six stages (five rows in flight).
 //
 // A workgroup of eight waves (two per SIMD) walks down a 64-column strip of one image.  A wave
 // owns one tile of 16 input channels, one half of the output channels (two tiles of 16) and all
@@ -35,6 +35,7 @@ constexpr int kWgPitch = kWgLanes * 16;           // 144 bytes: 66 x_pad columns
 constexpr int kWgRegion = 64 * kWgPitch;          // 9216 bytes: 64 channel rows
 constexpr int kWgStageBytes = 2 * kWgRegion;      // x_pad row, then dy row
 constexpr int kWgDmaPerStage = kWgStageBytes / 1024;  // 18 wave-wide copies
+constexpr int kWgStages = 6;                      // rows in LDS: the one being fetched + five on their way
 constexpr uint32_t kWgOutOfRange = 0x80000000u;
 constexpr uint32_t kWgPartialFloats = 64u * 64u * 9u;
 
@@ -56,6 +57,10 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
   __shared__ __attribute__((aligned(16))) uint8_t stage0[kWgStageBytes];
   __shared__ __attribute__((aligned(16))) uint8_t stage1[kWgStageBytes];
   __shared__ __attribute__((aligned(16))) uint8_t stage2[kWgStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t stage3[kWgStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t stage4[kWgStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t stage5[kWgStageBytes];
+  uint8_t *const stages[kWgStages] = {stage0, stage1, stage2, stage3, stage4, stage5};
 
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
@@ -123,41 +128,74 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
       }
     };
 
-    // dy rows r, r-1, r-2 as A operands: two column halves x two output-channel tiles each
-    u32x4 win[3][2][2];
+    // dy rows as A operands (two column halves x two output-channel tiles each): rows r, r-1, r-2
+    // in use plus row r+1 arriving, in four slots; x_pad rows as five dwords per column half, the
+    // row in use and the row arriving
+    u32x4 win[4][2][2];
 #pragma unroll
-    for (int a = 0; a < 3; ++a)
+    for (int a = 0; a < 4; ++a)
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int cot = 0; cot < 2; ++cot) win[a][kb][cot] = (u32x4){0u, 0u, 0u, 0u};
+    u32x4 xb[2][2];
+    uint32_t xe[2][2];
 
-    __syncthreads();  // the previous item's last rows have been read
-    dma_row(0, stage0);
-    if (last_row >= 1u) dma_row(1, stage1);
-
-    // one row; PH = r mod 3 picks the stage and the window slot that takes the new dy row
-    auto step = [&](auto ph, uint32_t r, uint8_t *cur, uint8_t *nxt2) {
+    // operands of row r from its stage: dy row r -> window slot r mod 4, x_pad row r -> parity r mod 2
+    auto fetch = [&](auto ph) {
       constexpr int PH = decltype(ph)::value;
-      // wait for this wave's copies of row r; those of row r + 1 may stay in flight
-      if (r + 1u <= last_row) {
-        if (wv < 2u) __builtin_amdgcn_s_waitcnt(0x0F70 | 3);
-        else __builtin_amdgcn_s_waitcnt(0x0F70 | 2);
-      } else {
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+      const uint8_t *src = stages[PH % kWgStages];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        xb[PH % 2][kb] = *reinterpret_cast<const u32x4 *>(src + b_off + kb * 64);
+        xe[PH % 2][kb] = *reinterpret_cast<const uint32_t *>(src + b_off + kb * 64 + 16);
       }
-      __syncthreads();  // row r is complete in LDS; everybody is done with row r - 1
-      if (r + 2u <= last_row) dma_row(r + 2u, nxt2);
-
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int cot = 0; cot < 2; ++cot)
-          win[PH][kb][cot] = *reinterpret_cast<const u32x4 *>(cur + a_off + cot * 16 * kWgPitch + kb * 64);
+          win[PH % 4][kb][cot] = *reinterpret_cast<const u32x4 *>(src + a_off + cot * 16 * kWgPitch + kb * 64);
+    };
+    // waits until this wave's copies of all rows but the newest `behind` have landed.  A wave
+    // issues two or three copies per row; counting two is the safe side.
+    auto wait_rows = [&](uint32_t behind) {
+      switch (behind) {
+        case 0: __builtin_amdgcn_s_waitcnt(0x0F70 | 0); break;
+        case 1: __builtin_amdgcn_s_waitcnt(0x0F70 | 2); break;
+        case 2: __builtin_amdgcn_s_waitcnt(0x0F70 | 4); break;
+        case 3: __builtin_amdgcn_s_waitcnt(0x0F70 | 6); break;
+        default: __builtin_amdgcn_s_waitcnt(0x0F70 | 8); break;
+      }
+    };
+
+    __syncthreads();  // the previous item's last rows have been read
+#pragma unroll
+    for (int q = 0; q < kWgStages; ++q)
+      if ((uint32_t)q <= last_row) dma_row((uint32_t)q, stages[q]);
+    wait_rows(last_row < (uint32_t)(kWgStages - 1) ? last_row : (uint32_t)(kWgStages - 1));
+    __syncthreads();
+    fetch(WgTag<0>());
+
+    // One row: the MFMAs of row r run on operands fetched a step ago, while the operands of row
+    // r + 1 are fetched.  PH = r mod 12 gives the stage (mod 6), the window slot (mod 4) and the
+    // x_pad register set (mod 2).
+    auto step = [&](auto ph, uint32_t r) {
+      constexpr int PH = decltype(ph)::value;
+      if (r < last_row) {
+        // row r + 1 must have landed; rows r + 2 .. r + 5 may stay in flight
+        const uint32_t rest = last_row - (r + 1u);
+        wait_rows(rest < (uint32_t)(kWgStages - 2) ? rest : (uint32_t)(kWgStages - 2));
+      }
+      __syncthreads();  // row r + 1 is complete in LDS; everybody has fetched row r
+#ifndef EXP_WG_NODMA
+      if (r + (uint32_t)kWgStages <= last_row) dma_row(r + (uint32_t)kWgStages, stages[PH % kWgStages]);
+#endif
+      if (r < last_row) fetch(WgTag<(PH + 1) % 12>());
+
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
-        const u32x4 b0 = *reinterpret_cast<const u32x4 *>(cur + b_off + kb * 64);
-        const uint32_t b4 = *reinterpret_cast<const uint32_t *>(cur + b_off + kb * 64 + 16);
+        const u32x4 b0 = xb[PH % 2][kb];
+        const uint32_t b4 = xe[PH % 2][kb];
         u32x4 b1;
         b1[0] = __builtin_amdgcn_alignbit(b0[1], b0[0], 16);
         b1[1] = __builtin_amdgcn_alignbit(b0[2], b0[1], 16);
@@ -167,11 +205,14 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
         const u32x4 bs[3] = {b0, b1, b2};
 #pragma unroll
         for (int kh = 0; kh < 3; ++kh) {
-          const int slot = (PH + 3 - kh) % 3;  // dy row r - kh
+          const int slot = (PH + 4 - kh) % 4;  // dy row r - kh
 #pragma unroll
           for (int kw = 0; kw < 3; ++kw)
 #pragma unroll
             for (int cot = 0; cot < 2; ++cot)
+#ifdef EXP_WG_NOMFMA
+              if (kh + kw == 0)
+#endif
               acc[kh][kw][cot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                   __builtin_bit_cast(bf16x8, win[slot][kb][cot]), __builtin_bit_cast(bf16x8, bs[kw]),
                   acc[kh][kw][cot], 0, 0, 0);
@@ -179,10 +220,19 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
       }
     };
 
-    for (uint32_t r = 0; r <= last_row; r += 3u) {
-      step(WgTag<0>(), r, stage0, stage2);
-      if (r + 1u <= last_row) step(WgTag<1>(), r + 1u, stage1, stage0);
-      if (r + 2u <= last_row) step(WgTag<2>(), r + 2u, stage2, stage1);
+    for (uint32_t r = 0; r <= last_row; r += 12u) {
+      step(WgTag<0>(), r);
+      if (r + 1u <= last_row) step(WgTag<1>(), r + 1u);
+      if (r + 2u <= last_row) step(WgTag<2>(), r + 2u);
+      if (r + 3u <= last_row) step(WgTag<3>(), r + 3u);
+      if (r + 4u <= last_row) step(WgTag<4>(), r + 4u);
+      if (r + 5u <= last_row) step(WgTag<5>(), r + 5u);
+      if (r + 6u <= last_row) step(WgTag<6>(), r + 6u);
+      if (r + 7u <= last_row) step(WgTag<7>(), r + 7u);
+      if (r + 8u <= last_row) step(WgTag<8>(), r + 8u);
+      if (r + 9u <= last_row) step(WgTag<9>(), r + 9u);
+      if (r + 10u <= last_row) step(WgTag<10>(), r + 10u);
+      if (r + 11u <= last_row) step(WgTag<11>(), r + 11u);
     }
   }
 
