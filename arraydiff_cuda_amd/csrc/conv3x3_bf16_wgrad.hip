@@ -60,6 +60,7 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
   __shared__ __attribute__((aligned(16))) uint8_t stage3[kWgStageBytes];
   __shared__ __attribute__((aligned(16))) uint8_t stage4[kWgStageBytes];
   __shared__ __attribute__((aligned(16))) uint8_t stage5[kWgStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t spare[1024];
   uint8_t *const stages[kWgStages] = {stage0, stage1, stage2, stage3, stage4, stage5};
 
   const uint32_t tid = threadIdx.x;
@@ -83,7 +84,11 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
   const uint32_t HP = P.H + 2u, WP = P.W + 2u;
   const uint32_t last_row = P.H + 1u;
 
-  for (uint32_t item = blockIdx.x; item < P.items; item += gridDim.x) {
+  // Workgroups are dealt to the eight XCDs (each with its own L2) in turn.  Renumber them so
+  // that an XCD works on neighbouring strips: those share the 128-byte lines at strip borders.
+  uint32_t vblock = blockIdx.x;
+  if ((gridDim.x & 7u) == 0u) vblock = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  for (uint32_t item = vblock; item < P.items; item += gridDim.x) {
     uint32_t strip, plane, tile, n;
     P.div_strips.divmod(item, plane, strip);
     P.div_N.divmod(plane, tile, n);
@@ -95,36 +100,34 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
     const __amdgpu_buffer_rsrc_t rsrc_dy =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(dy_img), 0, P.Cout * P.H * P.W * 2u, 0x00020000);
 
-    // per-lane source offsets of row 0 for the (up to) three copies; out of range where the
-    // channel, the piece or the column does not exist
-    uint32_t voff[3];
+    // Every wave issues three copies per row, numbers wv, wv + 8 and wv + 16 of the stage's 18
+    // (numbers 18 and up write zeros to a spare kilobyte: the same instruction count in every
+    // wave keeps the row loop free of branches and the wait counts exact).  Per-lane source
+    // offsets of row 0; out of range where the channel, the piece or the column does not exist.
+    uint32_t voff[3], rows_q[3], pitch_q[3], dst_q[3];
+    bool isx_q[3];
 #pragma unroll
     for (int q = 0; q < 3; ++q) {
-      const uint32_t k = wv + 8u * q;
+      const uint32_t k = wv + 8u * q;  // uniform
       const uint32_t j = (k % 9u) * 64u + lane;  // lane slot within the x_pad or dy region
       const uint32_t ch = j / kWgLanes, piece = j - ch * kWgLanes;
-      if (k < 9u) {
-        voff[q] = ch < P.Cin ? (ch * HP * WP + c0 + piece * 8u) * 2u : kWgOutOfRange;
-      } else {
-        const uint32_t col = c0 + piece * 8u;
-        voff[q] = (ch < P.Cout && piece < 8u && col < P.W) ? (ch * P.H * P.W + col) * 2u : kWgOutOfRange;
-      }
+      const uint32_t col = c0 + piece * 8u;
+      isx_q[q] = k < 9u;
+      const uint32_t vx = ch < P.Cin ? (ch * HP * WP + col) * 2u : kWgOutOfRange;
+      const uint32_t vd = (ch < P.Cout && piece < 8u && col < P.W) ? (ch * P.H * P.W + col) * 2u : kWgOutOfRange;
+      voff[q] = isx_q[q] ? vx : vd;
+      rows_q[q] = k >= (uint32_t)kWgDmaPerStage ? 0u : (isx_q[q] ? HP : P.H);
+      pitch_q[q] = isx_q[q] ? WP * 2u : P.W * 2u;
+      dst_q[q] = k * 1024u;
     }
 
     auto dma_row = [&](uint32_t r, uint8_t *stage) {
 #pragma unroll
       for (int q = 0; q < 3; ++q) {
-        const uint32_t k = wv + 8u * q;  // uniform
-        if (k >= (uint32_t)kWgDmaPerStage) continue;
-        uint8_t *dst = stage + k * 1024u;
-        if (k < 9u) {
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (__attribute__((address_space(3))) void *)dst, 16, voff[q],
-                                                   __builtin_amdgcn_readfirstlane(r * WP * 2u), 0, 0);
-        } else {
-          const uint32_t v = r < P.H ? voff[q] : kWgOutOfRange;
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_dy, (__attribute__((address_space(3))) void *)dst, 16, v,
-                                                   __builtin_amdgcn_readfirstlane(r * P.W * 2u), 0, 0);
-        }
+        uint8_t *dst = dst_q[q] < (uint32_t)kWgStageBytes ? stage + dst_q[q] : spare;
+        const uint32_t v = r < rows_q[q] ? voff[q] : kWgOutOfRange;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(isx_q[q] ? rsrc_x : rsrc_dy, (__attribute__((address_space(3))) void *)dst,
+                                                 16, v, __builtin_amdgcn_readfirstlane(r * pitch_q[q]), 0, 0);
       }
     };
 
@@ -156,15 +159,17 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
         for (int cot = 0; cot < 2; ++cot)
           win[PH % 4][kb][cot] = *reinterpret_cast<const u32x4 *>(src + a_off + cot * 16 * kWgPitch + kb * 64);
     };
-    // waits until this wave's copies of all rows but the newest `behind` have landed.  A wave
-    // issues two or three copies per row; counting two is the safe side.
+    // waits until this wave's copies (three per row) of all rows but the newest `behind` have landed
     auto wait_rows = [&](uint32_t behind) {
-      switch (behind) {
-        case 0: __builtin_amdgcn_s_waitcnt(0x0F70 | 0); break;
-        case 1: __builtin_amdgcn_s_waitcnt(0x0F70 | 2); break;
-        case 2: __builtin_amdgcn_s_waitcnt(0x0F70 | 4); break;
-        case 3: __builtin_amdgcn_s_waitcnt(0x0F70 | 6); break;
-        default: __builtin_amdgcn_s_waitcnt(0x0F70 | 8); break;
+      if (behind >= 4u) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | 12);
+      } else {
+        switch (behind) {
+          case 0: __builtin_amdgcn_s_waitcnt(0x0F70 | 0); break;
+          case 1: __builtin_amdgcn_s_waitcnt(0x0F70 | 3); break;
+          case 2: __builtin_amdgcn_s_waitcnt(0x0F70 | 6); break;
+          default: __builtin_amdgcn_s_waitcnt(0x0F70 | 9); break;
+        }
       }
     };
 
