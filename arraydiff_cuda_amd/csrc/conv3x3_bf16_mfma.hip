@@ -61,8 +61,11 @@ struct ConvBf16Params {
   uint32_t IH, IW, OH, OW;
   int32_t pad;              // input row/col = output row/col + tap - pad
   float beta;
-  uint32_t strips, segs, seg_rows, items;
-  FastDiv div_strips, div_segs, div_N;
+  // An item is a strip of an image (strip index fastest).  The first `whole_items` are dealt to
+  // the workgroups in turn, top to bottom each; what is left over (fewer items than workgroups)
+  // is cut into row segments of `seg_steps` steps so that it spreads over all of them.
+  uint32_t strips, items, whole_items, steps_per_item, seg_steps, segs, pieces;
+  FastDiv div_strips, div_N, div_rest;
 };
 
 // filter (Cout, Cin, 3, 3) -> matrix-operand order.  flip = 0 (forward): out = Cout index,
@@ -146,14 +149,25 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
   // that an XCD works on neighbouring strips: those share the 128-byte lines at strip borders.
   uint32_t vblock = blockIdx.x;
   if ((gridDim.x & 7u) == 0u) vblock = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  for (uint32_t item = vblock; item < P.items; item += gridDim.x) {
-    uint32_t strip, t1, seg, plane, tile, n;
-    P.div_strips.divmod(item, t1, strip);
-    P.div_segs.divmod(t1, plane, seg);
+  const uint32_t rest_items = P.items - P.whole_items;
+  for (uint32_t work = vblock; work < P.whole_items + P.pieces; work += gridDim.x) {
+    uint32_t item, seg = 0, seg_steps = P.steps_per_item;
+    if (work < P.whole_items) {
+      item = work;
+    } else {
+      // pieces of the left-over items, item index fastest: neighbouring workgroups get
+      // neighbouring strips at the same rows
+      uint32_t it;
+      P.div_rest.divmod(work - P.whole_items, seg, it);
+      item = P.whole_items + it;
+      seg_steps = P.seg_steps;
+    }
+    uint32_t strip, plane, tile, n;
+    P.div_strips.divmod(item, plane, strip);
     P.div_N.divmod(plane, tile, n);
     const int32_t c0 = (int32_t)(strip * kStripCols);
-    const uint32_t r_begin = seg * P.seg_rows;
-    const uint32_t r_end = r_begin + P.seg_rows < P.OH ? r_begin + P.seg_rows : P.OH;
+    const uint32_t r_begin = seg * seg_steps * kStepRows;
+    const uint32_t r_end = min(P.OH, r_begin + seg_steps * kStepRows);
     const uint32_t nsteps = (r_end - r_begin + kStepRows - 1) / kStepRows;
     const uint16_t *in_img = P.in[tile] + (size_t)n * P.Cred * P.IH * P.IW;
     uint16_t *out_img = P.out[tile] + (size_t)n * P.Cout * P.OH * P.OW;
@@ -567,25 +581,28 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
   const uint32_t cus = (uint32_t)num_cus();
   P.strips = (P.OW + kStripCols - 1) / kStripCols;
   const uint64_t base_items = (uint64_t)N * num_tiles * P.strips;
-  // split the rows of a strip into segments while that evens out the load over the CUs; a
-  // segment re-reads two input rows, so keep it at 16 rows or more
-  uint32_t segs = 1;
-  const uint32_t max_segs = (P.OH + 15u) / 16u;
-  const uint64_t want = 4ull * cus / groups;
-  while (segs < max_segs && base_items * segs < want) ++segs;
-  uint32_t seg_rows = (P.OH + segs - 1) / segs;
-  seg_rows = (seg_rows + kStepRows - 1) / kStepRows * kStepRows;
-  segs = (P.OH + seg_rows - 1) / seg_rows;
-  P.segs = segs;
-  P.seg_rows = seg_rows;
-  const uint64_t items = base_items * segs;
-  if (items >= (1ull << 31)) return ADH_EINVAL;
-  P.items = (uint32_t)items;
-  P.div_strips = FastDiv(P.strips);
-  P.div_segs = FastDiv(P.segs);
-  P.div_N = FastDiv(N);
+  if (base_items >= (1ull << 30)) return ADH_EINVAL;
+  P.items = (uint32_t)base_items;
+  P.steps_per_item = (P.OH + kStepRows - 1) / kStepRows;
   uint32_t gx = cus / groups ? cus / groups : 1u;
-  if (gx > P.items) gx = P.items;
+  if (gx > P.items * P.steps_per_item) gx = P.items * P.steps_per_item;
+  // whole items while they go round evenly; the rest in row segments of at least four steps
+  // (a segment re-reads two input rows and pays for filling the ring again)
+  P.whole_items = P.items / gx * gx;
+  const uint32_t rest = P.items - P.whole_items;
+  P.seg_steps = P.steps_per_item;
+  P.segs = 1;
+  if (rest) {
+    const uint32_t want_segs = gx / rest;  // >= 1
+    uint32_t seg_steps = (P.steps_per_item + want_segs - 1) / want_segs;
+    if (seg_steps < 4u) seg_steps = P.steps_per_item < 4u ? P.steps_per_item : 4u;
+    P.seg_steps = seg_steps;
+    P.segs = (P.steps_per_item + seg_steps - 1) / seg_steps;
+  }
+  P.pieces = rest * P.segs;
+  P.div_strips = FastDiv(P.strips);
+  P.div_N = FastDiv(N);
+  P.div_rest = FastDiv(rest ? rest : 1u);
   if (beta != 0.f)
     hipLaunchKernelGGL(conv3x3_bf16_kernel<true>, dim3(gx, groups), dim3(256), 0, st, P);
   else

@@ -192,9 +192,7 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
         wait_rows(rest < (uint32_t)(kWgStages - 2) ? rest : (uint32_t)(kWgStages - 2));
       }
       __syncthreads();  // row r + 1 is complete in LDS; everybody has fetched row r
-#ifndef EXP_WG_NODMA
       if (r + (uint32_t)kWgStages <= last_row) dma_row(r + (uint32_t)kWgStages, stages[PH % kWgStages]);
-#endif
       if (r < last_row) fetch(WgTag<(PH + 1) % 12>());
 
 #pragma unroll
@@ -215,9 +213,6 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
           for (int kw = 0; kw < 3; ++kw)
 #pragma unroll
             for (int cot = 0; cot < 2; ++cot)
-#ifdef EXP_WG_NOMFMA
-              if (kh + kw == 0)
-#endif
               acc[kh][kw][cot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                   __builtin_bit_cast(bf16x8, win[slot][kb][cot]), __builtin_bit_cast(bf16x8, bs[kw]),
                   acc[kh][kw][cot], 0, 0, 0);
