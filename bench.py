@@ -224,7 +224,7 @@ def main():
             lambda: lib.adh_tiles_unpack_nchw(1, K5, 1, W5, H5, C, N5, t5_tbl, Y5.data_ptr(), stream),
             "hbm", 2 * b5, HBM_PEAK_GBS, "GB/s")
         # config 5 slab conv on the bf16 matrix cores: fwd, bwd-data (beta = 1, as the reference
-        # accumulates input gradients), bwd-filter (bf16 widened to fp32, fp32 MFMA)
+        # accumulates input gradients), bwd-filter
         Ht5 = H5 // K5
         w5 = (torch.randn((C, C, 3, 3), device="cuda", generator=g) * (2.0 / (C * 9)) ** 0.5).to(torch.bfloat16)
         y5 = [torch.empty((N5, C, Ht5, W5), device="cuda", dtype=torch.bfloat16) for _ in range(K5)]
@@ -242,11 +242,10 @@ def main():
             lambda: lib.adh_conv3x3_slab_bwd_data_tiles(1, K5, N5, C, C, Ht5, W5, w5.data_ptr(), y5_tbl, t5_tbl, 1.0,
                                                         ws5.data_ptr(), ws5_bytes, stream),
             "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
-        reps, wu = 5, 1
-        add("conv bwd-filter cfg5 (bf16 in, widened, fp32 MFMA)",
+        add("conv bwd-filter cfg5 (bf16 in, fp32 filter gradient, two kernels)",
             lambda: lib.adh_conv3x3_slab_bwd_filter_tiles(1, K5, N5, C, C, Ht5, W5, t5_tbl, y5_tbl, gw5.data_ptr(), 0.0,
                                                           ws5.data_ptr(), ws5_bytes, stream),
-            "mfma", flops5, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+            "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
         del X5, t5, Y5, y5, ws5
         out["secondary"] = sec
 
