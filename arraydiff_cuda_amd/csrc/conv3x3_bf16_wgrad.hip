@@ -42,7 +42,7 @@ constexpr uint32_t kWgPartialFloats = 64u * 64u * 9u;
 struct WgradBf16Params {
   const uint16_t *x[ADH_MAX_TILES];
   const uint16_t *dy[ADH_MAX_TILES];
-  float *partial;  // [gridDim.x][64 co][64 ci][9]
+  float *partial;  // [gridDim.x][8 waves][9 taps][2 output-channel tiles][64 lanes][4]
   uint32_t N, Cin, Cout, H, W;
   uint32_t strips, items;
   FastDiv div_strips, div_N;
@@ -236,34 +236,30 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
     }
   }
 
-  // D[m = 4 g + i][n = l16]: output channel 32 coh + 16 cot + 4 g + i, input channel 16 cit + l16
-  float *part = P.partial + (size_t)blockIdx.x * kWgPartialFloats;
+  // D[m = 4 g + i][n = l16]: output channel 32 coh + 16 cot + 4 g + i, input channel 16 cit + l16.
+  // The partial is written in register order, [wave][tap][cot][lane][i], 16 contiguous bytes per
+  // lane: in filter order every lane would write lone floats 36 bytes apart, which costs five
+  // times the bytes in partial-sector writes.
+  floatx4 *part = reinterpret_cast<floatx4 *>(P.partial + (size_t)blockIdx.x * kWgPartialFloats) + wv * (18u * 64u) + lane;
 #pragma unroll
   for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
     for (int kw = 0; kw < 3; ++kw)
 #pragma unroll
-      for (int cot = 0; cot < 2; ++cot)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint32_t co = 32u * coh + 16u * cot + 4u * g + i, ci = 16u * cit + l16;
-          part[(co * 64u + ci) * 9u + kh * 3 + kw] = acc[kh][kw][cot][i];
-        }
+      for (int cot = 0; cot < 2; ++cot) part[((kh * 3 + kw) * 2 + cot) * 64] = acc[kh][kw][cot];
 }
 
-// dw[co][ci][tap] = beta * dw + sum over partials, in a fixed order: 64 elements per workgroup,
-// four quarters of the partials in parallel
+// dw[co][ci][tap] = beta * dw + sum over partials, in a fixed order.  A workgroup takes 64
+// consecutive elements in the partials' register order (coalesced reads), four quarters of the
+// partials in parallel, and scatters the 64 sums to their places in the filter.
 __global__ __launch_bounds__(256) void conv3x3_bf16_wgrad_reduce_kernel(const float *__restrict__ partial,
                                                                         uint32_t num_partials, float *dw, uint32_t Cin,
                                                                         uint32_t Cout, float beta) {
   __shared__ float part[4][64];
   const uint32_t q = threadIdx.x >> 6, j = threadIdx.x & 63u;
-  const uint32_t e = blockIdx.x * 64u + j;
-  const uint32_t total = Cout * Cin * 9u;
-  float s = 0.f;
-  if (e < total) {
-    const uint32_t tap = e % 9u, cc = e / 9u, ci = cc % Cin, co = cc / Cin;
-    const float *p = partial + (co * 64u + ci) * 9u + tap;
+  const uint32_t e = blockIdx.x * 64u + j;  // < kWgPartialFloats: the grid covers it exactly
+  {
+    const float *p = partial + e;
     const uint32_t per = (num_partials + 3u) / 4u;
     const uint32_t b0 = q * per, b1 = min(b0 + per, num_partials);
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
@@ -275,14 +271,20 @@ __global__ __launch_bounds__(256) void conv3x3_bf16_wgrad_reduce_kernel(const fl
       s3 += p[(size_t)(b + 3u) * kWgPartialFloats];
     }
     for (; b < b1; ++b) s0 += p[(size_t)b * kWgPartialFloats];
-    s = (s0 + s1) + (s2 + s3);
+    part[q][j] = (s0 + s1) + (s2 + s3);
   }
-  part[q][j] = s;
   __syncthreads();
-  if (q == 0 && e < total) {
-    float r = (part[0][j] + part[1][j]) + (part[2][j] + part[3][j]);
-    if (beta != 0.f) r += beta * dw[e];
-    dw[e] = r;
+  if (q == 0) {
+    // e = (((wave * 9 + tap) * 2 + cot) * 64 + lane) * 4 + i
+    const uint32_t i = e & 3u, lane = (e >> 2) & 63u, cot = (e >> 8) & 1u;
+    const uint32_t wt = e >> 9, tap = wt % 9u, wave = wt / 9u;
+    const uint32_t co = 32u * (wave >> 2) + 16u * cot + 4u * (lane >> 4) + i, ci = 16u * (wave & 3u) + (lane & 15u);
+    if (co < Cout && ci < Cin) {
+      float *d = dw + ((size_t)co * Cin + ci) * 9u + tap;
+      float r = (part[0][j] + part[1][j]) + (part[2][j] + part[3][j]);
+      if (beta != 0.f) r += beta * *d;
+      *d = r;
+    }
   }
 }
 
@@ -327,8 +329,7 @@ int conv_bf16_wgrad_mfma(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t 
   hipLaunchKernelGGL(conv3x3_bf16_wgrad_kernel, dim3(blocks), dim3(512), 0, st, P);
   int e = launch_status();
   if (e) return e;
-  const uint32_t total = Cout * Cin * 9u;
-  hipLaunchKernelGGL(conv3x3_bf16_wgrad_reduce_kernel, dim3((total + 63u) / 64u), dim3(256), 0, st,
+  hipLaunchKernelGGL(conv3x3_bf16_wgrad_reduce_kernel, dim3(kWgPartialFloats / 64u), dim3(256), 0, st,
                      reinterpret_cast<const float *>(workspace), blocks, dw, Cin, Cout, beta);
   return launch_status();
 }
