@@ -67,6 +67,43 @@ def test_bf16_conv_small_vs_oracle(oracle, K, N, Cin, Cout, H, W):
     assert capi.conv_fwd_tiles(d_xs, d_w, ys, N, Cin, Cout, H, W, ws=small) == capi.ADH_EWORKSPACE
 
 
+def test_bf16_conv_odd_pointers_and_many_images(oracle):
+    """Tile buffers that are only 2-byte aligned (views one element into an allocation), more work
+    items than workgroups, a one-row image and a single channel."""
+    rng = np.random.default_rng(404)
+    bf = lambda a: oracle.f32_to_bf16(a.astype(np.float32))
+    for (N, Cin, Cout, H, W) in ((300, 8, 8, 1, 8), (3, 1, 1, 5, 16), (2, 64, 64, 6, 64)):
+        x = bf(rng.uniform(-1, 1, size=(N, Cin, H + 2, W + 2)))
+        w = bf(rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9)))
+        dy = bf(rng.standard_normal((N, Cout, H, W)))
+
+        def odd(a):  # device copy whose first element sits at an odd 2-byte offset
+            buf = torch.empty(a.size + 1, device="cuda", dtype=torch.bfloat16)
+            v = buf[1:].view(a.shape)
+            v.copy_(dev(a).view(a.shape))
+            return v
+
+        d_x, d_dy, d_w = odd(x), odd(dy), dev(w)
+        y = odd(np.zeros((N, Cout, H, W), np.uint16))
+        gx = odd(np.zeros((N, Cin, H + 2, W + 2), np.uint16))
+        dw = torch.zeros((Cout, Cin, 3, 3), device="cuda")
+        capi.check(capi.conv_fwd_tiles([d_x], d_w, [y], N, Cin, Cout, H, W, ws=ws_for(capi.ADH_CONV_FWD, 1, N, Cin, Cout, H, W)))
+        capi.check(capi.conv_bwd_data_tiles(d_w, [d_dy], [gx], N, Cin, Cout, H, W,
+                                            ws=ws_for(capi.ADH_CONV_BWD_DATA, 1, N, Cin, Cout, H, W)))
+        capi.check(capi.conv_bwd_filter_tiles([d_x], [d_dy], dw, N, Cin, Cout, H, W,
+                                              ws=ws_for(capi.ADH_CONV_BWD_FILTER, 1, N, Cin, Cout, H, W)))
+        xf, dyf, wf = oracle.bf16_to_f32(x), oracle.bf16_to_f32(dy), oracle.bf16_to_f32(w)
+        y_want = np.empty((N, Cout, H, W), np.float32)
+        oracle.conv_slab_fwd(xf, wf, y_want)
+        assert rel_err(y.float().cpu().numpy(), y_want) <= 5e-3
+        g_want = np.empty((N, Cin, H + 2, W + 2), np.float32)
+        oracle.conv_slab_bwd_data(wf, dyf, g_want)
+        assert rel_err(gx.float().cpu().numpy(), g_want) <= 5e-3
+        dw_want = np.zeros((Cout, Cin, 3, 3), np.float32)
+        oracle.conv_slab_bwd_filter(xf, dyf, dw_want, beta=0.0)
+        assert rel_err(host(dw), dw_want) <= 1e-4
+
+
 def test_config5_highres_bf16_fwd_bwd_sampled(oracle):
     """bf16 N=2, C=64, 1024x2048 in 8 row-tiles of 128 rows + halo 1: pack, conv fwd, bwd-data +
     halo reduce + unpack, bwd-filter, each checked against the UNSPLIT convolution on samples."""
