@@ -12,6 +12,7 @@ ADH_F32 = 0
 ADH_BF16 = 1
 ADH_OK, ADH_EINVAL, ADH_EUNIMPL, ADH_ENULL, ADH_EALIGN, ADH_EWORKSPACE = 0, -1, -2, -3, -4, -5
 ADH_CONV_FWD, ADH_CONV_BWD_DATA, ADH_CONV_BWD_FILTER = 0, 1, 2
+ADH_POOL_AVG, ADH_POOL_MAX = 0, 1
 ADH_MAX_TILES = 16
 
 u32, u64, i32, f32, vp, sz = (ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int, ctypes.c_float,
@@ -46,6 +47,10 @@ SIGNATURES = {
     "adh_conv3x3_slab_bwd_data_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_filter": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_filter_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp, f32, vp, sz, vp]),
+    "adh_pool2d_slab_fwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp]),
+    "adh_pool2d_slab_fwd": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, vp, vp, vp]),
+    "adh_pool2d_slab_bwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vpp, vpp, vpp, f32, vp]),
+    "adh_pool2d_slab_bwd": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, vp, vp, vp, vp, f32, vp]),
     "adh_softmax_fwd": (i32, [u32, u32, vp, vp, vp]),
     "adh_softmax_nll_loss_fwd": (i32, [u32, u32, vp, vp, vp, vp]),
     "adh_softmax_nll_loss_bwd": (i32, [u32, u32, vp, vp, vp, vp, vp]),
@@ -224,6 +229,23 @@ def conv_bwd_data_tiles(w, dys, dxs, N, Cin, Cout, H, W, beta=0.0, ws=None):
     wp, wb = _ws(ws)
     return lib().adh_conv3x3_slab_bwd_data_tiles(_dt(dys[0]), len(dys), N, Cin, Cout, H, W, w.data_ptr(), dt, xt,
                                                  beta, wp, wb, _stream())
+
+
+def pool_fwd_tiles(mode, xs, ys, N, C, HP, WP, wh, ww, sh, sw):
+    _dev(*xs, *ys)
+    xt, k1 = _tbl(xs)
+    yt, k2 = _tbl(ys)
+    return lib().adh_pool2d_slab_fwd_tiles(_dt(xs[0]), mode, len(xs), N, C, HP, WP, wh, ww, sh, sw, xt, yt, _stream())
+
+
+def pool_bwd_tiles(mode, xs, ys, dys, dxs, N, C, HP, WP, wh, ww, sh, sw, beta=0.0):
+    _dev(*xs, *ys, *dys, *dxs)
+    xt, k1 = _tbl(xs)
+    yt, k2 = _tbl(ys)
+    dt, k3 = _tbl(dys)
+    gt, k4 = _tbl(dxs)
+    return lib().adh_pool2d_slab_bwd_tiles(_dt(dys[0]), mode, len(dys), N, C, HP, WP, wh, ww, sh, sw, xt, yt, dt, gt,
+                                           beta, _stream())
 
 
 def conv_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, H, W, beta=0.0, ws=None):

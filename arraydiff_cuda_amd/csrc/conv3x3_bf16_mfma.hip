@@ -149,7 +149,6 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
   // that an XCD works on neighbouring strips: those share the 128-byte lines at strip borders.
   uint32_t vblock = blockIdx.x;
   if ((gridDim.x & 7u) == 0u) vblock = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  const uint32_t rest_items = P.items - P.whole_items;
   for (uint32_t work = vblock; work < P.whole_items + P.pieces; work += gridDim.x) {
     uint32_t item, seg = 0, seg_steps = P.steps_per_item;
     if (work < P.whole_items) {

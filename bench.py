@@ -247,6 +247,28 @@ def main():
                                                           ws5.data_ptr(), ws5_bytes, stream),
             "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
         del X5, t5, Y5, y5, ws5
+        # pooling over the padded slab: the 3x3 stride-2 max pooling of a residual network's stem,
+        # 112x112 in 4 row-tiles of 28 rows with halo 1 -> 14x56 per tile
+        Hq, Wq = 28 + 2, 112 + 2
+        OHq, OWq = (Hq - 3) // 2 + 1, (Wq - 3) // 2 + 1
+        xq = [torch.rand((N, C, Hq, Wq), device="cuda", generator=g) for _ in range(K)]
+        yq = [torch.empty((N, C, OHq, OWq), device="cuda") for _ in range(K)]
+        dq = [torch.randn((N, C, OHq, OWq), device="cuda", generator=g) for _ in range(K)]
+        gq = [torch.empty((N, C, Hq, Wq), device="cuda") for _ in range(K)]
+        xq_tbl, _kq1 = capi.ptr_table([t.data_ptr() for t in xq])
+        yq_tbl, _kq2 = capi.ptr_table([t.data_ptr() for t in yq])
+        dq_tbl, _kq3 = capi.ptr_table([t.data_ptr() for t in dq])
+        gq_tbl, _kq4 = capi.ptr_table([t.data_ptr() for t in gq])
+        in_b, out_b = K * N * C * Hq * Wq * 4, K * N * C * OHq * OWq * 4
+        reps, wu = 100, 10
+        add("max pool 3x3 s2 fwd over padded tiles (fp32, 4 tiles of 30x114)",
+            lambda: lib.adh_pool2d_slab_fwd_tiles(0, 1, K, N, C, Hq, Wq, 3, 3, 2, 2, xq_tbl, yq_tbl, stream),
+            "hbm", in_b + out_b, HBM_PEAK_GBS, "GB/s")
+        add("max pool 3x3 s2 bwd over padded tiles (fp32)",
+            lambda: lib.adh_pool2d_slab_bwd_tiles(0, 1, K, N, C, Hq, Wq, 3, 3, 2, 2, xq_tbl, yq_tbl, dq_tbl, gq_tbl,
+                                                  0.0, stream),
+            "hbm", 2 * in_b + 2 * out_b, HBM_PEAK_GBS, "GB/s")
+        del xq, yq, dq, gq
         out["secondary"] = sec
 
     # ---- CPU baseline: the scalar port, single thread, on a bounded sample ----

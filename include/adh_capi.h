@@ -171,6 +171,34 @@ int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N,
                                       float *dw, float beta, void *workspace, size_t workspace_bytes,
                                       void *stream);
 
+/* ---- pooling over the halo-padded slab ------------------------------------- */
+/* CudnnPool2DOp with Pool2DShape::halo_padded_input (include/arraydiff/op.hh:2917-2925): the
+ * padded tile (N, C, HP, WP) with HP = H + 2*pad_h, WP = W + 2*pad_w is handed to cuDNN as a plain
+ * packed tensor with pooling pad 0 (src/op.cc:3424-3462), so the halo (neighbour rows after an
+ * exchange, zeros at the image border) takes part as ordinary data.  Output extents are
+ * OH = (HP - wh) / sh + 1, OW = (WP - ww) / sw + 1 (cudnnGetPooling2dForwardOutputDim).
+ * ADH_POOL_MAX = CUDNN_POOLING_MAX, ADH_POOL_AVG = CUDNN_POOLING_AVERAGE_COUNT_INCLUDE_PADDING
+ * (every window lies inside the padded tensor, so the divisor is always wh*ww).
+ * fwd, cudnnPoolingForward beta 0 (src/op.cc:3496-3503): y = pool(x_pad).
+ * bwd, cudnnPoolingBackward (src/op.cc:3610-3619): dx_pad = beta*dx_pad + pool'(dy), over the
+ * WHOLE padded tile (the reference zeroes it on first touch and calls with beta 1).  For MAX the
+ * gradient of a window goes to its first maximum in row-major window order; NaNs never win.
+ * dtype f32 or bf16 (arithmetic in fp32).  beta is 0 or 1.  One launch covers all tiles. */
+#define ADH_POOL_AVG 0 /* kAveragePool, include/arraydiff/op.hh:2912-2915 */
+#define ADH_POOL_MAX 1 /* kMaxPool */
+int adh_pool2d_slab_fwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t HP,
+                              uint32_t WP, uint32_t wh, uint32_t ww, uint32_t sh, uint32_t sw,
+                              const void *const *x_pad_tiles, void *const *y_tiles, void *stream);
+int adh_pool2d_slab_fwd(int dtype, int mode, uint32_t N, uint32_t C, uint32_t HP, uint32_t WP, uint32_t wh,
+                        uint32_t ww, uint32_t sh, uint32_t sw, const void *x_pad, void *y, void *stream);
+int adh_pool2d_slab_bwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t HP,
+                              uint32_t WP, uint32_t wh, uint32_t ww, uint32_t sh, uint32_t sw,
+                              const void *const *x_pad_tiles, const void *const *y_tiles,
+                              const void *const *dy_tiles, void *const *dx_pad_tiles, float beta, void *stream);
+int adh_pool2d_slab_bwd(int dtype, int mode, uint32_t N, uint32_t C, uint32_t HP, uint32_t WP, uint32_t wh,
+                        uint32_t ww, uint32_t sh, uint32_t sw, const void *x_pad, const void *y, const void *dy,
+                        void *dx_pad, float beta, void *stream);
+
 /* ---- L1/L2/L3: softmax + negative log likelihood (fp32) ------------------- */
 /* cudnnSoftmaxForward(ACCURATE, MODE_INSTANCE) on (N,C,1,1), src/op.cc:4129-4152 */
 int adh_softmax_fwd(uint32_t C, uint32_t N, const float *x, float *y, void *stream);

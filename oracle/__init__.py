@@ -194,6 +194,20 @@ def conv_slab_bwd_filter(x_pad, dy, dw, beta=0.0):
                                   _ptr(x_pad), _ptr(dy), ctypes.c_float(beta), _ptr(dw))
 
 
+def pool_slab_fwd(mode, x_pad, wh, ww, sh, sw, y):
+    """x_pad (N, C, HP, WP) float32 -> y (N, C, OH, OW); mode 1 = max, 0 = average."""
+    N, C, HP, WP = x_pad.shape
+    assert y.shape == (N, C, (HP - wh) // sh + 1, (WP - ww) // sw + 1)
+    _lib.orc_pool_slab_fwd(ctypes.c_int(mode), _u32(N), _u32(C), _u32(HP), _u32(WP), _u32(wh), _u32(ww),
+                           _u32(sh), _u32(sw), _ptr(x_pad), _ptr(y))
+
+
+def pool_slab_bwd(mode, x_pad, dy, wh, ww, sh, sw, dx_pad, beta=0.0):
+    N, C, HP, WP = x_pad.shape
+    _lib.orc_pool_slab_bwd(ctypes.c_int(mode), _u32(N), _u32(C), _u32(HP), _u32(WP), _u32(wh), _u32(ww),
+                           _u32(sh), _u32(sw), _ptr(x_pad), _ptr(dy), ctypes.c_float(beta), _ptr(dx_pad))
+
+
 def softmax_fwd(x, y):
     N, C = x.shape
     _lib.orc_softmax_fwd(_u32(C), _u32(N), _ptr(x), _ptr(y))

@@ -25,6 +25,10 @@
  *     conv2d + autograd on the CPU, delta / box / hot-pixel closed forms.
  *   - softmax / nll : pinned against scipy.special.log_softmax and closed
  *     forms (uniform logits, shift invariance, rows sum to one).
+ *   - pooling over the padded slab : pinned against torch max_pool2d /
+ *     avg_pool2d + autograd on the CPU; which element of a window receives the
+ *     max gradient when several are equal is cuDNN's choice and is parity
+ *     unpinned (this file and the kernels pick the first in row-major order).
  *   - cuDNN's exact fp32 summation order for conv and softmax: parity
  *     unpinned (not reproducible by the reference itself run to run); the
  *     tolerance-vs-unsplit criterion is used instead.
@@ -517,4 +521,68 @@ double orc_now_seconds(void) {
   struct timespec ts;
   clock_gettime(CLOCK_MONOTONIC, &ts);
   return (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
+}
+
+
+/* ------------------------------------------------------------------------- */
+/* pooling over the halo-padded slab                                          */
+/* ------------------------------------------------------------------------- */
+/* CudnnPool2DOp::_forward with halo_padded_input (src/op.cc:3424-3462, 3496-3503): the padded
+ * tile (WP, HP, C, N) is pooled as a plain packed tensor with pad 0; mode 1 = CUDNN_POOLING_MAX
+ * (NaNs never win, CUDNN_NOT_PROPAGATE_NAN), mode 0 = AVERAGE_COUNT_INCLUDE_PADDING (divisor
+ * wh*ww).  Output (OW, OH) = ((WP - ww)/sw + 1, (HP - wh)/sh + 1). */
+void orc_pool_slab_fwd(int mode, uint32_t N, uint32_t C, uint32_t HP, uint32_t WP, uint32_t wh, uint32_t ww,
+                       uint32_t sh, uint32_t sw, const float *x, float *y) {
+  const uint32_t OH = (HP - wh) / sh + 1u, OW = (WP - ww) / sw + 1u;
+  for (uint64_t pl = 0; pl < (uint64_t)N * C; ++pl) {
+    const float *xp = x + pl * HP * WP;
+    float *yp = y + pl * OH * OW;
+    for (uint32_t oh = 0; oh < OH; ++oh)
+      for (uint32_t ow = 0; ow < OW; ++ow) {
+        double sum = 0.0;
+        float mx = -INFINITY;
+        for (uint32_t a = 0; a < wh; ++a)
+          for (uint32_t b = 0; b < ww; ++b) {
+            const float v = xp[(uint64_t)(oh * sh + a) * WP + ow * sw + b];
+            sum += v;
+            if (v > mx) mx = v;
+          }
+        yp[(uint64_t)oh * OW + ow] = mode ? mx : (float)(sum / (double)(wh * ww));
+      }
+  }
+}
+
+/* CudnnPool2DOp::_backward (src/op.cc:3548-3619): dx_pad = beta*dx_pad + pool'(dy) over the whole
+ * padded tile.  MAX: a window's dy goes to its first maximum in row-major window order. */
+void orc_pool_slab_bwd(int mode, uint32_t N, uint32_t C, uint32_t HP, uint32_t WP, uint32_t wh, uint32_t ww,
+                       uint32_t sh, uint32_t sw, const float *x, const float *dy, float beta, float *dx) {
+  const uint32_t OH = (HP - wh) / sh + 1u, OW = (WP - ww) / sw + 1u;
+  const uint64_t plane = (uint64_t)HP * WP;
+  double *g = (double *)malloc(plane * sizeof(double));
+  for (uint64_t pl = 0; pl < (uint64_t)N * C; ++pl) {
+    const float *xp = x ? x + pl * plane : NULL;
+    const float *dyp = dy + pl * OH * OW;
+    float *dxp = dx + pl * plane;
+    for (uint64_t i = 0; i < plane; ++i) g[i] = 0.0;
+    for (uint32_t oh = 0; oh < OH; ++oh)
+      for (uint32_t ow = 0; ow < OW; ++ow) {
+        const float d = dyp[(uint64_t)oh * OW + ow];
+        if (mode) {
+          float mx = -INFINITY;
+          uint64_t arg = (uint64_t)(oh * sh) * WP + ow * sw;
+          for (uint32_t a = 0; a < wh; ++a)
+            for (uint32_t b = 0; b < ww; ++b) {
+              const uint64_t i = (uint64_t)(oh * sh + a) * WP + ow * sw + b;
+              if (xp[i] > mx) { mx = xp[i]; arg = i; }
+            }
+          g[arg] += d;
+        } else {
+          for (uint32_t a = 0; a < wh; ++a)
+            for (uint32_t b = 0; b < ww; ++b)
+              g[(uint64_t)(oh * sh + a) * WP + ow * sw + b] += (double)d / (double)(wh * ww);
+        }
+      }
+    for (uint64_t i = 0; i < plane; ++i) dxp[i] = (float)((beta != 0.f ? (double)beta * dxp[i] : 0.0) + g[i]);
+  }
+  free(g);
 }
