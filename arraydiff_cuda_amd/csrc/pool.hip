@@ -1,13 +1,19 @@
 // Pooling over the halo-padded slab (max / average, forward and backward): HBM-bound kernels.
 //
-// forward : one thread per output element, lanes along the output row; the wh x ww window reads
-//           overlap between neighbouring lanes and rows and are served by the caches, so HBM sees
-//           the padded tile once.
-// backward: one thread per element of the padded tile (a gather, no atomics): it visits the at
-//           most ceil(wh/sh) x ceil(ww/sw) windows that contain it.  For MAX it takes a window's
-//           gradient if it is that window's first maximum in row-major order: its value equals the
-//           stored maximum and no earlier element of the window does.
+// Banded kernels (the normal route): a block owns a band of rows of one plane.  The band of the
+// padded tile is a contiguous byte range, so it is staged into LDS with 16-byte loads whatever the
+// window and stride are, and the strided window reads then hit LDS instead of the vector caches.
+//   forward : stage the input band, one output element per thread and step, coalesced stores.
+//   backward: stage the input band and the band's dy rows; MAX first writes, per window, the
+//             position of its first maximum in row-major order (one byte); then one thread per
+//             element of the padded tile gathers the at most ceil(wh/sh) x ceil(ww/sw) windows
+//             that contain it in a fixed order (no atomics: results are reproducible) and stores
+//             dx coalesced.  y is not read: the maximum is recomputed from the staged input.
+// Direct kernels (rows too wide for LDS, windows of more than 256 elements): one thread per
+//   output (forward) or per padded element (backward), window reads served by the caches.
 #include "adh_common.h"
+
+#include <algorithm>
 
 namespace adh {
 
@@ -20,12 +26,247 @@ struct PoolParams {
   uint32_t HP, WP, OH, OW, wh, ww, sh, sw;
   float beta, inv_area;
   FastDiv div_sh, div_sw;
+  // banded kernels
+  uint32_t bands, band_rows;  // bands per plane; output rows (forward) / window rows (backward) per band
+  FastDiv div_bands, div_OW, div_WP;
 };
 
 __device__ __forceinline__ float ld_f(const float *p, size_t i) { return p[i]; }
 __device__ __forceinline__ float ld_f(const uint16_t *p, size_t i) { return bf16_bits_to_f32(p[i]); }
 __device__ __forceinline__ void st_f(float *p, size_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void st_f(uint16_t *p, size_t i, float v) { p[i] = f32_to_bf16_bits(v); }
+
+constexpr uint32_t kPoolThreads = 256;
+constexpr uint32_t kPoolBandBytes = 24u * 1024u;  // LDS aimed at per block (twice that for the max backward)
+constexpr uint32_t kPoolMaxLds = 64u * 1024u;
+
+// Copies n elements from src into LDS with 16-byte loads; lds is 16-byte aligned and has room for
+// n + 16 / sizeof(T) elements.  Returns the LDS address of element 0: it is shifted by the source's
+// misalignment so that aligned global vectors land on aligned LDS vectors.
+template <typename T>
+__device__ __forceinline__ T *stage_contiguous(T *lds, const T *__restrict__ src, uint32_t n) {
+  constexpr uint32_t VE = 16u / sizeof(T);
+  const uint32_t tid = threadIdx.x;
+  const uint32_t pad = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 15u) / (uint32_t)sizeof(T);
+  T *dst = lds + pad;
+  const uint32_t head = min(n, (VE - pad) & (VE - 1u));
+  const uint32_t nvec = (n - head) / VE;
+  const uint32_t tail0 = head + nvec * VE;
+  if (tid < head) dst[tid] = src[tid];
+  const uint4 *gv = reinterpret_cast<const uint4 *>(src + head);
+  uint4 *lv = reinterpret_cast<uint4 *>(dst + head);
+#pragma unroll 4
+  for (uint32_t v = tid; v < nvec; v += kPoolThreads) lv[v] = gv[v];
+  if (tid < n - tail0) dst[tail0 + tid] = src[tail0 + tid];
+  return dst;
+}
+
+__device__ __forceinline__ void vec_to_f32(const uint4 &v, float (&f)[4], const float *) {
+  f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y); f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+}
+__device__ __forceinline__ void vec_to_f32(const uint4 &v, float (&f)[8], const uint16_t *) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __uint_as_float(w[i] << 16);
+    f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ uint4 f32_to_vec(const float (&f)[4], const float *) {
+  return make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
+}
+__device__ __forceinline__ uint4 f32_to_vec(const float (&f)[8], const uint16_t *) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f32_to_bf16_bits(f[2 * i]) | ((uint32_t)f32_to_bf16_bits(f[2 * i + 1]) << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// dst[i] = src[i] (+ dst[i] when accumulate) for n elements with 16-byte stores; src is fp32 in LDS
+// and src - (dst's misalignment in elements) is 16-byte aligned.
+template <typename T>
+__device__ __forceinline__ void unstage_contiguous(T *__restrict__ dst, const float *src, uint32_t n, bool accumulate) {
+  constexpr uint32_t VE = 16u / sizeof(T);
+  const uint32_t tid = threadIdx.x;
+  const uint32_t pad = (uint32_t)(reinterpret_cast<uintptr_t>(dst) & 15u) / (uint32_t)sizeof(T);
+  const uint32_t head = min(n, (VE - pad) & (VE - 1u));
+  const uint32_t nvec = (n - head) / VE;
+  const uint32_t tail0 = head + nvec * VE;
+  if (tid < head) st_f(dst, tid, src[tid] + (accumulate ? ld_f(dst, tid) : 0.f));
+  uint4 *gv = reinterpret_cast<uint4 *>(dst + head);
+  const float4 *lv = reinterpret_cast<const float4 *>(src + head);
+#pragma unroll 2
+  for (uint32_t v = tid; v < nvec; v += kPoolThreads) {
+    float f[VE];
+#pragma unroll
+    for (uint32_t q = 0; q < VE / 4u; ++q) {
+      const float4 t = lv[v * (VE / 4u) + q];
+      f[4 * q] = t.x; f[4 * q + 1] = t.y; f[4 * q + 2] = t.z; f[4 * q + 3] = t.w;
+    }
+    if (accumulate) {
+      float o[VE];
+      vec_to_f32(gv[v], o, (const T *)nullptr);
+#pragma unroll
+      for (uint32_t q = 0; q < VE; ++q) f[q] += o[q];
+    }
+    gv[v] = f32_to_vec(f, (const T *)nullptr);
+  }
+  if (tid < n - tail0) st_f(dst, tail0 + tid, src[tail0 + tid] + (accumulate ? ld_f(dst, tail0 + tid) : 0.f));
+}
+
+template <int WH, int WW, bool MAX, typename T>
+__device__ __forceinline__ float window_reduce(const T *x, uint32_t base, uint32_t WP, uint32_t wh, uint32_t ww) {
+  float acc = MAX ? -__builtin_inff() : 0.f;
+  if (WH > 0) {
+#pragma unroll
+    for (int a = 0; a < WH; ++a)
+#pragma unroll
+      for (int b = 0; b < WW; ++b) {
+        const float v = ld_f(x, base + a * WP + b);
+        if (MAX) acc = v > acc ? v : acc;
+        else acc += v;
+      }
+  } else {
+    for (uint32_t a = 0; a < wh; ++a)
+      for (uint32_t b = 0; b < ww; ++b) {
+        const float v = ld_f(x, base + a * WP + b);
+        if (MAX) acc = v > acc ? v : acc;
+        else acc += v;
+      }
+  }
+  return acc;
+}
+
+// grid: planes * tiles * bands; block 256.  Band b: output rows [b * band_rows, ...), input rows
+// [b * band_rows * sh, last * sh + wh).
+template <typename T, bool MAX, int WH, int WW>
+__global__ __launch_bounds__(kPoolThreads) void pool_fwd_band_kernel(const PoolParams P) {
+  extern __shared__ __align__(16) unsigned char pool_lds[];
+  uint32_t pb, band;
+  P.div_bands.divmod(blockIdx.x, pb, band);
+  const uint32_t tile = pb / P.planes, plane = pb - tile * P.planes;
+  const uint32_t oh0 = band * P.band_rows, rows = min(P.band_rows, P.OH - oh0);
+  const uint32_t in_rows = (rows - 1u) * P.sh + P.wh;
+  const T *x = reinterpret_cast<const T *>(P.x[tile]) + (size_t)plane * P.HP * P.WP + (size_t)oh0 * P.sh * P.WP;
+  T *y = reinterpret_cast<T *>(P.out[tile]) + (size_t)plane * P.OH * P.OW + (size_t)oh0 * P.OW;
+  const T *xl = stage_contiguous(reinterpret_cast<T *>(pool_lds), x, in_rows * P.WP);
+  __syncthreads();
+  const uint32_t n_out = rows * P.OW;
+  for (uint32_t o = threadIdx.x; o < n_out; o += kPoolThreads) {
+    uint32_t oh, ow;
+    P.div_OW.divmod(o, oh, ow);
+    const float acc = window_reduce<WH, WW, MAX>(xl, oh * P.sh * P.WP + ow * P.sw, P.WP, P.wh, P.ww);
+    st_f(y, o, MAX ? acc : acc * P.inv_area);
+  }
+}
+
+// grid: planes * tiles * bands; block 256.  Band b owns the padded rows [b * band_rows * sh,
+// (b + 1) * band_rows * sh) (the last band: up to HP) and stages every window row that touches them.
+// WH, WW, S > 0: window and stride (both directions) known at compile time, 0: read from P.
+template <typename T, bool MAX, int WH, int WW, int S>
+__global__ __launch_bounds__(kPoolThreads) void pool_bwd_band_kernel(const PoolParams PP) {
+  extern __shared__ __align__(16) unsigned char pool_lds[];
+  constexpr uint32_t VE = 16u / sizeof(T);
+  struct Shape {
+    const PoolParams &p;
+    __device__ __forceinline__ uint32_t wh() const { return WH > 0 ? (uint32_t)WH : p.wh; }
+    __device__ __forceinline__ uint32_t ww() const { return WW > 0 ? (uint32_t)WW : p.ww; }
+    __device__ __forceinline__ uint32_t sh() const { return S > 0 ? (uint32_t)S : p.sh; }
+    __device__ __forceinline__ uint32_t sw() const { return S > 0 ? (uint32_t)S : p.sw; }
+    __device__ __forceinline__ uint32_t div_sh(uint32_t n) const { return S > 0 ? n / (uint32_t)S : p.div_sh.div(n); }
+    __device__ __forceinline__ uint32_t div_sw(uint32_t n) const { return S > 0 ? n / (uint32_t)S : p.div_sw.div(n); }
+  };
+  const Shape Q{PP};
+  const PoolParams &P = PP;
+  uint32_t pb, band;
+  P.div_bands.divmod(blockIdx.x, pb, band);
+  const uint32_t tile = pb / P.planes, plane = pb - tile * P.planes;
+  const uint32_t r0 = band * P.band_rows * Q.sh();
+  const uint32_t r1 = band + 1u == P.bands ? P.HP : r0 + P.band_rows * Q.sh();
+  // window rows that touch [r0, r1)
+  const uint32_t wr_lo = r0 + 1u > Q.wh() ? Q.div_sh(r0 + Q.sh() - Q.wh()) : 0u;
+  const uint32_t wr_hi = min(Q.div_sh(r1 - 1u), P.OH - 1u);
+  const uint32_t wrows = wr_hi + 1u - wr_lo;  // >= 1: r0 <= (OH - 1) * sh by the choice of bands
+  const uint32_t n_win = wrows * P.OW;
+  const uint32_t x_row0 = wr_lo * Q.sh(), x_rows = (wrows - 1u) * Q.sh() + Q.wh();
+  const T *dy = reinterpret_cast<const T *>(P.dy[tile]) + (size_t)plane * P.OH * P.OW + (size_t)wr_lo * P.OW;
+  T *dx = reinterpret_cast<T *>(P.out[tile]) + (size_t)plane * P.HP * P.WP;
+  // LDS: dy rows | input rows | first-maximum positions
+  T *lds_dy = reinterpret_cast<T *>(pool_lds);
+  const uint32_t dy_room = (n_win + VE + VE - 1u) & ~(VE - 1u);
+  const T *dyl = stage_contiguous(lds_dy, dy, n_win);
+  if (MAX) {
+    T *lds_x = lds_dy + dy_room;
+    const uint32_t x_room = (x_rows * P.WP + VE + VE - 1u) & ~(VE - 1u);
+    const T *x = reinterpret_cast<const T *>(P.x[tile]) + (size_t)plane * P.HP * P.WP + (size_t)x_row0 * P.WP;
+    const T *xl = stage_contiguous(lds_x, x, x_rows * P.WP);
+    // fp32 gradient of the owned rows, shifted like dx so that 16-byte stores line up
+    const uint32_t n_own = (r1 - r0) * P.WP;
+    T *dxo = dx + (size_t)r0 * P.WP;
+    float *gl_base = reinterpret_cast<float *>(lds_x + x_room);
+    const uint32_t gpad = (uint32_t)(reinterpret_cast<uintptr_t>(dxo) & 15u) / (uint32_t)sizeof(T);
+    float *gl = gl_base + gpad;
+    for (uint32_t v = threadIdx.x; v < (gpad + n_own + 3u) / 4u; v += kPoolThreads)
+      reinterpret_cast<float4 *>(gl_base)[v] = make_float4(0.f, 0.f, 0.f, 0.f);
+    __syncthreads();
+    // Windows whose row and column indices agree modulo ceil(wh / sh) and ceil(ww / sw) are disjoint:
+    // one class at a time, every window adds its dy onto its first maximum without atomics, and an
+    // element's terms are added in class order whatever the banding is.
+    const uint32_t ch = (Q.wh() + Q.sh() - 1u) / Q.sh(), cw = (Q.ww() + Q.sw() - 1u) / Q.sw();
+    const int32_t g_shift = ((int32_t)x_row0 - (int32_t)r0) * (int32_t)P.WP;
+    for (uint32_t ca = 0; ca < ch; ++ca)
+      for (uint32_t cb = 0; cb < cw; ++cb) {
+        const uint32_t first_oh = wr_lo + (ca + ch - wr_lo % ch) % ch;
+        const uint32_t nrow_c = first_oh <= wr_hi ? (wr_hi - first_oh) / ch + 1u : 0u;
+        const uint32_t ncol_c = cb < P.OW ? (P.OW - 1u - cb) / cw + 1u : 0u;
+        for (uint32_t t = threadIdx.x; t < nrow_c * ncol_c; t += kPoolThreads) {
+          const uint32_t wi = t / ncol_c, wj = t - wi * ncol_c;
+          const uint32_t ohl = first_oh - wr_lo + wi * ch, ow = cb + wj * cw;
+          const uint32_t base = ohl * Q.sh() * P.WP + ow * Q.sw();
+          float best = -__builtin_inff();
+          uint32_t at = base;
+          if (WH > 0) {
+#pragma unroll
+            for (int a = 0; a < WH; ++a)
+#pragma unroll
+              for (int b = 0; b < WW; ++b) {
+                const float v = ld_f(xl, base + a * P.WP + b);
+                if (v > best) { best = v; at = base + a * P.WP + b; }
+              }
+          } else {
+            for (uint32_t a = 0; a < Q.wh(); ++a)
+              for (uint32_t b = 0; b < Q.ww(); ++b) {
+                const float v = ld_f(xl, base + a * P.WP + b);
+                if (v > best) { best = v; at = base + a * P.WP + b; }
+              }
+          }
+          const uint32_t gi = (uint32_t)((int32_t)at + g_shift);
+          if (gi < n_own) gl[gi] += ld_f(dyl, ohl * P.OW + ow);
+        }
+        __syncthreads();
+      }
+    unstage_contiguous(dxo, gl, n_own, P.beta != 0.f);
+  } else {
+    __syncthreads();
+    const uint32_t n_own = (r1 - r0) * P.WP;
+    for (uint32_t j = threadIdx.x; j < n_own; j += kPoolThreads) {
+      uint32_t ihb, iw;
+      P.div_WP.divmod(j, ihb, iw);
+      const uint32_t ih = r0 + ihb;
+      const uint32_t oh_hi = min(Q.div_sh(ih), P.OH - 1u);
+      const uint32_t oh_lo = ih + 1u > Q.wh() ? Q.div_sh(ih + Q.sh() - Q.wh()) : 0u;
+      const uint32_t ow_hi = min(Q.div_sw(iw), P.OW - 1u);
+      const uint32_t ow_lo = iw + 1u > Q.ww() ? Q.div_sw(iw + Q.sw() - Q.ww()) : 0u;
+      float g = 0.f;
+      for (uint32_t oh = oh_lo; oh <= oh_hi; ++oh)
+        for (uint32_t ow = ow_lo; ow <= ow_hi; ++ow) g += ld_f(dyl, (oh - wr_lo) * P.OW + ow);
+      g *= P.inv_area;
+      const size_t i = (size_t)r0 * P.WP + j;
+      if (P.beta != 0.f) g += ld_f(dx, i);
+      st_f(dx, i, g);
+    }
+  }
+}
 
 // grid: (planes * tiles, ceil(OH / 4), ceil(OW / 64)); block 64 x 4 (4 output rows share a block)
 template <typename T, bool MAX>
@@ -117,6 +358,71 @@ static void launch_bwd(int dtype, const PoolParams &P, dim3 grid, hipStream_t st
   else hipLaunchKernelGGL((pool_bwd_kernel<uint16_t, MAX>), grid, dim3(64, 4), 0, st, P);
 }
 
+// ---- banded route: band size, LDS bytes, launches ----
+
+static size_t fwd_band_lds(const PoolParams &P, size_t es, uint32_t rows) {
+  return ((size_t)((rows - 1u) * P.sh + P.wh) * P.WP * es + 16u + 15u) & ~(size_t)15u;
+}
+static size_t bwd_band_lds(const PoolParams &P, size_t es, bool max, uint32_t rows) {
+  const uint64_t wrows = std::min<uint64_t>(P.OH, (uint64_t)rows + (P.wh - 1u) / P.sh);
+  const uint64_t n_win = wrows * P.OW;
+  size_t b = ((n_win * es + 16u + 15u) & ~(size_t)15u);
+  if (max) {
+    const uint64_t own_rows = std::min<uint64_t>(P.HP, (uint64_t)rows * P.sh + P.wh);
+    b += ((((wrows - 1u) * P.sh + P.wh) * P.WP * es + 16u + 15u) & ~(size_t)15u) + (own_rows * P.WP + 8u) * 4u;
+  }
+  return b;
+}
+
+// Picks the rows per band: as many as fit the LDS aimed at per block, fewer while the launch would
+// have too few blocks to fill the chip.  Returns 0 when not even one row fits (direct route).
+template <typename F>
+static uint32_t pick_band_rows(const PoolParams &P, uint32_t num_tiles, size_t aim, F lds_bytes) {
+  if (lds_bytes(1u) > kPoolMaxLds) return 0;
+  uint32_t rows = 1;
+  while (rows < P.OH && lds_bytes(rows + 1u) <= aim) ++rows;
+  const uint64_t pt = (uint64_t)P.planes * num_tiles;
+  while (rows > 1u && pt * ((P.OH + rows - 1u) / rows) < 2048u) rows = (rows + 1u) / 2u;
+  if (pt * ((P.OH + rows - 1u) / rows) >= (1ull << 24)) return 0;
+  return rows;
+}
+
+static void set_bands(PoolParams *P, uint32_t rows) {
+  P->band_rows = rows;
+  P->bands = (P->OH + rows - 1u) / rows;
+  P->div_bands = FastDiv(P->bands);
+  P->div_OW = FastDiv(P->OW);
+  P->div_WP = FastDiv(P->WP);
+}
+
+template <typename T, bool MAX>
+static void launch_fwd_band_t(const PoolParams &P, uint32_t blocks, size_t lds, hipStream_t st) {
+  if (P.wh == 3 && P.ww == 3)
+    hipLaunchKernelGGL((pool_fwd_band_kernel<T, MAX, 3, 3>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+  else if (P.wh == 2 && P.ww == 2)
+    hipLaunchKernelGGL((pool_fwd_band_kernel<T, MAX, 2, 2>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+  else
+    hipLaunchKernelGGL((pool_fwd_band_kernel<T, MAX, 0, 0>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+}
+template <typename T, bool MAX>
+static void launch_bwd_band_t(const PoolParams &P, uint32_t blocks, size_t lds, hipStream_t st) {
+  const bool s2 = P.sh == 2 && P.sw == 2;
+  if (P.wh == 3 && P.ww == 3 && s2)
+    hipLaunchKernelGGL((pool_bwd_band_kernel<T, MAX, 3, 3, 2>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+  else if (P.wh == 2 && P.ww == 2 && s2)
+    hipLaunchKernelGGL((pool_bwd_band_kernel<T, MAX, 2, 2, 2>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+  else
+    hipLaunchKernelGGL((pool_bwd_band_kernel<T, MAX, 0, 0, 0>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+}
+static void launch_fwd_band(int dtype, bool max, const PoolParams &P, uint32_t blocks, size_t lds, hipStream_t st) {
+  if (dtype == ADH_F32) max ? launch_fwd_band_t<float, true>(P, blocks, lds, st) : launch_fwd_band_t<float, false>(P, blocks, lds, st);
+  else max ? launch_fwd_band_t<uint16_t, true>(P, blocks, lds, st) : launch_fwd_band_t<uint16_t, false>(P, blocks, lds, st);
+}
+static void launch_bwd_band(int dtype, bool max, const PoolParams &P, uint32_t blocks, size_t lds, hipStream_t st) {
+  if (dtype == ADH_F32) max ? launch_bwd_band_t<float, true>(P, blocks, lds, st) : launch_bwd_band_t<float, false>(P, blocks, lds, st);
+  else max ? launch_bwd_band_t<uint16_t, true>(P, blocks, lds, st) : launch_bwd_band_t<uint16_t, false>(P, blocks, lds, st);
+}
+
 }  // namespace adh
 
 using namespace adh;
@@ -137,6 +443,13 @@ int adh_pool2d_slab_fwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t 
     if (!aligned_to(x_pad_tiles[t], es) || !aligned_to(y_tiles[t], es)) return ADH_EALIGN;
     P.x[t] = x_pad_tiles[t];
     P.out[t] = y_tiles[t];
+  }
+  const uint32_t band_rows = pick_band_rows(P, num_tiles, kPoolBandBytes, [&](uint32_t r) { return fwd_band_lds(P, es, r); });
+  if (band_rows) {
+    set_bands(&P, band_rows);
+    launch_fwd_band(dtype, mode == ADH_POOL_MAX, P, P.planes * num_tiles * P.bands, fwd_band_lds(P, es, band_rows),
+                    as_stream(stream));
+    return launch_status();
   }
   const uint64_t gz = (uint64_t)P.planes * num_tiles;
   if (gz >= (1ull << 26) || (P.OH + 3u) / 4u > 65535u || (P.OW + 63u) / 64u > 65535u) return ADH_EINVAL;
@@ -178,6 +491,15 @@ int adh_pool2d_slab_bwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t 
     P.out[t] = dx_pad_tiles[t];
   }
   P.beta = beta;
+  const bool is_max = mode == ADH_POOL_MAX;
+  const uint32_t band_rows =
+      wh * ww > 256u ? 0u : pick_band_rows(P, num_tiles, is_max ? 2u * kPoolBandBytes : kPoolBandBytes, [&](uint32_t r) { return bwd_band_lds(P, es, is_max, r); });
+  if (band_rows) {
+    set_bands(&P, band_rows);
+    launch_bwd_band(dtype, is_max, P, P.planes * num_tiles * P.bands, bwd_band_lds(P, es, is_max, band_rows),
+                    as_stream(stream));
+    return launch_status();
+  }
   const uint64_t gz = (uint64_t)P.planes * num_tiles;
   if (gz >= (1ull << 26) || (HP + 3u) / 4u > 65535u || (WP + 63u) / 64u > 65535u) return ADH_EINVAL;
   dim3 grid((uint32_t)gz, (HP + 3u) / 4u, (WP + 63u) / 64u);

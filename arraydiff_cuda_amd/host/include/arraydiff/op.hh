@@ -770,6 +770,103 @@ template <typename V, typename A, typename B = A>
 using CudnnConv2DOp = SlabConv2DOp<V, A>;
 
 // ---------------------------------------------------------------------------
+// pooling over the halo-padded slab
+// ---------------------------------------------------------------------------
+enum Pooling {
+  kAveragePool,
+  kMaxPool,
+};
+
+class Pool2DShape {
+public:
+  Pooling pooling;
+  array<size_t, 2> axes;
+  array<size_t, 2> window;
+  array<size_t, 2> stride;
+  array<size_t, 2> pad;
+  bool halo_padded_input;
+};
+
+// V = GPUBatchArray3D<float>.  With halo_padded_input the padded tile is pooled as a plain packed
+// tensor with pad 0 (the halo holds the padding: neighbour rows after a halo exchange, zeros at the
+// image border); without it the input must be packed and pad must be 0 (the global pooling before
+// the classifier).  Implicit zero padding of an unpadded input is not part of this path and throws
+// at construction.  One node serves all ranks it was made for: the K tiles go to the device in ONE
+// launch per pass.
+template <typename V>
+class SlabPool2DOp : public virtual Op, public virtual Var<V> {
+public:
+  static shared_ptr<Var<V>> Make(Pool2DShape shape, shared_ptr<Var<V>> input, shared_ptr<Context> ctx) {
+    return make_shared<SlabPool2DOp<V>>(shape, vector<shared_ptr<Var<V>>>{input}, ctx);
+  }
+  static vector<shared_ptr<Var<V>>> MakeParallel(Pool2DShape shape, vector<shared_ptr<Var<V>>> inputs,
+                                                 shared_ptr<Context> ctx) {
+    auto op = make_shared<SlabPool2DOp<V>>(shape, inputs, ctx);
+    vector<shared_ptr<Var<V>>> outputs;
+    for (size_t r = 0; r < inputs.size(); ++r) outputs.push_back(make_shared<NoOp<V>>(op, op->ys_.at(r).clone()));
+    return outputs;
+  }
+  SlabPool2DOp(Pool2DShape shape, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx)
+      : ctx_(ctx), shape_(shape), x_vars_(inputs) {
+    if (shape.pooling != kAveragePool && shape.pooling != kMaxPool)
+      throw std::invalid_argument("SlabPool2DOp: unknown pooling");
+    if (!shape.halo_padded_input && (shape.pad[0] != 0 || shape.pad[1] != 0))
+      throw std::invalid_argument("SlabPool2DOp: padding needs a halo-padded input");
+    if (shape.window[0] == 0 || shape.window[1] == 0 || shape.stride[0] == 0 || shape.stride[1] == 0)
+      throw std::invalid_argument("SlabPool2DOp: empty window or stride");
+    if (inputs.empty() || inputs.size() > ADH_MAX_TILES) throw std::invalid_argument("SlabPool2DOp: bad tile count");
+    for (size_t r = 0; r < inputs.size(); ++r) {
+      auto off = inputs[r]->offset();
+      if (off.shape[0] != shape.pad[0] || off.shape[1] != shape.pad[1] || off.shape[2] != 0)
+        throw std::invalid_argument("SlabPool2DOp: input halo must equal the pooling pad");
+      if (inputs[r]->shape() != inputs[0]->shape() || inputs[r]->batch_shape() != inputs[0]->batch_shape())
+        throw std::invalid_argument("SlabPool2DOp: all tiles must have one shape");
+      xs_.push_back(inputs[r]->data());
+      ys_.push_back(VarData<V>(_get_output_shape(inputs[r]->shape()), inputs[r]->batch_shape()));
+    }
+  }
+  // out = floor((in + 2 pad - window) / stride) + 1 per axis, channels kept (what
+  // cudnnGetPooling2dForwardOutputDim returns, op.cc:3346-3385)
+  Shape3D _get_output_shape(Shape3D in_shape) {
+    size_t out[2];
+    for (int a = 0; a < 2; ++a) {
+      const size_t padded = in_shape.shape[a] + 2 * shape_.pad[a];
+      if (padded < shape_.window[a]) throw std::invalid_argument("SlabPool2DOp: window larger than the padded input");
+      out[a] = (padded - shape_.window[a]) / shape_.stride[a] + 1;
+    }
+    return Shape3D(out[0], out[1], in_shape.shape[2]);
+  }
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) {
+      for (auto &x : x_vars_) x->_push(e, apply);
+      apply(this);
+    }
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) {
+      apply(this);
+      for (size_t r = x_vars_.size(); r-- > 0;) x_vars_[r]->_pop(e, apply);
+    }
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+  virtual typename V::Shape shape() { return ys_[0].shape(); }
+  virtual typename V::Shape offset() { return ys_[0].offset(); }
+  virtual typename V::Shape stride() { return ys_[0].stride(); }
+  virtual size_t batch_shape() { return ys_[0].batch_shape(); }
+  virtual VarData<V> data() { return ys_[0].clone(); }
+
+private:
+  shared_ptr<Context> ctx_;
+  Pool2DShape shape_;
+  vector<shared_ptr<Var<V>>> x_vars_;
+  vector<VarData<V>> xs_;
+  vector<VarData<V>> ys_;
+};
+template <typename V>
+using CudnnPool2DOp = SlabPool2DOp<V>;
+
+// ---------------------------------------------------------------------------
 // softmax + negative log likelihood (1-D logits)
 // ---------------------------------------------------------------------------
 template <typename V, typename Label, typename Loss>

@@ -446,6 +446,78 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
   }
 }
 
+// ---- SlabPool2DOp (op.cc:3405-3530 forward, 3532-3660 backward) ----
+template <>
+void SlabPool2DOp<V3>::_forward(TxnId txn) {
+  const size_t K = xs_.size();
+  const void *xt[ADH_MAX_TILES];
+  void *yt[ADH_MAX_TILES];
+  uint32_t n = 0;
+  TileDims d{};
+  for (size_t r = 0; r < K; ++r) {
+    if (!ys_[r].val().overwrite(txn, id(), rank_ctx(ctx_, r))) continue;
+    V3 &x = xs_[r].val().get(txn, id());
+    V3 &y = ys_[r].val().get_excl(txn, id());
+    d = dims_of(x);
+    y.set_batch_size(d.N);
+    if (shape_.halo_padded_input) {
+      if (shape_.pad[0] != shape_.pad[1]) throw std::invalid_argument("SlabPool2DOp: halo width must be one number");
+      check_padded(x, shape_.pad[0], "SlabPool2DOp");
+    } else {
+      check_packed(x, "SlabPool2DOp");
+    }
+    xt[n] = x.base_as_view().dptr();
+    yt[n] = y.as_view().dptr();
+    ++n;
+  }
+  if (n == 0) return;
+  GPUConn conn = rank_ctx(ctx_, 0)->conn();
+  adh_check(adh_pool2d_slab_fwd_tiles(ADH_F32, shape_.pooling == kMaxPool ? ADH_POOL_MAX : ADH_POOL_AVG, n, d.N, d.C,
+                                      d.H + 2 * (uint32_t)shape_.pad[1], d.W + 2 * (uint32_t)shape_.pad[0],
+                                      (uint32_t)shape_.window[1], (uint32_t)shape_.window[0], (uint32_t)shape_.stride[1],
+                                      (uint32_t)shape_.stride[0], xt, yt, conn.stream()),
+            "SlabPool2DOp::_forward");
+}
+
+template <>
+void SlabPool2DOp<V3>::_backward(TxnId txn) {
+  const size_t K = xs_.size();
+  const void *xt[ADH_MAX_TILES];
+  const void *yt[ADH_MAX_TILES];
+  const void *dyt[ADH_MAX_TILES];
+  void *dxt[ADH_MAX_TILES];
+  uint32_t n = 0;
+  TileDims d{};
+  // input gradient over the WHOLE padded tile, zeroed on first touch, beta = 1 (op.cc:3540-3550)
+  for (size_t r = 0; r < K; ++r) {
+    GPUContext *dc = rank_ctx(ctx_, r);
+    const size_t batch = xs_[r].val().get(txn, id()).batch_size();
+    if (!xs_[r].grad().accumulate(txn, id(), dc, [dc, batch](V3 *g) {
+          GPUConn conn = dc->conn();
+          g->set_batch_size(batch);
+          g->base_as_view().set_constant(0.0f, conn);
+        }))
+      continue;
+    V3 &x = xs_[r].val().get(txn, id());
+    V3 &dx = xs_[r].grad().get_mut(txn, id());
+    d = dims_of(x);
+    if (shape_.halo_padded_input) check_padded(dx, shape_.pad[0], "SlabPool2DOp");
+    else check_packed(dx, "SlabPool2DOp");
+    xt[n] = x.base_as_view().dptr();
+    yt[n] = ys_[r].val().get(txn, id()).as_view().dptr();
+    dyt[n] = ys_[r].grad().get(txn, id()).as_view().dptr();
+    dxt[n] = dx.base_as_view().dptr();
+    ++n;
+  }
+  if (n == 0) return;
+  GPUConn conn = rank_ctx(ctx_, 0)->conn();
+  adh_check(adh_pool2d_slab_bwd_tiles(ADH_F32, shape_.pooling == kMaxPool ? ADH_POOL_MAX : ADH_POOL_AVG, n, d.N, d.C,
+                                      d.H + 2 * (uint32_t)shape_.pad[1], d.W + 2 * (uint32_t)shape_.pad[0],
+                                      (uint32_t)shape_.window[1], (uint32_t)shape_.window[0], (uint32_t)shape_.stride[1],
+                                      (uint32_t)shape_.stride[0], xt, yt, dyt, dxt, 1.0f, conn.stream()),
+            "SlabPool2DOp::_backward");
+}
+
 // ---- SoftmaxNLLLossOp, 1-D logits (op.cc:4118-4188) ----
 typedef GPUBatchArray1D<float> V1;
 typedef GPUBatchArray0D<uint32_t> L0;

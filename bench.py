@@ -267,7 +267,7 @@ def main():
         add("max pool 3x3 s2 bwd over padded tiles (fp32)",
             lambda: lib.adh_pool2d_slab_bwd_tiles(0, 1, K, N, C, Hq, Wq, 3, 3, 2, 2, xq_tbl, yq_tbl, dq_tbl, gq_tbl,
                                                   0.0, stream),
-            "hbm", 2 * in_b + 2 * out_b, HBM_PEAK_GBS, "GB/s")
+            "hbm", 2 * in_b + out_b, HBM_PEAK_GBS, "GB/s", note="reads x and dy, writes dx; y is not read")
         del xq, yq, dq, gq
         out["secondary"] = sec
 

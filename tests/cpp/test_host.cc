@@ -25,6 +25,10 @@ void orc_halo_pad(int dtype, uint32_t p, uint32_t W, uint32_t H, uint32_t C, uin
 void orc_halo_unpad(int dtype, uint32_t p, uint32_t W, uint32_t H, uint32_t C, uint32_t N, const void *x, void *y);
 int orc_halo_op(int which, int dtype, uint32_t gw, uint32_t gh, uint32_t p, uint32_t W, uint32_t H, uint32_t C,
                 uint32_t N, void *const *tiles);
+void orc_pool_slab_fwd(int mode, uint32_t N, uint32_t C, uint32_t HP, uint32_t WP, uint32_t wh, uint32_t ww, uint32_t sh,
+                       uint32_t sw, const float *x, float *y);
+void orc_pool_slab_bwd(int mode, uint32_t N, uint32_t C, uint32_t HP, uint32_t WP, uint32_t wh, uint32_t ww, uint32_t sh,
+                       uint32_t sw, const float *x, const float *dy, float beta, float *dx);
 void orc_softmax_fwd(uint32_t C, uint32_t N, const float *x, float *y);
 void orc_softmax_nll_loss_fwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label, float *loss);
 void orc_softmax_nll_loss_bwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label, const float *dloss,
@@ -204,6 +208,54 @@ static void test_spatial_conv_graph(size_t K, size_t N, size_t C, size_t Co, siz
   }
 }
 
+// Scatter -> HaloPad(1) -> HaloExch(1) -> Pool(3x3, stride 2, pad 1, halo_padded_input) -> gather:
+// the stem pooling of src/zoo.cc:1562-1573 on K row-tiles of one GPU, against the oracle's pooling
+// of the zero-padded UNSPLIT tensor.
+static void test_spatial_pool_graph(Pooling pooling, size_t K, size_t N, size_t C, size_t H, size_t W) {
+  std::mt19937 gen(4321 + (unsigned)K);
+  auto ctx = MultiGPUContext::Make(K);
+  const size_t OH = (H + 2 - 3) / 2 + 1, OW = (W + 2 - 3) / 2 + 1;
+  std::vector<float> X = uniform(gen, N * C * H * W, -1, 1);
+  std::vector<float> dY = normal(gen, N * C * OH * OW, 1.0f);
+  typedef GPUBatchArray3D<float> V;
+  auto x_src = SrcOp<V>::Make(Shape3D(W, H, C), N, ctx->device_context(0));
+  vector<shared_ptr<Var<V>>> xs(K, x_src);
+  auto tiles = SpatialScatter2DOp<V>::MakeParallel(xs, ctx);
+  auto padded = HaloPad2DOp<V>::MakeParallel(1, tiles, ctx);
+  auto exch = HaloExch2DOp<V>::MakeParallel(1, padded, ctx);
+  Pool2DShape ps;
+  ps.pooling = pooling;
+  ps.axes = {0, 1};
+  ps.window = {3, 3};
+  ps.stride = {2, 2};
+  ps.pad = {1, 1};
+  ps.halo_padded_input = true;
+  auto ys = CudnnPool2DOp<V>::MakeParallel(ps, exch, ctx);
+  auto y_full = SpatialJoinedGather2DOp<V>::Make(ys, ctx);
+  auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
+  sink->set_host_grad(dY.data());
+  CHECK(ys[0]->shape() == Shape3D(OW, OH / K, C));
+  for (int rep = 0; rep < 2; ++rep) {
+    TxnId txn;
+    x_src->load(txn, X.data());
+    sink->gradient(txn);
+    ctx->sync();
+    std::vector<float> Y(dY.size()), dX(X.size());
+    sink->store_val(txn, Y.data());
+    x_src->store_grad(txn, dX.data());
+    std::vector<float> Xp(N * C * (H + 2) * (W + 2)), Yr(Y.size()), dXp(Xp.size()), dXr(X.size());
+    orc_halo_pad(0, 1, W, H, C, N, X.data(), Xp.data());
+    const int mode = pooling == kMaxPool ? 1 : 0;
+    orc_pool_slab_fwd(mode, N, C, H + 2, W + 2, 3, 3, 2, 2, Xp.data(), Yr.data());
+    orc_pool_slab_bwd(mode, N, C, H + 2, W + 2, 3, 3, 2, 2, Xp.data(), dY.data(), 0.f, dXp.data());
+    orc_halo_unpad(0, 1, W, H, C, N, dXp.data(), dXr.data());
+    const double ey = rel_err(Y, Yr), ex = rel_err(dX, dXr);
+    std::printf("pool graph %s K=%zu N=%zu C=%zu %zux%zu rep %d: rel-err y %.2e dx %.2e\n", mode ? "max" : "avg", K, N, C, H,
+                W, rep, ey, ex);
+    CHECK(ey <= 1e-5 && ex <= 1e-5);
+  }
+}
+
 // The call sequence of tools/microbench_spatial_conv.cc:227-263: raw buffers, per-rank
 // group_start / halo_exchange / group_end, no Op machinery.
 static void test_microbench_sequence() {
@@ -325,6 +377,31 @@ static void test_txn_hazards() {
     bad = true;
   }
   CHECK(bad);
+  bad = false;
+  try {
+    Pool2DShape ps{};
+    ps.pooling = kMaxPool; ps.window = {3, 3}; ps.stride = {2, 2}; ps.pad = {1, 1}; ps.halo_padded_input = false;
+    auto q = CudnnPool2DOp<V>::Make(ps, src, ctx);  // implicit zero padding is not on this path
+  } catch (const std::invalid_argument &) {
+    bad = true;
+  }
+  CHECK(bad);
+  // pooling a packed input without padding: the global average before the classifier
+  Pool2DShape gp{};
+  gp.pooling = kAveragePool; gp.window = {4, 4}; gp.stride = {4, 4}; gp.pad = {0, 0}; gp.halo_padded_input = false;
+  auto pooled = CudnnPool2DOp<V>::Make(gp, src, ctx);
+  CHECK(pooled->shape() == Shape3D(1, 1, 2));
+  auto psink = HostGradSinkOp<V>::Make(pooled, ctx);
+  std::vector<float> pg(2, 1.0f), py(2), pdx(32);
+  psink->set_host_grad(pg.data());
+  TxnId t3;
+  src->load(t3, x.data());
+  psink->gradient(t3);
+  ctx->sync();
+  psink->store_val(t3, py.data());
+  src->store_grad(t3, pdx.data());
+  CHECK(py[0] == 8.5f && py[1] == 24.5f);
+  for (float v : pdx) CHECK(v == 1.0f / 16);
 }
 
 int main(int argc, char **argv) {
@@ -338,6 +415,9 @@ int main(int argc, char **argv) {
     test_spatial_conv_graph(2, 3, 5, 7, 6, 9);
     test_spatial_conv_graph(1, 1, 16, 16, 5, 5);
     test_spatial_conv_graph(4, 4, 64, 64, 56, 56);
+    test_spatial_pool_graph(kMaxPool, 4, 2, 8, 16, 12);
+    test_spatial_pool_graph(kAveragePool, 2, 3, 5, 8, 10);
+    test_spatial_pool_graph(kMaxPool, 4, 8, 64, 112, 112);
     test_softmax_loss_op();
   }
   std::printf("%s: %d failure(s)\n", mode.c_str(), failures);

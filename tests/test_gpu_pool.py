@@ -15,7 +15,11 @@ pytestmark = pytest.mark.gpu
 TOL32, TOL16 = 1e-5, 2.0 ** -8
 
 CASES = [(1, 2, 3, 8, 9, 3, 3, 2, 2), (2, 1, 2, 7, 7, 2, 2, 2, 2), (1, 1, 1, 6, 70, 3, 3, 1, 1), (3, 2, 2, 9, 8, 3, 2, 2, 1),
-         (1, 1, 1, 5, 5, 5, 5, 1, 1), (1, 1, 2, 4, 6, 1, 1, 1, 1), (2, 1, 1, 10, 131, 2, 2, 3, 3), (4, 2, 5, 30, 114, 3, 3, 2, 2)]
+         (1, 1, 1, 5, 5, 5, 5, 1, 1), (1, 1, 2, 4, 6, 1, 1, 1, 1), (2, 1, 1, 10, 131, 2, 2, 3, 3), (4, 2, 5, 30, 114, 3, 3, 2, 2),
+         # several bands of several rows per plane (enough planes that the bands stay tall)
+         (1, 8, 64, 64, 200, 3, 3, 2, 2), (1, 8, 64, 61, 203, 2, 2, 2, 2), (1, 4, 64, 40, 150, 5, 3, 1, 2),
+         # rows too wide to stage / windows over 256 elements: the direct kernels
+         (1, 1, 1, 4, 11000, 3, 3, 1, 1), (1, 1, 2, 20, 21, 17, 17, 1, 2)]
 
 
 def out_dims(HP, WP, wh, ww, sh, sw):
@@ -53,7 +57,8 @@ def test_pool_f32_vs_oracle(oracle, mode, K, N, C, HP, WP, wh, ww, sh, sw):
 
 
 @pytest.mark.parametrize("mode", [capi.ADH_POOL_AVG, capi.ADH_POOL_MAX])
-@pytest.mark.parametrize("K,N,C,HP,WP,wh,ww,sh,sw", [CASES[0], CASES[3], CASES[6], CASES[7]])
+@pytest.mark.parametrize("K,N,C,HP,WP,wh,ww,sh,sw", [CASES[0], CASES[3], CASES[6], CASES[7], CASES[8], CASES[9], CASES[11],
+                                                     CASES[12]])
 def test_pool_bf16_vs_oracle(oracle, mode, K, N, C, HP, WP, wh, ww, sh, sw):
     rng = np.random.default_rng(32 + WP)
     OH, OW = out_dims(HP, WP, wh, ww, sh, sw)
