@@ -50,6 +50,17 @@ def time_gpu(fn, reps, warmup):
     return e0.elapsed_time(e1) / reps
 
 
+def time_gpu_flushed(fn, reps, scratch):
+    """Average milliseconds per call of fn() when every call is preceded by a rewrite of `scratch`
+    (512 MB, twice the on-package cache), so that fn's operands come from HBM: the time of a
+    (rewrite, fn) loop minus the time of the rewrite loop alone, best of three."""
+    both, alone = [], []
+    for i in range(3):
+        alone.append(time_gpu(lambda: scratch.fill_(1.0), reps, 3))
+        both.append(time_gpu(lambda: (scratch.fill_(1.0), fn()), reps, 3))
+    return max(min(both) - min(alone), 1e-6)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -156,11 +167,21 @@ def main():
         reps, wu = 200, 20
         sec = []
 
-        def add(name, fn, bound, work, peak, unit, note=None):
+        flush_scratch = torch.empty(128 * 1024 * 1024, device="cuda")  # 512 MB
+
+        def add(name, fn, bound, work, peak, unit, note=None, flushed=False):
             ms = time_gpu(fn, reps, wu)
             ach = work / (ms * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
             e = {"name": name, "ms": round(ms, 5), "bound": bound, "achieved": round(ach, 3), "peak": peak,
                  "unit": unit, "frac": round(ach / peak, 4), "work": work}
+            if flushed:
+                # the warm figure above has its operands resident in the 256 MB on-package cache;
+                # this one rewrites 512 MB before every call
+                msf = time_gpu_flushed(fn, 30, flush_scratch)
+                achf = work / (msf * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
+                e["ms_flushed"] = round(msf, 5)
+                e["achieved_flushed"] = round(achf, 3)
+                e["frac_flushed"] = round(achf / peak, 4)
             if note:
                 e["note"] = note
             sec.append(e)
@@ -169,10 +190,10 @@ def main():
         padded_b = K * N * C * (Ht + 2 * p) * (W + 2 * p) * es
         add("halo pack cfg1 (unsplit -> 4 padded tiles)",
             lambda: lib.adh_tiles_pack_nchw(0, K, p, W, H, C, N, X.data_ptr(), tile_tbl, stream),
-            "hbm", unsplit_b + padded_b, HBM_PEAK_GBS, "GB/s")
+            "hbm", unsplit_b + padded_b, HBM_PEAK_GBS, "GB/s", flushed=True)
         add("halo unpack cfg1 (4 padded tiles -> unsplit)",
             lambda: lib.adh_tiles_unpack_nchw(0, K, p, W, H, C, N, tile_tbl, Y.data_ptr(), stream),
-            "hbm", 2 * unsplit_b, HBM_PEAK_GBS, "GB/s")
+            "hbm", 2 * unsplit_b, HBM_PEAK_GBS, "GB/s", flushed=True)
         add("halo exchange cfg1 (6 strips)",
             lambda: lib.adh_halo_exchange_nchw(0, 1, K, p, W, Ht, C, N, tile_tbl, stream),
             "hbm", 2 * 2 * (K - 1) * strip, HBM_PEAK_GBS, "GB/s",
@@ -184,7 +205,7 @@ def main():
         add("channel slice [16,48) cfg4",
             lambda: lib.adh_slice_copy_nchw(0, W, H, 32, N, X.data_ptr(), W, H, C, 0, 0, 16, sl.data_ptr(), W, H, 32,
                                             0, 0, 0, stream),
-            "hbm", 2 * N * 32 * H * W * es, HBM_PEAK_GBS, "GB/s")
+            "hbm", 2 * N * 32 * H * W * es, HBM_PEAK_GBS, "GB/s", flushed=True)
         Ns, Cs = 256, 1000
         logits = torch.randn((Ns, Cs), device="cuda", generator=g) * 2
         labels = torch.randint(0, Cs, (Ns,), device="cuda", dtype=torch.int32)
@@ -195,7 +216,7 @@ def main():
         add("softmax + nll fwd cfg4 (256x1000)",
             lambda: lib.adh_softmax_xent_fwd(Cs, Ns, logits.data_ptr(), labels.data_ptr(), sy.data_ptr(),
                                              sloss.data_ptr(), stream),
-            "hbm", 2 * Ns * Cs * 4 + 8 * Ns, HBM_PEAK_GBS, "GB/s")
+            "hbm", 2 * Ns * Cs * 4 + 8 * Ns, HBM_PEAK_GBS, "GB/s", flushed=True)
         add("softmax-nll bwd cfg4 (256x1000)",
             lambda: lib.adh_softmax_nll_loss_bwd(Cs, Ns, sy.data_ptr(), labels.data_ptr(), dl.data_ptr(),
                                                  sdx.data_ptr(), stream),
@@ -268,7 +289,7 @@ def main():
             lambda: lib.adh_pool2d_slab_bwd_tiles(0, 1, K, N, C, Hq, Wq, 3, 3, 2, 2, xq_tbl, yq_tbl, dq_tbl, gq_tbl,
                                                   0.0, stream),
             "hbm", 2 * in_b + out_b, HBM_PEAK_GBS, "GB/s", note="reads x and dy, writes dx; y is not read")
-        del xq, yq, dq, gq
+        del xq, yq, dq, gq, flush_scratch
         out["secondary"] = sec
 
     # ---- CPU baseline: the scalar port, single thread, on a bounded sample ----
@@ -297,6 +318,23 @@ def main():
             oracle.halo_op(oracle.EXCH, 1, K, p, W, Ht, C, N, host_tiles)
         dt = (time.perf_counter() - t0) / reps_cpu
         out["cpu_baseline"]["halo_exchange_GBs"] = round(2 * 2 * (K - 1) * p * W * C * N * 4 / dt / 1e9, 3)
+        # configs[0]: pack (scatter + pad + exchange) and unpack (unpad + gather) of the unsplit tensor
+        host_X = X.cpu().numpy()
+        host_Y = np.empty_like(host_X)
+        reps_cpu = 3
+        t0 = time.perf_counter()
+        for _ in range(reps_cpu):
+            oracle.tiles_pack(K, p, W, H, C, N, host_X, host_tiles)
+        dt_pack = (time.perf_counter() - t0) / reps_cpu
+        t0 = time.perf_counter()
+        for _ in range(reps_cpu):
+            oracle.tiles_unpack(K, p, W, H, C, N, host_tiles, host_Y)
+        dt_unpack = (time.perf_counter() - t0) / reps_cpu
+        assert np.array_equal(host_Y, host_X)
+        unsplit_b = N * C * H * W * 4
+        padded_b = K * N * C * (Ht + 2 * p) * (W + 2 * p) * 4
+        out["cpu_baseline"]["halo_pack_GBs"] = round((unsplit_b + padded_b) / dt_pack / 1e9, 3)
+        out["cpu_baseline"]["halo_unpack_GBs"] = round(2 * unsplit_b / dt_unpack / 1e9, 3)
 
     print(json.dumps(out))
 
