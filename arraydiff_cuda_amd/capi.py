@@ -47,6 +47,9 @@ SIGNATURES = {
     "adh_conv3x3_slab_bwd_data_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_filter": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_filter_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp, f32, vp, sz, vp]),
+    "adh_conv2d_workspace_bytes": (sz, [i32, i32] + [u32] * 12),
+    "adh_conv2d_slab_fwd_tiles": (i32, [i32] + [u32] * 12 + [vpp, vp, vpp, f32, vp, sz, vp]),
+    "adh_conv2d_slab_bwd_data_tiles": (i32, [i32] + [u32] * 12 + [vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_pool2d_slab_fwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp]),
     "adh_pool2d_slab_fwd": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, vp, vp, vp]),
     "adh_pool2d_slab_bwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vpp, vpp, vpp, f32, vp]),
@@ -229,6 +232,28 @@ def conv_bwd_data_tiles(w, dys, dxs, N, Cin, Cout, H, W, beta=0.0, ws=None):
     wp, wb = _ws(ws)
     return lib().adh_conv3x3_slab_bwd_data_tiles(_dt(dys[0]), len(dys), N, Cin, Cout, H, W, w.data_ptr(), dt, xt,
                                                  beta, wp, wb, _stream())
+
+
+def conv2d_workspace_bytes(which, dtype, K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw):
+    return lib().adh_conv2d_workspace_bytes(which, dtype, K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw)
+
+
+def conv2d_fwd_tiles(xs, w, ys, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, beta=0.0, ws=None):
+    _dev(*xs, w, *ys)
+    xt, k1 = _tbl(xs)
+    yt, k2 = _tbl(ys)
+    wp, wb = _ws(ws)
+    return lib().adh_conv2d_slab_fwd_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, xt,
+                                           w.data_ptr(), yt, beta, wp, wb, _stream())
+
+
+def conv2d_bwd_data_tiles(w, dys, dxs, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, beta=0.0, ws=None):
+    _dev(w, *dys, *dxs)
+    dt, k1 = _tbl(dys)
+    gt, k2 = _tbl(dxs)
+    wp, wb = _ws(ws)
+    return lib().adh_conv2d_slab_bwd_data_tiles(_dt(dys[0]), len(dys), N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw,
+                                                w.data_ptr(), dt, gt, beta, wp, wb, _stream())
 
 
 def pool_fwd_tiles(mode, xs, ys, N, C, HP, WP, wh, ww, sh, sw):

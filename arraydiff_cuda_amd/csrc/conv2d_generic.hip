@@ -1,0 +1,465 @@
+// General slab convolution on the fp32 matrix cores: any window, stride and dilation, forward and
+// backward-data (the 7x7 stem, stride-2 3x3, 1x1 projections and dilated 3x3 of the networks that
+// feed halo-padded tiles to a convolution).  The 3x3 / stride-1 case has kernels of its own.
+//
+// One kernel serves both passes as a "tap correlation":
+//   out[m][o_r + i*so_r][o_c + j*so_c] (+)= sum over c and taps t of
+//       Wt[t][c][m] * in[c][i*si_r + off_r[t]][j*si_c + off_c[t]]          (zero outside `in`)
+//   forward      : in = padded tile, m = output channel, taps = all (a, b) with offsets (a*dh, b*dw),
+//                  si = stride, so = 1.
+//   backward-data: in = dy, m = input channel, out = the whole padded gradient tile.  Padded pixels
+//                  with the same residues (h' mod sh, w' mod sw) receive the same subset of taps, so
+//                  each residue class is a stride-1 correlation of dy with the taps that satisfy
+//                  a*dh = h' (mod sh), b*dw = w' (mod sw), offsets (h' - a*dh) / sh: up to sh*sw
+//                  sub-problems in one launch, written with output stride (sh, sw).
+// Implicit GEMM: M = 64 output channels per block, N = 16 x 16 output pixels per block (16 n-tiles
+// of 16 consecutive pixels of a row, 4 per wave), K = (tap, channel) in groups of 4 channels for
+// v_mfma_f32_16x16x4_f32.  Per channel chunk the input patch is staged in LDS once; the filter,
+// rewritten beforehand to [m group][chunk][tap][channel][64 m] in the workspace, is staged per tap
+// group.  bf16 tensors are widened while staging and rounded when stored: the arithmetic is fp32.
+#include "adh_common.h"
+
+#include <algorithm>
+#include <vector>
+
+namespace adh {
+
+constexpr int kGenMaxTaps = 64;
+constexpr int kGenMaxSub = 16;
+constexpr uint32_t kGenThreads = 256;
+constexpr uint32_t kGenWPitch = 80;  // floats per (tap, channel) row of 64 m: 4 channel groups on 4 x 16 banks
+constexpr uint32_t kGenLdsBytes = 64u * 1024u;
+
+struct GenSub {
+  uint32_t t0, t1;            // taps of this sub-problem
+  uint32_t GI, GJ, o_r, o_c;  // output sub-grid and where it starts
+  int32_t min_r, min_c;       // smallest tap offsets
+  uint32_t PR, PC;            // patch rows / columns
+  uint32_t nbj, blk0;         // block columns, first block of this sub-problem within an image
+  FastDiv div_PR, div_PC;
+};
+
+struct ConvGenParams {
+  const void *in[ADH_MAX_TILES];
+  void *out[ADH_MAX_TILES];
+  const float *wt;
+  uint32_t N, C, M, MG, in_H, in_W, out_H, out_W;
+  uint32_t si_r, si_c, so_r, so_c;
+  uint32_t CC, nchunks, ntaps, TG;
+  uint32_t TOH, TCT, log2_TCT;
+  uint32_t PCP, PP, w_lds_floats;
+  uint32_t nsub, blocks_per_image;
+  float beta;
+  FastDiv div_bpi, div_MG, div_N;
+  GenSub sub[kGenMaxSub];
+  int16_t off_r[kGenMaxTaps], off_c[kGenMaxTaps];
+};
+
+struct FilterGenParams {
+  const void *w;
+  float *wt;
+  uint32_t M, C, m_stride, c_stride, MG, nchunks, CC, ntaps;
+  uint16_t tap_index[kGenMaxTaps];
+};
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float gen_ld(const float *p, size_t i) { return p[i]; }
+__device__ __forceinline__ float gen_ld(const uint16_t *p, size_t i) { return bf16_bits_to_f32(p[i]); }
+__device__ __forceinline__ void gen_st(float *p, size_t i, float v) { p[i] = v; }
+__device__ __forceinline__ void gen_st(uint16_t *p, size_t i, float v) { p[i] = f32_to_bf16_bits(v); }
+
+// wt[((mg * nchunks + ch) * ntaps + t) * CC + c][m] = w[(mg*64 + m) * m_stride + (ch*CC + c) * c_stride + tap_index[t]]
+template <typename T>
+__global__ __launch_bounds__(256) void conv_gen_filter_kernel(const FilterGenParams F) {
+  const uint32_t total = F.MG * F.nchunks * F.ntaps * F.CC * 64u;
+  for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
+    const uint32_t m = e & 63u;
+    uint32_t r = e >> 6;
+    const uint32_t c = r % F.CC;
+    r /= F.CC;
+    const uint32_t t = r % F.ntaps;
+    r /= F.ntaps;
+    const uint32_t ch = r % F.nchunks, mg = r / F.nchunks;
+    const uint32_t mm = mg * 64u + m, cc = ch * F.CC + c;
+    float v = 0.f;
+    if (mm < F.M && cc < F.C)
+      v = gen_ld(reinterpret_cast<const T *>(F.w), (size_t)mm * F.m_stride + (size_t)cc * F.c_stride + F.tap_index[t]);
+    F.wt[e] = v;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenParams P) {
+  extern __shared__ __align__(16) float gen_lds[];
+  float *wl = gen_lds;
+  float *patch = gen_lds + P.w_lds_floats;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+
+  // block -> (tile, image, m group, sub-problem, block row, block column)
+  uint32_t outer, inner;
+  P.div_bpi.divmod(blockIdx.x, outer, inner);
+  uint32_t img, mg;
+  P.div_MG.divmod(outer, img, mg);
+  uint32_t tile, n;
+  P.div_N.divmod(img, tile, n);
+  uint32_t s = 0;
+  while (s + 1u < P.nsub && inner >= P.sub[s + 1u].blk0) ++s;
+  const GenSub &S = P.sub[s];
+  const uint32_t local = inner - S.blk0;
+  const uint32_t bi = local / S.nbj, bj = local - bi * S.nbj;
+
+  const T *src = reinterpret_cast<const T *>(P.in[tile]) + (size_t)n * P.C * P.in_H * P.in_W;
+  T *dst = reinterpret_cast<T *>(P.out[tile]) + (size_t)n * P.M * P.out_H * P.out_W;
+
+  // this wave's four n-tiles: row and column tile within the block's TOH x (16 * TCT) pixels
+  uint32_t pix[4], row_q[4], col_q[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const uint32_t t = wave * 4u + q;
+    row_q[q] = t >> P.log2_TCT;  // rows >= TOH (a block cut down to fit LDS) compute row 0 again and store nothing
+    col_q[q] = ((t & (P.TCT - 1u)) << 4) + l16;
+    pix[q] = (row_q[q] < P.TOH ? row_q[q] : 0u) * P.si_r * P.PCP + col_q[q] * P.si_c + g * P.PP;
+  }
+  floatx4 acc[4][4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[q][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int32_t in_r0 = (int32_t)(bi * P.TOH * P.si_r) + S.min_r;
+  const int32_t in_c0 = (int32_t)(bj * (P.TCT << 4) * P.si_c) + S.min_c;
+  const uint32_t patch_elems = P.CC * S.PR * S.PC;
+  const uint32_t cq_per_tap = P.CC >> 2, log2_cq = P.CC == 8u ? 1u : 0u;
+
+  if (S.t1 > S.t0) {
+    for (uint32_t ch = 0; ch < P.nchunks; ++ch) {
+      for (uint32_t tg0 = S.t0; tg0 < S.t1; tg0 += P.TG) {
+        const uint32_t ntg = min(P.TG, S.t1 - tg0);
+        __syncthreads();  // every wave is done with the filter rows (and, at a new chunk, the patch)
+        if (tg0 == S.t0) {
+          for (uint32_t e = tid; e < patch_elems; e += kGenThreads) {
+            uint32_t rc, col, c, r;
+            S.div_PC.divmod(e, rc, col);
+            S.div_PR.divmod(rc, c, r);
+            const int32_t gr = in_r0 + (int32_t)r, gc = in_c0 + (int32_t)col;
+            const uint32_t cg = ch * P.CC + c;
+            float v = 0.f;
+            if (gr >= 0 && gr < (int32_t)P.in_H && gc >= 0 && gc < (int32_t)P.in_W && cg < P.C)
+              v = gen_ld(src, ((size_t)cg * P.in_H + (uint32_t)gr) * P.in_W + (uint32_t)gc);
+            patch[c * P.PP + r * P.PCP + col] = v;
+          }
+        }
+        {
+          const float4 *wsrc = reinterpret_cast<const float4 *>(
+              P.wt + ((size_t)(mg * P.nchunks + ch) * P.ntaps + tg0) * P.CC * 64u);
+          const uint32_t n4 = ntg * P.CC * 16u;
+          for (uint32_t e = tid; e < n4; e += kGenThreads)
+            *reinterpret_cast<float4 *>(wl + (e >> 4) * kGenWPitch + ((e & 15u) << 2)) = wsrc[e];
+        }
+        // lane L keeps the patch offset of tap tg0 + L
+        int32_t delta_vec = 0;
+        if (lane < ntg)
+          delta_vec = ((int32_t)P.off_r[tg0 + lane] - S.min_r) * (int32_t)P.PCP + ((int32_t)P.off_c[tg0 + lane] - S.min_c);
+        __syncthreads();
+
+        const uint32_t steps = ntg << log2_cq;
+        float a_cur[4], b_cur[4], a_nxt[4], b_nxt[4];
+        auto fetch = [&](uint32_t step, float (&a)[4], float (&b)[4]) {
+          const uint32_t t = step >> log2_cq, cq = step & (cq_per_tap - 1u);
+          const int32_t delta = __builtin_amdgcn_readlane(delta_vec, (int)t);
+          const float *wrow = wl + ((t << (log2_cq + 2)) + (cq << 2) + g) * kGenWPitch + l16;
+          const float *prow = patch + (cq << 2) * P.PP + delta;
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt) a[mt] = wrow[mt * 16];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) b[q] = prow[pix[q]];
+        };
+        fetch(0, a_cur, b_cur);
+        for (uint32_t step = 0; step < steps; ++step) {
+          if (step + 1u < steps) fetch(step + 1u, a_nxt, b_nxt);
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt)
+              acc[q][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[mt], b_cur[q], acc[q][mt], 0, 0, 0);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            a_cur[k] = a_nxt[k];
+            b_cur[k] = b_nxt[k];
+          }
+        }
+      }
+    }
+  }
+
+  // the lane holds D[m = 4g + i][n = l16] of each 16 x 16 tile
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const uint32_t i = bi * P.TOH + row_q[q], j = bj * (P.TCT << 4) + col_q[q];
+    if (row_q[q] >= P.TOH || i >= S.GI || j >= S.GJ) continue;
+    const size_t pix_out = (size_t)(S.o_r + i * P.so_r) * P.out_W + (S.o_c + j * P.so_c);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t m = mg * 64u + mt * 16u + g * 4u + k;
+        if (m >= P.M) continue;
+        const size_t o = (size_t)m * P.out_H * P.out_W + pix_out;
+        float v = acc[q][mt][k];
+        if (P.beta != 0.f) v += gen_ld(dst, o);
+        gen_st(dst, o, v);
+      }
+  }
+}
+
+// ---- host side: tap tables, tiling, launches ----
+
+struct GenPlan {
+  ConvGenParams P;
+  FilterGenParams F;
+  size_t lds_bytes, wt_bytes;
+  uint64_t blocks;
+};
+
+// Fills the tiling fields of `plan` once the sub-problems' taps and grids are set.  Returns an error code.
+static int gen_finish_plan(GenPlan *plan) {
+  ConvGenParams &P = plan->P;
+  uint32_t max_GJ = 0, max_taps = 0;
+  for (uint32_t s = 0; s < P.nsub; ++s) {
+    max_GJ = std::max(max_GJ, P.sub[s].GJ);
+    max_taps = std::max(max_taps, P.sub[s].t1 - P.sub[s].t0);
+  }
+  P.TCT = max_GJ <= 16u ? 1u : max_GJ <= 32u ? 2u : 4u;
+  P.log2_TCT = P.TCT == 1u ? 0u : P.TCT == 2u ? 1u : 2u;
+  P.TOH = 16u / P.TCT;
+  P.CC = P.C >= 8u ? 8u : 4u;
+  P.nchunks = (P.C + P.CC - 1u) / P.CC;
+  P.MG = (P.M + 63u) / 64u;
+  uint32_t max_PR, max_PC, bpi;
+  size_t patch_bytes;
+  for (;;) {
+    max_PR = 1; max_PC = 1; bpi = 0;
+    for (uint32_t s = 0; s < P.nsub; ++s) {
+      GenSub &S = P.sub[s];
+      int32_t lo_r = 0, hi_r = 0, lo_c = 0, hi_c = 0;
+      for (uint32_t t = S.t0; t < S.t1; ++t) {
+        if (t == S.t0) {
+          lo_r = hi_r = P.off_r[t];
+          lo_c = hi_c = P.off_c[t];
+        }
+        lo_r = std::min<int32_t>(lo_r, P.off_r[t]);
+        hi_r = std::max<int32_t>(hi_r, P.off_r[t]);
+        lo_c = std::min<int32_t>(lo_c, P.off_c[t]);
+        hi_c = std::max<int32_t>(hi_c, P.off_c[t]);
+      }
+      S.min_r = lo_r;
+      S.min_c = lo_c;
+      S.PR = (P.TOH - 1u) * P.si_r + (uint32_t)(hi_r - lo_r) + 1u;
+      S.PC = (16u * P.TCT - 1u) * P.si_c + (uint32_t)(hi_c - lo_c) + 1u;
+      S.div_PR = FastDiv(S.PR);
+      S.div_PC = FastDiv(S.PC);
+      max_PR = std::max(max_PR, S.PR);
+      max_PC = std::max(max_PC, S.PC);
+      S.nbj = (S.GJ + 16u * P.TCT - 1u) / (16u * P.TCT);
+      S.blk0 = bpi;
+      bpi += S.nbj * ((S.GI + P.TOH - 1u) / P.TOH);
+    }
+    if (bpi == 0) return ADH_EINVAL;
+    P.PCP = max_PC;
+    // plane pitch: the four channel groups of a read start 16 banks apart
+    uint32_t pp = max_PR * P.PCP;
+    while (pp % 64u != 16u) ++pp;
+    P.PP = pp;
+    patch_bytes = (size_t)P.CC * P.PP * 4u;
+    if (patch_bytes + (size_t)P.CC * kGenWPitch * 4u <= kGenLdsBytes) break;
+    if (P.TOH == 1u) return ADH_EUNIMPL;
+    P.TOH /= 2u;  // fewer rows per block: the n-tiles of the dropped rows idle
+  }
+  P.blocks_per_image = bpi;
+  P.TG = (uint32_t)std::min<size_t>(std::min<uint32_t>(std::max(max_taps, 1u), 64u),
+                                    (kGenLdsBytes - patch_bytes) / ((size_t)P.CC * kGenWPitch * 4u));
+  P.w_lds_floats = P.TG * P.CC * kGenWPitch;
+  plan->lds_bytes = (size_t)P.w_lds_floats * 4u + patch_bytes;
+  plan->wt_bytes = (size_t)P.MG * P.nchunks * P.ntaps * P.CC * 64u * 4u;
+  P.div_bpi = FastDiv(bpi);
+  P.div_MG = FastDiv(P.MG);
+  P.div_N = FastDiv(P.N);
+  FilterGenParams &F = plan->F;
+  F.M = P.M;
+  F.C = P.C;
+  F.MG = P.MG;
+  F.nchunks = P.nchunks;
+  F.CC = P.CC;
+  F.ntaps = P.ntaps;
+  return ADH_OK;
+}
+
+struct GenShape {
+  uint32_t N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, OH, OW;
+};
+
+static int gen_check_shape(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP,
+                           uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, GenShape *g) {
+  if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
+  if (kh == 0 || kw == 0 || sh == 0 || sw == 0 || dh == 0 || dw == 0) return ADH_EINVAL;
+  if ((uint64_t)kh * kw > (uint64_t)kGenMaxTaps) return ADH_EUNIMPL;
+  if ((uint64_t)sh * sw > (uint64_t)kGenMaxSub) return ADH_EUNIMPL;
+  const uint64_t eh = (uint64_t)(kh - 1u) * dh + 1u, ew = (uint64_t)(kw - 1u) * dw + 1u;
+  if (eh > HP || ew > WP || eh > 4096u || ew > 4096u) return ADH_EINVAL;
+  if ((uint64_t)HP * WP >= (1ull << 31) || Cin >= (1u << 24) || Cout >= (1u << 24)) return ADH_EINVAL;
+  *g = GenShape{N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, (uint32_t)((HP - eh) / sh + 1u), (uint32_t)((WP - ew) / sw + 1u)};
+  return ADH_OK;
+}
+
+static int gen_plan_fwd(const GenShape &g, GenPlan *plan) {
+  ConvGenParams &P = plan->P;
+  P.N = g.N; P.C = g.Cin; P.M = g.Cout;
+  P.in_H = g.HP; P.in_W = g.WP; P.out_H = g.OH; P.out_W = g.OW;
+  P.si_r = g.sh; P.si_c = g.sw; P.so_r = 1; P.so_c = 1;
+  P.ntaps = g.kh * g.kw;
+  P.nsub = 1;
+  for (uint32_t a = 0; a < g.kh; ++a)
+    for (uint32_t b = 0; b < g.kw; ++b) {
+      const uint32_t t = a * g.kw + b;
+      P.off_r[t] = (int16_t)(a * g.dh);
+      P.off_c[t] = (int16_t)(b * g.dw);
+      plan->F.tap_index[t] = (uint16_t)t;
+    }
+  GenSub &S = P.sub[0];
+  S.t0 = 0; S.t1 = P.ntaps; S.GI = g.OH; S.GJ = g.OW; S.o_r = 0; S.o_c = 0;
+  plan->F.m_stride = g.Cin * g.kh * g.kw;
+  plan->F.c_stride = g.kh * g.kw;
+  return gen_finish_plan(plan);
+}
+
+static int gen_plan_bwd_data(const GenShape &g, GenPlan *plan) {
+  ConvGenParams &P = plan->P;
+  P.N = g.N; P.C = g.Cout; P.M = g.Cin;
+  P.in_H = g.OH; P.in_W = g.OW; P.out_H = g.HP; P.out_W = g.WP;
+  P.si_r = 1; P.si_c = 1; P.so_r = g.sh; P.so_c = g.sw;
+  P.ntaps = g.kh * g.kw;
+  uint32_t nsub = 0, t = 0;
+  for (uint32_t pr = 0; pr < g.sh && pr < g.HP; ++pr)
+    for (uint32_t pc = 0; pc < g.sw && pc < g.WP; ++pc) {
+      GenSub &S = P.sub[nsub++];
+      S.t0 = t;
+      for (uint32_t a = 0; a < g.kh; ++a)
+        for (uint32_t b = 0; b < g.kw; ++b) {
+          if ((a * g.dh) % g.sh != pr || (b * g.dw) % g.sw != pc) continue;
+          // dy row of padded row h' = pr + sh * i under tap a: (h' - a*dh) / sh = i + (pr - a*dh) / sh
+          P.off_r[t] = (int16_t)(((int32_t)pr - (int32_t)(a * g.dh)) / (int32_t)g.sh);
+          P.off_c[t] = (int16_t)(((int32_t)pc - (int32_t)(b * g.dw)) / (int32_t)g.sw);
+          plan->F.tap_index[t] = (uint16_t)(a * g.kw + b);
+          ++t;
+        }
+      S.t1 = t;
+      S.GI = (g.HP - pr + g.sh - 1u) / g.sh;
+      S.GJ = (g.WP - pc + g.sw - 1u) / g.sw;
+      S.o_r = pr;
+      S.o_c = pc;
+    }
+  P.nsub = nsub;
+  plan->F.m_stride = g.kh * g.kw;
+  plan->F.c_stride = g.Cin * g.kh * g.kw;
+  return gen_finish_plan(plan);
+}
+
+static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *w, void *workspace,
+                      size_t workspace_bytes, hipStream_t st) {
+  ConvGenParams &P = plan->P;
+  if (!workspace) return ADH_ENULL;
+  if (!aligned_to(workspace, 256)) return ADH_EALIGN;
+  if (workspace_bytes < plan->wt_bytes) return ADH_EWORKSPACE;
+  const uint64_t blocks = (uint64_t)num_tiles * P.N * P.MG * P.blocks_per_image;
+  if (blocks == 0) return ADH_OK;
+  if (blocks >= (1ull << 24)) return ADH_EINVAL;
+  plan->F.w = w;
+  plan->F.wt = reinterpret_cast<float *>(workspace);
+  P.wt = plan->F.wt;
+  const uint32_t fblocks = (uint32_t)std::min<size_t>(1024, (plan->wt_bytes / 4u + 255u) / 256u);
+  if (dtype == ADH_F32) {
+    hipLaunchKernelGGL(conv_gen_filter_kernel<float>, dim3(fblocks), dim3(256), 0, st, plan->F);
+    hipLaunchKernelGGL(conv_gen_kernel<float>, dim3((uint32_t)blocks), dim3(kGenThreads), plan->lds_bytes, st, P);
+  } else {
+    hipLaunchKernelGGL(conv_gen_filter_kernel<uint16_t>, dim3(fblocks), dim3(256), 0, st, plan->F);
+    hipLaunchKernelGGL(conv_gen_kernel<uint16_t>, dim3((uint32_t)blocks), dim3(kGenThreads), plan->lds_bytes, st, P);
+  }
+  return launch_status();
+}
+
+}  // namespace adh
+
+using namespace adh;
+
+extern "C" {
+
+size_t adh_conv2d_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                  uint32_t HP, uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw,
+                                  uint32_t dh, uint32_t dw) {
+  GenShape g;
+  if (!dtype_ok(dtype) || gen_check_shape(num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, &g)) return 0;
+  if (N == 0 || Cin == 0 || Cout == 0) return 0;
+  GenPlan plan = {};
+  int e = ADH_EINVAL;
+  if (which == ADH_CONV_FWD) e = gen_plan_fwd(g, &plan);
+  else if (which == ADH_CONV_BWD_DATA) e = gen_plan_bwd_data(g, &plan);
+  if (e) return 0;
+  return (plan.wt_bytes + 255u) & ~(size_t)255u;
+}
+
+int adh_conv2d_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,
+                              uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw,
+                              const void *const *x_pad_tiles, const void *w, void *const *y_tiles, float beta,
+                              void *workspace, size_t workspace_bytes, void *stream) {
+  if (!dtype_ok(dtype)) return ADH_EINVAL;
+  GenShape g;
+  int e = gen_check_shape(num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, &g);
+  if (e) return e;
+  if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
+  if (N == 0 || Cout == 0) return ADH_OK;
+  if (Cin == 0) return ADH_EINVAL;
+  if (!x_pad_tiles || !y_tiles || !w) return ADH_ENULL;
+  GenPlan plan = {};
+  e = gen_plan_fwd(g, &plan);
+  if (e) return e;
+  const size_t es = dtype_size(dtype);
+  if (!aligned_to(w, es)) return ADH_EALIGN;
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!x_pad_tiles[t] || !y_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(x_pad_tiles[t], es) || !aligned_to(y_tiles[t], es)) return ADH_EALIGN;
+    plan.P.in[t] = x_pad_tiles[t];
+    plan.P.out[t] = y_tiles[t];
+  }
+  plan.P.beta = beta;
+  return gen_launch(dtype, &plan, num_tiles, w, workspace, workspace_bytes, as_stream(stream));
+}
+
+int adh_conv2d_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,
+                                   uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh,
+                                   uint32_t dw, const void *w, const void *const *dy_tiles, void *const *dx_pad_tiles,
+                                   float beta, void *workspace, size_t workspace_bytes, void *stream) {
+  if (!dtype_ok(dtype)) return ADH_EINVAL;
+  GenShape g;
+  int e = gen_check_shape(num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, &g);
+  if (e) return e;
+  if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
+  if (N == 0 || Cin == 0) return ADH_OK;
+  if (Cout == 0) return ADH_EINVAL;
+  if (!dy_tiles || !dx_pad_tiles || !w) return ADH_ENULL;
+  GenPlan plan = {};
+  e = gen_plan_bwd_data(g, &plan);
+  if (e) return e;
+  const size_t es = dtype_size(dtype);
+  if (!aligned_to(w, es)) return ADH_EALIGN;
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!dy_tiles[t] || !dx_pad_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(dy_tiles[t], es) || !aligned_to(dx_pad_tiles[t], es)) return ADH_EALIGN;
+    plan.P.in[t] = dy_tiles[t];
+    plan.P.out[t] = dx_pad_tiles[t];
+  }
+  plan.P.beta = beta;
+  return gen_launch(dtype, &plan, num_tiles, w, workspace, workspace_bytes, as_stream(stream));
+}
+
+}  // extern "C"

@@ -171,6 +171,34 @@ int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N,
                                       float *dw, float beta, void *workspace, size_t workspace_bytes,
                                       void *stream);
 
+/* ---- general window / stride / dilation over the halo-padded slab ------------ */
+/* The other consumers of halo-padded input (CudnnConv2DSize with halo_padded_input,
+ * src/op.cc:1354-1410; the 7x7 stem src/zoo.cc:1528-1538, stride-2 3x3 src/zoo.cc:692-697, the
+ * dilated 3x3 of tools/microbench_spatial_conv.cc:25-32) and, with HP x WP the extents of a
+ * packed unpadded tensor, the 1x1 projections (src/zoo.cc:680-690): x_pad is a packed
+ * (N,Cin,HP,WP) tensor convolved with conv pad 0, filter KCRS (Cout,Cin,kh,kw), stride (sh,sw),
+ * dilation (dh,dw); OH = (HP - ((kh-1)*dh + 1)) / sh + 1, likewise OW
+ * (cudnnGetConvolution2dForwardOutputDim, src/op.cc:1512-1523).  kh*kw <= 64, sh*sw <= 16.
+ * fp32 arithmetic on the matrix cores; ADH_BF16 tensors are widened on load and rounded on store.
+ * The workspace (adh_conv2d_workspace_bytes, 256-byte aligned) holds the rewritten filter. */
+size_t adh_conv2d_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,
+                                  uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t kh, uint32_t kw,
+                                  uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw);
+/* cudnnConvolutionForward at src/op.cc:1576-1587:
+ * y[n,co,oh,ow] = beta*y + sum_{ci,a,b} w[co,ci,a,b] * x_pad[n,ci,oh*sh + a*dh, ow*sw + b*dw] */
+int adh_conv2d_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                              uint32_t HP, uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw,
+                              uint32_t dh, uint32_t dw, const void *const *x_pad_tiles, const void *w,
+                              void *const *y_tiles, float beta, void *workspace, size_t workspace_bytes,
+                              void *stream);
+/* cudnnConvolutionBackwardData at src/op.cc:1701-1712: the adjoint of the above, written over the
+ * WHOLE padded tile (padded pixels that no window reads get beta*dx_pad) */
+int adh_conv2d_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                   uint32_t HP, uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh,
+                                   uint32_t sw, uint32_t dh, uint32_t dw, const void *w,
+                                   const void *const *dy_tiles, void *const *dx_pad_tiles, float beta,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- pooling over the halo-padded slab ------------------------------------- */
 /* CudnnPool2DOp with Pool2DShape::halo_padded_input (include/arraydiff/op.hh:2917-2925): the
  * padded tile (N, C, HP, WP) with HP = H + 2*pad_h, WP = W + 2*pad_w is handed to cuDNN as a plain

@@ -194,6 +194,35 @@ def conv_slab_bwd_filter(x_pad, dy, dw, beta=0.0):
                                   _ptr(x_pad), _ptr(dy), ctypes.c_float(beta), _ptr(dw))
 
 
+def conv2d_out_dims(HP, WP, kh, kw, sh, sw, dh, dw):
+    return (HP - ((kh - 1) * dh + 1)) // sh + 1, (WP - ((kw - 1) * dw + 1)) // sw + 1
+
+
+def conv2d_slab_fwd(x_pad, wt, sh, sw, dh, dw, y, beta=0.0):
+    """General slab conv: x_pad (N,Cin,HP,WP), wt (Cout,Cin,kh,kw), pad 0, stride (sh,sw), dilation (dh,dw)."""
+    N, Cin, HP, WP = x_pad.shape
+    Cout, _, kh, kw = wt.shape
+    assert y.shape == (N, Cout) + conv2d_out_dims(HP, WP, kh, kw, sh, sw, dh, dw)
+    _lib.orc_conv2d_slab_fwd(_u32(N), _u32(Cin), _u32(Cout), _u32(HP), _u32(WP), _u32(kh), _u32(kw), _u32(sh), _u32(sw),
+                             _u32(dh), _u32(dw), _ptr(x_pad), _ptr(wt), ctypes.c_float(beta), _ptr(y))
+
+
+def conv2d_slab_bwd_data(wt, dy, sh, sw, dh, dw, dx_pad, beta=0.0):
+    N, Cin, HP, WP = dx_pad.shape
+    Cout, _, kh, kw = wt.shape
+    assert dy.shape == (N, Cout) + conv2d_out_dims(HP, WP, kh, kw, sh, sw, dh, dw)
+    _lib.orc_conv2d_slab_bwd_data(_u32(N), _u32(Cin), _u32(Cout), _u32(HP), _u32(WP), _u32(kh), _u32(kw), _u32(sh),
+                                  _u32(sw), _u32(dh), _u32(dw), _ptr(wt), _ptr(dy), ctypes.c_float(beta), _ptr(dx_pad))
+
+
+def conv2d_slab_bwd_filter(x_pad, dy, sh, sw, dh, dw, dwt, beta=0.0):
+    N, Cin, HP, WP = x_pad.shape
+    Cout, _, kh, kw = dwt.shape
+    assert dy.shape == (N, Cout) + conv2d_out_dims(HP, WP, kh, kw, sh, sw, dh, dw)
+    _lib.orc_conv2d_slab_bwd_filter(_u32(N), _u32(Cin), _u32(Cout), _u32(HP), _u32(WP), _u32(kh), _u32(kw), _u32(sh),
+                                    _u32(sw), _u32(dh), _u32(dw), _ptr(x_pad), _ptr(dy), ctypes.c_float(beta), _ptr(dwt))
+
+
 def pool_slab_fwd(mode, x_pad, wh, ww, sh, sw, y):
     """x_pad (N, C, HP, WP) float32 -> y (N, C, OH, OW); mode 1 = max, 0 = average."""
     N, C, HP, WP = x_pad.shape

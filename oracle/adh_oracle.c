@@ -25,6 +25,9 @@
  *     conv2d + autograd on the CPU, delta / box / hot-pixel closed forms.
  *   - softmax / nll : pinned against scipy.special.log_softmax and closed
  *     forms (uniform logits, shift invariance, rows sum to one).
+ *   - general conv (any window / stride / dilation) : pinned against torch
+ *     conv2d(stride, dilation) + autograd on the CPU and against the 3x3
+ *     stride-1 functions above.
  *   - pooling over the padded slab : pinned against torch max_pool2d /
  *     avg_pool2d + autograd on the CPU; which element of a window receives the
  *     max gradient when several are equal is cuDNN's choice and is parity
@@ -463,6 +466,82 @@ void orc_conv_slab_fwd_f32(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                 acc += wt[((co * (size_t)Cin + ci) * k + kh) * k + kw] *
                        x_pad[((n * (size_t)Cin + ci) * Hp + h + kh) * Wp + w + kw];
           y[((n * (size_t)Cout + co) * H + h) * W + w] = acc;
+        }
+}
+
+/* ------------------------------------------------------------------ */
+/* general window / stride / dilation over the halo-padded slab          */
+/* ------------------------------------------------------------------ */
+
+/* CudnnConv2DSize with halo_padded_input (src/op.cc:1354-1410): x = packed
+ * (N,Cin,HP,WP) with conv pad 0, stride (sh,sw), dilation (dh,dw), filter KCRS
+ * (Cout,Cin,kh,kw); output extents as cudnnGetConvolution2dForwardOutputDim,
+ * OH = (HP - ((kh-1)*dh + 1)) / sh + 1 (src/op.cc:1512-1523):
+ *   y[n,co,oh,ow] = beta*y + sum wt[co,ci,a,b] * x[n,ci,oh*sh + a*dh, ow*sw + b*dw] */
+void orc_conv2d_slab_fwd(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t kh, uint32_t kw,
+                         uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, const float *x_pad, const float *wt,
+                         float beta, float *y) {
+  const uint32_t OH = (HP - ((kh - 1) * dh + 1)) / sh + 1, OW = (WP - ((kw - 1) * dw + 1)) / sw + 1;
+  for (uint32_t n = 0; n < N; ++n)
+    for (uint32_t co = 0; co < Cout; ++co)
+      for (uint32_t oh = 0; oh < OH; ++oh)
+        for (uint32_t ow = 0; ow < OW; ++ow) {
+          double acc = 0.0;
+          for (uint32_t ci = 0; ci < Cin; ++ci)
+            for (uint32_t a = 0; a < kh; ++a)
+              for (uint32_t b = 0; b < kw; ++b)
+                acc += (double)wt[((co * (size_t)Cin + ci) * kh + a) * kw + b] *
+                       (double)x_pad[((n * (size_t)Cin + ci) * HP + oh * sh + a * dh) * WP + ow * sw + b * dw];
+          size_t yi = ((n * (size_t)Cout + co) * OH + oh) * OW + ow;
+          y[yi] = (float)(acc + (beta != 0.0f ? (double)beta * y[yi] : 0.0));
+        }
+}
+
+/* cudnnConvolutionBackwardData (src/op.cc:1701-1712) for the same descriptors, as the adjoint of
+ * the forward map written as a scatter: every (output pixel, tap) adds wt*dy onto the padded pixel
+ * it read.  Padded pixels that no window reads get beta*dx. */
+void orc_conv2d_slab_bwd_data(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t kh,
+                              uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, const float *wt,
+                              const float *dy, float beta, float *dx_pad) {
+  const uint32_t OH = (HP - ((kh - 1) * dh + 1)) / sh + 1, OW = (WP - ((kw - 1) * dw + 1)) / sw + 1;
+  const size_t plane = (size_t)HP * WP;
+  double *g = (double *)malloc(plane * sizeof(double));
+  for (uint32_t n = 0; n < N; ++n)
+    for (uint32_t ci = 0; ci < Cin; ++ci) {
+      for (size_t i = 0; i < plane; ++i) g[i] = 0.0;
+      for (uint32_t co = 0; co < Cout; ++co)
+        for (uint32_t oh = 0; oh < OH; ++oh)
+          for (uint32_t ow = 0; ow < OW; ++ow) {
+            const double d = dy[((n * (size_t)Cout + co) * OH + oh) * OW + ow];
+            for (uint32_t a = 0; a < kh; ++a)
+              for (uint32_t b = 0; b < kw; ++b)
+                g[(size_t)(oh * sh + a * dh) * WP + ow * sw + b * dw] +=
+                    (double)wt[((co * (size_t)Cin + ci) * kh + a) * kw + b] * d;
+          }
+      float *dxp = dx_pad + (n * (size_t)Cin + ci) * plane;
+      for (size_t i = 0; i < plane; ++i) dxp[i] = (float)(g[i] + (beta != 0.0f ? (double)beta * dxp[i] : 0.0));
+    }
+  free(g);
+}
+
+/* cudnnConvolutionBackwardFilter (src/op.cc:1660-1671) for the same descriptors:
+ *   dw[co,ci,a,b] = beta*dw + sum_{n,oh,ow} dy[n,co,oh,ow] * x[n,ci,oh*sh + a*dh, ow*sw + b*dw] */
+void orc_conv2d_slab_bwd_filter(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t kh,
+                                uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, const float *x_pad,
+                                const float *dy, float beta, float *dwt) {
+  const uint32_t OH = (HP - ((kh - 1) * dh + 1)) / sh + 1, OW = (WP - ((kw - 1) * dw + 1)) / sw + 1;
+  for (uint32_t co = 0; co < Cout; ++co)
+    for (uint32_t ci = 0; ci < Cin; ++ci)
+      for (uint32_t a = 0; a < kh; ++a)
+        for (uint32_t b = 0; b < kw; ++b) {
+          double acc = 0.0;
+          for (uint32_t n = 0; n < N; ++n)
+            for (uint32_t oh = 0; oh < OH; ++oh)
+              for (uint32_t ow = 0; ow < OW; ++ow)
+                acc += (double)dy[((n * (size_t)Cout + co) * OH + oh) * OW + ow] *
+                       (double)x_pad[((n * (size_t)Cin + ci) * HP + oh * sh + a * dh) * WP + ow * sw + b * dw];
+          size_t wi = ((co * (size_t)Cin + ci) * kh + a) * kw + b;
+          dwt[wi] = (float)(acc + (beta != 0.0f ? (double)beta * dwt[wi] : 0.0));
         }
 }
 

@@ -176,3 +176,44 @@ def test_softmax_vs_scipy_and_closed_forms(oracle):
     tl = F.cross_entropy(tx, torch.tensor(label.astype(np.int64)), reduction="mean")
     tl.backward()
     np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-5, atol=1e-9)
+
+
+GENERAL = [  # N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw
+    (2, 3, 4, 13, 15, 7, 7, 2, 2, 1, 1), (1, 4, 3, 9, 10, 3, 3, 2, 2, 1, 1), (1, 2, 2, 11, 12, 3, 3, 1, 1, 3, 3),
+    (2, 5, 3, 6, 7, 1, 1, 2, 2, 1, 1), (1, 2, 3, 10, 9, 3, 2, 2, 1, 2, 1), (1, 1, 1, 8, 8, 2, 2, 3, 3, 1, 1),
+    (1, 3, 2, 7, 9, 3, 3, 1, 1, 1, 1)]
+
+
+@pytest.mark.parametrize("N,Cin,Cout,HP,WP,kh,kw,sh,sw,dh,dw", GENERAL)
+def test_general_conv_vs_torch(oracle, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw):
+    rng = np.random.default_rng(20 + HP)
+    xp = rnd(rng, N, Cin, HP, WP)
+    wt = rnd(rng, Cout, Cin, kh, kw)
+    tx = torch.tensor(xp, dtype=torch.float64, requires_grad=True)
+    tw = torch.tensor(wt, dtype=torch.float64, requires_grad=True)
+    ty = F.conv2d(tx, tw, stride=(sh, sw), dilation=(dh, dw))
+    assert tuple(ty.shape[2:]) == oracle.conv2d_out_dims(HP, WP, kh, kw, sh, sw, dh, dw)
+    dy = rng.standard_normal(tuple(ty.shape)).astype(np.float32)
+    ty.backward(torch.tensor(dy, dtype=torch.float64))
+    y = np.full(tuple(ty.shape), np.nan, np.float32)
+    oracle.conv2d_slab_fwd(xp, wt, sh, sw, dh, dw, y)
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=0, atol=4e-6)
+    dx = np.full_like(xp, np.nan)
+    oracle.conv2d_slab_bwd_data(wt, dy, sh, sw, dh, dw, dx)
+    np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=0, atol=8e-6)
+    dwt = np.full_like(wt, np.nan)
+    oracle.conv2d_slab_bwd_filter(xp, dy, sh, sw, dh, dw, dwt)
+    np.testing.assert_allclose(dwt, tw.grad.numpy(), rtol=1e-6, atol=2e-5)
+    # beta = 1 accumulates
+    for fn, out, args in ((oracle.conv2d_slab_fwd, y, (xp, wt)), (oracle.conv2d_slab_bwd_data, dx, (wt, dy)),
+                          (oracle.conv2d_slab_bwd_filter, dwt, (xp, dy))):
+        twice = out.copy()
+        fn(*args, sh, sw, dh, dw, twice, beta=1.0)
+        np.testing.assert_allclose(twice, 2 * out, rtol=1e-6, atol=1e-6)
+    if (kh, kw, sh, sw, dh, dw) == (3, 3, 1, 1, 1, 1):  # the 3x3 stride-1 functions are the same map
+        y3 = np.empty_like(y)
+        oracle.conv_slab_fwd(xp, wt, y3)
+        assert np.array_equal(y3, y)
+        dx3 = np.empty_like(dx)
+        oracle.conv_slab_bwd_data(wt, dy, dx3)
+        np.testing.assert_allclose(dx3, dx, rtol=0, atol=1e-6)
