@@ -50,6 +50,7 @@ SIGNATURES = {
     "adh_conv2d_workspace_bytes": (sz, [i32, i32] + [u32] * 12),
     "adh_conv2d_slab_fwd_tiles": (i32, [i32] + [u32] * 12 + [vpp, vp, vpp, f32, vp, sz, vp]),
     "adh_conv2d_slab_bwd_data_tiles": (i32, [i32] + [u32] * 12 + [vp, vpp, vpp, f32, vp, sz, vp]),
+    "adh_conv2d_slab_bwd_filter_tiles": (i32, [i32] + [u32] * 12 + [vpp, vpp, vp, f32, vp, sz, vp]),
     "adh_pool2d_slab_fwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp]),
     "adh_pool2d_slab_fwd": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, vp, vp, vp]),
     "adh_pool2d_slab_bwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vpp, vpp, vpp, f32, vp]),
@@ -254,6 +255,15 @@ def conv2d_bwd_data_tiles(w, dys, dxs, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh,
     wp, wb = _ws(ws)
     return lib().adh_conv2d_slab_bwd_data_tiles(_dt(dys[0]), len(dys), N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw,
                                                 w.data_ptr(), dt, gt, beta, wp, wb, _stream())
+
+
+def conv2d_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw_, beta=0.0, ws=None):
+    _dev(*xs, *dys, dw)
+    xt, k1 = _tbl(xs)
+    dt, k2 = _tbl(dys)
+    wp, wb = _ws(ws)
+    return lib().adh_conv2d_slab_bwd_filter_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw_,
+                                                  xt, dt, dw.data_ptr(), beta, wp, wb, _stream())
 
 
 def pool_fwd_tiles(mode, xs, ys, N, C, HP, WP, wh, ww, sh, sw):

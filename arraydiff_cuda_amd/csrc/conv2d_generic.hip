@@ -390,6 +390,215 @@ static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *
 
 }  // namespace adh
 
+// ---------------------------------------------------------------------------------------------
+// backward-filter for any window / stride / dilation
+//   dw[co][ci][a][b] = beta*dw + sum over tiles, n, oh, ow of dy[n][co][oh][ow] * x[n][ci][oh*sh + a*dh][ow*sw + b*dw]
+// GEMM per tap: M = 64 output channels, N = 16 input channels, K = output pixels, four consecutive
+// pixels of a row per v_mfma_f32_16x16x4_f32.  A block owns (64 co, 16 ci, a group of T <= 9 taps)
+// and every PS-th unit of pixels (R output rows x OWT columns of one image); per unit it stages the dy
+// tile and the input patch in LDS, and its four waves split the unit's pixel groups, each keeping all
+// T x 4 accumulator tiles.  Every wave writes its sums in register order to the workspace; a second
+// kernel adds the 4 * PS partial sums in a fixed order (deterministic) and scatters them to KCRS.
+// ---------------------------------------------------------------------------------------------
+namespace adh {
+
+constexpr uint32_t kWgGenThreads = 256;
+
+struct WgradGenParams {
+  const void *x[ADH_MAX_TILES];
+  const void *dy[ADH_MAX_TILES];
+  float *partial;
+  uint32_t N, Cin, Cout, HP, WP, OH, OW, sh, sw;
+  uint32_t T, ntg, ntaps, COG, CIT;
+  uint32_t R, OWT, nrb, ncb, units, PS;
+  uint32_t PR, PC, PCP, PP, DP, dy_lds_floats;
+  FastDiv div_COG, div_CIT, div_ntg, div_ncb, div_nrb, div_N, div_OWT, div_PC, div_PR;
+  int16_t off_r[kGenMaxTaps], off_c[kGenMaxTaps];
+};
+
+template <typename T, int TAPS>
+__global__ __launch_bounds__(kWgGenThreads) void conv_gen_wgrad_kernel(const WgradGenParams P) {
+  extern __shared__ __align__(16) float gen_lds[];
+  float *dyl = gen_lds;
+  float *patch = gen_lds + P.dy_lds_floats;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+  uint32_t rest, rest2, cog, cit, tg, ps;
+  P.div_COG.divmod(blockIdx.x, rest, cog);
+  P.div_CIT.divmod(rest, rest2, cit);
+  P.div_ntg.divmod(rest2, ps, tg);
+
+  // lane L keeps the patch offset of tap tg * TAPS + L (absent taps of the last group read tap 0's place)
+  int32_t delta_vec = 0;
+  {
+    const uint32_t t = tg * TAPS + lane;
+    if (lane < (uint32_t)TAPS && t < P.ntaps) delta_vec = (int32_t)P.off_r[t] * (int32_t)P.PCP + (int32_t)P.off_c[t];
+  }
+  floatx4 acc[TAPS][4];
+#pragma unroll
+  for (int t = 0; t < TAPS; ++t)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const uint32_t unit_pix = P.R * P.OWT, ksteps = unit_pix >> 2;
+  const uint32_t patch_elems = 16u * P.PR * P.PC, dy_elems = 64u * unit_pix;
+  for (uint32_t u = ps; u < P.units; u += P.PS) {
+    uint32_t r2, r3, cb, rb, n, tile;
+    P.div_ncb.divmod(u, r2, cb);
+    P.div_nrb.divmod(r2, r3, rb);
+    P.div_N.divmod(r3, tile, n);
+    const T *xs = reinterpret_cast<const T *>(P.x[tile]) + ((size_t)n * P.Cin + cit * 16u) * P.HP * P.WP;
+    const T *ds = reinterpret_cast<const T *>(P.dy[tile]) + ((size_t)n * P.Cout + cog * 64u) * P.OH * P.OW;
+    const uint32_t oh0 = rb * P.R, ow0 = cb * P.OWT;
+    __syncthreads();  // every wave is done with the previous unit
+    for (uint32_t e = tid; e < dy_elems; e += kWgGenThreads) {
+      uint32_t co, pr, r, c;
+      co = e / unit_pix;
+      pr = e - co * unit_pix;
+      P.div_OWT.divmod(pr, r, c);
+      float v = 0.f;
+      if (cog * 64u + co < P.Cout && oh0 + r < P.OH && ow0 + c < P.OW)
+        v = gen_ld(ds, ((size_t)co * P.OH + oh0 + r) * P.OW + ow0 + c);
+      dyl[co * P.DP + pr] = v;
+    }
+    for (uint32_t e = tid; e < patch_elems; e += kWgGenThreads) {
+      uint32_t rc, col, c, r;
+      P.div_PC.divmod(e, rc, col);
+      P.div_PR.divmod(rc, c, r);
+      const uint32_t gr = oh0 * P.sh + r, gc = ow0 * P.sw + col;
+      float v = 0.f;
+      if (cit * 16u + c < P.Cin && gr < P.HP && gc < P.WP) v = gen_ld(xs, ((size_t)c * P.HP + gr) * P.WP + gc);
+      patch[c * P.PP + r * P.PCP + col] = v;
+    }
+    __syncthreads();
+    for (uint32_t ks = wave; ks < ksteps; ks += 4u) {
+      const uint32_t p0 = (ks << 2) + g;
+      uint32_t r, c;
+      P.div_OWT.divmod(p0, r, c);
+      const float *arow = dyl + l16 * P.DP + p0;
+      const float *brow = patch + l16 * P.PP + r * P.sh * P.PCP + c * P.sw;
+      float a[4], b[TAPS];
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) a[mt] = arow[mt * 16 * P.DP];
+#pragma unroll
+      for (int t = 0; t < TAPS; ++t) b[t] = brow[__builtin_amdgcn_readlane(delta_vec, t)];
+#pragma unroll
+      for (int t = 0; t < TAPS; ++t)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[mt], b[t], acc[t][mt], 0, 0, 0);
+    }
+  }
+  // partial[(ps * 4 + wave)][cog][cit][tg][t][mt][lane][4]
+  const size_t block_part = ((size_t)(cog * P.CIT + cit) * P.ntg + tg) * TAPS * 1024u;
+  const size_t stride = (size_t)P.COG * P.CIT * P.ntg * TAPS * 1024u;
+  float *dstp = P.partial + (size_t)(ps * 4u + wave) * stride + block_part;
+#pragma unroll
+  for (int t = 0; t < TAPS; ++t)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+      *reinterpret_cast<floatx4 *>(dstp + (t * 4 + mt) * 256 + lane * 4u) = acc[t][mt];
+}
+
+struct WgradGenReduceParams {
+  const float *partial;
+  float *dw;
+  uint32_t Cin, Cout, ntaps, T, ntg, COG, CIT, nparts;
+  float beta;
+};
+
+__global__ __launch_bounds__(256) void conv_gen_wgrad_reduce_kernel(const WgradGenReduceParams Q) {
+  const size_t stride = (size_t)Q.COG * Q.CIT * Q.ntg * Q.T * 1024u;
+  for (size_t e = (size_t)blockIdx.x * 256u + threadIdx.x; e < stride; e += (size_t)gridDim.x * 256u) {
+    const uint32_t i = (uint32_t)(e & 3u), lane = (uint32_t)((e >> 2) & 63u), mt = (uint32_t)((e >> 8) & 3u);
+    size_t r = e >> 10;
+    const uint32_t t = (uint32_t)(r % Q.T);
+    r /= Q.T;
+    const uint32_t tg = (uint32_t)(r % Q.ntg);
+    r /= Q.ntg;
+    const uint32_t cit = (uint32_t)(r % Q.CIT), cog = (uint32_t)(r / Q.CIT);
+    const uint32_t co = cog * 64u + mt * 16u + (lane >> 4) * 4u + i, ci = cit * 16u + (lane & 15u), tap = tg * Q.T + t;
+    if (co >= Q.Cout || ci >= Q.Cin || tap >= Q.ntaps) continue;
+    float sum = 0.f;
+    for (uint32_t p = 0; p < Q.nparts; ++p) sum += Q.partial[(size_t)p * stride + e];
+    float *out = Q.dw + ((size_t)co * Q.Cin + ci) * Q.ntaps + tap;
+    *out = Q.beta != 0.f ? *out + sum : sum;
+  }
+}
+
+struct WgradGenPlan {
+  WgradGenParams P;
+  size_t lds_bytes, partial_bytes;
+  uint32_t blocks, nparts;
+};
+
+static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *plan) {
+  WgradGenParams &P = plan->P;
+  P.N = g.N; P.Cin = g.Cin; P.Cout = g.Cout; P.HP = g.HP; P.WP = g.WP; P.OH = g.OH; P.OW = g.OW;
+  P.sh = g.sh; P.sw = g.sw;
+  P.ntaps = g.kh * g.kw;
+  P.T = P.ntaps == 1u ? 1u : P.ntaps <= 4u ? 4u : 9u;
+  P.ntg = (P.ntaps + P.T - 1u) / P.T;
+  for (uint32_t a = 0; a < g.kh; ++a)
+    for (uint32_t b = 0; b < g.kw; ++b) {
+      P.off_r[a * g.kw + b] = (int16_t)(a * g.dh);
+      P.off_c[a * g.kw + b] = (int16_t)(b * g.dw);
+    }
+  P.COG = (g.Cout + 63u) / 64u;
+  P.CIT = (g.Cin + 15u) / 16u;
+  P.OWT = std::min<uint32_t>((g.OW + 3u) & ~3u, 64u);
+  P.R = std::max<uint32_t>(1u, std::min<uint32_t>(g.OH, 64u / P.OWT));
+  const uint32_t span_r = (g.kh - 1u) * g.dh + 1u, span_c = (g.kw - 1u) * g.dw + 1u;
+  for (;;) {
+    P.PR = (P.R - 1u) * g.sh + span_r;
+    P.PC = (P.OWT - 1u) * g.sw + span_c;
+    P.PCP = P.PC;
+    uint32_t pp = P.PR * P.PCP;
+    while (pp % 64u != 4u * std::min<uint32_t>(g.sw, 4u) % 64u) ++pp;  // 16 channels x 4 pixels on distinct banks
+    P.PP = pp;
+    uint32_t dp = P.R * P.OWT;
+    while (dp % 64u != 4u) ++dp;
+    P.DP = dp;
+    P.dy_lds_floats = 64u * P.DP;
+    plan->lds_bytes = ((size_t)P.dy_lds_floats + 16u * (size_t)P.PP) * 4u;
+    if (plan->lds_bytes <= kGenLdsBytes) break;
+    if (P.R > 1u) P.R /= 2u;
+    else if (P.OWT > 4u) P.OWT = ((P.OWT / 2u) + 3u) & ~3u;
+    else return ADH_EUNIMPL;
+  }
+  P.nrb = (g.OH + P.R - 1u) / P.R;
+  P.ncb = (g.OW + P.OWT - 1u) / P.OWT;
+  const uint64_t units = (uint64_t)num_tiles * g.N * P.nrb * P.ncb;
+  if (units == 0 || units >= (1ull << 31)) return ADH_EINVAL;
+  P.units = (uint32_t)units;
+  const uint64_t fixed = (uint64_t)P.COG * P.CIT * P.ntg;
+  const size_t stride_bytes = (size_t)fixed * P.T * 1024u * 4u;
+  uint64_t ps = std::max<uint64_t>(1u, 1024u / fixed);
+  ps = std::min<uint64_t>(ps, units);
+  while (ps > 1u && ps * 4u * stride_bytes > (256ull << 20)) ps /= 2u;
+  if (fixed * ps >= (1ull << 24)) return ADH_EINVAL;
+  P.PS = (uint32_t)ps;
+  plan->nparts = P.PS * 4u;
+  plan->blocks = (uint32_t)(fixed * ps);
+  plan->partial_bytes = (size_t)plan->nparts * stride_bytes;
+  P.div_COG = FastDiv(P.COG); P.div_CIT = FastDiv(P.CIT); P.div_ntg = FastDiv(P.ntg);
+  P.div_ncb = FastDiv(P.ncb); P.div_nrb = FastDiv(P.nrb); P.div_N = FastDiv(g.N);
+  P.div_OWT = FastDiv(P.OWT); P.div_PC = FastDiv(P.PC); P.div_PR = FastDiv(P.PR);
+  return ADH_OK;
+}
+
+template <typename T>
+static void launch_wgrad_gen(const WgradGenPlan &plan, hipStream_t st) {
+  const WgradGenParams &P = plan.P;
+  if (P.T == 1u)
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 1>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+  else if (P.T == 4u)
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 4>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+  else
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 9>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+}
+
+}  // namespace adh
+
 using namespace adh;
 
 extern "C" {
@@ -400,6 +609,11 @@ size_t adh_conv2d_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint
   GenShape g;
   if (!dtype_ok(dtype) || gen_check_shape(num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, &g)) return 0;
   if (N == 0 || Cin == 0 || Cout == 0) return 0;
+  if (which == ADH_CONV_BWD_FILTER) {
+    WgradGenPlan wp = {};
+    if (gen_plan_wgrad(g, num_tiles, &wp)) return 0;
+    return (wp.partial_bytes + 255u) & ~(size_t)255u;
+  }
   GenPlan plan = {};
   int e = ADH_EINVAL;
   if (which == ADH_CONV_FWD) e = gen_plan_fwd(g, &plan);
@@ -460,6 +674,53 @@ int adh_conv2d_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, ui
   }
   plan.P.beta = beta;
   return gen_launch(dtype, &plan, num_tiles, w, workspace, workspace_bytes, as_stream(stream));
+}
+
+
+int adh_conv2d_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,
+                                     uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh,
+                                     uint32_t dw, const void *const *x_pad_tiles, const void *const *dy_tiles,
+                                     float *dwt, float beta, void *workspace, size_t workspace_bytes, void *stream) {
+  if (!dtype_ok(dtype)) return ADH_EINVAL;
+  GenShape g;
+  int e = gen_check_shape(num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, &g);
+  if (e) return e;
+  if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
+  if (Cin == 0 || Cout == 0) return ADH_OK;
+  if (!dwt) return ADH_ENULL;
+  if (!aligned_to(dwt, 4)) return ADH_EALIGN;
+  hipStream_t st = as_stream(stream);
+  if (N == 0) {  // an empty sum
+    if (beta == 0.f) return adh_fill_f32((uint64_t)Cout * Cin * kh * kw, 0.f, dwt, stream);
+    return ADH_OK;
+  }
+  if (!x_pad_tiles || !dy_tiles) return ADH_ENULL;
+  WgradGenPlan plan = {};
+  e = gen_plan_wgrad(g, num_tiles, &plan);
+  if (e) return e;
+  const size_t es = dtype_size(dtype);
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!x_pad_tiles[t] || !dy_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(x_pad_tiles[t], es) || !aligned_to(dy_tiles[t], es)) return ADH_EALIGN;
+    plan.P.x[t] = x_pad_tiles[t];
+    plan.P.dy[t] = dy_tiles[t];
+  }
+  if (!workspace) return ADH_ENULL;
+  if (!aligned_to(workspace, 256)) return ADH_EALIGN;
+  if (workspace_bytes < plan.partial_bytes) return ADH_EWORKSPACE;
+  plan.P.partial = reinterpret_cast<float *>(workspace);
+  if (dtype == ADH_F32) launch_wgrad_gen<float>(plan, st);
+  else launch_wgrad_gen<uint16_t>(plan, st);
+  WgradGenReduceParams Q;
+  Q.partial = plan.P.partial;
+  Q.dw = dwt;
+  Q.Cin = Cin; Q.Cout = Cout; Q.ntaps = plan.P.ntaps; Q.T = plan.P.T; Q.ntg = plan.P.ntg;
+  Q.COG = plan.P.COG; Q.CIT = plan.P.CIT; Q.nparts = plan.nparts;
+  Q.beta = beta;
+  const size_t stride = (size_t)Q.COG * Q.CIT * Q.ntg * Q.T * 1024u;
+  hipLaunchKernelGGL(conv_gen_wgrad_reduce_kernel, dim3((uint32_t)std::min<size_t>((stride + 255u) / 256u, 65535u)),
+                     dim3(256), 0, st, Q);
+  return launch_status();
 }
 
 }  // extern "C"

@@ -199,6 +199,15 @@ int adh_conv2d_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, ui
                                    const void *const *dy_tiles, void *const *dx_pad_tiles, float beta,
                                    void *workspace, size_t workspace_bytes, void *stream);
 
+/* cudnnConvolutionBackwardFilter at src/op.cc:1660-1671 for the same descriptors:
+ * dw[co,ci,a,b] = beta*dw + sum_{tiles,n,oh,ow} dy[n,co,oh,ow] * x_pad[n,ci,oh*sh + a*dh, ow*sw + b*dw];
+ * dw is always fp32; the workspace holds partial sums that are added in a fixed order. */
+int adh_conv2d_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                     uint32_t HP, uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh,
+                                     uint32_t sw, uint32_t dh, uint32_t dw, const void *const *x_pad_tiles,
+                                     const void *const *dy_tiles, float *dwt, float beta, void *workspace,
+                                     size_t workspace_bytes, void *stream);
+
 /* ---- pooling over the halo-padded slab ------------------------------------- */
 /* CudnnPool2DOp with Pool2DShape::halo_padded_input (include/arraydiff/op.hh:2917-2925): the
  * padded tile (N, C, HP, WP) with HP = H + 2*pad_h, WP = W + 2*pad_w is handed to cuDNN as a plain

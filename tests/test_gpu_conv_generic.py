@@ -72,7 +72,18 @@ def test_general_conv_f32_vs_oracle(oracle, K, N, Cin, Cout, HP, WP, kh, kw, sh,
         g1 = g0[r].copy()
         oracle.conv2d_slab_bwd_data(w, dys[r], sh, sw, dh, dw, g1, beta=1.0)
         assert rel_err(host(ga[r]), g1) <= TOL
+    # filter gradient summed over the tiles, beta = 0 then beta = 1
+    ws_w = ws_for(capi.ADH_CONV_BWD_FILTER, capi.ADH_F32, K, N, Cin, Cout, HP, WP, *geo)
+    gw = torch.full((Cout, Cin, kh, kw), float("nan"), device="cuda")
+    capi.check(capi.conv2d_bwd_filter_tiles(d_xs, d_dys, gw, N, Cin, Cout, HP, WP, *geo, ws=ws_w))
+    dw_want = np.zeros((Cout, Cin, kh, kw), np.float32)
+    for r in range(K):
+        oracle.conv2d_slab_bwd_filter(xs[r], dys[r], sh, sw, dh, dw, dw_want, beta=1.0)
+    assert rel_err(host(gw), dw_want) <= TOL
+    capi.check(capi.conv2d_bwd_filter_tiles(d_xs, d_dys, gw, N, Cin, Cout, HP, WP, *geo, beta=1.0, ws=ws_w))
+    assert rel_err(host(gw), 2 * dw_want) <= TOL
     small = torch.empty(8, device="cuda")
+    assert capi.conv2d_bwd_filter_tiles(d_xs, d_dys, gw, N, Cin, Cout, HP, WP, *geo, ws=small) == capi.ADH_EWORKSPACE
     assert capi.conv2d_fwd_tiles(d_xs, d_w, ys, N, Cin, Cout, HP, WP, *geo, ws=small) == capi.ADH_EWORKSPACE
     assert capi.conv2d_fwd_tiles(d_xs, d_w, ys, N, Cin, Cout, HP, WP, *geo) == capi.ADH_ENULL
 
@@ -101,6 +112,13 @@ def test_general_conv_bf16_vs_oracle(oracle, K, N, Cin, Cout, HP, WP, kh, kw, sh
         g = np.empty((N, Cin, HP, WP), np.float32)
         oracle.conv2d_slab_bwd_data(wf, oracle.bf16_to_f32(dys[r]), sh, sw, dh, dw, g)
         assert rel_err(oracle.bf16_to_f32(host(gs[r])), g) <= 5e-3
+    gw = torch.empty((Cout, Cin, kh, kw), device="cuda")
+    capi.check(capi.conv2d_bwd_filter_tiles(d_xs, d_dys, gw, N, Cin, Cout, HP, WP, *geo,
+                                            ws=ws_for(capi.ADH_CONV_BWD_FILTER, capi.ADH_BF16, K, N, Cin, Cout, HP, WP, *geo)))
+    dw_want = np.zeros((Cout, Cin, kh, kw), np.float32)
+    for r in range(K):
+        oracle.conv2d_slab_bwd_filter(oracle.bf16_to_f32(xs[r]), oracle.bf16_to_f32(dys[r]), sh, sw, dh, dw, dw_want, beta=1.0)
+    assert rel_err(host(gw), dw_want) <= 1e-4  # fp32 output, exact bf16 products
 
 
 def test_general_conv_stem_stitched_vs_unsplit():
@@ -137,6 +155,14 @@ def test_general_conv_stem_stitched_vs_unsplit():
     for r in range(K):
         total[:, :, r * Ht:r * Ht + Ht + 2 * p] += gs[r]
     assert float((total - xp.grad).abs().max() / xp.grad.abs().max()) <= TOL
+    # filter gradient summed over the tiles == the unsplit one
+    wsw = torch.empty(capi.conv2d_workspace_bytes(capi.ADH_CONV_BWD_FILTER, capi.ADH_F32, K, N, Cin, Cout, Ht + 2 * p,
+                                                  W + 2 * p, *geo) // 4, device="cuda")
+    gw = torch.empty_like(w)
+    capi.check(capi.conv2d_bwd_filter_tiles(tiles, dys, gw, N, Cin, Cout, Ht + 2 * p, W + 2 * p, *geo, ws=wsw))
+    wd = w.double().requires_grad_(True)
+    F.conv2d(xp.detach(), wd, stride=2).backward(dyu.double())
+    assert float((gw - wd.grad).abs().max() / wd.grad.abs().max()) <= TOL
 
 
 def test_general_conv_error_codes():
