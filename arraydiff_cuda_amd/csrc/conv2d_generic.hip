@@ -12,8 +12,8 @@
 //                  each residue class is a stride-1 correlation of dy with the taps that satisfy
 //                  a*dh = h' (mod sh), b*dw = w' (mod sw), offsets (h' - a*dh) / sh: up to sh*sw
 //                  sub-problems in one launch, written with output stride (sh, sw).
-// Implicit GEMM: M = 64 output channels per block, N = 16 x 16 output pixels per block (16 n-tiles
-// of 16 consecutive pixels of a row, 4 per wave), K = (tap, channel) in groups of 4 channels for
+// Implicit GEMM: M = 64 output channels per block, N = 256 output pixels per block (BR rows x BC columns, 16 n-tiles
+// of 16 consecutive pixels in row-major order, 4 per wave), K = (tap, channel) in groups of 4 channels for
 // v_mfma_f32_16x16x4_f32.  Per channel chunk the input patch is staged in LDS once; the filter,
 // rewritten beforehand to [m group][chunk][tap][channel][64 m] in the workspace, is staged per tap
 // group.  bf16 tensors are widened while staging and rounded when stored: the arithmetic is fp32.
@@ -27,7 +27,6 @@ namespace adh {
 constexpr int kGenMaxTaps = 64;
 constexpr int kGenMaxSub = 16;
 constexpr uint32_t kGenThreads = 256;
-constexpr uint32_t kGenWPitch = 80;  // floats per (tap, channel) row of 64 m: 4 channel groups on 4 x 16 banks
 constexpr uint32_t kGenLdsBytes = 64u * 1024u;
 
 struct GenSub {
@@ -36,7 +35,6 @@ struct GenSub {
   int32_t min_r, min_c;       // smallest tap offsets
   uint32_t PR, PC;            // patch rows / columns
   uint32_t nbj, blk0;         // block columns, first block of this sub-problem within an image
-  FastDiv div_PR, div_PC;
 };
 
 struct ConvGenParams {
@@ -46,11 +44,11 @@ struct ConvGenParams {
   uint32_t N, C, M, MG, in_H, in_W, out_H, out_W;
   uint32_t si_r, si_c, so_r, so_c;
   uint32_t CC, nchunks, ntaps, TG;
-  uint32_t TOH, TCT, log2_TCT;
+  uint32_t BR, BC;  // a block's output pixels: BR rows x BC columns, numbered row by row, 16 per n-tile
   uint32_t PCP, PP, w_lds_floats;
   uint32_t nsub, blocks_per_image;
   float beta;
-  FastDiv div_bpi, div_MG, div_N;
+  FastDiv div_bpi, div_MG, div_N, div_PCP, div_BC;
   GenSub sub[kGenMaxSub];
   int16_t off_r[kGenMaxTaps], off_c[kGenMaxTaps];
 };
@@ -58,7 +56,7 @@ struct ConvGenParams {
 struct FilterGenParams {
   const void *w;
   float *wt;
-  uint32_t M, C, m_stride, c_stride, MG, nchunks, CC, ntaps;
+  uint32_t M, C, m_stride, c_stride, MG, MW, nchunks, CC, ntaps;
   uint16_t tap_index[kGenMaxTaps];
 };
 
@@ -69,19 +67,19 @@ __device__ __forceinline__ float gen_ld(const uint16_t *p, size_t i) { return bf
 __device__ __forceinline__ void gen_st(float *p, size_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void gen_st(uint16_t *p, size_t i, float v) { p[i] = f32_to_bf16_bits(v); }
 
-// wt[((mg * nchunks + ch) * ntaps + t) * CC + c][m] = w[(mg*64 + m) * m_stride + (ch*CC + c) * c_stride + tap_index[t]]
+// wt[((mg * nchunks + ch) * ntaps + t) * CC + c][m] = w[(mg*MW + m) * m_stride + (ch*CC + c) * c_stride + tap_index[t]]
 template <typename T>
 __global__ __launch_bounds__(256) void conv_gen_filter_kernel(const FilterGenParams F) {
-  const uint32_t total = F.MG * F.nchunks * F.ntaps * F.CC * 64u;
+  const uint32_t total = F.MG * F.nchunks * F.ntaps * F.CC * F.MW;
   for (uint32_t e = blockIdx.x * 256u + threadIdx.x; e < total; e += gridDim.x * 256u) {
-    const uint32_t m = e & 63u;
-    uint32_t r = e >> 6;
+    const uint32_t m = e % F.MW;
+    uint32_t r = e / F.MW;
     const uint32_t c = r % F.CC;
     r /= F.CC;
     const uint32_t t = r % F.ntaps;
     r /= F.ntaps;
     const uint32_t ch = r % F.nchunks, mg = r / F.nchunks;
-    const uint32_t mm = mg * 64u + m, cc = ch * F.CC + c;
+    const uint32_t mm = mg * F.MW + m, cc = ch * F.CC + c;
     float v = 0.f;
     if (mm < F.M && cc < F.C)
       v = gen_ld(reinterpret_cast<const T *>(F.w), (size_t)mm * F.m_stride + (size_t)cc * F.c_stride + F.tap_index[t]);
@@ -89,8 +87,16 @@ __global__ __launch_bounds__(256) void conv_gen_filter_kernel(const FilterGenPar
   }
 }
 
-template <typename T>
+// CC: channels per chunk (4 or 8); MT: 16-wide m-tiles per block (1, 2 or 4).
+// The next (chunk, tap group)'s patch and filter rows are loaded into registers while the current
+// one is multiplied; they go to LDS after the barrier that ends the current one.
+template <typename T, int CC, int MT>
 __global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenParams P) {
+  constexpr uint32_t MW = 16u * MT;                         // m per block
+  constexpr uint32_t WPITCH = MT == 1 ? 16u : MW + 16u;     // filter row pitch: the 4 channel groups 16 banks apart
+  constexpr int PFC = 32 / CC;                              // prefetch registers per channel plane: PP <= 256 * PFC
+  constexpr int WF = 6;                                     // float4 filter registers: TG * CC * MW / 4 <= 256 * WF
+  constexpr uint32_t LOG2_CQ = CC == 8 ? 1u : 0u;
   extern __shared__ __align__(16) float gen_lds[];
   float *wl = gen_lds;
   float *patch = gen_lds + P.w_lds_floats;
@@ -112,66 +118,113 @@ __global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenPara
   const T *src = reinterpret_cast<const T *>(P.in[tile]) + (size_t)n * P.C * P.in_H * P.in_W;
   T *dst = reinterpret_cast<T *>(P.out[tile]) + (size_t)n * P.M * P.out_H * P.out_W;
 
-  // this wave's four n-tiles: row and column tile within the block's TOH x (16 * TCT) pixels
+  // this wave's four n-tiles: 16 consecutive pixels each of the block's BR x BC pixels numbered row by row;
+  // slots past the last pixel compute pixel 0 again and store nothing
   uint32_t pix[4], row_q[4], col_q[4];
+  bool live_q[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
-    const uint32_t t = wave * 4u + q;
-    row_q[q] = t >> P.log2_TCT;  // rows >= TOH (a block cut down to fit LDS) compute row 0 again and store nothing
-    col_q[q] = ((t & (P.TCT - 1u)) << 4) + l16;
-    pix[q] = (row_q[q] < P.TOH ? row_q[q] : 0u) * P.si_r * P.PCP + col_q[q] * P.si_c + g * P.PP;
+    const uint32_t f = ((wave * 4u + q) << 4) + l16;
+    P.div_BC.divmod(f, row_q[q], col_q[q]);
+    live_q[q] = f < P.BR * P.BC;
+    pix[q] = live_q[q] ? row_q[q] * P.si_r * P.PCP + col_q[q] * P.si_c : 0u;
+    pix[q] += g * P.PP;
   }
-  floatx4 acc[4][4];
+  floatx4 acc[4][MT];
 #pragma unroll
   for (int q = 0; q < 4; ++q)
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) acc[q][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt) acc[q][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const int32_t in_r0 = (int32_t)(bi * P.TOH * P.si_r) + S.min_r;
-  const int32_t in_c0 = (int32_t)(bj * (P.TCT << 4) * P.si_c) + S.min_c;
-  const uint32_t patch_elems = P.CC * S.PR * S.PC;
-  const uint32_t cq_per_tap = P.CC >> 2, log2_cq = P.CC == 8u ? 1u : 0u;
+  // where this thread's PFC elements of a channel plane come from (-1: outside the input or the patch)
+  const int32_t in_r0 = (int32_t)(bi * P.BR * P.si_r) + S.min_r;
+  const int32_t in_c0 = (int32_t)(bj * P.BC * P.si_c) + S.min_c;
+  int32_t src_off[PFC];
+#pragma unroll
+  for (int j = 0; j < PFC; ++j) {
+    const uint32_t e = tid + j * kGenThreads;
+    uint32_t r, col;
+    P.div_PCP.divmod(e, r, col);
+    const int32_t gr = in_r0 + (int32_t)r, gc = in_c0 + (int32_t)col;
+    const bool ok = e < P.PP && r < S.PR && col < S.PC && gr >= 0 && gr < (int32_t)P.in_H && gc >= 0 && gc < (int32_t)P.in_W;
+    src_off[j] = ok ? gr * (int32_t)P.in_W + gc : -1;
+  }
+  const size_t plane = (size_t)P.in_H * P.in_W;
 
-  if (S.t1 > S.t0) {
+  float pre[CC * PFC];
+  float4 wpre[WF];
+  auto load_patch = [&](uint32_t ch) {
+#pragma unroll
+    for (int c = 0; c < CC; ++c) {
+      const uint32_t cg = ch * CC + c;
+      const T *pl = src + (size_t)min(cg, P.C - 1u) * plane;
+#pragma unroll
+      for (int j = 0; j < PFC; ++j)
+        pre[c * PFC + j] = (src_off[j] >= 0 && cg < P.C) ? gen_ld(pl, (size_t)src_off[j]) : 0.f;
+    }
+  };
+  auto store_patch = [&]() {
+#pragma unroll
+    for (int c = 0; c < CC; ++c)
+#pragma unroll
+      for (int j = 0; j < PFC; ++j) {
+        const uint32_t e = tid + j * kGenThreads;
+        if (e < P.PP) patch[c * P.PP + e] = pre[c * PFC + j];
+      }
+  };
+  auto load_filter = [&](uint32_t ch, uint32_t tg0, uint32_t ntg) {
+    const float4 *wsrc =
+        reinterpret_cast<const float4 *>(P.wt + ((size_t)(mg * P.nchunks + ch) * P.ntaps + tg0) * CC * MW);
+    const uint32_t n4 = ntg * CC * (MW / 4u);
+#pragma unroll
+    for (int k = 0; k < WF; ++k) {
+      const uint32_t e = tid + k * kGenThreads;
+      wpre[k] = e < n4 ? wsrc[e] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  };
+  auto store_filter = [&](uint32_t ntg) {
+    const uint32_t n4 = ntg * CC * (MW / 4u);
+#pragma unroll
+    for (int k = 0; k < WF; ++k) {
+      const uint32_t e = tid + k * kGenThreads;
+      if (e < n4) *reinterpret_cast<float4 *>(wl + (e / (MW / 4u)) * WPITCH + (e % (MW / 4u)) * 4u) = wpre[k];
+    }
+  };
+
+  const uint32_t ntaps_s = S.t1 - S.t0;
+  if (ntaps_s > 0) {
+    const uint32_t ngroups = (ntaps_s + P.TG - 1u) / P.TG;
+    load_patch(0);
+    load_filter(0, S.t0, min(P.TG, ntaps_s));
     for (uint32_t ch = 0; ch < P.nchunks; ++ch) {
-      for (uint32_t tg0 = S.t0; tg0 < S.t1; tg0 += P.TG) {
+      for (uint32_t gi = 0; gi < ngroups; ++gi) {
+        const uint32_t tg0 = S.t0 + gi * P.TG;
         const uint32_t ntg = min(P.TG, S.t1 - tg0);
         __syncthreads();  // every wave is done with the filter rows (and, at a new chunk, the patch)
-        if (tg0 == S.t0) {
-          for (uint32_t e = tid; e < patch_elems; e += kGenThreads) {
-            uint32_t rc, col, c, r;
-            S.div_PC.divmod(e, rc, col);
-            S.div_PR.divmod(rc, c, r);
-            const int32_t gr = in_r0 + (int32_t)r, gc = in_c0 + (int32_t)col;
-            const uint32_t cg = ch * P.CC + c;
-            float v = 0.f;
-            if (gr >= 0 && gr < (int32_t)P.in_H && gc >= 0 && gc < (int32_t)P.in_W && cg < P.C)
-              v = gen_ld(src, ((size_t)cg * P.in_H + (uint32_t)gr) * P.in_W + (uint32_t)gc);
-            patch[c * P.PP + r * P.PCP + col] = v;
-          }
-        }
-        {
-          const float4 *wsrc = reinterpret_cast<const float4 *>(
-              P.wt + ((size_t)(mg * P.nchunks + ch) * P.ntaps + tg0) * P.CC * 64u);
-          const uint32_t n4 = ntg * P.CC * 16u;
-          for (uint32_t e = tid; e < n4; e += kGenThreads)
-            *reinterpret_cast<float4 *>(wl + (e >> 4) * kGenWPitch + ((e & 15u) << 2)) = wsrc[e];
-        }
+        if (gi == 0) store_patch();
+        store_filter(ntg);
         // lane L keeps the patch offset of tap tg0 + L
         int32_t delta_vec = 0;
         if (lane < ntg)
           delta_vec = ((int32_t)P.off_r[tg0 + lane] - S.min_r) * (int32_t)P.PCP + ((int32_t)P.off_c[tg0 + lane] - S.min_c);
         __syncthreads();
+        // registers for the next (chunk, tap group) while this one is multiplied
+        if (gi + 1u < ngroups) {
+          load_filter(ch, tg0 + P.TG, min(P.TG, S.t1 - tg0 - P.TG));
+        } else if (ch + 1u < P.nchunks) {
+          load_patch(ch + 1u);
+          load_filter(ch + 1u, S.t0, min(P.TG, ntaps_s));
+        }
 
-        const uint32_t steps = ntg << log2_cq;
-        float a_cur[4], b_cur[4], a_nxt[4], b_nxt[4];
-        auto fetch = [&](uint32_t step, float (&a)[4], float (&b)[4]) {
-          const uint32_t t = step >> log2_cq, cq = step & (cq_per_tap - 1u);
+        const uint32_t steps = ntg << LOG2_CQ;
+        float a_cur[MT], b_cur[4], a_nxt[MT], b_nxt[4];
+        auto fetch = [&](uint32_t step, float (&a)[MT], float (&b)[4]) {
+          const uint32_t t = step >> LOG2_CQ, cq = step & ((CC >> 2) - 1u);
           const int32_t delta = __builtin_amdgcn_readlane(delta_vec, (int)t);
-          const float *wrow = wl + ((t << (log2_cq + 2)) + (cq << 2) + g) * kGenWPitch + l16;
+          const float *wrow = wl + (t * CC + (cq << 2) + g) * WPITCH + l16;
           const float *prow = patch + (cq << 2) * P.PP + delta;
 #pragma unroll
-          for (int mt = 0; mt < 4; ++mt) a[mt] = wrow[mt * 16];
+          for (int mt = 0; mt < MT; ++mt) a[mt] = wrow[mt * 16];
 #pragma unroll
           for (int q = 0; q < 4; ++q) b[q] = prow[pix[q]];
         };
@@ -181,13 +234,12 @@ __global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenPara
 #pragma unroll
           for (int q = 0; q < 4; ++q)
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt)
+            for (int mt = 0; mt < MT; ++mt)
               acc[q][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[mt], b_cur[q], acc[q][mt], 0, 0, 0);
 #pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            a_cur[k] = a_nxt[k];
-            b_cur[k] = b_nxt[k];
-          }
+          for (int k = 0; k < MT; ++k) a_cur[k] = a_nxt[k];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) b_cur[k] = b_nxt[k];
         }
       }
     }
@@ -196,14 +248,14 @@ __global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenPara
   // the lane holds D[m = 4g + i][n = l16] of each 16 x 16 tile
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
-    const uint32_t i = bi * P.TOH + row_q[q], j = bj * (P.TCT << 4) + col_q[q];
-    if (row_q[q] >= P.TOH || i >= S.GI || j >= S.GJ) continue;
+    const uint32_t i = bi * P.BR + row_q[q], j = bj * P.BC + col_q[q];
+    if (!live_q[q] || i >= S.GI || j >= S.GJ) continue;
     const size_t pix_out = (size_t)(S.o_r + i * P.so_r) * P.out_W + (S.o_c + j * P.so_c);
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        const uint32_t m = mg * 64u + mt * 16u + g * 4u + k;
+        const uint32_t m = mg * MW + mt * 16u + g * 4u + k;
         if (m >= P.M) continue;
         const size_t o = (size_t)m * P.out_H * P.out_W + pix_out;
         float v = acc[q][mt][k];
@@ -219,7 +271,7 @@ struct GenPlan {
   ConvGenParams P;
   FilterGenParams F;
   size_t lds_bytes, wt_bytes;
-  uint64_t blocks;
+  uint32_t MT;
 };
 
 // Fills the tiling fields of `plan` once the sub-problems' taps and grids are set.  Returns an error code.
@@ -230,14 +282,25 @@ static int gen_finish_plan(GenPlan *plan) {
     max_GJ = std::max(max_GJ, P.sub[s].GJ);
     max_taps = std::max(max_taps, P.sub[s].t1 - P.sub[s].t0);
   }
-  P.TCT = max_GJ <= 16u ? 1u : max_GJ <= 32u ? 2u : 4u;
-  P.log2_TCT = P.TCT == 1u ? 0u : P.TCT == 2u ? 1u : 2u;
-  P.TOH = 16u / P.TCT;
-  P.CC = P.C >= 8u ? 8u : 4u;
-  P.nchunks = (P.C + P.CC - 1u) / P.CC;
-  P.MG = (P.M + 63u) / 64u;
+  uint32_t max_GI = 0;
+  for (uint32_t s = 0; s < P.nsub; ++s) max_GI = std::max(max_GI, P.sub[s].GI);
+  // block columns: the whole row when it has at most 64 pixels, else the width in [32, 64] that wastes least
+  if (max_GJ <= 64u) {
+    P.BC = std::max(max_GJ, 1u);
+  } else {
+    double best = -1.0;
+    for (uint32_t bc = 64u; bc >= 32u; --bc) {
+      const double used = (double)((256u / bc) * bc) / 256.0 * (double)max_GJ / (double)(((max_GJ + bc - 1u) / bc) * bc);
+      if (used > best + 1e-9) { best = used; P.BC = bc; }
+    }
+  }
+  P.BR = std::max(1u, std::min(256u / P.BC, std::max(max_GI, 1u)));
+  plan->MT = P.M <= 16u ? 1u : P.M <= 32u ? 2u : 4u;
+  const uint32_t MW = 16u * plan->MT, wpitch = plan->MT == 1u ? 16u : MW + 16u;
+  P.MG = (P.M + MW - 1u) / MW;
   uint32_t max_PR, max_PC, bpi;
   size_t patch_bytes;
+  P.CC = P.C >= 8u ? 8u : 4u;
   for (;;) {
     max_PR = 1; max_PC = 1; bpi = 0;
     for (uint32_t s = 0; s < P.nsub; ++s) {
@@ -255,15 +318,13 @@ static int gen_finish_plan(GenPlan *plan) {
       }
       S.min_r = lo_r;
       S.min_c = lo_c;
-      S.PR = (P.TOH - 1u) * P.si_r + (uint32_t)(hi_r - lo_r) + 1u;
-      S.PC = (16u * P.TCT - 1u) * P.si_c + (uint32_t)(hi_c - lo_c) + 1u;
-      S.div_PR = FastDiv(S.PR);
-      S.div_PC = FastDiv(S.PC);
+      S.PR = (P.BR - 1u) * P.si_r + (uint32_t)(hi_r - lo_r) + 1u;
+      S.PC = (P.BC - 1u) * P.si_c + (uint32_t)(hi_c - lo_c) + 1u;
       max_PR = std::max(max_PR, S.PR);
       max_PC = std::max(max_PC, S.PC);
-      S.nbj = (S.GJ + 16u * P.TCT - 1u) / (16u * P.TCT);
+      S.nbj = (S.GJ + P.BC - 1u) / P.BC;
       S.blk0 = bpi;
-      bpi += S.nbj * ((S.GI + P.TOH - 1u) / P.TOH);
+      bpi += S.nbj * ((S.GI + P.BR - 1u) / P.BR);
     }
     if (bpi == 0) return ADH_EINVAL;
     P.PCP = max_PC;
@@ -272,16 +333,27 @@ static int gen_finish_plan(GenPlan *plan) {
     while (pp % 64u != 16u) ++pp;
     P.PP = pp;
     patch_bytes = (size_t)P.CC * P.PP * 4u;
-    if (patch_bytes + (size_t)P.CC * kGenWPitch * 4u <= kGenLdsBytes) break;
-    if (P.TOH == 1u) return ADH_EUNIMPL;
-    P.TOH /= 2u;  // fewer rows per block: the n-tiles of the dropped rows idle
+    // a thread prefetches 32 / CC elements of each channel plane
+    if (P.PP <= 256u * (32u / P.CC) && patch_bytes + (size_t)P.CC * wpitch * 4u <= kGenLdsBytes) break;
+    if (P.CC == 8u) {
+      P.CC = 4u;  // half the channels per chunk: twice the room per plane
+      continue;
+    }
+    if (P.BR == 1u) return ADH_EUNIMPL;
+    P.BR -= 1u;  // fewer rows per block: the n-tiles of the dropped rows idle
+    P.CC = P.C >= 8u ? 8u : 4u;
   }
+  P.nchunks = (P.C + P.CC - 1u) / P.CC;
   P.blocks_per_image = bpi;
+  // taps per group: what fits LDS, a lane per tap, and six float4 prefetch registers per thread
   P.TG = (uint32_t)std::min<size_t>(std::min<uint32_t>(std::max(max_taps, 1u), 64u),
-                                    (kGenLdsBytes - patch_bytes) / ((size_t)P.CC * kGenWPitch * 4u));
-  P.w_lds_floats = P.TG * P.CC * kGenWPitch;
+                                    (kGenLdsBytes - patch_bytes) / ((size_t)P.CC * wpitch * 4u));
+  P.TG = std::min<uint32_t>(P.TG, 256u * 6u / (P.CC * MW / 4u));
+  P.w_lds_floats = P.TG * P.CC * wpitch;
+  P.div_PCP = FastDiv(P.PCP);
+  P.div_BC = FastDiv(P.BC);
   plan->lds_bytes = (size_t)P.w_lds_floats * 4u + patch_bytes;
-  plan->wt_bytes = (size_t)P.MG * P.nchunks * P.ntaps * P.CC * 64u * 4u;
+  plan->wt_bytes = (size_t)P.MG * P.nchunks * P.ntaps * P.CC * MW * 4u;
   P.div_bpi = FastDiv(bpi);
   P.div_MG = FastDiv(P.MG);
   P.div_N = FastDiv(P.N);
@@ -289,6 +361,7 @@ static int gen_finish_plan(GenPlan *plan) {
   F.M = P.M;
   F.C = P.C;
   F.MG = P.MG;
+  F.MW = MW;
   F.nchunks = P.nchunks;
   F.CC = P.CC;
   F.ntaps = P.ntaps;
@@ -365,6 +438,21 @@ static int gen_plan_bwd_data(const GenShape &g, GenPlan *plan) {
   return gen_finish_plan(plan);
 }
 
+template <typename T, int CC>
+static void launch_gen_cc(const GenPlan &plan, uint32_t blocks, hipStream_t st) {
+  if (plan.MT == 1u)
+    hipLaunchKernelGGL((conv_gen_kernel<T, CC, 1>), dim3(blocks), dim3(kGenThreads), plan.lds_bytes, st, plan.P);
+  else if (plan.MT == 2u)
+    hipLaunchKernelGGL((conv_gen_kernel<T, CC, 2>), dim3(blocks), dim3(kGenThreads), plan.lds_bytes, st, plan.P);
+  else
+    hipLaunchKernelGGL((conv_gen_kernel<T, CC, 4>), dim3(blocks), dim3(kGenThreads), plan.lds_bytes, st, plan.P);
+}
+template <typename T>
+static void launch_gen(const GenPlan &plan, uint32_t blocks, hipStream_t st) {
+  if (plan.P.CC == 8u) launch_gen_cc<T, 8>(plan, blocks, st);
+  else launch_gen_cc<T, 4>(plan, blocks, st);
+}
+
 static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *w, void *workspace,
                       size_t workspace_bytes, hipStream_t st) {
   ConvGenParams &P = plan->P;
@@ -380,10 +468,10 @@ static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *
   const uint32_t fblocks = (uint32_t)std::min<size_t>(1024, (plan->wt_bytes / 4u + 255u) / 256u);
   if (dtype == ADH_F32) {
     hipLaunchKernelGGL(conv_gen_filter_kernel<float>, dim3(fblocks), dim3(256), 0, st, plan->F);
-    hipLaunchKernelGGL(conv_gen_kernel<float>, dim3((uint32_t)blocks), dim3(kGenThreads), plan->lds_bytes, st, P);
+    launch_gen<float>(*plan, (uint32_t)blocks, st);
   } else {
     hipLaunchKernelGGL(conv_gen_filter_kernel<uint16_t>, dim3(fblocks), dim3(256), 0, st, plan->F);
-    hipLaunchKernelGGL(conv_gen_kernel<uint16_t>, dim3((uint32_t)blocks), dim3(kGenThreads), plan->lds_bytes, st, P);
+    launch_gen<uint16_t>(*plan, (uint32_t)blocks, st);
   }
   return launch_status();
 }
@@ -440,7 +528,10 @@ __global__ __launch_bounds__(kWgGenThreads) void conv_gen_wgrad_kernel(const Wgr
     for (int mt = 0; mt < 4; ++mt) acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   const uint32_t unit_pix = P.R * P.OWT, ksteps = unit_pix >> 2;
-  const uint32_t patch_elems = 16u * P.PR * P.PC, dy_elems = 64u * unit_pix;
+  // only the channels that exist are staged; lanes of absent channels read channel 0 and their sums are dropped
+  const uint32_t planes = min(16u, P.Cin - cit * 16u);
+  const uint32_t patch_elems = planes * P.PR * P.PC, dy_elems = 64u * unit_pix;
+  const uint32_t my_plane = l16 < planes ? l16 : 0u;
   for (uint32_t u = ps; u < P.units; u += P.PS) {
     uint32_t r2, r3, cb, rb, n, tile;
     P.div_ncb.divmod(u, r2, cb);
@@ -466,7 +557,7 @@ __global__ __launch_bounds__(kWgGenThreads) void conv_gen_wgrad_kernel(const Wgr
       P.div_PR.divmod(rc, c, r);
       const uint32_t gr = oh0 * P.sh + r, gc = ow0 * P.sw + col;
       float v = 0.f;
-      if (cit * 16u + c < P.Cin && gr < P.HP && gc < P.WP) v = gen_ld(xs, ((size_t)c * P.HP + gr) * P.WP + gc);
+      if (gr < P.HP && gc < P.WP) v = gen_ld(xs, ((size_t)c * P.HP + gr) * P.WP + gc);
       patch[c * P.PP + r * P.PCP + col] = v;
     }
     __syncthreads();
@@ -475,7 +566,7 @@ __global__ __launch_bounds__(kWgGenThreads) void conv_gen_wgrad_kernel(const Wgr
       uint32_t r, c;
       P.div_OWT.divmod(p0, r, c);
       const float *arow = dyl + l16 * P.DP + p0;
-      const float *brow = patch + l16 * P.PP + r * P.sh * P.PCP + c * P.sw;
+      const float *brow = patch + my_plane * P.PP + r * P.sh * P.PCP + c * P.sw;
       float a[4], b[TAPS];
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) a[mt] = arow[mt * 16 * P.DP];

@@ -290,6 +290,38 @@ def main():
                                                   0.0, stream),
             "hbm", 2 * in_b + out_b, HBM_PEAK_GBS, "GB/s", note="reads x and dy, writes dx; y is not read")
         del xq, yq, dq, gq, flush_scratch
+        # general slab conv (fp32 matrix cores): the 7x7 stride-2 stem over halo 3 (3 -> 64 channels, 224x224 in 4
+        # row-tiles) and a stride-2 3x3 (64 -> 128 channels) over cfg1's tiles
+        for label, Ci, Co, Hs, Ws, ph, geo in (("7x7 s2 stem 3->64, 4 tiles of 62x230", 3, 64, 56, 224, 3, (7, 7, 2, 2, 1, 1)),
+                                               ("3x3 s2 64->128, 4 tiles of 16x58", 64, 128, 14, 56, 1, (3, 3, 2, 2, 1, 1))):
+            HPs, WPs = Hs + 2 * ph, Ws + 2 * ph
+            OHs = (HPs - ((geo[0] - 1) * geo[4] + 1)) // geo[2] + 1
+            OWs = (WPs - ((geo[1] - 1) * geo[5] + 1)) // geo[3] + 1
+            xg = [torch.rand((N, Ci, HPs, WPs), device="cuda", generator=g) * 2 - 1 for _ in range(K)]
+            wg = torch.randn((Co, Ci, geo[0], geo[1]), device="cuda", generator=g) * (2.0 / (Ci * geo[0] * geo[1])) ** 0.5
+            yg = [torch.empty((N, Co, OHs, OWs), device="cuda") for _ in range(K)]
+            gg = [torch.empty((N, Ci, HPs, WPs), device="cuda") for _ in range(K)]
+            gwg = torch.empty_like(wg)
+            xg_tbl, _kg1 = capi.ptr_table([t.data_ptr() for t in xg])
+            yg_tbl, _kg2 = capi.ptr_table([t.data_ptr() for t in yg])
+            gg_tbl, _kg3 = capi.ptr_table([t.data_ptr() for t in gg])
+            wsg_bytes = max(lib.adh_conv2d_workspace_bytes(wh, 0, K, N, Ci, Co, HPs, WPs, *geo) for wh in (0, 1, 2))
+            wsg = torch.empty(wsg_bytes // 4 + 64, device="cuda")
+            fl = 2.0 * K * N * Co * Ci * geo[0] * geo[1] * OHs * OWs
+            reps, wu = 30, 5
+            add("general conv fwd " + label,
+                lambda: lib.adh_conv2d_slab_fwd_tiles(0, K, N, Ci, Co, HPs, WPs, *geo, xg_tbl, wg.data_ptr(), yg_tbl, 0.0,
+                                                      wsg.data_ptr(), wsg_bytes, stream),
+                "mfma", fl, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+            add("general conv bwd-data " + label,
+                lambda: lib.adh_conv2d_slab_bwd_data_tiles(0, K, N, Ci, Co, HPs, WPs, *geo, wg.data_ptr(), yg_tbl, gg_tbl,
+                                                           0.0, wsg.data_ptr(), wsg_bytes, stream),
+                "mfma", fl, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+            add("general conv bwd-filter " + label,
+                lambda: lib.adh_conv2d_slab_bwd_filter_tiles(0, K, N, Ci, Co, HPs, WPs, *geo, xg_tbl, yg_tbl, gwg.data_ptr(),
+                                                             0.0, wsg.data_ptr(), wsg_bytes, stream),
+                "mfma", fl, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+            del xg, yg, gg, wsg
         out["secondary"] = sec
 
     # ---- CPU baseline: the scalar port, single thread, on a bounded sample ----
