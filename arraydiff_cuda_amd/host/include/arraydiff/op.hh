@@ -685,8 +685,12 @@ public:
 };
 
 // V = GPUBatchArray3D<float>, A = GPUArray4D<float> (filter, Shape4D(kw,kh,Cin,Cout) = KCRS).
-// Supported: 3x3, stride 1, dilation 1, pad 1, halo_padded_input, no bias - the configuration of
-// the spatially-parallel blocks (src/zoo.cc:577-652); anything else throws at construction.
+// Any window / stride / dilation, no bias.  With halo_padded_input the input's halo must equal the
+// conv pad (the padded tile is convolved with pad 0, src/op.cc:1392-1410); without it the input
+// must be packed and pad must be 0 (the 1x1 projections, src/zoo.cc:680-690).  Implicit zero
+// padding of an unpadded input is not part of this path and throws at construction.  3x3 /
+// stride 1 / dilation 1 over halo 1 (the spatially-parallel blocks, src/zoo.cc:577-652) runs the
+// kernels written for it, everything else the general ones.
 // One node serves all ranks it was made for: the K slabs go to the device in ONE launch per
 // pass (the reference ran one cuDNN call per rank on K GPUs).  Make() is the one-rank form and
 // is itself the output variable; MakeParallel() returns per-rank views of one node.
@@ -710,15 +714,16 @@ public:
   SlabConv2DOp(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs, vector<shared_ptr<Var<A>>> kernels,
                shared_ptr<Context> ctx)
       : ctx_(ctx), shape_(shape), x_vars_(inputs), kernel_vars_(kernels) {
-    if (shape.kernel[0] != 3 || shape.kernel[1] != 3 || shape.stride[0] != 1 || shape.stride[1] != 1 ||
-        shape.dilate[0] != 1 || shape.dilate[1] != 1 || shape.pad[0] != 1 || shape.pad[1] != 1 ||
-        !shape.halo_padded_input)
-      throw std::invalid_argument("SlabConv2DOp: only 3x3 / stride 1 / dilation 1 / pad 1 over a halo-padded input");
+    if (shape.kernel[0] == 0 || shape.kernel[1] == 0 || shape.stride[0] == 0 || shape.stride[1] == 0 ||
+        shape.dilate[0] == 0 || shape.dilate[1] == 0)
+      throw std::invalid_argument("SlabConv2DOp: empty window, stride or dilation");
+    if (!shape.halo_padded_input && (shape.pad[0] != 0 || shape.pad[1] != 0))
+      throw std::invalid_argument("SlabConv2DOp: padding needs a halo-padded input");
     if (inputs.empty() || inputs.size() != kernels.size() || inputs.size() > ADH_MAX_TILES)
       throw std::invalid_argument("SlabConv2DOp: one kernel variable per input");
     for (size_t r = 0; r < inputs.size(); ++r) {
       auto off = inputs[r]->offset();
-      if (off.shape[0] != 1 || off.shape[1] != 1 || off.shape[2] != 0)
+      if (off.shape[0] != shape.pad[0] || off.shape[1] != shape.pad[1] || off.shape[2] != 0)
         throw std::invalid_argument("SlabConv2DOp: input halo must equal the conv pad");
       if (inputs[r]->shape() != inputs[0]->shape() || inputs[r]->batch_shape() != inputs[0]->batch_shape())
         throw std::invalid_argument("SlabConv2DOp: all slabs must have one shape");
@@ -727,9 +732,20 @@ public:
       ys_.push_back(VarData<V>(_get_output_shape(inputs[r]->shape(), inputs[r]->batch_shape()), inputs[r]->batch_shape()));
     }
   }
-  // out = floor((H + 2p - ((k-1)d+1)) / s) + 1 = H for 3x3/s1/p1 (op.cc:1512-1523)
+  // out = floor((in + 2p - ((k-1)d+1)) / s) + 1 per axis (op.cc:1512-1523)
   Shape3D _get_output_shape(Shape3D in_shape, size_t) {
-    return Shape3D(in_shape.shape[0], in_shape.shape[1], shape_.filters);
+    size_t out[2];
+    for (int a = 0; a < 2; ++a) {
+      const size_t padded = in_shape.shape[a] + 2 * shape_.pad[a], span = (shape_.kernel[a] - 1) * shape_.dilate[a] + 1;
+      if (padded < span) throw std::invalid_argument("SlabConv2DOp: window larger than the padded input");
+      out[a] = (padded - span) / shape_.stride[a] + 1;
+    }
+    return Shape3D(out[0], out[1], shape_.filters);
+  }
+  bool is_3x3_unit() const {
+    return shape_.kernel[0] == 3 && shape_.kernel[1] == 3 && shape_.stride[0] == 1 && shape_.stride[1] == 1 &&
+           shape_.dilate[0] == 1 && shape_.dilate[1] == 1 && shape_.pad[0] == 1 && shape_.pad[1] == 1 &&
+           shape_.halo_padded_input;
   }
   virtual void _push(EpochId e, function<void(Op *)> apply) {
     if (1 == stack_.push(e)) {

@@ -306,10 +306,33 @@ GPUContext *rank_ctx(const shared_ptr<Context> &ctx, size_t r) {
   if (MultiGPUContext *m = dynamic_cast<MultiGPUContext *>(ctx.get())) return m->device_context(r).get();
   return gpu_ctx_of(ctx);
 }
-void check_filter(A4 &w, size_t cin, size_t cout) {
-  if (w.dim() != Shape4D(3, 3, cin, cout) || !w.is_packed())
-    throw std::invalid_argument("SlabConv2DOp: filter must be a packed Shape4D(3,3,Cin,Cout)");
+void check_filter(A4 &w, const Conv2DShape &cs, size_t cin) {
+  if (w.dim() != Shape4D(cs.kernel[0], cs.kernel[1], cin, cs.filters) || !w.is_packed())
+    throw std::invalid_argument("SlabConv2DOp: filter must be a packed Shape4D(kw,kh,Cin,Cout)");
 }
+void check_conv_input(V3 &x, const Conv2DShape &cs) {
+  if (cs.halo_padded_input) {
+    if (cs.pad[0] != cs.pad[1]) throw std::invalid_argument("SlabConv2DOp: halo width must be one number");
+    check_padded(x, cs.pad[0], "SlabConv2DOp");
+  } else {
+    check_packed(x, "SlabConv2DOp");
+  }
+}
+// scratch of the rank's context, grown to what the general conv entry points ask for
+void *conv_scratch(GPUContext *dc, int which, uint32_t n, const TileDims &d, const Conv2DShape &cs, size_t *bytes) {
+  *bytes = adh_conv2d_workspace_bytes(which, ADH_F32, n, d.N, d.C, (uint32_t)cs.filters, d.H + 2 * (uint32_t)cs.pad[1],
+                                      d.W + 2 * (uint32_t)cs.pad[0], (uint32_t)cs.kernel[1], (uint32_t)cs.kernel[0],
+                                      (uint32_t)cs.stride[1], (uint32_t)cs.stride[0], (uint32_t)cs.dilate[1],
+                                      (uint32_t)cs.dilate[0]);
+  dc->reserve_scratch(*bytes);
+  auto scratch = dc->get_scratch();
+  *bytes = scratch->size();
+  return scratch->dptr();
+}
+#define ADH_CONV_GEOMETRY(d, cs)                                                                                    \
+  (d).H + 2 * (uint32_t)(cs).pad[1], (d).W + 2 * (uint32_t)(cs).pad[0], (uint32_t)(cs).kernel[1],                      \
+      (uint32_t)(cs).kernel[0], (uint32_t)(cs).stride[1], (uint32_t)(cs).stride[0], (uint32_t)(cs).dilate[1],          \
+      (uint32_t)(cs).dilate[0]
 }  // namespace
 
 template <>
@@ -336,16 +359,25 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
       V3 &y = ys_[r].val().get_excl(txn, id());
       d = dims_of(x);
       y.set_batch_size(d.N);
-      check_padded(x, 1, "SlabConv2DOp");
-      check_filter(w, d.C, shape_.filters);
+      check_conv_input(x, shape_);
+      check_filter(w, shape_, d.C);
       xt[n] = x.base_as_view().dptr();
       yt[n] = y.as_view().dptr();
       ++n;
     }
-    GPUConn conn = rank_ctx(ctx_, todo[0])->conn();
-    adh_check(adh_conv3x3_slab_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt, 0.0f,
-                                         nullptr, 0, conn.stream()),
-              "SlabConv2DOp::_forward");
+    GPUContext *dc = rank_ctx(ctx_, todo[0]);
+    GPUConn conn = dc->conn();
+    if (is_3x3_unit()) {
+      adh_check(adh_conv3x3_slab_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt, 0.0f,
+                                           nullptr, 0, conn.stream()),
+                "SlabConv2DOp::_forward");
+    } else {
+      size_t ws_bytes;
+      void *ws = conv_scratch(dc, ADH_CONV_FWD, n, d, shape_, &ws_bytes);
+      adh_check(adh_conv2d_slab_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, ADH_CONV_GEOMETRY(d, shape_),
+                                          xt, w0, yt, 0.0f, ws, ws_bytes, conn.stream()),
+                "SlabConv2DOp::_forward (general)");
+    }
     todo.swap(rest);
   }
 }
@@ -396,14 +428,23 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
       ++n;
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
-    const size_t ws = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
-                                                  d.H, d.W);
-    dc->reserve_scratch(ws);
-    auto scratch = dc->get_scratch();
     GPUConn conn = dc->conn();
-    adh_check(adh_conv3x3_slab_bwd_filter_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, dyt, dw,
-                                                1.0f, scratch->dptr(), scratch->size(), conn.stream()),
-              "SlabConv2DOp::_backward (filter)");
+    if (is_3x3_unit()) {
+      const size_t ws = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
+                                                    d.H, d.W);
+      dc->reserve_scratch(ws);
+      auto scratch = dc->get_scratch();
+      adh_check(adh_conv3x3_slab_bwd_filter_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, dyt, dw,
+                                                  1.0f, scratch->dptr(), scratch->size(), conn.stream()),
+                "SlabConv2DOp::_backward (filter)");
+    } else {
+      size_t ws_bytes;
+      void *ws = conv_scratch(dc, ADH_CONV_BWD_FILTER, n, d, shape_, &ws_bytes);
+      adh_check(adh_conv2d_slab_bwd_filter_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
+                                                 ADH_CONV_GEOMETRY(d, shape_), xt, dyt, dw, 1.0f, ws, ws_bytes,
+                                                 conn.stream()),
+                "SlabConv2DOp::_backward (filter, general)");
+    }
     todo.swap(rest);
   }
   // input gradient over the WHOLE padded slab, zeroed on first touch (op.cc:1687-1691), beta = 1
@@ -432,16 +473,26 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
       }
       V3 &dx = xs_[r].grad().get_mut(txn, id());
       V3 &dy = ys_[r].grad().get(txn, id());
-      check_padded(dx, 1, "SlabConv2DOp");
+      check_conv_input(dx, shape_);
       d = dims_of(dx);
       dyt[n] = dy.as_view().dptr();
       dxt[n] = dx.base_as_view().dptr();
       ++n;
     }
-    GPUConn conn = rank_ctx(ctx_, todo[0])->conn();
-    adh_check(adh_conv3x3_slab_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, w0, dyt, dxt,
-                                              1.0f, nullptr, 0, conn.stream()),
-              "SlabConv2DOp::_backward (data)");
+    GPUContext *dc = rank_ctx(ctx_, todo[0]);
+    GPUConn conn = dc->conn();
+    if (is_3x3_unit()) {
+      adh_check(adh_conv3x3_slab_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, w0, dyt, dxt,
+                                                1.0f, nullptr, 0, conn.stream()),
+                "SlabConv2DOp::_backward (data)");
+    } else {
+      size_t ws_bytes;
+      void *ws = conv_scratch(dc, ADH_CONV_BWD_DATA, n, d, shape_, &ws_bytes);
+      adh_check(adh_conv2d_slab_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
+                                               ADH_CONV_GEOMETRY(d, shape_), w0, dyt, dxt, 1.0f, ws, ws_bytes,
+                                               conn.stream()),
+                "SlabConv2DOp::_backward (data, general)");
+    }
     todo.swap(rest);
   }
 }

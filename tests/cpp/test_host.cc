@@ -21,6 +21,15 @@ void orc_conv_slab_bwd_data(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                             const float *wt, const float *dy, float beta, float *dx_pad);
 void orc_conv_slab_bwd_filter(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, uint32_t k,
                               const float *x_pad, const float *dy, float beta, float *dw);
+void orc_conv2d_slab_fwd(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t kh, uint32_t kw,
+                         uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, const float *x_pad, const float *wt,
+                         float beta, float *y);
+void orc_conv2d_slab_bwd_data(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t kh,
+                              uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, const float *wt,
+                              const float *dy, float beta, float *dx_pad);
+void orc_conv2d_slab_bwd_filter(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t kh,
+                                uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, const float *x_pad,
+                                const float *dy, float beta, float *dwt);
 void orc_halo_pad(int dtype, uint32_t p, uint32_t W, uint32_t H, uint32_t C, uint32_t N, const void *x, void *y);
 void orc_halo_unpad(int dtype, uint32_t p, uint32_t W, uint32_t H, uint32_t C, uint32_t N, const void *x, void *y);
 int orc_halo_op(int which, int dtype, uint32_t gw, uint32_t gh, uint32_t p, uint32_t W, uint32_t H, uint32_t C,
@@ -204,6 +213,65 @@ static void test_spatial_conv_graph(size_t K, size_t N, size_t C, size_t Co, siz
     const double ey = rel_err(Y, Yr), ex = rel_err(dX, dXr), ew = rel_err(dW, dWr);
     std::printf("graph K=%zu N=%zu C=%zu->%zu %zux%zu rep %d: rel-err y %.2e dx %.2e dw %.2e\n", K, N, C, Co, H, W, rep,
                 ey, ex, ew);
+    CHECK(ey <= 1e-5 && ex <= 1e-5 && ew <= 1e-5);
+  }
+}
+
+// The same graph with any window k, stride s, dilation d and halo p = d * (k - 1) / 2: the 7x7 stem
+// over halo 3 (src/zoo.cc:1525-1538), the stride-2 3x3 (src/zoo.cc:692-697) and the dilated 3x3 of
+// tools/microbench_spatial_conv.cc:25-32, against the oracle's UNSPLIT convolution.
+static void test_spatial_general_conv_graph(size_t K, size_t N, size_t C, size_t Co, size_t H, size_t W, size_t k,
+                                            size_t st, size_t dil) {
+  std::mt19937 gen(777 + (unsigned)(k * 10 + st));
+  const size_t p = dil * (k - 1) / 2;
+  const size_t OH = (H + 2 * p - (dil * (k - 1) + 1)) / st + 1, OW = (W + 2 * p - (dil * (k - 1) + 1)) / st + 1;
+  auto ctx = MultiGPUContext::Make(K);
+  std::vector<float> X = uniform(gen, N * C * H * W, -1, 1);
+  std::vector<float> Wt = normal(gen, Co * C * k * k, std::sqrt(2.0f / (C * k * k)));
+  std::vector<float> dY = normal(gen, N * Co * OH * OW, 1.0f);
+  typedef GPUBatchArray3D<float> V;
+  typedef GPUArray4D<float> A;
+  auto x_src = SrcOp<V>::Make(Shape3D(W, H, C), N, ctx->device_context(0));
+  auto w_src = ParamOp<A>::Make(Shape4D(k, k, C, Co), ctx->device_context(0));
+  vector<shared_ptr<Var<V>>> xs(K, x_src);
+  vector<shared_ptr<Var<A>>> ws(K, w_src);
+  auto tiles = SpatialScatter2DOp<V>::MakeParallel(xs, ctx);
+  auto padded = HaloPad2DOp<V>::MakeParallel(p, tiles, ctx);
+  auto exch = HaloExch2DOp<V>::MakeParallel(p, padded, ctx);
+  Conv2DShape cs;
+  cs.filters = Co;
+  cs.axes = {0, 1};
+  cs.kernel = {k, k};
+  cs.dilate = {dil, dil};
+  cs.stride = {st, st};
+  cs.pad = {p, p};
+  cs.halo_padded_input = true;
+  cs.enable_hmma = false;
+  auto ys = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch, ws, ctx);
+  CHECK(ys[0]->shape() == Shape3D(OW, OH / K, Co));
+  auto y_full = SpatialJoinedGather2DOp<V>::Make(ys, ctx);
+  auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
+  sink->set_host_grad(dY.data());
+  for (int rep = 0; rep < 2; ++rep) {
+    TxnId txn;
+    x_src->load(txn, X.data());
+    w_src->load(txn, Wt.data());
+    sink->gradient(txn);
+    ctx->sync();
+    std::vector<float> Y(dY.size()), dX(X.size()), dW(Wt.size());
+    sink->store_val(txn, Y.data());
+    x_src->store_grad(txn, dX.data());
+    w_src->store_grad(txn, dW.data());
+    const uint32_t HP = (uint32_t)(H + 2 * p), WP = (uint32_t)(W + 2 * p);
+    std::vector<float> Xp(N * C * HP * WP), Yr(Y.size()), dXp(Xp.size()), dXr(X.size()), dWr(Wt.size());
+    orc_halo_pad(0, (uint32_t)p, W, H, C, N, X.data(), Xp.data());
+    orc_conv2d_slab_fwd(N, C, Co, HP, WP, k, k, st, st, dil, dil, Xp.data(), Wt.data(), 0.f, Yr.data());
+    orc_conv2d_slab_bwd_data(N, C, Co, HP, WP, k, k, st, st, dil, dil, Wt.data(), dY.data(), 0.f, dXp.data());
+    orc_halo_unpad(0, (uint32_t)p, W, H, C, N, dXp.data(), dXr.data());
+    orc_conv2d_slab_bwd_filter(N, C, Co, HP, WP, k, k, st, st, dil, dil, Xp.data(), dY.data(), 0.f, dWr.data());
+    const double ey = rel_err(Y, Yr), ex = rel_err(dX, dXr), ew = rel_err(dW, dWr);
+    std::printf("general conv graph k=%zu s=%zu d=%zu K=%zu N=%zu C=%zu->%zu %zux%zu rep %d: rel-err y %.2e dx %.2e dw %.2e\n",
+                k, st, dil, K, N, C, Co, H, W, rep, ey, ex, ew);
     CHECK(ey <= 1e-5 && ex <= 1e-5 && ew <= 1e-5);
   }
 }
@@ -415,6 +483,10 @@ int main(int argc, char **argv) {
     test_spatial_conv_graph(2, 3, 5, 7, 6, 9);
     test_spatial_conv_graph(1, 1, 16, 16, 5, 5);
     test_spatial_conv_graph(4, 4, 64, 64, 56, 56);
+    test_spatial_general_conv_graph(4, 2, 3, 16, 32, 24, 7, 2, 1);   // the stem
+    test_spatial_general_conv_graph(2, 2, 8, 12, 16, 20, 3, 2, 1);   // stride-2 3x3
+    test_spatial_general_conv_graph(2, 1, 8, 8, 12, 14, 3, 1, 3);    // dilation 3 over halo 3
+    test_spatial_general_conv_graph(2, 2, 6, 10, 8, 9, 1, 1, 1);     // 1x1 over packed tiles (halo 0)
     test_spatial_pool_graph(kMaxPool, 4, 2, 8, 16, 12);
     test_spatial_pool_graph(kAveragePool, 2, 3, 5, 8, 10);
     test_spatial_pool_graph(kMaxPool, 4, 8, 64, 112, 112);
