@@ -51,6 +51,14 @@ SIGNATURES = {
     "adh_conv2d_slab_fwd_tiles": (i32, [i32] + [u32] * 12 + [vpp, vp, vpp, f32, vp, sz, vp]),
     "adh_conv2d_slab_bwd_data_tiles": (i32, [i32] + [u32] * 12 + [vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv2d_slab_bwd_filter_tiles": (i32, [i32] + [u32] * 12 + [vpp, vpp, vp, f32, vp, sz, vp]),
+    "adh_batchnorm2d_workspace_bytes": (sz, [u32, u32, u32]),
+    "adh_batchnorm2d_fwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, f32, i32, u32, vpp, vpp, vpp, vpp, vpp, vpp, vpp,
+                                        vpp, vpp, vpp, vp, sz, vp]),
+    "adh_batchnorm2d_bwd_tiles": (i32, [i32, u32, u32, u32, u32, u32, i32, u32, vpp, vpp, vpp, vpp, vpp, vpp, vpp, vpp, vpp,
+                                        f32, f32, vp, sz, vp]),
+    "adh_relu_fwd": (i32, [i32, ctypes.c_uint64, vp, vp, vp]),
+    "adh_relu_bwd": (i32, [i32, ctypes.c_uint64, vp, vp, vp, f32, vp]),
+    "adh_sum_fwd": (i32, [i32, u32, ctypes.c_uint64, vpp, vp, vp]),
     "adh_pool2d_slab_fwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp]),
     "adh_pool2d_slab_fwd": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, vp, vp, vp]),
     "adh_pool2d_slab_bwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vpp, vpp, vpp, f32, vp]),
@@ -264,6 +272,52 @@ def conv2d_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, HP, WP, kh, kw, sh, sw, d
     wp, wb = _ws(ws)
     return lib().adh_conv2d_slab_bwd_filter_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw_,
                                                   xt, dt, dw.data_ptr(), beta, wp, wb, _stream())
+
+
+def _opt_tbl(ts):
+    if ts is None:
+        return None, None
+    return _tbl(ts)
+
+
+def batchnorm_workspace_bytes(K, N, C):
+    return lib().adh_batchnorm2d_workspace_bytes(K, N, C)
+
+
+def batchnorm_fwd_tiles(xs, scales, shifts, ys, N, C, H, W, eps=1e-5, relu=0, out_halo=0, training=True, fixed_means=None,
+                        fixed_vars=None, run_means=None, run_vars=None, save_means=None, save_invstds=None, ws=None):
+    _dev(*xs, *ys, *scales, *shifts)
+    tabs = [_tbl(xs), _tbl(scales), _tbl(shifts), _opt_tbl(fixed_means), _opt_tbl(fixed_vars), _tbl(ys), _opt_tbl(run_means),
+            _opt_tbl(run_vars), _opt_tbl(save_means), _opt_tbl(save_invstds)]
+    wp, wb = _ws(ws)
+    return lib().adh_batchnorm2d_fwd_tiles(_dt(xs[0]), 1 if training else 0, len(xs), N, C, H, W, eps, relu, out_halo,
+                                           *[t[0] for t in tabs], wp, wb, _stream())
+
+
+def batchnorm_bwd_tiles(xs, dys, scales, shifts, save_means, save_invstds, dxs, dscales, dshifts, N, C, H, W, relu=0,
+                        dy_halo=0, beta_data=0.0, beta_param=0.0, ws=None):
+    _dev(*xs, *dys, *dxs)
+    tabs = [_tbl(xs), _tbl(dys), _tbl(scales), _opt_tbl(shifts), _tbl(save_means), _tbl(save_invstds), _tbl(dxs),
+            _tbl(dscales), _tbl(dshifts)]
+    wp, wb = _ws(ws)
+    return lib().adh_batchnorm2d_bwd_tiles(_dt(xs[0]), len(xs), N, C, H, W, relu, dy_halo, *[t[0] for t in tabs],
+                                           beta_data, beta_param, wp, wb, _stream())
+
+
+def relu_fwd(x, y):
+    _dev(x, y)
+    return lib().adh_relu_fwd(_dt(x), x.numel(), x.data_ptr(), y.data_ptr(), _stream())
+
+
+def relu_bwd(y, dy, dx, beta=0.0):
+    _dev(y, dy, dx)
+    return lib().adh_relu_bwd(_dt(y), y.numel(), y.data_ptr(), dy.data_ptr(), dx.data_ptr(), beta, _stream())
+
+
+def sum_fwd(xs, y):
+    _dev(*xs, y)
+    xt, keep = _tbl(xs)
+    return lib().adh_sum_fwd(_dt(y), len(xs), y.numel(), xt, y.data_ptr(), _stream())
 
 
 def pool_fwd_tiles(mode, xs, ys, N, C, HP, WP, wh, ww, sh, sw):

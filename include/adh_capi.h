@@ -208,6 +208,52 @@ int adh_conv2d_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, 
                                      const void *const *dy_tiles, float *dwt, float beta, void *workspace,
                                      size_t workspace_bytes, void *stream);
 
+/* ---- the shard-local ops between two halo exchanges ------------------------- */
+/* CudnnBatchNorm2DOp (src/op.cc:3907-4100) over K tiles in one call; as in the reference every
+ * tile (rank) has its own parameters and normalises with its OWN batch statistics over
+ * m = N*H*W elements per channel.  x, dx are packed (N,C,H,W); scale, shift, statistics and
+ * parameter gradients are fp32 vectors of C per tile (tables of K device pointers).
+ * training != 0: cudnnBatchNormalizationForwardTraining(SPATIAL, factor = 1, eps)
+ *   (src/op.cc:3996-4011): y = scale*(x-mean)/sqrt(var+eps) + shift; run_mean = mean,
+ *   run_var = var*m/(m-1), save_mean = mean, save_invstd = 1/sqrt(var+eps) (any of the four
+ *   tables, or entries, may be NULL).  training == 0: ...ForwardInference with fixed_mean /
+ *   fixed_var (src/op.cc:3978-3990).
+ * Fusions that have no counterpart in the reference (it ran three ops and three passes):
+ *   relu != 0 applies CudnnActivationOp's max(y,0) (src/op.cc:3189-3250) on the way out;
+ *   out_halo = p > 0 writes y into the interior of a (N,C,H+2p,W+2p) tile and zeroes its border,
+ *   i.e. HaloPad2DOp::_forward (src/op.cc:2573-2640); with relu = 0, out_halo = 0 it is the plain op.
+ * The workspace (adh_batchnorm2d_workspace_bytes, 256-byte aligned) holds partial sums. */
+size_t adh_batchnorm2d_workspace_bytes(uint32_t num_tiles, uint32_t N, uint32_t C);
+int adh_batchnorm2d_fwd_tiles(int dtype, int training, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H,
+                              uint32_t W, float eps, int relu, uint32_t out_halo, const void *const *x_tiles,
+                              const float *const *scale_tiles, const float *const *shift_tiles,
+                              const float *const *fixed_mean_tiles, const float *const *fixed_var_tiles,
+                              void *const *y_tiles, float *const *run_mean_tiles, float *const *run_var_tiles,
+                              float *const *save_mean_tiles, float *const *save_invstd_tiles, void *workspace,
+                              size_t workspace_bytes, void *stream);
+/* cudnnBatchNormalizationBackward (src/op.cc:4082-4097) with the saved statistics:
+ *   dshift = beta_param*dshift + sum dy', dscale = beta_param*dscale + sum dy'*xhat,
+ *   dx = beta_data*dx + scale*invstd*(dy' - sum dy'/m - xhat * sum dy'*xhat / m).
+ * relu != 0: dy' = dy where the fused forward output was positive (cudnnActivationBackward,
+ * src/op.cc:3252-3324; the mask is recomputed from x, y is not read); dy_halo = p > 0: dy is the
+ * interior of a gradient tile padded by p (HaloPad2DOp::_backward, src/op.cc:2642-2712).
+ * shift_tiles is only read when relu != 0. */
+int adh_batchnorm2d_bwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H, uint32_t W,
+                              int relu, uint32_t dy_halo, const void *const *x_tiles, const void *const *dy_tiles,
+                              const float *const *scale_tiles, const float *const *shift_tiles,
+                              const float *const *save_mean_tiles, const float *const *save_invstd_tiles,
+                              void *const *dx_tiles, float *const *dscale_tiles, float *const *dshift_tiles,
+                              float beta_data, float beta_param, void *workspace, size_t workspace_bytes,
+                              void *stream);
+/* CudnnActivationOp with kReluAct: cudnnActivationForward (src/op.cc:3236-3246), y = max(x, 0)
+ * (x == y allowed: relu_in_place), and cudnnActivationBackward (src/op.cc:3313-3322),
+ * dx = beta*dx + (y > 0 ? dy : 0). */
+int adh_relu_fwd(int dtype, uint64_t n, const void *x, void *y, void *stream);
+int adh_relu_bwd(int dtype, uint64_t n, const void *y, const void *dy, void *dx, float beta, void *stream);
+/* SumJoinOp::_forward (src/op.cc:744-806): y = x_0 + x_1 + ... (the residual join); its backward
+ * is adh_add_f32 / adh_slice_add_nchw of dy onto every input gradient. */
+int adh_sum_fwd(int dtype, uint32_t num_inputs, uint64_t n, const void *const *xs, void *y, void *stream);
+
 /* ---- pooling over the halo-padded slab ------------------------------------- */
 /* CudnnPool2DOp with Pool2DShape::halo_padded_input (include/arraydiff/op.hh:2917-2925): the
  * padded tile (N, C, HP, WP) with HP = H + 2*pad_h, WP = W + 2*pad_w is handed to cuDNN as a plain

@@ -223,6 +223,45 @@ def conv2d_slab_bwd_filter(x_pad, dy, sh, sw, dh, dw, dwt, beta=0.0):
                                     _u32(sw), _u32(dh), _u32(dw), _ptr(x_pad), _ptr(dy), ctypes.c_float(beta), _ptr(dwt))
 
 
+def _fp(a):
+    return _ptr(a) if a is not None else None
+
+
+def batchnorm2d_fwd_train(x, scale, shift, eps, relu, p, y, run_mean=None, run_var=None, save_mean=None, save_invstd=None):
+    N, C, H, W = x.shape
+    assert y.shape == (N, C, H + 2 * p, W + 2 * p)
+    _lib.orc_batchnorm2d_fwd_train(_u32(N), _u32(C), _u32(H), _u32(W), ctypes.c_float(eps), ctypes.c_int(relu), _u32(p),
+                                   _ptr(x), _ptr(scale), _ptr(shift), _ptr(y), _fp(run_mean), _fp(run_var), _fp(save_mean),
+                                   _fp(save_invstd))
+
+
+def batchnorm2d_fwd_infer(x, scale, shift, fixed_mean, fixed_var, eps, relu, p, y):
+    N, C, H, W = x.shape
+    assert y.shape == (N, C, H + 2 * p, W + 2 * p)
+    _lib.orc_batchnorm2d_fwd_infer(_u32(N), _u32(C), _u32(H), _u32(W), ctypes.c_float(eps), ctypes.c_int(relu), _u32(p),
+                                   _ptr(x), _ptr(scale), _ptr(shift), _ptr(fixed_mean), _ptr(fixed_var), _ptr(y))
+
+
+def batchnorm2d_bwd(x, dy, scale, shift, save_mean, save_invstd, relu, p, dx, dscale, dshift, beta_data=0.0, beta_param=0.0):
+    N, C, H, W = x.shape
+    assert dy.shape == (N, C, H + 2 * p, W + 2 * p)
+    _lib.orc_batchnorm2d_bwd(_u32(N), _u32(C), _u32(H), _u32(W), ctypes.c_int(relu), _u32(p), _ptr(x), _ptr(dy), _ptr(scale),
+                             _fp(shift), _ptr(save_mean), _ptr(save_invstd), ctypes.c_float(beta_data),
+                             ctypes.c_float(beta_param), _ptr(dx), _ptr(dscale), _ptr(dshift))
+
+
+def relu_fwd(x, y):
+    _lib.orc_relu_fwd(ctypes.c_uint64(x.size), _ptr(x), _ptr(y))
+
+
+def relu_bwd(y, dy, dx, beta=0.0):
+    _lib.orc_relu_bwd(ctypes.c_uint64(y.size), _ptr(y), _ptr(dy), ctypes.c_float(beta), _ptr(dx))
+
+
+def sum_fwd(xs, y):
+    _lib.orc_sum_fwd(_u32(len(xs)), ctypes.c_uint64(y.size), _ptr_array(xs), _ptr(y))
+
+
 def pool_slab_fwd(mode, x_pad, wh, ww, sh, sw, y):
     """x_pad (N, C, HP, WP) float32 -> y (N, C, OH, OW); mode 1 = max, 0 = average."""
     N, C, HP, WP = x_pad.shape

@@ -28,6 +28,9 @@
  *   - general conv (any window / stride / dilation) : pinned against torch
  *     conv2d(stride, dilation) + autograd on the CPU and against the 3x3
  *     stride-1 functions above.
+ *   - batch norm / rectifier / sum : pinned against torch batch_norm (training and
+ *     evaluation) + relu + constant_pad + autograd on the CPU, and closed forms
+ *     (normalised output has mean 0 / variance 1, dx sums to zero per channel).
  *   - pooling over the padded slab : pinned against torch max_pool2d /
  *     avg_pool2d + autograd on the CPU; which element of a window receives the
  *     max gradient when several are equal is cuDNN's choice and is parity
@@ -543,6 +546,122 @@ void orc_conv2d_slab_bwd_filter(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_
           size_t wi = ((co * (size_t)Cin + ci) * kh + a) * kw + b;
           dwt[wi] = (float)(acc + (beta != 0.0f ? (double)beta * dwt[wi] : 0.0));
         }
+}
+
+/* ------------------------------------------------------------------ */
+/* shard-local ops between halos: batch norm, rectifier, residual sum     */
+/* ------------------------------------------------------------------ */
+
+/* cudnnBatchNormalizationForwardTraining(CUDNN_BATCHNORM_SPATIAL, factor = 1, eps) at
+ * src/op.cc:3996-4011 over one tile (N,C,H,W): per channel over m = N*H*W elements
+ *   mean = sum x / m, var = sum (x-mean)^2 / m, y = scale*(x-mean)/sqrt(var+eps) + shift,
+ *   running mean = mean, running variance = var*m/(m-1) (factor 1 replaces the old values),
+ *   saved mean = mean, saved inverse std = 1/sqrt(var+eps).
+ * relu != 0 applies CudnnActivationOp's max(y,0) (src/op.cc:3189-3250) on the way out;
+ * p > 0 writes y into the interior of a tile padded by p and zeroes the border
+ * (HaloPad2DOp::_forward, src/op.cc:2573-2640).  Two passes in double. */
+void orc_batchnorm2d_fwd_train(uint32_t N, uint32_t C, uint32_t H, uint32_t W, float eps, int relu, uint32_t p,
+                               const float *x, const float *scale, const float *shift, float *y, float *run_mean,
+                               float *run_var, float *save_mean, float *save_invstd) {
+  const size_t HW = (size_t)H * W, WP = W + 2 * (size_t)p, HP = H + 2 * (size_t)p;
+  const double m = (double)N * (double)HW;
+  for (size_t i = 0; i < (size_t)N * C * HP * WP; ++i) y[i] = 0.0f;
+  for (uint32_t c = 0; c < C; ++c) {
+    double s = 0.0;
+    for (uint32_t n = 0; n < N; ++n)
+      for (size_t i = 0; i < HW; ++i) s += x[((size_t)n * C + c) * HW + i];
+    const double mean = s / m;
+    double v = 0.0;
+    for (uint32_t n = 0; n < N; ++n)
+      for (size_t i = 0; i < HW; ++i) {
+        const double d = x[((size_t)n * C + c) * HW + i] - mean;
+        v += d * d;
+      }
+    const double var = v / m, invstd = 1.0 / sqrt(var + (double)eps);
+    if (run_mean) run_mean[c] = (float)mean;
+    if (run_var) run_var[c] = (float)(m > 1.0 ? var * m / (m - 1.0) : var);
+    if (save_mean) save_mean[c] = (float)mean;
+    if (save_invstd) save_invstd[c] = (float)invstd;
+    for (uint32_t n = 0; n < N; ++n)
+      for (uint32_t h = 0; h < H; ++h)
+        for (uint32_t w = 0; w < W; ++w) {
+          double o = (double)scale[c] * (x[((size_t)n * C + c) * HW + (size_t)h * W + w] - mean) * invstd + (double)shift[c];
+          if (relu && o < 0.0) o = 0.0;
+          y[((size_t)n * C + c) * HP * WP + (size_t)(h + p) * WP + w + p] = (float)o;
+        }
+  }
+}
+
+/* cudnnBatchNormalizationForwardInference at src/op.cc:3978-3990:
+ *   y = scale*(x - fixed_mean)/sqrt(fixed_var + eps) + shift */
+void orc_batchnorm2d_fwd_infer(uint32_t N, uint32_t C, uint32_t H, uint32_t W, float eps, int relu, uint32_t p,
+                               const float *x, const float *scale, const float *shift, const float *fixed_mean,
+                               const float *fixed_var, float *y) {
+  const size_t HW = (size_t)H * W, WP = W + 2 * (size_t)p, HP = H + 2 * (size_t)p;
+  for (size_t i = 0; i < (size_t)N * C * HP * WP; ++i) y[i] = 0.0f;
+  for (uint32_t n = 0; n < N; ++n)
+    for (uint32_t c = 0; c < C; ++c) {
+      const double invstd = 1.0 / sqrt((double)fixed_var[c] + (double)eps);
+      for (uint32_t h = 0; h < H; ++h)
+        for (uint32_t w = 0; w < W; ++w) {
+          double o = (double)scale[c] * (x[((size_t)n * C + c) * HW + (size_t)h * W + w] - (double)fixed_mean[c]) * invstd +
+                     (double)shift[c];
+          if (relu && o < 0.0) o = 0.0;
+          y[((size_t)n * C + c) * HP * WP + (size_t)(h + p) * WP + w + p] = (float)o;
+        }
+    }
+}
+
+/* cudnnBatchNormalizationBackward(alpha = 1, beta as given for data and parameters) at
+ * src/op.cc:4082-4097 with the saved mean / inverse std of the forward pass:
+ *   dshift = sum dy', dscale = sum dy'*xhat, dx = scale*invstd*(dy' - dshift/m - xhat*dscale/m),
+ * xhat = (x-mean)*invstd.  relu != 0: dy' = dy where the forward output was positive
+ * (cudnnActivationBackward, src/op.cc:3252-3324); p > 0: dy is the interior of a gradient tile
+ * padded by p (HaloPad2DOp::_backward, src/op.cc:2642-2712). */
+void orc_batchnorm2d_bwd(uint32_t N, uint32_t C, uint32_t H, uint32_t W, int relu, uint32_t p, const float *x,
+                         const float *dy, const float *scale, const float *shift, const float *save_mean,
+                         const float *save_invstd, float beta_data, float beta_param, float *dx, float *dscale,
+                         float *dshift) {
+  const size_t HW = (size_t)H * W, WP = W + 2 * (size_t)p, HP = H + 2 * (size_t)p;
+  const double m = (double)N * (double)HW;
+  for (uint32_t c = 0; c < C; ++c) {
+    const double mean = save_mean[c], invstd = save_invstd[c], sc = scale[c], sh = shift ? shift[c] : 0.0;
+    double sd = 0.0, sdx = 0.0;
+    for (int pass = 0; pass < 2; ++pass)
+      for (uint32_t n = 0; n < N; ++n)
+        for (uint32_t h = 0; h < H; ++h)
+          for (uint32_t w = 0; w < W; ++w) {
+            const size_t xi = ((size_t)n * C + c) * HW + (size_t)h * W + w;
+            const double xhat = (x[xi] - mean) * invstd;
+            double d = dy[((size_t)n * C + c) * HP * WP + (size_t)(h + p) * WP + w + p];
+            if (relu && !(sc * xhat + sh > 0.0)) d = 0.0;
+            if (pass == 0) {
+              sd += d;
+              sdx += d * xhat;
+            } else {
+              const double g = sc * invstd * (d - sd / m - xhat * sdx / m);
+              dx[xi] = (float)(g + (beta_data != 0.0f ? (double)beta_data * dx[xi] : 0.0));
+            }
+          }
+    dscale[c] = (float)(sdx + (beta_param != 0.0f ? (double)beta_param * dscale[c] : 0.0));
+    dshift[c] = (float)(sd + (beta_param != 0.0f ? (double)beta_param * dshift[c] : 0.0));
+  }
+}
+
+/* cudnnActivationForward / Backward with CUDNN_ACTIVATION_RELU (src/op.cc:3189-3324) */
+void orc_relu_fwd(uint64_t n, const float *x, float *y) {
+  for (uint64_t i = 0; i < n; ++i) y[i] = x[i] > 0.0f ? x[i] : 0.0f;
+}
+void orc_relu_bwd(uint64_t n, const float *y, const float *dy, float beta, float *dx) {
+  for (uint64_t i = 0; i < n; ++i) dx[i] = (y[i] > 0.0f ? dy[i] : 0.0f) + (beta != 0.0f ? beta * dx[i] : 0.0f);
+}
+/* SumJoinOp::_forward (src/op.cc:744-806): y = x_0 + x_1 + ... in that order */
+void orc_sum_fwd(uint32_t count, uint64_t n, const float *const *xs, float *y) {
+  for (uint64_t i = 0; i < n; ++i) {
+    float v = xs[0][i];
+    for (uint32_t k = 1; k < count; ++k) v += xs[k][i];
+    y[i] = v;
+  }
 }
 
 /* ------------------------------------------------------------------ */
