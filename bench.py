@@ -290,6 +290,34 @@ def main():
                                                   0.0, stream),
             "hbm", 2 * in_b + out_b, HBM_PEAK_GBS, "GB/s", note="reads x and dy, writes dx; y is not read")
         del xq, yq, dq, gq, flush_scratch
+        # batch norm with tile-local statistics + rectifier + halo pad in one call (the BN -> ReLU -> HaloPad
+        # prefix of the spatially-parallel residual block) on cfg1's 4 tiles, and its backward
+        xb = [torch.randn((N, C, Ht, W), device="cuda", generator=g) + 0.5 for _ in range(K)]
+        sc = [torch.rand(C, device="cuda", generator=g) + 0.5 for _ in range(K)]
+        sh = [torch.rand(C, device="cuda", generator=g) - 0.5 for _ in range(K)]
+        sm = [torch.empty(C, device="cuda") for _ in range(K)]
+        si = [torch.empty(C, device="cuda") for _ in range(K)]
+        dsc = [torch.empty(C, device="cuda") for _ in range(K)]
+        dsh = [torch.empty(C, device="cuda") for _ in range(K)]
+        dxb = [torch.empty((N, C, Ht, W), device="cuda") for _ in range(K)]
+        tabs = {k: capi.ptr_table([t.data_ptr() for t in v]) for k, v in
+                (("x", xb), ("sc", sc), ("sh", sh), ("sm", sm), ("si", si), ("dsc", dsc), ("dsh", dsh), ("dx", dxb))}
+        bn_ws_bytes = lib.adh_batchnorm2d_workspace_bytes(K, N, C)
+        bn_ws = torch.empty(bn_ws_bytes // 4, device="cuda")
+        packed_b = K * N * C * Ht * W * 4
+        reps, wu = 100, 10
+        add("batch norm (training) + relu + halo pad fwd, cfg1 tiles (3 kernels)",
+            lambda: lib.adh_batchnorm2d_fwd_tiles(0, 1, K, N, C, Ht, W, 1e-5, 1, 1, tabs["x"][0], tabs["sc"][0], tabs["sh"][0],
+                                                  None, None, tile_tbl, None, None, tabs["sm"][0], tabs["si"][0],
+                                                  bn_ws.data_ptr(), bn_ws_bytes, stream),
+            "hbm", 2 * packed_b + padded_b, HBM_PEAK_GBS, "GB/s", note="x read for the statistics and again to normalise")
+        add("batch norm + relu + halo unpad bwd, cfg1 tiles (3 kernels)",
+            lambda: lib.adh_batchnorm2d_bwd_tiles(0, K, N, C, Ht, W, 1, 1, tabs["x"][0], g_tbl, tabs["sc"][0], tabs["sh"][0],
+                                                  tabs["sm"][0], tabs["si"][0], tabs["dx"][0], tabs["dsc"][0], tabs["dsh"][0],
+                                                  0.0, 0.0, bn_ws.data_ptr(), bn_ws_bytes, stream),
+            "hbm", 2 * (packed_b + packed_b) + packed_b, HBM_PEAK_GBS, "GB/s",
+            note="x and the interior of dy read twice (sums, then gradient), dx written")
+        del xb, dxb
         # general slab conv (fp32 matrix cores): the 7x7 stride-2 stem over halo 3 (3 -> 64 channels, 224x224 in 4
         # row-tiles) and a stride-2 3x3 (64 -> 128 channels) over cfg1's tiles
         for label, Ci, Co, Hs, Ws, ph, geo in (("7x7 s2 stem 3->64, 4 tiles of 62x230", 3, 64, 56, 224, 3, (7, 7, 2, 2, 1, 1)),
