@@ -786,6 +786,269 @@ template <typename V, typename A, typename B = A>
 using CudnnConv2DOp = SlabConv2DOp<V, A>;
 
 // ---------------------------------------------------------------------------
+// the shard-local ops between two halo exchanges: batch norm, rectifier, sum join
+// ---------------------------------------------------------------------------
+class VarIdSet {
+public:
+  void insert(VarId v) { ids_.insert(v.raw_id()); }
+  void insert_all(const VarIdSet &o) { ids_.insert(o.ids_.begin(), o.ids_.end()); }
+  bool contains(VarId v) const { return ids_.count(v.raw_id()) != 0; }
+  size_t size() const { return ids_.size(); }
+
+private:
+  std::set<uint64_t> ids_;
+};
+
+template <typename V, typename B>
+class BatchNormOutput {
+public:
+  shared_ptr<Var<V>> op;
+  shared_ptr<Var<B>> batch_mean;
+  shared_ptr<Var<B>> batch_variance;
+  shared_ptr<Var<B>> fixed_mean;
+  shared_ptr<Var<B>> fixed_variance;
+  shared_ptr<Var<B>> scale;
+  shared_ptr<Var<B>> shift;
+  VarIdSet params;
+  VarIdSet grads;
+  VarIdSet batch_stats;
+  VarIdSet fixed_stats;
+};
+
+// additions to the reference's struct: the per-rank parameter variables, so that a caller can load them
+template <typename V, typename B>
+class ParallelBatchNormOutput {
+public:
+  vector<shared_ptr<Var<V>>> ops;
+  vector<VarIdSet> params;
+  vector<VarIdSet> grads;
+  vector<VarIdSet> batch_stats;
+  vector<VarIdSet> fixed_stats;
+  vector<shared_ptr<ParamOp<B>>> scales, shifts, fixed_means, fixed_variances, batch_means, batch_variances;
+};
+
+// Switch = bool, V = GPUBatchArray3D<float>, B = GPUArray1D<float>.  *switch_var == false: batch
+// statistics of THIS rank's tile (training), true: the fixed statistics (evaluation; its backward
+// is unimplemented in the reference too, src/op.cc:4078-4080).  One node serves all ranks it was
+// made for (one launch per pass over all tiles); every rank keeps its own parameters and statistics.
+// Unlike the reference's Make(), the parameters start uninitialised: load scale / shift (and the fixed
+// statistics for evaluation) through the ParamOps in the output before the first transaction.
+template <typename Switch, typename V, typename B>
+class SlabBatchNorm2DOp : public virtual Op, public virtual Var<V> {
+public:
+  struct RankVars {
+    shared_ptr<ParamOp<B>> batch_mean, batch_variance, fixed_mean, fixed_variance, scale, shift;
+  };
+  static RankVars make_rank_vars(size_t channels, shared_ptr<Context> dev_ctx) {
+    RankVars v;
+    typename B::Shape s(channels);
+    v.batch_mean = ParamOp<B>::Make(s, dev_ctx);
+    v.batch_variance = ParamOp<B>::Make(s, dev_ctx);
+    v.fixed_mean = ParamOp<B>::Make(s, dev_ctx);
+    v.fixed_variance = ParamOp<B>::Make(s, dev_ctx);
+    v.scale = ParamOp<B>::Make(s, dev_ctx);
+    v.shift = ParamOp<B>::Make(s, dev_ctx);
+    return v;
+  }
+  static BatchNormOutput<V, B> Make(size_t channels, shared_ptr<Switch> switch_var, shared_ptr<Var<V>> input,
+                                    shared_ptr<Context> ctx) {
+    RankVars v = make_rank_vars(channels, ctx);
+    auto op = make_shared<SlabBatchNorm2DOp<Switch, V, B>>(switch_var, vector<shared_ptr<Var<V>>>{input},
+                                                           vector<RankVars>{v}, ctx);
+    BatchNormOutput<V, B> out;
+    out.op = op;
+    out.batch_mean = v.batch_mean; out.batch_variance = v.batch_variance;
+    out.fixed_mean = v.fixed_mean; out.fixed_variance = v.fixed_variance;
+    out.scale = v.scale; out.shift = v.shift;
+    fill_sets(v, &out.params, &out.grads, &out.batch_stats, &out.fixed_stats);
+    return out;
+  }
+  static ParallelBatchNormOutput<V, B> MakeParallel(size_t channels, shared_ptr<Switch> switch_var,
+                                                    vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+    MultiGPUContext *m = mgpu_ctx_of(ctx);
+    vector<RankVars> vars;
+    for (size_t r = 0; r < inputs.size(); ++r) vars.push_back(make_rank_vars(channels, m->device_context(r)));
+    auto op = make_shared<SlabBatchNorm2DOp<Switch, V, B>>(switch_var, inputs, vars, ctx);
+    ParallelBatchNormOutput<V, B> out;
+    for (size_t r = 0; r < inputs.size(); ++r) {
+      out.ops.push_back(make_shared<NoOp<V>>(op, op->ys_.at(r).clone()));
+      VarIdSet p, g, bs, fs;
+      fill_sets(vars[r], &p, &g, &bs, &fs);
+      out.params.push_back(p); out.grads.push_back(g); out.batch_stats.push_back(bs); out.fixed_stats.push_back(fs);
+      out.scales.push_back(vars[r].scale); out.shifts.push_back(vars[r].shift);
+      out.fixed_means.push_back(vars[r].fixed_mean); out.fixed_variances.push_back(vars[r].fixed_variance);
+      out.batch_means.push_back(vars[r].batch_mean); out.batch_variances.push_back(vars[r].batch_variance);
+    }
+    return out;
+  }
+  SlabBatchNorm2DOp(shared_ptr<Switch> switch_var, vector<shared_ptr<Var<V>>> inputs, vector<RankVars> vars,
+                    shared_ptr<Context> ctx)
+      : ctx_(ctx), switch_var_(switch_var), x_vars_(inputs), vars_(vars) {
+    if (inputs.empty() || inputs.size() != vars.size() || inputs.size() > ADH_MAX_TILES)
+      throw std::invalid_argument("SlabBatchNorm2DOp: one set of parameters per input");
+    for (size_t r = 0; r < inputs.size(); ++r) {
+      if (inputs[r]->shape() != inputs[0]->shape() || inputs[r]->batch_shape() != inputs[0]->batch_shape())
+        throw std::invalid_argument("SlabBatchNorm2DOp: all tiles must have one shape");
+      if (!inputs[r]->offset().is_zero())
+        throw std::invalid_argument("SlabBatchNorm2DOp: input must be packed");
+      xs_.push_back(inputs[r]->data());
+      ys_.push_back(VarData<V>(inputs[r]->shape(), inputs[r]->batch_shape()));
+      batch_mean_.push_back(vars[r].batch_mean->data());
+      batch_variance_.push_back(vars[r].batch_variance->data());
+      fixed_mean_.push_back(vars[r].fixed_mean->data());
+      fixed_variance_.push_back(vars[r].fixed_variance->data());
+      scale_.push_back(vars[r].scale->data());
+      shift_.push_back(vars[r].shift->data());
+      tmp_mean_.push_back(TxnVar<B>(_get_stat_shape(inputs[r]->shape())));
+      tmp_variance_.push_back(TxnVar<B>(_get_stat_shape(inputs[r]->shape())));
+    }
+  }
+  typename B::Shape _get_stat_shape(typename V::Shape in_shape) { return typename B::Shape(in_shape.shape[2]); }
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) {
+      for (size_t r = 0; r < x_vars_.size(); ++r) {
+        x_vars_[r]->_push(e, apply);
+        vars_[r].fixed_mean->_push(e, apply);
+        vars_[r].fixed_variance->_push(e, apply);
+        vars_[r].scale->_push(e, apply);
+        vars_[r].shift->_push(e, apply);
+      }
+      apply(this);
+    }
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) {
+      apply(this);
+      for (size_t r = x_vars_.size(); r-- > 0;) {
+        vars_[r].shift->_pop(e, apply);
+        vars_[r].scale->_pop(e, apply);
+        vars_[r].fixed_variance->_pop(e, apply);
+        vars_[r].fixed_mean->_pop(e, apply);
+        x_vars_[r]->_pop(e, apply);
+      }
+    }
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+  virtual typename V::Shape shape() { return ys_[0].shape(); }
+  virtual typename V::Shape offset() { return ys_[0].offset(); }
+  virtual typename V::Shape stride() { return ys_[0].stride(); }
+  virtual size_t batch_shape() { return ys_[0].batch_shape(); }
+  virtual VarData<V> data() { return ys_[0].clone(); }
+
+private:
+  static void fill_sets(const RankVars &v, VarIdSet *params, VarIdSet *grads, VarIdSet *batch_stats, VarIdSet *fixed_stats) {
+    batch_stats->insert(v.batch_mean->vars().at(0));
+    batch_stats->insert(v.batch_variance->vars().at(0));
+    fixed_stats->insert(v.fixed_mean->vars().at(0));
+    fixed_stats->insert(v.fixed_variance->vars().at(0));
+    params->insert(v.scale->vars().at(0));
+    params->insert(v.shift->vars().at(0));
+    grads->insert(v.scale->vars().at(1));
+    grads->insert(v.shift->vars().at(1));
+  }
+  shared_ptr<Context> ctx_;
+  shared_ptr<Switch> switch_var_;
+  vector<shared_ptr<Var<V>>> x_vars_;
+  vector<RankVars> vars_;
+  vector<VarData<V>> xs_, ys_;
+  vector<VarData<B>> batch_mean_, batch_variance_, fixed_mean_, fixed_variance_, scale_, shift_;
+  vector<TxnVar<B>> tmp_mean_, tmp_variance_;
+};
+template <typename Switch, typename V, typename B>
+using CudnnBatchNorm2DOp = SlabBatchNorm2DOp<Switch, V, B>;
+
+enum Activation {
+  kReluAct,
+};
+
+// y = max(x, 0); backward dx += (y > 0 ? dy : 0) (src/op.cc:3189-3324, the out-of-place form)
+template <typename V>
+class CudnnActivationOp : public UnaryVarOp<V> {
+public:
+  static shared_ptr<Var<V>> Make(Activation activation, shared_ptr<Var<V>> input, shared_ptr<Context> ctx) {
+    return make_shared<CudnnActivationOp<V>>(activation, input, ctx);
+  }
+  static vector<shared_ptr<Var<V>>> MakeParallel(Activation activation, vector<shared_ptr<Var<V>>> inputs,
+                                                 shared_ptr<Context> ctx) {
+    return make_per_rank<V>(ctx, [&](size_t r, shared_ptr<Context> dc) { return Make(activation, inputs.at(r), dc); });
+  }
+  CudnnActivationOp(Activation activation, shared_ptr<Var<V>> input, shared_ptr<Context> ctx) : UnaryVarOp<V>(input, ctx) {
+    if (activation != kReluAct) throw std::invalid_argument("CudnnActivationOp: only kReluAct");
+    if (!input->offset().is_zero()) throw std::invalid_argument("CudnnActivationOp: input must be packed");
+    this->y_ = VarData<V>(input->shape(), input->batch_shape());
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+};
+template <typename V>
+shared_ptr<Var<V>> relu(shared_ptr<Var<V>> input, shared_ptr<Context> ctx) {
+  return CudnnActivationOp<V>::Make(kReluAct, input, ctx);
+}
+template <typename V>
+vector<shared_ptr<Var<V>>> parallel_relu(vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+  return CudnnActivationOp<V>::MakeParallel(kReluAct, inputs, ctx);
+}
+
+// y = x_0 + x_1 + ...; backward adds dy onto every input's gradient (JoinOp<V, SumJoin>, src/op.cc:744-867)
+class SumJoin {};
+template <typename V, typename Join>
+class JoinOp : public virtual Op, public virtual Var<V> {
+public:
+  static shared_ptr<Var<V>> Make(Join join, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+    return make_shared<JoinOp<V, Join>>(join, false, inputs, ctx);
+  }
+  // inputs.at(j).at(rank)
+  static vector<shared_ptr<Var<V>>> MakeParallel(Join join, vector<vector<shared_ptr<Var<V>>>> inputs,
+                                                 shared_ptr<Context> ctx) {
+    return make_per_rank<V>(ctx, [&](size_t r, shared_ptr<Context> dc) {
+      vector<shared_ptr<Var<V>>> dev_inputs;
+      for (auto &in : inputs) dev_inputs.push_back(in.at(r));
+      return Make(join, dev_inputs, dc);
+    });
+  }
+  JoinOp(Join, bool in_place, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) : ctx_(ctx), inputs_(inputs) {
+    if (in_place) throw std::invalid_argument("JoinOp: the in-place form is not part of this path");
+    if (inputs.empty() || inputs.size() > ADH_MAX_TILES) throw std::invalid_argument("JoinOp: 1..16 inputs");
+    for (auto &in : inputs) {
+      if (in->shape() != inputs[0]->shape() || in->batch_shape() != inputs[0]->batch_shape() || !in->offset().is_zero())
+        throw std::invalid_argument("JoinOp: inputs must be packed and of one shape");
+      xs_.push_back(in->data());
+    }
+    y_ = VarData<V>(inputs[0]->shape(), inputs[0]->batch_shape());
+  }
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) {
+      for (auto &in : inputs_) in->_push(e, apply);
+      apply(this);
+    }
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) {
+      apply(this);
+      for (size_t j = inputs_.size(); j-- > 0;) inputs_[j]->_pop(e, apply);
+    }
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+  ARRAYDIFF_VAR_ACCESSORS(V)
+
+private:
+  shared_ptr<Context> ctx_;
+  vector<shared_ptr<Var<V>>> inputs_;
+  vector<VarData<V>> xs_;
+  VarData<V> y_;
+};
+template <typename V>
+shared_ptr<Var<V>> sum(vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+  return JoinOp<V, SumJoin>::Make(SumJoin(), inputs, ctx);
+}
+template <typename V>
+vector<shared_ptr<Var<V>>> parallel_sum(vector<vector<shared_ptr<Var<V>>>> inputs, shared_ptr<Context> ctx) {
+  return JoinOp<V, SumJoin>::MakeParallel(SumJoin(), inputs, ctx);
+}
+
+// ---------------------------------------------------------------------------
 // pooling over the halo-padded slab
 // ---------------------------------------------------------------------------
 enum Pooling {

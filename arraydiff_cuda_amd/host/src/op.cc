@@ -497,6 +497,184 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
   }
 }
 
+// ---- SlabBatchNorm2DOp (op.cc:3907-4100) ----
+typedef GPUArray1D<float> B1;
+
+template <>
+void SlabBatchNorm2DOp<bool, V3, B1>::_forward(TxnId txn) {
+  const size_t K = xs_.size();
+  const bool fixed = *switch_var_;
+  const void *xt[ADH_MAX_TILES];
+  void *yt[ADH_MAX_TILES];
+  const float *sc[ADH_MAX_TILES], *sh[ADH_MAX_TILES], *fm[ADH_MAX_TILES], *fv[ADH_MAX_TILES];
+  float *rm[ADH_MAX_TILES], *rv[ADH_MAX_TILES], *tm[ADH_MAX_TILES], *tv[ADH_MAX_TILES];
+  uint32_t n = 0;
+  TileDims d{};
+  for (size_t r = 0; r < K; ++r) {
+    GPUContext *dc = rank_ctx(ctx_, r);
+    if (!ys_[r].val().overwrite(txn, id(), dc)) continue;
+    V3 &x = xs_[r].val().get(txn, id());
+    V3 &y = ys_[r].val().get_excl(txn, id());
+    d = dims_of(x);
+    y.set_batch_size(d.N);
+    check_packed(x, "SlabBatchNorm2DOp");
+    xt[n] = x.as_view().dptr();
+    yt[n] = y.as_view().dptr();
+    sc[n] = scale_[r].val().get(txn, id()).dptr();
+    sh[n] = shift_[r].val().get(txn, id()).dptr();
+    if (fixed) {
+      fm[n] = fixed_mean_[r].val().get(txn, id()).dptr();
+      fv[n] = fixed_variance_[r].val().get(txn, id()).dptr();
+    } else {
+      // the reference asserts that it is the only writer of the four statistics (op.cc:3992-3995)
+      if (!batch_mean_[r].val().overwrite(txn, id(), dc) || !batch_variance_[r].val().overwrite(txn, id(), dc) ||
+          !tmp_mean_[r].overwrite(txn, id(), dc) || !tmp_variance_[r].overwrite(txn, id(), dc))
+        throw HazardError("SlabBatchNorm2DOp: batch statistics already written in this transaction");
+      rm[n] = batch_mean_[r].val().get_excl(txn, id()).dptr();
+      rv[n] = batch_variance_[r].val().get_excl(txn, id()).dptr();
+      tm[n] = tmp_mean_[r].get_excl(txn, id()).dptr();
+      tv[n] = tmp_variance_[r].get_excl(txn, id()).dptr();
+    }
+    ++n;
+  }
+  if (n == 0) return;
+  GPUContext *dc = rank_ctx(ctx_, 0);
+  const size_t ws = adh_batchnorm2d_workspace_bytes(n, d.N, d.C);
+  dc->reserve_scratch(ws);
+  auto scratch = dc->get_scratch();
+  GPUConn conn = dc->conn();
+  adh_check(adh_batchnorm2d_fwd_tiles(ADH_F32, fixed ? 0 : 1, n, d.N, d.C, d.H, d.W, 1.0e-5f, 0, 0, xt, sc, sh,
+                                      fixed ? fm : nullptr, fixed ? fv : nullptr, yt, fixed ? nullptr : rm,
+                                      fixed ? nullptr : rv, fixed ? nullptr : tm, fixed ? nullptr : tv, scratch->dptr(),
+                                      scratch->size(), conn.stream()),
+            "SlabBatchNorm2DOp::_forward");
+}
+
+template <>
+void SlabBatchNorm2DOp<bool, V3, B1>::_backward(TxnId txn) {
+  const size_t K = xs_.size();
+  const void *xt[ADH_MAX_TILES], *dyt[ADH_MAX_TILES];
+  void *dxt[ADH_MAX_TILES];
+  const float *sc[ADH_MAX_TILES], *sh[ADH_MAX_TILES], *tm[ADH_MAX_TILES], *tv[ADH_MAX_TILES];
+  float *dsc[ADH_MAX_TILES], *dsh[ADH_MAX_TILES];
+  uint32_t n = 0;
+  TileDims d{};
+  for (size_t r = 0; r < K; ++r) {
+    GPUContext *dc = rank_ctx(ctx_, r);
+    const size_t batch = xs_[r].val().get(txn, id()).batch_size();
+    if (!xs_[r].grad().accumulate(txn, id(), dc, [dc, batch](V3 *g) {
+          GPUConn conn = dc->conn();
+          g->set_batch_size(batch);
+          g->as_view().set_constant(0.0f, conn);
+        }))
+      continue;
+    if (*switch_var_) throw std::logic_error("SlabBatchNorm2DOp: backward with fixed statistics is unimplemented");
+    auto zero = [dc](B1 *g) {
+      GPUConn conn = dc->conn();
+      g->set_constant(0.0f, conn);
+    };
+    if (!scale_[r].grad().accumulate(txn, id(), dc, zero) || !shift_[r].grad().accumulate(txn, id(), dc, zero))
+      throw HazardError("SlabBatchNorm2DOp: parameter gradients already written by this node");
+    V3 &x = xs_[r].val().get(txn, id());
+    d = dims_of(x);
+    xt[n] = x.as_view().dptr();
+    dyt[n] = ys_[r].grad().get(txn, id()).as_view().dptr();
+    dxt[n] = xs_[r].grad().get_mut(txn, id()).as_view().dptr();
+    sc[n] = scale_[r].val().get(txn, id()).dptr();
+    sh[n] = shift_[r].val().get(txn, id()).dptr();
+    tm[n] = tmp_mean_[r].get(txn, id()).dptr();
+    tv[n] = tmp_variance_[r].get(txn, id()).dptr();
+    dsc[n] = scale_[r].grad().get_mut(txn, id()).dptr();
+    dsh[n] = shift_[r].grad().get_mut(txn, id()).dptr();
+    ++n;
+  }
+  if (n == 0) return;
+  GPUContext *dc = rank_ctx(ctx_, 0);
+  const size_t ws = adh_batchnorm2d_workspace_bytes(n, d.N, d.C);
+  dc->reserve_scratch(ws);
+  auto scratch = dc->get_scratch();
+  GPUConn conn = dc->conn();
+  adh_check(adh_batchnorm2d_bwd_tiles(ADH_F32, n, d.N, d.C, d.H, d.W, 0, 0, xt, dyt, sc, sh, tm, tv, dxt, dsc, dsh, 1.0f,
+                                      1.0f, scratch->dptr(), scratch->size(), conn.stream()),
+            "SlabBatchNorm2DOp::_backward");
+}
+
+// ---- CudnnActivationOp, kReluAct (op.cc:3189-3324) ----
+template <>
+void CudnnActivationOp<V3>::_forward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &x = x_.val().get(txn, id());
+  if (y_.val().overwrite(txn, id(), ctx)) {
+    GPUConn conn = ctx->conn();
+    V3 &y = y_.val().get_excl(txn, id());
+    const TileDims d = dims_of(x);
+    y.set_batch_size(d.N);
+    check_packed(x, "CudnnActivationOp");
+    adh_check(adh_relu_fwd(ADH_F32, (uint64_t)d.W * d.H * d.C * d.N, x.as_view().dptr(), y.as_view().dptr(), conn.stream()),
+              "CudnnActivationOp::_forward");
+  }
+}
+template <>
+void CudnnActivationOp<V3>::_backward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  const size_t batch = x_.val().get(txn, id()).batch_size();
+  if (x_.grad().accumulate(txn, id(), ctx, [ctx, batch](V3 *g) {
+        GPUConn conn = ctx->conn();
+        g->set_batch_size(batch);
+        g->as_view().set_constant(0.0f, conn);
+      })) {
+    GPUConn conn = ctx->conn();
+    V3 &y = y_.val().get(txn, id());
+    const TileDims d = dims_of(y);
+    adh_check(adh_relu_bwd(ADH_F32, (uint64_t)d.W * d.H * d.C * d.N, y.as_view().dptr(),
+                           y_.grad().get(txn, id()).as_view().dptr(), x_.grad().get_mut(txn, id()).as_view().dptr(), 1.0f,
+                           conn.stream()),
+              "CudnnActivationOp::_backward");
+  }
+}
+
+// ---- JoinOp<V, SumJoin> (op.cc:744-867) ----
+template <>
+void JoinOp<V3, SumJoin>::_forward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  if (y_.val().overwrite(txn, id(), ctx)) {
+    GPUConn conn = ctx->conn();
+    const void *xt[ADH_MAX_TILES];
+    TileDims d{};
+    for (size_t j = 0; j < xs_.size(); ++j) {
+      V3 &x = xs_[j].val().get(txn, id());
+      check_packed(x, "JoinOp");
+      d = dims_of(x);
+      xt[j] = x.as_view().dptr();
+    }
+    V3 &y = y_.val().get_excl(txn, id());
+    y.set_batch_size(d.N);
+    adh_check(adh_sum_fwd(ADH_F32, (uint32_t)xs_.size(), (uint64_t)d.W * d.H * d.C * d.N, xt, y.as_view().dptr(),
+                          conn.stream()),
+              "JoinOp::_forward");
+  }
+}
+template <>
+void JoinOp<V3, SumJoin>::_backward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &dy = y_.grad().get(txn, id());
+  const TileDims d = dims_of(dy);
+  const size_t batch = d.N;
+  for (size_t j = 0; j < xs_.size(); ++j) {
+    if (xs_[j].grad().accumulate(txn, id(), ctx, [ctx, batch](V3 *g) {
+          GPUConn conn = ctx->conn();
+          g->set_batch_size(batch);
+          g->as_view().set_constant(0.0f, conn);
+        })) {
+      GPUConn conn = ctx->conn();
+      V3 &dx = xs_[j].grad().get_mut(txn, id());
+      check_packed(dx, "JoinOp");
+      adh_check(adh_add_f32((uint64_t)d.W * d.H * d.C * d.N, dy.as_view().dptr(), dx.as_view().dptr(), conn.stream()),
+                "JoinOp::_backward");
+    }
+  }
+}
+
 // ---- SlabPool2DOp (op.cc:3405-3530 forward, 3532-3660 backward) ----
 template <>
 void SlabPool2DOp<V3>::_forward(TxnId txn) {

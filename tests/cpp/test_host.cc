@@ -38,6 +38,13 @@ void orc_pool_slab_fwd(int mode, uint32_t N, uint32_t C, uint32_t HP, uint32_t W
                        uint32_t sw, const float *x, float *y);
 void orc_pool_slab_bwd(int mode, uint32_t N, uint32_t C, uint32_t HP, uint32_t WP, uint32_t wh, uint32_t ww, uint32_t sh,
                        uint32_t sw, const float *x, const float *dy, float beta, float *dx);
+void orc_batchnorm2d_fwd_train(uint32_t N, uint32_t C, uint32_t H, uint32_t W, float eps, int relu, uint32_t p,
+                               const float *x, const float *scale, const float *shift, float *y, float *run_mean,
+                               float *run_var, float *save_mean, float *save_invstd);
+void orc_batchnorm2d_bwd(uint32_t N, uint32_t C, uint32_t H, uint32_t W, int relu, uint32_t p, const float *x,
+                         const float *dy, const float *scale, const float *shift, const float *save_mean,
+                         const float *save_invstd, float beta_data, float beta_param, float *dx, float *dscale,
+                         float *dshift);
 void orc_softmax_fwd(uint32_t C, uint32_t N, const float *x, float *y);
 void orc_softmax_nll_loss_fwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label, float *loss);
 void orc_softmax_nll_loss_bwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label, const float *dloss,
@@ -214,6 +221,144 @@ static void test_spatial_conv_graph(size_t K, size_t N, size_t C, size_t Co, siz
     std::printf("graph K=%zu N=%zu C=%zu->%zu %zux%zu rep %d: rel-err y %.2e dx %.2e dw %.2e\n", K, N, C, Co, H, W, rep,
                 ey, ex, ew);
     CHECK(ey <= 1e-5 && ex <= 1e-5 && ew <= 1e-5);
+  }
+}
+
+// rows [r*Ht, (r+1)*Ht) of an unsplit NCHW tensor <-> a packed tile
+static std::vector<float> tile_of(const std::vector<float> &full, size_t N, size_t C, size_t H, size_t W, size_t K, size_t r) {
+  const size_t Ht = H / K;
+  std::vector<float> t(N * C * Ht * W);
+  for (size_t nc = 0; nc < N * C; ++nc)
+    std::memcpy(&t[nc * Ht * W], &full[(nc * H + r * Ht) * W], Ht * W * sizeof(float));
+  return t;
+}
+static void put_tile(std::vector<float> &full, const std::vector<float> &t, size_t N, size_t C, size_t H, size_t W, size_t K,
+                     size_t r) {
+  const size_t Ht = H / K;
+  for (size_t nc = 0; nc < N * C; ++nc)
+    std::memcpy(&full[(nc * H + r * Ht) * W], &t[nc * Ht * W], Ht * W * sizeof(float));
+}
+
+// spatial_parallel_residual_v2_conv2d (src/zoo.cc:577-652) built with the reference's factories on K
+// row-tiles of one GPU:  x -> BN -> ReLU -> HaloPad -> HaloExch -> conv -> BN -> ReLU -> HaloPad ->
+// HaloExch -> conv -> (+ x).  Every rank's batch norm uses its own tile's statistics.  Oracle: the
+// same chain with per-tile batch norms and UNSPLIT convolutions.
+static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, size_t W) {
+  std::mt19937 gen(31337 + (unsigned)K);
+  auto ctx = MultiGPUContext::Make(K);
+  typedef GPUBatchArray3D<float> V;
+  typedef GPUArray4D<float> A;
+  typedef GPUArray1D<float> B;
+  const size_t Ht = H / K, full = N * C * H * W;
+  std::vector<float> X = uniform(gen, full, -1, 1), dY = normal(gen, full, 1.0f);
+  std::vector<float> W1 = normal(gen, C * C * 9, std::sqrt(2.0f / (C * 9))), W2 = normal(gen, C * C * 9, std::sqrt(2.0f / (C * 9)));
+  std::vector<std::vector<float>> sc0(K), sh0(K), sc1(K), sh1(K);
+  for (size_t r = 0; r < K; ++r) {
+    sc0[r] = uniform(gen, C, 0.5f, 1.5f); sh0[r] = uniform(gen, C, -0.5f, 0.5f);
+    sc1[r] = uniform(gen, C, 0.5f, 1.5f); sh1[r] = uniform(gen, C, -0.5f, 0.5f);
+  }
+  auto x_src = SrcOp<V>::Make(Shape3D(W, H, C), N, ctx->device_context(0));
+  auto w1_src = ParamOp<A>::Make(Shape4D(3, 3, C, C), ctx->device_context(0));
+  auto w2_src = ParamOp<A>::Make(Shape4D(3, 3, C, C), ctx->device_context(0));
+  vector<shared_ptr<Var<V>>> xs(K, x_src);
+  auto inputs = SpatialScatter2DOp<V>::MakeParallel(xs, ctx);
+  auto switch_var = std::make_shared<bool>(false);
+  Conv2DShape cs;
+  cs.filters = C; cs.axes = {0, 1}; cs.kernel = {3, 3}; cs.dilate = {1, 1}; cs.stride = {1, 1}; cs.pad = {1, 1};
+  cs.halo_padded_input = true; cs.enable_hmma = false;
+  auto bnorm0 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, inputs, ctx);
+  auto relu0 = parallel_relu<V>(bnorm0.ops, ctx);
+  auto pad1 = HaloPad2DOp<V>::MakeParallel(1, relu0, ctx);
+  auto exch1 = HaloExch2DOp<V>::MakeParallel(1, pad1, ctx);
+  auto conv1 = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch1, vector<shared_ptr<Var<A>>>(K, w1_src), ctx);
+  auto bnorm1 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, conv1, ctx);
+  auto relu1 = parallel_relu<V>(bnorm1.ops, ctx);
+  auto pad2 = HaloPad2DOp<V>::MakeParallel(1, relu1, ctx);
+  auto exch2 = HaloExch2DOp<V>::MakeParallel(1, pad2, ctx);
+  auto conv2 = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch2, vector<shared_ptr<Var<A>>>(K, w2_src), ctx);
+  vector<vector<shared_ptr<Var<V>>>> join_inputs{inputs, conv2};
+  auto join = parallel_sum<V>(join_inputs, ctx);
+  auto y_full = SpatialJoinedGather2DOp<V>::Make(join, ctx);
+  auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
+  sink->set_host_grad(dY.data());
+  CHECK(bnorm0.params.at(0).size() == 2 && bnorm0.grads.at(0).size() == 2);
+
+  for (int rep = 0; rep < 2; ++rep) {
+    TxnId txn;
+    x_src->load(txn, X.data());
+    w1_src->load(txn, W1.data());
+    w2_src->load(txn, W2.data());
+    for (size_t r = 0; r < K; ++r) {
+      bnorm0.scales[r]->load(txn, sc0[r].data()); bnorm0.shifts[r]->load(txn, sh0[r].data());
+      bnorm1.scales[r]->load(txn, sc1[r].data()); bnorm1.shifts[r]->load(txn, sh1[r].data());
+    }
+    sink->gradient(txn);
+    ctx->sync();
+    std::vector<float> Y(full), dX(full), dW1(W1.size()), dW2(W2.size());
+    sink->store_val(txn, Y.data());
+    x_src->store_grad(txn, dX.data());
+    w1_src->store_grad(txn, dW1.data());
+    w2_src->store_grad(txn, dW2.data());
+
+    // oracle forward
+    const float eps = 1.0e-5f;
+    std::vector<std::vector<float>> m0(K, std::vector<float>(C)), i0(K, std::vector<float>(C)), m1 = m0, i1 = i0;
+    std::vector<float> A0(full), C1(full), A1(full), C2(full), Yr(full);
+    for (size_t r = 0; r < K; ++r) {
+      auto xt = tile_of(X, N, C, H, W, K, r);
+      std::vector<float> yt(xt.size());
+      orc_batchnorm2d_fwd_train(N, C, Ht, W, eps, 1, 0, xt.data(), sc0[r].data(), sh0[r].data(), yt.data(), nullptr, nullptr,
+                                m0[r].data(), i0[r].data());
+      put_tile(A0, yt, N, C, H, W, K, r);
+    }
+    std::vector<float> A0p(N * C * (H + 2) * (W + 2)), A1p(A0p.size());
+    orc_halo_pad(0, 1, W, H, C, N, A0.data(), A0p.data());
+    orc_conv_slab_fwd(N, C, C, H, W, 3, A0p.data(), W1.data(), 0.f, C1.data());
+    for (size_t r = 0; r < K; ++r) {
+      auto xt = tile_of(C1, N, C, H, W, K, r);
+      std::vector<float> yt(xt.size());
+      orc_batchnorm2d_fwd_train(N, C, Ht, W, eps, 1, 0, xt.data(), sc1[r].data(), sh1[r].data(), yt.data(), nullptr, nullptr,
+                                m1[r].data(), i1[r].data());
+      put_tile(A1, yt, N, C, H, W, K, r);
+    }
+    orc_halo_pad(0, 1, W, H, C, N, A1.data(), A1p.data());
+    orc_conv_slab_fwd(N, C, C, H, W, 3, A1p.data(), W2.data(), 0.f, C2.data());
+    for (size_t i = 0; i < full; ++i) Yr[i] = X[i] + C2[i];
+    // oracle backward
+    std::vector<float> dA1p(A1p.size()), dA1(full), dC1(full), dA0p(A0p.size()), dA0(full), dXr(full), dW1r(W1.size()),
+        dW2r(W2.size());
+    orc_conv_slab_bwd_data(N, C, C, H, W, 3, W2.data(), dY.data(), 0.f, dA1p.data());
+    orc_conv_slab_bwd_filter(N, C, C, H, W, 3, A1p.data(), dY.data(), 0.f, dW2r.data());
+    orc_halo_unpad(0, 1, W, H, C, N, dA1p.data(), dA1.data());
+    double e_param = 0;
+    for (size_t r = 0; r < K; ++r) {
+      auto xt = tile_of(C1, N, C, H, W, K, r), dyt = tile_of(dA1, N, C, H, W, K, r);
+      std::vector<float> dxt(xt.size()), ds(C), db(C), got_ds(C), got_db(C);
+      orc_batchnorm2d_bwd(N, C, Ht, W, 1, 0, xt.data(), dyt.data(), sc1[r].data(), sh1[r].data(), m1[r].data(), i1[r].data(),
+                          0.f, 0.f, dxt.data(), ds.data(), db.data());
+      put_tile(dC1, dxt, N, C, H, W, K, r);
+      bnorm1.scales[r]->store_grad(txn, got_ds.data());
+      bnorm1.shifts[r]->store_grad(txn, got_db.data());
+      e_param = std::fmax(e_param, std::fmax(rel_err(got_ds, ds), rel_err(got_db, db)));
+    }
+    orc_conv_slab_bwd_data(N, C, C, H, W, 3, W1.data(), dC1.data(), 0.f, dA0p.data());
+    orc_conv_slab_bwd_filter(N, C, C, H, W, 3, A0p.data(), dC1.data(), 0.f, dW1r.data());
+    orc_halo_unpad(0, 1, W, H, C, N, dA0p.data(), dA0.data());
+    for (size_t r = 0; r < K; ++r) {
+      auto xt = tile_of(X, N, C, H, W, K, r), dyt = tile_of(dA0, N, C, H, W, K, r);
+      std::vector<float> dxt(xt.size()), ds(C), db(C), got_ds(C), got_db(C);
+      orc_batchnorm2d_bwd(N, C, Ht, W, 1, 0, xt.data(), dyt.data(), sc0[r].data(), sh0[r].data(), m0[r].data(), i0[r].data(),
+                          0.f, 0.f, dxt.data(), ds.data(), db.data());
+      put_tile(dXr, dxt, N, C, H, W, K, r);
+      bnorm0.scales[r]->store_grad(txn, got_ds.data());
+      bnorm0.shifts[r]->store_grad(txn, got_db.data());
+      e_param = std::fmax(e_param, std::fmax(rel_err(got_ds, ds), rel_err(got_db, db)));
+    }
+    for (size_t i = 0; i < full; ++i) dXr[i] += dY[i];
+    const double ey = rel_err(Y, Yr), ex = rel_err(dX, dXr), ew1 = rel_err(dW1, dW1r), ew2 = rel_err(dW2, dW2r);
+    std::printf("residual block K=%zu N=%zu C=%zu %zux%zu rep %d: rel-err y %.2e dx %.2e dw1 %.2e dw2 %.2e bn params %.2e\n",
+                K, N, C, H, W, rep, ey, ex, ew1, ew2, e_param);
+    CHECK(ey <= 1e-5 && ex <= 2e-5 && ew1 <= 2e-5 && ew2 <= 1e-5 && e_param <= 1e-4);
   }
 }
 
@@ -487,6 +632,8 @@ int main(int argc, char **argv) {
     test_spatial_general_conv_graph(2, 2, 8, 12, 16, 20, 3, 2, 1);   // stride-2 3x3
     test_spatial_general_conv_graph(2, 1, 8, 8, 12, 14, 3, 1, 3);    // dilation 3 over halo 3
     test_spatial_general_conv_graph(2, 2, 6, 10, 8, 9, 1, 1, 1);     // 1x1 over packed tiles (halo 0)
+    test_spatial_residual_block(4, 2, 8, 16, 12);
+    test_spatial_residual_block(2, 4, 64, 28, 28);
     test_spatial_pool_graph(kMaxPool, 4, 2, 8, 16, 12);
     test_spatial_pool_graph(kAveragePool, 2, 3, 5, 8, 10);
     test_spatial_pool_graph(kMaxPool, 4, 8, 64, 112, 112);
