@@ -447,27 +447,31 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     }
     todo.swap(rest);
   }
-  // input gradient over the WHOLE padded slab, zeroed on first touch (op.cc:1687-1691), beta = 1
+  // Input gradient over the WHOLE padded slab.  The reference zeroes it on first touch and always
+  // accumulates (beta = 1, op.cc:1687-1712); the kernel writes every element, so the first toucher of
+  // a transaction overwrites (beta = 0) instead: same values, one pass over the buffer instead of three.
   todo.clear();
+  bool fresh[ADH_MAX_TILES] = {};
   for (size_t r = 0; r < K; ++r) {
     GPUContext *dc = rank_ctx(ctx_, r);
     const size_t batch = xs_[r].val().get(txn, id()).batch_size();
-    if (xs_[r].grad().accumulate(txn, id(), dc, [dc, batch](V3 *g) {
-          GPUConn conn = dc->conn();
+    bool *first = &fresh[r];
+    if (xs_[r].grad().accumulate(txn, id(), dc, [batch, first](V3 *g) {
           g->set_batch_size(batch);
-          g->base_as_view().set_constant(0.0f, conn);
+          *first = true;
         }))
       todo.push_back(r);
   }
   while (!todo.empty()) {
     const float *w0 = kernels_[todo[0]].val().get(txn, id()).dptr();
+    const bool first = fresh[todo[0]];
     const void *dyt[ADH_MAX_TILES];
     void *dxt[ADH_MAX_TILES];
     uint32_t n = 0;
     TileDims d{};
     vector<size_t> rest;
     for (size_t r : todo) {
-      if (kernels_[r].val().get(txn, id()).dptr() != w0) {
+      if (kernels_[r].val().get(txn, id()).dptr() != w0 || fresh[r] != first) {
         rest.push_back(r);
         continue;
       }
@@ -481,15 +485,16 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
+    const float beta = first ? 0.0f : 1.0f;
     if (is_3x3_unit()) {
       adh_check(adh_conv3x3_slab_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, w0, dyt, dxt,
-                                                1.0f, nullptr, 0, conn.stream()),
+                                                beta, nullptr, 0, conn.stream()),
                 "SlabConv2DOp::_backward (data)");
     } else {
       size_t ws_bytes;
       void *ws = conv_scratch(dc, ADH_CONV_BWD_DATA, n, d, shape_, &ws_bytes);
       adh_check(adh_conv2d_slab_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
-                                               ADH_CONV_GEOMETRY(d, shape_), w0, dyt, dxt, 1.0f, ws, ws_bytes,
+                                               ADH_CONV_GEOMETRY(d, shape_), w0, dyt, dxt, beta, ws, ws_bytes,
                                                conn.stream()),
                 "SlabConv2DOp::_backward (data, general)");
     }
@@ -553,21 +558,18 @@ void SlabBatchNorm2DOp<bool, V3, B1>::_forward(TxnId txn) {
 template <>
 void SlabBatchNorm2DOp<bool, V3, B1>::_backward(TxnId txn) {
   const size_t K = xs_.size();
-  const void *xt[ADH_MAX_TILES], *dyt[ADH_MAX_TILES];
-  void *dxt[ADH_MAX_TILES];
-  const float *sc[ADH_MAX_TILES], *sh[ADH_MAX_TILES], *tm[ADH_MAX_TILES], *tv[ADH_MAX_TILES];
-  float *dsc[ADH_MAX_TILES], *dsh[ADH_MAX_TILES];
-  uint32_t n = 0;
-  TileDims d{};
+  // The first toucher of an input gradient overwrites it (the reference zeroes, then adds with beta = 1,
+  // op.cc:4026-4031, 4059-4060); parameter gradients are small and keep the zero-then-add form.
+  bool mine[ADH_MAX_TILES] = {}, fresh[ADH_MAX_TILES] = {};
   for (size_t r = 0; r < K; ++r) {
     GPUContext *dc = rank_ctx(ctx_, r);
     const size_t batch = xs_[r].val().get(txn, id()).batch_size();
-    if (!xs_[r].grad().accumulate(txn, id(), dc, [dc, batch](V3 *g) {
-          GPUConn conn = dc->conn();
-          g->set_batch_size(batch);
-          g->as_view().set_constant(0.0f, conn);
-        }))
-      continue;
+    bool *first = &fresh[r];
+    mine[r] = xs_[r].grad().accumulate(txn, id(), dc, [batch, first](V3 *g) {
+      g->set_batch_size(batch);
+      *first = true;
+    });
+    if (!mine[r]) continue;
     if (*switch_var_) throw std::logic_error("SlabBatchNorm2DOp: backward with fixed statistics is unimplemented");
     auto zero = [dc](B1 *g) {
       GPUConn conn = dc->conn();
@@ -575,28 +577,40 @@ void SlabBatchNorm2DOp<bool, V3, B1>::_backward(TxnId txn) {
     };
     if (!scale_[r].grad().accumulate(txn, id(), dc, zero) || !shift_[r].grad().accumulate(txn, id(), dc, zero))
       throw HazardError("SlabBatchNorm2DOp: parameter gradients already written by this node");
-    V3 &x = xs_[r].val().get(txn, id());
-    d = dims_of(x);
-    xt[n] = x.as_view().dptr();
-    dyt[n] = ys_[r].grad().get(txn, id()).as_view().dptr();
-    dxt[n] = xs_[r].grad().get_mut(txn, id()).as_view().dptr();
-    sc[n] = scale_[r].val().get(txn, id()).dptr();
-    sh[n] = shift_[r].val().get(txn, id()).dptr();
-    tm[n] = tmp_mean_[r].get(txn, id()).dptr();
-    tv[n] = tmp_variance_[r].get(txn, id()).dptr();
-    dsc[n] = scale_[r].grad().get_mut(txn, id()).dptr();
-    dsh[n] = shift_[r].grad().get_mut(txn, id()).dptr();
-    ++n;
   }
-  if (n == 0) return;
-  GPUContext *dc = rank_ctx(ctx_, 0);
-  const size_t ws = adh_batchnorm2d_workspace_bytes(n, d.N, d.C);
-  dc->reserve_scratch(ws);
-  auto scratch = dc->get_scratch();
-  GPUConn conn = dc->conn();
-  adh_check(adh_batchnorm2d_bwd_tiles(ADH_F32, n, d.N, d.C, d.H, d.W, 0, 0, xt, dyt, sc, sh, tm, tv, dxt, dsc, dsh, 1.0f,
-                                      1.0f, scratch->dptr(), scratch->size(), conn.stream()),
-            "SlabBatchNorm2DOp::_backward");
+  for (int pass = 0; pass < 2; ++pass) {
+    const bool first = pass == 0;
+    const void *xt[ADH_MAX_TILES], *dyt[ADH_MAX_TILES];
+    void *dxt[ADH_MAX_TILES];
+    const float *sc[ADH_MAX_TILES], *sh[ADH_MAX_TILES], *tm[ADH_MAX_TILES], *tv[ADH_MAX_TILES];
+    float *dsc[ADH_MAX_TILES], *dsh[ADH_MAX_TILES];
+    uint32_t n = 0;
+    TileDims d{};
+    for (size_t r = 0; r < K; ++r) {
+      if (!mine[r] || fresh[r] != first) continue;
+      V3 &x = xs_[r].val().get(txn, id());
+      d = dims_of(x);
+      xt[n] = x.as_view().dptr();
+      dyt[n] = ys_[r].grad().get(txn, id()).as_view().dptr();
+      dxt[n] = xs_[r].grad().get_mut(txn, id()).as_view().dptr();
+      sc[n] = scale_[r].val().get(txn, id()).dptr();
+      sh[n] = shift_[r].val().get(txn, id()).dptr();
+      tm[n] = tmp_mean_[r].get(txn, id()).dptr();
+      tv[n] = tmp_variance_[r].get(txn, id()).dptr();
+      dsc[n] = scale_[r].grad().get_mut(txn, id()).dptr();
+      dsh[n] = shift_[r].grad().get_mut(txn, id()).dptr();
+      ++n;
+    }
+    if (n == 0) continue;
+    GPUContext *dc = rank_ctx(ctx_, 0);
+    const size_t ws = adh_batchnorm2d_workspace_bytes(n, d.N, d.C);
+    dc->reserve_scratch(ws);
+    auto scratch = dc->get_scratch();
+    GPUConn conn = dc->conn();
+    adh_check(adh_batchnorm2d_bwd_tiles(ADH_F32, n, d.N, d.C, d.H, d.W, 0, 0, xt, dyt, sc, sh, tm, tv, dxt, dsc, dsh,
+                                        first ? 0.0f : 1.0f, 1.0f, scratch->dptr(), scratch->size(), conn.stream()),
+              "SlabBatchNorm2DOp::_backward");
+  }
 }
 
 // ---- CudnnActivationOp, kReluAct (op.cc:3189-3324) ----
@@ -618,17 +632,18 @@ template <>
 void CudnnActivationOp<V3>::_backward(TxnId txn) {
   GPUContext *ctx = gpu_ctx_of(ctx_);
   const size_t batch = x_.val().get(txn, id()).batch_size();
-  if (x_.grad().accumulate(txn, id(), ctx, [ctx, batch](V3 *g) {
-        GPUConn conn = ctx->conn();
+  // the first toucher of the input gradient overwrites it (the reference zeroes, then adds with beta = 1)
+  bool first = false;
+  if (x_.grad().accumulate(txn, id(), ctx, [batch, &first](V3 *g) {
         g->set_batch_size(batch);
-        g->as_view().set_constant(0.0f, conn);
+        first = true;
       })) {
     GPUConn conn = ctx->conn();
     V3 &y = y_.val().get(txn, id());
     const TileDims d = dims_of(y);
     adh_check(adh_relu_bwd(ADH_F32, (uint64_t)d.W * d.H * d.C * d.N, y.as_view().dptr(),
-                           y_.grad().get(txn, id()).as_view().dptr(), x_.grad().get_mut(txn, id()).as_view().dptr(), 1.0f,
-                           conn.stream()),
+                           y_.grad().get(txn, id()).as_view().dptr(), x_.grad().get_mut(txn, id()).as_view().dptr(),
+                           first ? 0.0f : 1.0f, conn.stream()),
               "CudnnActivationOp::_backward");
   }
 }
@@ -711,40 +726,48 @@ void SlabPool2DOp<V3>::_forward(TxnId txn) {
 template <>
 void SlabPool2DOp<V3>::_backward(TxnId txn) {
   const size_t K = xs_.size();
-  const void *xt[ADH_MAX_TILES];
-  const void *yt[ADH_MAX_TILES];
-  const void *dyt[ADH_MAX_TILES];
-  void *dxt[ADH_MAX_TILES];
-  uint32_t n = 0;
-  TileDims d{};
-  // input gradient over the WHOLE padded tile, zeroed on first touch, beta = 1 (op.cc:3540-3550)
+  // Input gradient over the WHOLE padded tile.  The reference zeroes it on first touch and accumulates
+  // (beta = 1, op.cc:3540-3550, 3610-3619); the kernel writes every element, so the first toucher of a
+  // transaction overwrites instead.
+  bool mine[ADH_MAX_TILES] = {}, fresh[ADH_MAX_TILES] = {};
   for (size_t r = 0; r < K; ++r) {
     GPUContext *dc = rank_ctx(ctx_, r);
     const size_t batch = xs_[r].val().get(txn, id()).batch_size();
-    if (!xs_[r].grad().accumulate(txn, id(), dc, [dc, batch](V3 *g) {
-          GPUConn conn = dc->conn();
-          g->set_batch_size(batch);
-          g->base_as_view().set_constant(0.0f, conn);
-        }))
-      continue;
-    V3 &x = xs_[r].val().get(txn, id());
-    V3 &dx = xs_[r].grad().get_mut(txn, id());
-    d = dims_of(x);
-    if (shape_.halo_padded_input) check_padded(dx, shape_.pad[0], "SlabPool2DOp");
-    else check_packed(dx, "SlabPool2DOp");
-    xt[n] = x.base_as_view().dptr();
-    yt[n] = ys_[r].val().get(txn, id()).as_view().dptr();
-    dyt[n] = ys_[r].grad().get(txn, id()).as_view().dptr();
-    dxt[n] = dx.base_as_view().dptr();
-    ++n;
+    bool *first = &fresh[r];
+    mine[r] = xs_[r].grad().accumulate(txn, id(), dc, [batch, first](V3 *g) {
+      g->set_batch_size(batch);
+      *first = true;
+    });
   }
-  if (n == 0) return;
-  GPUConn conn = rank_ctx(ctx_, 0)->conn();
-  adh_check(adh_pool2d_slab_bwd_tiles(ADH_F32, shape_.pooling == kMaxPool ? ADH_POOL_MAX : ADH_POOL_AVG, n, d.N, d.C,
-                                      d.H + 2 * (uint32_t)shape_.pad[1], d.W + 2 * (uint32_t)shape_.pad[0],
-                                      (uint32_t)shape_.window[1], (uint32_t)shape_.window[0], (uint32_t)shape_.stride[1],
-                                      (uint32_t)shape_.stride[0], xt, yt, dyt, dxt, 1.0f, conn.stream()),
-            "SlabPool2DOp::_backward");
+  for (int pass = 0; pass < 2; ++pass) {
+    const bool first = pass == 0;
+    const void *xt[ADH_MAX_TILES];
+    const void *yt[ADH_MAX_TILES];
+    const void *dyt[ADH_MAX_TILES];
+    void *dxt[ADH_MAX_TILES];
+    uint32_t n = 0;
+    TileDims d{};
+    for (size_t r = 0; r < K; ++r) {
+      if (!mine[r] || fresh[r] != first) continue;
+      V3 &x = xs_[r].val().get(txn, id());
+      V3 &dx = xs_[r].grad().get_mut(txn, id());
+      d = dims_of(x);
+      if (shape_.halo_padded_input) check_padded(dx, shape_.pad[0], "SlabPool2DOp");
+      else check_packed(dx, "SlabPool2DOp");
+      xt[n] = x.base_as_view().dptr();
+      yt[n] = ys_[r].val().get(txn, id()).as_view().dptr();
+      dyt[n] = ys_[r].grad().get(txn, id()).as_view().dptr();
+      dxt[n] = dx.base_as_view().dptr();
+      ++n;
+    }
+    if (n == 0) continue;
+    GPUConn conn = rank_ctx(ctx_, 0)->conn();
+    adh_check(adh_pool2d_slab_bwd_tiles(ADH_F32, shape_.pooling == kMaxPool ? ADH_POOL_MAX : ADH_POOL_AVG, n, d.N, d.C,
+                                        d.H + 2 * (uint32_t)shape_.pad[1], d.W + 2 * (uint32_t)shape_.pad[0],
+                                        (uint32_t)shape_.window[1], (uint32_t)shape_.window[0], (uint32_t)shape_.stride[1],
+                                        (uint32_t)shape_.stride[0], xt, yt, dyt, dxt, first ? 0.0f : 1.0f, conn.stream()),
+              "SlabPool2DOp::_backward");
+  }
 }
 
 // ---- SoftmaxNLLLossOp, 1-D logits (op.cc:4118-4188) ----

@@ -259,6 +259,10 @@ def main():
             lambda: lib.adh_conv3x3_slab_fwd_tiles(1, K5, N5, C, C, Ht5, W5, t5_tbl, w5.data_ptr(), y5_tbl, 0.0,
                                                    ws5.data_ptr(), ws5_bytes, stream),
             "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
+        add("conv bwd-data cfg5 (bf16, beta=0: first toucher of the gradient, what the host op issues)",
+            lambda: lib.adh_conv3x3_slab_bwd_data_tiles(1, K5, N5, C, C, Ht5, W5, w5.data_ptr(), y5_tbl, t5_tbl, 0.0,
+                                                        ws5.data_ptr(), ws5_bytes, stream),
+            "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
         add("conv bwd-data cfg5 (bf16, beta=1)",
             lambda: lib.adh_conv3x3_slab_bwd_data_tiles(1, K5, N5, C, C, Ht5, W5, w5.data_ptr(), y5_tbl, t5_tbl, 1.0,
                                                         ws5.data_ptr(), ws5_bytes, stream),
