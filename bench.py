@@ -69,6 +69,8 @@ def main():
                     help="untimed steps; a few hundred so that the GPU clocks have ramped up")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-secondary", action="store_true", help="time only the headline kernel")
+    ap.add_argument("--only", default=None,
+                    help="time only the secondary entries whose name contains this text (for profiling one kernel)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain copy of known size (1 GiB read + 1 GiB written) 10 times: the kernel "
                          "whose FETCH_SIZE / WRITE_SIZE readings calibrate the HBM traffic counters")
@@ -170,6 +172,8 @@ def main():
         flush_scratch = torch.empty(128 * 1024 * 1024, device="cuda")  # 512 MB
 
         def add(name, fn, bound, work, peak, unit, note=None, flushed=False):
+            if args.only is not None and args.only not in name:
+                return
             ms = time_gpu(fn, reps, wu)
             ach = work / (ms * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
             e = {"name": name, "ms": round(ms, 5), "bound": bound, "achieved": round(ach, 3), "peak": peak,
