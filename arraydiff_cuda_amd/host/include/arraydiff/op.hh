@@ -623,7 +623,7 @@ public:
                           input->batch_shape());
   }
   virtual void _forward(TxnId txn);
-  // the reference defines no backward for this op (SURVEY: op.cc:2872-2960 only)
+  // the reference defines no backward for this op (src/op.cc:2872-2960 holds the forward only)
   virtual void _backward(TxnId) { throw std::logic_error("HaloRepad2DOp has no backward"); }
 
 private:

@@ -91,7 +91,8 @@ def main():
     lib = capi.lib()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
-    # ---- workload: BASELINE configs[1] (conv) on the tensors of configs[0] (halo) ----
+    # ---- workload: the 3x3 slab conv forward (N=32, C=64, 4 row-tiles of 14 rows of a 56x56 image) on the tensors the halo
+    # pack / unpack entries use ----
     K, p, N, C, H, W = 4, 1, 32, 64, 56, 56
     Ht = H // K
     g = torch.Generator(device="cuda").manual_seed(0x5EED)
@@ -386,7 +387,7 @@ def main():
             oracle.halo_op(oracle.EXCH, 1, K, p, W, Ht, C, N, host_tiles)
         dt = (time.perf_counter() - t0) / reps_cpu
         out["cpu_baseline"]["halo_exchange_GBs"] = round(2 * 2 * (K - 1) * p * W * C * N * 4 / dt / 1e9, 3)
-        # configs[0]: pack (scatter + pad + exchange) and unpack (unpad + gather) of the unsplit tensor
+        # halo pack (scatter + pad + exchange) and unpack (unpad + gather) of the unsplit tensor on the host
         host_X = X.cpu().numpy()
         host_Y = np.empty_like(host_X)
         reps_cpu = 3
