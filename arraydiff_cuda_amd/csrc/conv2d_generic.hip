@@ -15,12 +15,11 @@
 // Implicit GEMM: M = 64 output channels per block, N = 256 output pixels per block (BR rows x BC columns, 16 n-tiles
 // of 16 consecutive pixels in row-major order, 4 per wave), K = (tap, channel) in groups of 4 channels for
 // v_mfma_f32_16x16x4_f32.  Per channel chunk the input patch is staged in LDS once; the filter,
-// rewritten beforehand to [m group][chunk][tap][channel][64 m] in the workspace, is staged per tap
+// rewritten beforehand to [m group][chunk][tap][channel][m] in the workspace, is staged per tap
 // group.  bf16 tensors are widened while staging and rounded when stored: the arithmetic is fp32.
 #include "adh_common.h"
 
 #include <algorithm>
-#include <vector>
 
 namespace adh {
 
@@ -90,11 +89,15 @@ __global__ __launch_bounds__(256) void conv_gen_filter_kernel(const FilterGenPar
 // CC: channels per chunk (4 or 8); MT: 16-wide m-tiles per block (1, 2 or 4).
 // The next (chunk, tap group)'s patch and filter rows are loaded into registers while the current
 // one is multiplied; they go to LDS after the barrier that ends the current one.
+// Patch and filter rows are loaded and staged between the two barriers of a (chunk, tap group); the registers they pass
+// through are dead during the multiplication, which leaves room for two workgroups per CU that hide each other's
+// staging.  (Loading the next chunk into registers during the multiplication instead takes the whole register file,
+// one workgroup per CU, and measured slower: 39 against 50 TFLOP/s on the 7x7 stem.)
 template <typename T, int CC, int MT>
 __global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenParams P) {
   constexpr uint32_t MW = 16u * MT;                         // m per block
   constexpr uint32_t WPITCH = MT == 1 ? 16u : MW + 16u;     // filter row pitch: the 4 channel groups 16 banks apart
-  constexpr int PFC = 32 / CC;                              // prefetch registers per channel plane: PP <= 256 * PFC
+  constexpr int PFC = 32 / CC;                              // staging registers per channel plane: PP <= 256 * PFC
   constexpr int WF = 6;                                     // float4 filter registers: TG * CC * MW / 4 <= 256 * WF
   constexpr uint32_t LOG2_CQ = CC == 8 ? 1u : 0u;
   extern __shared__ __align__(16) float gen_lds[];
@@ -194,28 +197,22 @@ __global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenPara
   const uint32_t ntaps_s = S.t1 - S.t0;
   if (ntaps_s > 0) {
     const uint32_t ngroups = (ntaps_s + P.TG - 1u) / P.TG;
-    load_patch(0);
-    load_filter(0, S.t0, min(P.TG, ntaps_s));
     for (uint32_t ch = 0; ch < P.nchunks; ++ch) {
       for (uint32_t gi = 0; gi < ngroups; ++gi) {
         const uint32_t tg0 = S.t0 + gi * P.TG;
         const uint32_t ntg = min(P.TG, S.t1 - tg0);
         __syncthreads();  // every wave is done with the filter rows (and, at a new chunk, the patch)
-        if (gi == 0) store_patch();
+        if (gi == 0) {
+          load_patch(ch);
+          store_patch();
+        }
+        load_filter(ch, tg0, ntg);
         store_filter(ntg);
         // lane L keeps the patch offset of tap tg0 + L
         int32_t delta_vec = 0;
         if (lane < ntg)
           delta_vec = ((int32_t)P.off_r[tg0 + lane] - S.min_r) * (int32_t)P.PCP + ((int32_t)P.off_c[tg0 + lane] - S.min_c);
         __syncthreads();
-        // registers for the next (chunk, tap group) while this one is multiplied
-        if (gi + 1u < ngroups) {
-          load_filter(ch, tg0 + P.TG, min(P.TG, S.t1 - tg0 - P.TG));
-        } else if (ch + 1u < P.nchunks) {
-          load_patch(ch + 1u);
-          load_filter(ch + 1u, S.t0, min(P.TG, ntaps_s));
-        }
-
         const uint32_t steps = ntg << LOG2_CQ;
         float a_cur[MT], b_cur[4], a_nxt[MT], b_nxt[4];
         auto fetch = [&](uint32_t step, float (&a)[MT], float (&b)[4]) {
@@ -333,7 +330,7 @@ static int gen_finish_plan(GenPlan *plan) {
     while (pp % 64u != 16u) ++pp;
     P.PP = pp;
     patch_bytes = (size_t)P.CC * P.PP * 4u;
-    // a thread prefetches 32 / CC elements of each channel plane
+    // a thread stages 32 / CC elements of each channel plane
     if (P.PP <= 256u * (32u / P.CC) && patch_bytes + (size_t)P.CC * wpitch * 4u <= kGenLdsBytes) break;
     if (P.CC == 8u) {
       P.CC = 4u;  // half the channels per chunk: twice the room per plane
@@ -345,7 +342,7 @@ static int gen_finish_plan(GenPlan *plan) {
   }
   P.nchunks = (P.C + P.CC - 1u) / P.CC;
   P.blocks_per_image = bpi;
-  // taps per group: what fits LDS, a lane per tap, and six float4 prefetch registers per thread
+  // taps per group: what fits LDS, a lane per tap, and six float4 staging registers per thread
   P.TG = (uint32_t)std::min<size_t>(std::min<uint32_t>(std::max(max_taps, 1u), 64u),
                                     (kGenLdsBytes - patch_bytes) / ((size_t)P.CC * wpitch * 4u));
   P.TG = std::min<uint32_t>(P.TG, 256u * 6u / (P.CC * MW / 4u));
@@ -485,8 +482,9 @@ static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *
 // pixels of a row per v_mfma_f32_16x16x4_f32.  A block owns (64 co, 16 ci, a group of T <= 9 taps)
 // and every PS-th unit of pixels (R output rows x OWT columns of one image); per unit it stages the dy
 // tile and the input patch in LDS, and its four waves split the unit's pixel groups, each keeping all
-// T x 4 accumulator tiles.  Every wave writes its sums in register order to the workspace; a second
-// kernel adds the 4 * PS partial sums in a fixed order (deterministic) and scatters them to KCRS.
+// T x 4 accumulator tiles.  The four waves' sums are added through LDS in wave order and written in
+// register order to the workspace; a second kernel adds the PS partial sums in a fixed order
+// (deterministic) and scatters them to KCRS.
 // ---------------------------------------------------------------------------------------------
 namespace adh {
 
@@ -505,7 +503,7 @@ struct WgradGenParams {
 };
 
 template <typename T, int TAPS>
-__global__ __launch_bounds__(kWgGenThreads) void conv_gen_wgrad_kernel(const WgradGenParams P) {
+__global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const WgradGenParams P) {
   extern __shared__ __align__(16) float gen_lds[];
   float *dyl = gen_lds;
   float *patch = gen_lds + P.dy_lds_floats;
@@ -530,8 +528,22 @@ __global__ __launch_bounds__(kWgGenThreads) void conv_gen_wgrad_kernel(const Wgr
   const uint32_t unit_pix = P.R * P.OWT, ksteps = unit_pix >> 2;
   // only the channels that exist are staged; lanes of absent channels read channel 0 and their sums are dropped
   const uint32_t planes = min(16u, P.Cin - cit * 16u);
-  const uint32_t patch_elems = planes * P.PR * P.PC, dy_elems = 64u * unit_pix;
   const uint32_t my_plane = l16 < planes ? l16 : 0u;
+  // What a thread stages is the same for every unit: the lane's pixel of the dy tile (a unit has at most 64
+  // pixels) for 16 output channels per wave, and up to four (row, column) places of every patch plane.
+  uint32_t dy_r, dy_c;
+  P.div_OWT.divmod(lane, dy_r, dy_c);
+  const bool dy_lane = lane < unit_pix;
+  constexpr int KP = 4;  // PR * PC <= 1024
+  uint32_t pr_rc[KP], pr_lds[KP];
+#pragma unroll
+  for (int k = 0; k < KP; ++k) {
+    const uint32_t e = tid + k * kWgGenThreads;
+    uint32_t r, col;
+    P.div_PC.divmod(e, r, col);
+    pr_rc[k] = e < P.PR * P.PC ? (r << 16) | col : 0xffffffffu;
+    pr_lds[k] = r * P.PCP + col;
+  }
   for (uint32_t u = ps; u < P.units; u += P.PS) {
     uint32_t r2, r3, cb, rb, n, tile;
     P.div_ncb.divmod(u, r2, cb);
@@ -541,24 +553,25 @@ __global__ __launch_bounds__(kWgGenThreads) void conv_gen_wgrad_kernel(const Wgr
     const T *ds = reinterpret_cast<const T *>(P.dy[tile]) + ((size_t)n * P.Cout + cog * 64u) * P.OH * P.OW;
     const uint32_t oh0 = rb * P.R, ow0 = cb * P.OWT;
     __syncthreads();  // every wave is done with the previous unit
-    for (uint32_t e = tid; e < dy_elems; e += kWgGenThreads) {
-      uint32_t co, pr, r, c;
-      co = e / unit_pix;
-      pr = e - co * unit_pix;
-      P.div_OWT.divmod(pr, r, c);
-      float v = 0.f;
-      if (cog * 64u + co < P.Cout && oh0 + r < P.OH && ow0 + c < P.OW)
-        v = gen_ld(ds, ((size_t)co * P.OH + oh0 + r) * P.OW + ow0 + c);
-      dyl[co * P.DP + pr] = v;
+    if (dy_lane) {
+      const bool in = oh0 + dy_r < P.OH && ow0 + dy_c < P.OW;
+      const size_t pix = (size_t)(oh0 + dy_r) * P.OW + ow0 + dy_c;
+#pragma unroll 4
+      for (uint32_t c = 0; c < 16u; ++c) {
+        const uint32_t co = wave * 16u + c;
+        float v = 0.f;
+        if (in && cog * 64u + co < P.Cout) v = gen_ld(ds, (size_t)co * P.OH * P.OW + pix);
+        dyl[co * P.DP + lane] = v;
+      }
     }
-    for (uint32_t e = tid; e < patch_elems; e += kWgGenThreads) {
-      uint32_t rc, col, c, r;
-      P.div_PC.divmod(e, rc, col);
-      P.div_PR.divmod(rc, c, r);
-      const uint32_t gr = oh0 * P.sh + r, gc = ow0 * P.sw + col;
-      float v = 0.f;
-      if (gr < P.HP && gc < P.WP) v = gen_ld(xs, ((size_t)c * P.HP + gr) * P.WP + gc);
-      patch[c * P.PP + r * P.PCP + col] = v;
+#pragma unroll
+    for (int k = 0; k < KP; ++k) {
+      if (pr_rc[k] == 0xffffffffu) continue;
+      const uint32_t gr = oh0 * P.sh + (pr_rc[k] >> 16), gc = ow0 * P.sw + (pr_rc[k] & 0xffffu);
+      const bool in = gr < P.HP && gc < P.WP;
+      const size_t pix = (size_t)gr * P.WP + gc;
+      for (uint32_t c = 0; c < planes; ++c)
+        patch[c * P.PP + pr_lds[k]] = in ? gen_ld(xs, (size_t)c * P.HP * P.WP + pix) : 0.f;
     }
     __syncthreads();
     for (uint32_t ks = wave; ks < ksteps; ks += 4u) {
@@ -579,15 +592,32 @@ __global__ __launch_bounds__(kWgGenThreads) void conv_gen_wgrad_kernel(const Wgr
           acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[mt], b[t], acc[t][mt], 0, 0, 0);
     }
   }
-  // partial[(ps * 4 + wave)][cog][cit][tg][t][mt][lane][4]
-  const size_t block_part = ((size_t)(cog * P.CIT + cit) * P.ntg + tg) * TAPS * 1024u;
-  const size_t stride = (size_t)P.COG * P.CIT * P.ntg * TAPS * 1024u;
-  float *dstp = P.partial + (size_t)(ps * 4u + wave) * stride + block_part;
+  // the four waves' sums are added in wave order through LDS (deterministic), then written once:
+  // partial[ps][cog][cit][tg][t][mt][lane][4]
+  floatx4 *red = reinterpret_cast<floatx4 *>(gen_lds);
+  for (uint32_t w = 0; w < 4u; ++w) {
+    __syncthreads();  // w = 0: every wave is done with the staged tiles
+    if (wave == w) {
 #pragma unroll
-  for (int t = 0; t < TAPS; ++t)
+      for (int t = 0; t < TAPS; ++t)
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
-      *reinterpret_cast<floatx4 *>(dstp + (t * 4 + mt) * 256 + lane * 4u) = acc[t][mt];
+        for (int mt = 0; mt < 4; ++mt) {
+          floatx4 &slot = red[(t * 4 + mt) * 64 + lane];
+          if (w > 0) acc[t][mt] += slot;
+          if (w < 3u) slot = acc[t][mt];
+        }
+    }
+  }
+  if (wave == 3u) {
+    const size_t block_part = ((size_t)(cog * P.CIT + cit) * P.ntg + tg) * TAPS * 1024u;
+    const size_t stride = (size_t)P.COG * P.CIT * P.ntg * TAPS * 1024u;
+    float *dstp = P.partial + (size_t)ps * stride + block_part;
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t)
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+        *reinterpret_cast<floatx4 *>(dstp + (t * 4 + mt) * 256 + lane * 4u) = acc[t][mt];
+  }
 }
 
 struct WgradGenReduceParams {
@@ -650,8 +680,8 @@ static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *p
     while (dp % 64u != 4u) ++dp;
     P.DP = dp;
     P.dy_lds_floats = 64u * P.DP;
-    plan->lds_bytes = ((size_t)P.dy_lds_floats + 16u * (size_t)P.PP) * 4u;
-    if (plan->lds_bytes <= kGenLdsBytes) break;
+    plan->lds_bytes = std::max<size_t>(((size_t)P.dy_lds_floats + 16u * (size_t)P.PP) * 4u, (size_t)P.T * 4096u);
+    if (plan->lds_bytes <= kGenLdsBytes && P.PR * P.PC <= 1024u) break;  // a thread stages up to four places per plane
     if (P.R > 1u) P.R /= 2u;
     else if (P.OWT > 4u) P.OWT = ((P.OWT / 2u) + 3u) & ~3u;
     else return ADH_EUNIMPL;
@@ -663,12 +693,12 @@ static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *p
   P.units = (uint32_t)units;
   const uint64_t fixed = (uint64_t)P.COG * P.CIT * P.ntg;
   const size_t stride_bytes = (size_t)fixed * P.T * 1024u * 4u;
-  uint64_t ps = std::max<uint64_t>(1u, 1024u / fixed);
+  uint64_t ps = std::max<uint64_t>(1u, 1024u / fixed);  // about four workgroups per CU: they hide each other's staging
   ps = std::min<uint64_t>(ps, units);
-  while (ps > 1u && ps * 4u * stride_bytes > (256ull << 20)) ps /= 2u;
+  while (ps > 1u && ps * stride_bytes > (256ull << 20)) ps /= 2u;
   if (fixed * ps >= (1ull << 24)) return ADH_EINVAL;
   P.PS = (uint32_t)ps;
-  plan->nparts = P.PS * 4u;
+  plan->nparts = P.PS;
   plan->blocks = (uint32_t)(fixed * ps);
   plan->partial_bytes = (size_t)plan->nparts * stride_bytes;
   P.div_COG = FastDiv(P.COG); P.div_CIT = FastDiv(P.CIT); P.div_ntg = FastDiv(P.ntg);
