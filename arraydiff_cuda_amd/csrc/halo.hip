@@ -216,7 +216,8 @@ struct StripParams {
   FastDiv div_run;
 };
 
-template <typename T, bool ADD, bool COLUMNS>
+// VEC elements per thread (row strips only): 16-byte accesses, which need no alignment beyond the element's.
+template <typename T, bool ADD, bool COLUMNS, int VEC>
 __global__ __launch_bounds__(kBlock) void halo_strip_kernel(const StripParams P) {
   const uint32_t idx = blockIdx.x * kBlock + threadIdx.x;
   if (idx >= P.total) return;
@@ -226,7 +227,8 @@ __global__ __launch_bounds__(kBlock) void halo_strip_kernel(const StripParams P)
   const int32_t dpos = job.dst_pos + P.inc[pair] * delta;
   const int32_t spos = job.src_pos + P.inc[pair] * delta;
   uint32_t cn, i;
-  P.div_run.divmod(idx, cn, i);
+  P.div_run.divmod(idx, cn, i);  // run is counted in groups of VEC elements
+  i *= (uint32_t)VEC;
   const uint64_t plane = (uint64_t)cn * P.PW * P.PH;
   uint64_t so, dof;
   if (COLUMNS) {
@@ -239,10 +241,21 @@ __global__ __launch_bounds__(kBlock) void halo_strip_kernel(const StripParams P)
   }
   const T *s = reinterpret_cast<const T *>(P.tiles[job.src_tile]) + so;
   T *d = reinterpret_cast<T *>(P.tiles[job.dst_tile]) + dof;
-  if (ADD)
-    *d = elem_add(*d, *s);
-  else
-    *d = *s;
+  if (VEC == 1) {
+    if (ADD)
+      *d = elem_add(*d, *s);
+    else
+      *d = *s;
+  } else {
+    struct __attribute__((packed, aligned(sizeof(T)))) Vec { T v[VEC]; };
+    Vec a = *reinterpret_cast<const Vec *>(s);
+    if (ADD) {
+      const Vec b = *reinterpret_cast<const Vec *>(d);
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) a.v[k] = elem_add(b.v[k], a.v[k]);
+    }
+    *reinterpret_cast<Vec *>(d) = a;
+  }
 }
 
 // rank == UINT32_MAX: all ranks.
@@ -293,18 +306,24 @@ static int halo_op(bool reduce, int dtype, uint32_t grid_w, uint32_t grid_h, uin
   P.halo_pad = p;
   P.W = W; P.H = H; P.PW = W + 2 * p; P.PH = H + 2 * p;
   P.run = columns ? H : W;
-  P.total = (uint32_t)total;
+  // row strips whose length is a whole number of 16-byte groups move 16 bytes per thread
+  const uint32_t vec = (uint32_t)(16 / dtype_size(dtype));
+  const bool wide = !columns && W % vec == 0;
+  if (wide) P.run = W / vec;
+  P.total = (uint32_t)(wide ? total / vec : total);
   P.div_run = FastDiv(P.run);
   dim3 grid((P.total + kBlock - 1) / kBlock, np * p, 1);
   if (grid.y > 65535u) return ADH_EINVAL;
-#define ADH_LAUNCH_STRIP(T, ADD, COL) \
-  hipLaunchKernelGGL((halo_strip_kernel<T, ADD, COL>), grid, dim3(kBlock), 0, st, P)
+#define ADH_LAUNCH_STRIP(T, ADD, COL, V) \
+  hipLaunchKernelGGL((halo_strip_kernel<T, ADD, COL, V>), grid, dim3(kBlock), 0, st, P)
   if (dtype == ADH_F32) {
-    if (reduce) { if (columns) ADH_LAUNCH_STRIP(float, true, true); else ADH_LAUNCH_STRIP(float, true, false); }
-    else        { if (columns) ADH_LAUNCH_STRIP(float, false, true); else ADH_LAUNCH_STRIP(float, false, false); }
+    if (columns) { if (reduce) ADH_LAUNCH_STRIP(float, true, true, 1); else ADH_LAUNCH_STRIP(float, false, true, 1); }
+    else if (wide) { if (reduce) ADH_LAUNCH_STRIP(float, true, false, 4); else ADH_LAUNCH_STRIP(float, false, false, 4); }
+    else { if (reduce) ADH_LAUNCH_STRIP(float, true, false, 1); else ADH_LAUNCH_STRIP(float, false, false, 1); }
   } else {
-    if (reduce) { if (columns) ADH_LAUNCH_STRIP(uint16_t, true, true); else ADH_LAUNCH_STRIP(uint16_t, true, false); }
-    else        { if (columns) ADH_LAUNCH_STRIP(uint16_t, false, true); else ADH_LAUNCH_STRIP(uint16_t, false, false); }
+    if (columns) { if (reduce) ADH_LAUNCH_STRIP(uint16_t, true, true, 1); else ADH_LAUNCH_STRIP(uint16_t, false, true, 1); }
+    else if (wide) { if (reduce) ADH_LAUNCH_STRIP(uint16_t, true, false, 8); else ADH_LAUNCH_STRIP(uint16_t, false, false, 8); }
+    else { if (reduce) ADH_LAUNCH_STRIP(uint16_t, true, false, 1); else ADH_LAUNCH_STRIP(uint16_t, false, false, 1); }
   }
 #undef ADH_LAUNCH_STRIP
   return launch_status();
