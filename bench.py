@@ -61,6 +61,32 @@ def time_gpu_flushed(fn, reps, scratch):
     return max(min(both) - min(alone), 1e-6)
 
 
+def time_gpu_graph(fn, per_graph=50, replays=10):
+    """Average milliseconds per call of fn() when `per_graph` calls are captured into one HIP graph and the
+    graph is replayed: the device-side time of a launch-bound loop, without the host's launch cost."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(per_graph):
+            fn()
+    graph.replay()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (replays * per_graph)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -172,7 +198,8 @@ def main():
 
         flush_scratch = torch.empty(128 * 1024 * 1024, device="cuda")  # 512 MB
 
-        def add(name, fn, bound, work, peak, unit, note=None, flushed=False):
+        def add(name, fn, bound, work, peak, unit, note=None, flushed=False, graph=False):
+            nonlocal stream
             if args.only is not None and args.only not in name:
                 return
             ms = time_gpu(fn, reps, wu)
@@ -187,6 +214,22 @@ def main():
                 e["ms_flushed"] = round(msf, 5)
                 e["achieved_flushed"] = round(achf, 3)
                 e["frac_flushed"] = round(achf / peak, 4)
+            if graph:
+                # launch-sized kernels: 50 launches captured into one HIP graph, replayed (the launches then come from
+                # the device's queue, not from this interpreter)
+                saved = stream
+
+                def fn_on_current_stream():
+                    nonlocal stream
+                    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                    fn()
+
+                msg = time_gpu_graph(fn_on_current_stream)
+                stream = saved
+                achg = work / (msg * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
+                e["ms_in_graph"] = round(msg, 5)
+                e["achieved_in_graph"] = round(achg, 3)
+                e["frac_in_graph"] = round(achg / peak, 4)
             if note:
                 e["note"] = note
             sec.append(e)
@@ -195,17 +238,17 @@ def main():
         padded_b = K * N * C * (Ht + 2 * p) * (W + 2 * p) * es
         add("halo pack cfg1 (unsplit -> 4 padded tiles)",
             lambda: lib.adh_tiles_pack_nchw(0, K, p, W, H, C, N, X.data_ptr(), tile_tbl, stream),
-            "hbm", unsplit_b + padded_b, HBM_PEAK_GBS, "GB/s", flushed=True)
+            "hbm", unsplit_b + padded_b, HBM_PEAK_GBS, "GB/s", flushed=True, graph=True)
         add("halo unpack cfg1 (4 padded tiles -> unsplit)",
             lambda: lib.adh_tiles_unpack_nchw(0, K, p, W, H, C, N, tile_tbl, Y.data_ptr(), stream),
-            "hbm", 2 * unsplit_b, HBM_PEAK_GBS, "GB/s", flushed=True)
+            "hbm", 2 * unsplit_b, HBM_PEAK_GBS, "GB/s", flushed=True, graph=True)
         add("halo exchange cfg1 (6 strips)",
             lambda: lib.adh_halo_exchange_nchw(0, 1, K, p, W, Ht, C, N, tile_tbl, stream),
             "hbm", 2 * 2 * (K - 1) * strip, HBM_PEAK_GBS, "GB/s",
-            note="reference figure of merit p*W*C*N*4/t = %d B / t" % strip)
+            note="reference figure of merit p*W*C*N*4/t = %d B / t" % strip, graph=True)
         add("halo reduce cfg1 (6 strips)",
             lambda: lib.adh_halo_reduce_nchw(0, 1, K, p, W, Ht, C, N, g_tbl, stream),
-            "hbm", 3 * 2 * (K - 1) * strip, HBM_PEAK_GBS, "GB/s")
+            "hbm", 3 * 2 * (K - 1) * strip, HBM_PEAK_GBS, "GB/s", graph=True)
         sl = torch.empty((N, 32, H, W), device="cuda")
         add("channel slice [16,48) cfg4",
             lambda: lib.adh_slice_copy_nchw(0, W, H, 32, N, X.data_ptr(), W, H, C, 0, 0, 16, sl.data_ptr(), W, H, 32,
@@ -221,11 +264,11 @@ def main():
         add("softmax + nll fwd cfg4 (256x1000)",
             lambda: lib.adh_softmax_xent_fwd(Cs, Ns, logits.data_ptr(), labels.data_ptr(), sy.data_ptr(),
                                              sloss.data_ptr(), stream),
-            "hbm", 2 * Ns * Cs * 4 + 8 * Ns, HBM_PEAK_GBS, "GB/s", flushed=True)
+            "hbm", 2 * Ns * Cs * 4 + 8 * Ns, HBM_PEAK_GBS, "GB/s", flushed=True, graph=True)
         add("softmax-nll bwd cfg4 (256x1000)",
             lambda: lib.adh_softmax_nll_loss_bwd(Cs, Ns, sy.data_ptr(), labels.data_ptr(), dl.data_ptr(),
                                                  sdx.data_ptr(), stream),
-            "hbm", 3 * Ns * Cs * 4 + 8 * Ns, HBM_PEAK_GBS, "GB/s")
+            "hbm", 3 * Ns * Cs * 4 + 8 * Ns, HBM_PEAK_GBS, "GB/s", graph=True)
         add("conv bwd-data cfg3 (4 tiles)",
             lambda: lib.adh_conv3x3_slab_bwd_data_tiles(0, K, N, C, C, Ht, W, wt.data_ptr(), dy_tbl, g_tbl, 0.0, None,
                                                         0, stream),
