@@ -37,16 +37,26 @@ struct BnParams {
   float *o3[ADH_MAX_TILES];               // forward: saved 1/sqrt(var + eps)
   float *partial;                         // [tile][c][split][2]
   float *coef;                            // [tile][c][8]
-  uint32_t N, C, H, W, HW, p, split, n_per_split, tiles;
+  uint32_t N, C, H, W, HW, p, split, n_per_split, tiles, groups_per_plane;
   float eps, beta;
   int relu;
-  FastDiv div_C, div_split, div_cols;  // div_cols: row length of the index that a kernel splits into (row, column)
+  FastDiv div_C, div_N, div_split, div_cols;  // div_cols: row length of the index that a kernel splits into (row, column)
 };
 
 __device__ __forceinline__ float bn_ld(const float *p, size_t i) { return p[i]; }
 __device__ __forceinline__ float bn_ld(const uint16_t *p, size_t i) { return bf16_bits_to_f32(p[i]); }
 __device__ __forceinline__ void bn_st(float *p, size_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void bn_st(uint16_t *p, size_t i, float v) { p[i] = f32_to_bf16_bits(v); }
+
+// VEC elements moved by one 16-byte access at element alignment (gfx950 takes unaligned vector accesses)
+template <typename T, int VEC>
+struct __attribute__((packed, aligned(sizeof(T)))) BnVec {
+  T v[VEC];
+};
+__device__ __forceinline__ float bn_f(float v) { return v; }
+__device__ __forceinline__ float bn_f(uint16_t v) { return bf16_bits_to_f32(v); }
+__device__ __forceinline__ void bn_t(float &d, float v) { d = v; }
+__device__ __forceinline__ void bn_t(uint16_t &d, float v) { d = f32_to_bf16_bits(v); }
 
 __device__ __forceinline__ float2 block_sum2(float a, float b) {
   __shared__ float red[2][kBnThreads / 64];
@@ -69,22 +79,29 @@ __device__ __forceinline__ float2 block_sum2(float a, float b) {
 
 // grid: tiles * C * split.  BWD = false: sums of (x - K), (x - K)^2.  BWD = true: sums of dy', dy' * (x - mean)
 // (dy' = dy where a*(x - mean) + shift > 0 when the rectifier was fused, else dy), dy at the interior of a tile padded by p.
-template <typename T, bool BWD>
+// VEC > 1: H*W (and, backward, W) are whole numbers of VEC-element groups, one 16-byte access per group.
+template <typename T, bool BWD, int VEC>
 __global__ __launch_bounds__(kBnThreads) void bn_reduce_kernel(const BnParams P) {
+  typedef BnVec<T, VEC> Vec;
   uint32_t tc, sp, tile, c;
   P.div_split.divmod(blockIdx.x, tc, sp);
   P.div_C.divmod(tc, tile, c);
   const T *x = reinterpret_cast<const T *>(P.x[tile]);
   const uint32_t n0 = sp * P.n_per_split, n1 = min(P.N, n0 + P.n_per_split);
+  const uint32_t groups = P.HW / (uint32_t)VEC;
   float s1 = 0.f, s2 = 0.f;
   if (!BWD) {
     const float K = bn_ld(x, (size_t)c * P.HW);
     for (uint32_t n = n0; n < n1; ++n) {
       const T *pl = x + ((size_t)n * P.C + c) * P.HW;
-      for (uint32_t i = threadIdx.x; i < P.HW; i += kBnThreads) {
-        const float v = bn_ld(pl, i) - K;
-        s1 += v;
-        s2 += v * v;
+      for (uint32_t i = threadIdx.x; i < groups; i += kBnThreads) {
+        const Vec xv = *reinterpret_cast<const Vec *>(pl + (size_t)i * VEC);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+          const float v = bn_f(xv.v[k]) - K;
+          s1 += v;
+          s2 += v * v;
+        }
       }
     }
   } else {
@@ -96,14 +113,19 @@ __global__ __launch_bounds__(kBnThreads) void bn_reduce_kernel(const BnParams P)
     for (uint32_t n = n0; n < n1; ++n) {
       const T *pl = x + ((size_t)n * P.C + c) * P.HW;
       const T *dl = dy + ((size_t)n * P.C + c) * HPp * WP + (size_t)P.p * WP + P.p;
-      for (uint32_t i = threadIdx.x; i < P.HW; i += kBnThreads) {
+      for (uint32_t i = threadIdx.x; i < groups; i += kBnThreads) {
         uint32_t h, w;
-        P.div_cols.divmod(i, h, w);
-        const float xv = bn_ld(pl, i);
-        float d = bn_ld(dl, (size_t)h * WP + w);
-        if (P.relu && !(a * (xv - mean) + b > 0.f)) d = 0.f;
-        s1 += d;
-        s2 += d * (xv - mean);
+        P.div_cols.divmod(i, h, w);  // groups per row
+        const Vec xv = *reinterpret_cast<const Vec *>(pl + (size_t)i * VEC);
+        const Vec dv = *reinterpret_cast<const Vec *>(dl + (size_t)h * WP + w * VEC);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+          const float xc = bn_f(xv.v[k]) - mean;
+          float d = bn_f(dv.v[k]);
+          if (P.relu && !(a * xc + b > 0.f)) d = 0.f;
+          s1 += d;
+          s2 += d * xc;
+        }
       }
     }
   }
@@ -177,43 +199,116 @@ __global__ __launch_bounds__(256) void bn_finalize_bwd_kernel(const BnParams P) 
   P.coef[(size_t)tc * 8u + 4u] = P.shift[tile][c];  // the rectifier's mask needs the forward output's sign
 }
 
-// grid: (tiles * N * C planes, bands of the padded output plane); one thread per padded output element
-template <typename T, bool BWD>
+// a thread moves VEC consecutive elements of the padded output
+// plane (forward: any shape, the last partial group element by element) or of the packed gradient plane (backward:
+// VEC > 1 needs H*W and W to be whole numbers of groups)
+template <typename T, bool BWD, int VEC>
 __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const BnParams P) {
-  uint32_t tn, c, tile, n;
-  P.div_C.divmod(blockIdx.x, tn, c);
-  tile = tn / P.N;
-  n = tn - tile * P.N;
+  typedef BnVec<T, VEC> Vec;
+  constexpr int U = 4;  // planes per workgroup: a thread moves the same group of each, all loads before the first store
   const uint32_t WP = P.W + 2u * P.p, HPp = P.H + 2u * P.p;
-  const float *cf = P.coef + ((size_t)tile * P.C + c) * 8u;
-  const T *x = reinterpret_cast<const T *>(P.x[tile]) + ((size_t)n * P.C + c) * P.HW;
+  const uint32_t total = HPp * WP;
+  const uint32_t planes = P.tiles * P.N * P.C;
+  const uint32_t gi = blockIdx.y * kBnThreads + threadIdx.x;  // group of VEC elements within a plane
+  if (gi >= P.groups_per_plane) return;
+  // where the group sits is the same for every plane
+  uint32_t r = 0, col = 0, in_off = 0, mask = 0;
+  bool whole = false;
   if (!BWD) {
-    const float a = cf[0], mean = cf[1], b = cf[2];
-    T *y = reinterpret_cast<T *>(P.out[tile]) + ((size_t)n * P.C + c) * HPp * WP;
-    const uint32_t total = HPp * WP;
-    for (uint32_t o = blockIdx.y * kBnThreads + threadIdx.x; o < total; o += gridDim.y * kBnThreads) {
-      uint32_t r, col;
-      P.div_cols.divmod(o, r, col);
-      float v = 0.f;
-      if (r - P.p < P.H && col - P.p < P.W) {
-        v = a * (bn_ld(x, (size_t)(r - P.p) * P.W + (col - P.p)) - mean) + b;
-        if (P.relu) v = v > 0.f ? v : 0.f;
+    P.div_cols.divmod(gi * VEC, r, col);
+    whole = VEC > 1 && r - P.p < P.H && col >= P.p && col + VEC <= P.p + P.W;  // inside one interior row
+    in_off = (r - P.p) * P.W + (col - P.p);
+    if (!whole) {
+      uint32_t rr = r, cc = col;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        if (rr - P.p < P.H && cc - P.p < P.W) mask |= 1u << k;
+        if (++cc == WP) {
+          cc = 0;
+          ++rr;
+        }
       }
-      bn_st(y, o, v);
+    } else {
+      mask = (1u << VEC) - 1u;
     }
   } else {
-    const float k1 = cf[0], k2 = cf[1], k3 = cf[2], mean = cf[3], b = cf[4];
-    const T *dy = reinterpret_cast<const T *>(P.dy[tile]) + ((size_t)n * P.C + c) * HPp * WP + (size_t)P.p * WP + P.p;
-    T *dx = reinterpret_cast<T *>(P.out[tile]) + ((size_t)n * P.C + c) * P.HW;
-    for (uint32_t i = blockIdx.y * kBnThreads + threadIdx.x; i < P.HW; i += gridDim.y * kBnThreads) {
-      uint32_t h, w;
-      P.div_cols.divmod(i, h, w);
-      const float xc = bn_ld(x, i) - mean;
-      float d = bn_ld(dy, (size_t)h * WP + w);
-      if (P.relu && !(k1 * xc + b > 0.f)) d = 0.f;
-      float g = k1 * d + k2 * xc + k3;
-      if (P.beta != 0.f) g += bn_ld(dx, i);
-      bn_st(dx, i, g);
+    uint32_t h, w;
+    P.div_cols.divmod(gi, h, w);  // groups per row
+    in_off = h * WP + w * VEC;     // within the interior of the padded gradient plane
+  }
+  Vec xv[U], dv[U], old[U];
+  const float *cf_u[U];
+  T *out_u[U];
+  bool live[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const uint32_t pl = blockIdx.x * U + u;
+    live[u] = pl < planes;
+    if (!live[u]) continue;
+    uint32_t tn, c, tile, n;
+    P.div_C.divmod(pl, tn, c);
+    P.div_N.divmod(tn, tile, n);
+    cf_u[u] = P.coef + ((size_t)tile * P.C + c) * 8u;
+    const T *x = reinterpret_cast<const T *>(P.x[tile]) + ((size_t)n * P.C + c) * P.HW;
+    if (!BWD) {
+      out_u[u] = reinterpret_cast<T *>(P.out[tile]) + ((size_t)n * P.C + c) * total;
+      if (whole) {
+        xv[u] = *reinterpret_cast<const Vec *>(x + in_off);
+      } else {
+        uint32_t rr = r, cc = col;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+          if (mask >> k & 1u) xv[u].v[k] = x[(size_t)(rr - P.p) * P.W + (cc - P.p)];
+          if (++cc == WP) {
+            cc = 0;
+            ++rr;
+          }
+        }
+      }
+    } else {
+      const T *dy = reinterpret_cast<const T *>(P.dy[tile]) + ((size_t)n * P.C + c) * total + (size_t)P.p * WP + P.p;
+      out_u[u] = reinterpret_cast<T *>(P.out[tile]) + ((size_t)n * P.C + c) * P.HW;
+      xv[u] = *reinterpret_cast<const Vec *>(x + (size_t)gi * VEC);
+      dv[u] = *reinterpret_cast<const Vec *>(dy + in_off);
+      if (P.beta != 0.f) old[u] = *reinterpret_cast<const Vec *>(out_u[u] + (size_t)gi * VEC);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (!live[u]) continue;
+    const float *cf = cf_u[u];
+    Vec out;
+    if (!BWD) {
+      const float a = cf[0], mean = cf[1], b = cf[2];
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        float v = 0.f;
+        if (mask >> k & 1u) {
+          v = a * (bn_f(xv[u].v[k]) - mean) + b;
+          if (P.relu) v = v > 0.f ? v : 0.f;
+        }
+        bn_t(out.v[k], v);
+      }
+      const uint32_t o = gi * VEC;
+      if (o + VEC <= total) {
+        *reinterpret_cast<Vec *>(out_u[u] + o) = out;
+      } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k)
+          if (o + k < total) out_u[u][o + k] = out.v[k];
+      }
+    } else {
+      const float k1 = cf[0], k2 = cf[1], k3 = cf[2], mean = cf[3], b = cf[4];
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        const float xc = bn_f(xv[u].v[k]) - mean;
+        float d = bn_f(dv[u].v[k]);
+        if (P.relu && !(k1 * xc + b > 0.f)) d = 0.f;
+        float g = k1 * d + k2 * xc + k3;
+        if (P.beta != 0.f) g += bn_f(old[u].v[k]);
+        bn_t(out.v[k], g);
+      }
+      *reinterpret_cast<Vec *>(out_u[u] + (size_t)gi * VEC) = out;
     }
   }
 }
@@ -279,11 +374,12 @@ static int bn_common(int dtype, uint32_t num_tiles, uint32_t N, uint32_t C, uint
   return ADH_OK;
 }
 
-static dim3 bn_apply_grid(const BnParams &P, uint32_t plane_elems) {
-  const uint64_t planes = (uint64_t)P.tiles * P.N * P.C;
-  uint32_t bands = (plane_elems + kBnThreads * 4u - 1u) / (kBnThreads * 4u);  // about 4 elements per thread
-  while (bands > 1u && planes * bands > (1ull << 22)) bands /= 2u;
-  return dim3((uint32_t)planes, std::min(std::max(bands, 1u), 65535u));
+// sets the apply kernel's work split and returns its grid: x = groups of four planes, y = bands of 256 groups of a plane
+static dim3 bn_apply_grid(BnParams *P, uint32_t groups_per_plane) {
+  P->groups_per_plane = groups_per_plane;
+  P->div_N = FastDiv(P->N);
+  const uint64_t planes = (uint64_t)P->tiles * P->N * P->C;
+  return dim3((uint32_t)((planes + 3u) / 4u), (groups_per_plane + kBnThreads - 1u) / kBnThreads);
 }
 
 }  // namespace adh
@@ -335,20 +431,26 @@ int adh_batchnorm2d_fwd_tiles(int dtype, int training, uint32_t num_tiles, uint3
   P.div_cols = FastDiv(W + 2u * out_halo);  // the apply kernel walks the padded output plane
   hipStream_t st = as_stream(stream);
   const uint32_t tc = num_tiles * C, fin_blocks = (tc + 255u) / 256u;
+  const uint32_t vec = (uint32_t)(16 / dtype_size(dtype));
+  const bool wide = (H * W) % vec == 0;  // the statistics pass reads whole 16-byte groups
+  const uint32_t gpp = ((H + 2u * out_halo) * (W + 2u * out_halo) + vec - 1u) / vec;
+  if ((gpp + kBnThreads - 1u) / kBnThreads > 65535u) return ADH_EINVAL;  // grid.y
   if (training) {
     if (dtype == ADH_F32) {
-      hipLaunchKernelGGL((bn_reduce_kernel<float, false>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
+      if (wide) hipLaunchKernelGGL((bn_reduce_kernel<float, false, 4>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
+      else hipLaunchKernelGGL((bn_reduce_kernel<float, false, 1>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
       hipLaunchKernelGGL(bn_finalize_fwd_kernel<float>, dim3(fin_blocks), dim3(256), 0, st, P);
     } else {
-      hipLaunchKernelGGL((bn_reduce_kernel<uint16_t, false>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
+      if (wide) hipLaunchKernelGGL((bn_reduce_kernel<uint16_t, false, 8>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
+      else hipLaunchKernelGGL((bn_reduce_kernel<uint16_t, false, 1>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
       hipLaunchKernelGGL(bn_finalize_fwd_kernel<uint16_t>, dim3(fin_blocks), dim3(256), 0, st, P);
     }
   } else {
     hipLaunchKernelGGL(bn_coef_infer_kernel, dim3(fin_blocks), dim3(256), 0, st, P);
   }
-  const dim3 grid = bn_apply_grid(P, (H + 2u * out_halo) * (W + 2u * out_halo));
-  if (dtype == ADH_F32) hipLaunchKernelGGL((bn_apply_kernel<float, false>), grid, dim3(kBnThreads), 0, st, P);
-  else hipLaunchKernelGGL((bn_apply_kernel<uint16_t, false>), grid, dim3(kBnThreads), 0, st, P);
+  const dim3 grid = bn_apply_grid(&P, gpp);
+  if (dtype == ADH_F32) hipLaunchKernelGGL((bn_apply_kernel<float, false, 4>), grid, dim3(kBnThreads), 0, st, P);
+  else hipLaunchKernelGGL((bn_apply_kernel<uint16_t, false, 8>), grid, dim3(kBnThreads), 0, st, P);
   return launch_status();
 }
 
@@ -385,17 +487,31 @@ int adh_batchnorm2d_bwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_
     P.o1[t] = dshift_tiles[t];
   }
   P.relu = relu ? 1 : 0;
-  P.div_cols = FastDiv(W);  // the reduce and apply kernels walk the packed plane
+  // the reduce and apply kernels walk the packed plane in groups of `vec` elements when rows are whole groups
+  const uint32_t vec = (uint32_t)(16 / dtype_size(dtype));
+  const bool wide = W % vec == 0;
+  P.div_cols = FastDiv(wide ? W / vec : W);
   hipStream_t st = as_stream(stream);
   const uint32_t tc = num_tiles * C, fin_blocks = (tc + 255u) / 256u;
+  if (((wide ? H * W / vec : H * W) + kBnThreads - 1u) / kBnThreads > 65535u) return ADH_EINVAL;  // grid.y
+  const dim3 rgrid(tc * P.split), agrid = bn_apply_grid(&P, wide ? H * W / vec : H * W);
   P.beta = beta_param;
-  if (dtype == ADH_F32) hipLaunchKernelGGL((bn_reduce_kernel<float, true>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
-  else hipLaunchKernelGGL((bn_reduce_kernel<uint16_t, true>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
+  if (dtype == ADH_F32) {
+    if (wide) hipLaunchKernelGGL((bn_reduce_kernel<float, true, 4>), rgrid, dim3(kBnThreads), 0, st, P);
+    else hipLaunchKernelGGL((bn_reduce_kernel<float, true, 1>), rgrid, dim3(kBnThreads), 0, st, P);
+  } else {
+    if (wide) hipLaunchKernelGGL((bn_reduce_kernel<uint16_t, true, 8>), rgrid, dim3(kBnThreads), 0, st, P);
+    else hipLaunchKernelGGL((bn_reduce_kernel<uint16_t, true, 1>), rgrid, dim3(kBnThreads), 0, st, P);
+  }
   hipLaunchKernelGGL(bn_finalize_bwd_kernel, dim3(fin_blocks), dim3(256), 0, st, P);
   P.beta = beta_data;
-  const dim3 grid = bn_apply_grid(P, H * W);
-  if (dtype == ADH_F32) hipLaunchKernelGGL((bn_apply_kernel<float, true>), grid, dim3(kBnThreads), 0, st, P);
-  else hipLaunchKernelGGL((bn_apply_kernel<uint16_t, true>), grid, dim3(kBnThreads), 0, st, P);
+  if (dtype == ADH_F32) {
+    if (wide) hipLaunchKernelGGL((bn_apply_kernel<float, true, 4>), agrid, dim3(kBnThreads), 0, st, P);
+    else hipLaunchKernelGGL((bn_apply_kernel<float, true, 1>), agrid, dim3(kBnThreads), 0, st, P);
+  } else {
+    if (wide) hipLaunchKernelGGL((bn_apply_kernel<uint16_t, true, 8>), agrid, dim3(kBnThreads), 0, st, P);
+    else hipLaunchKernelGGL((bn_apply_kernel<uint16_t, true, 1>), agrid, dim3(kBnThreads), 0, st, P);
+  }
   return launch_status();
 }
 
