@@ -1,0 +1,125 @@
+"""Seeded sweeps over small random shapes: general slab conv (forward, backward-data, backward-filter),
+pooling (max / average, forward, backward) and batch norm against the CPU oracle through the C ABI.
+They exist to hit tilings the hand-picked cases miss (block edges, residue classes with no taps,
+bands, channel counts off every step).  Tolerances as in the per-kernel tests."""
+import numpy as np
+import pytest
+import torch
+
+from arraydiff_cuda_amd import capi
+from gpu_util import dev, host, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _conv_cases(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        kh, kw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        sh, sw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        dh, dw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        eh, ew = (kh - 1) * dh + 1, (kw - 1) * dw + 1
+        HP, WP = eh + int(rng.integers(0, 12)), ew + int(rng.integers(0, 40))
+        out.append((int(rng.integers(1, 3)), int(rng.integers(1, 4)), int(rng.integers(1, 21)), int(rng.integers(1, 41)),
+                    HP, WP, kh, kw, sh, sw, dh, dw))
+    return out
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,HP,WP,kh,kw,sh,sw,dh,dw", _conv_cases(2024, 24))
+def test_general_conv_random(oracle, K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw):
+    rng = np.random.default_rng(HP * 131 + WP)
+    geo = (kh, kw, sh, sw, dh, dw)
+    OH, OW = oracle.conv2d_out_dims(HP, WP, *geo)
+    xs = [rng.uniform(-1, 1, size=(N, Cin, HP, WP)).astype(np.float32) for _ in range(K)]
+    w = rng.standard_normal((Cout, Cin, kh, kw)).astype(np.float32)
+    dys = [rng.standard_normal((N, Cout, OH, OW)).astype(np.float32) for _ in range(K)]
+    d_xs, d_dys, d_w = [dev(x) for x in xs], [dev(d) for d in dys], dev(w)
+    ws = torch.empty(max(capi.conv2d_workspace_bytes(wh, capi.ADH_F32, K, N, Cin, Cout, HP, WP, *geo) for wh in (0, 1, 2)) // 4,
+                     device="cuda")
+    ys = [torch.full((N, Cout, OH, OW), float("nan"), device="cuda") for _ in range(K)]
+    gs = [torch.full((N, Cin, HP, WP), float("nan"), device="cuda") for _ in range(K)]
+    gw = torch.full((Cout, Cin, kh, kw), float("nan"), device="cuda")
+    capi.check(capi.conv2d_fwd_tiles(d_xs, d_w, ys, N, Cin, Cout, HP, WP, *geo, ws=ws))
+    capi.check(capi.conv2d_bwd_data_tiles(d_w, d_dys, gs, N, Cin, Cout, HP, WP, *geo, ws=ws))
+    capi.check(capi.conv2d_bwd_filter_tiles(d_xs, d_dys, gw, N, Cin, Cout, HP, WP, *geo, ws=ws))
+    want_w = np.zeros_like(w)
+    for r in range(K):
+        y = np.empty((N, Cout, OH, OW), np.float32)
+        oracle.conv2d_slab_fwd(xs[r], w, sh, sw, dh, dw, y)
+        assert rel_err(host(ys[r]), y) <= 1e-5
+        g = np.empty((N, Cin, HP, WP), np.float32)
+        oracle.conv2d_slab_bwd_data(w, dys[r], sh, sw, dh, dw, g)
+        assert rel_err(host(gs[r]), g) <= 1e-5
+        oracle.conv2d_slab_bwd_filter(xs[r], dys[r], sh, sw, dh, dw, want_w, beta=1.0)
+    assert rel_err(host(gw), want_w) <= 1e-5
+
+
+def _pool_cases(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        wh, ww = int(rng.integers(1, 5)), int(rng.integers(1, 5))
+        out.append((int(rng.integers(1, 3)), int(rng.integers(1, 4)), int(rng.integers(1, 9)), wh + int(rng.integers(0, 20)),
+                    ww + int(rng.integers(0, 150)), wh, ww, int(rng.integers(1, 4)), int(rng.integers(1, 4)), int(rng.integers(0, 2))))
+    return out
+
+
+@pytest.mark.parametrize("K,N,C,HP,WP,wh,ww,sh,sw,mode", _pool_cases(2025, 20))
+def test_pool_random(oracle, K, N, C, HP, WP, wh, ww, sh, sw, mode):
+    rng = np.random.default_rng(HP * 977 + WP)
+    OH, OW = (HP - wh) // sh + 1, (WP - ww) // sw + 1
+    xs = [rng.uniform(-1, 1, size=(N, C, HP, WP)).astype(np.float32) for _ in range(K)]
+    dys = [rng.standard_normal((N, C, OH, OW)).astype(np.float32) for _ in range(K)]
+    d_xs, d_dys = [dev(x) for x in xs], [dev(d) for d in dys]
+    ys = [torch.full((N, C, OH, OW), float("nan"), device="cuda") for _ in range(K)]
+    gs = [torch.full((N, C, HP, WP), float("nan"), device="cuda") for _ in range(K)]
+    capi.check(capi.pool_fwd_tiles(mode, d_xs, ys, N, C, HP, WP, wh, ww, sh, sw))
+    capi.check(capi.pool_bwd_tiles(mode, d_xs, ys, d_dys, gs, N, C, HP, WP, wh, ww, sh, sw))
+    for r in range(K):
+        y = np.empty((N, C, OH, OW), np.float32)
+        oracle.pool_slab_fwd(mode, xs[r], wh, ww, sh, sw, y)
+        assert rel_err(host(ys[r]), y) <= 1e-5
+        g = np.empty((N, C, HP, WP), np.float32)
+        oracle.pool_slab_bwd(mode, xs[r], dys[r], wh, ww, sh, sw, g)
+        assert rel_err(host(gs[r]), g) <= 1e-5
+
+
+def _bn_cases(seed, count):
+    rng = np.random.default_rng(seed)
+    return [(int(rng.integers(1, 4)), int(rng.integers(1, 6)), int(rng.integers(1, 12)), int(rng.integers(1, 12)),
+             int(rng.integers(1, 40)), int(rng.integers(0, 2)), int(rng.integers(0, 3))) for _ in range(count)]
+
+
+@pytest.mark.parametrize("K,N,C,H,W,relu,p", _bn_cases(2026, 16))
+def test_batchnorm_random(oracle, K, N, C, H, W, relu, p):
+    rng = np.random.default_rng(H * 59 + W)
+    xs = [(rng.standard_normal((N, C, H, W)) + 1).astype(np.float32) for _ in range(K)]
+    sc = [rng.uniform(0.5, 1.5, C).astype(np.float32) for _ in range(K)]
+    sh = [rng.uniform(-0.5, 0.5, C).astype(np.float32) for _ in range(K)]
+    dys = [rng.standard_normal((N, C, H + 2 * p, W + 2 * p)).astype(np.float32) for _ in range(K)]
+    ws = torch.empty(capi.batchnorm_workspace_bytes(K, N, C) // 4, device="cuda")
+    d_xs, d_sc, d_sh, d_dys = ([dev(a) for a in l] for l in (xs, sc, sh, dys))
+    ys = [torch.full((N, C, H + 2 * p, W + 2 * p), float("nan"), device="cuda") for _ in range(K)]
+    sm = [torch.empty(C, device="cuda") for _ in range(K)]
+    si = [torch.empty(C, device="cuda") for _ in range(K)]
+    capi.check(capi.batchnorm_fwd_tiles(d_xs, d_sc, d_sh, ys, N, C, H, W, relu=relu, out_halo=p, save_means=sm, save_invstds=si,
+                                        ws=ws))
+    dxs = [torch.full((N, C, H, W), float("nan"), device="cuda") for _ in range(K)]
+    dsc, dsh = [torch.empty(C, device="cuda") for _ in range(K)], [torch.empty(C, device="cuda") for _ in range(K)]
+    capi.check(capi.batchnorm_bwd_tiles(d_xs, d_dys, d_sc, d_sh, sm, si, dxs, dsc, dsh, N, C, H, W, relu=relu, dy_halo=p, ws=ws))
+    for r in range(K):
+        y = np.empty((N, C, H + 2 * p, W + 2 * p), np.float32)
+        m, i = np.empty(C, np.float32), np.empty(C, np.float32)
+        oracle.batchnorm2d_fwd_train(xs[r], sc[r], sh[r], 1e-5, relu, p, y, None, None, m, i)
+        # a single value per channel has variance 0 and 1/sqrt(eps) ~ 316: its output is the shift, errors scale with it
+        assert rel_err(host(ys[r]), y) <= 2e-5
+        dx, ds, db = np.empty((N, C, H, W), np.float32), np.empty(C, np.float32), np.empty(C, np.float32)
+        oracle.batchnorm2d_bwd(xs[r], dys[r], sc[r], sh[r], m, i, relu, p, dx, ds, db)
+        pre = sc[r][None, :, None, None] * (xs[r].astype(np.float64) - m[None, :, None, None]) * i[None, :, None, None] + \
+            sh[r][None, :, None, None]
+        keep = (np.abs(pre) > 1e-4) if relu else np.ones_like(pre, bool)
+        if N * H * W > 1:
+            scale = max(float(np.abs(dx).max()), 1e-3)
+            assert np.max(np.abs(np.where(keep, host(dxs[r]) - dx, 0))) <= 5e-5 * max(scale, 1.0) * max(1.0, float(i.max()) / 10)
+        np.testing.assert_allclose(host(dsh[r]), db, rtol=1e-4, atol=1e-4 * max(1.0, float(np.abs(db).max())))
