@@ -67,6 +67,12 @@ SIGNATURES = {
     "adh_softmax_nll_loss_fwd": (i32, [u32, u32, vp, vp, vp, vp]),
     "adh_softmax_nll_loss_bwd": (i32, [u32, u32, vp, vp, vp, vp, vp]),
     "adh_softmax_xent_fwd": (i32, [u32, u32, vp, vp, vp, vp, vp]),
+    "adh_scale_add_f32": (i32, [u64, f32, vp, f32, vp, vp]),
+    "adh_add_online_f32": (i32, [u64, f32, vp, vp, vp]),
+    "adh_stat_step_f32": (i32, [u64, f32, vp, vp, vp, vp]),
+    "adh_flat_store_f32": (i32, [u32, vpp, ctypes.POINTER(u64), u64, vp, vp]),
+    "adh_flat_load_f32": (i32, [u32, vpp, ctypes.POINTER(u64), u64, vp, vp]),
+    "adh_sgd_step_f32": (i32, [u64, u32, vpp, f32, f32, f32, f32, i32, vp, vp, vp, vp, vp]),
 }
 
 
@@ -318,6 +324,53 @@ def sum_fwd(xs, y):
     _dev(*xs, y)
     xt, keep = _tbl(xs)
     return lib().adh_sum_fwd(_dt(y), len(xs), y.numel(), xt, y.data_ptr(), _stream())
+
+
+def scale_add(alpha, x, beta, y):
+    """y = alpha*x + beta*y over flat fp32 tensors."""
+    _dev(x, y)
+    return lib().adh_scale_add_f32(y.numel(), alpha, x.data_ptr(), beta, y.data_ptr(), _stream())
+
+
+def add_online(alpha, x, y):
+    """y = y + alpha*(x - y)."""
+    _dev(x, y)
+    return lib().adh_add_online_f32(y.numel(), alpha, x.data_ptr(), y.data_ptr(), _stream())
+
+
+def stat_step(rate, avg_stat, running_stat, stat):
+    _dev(avg_stat, running_stat, stat)
+    return lib().adh_stat_step_f32(stat.numel(), rate, avg_stat.data_ptr(), running_stat.data_ptr(), stat.data_ptr(),
+                                   _stream())
+
+
+def _lens(arrays):
+    return (u64 * len(arrays))(*[a.numel() for a in arrays])
+
+
+def flat_store(arrays, flat, offset=0):
+    """Copy the arrays, in order, into consecutive ranges of `flat` starting at element `offset`."""
+    _dev(*arrays, flat)
+    t, keep = _tbl(arrays)
+    return lib().adh_flat_store_f32(len(arrays), t, _lens(arrays), offset, flat.data_ptr(), _stream())
+
+
+def flat_load(arrays, flat, offset=0):
+    """The inverse of flat_store: consecutive ranges of `flat` into the arrays."""
+    _dev(*arrays, flat)
+    t, keep = _tbl(arrays)
+    return lib().adh_flat_load_f32(len(arrays), t, _lens(arrays), offset, flat.data_ptr(), _stream())
+
+
+def sgd_step(grads, param, momentum_grad, lagged_param=None, sum_grad=None, l2_reg=0.0, momentum=0.0, step_size=0.0,
+             next_step_size=0.0, nesterov=False):
+    """One fused optimizer update over flat fp32 vectors; grads is the list of per-rank gradient vectors."""
+    _dev(*grads, param, momentum_grad)
+    t, keep = _tbl(grads)
+    return lib().adh_sgd_step_f32(param.numel(), len(grads), t, l2_reg, momentum, step_size, next_step_size,
+                                  int(bool(nesterov)), param.data_ptr(), momentum_grad.data_ptr(),
+                                  lagged_param.data_ptr() if lagged_param is not None else None,
+                                  sum_grad.data_ptr() if sum_grad is not None else None, _stream())
 
 
 def pool_fwd_tiles(mode, xs, ys, N, C, HP, WP, wh, ww, sh, sw):

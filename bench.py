@@ -341,7 +341,7 @@ def main():
             lambda: lib.adh_pool2d_slab_bwd_tiles(0, 1, K, N, C, Hq, Wq, 3, 3, 2, 2, xq_tbl, yq_tbl, dq_tbl, gq_tbl,
                                                   0.0, stream),
             "hbm", 2 * in_b + out_b, HBM_PEAK_GBS, "GB/s", note="reads x and dy, writes dx; y is not read")
-        del xq, yq, dq, gq, flush_scratch
+        del xq, yq, dq, gq
         # batch norm with tile-local statistics + rectifier + halo pad in one call (the BN -> ReLU -> HaloPad
         # prefix of the spatially-parallel residual block) on cfg1's 4 tiles, and its backward
         xb = [torch.randn((N, C, Ht, W), device="cuda", generator=g) + 0.5 for _ in range(K)]
@@ -402,6 +402,38 @@ def main():
                                                              0.0, wsg.data_ptr(), wsg_bytes, stream),
                 "mfma", fl, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
             del xg, yg, gg, wsg
+
+        # the optimizer's flat vectors at ResNet-18's parameter count (11.69 M floats), gradients of 4 ranks
+        res18 = [(64, 3, 7, 7)]
+        for cin, cout, first in ((64, 64, False), (64, 128, True), (128, 256, True), (256, 512, True)):
+            for blk in range(2):
+                ci = cin if blk == 0 else cout
+                res18 += [(ci,), (ci,), (cout, ci, 3, 3), (cout,), (cout,), (cout, cout, 3, 3)]
+                if blk == 0 and first:
+                    res18 += [(cout, ci, 1, 1)]
+        res18 += [(512,), (512,), (1000, 512), (1000,)]
+        p_arrays = [torch.randn(sh, device="cuda", generator=g) * 0.05 for sh in res18]
+        pdim = sum(a.numel() for a in p_arrays)
+        flat_p = torch.empty(pdim, device="cuda")
+        flat_m = torch.zeros(pdim, device="cuda")
+        flat_lag = torch.empty(pdim, device="cuda")
+        flat_g = [torch.randn(pdim, device="cuda", generator=g) * 1e-3 for _ in range(K)]
+        pa_tbl, _kp1 = capi.ptr_table([a.data_ptr() for a in p_arrays])
+        pa_len = (ctypes.c_uint64 * len(p_arrays))(*[a.numel() for a in p_arrays])
+        fg_tbl, _kp2 = capi.ptr_table([t.data_ptr() for t in flat_g])
+        reps, wu = 50, 10
+        add("flat store: %d parameter arrays -> one vector of %d floats" % (len(p_arrays), pdim),
+            lambda: lib.adh_flat_store_f32(len(p_arrays), pa_tbl, pa_len, 0, flat_p.data_ptr(), stream),
+            "hbm", 2.0 * pdim * 4, HBM_PEAK_GBS, "GB/s", flushed=True, graph=True)
+        add("flat load: one vector -> %d parameter arrays" % len(p_arrays),
+            lambda: lib.adh_flat_load_f32(len(p_arrays), pa_tbl, pa_len, 0, flat_p.data_ptr(), stream),
+            "hbm", 2.0 * pdim * 4, HBM_PEAK_GBS, "GB/s", flushed=True, graph=True)
+        add("sgd step (4 rank gradients summed + l2 + Nesterov momentum + lagged copy, one pass)",
+            lambda: lib.adh_sgd_step_f32(pdim, K, fg_tbl, 1e-4, 0.9, 0.1, 0.1, 1, flat_p.data_ptr(), flat_m.data_ptr(),
+                                         flat_lag.data_ptr(), None, stream),
+            "hbm", (K + 2 + 3) * pdim * 4.0, HBM_PEAK_GBS, "GB/s", flushed=True,
+            note="reads 4 gradient vectors + parameters + momentum, writes momentum + parameters + lagged copy")
+        del p_arrays, flat_g, flush_scratch
         out["secondary"] = sec
 
     # ---- CPU baseline: the scalar port, single thread, on a bounded sample ----

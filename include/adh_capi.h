@@ -295,6 +295,39 @@ int adh_softmax_nll_loss_bwd(uint32_t C, uint32_t N, const float *y, const uint3
 int adh_softmax_xent_fwd(uint32_t C, uint32_t N, const float *x, const uint32_t *label, float *y,
                          float *loss, void *stream);
 
+/* ---- flat parameter vectors and the SGD update (fp32) ---------------------- */
+/* array_add_scaled_packed<float>, src/kernels/array.cu:97-110,211-222: y = alpha*x + beta*y,
+ * evaluated as fma(alpha, x, beta*y). */
+int adh_scale_add_f32(uint64_t n, float alpha, const float *x, float beta, float *y, void *stream);
+/* array_add_online_packed<float>, src/kernels/array.cu:112-124,224-234: y = y + alpha*(x - y),
+ * evaluated as fma(alpha, x - y, y). */
+int adh_add_online_f32(uint64_t n, float alpha, const float *x, float *y, void *stream);
+/* The running-statistics update of ParallelSGDOptimizer::step (include/arraydiff/optimize.hh:507-514):
+ * running_stat += rate*(avg_stat - running_stat); stat = running_stat, in one pass. */
+int adh_stat_step_f32(uint64_t n, float rate, const float *avg_stat, float *running_stat, float *stat,
+                      void *stream);
+/* Op::store_val / store_grad (src/op.cc:170-194) and Op::load_val (src/op.cc:148-158) for one flat
+ * vector: the arrays, in the order given, occupy consecutive ranges of `flat` starting at element
+ * flat_offset (array i of lens[i] floats; a zero length is skipped).  store copies arrays -> flat,
+ * load copies flat -> arrays.  One launch per 48 arrays instead of one copy per array. */
+int adh_flat_store_f32(uint32_t num_arrays, const float *const *arrays, const uint64_t *lens, uint64_t flat_offset,
+                       float *flat, void *stream);
+int adh_flat_load_f32(uint32_t num_arrays, float *const *arrays, const uint64_t *lens, uint64_t flat_offset,
+                      const float *flat, void *stream);
+/* The parameter update of ParallelSGDOptimizer::step (include/arraydiff/optimize.hh:443-505) in one pass
+ * over flat vectors of n floats:
+ *   g = grads[0] + grads[1] + ... + grads[num_grads-1]      (the ncclReduce to rank 0, in rank order)
+ *   if l2_reg != 0:  g = fma(l2_reg, param, g)
+ *   momentum_grad = g + momentum*momentum_grad              (product rounded, then the sum)
+ *   nesterov:  param = fma(-step_size, g, param); lagged_param = param;
+ *              param = fma(-next_step_size*momentum, momentum_grad, param)
+ *   else:      param = fma(-step_size, momentum_grad, param); lagged_param = param
+ * lagged_param and sum_grad (receives g) may be NULL.  sum_grad may be grads[0]; no other aliasing.
+ * 1 <= num_grads <= ADH_MAX_TILES. */
+int adh_sgd_step_f32(uint64_t n, uint32_t num_grads, const float *const *grads, float l2_reg, float momentum,
+                     float step_size, float next_step_size, int nesterov, float *param, float *momentum_grad,
+                     float *lagged_param, float *sum_grad, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

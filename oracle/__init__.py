@@ -262,6 +262,47 @@ def sum_fwd(xs, y):
     _lib.orc_sum_fwd(_u32(len(xs)), ctypes.c_uint64(y.size), _ptr_array(xs), _ptr(y))
 
 
+def array_add_scaled(alpha, x, beta, y):
+    """y = alpha*x + beta*y in place (flat float32)."""
+    _lib.orc_array_add_scaled(ctypes.c_uint64(y.size), ctypes.c_float(alpha), _ptr(x), ctypes.c_float(beta), _ptr(y))
+
+
+def array_add_online(alpha, x, y):
+    """y = y + alpha*(x - y) in place."""
+    _lib.orc_array_add_online(ctypes.c_uint64(y.size), ctypes.c_float(alpha), _ptr(x), _ptr(y))
+
+
+def _len_array(arrs):
+    return (ctypes.c_uint64 * len(arrs))(*[a.size for a in arrs])
+
+
+def flat_store(arrays, flat, offset=0):
+    """Arrays, in order, into consecutive ranges of flat from `offset`; returns the new offset.
+    flat=None only measures."""
+    _lib.orc_flat_store.restype = ctypes.c_uint64
+    return _lib.orc_flat_store(_u32(len(arrays)), _ptr_array(arrays), _len_array(arrays), ctypes.c_uint64(offset),
+                               _ptr(flat) if flat is not None else None)
+
+
+def flat_load(arrays, flat, offset=0):
+    _lib.orc_flat_load.restype = ctypes.c_uint64
+    return _lib.orc_flat_load(_u32(len(arrays)), _ptr_array(arrays), _len_array(arrays), ctypes.c_uint64(offset),
+                              _ptr(flat))
+
+
+def sgd_step(grads, param, momentum_grad, lagged, sum_grad, l2_reg, momentum, step_size, next_step_size, nesterov):
+    """The root-rank update of the parallel SGD optimizer, in place on param / momentum_grad;
+    lagged may be None; sum_grad receives the reduced (and l2-regularised) gradient."""
+    _lib.orc_sgd_step(ctypes.c_uint64(param.size), _u32(len(grads)), _ptr_array(grads), ctypes.c_float(l2_reg),
+                      ctypes.c_float(momentum), ctypes.c_float(step_size), ctypes.c_float(next_step_size),
+                      ctypes.c_int(int(bool(nesterov))), _ptr(param), _ptr(momentum_grad),
+                      _ptr(lagged) if lagged is not None else None, _ptr(sum_grad))
+
+
+def stat_step(rate, avg_stat, running_stat, stat):
+    _lib.orc_stat_step(ctypes.c_uint64(stat.size), ctypes.c_float(rate), _ptr(avg_stat), _ptr(running_stat), _ptr(stat))
+
+
 def pool_slab_fwd(mode, x_pad, wh, ww, sh, sw, y):
     """x_pad (N, C, HP, WP) float32 -> y (N, C, OH, OW); mode 1 = max, 0 = average."""
     N, C, HP, WP = x_pad.shape

@@ -665,6 +665,82 @@ void orc_sum_fwd(uint32_t count, uint64_t n, const float *const *xs, float *y) {
 }
 
 /* ------------------------------------------------------------------ */
+/* flat parameter vectors and the SGD update                            */
+/* ------------------------------------------------------------------ */
+
+/* arraydiff_array_add_scaled_packed_kernel (src/kernels/array.cu:97-110): y = alpha*x + beta*y.
+ * The compiler of the reference contracts the expression into one fused multiply-add; the form
+ * fma(alpha, x, beta*y), which contracts the first product, is fixed here.  With beta == 1 (every
+ * parameter update) both possible contractions give these bits; with alpha == 1 (the momentum
+ * update) the other contraction may differ in the last place. */
+void orc_array_add_scaled(uint64_t n, float alpha, const float *x, float beta, float *y) {
+  for (uint64_t i = 0; i < n; ++i) {
+    const float yi = y[i];
+    const float by = beta * yi;
+    y[i] = fmaf(alpha, x[i], by);
+  }
+}
+/* arraydiff_array_add_online_packed_kernel (src/kernels/array.cu:112-124): y = y + alpha*(x - y) */
+void orc_array_add_online(uint64_t n, float alpha, const float *x, float *y) {
+  for (uint64_t i = 0; i < n; ++i) {
+    const float yi = y[i];
+    const float d = x[i] - yi;
+    y[i] = fmaf(alpha, d, yi);
+  }
+}
+/* Op::store_val / store_grad walking the graph (src/op.cc:170-194): every array of the set is
+ * copied to the writer at the running offset, which advances by the array's size. */
+uint64_t orc_flat_store(uint32_t count, const float *const *arrays, const uint64_t *lens, uint64_t offset, float *flat) {
+  for (uint32_t k = 0; k < count; ++k) {
+    if (flat) memcpy(flat + offset, arrays[k], lens[k] * sizeof(float));
+    offset += lens[k];
+  }
+  return offset;
+}
+/* Op::load_val (src/op.cc:148-158): the inverse copy */
+uint64_t orc_flat_load(uint32_t count, float *const *arrays, const uint64_t *lens, uint64_t offset, const float *flat) {
+  for (uint32_t k = 0; k < count; ++k) {
+    memcpy(arrays[k], flat + offset, lens[k] * sizeof(float));
+    offset += lens[k];
+  }
+  return offset;
+}
+/* The root-rank part of ParallelSGDOptimizer::step (include/arraydiff/optimize.hh:443-505):
+ *   ncclReduce(sum) of the ranks' sum_grad vectors onto rank 0   (:443-451; summed here in rank order)
+ *   sum_grad += l2_reg * param                  if l2_reg != 0   (:481-483)
+ *   momentum_grad = 1*sum_grad + mu*momentum_grad                (:487)
+ *   nesterov:  param += -alpha*sum_grad; lagged = param; param += -next_alpha*mu*momentum_grad  (:488-492)
+ *   else:      param += -alpha*momentum_grad; lagged = param                                    (:493-496)
+ * sum_grad (n floats) is rank 0's vector on entry when grads == NULL, else scratch that receives
+ * the reduced gradient. */
+void orc_sgd_step(uint64_t n, uint32_t num_grads, const float *const *grads, float l2_reg, float mu, float alpha,
+                  float next_alpha, int nesterov, float *param, float *momentum_grad, float *lagged,
+                  float *sum_grad) {
+  if (grads) {
+    for (uint64_t i = 0; i < n; ++i) {
+      float g = grads[0][i];
+      for (uint32_t r = 1; r < num_grads; ++r) g += grads[r][i];
+      sum_grad[i] = g;
+    }
+  }
+  if (l2_reg != 0.0f) orc_array_add_scaled(n, l2_reg, param, 1.0f, sum_grad);
+  orc_array_add_scaled(n, 1.0f, sum_grad, mu, momentum_grad);
+  if (nesterov) {
+    orc_array_add_scaled(n, -alpha, sum_grad, 1.0f, param);
+    if (lagged) memcpy(lagged, param, n * sizeof(float));
+    orc_array_add_scaled(n, -next_alpha * mu, momentum_grad, 1.0f, param);
+  } else {
+    orc_array_add_scaled(n, -alpha, momentum_grad, 1.0f, param);
+    if (lagged) memcpy(lagged, param, n * sizeof(float));
+  }
+}
+/* running statistics (include/arraydiff/optimize.hh:507-514): running += rate*(avg - running); stat = running */
+void orc_stat_step(uint64_t n, float rate, const float *avg_stat, float *running_stat, float *stat) {
+  orc_array_add_online(n, rate, avg_stat, running_stat);
+  memcpy(stat, running_stat, n * sizeof(float));
+}
+
+/* ------------------------------------------------------------------ */
 /* L1/L2/L3: softmax + negative log likelihood                          */
 /* ------------------------------------------------------------------ */
 
