@@ -17,6 +17,7 @@
 #include <cassert>
 #include <cstdint>
 #include <memory>
+#include <stdexcept>
 
 namespace arraydiff {
 
@@ -38,6 +39,36 @@ public:
     ptr_ = std::shared_ptr<void>(gpu_alloc_bytes(bytes ? bytes : 4096), gpu_free_bytes);
   }
   void reallocate(size_t size, GPUContext *ctx) { *this = GPUMemory<T>(size, ctx); }
+  // array_gpu.hh:46-65
+  static GPUMemory Zeros(size_t size, GPUContext *ctx) {
+    static_assert(sizeof(T) == 4, "Zeros is a 32-bit fill");
+    GPUMemory m(size, ctx);
+    GPUConn conn = ctx->conn();
+    m.set_constant(T(), conn);
+    return m;
+  }
+  // whole-vector arithmetic of the optimizers (array_gpu.hh:150-215); ranges are checked here
+  void set_constant(T c, GPUConn &conn) {
+    float f;
+    __builtin_memcpy(&f, &c, 4);
+    array_set_constant_packed<float>((uint32_t)size_, f, reinterpret_cast<float *>(dptr()), conn.stream());
+  }
+  void add(GPUMemory<T> src, size_t buf_sz, size_t dst_offset, size_t src_offset, GPUConn &conn) {
+    check_range(src, buf_sz, dst_offset, src_offset);
+    array_add_packed<T>((uint32_t)buf_sz, src.dptr() + src_offset, dptr() + dst_offset, conn.stream());
+  }
+  void add_scaled(T alpha, GPUMemory<T> src, T beta, size_t buf_sz, size_t dst_offset, size_t src_offset, GPUConn &conn) {
+    check_range(src, buf_sz, dst_offset, src_offset);
+    array_add_scaled_packed<T>((uint32_t)buf_sz, alpha, beta, src.dptr() + src_offset, dptr() + dst_offset, conn.stream());
+  }
+  void add_online(T alpha, GPUMemory<T> src, size_t buf_sz, size_t dst_offset, size_t src_offset, GPUConn &conn) {
+    check_range(src, buf_sz, dst_offset, src_offset);
+    array_add_online_packed<T>((uint32_t)buf_sz, alpha, src.dptr() + src_offset, dptr() + dst_offset, conn.stream());
+  }
+  void copy(GPUMemory<T> src, size_t buf_sz, size_t dst_offset, size_t src_offset, GPUConn &conn) {
+    check_range(src, buf_sz, dst_offset, src_offset);
+    gpu_copy_d2d(dptr() + dst_offset, src.dptr() + src_offset, buf_sz * sizeof(T), conn.stream());
+  }
 
   T *dptr() const { return static_cast<T *>(ptr_.get()); }
   uintptr_t dptr_addr() const { return reinterpret_cast<uintptr_t>(ptr_.get()); }
@@ -55,6 +86,9 @@ public:
   }
 
 private:
+  void check_range(const GPUMemory<T> &src, size_t n, size_t dst_offset, size_t src_offset) const {
+    if (dst_offset + n > size_ || src_offset + n > src.size_) throw std::out_of_range("GPUMemory: range outside the buffer");
+  }
   std::shared_ptr<void> ptr_;
   size_t size_;
 };

@@ -31,6 +31,21 @@ inline void array_add_packed<float>(uint32_t dim, const float *x, float *y, hipS
   adh_check(adh_add_f32(dim, x, y, stream), "array_add_packed");
 }
 
+// src/kernels/array.cu:97-124, 211-234
+template <typename T>
+void array_add_scaled_packed(uint32_t dim, T alpha, T beta, const T *x, T *y, hipStream_t stream);
+template <>
+inline void array_add_scaled_packed<float>(uint32_t dim, float alpha, float beta, const float *x, float *y,
+                                           hipStream_t stream) {
+  adh_check(adh_scale_add_f32(dim, alpha, x, beta, y, stream), "array_add_scaled_packed");
+}
+template <typename T>
+void array_add_online_packed(uint32_t dim, T alpha, const T *x, T *y, hipStream_t stream);
+template <>
+inline void array_add_online_packed<float>(uint32_t dim, float alpha, const float *x, float *y, hipStream_t stream) {
+  adh_check(adh_add_online_f32(dim, alpha, x, y, stream), "array_add_online_packed");
+}
+
 // src/kernels/spatial.cu:455-510 (1x2), 596-652 (1x4), 708-731 (2x1): rank-wise launchers
 namespace detail {
 inline void halo_rank(bool reduce, uint32_t grid_w, uint32_t grid_h, uint32_t rank, uint32_t halo_pad, uint32_t w,

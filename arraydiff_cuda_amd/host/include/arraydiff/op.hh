@@ -66,6 +66,46 @@ public:
   explicit HazardError(const std::string &w) : std::logic_error(w) {}
 };
 
+// A set of variables to persist, load or store as one flat vector (op.hh:110-171).  While a walk
+// over the graph holds the lock, mask() lets every member through exactly once, so a variable
+// that several nodes share lands in the flat vector one time.
+class VarIdSet {
+public:
+  static VarIdSet Singleton(VarId v) {
+    VarIdSet s;
+    s.insert(v);
+    return s;
+  }
+  void insert(VarId v) {
+    if (locked_) throw HazardError("VarIdSet: insert while a walk holds the set");
+    ids_.insert(v.raw_id());
+  }
+  void insert_all(const VarIdSet &o) {
+    if (locked_) throw HazardError("VarIdSet: insert while a walk holds the set");
+    ids_.insert(o.ids_.begin(), o.ids_.end());
+  }
+  bool contains(VarId v) const { return ids_.count(v.raw_id()) != 0; }
+  size_t size() const { return ids_.size(); }
+  void lock() {
+    if (locked_) throw HazardError("VarIdSet: already locked");
+    seen_.clear();
+    locked_ = true;
+  }
+  void unlock() {
+    locked_ = false;
+    seen_.clear();
+  }
+  bool mask(VarId v) {
+    if (!locked_) throw HazardError("VarIdSet: mask outside a walk");
+    if (!ids_.count(v.raw_id())) return false;
+    return seen_.insert(v.raw_id()).second;
+  }
+
+private:
+  bool locked_ = false;
+  std::set<uint64_t> ids_, seen_;
+};
+
 // ---------------------------------------------------------------------------
 // TxnVar: one buffer, (re)initialised per transaction
 // ---------------------------------------------------------------------------
@@ -114,9 +154,22 @@ public:
     b.writers.insert(node.raw_id());
     return true;
   }
-  // Read access: the value must have been written in this transaction.
+  // Marks the value to be carried into `txn` by the first read there (op.hh:236-247); a write in
+  // the new transaction replaces it as usual.
+  void rollover(TxnId txn) {
+    Buf &b = *buf_;
+    if (!(b.has_txn && b.txn == txn.raw_id())) b.rollover = true;
+  }
+  // Read access: the value must have been written in this transaction, or carried into it.
   V &get(TxnId txn, NodeId node) {
     Buf &b = *buf_;
+    if (b.buffer && b.rollover && !(b.has_txn && b.txn == txn.raw_id())) {
+      b.has_txn = true;
+      b.txn = txn.raw_id();
+      b.writers.clear();
+      b.readers.clear();
+      b.rollover = false;
+    }
     if (!b.buffer || !b.has_txn || !(b.txn == txn.raw_id())) throw HazardError("read of a variable not written in this transaction");
     b.readers.insert(node.raw_id());
     return *b.buffer;
@@ -137,7 +190,7 @@ public:
 private:
   struct Buf {
     VarId var;
-    bool has_txn = false;
+    bool has_txn = false, rollover = false;
     uint64_t txn = 0;
     std::set<uint64_t> writers, readers;
     std::unique_ptr<V> buffer;
@@ -147,6 +200,7 @@ private:
     if (b.has_txn && b.txn == txn.raw_id()) return false;
     b.has_txn = true;
     b.txn = txn.raw_id();
+    b.rollover = false;
     b.writers.clear();
     b.readers.clear();
     if (!b.buffer) allocate(ctx);
@@ -178,6 +232,11 @@ public:
   VShape offset() const { return val_.offset(); }
   VShape stride() const { return val_.stride(); }
   size_t batch_shape() const { return val_.batch_shape(); }
+  // op.hh:569-581
+  void rollover_all(TxnId txn, VarIdSet &vars) {
+    if (vars.contains(val_.var())) val_.rollover(txn);
+    if (vars.contains(grad_.var())) grad_.rollover(txn);
+  }
 
 private:
   TxnVar<V> val_, grad_;
@@ -207,6 +266,21 @@ private:
   size_t pushes_ = 0, pops_ = 0;
 };
 
+// The arrays one walk over the graph contributes to (or takes from) a flat vector, in walk order.
+// The reference copies array by array as the walk proceeds (store_any / load_any through an `any`
+// reader or writer, op.hh:831-861); here the walk only collects and ONE batched copy follows it.
+struct FlatBatch {
+  vector<float *> arrays;
+  vector<uint64_t> lens;
+  hipStream_t stream = nullptr;
+  size_t push(float *dptr, size_t len, hipStream_t s) {
+    arrays.push_back(dptr);
+    lens.push_back(len);
+    stream = s;
+    return len;
+  }
+};
+
 class Op {
 public:
   Op() {}
@@ -218,6 +292,25 @@ public:
   virtual void _forward(TxnId txn) = 0;
   virtual void _backward(TxnId txn) = 0;
   virtual void _set_grad_sink(TxnId txn) { (void)txn; }
+  // Flat-vector plumbing (op.hh:630-658): a node that owns variables of `vars` adds them to the
+  // batch at the running offset and returns the advanced offset.  batch == NULL only measures.
+  virtual size_t _load_val(TxnId, VarIdSet &, size_t offset, FlatBatch *) { return offset; }
+  virtual size_t _load_grad(TxnId, VarIdSet &, size_t offset, FlatBatch *) { return offset; }
+  virtual size_t _store_val(TxnId, VarIdSet &, size_t offset, FlatBatch *) { return offset; }
+  virtual size_t _store_grad(TxnId, VarIdSet &, size_t offset, FlatBatch *) { return offset; }
+  // Only nodes that own long-lived variables (parameters, statistics, inputs) carry anything over.
+  virtual void _persist(TxnId, VarIdSet &) {}
+
+  // The members of `vars` reachable from this node, in the order the backward walk meets them, as
+  // consecutive ranges of a flat device vector starting at `offset`; returns the end offset
+  // (src/op.cc:148-194).  store_* with a NULL writer only measures.  One batched copy per call,
+  // enqueued on the stream of the variables' context.
+  size_t load_val(TxnId txn, VarIdSet &vars, size_t offset, GPUMemory<float> *reader);
+  size_t load_grad(TxnId txn, VarIdSet &vars, size_t offset, GPUMemory<float> *reader);
+  size_t store_val(TxnId txn, VarIdSet &vars, size_t offset, GPUMemory<float> *writer);
+  size_t store_grad(TxnId txn, VarIdSet &vars, size_t offset, GPUMemory<float> *writer);
+  // marks the members of `vars` to keep their value into transaction `txn` (src/op.cc:205-212)
+  void persist(TxnId txn, VarIdSet &vars);
 
   // forward pass of everything this node depends on, in dependency order (op.cc:196-221)
   void eval(TxnId txn) {
@@ -309,6 +402,7 @@ public:
   }
   virtual void _forward(TxnId) {}
   virtual void _backward(TxnId) {}
+  virtual void _persist(TxnId txn, VarIdSet &vars) { y_.rollover_all(txn, vars); }
   ARRAYDIFF_VAR_ACCESSORS(V)
 
 private:
@@ -337,6 +431,12 @@ public:
     GPUConn conn = gpu_ctx_of(ctx_)->conn();
     y_.grad().get(txn, id()).store_sync(host, conn);
   }
+  // the value as transaction txn sees it, copied out synchronously
+  template <typename T>
+  void store(TxnId txn, T *host) {
+    GPUConn conn = gpu_ctx_of(ctx_)->conn();
+    y_.val().get(txn, id()).store_sync(host, conn);
+  }
   virtual void _push(EpochId e, function<void(Op *)> apply) {
     if (1 == stack_.push(e)) apply(this);
   }
@@ -345,6 +445,20 @@ public:
   }
   virtual void _forward(TxnId) {}
   virtual void _backward(TxnId) {}
+  virtual void _persist(TxnId txn, VarIdSet &vars) { y_.rollover_all(txn, vars); }
+  // the value (gradient) is replaced from the flat vector: this node becomes its writer (op.hh:831-847)
+  virtual size_t _load_val(TxnId txn, VarIdSet &vars, size_t offset, FlatBatch *batch) {
+    return vars.mask(y_.val().var()) ? offset + flat_in(y_.val(), txn, batch) : offset;
+  }
+  virtual size_t _load_grad(TxnId txn, VarIdSet &vars, size_t offset, FlatBatch *batch) {
+    return vars.mask(y_.grad().var()) ? offset + flat_in(y_.grad(), txn, batch) : offset;
+  }
+  virtual size_t _store_val(TxnId txn, VarIdSet &vars, size_t offset, FlatBatch *batch) {
+    return vars.mask(y_.val().var()) ? offset + flat_out(y_.val(), txn, batch) : offset;
+  }
+  virtual size_t _store_grad(TxnId txn, VarIdSet &vars, size_t offset, FlatBatch *batch) {
+    return vars.mask(y_.grad().var()) ? offset + flat_out(y_.grad(), txn, batch) : offset;
+  }
   virtual typename A::Shape shape() { return y_.shape(); }
   virtual typename A::Shape offset() { return y_.offset(); }
   virtual typename A::Shape stride() { return y_.stride(); }
@@ -352,6 +466,19 @@ public:
   virtual VarData<A> data() { return y_.clone(); }
 
 private:
+  size_t flat_in(TxnVar<A> &v, TxnId txn, FlatBatch *batch) {
+    GPUContext *c = gpu_ctx_of(ctx_);
+    if (!v.overwrite(txn, id(), c)) throw HazardError("load of a variable another node wrote in this transaction");
+    A &a = v.get_excl(txn, id());
+    if (!a.is_packed()) throw std::invalid_argument("flat vectors hold packed arrays only");
+    return batch->push(reinterpret_cast<float *>(a.dptr()), a.dim().flat_size(), c->conn().stream());
+  }
+  size_t flat_out(TxnVar<A> &v, TxnId txn, FlatBatch *batch) {
+    if (!batch) return y_.shape().flat_size();
+    A &a = v.get(txn, id());
+    if (!a.is_packed()) throw std::invalid_argument("flat vectors hold packed arrays only");
+    return batch->push(reinterpret_cast<float *>(a.dptr()), a.dim().flat_size(), gpu_ctx_of(ctx_)->conn().stream());
+  }
   shared_ptr<Context> ctx_;
   VarData<A> y_;
 };
@@ -788,17 +915,6 @@ using CudnnConv2DOp = SlabConv2DOp<V, A>;
 // ---------------------------------------------------------------------------
 // the shard-local ops between two halo exchanges: batch norm, rectifier, sum join
 // ---------------------------------------------------------------------------
-class VarIdSet {
-public:
-  void insert(VarId v) { ids_.insert(v.raw_id()); }
-  void insert_all(const VarIdSet &o) { ids_.insert(o.ids_.begin(), o.ids_.end()); }
-  bool contains(VarId v) const { return ids_.count(v.raw_id()) != 0; }
-  size_t size() const { return ids_.size(); }
-
-private:
-  std::set<uint64_t> ids_;
-};
-
 template <typename V, typename B>
 class BatchNormOutput {
 public:
@@ -908,6 +1024,8 @@ public:
     if (1 == stack_.push(e)) {
       for (size_t r = 0; r < x_vars_.size(); ++r) {
         x_vars_[r]->_push(e, apply);
+        vars_[r].batch_mean->_push(e, apply);
+        vars_[r].batch_variance->_push(e, apply);
         vars_[r].fixed_mean->_push(e, apply);
         vars_[r].fixed_variance->_push(e, apply);
         vars_[r].scale->_push(e, apply);
@@ -924,6 +1042,8 @@ public:
         vars_[r].scale->_pop(e, apply);
         vars_[r].fixed_variance->_pop(e, apply);
         vars_[r].fixed_mean->_pop(e, apply);
+        vars_[r].batch_variance->_pop(e, apply);
+        vars_[r].batch_mean->_pop(e, apply);
         x_vars_[r]->_pop(e, apply);
       }
     }

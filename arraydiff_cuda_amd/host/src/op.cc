@@ -38,6 +38,67 @@ void check_packed(V3 &a, const char *who) {
 
 }  // namespace
 
+// ---- flat-vector plumbing (op.cc:148-212) ----
+namespace {
+enum FlatKind { kLoadVal, kLoadGrad, kStoreVal, kStoreGrad };
+
+// Visits every node once on the way back out of the graph (the order of the reference's walk),
+// collects the arrays of `vars`, then moves them with one batched copy.
+size_t flat_walk(Op *root, FlatKind kind, TxnId txn, VarIdSet &vars, size_t offset, GPUMemory<float> *mem) {
+  const bool is_load = kind == kLoadVal || kind == kLoadGrad;
+  if (is_load && !mem) throw std::invalid_argument("load from a flat vector needs the vector");
+  FlatBatch batch;
+  FlatBatch *b = mem ? &batch : nullptr;
+  size_t end = offset;
+  vars.lock();
+  try {
+    EpochId e;
+    root->_push(e, [](Op *) {});
+    root->_pop(e, [&](Op *op) {
+      switch (kind) {
+        case kLoadVal: end = op->_load_val(txn, vars, end, b); break;
+        case kLoadGrad: end = op->_load_grad(txn, vars, end, b); break;
+        case kStoreVal: end = op->_store_val(txn, vars, end, b); break;
+        case kStoreGrad: end = op->_store_grad(txn, vars, end, b); break;
+      }
+    });
+  } catch (...) {
+    vars.unlock();
+    throw;
+  }
+  vars.unlock();
+  if (!mem || batch.arrays.empty()) return end;
+  if (end > mem->size()) throw std::invalid_argument("flat vector shorter than the variables it should hold");
+  if (is_load)
+    adh_check(adh_flat_load_f32((uint32_t)batch.arrays.size(), batch.arrays.data(), batch.lens.data(), offset, mem->dptr(),
+                                batch.stream),
+              "Op::load_val");
+  else
+    adh_check(adh_flat_store_f32((uint32_t)batch.arrays.size(), batch.arrays.data(), batch.lens.data(), offset,
+                                 mem->dptr(), batch.stream),
+              "Op::store_val");
+  return end;
+}
+}  // namespace
+
+size_t Op::load_val(TxnId txn, VarIdSet &vars, size_t offset, GPUMemory<float> *reader) {
+  return flat_walk(this, kLoadVal, txn, vars, offset, reader);
+}
+size_t Op::load_grad(TxnId txn, VarIdSet &vars, size_t offset, GPUMemory<float> *reader) {
+  return flat_walk(this, kLoadGrad, txn, vars, offset, reader);
+}
+size_t Op::store_val(TxnId txn, VarIdSet &vars, size_t offset, GPUMemory<float> *writer) {
+  return flat_walk(this, kStoreVal, txn, vars, offset, writer);
+}
+size_t Op::store_grad(TxnId txn, VarIdSet &vars, size_t offset, GPUMemory<float> *writer) {
+  return flat_walk(this, kStoreGrad, txn, vars, offset, writer);
+}
+void Op::persist(TxnId txn, VarIdSet &vars) {
+  EpochId e;
+  _push(e, [txn, &vars](Op *op) { op->_persist(txn, vars); });
+  _pop(e, [](Op *) {});
+}
+
 // ---- SpatialScatter2DOp (op.cc:2396-2468) ----
 template <>
 void SpatialScatter2DOp<V3>::_forward(TxnId txn) {

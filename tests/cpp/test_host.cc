@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "arraydiff/op.hh"
+#include "arraydiff/optimize.hh"
 
 extern "C" {
 // CPU oracle (oracle/adh_oracle.c): the checker
@@ -49,6 +50,9 @@ void orc_softmax_fwd(uint32_t C, uint32_t N, const float *x, float *y);
 void orc_softmax_nll_loss_fwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label, float *loss);
 void orc_softmax_nll_loss_bwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label, const float *dloss,
                               float *dx);
+void orc_sgd_step(uint64_t n, uint32_t num_grads, const float *const *grads, float l2_reg, float mu, float alpha,
+                  float next_alpha, int nesterov, float *param, float *momentum_grad, float *lagged, float *sum_grad);
+void orc_stat_step(uint64_t n, float rate, const float *avg_stat, float *running_stat, float *stat);
 }
 
 using namespace arraydiff;
@@ -617,10 +621,275 @@ static void test_txn_hazards() {
   for (float v : pdx) CHECK(v == 1.0f / 16);
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// ParallelSGDOptimizer over the residual block: every rank owns its copies of the two filters and of
+// the batch-norm parameters, as in the reference's parallel nets; the optimizer sums the ranks'
+// gradients, updates and hands the result back to every rank.  The CPU side trains ONE set of
+// parameters on the unsplit convolution with the oracle's update and must stay in step.
+// ---------------------------------------------------------------------------------------------
+struct BlockParams {
+  std::vector<float> w1, w2, sc0, sh0, sc1, sh1;
+  std::vector<std::vector<float> *> all() { return {&w1, &w2, &sc0, &sh0, &sc1, &sh1}; }
+};
+
+// gradients of <dY, y> for y = x + conv2(relu(bn1(conv1(relu(bn0(x)))))) with tile-local batch-norm statistics;
+// the batch-norm parameter gradients are summed over the tiles.  stats[r] receives tile r's
+// (mean0, var0, mean1, var1) as the forward pass reports them.
+static BlockParams block_oracle_grads(size_t K, size_t N, size_t C, size_t H, size_t W, const std::vector<float> &X,
+                                      const std::vector<float> &dY, BlockParams &P,
+                                      std::vector<std::vector<std::vector<float>>> *stats) {
+  const size_t Ht = H / K, full = N * C * H * W;
+  const float eps = 1.0e-5f;
+  std::vector<std::vector<float>> m0(K, std::vector<float>(C)), i0 = m0, m1 = m0, i1 = m0;
+  std::vector<float> A0(full), C1(full), A1(full);
+  stats->assign(K, std::vector<std::vector<float>>(4, std::vector<float>(C)));
+  for (size_t r = 0; r < K; ++r) {
+    auto xt = tile_of(X, N, C, H, W, K, r);
+    std::vector<float> yt(xt.size());
+    orc_batchnorm2d_fwd_train(N, C, Ht, W, eps, 1, 0, xt.data(), P.sc0.data(), P.sh0.data(), yt.data(), (*stats)[r][0].data(),
+                              (*stats)[r][1].data(), m0[r].data(), i0[r].data());
+    put_tile(A0, yt, N, C, H, W, K, r);
+  }
+  std::vector<float> A0p(N * C * (H + 2) * (W + 2)), A1p(A0p.size());
+  orc_halo_pad(0, 1, W, H, C, N, A0.data(), A0p.data());
+  orc_conv_slab_fwd(N, C, C, H, W, 3, A0p.data(), P.w1.data(), 0.f, C1.data());
+  for (size_t r = 0; r < K; ++r) {
+    auto xt = tile_of(C1, N, C, H, W, K, r);
+    std::vector<float> yt(xt.size());
+    orc_batchnorm2d_fwd_train(N, C, Ht, W, eps, 1, 0, xt.data(), P.sc1.data(), P.sh1.data(), yt.data(), (*stats)[r][2].data(),
+                              (*stats)[r][3].data(), m1[r].data(), i1[r].data());
+    put_tile(A1, yt, N, C, H, W, K, r);
+  }
+  orc_halo_pad(0, 1, W, H, C, N, A1.data(), A1p.data());
+  BlockParams G;
+  G.w1.assign(P.w1.size(), 0.f); G.w2.assign(P.w2.size(), 0.f);
+  G.sc0.assign(C, 0.f); G.sh0.assign(C, 0.f); G.sc1.assign(C, 0.f); G.sh1.assign(C, 0.f);
+  std::vector<float> dA1p(A1p.size()), dA1(full), dC1(full), dA0p(A0p.size()), dA0(full);
+  orc_conv_slab_bwd_data(N, C, C, H, W, 3, P.w2.data(), dY.data(), 0.f, dA1p.data());
+  orc_conv_slab_bwd_filter(N, C, C, H, W, 3, A1p.data(), dY.data(), 0.f, G.w2.data());
+  orc_halo_unpad(0, 1, W, H, C, N, dA1p.data(), dA1.data());
+  for (size_t r = 0; r < K; ++r) {
+    auto xt = tile_of(C1, N, C, H, W, K, r), dyt = tile_of(dA1, N, C, H, W, K, r);
+    std::vector<float> dxt(xt.size()), ds(C), db(C);
+    orc_batchnorm2d_bwd(N, C, Ht, W, 1, 0, xt.data(), dyt.data(), P.sc1.data(), P.sh1.data(), m1[r].data(), i1[r].data(), 0.f,
+                        0.f, dxt.data(), ds.data(), db.data());
+    put_tile(dC1, dxt, N, C, H, W, K, r);
+    for (size_t c = 0; c < C; ++c) { G.sc1[c] += ds[c]; G.sh1[c] += db[c]; }
+  }
+  orc_conv_slab_bwd_data(N, C, C, H, W, 3, P.w1.data(), dC1.data(), 0.f, dA0p.data());
+  orc_conv_slab_bwd_filter(N, C, C, H, W, 3, A0p.data(), dC1.data(), 0.f, G.w1.data());
+  orc_halo_unpad(0, 1, W, H, C, N, dA0p.data(), dA0.data());
+  for (size_t r = 0; r < K; ++r) {
+    auto xt = tile_of(X, N, C, H, W, K, r), dyt = tile_of(dA0, N, C, H, W, K, r);
+    std::vector<float> dxt(xt.size()), ds(C), db(C);
+    orc_batchnorm2d_bwd(N, C, Ht, W, 1, 0, xt.data(), dyt.data(), P.sc0.data(), P.sh0.data(), m0[r].data(), i0[r].data(), 0.f,
+                        0.f, dxt.data(), ds.data(), db.data());
+    for (size_t c = 0; c < C; ++c) { G.sc0[c] += ds[c]; G.sh0[c] += db[c]; }
+  }
+  return G;
+}
+
+static void test_parallel_sgd(size_t K, size_t N, size_t C, size_t H, size_t W, bool nesterov, size_t num_batches) {
+  std::mt19937 gen(4242 + (unsigned)K + (nesterov ? 100 : 0));
+  auto ctx = MultiGPUContext::Make(K);
+  typedef GPUBatchArray3D<float> V;
+  typedef GPUArray4D<float> A;
+  typedef GPUArray1D<float> B;
+  const size_t full = N * C * H * W, steps = 3;
+  BlockParams P;
+  P.w1 = normal(gen, C * C * 9, std::sqrt(2.0f / (C * 9))); P.w2 = normal(gen, C * C * 9, std::sqrt(2.0f / (C * 9)));
+  P.sc0 = uniform(gen, C, 0.5f, 1.5f); P.sh0 = uniform(gen, C, -0.5f, 0.5f);
+  P.sc1 = uniform(gen, C, 0.5f, 1.5f); P.sh1 = uniform(gen, C, -0.5f, 0.5f);
+  std::vector<float> dY = normal(gen, full, 0.05f);
+
+  auto x_src = SrcOp<V>::Make(Shape3D(W, H, C), N, ctx->device_context(0));
+  vector<shared_ptr<ParamOp<A>>> w1(K), w2(K);
+  vector<shared_ptr<Var<A>>> w1v(K), w2v(K);
+  for (size_t r = 0; r < K; ++r) {
+    w1v[r] = w1[r] = ParamOp<A>::Make(Shape4D(3, 3, C, C), ctx->device_context(r));
+    w2v[r] = w2[r] = ParamOp<A>::Make(Shape4D(3, 3, C, C), ctx->device_context(r));
+  }
+  vector<shared_ptr<Var<V>>> xs(K, x_src);
+  auto inputs = SpatialScatter2DOp<V>::MakeParallel(xs, ctx);
+  auto switch_var = std::make_shared<bool>(false);
+  Conv2DShape cs;
+  cs.filters = C; cs.axes = {0, 1}; cs.kernel = {3, 3}; cs.dilate = {1, 1}; cs.stride = {1, 1}; cs.pad = {1, 1};
+  cs.halo_padded_input = true; cs.enable_hmma = false;
+  auto bnorm0 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, inputs, ctx);
+  auto relu0 = parallel_relu<V>(bnorm0.ops, ctx);
+  auto exch1 = HaloExch2DOp<V>::MakeParallel(1, HaloPad2DOp<V>::MakeParallel(1, relu0, ctx), ctx);
+  auto conv1 = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch1, w1v, ctx);
+  auto bnorm1 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, conv1, ctx);
+  auto relu1 = parallel_relu<V>(bnorm1.ops, ctx);
+  auto exch2 = HaloExch2DOp<V>::MakeParallel(1, HaloPad2DOp<V>::MakeParallel(1, relu1, ctx), ctx);
+  auto conv2 = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch2, w2v, ctx);
+  vector<vector<shared_ptr<Var<V>>>> join_inputs{inputs, conv2};
+  auto y_full = SpatialJoinedGather2DOp<V>::Make(parallel_sum<V>(join_inputs, ctx), ctx);
+  auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
+  sink->set_host_grad(dY.data());
+
+  vector<VarIdSet> params(K), grads(K), batch_stats(K), fixed_stats(K);
+  for (size_t r = 0; r < K; ++r) {
+    params[r].insert_all(bnorm0.params[r]); params[r].insert_all(bnorm1.params[r]);
+    grads[r].insert_all(bnorm0.grads[r]); grads[r].insert_all(bnorm1.grads[r]);
+    params[r].insert(w1[r]->vars().at(0)); params[r].insert(w2[r]->vars().at(0));
+    grads[r].insert(w1[r]->vars().at(1)); grads[r].insert(w2[r]->vars().at(1));
+    batch_stats[r].insert_all(bnorm0.batch_stats[r]); batch_stats[r].insert_all(bnorm1.batch_stats[r]);
+    fixed_stats[r].insert_all(bnorm0.fixed_stats[r]); fixed_stats[r].insert_all(bnorm1.fixed_stats[r]);
+  }
+  {  // initial values: rank 0 holds the real ones, the others something else that reset() must replace
+    TxnId init;
+    std::vector<float> zeros(C, 0.f);
+    for (size_t r = 0; r < K; ++r) {
+      const float f = r == 0 ? 1.0f : -3.0f;
+      auto scaled = [f](std::vector<float> v) { for (float &e : v) e *= f; return v; };
+      w1[r]->load(init, scaled(P.w1).data()); w2[r]->load(init, scaled(P.w2).data());
+      bnorm0.scales[r]->load(init, scaled(P.sc0).data()); bnorm0.shifts[r]->load(init, scaled(P.sh0).data());
+      bnorm1.scales[r]->load(init, scaled(P.sc1).data()); bnorm1.shifts[r]->load(init, scaled(P.sh1).data());
+      bnorm0.fixed_means[r]->load(init, zeros.data()); bnorm0.fixed_variances[r]->load(init, zeros.data());
+      bnorm1.fixed_means[r]->load(init, zeros.data()); bnorm1.fixed_variances[r]->load(init, zeros.data());
+    }
+  }
+  SGDConfig cfg;
+  cfg.minibatch_size = N * num_batches;
+  cfg.compute_batch_size = N;
+  cfg.step_size = std::make_shared<PiecewiseStepSchedule<double>>(0.05, 1, 0.03, 2, 0.02);
+  cfg.momentum = std::make_shared<ConstantSchedule<double>>(0.9);
+  cfg.nesterov = nesterov;
+  cfg.l2_reg = 1.0e-3;
+  cfg.batch_norm_rate = 0.25;
+  ParallelSGDOptimizer<float> opt(cfg, sink, params, grads, batch_stats, fixed_stats);
+  opt.reset(ctx);
+  CHECK(opt.param_dim() == 2 * C * C * 9 + 4 * C && opt.stat_dim() == 4 * C);
+
+  std::vector<std::vector<float>> batches;
+  size_t next_batch = 0;
+  function<void(TxnId, size_t, shared_ptr<Op>)> compute = [&](TxnId txn, size_t batch_size, shared_ptr<Op> loss) {
+    CHECK(batch_size == N);
+    for (size_t r = 0; r < K; ++r) {
+      loss->persist(txn, params[r]);
+      loss->persist(txn, fixed_stats[r]);
+    }
+    x_src->load(txn, batches.at(next_batch++).data());
+    loss->gradient(txn);
+  };
+
+  BlockParams M;  // momentum, per array
+  for (auto *v : {&M.w1, &M.w2}) v->assign(C * C * 9, 0.f);
+  for (auto *v : {&M.sc0, &M.sh0, &M.sc1, &M.sh1}) v->assign(C, 0.f);
+  BlockParams Lag = P;
+  const BlockParams P0 = P;
+  std::vector<std::vector<std::vector<float>>> running(K, std::vector<std::vector<float>>(4, std::vector<float>(C, 0.f)));
+  for (size_t t = 0; t < steps; ++t) {
+    batches.clear();
+    next_batch = 0;
+    for (size_t b = 0; b < num_batches; ++b) batches.push_back(uniform(gen, full, -1, 1));
+    opt.step(compute, ctx);
+    CHECK(next_batch == num_batches && opt.iter_count() == t + 1);
+
+    // CPU: gradients summed over the compute batches, statistics averaged online over them
+    BlockParams G;
+    std::vector<std::vector<std::vector<float>>> avg;
+    for (size_t b = 0; b < num_batches; ++b) {
+      std::vector<std::vector<std::vector<float>>> st;
+      BlockParams Gb = block_oracle_grads(K, N, C, H, W, batches[b], dY, P, &st);
+      if (b == 0) {
+        G = Gb;
+        avg = st;
+      } else {
+        auto ga = G.all(), gb = Gb.all();
+        for (size_t i = 0; i < ga.size(); ++i)
+          for (size_t j = 0; j < ga[i]->size(); ++j) (*ga[i])[j] += (*gb[i])[j];
+        const float a = 1.0f / (float)(b + 1);
+        for (size_t r = 0; r < K; ++r)
+          for (int q = 0; q < 4; ++q)
+            for (size_t c = 0; c < C; ++c) avg[r][q][c] += a * (st[r][q][c] - avg[r][q][c]);
+      }
+    }
+    const double steps_at[] = {0.05, 0.03, 0.02, 0.02};
+    auto pa = P.all(), ga = G.all(), ma = M.all(), la = Lag.all();
+    for (size_t i = 0; i < pa.size(); ++i) {
+      std::vector<float> sg(pa[i]->size());
+      const float *gl[1] = {ga[i]->data()};
+      orc_sgd_step(pa[i]->size(), 1, gl, 1.0e-3f, 0.9f, (float)steps_at[t], (float)steps_at[t + 1], nesterov ? 1 : 0,
+                   pa[i]->data(), ma[i]->data(), la[i]->data(), sg.data());
+    }
+    for (size_t r = 0; r < K; ++r)
+      for (int q = 0; q < 4; ++q) {
+        std::vector<float> stat(C);
+        orc_stat_step(C, 0.25f, avg[r][q].data(), running[r][q].data(), stat.data());
+      }
+
+    // every rank now holds the updated parameters; the fixed statistics hold the running ones
+    TxnId peek;
+    for (size_t r = 0; r < K; ++r) {
+      sink->persist(peek, params[r]);
+      sink->persist(peek, fixed_stats[r]);
+    }
+    ctx->sync();
+    double e_w = 0, e_bn = 0, e_stat = 0;
+    for (size_t r = 0; r < K; ++r) {
+      std::vector<float> g1(P.w1.size()), g2(P.w2.size()), a(C), b(C), c(C), d(C);
+      w1[r]->store(peek, g1.data()); w2[r]->store(peek, g2.data());
+      bnorm0.scales[r]->store(peek, a.data()); bnorm0.shifts[r]->store(peek, b.data());
+      bnorm1.scales[r]->store(peek, c.data()); bnorm1.shifts[r]->store(peek, d.data());
+      e_w = std::fmax(e_w, std::fmax(rel_err(g1, P.w1), rel_err(g2, P.w2)));
+      e_bn = std::fmax(e_bn, std::fmax(std::fmax(rel_err(a, P.sc0), rel_err(b, P.sh0)), std::fmax(rel_err(c, P.sc1), rel_err(d, P.sh1))));
+      std::vector<float> s(C);
+      bnorm0.fixed_means[r]->store(peek, s.data()); e_stat = std::fmax(e_stat, rel_err(s, running[r][0]));
+      bnorm0.fixed_variances[r]->store(peek, s.data()); e_stat = std::fmax(e_stat, rel_err(s, running[r][1]));
+      bnorm1.fixed_means[r]->store(peek, s.data()); e_stat = std::fmax(e_stat, rel_err(s, running[r][2]));
+      bnorm1.fixed_variances[r]->store(peek, s.data()); e_stat = std::fmax(e_stat, rel_err(s, running[r][3]));
+    }
+    std::printf("parallel sgd K=%zu N=%zu C=%zu %zux%zu nesterov=%d batches=%zu step %zu: rel-err filters %.2e bn %.2e stats %.2e\n",
+                K, N, C, H, W, (int)nesterov, num_batches, t, e_w, e_bn, e_stat);
+    CHECK(e_w <= 2e-5 && e_bn <= 2e-5 && e_stat <= 2e-5);
+  }
+  CHECK(rel_err(P.w1, P0.w1) > 1e-3 && rel_err(P.sc1, P0.sc1) > 1e-4);  // the steps did move the parameters
+  // the lagged parameters (before the look-ahead) come back on request
+  opt.reload_lagged_param(ctx);
+  {
+    TxnId peek;
+    sink->persist(peek, params[K - 1]);
+    std::vector<float> g1(P.w1.size());
+    w1[K - 1]->store(peek, g1.data());
+    CHECK(rel_err(g1, Lag.w1) <= 2e-5);
+    if (nesterov) CHECK(rel_err(g1, P.w1) > 1e-4);
+  }
+  opt.reload_param(ctx);
+}
+
+static void test_schedules() {
+  ConstantSchedule<double> c(0.1);
+  CHECK(c.at(0) == 0.1 && c.at(1000000) == 0.1);
+  PiecewiseStepSchedule<double> s(1.0, 10, 0.5, 20, 0.25);
+  CHECK(s.at(0) == 1.0 && s.at(9) == 1.0 && s.at(10) == 0.5 && s.at(19) == 0.5 && s.at(20) == 0.25 && s.at(99) == 0.25);
+  PiecewiseStepSchedule<double> s0(2.0);
+  CHECK(s0.at(5) == 2.0);
+  PiecewiseLinearSchedule<double> l(0.0, 10, 1.0);
+  CHECK(l.at(0) == 0.0 && std::fabs(l.at(5) - 0.5) < 1e-12 && l.at(10) == 1.0 && l.at(50) == 1.0);
+  PiecewiseLinearSchedule<double> l2(1.0, {{10, 2.0}, {30, 0.0}});
+  CHECK(std::fabs(l2.at(5) - 1.5) < 1e-12 && std::fabs(l2.at(20) - 1.0) < 1e-12 && l2.at(30) == 0.0);
+  VarIdSet set;
+  VarId a, b;
+  set.insert(a);
+  bool threw = false;
+  try { set.mask(a); } catch (const HazardError &) { threw = true; }
+  CHECK(threw);
+  set.lock();
+  CHECK(set.mask(a) && !set.mask(a) && !set.mask(b));
+  set.unlock();
+  set.lock();
+  CHECK(set.mask(a));
+  set.unlock();
+}
+
 int main(int argc, char **argv) {
   const std::string mode = argc > 1 ? argv[1] : "cpu";
   test_shapes();
   test_comm_protocol();
+  test_schedules();
   if (mode == "gpu") {
     test_txn_hazards();
     test_microbench_sequence();
@@ -638,6 +907,10 @@ int main(int argc, char **argv) {
     test_spatial_pool_graph(kAveragePool, 2, 3, 5, 8, 10);
     test_spatial_pool_graph(kMaxPool, 4, 8, 64, 112, 112);
     test_softmax_loss_op();
+    test_parallel_sgd(4, 2, 8, 16, 12, false, 1);
+    test_parallel_sgd(2, 2, 8, 8, 10, true, 1);
+    test_parallel_sgd(2, 2, 4, 8, 6, true, 2);
+    test_parallel_sgd(1, 3, 4, 6, 6, false, 2);
   }
   std::printf("%s: %d failure(s)\n", mode.c_str(), failures);
   return failures ? 1 : 0;
