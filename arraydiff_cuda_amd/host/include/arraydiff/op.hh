@@ -25,9 +25,11 @@
 
 #include <array>
 #include <cassert>
+#include <cmath>
 #include <functional>
 #include <map>
 #include <memory>
+#include <random>
 #include <set>
 #include <type_traits>
 #include <vector>
@@ -300,6 +302,8 @@ public:
   virtual size_t _store_grad(TxnId, VarIdSet &, size_t offset, FlatBatch *) { return offset; }
   // Only nodes that own long-lived variables (parameters, statistics, inputs) carry anything over.
   virtual void _persist(TxnId, VarIdSet &) {}
+  // Only parameters with an initialiser do anything (op.hh:654-656).
+  virtual void _init(TxnId, std::mt19937_64 *) {}
 
   // The members of `vars` reachable from this node, in the order the backward walk meets them, as
   // consecutive ranges of a flat device vector starting at `offset`; returns the end offset
@@ -311,6 +315,8 @@ public:
   size_t store_grad(TxnId txn, VarIdSet &vars, size_t offset, GPUMemory<float> *writer);
   // marks the members of `vars` to keep their value into transaction `txn` (src/op.cc:205-212)
   void persist(TxnId txn, VarIdSet &vars);
+  // gives every parameter below this node its initial value, in walk order (src/op.cc:196-203)
+  void init(TxnId txn, std::mt19937_64 *rng);
 
   // forward pass of everything this node depends on, in dependency order (op.cc:196-221)
   void eval(TxnId txn) {
@@ -418,6 +424,19 @@ public:
     return make_shared<ParamOp<A>>(shape, ctx);
   }
   ParamOp(typename A::Shape shape, shared_ptr<Context> ctx) : ctx_(ctx), y_(shape) {}
+  // The reference wraps a parameter in an InitOp (op.hh:1002-1060); here the parameter keeps its
+  // own initialiser, run by Op::init.
+  typedef function<void(A *, std::mt19937_64 *, shared_ptr<Context>)> InitFn;
+  static shared_ptr<ParamOp<A>> Make(typename A::Shape shape, InitFn init_fn, shared_ptr<Context> ctx) {
+    auto p = make_shared<ParamOp<A>>(shape, ctx);
+    p->init_fn_ = init_fn;
+    return p;
+  }
+  void set_init(InitFn init_fn) { init_fn_ = init_fn; }
+  virtual void _init(TxnId txn, std::mt19937_64 *rng) {
+    if (!init_fn_) return;
+    if (y_.val().overwrite(txn, id(), gpu_ctx_of(ctx_))) init_fn_(&y_.val().get_excl(txn, id()), rng, ctx_);
+  }
   template <typename T>
   void load(TxnId txn, const T *host) {
     GPUContext *c = gpu_ctx_of(ctx_);
@@ -481,7 +500,45 @@ private:
   }
   shared_ptr<Context> ctx_;
   VarData<A> y_;
+  InitFn init_fn_;
 };
+
+// Initialisers (src/op.cc:286-408): a constant, Xavier's uniform(+-sqrt(6/(fanin+fanout))) and
+// Kaiming's normal(0, sqrt(2/fanin)), drawn on the host in array order and copied in.
+template <typename A>
+typename ParamOp<A>::InitFn constant_init_gen(float c) {
+  return [c](A *val, std::mt19937_64 *, shared_ptr<Context> ctx) {
+    vector<float> buf(val->dim().flat_size(), c);
+    GPUConn conn = gpu_ctx_of(ctx)->conn();
+    val->load_sync(buf.data(), conn);
+  };
+}
+template <typename A>
+typename ParamOp<A>::InitFn zeros_init_gen() { return constant_init_gen<A>(0.0f); }
+template <typename A>
+typename ParamOp<A>::InitFn ones_init_gen() { return constant_init_gen<A>(1.0f); }
+template <typename A>
+typename ParamOp<A>::InitFn xavier_init_gen(size_t fanin, size_t fanout) {
+  return [fanin, fanout](A *val, std::mt19937_64 *rng, shared_ptr<Context> ctx) {
+    const float half_width = std::sqrt(6.0f / (float)(fanin + fanout));
+    std::uniform_real_distribution<float> dist(-half_width, half_width);
+    vector<float> buf(val->dim().flat_size());
+    for (float &v : buf) v = dist(*rng);
+    GPUConn conn = gpu_ctx_of(ctx)->conn();
+    val->load_sync(buf.data(), conn);
+  };
+}
+template <typename A>
+typename ParamOp<A>::InitFn kaiming_init_gen(size_t fanin, size_t fanout) {
+  (void)fanout;
+  return [fanin](A *val, std::mt19937_64 *rng, shared_ptr<Context> ctx) {
+    std::normal_distribution<float> dist(0.0f, std::sqrt(2.0f / (float)fanin));
+    vector<float> buf(val->dim().flat_size());
+    for (float &v : buf) v = dist(*rng);
+    GPUConn conn = gpu_ctx_of(ctx)->conn();
+    val->load_sync(buf.data(), conn);
+  };
+}
 
 // A variable that is a view of another op's data (outputs of HaloExch2DOp, op.hh:2653-2659).
 template <typename V>
@@ -958,12 +1015,13 @@ public:
   static RankVars make_rank_vars(size_t channels, shared_ptr<Context> dev_ctx) {
     RankVars v;
     typename B::Shape s(channels);
+    // initial values as in the reference's Make (op.hh:3173-3211): used only if Op::init runs
     v.batch_mean = ParamOp<B>::Make(s, dev_ctx);
     v.batch_variance = ParamOp<B>::Make(s, dev_ctx);
-    v.fixed_mean = ParamOp<B>::Make(s, dev_ctx);
-    v.fixed_variance = ParamOp<B>::Make(s, dev_ctx);
-    v.scale = ParamOp<B>::Make(s, dev_ctx);
-    v.shift = ParamOp<B>::Make(s, dev_ctx);
+    v.fixed_mean = ParamOp<B>::Make(s, zeros_init_gen<B>(), dev_ctx);
+    v.fixed_variance = ParamOp<B>::Make(s, ones_init_gen<B>(), dev_ctx);
+    v.scale = ParamOp<B>::Make(s, ones_init_gen<B>(), dev_ctx);
+    v.shift = ParamOp<B>::Make(s, zeros_init_gen<B>(), dev_ctx);
     return v;
   }
   static BatchNormOutput<V, B> Make(size_t channels, shared_ptr<Switch> switch_var, shared_ptr<Var<V>> input,
@@ -1109,6 +1167,24 @@ template <typename V>
 vector<shared_ptr<Var<V>>> parallel_relu(vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
   return CudnnActivationOp<V>::MakeParallel(kReluAct, inputs, ctx);
 }
+
+// y = scale * x; backward dx += scale * dy (ScaleOp, src/op.cc:1221-1290)
+template <typename T, typename V>
+class ScaleOp : public UnaryVarOp<V> {
+public:
+  static shared_ptr<Var<V>> Make(T scale, shared_ptr<Var<V>> input, shared_ptr<Context> ctx) {
+    return make_shared<ScaleOp<T, V>>(scale, input, ctx);
+  }
+  ScaleOp(T scale, shared_ptr<Var<V>> input, shared_ptr<Context> ctx) : UnaryVarOp<V>(input, ctx), scale_(scale) {
+    if (!input->offset().is_zero()) throw std::invalid_argument("ScaleOp: input must be packed");
+    this->y_ = VarData<V>(input->shape(), input->batch_shape());
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+
+private:
+  T scale_;
+};
 
 // y = x_0 + x_1 + ...; backward adds dy onto every input's gradient (JoinOp<V, SumJoin>, src/op.cc:744-867)
 class SumJoin {};
@@ -1268,6 +1344,46 @@ using CudnnPool2DOp = SlabPool2DOp<V>;
 // ---------------------------------------------------------------------------
 // softmax + negative log likelihood (1-D logits)
 // ---------------------------------------------------------------------------
+// (W, H, C) per example -> one vector of W*H*C per example, same order (parallel_flatten_nchw,
+// src/zoo.cc:1861): a copy forward, an accumulation backward.
+template <typename V, typename W>
+class FlattenNCHWOp : public virtual Op, public virtual Var<W> {
+public:
+  static shared_ptr<Var<W>> Make(shared_ptr<Var<V>> input, shared_ptr<Context> ctx) {
+    return make_shared<FlattenNCHWOp<V, W>>(input, ctx);
+  }
+  FlattenNCHWOp(shared_ptr<Var<V>> input, shared_ptr<Context> ctx)
+      : ctx_(ctx), input_(input), x_(input->data()),
+        y_(typename W::Shape(input->shape().flat_size()), input->batch_shape()) {
+    if (!input->offset().is_zero()) throw std::invalid_argument("FlattenNCHWOp: input must be packed");
+  }
+  virtual void _push(EpochId e, function<void(Op *)> apply) {
+    if (1 == stack_.push(e)) {
+      input_->_push(e, apply);
+      apply(this);
+    }
+  }
+  virtual void _pop(EpochId e, function<void(Op *)> apply) {
+    if (stack_.degree(e) == stack_.pop(e)) {
+      apply(this);
+      input_->_pop(e, apply);
+    }
+  }
+  virtual void _forward(TxnId txn);
+  virtual void _backward(TxnId txn);
+  virtual typename W::Shape shape() { return y_.shape(); }
+  virtual typename W::Shape offset() { return y_.offset(); }
+  virtual typename W::Shape stride() { return y_.stride(); }
+  virtual size_t batch_shape() { return y_.batch_shape(); }
+  virtual VarData<W> data() { return y_.clone(); }
+
+private:
+  shared_ptr<Context> ctx_;
+  shared_ptr<Var<V>> input_;
+  VarData<V> x_;
+  VarData<W> y_;
+};
+
 template <typename V, typename Label, typename Loss>
 class SoftmaxNLLLossOp : public virtual Op, public virtual Var<Loss> {
 public:
@@ -1294,11 +1410,15 @@ public:
   // same through batch_sum + ScaleOp, src/zoo.cc:1877-1878)
   virtual void _set_grad_sink(TxnId txn) {
     GPUContext *c = gpu_ctx_of(ctx_);
-    loss_.grad().accumulate(txn, id(), c, [c](Loss *g) {
+    const float seed = sink_grad_;
+    loss_.grad().accumulate(txn, id(), c, [c, seed](Loss *g) {
       GPUConn conn = c->conn();
-      g->as_view().set_constant(1.0f, conn);
+      g->as_view().set_constant(seed, conn);
     });
   }
+  // the gradient every example's loss is seeded with: 1 for the summed loss, 1/minibatch_size for
+  // the mean the trainers minimise (the ScaleOp before batch_sum, src/zoo.cc:1877)
+  void set_sink_grad(float g) { sink_grad_ = g; }
   template <typename T>
   void store_loss(TxnId txn, T *host) {
     GPUConn conn = gpu_ctx_of(ctx_)->conn();
@@ -1323,6 +1443,7 @@ private:
   VarData<V> y_;  // softmax output, kept for backward
   VarData<Label> label_;
   VarData<Loss> loss_;
+  float sink_grad_ = 1.0f;
 };
 template <typename V, typename Label, typename Loss>
 using CudnnSoftmaxNLLLossOp = SoftmaxNLLLossOp<V, Label, Loss>;

@@ -1,0 +1,194 @@
+// Builders of the spatially-parallel residual nets, by the reference's names
+// (include/arraydiff/zoo.hh:19-183, src/zoo.cc:133-161, 577-741, 1475-1909): parallel_conv2d,
+// spatial_parallel_residual_v2_conv2d, spatial_parallel_proj_residual_v2_conv2d and
+// ResNet<float>::MakeParallelResNet18.  Ranks are row-tiles of one GPU; every rank owns its copy
+// of every parameter, as in the reference, and ParallelSGDOptimizer keeps the copies equal.
+//
+// What differs from the reference's MakeParallelResNet18, all in the replicated tail after the
+// spatial part: the input arrives as NCHW floats (no transpose / scale ops); the tiles are
+// gathered once (SpatialJoinedGather2DOp replaces gather + all-reduce) and the global pooling,
+// the classifier and the loss run once instead of once per rank followed by a reduce and a
+// division by the rank count; the classifier is the 1x1 convolution over the pooled 1x1 image
+// that a bias-free linear layer is; the mean over the minibatch is the loss's sink gradient.
+#ifndef ARRAYDIFF_ZOO_HH
+#define ARRAYDIFF_ZOO_HH
+
+#include "arraydiff/op.hh"
+
+#include <memory>
+#include <vector>
+
+namespace arraydiff {
+
+template <typename V>
+class ParallelParamOp {
+public:
+  vector<shared_ptr<Var<V>>> ops;
+  vector<VarIdSet> params;
+  vector<VarIdSet> grads;
+};
+
+template <typename V>
+class ParallelBatchNormParamOp {
+public:
+  vector<shared_ptr<Var<V>>> ops;
+  vector<VarIdSet> params;
+  vector<VarIdSet> grads;
+  vector<VarIdSet> batch_stats;
+  vector<VarIdSet> fixed_stats;
+};
+
+inline void parallel_vars_insert_all(vector<VarIdSet> &dst, const vector<VarIdSet> &src) {
+  if (dst.size() != src.size()) throw std::invalid_argument("parallel_vars_insert_all: rank counts differ");
+  for (size_t rank = 0; rank < dst.size(); ++rank) dst[rank].insert_all(src[rank]);
+}
+
+// One filter variable per rank, one node for all of them (src/zoo.cc:133-161).  The reference's
+// enable_bias is false wherever the spatial nets call this; a bias is not implemented.
+template <typename V, typename A = GPUArray4D<float>>
+ParallelParamOp<V> parallel_conv2d(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs,
+                                   typename ParamOp<A>::InitFn kernel_init, bool enable_bias, shared_ptr<Context> ctx) {
+  if (enable_bias) throw std::invalid_argument("parallel_conv2d: bias is not implemented");
+  MultiGPUContext *mgpu_ctx = mgpu_ctx_of(ctx);
+  if (inputs.size() != mgpu_ctx->num_ranks()) throw std::invalid_argument("parallel_conv2d: one input per rank");
+  const size_t cin = inputs.at(0)->shape().shape[2];
+  ParallelParamOp<V> out;
+  vector<shared_ptr<Var<A>>> kernels;
+  for (size_t rank = 0; rank < inputs.size(); ++rank) {
+    auto kernel = ParamOp<A>::Make(Shape4D(shape.kernel[0], shape.kernel[1], cin, shape.filters), kernel_init,
+                                   mgpu_ctx->device_context(rank));
+    kernels.push_back(kernel);
+    out.params.push_back(VarIdSet::Singleton(kernel->vars().at(0)));
+    out.grads.push_back(VarIdSet::Singleton(kernel->vars().at(1)));
+  }
+  out.ops = CudnnConv2DOp<V, A, A>::MakeParallel(shape, inputs, kernels, ctx);
+  return out;
+}
+
+namespace detail {
+template <typename V>
+void add_batch_norm(ParallelBatchNormParamOp<V> &block, const ParallelBatchNormOutput<V, GPUArray1D<float>> &bn) {
+  parallel_vars_insert_all(block.params, bn.params);
+  parallel_vars_insert_all(block.grads, bn.grads);
+  parallel_vars_insert_all(block.batch_stats, bn.batch_stats);
+  parallel_vars_insert_all(block.fixed_stats, bn.fixed_stats);
+}
+template <typename V>
+ParallelBatchNormParamOp<V> empty_block(size_t num_ranks) {
+  ParallelBatchNormParamOp<V> b;
+  b.params.resize(num_ranks);
+  b.grads.resize(num_ranks);
+  b.batch_stats.resize(num_ranks);
+  b.fixed_stats.resize(num_ranks);
+  return b;
+}
+// batch norm -> rectifier -> halo pad -> halo exchange -> 3x3 conv with the given stride
+template <typename V>
+vector<shared_ptr<Var<V>>> padded_conv3x3(ParallelBatchNormParamOp<V> &block, Conv2DShape shape, size_t stride,
+                                          vector<shared_ptr<Var<V>>> activated, shared_ptr<Context> ctx) {
+  typedef GPUArray4D<float> A;
+  auto pad = HaloPad2DOp<V>::MakeParallel(1, activated, ctx);
+  auto exch = HaloExch2DOp<V>::MakeParallel(1, pad, ctx);
+  Conv2DShape cs = shape;
+  cs.stride = {stride, stride};
+  cs.halo_padded_input = true;
+  const size_t cin = activated.at(0)->shape().shape[2];
+  auto conv = parallel_conv2d<V, A>(cs, exch, kaiming_init_gen<A>(cin * shape.kernel[0] * shape.kernel[1], shape.filters),
+                                    false, ctx);
+  parallel_vars_insert_all(block.params, conv.params);
+  parallel_vars_insert_all(block.grads, conv.grads);
+  return conv.ops;
+}
+}  // namespace detail
+
+// x + conv(relu(bn(conv(relu(bn(x)))))) on every rank's tile (src/zoo.cc:577-652)
+template <typename V>
+ParallelBatchNormParamOp<V> spatial_parallel_residual_v2_conv2d(Conv2DShape shape, shared_ptr<bool> switch_var,
+                                                                vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+  typedef GPUArray1D<float> B;
+  const size_t cin = inputs.at(0)->shape().shape[2];
+  if (shape.filters != cin) throw std::invalid_argument("spatial_parallel_residual_v2_conv2d: the block keeps the channel count");
+  auto block = detail::empty_block<V>(inputs.size());
+  auto bnorm0 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(cin, switch_var, inputs, ctx);
+  detail::add_batch_norm(block, bnorm0);
+  auto conv1 = detail::padded_conv3x3(block, shape, 1, parallel_relu<V>(bnorm0.ops, ctx), ctx);
+  auto bnorm1 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(shape.filters, switch_var, conv1, ctx);
+  detail::add_batch_norm(block, bnorm1);
+  auto conv2 = detail::padded_conv3x3(block, shape, 1, parallel_relu<V>(bnorm1.ops, ctx), ctx);
+  vector<vector<shared_ptr<Var<V>>>> join_inputs{inputs, conv2};
+  block.ops = parallel_sum<V>(join_inputs, ctx);
+  return block;
+}
+
+// proj(a) + conv(relu(bn(conv_s(a)))) with a = relu(bn(x)), proj a strided 1x1 conv and conv_s the
+// strided 3x3 (src/zoo.cc:654-741): the block that changes extents and channel count
+template <typename V>
+ParallelBatchNormParamOp<V> spatial_parallel_proj_residual_v2_conv2d(Conv2DShape shape, size_t stride,
+                                                                     shared_ptr<bool> switch_var,
+                                                                     vector<shared_ptr<Var<V>>> inputs,
+                                                                     shared_ptr<Context> ctx) {
+  typedef GPUArray1D<float> B;
+  typedef GPUArray4D<float> A;
+  const size_t cin = inputs.at(0)->shape().shape[2];
+  auto block = detail::empty_block<V>(inputs.size());
+  auto bnorm0 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(cin, switch_var, inputs, ctx);
+  detail::add_batch_norm(block, bnorm0);
+  auto relu0 = parallel_relu<V>(bnorm0.ops, ctx);
+  Conv2DShape proj_shape = shape;
+  proj_shape.kernel = {1, 1};
+  proj_shape.stride = {stride, stride};
+  proj_shape.pad = {0, 0};
+  proj_shape.halo_padded_input = false;
+  auto proj = parallel_conv2d<V, A>(proj_shape, relu0, kaiming_init_gen<A>(cin, shape.filters), false, ctx);
+  parallel_vars_insert_all(block.params, proj.params);
+  parallel_vars_insert_all(block.grads, proj.grads);
+  auto conv1 = detail::padded_conv3x3(block, shape, stride, relu0, ctx);
+  auto bnorm1 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(shape.filters, switch_var, conv1, ctx);
+  detail::add_batch_norm(block, bnorm1);
+  auto conv2 = detail::padded_conv3x3(block, shape, 1, parallel_relu<V>(bnorm1.ops, ctx), ctx);
+  vector<vector<shared_ptr<Var<V>>>> join_inputs{proj.ops, conv2};
+  block.ops = parallel_sum<V>(join_inputs, ctx);
+  return block;
+}
+
+// include/arraydiff/zoo.hh:166-173
+class ConvNetConfig {
+public:
+  size_t input_w;
+  size_t input_h;
+  size_t batch_size;
+  size_t minibatch_size;
+};
+
+// include/arraydiff/zoo.hh:128-146, plus the two sources (the reference feeds them through
+// load_val on `inputs` / `labels`; here SrcOp::load does it)
+template <typename V, typename L>
+class ParallelCategoricalNLLBatchNormLoss {
+public:
+  shared_ptr<bool> batch_norm_use_fixed;
+  shared_ptr<Var<V>> op;                                   // logits
+  shared_ptr<SoftmaxNLLLossOp<V, GPUBatchArray0D<uint32_t>, L>> loss;  // per-example losses
+  shared_ptr<Op> sum_loss;                                 // what the optimizer differentiates
+  shared_ptr<SrcOp<GPUBatchArray3D<float>>> input;         // (W, H, 3) x batch, NCHW floats
+  shared_ptr<SrcOp<GPUBatchArray0D<uint32_t>>> label;
+  vector<VarIdSet> dev_params;
+  vector<VarIdSet> dev_grads;
+  vector<VarIdSet> dev_batch_stats;
+  vector<VarIdSet> dev_fixed_stats;
+};
+
+template <typename T>
+class ResNet {
+public:
+  // The reference's spatially-parallel 18-layer variant (src/zoo.cc:1475-1909): a 7x7 stem at
+  // stride 1 over halo 3, 3x3 max pooling at stride 2 over halo 1, then
+  // res2 x2 (64), res3 proj + plain (128), res4 proj + plain (256), res5 proj (512), res6 proj (512),
+  // batch norm, rectifier, global average pooling, a 1000-way classifier, softmax loss.
+  // Input extents must leave every stage's tile height even down to the last stride.
+  static ParallelCategoricalNLLBatchNormLoss<GPUBatchArray1D<T>, GPUBatchArray0D<T>> MakeParallelResNet18(
+      const ConvNetConfig &cfg, shared_ptr<Context> parallel_ctx, size_t num_classes = 1000);
+};
+
+}  // namespace arraydiff
+
+#endif

@@ -98,6 +98,11 @@ void Op::persist(TxnId txn, VarIdSet &vars) {
   _push(e, [txn, &vars](Op *op) { op->_persist(txn, vars); });
   _pop(e, [](Op *) {});
 }
+void Op::init(TxnId txn, std::mt19937_64 *rng) {
+  EpochId e;
+  _push(e, [txn, rng](Op *op) { op->_init(txn, rng); });
+  _pop(e, [](Op *) {});
+}
 
 // ---- SpatialScatter2DOp (op.cc:2396-2468) ----
 template <>
@@ -709,6 +714,41 @@ void CudnnActivationOp<V3>::_backward(TxnId txn) {
   }
 }
 
+// ---- ScaleOp (op.cc:1221-1290) ----
+template <>
+void ScaleOp<float, V3>::_forward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &x = x_.val().get(txn, id());
+  if (y_.val().overwrite(txn, id(), ctx)) {
+    GPUConn conn = ctx->conn();
+    V3 &y = y_.val().get_excl(txn, id());
+    const TileDims d = dims_of(x);
+    y.set_batch_size(d.N);
+    check_packed(x, "ScaleOp");
+    const uint64_t n = (uint64_t)d.W * d.H * d.C * d.N;
+    // y = scale * x + 0 * y needs a finite y: clear it first
+    adh_check(adh_fill_f32(n, 0.0f, y.as_view().dptr(), conn.stream()), "ScaleOp::_forward");
+    adh_check(adh_scale_add_f32(n, scale_, x.as_view().dptr(), 0.0f, y.as_view().dptr(), conn.stream()), "ScaleOp::_forward");
+  }
+}
+template <>
+void ScaleOp<float, V3>::_backward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  const size_t batch = x_.val().get(txn, id()).batch_size();
+  if (x_.grad().accumulate(txn, id(), ctx, [ctx, batch](V3 *g) {
+        GPUConn conn = ctx->conn();
+        g->set_batch_size(batch);
+        g->as_view().set_constant(0.0f, conn);
+      })) {
+    GPUConn conn = ctx->conn();
+    V3 &dy = y_.grad().get(txn, id());
+    const TileDims d = dims_of(dy);
+    adh_check(adh_scale_add_f32((uint64_t)d.W * d.H * d.C * d.N, scale_, dy.as_view().dptr(), 1.0f,
+                                x_.grad().get_mut(txn, id()).as_view().dptr(), conn.stream()),
+              "ScaleOp::_backward");
+  }
+}
+
 // ---- JoinOp<V, SumJoin> (op.cc:744-867) ----
 template <>
 void JoinOp<V3, SumJoin>::_forward(TxnId txn) {
@@ -835,6 +875,39 @@ void SlabPool2DOp<V3>::_backward(TxnId txn) {
 typedef GPUBatchArray1D<float> V1;
 typedef GPUBatchArray0D<uint32_t> L0;
 typedef GPUBatchArray0D<float> F0;
+
+// ---- FlattenNCHWOp (src/zoo.cc:1861) ----
+template <>
+void FlattenNCHWOp<V3, V1>::_forward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  V3 &x = x_.val().get(txn, id());
+  if (y_.val().overwrite(txn, id(), ctx)) {
+    GPUConn conn = ctx->conn();
+    V1 &y = y_.val().get_excl(txn, id());
+    check_packed(x, "FlattenNCHWOp");
+    y.set_batch_size(x.batch_size());
+    gpu_copy_d2d(y.as_view().dptr(), x.as_view().dptr(), x.dim().flat_size() * x.batch_size() * sizeof(float), conn.stream());
+  }
+}
+template <>
+void FlattenNCHWOp<V3, V1>::_backward(TxnId txn) {
+  GPUContext *ctx = gpu_ctx_of(ctx_);
+  const size_t batch = x_.val().get(txn, id()).batch_size();
+  bool first = false;
+  if (x_.grad().accumulate(txn, id(), ctx, [batch, &first](V3 *g) {
+        g->set_batch_size(batch);
+        first = true;
+      })) {
+    GPUConn conn = ctx->conn();
+    V3 &dx = x_.grad().get_mut(txn, id());
+    V1 &dy = y_.grad().get(txn, id());
+    const size_t n = dx.dim().flat_size() * batch;
+    if (first)
+      gpu_copy_d2d(dx.as_view().dptr(), dy.as_view().dptr(), n * sizeof(float), conn.stream());
+    else
+      array_add_packed<float>((uint32_t)n, dy.as_view().dptr(), dx.as_view().dptr(), conn.stream());
+  }
+}
 
 template <>
 void SoftmaxNLLLossOp<V1, L0, F0>::_forward(TxnId txn) {
