@@ -43,11 +43,15 @@ struct ConvGenParams {
   uint32_t N, C, M, MG, in_H, in_W, out_H, out_W;
   uint32_t si_r, si_c, so_r, so_c;
   uint32_t CC, nchunks, ntaps, TG;
-  uint32_t BR, BC;  // a block's output pixels: BR rows x BC columns, numbered row by row, 16 per n-tile
+  uint32_t BR, BC;  // a block's output pixels per image: BR rows x BC columns, numbered row by row, 16 per n-tile
+  // When an image's share (BR * BC = `live` pixels) fills at most half of the block's 256 pixel slots, the
+  // block takes NB consecutive images: slot f is pixel f % live of image f / live.  NG = ceil(N / NB) image
+  // groups per tile.  PPI: patch elements per image and channel; PP >= NB * PPI: pitch of a channel plane.
+  uint32_t NB, NG, live, PPI;
   uint32_t PCP, PP, w_lds_floats;
   uint32_t nsub, blocks_per_image;
   float beta;
-  FastDiv div_bpi, div_MG, div_N, div_PCP, div_BC;
+  FastDiv div_bpi, div_MG, div_N, div_PCP, div_BC, div_live, div_PPI;
   GenSub sub[kGenMaxSub];
   int16_t off_r[kGenMaxTaps], off_c[kGenMaxTaps];
 };
@@ -110,8 +114,9 @@ __global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenPara
   P.div_bpi.divmod(blockIdx.x, outer, inner);
   uint32_t img, mg;
   P.div_MG.divmod(outer, img, mg);
-  uint32_t tile, n;
-  P.div_N.divmod(img, tile, n);
+  uint32_t tile, ng;
+  P.div_N.divmod(img, tile, ng);
+  const uint32_t n = ng * P.NB;  // first image of this block
   uint32_t s = 0;
   while (s + 1u < P.nsub && inner >= P.sub[s + 1u].blk0) ++s;
   const GenSub &S = P.sub[s];
@@ -123,14 +128,16 @@ __global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenPara
 
   // this wave's four n-tiles: 16 consecutive pixels each of the block's BR x BC pixels numbered row by row;
   // slots past the last pixel compute pixel 0 again and store nothing
-  uint32_t pix[4], row_q[4], col_q[4];
+  uint32_t pix[4], row_q[4], col_q[4], img_q[4];
   bool live_q[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     const uint32_t f = ((wave * 4u + q) << 4) + l16;
-    P.div_BC.divmod(f, row_q[q], col_q[q]);
-    live_q[q] = f < P.BR * P.BC;
-    pix[q] = live_q[q] ? row_q[q] * P.si_r * P.PCP + col_q[q] * P.si_c : 0u;
+    uint32_t fi;
+    P.div_live.divmod(f, img_q[q], fi);
+    P.div_BC.divmod(fi, row_q[q], col_q[q]);
+    live_q[q] = img_q[q] < P.NB && n + img_q[q] < P.N;
+    pix[q] = live_q[q] ? img_q[q] * P.PPI + row_q[q] * P.si_r * P.PCP + col_q[q] * P.si_c : 0u;
     pix[q] += g * P.PP;
   }
   floatx4 acc[4][MT];
@@ -142,17 +149,20 @@ __global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenPara
   // where this thread's PFC elements of a channel plane come from (-1: outside the input or the patch)
   const int32_t in_r0 = (int32_t)(bi * P.BR * P.si_r) + S.min_r;
   const int32_t in_c0 = (int32_t)(bj * P.BC * P.si_c) + S.min_c;
+  const size_t plane = (size_t)P.in_H * P.in_W;
+  const int32_t image_elems = (int32_t)(P.C * (uint32_t)plane);  // only used when NB > 1 (the host bounds NB * C * plane)
   int32_t src_off[PFC];
 #pragma unroll
   for (int j = 0; j < PFC; ++j) {
     const uint32_t e = tid + j * kGenThreads;
-    uint32_t r, col;
-    P.div_PCP.divmod(e, r, col);
+    uint32_t b, ei, r, col;
+    P.div_PPI.divmod(e, b, ei);
+    P.div_PCP.divmod(ei, r, col);
     const int32_t gr = in_r0 + (int32_t)r, gc = in_c0 + (int32_t)col;
-    const bool ok = e < P.PP && r < S.PR && col < S.PC && gr >= 0 && gr < (int32_t)P.in_H && gc >= 0 && gc < (int32_t)P.in_W;
-    src_off[j] = ok ? gr * (int32_t)P.in_W + gc : -1;
+    const bool ok = b < P.NB && n + b < P.N && r < S.PR && col < S.PC && gr >= 0 && gr < (int32_t)P.in_H && gc >= 0 &&
+                    gc < (int32_t)P.in_W;
+    src_off[j] = ok ? (int32_t)b * image_elems + gr * (int32_t)P.in_W + gc : -1;
   }
-  const size_t plane = (size_t)P.in_H * P.in_W;
 
   float pre[CC * PFC];
   float4 wpre[WF];
@@ -247,7 +257,7 @@ __global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenPara
   for (int q = 0; q < 4; ++q) {
     const uint32_t i = bi * P.BR + row_q[q], j = bj * P.BC + col_q[q];
     if (!live_q[q] || i >= S.GI || j >= S.GJ) continue;
-    const size_t pix_out = (size_t)(S.o_r + i * P.so_r) * P.out_W + (S.o_c + j * P.so_c);
+    const size_t pix_out = (size_t)img_q[q] * P.M * P.out_H * P.out_W + (size_t)(S.o_r + i * P.so_r) * P.out_W + (S.o_c + j * P.so_c);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -325,13 +335,25 @@ static int gen_finish_plan(GenPlan *plan) {
     }
     if (bpi == 0) return ADH_EINVAL;
     P.PCP = max_PC;
-    // plane pitch: the four channel groups of a read start 16 banks apart
-    uint32_t pp = max_PR * P.PCP;
-    while (pp % 64u != 16u) ++pp;
-    P.PP = pp;
-    patch_bytes = (size_t)P.CC * P.PP * 4u;
-    // a thread stages 32 / CC elements of each channel plane
-    if (P.PP <= 256u * (32u / P.CC) && patch_bytes + (size_t)P.CC * wpitch * 4u <= kGenLdsBytes) break;
+    P.PPI = max_PR * P.PCP;
+    P.live = P.BR * P.BC;
+    // images per block: as many as fill the 256 pixel slots, fit LDS and the staging registers, and keep
+    // the offsets of a block's images within 31 bits
+    uint32_t nb = P.live <= 128u ? std::min(256u / P.live, std::max(P.N, 1u)) : 1u;
+    while (nb > 1u && (uint64_t)nb * P.C * P.in_H * P.in_W >= (1ull << 31)) --nb;
+    bool fits = false;
+    for (;; --nb) {
+      // plane pitch: the four channel groups of a read start 16 banks apart
+      uint32_t pp = nb * P.PPI;
+      while (pp % 64u != 16u) ++pp;
+      P.PP = pp;
+      patch_bytes = (size_t)P.CC * P.PP * 4u;
+      // a thread stages 32 / CC elements of each channel plane
+      fits = P.PP <= 256u * (32u / P.CC) && patch_bytes + (size_t)P.CC * wpitch * 4u <= kGenLdsBytes;
+      if (fits || nb == 1u) break;
+    }
+    P.NB = nb;
+    if (fits) break;
     if (P.CC == 8u) {
       P.CC = 4u;  // half the channels per chunk: twice the room per plane
       continue;
@@ -349,11 +371,14 @@ static int gen_finish_plan(GenPlan *plan) {
   P.w_lds_floats = P.TG * P.CC * wpitch;
   P.div_PCP = FastDiv(P.PCP);
   P.div_BC = FastDiv(P.BC);
+  P.div_live = FastDiv(P.live);
+  P.div_PPI = FastDiv(P.PPI);
+  P.NG = (P.N + P.NB - 1u) / P.NB;
   plan->lds_bytes = (size_t)P.w_lds_floats * 4u + patch_bytes;
   plan->wt_bytes = (size_t)P.MG * P.nchunks * P.ntaps * P.CC * MW * 4u;
   P.div_bpi = FastDiv(bpi);
   P.div_MG = FastDiv(P.MG);
-  P.div_N = FastDiv(P.N);
+  P.div_N = FastDiv(P.NG);
   FilterGenParams &F = plan->F;
   F.M = P.M;
   F.C = P.C;
@@ -456,7 +481,7 @@ static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *
   if (!workspace) return ADH_ENULL;
   if (!aligned_to(workspace, 256)) return ADH_EALIGN;
   if (workspace_bytes < plan->wt_bytes) return ADH_EWORKSPACE;
-  const uint64_t blocks = (uint64_t)num_tiles * P.N * P.MG * P.blocks_per_image;
+  const uint64_t blocks = (uint64_t)num_tiles * P.NG * P.MG * P.blocks_per_image;
   if (blocks == 0) return ADH_OK;
   if (blocks >= (1ull << 24)) return ADH_EINVAL;
   plan->F.w = w;

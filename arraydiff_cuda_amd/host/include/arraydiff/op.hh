@@ -304,6 +304,10 @@ public:
   virtual void _persist(TxnId, VarIdSet &) {}
   // Only parameters with an initialiser do anything (op.hh:654-656).
   virtual void _init(TxnId, std::mt19937_64 *) {}
+  // Not in the reference, which always computes every input gradient.  false: nothing below this
+  // node has parameters, so consumers need not produce (and this node's backward will not read)
+  // the gradient of its output; the first layer's input gradient is the case that matters.
+  virtual bool _requires_grad() { return true; }
 
   // The members of `vars` reachable from this node, in the order the backward walk meets them, as
   // consecutive ranges of a flat device vector starting at `offset`; returns the end offset
@@ -409,11 +413,15 @@ public:
   virtual void _forward(TxnId) {}
   virtual void _backward(TxnId) {}
   virtual void _persist(TxnId txn, VarIdSet &vars) { y_.rollover_all(txn, vars); }
+  // an input's gradient is computed (the reference's behaviour) unless the caller declines it
+  void set_requires_grad(bool r) { requires_grad_ = r; }
+  virtual bool _requires_grad() { return requires_grad_; }
   ARRAYDIFF_VAR_ACCESSORS(V)
 
 private:
   shared_ptr<Context> ctx_;
   VarData<V> y_;
+  bool requires_grad_ = true;
 };
 
 // A parameter (dense, no batch dimension), e.g. the conv filter GPUArray4D<float>.
@@ -553,6 +561,7 @@ public:
   }
   virtual void _forward(TxnId) {}
   virtual void _backward(TxnId) {}
+  virtual bool _requires_grad() { return op_->_requires_grad(); }
   ARRAYDIFF_VAR_ACCESSORS(V)
 
 private:
@@ -624,6 +633,8 @@ public:
       input_->_pop(e, apply);
     }
   }
+  // single-input ops have no parameters of their own
+  virtual bool _requires_grad() { return input_->_requires_grad(); }
   ARRAYDIFF_VAR_ACCESSORS(V)
 
 protected:
@@ -843,6 +854,11 @@ public:
       for (size_t r = inputs_.size(); r-- > 0;) inputs_.at(r)->_pop(e, apply);
     }
   }
+  virtual bool _requires_grad() {
+    for (auto &in : inputs_)
+      if (in->_requires_grad()) return true;
+    return false;
+  }
   virtual void _forward(TxnId txn);
   virtual void _backward(TxnId txn);
 
@@ -866,6 +882,12 @@ public:
   array<size_t, 2> pad;
   bool halo_padded_input;
   bool enable_hmma;
+  // Not in the reference.  A promise that the ranks' filter variables hold equal values (the
+  // parallel optimizer keeps them so): all tiles are then convolved in ONE launch with rank 0's
+  // filter, and the filter gradient of all tiles goes to rank 0's variable in one launch while
+  // the other ranks' gradients are zero.  The sum over ranks, which is all the optimizer uses,
+  // is the same.
+  bool replicated_filters = false;
 };
 
 // V = GPUBatchArray3D<float>, A = GPUArray4D<float> (filter, Shape4D(kw,kh,Cin,Cout) = KCRS).

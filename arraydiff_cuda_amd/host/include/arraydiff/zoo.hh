@@ -44,11 +44,16 @@ inline void parallel_vars_insert_all(vector<VarIdSet> &dst, const vector<VarIdSe
 }
 
 // One filter variable per rank, one node for all of them (src/zoo.cc:133-161).  The reference's
-// enable_bias is false wherever the spatial nets call this; a bias is not implemented.
+// enable_bias is false wherever the spatial nets call this; a bias is not implemented.  The node is
+// told that the copies are equal (Conv2DShape::replicated_filters): train such a graph with
+// ParallelSGDOptimizer, or load equal values into every rank's filter yourself.
 template <typename V, typename A = GPUArray4D<float>>
 ParallelParamOp<V> parallel_conv2d(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs,
                                    typename ParamOp<A>::InitFn kernel_init, bool enable_bias, shared_ptr<Context> ctx) {
   if (enable_bias) throw std::invalid_argument("parallel_conv2d: bias is not implemented");
+  // every rank's copy starts from rank 0's values (ParallelSGDOptimizer::reset) and receives the
+  // same update: one launch serves all tiles
+  shape.replicated_filters = true;
   MultiGPUContext *mgpu_ctx = mgpu_ctx_of(ctx);
   if (inputs.size() != mgpu_ctx->num_ranks()) throw std::invalid_argument("parallel_conv2d: one input per rank");
   const size_t cin = inputs.at(0)->shape().shape[2];

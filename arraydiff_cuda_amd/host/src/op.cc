@@ -122,6 +122,7 @@ void SpatialScatter2DOp<V3>::_forward(TxnId txn) {
 }
 template <>
 void SpatialScatter2DOp<V3>::_backward(TxnId txn) {
+  if (!_requires_grad()) return;  // nothing below needs this gradient, and nobody produced ours
   GPUContext *ctx = gpu_ctx_of(ctx_);
   V3 &dy = y_.grad().get(txn, id());
   const TileDims yd = dims_of(dy);
@@ -160,6 +161,7 @@ void SpatialGather2DOp<V3>::_forward(TxnId txn) {
 }
 template <>
 void SpatialGather2DOp<V3>::_backward(TxnId txn) {
+  if (!_requires_grad()) return;  // nothing below needs this gradient, and nobody produced ours
   GPUContext *ctx = gpu_ctx_of(ctx_);
   V3 &dy = y_.grad().get(txn, id());
   const TileDims yd = dims_of(dy);
@@ -207,16 +209,21 @@ void SpatialJoinedGather2DOp<V3>::_backward(TxnId txn) {
   const size_t batch = yd.N;
   for (size_t r = 0; r < xs_.size(); ++r) {
     GPUContext *dc = ctx->device_context(r).get();
-    if (xs_[r].grad().accumulate(txn, id(), dc, [dc, batch](V3 *g) {
-          GPUConn conn = dc->conn();
+    // the first toucher of a tile's gradient copies its rows, later ones add (the reference zeroes, then adds)
+    bool first = false;
+    if (xs_[r].grad().accumulate(txn, id(), dc, [batch, &first](V3 *g) {
           g->set_batch_size(batch);
-          g->as_view().set_constant(0.0f, conn);
+          first = true;
         })) {
       GPUConn conn = dc->conn();
       V3 &dx = xs_[r].grad().get_mut(txn, id());
       const TileDims xd = dims_of(dx);
-      slice2d_add_hw_nchw_packed<float>(xd.W, xd.H, yd.W, yd.H, xd.W, xd.H, xd.C, xd.N, dy.as_view().dptr(), 0,
-                                        (uint32_t)r * xd.H, dx.as_view().dptr(), 0, 0, conn.stream());
+      if (first)
+        slice2d_copy_hw_nchw_packed<float>(xd.W, xd.H, yd.W, yd.H, xd.W, xd.H, xd.C, xd.N, dy.as_view().dptr(), 0,
+                                           (uint32_t)r * xd.H, dx.as_view().dptr(), 0, 0, conn.stream());
+      else
+        slice2d_add_hw_nchw_packed<float>(xd.W, xd.H, yd.W, yd.H, xd.W, xd.H, xd.C, xd.N, dy.as_view().dptr(), 0,
+                                          (uint32_t)r * xd.H, dx.as_view().dptr(), 0, 0, conn.stream());
     }
   }
 }
@@ -243,20 +250,24 @@ void HaloPad2DOp<V3>::_forward(TxnId txn) {
 }
 template <>
 void HaloPad2DOp<V3>::_backward(TxnId txn) {
+  if (!_requires_grad()) return;  // nothing below needs this gradient, and nobody produced ours
   GPUContext *ctx = gpu_ctx_of(ctx_);
   V3 &dy = y_.grad().get(txn, id());
   const TileDims d = dims_of(dy);
   const size_t batch = d.N;
-  if (x_.grad().accumulate(txn, id(), ctx, [ctx, batch](V3 *g) {
-        GPUConn conn = ctx->conn();
+  // the first toucher of the input gradient overwrites it with the interior, later ones add
+  bool first = false;
+  if (x_.grad().accumulate(txn, id(), ctx, [batch, &first](V3 *g) {
         g->set_batch_size(batch);
-        g->as_view().set_constant(0.0f, conn);
+        first = true;
       })) {
     GPUConn conn = ctx->conn();
     V3 &dx = x_.grad().get_mut(txn, id());
     check_padded(dy, halo_pad_, "HaloPad2DOp");
-    adh_check(adh_halo_unpad_add_nchw(ADH_F32, (uint32_t)halo_pad_, d.W, d.H, d.C, d.N, dy.base_as_view().dptr(),
-                                      dx.as_view().dptr(), conn.stream()),
+    adh_check(first ? adh_halo_unpad_nchw(ADH_F32, (uint32_t)halo_pad_, d.W, d.H, d.C, d.N, dy.base_as_view().dptr(),
+                                          dx.as_view().dptr(), conn.stream())
+                    : adh_halo_unpad_add_nchw(ADH_F32, (uint32_t)halo_pad_, d.W, d.H, d.C, d.N, dy.base_as_view().dptr(),
+                                              dx.as_view().dptr(), conn.stream()),
               "HaloPad2DOp::_backward");
   }
 }
@@ -279,6 +290,7 @@ void HaloUnpad2DOp<V3>::_forward(TxnId txn) {
 }
 template <>
 void HaloUnpad2DOp<V3>::_backward(TxnId txn) {
+  if (!_requires_grad()) return;  // nothing below needs this gradient, and nobody produced ours
   GPUContext *ctx = gpu_ctx_of(ctx_);
   V3 &dy = y_.grad().get(txn, id());
   const TileDims d = dims_of(dy);
@@ -340,6 +352,7 @@ void HaloExch2DOp<V3>::_forward(TxnId txn) {
 }
 template <>
 void HaloExch2DOp<V3>::_backward(TxnId txn) {
+  if (!_requires_grad()) return;  // nothing below needs this gradient, and nobody produced ours
   MultiGPUContext *ctx = mgpu_ctx_of(ctx_);
   size_t num_writes = 0;
   for (size_t r = 0; r < ctx->num_ranks(); ++r) {
@@ -407,9 +420,11 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
   vector<size_t> todo;
   for (size_t r = 0; r < K; ++r)
     if (ys_[r].val().overwrite(txn, id(), rank_ctx(ctx_, r))) todo.push_back(r);
-  // group the ranks by filter buffer: one launch per distinct filter
+  // group the ranks by filter buffer: one launch per distinct filter (one in all when the filters
+  // are promised equal)
+  const bool replicated = shape_.replicated_filters;
   while (!todo.empty()) {
-    const float *w0 = kernels_[todo[0]].val().get(txn, id()).dptr();
+    const float *w0 = kernels_[replicated ? 0 : todo[0]].val().get(txn, id()).dptr();
     const void *xt[ADH_MAX_TILES];
     void *yt[ADH_MAX_TILES];
     uint32_t n = 0;
@@ -417,7 +432,7 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
     vector<size_t> rest;
     for (size_t r : todo) {
       A4 &w = kernels_[r].val().get(txn, id());
-      if (w.dptr() != w0) {
+      if (!replicated && w.dptr() != w0) {
         rest.push_back(r);
         continue;
       }
@@ -474,15 +489,21 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
         }
     }
   }
+  const bool replicated = shape_.replicated_filters;
+  if (replicated && !todo.empty()) {
+    // every rank's gradient was cleared above; all tiles now add into rank 0's
+    todo.clear();
+    for (size_t r = 0; r < K; ++r) todo.push_back(r);
+  }
   while (!todo.empty()) {
-    float *dw = kernels_[todo[0]].grad().get_mut(txn, id()).dptr();
+    float *dw = kernels_[replicated ? 0 : todo[0]].grad().get_mut(txn, id()).dptr();
     const void *xt[ADH_MAX_TILES];
     const void *dyt[ADH_MAX_TILES];
     uint32_t n = 0;
     TileDims d{};
     vector<size_t> rest;
     for (size_t r : todo) {
-      if (kernels_[r].grad().get(txn, id()).dptr() != dw) {
+      if (!replicated && kernels_[r].grad().get(txn, id()).dptr() != dw) {
         rest.push_back(r);
         continue;
       }
@@ -519,6 +540,7 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
   todo.clear();
   bool fresh[ADH_MAX_TILES] = {};
   for (size_t r = 0; r < K; ++r) {
+    if (!x_vars_[r]->_requires_grad()) continue;  // e.g. the first layer: nobody wants the image's gradient
     GPUContext *dc = rank_ctx(ctx_, r);
     const size_t batch = xs_[r].val().get(txn, id()).batch_size();
     bool *first = &fresh[r];
@@ -529,7 +551,7 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
       todo.push_back(r);
   }
   while (!todo.empty()) {
-    const float *w0 = kernels_[todo[0]].val().get(txn, id()).dptr();
+    const float *w0 = kernels_[replicated ? 0 : todo[0]].val().get(txn, id()).dptr();
     const bool first = fresh[todo[0]];
     const void *dyt[ADH_MAX_TILES];
     void *dxt[ADH_MAX_TILES];
@@ -537,7 +559,7 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     TileDims d{};
     vector<size_t> rest;
     for (size_t r : todo) {
-      if (kernels_[r].val().get(txn, id()).dptr() != w0 || fresh[r] != first) {
+      if ((!replicated && kernels_[r].val().get(txn, id()).dptr() != w0) || fresh[r] != first) {
         rest.push_back(r);
         continue;
       }
@@ -696,6 +718,7 @@ void CudnnActivationOp<V3>::_forward(TxnId txn) {
 }
 template <>
 void CudnnActivationOp<V3>::_backward(TxnId txn) {
+  if (!_requires_grad()) return;  // nothing below needs this gradient, and nobody produced ours
   GPUContext *ctx = gpu_ctx_of(ctx_);
   const size_t batch = x_.val().get(txn, id()).batch_size();
   // the first toucher of the input gradient overwrites it (the reference zeroes, then adds with beta = 1)
@@ -733,6 +756,7 @@ void ScaleOp<float, V3>::_forward(TxnId txn) {
 }
 template <>
 void ScaleOp<float, V3>::_backward(TxnId txn) {
+  if (!_requires_grad()) return;  // nothing below needs this gradient, and nobody produced ours
   GPUContext *ctx = gpu_ctx_of(ctx_);
   const size_t batch = x_.val().get(txn, id()).batch_size();
   if (x_.grad().accumulate(txn, id(), ctx, [ctx, batch](V3 *g) {
@@ -777,16 +801,20 @@ void JoinOp<V3, SumJoin>::_backward(TxnId txn) {
   const TileDims d = dims_of(dy);
   const size_t batch = d.N;
   for (size_t j = 0; j < xs_.size(); ++j) {
-    if (xs_[j].grad().accumulate(txn, id(), ctx, [ctx, batch](V3 *g) {
-          GPUConn conn = ctx->conn();
+    // the first toucher of an input's gradient copies dy into it, later ones add
+    bool first = false;
+    if (xs_[j].grad().accumulate(txn, id(), ctx, [batch, &first](V3 *g) {
           g->set_batch_size(batch);
-          g->as_view().set_constant(0.0f, conn);
+          first = true;
         })) {
       GPUConn conn = ctx->conn();
       V3 &dx = xs_[j].grad().get_mut(txn, id());
       check_packed(dx, "JoinOp");
-      adh_check(adh_add_f32((uint64_t)d.W * d.H * d.C * d.N, dy.as_view().dptr(), dx.as_view().dptr(), conn.stream()),
-                "JoinOp::_backward");
+      const uint64_t n = (uint64_t)d.W * d.H * d.C * d.N;
+      if (first)
+        gpu_copy_d2d(dx.as_view().dptr(), dy.as_view().dptr(), n * sizeof(float), conn.stream());
+      else
+        adh_check(adh_add_f32(n, dy.as_view().dptr(), dx.as_view().dptr(), conn.stream()), "JoinOp::_backward");
     }
   }
 }

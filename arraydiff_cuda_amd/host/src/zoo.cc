@@ -37,6 +37,7 @@ ParallelCategoricalNLLBatchNormLoss<V1, F0> ResNet<float>::MakeParallelResNet18(
 
   net.input = SrcOp<V3>::Make(Shape3D(cfg.input_w, cfg.input_h, 3), cfg.batch_size, root);
   net.label = SrcOp<L0>::Make(Shape0D(), cfg.batch_size, root);
+  net.input->set_requires_grad(false);  // the image's gradient is of no use to a trainer
 
   vector<shared_ptr<Var<V3>>> par_ys(num_ranks, net.input);
   par_ys = SpatialScatter2DOp<V3>::MakeParallel(par_ys, parallel_ctx);

@@ -25,6 +25,9 @@ CASES = [  # K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw
     (1, 1, 130, 20, 6, 6, 3, 3, 1, 1, 1, 1),   # many channel chunks, fewer than 16 columns
     (1, 1, 2, 3, 5, 5, 5, 5, 1, 1, 1, 1),      # a single output pixel
     (1, 1, 6, 5, 12, 70, 4, 4, 4, 4, 1, 1),    # 16 residue classes in backward-data
+    (1, 7, 12, 20, 10, 34, 3, 3, 2, 2, 1, 1),  # 4x16 outputs: four images per block, the last block holds three
+    (2, 5, 40, 48, 6, 18, 3, 3, 2, 2, 1, 1),   # 2x8 outputs (a late layer's tile): all five images in one block
+    (2, 6, 33, 20, 4, 16, 1, 1, 2, 2, 1, 1),   # strided 1x1 over a tiny tile, several images per block
 ]
 
 
