@@ -1059,12 +1059,17 @@ public:
     fill_sets(v, &out.params, &out.grads, &out.batch_stats, &out.fixed_stats);
     return out;
   }
+  // relu / out_halo (not in the reference): the node also applies the rectifier and writes into the
+  // interior of a tile padded by out_halo with a zeroed border, i.e. it stands for the chain
+  // CudnnBatchNorm2DOp -> CudnnActivationOp -> HaloPad2DOp (src/zoo.cc:596-604) in ONE pass over the
+  // data; its outputs then go straight to HaloExch2DOp.
   static ParallelBatchNormOutput<V, B> MakeParallel(size_t channels, shared_ptr<Switch> switch_var,
-                                                    vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+                                                    vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx,
+                                                    bool relu = false, size_t out_halo = 0) {
     MultiGPUContext *m = mgpu_ctx_of(ctx);
     vector<RankVars> vars;
     for (size_t r = 0; r < inputs.size(); ++r) vars.push_back(make_rank_vars(channels, m->device_context(r)));
-    auto op = make_shared<SlabBatchNorm2DOp<Switch, V, B>>(switch_var, inputs, vars, ctx);
+    auto op = make_shared<SlabBatchNorm2DOp<Switch, V, B>>(switch_var, inputs, vars, ctx, relu, out_halo);
     ParallelBatchNormOutput<V, B> out;
     for (size_t r = 0; r < inputs.size(); ++r) {
       out.ops.push_back(make_shared<NoOp<V>>(op, op->ys_.at(r).clone()));
@@ -1078,8 +1083,8 @@ public:
     return out;
   }
   SlabBatchNorm2DOp(shared_ptr<Switch> switch_var, vector<shared_ptr<Var<V>>> inputs, vector<RankVars> vars,
-                    shared_ptr<Context> ctx)
-      : ctx_(ctx), switch_var_(switch_var), x_vars_(inputs), vars_(vars) {
+                    shared_ptr<Context> ctx, bool relu = false, size_t out_halo = 0)
+      : ctx_(ctx), switch_var_(switch_var), x_vars_(inputs), vars_(vars), relu_(relu), out_halo_(out_halo) {
     if (inputs.empty() || inputs.size() != vars.size() || inputs.size() > ADH_MAX_TILES)
       throw std::invalid_argument("SlabBatchNorm2DOp: one set of parameters per input");
     for (size_t r = 0; r < inputs.size(); ++r) {
@@ -1088,7 +1093,14 @@ public:
       if (!inputs[r]->offset().is_zero())
         throw std::invalid_argument("SlabBatchNorm2DOp: input must be packed");
       xs_.push_back(inputs[r]->data());
-      ys_.push_back(VarData<V>(inputs[r]->shape(), inputs[r]->batch_shape()));
+      if (out_halo) {
+        const typename V::Shape sh = inputs[r]->shape();
+        ys_.push_back(VarData<V>(sh, typename V::Shape(out_halo, out_halo, 0),
+                                 typename V::Shape(sh.shape[0] + 2 * out_halo, sh.shape[1] + 2 * out_halo, sh.shape[2]).packed_stride(),
+                                 inputs[r]->batch_shape()));
+      } else {
+        ys_.push_back(VarData<V>(inputs[r]->shape(), inputs[r]->batch_shape()));
+      }
       batch_mean_.push_back(vars[r].batch_mean->data());
       batch_variance_.push_back(vars[r].batch_variance->data());
       fixed_mean_.push_back(vars[r].fixed_mean->data());
@@ -1154,6 +1166,8 @@ private:
   vector<VarData<V>> xs_, ys_;
   vector<VarData<B>> batch_mean_, batch_variance_, fixed_mean_, fixed_variance_, scale_, shift_;
   vector<TxnVar<B>> tmp_mean_, tmp_variance_;
+  bool relu_;
+  size_t out_halo_;
 };
 template <typename Switch, typename V, typename B>
 using CudnnBatchNorm2DOp = SlabBatchNorm2DOp<Switch, V, B>;

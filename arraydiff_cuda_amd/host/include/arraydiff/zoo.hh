@@ -87,22 +87,32 @@ ParallelBatchNormParamOp<V> empty_block(size_t num_ranks) {
   b.fixed_stats.resize(num_ranks);
   return b;
 }
-// batch norm -> rectifier -> halo pad -> halo exchange -> 3x3 conv with the given stride
+// halo exchange -> 3x3 conv with the given stride, over tiles that already carry a halo of 1
 template <typename V>
-vector<shared_ptr<Var<V>>> padded_conv3x3(ParallelBatchNormParamOp<V> &block, Conv2DShape shape, size_t stride,
-                                          vector<shared_ptr<Var<V>>> activated, shared_ptr<Context> ctx) {
+vector<shared_ptr<Var<V>>> exchanged_conv3x3(ParallelBatchNormParamOp<V> &block, Conv2DShape shape, size_t stride,
+                                             vector<shared_ptr<Var<V>>> padded, shared_ptr<Context> ctx) {
   typedef GPUArray4D<float> A;
-  auto pad = HaloPad2DOp<V>::MakeParallel(1, activated, ctx);
-  auto exch = HaloExch2DOp<V>::MakeParallel(1, pad, ctx);
+  auto exch = HaloExch2DOp<V>::MakeParallel(1, padded, ctx);
   Conv2DShape cs = shape;
   cs.stride = {stride, stride};
   cs.halo_padded_input = true;
-  const size_t cin = activated.at(0)->shape().shape[2];
+  const size_t cin = padded.at(0)->shape().shape[2];
   auto conv = parallel_conv2d<V, A>(cs, exch, kaiming_init_gen<A>(cin * shape.kernel[0] * shape.kernel[1], shape.filters),
                                     false, ctx);
   parallel_vars_insert_all(block.params, conv.params);
   parallel_vars_insert_all(block.grads, conv.grads);
   return conv.ops;
+}
+// batch norm -> rectifier -> halo pad as ONE node (the reference has three, src/zoo.cc:596-604),
+// then halo exchange -> 3x3 conv
+template <typename V>
+vector<shared_ptr<Var<V>>> bn_relu_pad_conv3x3(ParallelBatchNormParamOp<V> &block, Conv2DShape shape, size_t stride,
+                                               shared_ptr<bool> switch_var, vector<shared_ptr<Var<V>>> inputs,
+                                               shared_ptr<Context> ctx) {
+  const size_t cin = inputs.at(0)->shape().shape[2];
+  auto bnorm = CudnnBatchNorm2DOp<bool, V, GPUArray1D<float>>::MakeParallel(cin, switch_var, inputs, ctx, true, 1);
+  add_batch_norm(block, bnorm);
+  return exchanged_conv3x3(block, shape, stride, bnorm.ops, ctx);
 }
 }  // namespace detail
 
@@ -110,16 +120,11 @@ vector<shared_ptr<Var<V>>> padded_conv3x3(ParallelBatchNormParamOp<V> &block, Co
 template <typename V>
 ParallelBatchNormParamOp<V> spatial_parallel_residual_v2_conv2d(Conv2DShape shape, shared_ptr<bool> switch_var,
                                                                 vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
-  typedef GPUArray1D<float> B;
   const size_t cin = inputs.at(0)->shape().shape[2];
   if (shape.filters != cin) throw std::invalid_argument("spatial_parallel_residual_v2_conv2d: the block keeps the channel count");
   auto block = detail::empty_block<V>(inputs.size());
-  auto bnorm0 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(cin, switch_var, inputs, ctx);
-  detail::add_batch_norm(block, bnorm0);
-  auto conv1 = detail::padded_conv3x3(block, shape, 1, parallel_relu<V>(bnorm0.ops, ctx), ctx);
-  auto bnorm1 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(shape.filters, switch_var, conv1, ctx);
-  detail::add_batch_norm(block, bnorm1);
-  auto conv2 = detail::padded_conv3x3(block, shape, 1, parallel_relu<V>(bnorm1.ops, ctx), ctx);
+  auto conv1 = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, inputs, ctx);
+  auto conv2 = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, conv1, ctx);
   vector<vector<shared_ptr<Var<V>>>> join_inputs{inputs, conv2};
   block.ops = parallel_sum<V>(join_inputs, ctx);
   return block;
@@ -136,9 +141,10 @@ ParallelBatchNormParamOp<V> spatial_parallel_proj_residual_v2_conv2d(Conv2DShape
   typedef GPUArray4D<float> A;
   const size_t cin = inputs.at(0)->shape().shape[2];
   auto block = detail::empty_block<V>(inputs.size());
-  auto bnorm0 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(cin, switch_var, inputs, ctx);
+  // a = relu(bn(x)) feeds the unpadded projection and the padded 3x3: batch norm and rectifier fused, pad separate
+  auto bnorm0 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(cin, switch_var, inputs, ctx, true, 0);
   detail::add_batch_norm(block, bnorm0);
-  auto relu0 = parallel_relu<V>(bnorm0.ops, ctx);
+  auto relu0 = bnorm0.ops;
   Conv2DShape proj_shape = shape;
   proj_shape.kernel = {1, 1};
   proj_shape.stride = {stride, stride};
@@ -147,10 +153,8 @@ ParallelBatchNormParamOp<V> spatial_parallel_proj_residual_v2_conv2d(Conv2DShape
   auto proj = parallel_conv2d<V, A>(proj_shape, relu0, kaiming_init_gen<A>(cin, shape.filters), false, ctx);
   parallel_vars_insert_all(block.params, proj.params);
   parallel_vars_insert_all(block.grads, proj.grads);
-  auto conv1 = detail::padded_conv3x3(block, shape, stride, relu0, ctx);
-  auto bnorm1 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(shape.filters, switch_var, conv1, ctx);
-  detail::add_batch_norm(block, bnorm1);
-  auto conv2 = detail::padded_conv3x3(block, shape, 1, parallel_relu<V>(bnorm1.ops, ctx), ctx);
+  auto conv1 = detail::exchanged_conv3x3(block, shape, stride, HaloPad2DOp<V>::MakeParallel(1, relu0, ctx), ctx);
+  auto conv2 = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, conv1, ctx);
   vector<vector<shared_ptr<Var<V>>>> join_inputs{proj.ops, conv2};
   block.ops = parallel_sum<V>(join_inputs, ctx);
   return block;

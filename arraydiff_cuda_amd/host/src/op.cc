@@ -612,7 +612,7 @@ void SlabBatchNorm2DOp<bool, V3, B1>::_forward(TxnId txn) {
     y.set_batch_size(d.N);
     check_packed(x, "SlabBatchNorm2DOp");
     xt[n] = x.as_view().dptr();
-    yt[n] = y.as_view().dptr();
+    yt[n] = out_halo_ ? y.base_as_view().dptr() : y.as_view().dptr();
     sc[n] = scale_[r].val().get(txn, id()).dptr();
     sh[n] = shift_[r].val().get(txn, id()).dptr();
     if (fixed) {
@@ -636,7 +636,7 @@ void SlabBatchNorm2DOp<bool, V3, B1>::_forward(TxnId txn) {
   dc->reserve_scratch(ws);
   auto scratch = dc->get_scratch();
   GPUConn conn = dc->conn();
-  adh_check(adh_batchnorm2d_fwd_tiles(ADH_F32, fixed ? 0 : 1, n, d.N, d.C, d.H, d.W, 1.0e-5f, 0, 0, xt, sc, sh,
+  adh_check(adh_batchnorm2d_fwd_tiles(ADH_F32, fixed ? 0 : 1, n, d.N, d.C, d.H, d.W, 1.0e-5f, relu_ ? 1 : 0, (uint32_t)out_halo_, xt, sc, sh,
                                       fixed ? fm : nullptr, fixed ? fv : nullptr, yt, fixed ? nullptr : rm,
                                       fixed ? nullptr : rv, fixed ? nullptr : tm, fixed ? nullptr : tv, scratch->dptr(),
                                       scratch->size(), conn.stream()),
@@ -648,7 +648,7 @@ void SlabBatchNorm2DOp<bool, V3, B1>::_backward(TxnId txn) {
   const size_t K = xs_.size();
   // The first toucher of an input gradient overwrites it (the reference zeroes, then adds with beta = 1,
   // op.cc:4026-4031, 4059-4060); parameter gradients are small and keep the zero-then-add form.
-  bool mine[ADH_MAX_TILES] = {}, fresh[ADH_MAX_TILES] = {};
+  bool mine[ADH_MAX_TILES] = {}, fresh[ADH_MAX_TILES] = {}, pfresh[ADH_MAX_TILES] = {};
   for (size_t r = 0; r < K; ++r) {
     GPUContext *dc = rank_ctx(ctx_, r);
     const size_t batch = xs_[r].val().get(txn, id()).batch_size();
@@ -659,15 +659,19 @@ void SlabBatchNorm2DOp<bool, V3, B1>::_backward(TxnId txn) {
     });
     if (!mine[r]) continue;
     if (*switch_var_) throw std::logic_error("SlabBatchNorm2DOp: backward with fixed statistics is unimplemented");
-    auto zero = [dc](B1 *g) {
-      GPUConn conn = dc->conn();
-      g->set_constant(0.0f, conn);
-    };
-    if (!scale_[r].grad().accumulate(txn, id(), dc, zero) || !shift_[r].grad().accumulate(txn, id(), dc, zero))
+    // parameter gradients likewise: overwritten when this node is the first toucher of both
+    bool fresh_scale = false, fresh_shift = false;
+    if (!scale_[r].grad().accumulate(txn, id(), dc, [&fresh_scale](B1 *) { fresh_scale = true; }) ||
+        !shift_[r].grad().accumulate(txn, id(), dc, [&fresh_shift](B1 *) { fresh_shift = true; }))
       throw HazardError("SlabBatchNorm2DOp: parameter gradients already written by this node");
+    pfresh[r] = fresh_scale && fresh_shift;
+    if (fresh_scale != fresh_shift) {  // one was begun by another node: clear the other and add to both
+      GPUConn conn = dc->conn();
+      (fresh_scale ? scale_[r] : shift_[r]).grad().get_mut(txn, id()).set_constant(0.0f, conn);
+    }
   }
-  for (int pass = 0; pass < 2; ++pass) {
-    const bool first = pass == 0;
+  for (int pass = 0; pass < 4; ++pass) {
+    const bool first = (pass & 1) == 0, pfirst = (pass & 2) == 0;
     const void *xt[ADH_MAX_TILES], *dyt[ADH_MAX_TILES];
     void *dxt[ADH_MAX_TILES];
     const float *sc[ADH_MAX_TILES], *sh[ADH_MAX_TILES], *tm[ADH_MAX_TILES], *tv[ADH_MAX_TILES];
@@ -675,11 +679,12 @@ void SlabBatchNorm2DOp<bool, V3, B1>::_backward(TxnId txn) {
     uint32_t n = 0;
     TileDims d{};
     for (size_t r = 0; r < K; ++r) {
-      if (!mine[r] || fresh[r] != first) continue;
+      if (!mine[r] || fresh[r] != first || pfresh[r] != pfirst) continue;
       V3 &x = xs_[r].val().get(txn, id());
       d = dims_of(x);
       xt[n] = x.as_view().dptr();
-      dyt[n] = ys_[r].grad().get(txn, id()).as_view().dptr();
+      V3 &dy = ys_[r].grad().get(txn, id());
+      dyt[n] = out_halo_ ? dy.base_as_view().dptr() : dy.as_view().dptr();
       dxt[n] = xs_[r].grad().get_mut(txn, id()).as_view().dptr();
       sc[n] = scale_[r].val().get(txn, id()).dptr();
       sh[n] = shift_[r].val().get(txn, id()).dptr();
@@ -695,8 +700,9 @@ void SlabBatchNorm2DOp<bool, V3, B1>::_backward(TxnId txn) {
     dc->reserve_scratch(ws);
     auto scratch = dc->get_scratch();
     GPUConn conn = dc->conn();
-    adh_check(adh_batchnorm2d_bwd_tiles(ADH_F32, n, d.N, d.C, d.H, d.W, 0, 0, xt, dyt, sc, sh, tm, tv, dxt, dsc, dsh,
-                                        first ? 0.0f : 1.0f, 1.0f, scratch->dptr(), scratch->size(), conn.stream()),
+    adh_check(adh_batchnorm2d_bwd_tiles(ADH_F32, n, d.N, d.C, d.H, d.W, relu_ ? 1 : 0, (uint32_t)out_halo_, xt, dyt, sc, sh,
+                                        tm, tv, dxt, dsc, dsh, first ? 0.0f : 1.0f, pfirst ? 0.0f : 1.0f, scratch->dptr(),
+                                        scratch->size(), conn.stream()),
               "SlabBatchNorm2DOp::_backward");
   }
 }

@@ -84,12 +84,12 @@ ParallelCategoricalNLLBatchNormLoss<V1, F0> ResNet<float>::MakeParallelResNet18(
   proj(512);   // res5_1   (res5_2 is switched off in the reference, src/zoo.cc:1760)
   proj(512);   // res6_1   (res6_2 likewise, :1801)
 
-  auto bnorm_final = CudnnBatchNorm2DOp<bool, V3, B1>::MakeParallel(512, net.batch_norm_use_fixed, par_ys, parallel_ctx);
+  auto bnorm_final = CudnnBatchNorm2DOp<bool, V3, B1>::MakeParallel(512, net.batch_norm_use_fixed, par_ys, parallel_ctx, true, 0);
   parallel_vars_insert_all(net.dev_params, bnorm_final.params);
   parallel_vars_insert_all(net.dev_grads, bnorm_final.grads);
   parallel_vars_insert_all(net.dev_batch_stats, bnorm_final.batch_stats);
   parallel_vars_insert_all(net.dev_fixed_stats, bnorm_final.fixed_stats);
-  par_ys = parallel_relu<V3>(bnorm_final.ops, parallel_ctx);
+  par_ys = bnorm_final.ops;  // batch norm and rectifier in one node
 
   // The replicated tail (src/zoo.cc:1841-1873): every rank pools the gathered activation and applies
   // ITS copy of the classifier; the logits are summed over ranks and divided by the rank count.  With

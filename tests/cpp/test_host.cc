@@ -247,7 +247,8 @@ static void put_tile(std::vector<float> &full, const std::vector<float> &t, size
 // row-tiles of one GPU:  x -> BN -> ReLU -> HaloPad -> HaloExch -> conv -> BN -> ReLU -> HaloPad ->
 // HaloExch -> conv -> (+ x).  Every rank's batch norm uses its own tile's statistics.  Oracle: the
 // same chain with per-tile batch norms and UNSPLIT convolutions.
-static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, size_t W) {
+// fused: batch norm + rectifier + halo pad as one node (SlabBatchNorm2DOp with relu and out_halo) instead of three
+static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, size_t W, bool fused = false) {
   std::mt19937 gen(31337 + (unsigned)K);
   auto ctx = MultiGPUContext::Make(K);
   typedef GPUBatchArray3D<float> V;
@@ -270,14 +271,12 @@ static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, 
   Conv2DShape cs;
   cs.filters = C; cs.axes = {0, 1}; cs.kernel = {3, 3}; cs.dilate = {1, 1}; cs.stride = {1, 1}; cs.pad = {1, 1};
   cs.halo_padded_input = true; cs.enable_hmma = false;
-  auto bnorm0 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, inputs, ctx);
-  auto relu0 = parallel_relu<V>(bnorm0.ops, ctx);
-  auto pad1 = HaloPad2DOp<V>::MakeParallel(1, relu0, ctx);
+  auto bnorm0 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, inputs, ctx, fused, fused ? 1 : 0);
+  auto pad1 = fused ? bnorm0.ops : HaloPad2DOp<V>::MakeParallel(1, parallel_relu<V>(bnorm0.ops, ctx), ctx);
   auto exch1 = HaloExch2DOp<V>::MakeParallel(1, pad1, ctx);
   auto conv1 = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch1, vector<shared_ptr<Var<A>>>(K, w1_src), ctx);
-  auto bnorm1 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, conv1, ctx);
-  auto relu1 = parallel_relu<V>(bnorm1.ops, ctx);
-  auto pad2 = HaloPad2DOp<V>::MakeParallel(1, relu1, ctx);
+  auto bnorm1 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, conv1, ctx, fused, fused ? 1 : 0);
+  auto pad2 = fused ? bnorm1.ops : HaloPad2DOp<V>::MakeParallel(1, parallel_relu<V>(bnorm1.ops, ctx), ctx);
   auto exch2 = HaloExch2DOp<V>::MakeParallel(1, pad2, ctx);
   auto conv2 = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch2, vector<shared_ptr<Var<A>>>(K, w2_src), ctx);
   vector<vector<shared_ptr<Var<V>>>> join_inputs{inputs, conv2};
@@ -360,8 +359,8 @@ static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, 
     }
     for (size_t i = 0; i < full; ++i) dXr[i] += dY[i];
     const double ey = rel_err(Y, Yr), ex = rel_err(dX, dXr), ew1 = rel_err(dW1, dW1r), ew2 = rel_err(dW2, dW2r);
-    std::printf("residual block K=%zu N=%zu C=%zu %zux%zu rep %d: rel-err y %.2e dx %.2e dw1 %.2e dw2 %.2e bn params %.2e\n",
-                K, N, C, H, W, rep, ey, ex, ew1, ew2, e_param);
+    std::printf("residual block%s K=%zu N=%zu C=%zu %zux%zu rep %d: rel-err y %.2e dx %.2e dw1 %.2e dw2 %.2e bn params %.2e\n",
+                fused ? " (fused bn+relu+pad)" : "", K, N, C, H, W, rep, ey, ex, ew1, ew2, e_param);
     CHECK(ey <= 1e-5 && ex <= 2e-5 && ew1 <= 2e-5 && ew2 <= 1e-5 && e_param <= 1e-4);
   }
 }
@@ -903,6 +902,8 @@ int main(int argc, char **argv) {
     test_spatial_general_conv_graph(2, 2, 6, 10, 8, 9, 1, 1, 1);     // 1x1 over packed tiles (halo 0)
     test_spatial_residual_block(4, 2, 8, 16, 12);
     test_spatial_residual_block(2, 4, 64, 28, 28);
+    test_spatial_residual_block(4, 2, 8, 16, 12, true);
+    test_spatial_residual_block(2, 4, 64, 28, 28, true);
     test_spatial_pool_graph(kMaxPool, 4, 2, 8, 16, 12);
     test_spatial_pool_graph(kAveragePool, 2, 3, 5, 8, 10);
     test_spatial_pool_graph(kMaxPool, 4, 8, 64, 112, 112);
