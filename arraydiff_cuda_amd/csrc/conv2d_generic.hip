@@ -527,8 +527,11 @@ struct WgradGenParams {
   int16_t off_r[kGenMaxTaps], off_c[kGenMaxTaps];
 };
 
-template <typename T, int TAPS>
-__global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const WgradGenParams P) {
+// PACKED (few input channels, e.g. the 3-channel stem): the 16 columns of an accumulator tile are 16
+// (tap, input channel) pairs, pair q = 16 t + column = tap * Cin + ci, instead of 16 input channels of one tap;
+// all taps then fit one block and no matrix column is spent on channels that do not exist.
+template <typename T, int TAPS, bool PACKED>
+__global__ __launch_bounds__(kWgGenThreads, TAPS > 9 ? 1 : 2) void conv_gen_wgrad_kernel(const WgradGenParams P) {
   extern __shared__ __align__(16) float gen_lds[];
   float *dyl = gen_lds;
   float *patch = gen_lds + P.dy_lds_floats;
@@ -540,9 +543,19 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
 
   // lane L keeps the patch offset of tap tg * TAPS + L (absent taps of the last group read tap 0's place)
   int32_t delta_vec = 0;
-  {
+  if (!PACKED) {
     const uint32_t t = tg * TAPS + lane;
     if (lane < (uint32_t)TAPS && t < P.ntaps) delta_vec = (int32_t)P.off_r[t] * (int32_t)P.PCP + (int32_t)P.off_c[t];
+  }
+  // PACKED: this lane's (tap, channel) pair of every tile, as an offset into the patch (absent pairs read place 0)
+  int32_t pair_off[PACKED ? TAPS : 1];
+  if (PACKED) {
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t) {
+      const uint32_t q = (uint32_t)t * 16u + l16;
+      const uint32_t tap = q / P.Cin, ci = q - tap * P.Cin;
+      pair_off[t] = tap < P.ntaps ? (int32_t)(ci * P.PP) + (int32_t)P.off_r[tap] * (int32_t)P.PCP + (int32_t)P.off_c[tap] : 0;
+    }
   }
   floatx4 acc[TAPS][4];
 #pragma unroll
@@ -604,12 +617,12 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
       uint32_t r, c;
       P.div_OWT.divmod(p0, r, c);
       const float *arow = dyl + l16 * P.DP + p0;
-      const float *brow = patch + my_plane * P.PP + r * P.sh * P.PCP + c * P.sw;
+      const float *brow = patch + (PACKED ? 0u : my_plane * P.PP) + r * P.sh * P.PCP + c * P.sw;
       float a[4], b[TAPS];
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) a[mt] = arow[mt * 16 * P.DP];
 #pragma unroll
-      for (int t = 0; t < TAPS; ++t) b[t] = brow[__builtin_amdgcn_readlane(delta_vec, t)];
+      for (int t = 0; t < TAPS; ++t) b[t] = PACKED ? brow[pair_off[t]] : brow[__builtin_amdgcn_readlane(delta_vec, t)];
 #pragma unroll
       for (int t = 0; t < TAPS; ++t)
 #pragma unroll
@@ -648,7 +661,7 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
 struct WgradGenReduceParams {
   const float *partial;
   float *dw;
-  uint32_t Cin, Cout, ntaps, T, ntg, COG, CIT, nparts;
+  uint32_t Cin, Cout, ntaps, T, ntg, COG, CIT, nparts, packed;
   float beta;
 };
 
@@ -662,7 +675,13 @@ __global__ __launch_bounds__(256) void conv_gen_wgrad_reduce_kernel(const WgradG
     const uint32_t tg = (uint32_t)(r % Q.ntg);
     r /= Q.ntg;
     const uint32_t cit = (uint32_t)(r % Q.CIT), cog = (uint32_t)(r / Q.CIT);
-    const uint32_t co = cog * 64u + mt * 16u + (lane >> 4) * 4u + i, ci = cit * 16u + (lane & 15u), tap = tg * Q.T + t;
+    const uint32_t co = cog * 64u + mt * 16u + (lane >> 4) * 4u + i;
+    uint32_t ci = cit * 16u + (lane & 15u), tap = tg * Q.T + t;
+    if (Q.packed) {  // column = pair tap * Cin + ci
+      const uint32_t q = t * 16u + (lane & 15u);
+      tap = q / Q.Cin;
+      ci = q - tap * Q.Cin;
+    }
     if (co >= Q.Cout || ci >= Q.Cin || tap >= Q.ntaps) continue;
     float sum = 0.f;
     for (uint32_t p = 0; p < Q.nparts; ++p) sum += Q.partial[(size_t)p * stride + e];
@@ -675,6 +694,7 @@ struct WgradGenPlan {
   WgradGenParams P;
   size_t lds_bytes, partial_bytes;
   uint32_t blocks, nparts;
+  bool packed;
 };
 
 static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *plan) {
@@ -684,13 +704,20 @@ static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *p
   P.ntaps = g.kh * g.kw;
   P.T = P.ntaps == 1u ? 1u : P.ntaps <= 4u ? 4u : 9u;
   P.ntg = (P.ntaps + P.T - 1u) / P.T;
+  // few input channels and several taps: (tap, channel) pairs share the matrix columns, 4 or 10 tiles of 16
+  const uint32_t pairs = P.ntaps * g.Cin;
+  plan->packed = g.Cin <= 8u && P.ntaps > 1u && pairs <= 160u;
+  if (plan->packed) {
+    P.T = pairs <= 64u ? 4u : 10u;
+    P.ntg = 1;
+  }
   for (uint32_t a = 0; a < g.kh; ++a)
     for (uint32_t b = 0; b < g.kw; ++b) {
       P.off_r[a * g.kw + b] = (int16_t)(a * g.dh);
       P.off_c[a * g.kw + b] = (int16_t)(b * g.dw);
     }
   P.COG = (g.Cout + 63u) / 64u;
-  P.CIT = (g.Cin + 15u) / 16u;
+  P.CIT = plan->packed ? 1u : (g.Cin + 15u) / 16u;
   P.OWT = std::min<uint32_t>((g.OW + 3u) & ~3u, 64u);
   P.R = std::max<uint32_t>(1u, std::min<uint32_t>(g.OH, 64u / P.OWT));
   const uint32_t span_r = (g.kh - 1u) * g.dh + 1u, span_c = (g.kw - 1u) * g.dw + 1u;
@@ -735,12 +762,16 @@ static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *p
 template <typename T>
 static void launch_wgrad_gen(const WgradGenPlan &plan, hipStream_t st) {
   const WgradGenParams &P = plan.P;
-  if (P.T == 1u)
-    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 1>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+  if (plan.packed && P.T == 4u)
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 4, true>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+  else if (plan.packed)
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 10, true>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+  else if (P.T == 1u)
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 1, false>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
   else if (P.T == 4u)
-    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 4>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 4, false>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
   else
-    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 9>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 9, false>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
 }
 
 }  // namespace adh
@@ -862,6 +893,7 @@ int adh_conv2d_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, 
   Q.dw = dwt;
   Q.Cin = Cin; Q.Cout = Cout; Q.ntaps = plan.P.ntaps; Q.T = plan.P.T; Q.ntg = plan.P.ntg;
   Q.COG = plan.P.COG; Q.CIT = plan.P.CIT; Q.nparts = plan.nparts;
+  Q.packed = plan.packed ? 1u : 0u;
   Q.beta = beta;
   const size_t stride = (size_t)Q.COG * Q.CIT * Q.ntg * Q.T * 1024u;
   hipLaunchKernelGGL(conv_gen_wgrad_reduce_kernel, dim3((uint32_t)std::min<size_t>((stride + 255u) / 256u, 65535u)),
