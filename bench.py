@@ -106,6 +106,22 @@ def main():
               "inter-GPU collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
+    # End-to-end leg, run first as a child process (before this process touches the GPU): the synthetic-data trainer
+    # of the spatially-parallel ResNet-18 variant, every op of the path plus the optimizer, 4 row-tiles.
+    end_to_end = None
+    trainer = os.path.join(os.path.dirname(os.path.abspath(__file__)), "arraydiff_cuda_amd", "train_resnet18")
+    if not args.no_secondary and args.only is None:
+        import subprocess
+        if not os.path.exists(trainer):
+            print("bench.py: %s is not built (run __graft_entry__.build())" % trainer, file=sys.stderr)
+            sys.exit(3)
+        r = subprocess.run([trainer, "--ranks", "4", "--batch", "32", "--size", "256", "--steps", "10", "--warmup", "3"],
+                           capture_output=True, text=True, timeout=600)
+        if r.returncode != 0:
+            print("bench.py: the end-to-end trainer failed:\n" + r.stdout[-2000:] + r.stderr[-2000:], file=sys.stderr)
+            sys.exit(4)
+        end_to_end = json.loads(r.stdout.strip().splitlines()[-1])
+
     import numpy as np
     import torch
     from arraydiff_cuda_amd import capi
@@ -435,6 +451,8 @@ def main():
             note="reads 4 gradient vectors + parameters + momentum, writes momentum + parameters + lagged copy")
         del p_arrays, flat_g, flush_scratch
         out["secondary"] = sec
+    if end_to_end is not None:
+        out["end_to_end"] = end_to_end
 
     # ---- CPU baseline: the scalar port, single thread, on a bounded sample ----
     if not args.no_cpu:

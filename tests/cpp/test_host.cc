@@ -13,6 +13,7 @@
 
 #include "arraydiff/op.hh"
 #include "arraydiff/optimize.hh"
+#include "arraydiff/zoo.hh"
 
 extern "C" {
 // CPU oracle (oracle/adh_oracle.c): the checker
@@ -884,6 +885,71 @@ static void test_schedules() {
   set.unlock();
 }
 
+
+// The whole spatially-parallel ResNet-18 variant in evaluation mode (fixed batch-norm statistics, so that
+// nothing depends on how the rows are dealt to ranks): the logits for 2 and 4 row-tiles must equal those of
+// the unsplit net with the same parameters.  This exercises every halo exchange, the strided convolutions and
+// the pooling over tile borders, and the gather, end to end.
+static void test_resnet18_tiling_invariance() {
+  const size_t N = 2, H = 256, W = 32, classes = 10;
+  ConvNetConfig cfg;
+  cfg.input_w = W; cfg.input_h = H; cfg.batch_size = N; cfg.minibatch_size = N;
+  std::mt19937 gen(77);
+  std::vector<float> X = uniform(gen, N * 3 * H * W, 0.f, 1.f);
+  std::vector<uint32_t> labels = {3, 7};
+  std::vector<float> ref_logits, flat_host;
+  size_t param_dim = 0;
+  for (size_t K : {1, 2, 4}) {
+    auto ctx = MultiGPUContext::Make(K);
+    auto net = ResNet<float>::MakeParallelResNet18(cfg, ctx, classes);
+    std::mt19937_64 rng(1234);
+    {
+      TxnId init_txn;
+      net.sum_loss->init(init_txn, &rng);
+    }
+    TxnId txn;
+    for (size_t r = 0; r < K; ++r) {
+      net.sum_loss->persist(txn, net.dev_params[r]);
+      net.sum_loss->persist(txn, net.dev_fixed_stats[r]);
+    }
+    GPUContext *root = ctx->device_context(0).get();
+    if (K == 1) {
+      param_dim = net.sum_loss->store_val(txn, net.dev_params[0], 0, nullptr);
+      GPUMemory<float> flat = GPUMemory<float>::Zeros(param_dim, root);
+      CHECK(net.sum_loss->store_val(txn, net.dev_params[0], 0, &flat) == param_dim);
+      flat_host.resize(param_dim);
+      GPUConn conn = root->conn();
+      flat.store_sync(flat_host.data(), 0, param_dim, conn);
+    } else {
+      // every rank takes the unsplit net's parameters: a rank's variables come in the same order whatever K is
+      GPUMemory<float> flat(param_dim, root);
+      GPUConn conn = root->conn();
+      flat.load_sync(flat_host.data(), 0, param_dim, conn);
+      for (size_t r = 0; r < K; ++r) CHECK(net.sum_loss->load_val(txn, net.dev_params[r], 0, &flat) == param_dim);
+    }
+    *net.batch_norm_use_fixed = true;
+    net.input->load(txn, X.data());
+    net.label->load(txn, labels.data());
+    net.sum_loss->eval(txn);
+    ctx->sync();
+    std::vector<float> prob(N * classes), loss(N);
+    net.loss->store_prob(txn, prob.data());
+    net.loss->store_loss(txn, loss.data());
+    if (K == 1) {
+      ref_logits = prob;
+      bool spread = false;  // the net must not have collapsed to a constant output
+      for (size_t i = 1; i < classes; ++i) spread = spread || std::fabs(prob[i] - prob[0]) > 1e-4f;
+      CHECK(spread);
+      CHECK(param_dim > 11000000);
+    } else {
+      const double e = rel_err(prob, ref_logits);
+      std::printf("resnet18 eval, %zu row-tiles vs unsplit: rel-err of the class probabilities %.2e (loss %.5f %.5f)\n", K, e,
+                  loss[0], loss[1]);
+      CHECK(e <= 2e-5);
+    }
+  }
+}
+
 int main(int argc, char **argv) {
   const std::string mode = argc > 1 ? argv[1] : "cpu";
   test_shapes();
@@ -908,6 +974,7 @@ int main(int argc, char **argv) {
     test_spatial_pool_graph(kAveragePool, 2, 3, 5, 8, 10);
     test_spatial_pool_graph(kMaxPool, 4, 8, 64, 112, 112);
     test_softmax_loss_op();
+    test_resnet18_tiling_invariance();
     test_parallel_sgd(4, 2, 8, 16, 12, false, 1);
     test_parallel_sgd(2, 2, 8, 8, 10, true, 1);
     test_parallel_sgd(2, 2, 4, 8, 6, true, 2);
