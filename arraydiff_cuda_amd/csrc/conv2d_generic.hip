@@ -665,9 +665,14 @@ struct WgradGenReduceParams {
   float beta;
 };
 
+// 64 elements per workgroup; the partial sums of an element are dealt to four threads (part p to thread p % 4),
+// whose sums are then added in thread order: a fixed order, so the result has fixed bits.
 __global__ __launch_bounds__(256) void conv_gen_wgrad_reduce_kernel(const WgradGenReduceParams Q) {
+  __shared__ float part_sum[4][64];
   const size_t stride = (size_t)Q.COG * Q.CIT * Q.ntg * Q.T * 1024u;
-  for (size_t e = (size_t)blockIdx.x * 256u + threadIdx.x; e < stride; e += (size_t)gridDim.x * 256u) {
+  const uint32_t slice = threadIdx.x >> 6, le = threadIdx.x & 63u;
+  for (size_t e0 = (size_t)blockIdx.x * 64u; e0 < stride; e0 += (size_t)gridDim.x * 64u) {
+    const size_t e = e0 + le;  // stride is a multiple of 1024: every e is in range
     const uint32_t i = (uint32_t)(e & 3u), lane = (uint32_t)((e >> 2) & 63u), mt = (uint32_t)((e >> 8) & 3u);
     size_t r = e >> 10;
     const uint32_t t = (uint32_t)(r % Q.T);
@@ -682,11 +687,18 @@ __global__ __launch_bounds__(256) void conv_gen_wgrad_reduce_kernel(const WgradG
       tap = q / Q.Cin;
       ci = q - tap * Q.Cin;
     }
-    if (co >= Q.Cout || ci >= Q.Cin || tap >= Q.ntaps) continue;
+    const bool real = co < Q.Cout && ci < Q.Cin && tap < Q.ntaps;
     float sum = 0.f;
-    for (uint32_t p = 0; p < Q.nparts; ++p) sum += Q.partial[(size_t)p * stride + e];
-    float *out = Q.dw + ((size_t)co * Q.Cin + ci) * Q.ntaps + tap;
-    *out = Q.beta != 0.f ? *out + sum : sum;
+    if (real)
+      for (uint32_t p = slice; p < Q.nparts; p += 4u) sum += Q.partial[(size_t)p * stride + e];
+    __syncthreads();  // the previous round's sums have been read
+    part_sum[slice][le] = sum;
+    __syncthreads();
+    if (slice == 0u && real) {
+      sum = ((part_sum[0][le] + part_sum[1][le]) + part_sum[2][le]) + part_sum[3][le];
+      float *out = Q.dw + ((size_t)co * Q.Cin + ci) * Q.ntaps + tap;
+      *out = Q.beta != 0.f ? *out + sum : sum;
+    }
   }
 }
 
@@ -746,6 +758,7 @@ static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *p
   const uint64_t fixed = (uint64_t)P.COG * P.CIT * P.ntg;
   const size_t stride_bytes = (size_t)fixed * P.T * 1024u * 4u;
   uint64_t ps = std::max<uint64_t>(1u, 1024u / fixed);  // about four workgroups per CU: they hide each other's staging
+  if (P.T > 9u) ps = std::max<uint64_t>(1u, 256u / fixed);  // the ten-tile variant runs one workgroup per CU
   ps = std::min<uint64_t>(ps, units);
   while (ps > 1u && ps * stride_bytes > (256ull << 20)) ps /= 2u;
   if (fixed * ps >= (1ull << 24)) return ADH_EINVAL;
@@ -896,7 +909,7 @@ int adh_conv2d_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, 
   Q.packed = plan.packed ? 1u : 0u;
   Q.beta = beta;
   const size_t stride = (size_t)Q.COG * Q.CIT * Q.ntg * Q.T * 1024u;
-  hipLaunchKernelGGL(conv_gen_wgrad_reduce_kernel, dim3((uint32_t)std::min<size_t>((stride + 255u) / 256u, 65535u)),
+  hipLaunchKernelGGL(conv_gen_wgrad_reduce_kernel, dim3((uint32_t)std::min<size_t>((stride + 63u) / 64u, 65535u)),
                      dim3(256), 0, st, Q);
   return launch_status();
 }

@@ -95,6 +95,8 @@ def main():
                     help="untimed steps; a few hundred so that the GPU clocks have ramped up")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-secondary", action="store_true", help="time only the headline kernel")
+    ap.add_argument("--no-end-to-end", action="store_true",
+                    help="skip the end-to-end trainer leg (a child process; leave it out under a profiler)")
     ap.add_argument("--only", default=None,
                     help="time only the secondary entries whose name contains this text (for profiling one kernel)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -110,7 +112,7 @@ def main():
     # of the spatially-parallel ResNet-18 variant, every op of the path plus the optimizer, 4 row-tiles.
     end_to_end = None
     trainer = os.path.join(os.path.dirname(os.path.abspath(__file__)), "arraydiff_cuda_amd", "train_resnet18")
-    if not args.no_secondary and args.only is None:
+    if not args.no_secondary and not args.no_end_to_end and args.only is None:
         import subprocess
         if not os.path.exists(trainer):
             print("bench.py: %s is not built (run __graft_entry__.build())" % trainer, file=sys.stderr)
@@ -457,6 +459,12 @@ def main():
     # ---- CPU baseline: the scalar port, single thread, on a bounded sample ----
     if not args.no_cpu:
         import oracle
+        # the secondary entries above have written into the tiles (the halo reduce adds into them): pack and convolve
+        # once more so that the CPU and the GPU work on the same input
+        capi.check(capi.tiles_pack(K, p, W, H, C, N, X, tiles), "pack")
+        capi.check(lib.adh_conv3x3_slab_fwd_tiles(capi.ADH_F32, K, N, C, C, Ht, W, tile_tbl, wt.data_ptr(), y_tbl, 0.0,
+                                                  None, 0, stream), "conv fwd")
+        torch.cuda.synchronize()
         wn = wt.cpu().numpy()
         host_x = [t.cpu().numpy() for t in tiles]
         yc = np.empty((N, C, Ht, W), np.float32)
