@@ -398,6 +398,14 @@ void check_conv_input(V3 &x, const Conv2DShape &cs) {
   }
 }
 // scratch of the rank's context, grown to what the general conv entry points ask for
+// The 3x3 stride-1 kernels tile an image plane per workgroup; a tile of at most 64 pixels (the late layers of
+// a net split over several ranks) leaves them mostly idle, and the general kernel, which puts several images
+// into one workgroup, is 1.2 to 1.9 times faster there.
+template <typename Op>
+bool use_3x3_kernels(const Op &op, const TileDims &d) {
+  return op.is_3x3_unit() && (uint64_t)d.H * d.W > 64u;
+}
+
 void *conv_scratch(GPUContext *dc, int which, uint32_t n, const TileDims &d, const Conv2DShape &cs, size_t *bytes) {
   *bytes = adh_conv2d_workspace_bytes(which, ADH_F32, n, d.N, d.C, (uint32_t)cs.filters, d.H + 2 * (uint32_t)cs.pad[1],
                                       d.W + 2 * (uint32_t)cs.pad[0], (uint32_t)cs.kernel[1], (uint32_t)cs.kernel[0],
@@ -448,7 +456,7 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
-    if (is_3x3_unit()) {
+    if (use_3x3_kernels(*this, d)) {
       adh_check(adh_conv3x3_slab_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt, 0.0f,
                                            nullptr, 0, conn.stream()),
                 "SlabConv2DOp::_forward");
@@ -516,7 +524,7 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
-    if (is_3x3_unit()) {
+    if (use_3x3_kernels(*this, d)) {
       const size_t ws = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
                                                     d.H, d.W);
       dc->reserve_scratch(ws);
@@ -574,7 +582,7 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
     const float beta = first ? 0.0f : 1.0f;
-    if (is_3x3_unit()) {
+    if (use_3x3_kernels(*this, d)) {
       adh_check(adh_conv3x3_slab_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, w0, dyt, dxt,
                                                 beta, nullptr, 0, conn.stream()),
                 "SlabConv2DOp::_backward (data)");
