@@ -91,7 +91,7 @@ def test_general_conv_f32_vs_oracle(oracle, K, N, Cin, Cout, HP, WP, kh, kw, sh,
     assert capi.conv2d_fwd_tiles(d_xs, d_w, ys, N, Cin, Cout, HP, WP, *geo) == capi.ADH_ENULL
 
 
-@pytest.mark.parametrize("K,N,Cin,Cout,HP,WP,kh,kw,sh,sw,dh,dw", [CASES[0], CASES[2], CASES[3], CASES[4], CASES[6]])
+@pytest.mark.parametrize("K,N,Cin,Cout,HP,WP,kh,kw,sh,sw,dh,dw", [CASES[0], CASES[2], CASES[3], CASES[4], CASES[6], CASES[13]])
 def test_general_conv_bf16_vs_oracle(oracle, K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw):
     rng = np.random.default_rng(42 + WP)
     geo = (kh, kw, sh, sw, dh, dw)
