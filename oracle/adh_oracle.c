@@ -35,6 +35,12 @@
  *     avg_pool2d + autograd on the CPU; which element of a window receives the
  *     max gradient when several are equal is cuDNN's choice and is parity
  *     unpinned (this file and the kernels pick the first in row-major order).
+ *   - axpy / online average / flat copies / SGD step / running statistics :
+ *     pinned by closed forms (geometric momentum sum under a constant gradient,
+ *     (1 - step*l2)^t decay, textbook look-ahead Nesterov on a quadratic,
+ *     (1 - a)^t convergence of the online average) and round trips.  Which of
+ *     the two products of alpha*x + beta*y the reference's compiler fused, and
+ *     the order in which NCCL summed the ranks, are parity unpinned (one ulp).
  *   - cuDNN's exact fp32 summation order for conv and softmax: parity
  *     unpinned (not reproducible by the reference itself run to run); the
  *     tolerance-vs-unsplit criterion is used instead.
