@@ -130,16 +130,30 @@ __device__ __forceinline__ SgdOut sgd_elem(const SgdParams &P, float g, float p,
   return o;
 }
 
-template <bool VEC>
+// KG > 0: exactly KG gradient vectors, all of whose loads are issued before the first add (a loop over a
+// run-time count waits for each vector in turn); KG = 0: any count.
+template <bool VEC, int KG>
 __global__ __launch_bounds__(kOptBlock) void sgd_step_kernel(SgdParams P) {
   if (VEC) {
     const uint64_t stride = (uint64_t)gridDim.x * kOptBlock * 4;
     for (uint64_t i = ((uint64_t)blockIdx.x * kOptBlock + threadIdx.x) * 4; i < P.n; i += stride) {
       if (i + 4 <= P.n) {
-        float4 g = *reinterpret_cast<const float4 *>(P.grads[0] + i);
-        for (uint32_t r = 1; r < P.num_grads; ++r) {       // rank order: the result does not depend on timing
-          const float4 h = *reinterpret_cast<const float4 *>(P.grads[r] + i);
-          g.x += h.x; g.y += h.y; g.z += h.z; g.w += h.w;
+        float4 g;
+        if constexpr (KG > 0) {
+          float4 gv[KG];
+#pragma unroll
+          for (int r = 0; r < KG; ++r) gv[r] = *reinterpret_cast<const float4 *>(P.grads[r] + i);
+          g = gv[0];
+#pragma unroll
+          for (int r = 1; r < KG; ++r) {                     // rank order: the result does not depend on timing
+            g.x += gv[r].x; g.y += gv[r].y; g.z += gv[r].z; g.w += gv[r].w;
+          }
+        } else {
+          g = *reinterpret_cast<const float4 *>(P.grads[0] + i);
+          for (uint32_t r = 1; r < P.num_grads; ++r) {
+            const float4 h = *reinterpret_cast<const float4 *>(P.grads[r] + i);
+            g.x += h.x; g.y += h.y; g.z += h.z; g.w += h.w;
+          }
         }
         const float4 p = *reinterpret_cast<const float4 *>(P.param + i);
         const float4 m = *reinterpret_cast<const float4 *>(P.momentum + i);
@@ -341,10 +355,19 @@ int adh_sgd_step_f32(uint64_t n, uint32_t num_grads, const float *const *grads, 
   P.momentum = momentum_grad;
   P.lagged = lagged_param;
   P.sum_grad = sum_grad;
-  if (vec)
-    hipLaunchKernelGGL((sgd_step_kernel<true>), dim3(opt_grid(n, 4)), dim3(kOptBlock), 0, as_stream(stream), P);
+  const dim3 grid(opt_grid(n, vec ? 4 : 1)), block(kOptBlock);
+  if (!vec)
+    hipLaunchKernelGGL((sgd_step_kernel<false, 0>), grid, block, 0, as_stream(stream), P);
+  else if (num_grads == 1)
+    hipLaunchKernelGGL((sgd_step_kernel<true, 1>), grid, block, 0, as_stream(stream), P);
+  else if (num_grads == 2)
+    hipLaunchKernelGGL((sgd_step_kernel<true, 2>), grid, block, 0, as_stream(stream), P);
+  else if (num_grads == 4)
+    hipLaunchKernelGGL((sgd_step_kernel<true, 4>), grid, block, 0, as_stream(stream), P);
+  else if (num_grads == 8)
+    hipLaunchKernelGGL((sgd_step_kernel<true, 8>), grid, block, 0, as_stream(stream), P);
   else
-    hipLaunchKernelGGL((sgd_step_kernel<false>), dim3(opt_grid(n, 1)), dim3(kOptBlock), 0, as_stream(stream), P);
+    hipLaunchKernelGGL((sgd_step_kernel<true, 0>), grid, block, 0, as_stream(stream), P);
   return launch_status();
 }
 

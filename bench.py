@@ -51,13 +51,16 @@ def time_gpu(fn, reps, warmup):
 
 
 def time_gpu_flushed(fn, reps, scratch):
-    """Average milliseconds per call of fn() when every call is preceded by a rewrite of `scratch`
-    (512 MB, twice the on-package cache), so that fn's operands come from HBM: the time of a
-    (rewrite, fn) loop minus the time of the rewrite loop alone, best of three."""
+    """Average milliseconds per call of fn() when every call is preceded by a read of `scratch` (512 MB, twice
+    the on-package cache), so that fn's operands come from HBM and the cache holds clean lines: the time of a
+    (read, fn) loop minus the time of the read loop alone, best of three.  (Flushing by WRITING the buffer
+    leaves the cache full of dirty lines whose write-back is then charged to fn: about a fifth slower.)"""
+    import torch
     both, alone = [], []
+    flush = lambda: torch.amax(scratch)
     for i in range(3):
-        alone.append(time_gpu(lambda: scratch.fill_(1.0), reps, 3))
-        both.append(time_gpu(lambda: (scratch.fill_(1.0), fn()), reps, 3))
+        alone.append(time_gpu(flush, reps, 3))
+        both.append(time_gpu(lambda: (flush(), fn()), reps, 3))
     return max(min(both) - min(alone), 1e-6)
 
 
@@ -110,6 +113,10 @@ def main():
 
     # End-to-end leg, run first as a child process (before this process touches the GPU): the synthetic-data trainer
     # of the spatially-parallel ResNet-18 variant, every op of the path plus the optimizer, 4 row-tiles.
+    import torch
+    if torch.cuda.device_count() == 0:  # counting devices does not initialise the GPU
+        print("bench.py: no GPU visible; there is no CPU fallback", file=sys.stderr)
+        sys.exit(3)
     end_to_end = None
     trainer = os.path.join(os.path.dirname(os.path.abspath(__file__)), "arraydiff_cuda_amd", "train_resnet18")
     if not args.no_secondary and not args.no_end_to_end and args.only is None:
@@ -226,7 +233,7 @@ def main():
                  "unit": unit, "frac": round(ach / peak, 4), "work": work}
             if flushed:
                 # the warm figure above has its operands resident in the 256 MB on-package cache;
-                # this one rewrites 512 MB before every call
+                # this one reads 512 MB of something else before every call
                 msf = time_gpu_flushed(fn, 30, flush_scratch)
                 achf = work / (msf * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
                 e["ms_flushed"] = round(msf, 5)
