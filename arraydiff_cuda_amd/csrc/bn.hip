@@ -6,15 +6,16 @@
 //   bn_reduce_kernel<FWD>  per (tile, channel, split of the batch): sum (x - K) and sum (x - K)^2 with
 //                          K = the channel's first element, so that the sums stay small next to
 //                          the variance; fp32 per thread, tree over the block
-//   bn_finalize_fwd_kernel per (tile, channel): adds the splits in double; mean, 1/sqrt(var + eps),
-//                          running statistics, and a = scale / sqrt(var + eps)
-//   bn_apply_kernel        y = a*(x - mean) + shift (the difference first: the mean may be large next
+//   bn_apply_kernel        first, one thread per plane of the workgroup adds the channel's splits in double:
+//                          mean, 1/sqrt(var + eps), running statistics, a = scale / sqrt(var + eps) (there
+//                          is no finalize launch between the two passes); then
+//                          y = a*(x - mean) + shift (the difference first: the mean may be large next
 //                          to the deviation), optionally max(., 0), optionally written into the interior
 //                          of a halo-padded tile whose border it zeroes (BN -> ReLU -> HaloPad in
 //                          one pass over the data)
 // Backward mirrors it: reduce sum dy' and sum dy'*(x - mean) (dy' = dy masked by the rectifier, dy read
-// from the interior of the padded gradient tile when the forward wrote a padded tile), finalize
-// (parameter gradients, three coefficients), apply dx = beta*dx + k1*dy' + k2*(x - mean) + k3.
+// from the interior of the padded gradient tile when the forward wrote a padded tile); apply works out
+// the parameter gradients and three coefficients, then dx = beta*dx + k1*dy' + k2*(x - mean) + k3.
 #include "adh_common.h"
 
 #include <algorithm>
@@ -36,9 +37,8 @@ struct BnParams {
   float *o2[ADH_MAX_TILES];               // forward: saved mean
   float *o3[ADH_MAX_TILES];               // forward: saved 1/sqrt(var + eps)
   float *partial;                         // [tile][c][split][2]
-  float *coef;                            // [tile][c][8]
   uint32_t N, C, H, W, HW, p, split, n_per_split, tiles, groups_per_plane;
-  float eps, beta;
+  float eps, beta, beta_param;  // beta: input-gradient accumulation; beta_param: parameter-gradient accumulation
   int relu;
   FastDiv div_C, div_N, div_split, div_cols;  // div_cols: row length of the index that a kernel splits into (row, column)
 };
@@ -136,79 +136,85 @@ __global__ __launch_bounds__(kBnThreads) void bn_reduce_kernel(const BnParams P)
   }
 }
 
-// one thread per (tile, channel)
-template <typename T>
-__global__ __launch_bounds__(256) void bn_finalize_fwd_kernel(const BnParams P) {
-  const uint32_t tc = blockIdx.x * 256u + threadIdx.x;
-  if (tc >= P.tiles * P.C) return;
-  uint32_t tile, c;
-  P.div_C.divmod(tc, tile, c);
+// The five numbers the apply pass needs for one (tile, channel), worked out by ONE thread of every apply
+// workgroup that touches the channel (the sums of the splits are added in double, in split order, so every
+// workgroup gets the same bits).  `publish`: this thread also writes the channel's statistics (forward) or
+// parameter gradients (backward); exactly one thread per (tile, channel) in the grid is told to.
+//   MODE 0, training forward : cf = { a = scale / sqrt(var + eps), mean, shift }
+//   MODE 1, inference        : the same from the fixed statistics
+//   MODE 2, backward         : cf = { k1 = a, k2, k3, mean, shift };  dx = k1 dy' + k2 (x - mean) + k3
+template <typename T, int MODE>
+__device__ void bn_plane_coef(const BnParams &P, uint32_t tile, uint32_t c, bool publish, float *cf) {
+  const size_t tc = (size_t)tile * P.C + c;
+  if (MODE == 1) {
+    const double invstd = 1.0 / sqrt((double)P.second_in[tile][c] + (double)P.eps);
+    cf[0] = (float)((double)P.scale[tile][c] * invstd);
+    cf[1] = P.mean_in[tile][c];
+    cf[2] = P.shift[tile][c];
+    return;
+  }
   double s1 = 0.0, s2 = 0.0;
   for (uint32_t sp = 0; sp < P.split; ++sp) {
-    s1 += (double)P.partial[((size_t)tc * P.split + sp) * 2u];
-    s2 += (double)P.partial[((size_t)tc * P.split + sp) * 2u + 1u];
+    s1 += (double)P.partial[(tc * P.split + sp) * 2u];
+    s2 += (double)P.partial[(tc * P.split + sp) * 2u + 1u];
   }
   const double m = (double)P.N * (double)P.HW;
-  const double K = (double)bn_ld(reinterpret_cast<const T *>(P.x[tile]), (size_t)c * P.HW);
-  const double d = s1 / m, mean = K + d;
-  double var = s2 / m - d * d;
-  if (var < 0.0) var = 0.0;
-  const double invstd = 1.0 / sqrt(var + (double)P.eps);
-  if (P.o0[tile]) P.o0[tile][c] = (float)mean;
-  if (P.o1[tile]) P.o1[tile][c] = (float)(m > 1.0 ? var * m / (m - 1.0) : var);
-  if (P.o2[tile]) P.o2[tile][c] = (float)mean;
-  if (P.o3[tile]) P.o3[tile][c] = (float)invstd;
-  P.coef[(size_t)tc * 8u] = (float)((double)P.scale[tile][c] * invstd);
-  P.coef[(size_t)tc * 8u + 1u] = (float)mean;
-  P.coef[(size_t)tc * 8u + 2u] = P.shift[tile][c];
-}
-
-// inference: the same three numbers from fixed statistics
-__global__ __launch_bounds__(256) void bn_coef_infer_kernel(const BnParams P) {
-  const uint32_t tc = blockIdx.x * 256u + threadIdx.x;
-  if (tc >= P.tiles * P.C) return;
-  uint32_t tile, c;
-  P.div_C.divmod(tc, tile, c);
-  const double invstd = 1.0 / sqrt((double)P.second_in[tile][c] + (double)P.eps);
-  P.coef[(size_t)tc * 8u] = (float)((double)P.scale[tile][c] * invstd);
-  P.coef[(size_t)tc * 8u + 1u] = P.mean_in[tile][c];
-  P.coef[(size_t)tc * 8u + 2u] = P.shift[tile][c];
-}
-
-__global__ __launch_bounds__(256) void bn_finalize_bwd_kernel(const BnParams P) {
-  const uint32_t tc = blockIdx.x * 256u + threadIdx.x;
-  if (tc >= P.tiles * P.C) return;
-  uint32_t tile, c;
-  P.div_C.divmod(tc, tile, c);
-  double sd = 0.0, sdx = 0.0;
-  for (uint32_t sp = 0; sp < P.split; ++sp) {
-    sd += (double)P.partial[((size_t)tc * P.split + sp) * 2u];
-    sdx += (double)P.partial[((size_t)tc * P.split + sp) * 2u + 1u];
+  if (MODE == 0) {
+    const double K = (double)bn_ld(reinterpret_cast<const T *>(P.x[tile]), (size_t)c * P.HW);
+    const double d = s1 / m, mean = K + d;
+    double var = s2 / m - d * d;
+    if (var < 0.0) var = 0.0;
+    const double invstd = 1.0 / sqrt(var + (double)P.eps);
+    if (publish) {
+      if (P.o0[tile]) P.o0[tile][c] = (float)mean;
+      if (P.o1[tile]) P.o1[tile][c] = (float)(m > 1.0 ? var * m / (m - 1.0) : var);
+      if (P.o2[tile]) P.o2[tile][c] = (float)mean;
+      if (P.o3[tile]) P.o3[tile][c] = (float)invstd;
+    }
+    cf[0] = (float)((double)P.scale[tile][c] * invstd);
+    cf[1] = (float)mean;
+    cf[2] = P.shift[tile][c];
+  } else {
+    const double mean = P.mean_in[tile][c], invstd = P.second_in[tile][c], scale = P.scale[tile][c];
+    const double dshift = s1, dscale = s2 * invstd;  // sum dy' * (x - mean) * invstd
+    if (publish) {
+      P.o0[tile][c] = (float)((P.beta_param != 0.f ? (double)P.o0[tile][c] : 0.0) + dscale);
+      P.o1[tile][c] = (float)((P.beta_param != 0.f ? (double)P.o1[tile][c] : 0.0) + dshift);
+    }
+    // dx = a * (dy' - dshift/m - xhat * dscale/m),  xhat = (x - mean) * invstd
+    const double a = scale * invstd;
+    cf[0] = (float)a;
+    cf[1] = (float)(-a * invstd * dscale / m);
+    cf[2] = (float)(-a * dshift / m);
+    cf[3] = (float)mean;
+    cf[4] = P.shift[tile][c];  // the rectifier's mask needs the forward output's sign
   }
-  const double m = (double)P.N * (double)P.HW;
-  const double mean = P.mean_in[tile][c], invstd = P.second_in[tile][c], scale = P.scale[tile][c];
-  const double dshift = sd, dscale = sdx * invstd;  // sum dy' * (x - mean) * invstd
-  P.o0[tile][c] = (float)((P.beta != 0.f ? (double)P.o0[tile][c] : 0.0) + dscale);
-  P.o1[tile][c] = (float)((P.beta != 0.f ? (double)P.o1[tile][c] : 0.0) + dshift);
-  // dx = a * (dy' - dshift/m - xhat * dscale/m),  xhat = (x - mean) * invstd
-  const double a = scale * invstd;
-  P.coef[(size_t)tc * 8u] = (float)a;
-  P.coef[(size_t)tc * 8u + 1u] = (float)(-a * invstd * dscale / m);
-  P.coef[(size_t)tc * 8u + 2u] = (float)(-a * dshift / m);
-  P.coef[(size_t)tc * 8u + 3u] = (float)mean;
-  P.coef[(size_t)tc * 8u + 4u] = P.shift[tile][c];  // the rectifier's mask needs the forward output's sign
 }
 
 // a thread moves VEC consecutive elements of the padded output
 // plane (forward: any shape, the last partial group element by element) or of the packed gradient plane (backward:
 // VEC > 1 needs H*W and W to be whole numbers of groups)
-template <typename T, bool BWD, int VEC>
+// MODE as in bn_plane_coef: the first U threads of the workgroup work out the coefficients of its U planes
+// (there is no separate finalize launch), everyone else picks them up from LDS.
+template <typename T, int MODE, int VEC>
 __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const BnParams P) {
   typedef BnVec<T, VEC> Vec;
+  constexpr bool BWD = MODE == 2;
   constexpr int U = 4;  // planes per workgroup: a thread moves the same group of each, all loads before the first store
+  __shared__ float cf_s[U][8];
   const uint32_t WP = P.W + 2u * P.p, HPp = P.H + 2u * P.p;
   const uint32_t total = HPp * WP;
   const uint32_t planes = P.tiles * P.N * P.C;
+  if (threadIdx.x < (uint32_t)U) {
+    const uint32_t pl = blockIdx.x * U + threadIdx.x;
+    if (pl < planes) {
+      uint32_t tn, c, tile, n;
+      P.div_C.divmod(pl, tn, c);
+      P.div_N.divmod(tn, tile, n);
+      bn_plane_coef<T, MODE>(P, tile, c, blockIdx.y == 0u && n == 0u, cf_s[threadIdx.x]);
+    }
+  }
+  __syncthreads();
   const uint32_t gi = blockIdx.y * kBnThreads + threadIdx.x;  // group of VEC elements within a plane
   if (gi >= P.groups_per_plane) return;
   // where the group sits is the same for every plane
@@ -248,7 +254,7 @@ __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const BnParams P) 
     uint32_t tn, c, tile, n;
     P.div_C.divmod(pl, tn, c);
     P.div_N.divmod(tn, tile, n);
-    cf_u[u] = P.coef + ((size_t)tile * P.C + c) * 8u;
+    cf_u[u] = cf_s[u];
     const T *x = reinterpret_cast<const T *>(P.x[tile]) + ((size_t)n * P.C + c) * P.HW;
     if (!BWD) {
       out_u[u] = reinterpret_cast<T *>(P.out[tile]) + ((size_t)n * P.C + c) * total;
@@ -370,7 +376,6 @@ static int bn_common(int dtype, uint32_t num_tiles, uint32_t N, uint32_t C, uint
   if (!aligned_to(workspace, 256)) return ADH_EALIGN;
   if (workspace_bytes < bn_ws_bytes(num_tiles, C, P->split)) return ADH_EWORKSPACE;
   P->partial = reinterpret_cast<float *>(workspace);
-  P->coef = P->partial + (size_t)num_tiles * C * P->split * 2u;
   return ADH_OK;
 }
 
@@ -430,7 +435,7 @@ int adh_batchnorm2d_fwd_tiles(int dtype, int training, uint32_t num_tiles, uint3
   P.relu = relu ? 1 : 0;
   P.div_cols = FastDiv(W + 2u * out_halo);  // the apply kernel walks the padded output plane
   hipStream_t st = as_stream(stream);
-  const uint32_t tc = num_tiles * C, fin_blocks = (tc + 255u) / 256u;
+  const uint32_t tc = num_tiles * C;
   const uint32_t vec = (uint32_t)(16 / dtype_size(dtype));
   const bool wide = (H * W) % vec == 0;  // the statistics pass reads whole 16-byte groups
   const uint32_t gpp = ((H + 2u * out_halo) * (W + 2u * out_halo) + vec - 1u) / vec;
@@ -439,18 +444,19 @@ int adh_batchnorm2d_fwd_tiles(int dtype, int training, uint32_t num_tiles, uint3
     if (dtype == ADH_F32) {
       if (wide) hipLaunchKernelGGL((bn_reduce_kernel<float, false, 4>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
       else hipLaunchKernelGGL((bn_reduce_kernel<float, false, 1>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
-      hipLaunchKernelGGL(bn_finalize_fwd_kernel<float>, dim3(fin_blocks), dim3(256), 0, st, P);
     } else {
       if (wide) hipLaunchKernelGGL((bn_reduce_kernel<uint16_t, false, 8>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
       else hipLaunchKernelGGL((bn_reduce_kernel<uint16_t, false, 1>), dim3(tc * P.split), dim3(kBnThreads), 0, st, P);
-      hipLaunchKernelGGL(bn_finalize_fwd_kernel<uint16_t>, dim3(fin_blocks), dim3(256), 0, st, P);
     }
-  } else {
-    hipLaunchKernelGGL(bn_coef_infer_kernel, dim3(fin_blocks), dim3(256), 0, st, P);
   }
   const dim3 grid = bn_apply_grid(&P, gpp);
-  if (dtype == ADH_F32) hipLaunchKernelGGL((bn_apply_kernel<float, false, 4>), grid, dim3(kBnThreads), 0, st, P);
-  else hipLaunchKernelGGL((bn_apply_kernel<uint16_t, false, 8>), grid, dim3(kBnThreads), 0, st, P);
+  if (training) {
+    if (dtype == ADH_F32) hipLaunchKernelGGL((bn_apply_kernel<float, 0, 4>), grid, dim3(kBnThreads), 0, st, P);
+    else hipLaunchKernelGGL((bn_apply_kernel<uint16_t, 0, 8>), grid, dim3(kBnThreads), 0, st, P);
+  } else {
+    if (dtype == ADH_F32) hipLaunchKernelGGL((bn_apply_kernel<float, 1, 4>), grid, dim3(kBnThreads), 0, st, P);
+    else hipLaunchKernelGGL((bn_apply_kernel<uint16_t, 1, 8>), grid, dim3(kBnThreads), 0, st, P);
+  }
   return launch_status();
 }
 
@@ -492,10 +498,11 @@ int adh_batchnorm2d_bwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_
   const bool wide = W % vec == 0;
   P.div_cols = FastDiv(wide ? W / vec : W);
   hipStream_t st = as_stream(stream);
-  const uint32_t tc = num_tiles * C, fin_blocks = (tc + 255u) / 256u;
+  const uint32_t tc = num_tiles * C;
   if (((wide ? H * W / vec : H * W) + kBnThreads - 1u) / kBnThreads > 65535u) return ADH_EINVAL;  // grid.y
   const dim3 rgrid(tc * P.split), agrid = bn_apply_grid(&P, wide ? H * W / vec : H * W);
-  P.beta = beta_param;
+  P.beta = beta_data;
+  P.beta_param = beta_param;
   if (dtype == ADH_F32) {
     if (wide) hipLaunchKernelGGL((bn_reduce_kernel<float, true, 4>), rgrid, dim3(kBnThreads), 0, st, P);
     else hipLaunchKernelGGL((bn_reduce_kernel<float, true, 1>), rgrid, dim3(kBnThreads), 0, st, P);
@@ -503,14 +510,12 @@ int adh_batchnorm2d_bwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_
     if (wide) hipLaunchKernelGGL((bn_reduce_kernel<uint16_t, true, 8>), rgrid, dim3(kBnThreads), 0, st, P);
     else hipLaunchKernelGGL((bn_reduce_kernel<uint16_t, true, 1>), rgrid, dim3(kBnThreads), 0, st, P);
   }
-  hipLaunchKernelGGL(bn_finalize_bwd_kernel, dim3(fin_blocks), dim3(256), 0, st, P);
-  P.beta = beta_data;
   if (dtype == ADH_F32) {
-    if (wide) hipLaunchKernelGGL((bn_apply_kernel<float, true, 4>), agrid, dim3(kBnThreads), 0, st, P);
-    else hipLaunchKernelGGL((bn_apply_kernel<float, true, 1>), agrid, dim3(kBnThreads), 0, st, P);
+    if (wide) hipLaunchKernelGGL((bn_apply_kernel<float, 2, 4>), agrid, dim3(kBnThreads), 0, st, P);
+    else hipLaunchKernelGGL((bn_apply_kernel<float, 2, 1>), agrid, dim3(kBnThreads), 0, st, P);
   } else {
-    if (wide) hipLaunchKernelGGL((bn_apply_kernel<uint16_t, true, 8>), agrid, dim3(kBnThreads), 0, st, P);
-    else hipLaunchKernelGGL((bn_apply_kernel<uint16_t, true, 1>), agrid, dim3(kBnThreads), 0, st, P);
+    if (wide) hipLaunchKernelGGL((bn_apply_kernel<uint16_t, 2, 8>), agrid, dim3(kBnThreads), 0, st, P);
+    else hipLaunchKernelGGL((bn_apply_kernel<uint16_t, 2, 1>), agrid, dim3(kBnThreads), 0, st, P);
   }
   return launch_status();
 }

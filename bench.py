@@ -383,12 +383,12 @@ def main():
         bn_ws = torch.empty(bn_ws_bytes // 4, device="cuda")
         packed_b = K * N * C * Ht * W * 4
         reps, wu = 100, 10
-        add("batch norm (training) + relu + halo pad fwd, cfg1 tiles (3 kernels)",
+        add("batch norm (training) + relu + halo pad fwd, cfg1 tiles (2 kernels)",
             lambda: lib.adh_batchnorm2d_fwd_tiles(0, 1, K, N, C, Ht, W, 1e-5, 1, 1, tabs["x"][0], tabs["sc"][0], tabs["sh"][0],
                                                   None, None, tile_tbl, None, None, tabs["sm"][0], tabs["si"][0],
                                                   bn_ws.data_ptr(), bn_ws_bytes, stream),
             "hbm", 2 * packed_b + padded_b, HBM_PEAK_GBS, "GB/s", note="x read for the statistics and again to normalise")
-        add("batch norm + relu + halo unpad bwd, cfg1 tiles (3 kernels)",
+        add("batch norm + relu + halo unpad bwd, cfg1 tiles (2 kernels)",
             lambda: lib.adh_batchnorm2d_bwd_tiles(0, K, N, C, Ht, W, 1, 1, tabs["x"][0], g_tbl, tabs["sc"][0], tabs["sh"][0],
                                                   tabs["sm"][0], tabs["si"][0], tabs["dx"][0], tabs["dsc"][0], tabs["dsh"][0],
                                                   0.0, 0.0, bn_ws.data_ptr(), bn_ws_bytes, stream),
