@@ -106,6 +106,32 @@ private:
   Spatial2DComm *spatial_comms_;
 };
 
+// Everything enqueued on a stream between begin() and end(), recorded once as a HIP graph and replayed with
+// one launch: for loops that are bound by the host's launch rate (a training step at a small batch is a
+// thousand kernels of a few microseconds).  Not in the reference.  The host ops and the C ABI under them only
+// enqueue kernels and device-to-device copies, so a whole forward + backward + optimizer step can be recorded
+// once its buffers exist (run it eagerly first); host-to-device loads, read-backs and anything that
+// synchronises stay outside.  A replay repeats the recorded launches with the recorded arguments: values that
+// live in device memory (parameters, momentum, inputs copied into the same buffers) evolve, values that were
+// kernel arguments (this iteration's step size) do not.
+class StreamCapture {
+public:
+  explicit StreamCapture(hipStream_t stream) : stream_(stream), graph_(nullptr), exec_(nullptr) {}
+  ~StreamCapture();
+  StreamCapture(const StreamCapture &) = delete;
+  StreamCapture &operator=(const StreamCapture &) = delete;
+  void begin();
+  void end();
+  void replay();
+  size_t num_nodes() const { return num_nodes_; }
+
+private:
+  hipStream_t stream_;
+  hipGraph_t graph_;
+  hipGraphExec_t exec_;
+  size_t num_nodes_ = 0;
+};
+
 }  // namespace arraydiff
 
 #endif

@@ -105,4 +105,22 @@ Spatial2DComm *MultiGPUContext::spatial_comm(size_t rank) {
   return spatial_comms_ + rank;
 }
 
+StreamCapture::~StreamCapture() {
+  if (exec_) (void)hipGraphExecDestroy(exec_);
+  if (graph_) (void)hipGraphDestroy(graph_);
+}
+void StreamCapture::begin() {
+  if (graph_ || exec_) throw std::logic_error("StreamCapture: already recorded");
+  hip_check(hipStreamBeginCapture(stream_, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+}
+void StreamCapture::end() {
+  hip_check(hipStreamEndCapture(stream_, &graph_), "hipStreamEndCapture");
+  hip_check(hipGraphGetNodes(graph_, nullptr, &num_nodes_), "hipGraphGetNodes");
+  hip_check(hipGraphInstantiate(&exec_, graph_, nullptr, nullptr, 0), "hipGraphInstantiate");
+}
+void StreamCapture::replay() {
+  if (!exec_) throw std::logic_error("StreamCapture: nothing recorded");
+  hip_check(hipGraphLaunch(exec_, stream_), "hipGraphLaunch");
+}
+
 }  // namespace arraydiff

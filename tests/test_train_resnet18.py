@@ -13,9 +13,9 @@ BIN = os.path.join(os.path.dirname(HERE), "arraydiff_cuda_amd", "train_resnet18"
 ARGS = ["--ranks", "2", "--batch", "4", "--size", "128", "--steps", "6", "--warmup", "3", "--classes", "10"]
 
 
-def _run():
+def _run(extra=()):
     assert os.path.exists(BIN), "arraydiff_cuda_amd/train_resnet18 is not built: run __graft_entry__.build()"
-    r = subprocess.run([BIN] + ARGS, capture_output=True, text=True, timeout=240)
+    r = subprocess.run([BIN] + ARGS + list(extra), capture_output=True, text=True, timeout=240)
     assert r.returncode == 0, r.stdout + r.stderr
     return json.loads(r.stdout.strip().splitlines()[-1]), r.stdout
 
@@ -27,6 +27,16 @@ def test_loss_falls_and_run_is_deterministic():
     assert a["loss_last"] < 0.1 * a["loss_first"], out_a
     b, _ = _run()
     assert (a["loss_first"], a["loss_last"]) == (b["loss_first"], b["loss_last"])
+
+
+@pytest.mark.gpu
+def test_recorded_step_replays_to_the_same_losses():
+    """One step recorded as a HIP graph and replayed six times ends where six eager steps end (the step size
+    is constant, everything else that changes lives in device memory)."""
+    eager, _ = _run()
+    graph, out = _run(["--graph", "1"])
+    assert graph["graph"] is True and "graph nodes" in out
+    assert graph["loss_last"] == eager["loss_last"] and graph["loss_first"] == eager["loss_first"]
 
 
 def test_trainer_rejects_unknown_options():
