@@ -19,7 +19,9 @@ def rand_tiles(rng, K, N, C, PH, PW, dtype):
 
 SHAPES = [  # K, p, Ht, W, C, N
     (1, 1, 3, 4, 2, 1), (2, 1, 4, 5, 3, 2), (4, 1, 14, 56, 8, 3), (4, 2, 5, 7, 3, 2), (8, 1, 4, 6, 2, 2),
-    (3, 3, 6, 9, 2, 1), (16, 1, 2, 3, 1, 1), (4, 1, 3, 62, 5, 2)]
+    (3, 3, 6, 9, 2, 1), (16, 1, 2, 3, 1, 1), (4, 1, 3, 62, 5, 2),
+    # rows of 512 and more elements
+    (2, 1, 3, 520, 3, 2), (3, 2, 4, 517, 2, 1), (1, 3, 5, 1030, 1, 2)]
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.uint16])
