@@ -476,12 +476,21 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
   const size_t K = xs_.size();
   // filter gradient: dw += sum over the tiles that share the filter (zeroed on first touch,
   // op.cc:1651-1654; beta = 1, op.cc:1660-1671)
+  // (the first toucher of a filter gradient overwrites it, beta = 0, instead of clearing it and adding; with
+  // replicated filters rank 0's variable receives every tile's share and the other ranks' are cleared)
   vector<size_t> todo;
+  bool wfresh[ADH_MAX_TILES] = {};
+  const bool replicated_w = shape_.replicated_filters;
   for (size_t r = 0; r < K; ++r) {
     GPUContext *dc = rank_ctx(ctx_, r);
-    if (kernels_[r].grad().accumulate(txn, id(), dc, [dc](A4 *g) {
-          GPUConn conn = dc->conn();
-          g->set_constant(0.0f, conn);
+    bool *fresh_r = &wfresh[r];
+    const bool clear = replicated_w && r > 0;
+    if (kernels_[r].grad().accumulate(txn, id(), dc, [dc, fresh_r, clear](A4 *g) {
+          *fresh_r = true;
+          if (clear) {
+            GPUConn conn = dc->conn();
+            g->set_constant(0.0f, conn);
+          }
         }))
       todo.push_back(r);
   }
@@ -505,6 +514,7 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
   }
   while (!todo.empty()) {
     float *dw = kernels_[replicated ? 0 : todo[0]].grad().get_mut(txn, id()).dptr();
+    const float wbeta = wfresh[replicated ? 0 : todo[0]] ? 0.0f : 1.0f;
     const void *xt[ADH_MAX_TILES];
     const void *dyt[ADH_MAX_TILES];
     uint32_t n = 0;
@@ -530,13 +540,13 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
       dc->reserve_scratch(ws);
       auto scratch = dc->get_scratch();
       adh_check(adh_conv3x3_slab_bwd_filter_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, dyt, dw,
-                                                  1.0f, scratch->dptr(), scratch->size(), conn.stream()),
+                                                  wbeta, scratch->dptr(), scratch->size(), conn.stream()),
                 "SlabConv2DOp::_backward (filter)");
     } else {
       size_t ws_bytes;
       void *ws = conv_scratch(dc, ADH_CONV_BWD_FILTER, n, d, shape_, &ws_bytes);
       adh_check(adh_conv2d_slab_bwd_filter_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
-                                                 ADH_CONV_GEOMETRY(d, shape_), xt, dyt, dw, 1.0f, ws, ws_bytes,
+                                                 ADH_CONV_GEOMETRY(d, shape_), xt, dyt, dw, wbeta, ws, ws_bytes,
                                                  conn.stream()),
                 "SlabConv2DOp::_backward (filter, general)");
     }
