@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) void conv_gen_filter_kernel(const FilterGenPar
 // staging.  (Loading the next chunk into registers during the multiplication instead takes the whole register file,
 // one workgroup per CU, and measured slower: 39 against 50 TFLOP/s on the 7x7 stem.)
 template <typename T, int CC, int MT>
-__global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenParams P) {
+__global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenParams P) {
   constexpr uint32_t MW = 16u * MT;                         // m per block
   constexpr uint32_t WPITCH = MT == 1 ? 16u : MW + 16u;     // filter row pitch: the 4 channel groups 16 banks apart
   constexpr int PFC = 32 / CC;                              // staging registers per channel plane: PP <= 256 * PFC
@@ -207,47 +207,55 @@ __global__ __launch_bounds__(kGenThreads) void conv_gen_kernel(const ConvGenPara
   const uint32_t ntaps_s = S.t1 - S.t0;
   if (ntaps_s > 0) {
     const uint32_t ngroups = (ntaps_s + P.TG - 1u) / P.TG;
-    for (uint32_t ch = 0; ch < P.nchunks; ++ch) {
-      for (uint32_t gi = 0; gi < ngroups; ++gi) {
-        const uint32_t tg0 = S.t0 + gi * P.TG;
-        const uint32_t ntg = min(P.TG, S.t1 - tg0);
-        __syncthreads();  // every wave is done with the filter rows (and, at a new chunk, the patch)
-        if (gi == 0) {
-          load_patch(ch);
-          store_patch();
-        }
-        load_filter(ch, tg0, ntg);
-        store_filter(ntg);
-        // lane L keeps the patch offset of tap tg0 + L
-        int32_t delta_vec = 0;
-        if (lane < ntg)
-          delta_vec = ((int32_t)P.off_r[tg0 + lane] - S.min_r) * (int32_t)P.PCP + ((int32_t)P.off_c[tg0 + lane] - S.min_c);
-        __syncthreads();
-        const uint32_t steps = ntg << LOG2_CQ;
-        float a_cur[MT], b_cur[4], a_nxt[MT], b_nxt[4];
-        auto fetch = [&](uint32_t step, float (&a)[MT], float (&b)[4]) {
-          const uint32_t t = step >> LOG2_CQ, cq = step & ((CC >> 2) - 1u);
-          const int32_t delta = __builtin_amdgcn_readlane(delta_vec, (int)t);
-          const float *wrow = wl + (t * CC + (cq << 2) + g) * WPITCH + l16;
-          const float *prow = patch + (cq << 2) * P.PP + delta;
+    const uint32_t total = P.nchunks * ngroups;
+    uint32_t ch = 0, gi = 0;
+    load_patch(0);
+    load_filter(0, S.t0, min(P.TG, ntaps_s));
+    for (uint32_t it = 0; it < total; ++it) {
+      const uint32_t tg0 = S.t0 + gi * P.TG;
+      const uint32_t ntg = min(P.TG, S.t1 - tg0);
+      __syncthreads();  // every wave is done with the filter rows (and, at a new chunk, the patch)
+      if (gi == 0) store_patch();
+      store_filter(ntg);
+      // lane L keeps the patch offset of tap tg0 + L
+      int32_t delta_vec = 0;
+      if (lane < ntg)
+        delta_vec = ((int32_t)P.off_r[tg0 + lane] - S.min_r) * (int32_t)P.PCP + ((int32_t)P.off_c[tg0 + lane] - S.min_c);
+      __syncthreads();
+      // the next (chunk, tap group) is on its way from memory while this one is multiplied
+      if (++gi == ngroups) {
+        gi = 0;
+        ++ch;
+      }
+      if (it + 1u < total) {
+        if (gi == 0) load_patch(ch);
+        const uint32_t tn0 = S.t0 + gi * P.TG;
+        load_filter(ch, tn0, min(P.TG, S.t1 - tn0));
+      }
+      const uint32_t steps = ntg << LOG2_CQ;
+      float a_cur[MT], b_cur[4], a_nxt[MT], b_nxt[4];
+      auto fetch = [&](uint32_t step, float (&a)[MT], float (&b)[4]) {
+        const uint32_t t = step >> LOG2_CQ, cq = step & ((CC >> 2) - 1u);
+        const int32_t delta = __builtin_amdgcn_readlane(delta_vec, (int)t);
+        const float *wrow = wl + (t * CC + (cq << 2) + g) * WPITCH + l16;
+        const float *prow = patch + (cq << 2) * P.PP + delta;
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) a[mt] = wrow[mt * 16];
+        for (int mt = 0; mt < MT; ++mt) a[mt] = wrow[mt * 16];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) b[q] = prow[pix[q]];
-        };
-        fetch(0, a_cur, b_cur);
-        for (uint32_t step = 0; step < steps; ++step) {
-          if (step + 1u < steps) fetch(step + 1u, a_nxt, b_nxt);
+        for (int q = 0; q < 4; ++q) b[q] = prow[pix[q]];
+      };
+      fetch(0, a_cur, b_cur);
+      for (uint32_t step = 0; step < steps; ++step) {
+        if (step + 1u < steps) fetch(step + 1u, a_nxt, b_nxt);
 #pragma unroll
-          for (int q = 0; q < 4; ++q)
+        for (int q = 0; q < 4; ++q)
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-              acc[q][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[mt], b_cur[q], acc[q][mt], 0, 0, 0);
+          for (int mt = 0; mt < MT; ++mt)
+            acc[q][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[mt], b_cur[q], acc[q][mt], 0, 0, 0);
 #pragma unroll
-          for (int k = 0; k < MT; ++k) a_cur[k] = a_nxt[k];
+        for (int k = 0; k < MT; ++k) a_cur[k] = a_nxt[k];
 #pragma unroll
-          for (int k = 0; k < 4; ++k) b_cur[k] = b_nxt[k];
-        }
+        for (int k = 0; k < 4; ++k) b_cur[k] = b_nxt[k];
       }
     }
   }
@@ -278,31 +286,14 @@ struct GenPlan {
   ConvGenParams P;
   FilterGenParams F;
   size_t lds_bytes, wt_bytes;
-  uint32_t MT;
+  uint32_t MT, num_tiles;
 };
+// a launch of fewer blocks than this (two per compute unit) is split finer
+constexpr uint64_t kGenFillBlocks = 512;
 
-// Fills the tiling fields of `plan` once the sub-problems' taps and grids are set.  Returns an error code.
-static int gen_finish_plan(GenPlan *plan) {
+// The part of the tiling that depends on the block's width in output channels (16 * plan->MT); BR and BC are set.
+static int gen_tile_plan(GenPlan *plan, uint32_t max_taps) {
   ConvGenParams &P = plan->P;
-  uint32_t max_GJ = 0, max_taps = 0;
-  for (uint32_t s = 0; s < P.nsub; ++s) {
-    max_GJ = std::max(max_GJ, P.sub[s].GJ);
-    max_taps = std::max(max_taps, P.sub[s].t1 - P.sub[s].t0);
-  }
-  uint32_t max_GI = 0;
-  for (uint32_t s = 0; s < P.nsub; ++s) max_GI = std::max(max_GI, P.sub[s].GI);
-  // block columns: the whole row when it has at most 64 pixels, else the width in [32, 64] that wastes least
-  if (max_GJ <= 64u) {
-    P.BC = std::max(max_GJ, 1u);
-  } else {
-    double best = -1.0;
-    for (uint32_t bc = 64u; bc >= 32u; --bc) {
-      const double used = (double)((256u / bc) * bc) / 256.0 * (double)max_GJ / (double)(((max_GJ + bc - 1u) / bc) * bc);
-      if (used > best + 1e-9) { best = used; P.BC = bc; }
-    }
-  }
-  P.BR = std::max(1u, std::min(256u / P.BC, std::max(max_GI, 1u)));
-  plan->MT = P.M <= 16u ? 1u : P.M <= 32u ? 2u : 4u;
   const uint32_t MW = 16u * plan->MT, wpitch = plan->MT == 1u ? 16u : MW + 16u;
   P.MG = (P.M + MW - 1u) / MW;
   uint32_t max_PR, max_PC, bpi;
@@ -387,6 +378,40 @@ static int gen_finish_plan(GenPlan *plan) {
   F.nchunks = P.nchunks;
   F.CC = P.CC;
   F.ntaps = P.ntaps;
+  return ADH_OK;
+}
+
+// Fills the tiling fields of `plan` once the sub-problems' taps and grids are set.  Returns an error code.
+static int gen_finish_plan(GenPlan *plan) {
+  ConvGenParams &P = plan->P;
+  uint32_t max_GJ = 0, max_taps = 0;
+  for (uint32_t s = 0; s < P.nsub; ++s) {
+    max_GJ = std::max(max_GJ, P.sub[s].GJ);
+    max_taps = std::max(max_taps, P.sub[s].t1 - P.sub[s].t0);
+  }
+  uint32_t max_GI = 0;
+  for (uint32_t s = 0; s < P.nsub; ++s) max_GI = std::max(max_GI, P.sub[s].GI);
+  // block columns: the whole row when it has at most 64 pixels, else the width in [32, 64] that wastes least
+  if (max_GJ <= 64u) {
+    P.BC = std::max(max_GJ, 1u);
+  } else {
+    double best = -1.0;
+    for (uint32_t bc = 64u; bc >= 32u; --bc) {
+      const double used = (double)((256u / bc) * bc) / 256.0 * (double)max_GJ / (double)(((max_GJ + bc - 1u) / bc) * bc);
+      if (used > best + 1e-9) { best = used; P.BC = bc; }
+    }
+  }
+  P.BR = std::max(1u, std::min(256u / P.BC, std::max(max_GI, 1u)));
+  // Output channels per block: 64, or fewer when there are no more of them, or when the launch would
+  // leave compute units idle (a block's time is mostly the latency of staging its chunks, whatever its
+  // width, so narrower blocks on more units finish sooner).
+  plan->MT = P.M <= 16u ? 1u : P.M <= 32u ? 2u : 4u;
+  for (;; plan->MT /= 2u) {
+    const int e = gen_tile_plan(plan, max_taps);
+    if (e) return e;
+    const uint64_t blocks = (uint64_t)std::max(plan->num_tiles, 1u) * P.NG * P.MG * P.blocks_per_image;
+    if (plan->MT == 1u || blocks >= kGenFillBlocks) break;
+  }
   return ADH_OK;
 }
 
@@ -531,7 +556,7 @@ struct WgradGenParams {
 // (tap, input channel) pairs, pair q = 16 t + column = tap * Cin + ci, instead of 16 input channels of one tap;
 // all taps then fit one block and no matrix column is spent on channels that do not exist.
 template <typename T, int TAPS, bool PACKED>
-__global__ __launch_bounds__(kWgGenThreads, TAPS > 9 ? 1 : 2) void conv_gen_wgrad_kernel(const WgradGenParams P) {
+__global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const WgradGenParams P) {
   extern __shared__ __align__(16) float gen_lds[];
   float *dyl = gen_lds;
   float *patch = gen_lds + P.dy_lds_floats;
@@ -557,18 +582,17 @@ __global__ __launch_bounds__(kWgGenThreads, TAPS > 9 ? 1 : 2) void conv_gen_wgra
       pair_off[t] = tap < P.ntaps ? (int32_t)(ci * P.PP) + (int32_t)P.off_r[tap] * (int32_t)P.PCP + (int32_t)P.off_c[tap] : 0;
     }
   }
-  floatx4 acc[TAPS][4];
+  // wave w owns output channels 16 w .. 16 w + 15 of the block's 64: one accumulator tile per tap
+  floatx4 acc[TAPS];
 #pragma unroll
-  for (int t = 0; t < TAPS; ++t)
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < TAPS; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   const uint32_t unit_pix = P.R * P.OWT, ksteps = unit_pix >> 2;
   // only the channels that exist are staged; lanes of absent channels read channel 0 and their sums are dropped
   const uint32_t planes = min(16u, P.Cin - cit * 16u);
   const uint32_t my_plane = l16 < planes ? l16 : 0u;
   // What a thread stages is the same for every unit: the lane's pixel of the dy tile (a unit has at most 64
-  // pixels) for 16 output channels per wave, and up to four (row, column) places of every patch plane.
+  // pixels) for the wave's 16 output channels, and up to four (row, column) places of every patch plane.
   uint32_t dy_r, dy_c;
   P.div_OWT.divmod(lane, dy_r, dy_c);
   const bool dy_lane = lane < unit_pix;
@@ -582,7 +606,9 @@ __global__ __launch_bounds__(kWgGenThreads, TAPS > 9 ? 1 : 2) void conv_gen_wgra
     pr_rc[k] = e < P.PR * P.PC ? (r << 16) | col : 0xffffffffu;
     pr_lds[k] = r * P.PCP + col;
   }
-  for (uint32_t u = ps; u < P.units; u += P.PS) {
+  // A unit travels memory -> registers -> LDS; the next unit's loads are in flight while this one is multiplied.
+  float dy_pre[16], x_pre[KP][16];
+  auto load_unit = [&](uint32_t u) {
     uint32_t r2, r3, cb, rb, n, tile;
     P.div_ncb.divmod(u, r2, cb);
     P.div_nrb.divmod(r2, r3, rb);
@@ -590,72 +616,65 @@ __global__ __launch_bounds__(kWgGenThreads, TAPS > 9 ? 1 : 2) void conv_gen_wgra
     const T *xs = reinterpret_cast<const T *>(P.x[tile]) + ((size_t)n * P.Cin + cit * 16u) * P.HP * P.WP;
     const T *ds = reinterpret_cast<const T *>(P.dy[tile]) + ((size_t)n * P.Cout + cog * 64u) * P.OH * P.OW;
     const uint32_t oh0 = rb * P.R, ow0 = cb * P.OWT;
-    __syncthreads();  // every wave is done with the previous unit
-    if (dy_lane) {
-      const bool in = oh0 + dy_r < P.OH && ow0 + dy_c < P.OW;
+    {
+      const bool in = dy_lane && oh0 + dy_r < P.OH && ow0 + dy_c < P.OW;
       const size_t pix = (size_t)(oh0 + dy_r) * P.OW + ow0 + dy_c;
-#pragma unroll 4
+#pragma unroll
       for (uint32_t c = 0; c < 16u; ++c) {
         const uint32_t co = wave * 16u + c;
-        float v = 0.f;
-        if (in && cog * 64u + co < P.Cout) v = gen_ld(ds, (size_t)co * P.OH * P.OW + pix);
-        dyl[co * P.DP + lane] = v;
+        dy_pre[c] = (in && cog * 64u + co < P.Cout) ? gen_ld(ds, (size_t)co * P.OH * P.OW + pix) : 0.f;
       }
     }
 #pragma unroll
     for (int k = 0; k < KP; ++k) {
-      if (pr_rc[k] == 0xffffffffu) continue;
       const uint32_t gr = oh0 * P.sh + (pr_rc[k] >> 16), gc = ow0 * P.sw + (pr_rc[k] & 0xffffu);
-      const bool in = gr < P.HP && gc < P.WP;
+      const bool in = pr_rc[k] != 0xffffffffu && gr < P.HP && gc < P.WP;
       const size_t pix = (size_t)gr * P.WP + gc;
-      for (uint32_t c = 0; c < planes; ++c)
-        patch[c * P.PP + pr_lds[k]] = in ? gen_ld(xs, (size_t)c * P.HP * P.WP + pix) : 0.f;
-    }
-    __syncthreads();
-    for (uint32_t ks = wave; ks < ksteps; ks += 4u) {
-      const uint32_t p0 = (ks << 2) + g;
-      uint32_t r, c;
-      P.div_OWT.divmod(p0, r, c);
-      const float *arow = dyl + l16 * P.DP + p0;
-      const float *brow = patch + (PACKED ? 0u : my_plane * P.PP) + r * P.sh * P.PCP + c * P.sw;
-      float a[4], b[TAPS];
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt) a[mt] = arow[mt * 16 * P.DP];
+      for (uint32_t c = 0; c < 16u; ++c)
+        x_pre[k][c] = (in && c < planes) ? gen_ld(xs, (size_t)c * P.HP * P.WP + pix) : 0.f;
+    }
+  };
+  auto store_unit = [&]() {
+    if (dy_lane) {
+#pragma unroll
+      for (uint32_t c = 0; c < 16u; ++c) dyl[(wave * 16u + c) * P.DP + lane] = dy_pre[c];
+    }
+#pragma unroll
+    for (int k = 0; k < KP; ++k) {
+      if (pr_rc[k] == 0xffffffffu) continue;
+#pragma unroll
+      for (uint32_t c = 0; c < 16u; ++c)
+        if (c < planes) patch[c * P.PP + pr_lds[k]] = x_pre[k][c];
+    }
+  };
+  if (ps < P.units) load_unit(ps);
+  for (uint32_t u = ps; u < P.units; u += P.PS) {
+    __syncthreads();  // every wave is done with the previous unit
+    store_unit();
+    __syncthreads();
+    if (u + P.PS < P.units) load_unit(u + P.PS);
+    const float *arow = dyl + (wave * 16u + l16) * P.DP + g;
+    const float *bpl = patch + (PACKED ? 0u : my_plane * P.PP);
+#pragma unroll 2
+    for (uint32_t ks = 0; ks < ksteps; ++ks) {
+      uint32_t r, c;
+      P.div_OWT.divmod((ks << 2) + g, r, c);
+      const float *brow = bpl + r * P.sh * P.PCP + c * P.sw;
+      const float a = arow[ks << 2];
+      float b[TAPS];
 #pragma unroll
       for (int t = 0; t < TAPS; ++t) b[t] = PACKED ? brow[pair_off[t]] : brow[__builtin_amdgcn_readlane(delta_vec, t)];
 #pragma unroll
-      for (int t = 0; t < TAPS; ++t)
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[mt], b[t], acc[t][mt], 0, 0, 0);
+      for (int t = 0; t < TAPS; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[t], acc[t], 0, 0, 0);
     }
   }
-  // the four waves' sums are added in wave order through LDS (deterministic), then written once:
-  // partial[ps][cog][cit][tg][t][mt][lane][4]
-  floatx4 *red = reinterpret_cast<floatx4 *>(gen_lds);
-  for (uint32_t w = 0; w < 4u; ++w) {
-    __syncthreads();  // w = 0: every wave is done with the staged tiles
-    if (wave == w) {
+  // partial[ps][cog][cit][tg][t][mt = wave][lane][4]
+  const size_t block_part = ((size_t)(cog * P.CIT + cit) * P.ntg + tg) * TAPS * 1024u;
+  const size_t stride = (size_t)P.COG * P.CIT * P.ntg * TAPS * 1024u;
+  float *dstp = P.partial + (size_t)ps * stride + block_part;
 #pragma unroll
-      for (int t = 0; t < TAPS; ++t)
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
-          floatx4 &slot = red[(t * 4 + mt) * 64 + lane];
-          if (w > 0) acc[t][mt] += slot;
-          if (w < 3u) slot = acc[t][mt];
-        }
-    }
-  }
-  if (wave == 3u) {
-    const size_t block_part = ((size_t)(cog * P.CIT + cit) * P.ntg + tg) * TAPS * 1024u;
-    const size_t stride = (size_t)P.COG * P.CIT * P.ntg * TAPS * 1024u;
-    float *dstp = P.partial + (size_t)ps * stride + block_part;
-#pragma unroll
-    for (int t = 0; t < TAPS; ++t)
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
-        *reinterpret_cast<floatx4 *>(dstp + (t * 4 + mt) * 256 + lane * 4u) = acc[t][mt];
-  }
+  for (int t = 0; t < TAPS; ++t) *reinterpret_cast<floatx4 *>(dstp + (t * 4 + wave) * 256u + lane * 4u) = acc[t];
 }
 
 struct WgradGenReduceParams {
@@ -744,7 +763,7 @@ static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *p
     while (dp % 64u != 4u) ++dp;
     P.DP = dp;
     P.dy_lds_floats = 64u * P.DP;
-    plan->lds_bytes = std::max<size_t>(((size_t)P.dy_lds_floats + 16u * (size_t)P.PP) * 4u, (size_t)P.T * 4096u);
+    plan->lds_bytes = ((size_t)P.dy_lds_floats + 16u * (size_t)P.PP) * 4u;
     if (plan->lds_bytes <= kGenLdsBytes && P.PR * P.PC <= 1024u) break;  // a thread stages up to four places per plane
     if (P.R > 1u) P.R /= 2u;
     else if (P.OWT > 4u) P.OWT = ((P.OWT / 2u) + 3u) & ~3u;
@@ -805,6 +824,7 @@ size_t adh_conv2d_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint
     return (wp.partial_bytes + 255u) & ~(size_t)255u;
   }
   GenPlan plan = {};
+  plan.num_tiles = num_tiles;
   int e = ADH_EINVAL;
   if (which == ADH_CONV_FWD) e = gen_plan_fwd(g, &plan);
   else if (which == ADH_CONV_BWD_DATA) e = gen_plan_bwd_data(g, &plan);
@@ -825,6 +845,7 @@ int adh_conv2d_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_
   if (Cin == 0) return ADH_EINVAL;
   if (!x_pad_tiles || !y_tiles || !w) return ADH_ENULL;
   GenPlan plan = {};
+  plan.num_tiles = num_tiles;
   e = gen_plan_fwd(g, &plan);
   if (e) return e;
   const size_t es = dtype_size(dtype);
@@ -852,6 +873,7 @@ int adh_conv2d_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, ui
   if (Cout == 0) return ADH_EINVAL;
   if (!dy_tiles || !dx_pad_tiles || !w) return ADH_ENULL;
   GenPlan plan = {};
+  plan.num_tiles = num_tiles;
   e = gen_plan_bwd_data(g, &plan);
   if (e) return e;
   const size_t es = dtype_size(dtype);

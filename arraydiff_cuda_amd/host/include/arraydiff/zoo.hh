@@ -6,10 +6,11 @@
 //
 // What differs from the reference's MakeParallelResNet18, all in the replicated tail after the
 // spatial part: the input arrives as NCHW floats (no transpose / scale ops); the tiles are
-// gathered once (SpatialJoinedGather2DOp replaces gather + all-reduce) and the global pooling,
-// the classifier and the loss run once instead of once per rank followed by a reduce and a
-// division by the rank count; the classifier is the 1x1 convolution over the pooled 1x1 image
-// that a bias-free linear layer is; the mean over the minibatch is the loss's sink gradient.
+// gathered once (SpatialJoinedGather2DOp replaces gather + all-reduce); every rank then pools the
+// gathered activation and applies its own copy of the classifier, as in the reference, and the
+// logits are summed over ranks and divided by the rank count before ONE loss node (the reference
+// runs the loss per rank); the classifier is the 1x1 convolution over the pooled 1x1 image that a
+// bias-free linear layer is; the mean over the minibatch is the loss's sink gradient.
 #ifndef ARRAYDIFF_ZOO_HH
 #define ARRAYDIFF_ZOO_HH
 

@@ -104,15 +104,14 @@ ParallelCategoricalNLLBatchNormLoss<V1, F0> ResNet<float>::MakeParallelResNet18(
   Conv2DShape fc_shape;
   fc_shape.filters = num_classes; fc_shape.axes = {0, 1}; fc_shape.kernel = {1, 1}; fc_shape.dilate = {1, 1};
   fc_shape.stride = {1, 1}; fc_shape.pad = {0, 0}; fc_shape.halo_padded_input = false; fc_shape.enable_hmma = false;
-  vector<shared_ptr<Var<V3>>> rank_logits;
-  for (size_t rank = 0; rank < num_ranks; ++rank) {
-    shared_ptr<Context> dev = mgpu_ctx->device_context(rank);
-    auto pooled = CudnnPool2DOp<V3>::Make(global_pool_shape, gathered, dev);
-    auto fc_kernel = ParamOp<A4>::Make(Shape4D(1, 1, 512, num_classes), xavier_init_gen<A4>(512, num_classes), dev);
-    net.dev_params[rank].insert(fc_kernel->vars().at(0));
-    net.dev_grads[rank].insert(fc_kernel->vars().at(1));
-    rank_logits.push_back(CudnnConv2DOp<V3, A4, A4>::Make(fc_shape, pooled, fc_kernel, dev));
-  }
+  vector<shared_ptr<Var<V3>>> rank_pooled;
+  for (size_t rank = 0; rank < num_ranks; ++rank)
+    rank_pooled.push_back(CudnnPool2DOp<V3>::Make(global_pool_shape, gathered, mgpu_ctx->device_context(rank)));
+  // one node (and, the copies being equal, one launch per pass) applies every rank's classifier
+  auto fc = parallel_conv2d<V3, A4>(fc_shape, rank_pooled, xavier_init_gen<A4>(512, num_classes), false, parallel_ctx);
+  parallel_vars_insert_all(net.dev_params, fc.params);
+  parallel_vars_insert_all(net.dev_grads, fc.grads);
+  vector<shared_ptr<Var<V3>>> rank_logits = fc.ops;
   shared_ptr<Var<V3>> y = sum<V3>(rank_logits, root);
   y = ScaleOp<float, V3>::Make(1.0f / static_cast<float>(num_ranks), y, root);
   net.op = FlattenNCHWOp<V3, V1>::Make(y, root);
