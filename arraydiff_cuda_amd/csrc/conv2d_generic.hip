@@ -90,20 +90,17 @@ __global__ __launch_bounds__(256) void conv_gen_filter_kernel(const FilterGenPar
   }
 }
 
-// CC: channels per chunk (4 or 8); MT: 16-wide m-tiles per block (1, 2 or 4).
+// CC: channels per chunk (4, 8, 16 or 32: the more, the fewer barriers; the smaller the patch must be); MT: 16-wide m-tiles per block (1, 2 or 4).
 // The next (chunk, tap group)'s patch and filter rows are loaded into registers while the current
-// one is multiplied; they go to LDS after the barrier that ends the current one.
-// Patch and filter rows are loaded and staged between the two barriers of a (chunk, tap group); the registers they pass
-// through are dead during the multiplication, which leaves room for two workgroups per CU that hide each other's
-// staging.  (Loading the next chunk into registers during the multiplication instead takes the whole register file,
-// one workgroup per CU, and measured slower: 39 against 50 TFLOP/s on the 7x7 stem.)
+// one is multiplied; they go to LDS after the barrier that ends the current one.  The register
+// budget is held to half the file, so that two workgroups share a CU and hide each other's barriers.
 template <typename T, int CC, int MT>
 __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenParams P) {
   constexpr uint32_t MW = 16u * MT;                         // m per block
   constexpr uint32_t WPITCH = MT == 1 ? 16u : MW + 16u;     // filter row pitch: the 4 channel groups 16 banks apart
   constexpr int PFC = 32 / CC;                              // staging registers per channel plane: PP <= 256 * PFC
   constexpr int WF = 6;                                     // float4 filter registers: TG * CC * MW / 4 <= 256 * WF
-  constexpr uint32_t LOG2_CQ = CC == 8 ? 1u : 0u;
+  constexpr uint32_t LOG2_CQ = CC == 32 ? 3u : CC == 16 ? 2u : CC == 8 ? 1u : 0u;  // log2 of the chunk's groups of 4 channels
   extern __shared__ __align__(16) float gen_lds[];
   float *wl = gen_lds;
   float *patch = gen_lds + P.w_lds_floats;
@@ -298,7 +295,11 @@ static int gen_tile_plan(GenPlan *plan, uint32_t max_taps) {
   P.MG = (P.M + MW - 1u) / MW;
   uint32_t max_PR, max_PC, bpi;
   size_t patch_bytes;
-  P.CC = P.C >= 8u ? 8u : 4u;
+  // channels per chunk: 8 (4 when there are fewer), or 16 / 32 when the channel count is (nearly) a multiple and the
+  // patch is small enough for a thread's 32 staging registers without giving up images per block
+  // (a last chunk padded with zero channels is accepted when the padding is under an eighth of the channels)
+  auto pads_little = [&](uint32_t cc) { return ((P.C + cc - 1u) / cc * cc - P.C) * 8u <= P.C; };
+  P.CC = pads_little(32u) ? 32u : pads_little(16u) ? 16u : P.C >= 8u ? 8u : 4u;
   for (;;) {
     max_PR = 1; max_PC = 1; bpi = 0;
     for (uint32_t s = 0; s < P.nsub; ++s) {
@@ -341,12 +342,12 @@ static int gen_tile_plan(GenPlan *plan, uint32_t max_taps) {
       patch_bytes = (size_t)P.CC * P.PP * 4u;
       // a thread stages 32 / CC elements of each channel plane
       fits = P.PP <= 256u * (32u / P.CC) && patch_bytes + (size_t)P.CC * wpitch * 4u <= kGenLdsBytes;
-      if (fits || nb == 1u) break;
+      if (fits || nb == 1u || P.CC > 8u) break;
     }
     P.NB = nb;
     if (fits) break;
-    if (P.CC == 8u) {
-      P.CC = 4u;  // half the channels per chunk: twice the room per plane
+    if (P.CC > 4u) {
+      P.CC /= 2u;  // half the channels per chunk: twice the room per plane
       continue;
     }
     if (P.BR == 1u) return ADH_EUNIMPL;
@@ -496,7 +497,9 @@ static void launch_gen_cc(const GenPlan &plan, uint32_t blocks, hipStream_t st) 
 }
 template <typename T>
 static void launch_gen(const GenPlan &plan, uint32_t blocks, hipStream_t st) {
-  if (plan.P.CC == 8u) launch_gen_cc<T, 8>(plan, blocks, st);
+  if (plan.P.CC == 32u) launch_gen_cc<T, 32>(plan, blocks, st);
+  else if (plan.P.CC == 16u) launch_gen_cc<T, 16>(plan, blocks, st);
+  else if (plan.P.CC == 8u) launch_gen_cc<T, 8>(plan, blocks, st);
   else launch_gen_cc<T, 4>(plan, blocks, st);
 }
 
@@ -531,10 +534,10 @@ static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *
 // GEMM per tap: M = 64 output channels, N = 16 input channels, K = output pixels, four consecutive
 // pixels of a row per v_mfma_f32_16x16x4_f32.  A block owns (64 co, 16 ci, a group of T <= 9 taps)
 // and every PS-th unit of pixels (R output rows x OWT columns of one image); per unit it stages the dy
-// tile and the input patch in LDS, and its four waves split the unit's pixel groups, each keeping all
-// T x 4 accumulator tiles.  The four waves' sums are added through LDS in wave order and written in
-// register order to the workspace; a second kernel adds the PS partial sums in a fixed order
-// (deterministic) and scatters them to KCRS.
+// tile and the input patch in LDS, the next unit's loads already in flight in registers, and each of
+// its four waves multiplies the whole unit for its own 16 output channels, keeping T accumulator
+// tiles.  Every wave writes its sums in register order to the workspace; a second kernel adds the PS
+// partial sums in a fixed order (deterministic) and scatters them to KCRS.
 // ---------------------------------------------------------------------------------------------
 namespace adh {
 
