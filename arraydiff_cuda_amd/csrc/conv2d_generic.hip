@@ -67,6 +67,13 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float gen_ld(const float *p, size_t i) { return p[i]; }
 __device__ __forceinline__ float gen_ld(const uint16_t *p, size_t i) { return bf16_bits_to_f32(p[i]); }
+// base: the same address in every lane (it travels in scalar registers); boff: the lane's byte offset
+__device__ __forceinline__ float gen_ld_b(const float *base, uint32_t boff) {
+  return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(base) + boff);
+}
+__device__ __forceinline__ float gen_ld_b(const uint16_t *base, uint32_t boff) {
+  return bf16_bits_to_f32(*reinterpret_cast<const uint16_t *>(reinterpret_cast<const char *>(base) + boff));
+}
 __device__ __forceinline__ void gen_st(float *p, size_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void gen_st(uint16_t *p, size_t i, float v) { p[i] = f32_to_bf16_bits(v); }
 
@@ -148,7 +155,9 @@ __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenP
   const int32_t in_c0 = (int32_t)(bj * P.BC * P.si_c) + S.min_c;
   const size_t plane = (size_t)P.in_H * P.in_W;
   const int32_t image_elems = (int32_t)(P.C * (uint32_t)plane);  // only used when NB > 1 (the host bounds NB * C * plane)
-  int32_t src_off[PFC];
+  // a byte offset into the channel plane of the block's first image, and a bit per element that exists; the
+  // elements that do not (outside the input or the patch) load offset 0 and are replaced by zero
+  uint32_t src_boff[PFC], src_ok = 0;
 #pragma unroll
   for (int j = 0; j < PFC; ++j) {
     const uint32_t e = tid + j * kGenThreads;
@@ -158,38 +167,45 @@ __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenP
     const int32_t gr = in_r0 + (int32_t)r, gc = in_c0 + (int32_t)col;
     const bool ok = b < P.NB && n + b < P.N && r < S.PR && col < S.PC && gr >= 0 && gr < (int32_t)P.in_H && gc >= 0 &&
                     gc < (int32_t)P.in_W;
-    src_off[j] = ok ? (int32_t)b * image_elems + gr * (int32_t)P.in_W + gc : -1;
+    src_boff[j] = ok ? (uint32_t)((int32_t)b * image_elems + gr * (int32_t)P.in_W + gc) * (uint32_t)sizeof(T) : 0u;
+    src_ok |= ok ? 1u << j : 0u;
   }
 
   float pre[CC * PFC];
-  float4 wpre[WF];
+  floatx4 wpre[WF];
+  uint32_t pre_ch = 0;  // the chunk in `pre`
+  // (what does not exist is replaced by zero in store_patch, not here: a use of the loaded values next to
+  // the loads would make the wave wait for them before the multiplications they are meant to overlap)
   auto load_patch = [&](uint32_t ch) {
+    pre_ch = ch;
 #pragma unroll
     for (int c = 0; c < CC; ++c) {
-      const uint32_t cg = ch * CC + c;
-      const T *pl = src + (size_t)min(cg, P.C - 1u) * plane;
+      const T *pl = src + (size_t)min(ch * CC + c, P.C - 1u) * plane;
 #pragma unroll
-      for (int j = 0; j < PFC; ++j)
-        pre[c * PFC + j] = (src_off[j] >= 0 && cg < P.C) ? gen_ld(pl, (size_t)src_off[j]) : 0.f;
+      for (int j = 0; j < PFC; ++j) pre[c * PFC + j] = gen_ld_b(pl, src_boff[j]);
     }
   };
   auto store_patch = [&]() {
 #pragma unroll
-    for (int c = 0; c < CC; ++c)
+    for (int c = 0; c < CC; ++c) {
+      const bool chan = pre_ch * CC + c < P.C;
 #pragma unroll
       for (int j = 0; j < PFC; ++j) {
         const uint32_t e = tid + j * kGenThreads;
-        if (e < P.PP) patch[c * P.PP + e] = pre[c * PFC + j];
+        if (e < P.PP) patch[c * P.PP + e] = chan && ((src_ok >> j) & 1u) != 0u ? pre[c * PFC + j] : 0.f;
       }
+    }
   };
   auto load_filter = [&](uint32_t ch, uint32_t tg0, uint32_t ntg) {
-    const float4 *wsrc =
-        reinterpret_cast<const float4 *>(P.wt + ((size_t)(mg * P.nchunks + ch) * P.ntaps + tg0) * CC * MW);
+    const floatx4 *wsrc =
+        reinterpret_cast<const floatx4 *>(P.wt + ((size_t)(mg * P.nchunks + ch) * P.ntaps + tg0) * CC * MW);
     const uint32_t n4 = ntg * CC * (MW / 4u);
 #pragma unroll
     for (int k = 0; k < WF; ++k) {
+      // no branch and no default value: either would put a wait for the patch loads here (lanes past the end
+      // load the last piece again; store_filter drops it)
       const uint32_t e = tid + k * kGenThreads;
-      wpre[k] = e < n4 ? wsrc[e] : make_float4(0.f, 0.f, 0.f, 0.f);
+      wpre[k] = wsrc[min(e, n4 - 1u)];
     }
   };
   auto store_filter = [&](uint32_t ntg) {
@@ -197,7 +213,7 @@ __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenP
 #pragma unroll
     for (int k = 0; k < WF; ++k) {
       const uint32_t e = tid + k * kGenThreads;
-      if (e < n4) *reinterpret_cast<float4 *>(wl + (e / (MW / 4u)) * WPITCH + (e % (MW / 4u)) * 4u) = wpre[k];
+      if (e < n4) *reinterpret_cast<floatx4 *>(wl + (e / (MW / 4u)) * WPITCH + (e % (MW / 4u)) * 4u) = wpre[k];
     }
   };
 
@@ -241,18 +257,27 @@ __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenP
 #pragma unroll
         for (int q = 0; q < 4; ++q) b[q] = prow[pix[q]];
       };
-      fetch(0, a_cur, b_cur);
-      for (uint32_t step = 0; step < steps; ++step) {
-        if (step + 1u < steps) fetch(step + 1u, a_nxt, b_nxt);
+      auto multiply = [&](const float (&a)[MT], const float (&b)[4]) {
 #pragma unroll
         for (int q = 0; q < 4; ++q)
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            acc[q][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[mt], b_cur[q], acc[q][mt], 0, 0, 0);
-#pragma unroll
-        for (int k = 0; k < MT; ++k) a_cur[k] = a_nxt[k];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) b_cur[k] = b_nxt[k];
+          for (int mt = 0; mt < MT; ++mt) acc[q][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[mt], b[q], acc[q][mt], 0, 0, 0);
+      };
+      // two operand sets take turns: the reads of one step are in flight during the other step's multiplications
+      fetch(0, a_cur, b_cur);
+      // (a fetch past the last step repeats the last one: every pass has the same number of reads in flight, so
+      // the wait before a multiplication can leave the newer set outstanding)
+      // The scheduling barriers keep a set's reads together ahead of the other set's multiplications.
+      for (uint32_t step = 0; step < steps; step += 2u) {
+        fetch(min(step + 1u, steps - 1u), a_nxt, b_nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(a_cur, b_cur);
+        __builtin_amdgcn_sched_barrier(0);
+        if (step + 1u >= steps) break;
+        fetch(min(step + 2u, steps - 1u), a_cur, b_cur);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(a_nxt, b_nxt);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   }
@@ -330,9 +355,9 @@ static int gen_tile_plan(GenPlan *plan, uint32_t max_taps) {
     P.PPI = max_PR * P.PCP;
     P.live = P.BR * P.BC;
     // images per block: as many as fill the 256 pixel slots, fit LDS and the staging registers, and keep
-    // the offsets of a block's images within 31 bits
+    // the byte offsets of a block's images within 32 bits
     uint32_t nb = P.live <= 128u ? std::min(256u / P.live, std::max(P.N, 1u)) : 1u;
-    while (nb > 1u && (uint64_t)nb * P.C * P.in_H * P.in_W >= (1ull << 31)) --nb;
+    while (nb > 1u && (uint64_t)nb * P.C * P.in_H * P.in_W >= (1ull << 30)) --nb;
     bool fits = false;
     for (;; --nb) {
       // plane pitch: the four channel groups of a read start 16 banks apart
@@ -428,7 +453,8 @@ static int gen_check_shape(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_
   if ((uint64_t)sh * sw > (uint64_t)kGenMaxSub) return ADH_EUNIMPL;
   const uint64_t eh = (uint64_t)(kh - 1u) * dh + 1u, ew = (uint64_t)(kw - 1u) * dw + 1u;
   if (eh > HP || ew > WP || eh > 4096u || ew > 4096u) return ADH_EINVAL;
-  if ((uint64_t)HP * WP >= (1ull << 31) || Cin >= (1u << 24) || Cout >= (1u << 24)) return ADH_EINVAL;
+  // a lane's byte offset within a channel plane (within a block's images when it takes several) is 32 bits wide
+  if ((uint64_t)HP * WP >= (1ull << 30) || Cin >= (1u << 24) || Cout >= (1u << 24)) return ADH_EINVAL;
   *g = GenShape{N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, (uint32_t)((HP - eh) / sh + 1u), (uint32_t)((WP - ew) / sw + 1u)};
   return ADH_OK;
 }
@@ -595,12 +621,17 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
   const uint32_t planes = min(16u, P.Cin - cit * 16u);
   const uint32_t my_plane = l16 < planes ? l16 : 0u;
   // What a thread stages is the same for every unit: the lane's pixel of the dy tile (a unit has at most 64
-  // pixels) for the wave's 16 output channels, and up to four (row, column) places of every patch plane.
+  // pixels) for the wave's 16 output channels, and up to two (row, column) places of every patch plane.
+  // Loads take a base address that is the same in every lane (the unit's origin in the channel plane) plus the
+  // lane's 32-bit byte offset; places outside the tensors load offset 0 and are replaced by zero.
+  const uint32_t wave_u = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave);
   uint32_t dy_r, dy_c;
   P.div_OWT.divmod(lane, dy_r, dy_c);
   const bool dy_lane = lane < unit_pix;
-  constexpr int KP = 4;  // PR * PC <= 1024
-  uint32_t pr_rc[KP], pr_lds[KP];
+  const uint32_t dy_boff = (dy_r * P.OW + dy_c) * (uint32_t)sizeof(T);
+  const int32_t co_lim = (int32_t)P.Cout - (int32_t)(cog * 64u + wave_u * 16u);  // the wave's channels that exist
+  constexpr int KP = 2;  // PR * PC <= 512
+  uint32_t pr_rc[KP], pr_lds[KP], x_boff[KP];
 #pragma unroll
   for (int k = 0; k < KP; ++k) {
     const uint32_t e = tid + k * kWgGenThreads;
@@ -608,48 +639,64 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
     P.div_PC.divmod(e, r, col);
     pr_rc[k] = e < P.PR * P.PC ? (r << 16) | col : 0xffffffffu;
     pr_lds[k] = r * P.PCP + col;
+    x_boff[k] = (r * P.WP + col) * (uint32_t)sizeof(T);
   }
+  const size_t x_plane = (size_t)P.HP * P.WP, dy_plane = (size_t)P.OH * P.OW;
   // A unit travels memory -> registers -> LDS; the next unit's loads are in flight while this one is multiplied.
   float dy_pre[16], x_pre[KP][16];
+  uint32_t pre_in = 0;  // bit 0: the dy pixel exists; bit 1 + k: patch place k exists (of the unit in the registers)
+  // channels that do not exist load an existing one's place (no branch around a load); store_unit drops them
+  const int32_t dy_c0 = co_lim > 0 ? 0 : -(int32_t)(wave_u * 16u), dy_cmax = co_lim > 0 ? co_lim - 1 : 0;
   auto load_unit = [&](uint32_t u) {
     uint32_t r2, r3, cb, rb, n, tile;
     P.div_ncb.divmod(u, r2, cb);
     P.div_nrb.divmod(r2, r3, rb);
     P.div_N.divmod(r3, tile, n);
-    const T *xs = reinterpret_cast<const T *>(P.x[tile]) + ((size_t)n * P.Cin + cit * 16u) * P.HP * P.WP;
-    const T *ds = reinterpret_cast<const T *>(P.dy[tile]) + ((size_t)n * P.Cout + cog * 64u) * P.OH * P.OW;
     const uint32_t oh0 = rb * P.R, ow0 = cb * P.OWT;
-    {
-      const bool in = dy_lane && oh0 + dy_r < P.OH && ow0 + dy_c < P.OW;
-      const size_t pix = (size_t)(oh0 + dy_r) * P.OW + ow0 + dy_c;
+    const T *xs = reinterpret_cast<const T *>(P.x[tile]) + ((size_t)n * P.Cin + cit * 16u) * x_plane +
+                  (size_t)oh0 * P.sh * P.WP + (size_t)ow0 * P.sw;
+    const T *ds = reinterpret_cast<const T *>(P.dy[tile]) + ((size_t)n * P.Cout + cog * 64u + wave_u * 16u) * dy_plane +
+                  (size_t)oh0 * P.OW + ow0;
+    const bool dy_in = dy_lane && oh0 + dy_r < P.OH && ow0 + dy_c < P.OW;
+    pre_in = dy_in ? 1u : 0u;
+    const uint32_t dy_off = dy_in ? dy_boff : 0u;
 #pragma unroll
-      for (uint32_t c = 0; c < 16u; ++c) {
-        const uint32_t co = wave * 16u + c;
-        dy_pre[c] = (in && cog * 64u + co < P.Cout) ? gen_ld(ds, (size_t)co * P.OH * P.OW + pix) : 0.f;
-      }
-    }
+    for (int c = 0; c < 16; ++c)
+      dy_pre[c] = gen_ld_b(ds + (ptrdiff_t)(dy_c0 + min(c, dy_cmax)) * (ptrdiff_t)dy_plane, dy_off);
 #pragma unroll
     for (int k = 0; k < KP; ++k) {
-      const uint32_t gr = oh0 * P.sh + (pr_rc[k] >> 16), gc = ow0 * P.sw + (pr_rc[k] & 0xffffu);
-      const bool in = pr_rc[k] != 0xffffffffu && gr < P.HP && gc < P.WP;
-      const size_t pix = (size_t)gr * P.WP + gc;
+      const bool in = pr_rc[k] != 0xffffffffu && oh0 * P.sh + (pr_rc[k] >> 16) < P.HP && ow0 * P.sw + (pr_rc[k] & 0xffffu) < P.WP;
+      pre_in |= in ? 2u << k : 0u;
+      const uint32_t off = in ? x_boff[k] : 0u;
 #pragma unroll
-      for (uint32_t c = 0; c < 16u; ++c)
-        x_pre[k][c] = (in && c < planes) ? gen_ld(xs, (size_t)c * P.HP * P.WP + pix) : 0.f;
+      for (int c = 0; c < 16; ++c) x_pre[k][c] = gen_ld_b(xs + (size_t)min((uint32_t)c, planes - 1u) * x_plane, off);
     }
   };
   auto store_unit = [&]() {
     if (dy_lane) {
+      const bool in = (pre_in & 1u) != 0u;
 #pragma unroll
-      for (uint32_t c = 0; c < 16u; ++c) dyl[(wave * 16u + c) * P.DP + lane] = dy_pre[c];
+      for (int c = 0; c < 16; ++c) dyl[(wave * 16u + c) * P.DP + lane] = in && c < co_lim ? dy_pre[c] : 0.f;
     }
 #pragma unroll
     for (int k = 0; k < KP; ++k) {
       if (pr_rc[k] == 0xffffffffu) continue;
+      const bool in = ((pre_in >> (1 + k)) & 1u) != 0u;
 #pragma unroll
       for (uint32_t c = 0; c < 16u; ++c)
-        if (c < planes) patch[c * P.PP + pr_lds[k]] = x_pre[k][c];
+        if (c < planes) patch[c * P.PP + pr_lds[k]] = in ? x_pre[k][c] : 0.f;
     }
+  };
+  const float *arow = dyl + (wave * 16u + l16) * P.DP + g;
+  const float *bpl = patch + (PACKED ? 0u : my_plane * P.PP);
+  // the operands of k-step ks: four consecutive pixels of the unit, one per lane group
+  auto fetch = [&](uint32_t ks, float &a, float (&b)[TAPS]) {
+    uint32_t r, c;
+    P.div_OWT.divmod((ks << 2) + g, r, c);
+    const float *brow = bpl + r * P.sh * P.PCP + c * P.sw;
+    a = arow[ks << 2];
+#pragma unroll
+    for (int t = 0; t < TAPS; ++t) b[t] = PACKED ? brow[pair_off[t]] : brow[__builtin_amdgcn_readlane(delta_vec, t)];
   };
   if (ps < P.units) load_unit(ps);
   for (uint32_t u = ps; u < P.units; u += P.PS) {
@@ -657,19 +704,23 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
     store_unit();
     __syncthreads();
     if (u + P.PS < P.units) load_unit(u + P.PS);
-    const float *arow = dyl + (wave * 16u + l16) * P.DP + g;
-    const float *bpl = patch + (PACKED ? 0u : my_plane * P.PP);
-#pragma unroll 2
-    for (uint32_t ks = 0; ks < ksteps; ++ks) {
-      uint32_t r, c;
-      P.div_OWT.divmod((ks << 2) + g, r, c);
-      const float *brow = bpl + r * P.sh * P.PCP + c * P.sw;
-      const float a = arow[ks << 2];
-      float b[TAPS];
+    // two operand sets take turns: the reads of one k-step are in flight during the other's multiplications
+    float a_cur, a_nxt = 0.f, b_cur[TAPS], b_nxt[TAPS];
+    fetch(0, a_cur, b_cur);
+    // (a fetch past the last k-step repeats the last one: every pass has the same number of reads in flight, so
+    // the wait before a multiplication can leave the newer set outstanding)
+    for (uint32_t ks = 0; ks < ksteps; ks += 2u) {
+      fetch(min(ks + 1u, ksteps - 1u), a_nxt, b_nxt);
+      __builtin_amdgcn_sched_barrier(0);  // keeps a set's reads together ahead of the other set's multiplications
 #pragma unroll
-      for (int t = 0; t < TAPS; ++t) b[t] = PACKED ? brow[pair_off[t]] : brow[__builtin_amdgcn_readlane(delta_vec, t)];
+      for (int t = 0; t < TAPS; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur, b_cur[t], acc[t], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (ks + 1u >= ksteps) break;
+      fetch(min(ks + 2u, ksteps - 1u), a_cur, b_cur);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int t = 0; t < TAPS; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[t], acc[t], 0, 0, 0);
+      for (int t = 0; t < TAPS; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_nxt, b_nxt[t], acc[t], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
   // partial[ps][cog][cit][tg][t][mt = wave][lane][4]
@@ -767,7 +818,7 @@ static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *p
     P.DP = dp;
     P.dy_lds_floats = 64u * P.DP;
     plan->lds_bytes = ((size_t)P.dy_lds_floats + 16u * (size_t)P.PP) * 4u;
-    if (plan->lds_bytes <= kGenLdsBytes && P.PR * P.PC <= 1024u) break;  // a thread stages up to four places per plane
+    if (plan->lds_bytes <= kGenLdsBytes && P.PR * P.PC <= 512u) break;  // a thread stages up to two places per plane
     if (P.R > 1u) P.R /= 2u;
     else if (P.OWT > 4u) P.OWT = ((P.OWT / 2u) + 3u) & ~3u;
     else return ADH_EUNIMPL;
