@@ -178,7 +178,8 @@ int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N,
  * packed unpadded tensor, the 1x1 projections (src/zoo.cc:680-690): x_pad is a packed
  * (N,Cin,HP,WP) tensor convolved with conv pad 0, filter KCRS (Cout,Cin,kh,kw), stride (sh,sw),
  * dilation (dh,dw); OH = (HP - ((kh-1)*dh + 1)) / sh + 1, likewise OW
- * (cudnnGetConvolution2dForwardOutputDim, src/op.cc:1512-1523).  kh*kw <= 64, sh*sw <= 16.
+ * (cudnnGetConvolution2dForwardOutputDim, src/op.cc:1512-1523).  kh*kw <= 64, sh*sw <= 16,
+ * HP*WP < 2^30 (ADH_EINVAL beyond).
  * fp32 arithmetic on the matrix cores; ADH_BF16 tensors are widened on load and rounded on store.
  * The workspace (adh_conv2d_workspace_bytes, 256-byte aligned) holds the rewritten filter. */
 size_t adh_conv2d_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,

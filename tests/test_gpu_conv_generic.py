@@ -28,6 +28,11 @@ CASES = [  # K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw
     (1, 7, 12, 20, 10, 34, 3, 3, 2, 2, 1, 1),  # 4x16 outputs: four images per block, the last block holds three
     (2, 5, 40, 48, 6, 18, 3, 3, 2, 2, 1, 1),   # 2x8 outputs (a late layer's tile): all five images in one block
     (2, 6, 33, 20, 4, 16, 1, 1, 2, 2, 1, 1),   # strided 1x1 over a tiny tile, several images per block
+    (1, 2, 62, 30, 6, 10, 3, 3, 1, 1, 1, 1),   # 32-channel chunks whose last one is padded, in both passes
+    (1, 3, 31, 31, 8, 8, 1, 1, 1, 1, 1, 1),    # one padded 32-channel chunk
+    (1, 64, 8, 128, 18, 66, 3, 3, 1, 1, 1, 1), # enough blocks to keep them 64 output channels wide
+    (1, 32, 8, 128, 18, 66, 3, 3, 1, 1, 1, 1), # half as many: 32 output channels per block
+    (1, 48, 128, 8, 10, 66, 3, 3, 1, 1, 1, 1), # backward-data with 64-channel blocks and 32-channel chunks
 ]
 
 
