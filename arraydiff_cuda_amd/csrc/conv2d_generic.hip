@@ -428,6 +428,34 @@ static int gen_finish_plan(GenPlan *plan) {
     }
   }
   P.BR = std::max(1u, std::min(256u / P.BC, std::max(max_GI, 1u)));
+  // Fewer rows per block when that fills the 256 pixel slots better: a 9-row grid in blocks of 7 rows leaves the
+  // second block two rows, in blocks of 3 rows (two images per block) nothing.  Modelled time per pixel: the
+  // reciprocal of the filled share of the slots, times 1 + 0.39 * (patch rows staged per row of pixels); the
+  // factor is fitted to stride-2 backward-data on 17x65 and 9x33 grids, and a lower block must win by a tenth.
+  {
+    uint32_t span_r = 0;
+    for (uint32_t s = 0; s < P.nsub; ++s) {
+      int32_t lo = 0, hi = 0;
+      for (uint32_t t = P.sub[s].t0; t < P.sub[s].t1; ++t) {
+        if (t == P.sub[s].t0) lo = hi = P.off_r[t];
+        lo = std::min<int32_t>(lo, P.off_r[t]);
+        hi = std::max<int32_t>(hi, P.off_r[t]);
+      }
+      span_r = std::max(span_r, (uint32_t)(hi - lo));
+    }
+    const uint32_t gi = std::max(max_GI, 1u);
+    auto modelled = [&](uint32_t br) {
+      const uint32_t live = br * P.BC;
+      const uint32_t nb = live <= 128u ? std::min(256u / live, std::max(P.N, 1u)) : 1u;
+      const double filled = (double)gi / (double)(((gi + br - 1u) / br) * br) * (double)(nb * live) / 256.0;
+      const double patch_rows = (double)((br - 1u) * P.si_r + span_r + 1u) / (double)(br * P.si_r);
+      return (1.0 + 0.39 * patch_rows) / filled;
+    };
+    uint32_t best = P.BR;
+    for (uint32_t br = P.BR; br >= 1u; --br)
+      if (modelled(br) < modelled(best) - 1e-9) best = br;
+    if (modelled(best) < 0.9 * modelled(P.BR)) P.BR = best;
+  }
   // Output channels per block: 64, or fewer when there are no more of them, or when the launch would
   // leave compute units idle (a block's time is mostly the latency of staging its chunks, whatever its
   // width, so narrower blocks on more units finish sooner).
