@@ -432,7 +432,10 @@ static int gen_finish_plan(GenPlan *plan) {
   // second block two rows, in blocks of 3 rows (two images per block) nothing.  Modelled time per pixel: the
   // reciprocal of the filled share of the slots, times 1 + 0.39 * (patch rows staged per row of pixels); the
   // factor is fitted to stride-2 backward-data on 17x65 and 9x33 grids, and a lower block must win by a tenth.
-  {
+  // Only where the input is read at stride 1 (backward-data, stride-1 forward): a strided forward's patch has
+  // si_r rows per row of pixels, lower blocks push it out of the wider chunks, and the model does not hold
+  // (7x28 outputs of a stride-2 3x3: 9 one-row images per block ran 1.8 times slower than one 7-row image).
+  if (P.si_r == 1u) {
     uint32_t span_r = 0;
     for (uint32_t s = 0; s < P.nsub; ++s) {
       int32_t lo = 0, hi = 0;

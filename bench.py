@@ -130,6 +130,15 @@ def main():
             print("bench.py: the end-to-end trainer failed:\n" + r.stdout[-2000:] + r.stderr[-2000:], file=sys.stderr)
             sys.exit(4)
         end_to_end = json.loads(r.stdout.strip().splitlines()[-1])
+        # the same steps replayed from one recorded HIP graph (forward, backward, optimizer): reported beside the eager figure
+        g = subprocess.run([trainer, "--ranks", "4", "--batch", "32", "--size", "256", "--steps", "10", "--warmup", "3",
+                            "--graph", "1"], capture_output=True, text=True, timeout=600)
+        if g.returncode == 0:
+            replay = json.loads(g.stdout.strip().splitlines()[-1])
+            end_to_end["ms_per_step_graph_replay"] = replay["ms_per_step"]
+            end_to_end["graph_replay_same_loss"] = replay["loss_last"] == end_to_end["loss_last"]
+        else:
+            print("bench.py: the graph-replay run of the trainer failed:\n" + g.stdout[-1000:] + g.stderr[-1000:], file=sys.stderr)
 
     import numpy as np
     import torch
