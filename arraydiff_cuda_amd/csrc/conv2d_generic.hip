@@ -607,8 +607,12 @@ struct WgradGenParams {
   uint32_t N, Cin, Cout, HP, WP, OH, OW, sh, sw;
   uint32_t T, ntg, ntaps, COG, CIT;
   uint32_t R, OWT, nrb, ncb, units, PS;
+  // A unit is R x OWT pixels of one image, or, when that is a whole image of at most 32 pixel slots, of NBU
+  // consecutive images (unit pixel f is pixel f % img_pix of image f / img_pix; the images' patches lie side by
+  // side in a plane, PPI apart).  NG = ceil(N / NBU) image groups per tile.
+  uint32_t NBU, NG, img_pix, PPI;
   uint32_t PR, PC, PCP, PP, DP, dy_lds_floats;
-  FastDiv div_COG, div_CIT, div_ntg, div_ncb, div_nrb, div_N, div_OWT, div_PC, div_PR;
+  FastDiv div_COG, div_CIT, div_ntg, div_ncb, div_nrb, div_N, div_OWT, div_PC, div_PR, div_img_pix, div_PRPC;
   int16_t off_r[kGenMaxTaps], off_c[kGenMaxTaps];
 };
 
@@ -647,7 +651,7 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
 #pragma unroll
   for (int t = 0; t < TAPS; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const uint32_t unit_pix = P.R * P.OWT, ksteps = unit_pix >> 2;
+  const uint32_t unit_pix = P.NBU * P.img_pix, ksteps = unit_pix >> 2;
   // only the channels that exist are staged; lanes of absent channels read channel 0 and their sums are dropped
   const uint32_t planes = min(16u, P.Cin - cit * 16u);
   const uint32_t my_plane = l16 < planes ? l16 : 0u;
@@ -656,21 +660,24 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
   // Loads take a base address that is the same in every lane (the unit's origin in the channel plane) plus the
   // lane's 32-bit byte offset; places outside the tensors load offset 0 and are replaced by zero.
   const uint32_t wave_u = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave);
-  uint32_t dy_r, dy_c;
-  P.div_OWT.divmod(lane, dy_r, dy_c);
+  uint32_t dy_b, dy_p, dy_r, dy_c;
+  P.div_img_pix.divmod(lane, dy_b, dy_p);
+  P.div_OWT.divmod(dy_p, dy_r, dy_c);
   const bool dy_lane = lane < unit_pix;
-  const uint32_t dy_boff = (dy_r * P.OW + dy_c) * (uint32_t)sizeof(T);
+  const uint32_t dy_boff = (dy_b * P.Cout * P.OH * P.OW + dy_r * P.OW + dy_c) * (uint32_t)sizeof(T);
   const int32_t co_lim = (int32_t)P.Cout - (int32_t)(cog * 64u + wave_u * 16u);  // the wave's channels that exist
-  constexpr int KP = 2;  // PR * PC <= 512
-  uint32_t pr_rc[KP], pr_lds[KP], x_boff[KP];
+  constexpr int KP = 2;  // NBU * PR * PC <= 512
+  uint32_t pr_rc[KP], pr_b[KP], pr_lds[KP], x_boff[KP];
 #pragma unroll
   for (int k = 0; k < KP; ++k) {
     const uint32_t e = tid + k * kWgGenThreads;
-    uint32_t r, col;
-    P.div_PC.divmod(e, r, col);
-    pr_rc[k] = e < P.PR * P.PC ? (r << 16) | col : 0xffffffffu;
-    pr_lds[k] = r * P.PCP + col;
-    x_boff[k] = (r * P.WP + col) * (uint32_t)sizeof(T);
+    uint32_t b, ei, r, col;
+    P.div_PRPC.divmod(e, b, ei);
+    P.div_PC.divmod(ei, r, col);
+    pr_rc[k] = b < P.NBU ? (r << 16) | col : 0xffffffffu;
+    pr_b[k] = b;
+    pr_lds[k] = b * P.PPI + r * P.PCP + col;
+    x_boff[k] = (b * P.Cin * P.HP * P.WP + r * P.WP + col) * (uint32_t)sizeof(T);
   }
   const size_t x_plane = (size_t)P.HP * P.WP, dy_plane = (size_t)P.OH * P.OW;
   // A unit travels memory -> registers -> LDS; the next unit's loads are in flight while this one is multiplied.
@@ -683,12 +690,13 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
     P.div_ncb.divmod(u, r2, cb);
     P.div_nrb.divmod(r2, r3, rb);
     P.div_N.divmod(r3, tile, n);
+    n *= P.NBU;  // the unit's first image
     const uint32_t oh0 = rb * P.R, ow0 = cb * P.OWT;
     const T *xs = reinterpret_cast<const T *>(P.x[tile]) + ((size_t)n * P.Cin + cit * 16u) * x_plane +
                   (size_t)oh0 * P.sh * P.WP + (size_t)ow0 * P.sw;
     const T *ds = reinterpret_cast<const T *>(P.dy[tile]) + ((size_t)n * P.Cout + cog * 64u + wave_u * 16u) * dy_plane +
                   (size_t)oh0 * P.OW + ow0;
-    const bool dy_in = dy_lane && oh0 + dy_r < P.OH && ow0 + dy_c < P.OW;
+    const bool dy_in = dy_lane && n + dy_b < P.N && oh0 + dy_r < P.OH && ow0 + dy_c < P.OW;
     pre_in = dy_in ? 1u : 0u;
     const uint32_t dy_off = dy_in ? dy_boff : 0u;
 #pragma unroll
@@ -696,7 +704,8 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
       dy_pre[c] = gen_ld_b(ds + (ptrdiff_t)(dy_c0 + min(c, dy_cmax)) * (ptrdiff_t)dy_plane, dy_off);
 #pragma unroll
     for (int k = 0; k < KP; ++k) {
-      const bool in = pr_rc[k] != 0xffffffffu && oh0 * P.sh + (pr_rc[k] >> 16) < P.HP && ow0 * P.sw + (pr_rc[k] & 0xffffu) < P.WP;
+      const bool in = pr_rc[k] != 0xffffffffu && n + pr_b[k] < P.N && oh0 * P.sh + (pr_rc[k] >> 16) < P.HP &&
+                      ow0 * P.sw + (pr_rc[k] & 0xffffu) < P.WP;
       pre_in |= in ? 2u << k : 0u;
       const uint32_t off = in ? x_boff[k] : 0u;
 #pragma unroll
@@ -719,12 +728,15 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
     }
   };
   const float *arow = dyl + (wave * 16u + l16) * P.DP + g;
-  const float *bpl = patch + (PACKED ? 0u : my_plane * P.PP);
+  const float *bpl_g = patch + (PACKED ? 0u : my_plane * P.PP) + g * P.sw;
   // the operands of k-step ks: four consecutive pixels of the unit, one per lane group
   auto fetch = [&](uint32_t ks, float &a, float (&b)[TAPS]) {
-    uint32_t r, c;
-    P.div_OWT.divmod((ks << 2) + g, r, c);
-    const float *brow = bpl + r * P.sh * P.PCP + c * P.sw;
+    // the step's four pixels lie in one row (OWT is a multiple of 4): where the first one is is the same in every
+    // lane and is worked out on the scalar unit; the lane adds its own pixel (bpl_g)
+    uint32_t img, ip, r, c;
+    P.div_img_pix.divmod(ks << 2, img, ip);
+    P.div_OWT.divmod(ip, r, c);
+    const float *brow = bpl_g + (img * P.PPI + r * P.sh * P.PCP + c * P.sw);
     a = arow[ks << 2];
 #pragma unroll
     for (int t = 0; t < TAPS; ++t) b[t] = PACKED ? brow[pair_off[t]] : brow[__builtin_amdgcn_readlane(delta_vec, t)];
@@ -841,28 +853,37 @@ static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *p
     P.PR = (P.R - 1u) * g.sh + span_r;
     P.PC = (P.OWT - 1u) * g.sw + span_c;
     P.PCP = P.PC;
-    uint32_t pp = P.PR * P.PCP;
+    P.PPI = P.PR * P.PCP;
+    P.nrb = (g.OH + P.R - 1u) / P.R;
+    P.ncb = (g.OW + P.OWT - 1u) / P.OWT;
+    P.img_pix = P.R * P.OWT;
+    // several images per unit when a whole image takes at most half of a unit's 64 pixel slots; the images of a
+    // unit are reached from one base address by 32-bit byte offsets
+    P.NBU = P.nrb == 1u && P.ncb == 1u && P.img_pix <= 32u ? std::min(64u / P.img_pix, std::max(g.N, 1u)) : 1u;
+    while (P.NBU > 1u && (P.NBU * P.PR * P.PC > 512u ||
+                          (uint64_t)P.NBU * std::max((uint64_t)g.Cin * g.HP * g.WP, (uint64_t)g.Cout * g.OH * g.OW) >= (1ull << 30)))
+      --P.NBU;
+    uint32_t pp = P.NBU * P.PPI;
     while (pp % 64u != 4u * std::min<uint32_t>(g.sw, 4u) % 64u) ++pp;  // 16 channels x 4 pixels on distinct banks
     P.PP = pp;
-    uint32_t dp = P.R * P.OWT;
+    uint32_t dp = P.NBU * P.img_pix;
     while (dp % 64u != 4u) ++dp;
     P.DP = dp;
     P.dy_lds_floats = 64u * P.DP;
     plan->lds_bytes = ((size_t)P.dy_lds_floats + 16u * (size_t)P.PP) * 4u;
-    if (plan->lds_bytes <= kGenLdsBytes && P.PR * P.PC <= 512u) break;  // a thread stages up to two places per plane
+    if (plan->lds_bytes <= kGenLdsBytes && P.NBU * P.PR * P.PC <= 512u) break;  // a thread stages up to two places per plane
     if (P.R > 1u) P.R /= 2u;
     else if (P.OWT > 4u) P.OWT = ((P.OWT / 2u) + 3u) & ~3u;
     else return ADH_EUNIMPL;
   }
-  P.nrb = (g.OH + P.R - 1u) / P.R;
-  P.ncb = (g.OW + P.OWT - 1u) / P.OWT;
-  const uint64_t units = (uint64_t)num_tiles * g.N * P.nrb * P.ncb;
+  P.NG = (g.N + P.NBU - 1u) / P.NBU;
+  const uint64_t units = (uint64_t)num_tiles * P.NG * P.nrb * P.ncb;
   if (units == 0 || units >= (1ull << 31)) return ADH_EINVAL;
   P.units = (uint32_t)units;
   const uint64_t fixed = (uint64_t)P.COG * P.CIT * P.ntg;
   const size_t stride_bytes = (size_t)fixed * P.T * 1024u * 4u;
   uint64_t ps = std::max<uint64_t>(1u, 1024u / fixed);  // about four workgroups per CU: they hide each other's staging
-  if (P.T > 9u) ps = std::max<uint64_t>(1u, 256u / fixed);  // the ten-tile variant runs one workgroup per CU
+  if (P.T > 9u) ps = std::max<uint64_t>(1u, 512u / fixed);  // the ten-tile variant: two workgroups per CU, one round
   ps = std::min<uint64_t>(ps, units);
   while (ps > 1u && ps * stride_bytes > (256ull << 20)) ps /= 2u;
   if (fixed * ps >= (1ull << 24)) return ADH_EINVAL;
@@ -871,8 +892,9 @@ static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *p
   plan->blocks = (uint32_t)(fixed * ps);
   plan->partial_bytes = (size_t)plan->nparts * stride_bytes;
   P.div_COG = FastDiv(P.COG); P.div_CIT = FastDiv(P.CIT); P.div_ntg = FastDiv(P.ntg);
-  P.div_ncb = FastDiv(P.ncb); P.div_nrb = FastDiv(P.nrb); P.div_N = FastDiv(g.N);
+  P.div_ncb = FastDiv(P.ncb); P.div_nrb = FastDiv(P.nrb); P.div_N = FastDiv(P.NG);
   P.div_OWT = FastDiv(P.OWT); P.div_PC = FastDiv(P.PC); P.div_PR = FastDiv(P.PR);
+  P.div_img_pix = FastDiv(P.img_pix); P.div_PRPC = FastDiv(P.PR * P.PC);
   return ADH_OK;
 }
 
