@@ -56,10 +56,12 @@ struct ConvParams {
   FastDiv div_tiles_x, div_TW;
 };
 
-static constexpr int kPatchRows = 12;                                  // staged patch rows (>= R + 2)
-static constexpr int kChanStride = kPatchRows * kLdsPitch + 16;        // == 16 (mod 64)
-static constexpr int kPatchFloats = kChunk * kChanStride;
+// staged patch rows (>= R + 2): 12, or 20 in the tall variant of the kernel, which is a few percent slower per
+// flop (more rows to stage per wave) and is chosen where taller tiles waste fewer pixel slots
+static constexpr int kPatchRows = 12;
+static constexpr int kPatchRowsTall = 20;
 static constexpr int kMaxR = kPatchRows - 2;
+static constexpr int kMaxRTall = kPatchRowsTall - 2;
 
 template <int V>
 struct IntTag {
@@ -73,13 +75,15 @@ struct IntTag {
 //            other wave's MFMAs while every SIMD still carries exactly NT tile-MFMAs per k-step
 // FLIP  = false: forward (weights walked as w[o][k][tap]); true: backward-data
 //         (weights walked as w[k][o][8-tap]).
-template <int NT, int WAVES, bool FLIP>
+template <int NT, int WAVES, bool FLIP, int PROWS>
 __global__ __launch_bounds__(64 * WAVES, 1) void conv3x3_f32_kernel(const ConvParams P) {
+  constexpr int kChanStride = PROWS * kLdsPitch + 16;  // == 16 (mod 64)
+  constexpr int kPatchFloats = kChunk * kChanStride;
   constexpr int kThreads = 64 * WAVES;
   constexpr int G = WAVES / 4;                 // pixel groups
   constexpr int NTA = (NT + G - 1) / G;        // tiles of every group but the last
   constexpr int NTL = NT - (G - 1) * NTA;      // tiles of the last group
-  constexpr int RROWS = (kPatchRows + WAVES - 1) / WAVES;
+  constexpr int RROWS = (PROWS + WAVES - 1) / WAVES;
   constexpr int WLOADS = kWBufFloats / kThreads;
   static_assert(kWBufFloats % kThreads == 0 && NTL > 0, "bad configuration");
   // two patch buffers and two weight buffers as separate arrays: the compiler can then tell
@@ -137,7 +141,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void conv3x3_f32_kernel(const ConvPa
 #pragma unroll
     for (int rr = 0; rr < RROWS; ++rr) {
       const uint32_t prow = wv + (uint32_t)WAVES * rr;
-      if (kPatchRows % WAVES != 0 && prow >= (uint32_t)kPatchRows) continue;  // wave-uniform
+      if (PROWS % WAVES != 0 && prow >= (uint32_t)PROWS) continue;  // wave-uniform
 #pragma unroll
       for (int kl = 0; kl < kChunk; ++kl) {
         float *dst = buf + kl * kChanStride + prow * kLdsPitch;
@@ -330,14 +334,15 @@ static ConvTile choose_tile(uint32_t OH, uint32_t OW, uint64_t planes, uint32_t 
       const uint32_t TW = (OW + ncol - 1) / ncol;
       if (TW == 0 || TW > (uint32_t)kMaxTW || TW > cap) continue;
       uint32_t Rmax = cap / TW;
-      if (Rmax > (uint32_t)kMaxR) Rmax = (uint32_t)kMaxR;
+      const uint32_t max_r = nt == 8 ? (uint32_t)kMaxR : (uint32_t)kMaxRTall;  // the four-wave variant has no tall form
+      if (Rmax > max_r) Rmax = max_r;
       if (Rmax > OH) Rmax = OH;
       for (uint32_t R = 1; R <= Rmax; ++R) {
         const uint64_t tiles_y = (OH + R - 1) / R;
         const uint64_t blocks = tiles_y * ncol * planes * o_groups;
         const uint64_t rounds = (blocks + 255) / 256;
         // second-order term prefers fewer, fuller workgroups when rounds tie
-        const double rate = nt == 8 ? 0.68 : nt == 29 ? 0.95 : 1.0;
+        const double rate = (nt == 8 ? 0.68 : nt == 29 ? 0.95 : 1.0) * (R > (uint32_t)kMaxR ? 0.95 : 1.0);
         const double cost = ((double)rounds * nt + 1e-6 * (double)blocks * nt) / rate;
         if (cost < best_cost) {
           best_cost = cost;
@@ -349,12 +354,17 @@ static ConvTile choose_tile(uint32_t OH, uint32_t OW, uint64_t planes, uint32_t 
   return best;
 }
 
+template <int NT, int WAVES, int PROWS>
+static void launch_conv_rows(const ConvParams &P, dim3 grid, hipStream_t st) {
+  if (P.w_flip)
+    hipLaunchKernelGGL((conv3x3_f32_kernel<NT, WAVES, true, PROWS>), grid, dim3(64 * WAVES), 0, st, P);
+  else
+    hipLaunchKernelGGL((conv3x3_f32_kernel<NT, WAVES, false, PROWS>), grid, dim3(64 * WAVES), 0, st, P);
+}
 template <int NT, int WAVES>
 static void launch_conv(const ConvParams &P, dim3 grid, hipStream_t st) {
-  if (P.w_flip)
-    hipLaunchKernelGGL((conv3x3_f32_kernel<NT, WAVES, true>), grid, dim3(64 * WAVES), 0, st, P);
-  else
-    hipLaunchKernelGGL((conv3x3_f32_kernel<NT, WAVES, false>), grid, dim3(64 * WAVES), 0, st, P);
+  if (WAVES == 8 && P.R > (uint32_t)kMaxR) launch_conv_rows<NT, WAVES, (WAVES == 8 ? kPatchRowsTall : kPatchRows)>(P, grid, st);
+  else launch_conv_rows<NT, WAVES, kPatchRows>(P, grid, st);
 }
 
 int conv_bf16_via_f32(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
