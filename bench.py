@@ -207,7 +207,7 @@ def main():
         "config": {"workload": "configs[1]: 3x3 slab conv fwd, fp32 NCHW N=32 Cin=Cout=64, 4 row-tiles of "
                                "14(+2)x56(+2), one launch over all tiles",
                    "flops_per_step": flops_step, "tiles": K, "halo": p},
-        "roofline": {"kernel": "conv3x3_f32_kernel<25,8,false> (fwd)", "bound": "mfma", "achieved": round(achieved, 3),
+        "roofline": {"kernel": "conv3x3_f32_kernel<25,8,false,12> (fwd)", "bound": "mfma", "achieved": round(achieved, 3),
                      "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / MFMA_F32_PEAK_TFLOPS, 4),
                      "traffic": CONV_FWD_CFG2_TRAFFIC_BYTES, "launch_ms": round(kernel_ms, 5)},
     }
