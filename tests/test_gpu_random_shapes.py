@@ -12,7 +12,7 @@ from gpu_util import dev, host, rel_err
 pytestmark = pytest.mark.gpu
 
 
-def _conv_cases(seed, count):
+def _conv_cases(seed, count, max_n=3, max_cin=20, max_cout=40):
     rng = np.random.default_rng(seed)
     out = []
     while len(out) < count:
@@ -21,7 +21,8 @@ def _conv_cases(seed, count):
         dh, dw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
         eh, ew = (kh - 1) * dh + 1, (kw - 1) * dw + 1
         HP, WP = eh + int(rng.integers(0, 12)), ew + int(rng.integers(0, 40))
-        out.append((int(rng.integers(1, 3)), int(rng.integers(1, 4)), int(rng.integers(1, 21)), int(rng.integers(1, 41)),
+        out.append((int(rng.integers(1, 3)), int(rng.integers(1, max_n + 1)), int(rng.integers(1, max_cin + 1)),
+                    int(rng.integers(1, max_cout + 1)),
                     HP, WP, kh, kw, sh, sw, dh, dw))
     return out
 
@@ -63,6 +64,12 @@ def _pool_cases(seed, count):
         out.append((int(rng.integers(1, 3)), int(rng.integers(1, 4)), int(rng.integers(1, 9)), wh + int(rng.integers(0, 20)),
                     ww + int(rng.integers(0, 150)), wh, ww, int(rng.integers(1, 4)), int(rng.integers(1, 4)), int(rng.integers(0, 2))))
     return out
+
+
+# more images and channels: several images per block / per backward-filter unit, 16- and 32-channel chunks (some padded)
+@pytest.mark.parametrize("K,N,Cin,Cout,HP,WP,kh,kw,sh,sw,dh,dw", _conv_cases(7, 48, max_n=9, max_cin=70, max_cout=70))
+def test_general_conv_random_wide(oracle, K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw):
+    test_general_conv_random(oracle, K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw)
 
 
 @pytest.mark.parametrize("K,N,C,HP,WP,wh,ww,sh,sw,mode", _pool_cases(2025, 20))
