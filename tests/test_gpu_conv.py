@@ -26,7 +26,10 @@ def workspace(which, K, N, Cin, Cout, H, W):
 SMALL = [  # K, N, Cin, Cout, H, W
     (1, 1, 8, 16, 4, 8), (1, 2, 3, 5, 5, 7), (2, 2, 16, 16, 6, 17), (1, 1, 64, 64, 14, 56), (3, 1, 9, 70, 11, 13),
     (1, 1, 130, 20, 3, 60), (2, 3, 24, 40, 23, 5), (1, 2, 4, 4, 1, 1), (1, 1, 8, 8, 5, 61), (2, 1, 16, 8, 9, 150),
-    (1, 1, 4, 36, 3, 257)]
+    (1, 1, 4, 36, 3, 257),
+    # many planes of a 16x20 / 11x20 tile: the launch is large enough for the 8-wave kernels, whose tall form
+    # (tiles of up to 18 rows, 20 staged patch rows) then wins: forward 16 and 11 rows per tile, backward-data 18 and 13
+    (2, 96, 8, 8, 16, 20), (2, 96, 8, 16, 11, 20)]
 
 
 @pytest.mark.parametrize("K,N,Cin,Cout,H,W", SMALL)
