@@ -1,0 +1,59 @@
+// Declarations shared by the two bf16 matrix-core 3x3 slab convolution kernels
+// (conv3x3_bf16_mfma.hip: four waves, any shape; conv3x3_bf16_w8.hip: eight waves, even widths).
+#ifndef ADH_CONV3X3_BF16_MFMA_H
+#define ADH_CONV3X3_BF16_MFMA_H
+
+#include <utility>
+
+#include "adh_common.h"
+
+namespace adh {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
+
+constexpr int kStripCols = 64;                        // output columns per work item
+constexpr int kStepRows = 4;                          // output rows per step
+constexpr uint32_t kOutOfRange = 0x80000000u;
+constexpr uint32_t kWtGroupElems = 9u * 2u * 64u * 32u;  // transformed filter elements per group of 64 outputs
+
+struct ConvBf16Params {
+  const uint16_t *in[ADH_MAX_TILES];
+  uint16_t *out[ADH_MAX_TILES];
+  const uint16_t *wt;       // transformed filter: [group][tap][half][64 out][32 red]
+  uint32_t N, Cred, Cout;   // reduction and output channel counts as the kernel sees them
+  uint32_t IH, IW, OH, OW;
+  int32_t pad;              // input row/col = output row/col + tap - pad
+  float beta;
+  // An item is a strip of an image (strip index fastest).  The first `whole_items` are dealt to
+  // the workgroups in turn, top to bottom each; what is left over (fewer items than workgroups)
+  // is cut into row segments of `seg_steps` steps so that it spreads over all of them.
+  uint32_t strips, items, whole_items, steps_per_item, seg_steps, segs, pieces;
+  FastDiv div_strips, div_N, div_rest;
+};
+
+template <int V>
+struct IntTag { static constexpr int value = V; };
+template <int... T, typename F>
+__device__ __forceinline__ void for_each_int(std::integer_sequence<int, T...>, F &&f) {
+  (f(IntTag<T>()), ...);
+}
+
+// two floats -> two bf16 (round to nearest even) in one dword: one v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  const floatx2 f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+
+// the eight-wave kernel: shapes it takes, and its launch (grid.x workgroups per output group)
+bool conv_bf16_w8_takes(const ConvBf16Params &P, uint32_t num_tiles);
+int conv_bf16_w8_launch(const ConvBf16Params &P, uint32_t gx, uint32_t groups, hipStream_t st);
+
+}  // namespace adh
+
+#endif

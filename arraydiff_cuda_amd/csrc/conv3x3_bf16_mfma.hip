@@ -24,20 +24,10 @@
 //
 // Out-of-range rows, channels and buffer ends are handled by the buffer resource's range check
 // (out-of-range dwords read as zero); out-of-range columns by per-dword masks.
-#include <utility>
-
-#include "adh_common.h"
+#include "conv3x3_bf16_mfma.h"
 
 namespace adh {
 
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef u32x4 u32x4_unaligned __attribute__((aligned(2)));
-
-constexpr int kStripCols = 64;                        // output columns per work item
-constexpr int kStepRows = 4;                          // output rows per step
 constexpr int kRingRows = 10;                         // 6 rows in use + 4 rows being written
 constexpr int kPatchCols = kStripCols + 2;            // 66
 // LDS layout of a ring row: pixel px sits in slot px + px / 8 (one empty slot after every eight
@@ -50,23 +40,6 @@ constexpr int kRowSlots = kPatchCols + kPatchCols / 8;   // 74
 constexpr int kRowPitch = kRowSlots * kPxPitch;       // 11840
 constexpr int kRingBytes = kRingRows * kRowPitch;     // 118400
 __host__ __device__ constexpr int px_slot(int px) { return px + (px >> 3); }
-constexpr uint32_t kOutOfRange = 0x80000000u;
-constexpr uint32_t kWtGroupElems = 9u * 2u * 64u * 32u;  // transformed filter elements per group of 64 outputs
-
-struct ConvBf16Params {
-  const uint16_t *in[ADH_MAX_TILES];
-  uint16_t *out[ADH_MAX_TILES];
-  const uint16_t *wt;       // transformed filter: [group][tap][half][64 out][32 red]
-  uint32_t N, Cred, Cout;   // reduction and output channel counts as the kernel sees them
-  uint32_t IH, IW, OH, OW;
-  int32_t pad;              // input row/col = output row/col + tap - pad
-  float beta;
-  // An item is a strip of an image (strip index fastest).  The first `whole_items` are dealt to
-  // the workgroups in turn, top to bottom each; what is left over (fewer items than workgroups)
-  // is cut into row segments of `seg_steps` steps so that it spreads over all of them.
-  uint32_t strips, items, whole_items, steps_per_item, seg_steps, segs, pieces;
-  FastDiv div_strips, div_N, div_rest;
-};
 
 // filter (Cout, Cin, 3, 3) -> matrix-operand order.  flip = 0 (forward): out = Cout index,
 // red = Cin index, tap as is.  flip = 1 (backward-data): out = Cin index, red = Cout index,
@@ -86,22 +59,6 @@ __global__ __launch_bounds__(256) void conv3x3_bf16_filter_kernel(const uint16_t
     if (oc < Cin && rc < Cout) v = w[((uint64_t)rc * Cin + oc) * 9u + (8u - tap)];
   }
   wt[i] = v;
-}
-
-template <int V>
-struct IntTag { static constexpr int value = V; };
-template <int... T, typename F>
-__device__ __forceinline__ void for_each_int(std::integer_sequence<int, T...>, F &&f) {
-  (f(IntTag<T>()), ...);
-}
-
-typedef float floatx2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-
-// two floats -> two bf16 (round to nearest even) in one dword: one v_cvt_pk_bf16_f32
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  const floatx2 f = {a, b};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
 }
 
 template <bool BETA>
@@ -602,6 +559,7 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
   P.div_strips = FastDiv(P.strips);
   P.div_N = FastDiv(N);
   P.div_rest = FastDiv(rest ? rest : 1u);
+  if (conv_bf16_w8_takes(P, num_tiles)) return conv_bf16_w8_launch(P, gx, groups, st);
   if (beta != 0.f)
     hipLaunchKernelGGL(conv3x3_bf16_kernel<true>, dim3(gx, groups), dim3(256), 0, st, P);
   else

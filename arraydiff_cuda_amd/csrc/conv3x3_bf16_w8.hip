@@ -1,0 +1,554 @@
+// 3x3 slab convolution on the bf16 matrix cores (v_mfma_f32_16x16x32_bf16), forward and
+// backward-data, for up to 64 reduction channels: the eight-wave kernel, two waves per SIMD.
+//
+// A persistent workgroup of eight waves walks work items (image, 64-column strip, row segment)
+// four output rows at a time, like the four-wave kernel of conv3x3_bf16_mfma.hip, and keeps the
+// strip's input rows in LDS as a ring of ten rows in [pixel][channel] order, so that the matrix
+// operand of 16 pixels x 32 channels is one 16-byte LDS read per lane at any column shift.  What
+// differs is how rows get there and how the work is cut:
+//
+// * Rows arrive by `buffer_load ... lds` (16 bytes per lane, asynchronous, no registers) in the
+//   order they have in memory, [channel][pixel]: every wave copies eight channels x four rows x
+//   nine 8-pixel granules into a staging area of its own.  Rows, channels and granules that do
+//   not exist get an out-of-range offset and arrive as zeros.
+// * The wave then turns its own staging area into ring order with the transposing LDS read
+//   (ds_read_b64_tr_b16: inside a group of 16 lanes, four lanes read one channel's 16 pixels and
+//   every lane receives one pixel's four channels): two such reads and one 16-byte write per
+//   16 pixels x 8 channels per lane group, no byte permutes, no masks.  Because a wave only ever
+//   refills the staging area it has just read, one barrier per step is enough.
+// * A wave owns 32 output channels x 32 columns x 2 rows: 48 operand reads and 144 MFMAs per
+//   step, its filter share (9 taps x 64 x 32) in 144 registers; 8 accumulator tiles.  That fits
+//   256 registers, so two waves share a SIMD and one fills the other's stalls.  Waves 0-3
+//   transpose and request before they multiply, waves 4-7 after: the matrix pipe of every SIMD
+//   has work while its other wave moves data.
+// * The sequence of row groups runs on across work items (the first rows of the next item are
+//   requested during the last steps of the current one); an item costs one step without MFMAs.
+//
+// Forward takes the halo-padded input as it is (strip columns c0 .. c0 + 71).  Backward-data
+// reads the unpadded gradient from column c0 - 8 (granules stay 16-byte aligned and are wholly
+// inside or outside a row when the width is a multiple of 8) and finds its first column six
+// pixels into the ring row.
+#include "conv3x3_bf16_mfma.h"
+
+namespace adh {
+
+namespace {
+
+constexpr int kW8Threads = 512;
+constexpr int kW8PxBytes = 160;                          // 64 channels + 32 bytes: measured, 16-byte reads of 16 neighbouring pixels run at the linear rate (4.5 cycles per wave; 8 at 144 bytes)
+constexpr int kW8RowPx = 72;                             // nine granules of eight pixels
+constexpr int kW8RowBytes = kW8RowPx * kW8PxBytes;       // 11520
+constexpr int kW8RingRows = 10;                          // 6 rows in use + 4 rows being written
+constexpr int kW8RingBytes = kW8RingRows * kW8RowBytes;  // 115200
+constexpr int kW8RawCh = 144;                            // a channel row in the staging area: 72 pixels
+constexpr int kW8Copies = 5;                             // 4 rows x 8 channels x 9 granules = 288 lanes of 5 x 64
+constexpr int kW8RawWave = kW8Copies * 1024;
+constexpr int kW8RawBytes = 8 * kW8RawWave;              // 40960
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+#define ADH_LDS __attribute__((address_space(3)))
+
+__device__ __forceinline__ u32x2 lds_read_tr(const uint8_t *p) {
+  return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((ADH_LDS s16x4 *)p));
+}
+
+__device__ __forceinline__ uint32_t wrap_slot(uint32_t s) { return s >= (uint32_t)kW8RingRows ? s - (uint32_t)kW8RingRows : s; }
+
+#ifdef W8_TIMING
+__device__ uint64_t w8_dbg[64];
+#endif
+
+template <bool BETA>
+__global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16Params P) {
+#ifdef W8_TIMING
+  const uint64_t dbg_c0 = __builtin_readcyclecounter(), dbg_r0 = __builtin_amdgcn_s_memrealtime();
+  uint64_t dbg_move = 0, dbg_comp = 0, dbg_bar = 0, dbg_mm = 0, dbg_tb = 0, dbg_post = 0;
+#endif
+  __shared__ __attribute__((aligned(16))) uint8_t raw[kW8RawBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t ring[kW8RingBytes];
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
+  const uint32_t wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t h = wv & 1u, cw = (wv >> 1) & 1u, rp = wv >> 2;  // output-channel half, column half, row pair
+  const uint32_t grp = blockIdx.y;
+
+  // Workgroups are dealt to the eight XCDs (each with its own L2) in turn.  Renumber them so
+  // that an XCD works on neighbouring strips: those share the 128-byte lines at strip borders.
+  uint32_t vblock = blockIdx.x;
+  if ((gridDim.x & 7u) == 0u) vblock = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  const uint32_t total = P.whole_items + P.pieces;
+  if (vblock >= total) return;
+
+  // this wave's filter share, in B-operand order: lane (n = l16, k-block = g)
+  u32x4 wreg[9][2][2];
+  {
+    const u32x4 *wt = reinterpret_cast<const u32x4 *>(P.wt + (size_t)grp * kWtGroupElems);
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap)
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+          wreg[tap][half][ct] = wt[((tap * 2 + half) * 64 + (int)(32u * h + 16u * ct + l16)) * 4 + (int)g];
+  }
+
+  const uint32_t plane_bytes = P.IH * P.IW * 2u;
+  const uint32_t image_bytes = P.Cred * plane_bytes;
+  const uint32_t xoff = P.pad ? 6u : 0u;        // ring pixel of the strip's first output column at tap column 0
+  const int32_t col_back = P.pad ? 8 : 0;       // the staged row starts this many columns left of the strip
+
+  // ---- requests: copy q of a group moves staging slots 64 q + lane; slot = (row * 8 + channel) * 9 + granule
+  uint32_t ld_off[kW8Copies];   // byte offset of the slot's granule for row 0 of the group and strip column 0
+  uint32_t ld_rows = 0;         // 3 bits per copy: row of the group, bit 2 = the slot exists and so does its channel
+  uint32_t ld_gran = 0;         // 4 bits per copy: granule
+#pragma unroll
+  for (int q = 0; q < kW8Copies; ++q) {
+    const uint32_t slot = 64u * q + lane;
+    const uint32_t row = slot / 72u, rem = slot - row * 72u, ch = rem / 9u, gran = rem - ch * 9u;
+    const uint32_t chan = 8u * wv + ch;
+    const bool ok = slot < 288u && chan < P.Cred;
+    ld_off[q] = chan * plane_bytes + row * P.IW * 2u + gran * 16u;
+    ld_rows |= ((row & 3u) | (ok ? 4u : 0u)) << (3 * q);
+    ld_gran |= gran << (4 * q);
+  }
+  uint8_t *const raw_wave = raw + wv * kW8RawWave;
+
+  // ---- turning the staging area into ring order.  Lane (j = l16, g): rounds 0-3 handle row t,
+  // pixel block g; round 4 handles row g, pixel block 4 (pixels 64-71; its lanes 8-15 of a group
+  // hold pixels 72-79, which do not exist, and write to the unused tail of the staging area).  A
+  // transposing read takes channel j / 4 (+ 4 in the second read) at pixels 16 b + 4 (j % 4) and
+  // returns pixel 16 b + j.
+  const uint32_t tr_lane = (l16 >> 2) * kW8RawCh + (l16 & 3u) * 8u;
+  const uint8_t *const tr03 = raw_wave + tr_lane + g * 32u;                  // + t * 8 * kW8RawCh
+  const uint8_t *const tr4 = raw_wave + tr_lane + g * 8u * kW8RawCh + 128u;
+  const uint32_t wr03 = (16u * g + l16) * kW8PxBytes + wv * 16u;             // + slot(row t) * kW8RowBytes
+  const uint32_t wr4 = (64u + l16) * kW8PxBytes + wv * 16u;                  // + slot(row g) * kW8RowBytes
+  uint8_t *const wr4_dummy = raw_wave + 288 * 16 + ((l16 & 7u) + 8u * g) * 16u;
+
+  uint32_t tb = 0;  // ring slot the next transposed group starts at
+  struct TrPair { u32x2 lo, hi; };
+  auto tr_read = [&](auto tag, TrPair &T) {
+    constexpr int t = decltype(tag)::value;
+    if constexpr (t < 4) {
+      T.lo = lds_read_tr(tr03 + t * 8 * kW8RawCh);
+      T.hi = lds_read_tr(tr03 + t * 8 * kW8RawCh + 4 * kW8RawCh);
+    } else {
+      T.lo = lds_read_tr(tr4);
+      T.hi = lds_read_tr(tr4 + 4 * kW8RawCh);
+    }
+  };
+  auto tr_write = [&](auto tag, const TrPair &T) {
+    constexpr int t = decltype(tag)::value;
+    const u32x4 v = {T.lo[0], T.lo[1], T.hi[0], T.hi[1]};
+    if constexpr (t < 4) {
+      *reinterpret_cast<u32x4 *>(ring + wrap_slot(tb + (uint32_t)t) * kW8RowBytes + wr03) = v;
+    } else {
+      uint8_t *const dst = ring + wrap_slot(tb + g) * kW8RowBytes + wr4;
+      *reinterpret_cast<u32x4 *>(l16 < 8u ? dst : wr4_dummy) = v;
+    }
+  };
+
+  // ---- the loader's place in the sequence of row groups: work item, group -1 .. steps - 1
+  // (group k holds the item's ring-relative rows 4 k + 2 .. 4 k + 5; rows -2, -1 are never used)
+  uint32_t workL = vblock;
+  int32_t grpL = -1, stepsL = 0;
+  int32_t arow0L = 0, colL = 0;          // input row of ring-relative row 0, input column of staged pixel 0
+  uint32_t okL = 0;                      // 5 bits: copy q of this lane exists for this item (slot, channel, granule column)
+  __amdgpu_buffer_rsrc_t rsrcL = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(P.in[0]), 0, 0, 0x00020000);
+
+  // decodes a work number into (tile, image, first column, first and last output row)
+  auto decode = [&](uint32_t work, uint32_t &tile, uint32_t &n, uint32_t &c0, uint32_t &r_begin, uint32_t &r_end) {
+    uint32_t item, seg = 0, seg_steps = P.steps_per_item;
+    if (work < P.whole_items) {
+      item = work;
+    } else {
+      uint32_t it;
+      P.div_rest.divmod(work - P.whole_items, seg, it);
+      item = P.whole_items + it;
+      seg_steps = P.seg_steps;
+    }
+    uint32_t strip, plane;
+    P.div_strips.divmod(item, plane, strip);
+    P.div_N.divmod(plane, tile, n);
+    c0 = strip * kStripCols;
+    r_begin = seg * seg_steps * kStepRows;
+    r_end = min(P.OH, r_begin + seg_steps * kStepRows);
+  };
+
+  auto loader_open = [&]() {
+    uint32_t tile, n, c0, r_begin, r_end;
+    decode(workL, tile, n, c0, r_begin, r_end);
+    stepsL = (int32_t)((r_end - r_begin + kStepRows - 1) / kStepRows);
+    arow0L = (int32_t)r_begin - P.pad;
+    colL = (int32_t)c0 - col_back;
+    const uint16_t *in_img = P.in[tile] + (size_t)n * P.Cred * P.IH * P.IW;
+    rsrcL = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(in_img), 0, image_bytes, 0x00020000);
+    okL = 0;
+#pragma unroll
+    for (int q = 0; q < kW8Copies; ++q) {
+      const int32_t col = colL + 8 * (int32_t)((ld_gran >> (4 * q)) & 15u);
+      const bool ok = ((ld_rows >> (3 * q)) & 4u) && col >= 0 && col < (int32_t)P.IW;
+      okL |= (ok ? 1u : 0u) << q;
+    }
+    grpL = -1;
+  };
+  // Copy q of the loader's current group.  Once all work has been requested okL is zero and the
+  // copies only write zeros, which go to ring rows nobody reads: the sequence needs no branches.
+  auto request = [&](auto tag) {
+    constexpr int q = decltype(tag)::value;
+    const int32_t first = arow0L + 4 * grpL + 2;   // input row of the group's first row
+    const int32_t base = (first * (int32_t)P.IW + colL) * 2;
+    const int32_t arow = first + (int32_t)((ld_rows >> (3 * q)) & 3u);
+    const bool ok = ((okL >> q) & 1u) && (uint32_t)arow < P.IH;
+    const uint32_t v = ok ? ld_off[q] + (uint32_t)base : kOutOfRange;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcL, (ADH_LDS void *)(raw_wave + q * 1024), 16, v, 0, 0, 0);
+  };
+  auto loader_advance = [&]() {
+    if (workL >= total) return;
+    if (++grpL == stepsL) {
+      workL += gridDim.x;
+      if (workL < total)
+        loader_open();
+      else
+        okL = 0;
+    }
+  };
+
+  // ---- the multiplying side's place: work item and step
+  uint32_t workC = vblock;
+  int32_t stepC = -2, stepsC;
+  uint32_t c0C, r_beginC, r_endC;
+  // The MFMA leaves a lane with four neighbouring columns of one output channel in each of its
+  // two column tiles; a swap between lane rows (v_permlane16_swap) turns that into eight
+  // neighbouring columns, so a store moves 16 bytes per lane and four lanes fill a 64-byte run.
+  const uint32_t ocol_lane = 32u * cw + ((g & 1u) ? 16u : 0u) + (g >> 1) * 8u;  // + first column of the strip
+  const uint32_t co0 = grp * 64u + 32u * h + l16;
+  const bool okct[2] = {co0 < P.Cout, co0 + 16u < P.Cout};
+  const uint32_t out_image_bytes = P.Cout * P.OH * P.OW * 2u;
+  const uint32_t ct_bytes = 16u * P.OH * P.OW * 2u, orow_bytes = P.OW * 2u;
+  const uint32_t ooff_lane = (co0 * P.OH * P.OW + ocol_lane) * 2u;  // + (row * OW + first column) * 2
+  uint16_t *out_imgC = nullptr;
+  __amdgpu_buffer_rsrc_t rsrcC = __builtin_amdgcn_make_buffer_rsrc(P.out[0], 0, 0, 0x00020000);
+  bool wholeC = false;  // every lane of the wave stores eight whole columns of two existing channels
+  auto compute_open = [&]() {
+    uint32_t tile, n;
+    decode(workC, tile, n, c0C, r_beginC, r_endC);
+    stepsC = (int32_t)((r_endC - r_beginC + kStepRows - 1) / kStepRows);
+    out_imgC = P.out[tile] + (size_t)n * P.Cout * P.OH * P.OW;
+    rsrcC = __builtin_amdgcn_make_buffer_rsrc(out_imgC, 0, out_image_bytes, 0x00020000);
+    wholeC = __builtin_amdgcn_ballot_w64(!(c0C + ocol_lane + 7u < P.OW && okct[0] && okct[1])) == 0ull;
+  };
+  compute_open();
+
+  // operand reads: pixel (32 cw + 16 cti + l16 + kw + xoff) of a ring row, channels 8 g .. 8 g + 7 of a half
+  const uint32_t read_lane = (32u * cw + l16 + xoff) * kW8PxBytes + g * 16u;
+
+  u32x4 pk[2][2], old[2][2];  // [channel tile][row of the pair]: packed results, old values for beta = 1
+
+  // stores the packed results of a step lane by lane: edge strips and channel remainders
+  auto store_guarded = [&](uint32_t row0, uint32_t nrows) {
+    const uint32_t ocol = c0C + ocol_lane;
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+        if ((uint32_t)r < nrows && okct[ct]) {
+          uint16_t *p = out_imgC + ((size_t)(co0 + 16u * ct) * P.OH + row0 + r) * P.OW + ocol;
+          if (ocol + 7u < P.OW) {
+            *reinterpret_cast<u32x4_unaligned *>(p) = pk[ct][r];
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (ocol + e < P.OW) p[e] = (uint16_t)(pk[ct][r][e >> 1] >> ((e & 1) * 16));
+          }
+        }
+  };
+  auto load_old_guarded = [&](uint32_t row0, uint32_t nrows) {
+    const uint32_t ocol = c0C + ocol_lane;
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        old[ct][r] = (u32x4){0u, 0u, 0u, 0u};
+        if ((uint32_t)r < nrows && okct[ct]) {
+          const uint16_t *p = out_imgC + ((size_t)(co0 + 16u * ct) * P.OH + row0 + r) * P.OW + ocol;
+          if (ocol + 7u < P.OW) {
+            old[ct][r] = *reinterpret_cast<const u32x4_unaligned *>(p);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (ocol + e < P.OW) old[ct][r][e >> 1] |= (uint32_t)p[e] << ((e & 1) * 16);
+          }
+        }
+      }
+  };
+
+  // The matrix part of a step: 48 operand reads (input row, column shift, channel half, column
+  // tile), each fetched kAhead reads before its MFMAs; then the results are packed to bf16 and
+  // stored.  Rounds alternate between an input row that feeds one output row of the pair (two
+  // MFMAs) and one that feeds both (four), so that the reads run an even 240 or more matrix
+  // cycles ahead.  With SIDE everything else a wave does in a phase is dealt out between the
+  // rounds, one instruction at a time, so that no wave ever stands at a queue of memory
+  // instructions while its matrix pipe idles: the five transposing read pairs and ring writes
+  // of the row group that has landed, the five copies of the next group, and for beta = 1 the
+  // four loads of old values (buffer loads and stores: a row that does not exist gets an
+  // out-of-range offset, so the sequence has no branches).
+  auto compute = [&](uint32_t sb, auto side_tag, auto bar_tag, uint32_t row0, uint32_t nrows) {
+    constexpr bool SIDE = decltype(side_tag)::value != 0;
+    constexpr bool BAR = decltype(bar_tag)::value != 0;  // the phase's barrier comes between the rounds and the packing
+    const uint32_t cur_off = ooff_lane + (row0 * P.OW + c0C) * 2u;
+    const uint32_t off0 = nrows > 0u ? cur_off : kOutOfRange, off1 = nrows > 1u ? cur_off + orow_bytes : kOutOfRange;
+    floatx4 acc[2][2][2];  // [row][column tile][channel tile]
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+      for (int cti = 0; cti < 2; ++cti)
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) acc[r][cti][ct] = (floatx4){0.f, 0.f, 0.f, 0.f};
+    constexpr int kReads = 48, kAhead = BETA ? 3 : 4;
+    const uint8_t *row_ptr[4];
+#pragma unroll
+    for (int ir = 0; ir < 4; ++ir) row_ptr[ir] = ring + wrap_slot(sb + 2u * rp + (uint32_t)ir) * kW8RowBytes + read_lane;
+    u32x4 abuf[kAhead + 1];
+    TrPair trp[2];
+    // round t reads input row ir(t): 0, 1, 0, 1, .. for t < 24, then 2, 3, 2, 3, ..
+    auto fetch = [&](int t) {
+      const int ir = (t / 24) * 2 + (t & 1), j = (t % 24) >> 1, kw = j >> 2, half = (j >> 1) & 1, cti = j & 1;
+      abuf[t % (kAhead + 1)] =
+          *reinterpret_cast<const u32x4 *>(row_ptr[ir] + (cti * 16 + kw) * kW8PxBytes + half * 64);
+    };
+#pragma unroll
+    for (int t = 0; t < kAhead; ++t) fetch(t);
+    __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+    // The copies of the group to transpose have landed: everything but the previous step's four
+    // stores, which were issued after them (memory instructions complete in order).
+#ifdef W8_TIMING
+    __builtin_amdgcn_sched_barrier(0);
+    const uint64_t dbg_v0 = __builtin_readcyclecounter();
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+    if (SIDE) __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
+#ifdef W8_TIMING
+    __builtin_amdgcn_sched_barrier(0);
+    const uint64_t dbg_m0 = __builtin_readcyclecounter();
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    dbg_move += dbg_m0 - dbg_tb;
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+    auto round = [&](auto tag) {
+      constexpr int t = decltype(tag)::value;
+      if constexpr (t + kAhead < kReads) {
+        fetch(t + kAhead);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      constexpr int ir = (t / 24) * 2 + (t & 1), j = (t % 24) >> 1, kw = j >> 2, half = (j >> 1) & 1, cti = j & 1;
+      const bf16x8 a = __builtin_bit_cast(bf16x8, abuf[t % (kAhead + 1)]);
+      constexpr int kh_lo = ir - 1 > 0 ? ir - 1 : 0;
+      constexpr int kh_hi = ir < 2 ? ir : 2;
+#pragma unroll
+      for (int kh = kh_lo; kh <= kh_hi; ++kh) {
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+          acc[ir - kh][cti][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              a, __builtin_bit_cast(bf16x8, wreg[kh * 3 + kw][half][ct]), acc[ir - kh][cti][ct], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 2 * (kh_hi - kh_lo + 1), 0);
+      if constexpr (SIDE) {
+        // rounds 0, 2, .., 8: transposing read pair t / 2; rounds 3, 5, .., 11: ring write (t - 3) / 2
+        if constexpr (t % 2 == 0 && t <= 8) {
+          tr_read(IntTag<t / 2>(), trp[(t / 2) % 2]);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        if constexpr (t >= 3 && t % 2 == 1 && t <= 11) {
+          tr_write(IntTag<(t - 3) / 2>(), trp[((t - 3) / 2) % 2]);
+          __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
+        // rounds 13, 15, .., 21: copy (t - 13) / 2 of the next row group (every transposing read has returned)
+        if constexpr (t >= 13 && t % 2 == 1 && t <= 21) {
+          request(IntTag<(t - 13) / 2>());
+          __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        }
+        // rounds 28, 31, 34, 37: old value (t - 28) / 3 of this step
+        if constexpr (BETA && t >= 28 && (t - 28) % 3 == 0 && t <= 37) {
+          constexpr int i = (t - 28) / 3, ct = i >> 1, r = i & 1;
+          old[ct][r] = __builtin_amdgcn_raw_buffer_load_b128(rsrcC, r ? off1 : off0, ct ? ct_bytes : 0u, 0);
+          __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        }
+      }
+    };
+    for_each_int(std::make_integer_sequence<int, kReads>(), round);
+    __builtin_amdgcn_sched_barrier(0);
+#ifdef W8_TIMING
+    const uint64_t dbg_m1 = __builtin_readcyclecounter();
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    dbg_mm += dbg_m1 - dbg_m0;
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+    if constexpr (BAR) {
+      // every ring read and write of the phase is done (the operands have been multiplied)
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // pack: back to store order through the swap between lane rows
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+      for (int ct = 0; ct < 2; ++ct) {
+        floatx4 v0 = acc[r][0][ct], v1 = acc[r][1][ct];
+        if (BETA) {
+          // the old values, back in the MFMA's arrangement: the swap is its own inverse
+          const u32x2 s0 = __builtin_amdgcn_permlane16_swap(old[ct][r][0], old[ct][r][2], false, false);
+          const u32x2 s1 = __builtin_amdgcn_permlane16_swap(old[ct][r][1], old[ct][r][3], false, false);
+          v0[0] += __uint_as_float(s0[0] << 16);
+          v0[1] += __uint_as_float(s0[0] & 0xffff0000u);
+          v0[2] += __uint_as_float(s1[0] << 16);
+          v0[3] += __uint_as_float(s1[0] & 0xffff0000u);
+          v1[0] += __uint_as_float(s0[1] << 16);
+          v1[1] += __uint_as_float(s0[1] & 0xffff0000u);
+          v1[2] += __uint_as_float(s1[1] << 16);
+          v1[3] += __uint_as_float(s1[1] & 0xffff0000u);
+        }
+        const u32x2 q0 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[0], v0[1]), pack_bf16x2(v1[0], v1[1]), false, false);
+        const u32x2 q1 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[2], v0[3]), pack_bf16x2(v1[2], v1[3]), false, false);
+        pk[ct][r] = (u32x4){q0[0], q1[0], q0[1], q1[1]};
+#ifdef W8_NO_STORE
+        if (SIDE && P.N == 12345u) {
+#else
+        if constexpr (SIDE) {
+#endif
+#ifdef W8_DWORD_STORES
+          if (P.pad) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+              __builtin_amdgcn_raw_buffer_store_b32(pk[ct][r][d], rsrcC, (r ? off1 : off0) + 4 * d, ct ? ct_bytes : 0u, 0);
+          } else
+#endif
+          __builtin_amdgcn_raw_buffer_store_b128(pk[ct][r], rsrcC, r ? off1 : off0, ct ? ct_bytes : 0u, 0);
+        }
+      }
+    if constexpr (!SIDE) store_guarded(row0, nrows);
+#ifdef W8_TIMING
+    __builtin_amdgcn_sched_barrier(0);
+    dbg_post += __builtin_readcyclecounter() - dbg_m1;
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+#endif
+  };
+
+  // the same side work in one piece, for the phases that cannot take the interleaved form
+  auto move_rows_plain = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    TrPair T[5];
+    for_each_int(std::make_integer_sequence<int, 5>(), [&](auto tag) { tr_read(tag, T[decltype(tag)::value]); });
+    for_each_int(std::make_integer_sequence<int, 5>(), [&](auto tag) { tr_write(tag, T[decltype(tag)::value]); });
+    for_each_int(std::make_integer_sequence<int, 5>(), [&](auto tag) { request(tag); });
+  };
+
+  // One phase per step, plus one without MFMAs at the start of every item and a second one at the
+  // very start.  In phase f a wave transposes row group f + 1 (requested in phase f - 1) into
+  // the four ring slots that the step's six input rows leave free, requests group f + 2 and
+  // multiplies step f; the phase's barrier publishes the ring rows written in it and frees the
+  // ones read in it.
+  uint32_t sb = 4;  // ring slot of the first input row of the step multiplied in this phase
+  loader_open();
+  for_each_int(std::make_integer_sequence<int, 5>(), [&](auto tag) { request(tag); });
+  loader_advance();
+  // Every wave passes one barrier per phase, after its last ring access of the phase.
+  auto phase_barrier = [&]() {
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): LDS only; __syncthreads() would also wait for the copies in flight
+    __builtin_amdgcn_s_barrier();
+  };
+  for (;;) {
+#ifdef W8_TIMING
+    uint64_t dbg_t1 = __builtin_readcyclecounter();
+#endif
+#ifdef W8_TIMING
+    dbg_tb = dbg_t1;
+#endif
+    bool barrier_done = false;
+    if (stepC >= 0) {
+      const uint32_t row0 = r_beginC + (uint32_t)stepC * kStepRows + 2u * rp;  // this wave's first output row
+      const uint32_t nrows = row0 >= r_endC ? 0u : min(2u, r_endC - row0);
+      if (wholeC) {
+        // The older wave of a SIMD gets the matrix pipe first and finishes its rounds first: it
+        // packs and stores while it would wait, the younger one (row pair 1) after the barrier,
+        // while the older one already multiplies the next step.
+        if (rp == 0u) {
+          compute(sb, IntTag<1>(), IntTag<0>(), row0, nrows);
+        } else {
+          compute(sb, IntTag<1>(), IntTag<1>(), row0, nrows);
+          barrier_done = true;
+        }
+      } else {
+        if (BETA) load_old_guarded(row0, nrows);
+        move_rows_plain();
+        compute(sb, IntTag<0>(), IntTag<0>(), row0, nrows);
+      }
+    } else {
+      move_rows_plain();
+    }
+    loader_advance();
+#ifdef W8_TIMING
+    uint64_t dbg_t3 = __builtin_readcyclecounter();
+    dbg_comp += dbg_t3 - dbg_t1;
+#endif
+    if (!barrier_done) phase_barrier();
+#ifdef W8_TIMING
+    dbg_bar += __builtin_readcyclecounter() - dbg_t3;
+#endif
+    sb = wrap_slot(sb + kStepRows);
+    tb = wrap_slot(tb + kStepRows);
+    if (++stepC == stepsC) {
+      workC += gridDim.x;
+      if (workC >= total) break;
+      compute_open();
+      stepC = -1;
+    }
+  }
+#ifdef W8_TIMING
+  if (blockIdx.x == 8 && blockIdx.y == 0 && lane == 0) {
+    w8_dbg[wv * 8 + 0] = __builtin_readcyclecounter() - dbg_c0;
+    w8_dbg[wv * 8 + 1] = __builtin_amdgcn_s_memrealtime() - dbg_r0;
+    w8_dbg[wv * 8 + 2] = dbg_move;
+    w8_dbg[wv * 8 + 3] = dbg_comp;
+    w8_dbg[wv * 8 + 4] = dbg_bar;
+    w8_dbg[wv * 8 + 5] = 67;
+    w8_dbg[wv * 8 + 6] = dbg_mm;
+    w8_dbg[wv * 8 + 7] = dbg_post;
+  }
+#endif
+}
+
+}  // namespace
+
+#ifdef W8_TIMING
+extern "C" int adh_w8_dbg(uint64_t *host_out) {
+  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(w8_dbg), sizeof(uint64_t) * 64);
+}
+#endif
+
+// Shapes of the eight-wave kernel: rows that start on a 4-byte boundary (16 bytes for
+// backward-data, whose granules must lie wholly inside or outside a row), images whose byte
+// offsets fit the buffer range check's 31 bits.
+bool conv_bf16_w8_takes(const ConvBf16Params &P, uint32_t num_tiles) {
+  if (P.Cred > 64u) return false;
+  if (P.pad ? (P.IW % 8u) != 0u : (P.IW % 2u) != 0u) return false;
+  const uint64_t image_bytes = (uint64_t)P.Cred * P.IH * P.IW * 2u;
+  if (image_bytes >= (1ull << 31)) return false;
+  const size_t a = P.pad ? 16 : 4;
+  for (uint32_t t = 0; t < num_tiles; ++t)
+    if (!aligned_to(P.in[t], a)) return false;
+  return true;
+}
+
+int conv_bf16_w8_launch(const ConvBf16Params &P, uint32_t gx, uint32_t groups, hipStream_t st) {
+  if (P.beta != 0.f)
+    hipLaunchKernelGGL(conv3x3_bf16_w8_kernel<true>, dim3(gx, groups), dim3(kW8Threads), 0, st, P);
+  else
+    hipLaunchKernelGGL(conv3x3_bf16_w8_kernel<false>, dim3(gx, groups), dim3(kW8Threads), 0, st, P);
+  return launch_status();
+}
+
+}  // namespace adh
