@@ -18,9 +18,17 @@
 //   refills the staging area it has just read, one barrier per step is enough.
 // * A wave owns 32 output channels x 32 columns x 2 rows: 48 operand reads and 144 MFMAs per
 //   step, its filter share (9 taps x 64 x 32) in 144 registers; 8 accumulator tiles.  That fits
-//   256 registers, so two waves share a SIMD and one fills the other's stalls.  Waves 0-3
-//   transpose and request before they multiply, waves 4-7 after: the matrix pipe of every SIMD
-//   has work while its other wave moves data.
+//   256 registers, so two waves share a SIMD.  Everything else a wave does in a step (its copies,
+//   its transposition, its stores) is dealt out between the MFMA rounds one instruction at a
+//   time: issued in a burst, memory instructions fill the memory pipeline's queue and the wave
+//   stands at the next one with its MFMAs behind it.
+// * The SIMD gives the matrix pipe to its older wave first, so waves 0-3 (row pair 0) finish
+//   their rounds early and waves 4-7 late.  One barrier per step, after a wave's last ring
+//   access: the early waves pack and store before it (they would wait anyway), the late ones
+//   after it, while the early ones already multiply the next step.
+// * `__syncthreads()` would wait for the copies in flight (the compiler puts vmcnt(0) before the
+//   barrier); the barrier here waits for LDS only, and the wait for a row group's copies counts
+//   the stores issued after them (memory instructions of a wave complete in order).
 // * The sequence of row groups runs on across work items (the first rows of the next item are
 //   requested during the last steps of the current one); an item costs one step without MFMAs.
 //
@@ -54,16 +62,9 @@ __device__ __forceinline__ u32x2 lds_read_tr(const uint8_t *p) {
 
 __device__ __forceinline__ uint32_t wrap_slot(uint32_t s) { return s >= (uint32_t)kW8RingRows ? s - (uint32_t)kW8RingRows : s; }
 
-#ifdef W8_TIMING
-__device__ uint64_t w8_dbg[64];
-#endif
 
 template <bool BETA>
 __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16Params P) {
-#ifdef W8_TIMING
-  const uint64_t dbg_c0 = __builtin_readcyclecounter(), dbg_r0 = __builtin_amdgcn_s_memrealtime();
-  uint64_t dbg_move = 0, dbg_comp = 0, dbg_bar = 0, dbg_mm = 0, dbg_tb = 0, dbg_post = 0;
-#endif
   __shared__ __attribute__((aligned(16))) uint8_t raw[kW8RawBytes];
   __shared__ __attribute__((aligned(16))) uint8_t ring[kW8RingBytes];
 
@@ -312,9 +313,11 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     for (int ir = 0; ir < 4; ++ir) row_ptr[ir] = ring + wrap_slot(sb + 2u * rp + (uint32_t)ir) * kW8RowBytes + read_lane;
     u32x4 abuf[kAhead + 1];
     TrPair trp[2];
-    // round t reads input row ir(t): 0, 1, 0, 1, .. for t < 24, then 2, 3, 2, 3, ..
+    // round t reads input row 0, 1, 0, 1, .. for t < 24 (two and four MFMAs in turn), then row 2
+    // for twelve rounds and row 3 for the last twelve: output row 0 of the pair is complete after
+    // round 35 and is packed and stored between the two-MFMA rounds of row 3
     auto fetch = [&](int t) {
-      const int ir = (t / 24) * 2 + (t & 1), j = (t % 24) >> 1, kw = j >> 2, half = (j >> 1) & 1, cti = j & 1;
+      const int ir = t < 24 ? (t & 1) : t / 12, j = t < 24 ? t >> 1 : t % 12, kw = j >> 2, half = (j >> 1) & 1, cti = j & 1;
       abuf[t % (kAhead + 1)] =
           *reinterpret_cast<const u32x4 *>(row_ptr[ir] + (cti * 16 + kw) * kW8PxBytes + half * 64);
     };
@@ -323,27 +326,38 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
     // The copies of the group to transpose have landed: everything but the previous step's four
     // stores, which were issued after them (memory instructions complete in order).
-#ifdef W8_TIMING
-    __builtin_amdgcn_sched_barrier(0);
-    const uint64_t dbg_v0 = __builtin_readcyclecounter();
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    __builtin_amdgcn_sched_barrier(0);
-#endif
     if (SIDE) __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
-#ifdef W8_TIMING
-    __builtin_amdgcn_sched_barrier(0);
-    const uint64_t dbg_m0 = __builtin_readcyclecounter();
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    dbg_move += dbg_m0 - dbg_tb;
-    __builtin_amdgcn_sched_barrier(0);
-#endif
+    // packs tile i (row i / 2 of the pair, channel tile i % 2) back to store order through the
+    // swap between lane rows and, in the interleaved form, stores it
+    auto pack_tile = [&](auto tag) {
+      constexpr int r = decltype(tag)::value >> 1, ct = decltype(tag)::value & 1;
+      floatx4 v0 = acc[r][0][ct], v1 = acc[r][1][ct];
+      if (BETA) {
+        // the old values, back in the MFMA's arrangement: the swap is its own inverse
+        const u32x2 s0 = __builtin_amdgcn_permlane16_swap(old[ct][r][0], old[ct][r][2], false, false);
+        const u32x2 s1 = __builtin_amdgcn_permlane16_swap(old[ct][r][1], old[ct][r][3], false, false);
+        v0[0] += __uint_as_float(s0[0] << 16);
+        v0[1] += __uint_as_float(s0[0] & 0xffff0000u);
+        v0[2] += __uint_as_float(s1[0] << 16);
+        v0[3] += __uint_as_float(s1[0] & 0xffff0000u);
+        v1[0] += __uint_as_float(s0[1] << 16);
+        v1[1] += __uint_as_float(s0[1] & 0xffff0000u);
+        v1[2] += __uint_as_float(s1[1] << 16);
+        v1[3] += __uint_as_float(s1[1] & 0xffff0000u);
+      }
+      const u32x2 q0 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[0], v0[1]), pack_bf16x2(v1[0], v1[1]), false, false);
+      const u32x2 q1 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[2], v0[3]), pack_bf16x2(v1[2], v1[3]), false, false);
+      pk[ct][r] = (u32x4){q0[0], q1[0], q0[1], q1[1]};
+      if constexpr (SIDE)
+        __builtin_amdgcn_raw_buffer_store_b128(pk[ct][r], rsrcC, r ? off1 : off0, ct ? ct_bytes : 0u, 0);
+    };
     auto round = [&](auto tag) {
       constexpr int t = decltype(tag)::value;
       if constexpr (t + kAhead < kReads) {
         fetch(t + kAhead);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
-      constexpr int ir = (t / 24) * 2 + (t & 1), j = (t % 24) >> 1, kw = j >> 2, half = (j >> 1) & 1, cti = j & 1;
+      constexpr int ir = t < 24 ? (t & 1) : t / 12, j = t < 24 ? t >> 1 : t % 12, kw = j >> 2, half = (j >> 1) & 1, cti = j & 1;
       const bf16x8 a = __builtin_bit_cast(bf16x8, abuf[t % (kAhead + 1)]);
       constexpr int kh_lo = ir - 1 > 0 ? ir - 1 : 0;
       constexpr int kh_hi = ir < 2 ? ir : 2;
@@ -370,9 +384,14 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
           request(IntTag<(t - 13) / 2>());
           __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
         }
-        // rounds 28, 31, 34, 37: old value (t - 28) / 3 of this step
-        if constexpr (BETA && t >= 28 && (t - 28) % 3 == 0 && t <= 37) {
-          constexpr int i = (t - 28) / 3, ct = i >> 1, r = i & 1;
+        // rounds 38 and 42: output row 0, complete since round 35, is packed and stored
+        if constexpr (t == 38 || t == 42) {
+          pack_tile(IntTag<(t - 38) / 4>());
+          __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        }
+        // rounds 24, 27, 30, 33: old value (t - 24) / 3 of this step, row 0 first
+        if constexpr (BETA && t >= 24 && (t - 24) % 3 == 0 && t <= 33) {
+          constexpr int i = (t - 24) / 3, ct = i & 1, r = i >> 1;
           old[ct][r] = __builtin_amdgcn_raw_buffer_load_b128(rsrcC, r ? off1 : off0, ct ? ct_bytes : 0u, 0);
           __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
         }
@@ -380,61 +399,19 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     };
     for_each_int(std::make_integer_sequence<int, kReads>(), round);
     __builtin_amdgcn_sched_barrier(0);
-#ifdef W8_TIMING
-    const uint64_t dbg_m1 = __builtin_readcyclecounter();
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    dbg_mm += dbg_m1 - dbg_m0;
-    __builtin_amdgcn_sched_barrier(0);
-#endif
     if constexpr (BAR) {
       // every ring read and write of the phase is done (the operands have been multiplied)
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
     }
-    // pack: back to store order through the swap between lane rows
-#pragma unroll
-    for (int r = 0; r < 2; ++r)
-#pragma unroll
-      for (int ct = 0; ct < 2; ++ct) {
-        floatx4 v0 = acc[r][0][ct], v1 = acc[r][1][ct];
-        if (BETA) {
-          // the old values, back in the MFMA's arrangement: the swap is its own inverse
-          const u32x2 s0 = __builtin_amdgcn_permlane16_swap(old[ct][r][0], old[ct][r][2], false, false);
-          const u32x2 s1 = __builtin_amdgcn_permlane16_swap(old[ct][r][1], old[ct][r][3], false, false);
-          v0[0] += __uint_as_float(s0[0] << 16);
-          v0[1] += __uint_as_float(s0[0] & 0xffff0000u);
-          v0[2] += __uint_as_float(s1[0] << 16);
-          v0[3] += __uint_as_float(s1[0] & 0xffff0000u);
-          v1[0] += __uint_as_float(s0[1] << 16);
-          v1[1] += __uint_as_float(s0[1] & 0xffff0000u);
-          v1[2] += __uint_as_float(s1[1] << 16);
-          v1[3] += __uint_as_float(s1[1] & 0xffff0000u);
-        }
-        const u32x2 q0 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[0], v0[1]), pack_bf16x2(v1[0], v1[1]), false, false);
-        const u32x2 q1 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[2], v0[3]), pack_bf16x2(v1[2], v1[3]), false, false);
-        pk[ct][r] = (u32x4){q0[0], q1[0], q0[1], q1[1]};
-#ifdef W8_NO_STORE
-        if (SIDE && P.N == 12345u) {
-#else
-        if constexpr (SIDE) {
-#endif
-#ifdef W8_DWORD_STORES
-          if (P.pad) {
-#pragma unroll
-            for (int d = 0; d < 4; ++d)
-              __builtin_amdgcn_raw_buffer_store_b32(pk[ct][r][d], rsrcC, (r ? off1 : off0) + 4 * d, ct ? ct_bytes : 0u, 0);
-          } else
-#endif
-          __builtin_amdgcn_raw_buffer_store_b128(pk[ct][r], rsrcC, r ? off1 : off0, ct ? ct_bytes : 0u, 0);
-        }
-      }
+    if constexpr (!SIDE) {
+      for_each_int(std::make_integer_sequence<int, 4>(), pack_tile);
+    } else {
+      pack_tile(IntTag<2>());
+      pack_tile(IntTag<3>());
+    }
     if constexpr (!SIDE) store_guarded(row0, nrows);
-#ifdef W8_TIMING
-    __builtin_amdgcn_sched_barrier(0);
-    dbg_post += __builtin_readcyclecounter() - dbg_m1;
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-#endif
   };
 
   // the same side work in one piece, for the phases that cannot take the interleaved form
@@ -461,12 +438,6 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     __builtin_amdgcn_s_barrier();
   };
   for (;;) {
-#ifdef W8_TIMING
-    uint64_t dbg_t1 = __builtin_readcyclecounter();
-#endif
-#ifdef W8_TIMING
-    dbg_tb = dbg_t1;
-#endif
     bool barrier_done = false;
     if (stepC >= 0) {
       const uint32_t row0 = r_beginC + (uint32_t)stepC * kStepRows + 2u * rp;  // this wave's first output row
@@ -490,14 +461,7 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
       move_rows_plain();
     }
     loader_advance();
-#ifdef W8_TIMING
-    uint64_t dbg_t3 = __builtin_readcyclecounter();
-    dbg_comp += dbg_t3 - dbg_t1;
-#endif
     if (!barrier_done) phase_barrier();
-#ifdef W8_TIMING
-    dbg_bar += __builtin_readcyclecounter() - dbg_t3;
-#endif
     sb = wrap_slot(sb + kStepRows);
     tb = wrap_slot(tb + kStepRows);
     if (++stepC == stepsC) {
@@ -507,39 +471,22 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
       stepC = -1;
     }
   }
-#ifdef W8_TIMING
-  if (blockIdx.x == 8 && blockIdx.y == 0 && lane == 0) {
-    w8_dbg[wv * 8 + 0] = __builtin_readcyclecounter() - dbg_c0;
-    w8_dbg[wv * 8 + 1] = __builtin_amdgcn_s_memrealtime() - dbg_r0;
-    w8_dbg[wv * 8 + 2] = dbg_move;
-    w8_dbg[wv * 8 + 3] = dbg_comp;
-    w8_dbg[wv * 8 + 4] = dbg_bar;
-    w8_dbg[wv * 8 + 5] = 67;
-    w8_dbg[wv * 8 + 6] = dbg_mm;
-    w8_dbg[wv * 8 + 7] = dbg_post;
-  }
-#endif
 }
 
 }  // namespace
 
-#ifdef W8_TIMING
-extern "C" int adh_w8_dbg(uint64_t *host_out) {
-  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(w8_dbg), sizeof(uint64_t) * 64);
-}
-#endif
-
-// Shapes of the eight-wave kernel: rows that start on a 4-byte boundary (16 bytes for
-// backward-data, whose granules must lie wholly inside or outside a row), images whose byte
-// offsets fit the buffer range check's 31 bits.
+// Shapes of the eight-wave kernel: input and output rows that start on a 4-byte boundary (input
+// rows on 16 bytes for backward-data, whose granules must lie wholly inside or outside a row),
+// images whose byte offsets fit the buffer range check's 31 bits.
 bool conv_bf16_w8_takes(const ConvBf16Params &P, uint32_t num_tiles) {
   if (P.Cred > 64u) return false;
   if (P.pad ? (P.IW % 8u) != 0u : (P.IW % 2u) != 0u) return false;
   const uint64_t image_bytes = (uint64_t)P.Cred * P.IH * P.IW * 2u;
   if (image_bytes >= (1ull << 31)) return false;
+  if ((uint64_t)P.Cout * P.OH * P.OW * 2u >= (1ull << 31) || (P.OW % 2u) != 0u) return false;
   const size_t a = P.pad ? 16 : 4;
   for (uint32_t t = 0; t < num_tiles; ++t)
-    if (!aligned_to(P.in[t], a)) return false;
+    if (!aligned_to(P.in[t], a) || !aligned_to(P.out[t], 4)) return false;
   return true;
 }
 
