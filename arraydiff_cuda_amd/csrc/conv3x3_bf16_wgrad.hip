@@ -191,7 +191,11 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
         const uint32_t rest = last_row - (r + 1u);
         wait_rows(rest < (uint32_t)(kWgStages - 2) ? rest : (uint32_t)(kWgStages - 2));
       }
-      __syncthreads();  // row r + 1 is complete in LDS; everybody has fetched row r
+      // Row r + 1 is complete in LDS (every wave has waited for its own copies of it) and
+      // everybody has fetched row r.  Not __syncthreads(): the compiler would put vmcnt(0) before
+      // it and the rows meant to stay in flight would be waited for at every step.
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
       if (r + (uint32_t)kWgStages <= last_row) dma_row(r + (uint32_t)kWgStages, stages[PH % kWgStages]);
       if (r < last_row) fetch(WgTag<(PH + 1) % 12>());
 
