@@ -41,6 +41,7 @@ SIGNATURES = {
     "adh_tiles_pack_nchw": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vp]),
     "adh_tiles_unpack_nchw": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vp]),
     "adh_conv3x3_workspace_bytes": (sz, [i32, i32, u32, u32, u32, u32, u32, u32]),
+    "adh_conv3x3_kernel_name": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, f32, ctypes.c_char_p, sz]),
     "adh_conv3x3_slab_fwd": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_fwd_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_data": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
@@ -422,3 +423,10 @@ def softmax_nll_loss_bwd(y, label, dloss, dx):
     N, C = y.shape
     return lib().adh_softmax_nll_loss_bwd(C, N, y.data_ptr(), label.data_ptr(), dloss.data_ptr(), dx.data_ptr(),
                                           _stream())
+
+
+def conv_kernel_name(which, dtype, K, N, Cin, Cout, H, W, beta=0.0):
+    """Name of the kernel instance a 3x3 forward / backward-data call of this shape runs."""
+    buf = ctypes.create_string_buffer(128)
+    check(lib().adh_conv3x3_kernel_name(which, dtype, K, N, Cin, Cout, H, W, beta, buf, 128), "kernel name")
+    return buf.value.decode()

@@ -25,6 +25,8 @@
 //   * staging is asynchronous and register-free: global_load_lds writes each lane's dword
 //     straight into LDS.  The loads of chunk c+1 are issued before the MFMAs of chunk c into
 //     the other buffer pair; one barrier per chunk.
+#include <stdio.h>
+
 #include "adh_common.h"
 
 namespace adh {
@@ -428,11 +430,39 @@ static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uin
   return launch_status();
 }
 
+// name of the kernel instance conv_direct launches for a shape (fp32)
+static int conv_direct_kernel_name(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                                   uint32_t W, char *name, size_t name_bytes) {
+  const uint32_t OH = which == ADH_CONV_FWD ? H : H + 2u, OW = which == ADH_CONV_FWD ? W : W + 2u;
+  const uint32_t cout_k = which == ADH_CONV_FWD ? Cout : Cin;
+  const ConvTile tile = choose_tile(OH, OW, (uint64_t)N * num_tiles, (cout_k + 63u) / 64u);
+  if (tile.nt == 0) return ADH_EINVAL;
+  const int waves = tile.nt == 8 ? 4 : 8;
+  const int prows = (waves == 8 && tile.R > (uint32_t)kMaxR) ? kPatchRowsTall : kPatchRows;
+  snprintf(name, name_bytes, "conv3x3_f32_kernel<%d,%d,%s,%d>", tile.nt, waves, which == ADH_CONV_FWD ? "false" : "true", prows);
+  return ADH_OK;
+}
+
+const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t W, float beta);
+
 }  // namespace adh
 
 using namespace adh;
 
 extern "C" {
+
+int adh_conv3x3_kernel_name(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                            uint32_t H, uint32_t W, float beta, char *name, size_t name_bytes) {
+  if (!name || name_bytes == 0) return ADH_ENULL;
+  if (which != ADH_CONV_FWD && which != ADH_CONV_BWD_DATA) return ADH_EINVAL;
+  if (num_tiles == 0 || N == 0 || Cin == 0 || Cout == 0 || H == 0 || W == 0) return ADH_EINVAL;
+  if (dtype == ADH_BF16) {
+    snprintf(name, name_bytes, "%s", conv_bf16_kernel_name(which, Cin, Cout, W, beta));
+    return ADH_OK;
+  }
+  if (dtype != ADH_F32) return ADH_EINVAL;
+  return conv_direct_kernel_name(which, num_tiles, N, Cin, Cout, H, W, name, name_bytes);
+}
 
 int adh_conv3x3_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                                uint32_t W, const void *const *x_pad_tiles, const void *w, void *const *y_tiles,

@@ -499,6 +499,14 @@ bool conv_bf16_mfma_supported(int which, uint32_t Cin, uint32_t Cout) {
   return cred <= 64u;
 }
 
+// name of the kernel a bf16 forward / backward-data call runs, for tiles aligned to 16 bytes
+const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t W, float beta) {
+  if (!conv_bf16_mfma_supported(which, Cin, Cout)) return "widen_bf16_kernel + conv3x3_f32_kernel + narrow_bf16_kernel";
+  const bool w8 = which == ADH_CONV_FWD ? (W % 2u) == 0u : (W % 8u) == 0u;
+  if (w8) return beta != 0.f ? "conv3x3_bf16_w8_kernel<true>" : "conv3x3_bf16_w8_kernel<false>";
+  return beta != 0.f ? "conv3x3_bf16_kernel<true>" : "conv3x3_bf16_kernel<false>";
+}
+
 size_t conv_bf16_mfma_workspace_bytes(int which, uint32_t Cin, uint32_t Cout) {
   const uint32_t cout_k = which == ADH_CONV_FWD ? Cout : Cin;
   return (size_t)((cout_k + 63u) / 64u) * kWtGroupElems * 2u;

@@ -3,15 +3,20 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-A "step" is one pass of the hot path's dominant stage over one batch of synthetic input:
-the 3x3 slab convolution forward over the 4 halo-padded row-tiles of a ResNet-50
-conv2_x-shaped activation (fp32 NCHW N=32, Cin=Cout=64, 4 tiles of 14(+2) x 56(+2)), one launch
-through the C ABI, inputs resident in HBM.  One JSON line is printed: `value` is the conv
-throughput in TFLOP/s (algorithmic flops 2*N*Cout*Cin*H*W*9 per tile), `roofline` is that
-kernel against the fp32 MFMA peak, `cpu_baseline` is the scalar CPU port timed on this host,
-and `secondary` carries the HBM-bound kernels of the path (halo pack / unpack / exchange /
-reduce, channel slice, softmax-NLL) and the two backward convolutions with their own roofline
-figures.  Everything is timed with device events on the stream the kernels are launched on.
+A "step" is one pass of the hot path's dominant stage over one batch of synthetic input: the 3x3
+slab convolution forward of the largest configuration that fits one GPU, the high-resolution one
+(bf16 in HBM, fp32 accumulate, NCHW N=2, Cin=Cout=64, a 1024x2048 image in 8 row-tiles of 128(+2)
+x 2048(+2)), one call through the C ABI over all tiles, inputs resident in HBM.  Before the
+warm-up the same call is repeated, untimed, for at least 150 ms (`clock_ramp_ms`): the clocks of an
+idle GPU need tens of milliseconds to come up and, under this kernel, settle at what the power
+limit allows, so that 20 timed steps measure what 2000 would.  One JSON line is printed: `value`
+is the conv throughput in TFLOP/s (algorithmic flops 2*N*Cout*Cin*H*W*9 per tile), `roofline` is
+that kernel against the bf16 MFMA peak, `cpu_baseline` is the scalar CPU port timed on this host
+(one thread, and one thread per tile), and `secondary` carries every other kernel of the path with
+its own roofline figure: the fp32 conv of the ResNet-sized configurations, halo pack / unpack /
+exchange / reduce, channel slice, softmax-NLL, the backward convolutions, and the three shapes the
+reference's own microbenchmarks time.  Everything is timed with device events on the stream the
+kernels are launched on.
 """
 import argparse
 import ctypes
@@ -24,10 +29,14 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# HBM bytes per conv-forward launch on cfg2 measured with rocprofv3 PMC (FETCH_SIZE x 2.000 +
-# WRITE_SIZE x 1.000, factors from a 1 GiB plain copy); the summary with the commands is
-# profiles/conv3x3_fwd_cfg2_hbm_traffic.txt.  Not re-measured by this script.
-CONV_FWD_CFG2_TRAFFIC_BYTES = 64.07e6
+# HBM bytes per conv-forward launch measured with rocprofv3 PMC (FETCH_SIZE and WRITE_SIZE, each
+# scaled by what the same counter reads for a 1 GiB plain copy); the summaries with the commands
+# are profiles/conv3x3_bf16_fwd_cfg5_hbm_traffic.txt and profiles/conv3x3_fwd_cfg2_hbm_traffic.txt.
+# Not re-measured by this script; each figure belongs to the kernel instance named beside it and is
+# left out (null) when the library routes the shape to another instance.
+CONV_FWD_CFG5_TRAFFIC = ("conv3x3_bf16_w8_kernel<false>", None)
+CONV_FWD_CFG2_TRAFFIC = ("conv3x3_f32_kernel<25,8,false,12>", 64.07e6)
+CLOCK_RAMP_MS = 150.0
 HBM_PEAK_GBS = 8000.0
 MFMA_F32_PEAK_TFLOPS = 157.3
 MFMA_BF16_PEAK_TFLOPS = 2500.0
@@ -93,9 +102,9 @@ def time_gpu_graph(fn, per_graph=50, replays=10):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=500)
-    ap.add_argument("--warmup", type=int, default=300,
-                    help="untimed steps; a few hundred so that the GPU clocks have ramped up")
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20,
+                    help="untimed steps after the fixed clock-ramp phase")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-secondary", action="store_true", help="time only the headline kernel")
     ap.add_argument("--no-end-to-end", action="store_true",
@@ -151,11 +160,79 @@ def main():
     lib = capi.lib()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
-    # ---- workload: the 3x3 slab conv forward (N=32, C=64, 4 row-tiles of 14 rows of a 56x56 image) on the tensors the halo
-    # pack / unpack entries use ----
-    K, p, N, C, H, W = 4, 1, 32, 64, 56, 56
-    Ht = H // K
     g = torch.Generator(device="cuda").manual_seed(0x5EED)
+
+    # ---- workload: the 3x3 slab conv forward of the high-resolution configuration on the bf16 matrix cores ----
+    C = 64
+    K5, N5, H5, W5 = 8, 2, 1024, 2048
+    Ht5 = H5 // K5
+    X5 = (torch.rand((N5, C, H5, W5), device="cuda", generator=g) * 2 - 1).to(torch.bfloat16)
+    t5 = [torch.empty((N5, C, Ht5 + 2, W5 + 2), device="cuda", dtype=torch.bfloat16) for _ in range(K5)]
+    t5_tbl, _k5 = capi.ptr_table([t.data_ptr() for t in t5])
+    capi.check(lib.adh_tiles_pack_nchw(1, K5, 1, W5, H5, C, N5, X5.data_ptr(), t5_tbl, stream), "pack cfg5")
+    w5 = (torch.randn((C, C, 3, 3), device="cuda", generator=g) * (2.0 / (C * 9)) ** 0.5).to(torch.bfloat16)
+    y5 = [torch.empty((N5, C, Ht5, W5), device="cuda", dtype=torch.bfloat16) for _ in range(K5)]
+    y5_tbl, _ky = capi.ptr_table([t.data_ptr() for t in y5])
+    ws5_bytes = max(lib.adh_conv3x3_workspace_bytes(wh, 1, K5, N5, C, C, Ht5, W5) for wh in (0, 1, 2))
+    ws5 = torch.empty(ws5_bytes // 4 + 64, device="cuda")
+    flops5 = 2.0 * K5 * N5 * C * C * 9 * Ht5 * W5
+
+    def conv_fwd5():
+        return lib.adh_conv3x3_slab_fwd_tiles(1, K5, N5, C, C, Ht5, W5, t5_tbl, w5.data_ptr(), y5_tbl, 0.0,
+                                              ws5.data_ptr(), ws5_bytes, stream)
+
+    capi.check(conv_fwd5(), "conv fwd cfg5")
+
+    # ---- clock ramp: the same launch, untimed, until the clocks have settled ----
+    torch.cuda.synchronize()
+    t_ramp = time.perf_counter()
+    while (time.perf_counter() - t_ramp) * 1e3 < CLOCK_RAMP_MS:
+        for _ in range(20):
+            conv_fwd5()
+        torch.cuda.synchronize()
+    clock_ramp_ms = (time.perf_counter() - t_ramp) * 1e3
+
+    # ---- the timed region: W warmup steps, then exactly K steps between two synchronisations ----
+    for _ in range(args.warmup):
+        conv_fwd5()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        conv_fwd5()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    kernel_ms = e0.elapsed_time(e1) / args.steps
+    value = flops5 / (ms_per_step * 1e-3) / 1e12
+    achieved = flops5 / (kernel_ms * 1e-3) / 1e12
+    name5 = capi.conv_kernel_name(capi.ADH_CONV_FWD, capi.ADH_BF16, K5, N5, C, C, Ht5, W5)
+    in5_b = K5 * N5 * C * (Ht5 + 2) * (W5 + 2) * 2
+    out5_b = N5 * C * H5 * W5 * 2
+    ai5 = flops5 / (in5_b + out5_b + C * C * 9 * 2)
+
+    out = {
+        "metric": METRIC, "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "clock_ramp_ms": round(clock_ramp_ms, 1),
+        "config": {"workload": "configs[4]: 3x3 slab conv fwd, bf16 in / fp32 accumulate, NCHW N=2 Cin=Cout=64, "
+                               "1024x2048 image in 8 row-tiles of 128(+2)x2048(+2), one call over all tiles",
+                   "flops_per_step": flops5, "tiles": K5, "halo": 1},
+        "roofline": {"kernel": name5 + " (fwd; the call also runs the 2 us filter reordering kernel)", "bound": "mfma",
+                     "achieved": round(achieved, 3), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": CONV_FWD_CFG5_TRAFFIC[1] if name5 == CONV_FWD_CFG5_TRAFFIC[0] else None,
+                     "launch_ms": round(kernel_ms, 5),
+                     "compulsory_bytes": in5_b + out5_b + C * C * 9 * 2,
+                     "min_mfma_hbm_bound_TFLOPs": round(min(MFMA_BF16_PEAK_TFLOPS, HBM_PEAK_GBS * ai5 / 1e3), 1)},
+    }
+
+    # ---- the tensors of the ResNet-sized configurations (cfg1-cfg3): fp32 N=32, C=64, 56x56 in 4 row-tiles of 14 rows ----
+    K, p, N, H, W = 4, 1, 32, 56, 56
+    Ht = H // K
     X = torch.rand((N, C, H, W), device="cuda", generator=g) * 2 - 1
     wt = torch.randn((C, C, 3, 3), device="cuda", generator=g) * (2.0 / (C * 9)) ** 0.5
     dY = torch.randn((N, C, H, W), device="cuda", generator=g)
@@ -173,44 +250,9 @@ def main():
     g_tbl, _k4 = capi.ptr_table([t.data_ptr() for t in gs])
     ws_bytes = capi.conv_workspace_bytes(capi.ADH_CONV_BWD_FILTER, capi.ADH_F32, K, N, C, C, Ht, W)
     ws = torch.empty(max(ws_bytes // 4, 1), device="cuda")
-
-    def conv_fwd():
-        lib.adh_conv3x3_slab_fwd_tiles(capi.ADH_F32, K, N, C, C, Ht, W, tile_tbl, wt.data_ptr(), y_tbl, 0.0,
-                                       None, 0, stream)
-
+    flops_step = 2.0 * N * C * C * Ht * W * 9 * K
     capi.check(lib.adh_conv3x3_slab_fwd_tiles(capi.ADH_F32, K, N, C, C, Ht, W, tile_tbl, wt.data_ptr(), y_tbl, 0.0,
                                               None, 0, stream), "conv fwd")
-
-    # ---- the timed region: W warmup steps, then exactly K steps between two synchronisations ----
-    for _ in range(args.warmup):
-        conv_fwd()
-    torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(args.steps):
-        conv_fwd()
-    e1.record()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    kernel_ms = e0.elapsed_time(e1) / args.steps
-    flops_step = 2.0 * N * C * C * Ht * W * 9 * K
-    value = flops_step / (ms_per_step * 1e-3) / 1e12
-    achieved = flops_step / (kernel_ms * 1e-3) / 1e12
-
-    out = {
-        "metric": METRIC, "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "configs[1]: 3x3 slab conv fwd, fp32 NCHW N=32 Cin=Cout=64, 4 row-tiles of "
-                               "14(+2)x56(+2), one launch over all tiles",
-                   "flops_per_step": flops_step, "tiles": K, "halo": p},
-        "roofline": {"kernel": "conv3x3_f32_kernel<25,8,false,12> (fwd)", "bound": "mfma", "achieved": round(achieved, 3),
-                     "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / MFMA_F32_PEAK_TFLOPS, 4),
-                     "traffic": CONV_FWD_CFG2_TRAFFIC_BYTES, "launch_ms": round(kernel_ms, 5)},
-    }
 
     if args.copy_calibration:
         cw, chh, cc, cn = 1024, 1024, 64, 4  # 2^28 floats = 1 GiB each way, rows contiguous
@@ -232,7 +274,7 @@ def main():
 
         flush_scratch = torch.empty(128 * 1024 * 1024, device="cuda")  # 512 MB
 
-        def add(name, fn, bound, work, peak, unit, note=None, flushed=False, graph=False):
+        def add(name, fn, bound, work, peak, unit, note=None, flushed=False, graph=False, extra=None):
             nonlocal stream
             if args.only is not None and args.only not in name:
                 return
@@ -266,10 +308,20 @@ def main():
                 e["frac_in_graph"] = round(achg / peak, 4)
             if note:
                 e["note"] = note
+            if extra:
+                e.update(extra(ms) if callable(extra) else extra)
             sec.append(e)
 
         unsplit_b = N * C * H * W * es
         padded_b = K * N * C * (Ht + 2 * p) * (W + 2 * p) * es
+        name2 = capi.conv_kernel_name(capi.ADH_CONV_FWD, capi.ADH_F32, K, N, C, C, Ht, W)
+        reps, wu = 500, 300
+        add("conv fwd cfg2 (fp32, 4 tiles of 14(+2)x56(+2), one launch)",
+            lambda: lib.adh_conv3x3_slab_fwd_tiles(capi.ADH_F32, K, N, C, C, Ht, W, tile_tbl, wt.data_ptr(), y_tbl, 0.0,
+                                                   None, 0, stream),
+            "mfma", flops_step, MFMA_F32_PEAK_TFLOPS, "TFLOP/s",
+            extra={"kernel": name2, "traffic": CONV_FWD_CFG2_TRAFFIC[1] if name2 == CONV_FWD_CFG2_TRAFFIC[0] else None})
+        reps, wu = 200, 20
         add("halo pack cfg1 (unsplit -> 4 padded tiles)",
             lambda: lib.adh_tiles_pack_nchw(0, K, p, W, H, C, N, X.data_ptr(), tile_tbl, stream),
             "hbm", unsplit_b + padded_b, HBM_PEAK_GBS, "GB/s", flushed=True, graph=True)
@@ -279,7 +331,8 @@ def main():
         add("halo exchange cfg1 (6 strips)",
             lambda: lib.adh_halo_exchange_nchw(0, 1, K, p, W, Ht, C, N, tile_tbl, stream),
             "hbm", 2 * 2 * (K - 1) * strip, HBM_PEAK_GBS, "GB/s",
-            note="reference figure of merit p*W*C*N*4/t = %d B / t" % strip, graph=True)
+            graph=True, extra=lambda ms: {"reference_figure_GBs": round(strip / (ms * 1e-3) / 1e9, 3),
+                                          "reference_figure": "p*W*C*N*4 / t (tools/microbench_spatial.cc:100-101)"})
         add("halo reduce cfg1 (6 strips)",
             lambda: lib.adh_halo_reduce_nchw(0, 1, K, p, W, Ht, C, N, g_tbl, stream),
             "hbm", 3 * 2 * (K - 1) * strip, HBM_PEAK_GBS, "GB/s", graph=True)
@@ -313,10 +366,6 @@ def main():
             "mfma", flops_step, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
 
         # config 5 sized pack / unpack: 0.5 GB, larger than the on-package cache
-        K5, N5, H5, W5 = 8, 2, 1024, 2048
-        X5 = (torch.rand((N5, C, H5, W5), device="cuda", generator=g) * 2 - 1).to(torch.bfloat16)
-        t5 = [torch.empty((N5, C, H5 // K5 + 2, W5 + 2), device="cuda", dtype=torch.bfloat16) for _ in range(K5)]
-        t5_tbl, _k5 = capi.ptr_table([t.data_ptr() for t in t5])
         Y5 = torch.empty_like(X5)
         b5 = N5 * C * H5 * W5 * 2
         reps, wu = 50, 5
@@ -326,17 +375,11 @@ def main():
         add("halo unpack cfg5 (bf16)",
             lambda: lib.adh_tiles_unpack_nchw(1, K5, 1, W5, H5, C, N5, t5_tbl, Y5.data_ptr(), stream),
             "hbm", 2 * b5, HBM_PEAK_GBS, "GB/s")
-        # config 5 slab conv on the bf16 matrix cores: fwd, bwd-data (beta = 1, as the reference
-        # accumulates input gradients), bwd-filter
-        Ht5 = H5 // K5
-        w5 = (torch.randn((C, C, 3, 3), device="cuda", generator=g) * (2.0 / (C * 9)) ** 0.5).to(torch.bfloat16)
-        y5 = [torch.empty((N5, C, Ht5, W5), device="cuda", dtype=torch.bfloat16) for _ in range(K5)]
-        y5_tbl, _ky = capi.ptr_table([t.data_ptr() for t in y5])
+        # config 5 slab conv on the bf16 matrix cores: bwd-data (beta = 0, what the host op issues for the first
+        # toucher of a gradient, and beta = 1, as the reference accumulates input gradients), bwd-filter; the
+        # forward pass is the headline above
         gw5 = torch.zeros((C, C, 3, 3), device="cuda")
-        ws5_bytes = max(lib.adh_conv3x3_workspace_bytes(wh, 1, K5, N5, C, C, Ht5, W5) for wh in (0, 1, 2))
-        ws5 = torch.empty(ws5_bytes // 4 + 64, device="cuda")
-        flops5 = 2.0 * K5 * N5 * C * C * 9 * Ht5 * W5
-        reps, wu = 20, 3
+        reps, wu = 50, 10
         add("conv fwd cfg5 (bf16, 8 tiles)",
             lambda: lib.adh_conv3x3_slab_fwd_tiles(1, K5, N5, C, C, Ht5, W5, t5_tbl, w5.data_ptr(), y5_tbl, 0.0,
                                                    ws5.data_ptr(), ws5_bytes, stream),
@@ -353,7 +396,89 @@ def main():
             lambda: lib.adh_conv3x3_slab_bwd_filter_tiles(1, K5, N5, C, C, Ht5, W5, t5_tbl, y5_tbl, gw5.data_ptr(), 0.0,
                                                           ws5.data_ptr(), ws5_bytes, stream),
             "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
-        del X5, t5, Y5, y5, ws5
+        del Y5
+        # ---- the shapes the reference's own microbenchmarks time, with its own figures of merit ----
+        # tools/microbench_spatial.cc:23-28: halo exchange, fp32 N=32, C=64, W=256, H=256/ndev, p=1 (ndev = 4 tiles);
+        # it prints p*W*C*N*4 / t (:100-103)
+        Km, Nm, Wm, Hm, pm = 4, 32, 256, 256 // 4, 1
+        tm = [torch.rand((Nm, C, Hm + 2 * pm, Wm + 2 * pm), device="cuda", generator=g) for _ in range(Km)]
+        tm_tbl, _km = capi.ptr_table([t.data_ptr() for t in tm])
+        strip_m = pm * Wm * C * Nm * 4
+        reps, wu = 200, 20
+        add("reference microbench_spatial: halo exchange, N=32 C=64 W=256 H=64 per tile, p=1, 4 tiles",
+            lambda: lib.adh_halo_exchange_nchw(0, 1, Km, pm, Wm, Hm, C, Nm, tm_tbl, stream),
+            "hbm", 2 * 2 * (Km - 1) * strip_m, HBM_PEAK_GBS, "GB/s", graph=True,
+            extra=lambda ms: {"reference_figure_GBs": round(strip_m / (ms * 1e-3) / 1e9, 3),
+                              "reference_figure": "p*W*C*N*4 / t (tools/microbench_spatial.cc:100-101)"})
+        del tm
+        # tools/microbench_spatial_conv.cc:25-41: N=32, C=64, a 512x512 image in ndev row-tiles (4 tiles of 128 rows),
+        # 3x3 convolution with dilation 3 over halo 3: halo exchange, halo reduce (:227-269), conv forward and
+        # backward (:384-387, 473-476; it prints average milliseconds)
+        Kd, Nd, Wd, Hd, pd = 4, 32, 512, 512 // 4, 3
+        geo_d = (3, 3, 1, 1, 3, 3)
+        HPd, WPd = Hd + 2 * pd, Wd + 2 * pd
+        xd = [torch.rand((Nd, C, HPd, WPd), device="cuda", generator=g) * 2 - 1 for _ in range(Kd)]
+        yd = [torch.empty((Nd, C, Hd, Wd), device="cuda") for _ in range(Kd)]
+        gd = [torch.zeros((Nd, C, HPd, WPd), device="cuda") for _ in range(Kd)]
+        wd = torch.randn((C, C, 3, 3), device="cuda", generator=g) * (2.0 / (C * 9)) ** 0.5
+        gwd = torch.empty_like(wd)
+        xd_tbl, _kd1 = capi.ptr_table([t.data_ptr() for t in xd])
+        yd_tbl, _kd2 = capi.ptr_table([t.data_ptr() for t in yd])
+        gd_tbl, _kd3 = capi.ptr_table([t.data_ptr() for t in gd])
+        wsd_bytes = max(lib.adh_conv2d_workspace_bytes(wh, 0, Kd, Nd, C, C, HPd, WPd, *geo_d) for wh in (0, 1, 2))
+        wsd = torch.empty(wsd_bytes // 4 + 64, device="cuda")
+        strip_d = pd * Wd * C * Nd * 4
+        fl_d = 2.0 * Kd * Nd * C * C * 9 * Hd * Wd
+        reps, wu = 100, 10
+        add("reference microbench_spatial_conv: halo exchange, N=32 C=64 512x128 per tile, p=3, 4 tiles",
+            lambda: lib.adh_halo_exchange_nchw(0, 1, Kd, pd, Wd, Hd, C, Nd, xd_tbl, stream),
+            "hbm", 2 * 2 * (Kd - 1) * strip_d, HBM_PEAK_GBS, "GB/s",
+            extra=lambda ms: {"reference_figure_GBs": round(strip_d / (ms * 1e-3) / 1e9, 3)})
+        add("reference microbench_spatial_conv: halo reduce, same tiles",
+            lambda: lib.adh_halo_reduce_nchw(0, 1, Kd, pd, Wd, Hd, C, Nd, gd_tbl, stream),
+            "hbm", 3 * 2 * (Kd - 1) * strip_d, HBM_PEAK_GBS, "GB/s",
+            extra=lambda ms: {"reference_figure_GBs": round(strip_d / (ms * 1e-3) / 1e9, 3)})
+        reps, wu = 10, 3
+        add("reference microbench_spatial_conv: conv fwd 3x3 dilation 3 over halo 3 (fp32, 4 tiles, general kernel)",
+            lambda: lib.adh_conv2d_slab_fwd_tiles(0, Kd, Nd, C, C, HPd, WPd, *geo_d, xd_tbl, wd.data_ptr(), yd_tbl, 0.0,
+                                                  wsd.data_ptr(), wsd_bytes, stream),
+            "mfma", fl_d, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+        add("reference microbench_spatial_conv: conv bwd-filter, same shape",
+            lambda: lib.adh_conv2d_slab_bwd_filter_tiles(0, Kd, Nd, C, C, HPd, WPd, *geo_d, xd_tbl, yd_tbl, gwd.data_ptr(),
+                                                         0.0, wsd.data_ptr(), wsd_bytes, stream),
+            "mfma", fl_d, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+        add("reference microbench_spatial_conv: conv bwd-data, same shape",
+            lambda: lib.adh_conv2d_slab_bwd_data_tiles(0, Kd, Nd, C, C, HPd, WPd, *geo_d, wd.data_ptr(), yd_tbl, gd_tbl,
+                                                       0.0, wsd.data_ptr(), wsd_bytes, stream),
+            "mfma", fl_d, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+        del xd, yd, gd, wsd
+        # tools/microbench_conv.cc:30-54: one device, N=32, 64 -> 64 channels, 3x3 over a 64(+2) x 128(+2) slab,
+        # "est flops" 2*N*Co*Ci*H*W*9 = 9.66 GF (:53)
+        Nc, Hc, Wc = 32, 64, 128
+        xc = torch.rand((Nc, C, Hc + 2, Wc + 2), device="cuda", generator=g) * 2 - 1
+        yc_ = torch.empty((Nc, C, Hc, Wc), device="cuda")
+        fl_c = 2.0 * Nc * C * C * 9 * Hc * Wc
+        reps, wu = 100, 20
+        add("reference microbench_conv: conv fwd 3x3, N=32 64->64, 64(+2)x128(+2) slab (fp32, one tile)",
+            lambda: lib.adh_conv3x3_slab_fwd(0, Nc, C, C, Hc, Wc, xc.data_ptr(), wd.data_ptr(), yc_.data_ptr(), 0.0,
+                                             None, 0, stream),
+            "mfma", fl_c, MFMA_F32_PEAK_TFLOPS, "TFLOP/s",
+            extra={"kernel": capi.conv_kernel_name(capi.ADH_CONV_FWD, capi.ADH_F32, 1, Nc, C, C, Hc, Wc)})
+        del xc, yc_
+        # column halos (a K x 1 grid, src/kernels/spatial.cu:654-731): cfg1's tensor split into 4 column-tiles
+        # of 14 columns; a strip is p*H*C*N elements at row pitch
+        Wk, Hk = W // K, H
+        tk = [torch.rand((N, C, Hk + 2 * p, Wk + 2 * p), device="cuda", generator=g) for _ in range(K)]
+        tk_tbl, _kk = capi.ptr_table([t.data_ptr() for t in tk])
+        strip_k = p * Hk * C * N * es
+        reps, wu = 200, 20
+        add("column halo exchange (4 x 1 grid of 14-column tiles of cfg1's tensor, 6 strips)",
+            lambda: lib.adh_halo_exchange_nchw(0, K, 1, p, Wk, Hk, C, N, tk_tbl, stream),
+            "hbm", 2 * 2 * (K - 1) * strip_k, HBM_PEAK_GBS, "GB/s", graph=True)
+        add("column halo reduce (same tiles)",
+            lambda: lib.adh_halo_reduce_nchw(0, K, 1, p, Wk, Hk, C, N, tk_tbl, stream),
+            "hbm", 3 * 2 * (K - 1) * strip_k, HBM_PEAK_GBS, "GB/s", graph=True)
+        del tk
         # pooling over the padded slab: the 3x3 stride-2 max pooling of a residual network's stem,
         # 112x112 in 4 row-tiles of 28 rows with halo 1 -> 14x56 per tile
         Hq, Wq = 28 + 2, 112 + 2
@@ -472,55 +597,68 @@ def main():
     if end_to_end is not None:
         out["end_to_end"] = end_to_end
 
-    # ---- CPU baseline: the scalar port, single thread, on a bounded sample ----
+    # ---- CPU baseline: the scalar port on this host, one thread and one thread per tile, on a bounded sample ----
     if not args.no_cpu:
         import oracle
-        # the secondary entries above have written into the tiles (the halo reduce adds into them): pack and convolve
-        # once more so that the CPU and the GPU work on the same input
-        capi.check(capi.tiles_pack(K, p, W, H, C, N, X, tiles), "pack")
-        capi.check(lib.adh_conv3x3_slab_fwd_tiles(capi.ADH_F32, K, N, C, C, Ht, W, tile_tbl, wt.data_ptr(), y_tbl, 0.0,
-                                                  None, 0, stream), "conv fwd")
+        cores_on_box = oracle.hardware_threads()
+        # The sample: the first 8 output rows of image 0 of every one of the 8 tiles of the headline workload (same
+        # filter, same bf16 values widened to fp32: exact products, fp32 sums, the arithmetic the kernel does):
+        # 8 tiles x 64 x 64 x 9 x 8 x 2048 x 2 = 9.7 GFLOP per pass.  The secondary entries above have written into
+        # the tiles: pack and convolve once more so that the CPU and the GPU work on the same input.
+        capi.check(lib.adh_tiles_pack_nchw(1, K5, 1, W5, H5, C, N5, X5.data_ptr(), t5_tbl, stream), "pack cfg5")
+        capi.check(conv_fwd5(), "conv fwd cfg5")
         torch.cuda.synchronize()
-        wn = wt.cpu().numpy()
-        host_x = [t.cpu().numpy() for t in tiles]
-        yc = np.empty((N, C, Ht, W), np.float32)
-        cpu_reps = 2  # 2 passes over all 4 tiles = 14.8 GFLOP of scalar work
+        rows = 8
+        wn5 = w5.float().cpu().numpy()
+        host_x5 = [np.ascontiguousarray(t[0:1, :, 0:rows + 2, :].float().cpu().numpy()) for t in t5]
+        host_y5 = [np.empty((1, C, rows, W5), np.float32) for _ in range(K5)]
+        sample_flops = 2.0 * K5 * C * C * 9 * rows * W5
         t0 = time.perf_counter()
-        for _ in range(cpu_reps):
-            for r in range(K):
-                oracle.conv_slab_fwd_f32(host_x[r], wn, yc)
-        dt = (time.perf_counter() - t0) / cpu_reps
-        err = float(np.abs(yc - ys[K - 1].cpu().numpy()).max() / np.abs(yc).max())
+        for r in range(K5):
+            oracle.conv_slab_fwd_f32(host_x5[r], wn5, host_y5[r])
+        dt1 = time.perf_counter() - t0
+        err = max(float(np.abs(host_y5[r] - y5[r][0:1, :, 0:rows].float().cpu().numpy()).max() / np.abs(host_y5[r]).max())
+                  for r in range(K5))
+        t0 = time.perf_counter()
+        oracle.conv_slab_fwd_f32_threaded(host_x5, wn5, host_y5)
+        dtk = time.perf_counter() - t0
         out["cpu_baseline"] = {
-            "value": round(flops_step / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
-            "sample": "%d passes over the same 4 tiles (N=32, C=64, 14x56 outputs each, 7.4 GFLOP per pass), scalar "
-                      "fp32 direct conv, gcc -O2, one thread, %.2f s per pass; GPU result agrees to rel-err %.1e"
-                      % (cpu_reps, dt, err)}
-        # the reference kernels' own loop structure for the halo exchange (idx -> (w,c,n) by div/mod)
+            "value": round(sample_flops / dt1 / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "cores_on_box": cores_on_box,
+            "value_thread_per_tile": round(sample_flops / dtk / 1e12, 6), "threads_thread_per_tile": K5,
+            "sample": "rows 0-7 of image 0 of each of the 8 tiles of the headline workload (9.7 GFLOP): scalar fp32 "
+                      "direct conv of the widened bf16 values, gcc -O2, %.2f s on one thread, %.2f s with one thread "
+                      "per tile; GPU result (bf16) agrees to rel-err %.1e" % (dt1, dtk, err)}
+        # the reference kernels' own loop structure (idx -> (w,c,n) by div/mod) on cfg1: halo exchange, halo pack
+        # (scatter + pad + exchange) and unpack (unpad + gather), one thread and one thread per rank
+        capi.check(capi.tiles_pack(K, p, W, H, C, N, X, tiles), "pack")
+        torch.cuda.synchronize()
         host_tiles = [t.cpu().numpy() for t in tiles]
-        t0 = time.perf_counter()
-        reps_cpu = 20
-        for _ in range(reps_cpu):
-            oracle.halo_op(oracle.EXCH, 1, K, p, W, Ht, C, N, host_tiles)
-        dt = (time.perf_counter() - t0) / reps_cpu
-        out["cpu_baseline"]["halo_exchange_GBs"] = round(2 * 2 * (K - 1) * p * W * C * N * 4 / dt / 1e9, 3)
-        # halo pack (scatter + pad + exchange) and unpack (unpad + gather) of the unsplit tensor on the host
         host_X = X.cpu().numpy()
         host_Y = np.empty_like(host_X)
-        reps_cpu = 3
-        t0 = time.perf_counter()
-        for _ in range(reps_cpu):
-            oracle.tiles_pack(K, p, W, H, C, N, host_X, host_tiles)
-        dt_pack = (time.perf_counter() - t0) / reps_cpu
-        t0 = time.perf_counter()
-        for _ in range(reps_cpu):
-            oracle.tiles_unpack(K, p, W, H, C, N, host_tiles, host_Y)
-        dt_unpack = (time.perf_counter() - t0) / reps_cpu
-        assert np.array_equal(host_Y, host_X)
         unsplit_b = N * C * H * W * 4
         padded_b = K * N * C * (Ht + 2 * p) * (W + 2 * p) * 4
-        out["cpu_baseline"]["halo_pack_GBs"] = round((unsplit_b + padded_b) / dt_pack / 1e9, 3)
-        out["cpu_baseline"]["halo_unpack_GBs"] = round(2 * unsplit_b / dt_unpack / 1e9, 3)
+
+        def cpu_time(fn, reps_cpu):
+            t0 = time.perf_counter()
+            for _ in range(reps_cpu):
+                fn()
+            return (time.perf_counter() - t0) / reps_cpu
+
+        exch_b = 2 * 2 * (K - 1) * p * W * C * N * 4
+        cb = out["cpu_baseline"]
+        cb["halo_exchange_GBs"] = round(exch_b / cpu_time(lambda: oracle.halo_op(oracle.EXCH, 1, K, p, W, Ht, C, N, host_tiles), 20) / 1e9, 3)
+        cb["halo_exchange_GBs_thread_per_rank"] = round(
+            exch_b / cpu_time(lambda: oracle.halo_op_threaded(oracle.EXCH, 1, K, p, W, Ht, C, N, host_tiles), 20) / 1e9, 3)
+        cb["halo_pack_GBs"] = round((unsplit_b + padded_b) / cpu_time(lambda: oracle.tiles_pack(K, p, W, H, C, N, host_X, host_tiles), 3) / 1e9, 3)
+        cb["halo_pack_GBs_thread_per_rank"] = round(
+            (unsplit_b + padded_b) / cpu_time(lambda: oracle.tiles_pack_threaded(K, p, W, H, C, N, host_X, host_tiles), 3) / 1e9, 3)
+        cb["halo_unpack_GBs"] = round(2 * unsplit_b / cpu_time(lambda: oracle.tiles_unpack(K, p, W, H, C, N, host_tiles, host_Y), 3) / 1e9, 3)
+        assert np.array_equal(host_Y, host_X)
+        cb["halo_unpack_GBs_thread_per_rank"] = round(
+            2 * unsplit_b / cpu_time(lambda: oracle.tiles_unpack_threaded(K, p, W, H, C, N, host_tiles, host_Y), 3) / 1e9, 3)
+        assert np.array_equal(host_Y, host_X)
+        cb["threads_thread_per_rank"] = K
 
     print(json.dumps(out))
 

@@ -140,6 +140,12 @@ int adh_tiles_unpack_nchw(int dtype, uint32_t K, uint32_t halo_pad, uint32_t W, 
 #define ADH_CONV_BWD_FILTER 2
 size_t adh_conv3x3_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,
                                    uint32_t Cout, uint32_t H, uint32_t W);
+/* Name of the kernel instance a forward or backward-data call of this shape is routed to (tile
+ * buffers aligned to 16 bytes), written to `name`; for tools that match timings against a
+ * profiler's kernel trace.  Plays the part of the algorithm the reference reads back from
+ * cudnnFindConvolution*Algorithm and prints (src/op.cc:1463-1507). */
+int adh_conv3x3_kernel_name(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                            uint32_t H, uint32_t W, float beta, char *name, size_t name_bytes);
 /* cudnnConvolutionForward at src/op.cc:1576-1587:
  * y[n,co,h,w] = beta*y + sum_{ci,kh,kw} w[co,ci,kh,kw] * x_pad[n,ci,h+kh,w+kw] */
 int adh_conv3x3_slab_fwd(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,

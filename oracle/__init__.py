@@ -161,6 +161,42 @@ def tiles_unpack(K, p, W, H, C, N, tiles, y_unsplit):
                                  _ptr_array(tiles), _ptr(y_unsplit), _ptr(scratch))
 
 
+def hardware_threads():
+    """Hardware threads of this host (what std::thread::hardware_concurrency() reports)."""
+    _lib.orc_hardware_threads.restype = ctypes.c_uint32
+    return int(_lib.orc_hardware_threads())
+
+
+def halo_op_threaded(which, grid_w, grid_h, p, W, H, C, N, tiles):
+    """halo_op with one host thread per rank (the reference runs one kernel per rank)."""
+    dt = dtype_code(tiles[0])
+    return _lib.orc_halo_op_threaded(which, dt, _u32(grid_w), _u32(grid_h), _u32(p), _u32(W), _u32(H), _u32(C),
+                                     _u32(N), _ptr_array(tiles))
+
+
+def tiles_pack_threaded(K, p, W, H, C, N, x_unsplit, tiles):
+    dt = dtype_code(x_unsplit)
+    scratch = np.empty((max(K, 1), N, C, max(H // max(K, 1), 1), W), dtype=x_unsplit.dtype)
+    return _lib.orc_tiles_pack_threaded(dt, _u32(K), _u32(p), _u32(W), _u32(H), _u32(C), _u32(N),
+                                        _ptr(x_unsplit), _ptr_array(tiles), _ptr(scratch))
+
+
+def tiles_unpack_threaded(K, p, W, H, C, N, tiles, y_unsplit):
+    dt = dtype_code(y_unsplit)
+    scratch = np.empty((max(K, 1), N, C, max(H // max(K, 1), 1), W), dtype=y_unsplit.dtype)
+    return _lib.orc_tiles_unpack_threaded(dt, _u32(K), _u32(p), _u32(W), _u32(H), _u32(C), _u32(N),
+                                          _ptr_array(tiles), _ptr(y_unsplit), _ptr(scratch))
+
+
+def conv_slab_fwd_f32_threaded(x_pads, wt, ys):
+    """conv_slab_fwd_f32 of every tile, one host thread per tile."""
+    N, Cin, Hp, Wp = x_pads[0].shape
+    Cout, _, k, _ = wt.shape
+    H, W = Hp - k + 1, Wp - k + 1
+    return _lib.orc_conv_slab_fwd_f32_threaded(_u32(len(x_pads)), _u32(N), _u32(Cin), _u32(Cout), _u32(H), _u32(W),
+                                               _u32(k), _ptr_array(x_pads), _ptr(wt), _ptr_array(ys))
+
+
 def conv_slab_fwd(x_pad, wt, y, beta=0.0):
     N, Cin, Hp, Wp = x_pad.shape
     Cout, _, k, _ = wt.shape

@@ -866,3 +866,134 @@ void orc_pool_slab_bwd(int mode, uint32_t N, uint32_t C, uint32_t HP, uint32_t W
   }
   free(g);
 }
+
+/* ------------------------------------------------------------------ */
+/* one host thread per rank: the timed CPU baseline's parallel form     */
+/* ------------------------------------------------------------------ */
+
+/* The reference runs one kernel per rank on that rank's own device and stream
+ * (Spatial2DComm::group_end, src/spatial.cc:58-201, called once per rank at
+ * src/op.cc:2990-2999).  On the host the same split is one thread per rank,
+ * each running what orc_halo_op_rank / the per-rank part of pack and unpack /
+ * the slab conv runs for its tile.  Results are identical to the loops above:
+ * ranks write disjoint elements. */
+#include <pthread.h>
+#include <unistd.h>
+
+#define ORC_MAX_RANKS 64
+
+uint32_t orc_hardware_threads(void) {
+  long n = sysconf(_SC_NPROCESSORS_ONLN);
+  return n > 0 ? (uint32_t)n : 1u;
+}
+
+typedef struct {
+  int kind;  /* 0 halo op, 1 scatter + pad of one tile, 2 unpad + gather of one tile, 3 slab conv fwd f32 */
+  int which, dtype, status;
+  uint32_t grid_w, grid_h, rank, K, p, W, H, C, N, Cout, k;
+  void *const *tiles;
+  const void *x_unsplit;
+  void *y_unsplit, *scratch;
+  const float *x_pad, *wt;
+  float *y;
+} orc_job;
+
+static void *orc_job_run(void *arg) {
+  orc_job *j = (orc_job *)arg;
+  const uint32_t Ht = j->K ? j->H / j->K : 0;
+  j->status = ORC_OK;
+  switch (j->kind) {
+    case 0:
+      j->status = orc_halo_op_rank(j->which, j->dtype, j->grid_w, j->grid_h, j->rank, j->p, j->W, j->H, j->C, j->N, j->tiles);
+      break;
+    case 1:
+      j->status = orc_slice_nchw(ORC_OP_COPY, j->dtype, j->W, Ht, j->C, j->N, j->x_unsplit, j->W, j->H, j->C, 0,
+                                 j->rank * Ht, 0, j->scratch, j->W, Ht, j->C, 0, 0, 0);
+      if (!j->status) orc_halo_pad(j->dtype, j->p, j->W, Ht, j->C, j->N, j->scratch, j->tiles[j->rank]);
+      break;
+    case 2:
+      orc_halo_unpad(j->dtype, j->p, j->W, Ht, j->C, j->N, j->tiles[j->rank], j->scratch);
+      j->status = orc_slice_nchw(ORC_OP_COPY, j->dtype, j->W, Ht, j->C, j->N, j->scratch, j->W, Ht, j->C, 0, 0, 0,
+                                 j->y_unsplit, j->W, j->H, j->C, 0, j->rank * Ht, 0);
+      break;
+    default:
+      orc_conv_slab_fwd_f32(j->N, j->C, j->Cout, j->H, j->W, j->k, j->x_pad, j->wt, j->y);
+      break;
+  }
+  return NULL;
+}
+
+static int orc_run_jobs(orc_job *jobs, uint32_t count) {
+  pthread_t th[ORC_MAX_RANKS];
+  uint32_t started = 0;
+  int status = ORC_OK;
+  for (; started < count; ++started)
+    if (pthread_create(&th[started], NULL, orc_job_run, &jobs[started]) != 0) break;
+  for (uint32_t r = started; r < count; ++r) orc_job_run(&jobs[r]); /* could not start: run it here */
+  for (uint32_t r = 0; r < started; ++r) pthread_join(th[r], NULL);
+  for (uint32_t r = 0; r < count; ++r)
+    if (jobs[r].status) status = jobs[r].status;
+  return status;
+}
+
+/* orc_halo_op with one thread per rank.  An exchange only writes the caller's own halo rows and
+ * reads the neighbours' interiors, a reduce only writes interiors and reads halos, so the ranks
+ * do not race (the reference relies on the same fact between its per-rank kernels). */
+int orc_halo_op_threaded(int which, int dtype, uint32_t grid_w, uint32_t grid_h, uint32_t p, uint32_t W, uint32_t H,
+                         uint32_t C, uint32_t N, void *const *tiles) {
+  const uint32_t R = grid_w * grid_h;
+  if (R == 0 || R > ORC_MAX_RANKS) return ORC_EINVAL;
+  orc_job jobs[ORC_MAX_RANKS];
+  for (uint32_t r = 0; r < R; ++r) {
+    orc_job j = {0};
+    j.kind = 0; j.which = which; j.dtype = dtype; j.grid_w = grid_w; j.grid_h = grid_h; j.rank = r;
+    j.p = p; j.W = W; j.H = H; j.C = C; j.N = N; j.tiles = tiles;
+    jobs[r] = j;
+  }
+  return orc_run_jobs(jobs, R);
+}
+
+/* orc_tiles_pack / orc_tiles_unpack with one thread per tile; `scratch` holds K unpadded tiles. */
+int orc_tiles_pack_threaded(int dtype, uint32_t K, uint32_t p, uint32_t W, uint32_t H, uint32_t C, uint32_t N,
+                            const void *x_unsplit, void *const *tiles, void *scratch) {
+  if (K == 0 || K > ORC_MAX_RANKS || H % K != 0) return ORC_EINVAL;
+  const size_t tile_bytes = (size_t)N * C * (H / K) * W * orc_esize(dtype);
+  orc_job jobs[ORC_MAX_RANKS];
+  for (uint32_t r = 0; r < K; ++r) {
+    orc_job j = {0};
+    j.kind = 1; j.dtype = dtype; j.rank = r; j.K = K; j.p = p; j.W = W; j.H = H; j.C = C; j.N = N;
+    j.tiles = tiles; j.x_unsplit = x_unsplit; j.scratch = (char *)scratch + r * tile_bytes;
+    jobs[r] = j;
+  }
+  int e = orc_run_jobs(jobs, K);
+  if (e) return e;
+  return orc_halo_op_threaded(ORC_EXCH, dtype, 1, K, p, W, H / K, C, N, tiles);
+}
+
+int orc_tiles_unpack_threaded(int dtype, uint32_t K, uint32_t p, uint32_t W, uint32_t H, uint32_t C, uint32_t N,
+                              void *const *tiles, void *y_unsplit, void *scratch) {
+  if (K == 0 || K > ORC_MAX_RANKS || H % K != 0) return ORC_EINVAL;
+  const size_t tile_bytes = (size_t)N * C * (H / K) * W * orc_esize(dtype);
+  orc_job jobs[ORC_MAX_RANKS];
+  for (uint32_t r = 0; r < K; ++r) {
+    orc_job j = {0};
+    j.kind = 2; j.dtype = dtype; j.rank = r; j.K = K; j.p = p; j.W = W; j.H = H; j.C = C; j.N = N;
+    j.tiles = tiles; j.y_unsplit = y_unsplit; j.scratch = (char *)scratch + r * tile_bytes;
+    jobs[r] = j;
+  }
+  return orc_run_jobs(jobs, K);
+}
+
+/* orc_conv_slab_fwd_f32 of K tiles, one thread per tile (same filter, as the ranks' equal copies). */
+int orc_conv_slab_fwd_f32_threaded(uint32_t K, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                                   uint32_t k, const float *const *x_pads, const float *wt, float *const *ys) {
+  if (K == 0 || K > ORC_MAX_RANKS) return ORC_EINVAL;
+  orc_job jobs[ORC_MAX_RANKS];
+  for (uint32_t r = 0; r < K; ++r) {
+    orc_job j = {0};
+    j.kind = 3; j.N = N; j.C = Cin; j.Cout = Cout; j.H = H; j.W = W; j.k = k;
+    j.x_pad = x_pads[r]; j.wt = wt; j.y = ys[r];
+    jobs[r] = j;
+  }
+  return orc_run_jobs(jobs, K);
+}

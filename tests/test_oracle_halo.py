@@ -142,6 +142,76 @@ def test_reduce_is_adjoint_of_exchange(oracle, K, p, Ht, W, C, N):
         np.testing.assert_array_equal(RB[r][m], B[r][m])
 
 
+@pytest.mark.parametrize("K,p,H,Wt,C,N", [(2, 1, 4, 3, 2, 2), (3, 2, 3, 5, 1, 2), (4, 1, 2, 4, 3, 1)])
+def test_column_reduce_is_adjoint_of_column_exchange(oracle, K, p, H, Wt, C, N):
+    """K x 1 grid (column halos): <E a, b> == <a, R b> on small-integer floats, and the closed form
+    of the column reduce (right interior columns += next tile's left halo columns, left interior
+    columns += previous tile's right halo columns) written with numpy slices."""
+    rng = np.random.default_rng(31)
+    shape = (N, C, H + 2 * p, Wt + 2 * p)
+
+    def rand_int():
+        return [rng.integers(-8, 9, size=shape).astype(np.float32) for _ in range(K)]
+
+    A = rand_int()
+    for t in A:
+        m = np.zeros(shape, bool)
+        m[:, :, p:p + H, p:p + Wt] = True
+        t[~m] = 0
+    B = rand_int()
+    EA = [t.copy() for t in A]
+    assert oracle.halo_op(oracle.EXCH, K, 1, p, Wt, H, C, N, EA) == 0
+    RB = [t.copy() for t in B]
+    assert oracle.halo_op(oracle.REDUCE, K, 1, p, Wt, H, C, N, RB) == 0
+    lhs = sum(float(np.sum(EA[r].astype(np.float64) * B[r])) for r in range(K))
+    rhs = sum(float(np.sum(A[r][:, :, p:p + H, p:p + Wt].astype(np.float64) * RB[r][:, :, p:p + H, p:p + Wt]))
+              for r in range(K))
+    assert lhs == rhs
+    want = [b.copy() for b in B]
+    for r in range(K):
+        if r < K - 1:
+            want[r][:, :, p:p + H, Wt:Wt + p] += B[r + 1][:, :, p:p + H, 0:p]
+        if r > 0:
+            want[r][:, :, p:p + H, p:2 * p] += B[r - 1][:, :, p:p + H, Wt + p:Wt + 2 * p]
+    for r in range(K):
+        np.testing.assert_array_equal(RB[r], want[r])
+
+
+def test_thread_per_rank_forms_equal_the_serial_ones(oracle):
+    """The one-thread-per-rank forms timed as the parallel CPU baseline give the same bits as the loops."""
+    K, p, H, W, C, N = 4, 1, 8, 6, 3, 2
+    Ht = H // K
+    rng = np.random.default_rng(5)
+    X = rng.uniform(-1, 1, size=(N, C, H, W)).astype(np.float32)
+    a = [np.full((N, C, Ht + 2 * p, W + 2 * p), np.nan, np.float32) for _ in range(K)]
+    b = [t.copy() for t in a]
+    assert oracle.tiles_pack(K, p, W, H, C, N, X, a) == 0
+    assert oracle.tiles_pack_threaded(K, p, W, H, C, N, X, b) == 0
+    for r in range(K):
+        np.testing.assert_array_equal(a[r], b[r])
+    ya, yb = np.empty_like(X), np.empty_like(X)
+    assert oracle.tiles_unpack(K, p, W, H, C, N, a, ya) == 0
+    assert oracle.tiles_unpack_threaded(K, p, W, H, C, N, b, yb) == 0
+    np.testing.assert_array_equal(ya, X)
+    np.testing.assert_array_equal(yb, X)
+    for which in (oracle.EXCH, oracle.REDUCE):
+        ga = [rng.integers(-5, 6, size=a[0].shape).astype(np.float32) for _ in range(K)]
+        gb = [t.copy() for t in ga]
+        assert oracle.halo_op(which, 1, K, p, W, Ht, C, N, ga) == 0
+        assert oracle.halo_op_threaded(which, 1, K, p, W, Ht, C, N, gb) == 0
+        for r in range(K):
+            np.testing.assert_array_equal(ga[r], gb[r])
+    wt = rng.standard_normal((5, C, 3, 3)).astype(np.float32)
+    y1 = [np.empty((N, 5, Ht, W), np.float32) for _ in range(K)]
+    y2 = [np.empty((N, 5, Ht, W), np.float32) for _ in range(K)]
+    for r in range(K):
+        oracle.conv_slab_fwd_f32(a[r], wt, y1[r])
+    assert oracle.conv_slab_fwd_f32_threaded(a, wt, y2) == 0
+    for r in range(K):
+        np.testing.assert_array_equal(y1[r], y2[r])
+    assert oracle.hardware_threads() >= 1
+
+
 def test_reduce_closed_form_rows(oracle):
     K, p, Ht, W, C, N = 4, 2, 5, 3, 2, 1
     rng = np.random.default_rng(4)
