@@ -44,6 +44,7 @@ SIGNATURES = {
     "adh_conv3x3_kernel_name": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, f32, ctypes.c_char_p, sz]),
     "adh_conv3x3_slab_fwd": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_fwd_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp, sz, vp]),
+    "adh_conv3x3_slab_fwd_tiles_static": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp]),
     "adh_conv3x3_slab_bwd_data": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_data_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_filter": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),

@@ -576,3 +576,71 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
 }
 
 }  // namespace adh
+
+// ---------------------------------------------------------------------------
+// the forward entry point that allocates nothing
+// ---------------------------------------------------------------------------
+namespace {
+
+constexpr uint32_t kStaticGroups = 4;  // reordered filter of up to 256 output channels
+constexpr size_t kStaticScratchBytes = (size_t)kStaticGroups * adh::kWtGroupElems * 2u;  // 294,912 bytes
+constexpr int kStaticMaxDevices = 64;
+
+// The reordered filter of adh_conv3x3_slab_fwd_tiles_static lives here instead of in a caller's
+// workspace.  Every GPU the library runs on holds its own copy of the array until the process ends.
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on each device, looked up once per device with that device current.
+// In host code the array's name is only a handle for this lookup, never a device address.
+static void *g_scratch_ptr[kStaticMaxDevices];
+static int g_scratch_lock = 0;
+
+static int static_scratch(void **out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kStaticMaxDevices) return ADH_EINVAL;
+  while (__atomic_exchange_n(&g_scratch_lock, 1, __ATOMIC_ACQUIRE)) {
+  }
+  void *p = g_scratch_ptr[dev];
+  int status = ADH_OK;
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      status = e != hipSuccess ? (int)e : ADH_ENULL;
+      p = nullptr;
+    } else {
+      g_scratch_ptr[dev] = p;
+    }
+  }
+  __atomic_store_n(&g_scratch_lock, 0, __ATOMIC_RELEASE);
+  *out = p;
+  return status;
+}
+
+}  // namespace
+
+extern "C" int adh_conv3x3_slab_fwd_tiles_static(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                                 uint32_t H, uint32_t W, const void *const *x_pad_tiles,
+                                                 const void *w, void *const *y_tiles, float beta, void *stream) {
+  using namespace adh;
+  if (dtype != ADH_BF16) return ADH_EUNIMPL;
+  if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
+  if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
+  // beyond the static array: more than 256 output channels; beyond the matrix-core kernel: more than 64 input channels
+  if (Cout > 64u * kStaticGroups || !conv_bf16_mfma_supported(ADH_CONV_FWD, Cin, Cout)) return ADH_EWORKSPACE;
+  if (N == 0 || Cin == 0 || Cout == 0 || H == 0 || W == 0) return ADH_OK;
+  if (!x_pad_tiles || !y_tiles || !w) return ADH_ENULL;
+  if (!aligned_to(w, 2)) return ADH_EALIGN;
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!x_pad_tiles[t] || !y_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(x_pad_tiles[t], 2) || !aligned_to(y_tiles[t], 2)) return ADH_EALIGN;
+  }
+  const uint64_t cmax = Cin > Cout ? Cin : Cout;
+  if (cmax * (H + 2ull) * (W + 2ull) * 2u >= (1ull << 31) || (uint64_t)Cin * Cout * 18u >= (1ull << 31)) return ADH_EINVAL;
+  void *ws = nullptr;
+  const int e = static_scratch(&ws);
+  if (e) return e;
+  return conv_bf16_mfma(ADH_CONV_FWD, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, w, y_tiles, beta, ws, as_stream(stream));
+}
+

@@ -155,6 +155,17 @@ int adh_conv3x3_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32
                                uint32_t H, uint32_t W, const void *const *x_pad_tiles, const void *w,
                                void *const *y_tiles, float beta, void *workspace,
                                size_t workspace_bytes, void *stream);
+/* adh_conv3x3_slab_fwd_tiles for callers that cannot allocate and have no workspace to pass (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  dtype must be ADH_BF16 with Cin <= 64 and Cout <= 256 (else
+ * ADH_EWORKSPACE): the reordered filter, which the other entry point keeps in the caller's
+ * workspace, goes to a 294,912-byte array inside the library's device image, one copy per GPU,
+ * held until the process ends.  The call allocates and frees nothing.  Unlike every other entry
+ * point it is not re-entrant: all calls on a GPU share that GPU's array (each call rewrites the
+ * part it uses before reading it), so calls that overlap on one GPU, on any streams, race. */
+int adh_conv3x3_slab_fwd_tiles_static(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                      uint32_t H, uint32_t W, const void *const *x_pad_tiles, const void *w,
+                                      void *const *y_tiles, float beta, void *stream);
 /* cudnnConvolutionBackwardData at src/op.cc:1701-1712: writes the WHOLE padded slab
  * dx_pad[n,ci,h',w'] = beta*dx_pad + sum_{co,kh,kw} w[co,ci,kh,kw] * dy[n,co,h'-kh,w'-kw] */
 int adh_conv3x3_slab_bwd_data(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
