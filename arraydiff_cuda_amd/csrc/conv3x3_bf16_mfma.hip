@@ -559,7 +559,9 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
   if (rest) {
     const uint32_t want_segs = gx / rest;  // >= 1
     uint32_t seg_steps = (P.steps_per_item + want_segs - 1) / want_segs;
-    if (seg_steps < 4u) seg_steps = P.steps_per_item < 4u ? P.steps_per_item : 4u;
+    // the eight-wave kernel starts an item with one step without MFMAs; the four-wave one fills its ring first
+    const uint32_t min_steps = conv_bf16_w8_takes(P, num_tiles) ? 2u : 4u;
+    if (seg_steps < min_steps) seg_steps = P.steps_per_item < min_steps ? P.steps_per_item : min_steps;
     P.seg_steps = seg_steps;
     P.segs = (P.steps_per_item + seg_steps - 1) / seg_steps;
   }

@@ -40,8 +40,6 @@
 
 namespace adh {
 
-namespace {
-
 constexpr int kW8Threads = 512;
 constexpr int kW8PxBytes = 160;                          // 64 channels + 32 bytes: measured, 16-byte reads of 16 neighbouring pixels run at the linear rate (4.5 cycles per wave; 8 at 144 bytes)
 constexpr int kW8RowPx = 72;                             // nine granules of eight pixels
@@ -56,12 +54,11 @@ constexpr int kW8RawBytes = 8 * kW8RawWave;              // 40960
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 #define ADH_LDS __attribute__((address_space(3)))
 
-__device__ __forceinline__ u32x2 lds_read_tr(const uint8_t *p) {
+static __device__ __forceinline__ u32x2 lds_read_tr(const uint8_t *p) {
   return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((ADH_LDS s16x4 *)p));
 }
 
-__device__ __forceinline__ uint32_t wrap_slot(uint32_t s) { return s >= (uint32_t)kW8RingRows ? s - (uint32_t)kW8RingRows : s; }
-
+static __device__ __forceinline__ uint32_t wrap_slot(uint32_t s) { return s >= (uint32_t)kW8RingRows ? s - (uint32_t)kW8RingRows : s; }
 
 template <bool BETA>
 __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16Params P) {
@@ -472,8 +469,6 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     }
   }
 }
-
-}  // namespace
 
 // Shapes of the eight-wave kernel: input and output rows that start on a 4-byte boundary (input
 // rows on 16 bytes for backward-data, whose granules must lie wholly inside or outside a row),

@@ -137,6 +137,7 @@ int adh_softmax_fwd(uint32_t C, uint32_t N, const float *x, float *y, void *stre
   if (C == 0 || N == 0) return ADH_OK;
   if (!x || !y) return ADH_ENULL;
   if (!aligned_to(x, 4) || !aligned_to(y, 4)) return ADH_EALIGN;
+  if (x == y && C > 2048u) return ADH_EINVAL;  // rows past 2048 classes are read again after y is written
   hipLaunchKernelGGL((softmax_row_kernel<false>), dim3(N), dim3(kRowThreads), 0, as_stream(stream), C, N, x,
                      (const uint32_t *)nullptr, y, (float *)nullptr);
   return launch_status();
@@ -147,6 +148,7 @@ int adh_softmax_xent_fwd(uint32_t C, uint32_t N, const float *x, const uint32_t 
   if (C == 0 || N == 0) return ADH_OK;
   if (!x || !y || !label || !loss) return ADH_ENULL;
   if (!aligned_to(x, 4) || !aligned_to(y, 4) || !aligned_to(label, 4) || !aligned_to(loss, 4)) return ADH_EALIGN;
+  if (x == y && C > 2048u) return ADH_EINVAL;
   hipLaunchKernelGGL((softmax_row_kernel<true>), dim3(N), dim3(kRowThreads), 0, as_stream(stream), C, N, x, label, y, loss);
   return launch_status();
 }

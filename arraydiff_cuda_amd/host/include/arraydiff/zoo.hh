@@ -46,8 +46,11 @@ inline void parallel_vars_insert_all(vector<VarIdSet> &dst, const vector<VarIdSe
 
 // One filter variable per rank, one node for all of them (src/zoo.cc:133-161).  The reference's
 // enable_bias is false wherever the spatial nets call this; a bias is not implemented.  The node is
-// told that the copies are equal (Conv2DShape::replicated_filters): train such a graph with
-// ParallelSGDOptimizer, or load equal values into every rank's filter yourself.
+// told that the copies are equal (Conv2DShape::replicated_filters), and they are from the start:
+// Op::init draws rank 0's values and hands every other rank a copy of them (the reference draws
+// each rank's own and the optimizer's first broadcast overwrites them, optimize.hh:283-300).
+// ParallelSGDOptimizer keeps them equal; whoever loads values by hand must load the same ones
+// into every rank.
 template <typename V, typename A = GPUArray4D<float>>
 ParallelParamOp<V> parallel_conv2d(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs,
                                    typename ParamOp<A>::InitFn kernel_init, bool enable_bias, shared_ptr<Context> ctx) {
@@ -60,8 +63,22 @@ ParallelParamOp<V> parallel_conv2d(Conv2DShape shape, vector<shared_ptr<Var<V>>>
   const size_t cin = inputs.at(0)->shape().shape[2];
   ParallelParamOp<V> out;
   vector<shared_ptr<Var<A>>> kernels;
+  // the conv node visits rank 0's filter before the others (SlabConv2DOp::_push), so its values exist
+  // when the copies are made
+  auto drawn = make_shared<std::unique_ptr<A>>();
+  typename ParamOp<A>::InitFn draw = [kernel_init, drawn](A *a, std::mt19937_64 *rng, shared_ptr<Context> c) {
+    kernel_init(a, rng, c);
+    drawn->reset(new A(*a));  // a view of the same memory
+  };
+  typename ParamOp<A>::InitFn copy = [drawn](A *a, std::mt19937_64 *, shared_ptr<Context> c) {
+    if (!*drawn) throw std::logic_error("parallel_conv2d: rank 0's filter was not initialised before the others");
+    if (!a->is_packed() || !(*drawn)->is_packed() || a->dim() != (*drawn)->dim())
+      throw std::logic_error("parallel_conv2d: filter copies differ in shape");
+    GPUConn conn = gpu_ctx_of(c)->conn();
+    gpu_copy_d2d(a->dptr(), (*drawn)->dptr(), a->dim().flat_size() * sizeof(float), conn.stream());
+  };
   for (size_t rank = 0; rank < inputs.size(); ++rank) {
-    auto kernel = ParamOp<A>::Make(Shape4D(shape.kernel[0], shape.kernel[1], cin, shape.filters), kernel_init,
+    auto kernel = ParamOp<A>::Make(Shape4D(shape.kernel[0], shape.kernel[1], cin, shape.filters), rank == 0 ? draw : copy,
                                    mgpu_ctx->device_context(rank));
     kernels.push_back(kernel);
     out.params.push_back(VarIdSet::Singleton(kernel->vars().at(0)));

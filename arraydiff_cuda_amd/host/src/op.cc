@@ -401,15 +401,21 @@ void check_conv_input(V3 &x, const Conv2DShape &cs) {
 // The 3x3 stride-1 kernels tile an image plane per workgroup; a tile of at most 64 pixels (the late layers of
 // a net split over several ranks) leaves them mostly idle, and the general kernel, which puts several images
 // into one workgroup, is 1.2 to 1.9 times faster there.
+// The 3x3 entry points also have limits the general ones do not (images x tiles in one grid dimension,
+// one image inside a 2 GiB buffer range): shapes past them go to the general kernel instead of failing.
+inline bool fits_3x3_kernels(const TileDims &d, uint32_t n, size_t filters) {
+  const uint64_t cmax = d.C > filters ? d.C : filters;
+  return (uint64_t)d.N * n <= 65535u && cmax * (d.H + 2ull) * (d.W + 2ull) * 4u < (1ull << 31);
+}
 template <typename Op>
-bool use_3x3_kernels(const Op &op, const TileDims &d) {
-  return op.is_3x3_unit() && (uint64_t)d.H * d.W > 64u;
+bool use_3x3_kernels(const Op &op, const TileDims &d, uint32_t n, size_t filters) {
+  return op.is_3x3_unit() && (uint64_t)d.H * d.W > 64u && fits_3x3_kernels(d, n, filters);
 }
 // The 3x3 backward-filter kernel streams an image's rows through a ring and pays the ring's fill once per image:
 // on tiles of at most 256 pixels (8x32: 0.61 ms against 0.56) the general kernel's units of 64 pixels are faster.
 template <typename Op>
-bool use_3x3_filter_kernel(const Op &op, const TileDims &d) {
-  return op.is_3x3_unit() && (uint64_t)d.H * d.W > 256u;
+bool use_3x3_filter_kernel(const Op &op, const TileDims &d, uint32_t n, size_t filters) {
+  return op.is_3x3_unit() && (uint64_t)d.H * d.W > 256u && fits_3x3_kernels(d, n, filters);
 }
 
 void *conv_scratch(GPUContext *dc, int which, uint32_t n, const TileDims &d, const Conv2DShape &cs, size_t *bytes) {
@@ -462,7 +468,7 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
-    if (use_3x3_kernels(*this, d)) {
+    if (use_3x3_kernels(*this, d, n, shape_.filters)) {
       adh_check(adh_conv3x3_slab_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt, 0.0f,
                                            nullptr, 0, conn.stream()),
                 "SlabConv2DOp::_forward");
@@ -540,7 +546,7 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
-    if (use_3x3_filter_kernel(*this, d)) {
+    if (use_3x3_filter_kernel(*this, d, n, shape_.filters)) {
       const size_t ws = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
                                                     d.H, d.W);
       dc->reserve_scratch(ws);
@@ -598,7 +604,7 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
     const float beta = first ? 0.0f : 1.0f;
-    if (use_3x3_kernels(*this, d)) {
+    if (use_3x3_kernels(*this, d, n, shape_.filters)) {
       adh_check(adh_conv3x3_slab_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, w0, dyt, dxt,
                                                 beta, nullptr, 0, conn.stream()),
                 "SlabConv2DOp::_backward (data)");

@@ -118,6 +118,11 @@ int main(int argc, char **argv) {
     parallel_ctx->sync();
     read_loss = false;
     StreamCapture capture(dynamic_cast<MultiGPUContext *>(parallel_ctx.get())->stream());
+    if (use_graph && warmup < 1) {
+      // the first step allocates every buffer and sizes the scratch: that cannot happen inside a stream capture
+      std::fprintf(stderr, "train_resnet18: --graph 1 needs at least one warm-up step\n");
+      return 2;
+    }
     if (use_graph) {
       recording = true;
       capture.begin();

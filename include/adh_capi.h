@@ -301,7 +301,9 @@ int adh_pool2d_slab_bwd(int dtype, int mode, uint32_t N, uint32_t C, uint32_t HP
                         void *dx_pad, float beta, void *stream);
 
 /* ---- L1/L2/L3: softmax + negative log likelihood (fp32) ------------------- */
-/* cudnnSoftmaxForward(ACCURATE, MODE_INSTANCE) on (N,C,1,1), src/op.cc:4129-4152 */
+/* cudnnSoftmaxForward(ACCURATE, MODE_INSTANCE) on (N,C,1,1), src/op.cc:4129-4152 
+ * In place (y == x) is allowed up to 2048 classes; beyond that a row is read again after y
+ * has been written and the call returns ADH_EINVAL. */
 int adh_softmax_fwd(uint32_t C, uint32_t N, const float *x, float *y, void *stream);
 /* softmax_nll_loss_fwd<float>, src/kernels/softmax.cu:36-54,86-89 */
 int adh_softmax_nll_loss_fwd(uint32_t C, uint32_t N, const float *y, const uint32_t *label,

@@ -890,6 +890,45 @@ static void test_schedules() {
 // nothing depends on how the rows are dealt to ranks): the logits for 2 and 4 row-tiles must equal those of
 // the unsplit net with the same parameters.  This exercises every halo exchange, the strided convolutions and
 // the pooling over tile borders, and the gather, end to end.
+// Op::init alone (no optimizer reset, no hand-loaded values) must leave every rank's copy of a
+// parallel_conv2d filter equal to rank 0's: the node convolves all tiles with rank 0's filter.
+static void test_parallel_conv2d_init_gives_equal_copies() {
+  const size_t K = 4, N = 2, C = 8, Co = 16, H = 8, W = 12, Ht = H / K;
+  typedef GPUBatchArray3D<float> V3;
+  auto ctx = MultiGPUContext::Make(K);
+  std::vector<std::shared_ptr<Var<V3>>> xs;
+  std::vector<std::shared_ptr<SrcOp<V3>>> srcs;
+  for (size_t r = 0; r < K; ++r) {
+    auto src = SrcOp<V3>::Make(Shape3D(W, Ht, C), N, ctx->device_context(r));
+    srcs.push_back(src);
+    xs.push_back(src);
+  }
+  auto pad = HaloPad2DOp<V3>::MakeParallel(1, xs, ctx);
+  auto exch = HaloExch2DOp<V3>::MakeParallel(1, pad, ctx);
+  Conv2DShape cs;
+  cs.filters = Co; cs.axes = {0, 1}; cs.kernel = {3, 3}; cs.stride = {1, 1}; cs.dilate = {1, 1}; cs.pad = {1, 1};
+  cs.halo_padded_input = true; cs.enable_hmma = false;
+  auto conv = parallel_conv2d<V3>(cs, exch, kaiming_init_gen<GPUArray4D<float>>(C * 9, Co), false, ctx);
+  std::mt19937_64 rng(99);
+  TxnId init_txn;
+  for (size_t r = 0; r < K; ++r) conv.ops[r]->init(init_txn, &rng);
+  ctx->sync();
+  // read every rank's filter back through the flat-vector plumbing
+  const size_t wdim = Co * C * 9;
+  std::vector<std::vector<float>> w(K, std::vector<float>(wdim));
+  GPUContext *root = ctx->device_context(0).get();
+  for (size_t r = 0; r < K; ++r) {
+    GPUMemory<float> flat = GPUMemory<float>::Zeros(wdim, root);
+    CHECK(conv.ops[r]->store_val(init_txn, conv.params[r], 0, &flat) == wdim);
+    GPUConn conn = root->conn();
+    flat.store_sync(w[r].data(), 0, wdim, conn);
+  }
+  double norm = 0;
+  for (float v : w[0]) norm += (double)v * v;
+  CHECK(norm > 0.1);
+  for (size_t r = 1; r < K; ++r) CHECK(w[r] == w[0]);
+}
+
 static void test_resnet18_tiling_invariance() {
   const size_t N = 2, H = 256, W = 32, classes = 10;
   ConvNetConfig cfg;
@@ -974,6 +1013,7 @@ int main(int argc, char **argv) {
     test_spatial_pool_graph(kAveragePool, 2, 3, 5, 8, 10);
     test_spatial_pool_graph(kMaxPool, 4, 8, 64, 112, 112);
     test_softmax_loss_op();
+    test_parallel_conv2d_init_gives_equal_copies();
     test_resnet18_tiling_invariance();
     test_parallel_sgd(4, 2, 8, 16, 12, false, 1);
     test_parallel_sgd(2, 2, 8, 8, 10, true, 1);
