@@ -292,9 +292,11 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   // of the row group that has landed, the five copies of the next group, and for beta = 1 the
   // four loads of old values (buffer loads and stores: a row that does not exist gets an
   // out-of-range offset, so the sequence has no branches).
-  auto compute = [&](uint32_t sb, auto side_tag, auto bar_tag, uint32_t row0, uint32_t nrows) {
+  auto compute = [&](uint32_t sb, auto side_tag, auto bar_tag, uint32_t row0, uint32_t nrows, bool barrier_owed) {
     constexpr bool SIDE = decltype(side_tag)::value != 0;
-    constexpr bool BAR = decltype(bar_tag)::value != 0;  // the phase's barrier comes between the rounds and the packing
+    // 1: this phase's barrier comes between the rounds and the packing; 2: the previous phase's barrier, if still
+    // owed, comes after the first operand fetches (row pair 0 only: they read rows that step shares with this one)
+    constexpr int BAR = decltype(bar_tag)::value;
     const uint32_t cur_off = ooff_lane + (row0 * P.OW + c0C) * 2u;
     const uint32_t off0 = nrows > 0u ? cur_off : kOutOfRange, off1 = nrows > 1u ? cur_off + orow_bytes : kOutOfRange;
     floatx4 acc[2][2][2];  // [row][column tile][channel tile]
@@ -321,6 +323,14 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
 #pragma unroll
     for (int t = 0; t < kAhead; ++t) fetch(t);
     __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+    if constexpr (BAR == 2) {
+      if (barrier_owed) {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
     // The copies of the group to transpose have landed: everything but the previous step's four
     // stores, which were issued after them (memory instructions complete in order).
     if (SIDE) __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
@@ -396,7 +406,7 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     };
     for_each_int(std::make_integer_sequence<int, kReads>(), round);
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (BAR) {
+    if constexpr (BAR == 1) {
       // every ring read and write of the phase is done (the operands have been multiplied)
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
@@ -434,31 +444,44 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): LDS only; __syncthreads() would also wait for the copies in flight
     __builtin_amdgcn_s_barrier();
   };
+  // Row pair 0 (the older wave of every SIMD, which finishes its rounds early) owes each phase's barrier
+  // until the next phase has fetched its first operands: those come from the two rows a step shares
+  // with the one before it, which no wave overwrites meanwhile.  Its matrix pipe then starts the moment
+  // the late waves arrive.  Row pair 1 passes the barrier between its rounds and its packing.
+  bool barrier_owed = false;
   for (;;) {
+    const bool fast = stepC >= 0 && wholeC;
+    if (barrier_owed && !(fast && rp == 0u)) {
+      phase_barrier();
+      barrier_owed = false;
+    }
     bool barrier_done = false;
     if (stepC >= 0) {
       const uint32_t row0 = r_beginC + (uint32_t)stepC * kStepRows + 2u * rp;  // this wave's first output row
       const uint32_t nrows = row0 >= r_endC ? 0u : min(2u, r_endC - row0);
       if (wholeC) {
-        // The older wave of a SIMD gets the matrix pipe first and finishes its rounds first: it
-        // packs and stores while it would wait, the younger one (row pair 1) after the barrier,
-        // while the older one already multiplies the next step.
         if (rp == 0u) {
-          compute(sb, IntTag<1>(), IntTag<0>(), row0, nrows);
+          compute(sb, IntTag<1>(), IntTag<2>(), row0, nrows, barrier_owed);
+          barrier_owed = false;
         } else {
-          compute(sb, IntTag<1>(), IntTag<1>(), row0, nrows);
+          compute(sb, IntTag<1>(), IntTag<1>(), row0, nrows, false);
           barrier_done = true;
         }
       } else {
         if (BETA) load_old_guarded(row0, nrows);
         move_rows_plain();
-        compute(sb, IntTag<0>(), IntTag<0>(), row0, nrows);
+        compute(sb, IntTag<0>(), IntTag<0>(), row0, nrows, false);
       }
     } else {
       move_rows_plain();
     }
     loader_advance();
-    if (!barrier_done) phase_barrier();
+    if (!barrier_done) {
+      if (rp == 0u)
+        barrier_owed = true;
+      else
+        phase_barrier();
+    }
     sb = wrap_slot(sb + kStepRows);
     tb = wrap_slot(tb + kStepRows);
     if (++stepC == stepsC) {
@@ -468,6 +491,7 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
       stepC = -1;
     }
   }
+  if (barrier_owed) phase_barrier();
 }
 
 // Shapes of the eight-wave kernel: input and output rows that start on a 4-byte boundary (input
