@@ -5,7 +5,8 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libadh.so")
+# ADH_LIB names another build of the library (A/B measurements); the default is the one beside this file
+LIB_PATH = os.environ.get("ADH_LIB") or os.path.join(_HERE, "libadh.so")
 CSRC = os.path.join(_HERE, "csrc")
 
 ADH_F32 = 0

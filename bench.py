@@ -34,7 +34,7 @@ if ROOT not in sys.path:
 # are profiles/conv3x3_bf16_fwd_cfg5_hbm_traffic.txt and profiles/conv3x3_fwd_cfg2_hbm_traffic.txt.
 # Not re-measured by this script; each figure belongs to the kernel instance named beside it and is
 # left out (null) when the library routes the shape to another instance.
-CONV_FWD_CFG5_TRAFFIC = ("conv3x3_bf16_w8_kernel<false>", None)
+CONV_FWD_CFG5_TRAFFIC = ("conv3x3_bf16_w8_kernel<false>", 1085.8e6)
 CONV_FWD_CFG2_TRAFFIC = ("conv3x3_f32_kernel<25,8,false,12>", 64.07e6)
 CLOCK_RAMP_MS = 150.0
 HBM_PEAK_GBS = 8000.0
@@ -111,10 +111,14 @@ def main():
                     help="skip the end-to-end trainer leg (a child process; leave it out under a profiler)")
     ap.add_argument("--only", default=None,
                     help="time only the secondary entries whose name contains this text (for profiling one kernel)")
+    ap.add_argument("--lib", default=None,
+                    help="another build of libadh.so to load (A/B measurements of a kernel variant)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain copy of known size (1 GiB read + 1 GiB written) 10 times: the kernel "
                          "whose FETCH_SIZE / WRITE_SIZE readings calibrate the HBM traffic counters")
     args = ap.parse_args()
+    if args.lib:
+        os.environ["ADH_LIB"] = os.path.abspath(args.lib)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (the K row-tiles live in one HBM, there are no "
               "inter-GPU collectives); --gpus %d is not supported" % args.gpus, file=sys.stderr)
