@@ -45,11 +45,14 @@ SIGNATURES = {
     "adh_conv3x3_kernel_name": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, f32, ctypes.c_char_p, sz]),
     "adh_conv3x3_slab_fwd": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_fwd_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp, sz, vp]),
+    "adh_conv3x3_slab_fwd_tiles_unexchanged": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_fwd_tiles_static": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp]),
     "adh_conv3x3_slab_bwd_data": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_data_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_filter": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_filter_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp, f32, vp, sz, vp]),
+    "adh_conv3x3_slab_bwd_filter_tiles_unexchanged": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp, f32, vp, sz,
+                                                            vp]),
     "adh_conv2d_workspace_bytes": (sz, [i32, i32] + [u32] * 12),
     "adh_conv2d_slab_fwd_tiles": (i32, [i32] + [u32] * 12 + [vpp, vp, vpp, f32, vp, sz, vp]),
     "adh_conv2d_slab_bwd_data_tiles": (i32, [i32] + [u32] * 12 + [vp, vpp, vpp, f32, vp, sz, vp]),
@@ -234,12 +237,15 @@ def _ws(ws):
     return ws.data_ptr(), ws.numel() * ws.element_size()
 
 
-def conv_fwd_tiles(xs, w, ys, N, Cin, Cout, H, W, beta=0.0, ws=None):
+def conv_fwd_tiles(xs, w, ys, N, Cin, Cout, H, W, beta=0.0, ws=None, unexchanged=False):
+    """unexchanged: xs are the row tiles of one activation in rank order whose inner halo rows have not been
+    exchanged; the result equals halo_exchange followed by the ordinary forward."""
     _dev(w, *xs, *ys)
     xt, k1 = _tbl(xs)
     yt, k2 = _tbl(ys)
     wp, wb = _ws(ws)
-    return lib().adh_conv3x3_slab_fwd_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, xt, w.data_ptr(), yt, beta,
+    fn = lib().adh_conv3x3_slab_fwd_tiles_unexchanged if unexchanged else lib().adh_conv3x3_slab_fwd_tiles
+    return fn(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, xt, w.data_ptr(), yt, beta,
                                             wp, wb, _stream())
 
 
@@ -393,13 +399,14 @@ def pool_bwd_tiles(mode, xs, ys, dys, dxs, N, C, HP, WP, wh, ww, sh, sw, beta=0.
                                            beta, _stream())
 
 
-def conv_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, H, W, beta=0.0, ws=None):
+def conv_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, H, W, beta=0.0, ws=None, unexchanged=False):
     _dev(dw, *xs, *dys)
     xt, k1 = _tbl(xs)
     dt, k2 = _tbl(dys)
     wp, wb = _ws(ws)
-    return lib().adh_conv3x3_slab_bwd_filter_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, xt, dt, dw.data_ptr(),
-                                                   beta, wp, wb, _stream())
+    fn = (lib().adh_conv3x3_slab_bwd_filter_tiles_unexchanged if unexchanged
+          else lib().adh_conv3x3_slab_bwd_filter_tiles)
+    return fn(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, xt, dt, dw.data_ptr(), beta, wp, wb, _stream())
 
 
 def softmax_fwd(x, y):

@@ -54,6 +54,10 @@ struct ConvParams {
   uint32_t tiles_x;         // ceil(OW / TW); grid.x = tiles_x * ceil(OH / R)
   uint32_t w_out_stride, w_red_stride;  // weight address = o*w_out_stride + k*w_red_stride + tap'
   int32_t w_flip;           // tap' = w_flip ? 8 - tap : tap
+  // forward over the row tiles of one activation, in rank order: input row 0 of tile t > 0 is read
+  // from tile t-1's last interior row and input row IH-1 of tile t < num_tiles-1 from tile t+1's
+  // first interior row, which is what a halo exchange would have copied there
+  int32_t rows_from_neighbours;
   float beta;
   FastDiv div_tiles_x, div_TW;
 };
@@ -129,15 +133,29 @@ __global__ __launch_bounds__(64 * WAVES, 1) void conv3x3_f32_kernel(const ConvPa
   const bool col_ok = lane < P.TW + 2u && iw >= 0 && iw < (int32_t)P.IW;
   const uint32_t patch_rows = P.R + 2u;
   uint32_t row_voff[RROWS];
+  // a patch row is one wave's, so the image it is read from is a wave-uniform choice: one buffer
+  // resource per patch row of this wave
+  __amdgpu_buffer_rsrc_t rsrc_row[RROWS];
 #pragma unroll
   for (int rr = 0; rr < RROWS; ++rr) {
     const uint32_t prow = wv + (uint32_t)WAVES * rr;
-    const int32_t ih = (int32_t)(oh0 + prow) - P.pad;
+    int32_t ih = (int32_t)(oh0 + prow) - P.pad;
     const bool ok = col_ok && prow < patch_rows && ih >= 0 && ih < (int32_t)P.IH;
+    const float *src = in;
+    if (P.rows_from_neighbours) {
+      const int32_t interior = (int32_t)P.IH - 2;
+      if (ih == 0 && t > 0u) {
+        src = P.in[t - 1u] + (uint64_t)n * P.Cred * in_plane;
+        ih = interior;
+      } else if (ih == (int32_t)P.IH - 1 && t + 1u < P.num_tiles) {
+        src = P.in[t + 1u] + (uint64_t)n * P.Cred * in_plane;
+        ih = 1;
+      }
+    }
     row_voff[rr] = ok ? ((uint32_t)ih * P.IW + (uint32_t)iw) * 4u : kOutOfRange;
+    rsrc_row[rr] = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(src), 0,
+                                                     (int)(P.Cred * (uint32_t)in_plane * 4u), kBufferFlags);
   }
-  const __amdgpu_buffer_rsrc_t rsrc_in =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), 0, (int)(P.Cred * (uint32_t)in_plane * 4u), kBufferFlags);
   auto stage_patch = [&](float *buf, uint32_t k0) {
     const bool ragged = ragged_k && k0 + kChunk > P.Cred;  // uniform: a ragged last chunk
 #pragma unroll
@@ -148,11 +166,11 @@ __global__ __launch_bounds__(64 * WAVES, 1) void conv3x3_f32_kernel(const ConvPa
       for (int kl = 0; kl < kChunk; ++kl) {
         float *dst = buf + kl * kChanStride + prow * kLdsPitch;
         if (!ragged) {
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, dst, 4, row_voff[rr], (k0 + kl) * (uint32_t)in_plane * 4u, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_row[rr], dst, 4, row_voff[rr], (k0 + kl) * (uint32_t)in_plane * 4u, 0, 0);
         } else {  // channels past Cred are loaded as zero
           const bool k_ok = k0 + kl < P.Cred;
           const uint32_t soff = __builtin_amdgcn_readfirstlane(min(k0 + kl, P.Cred - 1u) * (uint32_t)in_plane * 4u);
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, dst, 4, k_ok ? row_voff[rr] : kOutOfRange, soff, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_row[rr], dst, 4, k_ok ? row_voff[rr] : kOutOfRange, soff, 0, 0);
         }
       }
     }
@@ -376,7 +394,7 @@ int conv_bf16_via_f32(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, u
 // which: ADH_CONV_FWD or ADH_CONV_BWD_DATA.  H, W are the interior extents.
 static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                        uint32_t W, const void *const *in_tiles, const void *w, void *const *out_tiles, float beta,
-                       hipStream_t st) {
+                       hipStream_t st, bool rows_from_neighbours = false) {
   if (!dtype_ok(dtype)) return ADH_EINVAL;
   if (dtype != ADH_F32) return ADH_EUNIMPL;
   if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
@@ -400,6 +418,7 @@ static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uin
   P.num_tiles = num_tiles;
   P.N = N;
   P.beta = beta;
+  P.rows_from_neighbours = (which == ADH_CONV_FWD && rows_from_neighbours) ? 1 : 0;
   if (which == ADH_CONV_FWD) {
     P.Cred = Cin; P.Cout = Cout;
     P.IH = (uint32_t)HP; P.IW = (uint32_t)WP; P.OH = H; P.OW = W;
@@ -472,6 +491,23 @@ int adh_conv3x3_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32
                              workspace_bytes, as_stream(stream));
   return conv_direct(ADH_CONV_FWD, dtype, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, w, y_tiles, beta,
                      as_stream(stream));
+}
+
+int adh_conv3x3_slab_fwd_tiles_unexchanged(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                           uint32_t H, uint32_t W, const void *const *x_pad_tiles, const void *w,
+                                           void *const *y_tiles, float beta, void *workspace, size_t workspace_bytes,
+                                           void *stream) {
+  if (dtype == ADH_BF16) {
+    // the bf16 kernels stream their rows from one image: exchange first, then the ordinary forward
+    const int rc = adh_halo_exchange_nchw(dtype, 1, num_tiles, 1, W, H, Cin, N,
+                                          const_cast<void *const *>(reinterpret_cast<const void *const *>(x_pad_tiles)),
+                                          stream);
+    if (rc != ADH_OK) return rc;
+    return adh_conv3x3_slab_fwd_tiles(dtype, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, w, y_tiles, beta, workspace,
+                                      workspace_bytes, stream);
+  }
+  return conv_direct(ADH_CONV_FWD, dtype, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, w, y_tiles, beta,
+                     as_stream(stream), true);
 }
 
 int adh_conv3x3_slab_fwd(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,

@@ -42,6 +42,10 @@ struct WgradParams {
   uint32_t cols_per_block, col_tiles;         // column tiles of a plane (<= kMaxW columns each)
   // grid.x = col_tiles * chunks_per_plane * N * num_tiles
   uint32_t ci_groups;        // grid.y = co_halves * ci_groups, co_halves = ceil(Cout/32)
+  // the tiles are the row tiles of one activation in rank order: slab row 0 of tile t > 0 is read from
+  // tile t-1's last interior row and slab row H+1 of tile t < num_tiles-1 from tile t+1's first
+  // interior row, which is what a halo exchange would have copied there
+  int32_t rows_from_neighbours;
   FastDiv div_chunks, div_tiles, div_ci_groups, div_cols;
 };
 
@@ -91,7 +95,24 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
   const uint32_t x_voff = lane < tw + 2u ? (w0 + lane) * 4u : kWgOutOfRange;
   const uint32_t d_voff = lane < tw ? (w0 + lane) * 4u : kWgOutOfRange;
   const bool ragged_c = (ci0 + 64u > P.Cin) || (co0 + 32u > P.Cout);  // uniform
+  // a slab row is uniform over the workgroup, and so is the image it comes from
+  const bool from_above = P.rows_from_neighbours && t > 0u;
+  const bool from_below = P.rows_from_neighbours && t + 1u < P.num_tiles;
+  const __amdgpu_buffer_rsrc_t rsrc_above = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(P.x[from_above ? t - 1u : t] + ((uint64_t)n * P.Cin) * HP * WP), 0, (int)(P.Cin * HP * WP * 4u),
+      kWgBufferFlags);
+  const __amdgpu_buffer_rsrc_t rsrc_below = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(P.x[from_below ? t + 1u : t] + ((uint64_t)n * P.Cin) * HP * WP), 0, (int)(P.Cin * HP * WP * 4u),
+      kWgBufferFlags);
   auto stage_x_row = [&](float *slot, uint32_t y) {  // slab row y of the 64 input channels
+    __amdgpu_buffer_rsrc_t rsrc = rsrc_x;
+    if (from_above && y == 0u) {
+      rsrc = rsrc_above;
+      y = P.H;
+    } else if (from_below && y == HP - 1u) {
+      rsrc = rsrc_below;
+      y = 1u;
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const uint32_t cl = wv * 8u + i;
@@ -101,7 +122,7 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
         voff = kWgOutOfRange;
         ci = 0;
       }
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, slot + cl * kRowPitch, 4, voff,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, slot + cl * kRowPitch, 4, voff,
                                                __builtin_amdgcn_readfirstlane((ci * HP + y) * WP * 4u), 0, 0);
     }
   };
@@ -319,11 +340,17 @@ size_t adh_conv3x3_workspace_bytes(int which, int dtype, uint32_t num_tiles, uin
   return dtype == ADH_F32 ? f32_bytes : 0;
 }
 
-int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
-                                      uint32_t H, uint32_t W, const void *const *x_pad_tiles,
-                                      const void *const *dy_tiles, float *dw, float beta, void *workspace,
-                                      size_t workspace_bytes, void *stream) {
+static int wgrad_entry(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                       const void *const *x_pad_tiles, const void *const *dy_tiles, float *dw, float beta,
+                       void *workspace, size_t workspace_bytes, void *stream, bool rows_from_neighbours) {
   if (!dtype_ok(dtype)) return ADH_EINVAL;
+  if (dtype == ADH_BF16 && rows_from_neighbours) {
+    // the bf16 kernels stream their rows from one image: exchange first, then the ordinary path
+    const int rc = adh_halo_exchange_nchw(dtype, 1, num_tiles, 1, W, H, Cin, N,
+                                          const_cast<void *const *>(reinterpret_cast<const void *const *>(x_pad_tiles)),
+                                          stream);
+    if (rc != ADH_OK) return rc;
+  }
   if (dtype == ADH_BF16)
     return conv_bf16_filter_via_f32(num_tiles, N, Cin, Cout, H, W, x_pad_tiles, dy_tiles, dw, beta, workspace,
                                     workspace_bytes, as_stream(stream));
@@ -363,6 +390,7 @@ int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N,
   P.div_chunks = FastDiv(plan.chunks_per_plane);
   P.div_tiles = FastDiv(num_tiles);
   P.div_ci_groups = FastDiv(P.ci_groups);
+  P.rows_from_neighbours = rows_from_neighbours ? 1 : 0;
   dim3 grid(plan.blocks_x, plan.groups, 1);
   if (grid.y > 65535u) return ADH_EINVAL;
   hipLaunchKernelGGL(conv3x3_wgrad_f32_kernel, grid, dim3(kWgThreads), 0, st, P);
@@ -375,6 +403,23 @@ int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N,
   R.div9 = FastDiv(9); R.div_cin = FastDiv(Cin);
   hipLaunchKernelGGL(conv3x3_wgrad_reduce_kernel, dim3((R.total + 63u) / 64u), dim3(256), 0, st, R);
   return launch_status();
+}
+
+int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                      uint32_t H, uint32_t W, const void *const *x_pad_tiles,
+                                      const void *const *dy_tiles, float *dw, float beta, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+  return wgrad_entry(dtype, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, dy_tiles, dw, beta, workspace, workspace_bytes,
+                     stream, false);
+}
+
+int adh_conv3x3_slab_bwd_filter_tiles_unexchanged(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,
+                                                  uint32_t Cout, uint32_t H, uint32_t W,
+                                                  const void *const *x_pad_tiles, const void *const *dy_tiles,
+                                                  float *dw, float beta, void *workspace, size_t workspace_bytes,
+                                                  void *stream) {
+  return wgrad_entry(dtype, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, dy_tiles, dw, beta, workspace, workspace_bytes,
+                     stream, true);
 }
 
 int adh_conv3x3_slab_bwd_filter(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,

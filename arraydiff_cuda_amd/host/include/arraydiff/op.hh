@@ -830,15 +830,19 @@ private:
 template <typename V>
 class HaloExch2DOp : public virtual Op {
 public:
+  // forward_by_consumer (not in the reference): the forward pass copies nothing, because the consumer is a
+  // convolution built with Conv2DShape::unexchanged_rows, which reads the neighbours' rows itself; the
+  // backward pass (the halo reduce of the gradient) is unchanged.
   static vector<shared_ptr<Var<V>>> MakeParallel(size_t halo_pad, vector<shared_ptr<Var<V>>> inputs,
-                                                 shared_ptr<Context> ctx) {
-    auto op = make_shared<HaloExch2DOp<V>>(halo_pad, inputs, ctx);
+                                                 shared_ptr<Context> ctx, bool forward_by_consumer = false) {
+    auto op = make_shared<HaloExch2DOp<V>>(halo_pad, inputs, ctx, forward_by_consumer);
     vector<shared_ptr<Var<V>>> outputs;
     for (size_t r = 0; r < inputs.size(); ++r) outputs.push_back(make_shared<NoOp<V>>(op, op->xs_.at(r).clone()));
     return outputs;
   }
-  HaloExch2DOp(size_t halo_pad, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx)
-      : ctx_(ctx), halo_pad_(halo_pad), inputs_(inputs) {
+  HaloExch2DOp(size_t halo_pad, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx,
+               bool forward_by_consumer = false)
+      : ctx_(ctx), halo_pad_(halo_pad), forward_by_consumer_(forward_by_consumer), inputs_(inputs) {
     if (inputs.size() != mgpu_ctx_of(ctx)->num_ranks()) throw std::invalid_argument("HaloExch2DOp: one input per rank");
     for (auto &in : inputs) xs_.push_back(in->data());
   }
@@ -865,6 +869,7 @@ public:
 private:
   shared_ptr<Context> ctx_;
   size_t halo_pad_;
+  bool forward_by_consumer_;
   vector<shared_ptr<Var<V>>> inputs_;
   vector<VarData<V>> xs_;
 };
@@ -888,6 +893,12 @@ public:
   // the other ranks' gradients are zero.  The sum over ranks, which is all the optimizer uses,
   // is the same.
   bool replicated_filters = false;
+  // Not in the reference.  The inputs are the row tiles of one activation in rank order (a 1 x K grid)
+  // whose inner halo rows nobody exchanged (HaloExch2DOp made with forward_by_consumer): the forward
+  // pass and the filter gradient read those rows from the neighbouring tiles, or exchange them first
+  // where the kernel for the shape cannot (or where the ranks' filters differ, so that one launch cannot
+  // hold every tile).
+  bool unexchanged_rows = false;
 };
 
 // V = GPUBatchArray3D<float>, A = GPUArray4D<float> (filter, Shape4D(kw,kh,Cin,Cout) = KCRS).
@@ -927,6 +938,8 @@ public:
       throw std::invalid_argument("SlabConv2DOp: padding needs a halo-padded input");
     if (inputs.empty() || inputs.size() != kernels.size() || inputs.size() > ADH_MAX_TILES)
       throw std::invalid_argument("SlabConv2DOp: one kernel variable per input");
+    if (shape.unexchanged_rows && !(shape.halo_padded_input && shape.pad[0] == 1 && shape.pad[1] == 1))
+      throw std::invalid_argument("SlabConv2DOp: unexchanged rows need a halo of one");
     for (size_t r = 0; r < inputs.size(); ++r) {
       auto off = inputs[r]->offset();
       if (off.shape[0] != shape.pad[0] || off.shape[1] != shape.pad[1] || off.shape[2] != 0)

@@ -110,10 +110,12 @@ template <typename V>
 vector<shared_ptr<Var<V>>> exchanged_conv3x3(ParallelBatchNormParamOp<V> &block, Conv2DShape shape, size_t stride,
                                              vector<shared_ptr<Var<V>>> padded, shared_ptr<Context> ctx) {
   typedef GPUArray4D<float> A;
-  auto exch = HaloExch2DOp<V>::MakeParallel(1, padded, ctx);
   Conv2DShape cs = shape;
   cs.stride = {stride, stride};
   cs.halo_padded_input = true;
+  // over row tiles the convolution reads its neighbours' rows itself and the exchange copies nothing
+  cs.unexchanged_rows = mgpu_ctx_of(ctx)->spatial_comm(0)->num_w_ranks == 1 && padded.size() > 1;
+  auto exch = HaloExch2DOp<V>::MakeParallel(1, padded, ctx, cs.unexchanged_rows);
   const size_t cin = padded.at(0)->shape().shape[2];
   auto conv = parallel_conv2d<V, A>(cs, exch, kaiming_init_gen<A>(cin * shape.kernel[0] * shape.kernel[1], shape.filters),
                                     false, ctx);

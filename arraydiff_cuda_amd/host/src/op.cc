@@ -339,6 +339,7 @@ void HaloExch2DOp<V3>::_forward(TxnId txn) {
     if (xs_.at(r).val().accumulate(txn, id(), ctx->device_context(r).get(), [](V3 *) {})) ++num_writes;
   if (num_writes != 0 && num_writes != ctx->num_ranks()) throw HazardError("HaloExch2DOp: some ranks already exchanged");
   if (num_writes == 0) return;
+  if (forward_by_consumer_) return;  // the consuming convolution reads the neighbours' rows itself
   for (size_t r = 0; r < ctx->num_ranks(); ++r) {
     V3 &x = xs_.at(r).val().get_mut(txn, id());
     check_padded(x, halo_pad_, "HaloExch2DOp");  // op.cc:2981-2982
@@ -418,6 +419,13 @@ bool use_3x3_filter_kernel(const Op &op, const TileDims &d, uint32_t n, size_t f
   return op.is_3x3_unit() && (uint64_t)d.H * d.W > 256u && fits_3x3_kernels(d, n, filters);
 }
 
+// With unexchanged rows the forward kernel and the filter-gradient kernel must both be the 3x3 ones, which can
+// read a halo row from the neighbouring tile; any other shape exchanges first and runs as usual.
+template <typename Op>
+bool reads_neighbour_rows(const Op &op, const Conv2DShape &cs, const TileDims &d, uint32_t n) {
+  return cs.unexchanged_rows && use_3x3_kernels(op, d, n, cs.filters) && use_3x3_filter_kernel(op, d, n, cs.filters);
+}
+
 void *conv_scratch(GPUContext *dc, int which, uint32_t n, const TileDims &d, const Conv2DShape &cs, size_t *bytes) {
   *bytes = adh_conv2d_workspace_bytes(which, ADH_F32, n, d.N, d.C, (uint32_t)cs.filters, d.H + 2 * (uint32_t)cs.pad[1],
                                       d.W + 2 * (uint32_t)cs.pad[0], (uint32_t)cs.kernel[1], (uint32_t)cs.kernel[0],
@@ -443,6 +451,7 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
   // group the ranks by filter buffer: one launch per distinct filter (one in all when the filters
   // are promised equal)
   const bool replicated = shape_.replicated_filters;
+  bool exchanged = false;
   while (!todo.empty()) {
     const float *w0 = kernels_[replicated ? 0 : todo[0]].val().get(txn, id()).dptr();
     const void *xt[ADH_MAX_TILES];
@@ -468,7 +477,21 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
-    if (use_3x3_kernels(*this, d, n, shape_.filters)) {
+    const bool in_kernel_rows = n == K && reads_neighbour_rows(*this, shape_, d, n);
+    if (shape_.unexchanged_rows && !in_kernel_rows && !exchanged) {
+      // no kernel for this shape reads across tiles (or this launch does not hold every tile): exchange over
+      // all ranks once, then the ordinary path
+      void *all[ADH_MAX_TILES];
+      for (size_t r = 0; r < K; ++r) all[r] = xs_[r].val().get(txn, id()).base_as_view().dptr();
+      adh_check(adh_halo_exchange_nchw(ADH_F32, 1, (uint32_t)K, 1, d.W, d.H, d.C, d.N, all, conn.stream()),
+                "SlabConv2DOp::_forward (exchange)");
+      exchanged = true;
+    }
+    if (in_kernel_rows) {
+      adh_check(adh_conv3x3_slab_fwd_tiles_unexchanged(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt,
+                                                       0.0f, nullptr, 0, conn.stream()),
+                "SlabConv2DOp::_forward (unexchanged)");
+    } else if (use_3x3_kernels(*this, d, n, shape_.filters)) {
       adh_check(adh_conv3x3_slab_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt, 0.0f,
                                            nullptr, 0, conn.stream()),
                 "SlabConv2DOp::_forward");
@@ -551,8 +574,11 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
                                                     d.H, d.W);
       dc->reserve_scratch(ws);
       auto scratch = dc->get_scratch();
-      adh_check(adh_conv3x3_slab_bwd_filter_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, dyt, dw,
-                                                  wbeta, scratch->dptr(), scratch->size(), conn.stream()),
+      // rows the forward pass read from the neighbours were never copied: read them there again
+      auto entry = n == K && reads_neighbour_rows(*this, shape_, d, n) ? adh_conv3x3_slab_bwd_filter_tiles_unexchanged
+                                                                       : adh_conv3x3_slab_bwd_filter_tiles;
+      adh_check(entry(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, dyt, dw, wbeta, scratch->dptr(),
+                      scratch->size(), conn.stream()),
                 "SlabConv2DOp::_backward (filter)");
     } else {
       size_t ws_bytes;

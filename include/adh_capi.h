@@ -155,6 +155,19 @@ int adh_conv3x3_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32
                                uint32_t H, uint32_t W, const void *const *x_pad_tiles, const void *w,
                                void *const *y_tiles, float beta, void *workspace,
                                size_t workspace_bytes, void *stream);
+/* HaloExch2DOp::_forward (src/op.cc:2963-3007) and the cudnnConvolutionForward of its consumer
+ * (src/op.cc:1576-1587) in one launch: x_pad_tiles are the row tiles of ONE activation in rank order
+ * (a 1 x num_tiles grid, halo width 1) whose inner halo rows have NOT been exchanged.  The result
+ * equals adh_halo_exchange_nchw followed by adh_conv3x3_slab_fwd_tiles, bit for bit: tile t reads
+ * its top halo row from tile t-1's last interior row and its bottom halo row from tile t+1's first.
+ * fp32 leaves the inner halo rows of x_pad unread and unwritten; bf16 exchanges and then convolves
+ * (two launches, the halo rows are refreshed).  The outer halo rows are read from each tile itself;
+ * the corner elements of an inner halo row, which an exchange does not touch, are taken from the
+ * neighbour's halo columns: both are zero after HaloPad2DOp, and must be equal for the equality to hold. */
+int adh_conv3x3_slab_fwd_tiles_unexchanged(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                           uint32_t H, uint32_t W, const void *const *x_pad_tiles,
+                                           const void *w, void *const *y_tiles, float beta, void *workspace,
+                                           size_t workspace_bytes, void *stream);
 /* adh_conv3x3_slab_fwd_tiles for callers that cannot allocate and have no workspace to pass (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  dtype must be ADH_BF16 with Cin <= 64 and Cout <= 256 (else
@@ -187,6 +200,14 @@ int adh_conv3x3_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N,
                                       const void *const *x_pad_tiles, const void *const *dy_tiles,
                                       float *dw, float beta, void *workspace, size_t workspace_bytes,
                                       void *stream);
+/* the filter gradient over tiles whose inner halo rows were never exchanged (the backward of a
+ * forward that went through adh_conv3x3_slab_fwd_tiles_unexchanged): equals adh_halo_exchange_nchw
+ * followed by adh_conv3x3_slab_bwd_filter_tiles, bit for bit. */
+int adh_conv3x3_slab_bwd_filter_tiles_unexchanged(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,
+                                                  uint32_t Cout, uint32_t H, uint32_t W,
+                                                  const void *const *x_pad_tiles, const void *const *dy_tiles,
+                                                  float *dw, float beta, void *workspace,
+                                                  size_t workspace_bytes, void *stream);
 
 /* ---- general window / stride / dilation over the halo-padded slab ------------ */
 /* The other consumers of halo-padded input (CudnnConv2DSize with halo_padded_input,
