@@ -73,6 +73,8 @@ SIGNATURES = {
     "adh_softmax_nll_loss_fwd": (i32, [u32, u32, vp, vp, vp, vp]),
     "adh_softmax_nll_loss_bwd": (i32, [u32, u32, vp, vp, vp, vp, vp]),
     "adh_softmax_xent_fwd": (i32, [u32, u32, vp, vp, vp, vp, vp]),
+    "adh_softmax_nll_loss_bwd_scaled": (i32, [u32, u32, vp, vp, vp, f32, f32, vp, vp]),
+    "adh_softmax_xent_fwd_bwd": (i32, [u32, u32, vp, vp, vp, f32, vp, vp, f32, vp, vp]),
     "adh_scale_add_f32": (i32, [u64, f32, vp, f32, vp, vp]),
     "adh_add_online_f32": (i32, [u64, f32, vp, vp, vp]),
     "adh_stat_step_f32": (i32, [u64, f32, vp, vp, vp, vp]),
@@ -432,6 +434,23 @@ def softmax_nll_loss_bwd(y, label, dloss, dx):
     N, C = y.shape
     return lib().adh_softmax_nll_loss_bwd(C, N, y.data_ptr(), label.data_ptr(), dloss.data_ptr(), dx.data_ptr(),
                                           _stream())
+
+
+def softmax_nll_loss_bwd_scaled(y, label, dloss, dloss_all, beta, dx):
+    """dx = beta*dx + dl*(y - onehot); dloss None: every example's dl is dloss_all."""
+    _dev(y, label, dx)
+    N, C = y.shape
+    return lib().adh_softmax_nll_loss_bwd_scaled(C, N, y.data_ptr(), label.data_ptr(),
+                                                 None if dloss is None else dloss.data_ptr(), dloss_all, beta,
+                                                 dx.data_ptr(), _stream())
+
+
+def softmax_xent_fwd_bwd(x, label, dloss, dloss_all, y, loss, beta, dx):
+    _dev(x, label, y, loss, dx)
+    N, C = x.shape
+    return lib().adh_softmax_xent_fwd_bwd(C, N, x.data_ptr(), label.data_ptr(),
+                                          None if dloss is None else dloss.data_ptr(), dloss_all, y.data_ptr(),
+                                          loss.data_ptr(), beta, dx.data_ptr(), _stream())
 
 
 def conv_kernel_name(which, dtype, K, N, Cin, Cout, H, W, beta=0.0):

@@ -1014,8 +1014,10 @@ void SoftmaxNLLLossOp<V1, L0, F0>::_forward(TxnId txn) {
     y.set_batch_size(N);
     loss.set_batch_size(N);
     if (label.batch_size() != N) throw std::invalid_argument("SoftmaxNLLLossOp: one label per example");
-    softmax_fwd<float>(C, N, x.as_view().dptr(), y.as_view().dptr(), conn.stream());
-    softmax_nll_loss_fwd<float>(C, N, y.as_view().dptr(), label.as_view().dptr(), loss.as_view().dptr(), conn.stream());
+    // softmax and loss in one launch (the reference: a cuDNN call, then its own kernel, op.cc:4129-4163)
+    adh_check(adh_softmax_xent_fwd(C, N, x.as_view().dptr(), label.as_view().dptr(), y.as_view().dptr(),
+                                   loss.as_view().dptr(), conn.stream()),
+              "SoftmaxNLLLossOp::_forward");
   }
 }
 template <>
@@ -1024,15 +1026,18 @@ void SoftmaxNLLLossOp<V1, L0, F0>::_backward(TxnId txn) {
   V1 &y = y_.val().get(txn, id());
   const uint32_t C = (uint32_t)y.dim().shape[0], N = (uint32_t)y.batch_size();
   const size_t batch = N;
-  if (x_.grad().accumulate(txn, id(), ctx, [ctx, batch](V1 *g) {
-        GPUConn conn = ctx->conn();
+  // the first toucher overwrites (beta = 0) where the reference clears the gradient and then adds
+  // (op.cc:4171-4176): the same values in one launch
+  bool first = false;
+  if (x_.grad().accumulate(txn, id(), ctx, [batch, &first](V1 *g) {
         g->set_batch_size(batch);
-        g->as_view().set_constant(0.0f, conn);
+        first = true;
       })) {
     GPUConn conn = ctx->conn();
-    softmax_nll_loss_bwd<float>(C, N, y.as_view().dptr(), label_.val().get(txn, id()).as_view().dptr(),
-                                loss_.grad().get(txn, id()).as_view().dptr(),
-                                x_.grad().get_mut(txn, id()).as_view().dptr(), conn.stream());
+    adh_check(adh_softmax_nll_loss_bwd_scaled(C, N, y.as_view().dptr(), label_.val().get(txn, id()).as_view().dptr(),
+                                              loss_.grad().get(txn, id()).as_view().dptr(), 0.0f, first ? 0.0f : 1.0f,
+                                              x_.grad().get_mut(txn, id()).as_view().dptr(), conn.stream()),
+              "SoftmaxNLLLossOp::_backward");
   }
 }
 

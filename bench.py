@@ -360,6 +360,14 @@ def main():
             lambda: lib.adh_softmax_nll_loss_bwd(Cs, Ns, sy.data_ptr(), labels.data_ptr(), dl.data_ptr(),
                                                  sdx.data_ptr(), stream),
             "hbm", 3 * Ns * Cs * 4 + 8 * Ns, HBM_PEAK_GBS, "GB/s", graph=True)
+        add("softmax + nll fwd and bwd in one kernel cfg4 (256x1000)",
+            lambda: lib.adh_softmax_xent_fwd_bwd(Cs, Ns, logits.data_ptr(), labels.data_ptr(), dl.data_ptr(), 0.0,
+                                                 sy.data_ptr(), sloss.data_ptr(), 0.0, sdx.data_ptr(), stream),
+            "hbm", 3 * Ns * Cs * 4 + 12 * Ns, HBM_PEAK_GBS, "GB/s", graph=True)
+        add("conv fwd cfg3 over unexchanged tiles (4 tiles, exchange + conv in one launch)",
+            lambda: lib.adh_conv3x3_slab_fwd_tiles_unexchanged(0, K, N, C, C, Ht, W, tile_tbl, wt.data_ptr(), y_tbl, 0.0,
+                                                               None, 0, stream),
+            "mfma", flops_step, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
         add("conv bwd-data cfg3 (4 tiles)",
             lambda: lib.adh_conv3x3_slab_bwd_data_tiles(0, K, N, C, C, Ht, W, wt.data_ptr(), dy_tbl, g_tbl, 0.0, None,
                                                         0, stream),

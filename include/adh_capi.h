@@ -335,6 +335,20 @@ int adh_softmax_nll_loss_bwd(uint32_t C, uint32_t N, const float *y, const uint3
 /* CudnnSoftmaxNLLLossOp::_forward, src/op.cc:4118-4163, in one kernel: y and loss together */
 int adh_softmax_xent_fwd(uint32_t C, uint32_t N, const float *x, const uint32_t *label, float *y,
                          float *loss, void *stream);
+/* softmax_nll_loss_bwd with the two launches the reference puts before it folded in
+ * (src/op.cc:4165-4188: the gradient is zeroed on first touch, then the kernel adds):
+ * dx = beta*dx + dl*(y - onehot), beta 0 or 1, dl = dloss ? dloss[i] : dloss_all (a loss that is the
+ * gradient sink seeds every example with one number, src/zoo.cc:1877-1878). */
+int adh_softmax_nll_loss_bwd_scaled(uint32_t C, uint32_t N, const float *y, const uint32_t *label,
+                                    const float *dloss, float dloss_all, float beta, float *dx,
+                                    void *stream);
+/* CudnnSoftmaxNLLLossOp::_forward and ::_backward (src/op.cc:4118-4188) in ONE kernel, for callers
+ * that know the loss gradient when the logits arrive (a training step whose loss is the sink):
+ * y and loss as adh_softmax_xent_fwd, dx as adh_softmax_nll_loss_bwd_scaled, bit for bit.
+ * dx may alias x up to 2048 classes; it may not alias y. */
+int adh_softmax_xent_fwd_bwd(uint32_t C, uint32_t N, const float *x, const uint32_t *label,
+                             const float *dloss, float dloss_all, float *y, float *loss, float beta,
+                             float *dx, void *stream);
 
 /* ---- flat parameter vectors and the SGD update (fp32) ---------------------- */
 /* array_add_scaled_packed<float>, src/kernels/array.cu:97-110,211-222: y = alpha*x + beta*y,

@@ -41,11 +41,30 @@ def test_softmax_nll_vs_oracle(oracle, N, C):
     gdx = dev(dx0)
     capi.check(capi.softmax_nll_loss_bwd(gy, gl, dev(dloss), gdx))
     assert rel_err(host(gdx), dx) <= TOL
-    # bwd on the oracle's y: same arithmetic up to the fused multiply-add the GPU compiler
-    # contracts `dx + dloss*(y-1)` into (one rounding instead of two)
+    # bwd on the oracle's y: the same arithmetic up to the fused multiply-add a host compiler may contract
+    # `dx + dloss*(y-1)` into (one rounding instead of the kernel's two)
     gdx2 = dev(dx0)
     capi.check(capi.softmax_nll_loss_bwd(dev(y), gl, dev(dloss), gdx2))
     np.testing.assert_allclose(host(gdx2), dx, rtol=1e-6, atol=1e-7)
+
+    # one kernel for y, loss and dx: the same bits as the separate entry points, for a per-example
+    # gradient and for one number, accumulating and overwriting
+    for beta in (1.0, 0.0):
+        for per_example in (True, False):
+            gdl = dev(dloss) if per_example else None
+            want = dev(dx0)
+            capi.check(capi.softmax_nll_loss_bwd_scaled(gy, gl, gdl, 1.0 / N, beta, want))
+            if per_example and beta == 1.0:
+                assert torch.equal(want, gdx)
+            if beta == 0.0:
+                ref = np.zeros_like(dx0)
+                oracle.softmax_nll_loss_bwd(host(gy), label, dloss, ref)
+                np.testing.assert_array_equal(host(want), ref)
+            gy3 = torch.full((N, C), float("nan"), device="cuda")
+            gloss3 = torch.full((N,), float("nan"), device="cuda")
+            got = dev(dx0)
+            capi.check(capi.softmax_xent_fwd_bwd(gx, gl, gdl, 1.0 / N, gy3, gloss3, beta, got))
+            assert torch.equal(gy3, gy) and torch.equal(gloss3, gloss) and torch.equal(got, want)
 
 
 def test_softmax_properties():
@@ -69,3 +88,19 @@ def test_softmax_properties():
     dl = torch.full((N,), 1.0 / N, device="cuda")
     capi.check(capi.softmax_nll_loss_bwd(y, labels, dl, dx))
     assert float(dx.double().sum(dim=1).abs().max()) < 1e-7
+
+
+def test_fused_forward_backward_error_codes():
+    x = torch.zeros(2, 8, device="cuda")
+    lab = torch.zeros(2, dtype=torch.int32, device="cuda")
+    y, dx, loss = torch.empty_like(x), torch.empty_like(x), torch.empty(2, device="cuda")
+    assert capi.softmax_xent_fwd_bwd(x, lab, None, 1.0, y, loss, 0.5, dx) == capi.ADH_EINVAL
+    assert capi.softmax_xent_fwd_bwd(x, lab, None, 1.0, y, loss, 0.0, y) == capi.ADH_EINVAL
+    assert capi.softmax_nll_loss_bwd_scaled(y, lab, None, 1.0, 2.0, dx) == capi.ADH_EINVAL
+    # the gradient may overwrite the logits of a short row
+    capi.check(capi.softmax_xent_fwd(x, lab, y, loss))
+    want = torch.empty_like(x)
+    capi.check(capi.softmax_nll_loss_bwd_scaled(y, lab, None, 0.5, 0.0, want))
+    xin = x.clone()
+    capi.check(capi.softmax_xent_fwd_bwd(xin, lab, None, 0.5, y, loss, 0.0, xin))
+    assert torch.equal(xin, want)
