@@ -368,6 +368,11 @@ def main():
             lambda: lib.adh_conv3x3_slab_fwd_tiles_unexchanged(0, K, N, C, C, Ht, W, tile_tbl, wt.data_ptr(), y_tbl, 0.0,
                                                                None, 0, stream),
             "mfma", flops_step, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+        add("halo exchange + conv fwd cfg3 (4 tiles, two launches: what the one above replaces)",
+            lambda: (lib.adh_halo_exchange_nchw(0, 1, K, p, W, Ht, C, N, tile_tbl, stream),
+                     lib.adh_conv3x3_slab_fwd_tiles(0, K, N, C, C, Ht, W, tile_tbl, wt.data_ptr(), y_tbl, 0.0, None, 0,
+                                                    stream))[1],
+            "mfma", flops_step, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
         add("conv bwd-data cfg3 (4 tiles)",
             lambda: lib.adh_conv3x3_slab_bwd_data_tiles(0, K, N, C, C, Ht, W, wt.data_ptr(), dy_tbl, g_tbl, 0.0, None,
                                                         0, stream),
