@@ -462,7 +462,7 @@ static int conv_direct_kernel_name(int which, uint32_t num_tiles, uint32_t N, ui
   return ADH_OK;
 }
 
-const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t W, float beta);
+const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, float beta);
 
 }  // namespace adh
 
@@ -476,7 +476,7 @@ int adh_conv3x3_kernel_name(int which, int dtype, uint32_t num_tiles, uint32_t N
   if (which != ADH_CONV_FWD && which != ADH_CONV_BWD_DATA) return ADH_EINVAL;
   if (num_tiles == 0 || N == 0 || Cin == 0 || Cout == 0 || H == 0 || W == 0) return ADH_EINVAL;
   if (dtype == ADH_BF16) {
-    snprintf(name, name_bytes, "%s", conv_bf16_kernel_name(which, Cin, Cout, W, beta));
+    snprintf(name, name_bytes, "%s", conv_bf16_kernel_name(which, Cin, Cout, H, W, beta));
     return ADH_OK;
   }
   if (dtype != ADH_F32) return ADH_EINVAL;

@@ -60,8 +60,9 @@ static uint32_t cvt_grid(uint64_t n) {
 // fp32 scratch copies live in 256-byte aligned consecutive regions of the workspace
 static size_t region(uint64_t elems) { return (size_t)((elems * 4u + 255u) / 256u * 256u); }
 
-bool conv_bf16_mfma_supported(int which, uint32_t Cin, uint32_t Cout);
-size_t conv_bf16_mfma_workspace_bytes(int which, uint32_t Cin, uint32_t Cout);
+bool conv_bf16_mfma_supported(int which, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W);
+size_t conv_bf16_mfma_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                                      uint32_t W);
 int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
                    const void *const *in_tiles, const void *w, void *const *out_tiles, float beta, void *workspace,
                    hipStream_t st);
@@ -76,8 +77,8 @@ size_t bf16_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t 
                             uint32_t W, size_t fp32_path_bytes) {
   if (which == ADH_CONV_BWD_FILTER && conv_bf16_wgrad_mfma_supported(Cin, Cout, W))
     return conv_bf16_wgrad_mfma_workspace_bytes(num_tiles, N, W);
-  if (which != ADH_CONV_BWD_FILTER && conv_bf16_mfma_supported(which, Cin, Cout))
-    return conv_bf16_mfma_workspace_bytes(which, Cin, Cout);
+  if (which != ADH_CONV_BWD_FILTER && conv_bf16_mfma_supported(which, Cin, Cout, H, W))
+    return conv_bf16_mfma_workspace_bytes(which, num_tiles, N, Cin, Cout, H, W);
   const uint64_t slab = (uint64_t)N * Cin * (H + 2) * (W + 2), out = (uint64_t)N * Cout * H * W;
   const uint64_t filt = (uint64_t)Cin * Cout * 9u;
   size_t total = 0;
@@ -123,7 +124,7 @@ int conv_bf16_via_f32(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, u
     if (!in_tiles[t] || !out_tiles[t]) return ADH_ENULL;
     if (!aligned_to(in_tiles[t], 2) || !aligned_to(out_tiles[t], 2)) return ADH_EALIGN;
   }
-  if (conv_bf16_mfma_supported(which, Cin, Cout)) {
+  if (conv_bf16_mfma_supported(which, Cin, Cout, H, W)) {
     // one image is addressed through a 32-bit buffer resource
     const uint64_t cmax = Cin > Cout ? Cin : Cout;
     if (cmax * (H + 2ull) * (W + 2ull) * 2u >= (1ull << 31) || (uint64_t)Cin * Cout * 18u >= (1ull << 31))

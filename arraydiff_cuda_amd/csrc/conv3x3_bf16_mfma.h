@@ -25,8 +25,13 @@ constexpr uint32_t kWtGroupElems = 9u * 2u * 64u * 32u;  // transformed filter e
 struct ConvBf16Params {
   const uint16_t *in[ADH_MAX_TILES];
   uint16_t *out[ADH_MAX_TILES];
-  const uint16_t *wt;       // transformed filter: [group][tap][half][64 out][32 red]
+  const uint16_t *wt;       // transformed filter: [group][pass][tap][half][64 out][32 red]
   uint32_t N, Cred, Cout;   // reduction and output channel counts as the kernel sees them
+  // More than 64 reduction channels take one launch per 64 (a pass): the pass multiplies channels
+  // chan0 .. chan0 + cred_pass - 1 and hands its sums to the next one as fp32 in `part`
+  // ([image][output channel][row][column] per tile); the last pass rounds to bf16 into `out`.
+  uint32_t pass, passes, chan0, cred_pass;
+  float *part[ADH_MAX_TILES];
   uint32_t IH, IW, OH, OW;
   int32_t pad;              // input row/col = output row/col + tap - pad
   float beta;
@@ -52,6 +57,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 
 // the eight-wave kernel: shapes it takes, and its launch (grid.x workgroups per output group)
 bool conv_bf16_w8_takes(const ConvBf16Params &P, uint32_t num_tiles);
+// launches pass P.pass of P.passes
 int conv_bf16_w8_launch(const ConvBf16Params &P, uint32_t gx, uint32_t groups, hipStream_t st);
 
 }  // namespace adh

@@ -44,14 +44,15 @@ __host__ __device__ constexpr int px_slot(int px) { return px + (px >> 3); }
 // filter (Cout, Cin, 3, 3) -> matrix-operand order.  flip = 0 (forward): out = Cout index,
 // red = Cin index, tap as is.  flip = 1 (backward-data): out = Cin index, red = Cout index,
 // tap mirrored.  Channels beyond the real extents are zero.
+// Reduction channels come in passes of 64: wt[group][pass][tap][half][64 out][32 red].
 __global__ __launch_bounds__(256) void conv3x3_bf16_filter_kernel(const uint16_t *__restrict__ w, uint16_t *__restrict__ wt,
                                                                   uint32_t Cin, uint32_t Cout, uint32_t flip,
-                                                                  uint32_t total) {
+                                                                  uint32_t passes, uint32_t total) {
   const uint32_t i = blockIdx.x * 256u + threadIdx.x;
   if (i >= total) return;
   const uint32_t r = i & 31u, o = (i >> 5) & 63u, half = (i >> 11) & 1u;
-  const uint32_t tg = i >> 12, tap = tg % 9u, grp = tg / 9u;
-  const uint32_t oc = grp * 64u + o, rc = half * 32u + r;
+  const uint32_t tg = i >> 12, tap = tg % 9u, gp = tg / 9u, pass = gp % passes, grp = gp / passes;
+  const uint32_t oc = grp * 64u + o, rc = pass * 64u + half * 32u + r;
   uint16_t v = 0;
   if (!flip) {
     if (oc < Cout && rc < Cin) v = w[((uint64_t)oc * Cin + rc) * 9u + tap];
@@ -494,22 +495,47 @@ static int num_cus() {
   return g_num_cus;
 }
 
-bool conv_bf16_mfma_supported(int which, uint32_t Cin, uint32_t Cout) {
+// Up to 64 reduction channels: any shape.  More: one pass of the eight-wave kernel per 64, with fp32 sums between
+// the passes; that kernel needs rows on a 4-byte boundary (forward: even width) or whole 16-byte granules
+// (backward-data: a width that is a multiple of 8), and the sums of one image inside a 2 GiB buffer range.
+bool conv_bf16_mfma_supported(int which, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W) {
   const uint32_t cred = which == ADH_CONV_FWD ? Cin : Cout;
-  return cred <= 64u;
+  if (cred <= 64u) return true;
+  const uint32_t cout_k = which == ADH_CONV_FWD ? Cout : Cin;
+  const uint64_t oh = which == ADH_CONV_FWD ? H : H + 2ull, ow = which == ADH_CONV_FWD ? W : W + 2ull;
+  if (cout_k * oh * ow * 4u >= (1ull << 31)) return false;
+  return which == ADH_CONV_FWD ? (W % 2u) == 0u : (W % 8u) == 0u;
+}
+static uint32_t conv_bf16_passes(int which, uint32_t Cin, uint32_t Cout) {
+  return ((which == ADH_CONV_FWD ? Cin : Cout) + 63u) / 64u;
 }
 
 // name of the kernel a bf16 forward / backward-data call runs, for tiles aligned to 16 bytes
-const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t W, float beta) {
-  if (!conv_bf16_mfma_supported(which, Cin, Cout)) return "widen_bf16_kernel + conv3x3_f32_kernel + narrow_bf16_kernel";
+const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, float beta) {
+  if (!conv_bf16_mfma_supported(which, Cin, Cout, H, W)) return "widen_bf16_kernel + conv3x3_f32_kernel + narrow_bf16_kernel";
+  if (conv_bf16_passes(which, Cin, Cout) > 1u)
+    return beta != 0.f ? "conv3x3_bf16_w8_kernel<true,false,true> + <false,true,true> per middle pass + <false,true,false>"
+                       : "conv3x3_bf16_w8_kernel<false,false,true> + <false,true,true> per middle pass + <false,true,false>";
   const bool w8 = which == ADH_CONV_FWD ? (W % 2u) == 0u : (W % 8u) == 0u;
   if (w8) return beta != 0.f ? "conv3x3_bf16_w8_kernel<true>" : "conv3x3_bf16_w8_kernel<false>";
   return beta != 0.f ? "conv3x3_bf16_kernel<true>" : "conv3x3_bf16_kernel<false>";
 }
 
-size_t conv_bf16_mfma_workspace_bytes(int which, uint32_t Cin, uint32_t Cout) {
+// the reordered filter, then (more than one pass) the fp32 sums of every tile, each region 256-byte aligned
+static size_t filter_region_bytes(int which, uint32_t Cin, uint32_t Cout) {
   const uint32_t cout_k = which == ADH_CONV_FWD ? Cout : Cin;
-  return (size_t)((cout_k + 63u) / 64u) * kWtGroupElems * 2u;
+  return (size_t)((cout_k + 63u) / 64u) * conv_bf16_passes(which, Cin, Cout) * kWtGroupElems * 2u;
+}
+static size_t part_region_bytes(int which, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W) {
+  const uint64_t cout_k = which == ADH_CONV_FWD ? Cout : Cin;
+  const uint64_t oh = which == ADH_CONV_FWD ? H : H + 2ull, ow = which == ADH_CONV_FWD ? W : W + 2ull;
+  return (size_t)((N * cout_k * oh * ow * 4u + 255u) / 256u * 256u);
+}
+size_t conv_bf16_mfma_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                                      uint32_t W) {
+  size_t bytes = filter_region_bytes(which, Cin, Cout);
+  if (conv_bf16_passes(which, Cin, Cout) > 1u) bytes += (size_t)num_tiles * part_region_bytes(which, N, Cin, Cout, H, W);
+  return bytes;
 }
 
 // which = ADH_CONV_FWD: in = x_pad tiles, out = y tiles; ADH_CONV_BWD_DATA: in = dy tiles,
@@ -535,10 +561,19 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
     P.pad = 2;
   }
   const uint32_t groups = (P.Cout + 63u) / 64u;
-  const uint32_t total = groups * kWtGroupElems;
+  P.passes = conv_bf16_passes(which, Cin, Cout);
+  P.pass = 0;
+  P.chan0 = 0;
+  P.cred_pass = P.Cred < 64u ? P.Cred : 64u;
+  if (P.passes > 1u) {
+    uint8_t *part = reinterpret_cast<uint8_t *>(workspace) + filter_region_bytes(which, Cin, Cout);
+    const size_t per_tile = part_region_bytes(which, N, Cin, Cout, H, W);
+    for (uint32_t t = 0; t < num_tiles; ++t) P.part[t] = reinterpret_cast<float *>(part + t * per_tile);
+  }
+  const uint32_t total = groups * P.passes * kWtGroupElems;
   hipLaunchKernelGGL(conv3x3_bf16_filter_kernel, dim3((total + 255u) / 256u), dim3(256), 0, st,
                      reinterpret_cast<const uint16_t *>(w), reinterpret_cast<uint16_t *>(workspace), Cin, Cout,
-                     which == ADH_CONV_FWD ? 0u : 1u, total);
+                     which == ADH_CONV_FWD ? 0u : 1u, P.passes, total);
   int e = launch_status();
   if (e) return e;
 
@@ -569,6 +604,17 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
   P.div_strips = FastDiv(P.strips);
   P.div_N = FastDiv(N);
   P.div_rest = FastDiv(rest ? rest : 1u);
+  if (P.passes > 1u) {
+    // conv_bf16_mfma_supported has checked widths and sizes; what is left is the tiles' alignment
+    if (!conv_bf16_w8_takes(P, num_tiles)) return ADH_EALIGN;
+    for (P.pass = 0; P.pass < P.passes; ++P.pass) {
+      P.chan0 = 64u * P.pass;
+      P.cred_pass = P.Cred - P.chan0 < 64u ? P.Cred - P.chan0 : 64u;
+      e = conv_bf16_w8_launch(P, gx, groups, st);
+      if (e) return e;
+    }
+    return ADH_OK;
+  }
   if (conv_bf16_w8_takes(P, num_tiles)) return conv_bf16_w8_launch(P, gx, groups, st);
   if (beta != 0.f)
     hipLaunchKernelGGL(conv3x3_bf16_kernel<true>, dim3(gx, groups), dim3(256), 0, st, P);
@@ -630,7 +676,7 @@ extern "C" int adh_conv3x3_slab_fwd_tiles_static(int dtype, uint32_t num_tiles, 
   if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
   if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
   // beyond the static array: more than 256 output channels; beyond the matrix-core kernel: more than 64 input channels
-  if (Cout > 64u * kStaticGroups || !conv_bf16_mfma_supported(ADH_CONV_FWD, Cin, Cout)) return ADH_EWORKSPACE;
+  if (Cout > 64u * kStaticGroups || Cin > 64u) return ADH_EWORKSPACE;
   if (N == 0 || Cin == 0 || Cout == 0 || H == 0 || W == 0) return ADH_OK;
   if (!x_pad_tiles || !y_tiles || !w) return ADH_ENULL;
   if (!aligned_to(w, 2)) return ADH_EALIGN;

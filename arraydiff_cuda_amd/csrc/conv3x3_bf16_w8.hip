@@ -60,8 +60,11 @@ static __device__ __forceinline__ u32x2 lds_read_tr(const uint8_t *p) {
 
 static __device__ __forceinline__ uint32_t wrap_slot(uint32_t s) { return s >= (uint32_t)kW8RingRows ? s - (uint32_t)kW8RingRows : s; }
 
-template <bool BETA>
+// BETA: the old output is added (in the first pass).  PIN: the sums of the passes before this one are read from
+// P.part and added.  POUT: the sums go to P.part as fp32 instead of to the output as bf16 (a later pass follows).
+template <bool BETA, bool PIN = false, bool POUT = false>
 __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16Params P) {
+  static_assert(!(BETA && PIN), "the old output is added in the first pass, which reads no sums");
   __shared__ __attribute__((aligned(16))) uint8_t raw[kW8RawBytes];
   __shared__ __attribute__((aligned(16))) uint8_t ring[kW8RingBytes];
 
@@ -81,7 +84,7 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   // this wave's filter share, in B-operand order: lane (n = l16, k-block = g)
   u32x4 wreg[9][2][2];
   {
-    const u32x4 *wt = reinterpret_cast<const u32x4 *>(P.wt + (size_t)grp * kWtGroupElems);
+    const u32x4 *wt = reinterpret_cast<const u32x4 *>(P.wt + ((size_t)grp * P.passes + P.pass) * kWtGroupElems);
 #pragma unroll
     for (int tap = 0; tap < 9; ++tap)
 #pragma unroll
@@ -105,8 +108,8 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     const uint32_t slot = 64u * q + lane;
     const uint32_t row = slot / 72u, rem = slot - row * 72u, ch = rem / 9u, gran = rem - ch * 9u;
     const uint32_t chan = 8u * wv + ch;
-    const bool ok = slot < 288u && chan < P.Cred;
-    ld_off[q] = chan * plane_bytes + row * P.IW * 2u + gran * 16u;
+    const bool ok = slot < 288u && chan < P.cred_pass;
+    ld_off[q] = (P.chan0 + chan) * plane_bytes + row * P.IW * 2u + gran * 16u;
     ld_rows |= ((row & 3u) | (ok ? 4u : 0u)) << (3 * q);
     ld_gran |= gran << (4 * q);
   }
@@ -228,6 +231,13 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   const uint32_t ooff_lane = (co0 * P.OH * P.OW + ocol_lane) * 2u;  // + (row * OW + first column) * 2
   uint16_t *out_imgC = nullptr;
   __amdgpu_buffer_rsrc_t rsrcC = __builtin_amdgcn_make_buffer_rsrc(P.out[0], 0, 0, 0x00020000);
+  // the fp32 sums between passes: the lane's own four columns of accumulator [row][column tile][channel tile]
+  // at (co0 + 16 ct, row, c0 + 32 cw + 16 cti + 4 g): 16 bytes per lane, 64 per output channel and lane row
+  constexpr bool PART = PIN || POUT;
+  const uint32_t poff_lane = (co0 * P.OH * P.OW + 32u * cw + 4u * g) * 4u;  // + (row * OW + first column) * 4
+  const uint32_t pct_bytes = 2u * ct_bytes, prow_bytes = 2u * orow_bytes;
+  float *part_imgC = nullptr;
+  __amdgpu_buffer_rsrc_t rsrcP = __builtin_amdgcn_make_buffer_rsrc(P.out[0], 0, 0, 0x00020000);
   bool wholeC = false;  // every lane of the wave stores eight whole columns of two existing channels
   auto compute_open = [&]() {
     uint32_t tile, n;
@@ -235,6 +245,10 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     stepsC = (int32_t)((r_endC - r_beginC + kStepRows - 1) / kStepRows);
     out_imgC = P.out[tile] + (size_t)n * P.Cout * P.OH * P.OW;
     rsrcC = __builtin_amdgcn_make_buffer_rsrc(out_imgC, 0, out_image_bytes, 0x00020000);
+    if constexpr (PART) {
+      part_imgC = P.part[tile] + (size_t)n * P.Cout * P.OH * P.OW;
+      rsrcP = __builtin_amdgcn_make_buffer_rsrc(part_imgC, 0, 2u * out_image_bytes, 0x00020000);
+    }
     wholeC = __builtin_amdgcn_ballot_w64(!(c0C + ocol_lane + 7u < P.OW && okct[0] && okct[1])) == 0ull;
   };
   compute_open();
@@ -282,6 +296,28 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
       }
   };
 
+  // the fp32 sums between passes, element by element: stored, or added to the accumulators
+  auto part_guarded = [&](floatx4 (&acc)[2][2][2], uint32_t row0, uint32_t nrows, bool store) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+      for (int cti = 0; cti < 2; ++cti)
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct)
+          if ((uint32_t)r < nrows && okct[ct]) {
+            const uint32_t col = c0C + 32u * cw + 16u * cti + 4u * g;
+            float *p = part_imgC + ((size_t)(co0 + 16u * ct) * P.OH + row0 + r) * P.OW + col;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (col + e < P.OW) {
+                if (store)
+                  p[e] = acc[r][cti][ct][e];
+                else
+                  acc[r][cti][ct][e] += p[e];
+              }
+          }
+  };
+
   // The matrix part of a step: 48 operand reads (input row, column shift, channel half, column
   // tile), each fetched kAhead reads before its MFMAs; then the results are packed to bf16 and
   // stored.  Rounds alternate between an input row that feeds one output row of the pair (two
@@ -299,6 +335,9 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     constexpr int BAR = decltype(bar_tag)::value;
     const uint32_t cur_off = ooff_lane + (row0 * P.OW + c0C) * 2u;
     const uint32_t off0 = nrows > 0u ? cur_off : kOutOfRange, off1 = nrows > 1u ? cur_off + orow_bytes : kOutOfRange;
+    const uint32_t pcur = poff_lane + (row0 * P.OW + c0C) * 4u;
+    const uint32_t poff0 = nrows > 0u ? pcur : kOutOfRange, poff1 = nrows > 1u ? pcur + prow_bytes : kOutOfRange;
+    floatx4 pin[2][2];  // [channel tile][column tile]: the earlier passes' sums of the output row being finished
     floatx4 acc[2][2][2];  // [row][column tile][channel tile]
 #pragma unroll
     for (int r = 0; r < 2; ++r)
@@ -306,7 +345,7 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
       for (int cti = 0; cti < 2; ++cti)
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) acc[r][cti][ct] = (floatx4){0.f, 0.f, 0.f, 0.f};
-    constexpr int kReads = 48, kAhead = BETA ? 3 : 4;
+    constexpr int kReads = 48, kAhead = (BETA || PIN) ? 3 : 4;
     const uint8_t *row_ptr[4];
 #pragma unroll
     for (int ir = 0; ir < 4; ++ir) row_ptr[ir] = ring + wrap_slot(sb + 2u * rp + (uint32_t)ir) * kW8RowBytes + read_lane;
@@ -333,7 +372,8 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     }
     // The copies of the group to transpose have landed: everything but the previous step's four
     // stores, which were issued after them (memory instructions complete in order).
-    if (SIDE) __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
+    // (eight stores when the sums go out as fp32)
+    if (SIDE) __builtin_amdgcn_s_waitcnt(POUT ? 0x0F78 : 0x0F74);  // vmcnt(8) : vmcnt(4)
     // packs tile i (row i / 2 of the pair, channel tile i % 2) back to store order through the
     // swap between lane rows and, in the interleaved form, stores it
     auto pack_tile = [&](auto tag) {
@@ -351,6 +391,21 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
         v1[1] += __uint_as_float(s0[1] & 0xffff0000u);
         v1[2] += __uint_as_float(s1[1] << 16);
         v1[3] += __uint_as_float(s1[1] & 0xffff0000u);
+      }
+      if constexpr (PIN && SIDE) {
+        v0 += pin[ct][0];
+        v1 += pin[ct][1];
+      }
+      if constexpr (POUT) {
+        if constexpr (SIDE) {
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v0), rsrcP, r ? poff1 : poff0, ct ? pct_bytes : 0u, 0);
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v1), rsrcP, (r ? poff1 : poff0) + 64u,
+                                                 ct ? pct_bytes : 0u, 0);
+        } else {
+          acc[r][0][ct] = v0;
+          acc[r][1][ct] = v1;
+        }
+        return;
       }
       const u32x2 q0 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[0], v0[1]), pack_bf16x2(v1[0], v1[1]), false, false);
       const u32x2 q1 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[2], v0[3]), pack_bf16x2(v1[2], v1[3]), false, false);
@@ -394,6 +449,20 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
         // rounds 38 and 42: output row 0, complete since round 35, is packed and stored
         if constexpr (t == 38 || t == 42) {
           pack_tile(IntTag<(t - 38) / 4>());
+          __builtin_amdgcn_sched_group_barrier(0x010, POUT ? 2 : 1, 0);
+        }
+        // the earlier passes' sums: output row 0 in rounds 24, 27, 30, 33; row 1 once row 0's have been used
+        // (rounds 39, 40 after the packing in round 38; rounds 43, 44 after the one in round 42)
+        if constexpr (PIN && t >= 24 && (t - 24) % 3 == 0 && t <= 33) {
+          constexpr int i = (t - 24) / 3, ct = i >> 1, cti = i & 1;
+          pin[ct][cti] = __builtin_bit_cast(
+              floatx4, __builtin_amdgcn_raw_buffer_load_b128(rsrcP, poff0 + 64u * cti, ct ? pct_bytes : 0u, 0));
+          __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        }
+        if constexpr (PIN && (t == 39 || t == 40 || t == 43 || t == 44)) {
+          constexpr int ct = t > 41 ? 1 : 0, cti = (t == 40 || t == 44) ? 1 : 0;
+          pin[ct][cti] = __builtin_bit_cast(
+              floatx4, __builtin_amdgcn_raw_buffer_load_b128(rsrcP, poff1 + 64u * cti, ct ? pct_bytes : 0u, 0));
           __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
         }
         // rounds 24, 27, 30, 33: old value (t - 24) / 3 of this step, row 0 first
@@ -413,12 +482,16 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (!SIDE) {
+      if constexpr (PIN) part_guarded(acc, row0, nrows, false);
       for_each_int(std::make_integer_sequence<int, 4>(), pack_tile);
+      if constexpr (POUT)
+        part_guarded(acc, row0, nrows, true);
+      else
+        store_guarded(row0, nrows);
     } else {
       pack_tile(IntTag<2>());
       pack_tile(IntTag<3>());
     }
-    if constexpr (!SIDE) store_guarded(row0, nrows);
   };
 
   // the same side work in one piece, for the phases that cannot take the interleaved form
@@ -498,7 +571,6 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
 // rows on 16 bytes for backward-data, whose granules must lie wholly inside or outside a row),
 // images whose byte offsets fit the buffer range check's 31 bits.
 bool conv_bf16_w8_takes(const ConvBf16Params &P, uint32_t num_tiles) {
-  if (P.Cred > 64u) return false;
   if (P.pad ? (P.IW % 8u) != 0u : (P.IW % 2u) != 0u) return false;
   const uint64_t image_bytes = (uint64_t)P.Cred * P.IH * P.IW * 2u;
   if (image_bytes >= (1ull << 31)) return false;
@@ -506,14 +578,32 @@ bool conv_bf16_w8_takes(const ConvBf16Params &P, uint32_t num_tiles) {
   const size_t a = P.pad ? 16 : 4;
   for (uint32_t t = 0; t < num_tiles; ++t)
     if (!aligned_to(P.in[t], a) || !aligned_to(P.out[t], 4)) return false;
+  if (P.Cred > 64u) {
+    // the fp32 sums between passes are addressed like the output, at four bytes an element
+    if ((uint64_t)P.Cout * P.OH * P.OW * 4u >= (1ull << 31)) return false;
+    for (uint32_t t = 0; t < num_tiles; ++t)
+      if (P.part[t] && !aligned_to(P.part[t], 16)) return false;
+  }
   return true;
 }
 
 int conv_bf16_w8_launch(const ConvBf16Params &P, uint32_t gx, uint32_t groups, hipStream_t st) {
-  if (P.beta != 0.f)
-    hipLaunchKernelGGL(conv3x3_bf16_w8_kernel<true>, dim3(gx, groups), dim3(kW8Threads), 0, st, P);
-  else
-    hipLaunchKernelGGL(conv3x3_bf16_w8_kernel<false>, dim3(gx, groups), dim3(kW8Threads), 0, st, P);
+  const dim3 grid(gx, groups), block(kW8Threads);
+  if (P.passes <= 1u) {
+    if (P.beta != 0.f)
+      hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<true>), grid, block, 0, st, P);
+    else
+      hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false>), grid, block, 0, st, P);
+  } else if (P.pass == 0u) {
+    if (P.beta != 0.f)
+      hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<true, false, true>), grid, block, 0, st, P);
+    else
+      hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, false, true>), grid, block, 0, st, P);
+  } else if (P.pass + 1u < P.passes) {
+    hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, true, true>), grid, block, 0, st, P);
+  } else {
+    hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, true, false>), grid, block, 0, st, P);
+  }
   return launch_status();
 }
 

@@ -28,7 +28,13 @@ def ws_for(which, K, N, Cin, Cout, H, W):
                                               (1, 1, 72, 64, 6, 20), (1, 1, 64, 72, 6, 20), (1, 3, 33, 40, 17, 31),
                                               # widths that are multiples of eight: the bf16 filter-gradient kernel
                                               (1, 2, 16, 24, 5, 8), (2, 1, 64, 64, 9, 72), (1, 1, 40, 48, 3, 136),
-                                              (3, 2, 7, 5, 1, 64), (1, 1, 64, 64, 2, 200)])
+                                              (3, 2, 7, 5, 1, 64), (1, 1, 64, 64, 2, 200),
+                                              # more than 64 reduction channels on the matrix cores: one pass per
+                                              # 64 with fp32 sums in between (two and three passes, a last pass of
+                                              # 36 channels, edge strips, output-channel remainders, both directions)
+                                              (2, 1, 128, 64, 12, 64), (1, 1, 192, 32, 9, 128), (1, 2, 100, 70, 8, 72),
+                                              (1, 1, 160, 16, 5, 16), (2, 1, 64, 128, 12, 64), (1, 1, 48, 130, 6, 24),
+                                              (1, 1, 256, 256, 4, 64)])
 def test_bf16_conv_small_vs_oracle(oracle, K, N, Cin, Cout, H, W):
     rng = np.random.default_rng(77 + Cin)
     bf = lambda a: oracle.f32_to_bf16(a.astype(np.float32))
