@@ -68,7 +68,7 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
                    hipStream_t st);
 
 bool conv_bf16_wgrad_mfma_supported(uint32_t Cin, uint32_t Cout, uint32_t W);
-size_t conv_bf16_wgrad_mfma_workspace_bytes(uint32_t num_tiles, uint32_t N, uint32_t W);
+size_t conv_bf16_wgrad_mfma_workspace_bytes(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t W);
 int conv_bf16_wgrad_mfma(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
                          const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta,
                          void *workspace, hipStream_t st);
@@ -76,7 +76,7 @@ int conv_bf16_wgrad_mfma(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t 
 size_t bf16_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                             uint32_t W, size_t fp32_path_bytes) {
   if (which == ADH_CONV_BWD_FILTER && conv_bf16_wgrad_mfma_supported(Cin, Cout, W))
-    return conv_bf16_wgrad_mfma_workspace_bytes(num_tiles, N, W);
+    return conv_bf16_wgrad_mfma_workspace_bytes(num_tiles, N, Cin, Cout, W);
   if (which != ADH_CONV_BWD_FILTER && conv_bf16_mfma_supported(which, Cin, Cout, H, W))
     return conv_bf16_mfma_workspace_bytes(which, num_tiles, N, Cin, Cout, H, W);
   const uint64_t slab = (uint64_t)N * Cin * (H + 2) * (W + 2), out = (uint64_t)N * Cout * H * W;
@@ -175,9 +175,9 @@ int conv_bf16_filter_via_f32(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint3
   if (conv_bf16_wgrad_mfma_supported(Cin, Cout, W)) {
     if (!workspace) return ADH_ENULL;
     if (!aligned_to(workspace, 256) || !aligned_to(dw, 4)) return ADH_EALIGN;
-    if (workspace_bytes < conv_bf16_wgrad_mfma_workspace_bytes(num_tiles, N, W)) return ADH_EWORKSPACE;
+    if (workspace_bytes < conv_bf16_wgrad_mfma_workspace_bytes(num_tiles, N, Cin, Cout, W)) return ADH_EWORKSPACE;
     // one image is addressed through a 32-bit buffer resource
-    if (64ull * (H + 2ull) * (W + 2ull) * 2u >= (1ull << 31)) return ADH_EINVAL;
+    if ((uint64_t)(Cin > Cout ? Cin : Cout) * (H + 2ull) * (W + 2ull) * 2u >= (1ull << 31)) return ADH_EINVAL;
     for (uint32_t t = 0; t < num_tiles; ++t) {
       if (!x_tiles[t] || !dy_tiles[t]) return ADH_ENULL;
       if (!aligned_to(x_tiles[t], 2) || !aligned_to(dy_tiles[t], 2)) return ADH_EALIGN;

@@ -42,8 +42,11 @@ constexpr uint32_t kWgPartialFloats = 64u * 64u * 9u;
 struct WgradBf16Params {
   const uint16_t *x[ADH_MAX_TILES];
   const uint16_t *dy[ADH_MAX_TILES];
-  float *partial;  // [gridDim.x][8 waves][9 taps][2 output-channel tiles][64 lanes][4]
+  float *partial;  // [gridDim.y][gridDim.x][8 waves][9 taps][2 output-channel tiles][64 lanes][4]
   uint32_t N, Cin, Cout, H, W;
+  // More than 64 channels on either side: blockIdx.y numbers the pairs (block of 64 output channels,
+  // block of 64 input channels), input block fastest; every pair is a problem of its own.
+  uint32_t ci_blocks;
   uint32_t strips, items;
   FastDiv div_strips, div_N;
 };
@@ -88,6 +91,8 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
   // that an XCD works on neighbouring strips: those share the 128-byte lines at strip borders.
   uint32_t vblock = blockIdx.x;
   if ((gridDim.x & 7u) == 0u) vblock = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  const uint32_t co_blk = blockIdx.y / P.ci_blocks, ci_blk = blockIdx.y - co_blk * P.ci_blocks;
+  const uint32_t ci0 = 64u * ci_blk, co0 = 64u * co_blk;
   for (uint32_t item = vblock; item < P.items; item += gridDim.x) {
     uint32_t strip, plane, tile, n;
     P.div_strips.divmod(item, plane, strip);
@@ -113,8 +118,9 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
       const uint32_t ch = j / kWgLanes, piece = j - ch * kWgLanes;
       const uint32_t col = c0 + piece * 8u;
       isx_q[q] = k < 9u;
-      const uint32_t vx = ch < P.Cin ? (ch * HP * WP + col) * 2u : kWgOutOfRange;
-      const uint32_t vd = (ch < P.Cout && piece < 8u && col < P.W) ? (ch * P.H * P.W + col) * 2u : kWgOutOfRange;
+      const uint32_t vx = ci0 + ch < P.Cin ? ((ci0 + ch) * HP * WP + col) * 2u : kWgOutOfRange;
+      const uint32_t vd =
+          (co0 + ch < P.Cout && piece < 8u && col < P.W) ? ((co0 + ch) * P.H * P.W + col) * 2u : kWgOutOfRange;
       voff[q] = isx_q[q] ? vx : vd;
       rows_q[q] = k >= (uint32_t)kWgDmaPerStage ? 0u : (isx_q[q] ? HP : P.H);
       pitch_q[q] = isx_q[q] ? WP * 2u : P.W * 2u;
@@ -244,7 +250,8 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
   // The partial is written in register order, [wave][tap][cot][lane][i], 16 contiguous bytes per
   // lane: in filter order every lane would write lone floats 36 bytes apart, which costs five
   // times the bytes in partial-sector writes.
-  floatx4 *part = reinterpret_cast<floatx4 *>(P.partial + (size_t)blockIdx.x * kWgPartialFloats) + wv * (18u * 64u) + lane;
+  floatx4 *part = reinterpret_cast<floatx4 *>(P.partial + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * kWgPartialFloats) +
+                  wv * (18u * 64u) + lane;
 #pragma unroll
   for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
@@ -258,12 +265,13 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
 // partials in parallel, and scatters the 64 sums to their places in the filter.
 __global__ __launch_bounds__(256) void conv3x3_bf16_wgrad_reduce_kernel(const float *__restrict__ partial,
                                                                         uint32_t num_partials, float *dw, uint32_t Cin,
-                                                                        uint32_t Cout, float beta) {
+                                                                        uint32_t Cout, uint32_t ci_blocks, float beta) {
   __shared__ float part[4][64];
   const uint32_t q = threadIdx.x >> 6, j = threadIdx.x & 63u;
   const uint32_t e = blockIdx.x * 64u + j;  // < kWgPartialFloats: the grid covers it exactly
+  const uint32_t co_blk = blockIdx.y / ci_blocks, ci_blk = blockIdx.y - co_blk * ci_blocks;
   {
-    const float *p = partial + e;
+    const float *p = partial + (size_t)blockIdx.y * num_partials * kWgPartialFloats + e;
     const uint32_t per = (num_partials + 3u) / 4u;
     const uint32_t b0 = q * per, b1 = min(b0 + per, num_partials);
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
@@ -282,7 +290,8 @@ __global__ __launch_bounds__(256) void conv3x3_bf16_wgrad_reduce_kernel(const fl
     // e = (((wave * 9 + tap) * 2 + cot) * 64 + lane) * 4 + i
     const uint32_t i = e & 3u, lane = (e >> 2) & 63u, cot = (e >> 8) & 1u;
     const uint32_t wt = e >> 9, tap = wt % 9u, wave = wt / 9u;
-    const uint32_t co = 32u * (wave >> 2) + 16u * cot + 4u * (lane >> 4) + i, ci = 16u * (wave & 3u) + (lane & 15u);
+    const uint32_t co = 64u * co_blk + 32u * (wave >> 2) + 16u * cot + 4u * (lane >> 4) + i;
+    const uint32_t ci = 64u * ci_blk + 16u * (wave & 3u) + (lane & 15u);
     if (co < Cout && ci < Cin) {
       float *d = dw + ((size_t)co * Cin + ci) * 9u + tap;
       float r = (part[0][j] + part[1][j]) + (part[2][j] + part[3][j]);
@@ -301,15 +310,16 @@ static uint32_t wgrad_bf16_blocks(uint64_t items) {
 }
 
 bool conv_bf16_wgrad_mfma_supported(uint32_t Cin, uint32_t Cout, uint32_t W) {
-  return Cin <= 64u && Cout <= 64u && (W % 8u) == 0u;
+  return (W % 8u) == 0u && (uint64_t)((Cin + 63u) / 64u) * ((Cout + 63u) / 64u) <= 65535u;
 }
 
 static uint64_t wgrad_bf16_items(uint32_t num_tiles, uint32_t N, uint32_t W) {
   return (uint64_t)num_tiles * N * ((W + kWgCols - 1) / kWgCols);
 }
 
-size_t conv_bf16_wgrad_mfma_workspace_bytes(uint32_t num_tiles, uint32_t N, uint32_t W) {
-  return (size_t)wgrad_bf16_blocks(wgrad_bf16_items(num_tiles, N, W)) * kWgPartialFloats * sizeof(float);
+size_t conv_bf16_wgrad_mfma_workspace_bytes(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t W) {
+  const size_t pairs = (size_t)((Cin + 63u) / 64u) * ((Cout + 63u) / 64u);
+  return pairs * wgrad_bf16_blocks(wgrad_bf16_items(num_tiles, N, W)) * kWgPartialFloats * sizeof(float);
 }
 
 // Arguments are validated by the caller (pointers, alignment, workspace size, extents > 0).
@@ -330,11 +340,13 @@ int conv_bf16_wgrad_mfma(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t 
   P.div_strips = FastDiv(P.strips);
   P.div_N = FastDiv(N);
   const uint32_t blocks = wgrad_bf16_blocks(items);
-  hipLaunchKernelGGL(conv3x3_bf16_wgrad_kernel, dim3(blocks), dim3(512), 0, st, P);
+  P.ci_blocks = (Cin + 63u) / 64u;
+  const uint32_t pairs = P.ci_blocks * ((Cout + 63u) / 64u);
+  hipLaunchKernelGGL(conv3x3_bf16_wgrad_kernel, dim3(blocks, pairs), dim3(512), 0, st, P);
   int e = launch_status();
   if (e) return e;
-  hipLaunchKernelGGL(conv3x3_bf16_wgrad_reduce_kernel, dim3(kWgPartialFloats / 64u), dim3(256), 0, st,
-                     reinterpret_cast<const float *>(workspace), blocks, dw, Cin, Cout, beta);
+  hipLaunchKernelGGL(conv3x3_bf16_wgrad_reduce_kernel, dim3(kWgPartialFloats / 64u, pairs), dim3(256), 0, st,
+                     reinterpret_cast<const float *>(workspace), blocks, dw, Cin, Cout, P.ci_blocks, beta);
   return launch_status();
 }
 
