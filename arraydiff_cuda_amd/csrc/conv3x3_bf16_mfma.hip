@@ -514,10 +514,10 @@ static uint32_t conv_bf16_passes(int which, uint32_t Cin, uint32_t Cout) {
 const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, float beta) {
   if (!conv_bf16_mfma_supported(which, Cin, Cout, H, W)) return "widen_bf16_kernel + conv3x3_f32_kernel + narrow_bf16_kernel";
   if (conv_bf16_passes(which, Cin, Cout) > 1u)
-    return beta != 0.f ? "conv3x3_bf16_w8_kernel<true,false,true> + <false,true,true> per middle pass + <false,true,false>"
-                       : "conv3x3_bf16_w8_kernel<false,false,true> + <false,true,true> per middle pass + <false,true,false>";
+    return beta != 0.f ? "conv3x3_bf16_w8_kernel<true, false, true> + <false, true, true> per middle pass + <false, true, false>"
+                       : "conv3x3_bf16_w8_kernel<false, false, true> + <false, true, true> per middle pass + <false, true, false>";
   const bool w8 = which == ADH_CONV_FWD ? (W % 2u) == 0u : (W % 8u) == 0u;
-  if (w8) return beta != 0.f ? "conv3x3_bf16_w8_kernel<true>" : "conv3x3_bf16_w8_kernel<false>";
+  if (w8) return beta != 0.f ? "conv3x3_bf16_w8_kernel<true, false, false>" : "conv3x3_bf16_w8_kernel<false, false, false>";
   return beta != 0.f ? "conv3x3_bf16_kernel<true>" : "conv3x3_bf16_kernel<false>";
 }
 
