@@ -54,10 +54,13 @@ struct ConvParams {
   uint32_t tiles_x;         // ceil(OW / TW); grid.x = tiles_x * ceil(OH / R)
   uint32_t w_out_stride, w_red_stride;  // weight address = o*w_out_stride + k*w_red_stride + tap'
   int32_t w_flip;           // tap' = w_flip ? 8 - tap : tap
-  // forward over the row tiles of one activation, in rank order: input row 0 of tile t > 0 is read
-  // from tile t-1's last interior row and input row IH-1 of tile t < num_tiles-1 from tile t+1's
-  // first interior row, which is what a halo exchange would have copied there
-  int32_t rows_from_neighbours;
+  // The tiles are the row tiles of one activation, in rank order, and two input rows come from the
+  // neighbouring tiles: row nb_lo of tile t > 0 is tile t-1's row nb_above, row nb_hi of tile
+  // t < num_tiles-1 is tile t+1's row nb_below.  Forward (padded input whose inner halo rows nobody
+  // exchanged): rows 0 and IH-1 are the neighbours' last and first interior rows, IH-2 and 1.
+  // Backward-data (unpadded dy): rows -1 and IH are the neighbours' rows IH-1 and 0, which makes
+  // the interior of the gradient tile complete, as after a halo reduce.
+  int32_t rows_from_neighbours, nb_lo, nb_hi, nb_above, nb_below;
   float beta;
   FastDiv div_tiles_x, div_TW;
 };
@@ -140,19 +143,21 @@ __global__ __launch_bounds__(64 * WAVES, 1) void conv3x3_f32_kernel(const ConvPa
   for (int rr = 0; rr < RROWS; ++rr) {
     const uint32_t prow = wv + (uint32_t)WAVES * rr;
     int32_t ih = (int32_t)(oh0 + prow) - P.pad;
-    const bool ok = col_ok && prow < patch_rows && ih >= 0 && ih < (int32_t)P.IH;
+    const bool ok = col_ok && prow < patch_rows;
     const float *src = in;
+    bool ok_row = ih >= 0 && ih < (int32_t)P.IH;
     if (P.rows_from_neighbours) {
-      const int32_t interior = (int32_t)P.IH - 2;
-      if (ih == 0 && t > 0u) {
+      if (ih == P.nb_lo && t > 0u) {
         src = P.in[t - 1u] + (uint64_t)n * P.Cred * in_plane;
-        ih = interior;
-      } else if (ih == (int32_t)P.IH - 1 && t + 1u < P.num_tiles) {
+        ih = P.nb_above;
+        ok_row = true;
+      } else if (ih == P.nb_hi && t + 1u < P.num_tiles) {
         src = P.in[t + 1u] + (uint64_t)n * P.Cred * in_plane;
-        ih = 1;
+        ih = P.nb_below;
+        ok_row = true;
       }
     }
-    row_voff[rr] = ok ? ((uint32_t)ih * P.IW + (uint32_t)iw) * 4u : kOutOfRange;
+    row_voff[rr] = ok && ok_row ? ((uint32_t)ih * P.IW + (uint32_t)iw) * 4u : kOutOfRange;
     rsrc_row[rr] = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(src), 0,
                                                      (int)(P.Cred * (uint32_t)in_plane * 4u), kBufferFlags);
   }
@@ -418,7 +423,12 @@ static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uin
   P.num_tiles = num_tiles;
   P.N = N;
   P.beta = beta;
-  P.rows_from_neighbours = (which == ADH_CONV_FWD && rows_from_neighbours) ? 1 : 0;
+  P.rows_from_neighbours = rows_from_neighbours ? 1 : 0;
+  if (which == ADH_CONV_FWD) {
+    P.nb_lo = 0; P.nb_hi = (int32_t)H + 1; P.nb_above = (int32_t)H; P.nb_below = 1;
+  } else {
+    P.nb_lo = -1; P.nb_hi = (int32_t)H; P.nb_above = (int32_t)H - 1; P.nb_below = 0;
+  }
   if (which == ADH_CONV_FWD) {
     P.Cred = Cin; P.Cout = Cout;
     P.IH = (uint32_t)HP; P.IW = (uint32_t)WP; P.OH = H; P.OW = W;
@@ -527,6 +537,22 @@ int adh_conv3x3_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, u
                              workspace, workspace_bytes, as_stream(stream));
   return conv_direct(ADH_CONV_BWD_DATA, dtype, num_tiles, N, Cin, Cout, H, W, dy_tiles, w, dx_pad_tiles, beta,
                      as_stream(stream));
+}
+
+int adh_conv3x3_slab_bwd_data_tiles_reduced(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                            uint32_t H, uint32_t W, const void *w, const void *const *dy_tiles,
+                                            void *const *dx_pad_tiles, float beta, void *workspace,
+                                            size_t workspace_bytes, void *stream) {
+  if (dtype == ADH_BF16) {
+    // the bf16 kernels stream their rows from one image: the ordinary backward-data, then the reduce
+    if (beta != 0.f) return ADH_EUNIMPL;  // a reduce after accumulating would add the old halo rows again
+    const int rc = adh_conv3x3_slab_bwd_data_tiles(dtype, num_tiles, N, Cin, Cout, H, W, w, dy_tiles, dx_pad_tiles, beta,
+                                                   workspace, workspace_bytes, stream);
+    if (rc != ADH_OK) return rc;
+    return adh_halo_reduce_nchw(dtype, 1, num_tiles, 1, W, H, Cin, N, dx_pad_tiles, stream);
+  }
+  return conv_direct(ADH_CONV_BWD_DATA, dtype, num_tiles, N, Cin, Cout, H, W, dy_tiles, w, dx_pad_tiles, beta,
+                     as_stream(stream), true);
 }
 
 int adh_conv3x3_slab_bwd_data(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,

@@ -830,9 +830,10 @@ private:
 template <typename V>
 class HaloExch2DOp : public virtual Op {
 public:
-  // forward_by_consumer (not in the reference): the forward pass copies nothing, because the consumer is a
-  // convolution built with Conv2DShape::unexchanged_rows, which reads the neighbours' rows itself; the
-  // backward pass (the halo reduce of the gradient) is unchanged.
+  // forward_by_consumer (not in the reference): neither pass launches anything, because the consumer is a
+  // convolution built with Conv2DShape::unexchanged_rows: its forward pass reads the neighbours' rows itself
+  // and its input gradient arrives reduced (the neighbours' gradient rows are multiplied by the tile that
+  // owns the result).
   static vector<shared_ptr<Var<V>>> MakeParallel(size_t halo_pad, vector<shared_ptr<Var<V>>> inputs,
                                                  shared_ptr<Context> ctx, bool forward_by_consumer = false) {
     auto op = make_shared<HaloExch2DOp<V>>(halo_pad, inputs, ctx, forward_by_consumer);
@@ -897,7 +898,9 @@ public:
   // whose inner halo rows nobody exchanged (HaloExch2DOp made with forward_by_consumer): the forward
   // pass and the filter gradient read those rows from the neighbouring tiles, or exchange them first
   // where the kernel for the shape cannot (or where the ranks' filters differ, so that one launch cannot
-  // hold every tile).
+  // hold every tile); the input gradient comes out as after the halo reduce (by a kernel that reads the
+  // neighbours' gradient rows, or by a reduce after the ordinary one).  The input gradient must have no
+  // other contributor.
   bool unexchanged_rows = false;
 };
 

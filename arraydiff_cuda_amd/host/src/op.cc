@@ -368,6 +368,7 @@ void HaloExch2DOp<V3>::_backward(TxnId txn) {
   }
   if (num_writes != 0 && num_writes != ctx->num_ranks()) throw HazardError("HaloExch2DOp: some ranks already reduced");
   if (num_writes == 0) return;
+  if (forward_by_consumer_) return;  // the consuming convolution's input gradient arrives reduced
   for (size_t r = 0; r < ctx->num_ranks(); ++r) {
     V3 &g = xs_.at(r).grad().get_mut(txn, id());
     check_padded(g, halo_pad_, "HaloExch2DOp");
@@ -595,6 +596,7 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
   // a transaction overwrites (beta = 0) instead: same values, one pass over the buffer instead of three.
   todo.clear();
   bool fresh[ADH_MAX_TILES] = {};
+  bool reduce_after = false;  // unexchanged rows, but a kernel that cannot read across tiles: reduce once at the end
   for (size_t r = 0; r < K; ++r) {
     if (!x_vars_[r]->_requires_grad()) continue;  // e.g. the first layer: nobody wants the image's gradient
     GPUContext *dc = rank_ctx(ctx_, r);
@@ -630,7 +632,18 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
     const float beta = first ? 0.0f : 1.0f;
-    if (use_3x3_kernels(*this, d, n, shape_.filters)) {
+    const bool in_kernel_rows = n == K && reads_neighbour_rows(*this, shape_, d, n);
+    if (shape_.unexchanged_rows && !in_kernel_rows) {
+      // a halo reduce after this pass would add what the halo rows held before it a second time
+      if (!first || n != K) throw HazardError("SlabConv2DOp: unexchanged rows need the input gradient to themselves");
+      reduce_after = true;
+    }
+    if (in_kernel_rows) {
+      // the neighbours' edge rows of dy are multiplied here: the interior comes out as after a halo reduce
+      adh_check(adh_conv3x3_slab_bwd_data_tiles_reduced(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, w0, dyt,
+                                                        dxt, beta, nullptr, 0, conn.stream()),
+                "SlabConv2DOp::_backward (data, reduced)");
+    } else if (use_3x3_kernels(*this, d, n, shape_.filters)) {
       adh_check(adh_conv3x3_slab_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, w0, dyt, dxt,
                                                 beta, nullptr, 0, conn.stream()),
                 "SlabConv2DOp::_backward (data)");
@@ -642,6 +655,9 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
                                                conn.stream()),
                 "SlabConv2DOp::_backward (data, general)");
     }
+    if (reduce_after)
+      adh_check(adh_halo_reduce_nchw(ADH_F32, 1, n, 1, d.W, d.H, d.C, d.N, dxt, conn.stream()),
+                "SlabConv2DOp::_backward (reduce)");
     todo.swap(rest);
   }
 }

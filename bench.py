@@ -377,6 +377,15 @@ def main():
             lambda: lib.adh_conv3x3_slab_bwd_data_tiles(0, K, N, C, C, Ht, W, wt.data_ptr(), dy_tbl, g_tbl, 0.0, None,
                                                         0, stream),
             "mfma", flops_step, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+        add("conv bwd-data cfg3 with the halo reduce folded in (4 tiles, one launch)",
+            lambda: lib.adh_conv3x3_slab_bwd_data_tiles_reduced(0, K, N, C, C, Ht, W, wt.data_ptr(), dy_tbl, g_tbl, 0.0,
+                                                                None, 0, stream),
+            "mfma", flops_step, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+        add("conv bwd-data cfg3 + halo reduce (two launches: what the one above replaces)",
+            lambda: (lib.adh_conv3x3_slab_bwd_data_tiles(0, K, N, C, C, Ht, W, wt.data_ptr(), dy_tbl, g_tbl, 0.0, None, 0,
+                                                         stream),
+                     lib.adh_halo_reduce_nchw(0, 1, K, p, W, Ht, C, N, g_tbl, stream))[1],
+            "mfma", flops_step, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
         add("conv bwd-filter cfg3 (4 tiles, two kernels)",
             lambda: lib.adh_conv3x3_slab_bwd_filter_tiles(0, K, N, C, C, Ht, W, tile_tbl, dy_tbl, gw.data_ptr(), 0.0,
                                                           ws.data_ptr(), ws_bytes, stream),

@@ -188,6 +188,19 @@ int adh_conv3x3_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, u
                                     uint32_t H, uint32_t W, const void *w, const void *const *dy_tiles,
                                     void *const *dx_pad_tiles, float beta, void *workspace,
                                     size_t workspace_bytes, void *stream);
+/* cudnnConvolutionBackwardData of the conv (src/op.cc:1701-1712) and HaloExch2DOp::_backward of
+ * its producer (the halo reduce, src/op.cc:3009-3052) in one launch: dy_tiles are the row tiles of
+ * ONE gradient in rank order (a 1 x num_tiles grid, halo width 1).  The interior of every
+ * dx_pad tile equals adh_conv3x3_slab_bwd_data_tiles followed by adh_halo_reduce_nchw up to the
+ * order of the additions (tile t also multiplies the last dy row of tile t-1 and the first of tile
+ * t+1); the inner halo rows of dx_pad hold partial sums nobody should read (HaloPad2DOp's
+ * backward reads the interior).  fp32: one launch, any beta in {0, 1}.  bf16: backward-data, then
+ * the reduce (two launches; beta = 1 returns ADH_EUNIMPL). */
+int adh_conv3x3_slab_bwd_data_tiles_reduced(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,
+                                            uint32_t Cout, uint32_t H, uint32_t W, const void *w,
+                                            const void *const *dy_tiles, void *const *dx_pad_tiles,
+                                            float beta, void *workspace, size_t workspace_bytes,
+                                            void *stream);
 /* cudnnConvolutionBackwardFilter at src/op.cc:1660-1671:
  * dw[co,ci,kh,kw] = beta*dw + sum_{tiles,n,h,w} dy[n,co,h,w] * x_pad[n,ci,h+kh,w+kw]
  * (the sum over tiles is what ParallelSGDOptimizer's ncclReduce did across ranks,

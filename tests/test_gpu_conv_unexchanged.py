@@ -1,4 +1,5 @@
-"""The exchange-free forms of the 3x3 slab convolution: forward and filter gradient over row tiles whose
+"""The exchange-free forms of the 3x3 slab convolution (the input gradient that needs no halo reduce is further
+down): forward and filter gradient over row tiles whose
 inner halo rows were never exchanged must equal halo exchange followed by the ordinary entry point, bit for
 bit (same kernels, same order of additions, only the address of two input rows per tile differs), and the
 fp32 forms must not read the inner halo rows at all (they hold NaN here).  One case is also checked against
@@ -79,6 +80,51 @@ def test_filter_gradient_equals_exchange_then_filter_gradient(K, N, Cin, Cout, H
                    "wgrad unexchanged")
         assert not torch.isnan(got).any()
         assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,H,W", SHAPES)
+def test_reduced_input_gradient_equals_backward_data_then_reduce(K, N, Cin, Cout, H, W):
+    rng = np.random.default_rng(4500 + K * 7 + Cin)
+    w = dev(he_normal(rng, Cout, Cin))
+    dys = [dev(rng.standard_normal((N, Cout, H, W)).astype(np.float32)) for _ in range(K)]
+    g0 = [dev(rng.standard_normal((N, Cin, H + 2, W + 2)).astype(np.float32)) for _ in range(K)]
+    for beta in (0.0, 1.0):
+        # the two-launch form: backward-data into a cleared buffer, halo reduce, then the accumulation
+        part = [torch.zeros_like(g) for g in g0]
+        capi.check(capi.conv_bwd_data_tiles(w, dys, part, N, Cin, Cout, H, W), "bwd-data")
+        if H >= 2:
+            capi.check(capi.halo_reduce(part, 1, K, 1, W, H, Cin, N), "reduce")
+        want = [p + beta * g for p, g in zip(part, g0)]
+        got = [g.clone() for g in g0]
+        capi.check(capi.conv_bwd_data_tiles(w, dys, got, N, Cin, Cout, H, W, beta=beta, reduced=True), "bwd-data reduced")
+        for r in range(K):
+            if H >= 2:
+                # same terms in another order of additions: fp32 tolerance 1e-5 of the largest value
+                # (interior columns: the reduce moves the W interior columns of a halo row, the halo columns of
+                # the gradient are read by nobody)
+                assert rel_err(host(got[r][:, :, 1:-1, 1:-1]), host(want[r][:, :, 1:-1, 1:-1])) <= 1e-5
+            # outer halo rows have no neighbour: the plain backward-data's values
+            if r == 0:
+                assert rel_err(host(got[r][:, :, 0, :]), host(want[r][:, :, 0, :])) <= 1e-5
+            if r == K - 1:
+                assert rel_err(host(got[r][:, :, -1, :]), host(want[r][:, :, -1, :])) <= 1e-5
+
+
+def test_reduced_input_gradient_vs_unsplit_oracle(oracle):
+    """The interiors of the K gradient tiles, stitched, are the unsplit convolution's input gradient."""
+    K, N, Cin, Cout, Ht, W = 4, 2, 6, 10, 5, 12
+    H = K * Ht
+    rng = np.random.default_rng(4600)
+    w = he_normal(rng, Cout, Cin)
+    dy = rng.standard_normal((N, Cout, H, W)).astype(np.float32)
+    want = np.zeros((N, Cin, H + 2, W + 2), np.float32)
+    oracle.conv_slab_bwd_data(w, dy, want)
+    dys = [dev(dy[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    gs = [torch.empty((N, Cin, Ht + 2, W + 2), device="cuda") for _ in range(K)]
+    capi.check(capi.conv_bwd_data_tiles(dev(w), dys, gs, N, Cin, Cout, Ht, W, reduced=True), "bwd-data reduced")
+    for r in range(K):
+        got = host(gs[r])[:, :, 1:-1, :]
+        assert rel_err(got, want[:, :, 1 + r * Ht:1 + (r + 1) * Ht, :]) <= 1e-5
 
 
 def test_forward_and_filter_gradient_vs_oracle(oracle):
