@@ -130,3 +130,98 @@ def test_batchnorm_random(oracle, K, N, C, H, W, relu, p):
             scale = max(float(np.abs(dx).max()), 1e-3)
             assert np.max(np.abs(np.where(keep, host(dxs[r]) - dx, 0))) <= 5e-5 * max(scale, 1.0) * max(1.0, float(i.max()) / 10)
         np.testing.assert_allclose(host(dsh[r]), db, rtol=1e-4, atol=1e-4 * max(1.0, float(np.abs(db).max())))
+
+
+def _row_tile_cases(seed, count, max_c):
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        out.append((int(rng.integers(1, 6)), int(rng.integers(1, 4)), int(rng.integers(1, max_c + 1)),
+                    int(rng.integers(1, max_c + 1)), int(rng.integers(1, 12)), int(rng.integers(1, 90))))
+    return out
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,Ht,W", _row_tile_cases(2027, 20, 40))
+def test_conv_over_row_tiles_without_halo_kernels_random(oracle, K, N, Cin, Cout, Ht, W):
+    """Forward over unexchanged tiles, the filter gradient over them and the input gradient with the reduce folded
+    in, against the UNSPLIT convolution of the stitched tensors (fp32, rel-err <= 1e-5)."""
+    rng = np.random.default_rng(K * 1000 + W)
+    H = K * Ht
+    x = rng.uniform(-1, 1, size=(N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))).astype(np.float32)
+    dy = rng.standard_normal((N, Cout, H, W)).astype(np.float32)
+    xp = np.zeros((N, Cin, H + 2, W + 2), np.float32)
+    xp[:, :, 1:-1, 1:-1] = x
+    y = np.empty((N, Cout, H, W), np.float32)
+    oracle.conv_slab_fwd(xp, w, y)
+    gx = np.empty_like(xp)
+    oracle.conv_slab_bwd_data(w, dy, gx)
+    gw = np.zeros_like(w)
+    oracle.conv_slab_bwd_filter(xp, dy, gw)
+    # tiles as after HaloPad2DOp: zero halo, nothing exchanged
+    xs = []
+    for r in range(K):
+        t = np.zeros((N, Cin, Ht + 2, W + 2), np.float32)
+        t[:, :, 1:-1, 1:-1] = x[:, :, r * Ht:(r + 1) * Ht, :]
+        xs.append(dev(t))
+    dys = [dev(dy[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    ys = [torch.full((N, Cout, Ht, W), float("nan"), device="cuda") for _ in range(K)]
+    gs = [torch.full((N, Cin, Ht + 2, W + 2), float("nan"), device="cuda") for _ in range(K)]
+    d_gw = torch.full((Cout, Cin, 3, 3), float("nan"), device="cuda")
+    nbytes = capi.conv_workspace_bytes(capi.ADH_CONV_BWD_FILTER, capi.ADH_F32, K, N, Cin, Cout, Ht, W)
+    ws = torch.empty(max(nbytes // 4, 1), device="cuda")
+    capi.check(capi.conv_fwd_tiles(xs, dev(w), ys, N, Cin, Cout, Ht, W, unexchanged=True))
+    capi.check(capi.conv_bwd_data_tiles(dev(w), dys, gs, N, Cin, Cout, Ht, W, reduced=True))
+    capi.check(capi.conv_bwd_filter_tiles(xs, dys, d_gw, N, Cin, Cout, Ht, W, ws=ws, unexchanged=True))
+    for r in range(K):
+        assert rel_err(host(ys[r]), y[:, :, r * Ht:(r + 1) * Ht, :]) <= 1e-5
+        assert rel_err(host(gs[r])[:, :, 1:-1, 1:-1], gx[:, :, 1 + r * Ht:1 + (r + 1) * Ht, 1:-1]) <= 1e-5
+    assert rel_err(host(d_gw), gw) <= 1e-5
+
+
+def _bf16_wide_cases(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        out.append((int(rng.integers(1, 4)), int(rng.integers(1, 3)), int(rng.integers(1, 200)), int(rng.integers(1, 200)),
+                    int(rng.integers(1, 11)), 8 * int(rng.integers(1, 12))))
+    return out
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,H,W", _bf16_wide_cases(2028, 16))
+def test_bf16_conv_random_channel_counts(oracle, K, N, Cin, Cout, H, W):
+    """bf16 forward, backward-data (beta 0 and 1) and filter gradient on the matrix cores for channel counts on
+    both sides of 64 and 128 (passes of 64 reduction channels, 64 x 64 pairs for the filter gradient), widths that
+    are multiples of 8.  Tolerances as in test_gpu_conv_bf16.py."""
+    rng = np.random.default_rng(Cin * 211 + Cout)
+    bf = lambda a: oracle.f32_to_bf16(a.astype(np.float32))
+    xs = [bf(rng.uniform(-1, 1, size=(N, Cin, H + 2, W + 2))) for _ in range(K)]
+    w = bf(rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9)))
+    dys = [bf(rng.standard_normal((N, Cout, H, W))) for _ in range(K)]
+    g0 = [bf(rng.standard_normal((N, Cin, H + 2, W + 2))) for _ in range(K)]
+    wf = oracle.bf16_to_f32(w)
+
+    def ws_for(which):
+        return torch.empty(capi.conv_workspace_bytes(which, capi.ADH_BF16, K, N, Cin, Cout, H, W) // 4 + 64, device="cuda")
+
+    d_xs, d_dys, d_w = [dev(a) for a in xs], [dev(a) for a in dys], dev(w)
+    ys = [torch.empty((N, Cout, H, W), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
+    gs = [torch.empty((N, Cin, H + 2, W + 2), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
+    ga = [dev(a) for a in g0]
+    dw = torch.full((Cout, Cin, 3, 3), float("nan"), device="cuda")
+    capi.check(capi.conv_fwd_tiles(d_xs, d_w, ys, N, Cin, Cout, H, W, ws=ws_for(capi.ADH_CONV_FWD)))
+    capi.check(capi.conv_bwd_data_tiles(d_w, d_dys, gs, N, Cin, Cout, H, W, ws=ws_for(capi.ADH_CONV_BWD_DATA)))
+    capi.check(capi.conv_bwd_data_tiles(d_w, d_dys, ga, N, Cin, Cout, H, W, beta=1.0, ws=ws_for(capi.ADH_CONV_BWD_DATA)))
+    capi.check(capi.conv_bwd_filter_tiles(d_xs, d_dys, dw, N, Cin, Cout, H, W, ws=ws_for(capi.ADH_CONV_BWD_FILTER)))
+    dw_want = np.zeros((Cout, Cin, 3, 3), np.float32)
+    for r in range(K):
+        xf, dyf = oracle.bf16_to_f32(xs[r]), oracle.bf16_to_f32(dys[r])
+        y = np.empty((N, Cout, H, W), np.float32)
+        oracle.conv_slab_fwd(xf, wf, y)
+        assert rel_err(oracle.bf16_to_f32(host(ys[r])), y) <= 5e-3
+        g = np.empty((N, Cin, H + 2, W + 2), np.float32)
+        oracle.conv_slab_bwd_data(wf, dyf, g)
+        assert rel_err(oracle.bf16_to_f32(host(gs[r])), g) <= 5e-3
+        assert rel_err(oracle.bf16_to_f32(host(ga[r])), g + oracle.bf16_to_f32(g0[r])) <= 5e-3
+        oracle.conv_slab_bwd_filter(xf, dyf, dw_want, beta=1.0)
+    assert rel_err(host(dw), dw_want) <= 1e-4
