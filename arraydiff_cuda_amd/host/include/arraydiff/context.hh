@@ -123,6 +123,9 @@ public:
   void begin();
   void end();
   void replay();
+  // ends a recording left open (the destructor calls it: an exception between begin() and end() leaves
+  // the stream usable)
+  void abort();
   size_t num_nodes() const { return num_nodes_; }
 
 private:

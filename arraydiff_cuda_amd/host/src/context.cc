@@ -70,6 +70,12 @@ shared_ptr<GPUMemory<uint8_t>> GPUContext::get_scratch() {
 
 void GPUContext::reserve_scratch(size_t min_scratch_size) {
   if (min_scratch_size <= scratch_size_) return;
+  // growing the scratch synchronises and reallocates, neither of which a stream that is being recorded
+  // into a graph allows: say so instead of invalidating the recording with an opaque error
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream_, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone)
+    throw std::logic_error("GPUContext::reserve_scratch: the scratch would grow while the stream is being recorded; "
+                           "run one step eagerly first");
   scratch_size_ = (min_scratch_size + 4095) / 4096 * 4096;
   if (scratch_) {
     sync();  // work queued on the old scratch must finish before it is released
@@ -106,8 +112,19 @@ Spatial2DComm *MultiGPUContext::spatial_comm(size_t rank) {
 }
 
 StreamCapture::~StreamCapture() {
+  abort();
   if (exec_) (void)hipGraphExecDestroy(exec_);
   if (graph_) (void)hipGraphDestroy(graph_);
+}
+// Ends a recording that is still open (an exception between begin() and end()) and drops what it held, so that
+// the stream is usable again.
+void StreamCapture::abort() {
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream_, &capturing) != hipSuccess || capturing == hipStreamCaptureStatusNone) return;
+  hipGraph_t partial = nullptr;
+  (void)hipStreamEndCapture(stream_, &partial);
+  if (partial) (void)hipGraphDestroy(partial);
+  (void)hipGetLastError();
 }
 void StreamCapture::begin() {
   if (graph_ || exec_) throw std::logic_error("StreamCapture: already recorded");

@@ -6,7 +6,9 @@
 //   train_resnet18 [--ranks K] [--batch N] [--size S] [--steps T] [--warmup W] [--classes C]
 //                  [--lr a] [--nesterov 0|1] [--graph 0|1]
 // --graph 1: after the warm-up steps one step (forward, backward, optimizer) is recorded as a HIP graph and
-// the timed steps replay it; the step size is constant here, so the replays compute what eager steps would.
+// the timed steps replay it; the step size and momentum are kernel arguments, fixed when the step is recorded,
+// and the optimizer's iteration counter does not advance during replays: this is right only because both
+// schedules are constant here (a varying schedule needs eager steps, or a new recording per value).
 #include <chrono>
 #include <cmath>
 #include <cstdio>
