@@ -189,3 +189,39 @@ def test_config5_highres_bf16_fwd_bwd_sampled(oracle):
                 errs.append(abs(gwh[co_, ci_, a, b] - ref1))
                 mags.append(abs(ref1))
     assert max(errs) / max(mags) <= 1e-3
+
+
+@pytest.mark.parametrize("dtype,K,N,C,Ht,W,eps", [(torch.bfloat16, 8, 2, 64, 128, 2048, 2.0 ** -9),
+                                                  (torch.bfloat16, 4, 1, 128, 64, 512, 2.0 ** -9),
+                                                  (torch.float32, 4, 32, 64, 14, 56, 2.0 ** -20)])
+def test_three_passes_agree_on_one_number(dtype, K, N, C, Ht, W, eps):
+    """<dy, conv(x, w)> = <x_pad, conv_bwd_data(w, dy)> = <w, conv_bwd_filter(x_pad, dy)>: the three kernels compute
+    the same trilinear form, at the full high-resolution configuration too (a size-independent check that ties
+    forward, backward-data and backward-filter together; a wrong tap, a transposed filter or a dropped row or
+    channel in any one of them breaks an equality).  The sums run in float64 on the GPU over the stored outputs.
+    The terms dy*y have random signs, so the number itself is a random-walk sum of size sqrt(sum (dy*y)^2), and each
+    stored output carries an independent relative rounding error eps (bf16: 2^-9; fp32: the order of its 576 or
+    1152 additions, 2^-20): the three numbers may differ by a few eps * sqrt(sum (dy*y)^2), six of which are
+    allowed.  One tap, row or channel dropped in one kernel moves its number by a tenth of that root or more."""
+    g = torch.Generator(device="cuda").manual_seed(31)
+    xs = [(torch.rand((N, C, Ht + 2, W + 2), device="cuda", generator=g) * 2 - 1).to(dtype) for _ in range(K)]
+    dys = [torch.randn((N, C, Ht, W), device="cuda", generator=g).to(dtype) for _ in range(K)]
+    w = (torch.randn((C, C, 3, 3), device="cuda", generator=g) * (2.0 / (C * 9)) ** 0.5).to(dtype)
+    code = capi.ADH_BF16 if dtype == torch.bfloat16 else capi.ADH_F32
+    nbytes = max(capi.conv_workspace_bytes(wh, code, K, N, C, C, Ht, W)
+                 for wh in (capi.ADH_CONV_FWD, capi.ADH_CONV_BWD_DATA, capi.ADH_CONV_BWD_FILTER))
+    ws = torch.empty(nbytes // 4 + 64, device="cuda")
+    ys = [torch.empty((N, C, Ht, W), device="cuda", dtype=dtype) for _ in range(K)]
+    gs = [torch.empty((N, C, Ht + 2, W + 2), device="cuda", dtype=dtype) for _ in range(K)]
+    gw = torch.empty((C, C, 3, 3), device="cuda")
+    capi.check(capi.conv_fwd_tiles(xs, w, ys, N, C, C, Ht, W, ws=ws))
+    capi.check(capi.conv_bwd_data_tiles(w, dys, gs, N, C, C, Ht, W, ws=ws))
+    capi.check(capi.conv_bwd_filter_tiles(xs, dys, gw, N, C, C, Ht, W, ws=ws))
+    dot = lambda a, b: float((a.double() * b.double()).sum())
+    via_fwd = sum(dot(dy, y) for dy, y in zip(dys, ys))
+    via_data = sum(dot(x, gx) for x, gx in zip(xs, gs))
+    via_filter = dot(w, gw)
+    walk = sum(float(((dy.double() * y.double()) ** 2).sum()) for dy, y in zip(dys, ys)) ** 0.5
+    assert abs(via_fwd) < 6.0 * walk  # sanity of the scale itself
+    assert abs(via_fwd - via_data) <= 6.0 * eps * walk
+    assert abs(via_fwd - via_filter) <= 6.0 * eps * walk
