@@ -32,6 +32,9 @@ struct ConvBf16Params {
   // ([image][output channel][row][column] per tile); the last pass rounds to bf16 into `out`.
   uint32_t pass, passes, chan0, cred_pass;
   float *part[ADH_MAX_TILES];
+  // the eight-wave kernel reads the filter as the caller holds it (no transformed copy): forward, a
+  // multiple of 64 input channels, 16-byte aligned; else null
+  const uint16_t *w_direct;
   uint32_t IH, IW, OH, OW;
   int32_t pad;              // input row/col = output row/col + tap - pad
   float beta;

@@ -570,12 +570,17 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
     const size_t per_tile = part_region_bytes(which, N, Cin, Cout, H, W);
     for (uint32_t t = 0; t < num_tiles; ++t) P.part[t] = reinterpret_cast<float *>(part + t * per_tile);
   }
-  const uint32_t total = groups * P.passes * kWtGroupElems;
-  hipLaunchKernelGGL(conv3x3_bf16_filter_kernel, dim3((total + 255u) / 256u), dim3(256), 0, st,
-                     reinterpret_cast<const uint16_t *>(w), reinterpret_cast<uint16_t *>(workspace), Cin, Cout,
-                     which == ADH_CONV_FWD ? 0u : 1u, P.passes, total);
-  int e = launch_status();
-  if (e) return e;
+  // the forward pass of the eight-wave kernel can read the caller's filter itself
+  const bool direct = which == ADH_CONV_FWD && (Cin % 64u) == 0u && aligned_to(w, 16) && (P.IW % 2u) == 0u;
+  int e = ADH_OK;
+  if (!direct) {
+    const uint32_t total = groups * P.passes * kWtGroupElems;
+    hipLaunchKernelGGL(conv3x3_bf16_filter_kernel, dim3((total + 255u) / 256u), dim3(256), 0, st,
+                       reinterpret_cast<const uint16_t *>(w), reinterpret_cast<uint16_t *>(workspace), Cin, Cout,
+                       which == ADH_CONV_FWD ? 0u : 1u, P.passes, total);
+    e = launch_status();
+    if (e) return e;
+  }
 
   const uint32_t cus = (uint32_t)num_cus();
   P.strips = (P.OW + kStripCols - 1) / kStripCols;
@@ -604,6 +609,17 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
   P.div_strips = FastDiv(P.strips);
   P.div_N = FastDiv(N);
   P.div_rest = FastDiv(rest ? rest : 1u);
+  if (direct && conv_bf16_w8_takes(P, num_tiles)) {
+    P.w_direct = reinterpret_cast<const uint16_t *>(w);
+  } else if (direct) {
+    // the four-wave kernel takes this shape after all (tile alignment): it needs the transformed copy
+    const uint32_t total = groups * P.passes * kWtGroupElems;
+    hipLaunchKernelGGL(conv3x3_bf16_filter_kernel, dim3((total + 255u) / 256u), dim3(256), 0, st,
+                       reinterpret_cast<const uint16_t *>(w), reinterpret_cast<uint16_t *>(workspace), Cin, Cout, 0u,
+                       P.passes, total);
+    e = launch_status();
+    if (e) return e;
+  }
   if (P.passes > 1u) {
     // conv_bf16_mfma_supported has checked widths and sizes; what is left is the tiles' alignment
     if (!conv_bf16_w8_takes(P, num_tiles)) return ADH_EALIGN;

@@ -83,7 +83,42 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
 
   // this wave's filter share, in B-operand order: lane (n = l16, k-block = g)
   u32x4 wreg[9][2][2];
-  {
+  if (P.w_direct) {
+    // Straight from the filter as the caller holds it (forward, (Cout, Cin, 3, 3), Cin a multiple of 64, 16-byte
+    // aligned): the lane's eight reduction channels x nine taps of one output channel are 72 consecutive
+    // elements, nine aligned 16-byte loads; what is left is to turn [channel][tap] into [tap][channel] in
+    // registers, one byte permute per dword.  No reordering kernel runs before this one.
+    const __amdgpu_buffer_rsrc_t rsrcW = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(P.w_direct), 0, (int)(P.Cout * P.Cred * 18u), 0x00020000);
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+      for (int ct = 0; ct < 2; ++ct) {
+        const uint32_t co = grp * 64u + 32u * h + 16u * ct + l16;
+        const uint32_t ci = P.chan0 + 32u * half + 8u * g;
+        // an output channel that does not exist lies past the end of the filter and loads as zero
+        const uint32_t off = co < P.Cout ? (co * P.Cred + ci) * 18u : kOutOfRange;
+        uint32_t d[36];
+#pragma unroll
+        for (int q = 0; q < 9; ++q) {
+          const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrcW, off, 16 * q, 0);
+          d[4 * q + 0] = v[0]; d[4 * q + 1] = v[1]; d[4 * q + 2] = v[2]; d[4 * q + 3] = v[3];
+        }
+        // element k = 9 * channel + tap sits in dword k / 2, half k % 2
+#pragma unroll
+        for (int tap = 0; tap < 9; ++tap) {
+          u32x4 r;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int klo = 18 * j + tap, khi = klo + 9;
+            // v_perm_b32 picks bytes from {first operand: bytes 4-7, second operand: bytes 0-3}
+            const uint32_t sel = ((khi & 1) ? 0x07060000u : 0x05040000u) | ((klo & 1) ? 0x00000302u : 0x00000100u);
+            r[j] = __builtin_amdgcn_perm(d[khi >> 1], d[klo >> 1], sel);
+          }
+          wreg[tap][half][ct] = r;
+        }
+      }
+  } else {
     const u32x4 *wt = reinterpret_cast<const u32x4 *>(P.wt + ((size_t)grp * P.passes + P.pass) * kWtGroupElems);
 #pragma unroll
     for (int tap = 0; tap < 9; ++tap)

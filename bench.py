@@ -225,7 +225,7 @@ def main():
         "config": {"workload": "configs[4]: 3x3 slab conv fwd, bf16 in / fp32 accumulate, NCHW N=2 Cin=Cout=64, "
                                "1024x2048 image in 8 row-tiles of 128(+2)x2048(+2), one call over all tiles",
                    "flops_per_step": flops5, "tiles": K5, "halo": 1},
-        "roofline": {"kernel": name5 + " (fwd; the call also runs the 2 us filter reordering kernel)", "bound": "mfma",
+        "roofline": {"kernel": name5 + " (fwd; the only kernel of the call: it reads the filter as the caller holds it)", "bound": "mfma",
                      "achieved": round(achieved, 3), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": CONV_FWD_CFG5_TRAFFIC[1] if name5 == CONV_FWD_CFG5_TRAFFIC[0] else None,
