@@ -47,6 +47,8 @@ SIGNATURES = {
     "adh_conv3x3_slab_fwd_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_fwd_tiles_unexchanged": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_data_tiles_reduced": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
+    "adh_conv3x3_unpadded_fwd_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp, sz, vp]),
+    "adh_conv3x3_unpadded_bwd_data_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_fwd_tiles_static": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp]),
     "adh_conv3x3_slab_bwd_data": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_data_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
@@ -261,6 +263,25 @@ def conv_bwd_data_tiles(w, dys, dxs, N, Cin, Cout, H, W, beta=0.0, ws=None, redu
     wp, wb = _ws(ws)
     fn = lib().adh_conv3x3_slab_bwd_data_tiles_reduced if reduced else lib().adh_conv3x3_slab_bwd_data_tiles
     return fn(_dt(dys[0]), len(dys), N, Cin, Cout, H, W, w.data_ptr(), dt, xt, beta, wp, wb, _stream())
+
+
+def conv_unpadded_fwd_tiles(xs, w, ys, N, Cin, Cout, H, W, beta=0.0, ws=None):
+    """xs, ys: the row tiles (H x W, no halo) of one tensor in rank order."""
+    _dev(w, *xs, *ys)
+    xt, k1 = _tbl(xs)
+    yt, k2 = _tbl(ys)
+    wp, wb = _ws(ws)
+    return lib().adh_conv3x3_unpadded_fwd_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, xt, w.data_ptr(), yt, beta, wp,
+                                                wb, _stream())
+
+
+def conv_unpadded_bwd_data_tiles(w, dys, dxs, N, Cin, Cout, H, W, beta=0.0, ws=None):
+    _dev(w, *dys, *dxs)
+    dt, k1 = _tbl(dys)
+    xt, k2 = _tbl(dxs)
+    wp, wb = _ws(ws)
+    return lib().adh_conv3x3_unpadded_bwd_data_tiles(_dt(dys[0]), len(dys), N, Cin, Cout, H, W, w.data_ptr(), dt, xt,
+                                                     beta, wp, wb, _stream())
 
 
 def conv2d_workspace_bytes(which, dtype, K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw):

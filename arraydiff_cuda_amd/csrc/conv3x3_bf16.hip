@@ -65,7 +65,7 @@ size_t conv_bf16_mfma_workspace_bytes(int which, uint32_t num_tiles, uint32_t N,
                                       uint32_t W);
 int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
                    const void *const *in_tiles, const void *w, void *const *out_tiles, float beta, void *workspace,
-                   hipStream_t st);
+                   hipStream_t st, bool halofree = false);
 
 bool conv_bf16_wgrad_mfma_supported(uint32_t Cin, uint32_t Cout, uint32_t W);
 size_t conv_bf16_wgrad_mfma_workspace_bytes(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t W);

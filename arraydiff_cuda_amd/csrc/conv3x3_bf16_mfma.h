@@ -35,6 +35,8 @@ struct ConvBf16Params {
   // the eight-wave kernel reads the filter as the caller holds it (no transformed copy): forward, a
   // multiple of 64 input channels, 16-byte aligned; else null
   const uint16_t *w_direct;
+  // the eight-wave kernel over tiles without halo (pad 1): rows -1 and IH come from the neighbouring tiles
+  uint32_t neighbour_rows, num_tiles;
   uint32_t IH, IW, OH, OW;
   int32_t pad;              // input row/col = output row/col + tap - pad
   float beta;

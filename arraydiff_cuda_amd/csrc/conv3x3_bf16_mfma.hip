@@ -540,9 +540,13 @@ size_t conv_bf16_mfma_workspace_bytes(int which, uint32_t num_tiles, uint32_t N,
 
 // which = ADH_CONV_FWD: in = x_pad tiles, out = y tiles; ADH_CONV_BWD_DATA: in = dy tiles,
 // out = dx_pad tiles.  Arguments are validated by the caller.
+// halofree: no tile carries a halo (in and out are H x W), the tiles are the row tiles of one tensor in rank order
+// and a tile's rows -1 and H are its neighbours' last and first rows (zeros at the tensor's own border): the
+// unsplit convolution with zero padding, restricted to the tile.  Only shapes the eight-wave kernel takes
+// (ADH_EUNIMPL otherwise).
 int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
                    const void *const *in_tiles, const void *w, void *const *out_tiles, float beta, void *workspace,
-                   hipStream_t st) {
+                   hipStream_t st, bool halofree) {
   ConvBf16Params P = {};
   for (uint32_t t = 0; t < num_tiles; ++t) {
     P.in[t] = reinterpret_cast<const uint16_t *>(in_tiles[t]);
@@ -560,6 +564,12 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
     P.IH = H; P.IW = W; P.OH = H + 2; P.OW = W + 2;
     P.pad = 2;
   }
+  if (halofree) {
+    P.IH = P.OH = H; P.IW = P.OW = W;
+    P.pad = 1;
+    P.neighbour_rows = 1;
+    P.num_tiles = num_tiles;
+  }
   const uint32_t groups = (P.Cout + 63u) / 64u;
   P.passes = conv_bf16_passes(which, Cin, Cout);
   P.pass = 0;
@@ -570,6 +580,7 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
     const size_t per_tile = part_region_bytes(which, N, Cin, Cout, H, W);
     for (uint32_t t = 0; t < num_tiles; ++t) P.part[t] = reinterpret_cast<float *>(part + t * per_tile);
   }
+  if (halofree && !conv_bf16_w8_takes(P, num_tiles)) return ADH_EUNIMPL;
   // the forward pass of the eight-wave kernel can read the caller's filter itself
   const bool direct = which == ADH_CONV_FWD && (Cin % 64u) == 0u && aligned_to(w, 16) && (P.IW % 2u) == 0u;
   int e = ADH_OK;
@@ -705,6 +716,55 @@ extern "C" int adh_conv3x3_slab_fwd_tiles_static(int dtype, uint32_t num_tiles, 
   void *ws = nullptr;
   const int e = static_scratch(&ws);
   if (e) return e;
-  return conv_bf16_mfma(ADH_CONV_FWD, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, w, y_tiles, beta, ws, as_stream(stream));
+  return conv_bf16_mfma(ADH_CONV_FWD, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, w, y_tiles, beta, ws, as_stream(stream),
+                        false);
 }
 
+// ---------------------------------------------------------------------------
+// convolution over row tiles that carry no halo
+// ---------------------------------------------------------------------------
+namespace {
+int unpadded_entry(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                   const void *const *in_tiles, const void *w, void *const *out_tiles, float beta, void *workspace,
+                   size_t workspace_bytes, void *stream) {
+  using namespace adh;
+  if (!dtype_ok(dtype)) return ADH_EINVAL;
+  if (dtype != ADH_BF16) return ADH_EUNIMPL;
+  if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
+  if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
+  if (N == 0 || Cin == 0 || Cout == 0 || H == 0 || W == 0) return ADH_OK;
+  if (!in_tiles || !out_tiles || !w) return ADH_ENULL;
+  if ((W % 8u) != 0u) return ADH_EUNIMPL;  // whole 16-byte granules per row
+  if (!aligned_to(w, 2)) return ADH_EALIGN;
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!in_tiles[t] || !out_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(in_tiles[t], 16) || !aligned_to(out_tiles[t], 4)) return ADH_EALIGN;
+  }
+  const uint64_t cmax = Cin > Cout ? Cin : Cout;
+  if (cmax * (H + 2ull) * (W + 2ull) * 2u >= (1ull << 31) || (uint64_t)Cin * Cout * 18u >= (1ull << 31)) return ADH_EINVAL;
+  if (!conv_bf16_mfma_supported(which, Cin, Cout, H, W)) return ADH_EUNIMPL;
+  // the same workspace as the padded entry point of this pass (the transformed filter; the sums between passes)
+  const size_t need = conv_bf16_mfma_workspace_bytes(which, num_tiles, N, Cin, Cout, H, W);
+  if (!workspace) return ADH_ENULL;
+  if (!aligned_to(workspace, 256)) return ADH_EALIGN;
+  if (workspace_bytes < need) return ADH_EWORKSPACE;
+  return conv_bf16_mfma(which, num_tiles, N, Cin, Cout, H, W, in_tiles, w, out_tiles, beta, workspace, as_stream(stream),
+                        true);
+}
+}  // namespace
+
+extern "C" int adh_conv3x3_unpadded_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                              uint32_t H, uint32_t W, const void *const *x_tiles, const void *w,
+                                              void *const *y_tiles, float beta, void *workspace, size_t workspace_bytes,
+                                              void *stream) {
+  return unpadded_entry(ADH_CONV_FWD, dtype, num_tiles, N, Cin, Cout, H, W, x_tiles, w, y_tiles, beta, workspace,
+                        workspace_bytes, stream);
+}
+
+extern "C" int adh_conv3x3_unpadded_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                                   uint32_t H, uint32_t W, const void *w, const void *const *dy_tiles,
+                                                   void *const *dx_tiles, float beta, void *workspace,
+                                                   size_t workspace_bytes, void *stream) {
+  return unpadded_entry(ADH_CONV_BWD_DATA, dtype, num_tiles, N, Cin, Cout, H, W, dy_tiles, w, dx_tiles, beta, workspace,
+                        workspace_bytes, stream);
+}

@@ -62,11 +62,19 @@ static __device__ __forceinline__ uint32_t wrap_slot(uint32_t s) { return s >= (
 
 // BETA: the old output is added (in the first pass).  PIN: the sums of the passes before this one are read from
 // P.part and added.  POUT: the sums go to P.part as fp32 instead of to the output as bf16 (a later pass follows).
-template <bool BETA, bool PIN = false, bool POUT = false>
+// HF (P.pad == 1): neither the input nor the output carries a halo.  An output strip of 64 columns then needs
+// input columns c0 - 1 .. c0 + 64, one more than the nine granules from c0 - 8 hold: the 32 lanes that copy 4
+// leaves idle fetch the tenth granule of every row and channel into the idle tail of the staging area, and a
+// sixth transposing read turns its first pixel into ring pixel 72 (rows of 73 pixels).  Rows -1 and IH come
+// from the neighbouring tiles (P.neighbour_rows).
+template <bool BETA, bool PIN = false, bool POUT = false, bool HF = false>
 __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16Params P) {
   static_assert(!(BETA && PIN), "the old output is added in the first pass, which reads no sums");
+  constexpr int kRowBytes = (HF ? kW8RowPx + 1 : kW8RowPx) * kW8PxBytes;
+  constexpr int kRingBytes = kW8RingRows * kRowBytes;
+  constexpr int kGroups = HF ? 6 : 5;  // transposing read pairs (and ring writes) per row group
   __shared__ __attribute__((aligned(16))) uint8_t raw[kW8RawBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t ring[kW8RingBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t ring[kRingBytes];
 
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
@@ -131,7 +139,9 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
 
   const uint32_t plane_bytes = P.IH * P.IW * 2u;
   const uint32_t image_bytes = P.Cred * plane_bytes;
-  const uint32_t xoff = P.pad ? 6u : 0u;        // ring pixel of the strip's first output column at tap column 0
+  // ring pixel of the strip's first output column at tap column 0: the staged row starts eight columns left of
+  // the strip whenever the input has no halo of its own (pad 1: unpadded in and out; pad 2: backward-data into a padded slab)
+  const uint32_t xoff = P.pad ? 8u - (uint32_t)P.pad : 0u;
   const int32_t col_back = P.pad ? 8 : 0;       // the staged row starts this many columns left of the strip
 
   // ---- requests: copy q of a group moves staging slots 64 q + lane; slot = (row * 8 + channel) * 9 + granule
@@ -141,9 +151,14 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
 #pragma unroll
   for (int q = 0; q < kW8Copies; ++q) {
     const uint32_t slot = 64u * q + lane;
-    const uint32_t row = slot / 72u, rem = slot - row * 72u, ch = rem / 9u, gran = rem - ch * 9u;
+    uint32_t row = slot / 72u, rem = slot - row * 72u, ch = rem / 9u, gran = rem - ch * 9u;
+    if (HF && slot >= 288u) {  // the tenth granule: slot 288 + 8 row + channel
+      row = (slot - 288u) >> 3;
+      ch = slot & 7u;
+      gran = 9u;
+    }
     const uint32_t chan = 8u * wv + ch;
-    const bool ok = slot < 288u && chan < P.cred_pass;
+    const bool ok = (HF || slot < 288u) && chan < P.cred_pass;
     ld_off[q] = (P.chan0 + chan) * plane_bytes + row * P.IW * 2u + gran * 16u;
     ld_rows |= ((row & 3u) | (ok ? 4u : 0u)) << (3 * q);
     ld_gran |= gran << (4 * q);
@@ -161,6 +176,10 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   const uint32_t wr03 = (16u * g + l16) * kW8PxBytes + wv * 16u;             // + slot(row t) * kW8RowBytes
   const uint32_t wr4 = (64u + l16) * kW8PxBytes + wv * 16u;                  // + slot(row g) * kW8RowBytes
   uint8_t *const wr4_dummy = raw_wave + 288 * 16 + ((l16 & 7u) + 8u * g) * 16u;
+  // HF, round 5: row g's tenth granule, [channel][8 pixels] at slot 288 + 8 g + channel; lane 0 of the group
+  // receives its first pixel (the reads of the other lanes run on into the next slots and are not used)
+  const uint8_t *const tr5 = raw_wave + (288u + 8u * g + (l16 >> 2)) * 16u + (l16 & 3u) * 8u;
+  const uint32_t wr5 = (uint32_t)kW8RowPx * kW8PxBytes + wv * 16u;           // + slot(row g) * kRowBytes
 
   uint32_t tb = 0;  // ring slot the next transposed group starts at
   struct TrPair { u32x2 lo, hi; };
@@ -169,19 +188,24 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     if constexpr (t < 4) {
       T.lo = lds_read_tr(tr03 + t * 8 * kW8RawCh);
       T.hi = lds_read_tr(tr03 + t * 8 * kW8RawCh + 4 * kW8RawCh);
-    } else {
+    } else if constexpr (t == 4) {
       T.lo = lds_read_tr(tr4);
       T.hi = lds_read_tr(tr4 + 4 * kW8RawCh);
+    } else {
+      T.lo = lds_read_tr(tr5);
+      T.hi = lds_read_tr(tr5 + 4 * 16);
     }
   };
   auto tr_write = [&](auto tag, const TrPair &T) {
     constexpr int t = decltype(tag)::value;
     const u32x4 v = {T.lo[0], T.lo[1], T.hi[0], T.hi[1]};
     if constexpr (t < 4) {
-      *reinterpret_cast<u32x4 *>(ring + wrap_slot(tb + (uint32_t)t) * kW8RowBytes + wr03) = v;
-    } else {
-      uint8_t *const dst = ring + wrap_slot(tb + g) * kW8RowBytes + wr4;
+      *reinterpret_cast<u32x4 *>(ring + wrap_slot(tb + (uint32_t)t) * kRowBytes + wr03) = v;
+    } else if constexpr (t == 4) {
+      uint8_t *const dst = ring + wrap_slot(tb + g) * kRowBytes + wr4;
       *reinterpret_cast<u32x4 *>(l16 < 8u ? dst : wr4_dummy) = v;
+    } else {
+      if (l16 == 0u) *reinterpret_cast<u32x4 *>(ring + wrap_slot(tb + g) * kRowBytes + wr5) = v;
     }
   };
 
@@ -192,6 +216,10 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   int32_t arow0L = 0, colL = 0;          // input row of ring-relative row 0, input column of staged pixel 0
   uint32_t okL = 0;                      // 5 bits: copy q of this lane exists for this item (slot, channel, granule column)
   __amdgpu_buffer_rsrc_t rsrcL = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(P.in[0]), 0, 0, 0x00020000);
+  // P.neighbour_rows: the tiles are the row tiles of one tensor in rank order and carry no halo; input row -1 of
+  // tile t > 0 is the last row of tile t - 1 and input row IH of tile t < tiles - 1 the first row of tile t + 1
+  __amdgpu_buffer_rsrc_t rsrcUp = rsrcL, rsrcDn = rsrcL;
+  bool hasUpL = false, hasDnL = false;
 
   // decodes a work number into (tile, image, first column, first and last output row)
   auto decode = [&](uint32_t work, uint32_t &tile, uint32_t &n, uint32_t &c0, uint32_t &r_begin, uint32_t &r_end) {
@@ -220,6 +248,15 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     colL = (int32_t)c0 - col_back;
     const uint16_t *in_img = P.in[tile] + (size_t)n * P.Cred * P.IH * P.IW;
     rsrcL = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(in_img), 0, image_bytes, 0x00020000);
+    if (P.neighbour_rows) {
+      hasUpL = tile > 0u;
+      hasDnL = tile + 1u < P.num_tiles;
+      const size_t img_off = (size_t)n * P.Cred * P.IH * P.IW;
+      rsrcUp = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(P.in[hasUpL ? tile - 1u : tile] + img_off), 0,
+                                                 image_bytes, 0x00020000);
+      rsrcDn = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(P.in[hasDnL ? tile + 1u : tile] + img_off), 0,
+                                                 image_bytes, 0x00020000);
+    }
     okL = 0;
 #pragma unroll
     for (int q = 0; q < kW8Copies; ++q) {
@@ -231,14 +268,39 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   };
   // Copy q of the loader's current group.  Once all work has been requested okL is zero and the
   // copies only write zeros, which go to ring rows nobody reads: the sequence needs no branches.
-  auto request = [&](auto tag) {
+  // NBR: the group holds a row that comes from a neighbouring tile.  A copy instruction has one buffer, so the
+  // lanes of that row take an instruction of their own with the neighbour's (lanes that are switched off write
+  // nothing to LDS); one image plane further on or back turns row -1 into the neighbour's last row and row IH
+  // into its first.
+  auto request = [&](auto tag, auto nbr_tag) {
     constexpr int q = decltype(tag)::value;
+    constexpr bool NBR = decltype(nbr_tag)::value != 0;
     const int32_t first = arow0L + 4 * grpL + 2;   // input row of the group's first row
     const int32_t base = (first * (int32_t)P.IW + colL) * 2;
     const int32_t arow = first + (int32_t)((ld_rows >> (3 * q)) & 3u);
     const bool ok = ((okL >> q) & 1u) && (uint32_t)arow < P.IH;
     const uint32_t v = ok ? ld_off[q] + (uint32_t)base : kOutOfRange;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcL, (ADH_LDS void *)(raw_wave + q * 1024), 16, v, 0, 0, 0);
+    if constexpr (!NBR) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcL, (ADH_LDS void *)(raw_wave + q * 1024), 16, v, 0, 0, 0);
+    } else {
+      const bool slot = ((okL >> q) & 1u) != 0u;
+      const bool up = slot && hasUpL && arow == -1, dn = slot && hasDnL && arow == (int32_t)P.IH;
+      if (up) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcUp, (ADH_LDS void *)(raw_wave + q * 1024), 16,
+                                                 ld_off[q] + (uint32_t)base + plane_bytes, 0, 0, 0);
+      } else if (dn) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcDn, (ADH_LDS void *)(raw_wave + q * 1024), 16,
+                                                 ld_off[q] + (uint32_t)base - plane_bytes, 0, 0, 0);
+      } else {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcL, (ADH_LDS void *)(raw_wave + q * 1024), 16, v, 0, 0, 0);
+      }
+    }
+  };
+  // does the group the loader stands at hold a neighbour's row?  (the same in every lane)
+  auto group_has_neighbour_row = [&]() -> bool {
+    if (!P.neighbour_rows || workL >= total) return false;
+    const int32_t first = arow0L + 4 * grpL + 2;
+    return (hasUpL && first <= -1 && -1 <= first + 3) || (hasDnL && first <= (int32_t)P.IH && (int32_t)P.IH <= first + 3);
   };
   auto loader_advance = [&]() {
     if (workL >= total) return;
@@ -363,7 +425,7 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   // of the row group that has landed, the five copies of the next group, and for beta = 1 the
   // four loads of old values (buffer loads and stores: a row that does not exist gets an
   // out-of-range offset, so the sequence has no branches).
-  auto compute = [&](uint32_t sb, auto side_tag, auto bar_tag, uint32_t row0, uint32_t nrows, bool barrier_owed) {
+  auto compute = [&](uint32_t sb, auto side_tag, auto bar_tag, auto nbr_tag, uint32_t row0, uint32_t nrows, bool barrier_owed) {
     constexpr bool SIDE = decltype(side_tag)::value != 0;
     // 1: this phase's barrier comes between the rounds and the packing; 2: the previous phase's barrier, if still
     // owed, comes after the first operand fetches (row pair 0 only: they read rows that step shares with this one)
@@ -380,10 +442,10 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
       for (int cti = 0; cti < 2; ++cti)
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) acc[r][cti][ct] = (floatx4){0.f, 0.f, 0.f, 0.f};
-    constexpr int kReads = 48, kAhead = (BETA || PIN) ? 3 : 4;
+    constexpr int kReads = 48, kAhead = HF ? ((BETA || PIN) ? 2 : 2) : ((BETA || PIN) ? 3 : 4);
     const uint8_t *row_ptr[4];
 #pragma unroll
-    for (int ir = 0; ir < 4; ++ir) row_ptr[ir] = ring + wrap_slot(sb + 2u * rp + (uint32_t)ir) * kW8RowBytes + read_lane;
+    for (int ir = 0; ir < 4; ++ir) row_ptr[ir] = ring + wrap_slot(sb + 2u * rp + (uint32_t)ir) * kRowBytes + read_lane;
     u32x4 abuf[kAhead + 1];
     TrPair trp[2];
     // round t reads input row 0, 1, 0, 1, .. for t < 24 (two and four MFMAs in turn), then row 2
@@ -467,19 +529,20 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
       }
       __builtin_amdgcn_sched_group_barrier(0x008, 2 * (kh_hi - kh_lo + 1), 0);
       if constexpr (SIDE) {
-        // rounds 0, 2, .., 8: transposing read pair t / 2; rounds 3, 5, .., 11: ring write (t - 3) / 2
-        if constexpr (t % 2 == 0 && t <= 8) {
+        // rounds 0, 2, .., 8 (HF: 10): transposing read pair t / 2; rounds 3, 5, .., 11 (13): ring write (t - 3) / 2
+        if constexpr (t % 2 == 0 && t <= 2 * (kGroups - 1)) {
           tr_read(IntTag<t / 2>(), trp[(t / 2) % 2]);
           __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         }
-        if constexpr (t >= 3 && t % 2 == 1 && t <= 11) {
+        if constexpr (t >= 3 && t % 2 == 1 && t <= 2 * kGroups + 1) {
           tr_write(IntTag<(t - 3) / 2>(), trp[((t - 3) / 2) % 2]);
           __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
-        // rounds 13, 15, .., 21: copy (t - 13) / 2 of the next row group (every transposing read has returned)
-        if constexpr (t >= 13 && t % 2 == 1 && t <= 21) {
-          request(IntTag<(t - 13) / 2>());
-          __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        // rounds 13, 15, .., 21 (HF: 15 .. 23): copy of the next row group (every transposing read has returned)
+        constexpr int kReq0 = HF ? 15 : 13;
+        if constexpr (t >= kReq0 && t % 2 == 1 && t <= kReq0 + 8) {
+          request(IntTag<(t - kReq0) / 2>(), nbr_tag);
+          if constexpr (!decltype(nbr_tag)::value) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
         }
         // rounds 38 and 42: output row 0, complete since round 35, is packed and stored
         if constexpr (t == 38 || t == 42) {
@@ -532,10 +595,10 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   // the same side work in one piece, for the phases that cannot take the interleaved form
   auto move_rows_plain = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    TrPair T[5];
-    for_each_int(std::make_integer_sequence<int, 5>(), [&](auto tag) { tr_read(tag, T[decltype(tag)::value]); });
-    for_each_int(std::make_integer_sequence<int, 5>(), [&](auto tag) { tr_write(tag, T[decltype(tag)::value]); });
-    for_each_int(std::make_integer_sequence<int, 5>(), [&](auto tag) { request(tag); });
+    TrPair T[kGroups];
+    for_each_int(std::make_integer_sequence<int, kGroups>(), [&](auto tag) { tr_read(tag, T[decltype(tag)::value]); });
+    for_each_int(std::make_integer_sequence<int, kGroups>(), [&](auto tag) { tr_write(tag, T[decltype(tag)::value]); });
+    for_each_int(std::make_integer_sequence<int, 5>(), [&](auto tag) { request(tag, IntTag<HF ? 1 : 0>()); });
   };
 
   // One phase per step, plus one without MFMAs at the start of every item and a second one at the
@@ -545,7 +608,7 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   // ones read in it.
   uint32_t sb = 4;  // ring slot of the first input row of the step multiplied in this phase
   loader_open();
-  for_each_int(std::make_integer_sequence<int, 5>(), [&](auto tag) { request(tag); });
+  for_each_int(std::make_integer_sequence<int, 5>(), [&](auto tag) { request(tag, IntTag<HF ? 1 : 0>()); });
   loader_advance();
   // Every wave passes one barrier per phase, after its last ring access of the phase.
   auto phase_barrier = [&]() {
@@ -568,17 +631,30 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
       const uint32_t row0 = r_beginC + (uint32_t)stepC * kStepRows + 2u * rp;  // this wave's first output row
       const uint32_t nrows = row0 >= r_endC ? 0u : min(2u, r_endC - row0);
       if (wholeC) {
+        // (the few steps whose next row group holds a neighbour's row run a second instance of the step)
+        bool nbr = false;
+        if constexpr (HF) nbr = group_has_neighbour_row();
         if (rp == 0u) {
-          compute(sb, IntTag<1>(), IntTag<2>(), row0, nrows, barrier_owed);
+          if constexpr (HF) {
+            if (nbr) compute(sb, IntTag<1>(), IntTag<2>(), IntTag<1>(), row0, nrows, barrier_owed);
+            else compute(sb, IntTag<1>(), IntTag<2>(), IntTag<0>(), row0, nrows, barrier_owed);
+          } else {
+            compute(sb, IntTag<1>(), IntTag<2>(), IntTag<0>(), row0, nrows, barrier_owed);
+          }
           barrier_owed = false;
         } else {
-          compute(sb, IntTag<1>(), IntTag<1>(), row0, nrows, false);
+          if constexpr (HF) {
+            if (nbr) compute(sb, IntTag<1>(), IntTag<1>(), IntTag<1>(), row0, nrows, false);
+            else compute(sb, IntTag<1>(), IntTag<1>(), IntTag<0>(), row0, nrows, false);
+          } else {
+            compute(sb, IntTag<1>(), IntTag<1>(), IntTag<0>(), row0, nrows, false);
+          }
           barrier_done = true;
         }
       } else {
         if (BETA) load_old_guarded(row0, nrows);
         move_rows_plain();
-        compute(sb, IntTag<0>(), IntTag<0>(), row0, nrows, false);
+        compute(sb, IntTag<0>(), IntTag<0>(), IntTag<0>(), row0, nrows, false);
       }
     } else {
       move_rows_plain();
@@ -607,6 +683,7 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
 // images whose byte offsets fit the buffer range check's 31 bits.
 bool conv_bf16_w8_takes(const ConvBf16Params &P, uint32_t num_tiles) {
   if (P.pad ? (P.IW % 8u) != 0u : (P.IW % 2u) != 0u) return false;
+  if (P.neighbour_rows && P.IH == 0u) return false;
   const uint64_t image_bytes = (uint64_t)P.Cred * P.IH * P.IW * 2u;
   if (image_bytes >= (1ull << 31)) return false;
   if ((uint64_t)P.Cout * P.OH * P.OW * 2u >= (1ull << 31) || (P.OW % 2u) != 0u) return false;
@@ -624,6 +701,24 @@ bool conv_bf16_w8_takes(const ConvBf16Params &P, uint32_t num_tiles) {
 
 int conv_bf16_w8_launch(const ConvBf16Params &P, uint32_t gx, uint32_t groups, hipStream_t st) {
   const dim3 grid(gx, groups), block(kW8Threads);
+  if (P.pad == 1) {  // no halo on either side
+    if (P.passes <= 1u) {
+      if (P.beta != 0.f)
+        hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<true, false, false, true>), grid, block, 0, st, P);
+      else
+        hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, false, false, true>), grid, block, 0, st, P);
+    } else if (P.pass == 0u) {
+      if (P.beta != 0.f)
+        hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<true, false, true, true>), grid, block, 0, st, P);
+      else
+        hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, false, true, true>), grid, block, 0, st, P);
+    } else if (P.pass + 1u < P.passes) {
+      hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, true, true, true>), grid, block, 0, st, P);
+    } else {
+      hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, true, false, true>), grid, block, 0, st, P);
+    }
+    return launch_status();
+  }
   if (P.passes <= 1u) {
     if (P.beta != 0.f)
       hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<true>), grid, block, 0, st, P);

@@ -422,7 +422,23 @@ def main():
             lambda: lib.adh_conv3x3_slab_bwd_filter_tiles(1, K5, N5, C, C, Ht5, W5, t5_tbl, y5_tbl, gw5.data_ptr(), 0.0,
                                                           ws5.data_ptr(), ws5_bytes, stream),
             "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
-        del Y5
+        # the same convolution over tiles WITHOUT halo: one launch does what pack (pad + exchange) + conv, and conv
+        # backward-data + halo reduce + unpack, do in two and three
+        xu = [X5[:, :, r * Ht5:(r + 1) * Ht5, :].contiguous() for r in range(K5)]
+        yu = [torch.empty((N5, C, Ht5, W5), device="cuda", dtype=torch.bfloat16) for _ in range(K5)]
+        xu_tbl, _ku1 = capi.ptr_table([t.data_ptr() for t in xu])
+        yu_tbl, _ku2 = capi.ptr_table([t.data_ptr() for t in yu])
+        add("conv fwd cfg5 over tiles without halo (bf16; pad, exchange and conv in one launch)",
+            lambda: lib.adh_conv3x3_unpadded_fwd_tiles(1, K5, N5, C, C, Ht5, W5, xu_tbl, w5.data_ptr(), yu_tbl, 0.0,
+                                                       ws5.data_ptr(), ws5_bytes, stream),
+            "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s",
+            note="replaces halo pack cfg5 + conv fwd cfg5 above (their times add)")
+        add("conv bwd-data cfg5 into tiles without halo (bf16, beta=0; conv, halo reduce and unpad in one launch)",
+            lambda: lib.adh_conv3x3_unpadded_bwd_data_tiles(1, K5, N5, C, C, Ht5, W5, w5.data_ptr(), y5_tbl, xu_tbl, 0.0,
+                                                            ws5.data_ptr(), ws5_bytes, stream),
+            "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s",
+            note="replaces conv bwd-data cfg5 + halo reduce + halo unpack cfg5 above (their times add)")
+        del Y5, xu, yu
         # 128 channels on the bf16 matrix cores (two passes of 64 reduction channels with fp32 sums in between;
         # the filter gradient as four 64 x 64 channel pairs): the high-resolution tiles at half the width
         Cw, Ww = 128, W5 // 2

@@ -201,6 +201,25 @@ int adh_conv3x3_slab_bwd_data_tiles_reduced(int dtype, uint32_t num_tiles, uint3
                                             const void *const *dy_tiles, void *const *dx_pad_tiles,
                                             float beta, void *workspace, size_t workspace_bytes,
                                             void *stream);
+/* The whole forward chain HaloPad2DOp -> HaloExch2DOp -> CudnnConv2DOp (src/op.cc:2574-2641, 2963-3007,
+ * 1576-1587) and the whole backward chain conv backward-data -> halo reduce -> HaloPad2DOp::_backward
+ * (src/op.cc:1701-1712, 3009-3052, 2643-2700) as ONE launch each over row tiles that carry NO halo:
+ * x_tiles / y_tiles / dy_tiles / dx_tiles are the K row tiles (H x W each, packed NCHW) of one tensor in
+ * rank order.  A tile's rows -1 and H are read from its neighbours' last and first rows, the tensor's own
+ * border is zero: tile t of the result is rows [t*H, (t+1)*H) of the unsplit 3x3 convolution with zero
+ * padding 1 (forward: y = beta*y + conv(x, w); backward-data: dx = beta*dx + conv^T(dy, w)).  No padded
+ * copy of the activation or of its gradient exists, so the pad, exchange, reduce and unpad passes and
+ * their buffers disappear.  bf16 with W a multiple of 8 and 16-byte aligned tiles (the bf16 matrix-core
+ * kernel); other dtypes and widths return ADH_EUNIMPL: use the padded entry points.  Workspace as for
+ * adh_conv3x3_slab_fwd_tiles / adh_conv3x3_slab_bwd_data_tiles of the same shape. */
+int adh_conv3x3_unpadded_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                   uint32_t H, uint32_t W, const void *const *x_tiles, const void *w,
+                                   void *const *y_tiles, float beta, void *workspace, size_t workspace_bytes,
+                                   void *stream);
+int adh_conv3x3_unpadded_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                        uint32_t H, uint32_t W, const void *w, const void *const *dy_tiles,
+                                        void *const *dx_tiles, float beta, void *workspace,
+                                        size_t workspace_bytes, void *stream);
 /* cudnnConvolutionBackwardFilter at src/op.cc:1660-1671:
  * dw[co,ci,kh,kw] = beta*dw + sum_{tiles,n,h,w} dy[n,co,h,w] * x_pad[n,ci,h+kh,w+kw]
  * (the sum over tiles is what ParallelSGDOptimizer's ncclReduce did across ranks,
