@@ -49,6 +49,7 @@ SIGNATURES = {
     "adh_conv3x3_slab_bwd_data_tiles_reduced": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_unpadded_fwd_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_unpadded_bwd_data_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
+    "adh_conv3x3_unpadded_bwd_filter_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_fwd_tiles_static": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp]),
     "adh_conv3x3_slab_bwd_data": (i32, [i32, u32, u32, u32, u32, u32, vp, vp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_data_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
@@ -282,6 +283,15 @@ def conv_unpadded_bwd_data_tiles(w, dys, dxs, N, Cin, Cout, H, W, beta=0.0, ws=N
     wp, wb = _ws(ws)
     return lib().adh_conv3x3_unpadded_bwd_data_tiles(_dt(dys[0]), len(dys), N, Cin, Cout, H, W, w.data_ptr(), dt, xt,
                                                      beta, wp, wb, _stream())
+
+
+def conv_unpadded_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, H, W, beta=0.0, ws=None):
+    _dev(dw, *xs, *dys)
+    xt, k1 = _tbl(xs)
+    dt, k2 = _tbl(dys)
+    wp, wb = _ws(ws)
+    return lib().adh_conv3x3_unpadded_bwd_filter_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, xt, dt, dw.data_ptr(),
+                                                       beta, wp, wb, _stream())
 
 
 def conv2d_workspace_bytes(which, dtype, K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw):

@@ -71,7 +71,7 @@ bool conv_bf16_wgrad_mfma_supported(uint32_t Cin, uint32_t Cout, uint32_t W);
 size_t conv_bf16_wgrad_mfma_workspace_bytes(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t W);
 int conv_bf16_wgrad_mfma(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
                          const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta,
-                         void *workspace, hipStream_t st);
+                         void *workspace, hipStream_t st, bool unpadded);
 
 size_t bf16_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                             uint32_t W, size_t fp32_path_bytes) {
@@ -182,7 +182,7 @@ int conv_bf16_filter_via_f32(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint3
       if (!x_tiles[t] || !dy_tiles[t]) return ADH_ENULL;
       if (!aligned_to(x_tiles[t], 2) || !aligned_to(dy_tiles[t], 2)) return ADH_EALIGN;
     }
-    return conv_bf16_wgrad_mfma(num_tiles, N, Cin, Cout, H, W, x_tiles, dy_tiles, dw, beta, workspace, st);
+    return conv_bf16_wgrad_mfma(num_tiles, N, Cin, Cout, H, W, x_tiles, dy_tiles, dw, beta, workspace, st, false);
   }
   const size_t f32_bytes = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, num_tiles, N, Cin, Cout, H, W);
   if (f32_bytes == 0) return ADH_EUNIMPL;
@@ -212,3 +212,33 @@ int conv_bf16_filter_via_f32(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint3
 }
 
 }  // namespace adh
+
+// The filter gradient over tiles without halo: see adh_conv3x3_unpadded_fwd_tiles.
+extern "C" int adh_conv3x3_unpadded_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                                     uint32_t H, uint32_t W, const void *const *x_tiles,
+                                                     const void *const *dy_tiles, float *dw, float beta, void *workspace,
+                                                     size_t workspace_bytes, void *stream) {
+  using namespace adh;
+  if (!dtype_ok(dtype)) return ADH_EINVAL;
+  if (dtype != ADH_BF16) return ADH_EUNIMPL;
+  if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
+  if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
+  if (Cin == 0 || Cout == 0) return ADH_OK;
+  if (!dw) return ADH_ENULL;
+  if (!aligned_to(dw, 4)) return ADH_EALIGN;
+  if (N == 0 || H == 0 || W == 0) {
+    if (beta == 0.f) return adh_fill_f32((uint64_t)Cin * Cout * 9u, 0.f, dw, stream);  // an empty sum
+    return ADH_OK;
+  }
+  if (!x_tiles || !dy_tiles) return ADH_ENULL;
+  if (!conv_bf16_wgrad_mfma_supported(Cin, Cout, W)) return ADH_EUNIMPL;  // whole 16-byte granules per row
+  if (!workspace) return ADH_ENULL;
+  if (!aligned_to(workspace, 256)) return ADH_EALIGN;
+  if (workspace_bytes < conv_bf16_wgrad_mfma_workspace_bytes(num_tiles, N, Cin, Cout, W)) return ADH_EWORKSPACE;
+  if ((uint64_t)(Cin > Cout ? Cin : Cout) * (H + 2ull) * (W + 2ull) * 2u >= (1ull << 31)) return ADH_EINVAL;
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!x_tiles[t] || !dy_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(x_tiles[t], 16) || !aligned_to(dy_tiles[t], 2)) return ADH_EALIGN;
+  }
+  return conv_bf16_wgrad_mfma(num_tiles, N, Cin, Cout, H, W, x_tiles, dy_tiles, dw, beta, workspace, as_stream(stream), true);
+}

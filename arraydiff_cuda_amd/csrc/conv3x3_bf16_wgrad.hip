@@ -47,6 +47,9 @@ struct WgradBf16Params {
   // More than 64 channels on either side: blockIdx.y numbers the pairs (block of 64 output channels,
   // block of 64 input channels), input block fastest; every pair is a problem of its own.
   uint32_t ci_blocks;
+  // UNP instance: x carries no halo (H x W like dy); the tiles are the row tiles of one tensor in rank
+  // order, and a tile's rows -1 and H are its neighbours' last and first rows
+  uint32_t num_tiles;
   uint32_t strips, items;
   FastDiv div_strips, div_N;
 };
@@ -54,15 +57,25 @@ struct WgradBf16Params {
 template <int V>
 struct WgTag { static constexpr int value = V; };
 
+// UNP: x has no halo.  The x row of a stage is then the unpadded row r - 1 (from a neighbouring tile at the
+// tile's ends, zeros at the tensor's), and a strip's 64 dy columns meet x columns c0 - 1 .. c0 + 64: ten
+// aligned granules from c0 - 8 per channel row (pitch 160 bytes), the operand for column shift kw = 0 made from
+// the aligned 16 bytes and the dword BEFORE them, kw = 2 from the dword after.
+template <bool UNP>
 __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Params P) {
+  constexpr int kXLanes = UNP ? 10 : kWgLanes;          // 16-byte lanes per x channel row
+  constexpr int kXPitch = kXLanes * 16;
+  constexpr int kXRegion = 64 * kXPitch;                // 64 channel rows of x
+  constexpr int kStageBytes = kXRegion + kWgRegion;     // x row, then dy row
+  constexpr int kDmaPerStage = kStageBytes / 1024;      // 18 (19) wave-wide copies
   // one array per stage: the compiler can then tell the asynchronous writes of one stage from
   // the reads of another
-  __shared__ __attribute__((aligned(16))) uint8_t stage0[kWgStageBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t stage1[kWgStageBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t stage2[kWgStageBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t stage3[kWgStageBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t stage4[kWgStageBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t stage5[kWgStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t stage0[kStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t stage1[kStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t stage2[kStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t stage3[kStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t stage4[kStageBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t stage5[kStageBytes];
   __shared__ __attribute__((aligned(16))) uint8_t spare[1024];
   uint8_t *const stages[kWgStages] = {stage0, stage1, stage2, stage3, stage4, stage5};
 
@@ -80,11 +93,12 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
       for (int cot = 0; cot < 2; ++cot) acc[kh][kw][cot] = (floatx4){0.f, 0.f, 0.f, 0.f};
 
   // operand addresses inside a stage, for the left 32 columns (+ 64 bytes for the right ones)
-  const uint32_t b_off = (16u * cit + l16) * kWgPitch + g * 16u;
-  const uint32_t a_off = kWgRegion + (32u * coh + l16) * kWgPitch + g * 16u;  // + cot * 16 * kWgPitch
+  // (UNP: the row in LDS starts eight columns left of the strip)
+  const uint32_t b_off = (16u * cit + l16) * kXPitch + g * 16u + (UNP ? 16u : 0u);
+  const uint32_t a_off = kXRegion + (32u * coh + l16) * kWgPitch + g * 16u;  // + cot * 16 * kWgPitch
 
-  // copies this wave issues per stage: numbers wv, wv + 8, wv + 16 of the 18
-  const uint32_t HP = P.H + 2u, WP = P.W + 2u;
+  // copies this wave issues per stage: numbers wv, wv + 8, wv + 16 of the 18 (19)
+  const uint32_t HP = UNP ? P.H : P.H + 2u, WP = UNP ? P.W : P.W + 2u;  // extents of an x plane in memory
   const uint32_t last_row = P.H + 1u;
 
   // Workgroups are dealt to the eight XCDs (each with its own L2) in turn.  Renumber them so
@@ -102,6 +116,13 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
     const uint16_t *dy_img = P.dy[tile] + (size_t)n * P.Cout * P.H * P.W;
     const __amdgpu_buffer_rsrc_t rsrc_x =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(x_img), 0, P.Cin * HP * WP * 2u, 0x00020000);
+    const bool has_up = UNP && tile > 0u, has_dn = UNP && tile + 1u < P.num_tiles;
+    const __amdgpu_buffer_rsrc_t rsrc_up = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(P.x[has_up ? tile - 1u : tile] + (size_t)n * P.Cin * HP * WP), 0, P.Cin * HP * WP * 2u,
+        0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_dn = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(P.x[has_dn ? tile + 1u : tile] + (size_t)n * P.Cin * HP * WP), 0, P.Cin * HP * WP * 2u,
+        0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_dy =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t *>(dy_img), 0, P.Cout * P.H * P.W * 2u, 0x00020000);
 
@@ -114,15 +135,22 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
 #pragma unroll
     for (int q = 0; q < 3; ++q) {
       const uint32_t k = wv + 8u * q;  // uniform
-      const uint32_t j = (k % 9u) * 64u + lane;  // lane slot within the x_pad or dy region
-      const uint32_t ch = j / kWgLanes, piece = j - ch * kWgLanes;
+      isx_q[q] = k < (uint32_t)kXLanes;
+      const uint32_t j = (isx_q[q] ? k : k - (uint32_t)kXLanes) * 64u + lane;  // lane slot within the x or dy region
+      const uint32_t lanes_per_row = isx_q[q] ? (uint32_t)kXLanes : (uint32_t)kWgLanes;
+      const uint32_t ch = j / lanes_per_row, piece = j - ch * lanes_per_row;
       const uint32_t col = c0 + piece * 8u;
-      isx_q[q] = k < 9u;
-      const uint32_t vx = ci0 + ch < P.Cin ? ((ci0 + ch) * HP * WP + col) * 2u : kWgOutOfRange;
+      uint32_t vx;
+      if (UNP) {
+        const int32_t xcol = (int32_t)col - 8;  // whole granules lie inside or outside a row (W is a multiple of 8)
+        vx = (ci0 + ch < P.Cin && xcol >= 0 && xcol < (int32_t)P.W) ? ((ci0 + ch) * HP * WP + (uint32_t)xcol) * 2u : kWgOutOfRange;
+      } else {
+        vx = ci0 + ch < P.Cin ? ((ci0 + ch) * HP * WP + col) * 2u : kWgOutOfRange;
+      }
       const uint32_t vd =
           (co0 + ch < P.Cout && piece < 8u && col < P.W) ? ((co0 + ch) * P.H * P.W + col) * 2u : kWgOutOfRange;
       voff[q] = isx_q[q] ? vx : vd;
-      rows_q[q] = k >= (uint32_t)kWgDmaPerStage ? 0u : (isx_q[q] ? HP : P.H);
+      rows_q[q] = k >= (uint32_t)kDmaPerStage ? 0u : (isx_q[q] ? P.H + 2u : P.H);
       pitch_q[q] = isx_q[q] ? WP * 2u : P.W * 2u;
       dst_q[q] = k * 1024u;
     }
@@ -130,10 +158,27 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
     auto dma_row = [&](uint32_t r, uint8_t *stage) {
 #pragma unroll
       for (int q = 0; q < 3; ++q) {
-        uint8_t *dst = dst_q[q] < (uint32_t)kWgStageBytes ? stage + dst_q[q] : spare;
-        const uint32_t v = r < rows_q[q] ? voff[q] : kWgOutOfRange;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(isx_q[q] ? rsrc_x : rsrc_dy, (__attribute__((address_space(3))) void *)dst,
-                                                 16, v, __builtin_amdgcn_readfirstlane(r * pitch_q[q]), 0, 0);
+        uint8_t *dst = dst_q[q] < (uint32_t)kStageBytes ? stage + dst_q[q] : spare;
+        uint32_t v = r < rows_q[q] ? voff[q] : kWgOutOfRange;
+        if (UNP && isx_q[q]) {
+          // stage row r holds x row r - 1: the neighbour's last row, the tile's own rows, the other neighbour's first
+          __amdgpu_buffer_rsrc_t rs = rsrc_x;
+          uint32_t row = r - 1u;
+          if (r == 0u) {
+            rs = rsrc_up;
+            row = P.H - 1u;
+            if (!has_up) v = kWgOutOfRange;
+          } else if (r == P.H + 1u) {
+            rs = rsrc_dn;
+            row = 0u;
+            if (!has_dn) v = kWgOutOfRange;
+          }
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void *)dst, 16, v,
+                                                   __builtin_amdgcn_readfirstlane(row * pitch_q[q]), 0, 0);
+        } else {
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(isx_q[q] ? rsrc_x : rsrc_dy, (__attribute__((address_space(3))) void *)dst,
+                                                   16, v, __builtin_amdgcn_readfirstlane(r * pitch_q[q]), 0, 0);
+        }
       }
     };
 
@@ -148,7 +193,7 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
 #pragma unroll
         for (int cot = 0; cot < 2; ++cot) win[a][kb][cot] = (u32x4){0u, 0u, 0u, 0u};
     u32x4 xb[2][2];
-    uint32_t xe[2][2];
+    uint32_t xe[2][2], xm[2][2];  // the dword after the 16 bytes; UNP: and the one before
 
     // operands of row r from its stage: dy row r -> window slot r mod 4, x_pad row r -> parity r mod 2
     auto fetch = [&](auto ph) {
@@ -158,6 +203,7 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
       for (int kb = 0; kb < 2; ++kb) {
         xb[PH % 2][kb] = *reinterpret_cast<const u32x4 *>(src + b_off + kb * 64);
         xe[PH % 2][kb] = *reinterpret_cast<const uint32_t *>(src + b_off + kb * 64 + 16);
+        if (UNP) xm[PH % 2][kb] = *reinterpret_cast<const uint32_t *>(src + b_off + kb * 64 - 4);
       }
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
@@ -215,7 +261,15 @@ __global__ __launch_bounds__(512, 1) void conv3x3_bf16_wgrad_kernel(WgradBf16Par
         b1[2] = __builtin_amdgcn_alignbit(b0[3], b0[2], 16);
         b1[3] = __builtin_amdgcn_alignbit(b4, b0[3], 16);
         const u32x4 b2 = (u32x4){b0[1], b0[2], b0[3], b4};
-        const u32x4 bs[3] = {b0, b1, b2};
+        u32x4 bm;  // UNP: one column to the left
+        if (UNP) {
+          bm[0] = __builtin_amdgcn_alignbit(b0[0], xm[PH % 2][kb], 16);
+          bm[1] = __builtin_amdgcn_alignbit(b0[1], b0[0], 16);
+          bm[2] = __builtin_amdgcn_alignbit(b0[2], b0[1], 16);
+          bm[3] = __builtin_amdgcn_alignbit(b0[3], b0[2], 16);
+        }
+        // column shifts kw = 0, 1, 2: padded x: 0, +1, +2 columns from the strip's first; unpadded: -1, 0, +1
+        const u32x4 bs[3] = {UNP ? bm : b0, UNP ? b0 : b1, UNP ? b1 : b2};
 #pragma unroll
         for (int kh = 0; kh < 3; ++kh) {
           const int slot = (PH + 4 - kh) % 4;  // dy row r - kh
@@ -325,7 +379,7 @@ size_t conv_bf16_wgrad_mfma_workspace_bytes(uint32_t num_tiles, uint32_t N, uint
 // Arguments are validated by the caller (pointers, alignment, workspace size, extents > 0).
 int conv_bf16_wgrad_mfma(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
                          const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta,
-                         void *workspace, hipStream_t st) {
+                         void *workspace, hipStream_t st, bool unpadded) {
   WgradBf16Params P = {};
   for (uint32_t t = 0; t < num_tiles; ++t) {
     P.x[t] = reinterpret_cast<const uint16_t *>(x_tiles[t]);
@@ -342,7 +396,11 @@ int conv_bf16_wgrad_mfma(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t 
   const uint32_t blocks = wgrad_bf16_blocks(items);
   P.ci_blocks = (Cin + 63u) / 64u;
   const uint32_t pairs = P.ci_blocks * ((Cout + 63u) / 64u);
-  hipLaunchKernelGGL(conv3x3_bf16_wgrad_kernel, dim3(blocks, pairs), dim3(512), 0, st, P);
+  P.num_tiles = num_tiles;
+  if (unpadded)
+    hipLaunchKernelGGL(conv3x3_bf16_wgrad_kernel<true>, dim3(blocks, pairs), dim3(512), 0, st, P);
+  else
+    hipLaunchKernelGGL(conv3x3_bf16_wgrad_kernel<false>, dim3(blocks, pairs), dim3(512), 0, st, P);
   int e = launch_status();
   if (e) return e;
   hipLaunchKernelGGL(conv3x3_bf16_wgrad_reduce_kernel, dim3(kWgPartialFloats / 64u, pairs), dim3(256), 0, st,

@@ -438,6 +438,10 @@ def main():
                                                             ws5.data_ptr(), ws5_bytes, stream),
             "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s",
             note="replaces conv bwd-data cfg5 + halo reduce + halo unpack cfg5 above (their times add)")
+        add("conv bwd-filter cfg5 over tiles without halo (bf16 in, fp32 filter gradient, two kernels)",
+            lambda: lib.adh_conv3x3_unpadded_bwd_filter_tiles(1, K5, N5, C, C, Ht5, W5, xu_tbl, y5_tbl, gw5.data_ptr(), 0.0,
+                                                              ws5.data_ptr(), ws5_bytes, stream),
+            "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
         del Y5, xu, yu
         # 128 channels on the bf16 matrix cores (two passes of 64 reduction channels with fp32 sums in between;
         # the filter gradient as four 64 x 64 channel pairs): the high-resolution tiles at half the width

@@ -220,6 +220,13 @@ int adh_conv3x3_unpadded_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t 
                                         uint32_t H, uint32_t W, const void *w, const void *const *dy_tiles,
                                         void *const *dx_tiles, float beta, void *workspace,
                                         size_t workspace_bytes, void *stream);
+/* the filter gradient of the same convolution (cudnnConvolutionBackwardFilter, src/op.cc:1660-1671, over
+ * the tiles HaloPad2DOp and HaloExch2DOp would have prepared): dw = beta*dw + sum over tiles of
+ * dy (*) x with x read as above.  Workspace as for adh_conv3x3_slab_bwd_filter_tiles. */
+int adh_conv3x3_unpadded_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                          uint32_t H, uint32_t W, const void *const *x_tiles,
+                                          const void *const *dy_tiles, float *dw, float beta, void *workspace,
+                                          size_t workspace_bytes, void *stream);
 /* cudnnConvolutionBackwardFilter at src/op.cc:1660-1671:
  * dw[co,ci,kh,kw] = beta*dw + sum_{tiles,n,h,w} dy[n,co,h,w] * x_pad[n,ci,h+kh,w+kw]
  * (the sum over tiles is what ParallelSGDOptimizer's ncclReduce did across ranks,

@@ -1,4 +1,4 @@
-"""Convolution over row tiles that carry no halo (adh_conv3x3_unpadded_{fwd,bwd_data}_tiles): tile t of the
+"""Convolution over row tiles that carry no halo (adh_conv3x3_unpadded_{fwd,bwd_data,bwd_filter}_tiles): tile t of the
 result must be rows [t*H, (t+1)*H) of the UNSPLIT 3x3 convolution with zero padding 1 - what pad -> exchange ->
 conv (forward) and conv backward-data -> reduce -> unpad (backward) compute in the reference's graph.  Checked
 against the CPU oracle's unsplit convolution and, bit for bit, against this library's own padded chain.
@@ -40,12 +40,15 @@ def test_unpadded_tiles_vs_unsplit_oracle(oracle, K, N, Cin, Cout, Ht, W):
     gx_want = np.empty((N, Cin, H + 2, W + 2), np.float32)
     oracle.conv_slab_bwd_data(wf, dyf, gx_want)
     gx_want = gx_want[:, :, 1:-1, 1:-1]
+    dw_want = np.zeros((Cout, Cin, 3, 3), np.float32)
+    oracle.conv_slab_bwd_filter(xp, dyf, dw_want)
 
     xs = [dev(x[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
     dys = [dev(dy[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
     y0 = [dev(bf(rng.standard_normal((N, Cout, Ht, W)))) for _ in range(K)]
     g0 = [dev(bf(rng.standard_normal((N, Cin, Ht, W)))) for _ in range(K)]
     d_w = dev(w)
+    dw0 = dev(rng.standard_normal((Cout, Cin, 3, 3)).astype(np.float32))
     for beta in (0.0, 1.0):
         ys = [t.clone() for t in y0]
         gs = [t.clone() for t in g0]
@@ -53,6 +56,10 @@ def test_unpadded_tiles_vs_unsplit_oracle(oracle, K, N, Cin, Cout, Ht, W):
                                                 ws=ws_for(capi.ADH_CONV_FWD, K, N, Cin, Cout, Ht, W)), "fwd")
         capi.check(capi.conv_unpadded_bwd_data_tiles(d_w, dys, gs, N, Cin, Cout, Ht, W, beta=beta,
                                                      ws=ws_for(capi.ADH_CONV_BWD_DATA, K, N, Cin, Cout, Ht, W)), "bwd-data")
+        dw = dw0.clone()
+        capi.check(capi.conv_unpadded_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, Ht, W, beta=beta,
+                                                       ws=ws_for(capi.ADH_CONV_BWD_FILTER, K, N, Cin, Cout, Ht, W)), "bwd-filter")
+        assert rel_err(host(dw), dw_want + beta * host(dw0)) <= 1e-4  # fp32 output, exact bf16 products
         for r in range(K):
             want_y = y_want[:, :, r * Ht:(r + 1) * Ht, :] + beta * oracle.bf16_to_f32(host(y0[r]))
             want_g = gx_want[:, :, r * Ht:(r + 1) * Ht, :] + beta * oracle.bf16_to_f32(host(g0[r]))
