@@ -225,3 +225,39 @@ def test_bf16_conv_random_channel_counts(oracle, K, N, Cin, Cout, H, W):
         assert rel_err(oracle.bf16_to_f32(host(ga[r])), g + oracle.bf16_to_f32(g0[r])) <= 5e-3
         oracle.conv_slab_bwd_filter(xf, dyf, dw_want, beta=1.0)
     assert rel_err(host(dw), dw_want) <= 1e-4
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,Ht,W", _bf16_wide_cases(2029, 16))
+def test_bf16_conv_over_tiles_without_halo_random(oracle, K, N, Cin, Cout, Ht, W):
+    """adh_conv3x3_unpadded_{fwd,bwd_data,bwd_filter}_tiles against the UNSPLIT convolution with zero padding."""
+    rng = np.random.default_rng(Cin * 311 + Cout + K)
+    bf = lambda a: oracle.f32_to_bf16(a.astype(np.float32))
+    H = K * Ht
+    x = bf(rng.uniform(-1, 1, size=(N, Cin, H, W)))
+    w = bf(rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9)))
+    dy = bf(rng.standard_normal((N, Cout, H, W)))
+    xf, wf, dyf = oracle.bf16_to_f32(x), oracle.bf16_to_f32(w), oracle.bf16_to_f32(dy)
+    xp = np.zeros((N, Cin, H + 2, W + 2), np.float32)
+    xp[:, :, 1:-1, 1:-1] = xf
+    y_want = np.empty((N, Cout, H, W), np.float32)
+    oracle.conv_slab_fwd(xp, wf, y_want)
+    gx_want = np.empty((N, Cin, H + 2, W + 2), np.float32)
+    oracle.conv_slab_bwd_data(wf, dyf, gx_want)
+    dw_want = np.zeros((Cout, Cin, 3, 3), np.float32)
+    oracle.conv_slab_bwd_filter(xp, dyf, dw_want)
+
+    def ws_for(which):
+        return torch.empty(capi.conv_workspace_bytes(which, capi.ADH_BF16, K, N, Cin, Cout, Ht, W) // 4 + 64, device="cuda")
+
+    xs = [dev(x[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    dys = [dev(dy[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    ys = [torch.empty((N, Cout, Ht, W), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
+    gs = [torch.empty((N, Cin, Ht, W), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
+    dw = torch.full((Cout, Cin, 3, 3), float("nan"), device="cuda")
+    capi.check(capi.conv_unpadded_fwd_tiles(xs, dev(w), ys, N, Cin, Cout, Ht, W, ws=ws_for(capi.ADH_CONV_FWD)))
+    capi.check(capi.conv_unpadded_bwd_data_tiles(dev(w), dys, gs, N, Cin, Cout, Ht, W, ws=ws_for(capi.ADH_CONV_BWD_DATA)))
+    capi.check(capi.conv_unpadded_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, Ht, W, ws=ws_for(capi.ADH_CONV_BWD_FILTER)))
+    for r in range(K):
+        assert rel_err(oracle.bf16_to_f32(host(ys[r])), y_want[:, :, r * Ht:(r + 1) * Ht, :]) <= 5e-3
+        assert rel_err(oracle.bf16_to_f32(host(gs[r])), gx_want[:, :, 1 + r * Ht:1 + (r + 1) * Ht, 1:-1]) <= 5e-3
+    assert rel_err(host(dw), dw_want) <= 1e-4
