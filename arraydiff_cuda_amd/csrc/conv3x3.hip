@@ -399,7 +399,7 @@ int conv_bf16_via_f32(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, u
 // which: ADH_CONV_FWD or ADH_CONV_BWD_DATA.  H, W are the interior extents.
 static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                        uint32_t W, const void *const *in_tiles, const void *w, void *const *out_tiles, float beta,
-                       hipStream_t st, bool rows_from_neighbours = false) {
+                       hipStream_t st, bool rows_from_neighbours = false, bool unpadded = false) {
   if (!dtype_ok(dtype)) return ADH_EINVAL;
   if (dtype != ADH_F32) return ADH_EUNIMPL;
   if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
@@ -440,6 +440,14 @@ static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uin
     P.pad = 2;
     P.w_out_stride = 9u; P.w_red_stride = Cin * 9u; P.w_flip = 1;
   }
+  if (unpadded) {
+    // neither side carries a halo: the unsplit convolution with zero padding 1, restricted to the tile; rows -1
+    // and H come from the neighbouring tiles (zero columns and the tensor's own border through the range check)
+    P.IH = P.OH = H; P.IW = P.OW = W;
+    P.pad = 1;
+    P.rows_from_neighbours = 1;
+    P.nb_lo = -1; P.nb_hi = (int32_t)H; P.nb_above = (int32_t)H - 1; P.nb_below = 0;
+  }
   const uint32_t o_groups = (P.Cout + 63u) / 64u;
   const ConvTile tile = choose_tile(P.OH, P.OW, (uint64_t)N * num_tiles, o_groups);
   if (tile.nt == 0) return ADH_EINVAL;
@@ -473,6 +481,9 @@ static int conv_direct_kernel_name(int which, uint32_t num_tiles, uint32_t N, ui
 }
 
 const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, float beta);
+int conv_bf16_unpadded(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                       const void *const *in_tiles, const void *w, void *const *out_tiles, float beta, void *workspace,
+                       size_t workspace_bytes, hipStream_t st);
 
 }  // namespace adh
 
@@ -553,6 +564,26 @@ int adh_conv3x3_slab_bwd_data_tiles_reduced(int dtype, uint32_t num_tiles, uint3
   }
   return conv_direct(ADH_CONV_BWD_DATA, dtype, num_tiles, N, Cin, Cout, H, W, dy_tiles, w, dx_pad_tiles, beta,
                      as_stream(stream), true);
+}
+
+int adh_conv3x3_unpadded_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                                   uint32_t W, const void *const *x_tiles, const void *w, void *const *y_tiles, float beta,
+                                   void *workspace, size_t workspace_bytes, void *stream) {
+  if (dtype == ADH_F32)
+    return conv_direct(ADH_CONV_FWD, dtype, num_tiles, N, Cin, Cout, H, W, x_tiles, w, y_tiles, beta, as_stream(stream),
+                       true, true);
+  return conv_bf16_unpadded(ADH_CONV_FWD, dtype, num_tiles, N, Cin, Cout, H, W, x_tiles, w, y_tiles, beta, workspace,
+                            workspace_bytes, as_stream(stream));
+}
+
+int adh_conv3x3_unpadded_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                                        uint32_t W, const void *w, const void *const *dy_tiles, void *const *dx_tiles,
+                                        float beta, void *workspace, size_t workspace_bytes, void *stream) {
+  if (dtype == ADH_F32)
+    return conv_direct(ADH_CONV_BWD_DATA, dtype, num_tiles, N, Cin, Cout, H, W, dy_tiles, w, dx_tiles, beta,
+                       as_stream(stream), true, true);
+  return conv_bf16_unpadded(ADH_CONV_BWD_DATA, dtype, num_tiles, N, Cin, Cout, H, W, dy_tiles, w, dx_tiles, beta, workspace,
+                            workspace_bytes, as_stream(stream));
 }
 
 int adh_conv3x3_slab_bwd_data(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,

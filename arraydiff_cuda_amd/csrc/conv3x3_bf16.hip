@@ -213,6 +213,12 @@ int conv_bf16_filter_via_f32(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint3
 
 }  // namespace adh
 
+namespace adh {
+int conv_wgrad_f32_unpadded(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                            const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta, void *workspace,
+                            size_t workspace_bytes, void *stream);
+}
+
 // The filter gradient over tiles without halo: see adh_conv3x3_unpadded_fwd_tiles.
 extern "C" int adh_conv3x3_unpadded_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
                                                      uint32_t H, uint32_t W, const void *const *x_tiles,
@@ -220,7 +226,9 @@ extern "C" int adh_conv3x3_unpadded_bwd_filter_tiles(int dtype, uint32_t num_til
                                                      size_t workspace_bytes, void *stream) {
   using namespace adh;
   if (!dtype_ok(dtype)) return ADH_EINVAL;
-  if (dtype != ADH_BF16) return ADH_EUNIMPL;
+  if (dtype == ADH_F32)
+    return conv_wgrad_f32_unpadded(num_tiles, N, Cin, Cout, H, W, x_tiles, dy_tiles, dw, beta, workspace, workspace_bytes,
+                                   stream);
   if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
   if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
   if (Cin == 0 || Cout == 0) return ADH_OK;

@@ -721,13 +721,12 @@ extern "C" int adh_conv3x3_slab_fwd_tiles_static(int dtype, uint32_t num_tiles, 
 }
 
 // ---------------------------------------------------------------------------
-// convolution over row tiles that carry no halo
+// convolution over row tiles that carry no halo (bf16; the entry points are in conv3x3.hip)
 // ---------------------------------------------------------------------------
-namespace {
-int unpadded_entry(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
-                   const void *const *in_tiles, const void *w, void *const *out_tiles, float beta, void *workspace,
-                   size_t workspace_bytes, void *stream) {
-  using namespace adh;
+namespace adh {
+int conv_bf16_unpadded(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                       const void *const *in_tiles, const void *w, void *const *out_tiles, float beta, void *workspace,
+                       size_t workspace_bytes, hipStream_t st) {
   if (!dtype_ok(dtype)) return ADH_EINVAL;
   if (dtype != ADH_BF16) return ADH_EUNIMPL;
   if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
@@ -748,23 +747,6 @@ int unpadded_entry(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_
   if (!workspace) return ADH_ENULL;
   if (!aligned_to(workspace, 256)) return ADH_EALIGN;
   if (workspace_bytes < need) return ADH_EWORKSPACE;
-  return conv_bf16_mfma(which, num_tiles, N, Cin, Cout, H, W, in_tiles, w, out_tiles, beta, workspace, as_stream(stream),
-                        true);
+  return conv_bf16_mfma(which, num_tiles, N, Cin, Cout, H, W, in_tiles, w, out_tiles, beta, workspace, st, true);
 }
-}  // namespace
-
-extern "C" int adh_conv3x3_unpadded_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
-                                              uint32_t H, uint32_t W, const void *const *x_tiles, const void *w,
-                                              void *const *y_tiles, float beta, void *workspace, size_t workspace_bytes,
-                                              void *stream) {
-  return unpadded_entry(ADH_CONV_FWD, dtype, num_tiles, N, Cin, Cout, H, W, x_tiles, w, y_tiles, beta, workspace,
-                        workspace_bytes, stream);
-}
-
-extern "C" int adh_conv3x3_unpadded_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
-                                                   uint32_t H, uint32_t W, const void *w, const void *const *dy_tiles,
-                                                   void *const *dx_tiles, float beta, void *workspace,
-                                                   size_t workspace_bytes, void *stream) {
-  return unpadded_entry(ADH_CONV_BWD_DATA, dtype, num_tiles, N, Cin, Cout, H, W, dy_tiles, w, dx_tiles, beta, workspace,
-                        workspace_bytes, stream);
-}
+}  // namespace adh

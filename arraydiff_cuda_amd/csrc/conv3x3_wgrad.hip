@@ -46,6 +46,9 @@ struct WgradParams {
   // tile t-1's last interior row and slab row H+1 of tile t < num_tiles-1 from tile t+1's first
   // interior row, which is what a halo exchange would have copied there
   int32_t rows_from_neighbours;
+  // x carries no halo (H x W like dy): slab row y is x row y - 1, slab column c is x column c - 1, what lies
+  // outside is zero or, for rows -1 and H with rows_from_neighbours, the neighbouring tile's last / first row
+  int32_t unpadded;
   FastDiv div_chunks, div_tiles, div_ci_groups, div_cols;
 };
 
@@ -72,7 +75,7 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
   P.div_ci_groups.divmod(blockIdx.y, coh, cig);
   const uint32_t r0 = chunk * P.rows_per_block;
   const uint32_t r1 = min(r0 + P.rows_per_block, P.H);
-  const uint32_t WP = P.W + 2u, HP = P.H + 2u;
+  const uint32_t WP = P.unpadded ? P.W : P.W + 2u, HP = P.unpadded ? P.H : P.H + 2u;  // an x plane in memory
   const uint32_t ci0 = cig * 64u, co0 = coh * 32u;
   const float *__restrict__ x = P.x[t] + ((uint64_t)n * P.Cin) * HP * WP;
   const float *__restrict__ dy = P.dy[t] + ((uint64_t)n * P.Cout) * P.H * P.W;
@@ -92,7 +95,11 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
       __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(dy), 0, (int)(P.Cout * P.H * P.W * 4u), kWgBufferFlags);
   const uint32_t w0 = ctile * P.cols_per_block;
   const uint32_t tw = min(P.cols_per_block, P.W - w0);  // columns of this workgroup
-  const uint32_t x_voff = lane < tw + 2u ? (w0 + lane) * 4u : kWgOutOfRange;
+  uint32_t x_voff = lane < tw + 2u ? (w0 + lane) * 4u : kWgOutOfRange;
+  if (P.unpadded) {
+    const int32_t col = (int32_t)(w0 + lane) - 1;
+    x_voff = (lane < tw + 2u && col >= 0 && col < (int32_t)P.W) ? (uint32_t)col * 4u : kWgOutOfRange;
+  }
   const uint32_t d_voff = lane < tw ? (w0 + lane) * 4u : kWgOutOfRange;
   const bool ragged_c = (ci0 + 64u > P.Cin) || (co0 + 32u > P.Cout);  // uniform
   // a slab row is uniform over the workgroup, and so is the image it comes from
@@ -106,7 +113,20 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
       kWgBufferFlags);
   auto stage_x_row = [&](float *slot, uint32_t y) {  // slab row y of the 64 input channels
     __amdgpu_buffer_rsrc_t rsrc = rsrc_x;
-    if (from_above && y == 0u) {
+    bool none = false;  // a row of zeros
+    if (P.unpadded) {
+      if (y == 0u) {
+        rsrc = rsrc_above;
+        none = !from_above;
+        y = P.H - 1u;
+      } else if (y == P.H + 1u) {
+        rsrc = rsrc_below;
+        none = !from_below;
+        y = 0u;
+      } else {
+        y -= 1u;
+      }
+    } else if (from_above && y == 0u) {
       rsrc = rsrc_above;
       y = P.H;
     } else if (from_below && y == HP - 1u) {
@@ -116,7 +136,7 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const uint32_t cl = wv * 8u + i;
-      uint32_t voff = x_voff;
+      uint32_t voff = none ? kWgOutOfRange : x_voff;
       uint32_t ci = ci0 + cl;
       if (ragged_c && ci >= P.Cin) {
         voff = kWgOutOfRange;
@@ -342,8 +362,10 @@ size_t adh_conv3x3_workspace_bytes(int which, int dtype, uint32_t num_tiles, uin
 
 static int wgrad_entry(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
                        const void *const *x_pad_tiles, const void *const *dy_tiles, float *dw, float beta,
-                       void *workspace, size_t workspace_bytes, void *stream, bool rows_from_neighbours) {
+                       void *workspace, size_t workspace_bytes, void *stream, bool rows_from_neighbours,
+                       bool unpadded = false) {
   if (!dtype_ok(dtype)) return ADH_EINVAL;
+  if (unpadded && dtype != ADH_F32) return ADH_EINVAL;  // the bf16 form has an entry of its own
   if (dtype == ADH_BF16 && rows_from_neighbours) {
     // the bf16 kernels stream their rows from one image: exchange first, then the ordinary path
     const int rc = adh_halo_exchange_nchw(dtype, 1, num_tiles, 1, W, H, Cin, N,
@@ -391,6 +413,7 @@ static int wgrad_entry(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, 
   P.div_tiles = FastDiv(num_tiles);
   P.div_ci_groups = FastDiv(P.ci_groups);
   P.rows_from_neighbours = rows_from_neighbours ? 1 : 0;
+  P.unpadded = unpadded ? 1 : 0;
   dim3 grid(plan.blocks_x, plan.groups, 1);
   if (grid.y > 65535u) return ADH_EINVAL;
   hipLaunchKernelGGL(conv3x3_wgrad_f32_kernel, grid, dim3(kWgThreads), 0, st, P);
@@ -421,6 +444,20 @@ int adh_conv3x3_slab_bwd_filter_tiles_unexchanged(int dtype, uint32_t num_tiles,
   return wgrad_entry(dtype, num_tiles, N, Cin, Cout, H, W, x_pad_tiles, dy_tiles, dw, beta, workspace, workspace_bytes,
                      stream, true);
 }
+
+}  // extern "C"
+
+// the fp32 leg of adh_conv3x3_unpadded_bwd_filter_tiles
+namespace adh {
+int conv_wgrad_f32_unpadded(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                            const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta, void *workspace,
+                            size_t workspace_bytes, void *stream) {
+  return wgrad_entry(ADH_F32, num_tiles, N, Cin, Cout, H, W, x_tiles, dy_tiles, dw, beta, workspace, workspace_bytes, stream,
+                     true, true);
+}
+}  // namespace adh
+
+extern "C" {
 
 int adh_conv3x3_slab_bwd_filter(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
                                 const void *x_pad, const void *dy, float *dw, float beta, void *workspace,

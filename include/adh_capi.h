@@ -209,9 +209,10 @@ int adh_conv3x3_slab_bwd_data_tiles_reduced(int dtype, uint32_t num_tiles, uint3
  * border is zero: tile t of the result is rows [t*H, (t+1)*H) of the unsplit 3x3 convolution with zero
  * padding 1 (forward: y = beta*y + conv(x, w); backward-data: dx = beta*dx + conv^T(dy, w)).  No padded
  * copy of the activation or of its gradient exists, so the pad, exchange, reduce and unpad passes and
- * their buffers disappear.  bf16 with W a multiple of 8 and 16-byte aligned tiles (the bf16 matrix-core
- * kernel); other dtypes and widths return ADH_EUNIMPL: use the padded entry points.  Workspace as for
- * adh_conv3x3_slab_fwd_tiles / adh_conv3x3_slab_bwd_data_tiles of the same shape. */
+ * their buffers disappear.  fp32: any shape the padded entry points take, no workspace.  bf16: W a
+ * multiple of 8 and 16-byte aligned tiles (the bf16 matrix-core kernel; other widths return
+ * ADH_EUNIMPL: use the padded entry points), workspace as for adh_conv3x3_slab_fwd_tiles /
+ * adh_conv3x3_slab_bwd_data_tiles of the same shape. */
 int adh_conv3x3_unpadded_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
                                    uint32_t H, uint32_t W, const void *const *x_tiles, const void *w,
                                    void *const *y_tiles, float beta, void *workspace, size_t workspace_bytes,

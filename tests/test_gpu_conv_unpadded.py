@@ -93,8 +93,43 @@ def test_unpadded_entry_limits():
     w = torch.zeros((8, 8, 3, 3), device="cuda", dtype=torch.bfloat16)
     ws = torch.empty(1 << 16, device="cuda")
     assert capi.conv_unpadded_fwd_tiles(x, w, y, 1, 8, 8, 4, 12, ws=ws) == capi.ADH_EUNIMPL  # width not a multiple of 8
-    xf = [torch.zeros((1, 8, 4, 16), device="cuda")]
-    assert capi.conv_unpadded_fwd_tiles(xf, w.float(), [torch.zeros_like(xf[0])], 1, 8, 8, 4, 16, ws=ws) == capi.ADH_EUNIMPL
     x16 = [torch.zeros((1, 8, 4, 16), device="cuda", dtype=torch.bfloat16)]
     assert capi.conv_unpadded_fwd_tiles(x16, w, [torch.zeros_like(x16[0])], 1, 8, 8, 4, 16, beta=0.5, ws=ws) == capi.ADH_EINVAL
     assert capi.conv_unpadded_fwd_tiles(x16, w, [torch.zeros_like(x16[0])], 1, 8, 8, 4, 16, ws=None) == capi.ADH_ENULL
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,Ht,W", [(1, 2, 8, 16, 5, 9), (2, 1, 19, 7, 6, 33), (4, 2, 9, 70, 1, 13), (3, 1, 24, 40, 23, 5),
+                                              (4, 32, 64, 64, 14, 56), (2, 96, 8, 16, 11, 20), (5, 1, 16, 8, 3, 150)])
+def test_unpadded_tiles_fp32_vs_unsplit_oracle(oracle, K, N, Cin, Cout, Ht, W):
+    """The fp32 forms (any width): forward, backward-data and filter gradient over tiles without halo against the
+    unsplit convolution, rel-err <= 1e-5, beta 0 and 1."""
+    rng = np.random.default_rng(5200 + K * 13 + Cin)
+    H = K * Ht
+    x = rng.uniform(-1, 1, size=(N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))).astype(np.float32)
+    dy = rng.standard_normal((N, Cout, H, W)).astype(np.float32)
+    xp = np.zeros((N, Cin, H + 2, W + 2), np.float32)
+    xp[:, :, 1:-1, 1:-1] = x
+    y_want = np.empty((N, Cout, H, W), np.float32)
+    oracle.conv_slab_fwd(xp, w, y_want)
+    gx_want = np.empty((N, Cin, H + 2, W + 2), np.float32)
+    oracle.conv_slab_bwd_data(w, dy, gx_want)
+    gx_want = gx_want[:, :, 1:-1, 1:-1]
+    dw_want = np.zeros((Cout, Cin, 3, 3), np.float32)
+    oracle.conv_slab_bwd_filter(xp, dy, dw_want)
+    xs = [dev(x[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    dys = [dev(dy[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    y0 = [dev(rng.standard_normal((N, Cout, Ht, W)).astype(np.float32)) for _ in range(K)]
+    g0 = [dev(rng.standard_normal((N, Cin, Ht, W)).astype(np.float32)) for _ in range(K)]
+    dw0 = dev(rng.standard_normal((Cout, Cin, 3, 3)).astype(np.float32))
+    nbytes = capi.conv_workspace_bytes(capi.ADH_CONV_BWD_FILTER, capi.ADH_F32, K, N, Cin, Cout, Ht, W)
+    ws = torch.empty(max(nbytes // 4, 1), device="cuda")
+    for beta in (0.0, 1.0):
+        ys, gs, dw = [t.clone() for t in y0], [t.clone() for t in g0], dw0.clone()
+        capi.check(capi.conv_unpadded_fwd_tiles(xs, dev(w), ys, N, Cin, Cout, Ht, W, beta=beta), "fwd")
+        capi.check(capi.conv_unpadded_bwd_data_tiles(dev(w), dys, gs, N, Cin, Cout, Ht, W, beta=beta), "bwd-data")
+        capi.check(capi.conv_unpadded_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, Ht, W, beta=beta, ws=ws), "bwd-filter")
+        assert rel_err(host(dw), dw_want + beta * host(dw0)) <= 1e-5
+        for r in range(K):
+            assert rel_err(host(ys[r]), y_want[:, :, r * Ht:(r + 1) * Ht, :] + beta * host(y0[r])) <= 1e-5
+            assert rel_err(host(gs[r]), gx_want[:, :, r * Ht:(r + 1) * Ht, :] + beta * host(g0[r])) <= 1e-5
