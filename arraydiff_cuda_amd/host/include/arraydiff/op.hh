@@ -902,6 +902,12 @@ public:
   // neighbours' gradient rows, or by a reduce after the ordinary one).  The input gradient must have no
   // other contributor.
   bool unexchanged_rows = false;
+  // Not in the reference.  The inputs are the row tiles of one activation in rank order (a 1 x K grid) and
+  // carry NO halo (halo_padded_input = false, pad = {1, 1}, 3x3, stride 1, dilation 1): the op is the
+  // reference's HaloPad2DOp -> HaloExch2DOp -> conv chain in one node.  Zero padding at the tensor's border
+  // and the neighbours' rows at the tiles' borders are read by the kernels; the input gradient comes out
+  // unpadded and complete.
+  bool unpadded_tiles = false;
 };
 
 // V = GPUBatchArray3D<float>, A = GPUArray4D<float> (filter, Shape4D(kw,kh,Cin,Cout) = KCRS).
@@ -937,7 +943,11 @@ public:
     if (shape.kernel[0] == 0 || shape.kernel[1] == 0 || shape.stride[0] == 0 || shape.stride[1] == 0 ||
         shape.dilate[0] == 0 || shape.dilate[1] == 0)
       throw std::invalid_argument("SlabConv2DOp: empty window, stride or dilation");
-    if (!shape.halo_padded_input && (shape.pad[0] != 0 || shape.pad[1] != 0))
+    if (shape.unpadded_tiles) {
+      if (shape.halo_padded_input || shape.kernel[0] != 3 || shape.kernel[1] != 3 || shape.stride[0] != 1 ||
+          shape.stride[1] != 1 || shape.dilate[0] != 1 || shape.dilate[1] != 1 || shape.pad[0] != 1 || shape.pad[1] != 1)
+        throw std::invalid_argument("SlabConv2DOp: tiles without halo take 3x3, stride 1, dilation 1, padding 1");
+    } else if (!shape.halo_padded_input && (shape.pad[0] != 0 || shape.pad[1] != 0))
       throw std::invalid_argument("SlabConv2DOp: padding needs a halo-padded input");
     if (inputs.empty() || inputs.size() != kernels.size() || inputs.size() > ADH_MAX_TILES)
       throw std::invalid_argument("SlabConv2DOp: one kernel variable per input");
@@ -945,7 +955,8 @@ public:
       throw std::invalid_argument("SlabConv2DOp: unexchanged rows need a halo of one");
     for (size_t r = 0; r < inputs.size(); ++r) {
       auto off = inputs[r]->offset();
-      if (off.shape[0] != shape.pad[0] || off.shape[1] != shape.pad[1] || off.shape[2] != 0)
+      const size_t halo0 = shape.unpadded_tiles ? 0 : shape.pad[0], halo1 = shape.unpadded_tiles ? 0 : shape.pad[1];
+      if (off.shape[0] != halo0 || off.shape[1] != halo1 || off.shape[2] != 0)
         throw std::invalid_argument("SlabConv2DOp: input halo must equal the conv pad");
       if (inputs[r]->shape() != inputs[0]->shape() || inputs[r]->batch_shape() != inputs[0]->batch_shape())
         throw std::invalid_argument("SlabConv2DOp: all slabs must have one shape");

@@ -130,6 +130,26 @@ vector<shared_ptr<Var<V>>> bn_relu_pad_conv3x3(ParallelBatchNormParamOp<V> &bloc
                                                shared_ptr<bool> switch_var, vector<shared_ptr<Var<V>>> inputs,
                                                shared_ptr<Context> ctx) {
   const size_t cin = inputs.at(0)->shape().shape[2];
+  // On row tiles of more than 256 pixels a stride-1 3x3 runs over tiles WITHOUT halo: the batch norm does not
+  // pad, no exchange node exists, and the conv node reads zero padding and its neighbours' rows itself (the
+  // 3x3 kernels serve every pass from that size on; smaller tiles keep the padded chain and the general kernels).
+  const auto tile = inputs.at(0)->shape();
+  const bool halo_free = stride == 1 && mgpu_ctx_of(ctx)->spatial_comm(0)->num_w_ranks == 1 && tile.shape[0] * tile.shape[1] > 256 &&
+                         shape.kernel[0] == 3 && shape.kernel[1] == 3 && shape.dilate[0] == 1 && shape.dilate[1] == 1 &&
+                         shape.pad[0] == 1 && shape.pad[1] == 1;
+  if (halo_free) {
+    typedef GPUArray4D<float> A;
+    auto bnorm = CudnnBatchNorm2DOp<bool, V, GPUArray1D<float>>::MakeParallel(cin, switch_var, inputs, ctx, true, 0);
+    add_batch_norm(block, bnorm);
+    Conv2DShape cs = shape;
+    cs.stride = {1, 1};
+    cs.halo_padded_input = false;
+    cs.unpadded_tiles = true;
+    auto conv = parallel_conv2d<V, A>(cs, bnorm.ops, kaiming_init_gen<A>(cin * 9, shape.filters), false, ctx);
+    parallel_vars_insert_all(block.params, conv.params);
+    parallel_vars_insert_all(block.grads, conv.grads);
+    return conv.ops;
+  }
   auto bnorm = CudnnBatchNorm2DOp<bool, V, GPUArray1D<float>>::MakeParallel(cin, switch_var, inputs, ctx, true, 1);
   add_batch_norm(block, bnorm);
   return exchanged_conv3x3(block, shape, stride, bnorm.ops, ctx);

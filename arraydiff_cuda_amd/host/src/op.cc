@@ -478,6 +478,14 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
+    if (shape_.unpadded_tiles) {
+      if (n != K) throw HazardError("SlabConv2DOp: tiles without halo need every rank in one pass");
+      adh_check(adh_conv3x3_unpadded_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt, 0.0f,
+                                               nullptr, 0, conn.stream()),
+                "SlabConv2DOp::_forward (tiles without halo)");
+      todo.swap(rest);
+      continue;
+    }
     const bool in_kernel_rows = n == K && reads_neighbour_rows(*this, shape_, d, n);
     if (shape_.unexchanged_rows && !in_kernel_rows && !exchanged) {
       // no kernel for this shape reads across tiles (or this launch does not hold every tile): exchange over
@@ -570,7 +578,16 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
-    if (use_3x3_filter_kernel(*this, d, n, shape_.filters)) {
+    if (shape_.unpadded_tiles) {
+      if (n != K) throw HazardError("SlabConv2DOp: tiles without halo need every rank in one pass");
+      const size_t ws = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
+                                                    d.H, d.W);
+      dc->reserve_scratch(ws);
+      auto scratch = dc->get_scratch();
+      adh_check(adh_conv3x3_unpadded_bwd_filter_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, dyt, dw,
+                                                      wbeta, scratch->dptr(), scratch->size(), conn.stream()),
+                "SlabConv2DOp::_backward (filter, tiles without halo)");
+    } else if (use_3x3_filter_kernel(*this, d, n, shape_.filters)) {
       const size_t ws = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
                                                     d.H, d.W);
       dc->reserve_scratch(ws);
@@ -632,6 +649,14 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
     const float beta = first ? 0.0f : 1.0f;
+    if (shape_.unpadded_tiles) {
+      if (n != K) throw HazardError("SlabConv2DOp: tiles without halo need every rank in one pass");
+      adh_check(adh_conv3x3_unpadded_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, w0, dyt, dxt,
+                                                    beta, nullptr, 0, conn.stream()),
+                "SlabConv2DOp::_backward (data, tiles without halo)");
+      todo.swap(rest);
+      continue;
+    }
     const bool in_kernel_rows = n == K && reads_neighbour_rows(*this, shape_, d, n);
     if (shape_.unexchanged_rows && !in_kernel_rows) {
       // a halo reduce after this pass would add what the halo rows held before it a second time

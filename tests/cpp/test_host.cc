@@ -171,7 +171,9 @@ static std::vector<float> normal(std::mt19937 &g, size_t n, float s) {
 // of src/zoo.cc:577-652 and :1522-1526, on K row-tiles of one GPU.
 // unexchanged: the exchange node copies nothing in the forward pass and the convolution reads its neighbours'
 // rows itself (tiles of more than 256 pixels) or exchanges first (smaller ones)
-static void test_spatial_conv_graph(size_t K, size_t N, size_t C, size_t Co, size_t H, size_t W, bool unexchanged = false) {
+// halo_free: no pad and no exchange node at all: the conv node takes the scattered tiles as they are
+static void test_spatial_conv_graph(size_t K, size_t N, size_t C, size_t Co, size_t H, size_t W, bool unexchanged = false,
+                                    bool halo_free = false) {
   std::mt19937 gen(1234 + (unsigned)K);
   auto ctx = MultiGPUContext::Make(K);
   std::vector<float> X = uniform(gen, N * C * H * W, -1, 1);
@@ -194,10 +196,11 @@ static void test_spatial_conv_graph(size_t K, size_t N, size_t C, size_t Co, siz
   cs.dilate = {1, 1};
   cs.stride = {1, 1};
   cs.pad = {1, 1};
-  cs.halo_padded_input = true;
+  cs.halo_padded_input = !halo_free;
   cs.enable_hmma = false;
   cs.unexchanged_rows = unexchanged;
-  auto ys = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch, ws, ctx);
+  cs.unpadded_tiles = halo_free;
+  auto ys = CudnnConv2DOp<V, A, A>::MakeParallel(cs, halo_free ? tiles : exch, ws, ctx);
   auto y_full = SpatialJoinedGather2DOp<V>::Make(ys, ctx);
   auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
   sink->set_host_grad(dY.data());
@@ -227,7 +230,7 @@ static void test_spatial_conv_graph(size_t K, size_t N, size_t C, size_t Co, siz
     orc_conv_slab_bwd_filter(N, C, Co, H, W, 3, Xp.data(), dY.data(), 0.f, dWr.data());
     const double ey = rel_err(Y, Yr), ex = rel_err(dX, dXr), ew = rel_err(dW, dWr);
     std::printf("graph K=%zu N=%zu C=%zu->%zu %zux%zu%s rep %d: rel-err y %.2e dx %.2e dw %.2e\n", K, N, C, Co, H, W,
-                unexchanged ? " unexchanged" : "", rep, ey, ex, ew);
+                halo_free ? " tiles without halo" : unexchanged ? " unexchanged" : "", rep, ey, ex, ew);
     CHECK(ey <= 1e-5 && ex <= 1e-5 && ew <= 1e-5);
   }
 }
@@ -1007,6 +1010,10 @@ int main(int argc, char **argv) {
     test_spatial_conv_graph(4, 4, 64, 64, 56, 56, true);
     test_spatial_conv_graph(2, 3, 5, 7, 40, 30, true);
     test_spatial_conv_graph(4, 2, 8, 16, 8, 12, true);
+    test_spatial_conv_graph(4, 4, 64, 64, 56, 56, false, true);
+    test_spatial_conv_graph(2, 3, 5, 7, 40, 30, false, true);
+    test_spatial_conv_graph(4, 2, 8, 16, 8, 12, false, true);
+    test_spatial_conv_graph(1, 1, 16, 16, 5, 5, false, true);
     test_spatial_general_conv_graph(4, 2, 3, 16, 32, 24, 7, 2, 1);   // the stem
     test_spatial_general_conv_graph(2, 2, 8, 12, 16, 20, 3, 2, 1);   // stride-2 3x3
     test_spatial_general_conv_graph(2, 1, 8, 8, 12, 14, 3, 1, 3);    // dilation 3 over halo 3
