@@ -130,11 +130,11 @@ vector<shared_ptr<Var<V>>> bn_relu_pad_conv3x3(ParallelBatchNormParamOp<V> &bloc
                                                shared_ptr<bool> switch_var, vector<shared_ptr<Var<V>>> inputs,
                                                shared_ptr<Context> ctx) {
   const size_t cin = inputs.at(0)->shape().shape[2];
-  // On row tiles of more than 256 pixels a stride-1 3x3 runs over tiles WITHOUT halo: the batch norm does not
+  // On row tiles of at least 256 pixels a stride-1 3x3 runs over tiles WITHOUT halo: the batch norm does not
   // pad, no exchange node exists, and the conv node reads zero padding and its neighbours' rows itself (the
   // 3x3 kernels serve every pass from that size on; smaller tiles keep the padded chain and the general kernels).
   const auto tile = inputs.at(0)->shape();
-  const bool halo_free = stride == 1 && mgpu_ctx_of(ctx)->spatial_comm(0)->num_w_ranks == 1 && tile.shape[0] * tile.shape[1] > 256 &&
+  const bool halo_free = stride == 1 && mgpu_ctx_of(ctx)->spatial_comm(0)->num_w_ranks == 1 && tile.shape[0] * tile.shape[1] >= 256 &&
                          shape.kernel[0] == 3 && shape.kernel[1] == 3 && shape.dilate[0] == 1 && shape.dilate[1] == 1 &&
                          shape.pad[0] == 1 && shape.pad[1] == 1;
   if (halo_free) {
