@@ -39,8 +39,9 @@ struct WgradParams {
   float *partial;            // [grid.y][grid.x][32*64*9] in (co, ci, tap) order, local to the group
   uint32_t num_tiles, N, Cin, Cout, H, W;
   uint32_t rows_per_block, chunks_per_plane;  // row chunks of a plane
+  uint32_t planes_per_block;                  // image planes a workgroup walks (same rows and columns of each)
   uint32_t cols_per_block, col_tiles;         // column tiles of a plane (<= kMaxW columns each)
-  // grid.x = col_tiles * chunks_per_plane * N * num_tiles
+  // grid.x = col_tiles * chunks_per_plane * ceil(N * num_tiles / planes_per_block)
   uint32_t ci_groups;        // grid.y = co_halves * ci_groups, co_halves = ceil(Cout/32)
   // the tiles are the row tiles of one activation in rank order: slab row 0 of tile t > 0 is read from
   // tile t-1's last interior row and slab row H+1 of tile t < num_tiles-1 from tile t+1's first
@@ -66,19 +67,15 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
   const uint32_t ot = wv & 1u;   // co tile inside the 32-channel half
   const uint32_t ct = wv >> 1;   // ci tile
 
-  uint32_t rest, ctile, plane, chunk;
+  uint32_t rest, ctile, pgroup, chunk;
   P.div_cols.divmod(blockIdx.x, rest, ctile);
-  P.div_chunks.divmod(rest, plane, chunk);
-  uint32_t n, t;
-  P.div_tiles.divmod(plane, n, t);
+  P.div_chunks.divmod(rest, pgroup, chunk);
   uint32_t coh, cig;
   P.div_ci_groups.divmod(blockIdx.y, coh, cig);
   const uint32_t r0 = chunk * P.rows_per_block;
   const uint32_t r1 = min(r0 + P.rows_per_block, P.H);
   const uint32_t WP = P.unpadded ? P.W : P.W + 2u, HP = P.unpadded ? P.H : P.H + 2u;  // an x plane in memory
   const uint32_t ci0 = cig * 64u, co0 = coh * 32u;
-  const float *__restrict__ x = P.x[t] + ((uint64_t)n * P.Cin) * HP * WP;
-  const float *__restrict__ dy = P.dy[t] + ((uint64_t)n * P.Cout) * P.H * P.W;
 
   // columns 64..67 of every staged row are read by the last k-steps of wide rows but never
   // written by the 64-lane loads: clear them once
@@ -89,10 +86,6 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
 
   // ---- staging: one 64-lane load = one channel row; wave v loads slab channels [8v,8v+8) and
   // dy channels [4v,4v+4) ----
-  const __amdgpu_buffer_rsrc_t rsrc_x =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(x), 0, (int)(P.Cin * HP * WP * 4u), kWgBufferFlags);
-  const __amdgpu_buffer_rsrc_t rsrc_dy =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(dy), 0, (int)(P.Cout * P.H * P.W * 4u), kWgBufferFlags);
   const uint32_t w0 = ctile * P.cols_per_block;
   const uint32_t tw = min(P.cols_per_block, P.W - w0);  // columns of this workgroup
   uint32_t x_voff = lane < tw + 2u ? (w0 + lane) * 4u : kWgOutOfRange;
@@ -102,15 +95,26 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
   }
   const uint32_t d_voff = lane < tw ? (w0 + lane) * 4u : kWgOutOfRange;
   const bool ragged_c = (ci0 + 64u > P.Cin) || (co0 + 32u > P.Cout);  // uniform
-  // a slab row is uniform over the workgroup, and so is the image it comes from
-  const bool from_above = P.rows_from_neighbours && t > 0u;
-  const bool from_below = P.rows_from_neighbours && t + 1u < P.num_tiles;
-  const __amdgpu_buffer_rsrc_t rsrc_above = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float *>(P.x[from_above ? t - 1u : t] + ((uint64_t)n * P.Cin) * HP * WP), 0, (int)(P.Cin * HP * WP * 4u),
-      kWgBufferFlags);
-  const __amdgpu_buffer_rsrc_t rsrc_below = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<float *>(P.x[from_below ? t + 1u : t] + ((uint64_t)n * P.Cin) * HP * WP), 0, (int)(P.Cin * HP * WP * 4u),
-      kWgBufferFlags);
+  // The image plane (tile, image) the workgroup stands at; it walks planes_per_block of them with the same
+  // accumulators.  A slab row is uniform over the workgroup, and so is the image it comes from.
+  const int x_bytes = (int)(P.Cin * HP * WP * 4u), dy_bytes = (int)(P.Cout * P.H * P.W * 4u);
+  __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.x[0]), 0, 0, kWgBufferFlags);
+  __amdgpu_buffer_rsrc_t rsrc_dy = rsrc_x, rsrc_above = rsrc_x, rsrc_below = rsrc_x;
+  bool from_above = false, from_below = false;
+  auto open_plane = [&](uint32_t plane) {
+    uint32_t n, t;
+    P.div_tiles.divmod(plane, n, t);
+    const uint64_t x_img = ((uint64_t)n * P.Cin) * HP * WP;
+    rsrc_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.x[t] + x_img), 0, x_bytes, kWgBufferFlags);
+    rsrc_dy = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.dy[t] + ((uint64_t)n * P.Cout) * P.H * P.W), 0,
+                                                dy_bytes, kWgBufferFlags);
+    from_above = P.rows_from_neighbours && t > 0u;
+    from_below = P.rows_from_neighbours && t + 1u < P.num_tiles;
+    rsrc_above = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.x[from_above ? t - 1u : t] + x_img), 0, x_bytes,
+                                                   kWgBufferFlags);
+    rsrc_below = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.x[from_below ? t + 1u : t] + x_img), 0, x_bytes,
+                                                   kWgBufferFlags);
+  };
   auto stage_x_row = [&](float *slot, uint32_t y) {  // slab row y of the 64 input channels
     __amdgpu_buffer_rsrc_t rsrc = rsrc_x;
     bool none = false;  // a row of zeros
@@ -204,35 +208,40 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
     }
   };
 
-  // prologue: slab rows r0, r0+1, r0+2 -> slots 0,1,2 and dy row r0 -> slot 0
-  stage_x_row(xs0, r0);
-  stage_x_row(xs1, r0 + 1u);
-  stage_x_row(xs2, r0 + 2u);
-  stage_dy_row(dys0, r0);
-  __syncthreads();
+  const uint32_t plane0 = pgroup * P.planes_per_block;
+  const uint32_t plane1 = min(plane0 + P.planes_per_block, P.num_tiles * P.N);
+  for (uint32_t plane = plane0; plane < plane1; ++plane) {
+    open_plane(plane);
+    // prologue: slab rows r0, r0+1, r0+2 -> slots 0,1,2 and dy row r0 -> slot 0
+    stage_x_row(xs0, r0);
+    stage_x_row(xs1, r0 + 1u);
+    stage_x_row(xs2, r0 + 2u);
+    stage_dy_row(dys0, r0);
+    __syncthreads();
 
-  // four rows per trip: each phase names its ring slots statically
-  for (uint32_t r = r0;;) {
-    if (r + 1u < r1) { stage_x_row(xs3, r + 3u); stage_dy_row(dys1, r + 1u); }
-    __builtin_amdgcn_sched_barrier(0);
-    compute_row(dys0, xs0, xs1, xs2);
-    __syncthreads();
-    if (++r == r1) break;
-    if (r + 1u < r1) { stage_x_row(xs0, r + 3u); stage_dy_row(dys0, r + 1u); }
-    __builtin_amdgcn_sched_barrier(0);
-    compute_row(dys1, xs1, xs2, xs3);
-    __syncthreads();
-    if (++r == r1) break;
-    if (r + 1u < r1) { stage_x_row(xs1, r + 3u); stage_dy_row(dys1, r + 1u); }
-    __builtin_amdgcn_sched_barrier(0);
-    compute_row(dys0, xs2, xs3, xs0);
-    __syncthreads();
-    if (++r == r1) break;
-    if (r + 1u < r1) { stage_x_row(xs2, r + 3u); stage_dy_row(dys0, r + 1u); }
-    __builtin_amdgcn_sched_barrier(0);
-    compute_row(dys1, xs3, xs0, xs1);
-    __syncthreads();
-    if (++r == r1) break;
+    // four rows per trip: each phase names its ring slots statically
+    for (uint32_t r = r0;;) {
+      if (r + 1u < r1) { stage_x_row(xs3, r + 3u); stage_dy_row(dys1, r + 1u); }
+      __builtin_amdgcn_sched_barrier(0);
+      compute_row(dys0, xs0, xs1, xs2);
+      __syncthreads();
+      if (++r == r1) break;
+      if (r + 1u < r1) { stage_x_row(xs0, r + 3u); stage_dy_row(dys0, r + 1u); }
+      __builtin_amdgcn_sched_barrier(0);
+      compute_row(dys1, xs1, xs2, xs3);
+      __syncthreads();
+      if (++r == r1) break;
+      if (r + 1u < r1) { stage_x_row(xs1, r + 3u); stage_dy_row(dys1, r + 1u); }
+      __builtin_amdgcn_sched_barrier(0);
+      compute_row(dys0, xs2, xs3, xs0);
+      __syncthreads();
+      if (++r == r1) break;
+      if (r + 1u < r1) { stage_x_row(xs2, r + 3u); stage_dy_row(dys0, r + 1u); }
+      __builtin_amdgcn_sched_barrier(0);
+      compute_row(dys1, xs3, xs0, xs1);
+      __syncthreads();
+      if (++r == r1) break;
+    }
   }
 
   // ---- epilogue: lane holds D[co = 4g+i][ci = l16] of each tap tile ----
@@ -293,7 +302,7 @@ __global__ __launch_bounds__(256) void conv3x3_wgrad_reduce_kernel(const WgradRe
 }
 
 struct WgradPlan {
-  uint32_t rows_per_block, chunks_per_plane, cols_per_block, col_tiles, blocks_x, groups;
+  uint32_t rows_per_block, chunks_per_plane, planes_per_block, cols_per_block, col_tiles, blocks_x, groups;
   size_t workspace_bytes;
 };
 
@@ -303,30 +312,39 @@ static bool wgrad_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Co
   const uint32_t groups = ((Cin + 63u) / 64u) * ((Cout + 31u) / 32u);
   const uint32_t col_tiles = (W + kMaxW - 1) / kMaxW;
   const uint32_t cols = (W + col_tiles - 1) / col_tiles;
-  // Row chunks per plane: a workgroup's time grows with its rows, 256 CUs run one workgroup each
-  // per round, and every workgroup costs one partial block to write and reduce (priced here as
-  // two rows of work).  Pick the chunk count with the least modelled time.
-  const uint64_t per_chunk = planes * col_tiles * groups;
-  uint32_t best_chunks = 1;
+  // Row chunks per plane and planes per workgroup.  256 CUs run one workgroup each per round.  A workgroup
+  // spends 576 matrix-core cycles per k-step of four columns (9 MFMAs of 32 cycles, two waves a SIMD) on every
+  // row, about 4000 cycles per plane waiting for its first rows, and about 19000 cycles on being launched and
+  // on writing the partial block that the second kernel then reads back.  Pick the pair with the least modelled time.
+  const double row_cycles = 576.0 * ((cols + 3u) / 4u), plane_cycles = 4000.0, block_cycles = 19000.0;
+  const uint64_t per_chunk = (uint64_t)col_tiles * groups;
+  uint32_t best_chunks = 1, best_ppb = 1;
   double best_cost = 1e300;
   for (uint32_t chunks = 1; chunks <= H; ++chunks) {
     const uint32_t rows = (H + chunks - 1) / chunks;
     if ((H + rows - 1) / rows != chunks) continue;  // same row count as a smaller chunk number
-    const uint64_t blocks = per_chunk * chunks;
-    const double cost = (double)((blocks + 255) / 256) * (rows + 2.0);
-    if (cost < best_cost) {
-      best_cost = cost;
-      best_chunks = chunks;
+    for (uint64_t ppb = 1; ppb <= planes; ++ppb) {
+      const uint64_t pgroups = (planes + ppb - 1) / ppb;
+      if ((planes + pgroups - 1) / pgroups != ppb) continue;  // same group count as a smaller number of planes
+      const uint64_t blocks = per_chunk * chunks * pgroups;
+      const double cost = (double)((blocks + 255) / 256) * ((double)ppb * (rows * row_cycles + plane_cycles) + block_cycles);
+      if (cost < best_cost) {
+        best_cost = cost;
+        best_chunks = chunks;
+        best_ppb = (uint32_t)ppb;
+      }
+      if (blocks < 256) break;  // more planes per workgroup only leave more CUs idle
     }
-    if (blocks >= 4096) break;
+    if (per_chunk * chunks * planes >= 4096) break;
   }
   const uint32_t rows = (H + best_chunks - 1) / best_chunks;
-  const uint64_t blocks_x = planes * best_chunks * col_tiles;
+  const uint64_t blocks_x = ((planes + best_ppb - 1) / best_ppb) * best_chunks * col_tiles;
   if (blocks_x > 0x7fffffffull) return false;
   // one image of x / dy is addressed through a 32-bit buffer resource
   if ((uint64_t)Cin * (H + 2) * (W + 2) * 4u >= (1ull << 31) || (uint64_t)Cout * H * W * 4u >= (1ull << 31)) return false;
   plan->rows_per_block = rows;
   plan->chunks_per_plane = best_chunks;
+  plan->planes_per_block = best_ppb;
   plan->cols_per_block = cols;
   plan->col_tiles = col_tiles;
   plan->blocks_x = (uint32_t)blocks_x;
@@ -405,6 +423,7 @@ static int wgrad_entry(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, 
   P.num_tiles = num_tiles; P.N = N; P.Cin = Cin; P.Cout = Cout; P.H = H; P.W = W;
   P.rows_per_block = plan.rows_per_block;
   P.chunks_per_plane = plan.chunks_per_plane;
+  P.planes_per_block = plan.planes_per_block;
   P.cols_per_block = plan.cols_per_block;
   P.col_tiles = plan.col_tiles;
   P.div_cols = FastDiv(plan.col_tiles);
