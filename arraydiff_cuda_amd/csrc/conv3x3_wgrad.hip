@@ -12,6 +12,10 @@
 //     buffer_load ... lds, while the previous row is being multiplied; lanes past the row end
 //     carry an out-of-range offset and the hardware writes zero.  Channel pitch 68 floats
 //     (== 4 mod 64): the 16 channels x 4 pixels of one operand read hit 64 different banks.
+//     Column tiles of at most 36 pixels take pitch 44 instead (16 channels x 44 floats fall on 16
+//     different groups of four banks too): the rings then need 56 KB, two workgroups share a CU and
+//     each one's waits (first rows of a plane, the barrier after a row, the partial block's stores)
+//     are the other's matrix-core time.
 //   * LDS reads of k-step s+1 are interleaved 1:1 with the MFMAs of k-step s (two-deep register
 //     buffer, pinned with scheduling-group barriers).
 //   * every workgroup writes its partial 32x64x9 block to the workspace and a second kernel
@@ -24,11 +28,10 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 static constexpr int kWgWaves = 8;
 static constexpr int kWgThreads = 64 * kWgWaves;
-static constexpr int kRowPitch = 68;              // floats per staged channel row, == 4 (mod 64)
-static constexpr int kXSlotFloats = 64 * kRowPitch;
-static constexpr int kDSlotFloats = 32 * kRowPitch;
-// the last k-step reads columns up to 4*ceil(W/4)+5 < kRowPitch, and a row is one 64-lane load
-static constexpr int kMaxW = 60;
+// floats per staged channel row (PITCH): 68 or 44.  A row is one load of min(64, PITCH) lanes, and the k-steps
+// run in pairs: the last one reads columns up to 8 * ceil(ceil(W / 4) / 2) + 1 < PITCH.
+static constexpr int kMaxW = 60;        // widest column tile at pitch 68
+static constexpr int kMaxWNarrow = 40;  // at pitch 44
 static constexpr int kPartialFloats = 32 * 64 * 9;
 static constexpr int kWgBufferFlags = 0x00020000;
 static constexpr uint32_t kWgOutOfRange = 0x80000000u;
@@ -53,7 +56,10 @@ struct WgradParams {
   FastDiv div_chunks, div_tiles, div_ci_groups, div_cols;
 };
 
-__global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const WgradParams P) {
+template <int PITCH>
+__global__ __launch_bounds__(kWgThreads, PITCH == 44 ? 2 : 1) void conv3x3_wgrad_f32_kernel(const WgradParams P) {
+  constexpr int kRowPitch = PITCH;
+  constexpr int kXSlotFloats = 64 * kRowPitch, kDSlotFloats = 32 * kRowPitch;
   __shared__ float xs0[kXSlotFloats];
   __shared__ float xs1[kXSlotFloats];
   __shared__ float xs2[kXSlotFloats];
@@ -79,10 +85,15 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
 
   // columns 64..67 of every staged row are read by the last k-steps of wide rows but never
   // written by the 64-lane loads: clear them once
-  for (uint32_t i = tid; i < 64u * 4u; i += kWgThreads) {
-    const uint32_t o = (i >> 2) * kRowPitch + 64u + (i & 3u);
-    xs0[o] = 0.f; xs1[o] = 0.f; xs2[o] = 0.f; xs3[o] = 0.f;
+  if constexpr (PITCH > 64) {
+    for (uint32_t i = tid; i < 64u * 4u; i += kWgThreads) {
+      const uint32_t o = (i >> 2) * kRowPitch + 64u + (i & 3u);
+      xs0[o] = 0.f; xs1[o] = 0.f; xs2[o] = 0.f; xs3[o] = 0.f;
+    }
   }
+  // a load writes one dword per lane from the row's start on: lanes past the pitch would land in the next
+  // channel's row, so they are switched off (a lane that is switched off writes nothing)
+  const bool row_lane = PITCH >= 64 || lane < (uint32_t)PITCH;
 
   // ---- staging: one 64-lane load = one channel row; wave v loads slab channels [8v,8v+8) and
   // dy channels [4v,4v+4) ----
@@ -137,6 +148,7 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
       rsrc = rsrc_below;
       y = 1u;
     }
+    if (!row_lane) return;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const uint32_t cl = wv * 8u + i;
@@ -151,6 +163,7 @@ __global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_f32_kernel(const 
     }
   };
   auto stage_dy_row = [&](float *slot, uint32_t r) {  // output row r of the 32 output channels
+    if (!row_lane) return;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t cl = wv * 4u + i;
@@ -303,23 +316,24 @@ __global__ __launch_bounds__(256) void conv3x3_wgrad_reduce_kernel(const WgradRe
 
 struct WgradPlan {
   uint32_t rows_per_block, chunks_per_plane, planes_per_block, cols_per_block, col_tiles, blocks_x, groups;
+  bool narrow;  // column tiles of at most kMaxWNarrow pixels: row pitch 44, two workgroups per CU
   size_t workspace_bytes;
 };
 
-static bool wgrad_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
-                       WgradPlan *plan) {
-  const uint64_t planes = (uint64_t)num_tiles * N;
-  const uint32_t groups = ((Cin + 63u) / 64u) * ((Cout + 31u) / 32u);
-  const uint32_t col_tiles = (W + kMaxW - 1) / kMaxW;
-  const uint32_t cols = (W + col_tiles - 1) / col_tiles;
-  // Row chunks per plane and planes per workgroup.  256 CUs run one workgroup each per round.  A workgroup
-  // spends 576 matrix-core cycles per k-step of four columns (9 MFMAs of 32 cycles, two waves a SIMD) on every
-  // row, about 4000 cycles per plane waiting for its first rows, and about 19000 cycles on being launched and
-  // on writing the partial block that the second kernel then reads back.  Pick the pair with the least modelled time.
-  const double row_cycles = 576.0 * ((cols + 3u) / 4u), plane_cycles = 4000.0, block_cycles = 19000.0;
-  const uint64_t per_chunk = (uint64_t)col_tiles * groups;
-  uint32_t best_chunks = 1, best_ppb = 1;
+// Row chunks per plane and planes per workgroup for column tiles of `cols` pixels, `per_cu` workgroups sharing a
+// CU.  A workgroup spends 576 matrix-core cycles per k-step of four columns (9 MFMAs of 32 cycles, two waves a SIMD)
+// on every row, about 4000 cycles per plane waiting for its first rows, and about 19000 cycles on being launched
+// and on writing the partial block that the second kernel then reads back; workgroups that share a CU share its
+// matrix cores, and one's waits are the other's multiplications.  Every partial block is 74 KB written and read
+// once more, about 100 cycles of the whole chip's memory bandwidth.  Returns the least modelled time.
+static double wgrad_plan_rows(uint64_t planes, uint64_t per_chunk, uint32_t H, uint32_t cols, uint32_t per_cu,
+                              uint32_t *best_chunks, uint32_t *best_ppb) {
+  const double row_cycles = 576.0 * ((cols + 3u) / 4u) * per_cu;
+  const double plane_cycles = per_cu > 1u ? 1000.0 : 4000.0, block_cycles = per_cu > 1u ? 8000.0 : 19000.0;
+  const uint64_t slots = 256ull * per_cu;
   double best_cost = 1e300;
+  *best_chunks = 1;
+  *best_ppb = 1;
   for (uint32_t chunks = 1; chunks <= H; ++chunks) {
     const uint32_t rows = (H + chunks - 1) / chunks;
     if ((H + rows - 1) / rows != chunks) continue;  // same row count as a smaller chunk number
@@ -327,26 +341,45 @@ static bool wgrad_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Co
       const uint64_t pgroups = (planes + ppb - 1) / ppb;
       if ((planes + pgroups - 1) / pgroups != ppb) continue;  // same group count as a smaller number of planes
       const uint64_t blocks = per_chunk * chunks * pgroups;
-      const double cost = (double)((blocks + 255) / 256) * ((double)ppb * (rows * row_cycles + plane_cycles) + block_cycles);
+      const double cost = (double)((blocks + slots - 1) / slots) * ((double)ppb * (rows * row_cycles + plane_cycles) + block_cycles) +
+                          100.0 * (double)blocks;
       if (cost < best_cost) {
         best_cost = cost;
-        best_chunks = chunks;
-        best_ppb = (uint32_t)ppb;
+        *best_chunks = chunks;
+        *best_ppb = (uint32_t)ppb;
       }
-      if (blocks < 256) break;  // more planes per workgroup only leave more CUs idle
+      if (blocks < slots) break;  // more planes per workgroup only leave more CUs idle
     }
-    if (per_chunk * chunks * planes >= 4096) break;
+    if (per_chunk * chunks * planes >= 16u * slots) break;
   }
-  const uint32_t rows = (H + best_chunks - 1) / best_chunks;
-  const uint64_t blocks_x = ((planes + best_ppb - 1) / best_ppb) * best_chunks * col_tiles;
+  return best_cost;
+}
+
+static bool wgrad_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                       WgradPlan *plan) {
+  const uint64_t planes = (uint64_t)num_tiles * N;
+  const uint32_t groups = ((Cin + 63u) / 64u) * ((Cout + 31u) / 32u);
+  uint32_t chunks[2], ppb[2], col_tiles[2], cols[2];
+  double cost[2];
+  for (int narrow = 0; narrow < 2; ++narrow) {
+    const uint32_t max_w = narrow ? kMaxWNarrow : kMaxW;
+    col_tiles[narrow] = (W + max_w - 1) / max_w;
+    cols[narrow] = (W + col_tiles[narrow] - 1) / col_tiles[narrow];
+    cost[narrow] = wgrad_plan_rows(planes, (uint64_t)col_tiles[narrow] * groups, H, cols[narrow], narrow ? 2u : 1u,
+                                   &chunks[narrow], &ppb[narrow]);
+  }
+  const int pick = cost[1] <= cost[0] ? 1 : 0;
+  const uint32_t rows = (H + chunks[pick] - 1) / chunks[pick];
+  const uint64_t blocks_x = ((planes + ppb[pick] - 1) / ppb[pick]) * chunks[pick] * col_tiles[pick];
   if (blocks_x > 0x7fffffffull) return false;
   // one image of x / dy is addressed through a 32-bit buffer resource
   if ((uint64_t)Cin * (H + 2) * (W + 2) * 4u >= (1ull << 31) || (uint64_t)Cout * H * W * 4u >= (1ull << 31)) return false;
   plan->rows_per_block = rows;
-  plan->chunks_per_plane = best_chunks;
-  plan->planes_per_block = best_ppb;
-  plan->cols_per_block = cols;
-  plan->col_tiles = col_tiles;
+  plan->chunks_per_plane = chunks[pick];
+  plan->planes_per_block = ppb[pick];
+  plan->cols_per_block = cols[pick];
+  plan->col_tiles = col_tiles[pick];
+  plan->narrow = pick == 1;
   plan->blocks_x = (uint32_t)blocks_x;
   plan->groups = groups;
   plan->workspace_bytes = (size_t)plan->blocks_x * groups * kPartialFloats * sizeof(float);
@@ -435,7 +468,10 @@ static int wgrad_entry(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, 
   P.unpadded = unpadded ? 1 : 0;
   dim3 grid(plan.blocks_x, plan.groups, 1);
   if (grid.y > 65535u) return ADH_EINVAL;
-  hipLaunchKernelGGL(conv3x3_wgrad_f32_kernel, grid, dim3(kWgThreads), 0, st, P);
+  if (plan.narrow)
+    hipLaunchKernelGGL(conv3x3_wgrad_f32_kernel<44>, grid, dim3(kWgThreads), 0, st, P);
+  else
+    hipLaunchKernelGGL(conv3x3_wgrad_f32_kernel<68>, grid, dim3(kWgThreads), 0, st, P);
   int e = launch_status();
   if (e) return e;
   WgradReduceParams R = {};
