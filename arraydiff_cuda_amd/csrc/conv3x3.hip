@@ -66,11 +66,15 @@ struct ConvParams {
 };
 
 // staged patch rows (>= R + 2): 12, or 20 in the tall variant of the kernel, which is a few percent slower per
-// flop (more rows to stage per wave) and is chosen where taller tiles waste fewer pixel slots
+// flop (more rows to stage per wave) and is chosen where taller tiles waste fewer pixel slots, or 10 in the
+// short variant of the 16-tile kernel: its buffers then take 77 KB, two workgroups share a CU and the waits of
+// one (its first chunk, the barrier after every chunk, its stores) are the other's matrix-core time
 static constexpr int kPatchRows = 12;
 static constexpr int kPatchRowsTall = 20;
+static constexpr int kPatchRowsShort = 10;
 static constexpr int kMaxR = kPatchRows - 2;
 static constexpr int kMaxRTall = kPatchRowsTall - 2;
+static constexpr int kMaxRShort = kPatchRowsShort - 2;
 
 template <int V>
 struct IntTag {
@@ -85,7 +89,7 @@ struct IntTag {
 // FLIP  = false: forward (weights walked as w[o][k][tap]); true: backward-data
 //         (weights walked as w[k][o][8-tap]).
 template <int NT, int WAVES, bool FLIP, int PROWS>
-__global__ __launch_bounds__(64 * WAVES, 1) void conv3x3_f32_kernel(const ConvParams P) {
+__global__ __launch_bounds__(64 * WAVES, PROWS == kPatchRowsShort ? 2 : 1) void conv3x3_f32_kernel(const ConvParams P) {
   constexpr int kChanStride = PROWS * kLdsPitch + 16;  // == 16 (mod 64)
   constexpr int kPatchFloats = kChunk * kChanStride;
   constexpr int kThreads = 64 * WAVES;
@@ -345,18 +349,30 @@ struct ConvTile {
 
 static const int kNtVariants[] = {8, 16, 25, 29};
 
-// Picks (NT, R, TW) minimising the modelled time ceil(blocks / 256) * NT / rate(NT): a workgroup's
-// time is proportional to NT, 256 CUs run one workgroup each per round, and the four-wave variant
-// (NT = 8) stages the same filter chunk for a third of the pixels: measured at full tiles it
-// reaches 0.68 of the rate of the eight-wave variants (80 against 115-120 TFLOP/s), NT = 29 0.95.
+// staged patch rows of the instance that serves R output rows per workgroup
+static int patch_rows_for(int nt, uint32_t R) {
+  if (nt == 8) return kPatchRows;  // the four-wave variant has one form
+  if (R > (uint32_t)kMaxR) return kPatchRowsTall;
+  return nt == 16 && R <= (uint32_t)kMaxRShort ? kPatchRowsShort : kPatchRows;
+}
+
+// Picks (NT, R, TW) minimising the modelled time: a workgroup's time is proportional to NT / rate(NT) and 256 CUs
+// run one workgroup each per round.  Rates measured at full tiles, relative to NT = 25 (115-120 TFLOP/s): the
+// four-wave variant (NT = 8) stages the same filter chunk for a third of the pixels, 0.68; NT = 16 alone on a
+// CU 0.9; NT = 29 0.95; the tall variant 0.95 of its NT's.  The short variant of NT = 16 runs two workgroups per
+// CU, each at half the pace of NT = 16 at rate 1.0 (125-133 TFLOP/s at 8 x 32 tiles); a last round that leaves
+// every CU one workgroup runs like NT = 16 alone.
 static ConvTile choose_tile(uint32_t OH, uint32_t OW, uint64_t planes, uint32_t o_groups) {
   ConvTile best = {0, 0, 0, 0};
   double best_cost = 1e300;
   for (int nt : kNtVariants) {
     const uint32_t cap = 16u * nt;
     const uint32_t max_cols = OW < (uint32_t)kMaxTW ? OW : (uint32_t)kMaxTW;
-    for (uint32_t ncol = (OW + max_cols - 1) / max_cols; ncol <= OW && ncol <= (OW + max_cols - 1) / max_cols + 2; ++ncol) {
+    const uint32_t ncol0 = (OW + max_cols - 1) / max_cols;
+    for (uint32_t ncol = ncol0; ncol <= OW; ++ncol) {
       const uint32_t TW = (OW + ncol - 1) / ncol;
+      // the widest few column tilings, and for the 16-tile variants everything down to 24 columns (8 x 32 fills it)
+      if (ncol > ncol0 + 2 && !(nt == 16 && TW >= 24u)) break;
       if (TW == 0 || TW > (uint32_t)kMaxTW || TW > cap) continue;
       uint32_t Rmax = cap / TW;
       const uint32_t max_r = nt == 8 ? (uint32_t)kMaxR : (uint32_t)kMaxRTall;  // the four-wave variant has no tall form
@@ -365,10 +381,16 @@ static ConvTile choose_tile(uint32_t OH, uint32_t OW, uint64_t planes, uint32_t 
       for (uint32_t R = 1; R <= Rmax; ++R) {
         const uint64_t tiles_y = (OH + R - 1) / R;
         const uint64_t blocks = tiles_y * ncol * planes * o_groups;
-        const uint64_t rounds = (blocks + 255) / 256;
-        // second-order term prefers fewer, fuller workgroups when rounds tie
-        const double rate = (nt == 8 ? 0.68 : nt == 29 ? 0.95 : 1.0) * (R > (uint32_t)kMaxR ? 0.95 : 1.0);
-        const double cost = ((double)rounds * nt + 1e-6 * (double)blocks * nt) / rate;
+        const int prows = patch_rows_for(nt, R);
+        double cost;
+        if (prows == kPatchRowsShort) {
+          const uint64_t rest = blocks % 512;
+          cost = (double)(blocks / 512) * 2.0 * nt + (rest == 0 ? 0.0 : rest <= 256 ? nt / 0.9 : 2.0 * nt);
+        } else {
+          const double rate = (nt == 8 ? 0.68 : nt == 16 ? 0.9 : nt == 29 ? 0.95 : 1.0) * (prows == kPatchRowsTall ? 0.95 : 1.0);
+          cost = (double)((blocks + 255) / 256) * nt / rate;
+        }
+        cost += 1e-6 * (double)blocks * nt;  // prefers fewer, fuller workgroups when rounds tie
         if (cost < best_cost) {
           best_cost = cost;
           best.nt = nt; best.R = R; best.TW = TW; best.blocks = blocks;
@@ -388,7 +410,9 @@ static void launch_conv_rows(const ConvParams &P, dim3 grid, hipStream_t st) {
 }
 template <int NT, int WAVES>
 static void launch_conv(const ConvParams &P, dim3 grid, hipStream_t st) {
-  if (WAVES == 8 && P.R > (uint32_t)kMaxR) launch_conv_rows<NT, WAVES, (WAVES == 8 ? kPatchRowsTall : kPatchRows)>(P, grid, st);
+  const int prows = patch_rows_for(NT, P.R);
+  if (WAVES == 8 && prows == kPatchRowsTall) launch_conv_rows<NT, WAVES, (WAVES == 8 ? kPatchRowsTall : kPatchRows)>(P, grid, st);
+  else if (NT == 16 && prows == kPatchRowsShort) launch_conv_rows<NT, WAVES, (NT == 16 ? kPatchRowsShort : kPatchRows)>(P, grid, st);
   else launch_conv_rows<NT, WAVES, kPatchRows>(P, grid, st);
 }
 
@@ -475,7 +499,7 @@ static int conv_direct_kernel_name(int which, uint32_t num_tiles, uint32_t N, ui
   const ConvTile tile = choose_tile(OH, OW, (uint64_t)N * num_tiles, (cout_k + 63u) / 64u);
   if (tile.nt == 0) return ADH_EINVAL;
   const int waves = tile.nt == 8 ? 4 : 8;
-  const int prows = (waves == 8 && tile.R > (uint32_t)kMaxR) ? kPatchRowsTall : kPatchRows;
+  const int prows = patch_rows_for(tile.nt, tile.R);
   snprintf(name, name_bytes, "conv3x3_f32_kernel<%d, %d, %s, %d>", tile.nt, waves, which == ADH_CONV_FWD ? "false" : "true", prows);
   return ADH_OK;
 }
