@@ -413,11 +413,14 @@ template <typename Op>
 bool use_3x3_kernels(const Op &op, const TileDims &d, uint32_t n, size_t filters) {
   return op.is_3x3_unit() && (uint64_t)d.H * d.W > 64u && fits_3x3_kernels(d, n, filters);
 }
-// The 3x3 backward-filter kernel streams an image's rows through a ring and pays the ring's fill once per image:
-// on tiles of at most 256 pixels (8x32: 0.61 ms against 0.56) the general kernel's units of 64 pixels are faster.
+// The 3x3 backward-filter kernel streams an image's rows through a ring and pays the ring's fill once per image
+// plane; its workgroups walk several planes, so with many planes (images x tiles) it is the faster one down to
+// tiles of 64 pixels (4x16 tiles, 128 planes, 512 channels: 0.48 ms against 0.57; 2x8: 0.21 against 0.17).  With
+// few planes the general kernel's units of 64 pixels win on tiles of at most 256 pixels.
 template <typename Op>
 bool use_3x3_filter_kernel(const Op &op, const TileDims &d, uint32_t n, size_t filters) {
-  return op.is_3x3_unit() && (uint64_t)d.H * d.W > 256u && fits_3x3_kernels(d, n, filters);
+  const uint64_t pixels = (uint64_t)d.H * d.W;
+  return op.is_3x3_unit() && (pixels > 256u || (pixels >= 64u && (uint64_t)d.N * n >= 64u)) && fits_3x3_kernels(d, n, filters);
 }
 
 // With unexchanged rows the forward kernel and the filter-gradient kernel must both be the 3x3 ones, which can
