@@ -61,6 +61,10 @@ SIGNATURES = {
     "adh_conv2d_slab_fwd_tiles": (i32, [i32] + [u32] * 12 + [vpp, vp, vpp, f32, vp, sz, vp]),
     "adh_conv2d_slab_bwd_data_tiles": (i32, [i32] + [u32] * 12 + [vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv2d_slab_bwd_filter_tiles": (i32, [i32] + [u32] * 12 + [vpp, vpp, vp, f32, vp, sz, vp]),
+    "adh_conv2d_unpadded_workspace_bytes": (sz, [i32, i32] + [u32] * 14),
+    "adh_conv2d_unpadded_fwd_tiles": (i32, [i32] + [u32] * 14 + [vpp, vp, vpp, f32, vp, sz, vp]),
+    "adh_conv2d_unpadded_bwd_data_tiles": (i32, [i32] + [u32] * 14 + [vp, vpp, vpp, f32, vp, sz, vp]),
+    "adh_conv2d_unpadded_bwd_filter_tiles": (i32, [i32] + [u32] * 14 + [vpp, vpp, vp, f32, vp, sz, vp]),
     "adh_batchnorm2d_workspace_bytes": (sz, [u32, u32, u32]),
     "adh_batchnorm2d_fwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, f32, i32, u32, vpp, vpp, vpp, vpp, vpp, vpp, vpp,
                                         vpp, vpp, vpp, vp, sz, vp]),
@@ -323,6 +327,38 @@ def conv2d_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, HP, WP, kh, kw, sh, sw, d
     wp, wb = _ws(ws)
     return lib().adh_conv2d_slab_bwd_filter_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw_,
                                                   xt, dt, dw.data_ptr(), beta, wp, wb, _stream())
+
+
+def conv2d_unpadded_workspace_bytes(which, dtype, K, N, Cin, Cout, H, W, kh, kw, sh, sw, dh, dw, pad_h, pad_w):
+    return lib().adh_conv2d_unpadded_workspace_bytes(which, dtype, K, N, Cin, Cout, H, W, kh, kw, sh, sw, dh, dw, pad_h, pad_w)
+
+
+def conv2d_unpadded_fwd_tiles(xs, w, ys, N, Cin, Cout, H, W, kh, kw, sh, sw, dh, dw, pad_h, pad_w, beta=0.0, ws=None):
+    """Row tiles without halo, any window / stride / dilation: rows outside a tile come from its neighbours."""
+    _dev(*xs, w, *ys)
+    xt, k1 = _tbl(xs)
+    yt, k2 = _tbl(ys)
+    wp, wb = _ws(ws)
+    return lib().adh_conv2d_unpadded_fwd_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, kh, kw, sh, sw, dh, dw, pad_h, pad_w,
+                                               xt, w.data_ptr(), yt, beta, wp, wb, _stream())
+
+
+def conv2d_unpadded_bwd_data_tiles(w, dys, dxs, N, Cin, Cout, H, W, kh, kw, sh, sw, dh, dw, pad_h, pad_w, beta=0.0, ws=None):
+    _dev(w, *dys, *dxs)
+    dt, k1 = _tbl(dys)
+    gt, k2 = _tbl(dxs)
+    wp, wb = _ws(ws)
+    return lib().adh_conv2d_unpadded_bwd_data_tiles(_dt(dys[0]), len(dys), N, Cin, Cout, H, W, kh, kw, sh, sw, dh, dw, pad_h,
+                                                    pad_w, w.data_ptr(), dt, gt, beta, wp, wb, _stream())
+
+
+def conv2d_unpadded_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, H, W, kh, kw, sh, sw, dh, dw_, pad_h, pad_w, beta=0.0, ws=None):
+    _dev(*xs, *dys, dw)
+    xt, k1 = _tbl(xs)
+    dt, k2 = _tbl(dys)
+    wp, wb = _ws(ws)
+    return lib().adh_conv2d_unpadded_bwd_filter_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, kh, kw, sh, sw, dh, dw_, pad_h,
+                                                      pad_w, xt, dt, dw.data_ptr(), beta, wp, wb, _stream())
 
 
 def _opt_tbl(ts):

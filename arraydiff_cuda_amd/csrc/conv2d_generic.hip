@@ -50,6 +50,10 @@ struct ConvGenParams {
   uint32_t NB, NG, live, PPI;
   uint32_t PCP, PP, w_lds_floats;
   uint32_t nsub, blocks_per_image;
+  // the tiles are the row tiles of one tensor in rank order and carry no halo (the NBR instances of the kernel):
+  // input rows -in_H .. -1 of tile t > 0 are the last rows of tile t - 1, rows in_H .. 2 in_H - 1 of tile
+  // t < num_tiles - 1 the first rows of tile t + 1; what lies outside the tensor is zero
+  uint32_t num_tiles;
   float beta;
   FastDiv div_bpi, div_MG, div_N, div_PCP, div_BC, div_live, div_PPI;
   GenSub sub[kGenMaxSub];
@@ -73,6 +77,11 @@ __device__ __forceinline__ float gen_ld_b(const float *base, uint32_t boff) {
 }
 __device__ __forceinline__ float gen_ld_b(const uint16_t *base, uint32_t boff) {
   return bf16_bits_to_f32(*reinterpret_cast<const uint16_t *>(reinterpret_cast<const char *>(base) + boff));
+}
+// p: the lane's own address
+__device__ __forceinline__ float gen_ld_p(const float *, const char *p) { return *reinterpret_cast<const float *>(p); }
+__device__ __forceinline__ float gen_ld_p(const uint16_t *, const char *p) {
+  return bf16_bits_to_f32(*reinterpret_cast<const uint16_t *>(p));
 }
 __device__ __forceinline__ void gen_st(float *p, size_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void gen_st(uint16_t *p, size_t i, float v) { p[i] = f32_to_bf16_bits(v); }
@@ -101,7 +110,9 @@ __global__ __launch_bounds__(256) void conv_gen_filter_kernel(const FilterGenPar
 // The next (chunk, tap group)'s patch and filter rows are loaded into registers while the current
 // one is multiplied; they go to LDS after the barrier that ends the current one.  The register
 // budget is held to half the file, so that two workgroups share a CU and hide each other's barriers.
-template <typename T, int CC, int MT>
+// NBR: the input tiles carry no halo and rows outside a tile are read from the neighbouring tiles (P.num_tiles):
+// a staged element then has an address of its own instead of an offset from the tile's.
+template <typename T, int CC, int MT, bool NBR = false>
 __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenParams P) {
   constexpr uint32_t MW = 16u * MT;                         // m per block
   constexpr uint32_t WPITCH = MT == 1 ? 16u : MW + 16u;     // filter row pitch: the 4 channel groups 16 banks apart
@@ -158,6 +169,7 @@ __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenP
   // a byte offset into the channel plane of the block's first image, and a bit per element that exists; the
   // elements that do not (outside the input or the patch) load offset 0 and are replaced by zero
   uint32_t src_boff[PFC], src_ok = 0;
+  const char *src_ptr[NBR ? PFC : 1];  // NBR: the element's address in channel 0 of the block's first image
 #pragma unroll
   for (int j = 0; j < PFC; ++j) {
     const uint32_t e = tid + j * kGenThreads;
@@ -165,9 +177,28 @@ __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenP
     P.div_PPI.divmod(e, b, ei);
     P.div_PCP.divmod(ei, r, col);
     const int32_t gr = in_r0 + (int32_t)r, gc = in_c0 + (int32_t)col;
-    const bool ok = b < P.NB && n + b < P.N && r < S.PR && col < S.PC && gr >= 0 && gr < (int32_t)P.in_H && gc >= 0 &&
-                    gc < (int32_t)P.in_W;
-    src_boff[j] = ok ? (uint32_t)((int32_t)b * image_elems + gr * (int32_t)P.in_W + gc) * (uint32_t)sizeof(T) : 0u;
+    bool ok = b < P.NB && n + b < P.N && r < S.PR && col < S.PC && gc >= 0 && gc < (int32_t)P.in_W;
+    if constexpr (!NBR) {
+      ok = ok && gr >= 0 && gr < (int32_t)P.in_H;
+      src_boff[j] = ok ? (uint32_t)((int32_t)b * image_elems + gr * (int32_t)P.in_W + gc) * (uint32_t)sizeof(T) : 0u;
+    } else {
+      int32_t row = gr;
+      uint32_t from = tile;
+      if (gr < 0) {
+        row = gr + (int32_t)P.in_H;
+        ok = ok && tile > 0u;
+        from = tile > 0u ? tile - 1u : tile;
+      } else if (gr >= (int32_t)P.in_H) {
+        row = gr - (int32_t)P.in_H;
+        ok = ok && tile + 1u < P.num_tiles;
+        from = tile + 1u < P.num_tiles ? tile + 1u : tile;
+      }
+      ok = ok && row >= 0 && row < (int32_t)P.in_H;
+      const T *base = reinterpret_cast<const T *>(P.in[from]) + (size_t)n * P.C * P.in_H * P.in_W;
+      src_boff[j] = 0u;
+      src_ptr[j] = reinterpret_cast<const char *>(base) +
+                   (ok ? (size_t)((int32_t)b * image_elems + row * (int32_t)P.in_W + gc) * sizeof(T) : (size_t)0);
+    }
     src_ok |= ok ? 1u << j : 0u;
   }
 
@@ -180,9 +211,13 @@ __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenP
     pre_ch = ch;
 #pragma unroll
     for (int c = 0; c < CC; ++c) {
-      const T *pl = src + (size_t)min(ch * CC + c, P.C - 1u) * plane;
+      const size_t chan = (size_t)min(ch * CC + c, P.C - 1u) * plane;
+      const T *pl = src + chan;
 #pragma unroll
-      for (int j = 0; j < PFC; ++j) pre[c * PFC + j] = gen_ld_b(pl, src_boff[j]);
+      for (int j = 0; j < PFC; ++j) {
+        if constexpr (NBR) pre[c * PFC + j] = gen_ld_p(src, src_ptr[j] + chan * sizeof(T));
+        else pre[c * PFC + j] = gen_ld_b(pl, src_boff[j]);
+      }
     }
   };
   auto store_patch = [&]() {
@@ -309,6 +344,7 @@ struct GenPlan {
   FilterGenParams F;
   size_t lds_bytes, wt_bytes;
   uint32_t MT, num_tiles;
+  bool nbr;  // tiles without halo: the kernel instances that read rows from the neighbouring tiles
 };
 // a launch of fewer blocks than this (two per compute unit) is split finer
 constexpr uint64_t kGenFillBlocks = 512;
@@ -490,18 +526,20 @@ static int gen_check_shape(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_
   return ADH_OK;
 }
 
-static int gen_plan_fwd(const GenShape &g, GenPlan *plan) {
+// pad_h, pad_w: the input tile carries no halo (it is g.HP - 2 pad_h rows by g.WP - 2 pad_w columns) and the taps
+// reach pad_h rows and pad_w columns before its first pixel
+static int gen_plan_fwd(const GenShape &g, GenPlan *plan, uint32_t pad_h = 0, uint32_t pad_w = 0) {
   ConvGenParams &P = plan->P;
   P.N = g.N; P.C = g.Cin; P.M = g.Cout;
-  P.in_H = g.HP; P.in_W = g.WP; P.out_H = g.OH; P.out_W = g.OW;
+  P.in_H = g.HP - 2u * pad_h; P.in_W = g.WP - 2u * pad_w; P.out_H = g.OH; P.out_W = g.OW;
   P.si_r = g.sh; P.si_c = g.sw; P.so_r = 1; P.so_c = 1;
   P.ntaps = g.kh * g.kw;
   P.nsub = 1;
   for (uint32_t a = 0; a < g.kh; ++a)
     for (uint32_t b = 0; b < g.kw; ++b) {
       const uint32_t t = a * g.kw + b;
-      P.off_r[t] = (int16_t)(a * g.dh);
-      P.off_c[t] = (int16_t)(b * g.dw);
+      P.off_r[t] = (int16_t)((int32_t)(a * g.dh) - (int32_t)pad_h);
+      P.off_c[t] = (int16_t)((int32_t)(b * g.dw) - (int32_t)pad_w);
       plan->F.tap_index[t] = (uint16_t)t;
     }
   GenSub &S = P.sub[0];
@@ -511,31 +549,39 @@ static int gen_plan_fwd(const GenShape &g, GenPlan *plan) {
   return gen_finish_plan(plan);
 }
 
-static int gen_plan_bwd_data(const GenShape &g, GenPlan *plan) {
+// pad_h, pad_w (with `unpadded`): the gradient tile carries no halo: only the pixels pad_h .. pad_h + H - 1 by
+// pad_w .. pad_w + W - 1 of the padded gradient are computed, and they are stored from (0, 0) on.
+static int gen_plan_bwd_data(const GenShape &g, GenPlan *plan, bool unpadded = false, uint32_t pad_h = 0, uint32_t pad_w = 0) {
   ConvGenParams &P = plan->P;
+  if (!unpadded) pad_h = pad_w = 0;
+  const uint32_t H = g.HP - 2u * pad_h, W = g.WP - 2u * pad_w;  // the gradient tile
   P.N = g.N; P.C = g.Cout; P.M = g.Cin;
-  P.in_H = g.OH; P.in_W = g.OW; P.out_H = g.HP; P.out_W = g.WP;
+  P.in_H = g.OH; P.in_W = g.OW; P.out_H = H; P.out_W = W;
   P.si_r = 1; P.si_c = 1; P.so_r = g.sh; P.so_c = g.sw;
   P.ntaps = g.kh * g.kw;
   uint32_t nsub = 0, t = 0;
   for (uint32_t pr = 0; pr < g.sh && pr < g.HP; ++pr)
     for (uint32_t pc = 0; pc < g.sw && pc < g.WP; ++pc) {
       GenSub &S = P.sub[nsub++];
+      // the class's first padded row / column inside the tile: pr + sh * i0 >= pad_h
+      const uint32_t i0 = pad_h > pr ? (pad_h - pr + g.sh - 1u) / g.sh : 0u;
+      const uint32_t j0 = pad_w > pc ? (pad_w - pc + g.sw - 1u) / g.sw : 0u;
+      const uint32_t r_first = pr + g.sh * i0 - pad_h, c_first = pc + g.sw * j0 - pad_w;
       S.t0 = t;
       for (uint32_t a = 0; a < g.kh; ++a)
         for (uint32_t b = 0; b < g.kw; ++b) {
           if ((a * g.dh) % g.sh != pr || (b * g.dw) % g.sw != pc) continue;
-          // dy row of padded row h' = pr + sh * i under tap a: (h' - a*dh) / sh = i + (pr - a*dh) / sh
-          P.off_r[t] = (int16_t)(((int32_t)pr - (int32_t)(a * g.dh)) / (int32_t)g.sh);
-          P.off_c[t] = (int16_t)(((int32_t)pc - (int32_t)(b * g.dw)) / (int32_t)g.sw);
+          // dy row of padded row h' = pr + sh * (i0 + i) under tap a: (h' - a*dh) / sh = i + i0 + (pr - a*dh) / sh
+          P.off_r[t] = (int16_t)((int32_t)i0 + ((int32_t)pr - (int32_t)(a * g.dh)) / (int32_t)g.sh);
+          P.off_c[t] = (int16_t)((int32_t)j0 + ((int32_t)pc - (int32_t)(b * g.dw)) / (int32_t)g.sw);
           plan->F.tap_index[t] = (uint16_t)(a * g.kw + b);
           ++t;
         }
       S.t1 = t;
-      S.GI = (g.HP - pr + g.sh - 1u) / g.sh;
-      S.GJ = (g.WP - pc + g.sw - 1u) / g.sw;
-      S.o_r = pr;
-      S.o_c = pc;
+      S.GI = r_first < H ? (H - r_first + g.sh - 1u) / g.sh : 0u;
+      S.GJ = c_first < W ? (W - c_first + g.sw - 1u) / g.sw : 0u;
+      S.o_r = r_first;
+      S.o_c = c_first;
     }
   P.nsub = nsub;
   plan->F.m_stride = g.kh * g.kw;
@@ -543,21 +589,26 @@ static int gen_plan_bwd_data(const GenShape &g, GenPlan *plan) {
   return gen_finish_plan(plan);
 }
 
-template <typename T, int CC>
+template <typename T, int CC, bool NBR>
 static void launch_gen_cc(const GenPlan &plan, uint32_t blocks, hipStream_t st) {
   if (plan.MT == 1u)
-    hipLaunchKernelGGL((conv_gen_kernel<T, CC, 1>), dim3(blocks), dim3(kGenThreads), plan.lds_bytes, st, plan.P);
+    hipLaunchKernelGGL((conv_gen_kernel<T, CC, 1, NBR>), dim3(blocks), dim3(kGenThreads), plan.lds_bytes, st, plan.P);
   else if (plan.MT == 2u)
-    hipLaunchKernelGGL((conv_gen_kernel<T, CC, 2>), dim3(blocks), dim3(kGenThreads), plan.lds_bytes, st, plan.P);
+    hipLaunchKernelGGL((conv_gen_kernel<T, CC, 2, NBR>), dim3(blocks), dim3(kGenThreads), plan.lds_bytes, st, plan.P);
   else
-    hipLaunchKernelGGL((conv_gen_kernel<T, CC, 4>), dim3(blocks), dim3(kGenThreads), plan.lds_bytes, st, plan.P);
+    hipLaunchKernelGGL((conv_gen_kernel<T, CC, 4, NBR>), dim3(blocks), dim3(kGenThreads), plan.lds_bytes, st, plan.P);
+}
+template <typename T, bool NBR>
+static void launch_gen_nbr(const GenPlan &plan, uint32_t blocks, hipStream_t st) {
+  if (plan.P.CC == 32u) launch_gen_cc<T, 32, NBR>(plan, blocks, st);
+  else if (plan.P.CC == 16u) launch_gen_cc<T, 16, NBR>(plan, blocks, st);
+  else if (plan.P.CC == 8u) launch_gen_cc<T, 8, NBR>(plan, blocks, st);
+  else launch_gen_cc<T, 4, NBR>(plan, blocks, st);
 }
 template <typename T>
 static void launch_gen(const GenPlan &plan, uint32_t blocks, hipStream_t st) {
-  if (plan.P.CC == 32u) launch_gen_cc<T, 32>(plan, blocks, st);
-  else if (plan.P.CC == 16u) launch_gen_cc<T, 16>(plan, blocks, st);
-  else if (plan.P.CC == 8u) launch_gen_cc<T, 8>(plan, blocks, st);
-  else launch_gen_cc<T, 4>(plan, blocks, st);
+  if (plan.nbr) launch_gen_nbr<T, true>(plan, blocks, st);
+  else launch_gen_nbr<T, false>(plan, blocks, st);
 }
 
 static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *w, void *workspace,
@@ -572,6 +623,7 @@ static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *
   plan->F.w = w;
   plan->F.wt = reinterpret_cast<float *>(workspace);
   P.wt = plan->F.wt;
+  P.num_tiles = num_tiles;
   const uint32_t fblocks = (uint32_t)std::min<size_t>(1024, (plan->wt_bytes / 4u + 255u) / 256u);
   if (dtype == ADH_F32) {
     hipLaunchKernelGGL(conv_gen_filter_kernel<float>, dim3(fblocks), dim3(256), 0, st, plan->F);
@@ -612,6 +664,10 @@ struct WgradGenParams {
   // side in a plane, PPI apart).  NG = ceil(N / NBU) image groups per tile.
   uint32_t NBU, NG, img_pix, PPI;
   uint32_t PR, PC, PCP, PP, DP, dy_lds_floats;
+  // the NBR instances: x carries no halo (HP x WP is the tile itself), the taps reach pad_h rows and pad_w columns
+  // before its first pixel, rows outside the tile are the neighbouring row tiles' (tiles in rank order), what
+  // lies outside the tensor is zero
+  uint32_t pad_h, pad_w, num_tiles;
   FastDiv div_COG, div_CIT, div_ntg, div_ncb, div_nrb, div_N, div_OWT, div_PC, div_PR, div_img_pix, div_PRPC;
   int16_t off_r[kGenMaxTaps], off_c[kGenMaxTaps];
 };
@@ -619,7 +675,7 @@ struct WgradGenParams {
 // PACKED (few input channels, e.g. the 3-channel stem): the 16 columns of an accumulator tile are 16
 // (tap, input channel) pairs, pair q = 16 t + column = tap * Cin + ci, instead of 16 input channels of one tap;
 // all taps then fit one block and no matrix column is spent on channels that do not exist.
-template <typename T, int TAPS, bool PACKED>
+template <typename T, int TAPS, bool PACKED, bool NBR = false>
 __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const WgradGenParams P) {
   extern __shared__ __align__(16) float gen_lds[];
   float *dyl = gen_lds;
@@ -704,12 +760,38 @@ __global__ __launch_bounds__(kWgGenThreads, 2) void conv_gen_wgrad_kernel(const 
       dy_pre[c] = gen_ld_b(ds + (ptrdiff_t)(dy_c0 + min(c, dy_cmax)) * (ptrdiff_t)dy_plane, dy_off);
 #pragma unroll
     for (int k = 0; k < KP; ++k) {
-      const bool in = pr_rc[k] != 0xffffffffu && n + pr_b[k] < P.N && oh0 * P.sh + (pr_rc[k] >> 16) < P.HP &&
-                      ow0 * P.sw + (pr_rc[k] & 0xffffu) < P.WP;
-      pre_in |= in ? 2u << k : 0u;
-      const uint32_t off = in ? x_boff[k] : 0u;
+      if constexpr (!NBR) {
+        const bool in = pr_rc[k] != 0xffffffffu && n + pr_b[k] < P.N && oh0 * P.sh + (pr_rc[k] >> 16) < P.HP &&
+                        ow0 * P.sw + (pr_rc[k] & 0xffffu) < P.WP;
+        pre_in |= in ? 2u << k : 0u;
+        const uint32_t off = in ? x_boff[k] : 0u;
 #pragma unroll
-      for (int c = 0; c < 16; ++c) x_pre[k][c] = gen_ld_b(xs + (size_t)min((uint32_t)c, planes - 1u) * x_plane, off);
+        for (int c = 0; c < 16; ++c) x_pre[k][c] = gen_ld_b(xs + (size_t)min((uint32_t)c, planes - 1u) * x_plane, off);
+      } else {
+        // the place's row and column in the tile; a row outside it is the neighbouring tile's
+        const int32_t gr = (int32_t)(oh0 * P.sh + (pr_rc[k] >> 16)) - (int32_t)P.pad_h;
+        const int32_t gc = (int32_t)(ow0 * P.sw + (pr_rc[k] & 0xffffu)) - (int32_t)P.pad_w;
+        int32_t row = gr;
+        uint32_t from = tile;
+        bool in = pr_rc[k] != 0xffffffffu && n + pr_b[k] < P.N && gc >= 0 && gc < (int32_t)P.WP;
+        if (gr < 0) {
+          row = gr + (int32_t)P.HP;
+          in = in && tile > 0u;
+          from = tile > 0u ? tile - 1u : tile;
+        } else if (gr >= (int32_t)P.HP) {
+          row = gr - (int32_t)P.HP;
+          in = in && tile + 1u < P.num_tiles;
+          from = tile + 1u < P.num_tiles ? tile + 1u : tile;
+        }
+        in = in && row >= 0 && row < (int32_t)P.HP;
+        pre_in |= in ? 2u << k : 0u;
+        // a place that does not exist loads the first element of the unit's first image instead
+        const char *px = reinterpret_cast<const char *>(reinterpret_cast<const T *>(P.x[from]) + ((size_t)n * P.Cin + cit * 16u) * x_plane) +
+                         (in ? ((size_t)pr_b[k] * P.Cin * x_plane + (size_t)row * P.WP + (size_t)gc) * sizeof(T) : (size_t)0);
+#pragma unroll
+        for (int c = 0; c < 16; ++c)
+          x_pre[k][c] = gen_ld_p(xs, px + (size_t)min((uint32_t)c, planes - 1u) * x_plane * sizeof(T));
+      }
     }
   };
   auto store_unit = [&]() {
@@ -822,12 +904,17 @@ struct WgradGenPlan {
   WgradGenParams P;
   size_t lds_bytes, partial_bytes;
   uint32_t blocks, nparts;
-  bool packed;
+  bool packed, nbr;
 };
 
-static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *plan) {
+// pad_h, pad_w (with `unpadded`): x carries no halo and is g.HP - 2 pad_h rows by g.WP - 2 pad_w columns
+static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *plan, bool unpadded = false, uint32_t pad_h = 0,
+                          uint32_t pad_w = 0) {
   WgradGenParams &P = plan->P;
-  P.N = g.N; P.Cin = g.Cin; P.Cout = g.Cout; P.HP = g.HP; P.WP = g.WP; P.OH = g.OH; P.OW = g.OW;
+  if (!unpadded) pad_h = pad_w = 0;
+  plan->nbr = unpadded;
+  P.pad_h = pad_h; P.pad_w = pad_w; P.num_tiles = num_tiles;
+  P.N = g.N; P.Cin = g.Cin; P.Cout = g.Cout; P.HP = g.HP - 2u * pad_h; P.WP = g.WP - 2u * pad_w; P.OH = g.OH; P.OW = g.OW;
   P.sh = g.sh; P.sw = g.sw;
   P.ntaps = g.kh * g.kw;
   P.T = P.ntaps == 1u ? 1u : P.ntaps <= 4u ? 4u : 9u;
@@ -898,51 +985,73 @@ static int gen_plan_wgrad(const GenShape &g, uint32_t num_tiles, WgradGenPlan *p
   return ADH_OK;
 }
 
-template <typename T>
-static void launch_wgrad_gen(const WgradGenPlan &plan, hipStream_t st) {
+template <typename T, bool NBR>
+static void launch_wgrad_gen_nbr(const WgradGenPlan &plan, hipStream_t st) {
   const WgradGenParams &P = plan.P;
   if (plan.packed && P.T == 4u)
-    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 4, true>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 4, true, NBR>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
   else if (plan.packed)
-    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 10, true>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 10, true, NBR>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
   else if (P.T == 1u)
-    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 1, false>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 1, false, NBR>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
   else if (P.T == 4u)
-    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 4, false>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 4, false, NBR>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
   else
-    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 9, false>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+    hipLaunchKernelGGL((conv_gen_wgrad_kernel<T, 9, false, NBR>), dim3(plan.blocks), dim3(kWgGenThreads), plan.lds_bytes, st, P);
+}
+template <typename T>
+static void launch_wgrad_gen(const WgradGenPlan &plan, hipStream_t st) {
+  if (plan.nbr) launch_wgrad_gen_nbr<T, true>(plan, st);
+  else launch_wgrad_gen_nbr<T, false>(plan, st);
 }
 
 }  // namespace adh
 
 using namespace adh;
 
-extern "C" {
+namespace {
 
-size_t adh_conv2d_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
-                                  uint32_t HP, uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw,
-                                  uint32_t dh, uint32_t dw) {
+// Tiles without halo: the extents the padded form of the same convolution would have, and whether the row split
+// is one the kernels serve.  H, W: the tile.  The tile's output must be H / sh rows (then any number of row tiles
+// stitches to the unsplit output), and the taps may reach into the neighbouring tiles only.
+int unpadded_geometry(uint32_t H, uint32_t W, uint32_t kh, uint32_t sh, uint32_t dh, uint32_t pad_h, uint32_t pad_w,
+                      uint32_t *HP, uint32_t *WP) {
+  if (H == 0 || W == 0 || sh == 0 || kh == 0 || dh == 0) return ADH_EINVAL;
+  if (pad_h > 4096u || pad_w > 4096u) return ADH_EINVAL;
+  const uint64_t eh = (uint64_t)(kh - 1u) * dh + 1u;
+  if (H % sh != 0u) return ADH_EINVAL;
+  // floor((H + 2 pad_h - eh) / sh) + 1 == H / sh
+  if (2ull * pad_h >= eh || eh - 2ull * pad_h > sh) return ADH_EINVAL;
+  if (pad_h > H || eh - 1u - pad_h > H) return ADH_EINVAL;
+  *HP = H + 2u * pad_h;
+  *WP = W + 2u * pad_w;
+  return ADH_OK;
+}
+
+size_t conv2d_workspace(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,
+                        uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw,
+                        bool unpadded, uint32_t pad_h, uint32_t pad_w) {
   GenShape g;
   if (!dtype_ok(dtype) || gen_check_shape(num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, &g)) return 0;
   if (N == 0 || Cin == 0 || Cout == 0) return 0;
   if (which == ADH_CONV_BWD_FILTER) {
     WgradGenPlan wp = {};
-    if (gen_plan_wgrad(g, num_tiles, &wp)) return 0;
+    if (gen_plan_wgrad(g, num_tiles, &wp, unpadded, pad_h, pad_w)) return 0;
     return (wp.partial_bytes + 255u) & ~(size_t)255u;
   }
   GenPlan plan = {};
   plan.num_tiles = num_tiles;
   int e = ADH_EINVAL;
-  if (which == ADH_CONV_FWD) e = gen_plan_fwd(g, &plan);
-  else if (which == ADH_CONV_BWD_DATA) e = gen_plan_bwd_data(g, &plan);
+  if (which == ADH_CONV_FWD) e = gen_plan_fwd(g, &plan, unpadded ? pad_h : 0u, unpadded ? pad_w : 0u);
+  else if (which == ADH_CONV_BWD_DATA) e = gen_plan_bwd_data(g, &plan, unpadded, pad_h, pad_w);
   if (e) return 0;
   return (plan.wt_bytes + 255u) & ~(size_t)255u;
 }
 
-int adh_conv2d_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,
-                              uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw,
-                              const void *const *x_pad_tiles, const void *w, void *const *y_tiles, float beta,
-                              void *workspace, size_t workspace_bytes, void *stream) {
+int conv2d_fwd(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP,
+               uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, bool unpadded, uint32_t pad_h,
+               uint32_t pad_w, const void *const *x_tiles, const void *w, void *const *y_tiles, float beta, void *workspace,
+               size_t workspace_bytes, void *stream) {
   if (!dtype_ok(dtype)) return ADH_EINVAL;
   GenShape g;
   int e = gen_check_shape(num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, &g);
@@ -950,27 +1059,28 @@ int adh_conv2d_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_
   if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
   if (N == 0 || Cout == 0) return ADH_OK;
   if (Cin == 0) return ADH_EINVAL;
-  if (!x_pad_tiles || !y_tiles || !w) return ADH_ENULL;
+  if (!x_tiles || !y_tiles || !w) return ADH_ENULL;
   GenPlan plan = {};
   plan.num_tiles = num_tiles;
-  e = gen_plan_fwd(g, &plan);
+  plan.nbr = unpadded;
+  e = gen_plan_fwd(g, &plan, unpadded ? pad_h : 0u, unpadded ? pad_w : 0u);
   if (e) return e;
   const size_t es = dtype_size(dtype);
   if (!aligned_to(w, es)) return ADH_EALIGN;
   for (uint32_t t = 0; t < num_tiles; ++t) {
-    if (!x_pad_tiles[t] || !y_tiles[t]) return ADH_ENULL;
-    if (!aligned_to(x_pad_tiles[t], es) || !aligned_to(y_tiles[t], es)) return ADH_EALIGN;
-    plan.P.in[t] = x_pad_tiles[t];
+    if (!x_tiles[t] || !y_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(x_tiles[t], es) || !aligned_to(y_tiles[t], es)) return ADH_EALIGN;
+    plan.P.in[t] = x_tiles[t];
     plan.P.out[t] = y_tiles[t];
   }
   plan.P.beta = beta;
   return gen_launch(dtype, &plan, num_tiles, w, workspace, workspace_bytes, as_stream(stream));
 }
 
-int adh_conv2d_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,
-                                   uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh,
-                                   uint32_t dw, const void *w, const void *const *dy_tiles, void *const *dx_pad_tiles,
-                                   float beta, void *workspace, size_t workspace_bytes, void *stream) {
+int conv2d_bwd_data(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP,
+                    uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, bool unpadded,
+                    uint32_t pad_h, uint32_t pad_w, const void *w, const void *const *dy_tiles, void *const *dx_tiles,
+                    float beta, void *workspace, size_t workspace_bytes, void *stream) {
   if (!dtype_ok(dtype)) return ADH_EINVAL;
   GenShape g;
   int e = gen_check_shape(num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, &g);
@@ -978,28 +1088,28 @@ int adh_conv2d_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, ui
   if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
   if (N == 0 || Cin == 0) return ADH_OK;
   if (Cout == 0) return ADH_EINVAL;
-  if (!dy_tiles || !dx_pad_tiles || !w) return ADH_ENULL;
+  if (!dy_tiles || !dx_tiles || !w) return ADH_ENULL;
   GenPlan plan = {};
   plan.num_tiles = num_tiles;
-  e = gen_plan_bwd_data(g, &plan);
+  plan.nbr = unpadded;
+  e = gen_plan_bwd_data(g, &plan, unpadded, pad_h, pad_w);
   if (e) return e;
   const size_t es = dtype_size(dtype);
   if (!aligned_to(w, es)) return ADH_EALIGN;
   for (uint32_t t = 0; t < num_tiles; ++t) {
-    if (!dy_tiles[t] || !dx_pad_tiles[t]) return ADH_ENULL;
-    if (!aligned_to(dy_tiles[t], es) || !aligned_to(dx_pad_tiles[t], es)) return ADH_EALIGN;
+    if (!dy_tiles[t] || !dx_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(dy_tiles[t], es) || !aligned_to(dx_tiles[t], es)) return ADH_EALIGN;
     plan.P.in[t] = dy_tiles[t];
-    plan.P.out[t] = dx_pad_tiles[t];
+    plan.P.out[t] = dx_tiles[t];
   }
   plan.P.beta = beta;
   return gen_launch(dtype, &plan, num_tiles, w, workspace, workspace_bytes, as_stream(stream));
 }
 
-
-int adh_conv2d_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,
-                                     uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh,
-                                     uint32_t dw, const void *const *x_pad_tiles, const void *const *dy_tiles,
-                                     float *dwt, float beta, void *workspace, size_t workspace_bytes, void *stream) {
+int conv2d_bwd_filter(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP,
+                      uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, bool unpadded,
+                      uint32_t pad_h, uint32_t pad_w, const void *const *x_tiles, const void *const *dy_tiles, float *dwt,
+                      float beta, void *workspace, size_t workspace_bytes, void *stream) {
   if (!dtype_ok(dtype)) return ADH_EINVAL;
   GenShape g;
   int e = gen_check_shape(num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, &g);
@@ -1013,15 +1123,15 @@ int adh_conv2d_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, 
     if (beta == 0.f) return adh_fill_f32((uint64_t)Cout * Cin * kh * kw, 0.f, dwt, stream);
     return ADH_OK;
   }
-  if (!x_pad_tiles || !dy_tiles) return ADH_ENULL;
+  if (!x_tiles || !dy_tiles) return ADH_ENULL;
   WgradGenPlan plan = {};
-  e = gen_plan_wgrad(g, num_tiles, &plan);
+  e = gen_plan_wgrad(g, num_tiles, &plan, unpadded, pad_h, pad_w);
   if (e) return e;
   const size_t es = dtype_size(dtype);
   for (uint32_t t = 0; t < num_tiles; ++t) {
-    if (!x_pad_tiles[t] || !dy_tiles[t]) return ADH_ENULL;
-    if (!aligned_to(x_pad_tiles[t], es) || !aligned_to(dy_tiles[t], es)) return ADH_EALIGN;
-    plan.P.x[t] = x_pad_tiles[t];
+    if (!x_tiles[t] || !dy_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(x_tiles[t], es) || !aligned_to(dy_tiles[t], es)) return ADH_EALIGN;
+    plan.P.x[t] = x_tiles[t];
     plan.P.dy[t] = dy_tiles[t];
   }
   if (!workspace) return ADH_ENULL;
@@ -1041,6 +1151,83 @@ int adh_conv2d_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, 
   hipLaunchKernelGGL(conv_gen_wgrad_reduce_kernel, dim3((uint32_t)std::min<size_t>((stride + 63u) / 64u, 65535u)),
                      dim3(256), 0, st, Q);
   return launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t adh_conv2d_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                  uint32_t HP, uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw,
+                                  uint32_t dh, uint32_t dw) {
+  return conv2d_workspace(which, dtype, num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, false, 0, 0);
+}
+
+int adh_conv2d_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,
+                              uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw,
+                              const void *const *x_pad_tiles, const void *w, void *const *y_tiles, float beta,
+                              void *workspace, size_t workspace_bytes, void *stream) {
+  return conv2d_fwd(dtype, num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, false, 0, 0, x_pad_tiles, w, y_tiles, beta,
+                    workspace, workspace_bytes, stream);
+}
+
+int adh_conv2d_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,
+                                   uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh,
+                                   uint32_t dw, const void *w, const void *const *dy_tiles, void *const *dx_pad_tiles,
+                                   float beta, void *workspace, size_t workspace_bytes, void *stream) {
+  return conv2d_bwd_data(dtype, num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, false, 0, 0, w, dy_tiles,
+                         dx_pad_tiles, beta, workspace, workspace_bytes, stream);
+}
+
+int adh_conv2d_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,
+                                     uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh,
+                                     uint32_t dw, const void *const *x_pad_tiles, const void *const *dy_tiles,
+                                     float *dwt, float beta, void *workspace, size_t workspace_bytes, void *stream) {
+  return conv2d_bwd_filter(dtype, num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, false, 0, 0, x_pad_tiles, dy_tiles,
+                           dwt, beta, workspace, workspace_bytes, stream);
+}
+
+size_t adh_conv2d_unpadded_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,
+                                           uint32_t Cout, uint32_t H, uint32_t W, uint32_t kh, uint32_t kw, uint32_t sh,
+                                           uint32_t sw, uint32_t dh, uint32_t dw, uint32_t pad_h, uint32_t pad_w) {
+  uint32_t HP, WP;
+  if (unpadded_geometry(H, W, kh, sh, dh, pad_h, pad_w, &HP, &WP)) return 0;
+  return conv2d_workspace(which, dtype, num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, true, pad_h, pad_w);
+}
+
+int adh_conv2d_unpadded_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                                  uint32_t W, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw,
+                                  uint32_t pad_h, uint32_t pad_w, const void *const *x_tiles, const void *w,
+                                  void *const *y_tiles, float beta, void *workspace, size_t workspace_bytes, void *stream) {
+  uint32_t HP, WP;
+  const int e = unpadded_geometry(H, W, kh, sh, dh, pad_h, pad_w, &HP, &WP);
+  if (e) return e;
+  return conv2d_fwd(dtype, num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, true, pad_h, pad_w, x_tiles, w, y_tiles,
+                    beta, workspace, workspace_bytes, stream);
+}
+
+int adh_conv2d_unpadded_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                                       uint32_t W, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh,
+                                       uint32_t dw, uint32_t pad_h, uint32_t pad_w, const void *w,
+                                       const void *const *dy_tiles, void *const *dx_tiles, float beta, void *workspace,
+                                       size_t workspace_bytes, void *stream) {
+  uint32_t HP, WP;
+  const int e = unpadded_geometry(H, W, kh, sh, dh, pad_h, pad_w, &HP, &WP);
+  if (e) return e;
+  return conv2d_bwd_data(dtype, num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, true, pad_h, pad_w, w, dy_tiles,
+                         dx_tiles, beta, workspace, workspace_bytes, stream);
+}
+
+int adh_conv2d_unpadded_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                                         uint32_t W, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh,
+                                         uint32_t dw, uint32_t pad_h, uint32_t pad_w, const void *const *x_tiles,
+                                         const void *const *dy_tiles, float *dwt, float beta, void *workspace,
+                                         size_t workspace_bytes, void *stream) {
+  uint32_t HP, WP;
+  const int e = unpadded_geometry(H, W, kh, sh, dh, pad_h, pad_w, &HP, &WP);
+  if (e) return e;
+  return conv2d_bwd_filter(dtype, num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, true, pad_h, pad_w, x_tiles,
+                           dy_tiles, dwt, beta, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

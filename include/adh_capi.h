@@ -287,6 +287,40 @@ int adh_conv2d_slab_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, 
                                      const void *const *dy_tiles, float *dwt, float beta, void *workspace,
                                      size_t workspace_bytes, void *stream);
 
+/* The same three passes over row tiles that carry NO halo, for any window / stride / dilation: the chains
+ * HaloPad2DOp -> HaloExch2DOp -> CudnnConv2DOp and conv backward-data -> halo reduce -> HaloPad2DOp::_backward
+ * (src/op.cc:2574-2641, 2963-3007, 1576-1587; 1701-1712, 3009-3052, 2643-2700) as one convolution launch each
+ * (the strided 3x3 and the 7x7 stem of src/zoo.cc:692-697, 1528-1538 without their pad, exchange, reduce and unpad
+ * passes).  x_tiles / dx_tiles are the K row tiles (H x W, packed NCHW) of one tensor in rank order, y_tiles /
+ * dy_tiles the row tiles (H / sh rows, OW = (W + 2 pad_w - ((kw-1)*dw + 1)) / sw + 1 columns) of the result.  Rows
+ * a window reaches outside a tile are read from the neighbouring tiles, the tensor's own border is zero
+ * padding (pad_h, pad_w): tile t of y is rows [t*H/sh, (t+1)*H/sh) of the unsplit convolution with that padding;
+ * backward-data computes the tile's own gradient completely (what the reduce would have added comes from the
+ * neighbours' dy rows) and never the halo pixels' (a 4 x 16 tile has 64 pixels, its padded form 108).
+ * Limits: H a multiple of sh; 0 < (kh-1)*dh + 1 - 2 pad_h <= sh (then H / sh output rows per tile stitch to the
+ * unsplit output: 3x3 pad 1 at stride 1 or 2, 7x7 pad 3, 1x1 pad 0 ...); pad_h <= H and (kh-1)*dh - pad_h <= H
+ * (a window reaches the adjacent tiles only); otherwise as the padded entry points above with HP = H + 2 pad_h,
+ * WP = W + 2 pad_w.  ADH_EINVAL outside these limits. */
+size_t adh_conv2d_unpadded_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,
+                                           uint32_t Cout, uint32_t H, uint32_t W, uint32_t kh, uint32_t kw,
+                                           uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, uint32_t pad_h,
+                                           uint32_t pad_w);
+int adh_conv2d_unpadded_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                  uint32_t H, uint32_t W, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw,
+                                  uint32_t dh, uint32_t dw, uint32_t pad_h, uint32_t pad_w,
+                                  const void *const *x_tiles, const void *w, void *const *y_tiles, float beta,
+                                  void *workspace, size_t workspace_bytes, void *stream);
+int adh_conv2d_unpadded_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                       uint32_t H, uint32_t W, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw,
+                                       uint32_t dh, uint32_t dw, uint32_t pad_h, uint32_t pad_w, const void *w,
+                                       const void *const *dy_tiles, void *const *dx_tiles, float beta,
+                                       void *workspace, size_t workspace_bytes, void *stream);
+int adh_conv2d_unpadded_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                         uint32_t H, uint32_t W, uint32_t kh, uint32_t kw, uint32_t sh,
+                                         uint32_t sw, uint32_t dh, uint32_t dw, uint32_t pad_h, uint32_t pad_w,
+                                         const void *const *x_tiles, const void *const *dy_tiles, float *dwt,
+                                         float beta, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- the shard-local ops between two halo exchanges ------------------------- */
 /* CudnnBatchNorm2DOp (src/op.cc:3907-4100) over K tiles in one call; as in the reference every
  * tile (rank) has its own parameters and normalises with its OWN batch statistics over
