@@ -903,10 +903,12 @@ public:
   // other contributor.
   bool unexchanged_rows = false;
   // Not in the reference.  The inputs are the row tiles of one activation in rank order (a 1 x K grid) and
-  // carry NO halo (halo_padded_input = false, pad = {1, 1}, 3x3, stride 1, dilation 1): the op is the
-  // reference's HaloPad2DOp -> HaloExch2DOp -> conv chain in one node.  Zero padding at the tensor's border
+  // carry NO halo (halo_padded_input = false; pad is the zero padding of the unsplit convolution): the op is
+  // the reference's HaloPad2DOp -> HaloExch2DOp -> conv chain in one node.  Zero padding at the tensor's border
   // and the neighbours' rows at the tiles' borders are read by the kernels; the input gradient comes out
-  // unpadded and complete.
+  // unpadded and complete.  Any window whose row split stitches: tile height a multiple of the row stride,
+  // 0 < (kernel - 1) * dilation + 1 - 2 * pad <= stride along the rows, a window that reaches the adjacent
+  // tiles only (3x3 pad 1 at stride 1 or 2, the 7x7 stem with pad 3, 1x1 pad 0 ...).
   bool unpadded_tiles = false;
 };
 
@@ -944,9 +946,11 @@ public:
         shape.dilate[0] == 0 || shape.dilate[1] == 0)
       throw std::invalid_argument("SlabConv2DOp: empty window, stride or dilation");
     if (shape.unpadded_tiles) {
-      if (shape.halo_padded_input || shape.kernel[0] != 3 || shape.kernel[1] != 3 || shape.stride[0] != 1 ||
-          shape.stride[1] != 1 || shape.dilate[0] != 1 || shape.dilate[1] != 1 || shape.pad[0] != 1 || shape.pad[1] != 1)
-        throw std::invalid_argument("SlabConv2DOp: tiles without halo take 3x3, stride 1, dilation 1, padding 1");
+      const size_t span = (shape.kernel[1] - 1) * shape.dilate[1] + 1;
+      const size_t tile_h = inputs.empty() ? 0 : inputs[0]->shape().shape[1];
+      if (shape.halo_padded_input || 2 * shape.pad[1] >= span || span - 2 * shape.pad[1] > shape.stride[1] ||
+          tile_h % shape.stride[1] != 0 || shape.pad[1] > tile_h || span - 1 - shape.pad[1] > tile_h)
+        throw std::invalid_argument("SlabConv2DOp: tiles without halo need a row split whose outputs stitch");
     } else if (!shape.halo_padded_input && (shape.pad[0] != 0 || shape.pad[1] != 0))
       throw std::invalid_argument("SlabConv2DOp: padding needs a halo-padded input");
     if (inputs.empty() || inputs.size() != kernels.size() || inputs.size() > ADH_MAX_TILES)
@@ -974,6 +978,11 @@ public:
       out[a] = (padded - span) / shape_.stride[a] + 1;
     }
     return Shape3D(out[0], out[1], shape_.filters);
+  }
+  bool is_3x3_unit_unpadded() const {
+    return shape_.kernel[0] == 3 && shape_.kernel[1] == 3 && shape_.stride[0] == 1 && shape_.stride[1] == 1 &&
+           shape_.dilate[0] == 1 && shape_.dilate[1] == 1 && shape_.pad[0] == 1 && shape_.pad[1] == 1 &&
+           !shape_.halo_padded_input && shape_.unpadded_tiles;
   }
   bool is_3x3_unit() const {
     return shape_.kernel[0] == 3 && shape_.kernel[1] == 3 && shape_.stride[0] == 1 && shape_.stride[1] == 1 &&

@@ -123,32 +123,43 @@ vector<shared_ptr<Var<V>>> exchanged_conv3x3(ParallelBatchNormParamOp<V> &block,
   parallel_vars_insert_all(block.grads, conv.grads);
   return conv.ops;
 }
+// A conv over row tiles WITHOUT halo (Conv2DShape::unpadded_tiles): no pad and no exchange node, the conv node reads
+// zero padding and its neighbours' rows itself and leaves an unpadded, complete input gradient.  Row tiles only,
+// and a tile height the row stride divides.
+template <typename V>
+bool halo_free_conv(const Conv2DShape &shape, size_t stride, const vector<shared_ptr<Var<V>>> &inputs, shared_ptr<Context> ctx) {
+  const auto tile = inputs.at(0)->shape();
+  const size_t span = (shape.kernel[1] - 1) * shape.dilate[1] + 1;
+  return mgpu_ctx_of(ctx)->spatial_comm(0)->num_w_ranks == 1 && tile.shape[1] % stride == 0 && 2 * shape.pad[1] < span &&
+         span - 2 * shape.pad[1] <= stride && shape.pad[1] <= tile.shape[1] && span - 1 - shape.pad[1] <= tile.shape[1];
+}
+template <typename V>
+vector<shared_ptr<Var<V>>> unpadded_conv(ParallelBatchNormParamOp<V> &block, Conv2DShape shape, size_t stride,
+                                         vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+  typedef GPUArray4D<float> A;
+  Conv2DShape cs = shape;
+  cs.stride = {stride, stride};
+  cs.halo_padded_input = false;
+  cs.unpadded_tiles = true;
+  const size_t cin = inputs.at(0)->shape().shape[2];
+  auto conv = parallel_conv2d<V, A>(cs, inputs, kaiming_init_gen<A>(cin * shape.kernel[0] * shape.kernel[1], shape.filters),
+                                    false, ctx);
+  parallel_vars_insert_all(block.params, conv.params);
+  parallel_vars_insert_all(block.grads, conv.grads);
+  return conv.ops;
+}
 // batch norm -> rectifier -> halo pad as ONE node (the reference has three, src/zoo.cc:596-604),
-// then halo exchange -> 3x3 conv
+// then halo exchange -> 3x3 conv; over row tiles the batch norm does not pad and the conv runs over tiles
+// without halo
 template <typename V>
 vector<shared_ptr<Var<V>>> bn_relu_pad_conv3x3(ParallelBatchNormParamOp<V> &block, Conv2DShape shape, size_t stride,
                                                shared_ptr<bool> switch_var, vector<shared_ptr<Var<V>>> inputs,
                                                shared_ptr<Context> ctx) {
   const size_t cin = inputs.at(0)->shape().shape[2];
-  // On row tiles of at least 256 pixels a stride-1 3x3 runs over tiles WITHOUT halo: the batch norm does not
-  // pad, no exchange node exists, and the conv node reads zero padding and its neighbours' rows itself (the
-  // 3x3 kernels serve every pass from that size on; smaller tiles keep the padded chain and the general kernels).
-  const auto tile = inputs.at(0)->shape();
-  const bool halo_free = stride == 1 && mgpu_ctx_of(ctx)->spatial_comm(0)->num_w_ranks == 1 && tile.shape[0] * tile.shape[1] >= 256 &&
-                         shape.kernel[0] == 3 && shape.kernel[1] == 3 && shape.dilate[0] == 1 && shape.dilate[1] == 1 &&
-                         shape.pad[0] == 1 && shape.pad[1] == 1;
-  if (halo_free) {
-    typedef GPUArray4D<float> A;
+  if (halo_free_conv(shape, stride, inputs, ctx)) {
     auto bnorm = CudnnBatchNorm2DOp<bool, V, GPUArray1D<float>>::MakeParallel(cin, switch_var, inputs, ctx, true, 0);
     add_batch_norm(block, bnorm);
-    Conv2DShape cs = shape;
-    cs.stride = {1, 1};
-    cs.halo_padded_input = false;
-    cs.unpadded_tiles = true;
-    auto conv = parallel_conv2d<V, A>(cs, bnorm.ops, kaiming_init_gen<A>(cin * 9, shape.filters), false, ctx);
-    parallel_vars_insert_all(block.params, conv.params);
-    parallel_vars_insert_all(block.grads, conv.grads);
-    return conv.ops;
+    return unpadded_conv(block, shape, stride, bnorm.ops, ctx);
   }
   auto bnorm = CudnnBatchNorm2DOp<bool, V, GPUArray1D<float>>::MakeParallel(cin, switch_var, inputs, ctx, true, 1);
   add_batch_norm(block, bnorm);
@@ -193,7 +204,9 @@ ParallelBatchNormParamOp<V> spatial_parallel_proj_residual_v2_conv2d(Conv2DShape
   auto proj = parallel_conv2d<V, A>(proj_shape, relu0, kaiming_init_gen<A>(cin, shape.filters), false, ctx);
   parallel_vars_insert_all(block.params, proj.params);
   parallel_vars_insert_all(block.grads, proj.grads);
-  auto conv1 = detail::exchanged_conv3x3(block, shape, stride, HaloPad2DOp<V>::MakeParallel(1, relu0, ctx), ctx);
+  auto conv1 = detail::halo_free_conv(shape, stride, relu0, ctx)
+                   ? detail::unpadded_conv(block, shape, stride, relu0, ctx)
+                   : detail::exchanged_conv3x3(block, shape, stride, HaloPad2DOp<V>::MakeParallel(1, relu0, ctx), ctx);
   auto conv2 = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, conv1, ctx);
   vector<vector<shared_ptr<Var<V>>>> join_inputs{proj.ops, conv2};
   block.ops = parallel_sum<V>(join_inputs, ctx);

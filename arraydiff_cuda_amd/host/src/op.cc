@@ -430,6 +430,28 @@ bool reads_neighbour_rows(const Op &op, const Conv2DShape &cs, const TileDims &d
   return cs.unexchanged_rows && use_3x3_kernels(op, d, n, cs.filters) && use_3x3_filter_kernel(op, d, n, cs.filters);
 }
 
+// Tiles without halo: the 3x3 kernels where they are the faster ones (as over padded tiles), else the general ones
+template <typename Op>
+bool unpadded_3x3_kernels(const Op &op, const TileDims &d, uint32_t n, size_t filters) {
+  return op.is_3x3_unit_unpadded() && (uint64_t)d.H * d.W > 64u && fits_3x3_kernels(d, n, filters);
+}
+template <typename Op>
+bool unpadded_3x3_filter_kernel(const Op &op, const TileDims &d, uint32_t n, size_t filters) {
+  const uint64_t pixels = (uint64_t)d.H * d.W;
+  return op.is_3x3_unit_unpadded() && (pixels > 256u || (pixels >= 64u && (uint64_t)d.N * n >= 64u)) &&
+         fits_3x3_kernels(d, n, filters);
+}
+#define ADH_UNPADDED_GEOMETRY(d, cs)                                                                                \
+  (d).H, (d).W, (uint32_t)(cs).kernel[1], (uint32_t)(cs).kernel[0], (uint32_t)(cs).stride[1], (uint32_t)(cs).stride[0], \
+      (uint32_t)(cs).dilate[1], (uint32_t)(cs).dilate[0], (uint32_t)(cs).pad[1], (uint32_t)(cs).pad[0]
+void *unpadded_conv_scratch(GPUContext *dc, int which, uint32_t n, const TileDims &d, const Conv2DShape &cs, size_t *bytes) {
+  *bytes = adh_conv2d_unpadded_workspace_bytes(which, ADH_F32, n, d.N, d.C, (uint32_t)cs.filters, ADH_UNPADDED_GEOMETRY(d, cs));
+  dc->reserve_scratch(*bytes);
+  auto scratch = dc->get_scratch();
+  *bytes = scratch->size();
+  return scratch->dptr();
+}
+
 void *conv_scratch(GPUContext *dc, int which, uint32_t n, const TileDims &d, const Conv2DShape &cs, size_t *bytes) {
   *bytes = adh_conv2d_workspace_bytes(which, ADH_F32, n, d.N, d.C, (uint32_t)cs.filters, d.H + 2 * (uint32_t)cs.pad[1],
                                       d.W + 2 * (uint32_t)cs.pad[0], (uint32_t)cs.kernel[1], (uint32_t)cs.kernel[0],
@@ -483,9 +505,17 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
     GPUConn conn = dc->conn();
     if (shape_.unpadded_tiles) {
       if (n != K) throw HazardError("SlabConv2DOp: tiles without halo need every rank in one pass");
-      adh_check(adh_conv3x3_unpadded_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt, 0.0f,
-                                               nullptr, 0, conn.stream()),
-                "SlabConv2DOp::_forward (tiles without halo)");
+      if (unpadded_3x3_kernels(*this, d, n, shape_.filters)) {
+        adh_check(adh_conv3x3_unpadded_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt, 0.0f,
+                                                 nullptr, 0, conn.stream()),
+                  "SlabConv2DOp::_forward (tiles without halo)");
+      } else {
+        size_t ws_bytes;
+        void *ws = unpadded_conv_scratch(dc, ADH_CONV_FWD, n, d, shape_, &ws_bytes);
+        adh_check(adh_conv2d_unpadded_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, ADH_UNPADDED_GEOMETRY(d, shape_),
+                                                xt, w0, yt, 0.0f, ws, ws_bytes, conn.stream()),
+                  "SlabConv2DOp::_forward (tiles without halo, general)");
+      }
       todo.swap(rest);
       continue;
     }
@@ -583,13 +613,22 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     GPUConn conn = dc->conn();
     if (shape_.unpadded_tiles) {
       if (n != K) throw HazardError("SlabConv2DOp: tiles without halo need every rank in one pass");
-      const size_t ws = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
-                                                    d.H, d.W);
-      dc->reserve_scratch(ws);
-      auto scratch = dc->get_scratch();
-      adh_check(adh_conv3x3_unpadded_bwd_filter_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, dyt, dw,
-                                                      wbeta, scratch->dptr(), scratch->size(), conn.stream()),
-                "SlabConv2DOp::_backward (filter, tiles without halo)");
+      if (unpadded_3x3_filter_kernel(*this, d, n, shape_.filters)) {
+        const size_t ws = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
+                                                      d.H, d.W);
+        dc->reserve_scratch(ws);
+        auto scratch = dc->get_scratch();
+        adh_check(adh_conv3x3_unpadded_bwd_filter_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, dyt, dw,
+                                                        wbeta, scratch->dptr(), scratch->size(), conn.stream()),
+                  "SlabConv2DOp::_backward (filter, tiles without halo)");
+      } else {
+        size_t ws_bytes;
+        void *ws = unpadded_conv_scratch(dc, ADH_CONV_BWD_FILTER, n, d, shape_, &ws_bytes);
+        adh_check(adh_conv2d_unpadded_bwd_filter_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
+                                                       ADH_UNPADDED_GEOMETRY(d, shape_), xt, dyt, dw, wbeta, ws, ws_bytes,
+                                                       conn.stream()),
+                  "SlabConv2DOp::_backward (filter, tiles without halo, general)");
+      }
     } else if (use_3x3_filter_kernel(*this, d, n, shape_.filters)) {
       const size_t ws = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
                                                     d.H, d.W);
@@ -654,9 +693,18 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     const float beta = first ? 0.0f : 1.0f;
     if (shape_.unpadded_tiles) {
       if (n != K) throw HazardError("SlabConv2DOp: tiles without halo need every rank in one pass");
-      adh_check(adh_conv3x3_unpadded_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, w0, dyt, dxt,
-                                                    beta, nullptr, 0, conn.stream()),
-                "SlabConv2DOp::_backward (data, tiles without halo)");
+      if (unpadded_3x3_kernels(*this, d, n, shape_.filters)) {
+        adh_check(adh_conv3x3_unpadded_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, w0, dyt, dxt,
+                                                      beta, nullptr, 0, conn.stream()),
+                  "SlabConv2DOp::_backward (data, tiles without halo)");
+      } else {
+        size_t ws_bytes;
+        void *ws = unpadded_conv_scratch(dc, ADH_CONV_BWD_DATA, n, d, shape_, &ws_bytes);
+        adh_check(adh_conv2d_unpadded_bwd_data_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters,
+                                                     ADH_UNPADDED_GEOMETRY(d, shape_), w0, dyt, dxt, beta, ws, ws_bytes,
+                                                     conn.stream()),
+                  "SlabConv2DOp::_backward (data, tiles without halo, general)");
+      }
       todo.swap(rest);
       continue;
     }
