@@ -375,8 +375,9 @@ static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, 
 // The same graph with any window k, stride s, dilation d and halo p = d * (k - 1) / 2: the 7x7 stem
 // over halo 3 (src/zoo.cc:1525-1538), the stride-2 3x3 (src/zoo.cc:692-697) and the dilated 3x3 of
 // tools/microbench_spatial_conv.cc:25-32, against the oracle's UNSPLIT convolution.
+// halo_free: no pad and no exchange node: the conv node takes the scattered tiles as they are
 static void test_spatial_general_conv_graph(size_t K, size_t N, size_t C, size_t Co, size_t H, size_t W, size_t k,
-                                            size_t st, size_t dil) {
+                                            size_t st, size_t dil, bool halo_free = false) {
   std::mt19937 gen(777 + (unsigned)(k * 10 + st));
   const size_t p = dil * (k - 1) / 2;
   const size_t OH = (H + 2 * p - (dil * (k - 1) + 1)) / st + 1, OW = (W + 2 * p - (dil * (k - 1) + 1)) / st + 1;
@@ -400,9 +401,10 @@ static void test_spatial_general_conv_graph(size_t K, size_t N, size_t C, size_t
   cs.dilate = {dil, dil};
   cs.stride = {st, st};
   cs.pad = {p, p};
-  cs.halo_padded_input = true;
+  cs.halo_padded_input = !halo_free;
+  cs.unpadded_tiles = halo_free;
   cs.enable_hmma = false;
-  auto ys = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch, ws, ctx);
+  auto ys = CudnnConv2DOp<V, A, A>::MakeParallel(cs, halo_free ? tiles : exch, ws, ctx);
   CHECK(ys[0]->shape() == Shape3D(OW, OH / K, Co));
   auto y_full = SpatialJoinedGather2DOp<V>::Make(ys, ctx);
   auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
@@ -425,8 +427,8 @@ static void test_spatial_general_conv_graph(size_t K, size_t N, size_t C, size_t
     orc_halo_unpad(0, (uint32_t)p, W, H, C, N, dXp.data(), dXr.data());
     orc_conv2d_slab_bwd_filter(N, C, Co, HP, WP, k, k, st, st, dil, dil, Xp.data(), dY.data(), 0.f, dWr.data());
     const double ey = rel_err(Y, Yr), ex = rel_err(dX, dXr), ew = rel_err(dW, dWr);
-    std::printf("general conv graph k=%zu s=%zu d=%zu K=%zu N=%zu C=%zu->%zu %zux%zu rep %d: rel-err y %.2e dx %.2e dw %.2e\n",
-                k, st, dil, K, N, C, Co, H, W, rep, ey, ex, ew);
+    std::printf("general conv graph k=%zu s=%zu d=%zu K=%zu N=%zu C=%zu->%zu %zux%zu%s rep %d: rel-err y %.2e dx %.2e dw %.2e\n",
+                k, st, dil, K, N, C, Co, H, W, halo_free ? " tiles without halo" : "", rep, ey, ex, ew);
     CHECK(ey <= 1e-5 && ex <= 1e-5 && ew <= 1e-5);
   }
 }
@@ -1018,6 +1020,12 @@ int main(int argc, char **argv) {
     test_spatial_general_conv_graph(2, 2, 8, 12, 16, 20, 3, 2, 1);   // stride-2 3x3
     test_spatial_general_conv_graph(2, 1, 8, 8, 12, 14, 3, 1, 3);    // dilation 3 over halo 3
     test_spatial_general_conv_graph(2, 2, 6, 10, 8, 9, 1, 1, 1);     // 1x1 over packed tiles (halo 0)
+    test_spatial_general_conv_graph(4, 2, 3, 16, 32, 24, 7, 2, 1, true);   // the same four over tiles without halo
+    test_spatial_general_conv_graph(2, 2, 8, 12, 16, 20, 3, 2, 1, true);
+    test_spatial_general_conv_graph(2, 1, 8, 8, 12, 14, 3, 1, 3, true);
+    test_spatial_general_conv_graph(4, 3, 3, 16, 32, 24, 7, 1, 1, true);   // the stem as the spatial net builds it (stride 1)
+    test_spatial_general_conv_graph(4, 4, 24, 24, 16, 16, 3, 1, 1, true);  // 4x16 tiles: stride-1 3x3 through the general kernels
+    test_spatial_general_conv_graph(4, 4, 16, 24, 8, 8, 3, 2, 1, true);    // 2x8 tiles at stride 2
     test_spatial_residual_block(4, 2, 8, 16, 12);
     test_spatial_residual_block(2, 4, 64, 28, 28);
     test_spatial_residual_block(4, 2, 8, 16, 12, true);
