@@ -144,6 +144,7 @@ public:
     if (b.readers.count(node.raw_id())) throw HazardError("overwrite after read by the same node");
     if (!b.writers.empty() && !b.writers.count(node.raw_id())) return false;
     b.writers.insert(node.raw_id());
+    b.all_zero = false;
     return true;
   }
   // Accumulating write.  The first toucher of a transaction runs init_fn on the buffer; the
@@ -154,7 +155,19 @@ public:
     if (fresh) init_fn(b.buffer.get());
     if (b.writers.count(node.raw_id())) return false;
     b.writers.insert(node.raw_id());
+    b.all_zero = false;
     return true;
+  }
+  // Not in the reference.  True while the buffer is known to hold nothing but zeros: it was allocated (cleared) or
+  // a writer declared it so, and no write access has been handed out since.  A node that would clear the buffer
+  // again can skip the fill.
+  bool known_zero() const { return buf_->buffer && buf_->all_zero; }
+  // a writer of this transaction states that the buffer holds only zeros now
+  void declare_zero(TxnId txn, NodeId node) {
+    Buf &b = *buf_;
+    if (!b.buffer || !b.has_txn || !(b.txn == txn.raw_id()) || !b.writers.count(node.raw_id()))
+      throw HazardError("declare_zero by a node that is not a writer of this transaction");
+    b.all_zero = true;
   }
   // Marks the value to be carried into `txn` by the first read there (op.hh:236-247); a write in
   // the new transaction replaces it as usual.
@@ -180,6 +193,7 @@ public:
     Buf &b = *buf_;
     if (!b.buffer || !b.has_txn || !(b.txn == txn.raw_id()) || !b.writers.count(node.raw_id()))
       throw HazardError("get_mut by a node that is not a writer of this transaction");
+    b.all_zero = false;
     return *b.buffer;
   }
   V &get_excl(TxnId txn, NodeId node) {
@@ -192,7 +206,7 @@ public:
 private:
   struct Buf {
     VarId var;
-    bool has_txn = false, rollover = false;
+    bool has_txn = false, rollover = false, all_zero = false;
     uint64_t txn = 0;
     std::set<uint64_t> writers, readers;
     std::unique_ptr<V> buffer;
@@ -213,6 +227,7 @@ private:
       buf_->buffer.reset(new V(V::ZerosPadded(shape_, offset_, stride_, batch_shape_, ctx)));
     else
       buf_->buffer.reset(new V(V::Zeros(shape_, ctx)));
+    buf_->all_zero = true;
   }
   VShape shape_, offset_, stride_;
   size_t batch_shape_ = 0;

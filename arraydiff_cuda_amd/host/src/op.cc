@@ -561,15 +561,18 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
   for (size_t r = 0; r < K; ++r) {
     GPUContext *dc = rank_ctx(ctx_, r);
     bool *fresh_r = &wfresh[r];
-    const bool clear = replicated_w && r > 0;
+    // (a gradient that is still all zeros from the last time - nobody writes the other ranks' - is not cleared again)
+    const bool clear = replicated_w && r > 0 && !kernels_[r].grad().known_zero();
     if (kernels_[r].grad().accumulate(txn, id(), dc, [dc, fresh_r, clear](A4 *g) {
           *fresh_r = true;
           if (clear) {
             GPUConn conn = dc->conn();
             g->set_constant(0.0f, conn);
           }
-        }))
+        })) {
       todo.push_back(r);
+      if (replicated_w && r > 0 && wfresh[r]) kernels_[r].grad().declare_zero(txn, id());
+    }
   }
   // ranks whose kernel variable was already counted through a shared VarData still contribute
   for (size_t r = 0; r < K; ++r) {
