@@ -77,6 +77,8 @@ SIGNATURES = {
     "adh_pool2d_slab_fwd": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, vp, vp, vp]),
     "adh_pool2d_slab_bwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vpp, vpp, vpp, f32, vp]),
     "adh_pool2d_slab_bwd": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, vp, vp, vp, vp, f32, vp]),
+    "adh_pool2d_unpadded_fwd_tiles": (i32, [i32, i32] + [u32] * 11 + [vpp, vpp, vp]),
+    "adh_pool2d_unpadded_bwd_tiles": (i32, [i32, i32] + [u32] * 11 + [vpp, vpp, vpp, vpp, f32, vp]),
     "adh_softmax_fwd": (i32, [u32, u32, vp, vp, vp]),
     "adh_softmax_nll_loss_fwd": (i32, [u32, u32, vp, vp, vp, vp]),
     "adh_softmax_nll_loss_bwd": (i32, [u32, u32, vp, vp, vp, vp, vp]),
@@ -469,6 +471,25 @@ def pool_bwd_tiles(mode, xs, ys, dys, dxs, N, C, HP, WP, wh, ww, sh, sw, beta=0.
     gt, k4 = _tbl(dxs)
     return lib().adh_pool2d_slab_bwd_tiles(_dt(dys[0]), mode, len(dys), N, C, HP, WP, wh, ww, sh, sw, xt, yt, dt, gt,
                                            beta, _stream())
+
+
+def pool_unpadded_fwd_tiles(mode, xs, ys, N, C, H, W, wh, ww, sh, sw, pad_h, pad_w):
+    """Pooling over row tiles without halo: rows outside a tile come from its neighbours, zeros outside the tensor."""
+    _dev(*xs, *ys)
+    xt, k1 = _tbl(xs)
+    yt, k2 = _tbl(ys)
+    return lib().adh_pool2d_unpadded_fwd_tiles(_dt(xs[0]), mode, len(xs), N, C, H, W, wh, ww, sh, sw, pad_h, pad_w, xt, yt,
+                                               _stream())
+
+
+def pool_unpadded_bwd_tiles(mode, xs, ys, dys, dxs, N, C, H, W, wh, ww, sh, sw, pad_h, pad_w, beta=0.0):
+    _dev(*xs, *dys, *dxs)
+    xt, k1 = _tbl(xs)
+    yt, k2 = _opt_tbl(ys)
+    dt, k3 = _tbl(dys)
+    gt, k4 = _tbl(dxs)
+    return lib().adh_pool2d_unpadded_bwd_tiles(_dt(dys[0]), mode, len(dys), N, C, H, W, wh, ww, sh, sw, pad_h, pad_w, xt, yt,
+                                               dt, gt, beta, _stream())
 
 
 def conv_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, H, W, beta=0.0, ws=None, unexchanged=False):

@@ -11,6 +11,13 @@
 //             dx coalesced.  y is not read: the maximum is recomputed from the staged input.
 // Direct kernels (rows too wide for LDS, windows of more than 256 elements): one thread per
 //   output (forward) or per padded element (backward), window reads served by the caches.
+// Tiles without halo (the UNP instances of the banded kernels): the tiles are the row tiles of one tensor in rank
+//   order; a block stages its band of the PADDED tile into LDS element by element, reading rows outside the
+//   tile from the neighbouring tiles and zeros outside the tensor, and then works as over a padded tile.
+//   Backward also takes the windows of the tiles above and below that reach into this tile (the padded plane
+//   is continued upward by `up` window rows and downward as far as needed, so that they are the windows
+//   0 .. up - 1 and up + OH .. of one row numbering) and stores interior pixels only: the gradient tile comes
+//   out complete, as after a halo reduce and an unpad.
 #include "adh_common.h"
 
 #include <algorithm>
@@ -29,7 +36,41 @@ struct PoolParams {
   // banded kernels
   uint32_t bands, band_rows;  // bands per plane; output rows (forward) / window rows (backward) per band
   FastDiv div_bands, div_OW, div_WP;
+  // tiles without halo: the tile is H x W and WP = W + 2 pad_w; pad_top rows lie above the tile's first row in
+  // the launch's row numbering (forward: pad_h, HP = H + 2 pad_h; backward: pad_h + up * sh, HP = pad_top + H +
+  // pad_h); up / extra = windows of the tile above / below that reach into this tile's rows (backward)
+  uint32_t H, W, pad_h, pad_w, pad_top, num_tiles, up, extra;
 };
+
+// element (vr, vc) of tile `tile`'s padded plane, read through the row tiles that carry no halo
+template <typename T>
+__device__ __forceinline__ T virt_at(const PoolParams &P, const void *const *tiles, uint32_t tile, uint32_t plane, uint32_t vr,
+                                     uint32_t vc) {
+  const int32_t c = (int32_t)vc - (int32_t)P.pad_w;
+  int32_t r = (int32_t)vr - (int32_t)P.pad_top;
+  if (c < 0 || c >= (int32_t)P.W) return (T)0;
+  uint32_t from = tile;
+  if (r < 0) {
+    r += (int32_t)P.H;
+    if (tile == 0u || r < 0) return (T)0;
+    from = tile - 1u;
+  } else if (r >= (int32_t)P.H) {
+    r -= (int32_t)P.H;
+    if (tile + 1u >= P.num_tiles || r >= (int32_t)P.H) return (T)0;
+    from = tile + 1u;
+  }
+  return reinterpret_cast<const T *>(tiles[from])[((size_t)plane * P.H + (uint32_t)r) * P.W + (uint32_t)c];
+}
+// rows [v0, v0 + nrows) of the padded plane into LDS, row pitch WP
+template <typename T>
+__device__ __forceinline__ void stage_virtual(T *lds, const PoolParams &P, uint32_t tile, uint32_t plane, uint32_t v0, uint32_t nrows) {
+  const uint32_t n = nrows * P.WP;
+  for (uint32_t e = threadIdx.x; e < n; e += 256u) {
+    uint32_t r, c;
+    P.div_WP.divmod(e, r, c);
+    lds[e] = virt_at<T>(P, P.x, tile, plane, v0 + r, c);
+  }
+}
 
 __device__ __forceinline__ float ld_f(const float *p, size_t i) { return p[i]; }
 __device__ __forceinline__ float ld_f(const uint16_t *p, size_t i) { return bf16_bits_to_f32(p[i]); }
@@ -139,7 +180,7 @@ __device__ __forceinline__ float window_reduce(const T *x, uint32_t base, uint32
 
 // grid: planes * tiles * bands; block 256.  Band b: output rows [b * band_rows, ...), input rows
 // [b * band_rows * sh, last * sh + wh).
-template <typename T, bool MAX, int WH, int WW>
+template <typename T, bool MAX, int WH, int WW, bool UNP = false>
 __global__ __launch_bounds__(kPoolThreads) void pool_fwd_band_kernel(const PoolParams P) {
   extern __shared__ __align__(16) unsigned char pool_lds[];
   uint32_t pb, band;
@@ -147,9 +188,15 @@ __global__ __launch_bounds__(kPoolThreads) void pool_fwd_band_kernel(const PoolP
   const uint32_t tile = pb / P.planes, plane = pb - tile * P.planes;
   const uint32_t oh0 = band * P.band_rows, rows = min(P.band_rows, P.OH - oh0);
   const uint32_t in_rows = (rows - 1u) * P.sh + P.wh;
-  const T *x = reinterpret_cast<const T *>(P.x[tile]) + (size_t)plane * P.HP * P.WP + (size_t)oh0 * P.sh * P.WP;
   T *y = reinterpret_cast<T *>(P.out[tile]) + (size_t)plane * P.OH * P.OW + (size_t)oh0 * P.OW;
-  const T *xl = stage_contiguous(reinterpret_cast<T *>(pool_lds), x, in_rows * P.WP);
+  const T *xl;
+  if constexpr (UNP) {
+    stage_virtual(reinterpret_cast<T *>(pool_lds), P, tile, plane, oh0 * P.sh, in_rows);
+    xl = reinterpret_cast<const T *>(pool_lds);
+  } else {
+    const T *x = reinterpret_cast<const T *>(P.x[tile]) + (size_t)plane * P.HP * P.WP + (size_t)oh0 * P.sh * P.WP;
+    xl = stage_contiguous(reinterpret_cast<T *>(pool_lds), x, in_rows * P.WP);
+  }
   __syncthreads();
   const uint32_t n_out = rows * P.OW;
   for (uint32_t o = threadIdx.x; o < n_out; o += kPoolThreads) {
@@ -163,7 +210,7 @@ __global__ __launch_bounds__(kPoolThreads) void pool_fwd_band_kernel(const PoolP
 // grid: planes * tiles * bands; block 256.  Band b owns the padded rows [b * band_rows * sh,
 // (b + 1) * band_rows * sh) (the last band: up to HP) and stages every window row that touches them.
 // WH, WW, S > 0: window and stride (both directions) known at compile time, 0: read from P.
-template <typename T, bool MAX, int WH, int WW, int S>
+template <typename T, bool MAX, int WH, int WW, int S, bool UNP = false>
 __global__ __launch_bounds__(kPoolThreads) void pool_bwd_band_kernel(const PoolParams PP) {
   extern __shared__ __align__(16) unsigned char pool_lds[];
   constexpr uint32_t VE = 16u / sizeof(T);
@@ -184,27 +231,71 @@ __global__ __launch_bounds__(kPoolThreads) void pool_bwd_band_kernel(const PoolP
   const uint32_t r0 = band * P.band_rows * Q.sh();
   const uint32_t r1 = band + 1u == P.bands ? P.HP : r0 + P.band_rows * Q.sh();
   // window rows that touch [r0, r1)
-  const uint32_t wr_lo = r0 + 1u > Q.wh() ? Q.div_sh(r0 + Q.sh() - Q.wh()) : 0u;
-  const uint32_t wr_hi = min(Q.div_sh(r1 - 1u), P.OH - 1u);
+  // tiles without halo: window rows 0 .. up - 1 are the last windows of the tile above (none for the first
+  // tile), up .. up + OH - 1 this tile's, the next `extra` the first windows of the tile below
+  const uint32_t up = UNP ? P.up : 0u;
+  const uint32_t w_first = UNP && tile == 0u ? up : 0u;
+  const uint32_t OHv = up + P.OH + (UNP && tile + 1u < P.num_tiles ? P.extra : 0u);
+  const uint32_t wr_lo = max(r0 + 1u > Q.wh() ? Q.div_sh(r0 + Q.sh() - Q.wh()) : 0u, w_first);
+  const uint32_t wr_hi = min(Q.div_sh(r1 - 1u), OHv - 1u);
+  if (UNP && wr_hi < wr_lo) return;  // (uniform) a band of the first tile that only the absent tile above would touch
   const uint32_t wrows = wr_hi + 1u - wr_lo;  // >= 1: r0 <= (OH - 1) * sh by the choice of bands
   const uint32_t n_win = wrows * P.OW;
   const uint32_t x_row0 = wr_lo * Q.sh(), x_rows = (wrows - 1u) * Q.sh() + Q.wh();
-  const T *dy = reinterpret_cast<const T *>(P.dy[tile]) + (size_t)plane * P.OH * P.OW + (size_t)wr_lo * P.OW;
-  T *dx = reinterpret_cast<T *>(P.out[tile]) + (size_t)plane * P.HP * P.WP;
+  // padded: the tile's padded gradient plane; tiles without halo: the H x W plane
+  T *dx = reinterpret_cast<T *>(P.out[tile]) + (size_t)plane * (UNP ? P.H * P.W : P.HP * P.WP);
   // LDS: dy rows | input rows | first-maximum positions
   T *lds_dy = reinterpret_cast<T *>(pool_lds);
   const uint32_t dy_room = (n_win + VE + VE - 1u) & ~(VE - 1u);
-  const T *dyl = stage_contiguous(lds_dy, dy, n_win);
+  const T *dyl;
+  if constexpr (UNP) {
+    for (uint32_t e = threadIdx.x; e < n_win; e += kPoolThreads) {
+      uint32_t wr, ow;
+      P.div_OW.divmod(e, wr, ow);
+      const uint32_t row = wr_lo + wr;
+      uint32_t from = tile, drow = row - up;
+      if (row < up) {
+        from = tile - 1u;
+        drow = P.OH - up + row;
+      } else if (row >= up + P.OH) {
+        from = tile + 1u;
+        drow = row - up - P.OH;
+      }
+      lds_dy[e] = reinterpret_cast<const T *>(P.dy[from])[((size_t)plane * P.OH + drow) * P.OW + ow];
+    }
+    dyl = lds_dy;
+  } else {
+    const T *dy = reinterpret_cast<const T *>(P.dy[tile]) + (size_t)plane * P.OH * P.OW + (size_t)wr_lo * P.OW;
+    dyl = stage_contiguous(lds_dy, dy, n_win);
+  }
+  // stores the owned rows' gradient g (LDS, fp32, padded pitch): all of it into the padded plane, or the
+  // interior pixels into the plane without halo
+  auto store_unpadded = [&](const float *g, uint32_t n_own) {
+    for (uint32_t e = threadIdx.x; e < n_own; e += kPoolThreads) {
+      uint32_t rb, vc;
+      P.div_WP.divmod(e, rb, vc);
+      const int32_t r = (int32_t)(r0 + rb) - (int32_t)P.pad_top, c = (int32_t)vc - (int32_t)P.pad_w;
+      if (r < 0 || r >= (int32_t)P.H || c < 0 || c >= (int32_t)P.W) continue;
+      const size_t i = (size_t)r * P.W + (uint32_t)c;
+      st_f(dx, i, g[e] + (P.beta != 0.f ? ld_f(dx, i) : 0.f));
+    }
+  };
   if (MAX) {
     T *lds_x = lds_dy + dy_room;
     const uint32_t x_room = (x_rows * P.WP + VE + VE - 1u) & ~(VE - 1u);
-    const T *x = reinterpret_cast<const T *>(P.x[tile]) + (size_t)plane * P.HP * P.WP + (size_t)x_row0 * P.WP;
-    const T *xl = stage_contiguous(lds_x, x, x_rows * P.WP);
+    const T *xl;
+    if constexpr (UNP) {
+      stage_virtual(lds_x, P, tile, plane, x_row0, x_rows);
+      xl = lds_x;
+    } else {
+      const T *x = reinterpret_cast<const T *>(P.x[tile]) + (size_t)plane * P.HP * P.WP + (size_t)x_row0 * P.WP;
+      xl = stage_contiguous(lds_x, x, x_rows * P.WP);
+    }
     // fp32 gradient of the owned rows, shifted like dx so that 16-byte stores line up
     const uint32_t n_own = (r1 - r0) * P.WP;
     T *dxo = dx + (size_t)r0 * P.WP;
     float *gl_base = reinterpret_cast<float *>(lds_x + x_room);
-    const uint32_t gpad = (uint32_t)(reinterpret_cast<uintptr_t>(dxo) & 15u) / (uint32_t)sizeof(T);
+    const uint32_t gpad = UNP ? 0u : (uint32_t)(reinterpret_cast<uintptr_t>(dxo) & 15u) / (uint32_t)sizeof(T);
     float *gl = gl_base + gpad;
     for (uint32_t v = threadIdx.x; v < (gpad + n_own + 3u) / 4u; v += kPoolThreads)
       reinterpret_cast<float4 *>(gl_base)[v] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -245,7 +336,8 @@ __global__ __launch_bounds__(kPoolThreads) void pool_bwd_band_kernel(const PoolP
         }
         __syncthreads();
       }
-    unstage_contiguous(dxo, gl, n_own, P.beta != 0.f);
+    if constexpr (UNP) store_unpadded(gl, n_own);
+    else unstage_contiguous(dxo, gl, n_own, P.beta != 0.f);
   } else {
     __syncthreads();
     const uint32_t n_own = (r1 - r0) * P.WP;
@@ -253,15 +345,18 @@ __global__ __launch_bounds__(kPoolThreads) void pool_bwd_band_kernel(const PoolP
       uint32_t ihb, iw;
       P.div_WP.divmod(j, ihb, iw);
       const uint32_t ih = r0 + ihb;
-      const uint32_t oh_hi = min(Q.div_sh(ih), P.OH - 1u);
-      const uint32_t oh_lo = ih + 1u > Q.wh() ? Q.div_sh(ih + Q.sh() - Q.wh()) : 0u;
+      if constexpr (UNP) {  // interior pixels only
+        if (ih < P.pad_top || ih >= P.pad_top + P.H || iw < P.pad_w || iw >= P.pad_w + P.W) continue;
+      }
+      const uint32_t oh_hi = min(Q.div_sh(ih), OHv - 1u);
+      const uint32_t oh_lo = max(ih + 1u > Q.wh() ? Q.div_sh(ih + Q.sh() - Q.wh()) : 0u, w_first);
       const uint32_t ow_hi = min(Q.div_sw(iw), P.OW - 1u);
       const uint32_t ow_lo = iw + 1u > Q.ww() ? Q.div_sw(iw + Q.sw() - Q.ww()) : 0u;
       float g = 0.f;
       for (uint32_t oh = oh_lo; oh <= oh_hi; ++oh)
         for (uint32_t ow = ow_lo; ow <= ow_hi; ++ow) g += ld_f(dyl, (oh - wr_lo) * P.OW + ow);
       g *= P.inv_area;
-      const size_t i = (size_t)r0 * P.WP + j;
+      const size_t i = UNP ? (size_t)(ih - P.pad_top) * P.W + (iw - P.pad_w) : (size_t)r0 * P.WP + j;
       if (P.beta != 0.f) g += ld_f(dx, i);
       st_f(dx, i, g);
     }
@@ -364,7 +459,7 @@ static size_t fwd_band_lds(const PoolParams &P, size_t es, uint32_t rows) {
   return ((size_t)((rows - 1u) * P.sh + P.wh) * P.WP * es + 16u + 15u) & ~(size_t)15u;
 }
 static size_t bwd_band_lds(const PoolParams &P, size_t es, bool max, uint32_t rows) {
-  const uint64_t wrows = std::min<uint64_t>(P.OH, (uint64_t)rows + (P.wh - 1u) / P.sh);
+  const uint64_t wrows = std::min<uint64_t>(P.OH + P.up + P.extra, (uint64_t)rows + (P.wh - 1u) / P.sh + P.extra);
   const uint64_t n_win = wrows * P.OW;
   size_t b = ((n_win * es + 16u + 15u) & ~(size_t)15u);
   if (max) {
@@ -389,38 +484,68 @@ static uint32_t pick_band_rows(const PoolParams &P, uint32_t num_tiles, size_t a
 
 static void set_bands(PoolParams *P, uint32_t rows) {
   P->band_rows = rows;
-  P->bands = (P->OH + rows - 1u) / rows;
+  P->bands = (P->OH + P->up + rows - 1u) / rows;  // (up: window rows of the tile above, backward over tiles without halo)
   P->div_bands = FastDiv(P->bands);
   P->div_OW = FastDiv(P->OW);
   P->div_WP = FastDiv(P->WP);
 }
 
-template <typename T, bool MAX>
+template <typename T, bool MAX, bool UNP>
 static void launch_fwd_band_t(const PoolParams &P, uint32_t blocks, size_t lds, hipStream_t st) {
   if (P.wh == 3 && P.ww == 3)
-    hipLaunchKernelGGL((pool_fwd_band_kernel<T, MAX, 3, 3>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+    hipLaunchKernelGGL((pool_fwd_band_kernel<T, MAX, 3, 3, UNP>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
   else if (P.wh == 2 && P.ww == 2)
-    hipLaunchKernelGGL((pool_fwd_band_kernel<T, MAX, 2, 2>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+    hipLaunchKernelGGL((pool_fwd_band_kernel<T, MAX, 2, 2, UNP>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
   else
-    hipLaunchKernelGGL((pool_fwd_band_kernel<T, MAX, 0, 0>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+    hipLaunchKernelGGL((pool_fwd_band_kernel<T, MAX, 0, 0, UNP>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
 }
-template <typename T, bool MAX>
+template <typename T, bool MAX, bool UNP>
 static void launch_bwd_band_t(const PoolParams &P, uint32_t blocks, size_t lds, hipStream_t st) {
   const bool s2 = P.sh == 2 && P.sw == 2;
   if (P.wh == 3 && P.ww == 3 && s2)
-    hipLaunchKernelGGL((pool_bwd_band_kernel<T, MAX, 3, 3, 2>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+    hipLaunchKernelGGL((pool_bwd_band_kernel<T, MAX, 3, 3, 2, UNP>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
   else if (P.wh == 2 && P.ww == 2 && s2)
-    hipLaunchKernelGGL((pool_bwd_band_kernel<T, MAX, 2, 2, 2>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+    hipLaunchKernelGGL((pool_bwd_band_kernel<T, MAX, 2, 2, 2, UNP>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
   else
-    hipLaunchKernelGGL((pool_bwd_band_kernel<T, MAX, 0, 0, 0>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+    hipLaunchKernelGGL((pool_bwd_band_kernel<T, MAX, 0, 0, 0, UNP>), dim3(blocks), dim3(kPoolThreads), lds, st, P);
+}
+template <bool UNP>
+static void launch_fwd_band_u(int dtype, bool max, const PoolParams &P, uint32_t blocks, size_t lds, hipStream_t st) {
+  if (dtype == ADH_F32) max ? launch_fwd_band_t<float, true, UNP>(P, blocks, lds, st) : launch_fwd_band_t<float, false, UNP>(P, blocks, lds, st);
+  else max ? launch_fwd_band_t<uint16_t, true, UNP>(P, blocks, lds, st) : launch_fwd_band_t<uint16_t, false, UNP>(P, blocks, lds, st);
+}
+template <bool UNP>
+static void launch_bwd_band_u(int dtype, bool max, const PoolParams &P, uint32_t blocks, size_t lds, hipStream_t st) {
+  if (dtype == ADH_F32) max ? launch_bwd_band_t<float, true, UNP>(P, blocks, lds, st) : launch_bwd_band_t<float, false, UNP>(P, blocks, lds, st);
+  else max ? launch_bwd_band_t<uint16_t, true, UNP>(P, blocks, lds, st) : launch_bwd_band_t<uint16_t, false, UNP>(P, blocks, lds, st);
 }
 static void launch_fwd_band(int dtype, bool max, const PoolParams &P, uint32_t blocks, size_t lds, hipStream_t st) {
-  if (dtype == ADH_F32) max ? launch_fwd_band_t<float, true>(P, blocks, lds, st) : launch_fwd_band_t<float, false>(P, blocks, lds, st);
-  else max ? launch_fwd_band_t<uint16_t, true>(P, blocks, lds, st) : launch_fwd_band_t<uint16_t, false>(P, blocks, lds, st);
+  launch_fwd_band_u<false>(dtype, max, P, blocks, lds, st);
 }
 static void launch_bwd_band(int dtype, bool max, const PoolParams &P, uint32_t blocks, size_t lds, hipStream_t st) {
-  if (dtype == ADH_F32) max ? launch_bwd_band_t<float, true>(P, blocks, lds, st) : launch_bwd_band_t<float, false>(P, blocks, lds, st);
-  else max ? launch_bwd_band_t<uint16_t, true>(P, blocks, lds, st) : launch_bwd_band_t<uint16_t, false>(P, blocks, lds, st);
+  launch_bwd_band_u<false>(dtype, max, P, blocks, lds, st);
+}
+
+// Tiles without halo: fills the padded extents and the split's fields; the same limits as the convolution over
+// such tiles (H / sh output rows per tile must stitch, a window reaches the adjacent tiles only).
+static int pool_check_unpadded(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H, uint32_t W,
+                               uint32_t wh, uint32_t ww, uint32_t sh, uint32_t sw, uint32_t pad_h, uint32_t pad_w,
+                               PoolParams *P) {
+  if (H == 0 || W == 0 || sh == 0 || wh == 0 || pad_h > 4096u || pad_w > 4096u) return ADH_EINVAL;
+  if (H % sh != 0u || 2u * pad_h >= wh || wh - 2u * pad_h > sh || pad_h > H || wh - 1u - pad_h > H) return ADH_EINVAL;
+  const int e = pool_check(dtype, mode, num_tiles, N, C, H + 2u * pad_h, W + 2u * pad_w, wh, ww, sh, sw, P);
+  if (e) return e;
+  P->H = H; P->W = W; P->pad_h = pad_h; P->pad_w = pad_w; P->pad_top = pad_h; P->num_tiles = num_tiles;
+  return ADH_OK;
+}
+// the backward launch's row numbering: continued upward by the window rows of the tile above that reach this tile
+static int pool_unpadded_bwd_rows(PoolParams *P) {
+  P->extra = (P->pad_h + P->sh - 1u) / P->sh;     // windows j of the tile below with j * sh < pad_h
+  P->up = (P->wh - 1u - P->pad_h) / P->sh;        // windows OH - j of the tile above with j * sh <= wh - 1 - pad_h
+  P->pad_top = P->pad_h + P->up * P->sh;
+  if (P->pad_top > P->H) return ADH_EINVAL;       // they start inside the tile above
+  P->HP = P->pad_top + P->H + P->pad_h;
+  return ADH_OK;
 }
 
 }  // namespace adh
@@ -516,6 +641,66 @@ int adh_pool2d_slab_bwd(int dtype, int mode, uint32_t N, uint32_t C, uint32_t HP
   const void *dys[1] = {dy};
   void *dxs[1] = {dx_pad};
   return adh_pool2d_slab_bwd_tiles(dtype, mode, 1, N, C, HP, WP, wh, ww, sh, sw, xs, ys, dys, dxs, beta, stream);
+}
+
+int adh_pool2d_unpadded_fwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H, uint32_t W,
+                                  uint32_t wh, uint32_t ww, uint32_t sh, uint32_t sw, uint32_t pad_h, uint32_t pad_w,
+                                  const void *const *x_tiles, void *const *y_tiles, void *stream) {
+  PoolParams P = {};
+  int e = pool_check_unpadded(dtype, mode, num_tiles, N, C, H, W, wh, ww, sh, sw, pad_h, pad_w, &P);
+  if (e) return e;
+  if (N == 0 || C == 0) return ADH_OK;
+  if (!x_tiles || !y_tiles) return ADH_ENULL;
+  const size_t es = dtype_size(dtype);
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!x_tiles[t] || !y_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(x_tiles[t], es) || !aligned_to(y_tiles[t], es)) return ADH_EALIGN;
+    P.x[t] = x_tiles[t];
+    P.out[t] = y_tiles[t];
+  }
+  const uint32_t band_rows = pick_band_rows(P, num_tiles, kPoolBandBytes, [&](uint32_t r) { return fwd_band_lds(P, es, r); });
+  if (!band_rows) return ADH_EUNIMPL;  // rows too wide for a band in LDS: use the padded entry points
+  set_bands(&P, band_rows);
+  launch_fwd_band_u<true>(dtype, mode == ADH_POOL_MAX, P, P.planes * num_tiles * P.bands, fwd_band_lds(P, es, band_rows),
+                          as_stream(stream));
+  return launch_status();
+}
+
+int adh_pool2d_unpadded_bwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H, uint32_t W,
+                                  uint32_t wh, uint32_t ww, uint32_t sh, uint32_t sw, uint32_t pad_h, uint32_t pad_w,
+                                  const void *const *x_tiles, const void *const *y_tiles, const void *const *dy_tiles,
+                                  void *const *dx_tiles, float beta, void *stream) {
+  PoolParams P = {};
+  int e = pool_check_unpadded(dtype, mode, num_tiles, N, C, H, W, wh, ww, sh, sw, pad_h, pad_w, &P);
+  if (e) return e;
+  if (beta != 0.f && beta != 1.f) return ADH_EINVAL;
+  if (N == 0 || C == 0) return ADH_OK;
+  if (!dy_tiles || !dx_tiles) return ADH_ENULL;
+  const bool is_max = mode == ADH_POOL_MAX;
+  if (is_max && !x_tiles) return ADH_ENULL;
+  const size_t es = dtype_size(dtype);
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!dy_tiles[t] || !dx_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(dy_tiles[t], es) || !aligned_to(dx_tiles[t], es)) return ADH_EALIGN;
+    if (is_max) {
+      if (!x_tiles[t]) return ADH_ENULL;
+      if (!aligned_to(x_tiles[t], es)) return ADH_EALIGN;
+      P.x[t] = x_tiles[t];
+      P.y[t] = y_tiles ? y_tiles[t] : nullptr;  // not read: the maximum is recomputed from the staged input
+    }
+    P.dy[t] = dy_tiles[t];
+    P.out[t] = dx_tiles[t];
+  }
+  P.beta = beta;
+  e = pool_unpadded_bwd_rows(&P);
+  if (e) return e;
+  const uint32_t band_rows =
+      wh * ww > 256u ? 0u : pick_band_rows(P, num_tiles, is_max ? 2u * kPoolBandBytes : kPoolBandBytes, [&](uint32_t r) { return bwd_band_lds(P, es, is_max, r); });
+  if (!band_rows) return ADH_EUNIMPL;
+  set_bands(&P, band_rows);
+  launch_bwd_band_u<true>(dtype, is_max, P, P.planes * num_tiles * P.bands, bwd_band_lds(P, es, is_max, band_rows),
+                          as_stream(stream));
+  return launch_status();
 }
 
 }  // extern "C"

@@ -394,6 +394,24 @@ int adh_pool2d_slab_bwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t 
 int adh_pool2d_slab_bwd(int dtype, int mode, uint32_t N, uint32_t C, uint32_t HP, uint32_t WP, uint32_t wh,
                         uint32_t ww, uint32_t sh, uint32_t sw, const void *x_pad, const void *y, const void *dy,
                         void *dx_pad, float beta, void *stream);
+/* The chains HaloPad2DOp -> HaloExch2DOp -> CudnnPool2DOp and pooling backward -> halo reduce ->
+ * HaloPad2DOp::_backward (src/zoo.cc:1562-1574 with src/op.cc:2574-2700, 2963-3052, 3496-3503, 3610-3619) as ONE
+ * launch each over row tiles that carry NO halo: x_tiles / dx_tiles are the K row tiles (H x W, packed NCHW) of
+ * one tensor in rank order, y_tiles / dy_tiles the tiles (H / sh rows, OW = (W + 2 pad_w - ww) / sw + 1 columns) of
+ * the result.  Rows a window reaches outside a tile are read from the neighbouring tiles; outside the tensor a
+ * window sees ZEROS, which take part as data exactly as the zeroed halo of the padded tile does (a window of
+ * negative values at the border has maximum 0, and its gradient then belongs to no pixel).  Backward computes the
+ * tile's own gradient completely: the windows of the tile below that reach into this tile are evaluated here too.
+ * Limits: H a multiple of sh, 0 < wh - 2 pad_h <= sh, pad_h <= H, wh - 1 - pad_h <= H (ADH_EINVAL otherwise); a band
+ * of window rows must fit in LDS (rows of up to a few thousand elements; ADH_EUNIMPL beyond: use the padded entry
+ * points).  y_tiles of the backward call is not read (the maximum is recomputed) and may be NULL. */
+int adh_pool2d_unpadded_fwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H,
+                                  uint32_t W, uint32_t wh, uint32_t ww, uint32_t sh, uint32_t sw, uint32_t pad_h,
+                                  uint32_t pad_w, const void *const *x_tiles, void *const *y_tiles, void *stream);
+int adh_pool2d_unpadded_bwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H,
+                                  uint32_t W, uint32_t wh, uint32_t ww, uint32_t sh, uint32_t sw, uint32_t pad_h,
+                                  uint32_t pad_w, const void *const *x_tiles, const void *const *y_tiles,
+                                  const void *const *dy_tiles, void *const *dx_tiles, float beta, void *stream);
 
 /* ---- L1/L2/L3: softmax + negative log likelihood (fp32) ------------------- */
 /* cudnnSoftmaxForward(ACCURATE, MODE_INSTANCE) on (N,C,1,1), src/op.cc:4129-4152 
