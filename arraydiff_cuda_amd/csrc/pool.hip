@@ -40,37 +40,11 @@ struct PoolParams {
   // the launch's row numbering (forward: pad_h, HP = H + 2 pad_h; backward: pad_h + up * sh, HP = pad_top + H +
   // pad_h); up / extra = windows of the tile above / below that reach into this tile's rows (backward)
   uint32_t H, W, pad_h, pad_w, pad_top, num_tiles, up, extra;
+  // rows of W (x, dx) and OW (dy) elements are copied as 16-byte vectors when their width is a multiple of the
+  // vector and the tiles are 16-byte aligned; x_items / dy_items = vectors (or elements) per row
+  uint32_t x_vec, dy_vec, x_items, dy_items;
+  FastDiv div_x_items, div_dy_items, div_side;
 };
-
-// element (vr, vc) of tile `tile`'s padded plane, read through the row tiles that carry no halo
-template <typename T>
-__device__ __forceinline__ T virt_at(const PoolParams &P, const void *const *tiles, uint32_t tile, uint32_t plane, uint32_t vr,
-                                     uint32_t vc) {
-  const int32_t c = (int32_t)vc - (int32_t)P.pad_w;
-  int32_t r = (int32_t)vr - (int32_t)P.pad_top;
-  if (c < 0 || c >= (int32_t)P.W) return (T)0;
-  uint32_t from = tile;
-  if (r < 0) {
-    r += (int32_t)P.H;
-    if (tile == 0u || r < 0) return (T)0;
-    from = tile - 1u;
-  } else if (r >= (int32_t)P.H) {
-    r -= (int32_t)P.H;
-    if (tile + 1u >= P.num_tiles || r >= (int32_t)P.H) return (T)0;
-    from = tile + 1u;
-  }
-  return reinterpret_cast<const T *>(tiles[from])[((size_t)plane * P.H + (uint32_t)r) * P.W + (uint32_t)c];
-}
-// rows [v0, v0 + nrows) of the padded plane into LDS, row pitch WP
-template <typename T>
-__device__ __forceinline__ void stage_virtual(T *lds, const PoolParams &P, uint32_t tile, uint32_t plane, uint32_t v0, uint32_t nrows) {
-  const uint32_t n = nrows * P.WP;
-  for (uint32_t e = threadIdx.x; e < n; e += 256u) {
-    uint32_t r, c;
-    P.div_WP.divmod(e, r, c);
-    lds[e] = virt_at<T>(P, P.x, tile, plane, v0 + r, c);
-  }
-}
 
 __device__ __forceinline__ float ld_f(const float *p, size_t i) { return p[i]; }
 __device__ __forceinline__ float ld_f(const uint16_t *p, size_t i) { return bf16_bits_to_f32(p[i]); }
@@ -80,6 +54,80 @@ __device__ __forceinline__ void st_f(uint16_t *p, size_t i, float v) { p[i] = f3
 constexpr uint32_t kPoolThreads = 256;
 constexpr uint32_t kPoolBandBytes = 24u * 1024u;  // LDS aimed at per block (twice that for the max backward)
 constexpr uint32_t kPoolMaxLds = 64u * 1024u;
+
+// Copies nrows rows of `items` vectors (vec: 16 bytes each) or elements into LDS rows of `pitch` elements, from
+// column col0 on.  src(row) is the row's first element in memory, or nullptr for a row of zeros; `any` is an
+// address that can always be read (a row of zeros loads from there and drops what it loaded: no branch around
+// the loads, so that several are in flight).
+template <typename T, typename F>
+__device__ __forceinline__ void stage_rows(T *lds, uint32_t pitch, uint32_t col0, uint32_t nrows, uint32_t items,
+                                           const FastDiv &div_items, bool vec, const T *any, F src) {
+  constexpr uint32_t VE = 16u / sizeof(T);
+  const uint32_t n = nrows * items;
+  if (vec) {
+#pragma unroll 4
+    for (uint32_t e = threadIdx.x; e < n; e += 256u) {
+      uint32_t row, it;
+      div_items.divmod(e, row, it);
+      const T *sp = src(row);
+      const bool have = sp != nullptr;
+      uint4 v = reinterpret_cast<const uint4 *>(have ? sp : any)[have ? it : 0u];
+      if (!have) v = make_uint4(0u, 0u, 0u, 0u);
+      T *d = lds + row * pitch + col0 + it * VE;
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      if constexpr (sizeof(T) == 4) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) reinterpret_cast<uint32_t *>(d)[k] = w[k];
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          d[2 * k] = (T)(w[k] & 0xffffu);
+          d[2 * k + 1] = (T)(w[k] >> 16);
+        }
+      }
+    }
+  } else {
+#pragma unroll 4
+    for (uint32_t e = threadIdx.x; e < n; e += 256u) {
+      uint32_t row, it;
+      div_items.divmod(e, row, it);
+      const T *sp = src(row);
+      const bool have = sp != nullptr;
+      const T v = (have ? sp : any)[have ? it : 0u];
+      lds[row * pitch + col0 + it] = have ? v : (T)0;
+    }
+  }
+}
+// rows [v0, v0 + nrows) of tile `tile`'s padded plane into LDS (row pitch WP), read through the row tiles that
+// carry no halo: rows outside the tile from the neighbouring tiles, zeros outside the tensor
+template <typename T>
+__device__ __forceinline__ void stage_virtual(T *lds, const PoolParams &P, uint32_t tile, uint32_t plane, uint32_t v0, uint32_t nrows) {
+  // the three planes a row can come from (chosen per row by selects: an index into the table of tiles that
+  // differs between lanes would be looked up one lane group at a time)
+  const size_t plane_off = (size_t)plane * P.H * P.W;
+  const T *own = reinterpret_cast<const T *>(P.x[tile]) + plane_off;
+  const T *above = tile > 0u ? reinterpret_cast<const T *>(P.x[tile - 1u]) + plane_off : nullptr;
+  const T *below = tile + 1u < P.num_tiles ? reinterpret_cast<const T *>(P.x[tile + 1u]) + plane_off : nullptr;
+  stage_rows(lds, P.WP, P.pad_w, nrows, P.x_items, P.div_x_items, P.x_vec != 0u, own, [&](uint32_t row) -> const T * {
+    int32_t r = (int32_t)(v0 + row) - (int32_t)P.pad_top;
+    const T *from = own;
+    if (r < 0) {
+      r += (int32_t)P.H;
+      from = r >= 0 ? above : nullptr;
+    } else if (r >= (int32_t)P.H) {
+      r -= (int32_t)P.H;
+      from = r < (int32_t)P.H ? below : nullptr;
+    }
+    return from ? from + (size_t)(uint32_t)r * P.W : nullptr;
+  });
+  // the zero columns left and right of every row
+  const uint32_t side = P.WP - P.W;
+  for (uint32_t e = threadIdx.x; e < nrows * side; e += 256u) {
+    uint32_t row, k;
+    P.div_side.divmod(e, row, k);
+    lds[row * P.WP + (k < P.pad_w ? k : P.W + k)] = (T)0;
+  }
+}
 
 // Copies n elements from src into LDS with 16-byte loads; lds is 16-byte aligned and has room for
 // n + 16 / sizeof(T) elements.  Returns the LDS address of element 0: it is shifted by the source's
@@ -249,20 +297,23 @@ __global__ __launch_bounds__(kPoolThreads) void pool_bwd_band_kernel(const PoolP
   const uint32_t dy_room = (n_win + VE + VE - 1u) & ~(VE - 1u);
   const T *dyl;
   if constexpr (UNP) {
-    for (uint32_t e = threadIdx.x; e < n_win; e += kPoolThreads) {
-      uint32_t wr, ow;
-      P.div_OW.divmod(e, wr, ow);
+    const size_t dy_plane_off = (size_t)plane * P.OH * P.OW;
+    const T *own_dy = reinterpret_cast<const T *>(P.dy[tile]) + dy_plane_off;
+    const T *dy_above = tile > 0u ? reinterpret_cast<const T *>(P.dy[tile - 1u]) + dy_plane_off : own_dy;
+    const T *dy_below = tile + 1u < P.num_tiles ? reinterpret_cast<const T *>(P.dy[tile + 1u]) + dy_plane_off : own_dy;
+    stage_rows(lds_dy, P.OW, 0u, wrows, P.dy_items, P.div_dy_items, P.dy_vec != 0u, own_dy, [&](uint32_t wr) -> const T * {
       const uint32_t row = wr_lo + wr;
-      uint32_t from = tile, drow = row - up;
+      const T *from = own_dy;
+      uint32_t drow = row - up;
       if (row < up) {
-        from = tile - 1u;
+        from = dy_above;
         drow = P.OH - up + row;
       } else if (row >= up + P.OH) {
-        from = tile + 1u;
+        from = dy_below;
         drow = row - up - P.OH;
       }
-      lds_dy[e] = reinterpret_cast<const T *>(P.dy[from])[((size_t)plane * P.OH + drow) * P.OW + ow];
-    }
+      return from + (size_t)drow * P.OW;
+    });
     dyl = lds_dy;
   } else {
     const T *dy = reinterpret_cast<const T *>(P.dy[tile]) + (size_t)plane * P.OH * P.OW + (size_t)wr_lo * P.OW;
@@ -271,13 +322,34 @@ __global__ __launch_bounds__(kPoolThreads) void pool_bwd_band_kernel(const PoolP
   // stores the owned rows' gradient g (LDS, fp32, padded pitch): all of it into the padded plane, or the
   // interior pixels into the plane without halo
   auto store_unpadded = [&](const float *g, uint32_t n_own) {
-    for (uint32_t e = threadIdx.x; e < n_own; e += kPoolThreads) {
-      uint32_t rb, vc;
-      P.div_WP.divmod(e, rb, vc);
-      const int32_t r = (int32_t)(r0 + rb) - (int32_t)P.pad_top, c = (int32_t)vc - (int32_t)P.pad_w;
-      if (r < 0 || r >= (int32_t)P.H || c < 0 || c >= (int32_t)P.W) continue;
-      const size_t i = (size_t)r * P.W + (uint32_t)c;
-      st_f(dx, i, g[e] + (P.beta != 0.f ? ld_f(dx, i) : 0.f));
+    // the owned rows that are the tile's own: rows [i0, i1) of the H x W plane
+    const uint32_t i0 = r0 > P.pad_top ? r0 - P.pad_top : 0u;
+    const uint32_t i1 = min(P.H, r1 > P.pad_top ? r1 - P.pad_top : 0u);
+    if (i1 <= i0) return;
+    const uint32_t n = (i1 - i0) * P.x_items;
+    (void)n_own;
+#pragma unroll 2
+    for (uint32_t e = threadIdx.x; e < n; e += kPoolThreads) {
+      uint32_t rb, it;
+      P.div_x_items.divmod(e, rb, it);
+      const uint32_t r = i0 + rb;
+      const float *gs = g + (r + P.pad_top - r0) * P.WP + P.pad_w;
+      T *drow = dx + (size_t)r * P.W;
+      if (P.x_vec) {
+        float f[VE];
+#pragma unroll
+        for (uint32_t k = 0; k < VE; ++k) f[k] = gs[it * VE + k];
+        uint4 *dv = reinterpret_cast<uint4 *>(drow) + it;
+        if (P.beta != 0.f) {
+          float o[VE];
+          vec_to_f32(*dv, o, (const T *)nullptr);
+#pragma unroll
+          for (uint32_t k = 0; k < VE; ++k) f[k] += o[k];
+        }
+        *dv = f32_to_vec(f, (const T *)nullptr);
+      } else {
+        st_f(drow, it, gs[it] + (P.beta != 0.f ? ld_f(drow, it) : 0.f));
+      }
     }
   };
   if (MAX) {
@@ -536,7 +608,23 @@ static int pool_check_unpadded(int dtype, int mode, uint32_t num_tiles, uint32_t
   const int e = pool_check(dtype, mode, num_tiles, N, C, H + 2u * pad_h, W + 2u * pad_w, wh, ww, sh, sw, P);
   if (e) return e;
   P->H = H; P->W = W; P->pad_h = pad_h; P->pad_w = pad_w; P->pad_top = pad_h; P->num_tiles = num_tiles;
+  P->div_side = FastDiv(std::max(1u, 2u * pad_w));
   return ADH_OK;
+}
+// rows as 16-byte vectors where widths and addresses allow
+static void pool_unpadded_vectors(PoolParams *P, size_t es, uint32_t num_tiles, bool with_dy) {
+  const uint32_t ve = (uint32_t)(16u / es);
+  bool x_ok = P->W % ve == 0u, dy_ok = with_dy && P->OW % ve == 0u;
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    x_ok = x_ok && (!P->x[t] || aligned_to(P->x[t], 16)) && (!with_dy || aligned_to(P->out[t], 16));
+    dy_ok = dy_ok && aligned_to(P->dy[t], 16);
+  }
+  P->x_vec = x_ok ? 1u : 0u;
+  P->dy_vec = dy_ok ? 1u : 0u;
+  P->x_items = x_ok ? P->W / ve : P->W;
+  P->dy_items = dy_ok ? P->OW / ve : P->OW;
+  P->div_x_items = FastDiv(P->x_items);
+  P->div_dy_items = FastDiv(std::max(1u, P->dy_items));
 }
 // the backward launch's row numbering: continued upward by the window rows of the tile above that reach this tile
 static int pool_unpadded_bwd_rows(PoolParams *P) {
@@ -658,6 +746,7 @@ int adh_pool2d_unpadded_fwd_tiles(int dtype, int mode, uint32_t num_tiles, uint3
     P.x[t] = x_tiles[t];
     P.out[t] = y_tiles[t];
   }
+  pool_unpadded_vectors(&P, es, num_tiles, false);
   const uint32_t band_rows = pick_band_rows(P, num_tiles, kPoolBandBytes, [&](uint32_t r) { return fwd_band_lds(P, es, r); });
   if (!band_rows) return ADH_EUNIMPL;  // rows too wide for a band in LDS: use the padded entry points
   set_bands(&P, band_rows);
@@ -694,6 +783,7 @@ int adh_pool2d_unpadded_bwd_tiles(int dtype, int mode, uint32_t num_tiles, uint3
   P.beta = beta;
   e = pool_unpadded_bwd_rows(&P);
   if (e) return e;
+  pool_unpadded_vectors(&P, es, num_tiles, true);
   const uint32_t band_rows =
       wh * ww > 256u ? 0u : pick_band_rows(P, num_tiles, is_max ? 2u * kPoolBandBytes : kPoolBandBytes, [&](uint32_t r) { return bwd_band_lds(P, es, is_max, r); });
   if (!band_rows) return ADH_EUNIMPL;

@@ -1347,6 +1347,12 @@ public:
   array<size_t, 2> stride;
   array<size_t, 2> pad;
   bool halo_padded_input;
+  // Not in the reference.  The inputs are the row tiles of one activation in rank order (a 1 x K grid) and carry
+  // NO halo (halo_padded_input = false; pad is the zero padding of the unsplit pooling): the op is the reference's
+  // HaloPad2DOp -> HaloExch2DOp -> pool chain in one node, and its input gradient comes out unpadded and complete.
+  // The row split must stitch: tile height a multiple of the row stride, 0 < window - 2 * pad <= stride along the
+  // rows, windows that reach the adjacent tiles only.
+  bool unpadded_tiles = false;
 };
 
 // V = GPUBatchArray3D<float>.  With halo_padded_input the padded tile is pooled as a plain packed
@@ -1372,14 +1378,20 @@ public:
       : ctx_(ctx), shape_(shape), x_vars_(inputs) {
     if (shape.pooling != kAveragePool && shape.pooling != kMaxPool)
       throw std::invalid_argument("SlabPool2DOp: unknown pooling");
-    if (!shape.halo_padded_input && (shape.pad[0] != 0 || shape.pad[1] != 0))
-      throw std::invalid_argument("SlabPool2DOp: padding needs a halo-padded input");
     if (shape.window[0] == 0 || shape.window[1] == 0 || shape.stride[0] == 0 || shape.stride[1] == 0)
       throw std::invalid_argument("SlabPool2DOp: empty window or stride");
     if (inputs.empty() || inputs.size() > ADH_MAX_TILES) throw std::invalid_argument("SlabPool2DOp: bad tile count");
+    if (shape.unpadded_tiles) {
+      const size_t tile_h = inputs[0]->shape().shape[1];
+      if (shape.halo_padded_input || 2 * shape.pad[1] >= shape.window[1] || shape.window[1] - 2 * shape.pad[1] > shape.stride[1] ||
+          tile_h % shape.stride[1] != 0 || shape.pad[1] > tile_h || shape.window[1] - 1 - shape.pad[1] > tile_h)
+        throw std::invalid_argument("SlabPool2DOp: tiles without halo need a row split whose outputs stitch");
+    } else if (!shape.halo_padded_input && (shape.pad[0] != 0 || shape.pad[1] != 0))
+      throw std::invalid_argument("SlabPool2DOp: padding needs a halo-padded input");
     for (size_t r = 0; r < inputs.size(); ++r) {
       auto off = inputs[r]->offset();
-      if (off.shape[0] != shape.pad[0] || off.shape[1] != shape.pad[1] || off.shape[2] != 0)
+      const size_t halo0 = shape.unpadded_tiles ? 0 : shape.pad[0], halo1 = shape.unpadded_tiles ? 0 : shape.pad[1];
+      if (off.shape[0] != halo0 || off.shape[1] != halo1 || off.shape[2] != 0)
         throw std::invalid_argument("SlabPool2DOp: input halo must equal the pooling pad");
       if (inputs[r]->shape() != inputs[0]->shape() || inputs[r]->batch_shape() != inputs[0]->batch_shape())
         throw std::invalid_argument("SlabPool2DOp: all tiles must have one shape");

@@ -1002,6 +1002,15 @@ void SlabPool2DOp<V3>::_forward(TxnId txn) {
   }
   if (n == 0) return;
   GPUConn conn = rank_ctx(ctx_, 0)->conn();
+  if (shape_.unpadded_tiles) {
+    if (n != K) throw HazardError("SlabPool2DOp: tiles without halo need every rank in one pass");
+    adh_check(adh_pool2d_unpadded_fwd_tiles(ADH_F32, shape_.pooling == kMaxPool ? ADH_POOL_MAX : ADH_POOL_AVG, n, d.N, d.C, d.H,
+                                            d.W, (uint32_t)shape_.window[1], (uint32_t)shape_.window[0],
+                                            (uint32_t)shape_.stride[1], (uint32_t)shape_.stride[0], (uint32_t)shape_.pad[1],
+                                            (uint32_t)shape_.pad[0], xt, yt, conn.stream()),
+              "SlabPool2DOp::_forward (tiles without halo)");
+    return;
+  }
   adh_check(adh_pool2d_slab_fwd_tiles(ADH_F32, shape_.pooling == kMaxPool ? ADH_POOL_MAX : ADH_POOL_AVG, n, d.N, d.C,
                                       d.H + 2 * (uint32_t)shape_.pad[1], d.W + 2 * (uint32_t)shape_.pad[0],
                                       (uint32_t)shape_.window[1], (uint32_t)shape_.window[0], (uint32_t)shape_.stride[1],
@@ -1048,6 +1057,15 @@ void SlabPool2DOp<V3>::_backward(TxnId txn) {
     }
     if (n == 0) continue;
     GPUConn conn = rank_ctx(ctx_, 0)->conn();
+    if (shape_.unpadded_tiles) {
+      if (n != K) throw HazardError("SlabPool2DOp: tiles without halo need every rank in one pass");
+      adh_check(adh_pool2d_unpadded_bwd_tiles(ADH_F32, shape_.pooling == kMaxPool ? ADH_POOL_MAX : ADH_POOL_AVG, n, d.N, d.C,
+                                              d.H, d.W, (uint32_t)shape_.window[1], (uint32_t)shape_.window[0],
+                                              (uint32_t)shape_.stride[1], (uint32_t)shape_.stride[0], (uint32_t)shape_.pad[1],
+                                              (uint32_t)shape_.pad[0], xt, yt, dyt, dxt, first ? 0.0f : 1.0f, conn.stream()),
+                "SlabPool2DOp::_backward (tiles without halo)");
+      continue;
+    }
     adh_check(adh_pool2d_slab_bwd_tiles(ADH_F32, shape_.pooling == kMaxPool ? ADH_POOL_MAX : ADH_POOL_AVG, n, d.N, d.C,
                                         d.H + 2 * (uint32_t)shape_.pad[1], d.W + 2 * (uint32_t)shape_.pad[0],
                                         (uint32_t)shape_.window[1], (uint32_t)shape_.window[0], (uint32_t)shape_.stride[1],

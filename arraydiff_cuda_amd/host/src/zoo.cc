@@ -55,10 +55,17 @@ ParallelCategoricalNLLBatchNormLoss<V1, F0> ResNet<float>::MakeParallelResNet18(
   par_ys = conv1.ops;
 
   // pool1: 3x3 max at stride 2 over halo 1 (src/zoo.cc:1562-1574)
-  par_ys = HaloExch2DOp<V3>::MakeParallel(1, HaloPad2DOp<V3>::MakeParallel(1, par_ys, parallel_ctx), parallel_ctx);
   Pool2DShape pool1_shape;
   pool1_shape.pooling = kMaxPool; pool1_shape.axes = {0, 1}; pool1_shape.window = {3, 3}; pool1_shape.stride = {2, 2};
   pool1_shape.pad = {1, 1}; pool1_shape.halo_padded_input = true;
+  if (mgpu_ctx->spatial_comm(0)->num_w_ranks == 1 && par_ys.at(0)->shape().shape[1] % 2 == 0) {
+    // over row tiles the pooling reads its zero padding and its neighbours' rows itself: no pad, no exchange, and
+    // the stem's output gradient comes out unpadded (two passes over the largest activation of the net fewer)
+    pool1_shape.halo_padded_input = false;
+    pool1_shape.unpadded_tiles = true;
+  } else {
+    par_ys = HaloExch2DOp<V3>::MakeParallel(1, HaloPad2DOp<V3>::MakeParallel(1, par_ys, parallel_ctx), parallel_ctx);
+  }
   par_ys = CudnnPool2DOp<V3>::MakeParallel(pool1_shape, par_ys, parallel_ctx);
 
   auto res_shape = [](size_t filters) {

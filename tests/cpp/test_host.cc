@@ -436,7 +436,8 @@ static void test_spatial_general_conv_graph(size_t K, size_t N, size_t C, size_t
 // Scatter -> HaloPad(1) -> HaloExch(1) -> Pool(3x3, stride 2, pad 1, halo_padded_input) -> gather:
 // the stem pooling of src/zoo.cc:1562-1573 on K row-tiles of one GPU, against the oracle's pooling
 // of the zero-padded UNSPLIT tensor.
-static void test_spatial_pool_graph(Pooling pooling, size_t K, size_t N, size_t C, size_t H, size_t W) {
+// halo_free: no pad and no exchange node: the pooling node takes the scattered tiles as they are
+static void test_spatial_pool_graph(Pooling pooling, size_t K, size_t N, size_t C, size_t H, size_t W, bool halo_free = false) {
   std::mt19937 gen(4321 + (unsigned)K);
   auto ctx = MultiGPUContext::Make(K);
   const size_t OH = (H + 2 - 3) / 2 + 1, OW = (W + 2 - 3) / 2 + 1;
@@ -454,8 +455,9 @@ static void test_spatial_pool_graph(Pooling pooling, size_t K, size_t N, size_t 
   ps.window = {3, 3};
   ps.stride = {2, 2};
   ps.pad = {1, 1};
-  ps.halo_padded_input = true;
-  auto ys = CudnnPool2DOp<V>::MakeParallel(ps, exch, ctx);
+  ps.halo_padded_input = !halo_free;
+  ps.unpadded_tiles = halo_free;
+  auto ys = CudnnPool2DOp<V>::MakeParallel(ps, halo_free ? tiles : exch, ctx);
   auto y_full = SpatialJoinedGather2DOp<V>::Make(ys, ctx);
   auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
   sink->set_host_grad(dY.data());
@@ -475,8 +477,8 @@ static void test_spatial_pool_graph(Pooling pooling, size_t K, size_t N, size_t 
     orc_pool_slab_bwd(mode, N, C, H + 2, W + 2, 3, 3, 2, 2, Xp.data(), dY.data(), 0.f, dXp.data());
     orc_halo_unpad(0, 1, W, H, C, N, dXp.data(), dXr.data());
     const double ey = rel_err(Y, Yr), ex = rel_err(dX, dXr);
-    std::printf("pool graph %s K=%zu N=%zu C=%zu %zux%zu rep %d: rel-err y %.2e dx %.2e\n", mode ? "max" : "avg", K, N, C, H,
-                W, rep, ey, ex);
+    std::printf("pool graph %s K=%zu N=%zu C=%zu %zux%zu%s rep %d: rel-err y %.2e dx %.2e\n", mode ? "max" : "avg", K, N, C, H,
+                W, halo_free ? " tiles without halo" : "", rep, ey, ex);
     CHECK(ey <= 1e-5 && ex <= 1e-5);
   }
 }
@@ -1033,6 +1035,9 @@ int main(int argc, char **argv) {
     test_spatial_pool_graph(kMaxPool, 4, 2, 8, 16, 12);
     test_spatial_pool_graph(kAveragePool, 2, 3, 5, 8, 10);
     test_spatial_pool_graph(kMaxPool, 4, 8, 64, 112, 112);
+    test_spatial_pool_graph(kMaxPool, 4, 2, 8, 16, 12, true);
+    test_spatial_pool_graph(kAveragePool, 2, 3, 5, 8, 10, true);
+    test_spatial_pool_graph(kMaxPool, 4, 8, 64, 112, 112, true);
     test_softmax_loss_op();
     test_parallel_conv2d_init_gives_equal_copies();
     test_resnet18_tiling_invariance();
