@@ -572,7 +572,56 @@ def main():
             lambda: lib.adh_pool2d_slab_bwd_tiles(0, 1, K, N, C, Hq, Wq, 3, 3, 2, 2, xq_tbl, yq_tbl, dq_tbl, gq_tbl,
                                                   0.0, stream),
             "hbm", 2 * in_b + out_b, HBM_PEAK_GBS, "GB/s", note="reads x and dy, writes dx; y is not read")
-        del xq, yq, dq, gq
+        # the same pooling over tiles without halo (no pad, exchange, reduce or unpad pass around it)
+        xqu = [torch.rand((N, C, 28, 112), device="cuda", generator=g) for _ in range(K)]
+        gqu = [torch.empty((N, C, 28, 112), device="cuda") for _ in range(K)]
+        xqu_tbl, _kq5 = capi.ptr_table([t.data_ptr() for t in xqu])
+        gqu_tbl, _kq6 = capi.ptr_table([t.data_ptr() for t in gqu])
+        in_u = K * N * C * 28 * 112 * 4
+        add("max pool 3x3 s2 fwd over tiles without halo (fp32, 4 tiles of 28x112; pad, exchange and pooling in one launch)",
+            lambda: lib.adh_pool2d_unpadded_fwd_tiles(0, 1, K, N, C, 28, 112, 3, 3, 2, 2, 1, 1, xqu_tbl, yq_tbl, stream),
+            "hbm", in_u + out_b, HBM_PEAK_GBS, "GB/s")
+        add("max pool 3x3 s2 bwd into tiles without halo (fp32; pooling backward, halo reduce and unpad in one launch)",
+            lambda: lib.adh_pool2d_unpadded_bwd_tiles(0, 1, K, N, C, 28, 112, 3, 3, 2, 2, 1, 1, xqu_tbl, yq_tbl, dq_tbl, gqu_tbl,
+                                                      0.0, stream),
+            "hbm", 2 * in_u + out_b, HBM_PEAK_GBS, "GB/s")
+        del xq, yq, dq, gq, xqu, gqu
+        # the 3x3 kernels and the general kernels over tiles without halo, at the shapes of the spatially-parallel
+        # ResNet-18 (batch 32, 4 row tiles): a 64-channel 3x3 on 32x128 tiles, the stride-2 3x3 64 -> 128 on the same
+        # tiles, and a 512-channel 3x3 on 4x16 tiles (the general kernels; padded tiles of 6x18 hold 1.7 times the pixels)
+        for (nm, Ci, Co, Hu, Wu, su) in (("3x3 64->64 on 32x128 tiles", 64, 64, 32, 128, 1), ("3x3 stride 2 64->128 on 32x128 tiles", 64, 128, 32, 128, 2),
+                                         ("3x3 512->512 on 4x16 tiles", 512, 512, 4, 16, 1)):
+            OHu, OWu = Hu // su, (Wu + 2 - 3) // su + 1
+            xu = [torch.randn((N, Ci, Hu, Wu), device="cuda", generator=g) for _ in range(K)]
+            yu = [torch.randn((N, Co, OHu, OWu), device="cuda", generator=g) for _ in range(K)]
+            wu_ = torch.randn((Co, Ci, 3, 3), device="cuda", generator=g) * (2.0 / (Ci * 9)) ** 0.5
+            gwu = torch.empty((Co, Ci, 3, 3), device="cuda")
+            xu_tbl, _ku1 = capi.ptr_table([t.data_ptr() for t in xu])
+            yu_tbl, _ku2 = capi.ptr_table([t.data_ptr() for t in yu])
+            small = su == 1 and Hu * Wu > 64  # the 3x3 kernels serve it; else the general ones
+            wsb = max([lib.adh_conv2d_unpadded_workspace_bytes(wh, 0, K, N, Ci, Co, Hu, Wu, 3, 3, su, su, 1, 1, 1, 1) for wh in (0, 1, 2)] +
+                      [lib.adh_conv3x3_workspace_bytes(2, 0, K, N, Ci, Co, Hu, Wu)])
+            wsu = torch.empty(wsb // 4 + 64, device="cuda")
+            flop = 2.0 * K * N * Ci * Co * 9 * OHu * OWu
+            reps, wu = 50, 10
+            if small:
+                f = lambda: lib.adh_conv3x3_unpadded_fwd_tiles(0, K, N, Ci, Co, Hu, Wu, xu_tbl, wu_.data_ptr(), yu_tbl, 0.0, None, 0, stream)
+                b = lambda: lib.adh_conv3x3_unpadded_bwd_data_tiles(0, K, N, Ci, Co, Hu, Wu, wu_.data_ptr(), yu_tbl, xu_tbl, 0.0, None, 0, stream)
+            else:
+                f = lambda: lib.adh_conv2d_unpadded_fwd_tiles(0, K, N, Ci, Co, Hu, Wu, 3, 3, su, su, 1, 1, 1, 1, xu_tbl, wu_.data_ptr(), yu_tbl,
+                                                              0.0, wsu.data_ptr(), wsb, stream)
+                b = lambda: lib.adh_conv2d_unpadded_bwd_data_tiles(0, K, N, Ci, Co, Hu, Wu, 3, 3, su, su, 1, 1, 1, 1, wu_.data_ptr(), yu_tbl,
+                                                                   xu_tbl, 0.0, wsu.data_ptr(), wsb, stream)
+            if su == 1:
+                wgf = lambda: lib.adh_conv3x3_unpadded_bwd_filter_tiles(0, K, N, Ci, Co, Hu, Wu, xu_tbl, yu_tbl, gwu.data_ptr(), 0.0,
+                                                                        wsu.data_ptr(), wsb, stream)
+            else:
+                wgf = lambda: lib.adh_conv2d_unpadded_bwd_filter_tiles(0, K, N, Ci, Co, Hu, Wu, 3, 3, su, su, 1, 1, 1, 1, xu_tbl, yu_tbl,
+                                                                       gwu.data_ptr(), 0.0, wsu.data_ptr(), wsb, stream)
+            add("conv fwd over tiles without halo, fp32, N=32, 4 tiles: " + nm, f, "mfma", flop, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+            add("conv bwd-data into tiles without halo, fp32: " + nm, b, "mfma", flop, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+            add("conv bwd-filter over tiles without halo, fp32: " + nm, wgf, "mfma", flop, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
+            del xu, yu, wu_, gwu, wsu
         # batch norm with tile-local statistics + rectifier + halo pad in one call (the BN -> ReLU -> HaloPad
         # prefix of the spatially-parallel residual block) on cfg1's 4 tiles, and its backward
         xb = [torch.randn((N, C, Ht, W), device="cuda", generator=g) + 0.5 for _ in range(K)]
