@@ -510,14 +510,15 @@ static uint32_t conv_bf16_passes(int which, uint32_t Cin, uint32_t Cout) {
   return ((which == ADH_CONV_FWD ? Cin : Cout) + 63u) / 64u;
 }
 
-// name of the kernel a bf16 forward / backward-data call runs, for tiles aligned to 16 bytes
+// name of the kernel a bf16 forward / backward-data call over padded tiles runs, for tiles aligned to 16 bytes
+// (template arguments: old output added, sums of earlier passes read, sums written for a later pass, tiles without halo)
 const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, float beta) {
   if (!conv_bf16_mfma_supported(which, Cin, Cout, H, W)) return "widen_bf16_kernel + conv3x3_f32_kernel + narrow_bf16_kernel";
   if (conv_bf16_passes(which, Cin, Cout) > 1u)
-    return beta != 0.f ? "conv3x3_bf16_w8_kernel<true, false, true> + <false, true, true> per middle pass + <false, true, false>"
-                       : "conv3x3_bf16_w8_kernel<false, false, true> + <false, true, true> per middle pass + <false, true, false>";
+    return beta != 0.f ? "conv3x3_bf16_w8_kernel<true, false, true, false> + <false, true, true, false> per middle pass + <false, true, false, false>"
+                       : "conv3x3_bf16_w8_kernel<false, false, true, false> + <false, true, true, false> per middle pass + <false, true, false, false>";
   const bool w8 = which == ADH_CONV_FWD ? (W % 2u) == 0u : (W % 8u) == 0u;
-  if (w8) return beta != 0.f ? "conv3x3_bf16_w8_kernel<true, false, false>" : "conv3x3_bf16_w8_kernel<false, false, false>";
+  if (w8) return beta != 0.f ? "conv3x3_bf16_w8_kernel<true, false, false, false>" : "conv3x3_bf16_w8_kernel<false, false, false, false>";
   return beta != 0.f ? "conv3x3_bf16_kernel<true>" : "conv3x3_bf16_kernel<false>";
 }
 

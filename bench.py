@@ -34,7 +34,7 @@ if ROOT not in sys.path:
 # are profiles/conv3x3_bf16_fwd_cfg5_hbm_traffic.txt and profiles/conv3x3_fwd_cfg2_hbm_traffic.txt.
 # Not re-measured by this script; each figure belongs to the kernel instance named beside it and is
 # left out (null) when the library routes the shape to another instance.
-CONV_FWD_CFG5_TRAFFIC = ("conv3x3_bf16_w8_kernel<false, false, false>", 1085.7e6)
+CONV_FWD_CFG5_TRAFFIC = ("conv3x3_bf16_w8_kernel<false, false, false, false>", 1085.7e6)
 CONV_FWD_CFG2_TRAFFIC = ("conv3x3_f32_kernel<25, 8, false, 12>", 64.07e6)
 CLOCK_RAMP_MS = 150.0
 HBM_PEAK_GBS = 8000.0
