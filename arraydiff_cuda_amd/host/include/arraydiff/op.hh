@@ -243,6 +243,14 @@ public:
   VarData(VShape shape, VShape offset, VShape stride, size_t batch_shape)
       : val_(shape, offset, stride, batch_shape), grad_(shape, offset, stride, batch_shape) {}
   VarData clone() const { return *this; }
+  // Not in the reference.  This variable's gradient becomes the SAME buffer as `other`'s (same shape): whoever
+  // writes one writes the other.  For a node whose input gradient equals its output gradient (a sum's) and whose
+  // input has no other consumer: no copy is needed.
+  void alias_grad(VarData &other) {
+    if (other.shape() != shape() || other.offset() != offset() || other.stride() != stride() || other.batch_shape() != batch_shape())
+      throw std::invalid_argument("VarData::alias_grad: the two variables must have one layout");
+    grad_ = other.grad_;
+  }
   TxnVar<V> &val() { return val_; }
   TxnVar<V> &grad() { return grad_; }
   VShape shape() const { return val_.shape(); }
@@ -1278,19 +1286,25 @@ class SumJoin {};
 template <typename V, typename Join>
 class JoinOp : public virtual Op, public virtual Var<V> {
 public:
-  static shared_ptr<Var<V>> Make(Join join, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
-    return make_shared<JoinOp<V, Join>>(join, false, inputs, ctx);
+  // sole_consumer_of (not in the reference): the index of an input that NO other node consumes, or -1.  The gradient
+  // of such an input is the output's gradient and nothing else, so the output's gradient variable takes the
+  // input's buffer and the backward pass copies nothing for it.  (An input that another node also consumes must not
+  // be named: that node's contribution would land in the output's gradient and reach the other inputs.)
+  static shared_ptr<Var<V>> Make(Join join, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx,
+                                 int sole_consumer_of = -1) {
+    return make_shared<JoinOp<V, Join>>(join, false, inputs, ctx, sole_consumer_of);
   }
   // inputs.at(j).at(rank)
   static vector<shared_ptr<Var<V>>> MakeParallel(Join join, vector<vector<shared_ptr<Var<V>>>> inputs,
-                                                 shared_ptr<Context> ctx) {
+                                                 shared_ptr<Context> ctx, int sole_consumer_of = -1) {
     return make_per_rank<V>(ctx, [&](size_t r, shared_ptr<Context> dc) {
       vector<shared_ptr<Var<V>>> dev_inputs;
       for (auto &in : inputs) dev_inputs.push_back(in.at(r));
-      return Make(join, dev_inputs, dc);
+      return Make(join, dev_inputs, dc, sole_consumer_of);
     });
   }
-  JoinOp(Join, bool in_place, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) : ctx_(ctx), inputs_(inputs) {
+  JoinOp(Join, bool in_place, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx, int sole_consumer_of = -1)
+      : ctx_(ctx), inputs_(inputs) {
     if (in_place) throw std::invalid_argument("JoinOp: the in-place form is not part of this path");
     if (inputs.empty() || inputs.size() > ADH_MAX_TILES) throw std::invalid_argument("JoinOp: 1..16 inputs");
     for (auto &in : inputs) {
@@ -1299,6 +1313,12 @@ public:
       xs_.push_back(in->data());
     }
     y_ = VarData<V>(inputs[0]->shape(), inputs[0]->batch_shape());
+    grad_shared_.assign(inputs.size(), false);
+    if (sole_consumer_of >= 0) {
+      if ((size_t)sole_consumer_of >= inputs.size()) throw std::invalid_argument("JoinOp: no such input");
+      y_.alias_grad(xs_[(size_t)sole_consumer_of]);
+      grad_shared_[(size_t)sole_consumer_of] = true;
+    }
   }
   virtual void _push(EpochId e, function<void(Op *)> apply) {
     if (1 == stack_.push(e)) {
@@ -1321,14 +1341,16 @@ private:
   vector<shared_ptr<Var<V>>> inputs_;
   vector<VarData<V>> xs_;
   VarData<V> y_;
+  vector<bool> grad_shared_;  // the input's gradient buffer is the output's
 };
 template <typename V>
 shared_ptr<Var<V>> sum(vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
   return JoinOp<V, SumJoin>::Make(SumJoin(), inputs, ctx);
 }
 template <typename V>
-vector<shared_ptr<Var<V>>> parallel_sum(vector<vector<shared_ptr<Var<V>>>> inputs, shared_ptr<Context> ctx) {
-  return JoinOp<V, SumJoin>::MakeParallel(SumJoin(), inputs, ctx);
+vector<shared_ptr<Var<V>>> parallel_sum(vector<vector<shared_ptr<Var<V>>>> inputs, shared_ptr<Context> ctx,
+                                        int sole_consumer_of = -1) {
+  return JoinOp<V, SumJoin>::MakeParallel(SumJoin(), inputs, ctx, sole_consumer_of);
 }
 
 // ---------------------------------------------------------------------------

@@ -958,6 +958,7 @@ void JoinOp<V3, SumJoin>::_backward(TxnId txn) {
   const TileDims d = dims_of(dy);
   const size_t batch = d.N;
   for (size_t j = 0; j < xs_.size(); ++j) {
+    if (grad_shared_[j]) continue;  // the input's gradient IS dy (one buffer): nothing to copy
     // the first toucher of an input's gradient copies dy into it, later ones add
     bool first = false;
     if (xs_[j].grad().accumulate(txn, id(), ctx, [batch, &first](V3 *g) {

@@ -255,7 +255,10 @@ static void put_tile(std::vector<float> &full, const std::vector<float> &t, size
 // HaloExch -> conv -> (+ x).  Every rank's batch norm uses its own tile's statistics.  Oracle: the
 // same chain with per-tile batch norms and UNSPLIT convolutions.
 // fused: batch norm + rectifier + halo pad as one node (SlabBatchNorm2DOp with relu and out_halo) instead of three
-static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, size_t W, bool fused = false) {
+// shared_grad: the sum's output gradient and the second conv's output gradient are one buffer (JoinOp's
+// sole_consumer_of): the backward pass copies dy once instead of twice
+static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, size_t W, bool fused = false,
+                                        bool shared_grad = false) {
   std::mt19937 gen(31337 + (unsigned)K);
   auto ctx = MultiGPUContext::Make(K);
   typedef GPUBatchArray3D<float> V;
@@ -287,7 +290,7 @@ static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, 
   auto exch2 = HaloExch2DOp<V>::MakeParallel(1, pad2, ctx);
   auto conv2 = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch2, vector<shared_ptr<Var<A>>>(K, w2_src), ctx);
   vector<vector<shared_ptr<Var<V>>>> join_inputs{inputs, conv2};
-  auto join = parallel_sum<V>(join_inputs, ctx);
+  auto join = parallel_sum<V>(join_inputs, ctx, shared_grad ? 1 : -1);
   auto y_full = SpatialJoinedGather2DOp<V>::Make(join, ctx);
   auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
   sink->set_host_grad(dY.data());
@@ -1032,6 +1035,8 @@ int main(int argc, char **argv) {
     test_spatial_residual_block(2, 4, 64, 28, 28);
     test_spatial_residual_block(4, 2, 8, 16, 12, true);
     test_spatial_residual_block(2, 4, 64, 28, 28, true);
+    test_spatial_residual_block(4, 2, 8, 16, 12, true, true);
+    test_spatial_residual_block(2, 4, 64, 28, 28, false, true);
     test_spatial_pool_graph(kMaxPool, 4, 2, 8, 16, 12);
     test_spatial_pool_graph(kAveragePool, 2, 3, 5, 8, 10);
     test_spatial_pool_graph(kMaxPool, 4, 8, 64, 112, 112);
