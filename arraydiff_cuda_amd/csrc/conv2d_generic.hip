@@ -54,8 +54,13 @@ struct ConvGenParams {
   // input rows -in_H .. -1 of tile t > 0 are the last rows of tile t - 1, rows in_H .. 2 in_H - 1 of tile
   // t < num_tiles - 1 the first rows of tile t + 1; what lies outside the tensor is zero
   uint32_t num_tiles;
+  // ksplit > 1: the channel chunks are dealt to ksplit workgroups per block of pixels; each writes its fp32 sums
+  // to part[split][tile] (laid out like an output tile) and a second kernel adds them in a fixed order
+  uint32_t ksplit, chunks_per_split;
+  float *part;
+  uint64_t part_tile_elems;
   float beta;
-  FastDiv div_bpi, div_MG, div_N, div_PCP, div_BC, div_live, div_PPI;
+  FastDiv div_bpi, div_MG, div_N, div_PCP, div_BC, div_live, div_PPI, div_ksplit;
   GenSub sub[kGenMaxSub];
   int16_t off_r[kGenMaxTaps], off_c[kGenMaxTaps];
 };
@@ -124,9 +129,11 @@ __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenP
   float *patch = gen_lds + P.w_lds_floats;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
 
-  // block -> (tile, image, m group, sub-problem, block row, block column)
-  uint32_t outer, inner;
-  P.div_bpi.divmod(blockIdx.x, outer, inner);
+  // block -> (tile, image, m group, sub-problem, block row, block column), split of the channel chunks
+  uint32_t outer, inner, bid = blockIdx.x, ks = 0;
+  if (P.ksplit > 1u) P.div_ksplit.divmod(blockIdx.x, bid, ks);
+  const uint32_t ch_lo = ks * P.chunks_per_split, ch_hi = min(P.nchunks, ch_lo + P.chunks_per_split);
+  P.div_bpi.divmod(bid, outer, inner);
   uint32_t img, mg;
   P.div_MG.divmod(outer, img, mg);
   uint32_t tile, ng;
@@ -253,12 +260,12 @@ __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenP
   };
 
   const uint32_t ntaps_s = S.t1 - S.t0;
-  if (ntaps_s > 0) {
+  if (ntaps_s > 0 && ch_lo < ch_hi) {
     const uint32_t ngroups = (ntaps_s + P.TG - 1u) / P.TG;
-    const uint32_t total = P.nchunks * ngroups;
-    uint32_t ch = 0, gi = 0;
-    load_patch(0);
-    load_filter(0, S.t0, min(P.TG, ntaps_s));
+    const uint32_t total = (ch_hi - ch_lo) * ngroups;
+    uint32_t ch = ch_lo, gi = 0;
+    load_patch(ch_lo);
+    load_filter(ch_lo, S.t0, min(P.TG, ntaps_s));
     for (uint32_t it = 0; it < total; ++it) {
       const uint32_t tg0 = S.t0 + gi * P.TG;
       const uint32_t ntg = min(P.TG, S.t1 - tg0);
@@ -331,9 +338,33 @@ __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenP
         if (m >= P.M) continue;
         const size_t o = (size_t)m * P.out_H * P.out_W + pix_out;
         float v = acc[q][mt][k];
+        if (P.ksplit > 1u) {
+          P.part[((size_t)ks * P.num_tiles + tile) * P.part_tile_elems + (size_t)n * P.M * P.out_H * P.out_W + o] = v;
+          continue;
+        }
         if (P.beta != 0.f) v += gen_ld(dst, o);
         gen_st(dst, o, v);
       }
+  }
+}
+
+// out[tile][e] = beta * out[tile][e] + part[0][tile][e] + part[1][tile][e] + ... (a fixed order: reproducible)
+struct SplitReduceParams {
+  void *out[ADH_MAX_TILES];
+  const float *part;
+  uint64_t tile_elems;
+  uint32_t num_tiles, ksplit;
+  float beta;
+};
+template <typename T>
+__global__ __launch_bounds__(256) void conv_gen_split_reduce_kernel(const SplitReduceParams R) {
+  const uint32_t tile = blockIdx.y;
+  T *out = reinterpret_cast<T *>(R.out[tile]);
+  for (uint64_t e = (uint64_t)blockIdx.x * 256u + threadIdx.x; e < R.tile_elems; e += (uint64_t)gridDim.x * 256u) {
+    float v = R.part[(size_t)tile * R.tile_elems + e];
+    for (uint32_t k = 1; k < R.ksplit; ++k) v += R.part[((size_t)k * R.num_tiles + tile) * R.tile_elems + e];
+    if (R.beta != 0.f) v += gen_ld(out, e);
+    gen_st(out, e, v);
   }
 }
 
@@ -342,7 +373,7 @@ __global__ __launch_bounds__(kGenThreads, 2) void conv_gen_kernel(const ConvGenP
 struct GenPlan {
   ConvGenParams P;
   FilterGenParams F;
-  size_t lds_bytes, wt_bytes;
+  size_t lds_bytes, wt_bytes, part_bytes;  // part_bytes: the partial sums of a launch whose channel chunks are split
   uint32_t MT, num_tiles;
   bool nbr;  // tiles without halo: the kernel instances that read rows from the neighbouring tiles
 };
@@ -505,6 +536,19 @@ static int gen_finish_plan(GenPlan *plan) {
     const uint64_t blocks = (uint64_t)std::max(plan->num_tiles, 1u) * P.NG * P.MG * P.blocks_per_image;
     if (plan->MT == 1u || blocks >= kGenFillBlocks) break;
   }
+  // Still a thin launch at 16 output channels per block (the late layers of a net split over ranks: a 2x8 tile
+  // with 512 channels makes 256 workgroups, one wave per SIMD, each waiting for its next chunk with nothing else
+  // to run): deal the channel chunks to up to four workgroups per block of pixels, three of which share a CU,
+  // and add their sums in a second kernel.
+  const uint64_t blocks = (uint64_t)std::max(plan->num_tiles, 1u) * P.NG * P.MG * P.blocks_per_image;
+  P.ksplit = 1;
+  if (blocks < kGenFillBlocks && P.nchunks >= 8u)
+    P.ksplit = (uint32_t)std::min<uint64_t>(std::min<uint64_t>(4u, P.nchunks / 4u), (768u + blocks - 1u) / blocks);
+  P.chunks_per_split = (P.nchunks + P.ksplit - 1u) / P.ksplit;
+  P.ksplit = (P.nchunks + P.chunks_per_split - 1u) / P.chunks_per_split;  // no split without chunks
+  P.div_ksplit = FastDiv(P.ksplit);
+  P.part_tile_elems = (uint64_t)P.N * P.M * P.out_H * P.out_W;
+  plan->part_bytes = P.ksplit > 1u ? (size_t)P.ksplit * std::max(plan->num_tiles, 1u) * P.part_tile_elems * 4u : 0u;
   return ADH_OK;
 }
 
@@ -616,14 +660,16 @@ static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *
   ConvGenParams &P = plan->P;
   if (!workspace) return ADH_ENULL;
   if (!aligned_to(workspace, 256)) return ADH_EALIGN;
-  if (workspace_bytes < plan->wt_bytes) return ADH_EWORKSPACE;
-  const uint64_t blocks = (uint64_t)num_tiles * P.NG * P.MG * P.blocks_per_image;
+  const size_t wt_room = (plan->wt_bytes + 255u) & ~(size_t)255u;
+  if (workspace_bytes < wt_room + plan->part_bytes) return ADH_EWORKSPACE;
+  const uint64_t blocks = (uint64_t)num_tiles * P.NG * P.MG * P.blocks_per_image * P.ksplit;
   if (blocks == 0) return ADH_OK;
   if (blocks >= (1ull << 24)) return ADH_EINVAL;
   plan->F.w = w;
   plan->F.wt = reinterpret_cast<float *>(workspace);
   P.wt = plan->F.wt;
   P.num_tiles = num_tiles;
+  P.part = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + wt_room);
   const uint32_t fblocks = (uint32_t)std::min<size_t>(1024, (plan->wt_bytes / 4u + 255u) / 256u);
   if (dtype == ADH_F32) {
     hipLaunchKernelGGL(conv_gen_filter_kernel<float>, dim3(fblocks), dim3(256), 0, st, plan->F);
@@ -631,6 +677,20 @@ static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *
   } else {
     hipLaunchKernelGGL(conv_gen_filter_kernel<uint16_t>, dim3(fblocks), dim3(256), 0, st, plan->F);
     launch_gen<uint16_t>(*plan, (uint32_t)blocks, st);
+  }
+  if (P.ksplit > 1u) {
+    SplitReduceParams R = {};
+    for (uint32_t t = 0; t < num_tiles; ++t) R.out[t] = P.out[t];
+    R.part = P.part;
+    R.tile_elems = P.part_tile_elems;
+    R.num_tiles = num_tiles;
+    R.ksplit = P.ksplit;
+    R.beta = P.beta;
+    const uint32_t rb = (uint32_t)std::min<uint64_t>((P.part_tile_elems + 255u) / 256u, 2048u);
+    if (dtype == ADH_F32)
+      hipLaunchKernelGGL(conv_gen_split_reduce_kernel<float>, dim3(rb, num_tiles), dim3(256), 0, st, R);
+    else
+      hipLaunchKernelGGL(conv_gen_split_reduce_kernel<uint16_t>, dim3(rb, num_tiles), dim3(256), 0, st, R);
   }
   return launch_status();
 }
@@ -1045,7 +1105,7 @@ size_t conv2d_workspace(int which, int dtype, uint32_t num_tiles, uint32_t N, ui
   if (which == ADH_CONV_FWD) e = gen_plan_fwd(g, &plan, unpadded ? pad_h : 0u, unpadded ? pad_w : 0u);
   else if (which == ADH_CONV_BWD_DATA) e = gen_plan_bwd_data(g, &plan, unpadded, pad_h, pad_w);
   if (e) return 0;
-  return (plan.wt_bytes + 255u) & ~(size_t)255u;
+  return ((plan.wt_bytes + 255u) & ~(size_t)255u) + ((plan.part_bytes + 255u) & ~(size_t)255u);
 }
 
 int conv2d_fwd(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP,
