@@ -605,6 +605,8 @@ static int pool_check_unpadded(int dtype, int mode, uint32_t num_tiles, uint32_t
                                PoolParams *P) {
   if (H == 0 || W == 0 || sh == 0 || wh == 0 || pad_h > 4096u || pad_w > 4096u) return ADH_EINVAL;
   if (H % sh != 0u || 2u * pad_h >= wh || wh - 2u * pad_h > sh || pad_h > H || wh - 1u - pad_h > H) return ADH_EINVAL;
+  // (backward) the windows of the tile above that reach into this tile must start inside that tile
+  if (pad_h + (wh - 1u - pad_h) / sh * sh > H) return ADH_EINVAL;
   const int e = pool_check(dtype, mode, num_tiles, N, C, H + 2u * pad_h, W + 2u * pad_w, wh, ww, sh, sw, P);
   if (e) return e;
   P->H = H; P->W = W; P->pad_h = pad_h; P->pad_w = pad_w; P->pad_top = pad_h; P->num_tiles = num_tiles;

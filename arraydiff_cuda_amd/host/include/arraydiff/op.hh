@@ -1406,7 +1406,8 @@ public:
     if (shape.unpadded_tiles) {
       const size_t tile_h = inputs[0]->shape().shape[1];
       if (shape.halo_padded_input || 2 * shape.pad[1] >= shape.window[1] || shape.window[1] - 2 * shape.pad[1] > shape.stride[1] ||
-          tile_h % shape.stride[1] != 0 || shape.pad[1] > tile_h || shape.window[1] - 1 - shape.pad[1] > tile_h)
+          tile_h % shape.stride[1] != 0 || shape.window[1] - 1 - shape.pad[1] > tile_h ||
+          shape.pad[1] + (shape.window[1] - 1 - shape.pad[1]) / shape.stride[1] * shape.stride[1] > tile_h)
         throw std::invalid_argument("SlabPool2DOp: tiles without halo need a row split whose outputs stitch");
     } else if (!shape.halo_padded_input && (shape.pad[0] != 0 || shape.pad[1] != 0))
       throw std::invalid_argument("SlabPool2DOp: padding needs a halo-padded input");

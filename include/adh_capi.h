@@ -404,7 +404,8 @@ int adh_pool2d_slab_bwd(int dtype, int mode, uint32_t N, uint32_t C, uint32_t HP
  * window sees ZEROS, which take part as data exactly as the zeroed halo of the padded tile does (a window of
  * negative values at the border has maximum 0, and its gradient then belongs to no pixel).  Backward computes the
  * tile's own gradient completely: the windows of the tile below that reach into this tile are evaluated here too.
- * Limits: H a multiple of sh, 0 < wh - 2 pad_h <= sh, pad_h <= H, wh - 1 - pad_h <= H (ADH_EINVAL otherwise); a band
+ * Limits: H a multiple of sh, 0 < wh - 2 pad_h <= sh, pad_h + floor((wh - 1 - pad_h) / sh) * sh <= H and
+ * wh - 1 - pad_h <= H (windows, the neighbours' too, touch adjacent tiles only; ADH_EINVAL otherwise); a band
  * of window rows must fit in LDS (rows of up to a few thousand elements; ADH_EUNIMPL beyond: use the padded entry
  * points).  y_tiles of the backward call is not read (the maximum is recomputed) and may be NULL. */
 int adh_pool2d_unpadded_fwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H,

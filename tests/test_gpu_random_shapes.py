@@ -261,3 +261,101 @@ def test_bf16_conv_over_tiles_without_halo_random(oracle, K, N, Cin, Cout, Ht, W
         assert rel_err(oracle.bf16_to_f32(host(ys[r])), y_want[:, :, r * Ht:(r + 1) * Ht, :]) <= 5e-3
         assert rel_err(oracle.bf16_to_f32(host(gs[r])), gx_want[:, :, 1 + r * Ht:1 + (r + 1) * Ht, 1:-1]) <= 5e-3
     assert rel_err(host(dw), dw_want) <= 1e-4
+
+
+def _unpadded_geometries(seed, count, max_k):
+    """(K, Ht, W, k_h, k_w, s_h, s_w, d_h, d_w, pad_h, pad_w) whose row split stitches: Ht a multiple of s_h,
+    0 < (k_h - 1) d_h + 1 - 2 pad_h <= s_h, a window that reaches the adjacent tiles only."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        kh, kw = int(rng.integers(1, max_k + 1)), int(rng.integers(1, max_k + 1))
+        sh, sw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        dh, dw = int(rng.integers(1, 3)), int(rng.integers(1, 3))
+        eh, ew = (kh - 1) * dh + 1, (kw - 1) * dw + 1
+        pads = [p for p in range(0, eh) if 0 < eh - 2 * p <= sh]
+        if not pads:
+            continue
+        pad_h = int(rng.choice(pads))
+        pad_w = int(rng.integers(0, ew))
+        Ht = sh * int(rng.integers(1, 6))
+        if pad_h > Ht or eh - 1 - pad_h > Ht:
+            continue
+        W = max(1, ew - 2 * pad_w) + int(rng.integers(0, 30))
+        out.append((int(rng.integers(1, 5)), Ht, W, kh, kw, sh, sw, dh, dw, pad_h, pad_w))
+    return out
+
+
+@pytest.mark.parametrize("K,Ht,W,kh,kw,sh,sw,dh,dw,pad_h,pad_w", _unpadded_geometries(2030, 32, 5))
+def test_general_conv_over_tiles_without_halo_random(oracle, K, Ht, W, kh, kw, sh, sw, dh, dw, pad_h, pad_w):
+    """adh_conv2d_unpadded_*_tiles against the oracle's convolution of the unsplit zero-padded tensor (rel-err 1e-5)."""
+    rng = np.random.default_rng(Ht * 977 + W * 13 + kh)
+    N, Cin, Cout = int(rng.integers(1, 4)), int(rng.integers(1, 40)), int(rng.integers(1, 40))
+    geo = (kh, kw, sh, sw, dh, dw)
+    H, OHt = K * Ht, Ht // sh
+    OW = (W + 2 * pad_w - ((kw - 1) * dw + 1)) // sw + 1
+    x = rng.uniform(-1, 1, size=(N, Cin, H, W)).astype(np.float32)
+    w = rng.standard_normal((Cout, Cin, kh, kw)).astype(np.float32)
+    dy = rng.standard_normal((N, Cout, K * OHt, OW)).astype(np.float32)
+    xp = np.zeros((N, Cin, H + 2 * pad_h, W + 2 * pad_w), np.float32)
+    xp[:, :, pad_h:pad_h + H, pad_w:pad_w + W] = x
+    y_want = np.empty(dy.shape, np.float32)
+    oracle.conv2d_slab_fwd(xp, w, sh, sw, dh, dw, y_want)
+    gp = np.empty(xp.shape, np.float32)
+    oracle.conv2d_slab_bwd_data(w, dy, sh, sw, dh, dw, gp)
+    g_want = gp[:, :, pad_h:pad_h + H, pad_w:pad_w + W]
+    gw_want = np.zeros(w.shape, np.float32)
+    oracle.conv2d_slab_bwd_filter(xp, dy, sh, sw, dh, dw, gw_want)
+    xs = [dev(x[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    dys = [dev(dy[:, :, r * OHt:(r + 1) * OHt, :].copy()) for r in range(K)]
+    d_w = dev(w)
+    ws = torch.empty(max(capi.conv2d_unpadded_workspace_bytes(wh, capi.ADH_F32, K, N, Cin, Cout, Ht, W, *geo, pad_h, pad_w)
+                         for wh in (0, 1, 2)) // 4, device="cuda")
+    ys = [torch.full((N, Cout, OHt, OW), float("nan"), device="cuda") for _ in range(K)]
+    gs = [torch.full((N, Cin, Ht, W), float("nan"), device="cuda") for _ in range(K)]
+    gw = torch.full(w.shape, float("nan"), device="cuda")
+    capi.check(capi.conv2d_unpadded_fwd_tiles(xs, d_w, ys, N, Cin, Cout, Ht, W, *geo, pad_h, pad_w, ws=ws), "fwd")
+    capi.check(capi.conv2d_unpadded_bwd_data_tiles(d_w, dys, gs, N, Cin, Cout, Ht, W, *geo, pad_h, pad_w, ws=ws), "bwd-data")
+    capi.check(capi.conv2d_unpadded_bwd_filter_tiles(xs, dys, gw, N, Cin, Cout, Ht, W, *geo, pad_h, pad_w, ws=ws), "bwd-filter")
+    assert rel_err(host(gw), gw_want) <= 1e-5
+    for r in range(K):
+        assert rel_err(host(ys[r]), y_want[:, :, r * OHt:(r + 1) * OHt, :]) <= 1e-5
+        assert rel_err(host(gs[r]), g_want[:, :, r * Ht:(r + 1) * Ht, :]) <= 1e-5
+
+
+@pytest.mark.parametrize("K,Ht,W,wh,ww,sh,sw,dh,dw,pad_h,pad_w", _unpadded_geometries(2031, 24, 4))
+def test_pool_over_tiles_without_halo_random(oracle, K, Ht, W, wh, ww, sh, sw, dh, dw, pad_h, pad_w):
+    """adh_pool2d_unpadded_*_tiles against the oracle's pooling of the unsplit zero-padded tensor (windows without
+    dilation: the geometry's dilation is dropped and the row padding chosen again for the plain window)."""
+    pads = [p for p in range(0, wh) if 0 < wh - 2 * p <= sh and p + (wh - 1 - p) // sh * sh <= Ht and wh - 1 - p <= Ht]
+    if not pads:
+        pytest.skip("no row padding stitches for this window and stride")
+    pad_h = pads[0]
+    pad_w = min(pad_w, ww - 1)
+    rng = np.random.default_rng(Ht * 31 + W * 7 + wh)
+    W = max(W, ww)
+    N, C = int(rng.integers(1, 4)), int(rng.integers(1, 9))
+    H, OHt, OW = K * Ht, Ht // sh, (W + 2 * pad_w - ww) // sw + 1
+    x = rng.uniform(-1, 1, size=(N, C, H, W)).astype(np.float32)
+    dy = rng.standard_normal((N, C, K * OHt, OW)).astype(np.float32)
+    xp = np.zeros((N, C, H + 2 * pad_h, W + 2 * pad_w), np.float32)
+    xp[:, :, pad_h:pad_h + H, pad_w:pad_w + W] = x
+    xs = [dev(x[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    dys = [dev(dy[:, :, r * OHt:(r + 1) * OHt, :].copy()) for r in range(K)]
+    for mode in (capi.ADH_POOL_AVG, capi.ADH_POOL_MAX):
+        y_want = np.empty(dy.shape, np.float32)
+        oracle.pool_slab_fwd(mode, xp, wh, ww, sh, sw, y_want)
+        gp = np.empty(xp.shape, np.float32)
+        oracle.pool_slab_bwd(mode, xp, dy, wh, ww, sh, sw, gp)
+        g_want = gp[:, :, pad_h:pad_h + H, pad_w:pad_w + W]
+        ys = [torch.full((N, C, OHt, OW), float("nan"), device="cuda") for _ in range(K)]
+        gs = [torch.full((N, C, Ht, W), float("nan"), device="cuda") for _ in range(K)]
+        capi.check(capi.pool_unpadded_fwd_tiles(mode, xs, ys, N, C, Ht, W, wh, ww, sh, sw, pad_h, pad_w), "fwd")
+        capi.check(capi.pool_unpadded_bwd_tiles(mode, xs, ys, dys, gs, N, C, Ht, W, wh, ww, sh, sw, pad_h, pad_w), "bwd")
+        for r in range(K):
+            want_y = y_want[:, :, r * OHt:(r + 1) * OHt, :]
+            if mode == capi.ADH_POOL_MAX:
+                assert np.array_equal(host(ys[r]), want_y)
+            else:
+                assert rel_err(host(ys[r]), want_y) <= 1e-5
+            assert rel_err(host(gs[r]), g_want[:, :, r * Ht:(r + 1) * Ht, :]) <= 1e-5
