@@ -43,9 +43,7 @@ namespace adh {
 constexpr int kW8Threads = 512;
 constexpr int kW8PxBytes = 160;                          // 64 channels + 32 bytes: measured, 16-byte reads of 16 neighbouring pixels run at the linear rate (4.5 cycles per wave; 8 at 144 bytes)
 constexpr int kW8RowPx = 72;                             // nine granules of eight pixels
-constexpr int kW8RowBytes = kW8RowPx * kW8PxBytes;       // 11520
-constexpr int kW8RingRows = 10;                          // 6 rows in use + 4 rows being written
-constexpr int kW8RingBytes = kW8RingRows * kW8RowBytes;  // 115200
+constexpr int kW8RingRows = 10;                          // 6 rows in use + 4 rows being written: a ring of 115200 bytes (157760 with 73-pixel rows)
 constexpr int kW8RawCh = 144;                            // a channel row in the staging area: 72 pixels
 constexpr int kW8Copies = 5;                             // 4 rows x 8 channels x 9 granules = 288 lanes of 5 x 64
 constexpr int kW8RawWave = kW8Copies * 1024;
@@ -173,8 +171,8 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   const uint32_t tr_lane = (l16 >> 2) * kW8RawCh + (l16 & 3u) * 8u;
   const uint8_t *const tr03 = raw_wave + tr_lane + g * 32u;                  // + t * 8 * kW8RawCh
   const uint8_t *const tr4 = raw_wave + tr_lane + g * 8u * kW8RawCh + 128u;
-  const uint32_t wr03 = (16u * g + l16) * kW8PxBytes + wv * 16u;             // + slot(row t) * kW8RowBytes
-  const uint32_t wr4 = (64u + l16) * kW8PxBytes + wv * 16u;                  // + slot(row g) * kW8RowBytes
+  const uint32_t wr03 = (16u * g + l16) * kW8PxBytes + wv * 16u;             // + slot(row t) * kRowBytes
+  const uint32_t wr4 = (64u + l16) * kW8PxBytes + wv * 16u;                  // + slot(row g) * kRowBytes
   uint8_t *const wr4_dummy = raw_wave + 288 * 16 + ((l16 & 7u) + 8u * g) * 16u;
   // HF, round 5: row g's tenth granule, [channel][8 pixels] at slot 288 + 8 g + channel; lane 0 of the group
   // receives its first pixel (the reads of the other lanes run on into the next slots and are not used)

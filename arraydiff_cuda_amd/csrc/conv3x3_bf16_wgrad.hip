@@ -33,8 +33,6 @@ constexpr int kWgCols = 64;                       // dy columns per strip
 constexpr int kWgLanes = 9;                       // 16-byte lanes per channel row in LDS
 constexpr int kWgPitch = kWgLanes * 16;           // 144 bytes: 66 x_pad columns, or 64 dy columns + pad
 constexpr int kWgRegion = 64 * kWgPitch;          // 9216 bytes: 64 channel rows
-constexpr int kWgStageBytes = 2 * kWgRegion;      // x_pad row, then dy row
-constexpr int kWgDmaPerStage = kWgStageBytes / 1024;  // 18 wave-wide copies
 constexpr int kWgStages = 6;                      // rows in LDS: the one being fetched + five on their way
 constexpr uint32_t kWgOutOfRange = 0x80000000u;
 constexpr uint32_t kWgPartialFloats = 64u * 64u * 9u;
