@@ -438,6 +438,13 @@ def main():
                                                             ws5.data_ptr(), ws5_bytes, stream),
             "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s",
             note="replaces conv bwd-data cfg5 + halo reduce + halo unpack cfg5 above (their times add)")
+        gu = [torch.zeros((N5, C, Ht5, W5), device="cuda", dtype=torch.bfloat16) for _ in range(K5)]
+        gu_tbl, _ku3 = capi.ptr_table([t.data_ptr() for t in gu])
+        add("conv bwd-data cfg5 into tiles without halo (bf16, beta=1: accumulates into the gradient tiles)",
+            lambda: lib.adh_conv3x3_unpadded_bwd_data_tiles(1, K5, N5, C, C, Ht5, W5, w5.data_ptr(), y5_tbl, gu_tbl, 1.0,
+                                                            ws5.data_ptr(), ws5_bytes, stream),
+            "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
+        del gu
         add("conv bwd-filter cfg5 over tiles without halo (bf16 in, fp32 filter gradient, two kernels)",
             lambda: lib.adh_conv3x3_unpadded_bwd_filter_tiles(1, K5, N5, C, C, Ht5, W5, xu_tbl, y5_tbl, gw5.data_ptr(), 0.0,
                                                               ws5.data_ptr(), ws5_bytes, stream),
