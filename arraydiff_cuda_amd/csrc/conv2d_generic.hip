@@ -556,6 +556,26 @@ struct GenShape {
   uint32_t N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, OH, OW;
 };
 
+// conv1x1.hip: forward / backward-data of a 1x1 window at stride 1 or 2 in fp32; ADH_EUNIMPL (and nothing
+// launched) for a shape it does not serve
+int conv1x1_try(bool bwd, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                uint32_t OH, uint32_t OW, uint32_t s, const void *const *in_tiles, const void *w,
+                void *const *out_tiles, float beta, hipStream_t st);
+
+size_t conv1x1_wgrad_workspace(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t OH, uint32_t OW);
+int conv1x1_wgrad_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, uint32_t OH,
+                      uint32_t OW, uint32_t sh, uint32_t sw, const void *const *x_tiles, const void *const *dy_tiles,
+                      float *dwt, float beta, void *workspace, hipStream_t st);
+
+// a window of one tap reads no neighbour and no padding: tiles with and without halo are the same thing
+static bool gen_is_pointwise(int dtype, const GenShape &g, bool unpadded, uint32_t pad_h, uint32_t pad_w) {
+  return dtype == ADH_F32 && g.kh == 1u && g.kw == 1u && g.sh == g.sw && (!unpadded || (pad_h == 0u && pad_w == 0u));
+}
+// the filter gradient's kernel takes any pair of strides
+static bool gen_is_pointwise_wgrad(int dtype, const GenShape &g, bool unpadded, uint32_t pad_h, uint32_t pad_w) {
+  return dtype == ADH_F32 && g.kh == 1u && g.kw == 1u && (!unpadded || (pad_h == 0u && pad_w == 0u));
+}
+
 static int gen_check_shape(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP,
                            uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, GenShape *g) {
   if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
@@ -655,13 +675,20 @@ static void launch_gen(const GenPlan &plan, uint32_t blocks, hipStream_t st) {
   else launch_gen_nbr<T, false>(plan, blocks, st);
 }
 
+static int gen_check_workspace(const GenPlan &plan, const void *workspace, size_t workspace_bytes) {
+  if (!workspace) return ADH_ENULL;
+  if (!aligned_to(workspace, 256)) return ADH_EALIGN;
+  const size_t wt_room = (plan.wt_bytes + 255u) & ~(size_t)255u;
+  if (workspace_bytes < wt_room + plan.part_bytes) return ADH_EWORKSPACE;
+  return ADH_OK;
+}
+
 static int gen_launch(int dtype, GenPlan *plan, uint32_t num_tiles, const void *w, void *workspace,
                       size_t workspace_bytes, hipStream_t st) {
   ConvGenParams &P = plan->P;
-  if (!workspace) return ADH_ENULL;
-  if (!aligned_to(workspace, 256)) return ADH_EALIGN;
+  const int ws = gen_check_workspace(*plan, workspace, workspace_bytes);
+  if (ws) return ws;
   const size_t wt_room = (plan->wt_bytes + 255u) & ~(size_t)255u;
-  if (workspace_bytes < wt_room + plan->part_bytes) return ADH_EWORKSPACE;
   const uint64_t blocks = (uint64_t)num_tiles * P.NG * P.MG * P.blocks_per_image * P.ksplit;
   if (blocks == 0) return ADH_OK;
   if (blocks >= (1ull << 24)) return ADH_EINVAL;
@@ -1097,7 +1124,10 @@ size_t conv2d_workspace(int which, int dtype, uint32_t num_tiles, uint32_t N, ui
   if (which == ADH_CONV_BWD_FILTER) {
     WgradGenPlan wp = {};
     if (gen_plan_wgrad(g, num_tiles, &wp, unpadded, pad_h, pad_w)) return 0;
-    return (wp.partial_bytes + 255u) & ~(size_t)255u;
+    size_t bytes = wp.partial_bytes;
+    if (gen_is_pointwise_wgrad(dtype, g, unpadded, pad_h, pad_w))
+      bytes = std::max(bytes, conv1x1_wgrad_workspace(num_tiles, N, Cin, Cout, g.OH, g.OW));
+    return (bytes + 255u) & ~(size_t)255u;
   }
   GenPlan plan = {};
   plan.num_tiles = num_tiles;
@@ -1134,6 +1164,12 @@ int conv2d_fwd(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t
     plan.P.out[t] = y_tiles[t];
   }
   plan.P.beta = beta;
+  if (gen_is_pointwise(dtype, g, unpadded, pad_h, pad_w)) {
+    e = gen_check_workspace(plan, workspace, workspace_bytes);  // not used, but the contract is one for all shapes
+    if (e) return e;
+    e = conv1x1_try(false, num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, g.sh, x_tiles, w, y_tiles, beta, as_stream(stream));
+    if (e != ADH_EUNIMPL) return e;
+  }
   return gen_launch(dtype, &plan, num_tiles, w, workspace, workspace_bytes, as_stream(stream));
 }
 
@@ -1163,6 +1199,12 @@ int conv2d_bwd_data(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uin
     plan.P.out[t] = dx_tiles[t];
   }
   plan.P.beta = beta;
+  if (gen_is_pointwise(dtype, g, unpadded, pad_h, pad_w)) {
+    e = gen_check_workspace(plan, workspace, workspace_bytes);
+    if (e) return e;
+    e = conv1x1_try(true, num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, g.sh, dy_tiles, w, dx_tiles, beta, as_stream(stream));
+    if (e != ADH_EUNIMPL) return e;
+  }
   return gen_launch(dtype, &plan, num_tiles, w, workspace, workspace_bytes, as_stream(stream));
 }
 
@@ -1197,6 +1239,15 @@ int conv2d_bwd_filter(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, u
   if (!workspace) return ADH_ENULL;
   if (!aligned_to(workspace, 256)) return ADH_EALIGN;
   if (workspace_bytes < plan.partial_bytes) return ADH_EWORKSPACE;
+  if (gen_is_pointwise_wgrad(dtype, g, unpadded, pad_h, pad_w)) {
+    const size_t need = conv1x1_wgrad_workspace(num_tiles, N, Cin, Cout, g.OH, g.OW);
+    if (need != 0) {
+      if (workspace_bytes < need) return ADH_EWORKSPACE;
+      e = conv1x1_wgrad_try(num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, g.sh, g.sw, x_tiles, dy_tiles, dwt, beta,
+                            workspace, st);
+      if (e != ADH_EUNIMPL) return e;
+    }
+  }
   plan.P.partial = reinterpret_cast<float *>(workspace);
   if (dtype == ADH_F32) launch_wgrad_gen<float>(plan, st);
   else launch_wgrad_gen<uint16_t>(plan, st);

@@ -629,6 +629,35 @@ def main():
             add("conv bwd-data into tiles without halo, fp32: " + nm, b, "mfma", flop, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
             add("conv bwd-filter over tiles without halo, fp32: " + nm, wgf, "mfma", flop, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")
             del xu, yu, wu_, gwu, wsu
+        # the 1x1 stride-2 projection shortcuts of the same net (matrix-product kernels of their own): the first is
+        # sized by memory (priced by the bytes of the pixels it uses and writes), the third by the matrix cores
+        for (Ci, Co, Hu, Wu, bound) in ((64, 128, 32, 128, "hbm"), (256, 512, 8, 32, "mfma")):
+            OHu, OWu = Hu // 2, Wu // 2
+            xu = [torch.randn((N, Ci, Hu, Wu), device="cuda", generator=g) for _ in range(K)]
+            yu = [torch.randn((N, Co, OHu, OWu), device="cuda", generator=g) for _ in range(K)]
+            wu_ = torch.randn((Co, Ci, 1, 1), device="cuda", generator=g) * (2.0 / Ci) ** 0.5
+            gwu = torch.empty((Co, Ci, 1, 1), device="cuda")
+            xu_tbl, _ku1 = capi.ptr_table([t.data_ptr() for t in xu])
+            yu_tbl, _ku2 = capi.ptr_table([t.data_ptr() for t in yu])
+            geo1 = (1, 1, 2, 2, 1, 1)
+            wsb = max(lib.adh_conv2d_workspace_bytes(wh, 0, K, N, Ci, Co, Hu, Wu, *geo1) for wh in (0, 1, 2))
+            wsu = torch.empty(wsb // 4 + 64, device="cuda")
+            flop = 2.0 * K * N * Ci * Co * OHu * OWu
+            used = 4.0 * K * N * (Ci + Co) * OHu * OWu               # sampled pixels of x + y
+            grad = 4.0 * K * N * (Ci * Hu * Wu + Co * OHu * OWu)     # dy read, the whole of dx written
+            reps, wu = 50, 10
+            nm = "1x1 stride 2 %d->%d on %dx%d tiles, fp32, N=32, 4 tiles" % (Ci, Co, Hu, Wu)
+            price = (lambda b: (b, HBM_PEAK_GBS, "GB/s")) if bound == "hbm" else (lambda b: (flop, MFMA_F32_PEAK_TFLOPS, "TFLOP/s"))
+            add("conv fwd " + nm,
+                lambda: lib.adh_conv2d_slab_fwd_tiles(0, K, N, Ci, Co, Hu, Wu, *geo1, xu_tbl, wu_.data_ptr(), yu_tbl, 0.0,
+                                                      wsu.data_ptr(), wsb, stream), bound, *price(used))
+            add("conv bwd-data " + nm,
+                lambda: lib.adh_conv2d_slab_bwd_data_tiles(0, K, N, Ci, Co, Hu, Wu, *geo1, wu_.data_ptr(), yu_tbl, xu_tbl, 0.0,
+                                                           wsu.data_ptr(), wsb, stream), bound, *price(grad))
+            add("conv bwd-filter " + nm + " (2 kernels)",
+                lambda: lib.adh_conv2d_slab_bwd_filter_tiles(0, K, N, Ci, Co, Hu, Wu, *geo1, xu_tbl, yu_tbl, gwu.data_ptr(), 0.0,
+                                                             wsu.data_ptr(), wsb, stream), bound, *price(used))
+            del xu, yu, wu_, gwu, wsu
         # batch norm with tile-local statistics + rectifier + halo pad in one call (the BN -> ReLU -> HaloPad
         # prefix of the spatially-parallel residual block) on cfg1's 4 tiles, and its backward
         xb = [torch.randn((N, C, Ht, W), device="cuda", generator=g) + 0.5 for _ in range(K)]

@@ -33,6 +33,12 @@ CASES = [  # K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw
     (1, 64, 8, 128, 18, 66, 3, 3, 1, 1, 1, 1), # enough blocks to keep them 64 output channels wide
     (1, 32, 8, 128, 18, 66, 3, 3, 1, 1, 1, 1), # half as many: 32 output channels per block
     (1, 48, 128, 8, 10, 66, 3, 3, 1, 1, 1, 1), # backward-data with 64-channel blocks and 32-channel chunks
+    # 1x1 windows with output rows of a multiple of 4 pixels take the matrix-product kernels of their own
+    (4, 5, 64, 128, 8, 32, 1, 1, 2, 2, 1, 1),    # a projection shortcut: 64 pixels x 64 channels per workgroup
+    (2, 3, 70, 150, 6, 24, 1, 1, 2, 2, 1, 1),    # channel counts off every step: padded chunks and channel blocks
+    (4, 16, 16, 130, 64, 64, 1, 1, 2, 2, 1, 1),  # 128 x 128 blocks forward (the last channel block holds 2), 128 x 64 backward
+    (4, 16, 72, 24, 32, 64, 1, 1, 1, 1, 1, 1),   # stride 1: 128 x 64 blocks forward, 128 x 128 backward
+    (3, 2, 5, 3, 2, 4, 1, 1, 2, 2, 1, 1),        # a single row of four pixels per image: most of the block is idle
 ]
 
 
