@@ -567,6 +567,11 @@ int conv1x1_wgrad_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cou
                       uint32_t OW, uint32_t sh, uint32_t sw, const void *const *x_tiles, const void *const *dy_tiles,
                       float *dwt, float beta, void *workspace, hipStream_t st);
 
+// conv3x3s2.hip: backward-data of a 3x3 window at stride 2, padding 1, over fp32 tiles of H x W without halo
+int conv3x3s2_bwd_data_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                           const void *w, const void *const *dy_tiles, void *const *dx_tiles, float beta,
+                           hipStream_t st);
+
 // a window of one tap reads no neighbour and no padding: tiles with and without halo are the same thing
 static bool gen_is_pointwise(int dtype, const GenShape &g, bool unpadded, uint32_t pad_h, uint32_t pad_w) {
   return dtype == ADH_F32 && g.kh == 1u && g.kw == 1u && g.sh == g.sw && (!unpadded || (pad_h == 0u && pad_w == 0u));
@@ -1203,6 +1208,13 @@ int conv2d_bwd_data(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uin
     e = gen_check_workspace(plan, workspace, workspace_bytes);
     if (e) return e;
     e = conv1x1_try(true, num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, g.sh, dy_tiles, w, dx_tiles, beta, as_stream(stream));
+    if (e != ADH_EUNIMPL) return e;
+  }
+  if (dtype == ADH_F32 && unpadded && kh == 3u && kw == 3u && sh == 2u && sw == 2u && dh == 1u && dw == 1u && pad_h == 1u &&
+      pad_w == 1u) {
+    e = gen_check_workspace(plan, workspace, workspace_bytes);
+    if (e) return e;
+    e = conv3x3s2_bwd_data_try(num_tiles, N, Cin, Cout, g.HP - 2u, g.WP - 2u, w, dy_tiles, dx_tiles, beta, as_stream(stream));
     if (e != ADH_EUNIMPL) return e;
   }
   return gen_launch(dtype, &plan, num_tiles, w, workspace, workspace_bytes, as_stream(stream));

@@ -1,0 +1,267 @@
+// 3x3 convolution at stride 2 with padding 1 over row tiles WITHOUT halo, fp32 matrix cores: backward-data.
+//
+// A gradient pixel dx[h][w] receives dy[i'][j'] through tap (a, b) when h = 2 i' + a - 1 and w = 2 j' + b - 1.  The
+// 2 x 2 pixels dx[2i .. 2i+1][2j .. 2j+1] (a "quad", one per dy pixel (i, j)) therefore need, per channel pair,
+//   dx[2i  ][2j  ] : tap (1,1) dy[i][j]
+//   dx[2i  ][2j+1] : tap (1,0) dy[i][j+1] + tap (1,2) dy[i][j]
+//   dx[2i+1][2j  ] : tap (0,1) dy[i+1][j] + tap (2,1) dy[i][j]
+//   dx[2i+1][2j+1] : tap (0,0) dy[i+1][j+1] + tap (0,2) dy[i+1][j] + tap (2,0) dy[i][j+1] + tap (2,2) dy[i][j]
+// nine multiplications of the dy patch (shifted by 0 or 1) with one tap each, into four accumulator sets.  The
+// general kernel makes the four sets four workgroups that stage the same dy patch four times, hold 1, 2, 2 and 4
+// taps, and write every cache line of dx in four pieces; here a workgroup owns 64 quads x 64 input channels, stages
+// the dy patch and the filter rows (read as the caller holds them) once per 16 output channels, and a lane, which
+// ends up with four neighbouring quads of one channel, writes two rows of eight consecutive pixels.
+// dy row OH of a tile is the first row of the tile below (zero below the last tile); dy column OW is zero.
+#include "adh_common.h"
+
+#include <algorithm>
+
+namespace adh {
+
+constexpr uint32_t kS2Threads = 256;
+constexpr uint32_t kS2CC = 16;       // output channels (the reduction) per staged chunk
+constexpr uint32_t kS2Quads = 64;    // quads per workgroup
+constexpr uint32_t kS2BM = 64;       // input channels per workgroup
+constexpr uint32_t kS2WPitch = kS2BM * 9u + 16u;  // floats per staged output channel of the filter
+
+struct S2BwdParams {
+  const float *dy[ADH_MAX_TILES];
+  float *dx[ADH_MAX_TILES];
+  const float *w;
+  uint32_t num_tiles, N, Cin, Cout;
+  uint32_t OH, OW;          // a dy tile; the gradient tile is 2 OH x 2 OW
+  uint32_t QR, QC, NBI;     // a workgroup's quads: NBI images x QR rows x QC columns (= 64)
+  uint32_t PRW, PPI, PPITCH;  // patch row width (QC + 1), floats per image ((QR + 1) PRW), per staged channel
+  uint32_t RB, CB, NG, MG;  // row blocks and column blocks per image and tile, image groups, input-channel groups
+  float beta;
+  FastDiv div_MG, div_CB, div_RB, div_NG;
+};
+
+typedef float s2_floatx4 __attribute__((ext_vector_type(4)));
+
+// PJ: patch elements a thread stages per chunk (kS2CC * NBI * PPI <= 256 PJ)
+template <int PJ>
+__global__ __launch_bounds__(kS2Threads, 2) void conv3x3s2_bwd_data_kernel(const S2BwdParams P) {
+  constexpr int WJ = (int)(kS2CC * kS2BM * 9u / 4u / kS2Threads);  // 16-byte filter pieces a thread stages per chunk
+  extern __shared__ __align__(16) float s2_lds[];
+  float *wl = s2_lds;                        // [kS2CC][kS2WPitch]
+  float *patch = s2_lds + kS2CC * kS2WPitch;  // [kS2CC][PPITCH]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+  const uint32_t wq = wave & 1u, wm = wave >> 1;  // quad half, channel half
+
+  uint32_t vb = blockIdx.x;
+  if ((gridDim.x & 7u) == 0u) vb = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  uint32_t r1, r2, r3, mg, cb, rb, ng, tile;
+  P.div_MG.divmod(vb, r1, mg);
+  P.div_CB.divmod(r1, r2, cb);
+  P.div_RB.divmod(r2, r3, rb);
+  P.div_NG.divmod(r3, tile, ng);
+  const uint32_t n0 = ng * P.NBI, i0 = rb * P.QR, j0 = cb * P.QC, m0 = mg * kS2BM;
+  const uint32_t y_plane = P.OH * P.OW;
+  const size_t y_image = (size_t)P.Cout * y_plane;
+
+  // ---- staging: the thread's patch elements (output channel within the chunk, place in the patch) and where
+  // they come from; an element outside the tensor points at the tile's first element and is replaced by zero
+  const float *p_ptr[PJ];
+  uint32_t p_dst[PJ];      // where the element goes in LDS (no place: past the end, never stored)
+  uint32_t p_ok = 0;       // bit j: the element lies inside the tensor
+  uint32_t p_k = 0;        // 4 bits per element: its output channel within the chunk
+  const uint32_t pp = P.NBI * P.PPI;
+  constexpr uint32_t kNoPlace = 0xffffffffu;
+#pragma unroll
+  for (int j = 0; j < PJ; ++j) {
+    const uint32_t f = tid + (uint32_t)j * kS2Threads;
+    const uint32_t k = f / pp, e = f - k * pp;
+    const uint32_t b = e / P.PPI, e2 = e - b * P.PPI;
+    const uint32_t pr = e2 / P.PRW, pc = e2 - pr * P.PRW;
+    const uint32_t row = i0 + pr, col = j0 + pc;
+    bool ok = k < kS2CC && n0 + b < P.N && col < P.OW && row <= P.OH;
+    uint32_t from = tile, rr = row;
+    if (row >= P.OH) {  // the row below the tile
+      rr = 0;
+      from = tile + 1u < P.num_tiles ? tile + 1u : tile;
+      ok = ok && tile + 1u < P.num_tiles;
+    }
+    p_ptr[j] = P.dy[from] + (ok ? (size_t)(n0 + b) * y_image + rr * P.OW + col : (size_t)0);
+    p_dst[j] = k < kS2CC ? k * P.PPITCH + e : kNoPlace;
+    p_ok |= ok ? 1u << j : 0u;
+    p_k |= (k & 15u) << (4 * j);
+  }
+  // the filter: for output channel co0 + k the 576 consecutive floats from input channel m0 on, 16 bytes at a
+  // time (Cin is a multiple of 4, so a piece lies wholly inside or outside the filter)
+  const uint32_t w_row = m0 * 9u, w_end = P.Cin * 9u;
+  float ppre[PJ];
+  s2_floatx4 wpre[WJ];
+  uint32_t pre_co = 0;
+  // (an element that does not exist loads one that does and becomes zero on the way to LDS: the selects sit on
+  // the addresses, never on the loaded values, which nothing may touch before the multiplications they overlap)
+  auto load_chunk = [&](uint32_t co0) {
+    pre_co = co0;
+#pragma unroll
+    for (int j = 0; j < PJ; ++j) {
+      const uint32_t co = min(co0 + ((p_k >> (4 * j)) & 15u), P.Cout - 1u);
+      ppre[j] = p_ptr[j][((p_ok >> j) & 1u) ? (size_t)co * y_plane : (size_t)0];
+    }
+#pragma unroll
+    for (int j = 0; j < WJ; ++j) {
+      const uint32_t f = tid + (uint32_t)j * kS2Threads;
+      const uint32_t k = f / (kS2BM * 9u / 4u), rr = (f - k * (kS2BM * 9u / 4u)) * 4u;
+      const uint32_t co = min(co0 + k, P.Cout - 1u);
+      wpre[j] = *reinterpret_cast<const s2_floatx4 *>(P.w + (w_row + rr < w_end ? co * w_end + w_row + rr : 0u));
+    }
+  };
+  auto store_chunk = [&]() {
+#pragma unroll
+    for (int j = 0; j < PJ; ++j) {
+      const uint32_t k = (p_k >> (4 * j)) & 15u;
+      if (p_dst[j] != kNoPlace) patch[p_dst[j]] = ((p_ok >> j) & 1u) && pre_co + k < P.Cout ? ppre[j] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < WJ; ++j) {
+      const uint32_t f = tid + (uint32_t)j * kS2Threads;
+      const uint32_t k = f / (kS2BM * 9u / 4u), rr = (f - k * (kS2BM * 9u / 4u)) * 4u;
+      const bool ok = w_row + rr < w_end && pre_co + k < P.Cout;
+      *reinterpret_cast<s2_floatx4 *>(wl + k * kS2WPitch + rr) = ok ? wpre[j] : s2_floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+
+  // ---- this lane's quads: quad l16 of each of its wave's two 16-quad tiles, as an offset into a patch plane
+  uint32_t q_off[2];
+#pragma unroll
+  for (int pt = 0; pt < 2; ++pt) {
+    const uint32_t q = wq * 32u + (uint32_t)pt * 16u + l16;
+    const uint32_t per = P.QR * P.QC;
+    const uint32_t b = q / per, q2 = q - b * per;
+    const uint32_t qi = q2 / P.QC, qj = q2 - qi * P.QC;
+    q_off[pt] = b * P.PPI + qi * P.PRW + qj + g * P.PPITCH;
+  }
+  const float *b_base = wl + g * kS2WPitch + (wm * 32u + l16) * 9u;
+
+  // acc[class 2 pr + pc][quad tile][channel tile]
+  s2_floatx4 acc[4][2][2];
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+#pragma unroll
+    for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+      for (int ct = 0; ct < 2; ++ct) acc[c][pt][ct] = s2_floatx4{0.f, 0.f, 0.f, 0.f};
+
+  load_chunk(0);
+  for (uint32_t co0 = 0; co0 < P.Cout; co0 += kS2CC) {
+    __syncthreads();
+    store_chunk();
+    __syncthreads();
+    if (co0 + kS2CC < P.Cout) load_chunk(co0 + kS2CC);
+#pragma unroll
+    for (int kk = 0; kk < (int)kS2CC / 4; ++kk) {
+      // the patch at the four shifts (di, dj), then tap by tap
+      float a[2][2][2];
+#pragma unroll
+      for (int di = 0; di < 2; ++di)
+#pragma unroll
+        for (int dj = 0; dj < 2; ++dj)
+#pragma unroll
+          for (int pt = 0; pt < 2; ++pt) a[di][dj][pt] = patch[(uint32_t)(4 * kk) * P.PPITCH + q_off[pt] + (uint32_t)di * P.PRW + (uint32_t)dj];
+#pragma unroll
+      for (int ta = 0; ta < 3; ++ta)
+#pragma unroll
+        for (int tb = 0; tb < 3; ++tb) {
+          float b[2];
+#pragma unroll
+          for (int ct = 0; ct < 2; ++ct) b[ct] = b_base[(4 * kk) * (int)kS2WPitch + ct * 144 + ta * 3 + tb];
+          const int cls = (ta == 1 ? 0 : 2) + (tb == 1 ? 0 : 1);
+          const int di = ta == 0 ? 1 : 0, dj = tb == 0 ? 1 : 0;
+#pragma unroll
+          for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+            for (int ct = 0; ct < 2; ++ct)
+              acc[cls][pt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[di][dj][pt], b[ct], acc[cls][pt][ct], 0, 0, 0);
+        }
+    }
+  }
+
+  // ---- the lane holds quads 4 g .. 4 g + 3 of each tile (one dy row: QC is a multiple of 4) for channel l16 of
+  // each channel tile: two rows of eight consecutive gradient pixels
+  const uint32_t W = 2u * P.OW;
+  const size_t x_plane = (size_t)(2u * P.OH) * W;
+#pragma unroll
+  for (int pt = 0; pt < 2; ++pt) {
+    const uint32_t q = wq * 32u + (uint32_t)pt * 16u + 4u * g;
+    const uint32_t per = P.QR * P.QC;
+    const uint32_t b = q / per, q2 = q - b * per;
+    const uint32_t qi = q2 / P.QC, qj = q2 - qi * P.QC;
+    if (b >= P.NBI || n0 + b >= P.N || i0 + qi >= P.OH || j0 + qj >= P.OW) continue;
+    float *o_px = P.dx[tile] + (size_t)(n0 + b) * P.Cin * x_plane + (size_t)(2u * (i0 + qi)) * W + 2u * (j0 + qj);
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) {
+      const uint32_t m = m0 + wm * 32u + (uint32_t)ct * 16u + l16;
+      if (m >= P.Cin) continue;
+      float *o = o_px + (size_t)m * x_plane;
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        const s2_floatx4 e = acc[2 * pr][pt][ct], d = acc[2 * pr + 1][pt][ct];
+        s2_floatx4 lo = {e[0], d[0], e[1], d[1]}, hi = {e[2], d[2], e[3], d[3]};
+        float *row = o + (size_t)pr * W;
+        if (P.beta != 0.f) {
+          lo += *reinterpret_cast<const s2_floatx4 *>(row);
+          hi += *reinterpret_cast<const s2_floatx4 *>(row + 4);
+        }
+        *reinterpret_cast<s2_floatx4 *>(row) = lo;
+        *reinterpret_cast<s2_floatx4 *>(row + 4) = hi;
+      }
+    }
+  }
+}
+
+// Backward-data of a 3x3 window at stride 2, padding 1, over fp32 tiles of H x W without halo (dy tiles of
+// H/2 x W/2).  ADH_EUNIMPL: not a shape this kernel serves (the caller takes the general kernel); nothing launched.
+int conv3x3s2_bwd_data_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                           const void *w, const void *const *dy_tiles, void *const *dx_tiles, float beta,
+                           hipStream_t st) {
+  if (H % 2u != 0u || W % 2u != 0u || H == 0 || W == 0) return ADH_EUNIMPL;
+  const uint32_t OH = H / 2u, OW = W / 2u;
+  // a workgroup's 64 quads: rows of 8 or 16 dy pixels
+  if (OW != 8u && OW % 16u != 0u) return ADH_EUNIMPL;
+  const uint32_t QC = std::min(OW, 16u);
+  uint32_t QR = std::min(OH, kS2Quads / QC);
+  while (QR > 1u && OH % QR != 0u) --QR;
+  if ((kS2Quads / QC) % QR != 0u) return ADH_EUNIMPL;
+  const uint32_t NBI = kS2Quads / (QC * QR);
+  if (!aligned_to(w, 16) || Cin % 4u != 0u) return ADH_EUNIMPL;
+  for (uint32_t t = 0; t < num_tiles; ++t)
+    if (!aligned_to(dx_tiles[t], 16) || !aligned_to(dy_tiles[t], 4)) return ADH_EUNIMPL;
+  if ((uint64_t)Cin * Cout * 9u >= (1ull << 31) || (uint64_t)H * W >= (1ull << 30)) return ADH_EUNIMPL;
+
+  S2BwdParams P = {};
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    P.dy[t] = reinterpret_cast<const float *>(dy_tiles[t]);
+    P.dx[t] = reinterpret_cast<float *>(dx_tiles[t]);
+  }
+  P.w = reinterpret_cast<const float *>(w);
+  P.num_tiles = num_tiles; P.N = N; P.Cin = Cin; P.Cout = Cout;
+  P.OH = OH; P.OW = OW;
+  P.QR = QR; P.QC = QC; P.NBI = NBI;
+  P.PRW = QC + 1u;
+  P.PPI = (QR + 1u) * P.PRW;
+  const uint32_t pp = NBI * P.PPI;
+  // the four shifted reads of a wave cover runs of 16 consecutive floats in 4 channel planes: planes 16 banks apart
+  P.PPITCH = (pp + 63u) / 64u * 64u + 16u;
+  P.RB = OH / QR; P.CB = OW / QC; P.NG = (N + NBI - 1u) / NBI; P.MG = (Cin + kS2BM - 1u) / kS2BM;
+  P.beta = beta;
+  P.div_MG = FastDiv(P.MG); P.div_CB = FastDiv(P.CB); P.div_RB = FastDiv(P.RB); P.div_NG = FastDiv(P.NG);
+  const uint64_t blocks = (uint64_t)num_tiles * P.NG * P.RB * P.CB * P.MG;
+  if (blocks == 0 || blocks >= (1ull << 31)) return ADH_EUNIMPL;
+  const uint32_t pj = (kS2CC * pp + kS2Threads - 1u) / kS2Threads;
+  const size_t lds = (size_t)(kS2CC * kS2WPitch + kS2CC * P.PPITCH) * sizeof(float);
+  if (lds > 64u * 1024u) return ADH_EUNIMPL;
+  if (pj <= 6u)
+    hipLaunchKernelGGL((conv3x3s2_bwd_data_kernel<6>), dim3((uint32_t)blocks), dim3(kS2Threads), lds, st, P);
+  else if (pj <= 8u)
+    hipLaunchKernelGGL((conv3x3s2_bwd_data_kernel<8>), dim3((uint32_t)blocks), dim3(kS2Threads), lds, st, P);
+  else
+    return ADH_EUNIMPL;
+  return launch_status();
+}
+
+}  // namespace adh

@@ -28,6 +28,11 @@ CASES = [  # K, N, Cin, Cout, Ht, W, kh, kw, sh, sw, dh, dw, pad_h, pad_w
     (5, 2, 64, 64, 2, 72, 3, 3, 1, 1, 1, 1, 1, 1),    # wide rows, five tiles of two rows
     (2, 1, 12, 20, 4, 12, 5, 5, 1, 1, 1, 1, 2, 2),    # 5x5: two rows from each neighbour
     (4, 32, 8, 16, 2, 8, 3, 3, 2, 2, 1, 1, 1, 1),     # 1x4 outputs per tile: many images per block
+    # stride-2 3x3 whose backward-data takes the kernel of its own (fp32, output rows of 8 or a multiple of 16 pixels)
+    (2, 6, 20, 24, 4, 16, 3, 3, 2, 2, 1, 1, 1, 1),    # 2x8 outputs: four images per workgroup, the second group holds two
+    (3, 2, 8, 40, 16, 64, 3, 3, 2, 2, 1, 1, 1, 1),    # 8x32 outputs: two row blocks and two column blocks per image
+    (2, 3, 68, 16, 4, 32, 3, 3, 2, 2, 1, 1, 1, 1),    # 2x16 outputs: two images per workgroup, a second channel group of 4
+    (1, 2, 4, 4, 16, 16, 3, 3, 2, 2, 1, 1, 1, 1),     # 8x8 outputs on a single tile: zeros below
 ]
 
 
