@@ -39,6 +39,8 @@ struct S2BwdParams {
 
 typedef float s2_floatx4 __attribute__((ext_vector_type(4)));
 
+static bool s2_quads(uint32_t OH, uint32_t OW, uint32_t *QR, uint32_t *QC, uint32_t *NBI);
+
 // PJ: patch elements a thread stages per chunk (kS2CC * NBI * PPI <= 256 PJ)
 template <int PJ>
 __global__ __launch_bounds__(kS2Threads, 2) void conv3x3s2_bwd_data_kernel(const S2BwdParams P) {
@@ -221,13 +223,8 @@ int conv3x3s2_bwd_data_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_
                            hipStream_t st) {
   if (H % 2u != 0u || W % 2u != 0u || H == 0 || W == 0) return ADH_EUNIMPL;
   const uint32_t OH = H / 2u, OW = W / 2u;
-  // a workgroup's 64 quads: rows of 8 or 16 dy pixels
-  if (OW != 8u && OW % 16u != 0u) return ADH_EUNIMPL;
-  const uint32_t QC = std::min(OW, 16u);
-  uint32_t QR = std::min(OH, kS2Quads / QC);
-  while (QR > 1u && OH % QR != 0u) --QR;
-  if ((kS2Quads / QC) % QR != 0u) return ADH_EUNIMPL;
-  const uint32_t NBI = kS2Quads / (QC * QR);
+  uint32_t QR, QC, NBI;
+  if (!s2_quads(OH, OW, &QR, &QC, &NBI)) return ADH_EUNIMPL;
   if (!aligned_to(w, 16) || Cin % 4u != 0u) return ADH_EUNIMPL;
   for (uint32_t t = 0; t < num_tiles; ++t)
     if (!aligned_to(dx_tiles[t], 16) || !aligned_to(dy_tiles[t], 4)) return ADH_EUNIMPL;
@@ -261,6 +258,247 @@ int conv3x3s2_bwd_data_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_
     hipLaunchKernelGGL((conv3x3s2_bwd_data_kernel<8>), dim3((uint32_t)blocks), dim3(kS2Threads), lds, st, P);
   else
     return ADH_EUNIMPL;
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward: y[co][i][j] = sum over ci and taps of w[co][ci][a][b] * x[ci][2 i + a - 1][2 j + b - 1]
+// A workgroup owns 64 output pixels (NBI images x QR rows x QC columns) x 64 output channels and stages, per 16
+// input channels, the (2 QR + 1) x (2 QC + 1) input patch of every image and the filter rows as the caller holds
+// them.  A patch row is stored with its even columns first and its odd columns after them, so that the 16
+// pixels of a matrix tile read 16 consecutive floats for every tap.  Input row -1 of a tile is the last row of
+// the tile above (zero above the first tile); column -1 is zero.
+// ---------------------------------------------------------------------------------------------
+constexpr uint32_t kS2FwdWPitch = kS2CC * 9u + 4u;  // floats per staged output channel: 16 input channels x 9 taps
+
+struct S2FwdParams {
+  const float *x[ADH_MAX_TILES];
+  float *y[ADH_MAX_TILES];
+  const float *w;
+  uint32_t num_tiles, N, Cin, Cout;
+  uint32_t OH, OW;
+  uint32_t QR, QC, NBI;
+  uint32_t PRW, PPI, PPITCH;  // patch row width (2 QC + 1), floats per image ((2 QR + 1) PRW), per staged channel
+  uint32_t RB, CB, NG, MG;
+  float beta;
+  FastDiv div_MG, div_CB, div_RB, div_NG, div_PPI, div_PRW;
+};
+
+// NP: patch places a thread stages (NBI * PPI <= 128 NP); threads 0-127 stage them for the chunk's first eight
+// input channels, threads 128-255 for the other eight
+template <int NP>
+__global__ __launch_bounds__(kS2Threads, 2) void conv3x3s2_fwd_kernel(const S2FwdParams P) {
+  constexpr int WJ = (int)(kS2BM * kS2CC * 9u / 4u / kS2Threads);  // 16-byte filter pieces per thread and chunk
+  constexpr uint32_t kRowPieces = kS2CC * 9u / 4u;                  // pieces per output channel
+  extern __shared__ __align__(16) float s2_lds[];
+  float *wl = s2_lds;                            // [kS2BM][kS2FwdWPitch]
+  float *patch = s2_lds + kS2BM * kS2FwdWPitch;  // [kS2CC][PPITCH]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+  const uint32_t wq = wave & 1u, wm = wave >> 1;
+
+  uint32_t vb = blockIdx.x;
+  if ((gridDim.x & 7u) == 0u) vb = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  uint32_t r1, r2, r3, mg, cb, rb, ng, tile;
+  P.div_MG.divmod(vb, r1, mg);
+  P.div_CB.divmod(r1, r2, cb);
+  P.div_RB.divmod(r2, r3, rb);
+  P.div_NG.divmod(r3, tile, ng);
+  const uint32_t n0 = ng * P.NBI, i0 = rb * P.QR, j0 = cb * P.QC, m0 = mg * kS2BM;
+  const uint32_t H = 2u * P.OH, W = 2u * P.OW;
+  const uint32_t x_plane = H * W;
+  const float *x_own = P.x[tile];
+  const float *x_up = P.x[tile > 0u ? tile - 1u : tile];
+
+  // ---- staging: the thread's places in the patch (the same for each of its eight channels).  Offsets are relative
+  // to the tile, or to the tile above for input row -1
+  const uint32_t half = tid >> 7, t128 = tid & 127u;
+  uint32_t p_off[NP], p_dst[NP];
+  uint32_t p_ok = 0, p_up = 0, p_has = 0;  // inside the tensor / from the tile above / a place of the patch
+  const uint32_t even_cols = P.QC + 1u;
+  const uint32_t pp = P.NBI * P.PPI;
+#pragma unroll
+  for (int j = 0; j < NP; ++j) {
+    const uint32_t e = t128 + (uint32_t)j * 128u;
+    uint32_t b, e2, pr, pc;
+    P.div_PPI.divmod(e, b, e2);
+    P.div_PRW.divmod(e2, pr, pc);
+    const int32_t row = (int32_t)(2u * i0 + pr) - 1, col = (int32_t)(2u * j0 + pc) - 1;
+    const bool has = e < pp;
+    bool ok = has && n0 + b < P.N && col >= 0;
+    const bool up = row < 0;
+    if (up) ok = ok && tile > 0u;
+    const uint32_t rr = up ? H - 1u : (uint32_t)row;
+    p_off[j] = ok ? (n0 + b) * P.Cin * x_plane + rr * W + (uint32_t)col : 0u;
+    // even columns of the patch row first, odd ones after them
+    p_dst[j] = b * P.PPI + pr * P.PRW + ((pc & 1u) ? even_cols + (pc >> 1) : (pc >> 1));
+    p_ok |= ok ? 1u << j : 0u;
+    p_up |= (ok && up) ? 1u << j : 0u;
+    p_has |= has ? 1u << j : 0u;
+  }
+  const uint32_t w_end = P.Cin * 9u;
+
+  float ppre[NP][8];
+  s2_floatx4 wpre[WJ];
+  uint32_t pre_ci = 0;
+  auto load_chunk = [&](uint32_t ci0) {
+    pre_ci = ci0;
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+      const float *base = ((p_up >> j) & 1u) ? x_up : x_own;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const uint32_t ci = min(ci0 + half * 8u + (uint32_t)c, P.Cin - 1u);
+        ppre[j][c] = base[((p_ok >> j) & 1u) ? p_off[j] + ci * x_plane : 0u];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < WJ; ++j) {
+      const uint32_t f = tid + (uint32_t)j * kS2Threads;
+      const uint32_t co_l = f / kRowPieces, rr = (f - co_l * kRowPieces) * 4u;
+      const uint32_t co = min(m0 + co_l, P.Cout - 1u);
+      const uint32_t at = ci0 * 9u + rr;  // within the output channel's Cin * 9 floats
+      wpre[j] = *reinterpret_cast<const s2_floatx4 *>(P.w + (at < w_end ? co * w_end + at : 0u));
+    }
+  };
+  auto store_chunk = [&]() {
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+      if (!((p_has >> j) & 1u)) continue;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const uint32_t k = half * 8u + (uint32_t)c;
+        patch[k * P.PPITCH + p_dst[j]] = ((p_ok >> j) & 1u) && pre_ci + k < P.Cin ? ppre[j][c] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < WJ; ++j) {
+      const uint32_t f = tid + (uint32_t)j * kS2Threads;
+      const uint32_t co_l = f / kRowPieces, rr = (f - co_l * kRowPieces) * 4u;
+      const bool ok = pre_ci * 9u + rr < w_end && m0 + co_l < P.Cout;
+      *reinterpret_cast<s2_floatx4 *>(wl + co_l * kS2FwdWPitch + rr) = ok ? wpre[j] : s2_floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+
+  // ---- this lane's pixels: pixel l16 of each of its wave's two 16-pixel tiles
+  uint32_t q_off[2];
+#pragma unroll
+  for (int pt = 0; pt < 2; ++pt) {
+    const uint32_t q = wq * 32u + (uint32_t)pt * 16u + l16;
+    const uint32_t per = P.QR * P.QC;
+    const uint32_t b = q / per, q2 = q - b * per;
+    const uint32_t qi = q2 / P.QC, qj = q2 - qi * P.QC;
+    q_off[pt] = b * P.PPI + 2u * qi * P.PRW + qj + g * P.PPITCH;
+  }
+  const float *b_base = wl + (wm * 32u + l16) * kS2FwdWPitch + g * 9u;
+  // where tap column tb = 0, 1, 2 lies relative to the pixel's place in the even half of a patch row
+  const uint32_t tap_col[3] = {0u, even_cols, 1u};
+
+  s2_floatx4 acc[2][2];
+#pragma unroll
+  for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) acc[pt][ct] = s2_floatx4{0.f, 0.f, 0.f, 0.f};
+
+  load_chunk(0);
+  for (uint32_t ci0 = 0; ci0 < P.Cin; ci0 += kS2CC) {
+    __syncthreads();
+    store_chunk();
+    __syncthreads();
+    if (ci0 + kS2CC < P.Cin) load_chunk(ci0 + kS2CC);
+#pragma unroll
+    for (int kk = 0; kk < (int)kS2CC / 4; ++kk) {
+#pragma unroll
+      for (int ta = 0; ta < 3; ++ta)
+#pragma unroll
+        for (int tb = 0; tb < 3; ++tb) {
+          float a[2], b[2];
+#pragma unroll
+          for (int pt = 0; pt < 2; ++pt)
+            a[pt] = patch[(uint32_t)(4 * kk) * P.PPITCH + q_off[pt] + (uint32_t)ta * P.PRW + tap_col[tb]];
+#pragma unroll
+          for (int ct = 0; ct < 2; ++ct) b[ct] = b_base[ct * 16 * (int)kS2FwdWPitch + kk * 36 + ta * 3 + tb];
+#pragma unroll
+          for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+            for (int ct = 0; ct < 2; ++ct)
+              acc[pt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[pt], b[ct], acc[pt][ct], 0, 0, 0);
+        }
+    }
+  }
+
+  // ---- the lane holds pixels 4 g .. 4 g + 3 of each tile (one output row) for channel l16 of each channel tile
+  const size_t y_plane = (size_t)P.OH * P.OW;
+#pragma unroll
+  for (int pt = 0; pt < 2; ++pt) {
+    const uint32_t q = wq * 32u + (uint32_t)pt * 16u + 4u * g;
+    const uint32_t per = P.QR * P.QC;
+    const uint32_t b = q / per, q2 = q - b * per;
+    const uint32_t qi = q2 / P.QC, qj = q2 - qi * P.QC;
+    if (n0 + b >= P.N) continue;
+    float *o_px = P.y[tile] + (size_t)(n0 + b) * P.Cout * y_plane + (size_t)(i0 + qi) * P.OW + (j0 + qj);
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) {
+      const uint32_t m = m0 + wm * 32u + (uint32_t)ct * 16u + l16;
+      if (m >= P.Cout) continue;
+      float *o = o_px + (size_t)m * y_plane;
+      s2_floatx4 v = acc[pt][ct];
+      if (P.beta != 0.f) v += *reinterpret_cast<const s2_floatx4 *>(o);
+      *reinterpret_cast<s2_floatx4 *>(o) = v;
+    }
+  }
+}
+
+// the split of a tile's H/2 x W/2 output pixels into workgroups of 64: rows of 8 or 16 pixels
+static bool s2_quads(uint32_t OH, uint32_t OW, uint32_t *QR, uint32_t *QC, uint32_t *NBI) {
+  if (OW != 8u && OW % 16u != 0u) return false;
+  *QC = std::min(OW, 16u);
+  *QR = std::min(OH, kS2Quads / *QC);
+  while (*QR > 1u && OH % *QR != 0u) --*QR;
+  if ((kS2Quads / *QC) % *QR != 0u) return false;
+  *NBI = kS2Quads / (*QC * *QR);
+  return true;
+}
+
+// Forward of a 3x3 window at stride 2, padding 1, over fp32 tiles of H x W without halo (y tiles of H/2 x W/2).
+// ADH_EUNIMPL: not a shape this kernel serves; nothing launched.
+int conv3x3s2_fwd_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                      const void *const *x_tiles, const void *w, void *const *y_tiles, float beta, hipStream_t st) {
+  if (H % 2u != 0u || W % 2u != 0u || H == 0 || W == 0) return ADH_EUNIMPL;
+  const uint32_t OH = H / 2u, OW = W / 2u;
+  uint32_t QR, QC, NBI;
+  if (!s2_quads(OH, OW, &QR, &QC, &NBI)) return ADH_EUNIMPL;
+  // With few input channels a workgroup's set-up and its first chunk, which nothing overlaps, weigh more than
+  // what the kernel saves: 64 -> 128 on 32x128 tiles 0.23-0.24 ms against the general kernel's 0.22, 128 -> 256 on
+  // 16x64 0.215-0.225 against 0.205; 256 -> 512 on 8x32 0.21 against 0.36, 512 -> 512 on 4x16 0.13 against 0.27.
+  if (Cin < 256u) return ADH_EUNIMPL;
+  if (!aligned_to(w, 16) || Cin % 4u != 0u) return ADH_EUNIMPL;
+  for (uint32_t t = 0; t < num_tiles; ++t)
+    if (!aligned_to(y_tiles[t], 16) || !aligned_to(x_tiles[t], 4)) return ADH_EUNIMPL;
+  if ((uint64_t)Cin * Cout * 9u >= (1ull << 31) || (uint64_t)N * Cin * H * W >= (1ull << 31)) return ADH_EUNIMPL;
+
+  S2FwdParams P = {};
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    P.x[t] = reinterpret_cast<const float *>(x_tiles[t]);
+    P.y[t] = reinterpret_cast<float *>(y_tiles[t]);
+  }
+  P.w = reinterpret_cast<const float *>(w);
+  P.num_tiles = num_tiles; P.N = N; P.Cin = Cin; P.Cout = Cout;
+  P.OH = OH; P.OW = OW;
+  P.QR = QR; P.QC = QC; P.NBI = NBI;
+  P.PRW = 2u * QC + 1u;
+  P.PPI = (2u * QR + 1u) * P.PRW;
+  const uint32_t pp = NBI * P.PPI;
+  P.PPITCH = (pp + 63u) / 64u * 64u + 16u;
+  P.RB = OH / QR; P.CB = OW / QC; P.NG = (N + NBI - 1u) / NBI; P.MG = (Cout + kS2BM - 1u) / kS2BM;
+  P.beta = beta;
+  P.div_MG = FastDiv(P.MG); P.div_CB = FastDiv(P.CB); P.div_RB = FastDiv(P.RB); P.div_NG = FastDiv(P.NG);
+  P.div_PPI = FastDiv(P.PPI); P.div_PRW = FastDiv(P.PRW);
+  const uint64_t blocks = (uint64_t)num_tiles * P.NG * P.RB * P.CB * P.MG;
+  if (blocks == 0 || blocks >= (1ull << 31)) return ADH_EUNIMPL;
+  const size_t lds = (size_t)(kS2BM * kS2FwdWPitch + kS2CC * P.PPITCH) * sizeof(float);
+  if (lds > 64u * 1024u || pp > 3u * 128u) return ADH_EUNIMPL;
+  hipLaunchKernelGGL((conv3x3s2_fwd_kernel<3>), dim3((uint32_t)blocks), dim3(kS2Threads), lds, st, P);
   return launch_status();
 }
 

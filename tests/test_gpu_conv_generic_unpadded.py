@@ -33,6 +33,11 @@ CASES = [  # K, N, Cin, Cout, Ht, W, kh, kw, sh, sw, dh, dw, pad_h, pad_w
     (3, 2, 8, 40, 16, 64, 3, 3, 2, 2, 1, 1, 1, 1),    # 8x32 outputs: two row blocks and two column blocks per image
     (2, 3, 68, 16, 4, 32, 3, 3, 2, 2, 1, 1, 1, 1),    # 2x16 outputs: two images per workgroup, a second channel group of 4
     (1, 2, 4, 4, 16, 16, 3, 3, 2, 2, 1, 1, 1, 1),     # 8x8 outputs on a single tile: zeros below
+    # ... and with at least 256 input channels the forward takes its own kernel too
+    (2, 5, 256, 72, 4, 16, 3, 3, 2, 2, 1, 1, 1, 1),   # 2x8 outputs, four images per workgroup (then one), 64 + 8 output channels
+    (2, 2, 260, 16, 8, 32, 3, 3, 2, 2, 1, 1, 1, 1),   # 4x16 outputs, a last chunk of four input channels
+    (3, 1, 256, 8, 16, 64, 3, 3, 2, 2, 1, 1, 1, 1),   # 8x32 outputs over three tiles: row -1 from the tile above
+    (1, 1, 256, 8, 16, 16, 3, 3, 2, 2, 1, 1, 1, 1),   # 8x8 outputs on a single tile: zeros above
 ]
 
 
