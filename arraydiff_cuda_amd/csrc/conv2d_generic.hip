@@ -575,6 +575,15 @@ int conv3x3s2_bwd_data_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_
 int conv3x3s2_fwd_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
                       const void *const *x_tiles, const void *w, void *const *y_tiles, float beta, hipStream_t st);
 
+size_t conv3x3s2_wgrad_workspace(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W);
+int conv3x3s2_wgrad_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                        const void *const *x_tiles, const void *const *dy_tiles, float *dwt, float beta, void *workspace,
+                        hipStream_t st);
+static bool gen_is_3x3s2_unpadded(int dtype, const GenShape &g, bool unpadded, uint32_t pad_h, uint32_t pad_w) {
+  return dtype == ADH_F32 && unpadded && g.kh == 3u && g.kw == 3u && g.sh == 2u && g.sw == 2u && g.dh == 1u && g.dw == 1u &&
+         pad_h == 1u && pad_w == 1u;
+}
+
 // a window of one tap reads no neighbour and no padding: tiles with and without halo are the same thing
 static bool gen_is_pointwise(int dtype, const GenShape &g, bool unpadded, uint32_t pad_h, uint32_t pad_w) {
   return dtype == ADH_F32 && g.kh == 1u && g.kw == 1u && g.sh == g.sw && (!unpadded || (pad_h == 0u && pad_w == 0u));
@@ -1135,6 +1144,8 @@ size_t conv2d_workspace(int which, int dtype, uint32_t num_tiles, uint32_t N, ui
     size_t bytes = wp.partial_bytes;
     if (gen_is_pointwise_wgrad(dtype, g, unpadded, pad_h, pad_w))
       bytes = std::max(bytes, conv1x1_wgrad_workspace(num_tiles, N, Cin, Cout, g.OH, g.OW));
+    if (gen_is_3x3s2_unpadded(dtype, g, unpadded, pad_h, pad_w))
+      bytes = std::max(bytes, conv3x3s2_wgrad_workspace(num_tiles, N, Cin, Cout, g.HP - 2u, g.WP - 2u));
     return (bytes + 255u) & ~(size_t)255u;
   }
   GenPlan plan = {};
@@ -1267,6 +1278,14 @@ int conv2d_bwd_filter(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, u
       if (workspace_bytes < need) return ADH_EWORKSPACE;
       e = conv1x1_wgrad_try(num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, g.sh, g.sw, x_tiles, dy_tiles, dwt, beta,
                             workspace, st);
+      if (e != ADH_EUNIMPL) return e;
+    }
+  }
+  if (gen_is_3x3s2_unpadded(dtype, g, unpadded, pad_h, pad_w)) {
+    const size_t need = conv3x3s2_wgrad_workspace(num_tiles, N, Cin, Cout, g.HP - 2u, g.WP - 2u);
+    if (need != 0) {
+      if (workspace_bytes < need) return ADH_EWORKSPACE;
+      e = conv3x3s2_wgrad_try(num_tiles, N, Cin, Cout, g.HP - 2u, g.WP - 2u, x_tiles, dy_tiles, dwt, beta, workspace, st);
       if (e != ADH_EUNIMPL) return e;
     }
   }

@@ -502,4 +502,293 @@ int conv3x3s2_fwd_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cou
   return launch_status();
 }
 
+// ---------------------------------------------------------------------------------------------
+// backward-filter: dw[co][ci][a][b] = beta dw + sum over tiles, n, i, j of dy[n][co][i][j] * x[n][ci][2i+a-1][2j+b-1]
+// Per tap a matrix product whose reduction runs over the pixels.  A workgroup owns 64 output channels x 32 input
+// channels x 9 taps and a run of 32-pixel chunks (NBI images x QR rows x QC columns of dy); per chunk it stages the
+// dy pixels and the input patch (rows split into even and odd columns, as in the forward kernel), and each wave
+// multiplies four consecutive pixels of a row at a time: one dy operand serves all nine taps.  The sums go to
+// part[split][tap][co][ci]; a second kernel adds the splits in a fixed order and writes the filter's own layout.
+// ---------------------------------------------------------------------------------------------
+constexpr uint32_t kS2WgPx = 32;   // pixels per chunk
+constexpr uint32_t kS2WgCo = 64;   // output channels per workgroup
+constexpr uint32_t kS2WgCi = 32;   // input channels per workgroup
+constexpr uint32_t kS2WgYPitch = kS2WgPx + 4u;
+
+struct S2WgradParams {
+  const float *x[ADH_MAX_TILES];
+  const float *dy[ADH_MAX_TILES];
+  float *part;
+  uint32_t num_tiles, N, Cin, Cout;
+  uint32_t OH, OW;
+  uint32_t QR, QC, NBI;
+  uint32_t PRW, PPI, XP;     // patch row width, floats per image, per staged input channel (4 mod 64)
+  uint32_t RB, CB, NG;
+  uint32_t COB, CIB;         // blocks of output / input channels
+  uint32_t chunks, chunks_per_split;
+  FastDiv div_CIB, div_COB, div_CB, div_RB, div_NG, div_PPI, div_PRW;
+};
+
+__global__ __launch_bounds__(kS2Threads, 2) void conv3x3s2_wgrad_kernel(const S2WgradParams P) {
+  constexpr int NP = 3;  // patch places per lane (NBI * PPI <= 192), each for eight input channels
+  extern __shared__ __align__(16) float s2_lds[];
+  float *yl = s2_lds;                               // [kS2WgCo][kS2WgYPitch]
+  float *xl = s2_lds + kS2WgCo * kS2WgYPitch;       // [kS2WgCi][XP]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+  const uint32_t wo = wave & 1u, wi = wave >> 1;  // output-channel half (32), input-channel half (16)
+
+  uint32_t vb = blockIdx.x;
+  if ((gridDim.x & 7u) == 0u) vb = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  uint32_t r1, cib, cob, split;
+  P.div_CIB.divmod(vb, r1, cib);
+  P.div_COB.divmod(r1, split, cob);
+  const uint32_t co0 = cob * kS2WgCo, ci0 = cib * kS2WgCi;
+  const uint32_t c_lo = split * P.chunks_per_split, c_hi = min(P.chunks, c_lo + P.chunks_per_split);
+  const uint32_t H = 2u * P.OH, W = 2u * P.OW;
+  const uint32_t x_plane = H * W, y_plane = P.OH * P.OW;
+  const uint32_t pp = P.NBI * P.PPI;
+  const uint32_t even_cols = P.QC + 1u;
+
+  // ---- what a thread stages is the same for every chunk but for the chunk's place in the tensor
+  // dy: pixel tid % 32 of the chunk for output channels tid / 32 + 8 c
+  const uint32_t ypx = tid & (kS2WgPx - 1u), yco = tid >> 5;
+  uint32_t y_b, y_rel;
+  {
+    const uint32_t per = P.QR * P.QC;
+    y_b = ypx / per;
+    const uint32_t q2 = ypx - y_b * per, qi = q2 / P.QC, qj = q2 - qi * P.QC;
+    y_rel = y_b * P.Cout * y_plane + qi * P.OW + qj;
+  }
+  // x: patch places lane + 64 j for input channels 8 wave + c
+  uint32_t x_rel[NP], x_dst[NP], x_b[NP];
+  uint32_t x_has = 0, x_row0 = 0, x_col0 = 0;  // bit j: a place of the patch / in its first row / in its first column
+#pragma unroll
+  for (int j = 0; j < NP; ++j) {
+    const uint32_t e = lane + 64u * (uint32_t)j;
+    uint32_t b, e2, pr, pc;
+    P.div_PPI.divmod(e, b, e2);
+    P.div_PRW.divmod(e2, pr, pc);
+    x_b[j] = b;
+    x_rel[j] = b * P.Cin * x_plane + pr * W + pc;
+    x_dst[j] = b * P.PPI + pr * P.PRW + ((pc & 1u) ? even_cols + (pc >> 1) : (pc >> 1));
+    x_has |= e < pp ? 1u << j : 0u;
+    x_row0 |= pr == 0u ? 1u << j : 0u;
+    x_col0 |= pc == 0u ? 1u << j : 0u;
+  }
+
+  float ypre[8], xpre[NP][8];
+  uint32_t pre_y_ok = 0, pre_x_ok = 0;
+  auto load_chunk = [&](uint32_t c) {
+    uint32_t q1, q2, cb, rb, ng, tile;
+    P.div_CB.divmod(c, q1, cb);
+    P.div_RB.divmod(q1, q2, rb);
+    P.div_NG.divmod(q2, tile, ng);
+    const uint32_t n0 = ng * P.NBI, i0 = rb * P.QR, j0 = cb * P.QC;
+    const float *yb = P.dy[tile] + (size_t)n0 * P.Cout * y_plane + i0 * P.OW + j0;
+    pre_y_ok = n0 + y_b < P.N ? 1u : 0u;
+#pragma unroll
+    for (int cc = 0; cc < 8; ++cc) {
+      const uint32_t co = min(co0 + yco + 8u * (uint32_t)cc, P.Cout - 1u);
+      ypre[cc] = yb[pre_y_ok ? y_rel + co * y_plane : 0u];
+    }
+    // the patch starts one row above and one column left of the chunk's first input pixel
+    const float *x_own = P.x[tile];
+    const float *x_up = P.x[tile > 0u ? tile - 1u : tile];
+    const int32_t base = (int32_t)(n0 * P.Cin * x_plane) + ((int32_t)(2u * i0) - 1) * (int32_t)W + (int32_t)(2u * j0) - 1;
+    pre_x_ok = 0;
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+      const bool up = i0 == 0u && ((x_row0 >> j) & 1u);
+      const bool left = j0 == 0u && ((x_col0 >> j) & 1u);
+      const bool ok = ((x_has >> j) & 1u) && n0 + x_b[j] < P.N && !left && (!up || tile > 0u);
+      pre_x_ok |= ok ? 1u << j : 0u;
+      // row -1 of this tile is row H - 1 of the tile above; a place outside the tensor reads the tile's first element
+      const float *xb = ok && up ? x_up + x_plane : x_own;
+      const int32_t off = ok ? base + (int32_t)x_rel[j] : 0;
+#pragma unroll
+      for (int cc = 0; cc < 8; ++cc) {
+        const uint32_t ci = min(ci0 + 8u * wave + (uint32_t)cc, P.Cin - 1u);
+        xpre[j][cc] = xb[off + (ok ? (int32_t)(ci * x_plane) : 0)];
+      }
+    }
+  };
+  auto store_chunk = [&]() {
+#pragma unroll
+    for (int cc = 0; cc < 8; ++cc) {
+      const uint32_t cl = yco + 8u * (uint32_t)cc;
+      yl[cl * kS2WgYPitch + ypx] = pre_y_ok && co0 + cl < P.Cout ? ypre[cc] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+      if (!((x_has >> j) & 1u)) continue;
+#pragma unroll
+      for (int cc = 0; cc < 8; ++cc) {
+        const uint32_t cl = 8u * wave + (uint32_t)cc;
+        xl[cl * P.XP + x_dst[j]] = ((pre_x_ok >> j) & 1u) && ci0 + cl < P.Cin ? xpre[j][cc] : 0.f;
+      }
+    }
+  };
+
+  // ---- the eight groups of four consecutive pixels of a chunk: where the group's first pixel lies in the even half
+  // of its patch row (this lane reads pixel g of the group)
+  uint32_t goff[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const uint32_t p = 4u * (uint32_t)q, per = P.QR * P.QC;
+    const uint32_t b = p / per, q2 = p - b * per, qi = q2 / P.QC, qj = q2 - qi * P.QC;
+    goff[q] = b * P.PPI + 2u * qi * P.PRW + qj + g;
+  }
+  const float *a_base = yl + (wo * 32u + l16) * kS2WgYPitch + g;
+  const float *b_base = xl + (wi * 16u + l16) * P.XP;
+  const uint32_t tap_col[3] = {0u, even_cols, 1u};
+
+  s2_floatx4 acc[9][2];
+#pragma unroll
+  for (int t = 0; t < 9; ++t)
+#pragma unroll
+    for (int ot = 0; ot < 2; ++ot) acc[t][ot] = s2_floatx4{0.f, 0.f, 0.f, 0.f};
+
+  if (c_lo < c_hi) load_chunk(c_lo);
+  for (uint32_t c = c_lo; c < c_hi; ++c) {
+    __syncthreads();
+    store_chunk();
+    __syncthreads();
+    if (c + 1u < c_hi) load_chunk(c + 1u);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      float a[2];
+#pragma unroll
+      for (int ot = 0; ot < 2; ++ot) a[ot] = a_base[ot * 16 * (int)kS2WgYPitch + 4 * q];
+#pragma unroll
+      for (int ta = 0; ta < 3; ++ta)
+#pragma unroll
+        for (int tb = 0; tb < 3; ++tb) {
+          const float b = b_base[goff[q] + (uint32_t)ta * P.PRW + tap_col[tb]];
+#pragma unroll
+          for (int ot = 0; ot < 2; ++ot)
+            acc[ta * 3 + tb][ot] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[ot], b, acc[ta * 3 + tb][ot], 0, 0, 0);
+        }
+    }
+  }
+
+  // ---- the lane holds output channels 4 g .. 4 g + 3 of each tile for input channel l16, per tap
+  const uint32_t ci = ci0 + wi * 16u + l16;
+  const size_t taps_stride = (size_t)P.Cout * P.Cin;
+  float *part = P.part + (size_t)split * 9u * taps_stride;
+  if (ci < P.Cin) {
+#pragma unroll
+    for (int t = 0; t < 9; ++t)
+#pragma unroll
+      for (int ot = 0; ot < 2; ++ot)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const uint32_t co = co0 + wo * 32u + (uint32_t)ot * 16u + 4u * g + (uint32_t)k;
+          if (co < P.Cout) part[(size_t)t * taps_stride + (size_t)co * P.Cin + ci] = acc[t][ot][k];
+        }
+  }
+}
+
+// dw[pair][tap] = beta dw + sum over the splits of part[split][tap][pair]: a workgroup takes 64 (co, ci) pairs; its
+// four waves take every fourth split each, and the four sums are added in order (the same bits on every run)
+__global__ __launch_bounds__(256) void conv3x3s2_wgrad_reduce_kernel(const float *part, float *dw, uint32_t pairs,
+                                                                     uint32_t nsplit, float beta) {
+  __shared__ float sums[4][9][64];
+  const uint32_t l = threadIdx.x & 63u, sg = threadIdx.x >> 6;
+  const uint32_t pair = blockIdx.x * 64u + l;
+  float s[9];
+#pragma unroll
+  for (int t = 0; t < 9; ++t) s[t] = 0.f;
+  if (pair < pairs)
+    for (uint32_t sp = sg; sp < nsplit; sp += 4u)
+#pragma unroll
+      for (int t = 0; t < 9; ++t) s[t] += part[((size_t)sp * 9u + (uint32_t)t) * pairs + pair];
+#pragma unroll
+  for (int t = 0; t < 9; ++t) sums[sg][t][l] = s[t];
+  __syncthreads();
+  // the block's 64 x 9 results are consecutive in dw
+  for (uint32_t e = threadIdx.x; e < 576u; e += 256u) {
+    const uint32_t pl = e / 9u, t = e - pl * 9u;
+    if (blockIdx.x * 64u + pl >= pairs) continue;
+    const float total = ((sums[0][t][pl] + sums[1][t][pl]) + sums[2][t][pl]) + sums[3][t][pl];
+    const size_t o = (size_t)blockIdx.x * 576u + e;
+    dw[o] = beta != 0.f ? dw[o] + total : total;
+  }
+}
+
+struct S2WgradPlan {
+  uint32_t QR, QC, NBI, nsplit, chunks, chunks_per_split;
+  size_t part_bytes;
+};
+
+static bool s2_wgrad_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                          S2WgradPlan *plan) {
+  if (H % 2u != 0u || W % 2u != 0u || H == 0 || W == 0 || N == 0) return false;
+  const uint32_t OH = H / 2u, OW = W / 2u;
+  if (OW != 8u && OW % 16u != 0u) return false;
+  plan->QC = std::min(OW, 16u);
+  plan->QR = std::min(OH, kS2WgPx / plan->QC);
+  while (plan->QR > 1u && OH % plan->QR != 0u) --plan->QR;
+  if ((kS2WgPx / plan->QC) % plan->QR != 0u) return false;
+  plan->NBI = kS2WgPx / (plan->QC * plan->QR);
+  if (plan->NBI * (2u * plan->QR + 1u) * (2u * plan->QC + 1u) > 192u) return false;
+  if ((uint64_t)Cin * Cout * 9u >= (1ull << 31) || (uint64_t)N * Cin * H * W >= (1ull << 31)) return false;
+  const uint64_t chunks = (uint64_t)num_tiles * ((N + plan->NBI - 1u) / plan->NBI) * (OH / plan->QR) * (OW / plan->QC);
+  if (chunks == 0 || chunks >= (1ull << 31)) return false;
+  plan->chunks = (uint32_t)chunks;
+  const uint32_t out_tiles = ((Cout + kS2WgCo - 1u) / kS2WgCo) * ((Cin + kS2WgCi - 1u) / kS2WgCi);
+  // two workgroups per CU, and at least four chunks each: every split writes and re-reads a whole filter gradient
+  const uint32_t nsplit = std::max(1u, std::min(plan->chunks / 4u, (512u + out_tiles - 1u) / out_tiles));
+  plan->chunks_per_split = (plan->chunks + nsplit - 1u) / nsplit;
+  plan->nsplit = (plan->chunks + plan->chunks_per_split - 1u) / plan->chunks_per_split;
+  plan->part_bytes = (size_t)plan->nsplit * 9u * Cout * Cin * sizeof(float);
+  return true;
+}
+
+// the partial sums of conv3x3s2_wgrad_try (0: not a shape it serves)
+size_t conv3x3s2_wgrad_workspace(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W) {
+  S2WgradPlan plan;
+  if (!s2_wgrad_plan(num_tiles, N, Cin, Cout, H, W, &plan)) return 0;
+  return plan.part_bytes;
+}
+
+// Filter gradient of a 3x3 window at stride 2, padding 1, over fp32 tiles of H x W without halo.  `workspace` holds
+// conv3x3s2_wgrad_workspace bytes.  ADH_EUNIMPL: not a shape this kernel serves; nothing launched.
+int conv3x3s2_wgrad_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                        const void *const *x_tiles, const void *const *dy_tiles, float *dwt, float beta, void *workspace,
+                        hipStream_t st) {
+  S2WgradPlan plan;
+  if (!s2_wgrad_plan(num_tiles, N, Cin, Cout, H, W, &plan)) return ADH_EUNIMPL;
+  S2WgradParams P = {};
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!aligned_to(x_tiles[t], 4) || !aligned_to(dy_tiles[t], 4)) return ADH_EUNIMPL;
+    P.x[t] = reinterpret_cast<const float *>(x_tiles[t]);
+    P.dy[t] = reinterpret_cast<const float *>(dy_tiles[t]);
+  }
+  P.part = reinterpret_cast<float *>(workspace);
+  P.num_tiles = num_tiles; P.N = N; P.Cin = Cin; P.Cout = Cout;
+  P.OH = H / 2u; P.OW = W / 2u;
+  P.QR = plan.QR; P.QC = plan.QC; P.NBI = plan.NBI;
+  P.PRW = 2u * plan.QC + 1u;
+  P.PPI = (2u * plan.QR + 1u) * P.PRW;
+  const uint32_t pp = plan.NBI * P.PPI;
+  P.XP = (pp + 63u) / 64u * 64u + 4u;
+  P.RB = P.OH / plan.QR; P.CB = P.OW / plan.QC; P.NG = (N + plan.NBI - 1u) / plan.NBI;
+  P.COB = (Cout + kS2WgCo - 1u) / kS2WgCo; P.CIB = (Cin + kS2WgCi - 1u) / kS2WgCi;
+  P.chunks = plan.chunks; P.chunks_per_split = plan.chunks_per_split;
+  P.div_CIB = FastDiv(P.CIB); P.div_COB = FastDiv(P.COB); P.div_CB = FastDiv(P.CB); P.div_RB = FastDiv(P.RB);
+  P.div_NG = FastDiv(P.NG); P.div_PPI = FastDiv(P.PPI); P.div_PRW = FastDiv(P.PRW);
+  const uint64_t blocks = (uint64_t)plan.nsplit * P.COB * P.CIB;
+  if (blocks >= (1ull << 31)) return ADH_EUNIMPL;
+  const size_t lds = (size_t)(kS2WgCo * kS2WgYPitch + kS2WgCi * P.XP) * sizeof(float);
+  if (lds > 64u * 1024u) return ADH_EUNIMPL;
+  hipLaunchKernelGGL(conv3x3s2_wgrad_kernel, dim3((uint32_t)blocks), dim3(kS2Threads), lds, st, P);
+  int e = launch_status();
+  if (e) return e;
+  const uint32_t pairs = Cout * Cin;
+  hipLaunchKernelGGL(conv3x3s2_wgrad_reduce_kernel, dim3((pairs + 63u) / 64u), dim3(256), 0, st, P.part, dwt, pairs,
+                     plan.nsplit, beta);
+  return launch_status();
+}
+
 }  // namespace adh
