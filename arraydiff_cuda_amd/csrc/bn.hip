@@ -37,7 +37,7 @@ struct BnParams {
   float *o2[ADH_MAX_TILES];               // forward: saved mean
   float *o3[ADH_MAX_TILES];               // forward: saved 1/sqrt(var + eps)
   float *partial;                         // [tile][c][split][2]
-  uint32_t N, C, H, W, HW, p, split, n_per_split, tiles, groups_per_plane;
+  uint32_t N, C, H, W, HW, p, split, n_per_split, tiles, groups_per_plane, slots_log2;
   float eps, beta, beta_param;  // beta: input-gradient accumulation; beta_param: parameter-gradient accumulation
   int relu;
   FastDiv div_C, div_N, div_split, div_groups, div_cols;  // div_groups: the 16-byte groups of a plane; div_cols: row length of the index that a kernel splits into (row, column)
@@ -202,13 +202,17 @@ template <typename T, int MODE, int VEC>
 __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const BnParams P) {
   typedef BnVec<T, VEC> Vec;
   constexpr bool BWD = MODE == 2;
-  constexpr int U = 4;  // planes per workgroup: a thread moves the same group of each, all loads before the first store
-  __shared__ float cf_s[U][8];
+  constexpr int U = 4;  // planes per thread: a thread moves the same group of each, all loads before the first store
+  // A plane of at most 128 groups (the late layers' tiles) takes P.slots = 16 .. 128 threads, and the workgroup's
+  // 256 / P.slots parts take U planes each; a larger plane takes the whole workgroup, band by band (blockIdx.y).
+  __shared__ float cf_s[U * 16][8];
   const uint32_t WP = P.W + 2u * P.p, HPp = P.H + 2u * P.p;
   const uint32_t total = HPp * WP;
   const uint32_t planes = P.tiles * P.N * P.C;
-  if (threadIdx.x < (uint32_t)U) {
-    const uint32_t pl = blockIdx.x * U + threadIdx.x;
+  const uint32_t parts = kBnThreads >> P.slots_log2;
+  const uint32_t part = threadIdx.x >> P.slots_log2;
+  if (threadIdx.x < (uint32_t)U * parts) {
+    const uint32_t pl = blockIdx.x * U * parts + threadIdx.x;
     if (pl < planes) {
       uint32_t tn, c, tile, n;
       P.div_C.divmod(pl, tn, c);
@@ -217,7 +221,7 @@ __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const BnParams P) 
     }
   }
   __syncthreads();
-  const uint32_t gi = blockIdx.y * kBnThreads + threadIdx.x;  // group of VEC elements within a plane
+  const uint32_t gi = blockIdx.y * kBnThreads + (threadIdx.x & ((1u << P.slots_log2) - 1u));  // group of VEC elements within a plane
   if (gi >= P.groups_per_plane) return;
   // where the group sits is the same for every plane
   uint32_t r = 0, col = 0, in_off = 0, mask = 0;
@@ -250,13 +254,13 @@ __global__ __launch_bounds__(kBnThreads) void bn_apply_kernel(const BnParams P) 
   bool live[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    const uint32_t pl = blockIdx.x * U + u;
+    const uint32_t pl = (blockIdx.x * parts + part) * U + u;
     live[u] = pl < planes;
     if (!live[u]) continue;
     uint32_t tn, c, tile, n;
     P.div_C.divmod(pl, tn, c);
     P.div_N.divmod(tn, tile, n);
-    cf_u[u] = cf_s[u];
+    cf_u[u] = cf_s[part * U + u];
     const T *x = reinterpret_cast<const T *>(P.x[tile]) + ((size_t)n * P.C + c) * P.HW;
     if (!BWD) {
       out_u[u] = reinterpret_cast<T *>(P.out[tile]) + ((size_t)n * P.C + c) * total;
@@ -385,8 +389,15 @@ static int bn_common(int dtype, uint32_t num_tiles, uint32_t N, uint32_t C, uint
 static dim3 bn_apply_grid(BnParams *P, uint32_t groups_per_plane) {
   P->groups_per_plane = groups_per_plane;
   P->div_N = FastDiv(P->N);
+  // threads per plane: the whole workgroup, or for planes of at most 128 groups the power of two that holds them
+  P->slots_log2 = 8;
+  if (groups_per_plane <= kBnThreads / 2u) {
+    P->slots_log2 = 4;
+    while ((1u << P->slots_log2) < groups_per_plane) ++P->slots_log2;
+  }
   const uint64_t planes = (uint64_t)P->tiles * P->N * P->C;
-  return dim3((uint32_t)((planes + 3u) / 4u), (groups_per_plane + kBnThreads - 1u) / kBnThreads);
+  const uint64_t per_block = 4u * (kBnThreads >> P->slots_log2);
+  return dim3((uint32_t)((planes + per_block - 1u) / per_block), (groups_per_plane + kBnThreads - 1u) / kBnThreads);
 }
 
 }  // namespace adh
