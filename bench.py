@@ -445,6 +445,16 @@ def main():
                                                             ws5.data_ptr(), ws5_bytes, stream),
             "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
         del gu
+        # the clock under this kernel is set by power and the power by the data: the same launch on rectified
+        # activations (what a BN -> ReLU -> conv block feeds its convolution: half the values are zero)
+        xr = [t.clamp_min(0) for t in xu]
+        xr_tbl, _ku4 = capi.ptr_table([t.data_ptr() for t in xr])
+        add("conv fwd cfg5 over tiles without halo on rectified activations (bf16; the same launch, max(x, 0) as input)",
+            lambda: lib.adh_conv3x3_unpadded_fwd_tiles(1, K5, N5, C, C, Ht5, W5, xr_tbl, w5.data_ptr(), yu_tbl, 0.0,
+                                                       ws5.data_ptr(), ws5_bytes, stream),
+            "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s",
+            note="not the headline's data: shows how much of the distance to the peak is the clock the device picks for the data")
+        del xr
         add("conv bwd-filter cfg5 over tiles without halo (bf16 in, fp32 filter gradient, two kernels)",
             lambda: lib.adh_conv3x3_unpadded_bwd_filter_tiles(1, K5, N5, C, C, Ht5, W5, xu_tbl, y5_tbl, gw5.data_ptr(), 0.0,
                                                               ws5.data_ptr(), ws5_bytes, stream),
@@ -595,9 +605,10 @@ def main():
         del xq, yq, dq, gq, xqu, gqu
         # the 3x3 kernels and the general kernels over tiles without halo, at the shapes of the spatially-parallel
         # ResNet-18 (batch 32, 4 row tiles): a 64-channel 3x3 on 32x128 tiles, the stride-2 3x3 64 -> 128 on the same
-        # tiles, and a 512-channel 3x3 on 4x16 tiles (the general kernels; padded tiles of 6x18 hold 1.7 times the pixels)
+        # tiles and 256 -> 512 on 8x32 tiles (kernels of their own for backward-data, backward-filter and, from 256 input
+        # channels on, forward), and a 512-channel 3x3 on 4x16 tiles (the general kernels; padded tiles of 6x18 hold 1.7 times the pixels)
         for (nm, Ci, Co, Hu, Wu, su) in (("3x3 64->64 on 32x128 tiles", 64, 64, 32, 128, 1), ("3x3 stride 2 64->128 on 32x128 tiles", 64, 128, 32, 128, 2),
-                                         ("3x3 512->512 on 4x16 tiles", 512, 512, 4, 16, 1)):
+                                         ("3x3 stride 2 256->512 on 8x32 tiles", 256, 512, 8, 32, 2), ("3x3 512->512 on 4x16 tiles", 512, 512, 4, 16, 1)):
             OHu, OWu = Hu // su, (Wu + 2 - 3) // su + 1
             xu = [torch.randn((N, Ci, Hu, Wu), device="cuda", generator=g) for _ in range(K)]
             yu = [torch.randn((N, Co, OHu, OWu), device="cuda", generator=g) for _ in range(K)]
