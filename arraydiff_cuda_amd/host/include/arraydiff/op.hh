@@ -130,7 +130,17 @@ public:
       : shape_(shape), offset_(offset), stride_(stride), batch_shape_(batch_shape), buf_(make_shared<Buf>()) {}
 
   TxnVar clone() const { return *this; }  // shares the buffer
-  VarId var() const { return buf_->var; }
+  VarId var() const { return buf().var; }
+  // Not in the reference.  From now on this variable (and every copy of it that a node already holds) IS `target`:
+  // one buffer, one transaction state.  Both must have one layout.
+  void forward_to(TxnVar &target) {
+    if (target.shape_ != shape_ || target.offset_ != offset_ || target.stride_ != stride_ || target.batch_shape_ != batch_shape_)
+      throw std::invalid_argument("TxnVar::forward_to: the two variables must have one layout");
+    shared_ptr<Buf> mine = root(), theirs = target.root();
+    if (mine == theirs) return;
+    if (mine->buffer) throw HazardError("TxnVar::forward_to after the buffer was allocated");
+    mine->forward = theirs;
+  }
   VShape shape() const { return shape_; }
   VShape offset() const { return offset_; }
   VShape stride() const { return stride_; }
@@ -140,7 +150,7 @@ public:
   // and must produce the value; false: another node already produced it.
   bool overwrite(TxnId txn, NodeId node, Ctx *ctx) {
     begin(txn, ctx);
-    Buf &b = *buf_;
+    Buf &b = buf();
     if (b.readers.count(node.raw_id())) throw HazardError("overwrite after read by the same node");
     if (!b.writers.empty() && !b.writers.count(node.raw_id())) return false;
     b.writers.insert(node.raw_id());
@@ -151,7 +161,7 @@ public:
   // return value says whether THIS node still has to add its contribution.
   bool accumulate(TxnId txn, NodeId node, Ctx *ctx, function<void(V *)> init_fn) {
     const bool fresh = begin(txn, ctx);
-    Buf &b = *buf_;
+    Buf &b = buf();
     if (fresh) init_fn(b.buffer.get());
     if (b.writers.count(node.raw_id())) return false;
     b.writers.insert(node.raw_id());
@@ -161,10 +171,10 @@ public:
   // Not in the reference.  True while the buffer is known to hold nothing but zeros: it was allocated (cleared) or
   // a writer declared it so, and no write access has been handed out since.  A node that would clear the buffer
   // again can skip the fill.
-  bool known_zero() const { return buf_->buffer && buf_->all_zero; }
+  bool known_zero() const { return buf().buffer && buf().all_zero; }
   // a writer of this transaction states that the buffer holds only zeros now
   void declare_zero(TxnId txn, NodeId node) {
-    Buf &b = *buf_;
+    Buf &b = buf();
     if (!b.buffer || !b.has_txn || !(b.txn == txn.raw_id()) || !b.writers.count(node.raw_id()))
       throw HazardError("declare_zero by a node that is not a writer of this transaction");
     b.all_zero = true;
@@ -172,12 +182,12 @@ public:
   // Marks the value to be carried into `txn` by the first read there (op.hh:236-247); a write in
   // the new transaction replaces it as usual.
   void rollover(TxnId txn) {
-    Buf &b = *buf_;
+    Buf &b = buf();
     if (!(b.has_txn && b.txn == txn.raw_id())) b.rollover = true;
   }
   // Read access: the value must have been written in this transaction, or carried into it.
   V &get(TxnId txn, NodeId node) {
-    Buf &b = *buf_;
+    Buf &b = buf();
     if (b.buffer && b.rollover && !(b.has_txn && b.txn == txn.raw_id())) {
       b.has_txn = true;
       b.txn = txn.raw_id();
@@ -190,7 +200,7 @@ public:
     return *b.buffer;
   }
   V &get_mut(TxnId txn, NodeId node) {
-    Buf &b = *buf_;
+    Buf &b = buf();
     if (!b.buffer || !b.has_txn || !(b.txn == txn.raw_id()) || !b.writers.count(node.raw_id()))
       throw HazardError("get_mut by a node that is not a writer of this transaction");
     b.all_zero = false;
@@ -198,10 +208,10 @@ public:
   }
   V &get_excl(TxnId txn, NodeId node) {
     V &v = get_mut(txn, node);
-    if (buf_->writers.size() != 1) throw HazardError("get_excl with more than one writer");
+    if (buf().writers.size() != 1) throw HazardError("get_excl with more than one writer");
     return v;
   }
-  bool written(TxnId txn) const { return buf_->has_txn && buf_->txn == txn.raw_id() && !buf_->writers.empty(); }
+  bool written(TxnId txn) const { return buf().has_txn && buf().txn == txn.raw_id() && !buf().writers.empty(); }
 
 private:
   struct Buf {
@@ -210,9 +220,20 @@ private:
     uint64_t txn = 0;
     std::set<uint64_t> writers, readers;
     std::unique_ptr<V> buffer;
+    shared_ptr<Buf> forward;  // set: this variable is that one (forward_to)
   };
+  shared_ptr<Buf> root() const {
+    shared_ptr<Buf> b = buf_;
+    while (b->forward) b = b->forward;
+    return b;
+  }
+  Buf &buf() const {
+    Buf *b = buf_.get();
+    while (b->forward) b = b->forward.get();
+    return *b;
+  }
   bool begin(TxnId txn, Ctx *ctx) {
-    Buf &b = *buf_;
+    Buf &b = buf();
     if (b.has_txn && b.txn == txn.raw_id()) return false;
     b.has_txn = true;
     b.txn = txn.raw_id();
@@ -224,10 +245,10 @@ private:
   }
   void allocate(Ctx *ctx) {
     if constexpr (IsBatchArray<V>::value)
-      buf_->buffer.reset(new V(V::ZerosPadded(shape_, offset_, stride_, batch_shape_, ctx)));
+      buf().buffer.reset(new V(V::ZerosPadded(shape_, offset_, stride_, batch_shape_, ctx)));
     else
-      buf_->buffer.reset(new V(V::Zeros(shape_, ctx)));
-    buf_->all_zero = true;
+      buf().buffer.reset(new V(V::Zeros(shape_, ctx)));
+    buf().all_zero = true;
   }
   VShape shape_, offset_, stride_;
   size_t batch_shape_ = 0;
@@ -251,6 +272,9 @@ public:
       throw std::invalid_argument("VarData::alias_grad: the two variables must have one layout");
     grad_ = other.grad_;
   }
+  // Not in the reference.  `other`'s gradient, in every copy of `other` that a node already holds, becomes this
+  // variable's gradient buffer.
+  void absorb_grad(VarData &other) { other.grad_.forward_to(grad_); }
   TxnVar<V> &val() { return val_; }
   TxnVar<V> &grad() { return grad_; }
   VShape shape() const { return val_.shape(); }
@@ -1290,20 +1314,27 @@ public:
   // of such an input is the output's gradient and nothing else, so the output's gradient variable takes the
   // input's buffer and the backward pass copies nothing for it.  (An input that another node also consumes must not
   // be named: that node's contribution would land in the output's gradient and reach the other inputs.)
+  // trunk_input (not in the reference): the index of an input that other nodes consume too, all of which lie
+  // UPSTREAM of the join's remaining inputs (the block input of a residual block: its other consumer is the first
+  // node of the path that ends in the join's second input), or -1.  Its gradient is the output's gradient plus what
+  // those nodes add - and they run their backward pass after every node that reads the output's gradient, and add
+  // in place.  So this input's gradient too can be the output's buffer: the gradient of a whole chain of residual
+  // blocks is then one buffer that each block's first node adds to, and the sum's backward pass copies nothing.
   static shared_ptr<Var<V>> Make(Join join, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx,
-                                 int sole_consumer_of = -1) {
-    return make_shared<JoinOp<V, Join>>(join, false, inputs, ctx, sole_consumer_of);
+                                 int sole_consumer_of = -1, int trunk_input = -1) {
+    return make_shared<JoinOp<V, Join>>(join, false, inputs, ctx, sole_consumer_of, trunk_input);
   }
   // inputs.at(j).at(rank)
   static vector<shared_ptr<Var<V>>> MakeParallel(Join join, vector<vector<shared_ptr<Var<V>>>> inputs,
-                                                 shared_ptr<Context> ctx, int sole_consumer_of = -1) {
+                                                 shared_ptr<Context> ctx, int sole_consumer_of = -1, int trunk_input = -1) {
     return make_per_rank<V>(ctx, [&](size_t r, shared_ptr<Context> dc) {
       vector<shared_ptr<Var<V>>> dev_inputs;
       for (auto &in : inputs) dev_inputs.push_back(in.at(r));
-      return Make(join, dev_inputs, dc, sole_consumer_of);
+      return Make(join, dev_inputs, dc, sole_consumer_of, trunk_input);
     });
   }
-  JoinOp(Join, bool in_place, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx, int sole_consumer_of = -1)
+  JoinOp(Join, bool in_place, vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx, int sole_consumer_of = -1,
+         int trunk_input = -1)
       : ctx_(ctx), inputs_(inputs) {
     if (in_place) throw std::invalid_argument("JoinOp: the in-place form is not part of this path");
     if (inputs.empty() || inputs.size() > ADH_MAX_TILES) throw std::invalid_argument("JoinOp: 1..16 inputs");
@@ -1318,6 +1349,12 @@ public:
       if ((size_t)sole_consumer_of >= inputs.size()) throw std::invalid_argument("JoinOp: no such input");
       y_.alias_grad(xs_[(size_t)sole_consumer_of]);
       grad_shared_[(size_t)sole_consumer_of] = true;
+    }
+    if (trunk_input >= 0) {
+      if ((size_t)trunk_input >= inputs.size() || trunk_input == sole_consumer_of) throw std::invalid_argument("JoinOp: no such input");
+      // the nodes that hold copies of this input must see the shared buffer too: its variable forwards to the output's
+      y_.absorb_grad(xs_[(size_t)trunk_input]);
+      grad_shared_[(size_t)trunk_input] = true;
     }
   }
   virtual void _push(EpochId e, function<void(Op *)> apply) {
@@ -1349,8 +1386,8 @@ shared_ptr<Var<V>> sum(vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ct
 }
 template <typename V>
 vector<shared_ptr<Var<V>>> parallel_sum(vector<vector<shared_ptr<Var<V>>>> inputs, shared_ptr<Context> ctx,
-                                        int sole_consumer_of = -1) {
-  return JoinOp<V, SumJoin>::MakeParallel(SumJoin(), inputs, ctx, sole_consumer_of);
+                                        int sole_consumer_of = -1, int trunk_input = -1) {
+  return JoinOp<V, SumJoin>::MakeParallel(SumJoin(), inputs, ctx, sole_consumer_of, trunk_input);
 }
 
 // ---------------------------------------------------------------------------

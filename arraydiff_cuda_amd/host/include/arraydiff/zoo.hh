@@ -177,7 +177,9 @@ ParallelBatchNormParamOp<V> spatial_parallel_residual_v2_conv2d(Conv2DShape shap
   auto conv1 = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, inputs, ctx);
   auto conv2 = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, conv1, ctx);
   vector<vector<shared_ptr<Var<V>>>> join_inputs{inputs, conv2};
-  block.ops = parallel_sum<V>(join_inputs, ctx, 1);  // conv2 feeds the sum only: its gradient is the sum's, one buffer
+  // conv2 feeds the sum only, and the block input's other consumer (the first batch norm) lies upstream of conv2:
+  // both gradients are the sum's output gradient, one buffer that the batch norm's backward pass adds to in place
+  block.ops = parallel_sum<V>(join_inputs, ctx, 1, 0);
   return block;
 }
 
@@ -209,7 +211,7 @@ ParallelBatchNormParamOp<V> spatial_parallel_proj_residual_v2_conv2d(Conv2DShape
                    : detail::exchanged_conv3x3(block, shape, stride, HaloPad2DOp<V>::MakeParallel(1, relu0, ctx), ctx);
   auto conv2 = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, conv1, ctx);
   vector<vector<shared_ptr<Var<V>>>> join_inputs{proj.ops, conv2};
-  block.ops = parallel_sum<V>(join_inputs, ctx, 1);  // conv2 feeds the sum only: its gradient is the sum's, one buffer
+  block.ops = parallel_sum<V>(join_inputs, ctx, 1, 0);  // both convs feed the sum only: their gradients are the sum's, one buffer
   return block;
 }
 

@@ -255,8 +255,8 @@ static void put_tile(std::vector<float> &full, const std::vector<float> &t, size
 // HaloExch -> conv -> (+ x).  Every rank's batch norm uses its own tile's statistics.  Oracle: the
 // same chain with per-tile batch norms and UNSPLIT convolutions.
 // fused: batch norm + rectifier + halo pad as one node (SlabBatchNorm2DOp with relu and out_halo) instead of three
-// shared_grad: the sum's output gradient and the second conv's output gradient are one buffer (JoinOp's
-// sole_consumer_of): the backward pass copies dy once instead of twice
+// shared_grad: the sum's output gradient, the second conv's output gradient (JoinOp's sole_consumer_of) and the block
+// input's gradient (trunk_input: the first batch norm adds to it in place) are one buffer: the sum's backward pass copies nothing
 static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, size_t W, bool fused = false,
                                         bool shared_grad = false) {
   std::mt19937 gen(31337 + (unsigned)K);
@@ -290,7 +290,7 @@ static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, 
   auto exch2 = HaloExch2DOp<V>::MakeParallel(1, pad2, ctx);
   auto conv2 = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch2, vector<shared_ptr<Var<A>>>(K, w2_src), ctx);
   vector<vector<shared_ptr<Var<V>>>> join_inputs{inputs, conv2};
-  auto join = parallel_sum<V>(join_inputs, ctx, shared_grad ? 1 : -1);
+  auto join = parallel_sum<V>(join_inputs, ctx, shared_grad ? 1 : -1, shared_grad ? 0 : -1);
   auto y_full = SpatialJoinedGather2DOp<V>::Make(join, ctx);
   auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
   sink->set_host_grad(dY.data());
