@@ -323,6 +323,74 @@ def test_general_conv_over_tiles_without_halo_random(oracle, K, Ht, W, kh, kw, s
         assert rel_err(host(gs[r]), g_want[:, :, r * Ht:(r + 1) * Ht, :]) <= 1e-5
 
 
+def _own_kernel_cases(seed, count):
+    """(K, N, Cin, Cout, Ht, W, k, s, pad) that the 1x1 kernels (output rows of a multiple of 4 pixels, tile sides a
+    multiple of the stride) and the stride-2 3x3 kernels (output rows of 8 or a multiple of 16 pixels, input channels a
+    multiple of 4; the forward one from 256 input channels on) take instead of the general kernel."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        k = int(rng.choice([1, 3]))
+        if k == 1:
+            s = int(rng.integers(1, 3))
+            OW, OH = 4 * int(rng.integers(1, 9)), int(rng.integers(1, 7))
+            Cin, Cout = int(rng.integers(1, 150)), int(rng.integers(1, 150))
+        else:
+            s = 2
+            OW, OH = int(rng.choice([8, 16, 32, 48])), int(rng.choice([1, 2, 3, 4, 6, 8]))
+            Cin = 4 * int(rng.integers(1, 20)) if rng.integers(0, 3) else 256 + 4 * int(rng.integers(0, 5))
+            Cout = int(rng.integers(1, 90 if Cin < 256 else 20))
+        K, N = int(rng.integers(1, 5)), int(rng.integers(1, 7))
+        if K * N * Cin * Cout * k * k * OH * OW > 6e7:  # keeps the scalar oracle to a second or two
+            continue
+        out.append((K, N, Cin, Cout, s * OH, s * OW, k, s, k // 2))
+    return out
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,Ht,W,k,s,pad", _own_kernel_cases(2033, 40))
+def test_pointwise_and_strided_3x3_kernels_random(oracle, K, N, Cin, Cout, Ht, W, k, s, pad):
+    """The three passes (backward-data with beta 0 and 1, the filter gradient with beta 0 and 1) of the shapes that have
+    kernels of their own behind adh_conv2d_unpadded_*_tiles, against the oracle's convolution of the unsplit
+    zero-padded tensor (fp32, rel-err <= 1e-5)."""
+    rng = np.random.default_rng(Cin * 131 + Cout * 7 + W)
+    geo = (k, k, s, s, 1, 1)
+    H, OHt, OW = K * Ht, Ht // s, W // s
+    x = rng.uniform(-1, 1, size=(N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, k, k)) * np.sqrt(2.0 / (Cin * k * k))).astype(np.float32)
+    dy = rng.standard_normal((N, Cout, K * OHt, OW)).astype(np.float32)
+    g0 = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    gw0 = rng.standard_normal(w.shape).astype(np.float32)
+    xp = np.zeros((N, Cin, H + 2 * pad, W + 2 * pad), np.float32)
+    xp[:, :, pad:pad + H, pad:pad + W] = x
+    y_want = np.empty(dy.shape, np.float32)
+    oracle.conv2d_slab_fwd(xp, w, s, s, 1, 1, y_want)
+    gp = np.empty(xp.shape, np.float32)
+    oracle.conv2d_slab_bwd_data(w, dy, s, s, 1, 1, gp)
+    g_want = gp[:, :, pad:pad + H, pad:pad + W]
+    gw_want = np.zeros(w.shape, np.float32)
+    oracle.conv2d_slab_bwd_filter(xp, dy, s, s, 1, 1, gw_want)
+    xs = [dev(x[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    dys = [dev(dy[:, :, r * OHt:(r + 1) * OHt, :].copy()) for r in range(K)]
+    d_w = dev(w)
+    ws = torch.empty(max(capi.conv2d_unpadded_workspace_bytes(wh, capi.ADH_F32, K, N, Cin, Cout, Ht, W, *geo, pad, pad)
+                         for wh in (0, 1, 2)) // 4, device="cuda")
+    ys = [torch.full((N, Cout, OHt, OW), float("nan"), device="cuda") for _ in range(K)]
+    gs = [torch.full((N, Cin, Ht, W), float("nan"), device="cuda") for _ in range(K)]
+    ga = [dev(g0[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    gw, gwa = torch.full(w.shape, float("nan"), device="cuda"), dev(gw0)
+    capi.check(capi.conv2d_unpadded_fwd_tiles(xs, d_w, ys, N, Cin, Cout, Ht, W, *geo, pad, pad, ws=ws), "fwd")
+    capi.check(capi.conv2d_unpadded_bwd_data_tiles(d_w, dys, gs, N, Cin, Cout, Ht, W, *geo, pad, pad, ws=ws), "bwd-data")
+    capi.check(capi.conv2d_unpadded_bwd_data_tiles(d_w, dys, ga, N, Cin, Cout, Ht, W, *geo, pad, pad, beta=1.0, ws=ws), "bwd-data +")
+    capi.check(capi.conv2d_unpadded_bwd_filter_tiles(xs, dys, gw, N, Cin, Cout, Ht, W, *geo, pad, pad, ws=ws), "bwd-filter")
+    capi.check(capi.conv2d_unpadded_bwd_filter_tiles(xs, dys, gwa, N, Cin, Cout, Ht, W, *geo, pad, pad, beta=1.0, ws=ws), "bwd-filter +")
+    assert rel_err(host(gw), gw_want) <= 1e-5
+    assert rel_err(host(gwa), gw0 + gw_want) <= 1e-5
+    for r in range(K):
+        assert rel_err(host(ys[r]), y_want[:, :, r * OHt:(r + 1) * OHt, :]) <= 1e-5
+        assert rel_err(host(gs[r]), g_want[:, :, r * Ht:(r + 1) * Ht, :]) <= 1e-5
+        assert rel_err(host(ga[r]), (g0 + g_want)[:, :, r * Ht:(r + 1) * Ht, :]) <= 1e-5
+
+
 @pytest.mark.parametrize("K,Ht,W,wh,ww,sh,sw,dh,dw,pad_h,pad_w", _unpadded_geometries(2031, 24, 4))
 def test_pool_over_tiles_without_halo_random(oracle, K, Ht, W, wh, ww, sh, sw, dh, dw, pad_h, pad_w):
     """adh_pool2d_unpadded_*_tiles against the oracle's pooling of the unsplit zero-padded tensor (windows without
