@@ -584,6 +584,11 @@ static bool gen_is_3x3s2_unpadded(int dtype, const GenShape &g, bool unpadded, u
          pad_h == 1u && pad_w == 1u;
 }
 
+// conv_thin.hip: forward over halo-padded fp32 tiles for at most three input channels (a network's stem)
+int conv_thin_fwd_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t OH,
+                      uint32_t OW, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, const void *const *x_tiles,
+                      const void *w, void *const *y_tiles, float beta, hipStream_t st);
+
 // a window of one tap reads no neighbour and no padding: tiles with and without halo are the same thing
 static bool gen_is_pointwise(int dtype, const GenShape &g, bool unpadded, uint32_t pad_h, uint32_t pad_w) {
   return dtype == ADH_F32 && g.kh == 1u && g.kw == 1u && g.sh == g.sw && (!unpadded || (pad_h == 0u && pad_w == 0u));
@@ -1187,6 +1192,13 @@ int conv2d_fwd(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t
     e = gen_check_workspace(plan, workspace, workspace_bytes);  // not used, but the contract is one for all shapes
     if (e) return e;
     e = conv1x1_try(false, num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, g.sh, x_tiles, w, y_tiles, beta, as_stream(stream));
+    if (e != ADH_EUNIMPL) return e;
+  }
+  if (dtype == ADH_F32 && !unpadded && dh == 1u && dw == 1u && Cin <= 3u && (kh > 1u || kw > 1u)) {
+    e = gen_check_workspace(plan, workspace, workspace_bytes);
+    if (e) return e;
+    e = conv_thin_fwd_try(num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, kh, kw, sh, sw, x_tiles, w, y_tiles, beta,
+                          as_stream(stream));
     if (e != ADH_EUNIMPL) return e;
   }
   if (dtype == ADH_F32 && unpadded && kh == 3u && kw == 3u && sh == 2u && sw == 2u && dh == 1u && dw == 1u && pad_h == 1u &&

@@ -39,6 +39,10 @@ CASES = [  # K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw
     (4, 16, 16, 130, 64, 64, 1, 1, 2, 2, 1, 1),  # 128 x 128 blocks forward (the last channel block holds 2), 128 x 64 backward
     (4, 16, 72, 24, 32, 64, 1, 1, 1, 1, 1, 1),   # stride 1: 128 x 64 blocks forward, 128 x 128 backward
     (3, 2, 5, 3, 2, 4, 1, 1, 2, 2, 1, 1),        # a single row of four pixels per image: most of the block is idle
+    # at most three input channels: the forward pass flattens (channel, tap) pairs and stages the whole filter once
+    (1, 2, 3, 64, 22, 70, 7, 7, 1, 1, 1, 1),     # the stem on 16x64 outputs: two row blocks and two column blocks, 16-byte stores
+    (3, 2, 3, 70, 14, 45, 7, 7, 1, 1, 1, 1),     # 39 output columns (stores element by element), 64 + 6 output channels
+    (2, 3, 1, 20, 19, 71, 3, 3, 2, 2, 1, 1),     # one input channel, stride 2
 ]
 
 
