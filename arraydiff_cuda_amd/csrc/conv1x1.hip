@@ -414,6 +414,13 @@ __global__ __launch_bounds__(256) void conv1x1_wgrad_reduce_kernel(const float *
   }
 }
 
+// dw[e] = beta dw[e] + the sum over the splits of part[split][e], for any kernel whose partial sums have the
+// filter gradient's own layout
+int split_sum_launch(const float *part, float *dw, uint32_t elems, uint32_t nsplit, float beta, hipStream_t st) {
+  hipLaunchKernelGGL(conv1x1_wgrad_reduce_kernel, dim3((elems + 63u) / 64u), dim3(256), 0, st, part, dw, elems, nsplit, beta);
+  return launch_status();
+}
+
 struct PwWgradPlan {
   uint32_t ot, it, nsplit, chunks_per_split;
   size_t part_bytes;

@@ -589,6 +589,15 @@ int conv_thin_fwd_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cou
                       uint32_t OW, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, const void *const *x_tiles,
                       const void *w, void *const *y_tiles, float beta, hipStream_t st);
 
+size_t conv_thin_wgrad_workspace(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP,
+                                 uint32_t OH, uint32_t OW, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw);
+int conv_thin_wgrad_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t OH,
+                        uint32_t OW, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, const void *const *x_tiles,
+                        const void *const *dy_tiles, float *dwt, float beta, void *workspace, hipStream_t st);
+static bool gen_is_thin(int dtype, const GenShape &g, bool unpadded) {
+  return dtype == ADH_F32 && !unpadded && g.dh == 1u && g.dw == 1u && g.Cin <= 3u && (g.kh > 1u || g.kw > 1u);
+}
+
 // a window of one tap reads no neighbour and no padding: tiles with and without halo are the same thing
 static bool gen_is_pointwise(int dtype, const GenShape &g, bool unpadded, uint32_t pad_h, uint32_t pad_w) {
   return dtype == ADH_F32 && g.kh == 1u && g.kw == 1u && g.sh == g.sw && (!unpadded || (pad_h == 0u && pad_w == 0u));
@@ -1151,6 +1160,8 @@ size_t conv2d_workspace(int which, int dtype, uint32_t num_tiles, uint32_t N, ui
       bytes = std::max(bytes, conv1x1_wgrad_workspace(num_tiles, N, Cin, Cout, g.OH, g.OW));
     if (gen_is_3x3s2_unpadded(dtype, g, unpadded, pad_h, pad_w))
       bytes = std::max(bytes, conv3x3s2_wgrad_workspace(num_tiles, N, Cin, Cout, g.HP - 2u, g.WP - 2u));
+    if (gen_is_thin(dtype, g, unpadded))
+      bytes = std::max(bytes, conv_thin_wgrad_workspace(num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, kh, kw, sh, sw));
     return (bytes + 255u) & ~(size_t)255u;
   }
   GenPlan plan = {};
@@ -1194,7 +1205,7 @@ int conv2d_fwd(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t
     e = conv1x1_try(false, num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, g.sh, x_tiles, w, y_tiles, beta, as_stream(stream));
     if (e != ADH_EUNIMPL) return e;
   }
-  if (dtype == ADH_F32 && !unpadded && dh == 1u && dw == 1u && Cin <= 3u && (kh > 1u || kw > 1u)) {
+  if (gen_is_thin(dtype, g, unpadded)) {
     e = gen_check_workspace(plan, workspace, workspace_bytes);
     if (e) return e;
     e = conv_thin_fwd_try(num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, kh, kw, sh, sw, x_tiles, w, y_tiles, beta,
@@ -1290,6 +1301,15 @@ int conv2d_bwd_filter(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, u
       if (workspace_bytes < need) return ADH_EWORKSPACE;
       e = conv1x1_wgrad_try(num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, g.sh, g.sw, x_tiles, dy_tiles, dwt, beta,
                             workspace, st);
+      if (e != ADH_EUNIMPL) return e;
+    }
+  }
+  if (gen_is_thin(dtype, g, unpadded)) {
+    const size_t need = conv_thin_wgrad_workspace(num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, kh, kw, sh, sw);
+    if (need != 0) {
+      if (workspace_bytes < need) return ADH_EWORKSPACE;
+      e = conv_thin_wgrad_try(num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, kh, kw, sh, sw, x_tiles, dy_tiles, dwt, beta,
+                              workspace, st);
       if (e != ADH_EUNIMPL) return e;
     }
   }

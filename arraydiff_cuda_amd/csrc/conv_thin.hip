@@ -138,17 +138,33 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_fwd_kernel(const Th
 
     __syncthreads();  // the patch (and, the first time, the filter) is in place
     if (tt + 1u < kThinTiles && i0 + kThinBR < P.OH) load_patch(i0 + kThinBR);
-#pragma unroll
-    for (int q = 0; q < (int)kThinSteps; ++q) {
-      float a[8], b[2];
+    // Two operand sets take turns: the reads of step q + 1 are issued, then the multiplications of step q (left
+    // to itself the compiler waits for every read right before the multiplication that uses it).
+    auto fetch = [&](int q, float (&a)[8], float (&b)[2]) {
 #pragma unroll
       for (int pt = 0; pt < 8; ++pt) a[pt] = patch[koff[q] + pix_t[pt]];
 #pragma unroll
       for (int ct = 0; ct < 2; ++ct) b[ct] = b_base[(4 * q) * (int)kThinWPitch + 16 * ct];
+    };
+    auto multiply = [&](const float (&a)[8], const float (&b)[2]) {
 #pragma unroll
       for (int pt = 0; pt < 8; ++pt)
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) acc[pt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[pt], b[ct], acc[pt][ct], 0, 0, 0);
+    };
+    float a0[8], b0[2], a1[8], b1[2];
+    fetch(0, a0, b0);
+#pragma unroll
+    for (int q = 0; q < (int)kThinSteps; q += 2) {
+      fetch(q + 1 < (int)kThinSteps ? q + 1 : (int)kThinSteps - 1, a1, b1);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(a0, b0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (q + 1 >= (int)kThinSteps) break;
+      fetch(q + 2 < (int)kThinSteps ? q + 2 : (int)kThinSteps - 1, a0, b0);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(a1, b1);
+      __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- the lane holds pixels 4 g .. 4 g + 3 of each tile for channel l16 of each channel tile
@@ -210,6 +226,233 @@ int conv_thin_fwd_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cou
   if (vec) hipLaunchKernelGGL((conv_thin_fwd_kernel<true>), dim3((uint32_t)blocks), dim3(kThinThreads), lds, st, P);
   else hipLaunchKernelGGL((conv_thin_fwd_kernel<false>), dim3((uint32_t)blocks), dim3(kThinThreads), lds, st, P);
   return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// backward-filter of the same convolutions: dw[co][k] = beta dw + sum over pixels of dy[co][px] * x[pair k at px], a
+// matrix product whose reduction runs over the pixels and whose columns are the (channel, tap) pairs (ten tiles of
+// 16 for a 7x7x3 window: 147 of 160 columns real).  A workgroup owns 64 output channels x all pairs and a run of
+// 64-pixel chunks (2 rows x 32 columns); each of its four waves takes 16 output channels: one dy operand per step
+// serves the ten column tiles.  The sums go to part[split][co][k] (the filter's own layout) and a second kernel adds
+// the splits in a fixed order.
+// ---------------------------------------------------------------------------------------------
+constexpr uint32_t kThinWgRows = 2, kThinWgCols = 32, kThinWgPx = kThinWgRows * kThinWgCols;
+constexpr uint32_t kThinWgYPitch = kThinWgPx + 4u;
+constexpr int kThinKT = 10;  // column tiles: up to 160 pairs
+
+struct ThinWgradParams {
+  const float *x[ADH_MAX_TILES];
+  const float *dy[ADH_MAX_TILES];
+  float *part;
+  uint32_t N, C, M, HP, WP, OH, OW, kh, kw, sh, sw, KK;
+  uint32_t PRH, PRW, PP;
+  uint32_t NRC, NCC, MG;  // row chunks and column chunks per image and tile, output-channel groups
+  uint32_t chunks, chunks_per_split;
+  FastDiv div_MG, div_NCC, div_NRC, div_N, div_PRW, div_PP, div_kw, div_khw;
+};
+
+int split_sum_launch(const float *part, float *dw, uint32_t elems, uint32_t nsplit, float beta, hipStream_t st);
+
+__global__ __launch_bounds__(kThinThreads, 2) void conv_thin_wgrad_kernel(const ThinWgradParams P) {
+  extern __shared__ __align__(16) float thin_lds[];
+  float *yl = thin_lds;                               // [64 co][kThinWgYPitch]
+  float *patch = thin_lds + kThinCo * kThinWgYPitch;  // [C][PP]
+
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+  uint32_t split, mg;
+  P.div_MG.divmod(blockIdx.x, split, mg);
+  const uint32_t m0 = mg * kThinCo;
+  const uint32_t c_lo = split * P.chunks_per_split, c_hi = min(P.chunks, c_lo + P.chunks_per_split);
+  const uint32_t total = P.C * P.PP;
+
+  // what a thread stages of a chunk: pixel tid % 64 of dy for output channels tid / 64 + 4 j; patch elements tid + 256 j
+  const uint32_t ypx = tid & 63u, yrow = ypx >> 5, ycol = ypx & 31u;
+  uint32_t p_rel[4], p_rc[4];  // offset in the image of the element for the chunk at (0, 0); patch row << 16 | column
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t e = tid + (uint32_t)j * kThinThreads;
+    uint32_t c, e2, pr, pc;
+    P.div_PP.divmod(e, c, e2);
+    P.div_PRW.divmod(e2, pr, pc);
+    p_rel[j] = (c * P.HP + pr) * P.WP + pc;
+    p_rc[j] = pr << 16 | pc;
+  }
+
+  float ypre[16], ppre[4];
+  uint32_t y_ok = 0, p_ok = 0;
+  auto load_chunk = [&](uint32_t ch) {
+    uint32_t q1, q2, q3, cc, rc, n, tile;
+    P.div_NCC.divmod(ch, q1, cc);
+    P.div_NRC.divmod(q1, q2, rc);
+    P.div_N.divmod(q2, tile, n);
+    const uint32_t i0 = rc * kThinWgRows, j0 = cc * kThinWgCols;
+    const float *yb = P.dy[tile] + (size_t)n * P.M * P.OH * P.OW;
+    y_ok = i0 + yrow < P.OH && j0 + ycol < P.OW ? 1u : 0u;
+    const uint32_t y_off = y_ok ? (i0 + yrow) * P.OW + j0 + ycol : 0u;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const uint32_t co = min(m0 + wave + 4u * (uint32_t)j, P.M - 1u);
+      ypre[j] = yb[y_ok ? (size_t)co * P.OH * P.OW + y_off : (size_t)0];
+    }
+    const float *xb = P.x[tile] + (size_t)n * P.C * P.HP * P.WP;
+    const uint32_t base = i0 * P.sh * P.WP + j0 * P.sw;
+    p_ok = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t e = tid + (uint32_t)j * kThinThreads;
+      const bool ok = e < total && i0 * P.sh + (p_rc[j] >> 16) < P.HP && j0 * P.sw + (p_rc[j] & 0xffffu) < P.WP;
+      p_ok |= ok ? 1u << j : 0u;
+      ppre[j] = xb[ok ? base + p_rel[j] : 0u];
+    }
+  };
+  auto store_chunk = [&]() {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const uint32_t cl = wave + 4u * (uint32_t)j;
+      yl[cl * kThinWgYPitch + ypx] = y_ok && m0 + cl < P.M ? ypre[j] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t e = tid + (uint32_t)j * kThinThreads;
+      if (e < total) patch[e] = ((p_ok >> j) & 1u) ? ppre[j] : 0.f;
+    }
+  };
+
+  // column l16 of column tile kt is pair kt * 16 + l16: where it lies in the patch (a pair that does not exist reads
+  // the patch's first element: its column of the result is never stored)
+  uint32_t kB[kThinKT];
+#pragma unroll
+  for (int kt = 0; kt < kThinKT; ++kt) {
+    const uint32_t k = 16u * (uint32_t)kt + l16;
+    uint32_t c, t, a, b;
+    P.div_khw.divmod(k, c, t);
+    P.div_kw.divmod(t, a, b);
+    kB[kt] = k < P.KK ? c * P.PP + a * P.PRW + b : 0u;
+  }
+  const float *a_base = yl + (wave * 16u + l16) * kThinWgYPitch + g;
+
+  thin_floatx4 acc[kThinKT];
+#pragma unroll
+  for (int kt = 0; kt < kThinKT; ++kt) acc[kt] = thin_floatx4{0.f, 0.f, 0.f, 0.f};
+
+  if (c_lo < c_hi) load_chunk(c_lo);
+#pragma unroll 1
+  for (uint32_t ch = c_lo; ch < c_hi; ++ch) {
+    __syncthreads();
+    store_chunk();
+    __syncthreads();
+    if (ch + 1u < c_hi) load_chunk(ch + 1u);
+    // the sums kB + pixel offset are the same for every chunk: a zero the compiler cannot see through keeps them
+    // from being worked out (160 registers) ahead of the loop
+    uint32_t here = 0;
+    asm volatile("" : "+v"(here));
+    // Two operand sets take turns: the reads of step q + 1 are issued, then the multiplications of step q (left
+    // to itself the compiler waits for every read right before the multiplication that uses it).
+    auto fetch = [&](int q, float &a, float (&b)[kThinKT]) {
+      // pixels 4 q .. 4 q + 3: row q / 8, columns 4 (q % 8) ..; this lane reads pixel g of them
+      const uint32_t px_off = (uint32_t)(q >> 3) * P.sh * P.PRW + (4u * (uint32_t)(q & 7) + g) * P.sw + here;
+      a = a_base[4 * q];
+#pragma unroll
+      for (int kt = 0; kt < kThinKT; ++kt) b[kt] = patch[kB[kt] + px_off];
+    };
+    auto multiply = [&](float a, const float (&b)[kThinKT]) {
+#pragma unroll
+      for (int kt = 0; kt < kThinKT; ++kt) acc[kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[kt], acc[kt], 0, 0, 0);
+    };
+    constexpr int kSteps = (int)kThinWgPx / 4;
+    float a0, a1, b0[kThinKT], b1[kThinKT];
+    fetch(0, a0, b0);
+#pragma unroll
+    for (int q = 0; q < kSteps; q += 2) {
+      fetch(q + 1, a1, b1);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(a0, b0);
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(q + 2 < kSteps ? q + 2 : kSteps - 1, a0, b0);  // past the end: the last step again, so that every pass has the same reads in flight
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(a1, b1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // the lane holds output channels 4 g .. 4 g + 3 of its wave's 16 for pair l16 of each column tile
+  float *part = P.part + (size_t)split * P.M * P.KK;
+#pragma unroll
+  for (int kt = 0; kt < kThinKT; ++kt) {
+    const uint32_t k = 16u * (uint32_t)kt + l16;
+    if (k >= P.KK) continue;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const uint32_t co = m0 + wave * 16u + 4u * g + (uint32_t)r;
+      if (co < P.M) part[(size_t)co * P.KK + k] = acc[kt][r];
+    }
+  }
+}
+
+struct ThinWgradPlan {
+  uint32_t nsplit, chunks, chunks_per_split, PRH, PRW;
+  size_t part_bytes, lds;
+};
+
+static bool thin_wgrad_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP,
+                            uint32_t OH, uint32_t OW, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw,
+                            ThinWgradPlan *plan) {
+  if (Cin == 0 || Cin > 3u || Cin * kh * kw > 16u * (uint32_t)kThinKT || N == 0 || OH == 0 || OW == 0) return false;
+  plan->PRH = (kThinWgRows - 1u) * sh + kh;
+  plan->PRW = (kThinWgCols - 1u) * sw + kw;
+  if (plan->PRH >= (1u << 16) || plan->PRW >= (1u << 16)) return false;
+  const uint32_t total = Cin * plan->PRH * plan->PRW;
+  if (total > 4u * kThinThreads) return false;
+  plan->lds = (size_t)(kThinCo * kThinWgYPitch + total) * sizeof(float);
+  if ((uint64_t)Cin * HP * WP >= (1ull << 31) || (uint64_t)Cout * Cin * kh * kw >= (1ull << 31)) return false;
+  const uint64_t chunks = (uint64_t)num_tiles * N * ((OH + kThinWgRows - 1u) / kThinWgRows) * ((OW + kThinWgCols - 1u) / kThinWgCols);
+  if (chunks >= (1ull << 31)) return false;
+  plan->chunks = (uint32_t)chunks;
+  const uint32_t mg = (Cout + kThinCo - 1u) / kThinCo;
+  // two workgroups per CU; at least sixteen chunks each
+  const uint32_t nsplit = std::max(1u, std::min(plan->chunks / 16u, (512u + mg - 1u) / mg));
+  plan->chunks_per_split = (plan->chunks + nsplit - 1u) / nsplit;
+  plan->nsplit = (plan->chunks + plan->chunks_per_split - 1u) / plan->chunks_per_split;
+  plan->part_bytes = (size_t)plan->nsplit * Cout * Cin * kh * kw * sizeof(float);
+  return true;
+}
+
+// the partial sums of conv_thin_wgrad_try (0: not a shape it serves)
+size_t conv_thin_wgrad_workspace(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP,
+                                 uint32_t OH, uint32_t OW, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw) {
+  ThinWgradPlan plan;
+  if (!thin_wgrad_plan(num_tiles, N, Cin, Cout, HP, WP, OH, OW, kh, kw, sh, sw, &plan)) return 0;
+  return plan.part_bytes;
+}
+
+// Filter gradient over halo-padded fp32 tiles for at most three input channels and Cin kh kw <= 160, any stride, no
+// dilation.  `workspace` holds conv_thin_wgrad_workspace bytes.  ADH_EUNIMPL: not served; nothing launched.
+int conv_thin_wgrad_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t OH,
+                        uint32_t OW, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, const void *const *x_tiles,
+                        const void *const *dy_tiles, float *dwt, float beta, void *workspace, hipStream_t st) {
+  ThinWgradPlan plan;
+  if (!thin_wgrad_plan(num_tiles, N, Cin, Cout, HP, WP, OH, OW, kh, kw, sh, sw, &plan)) return ADH_EUNIMPL;
+  ThinWgradParams P = {};
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!aligned_to(x_tiles[t], 4) || !aligned_to(dy_tiles[t], 4)) return ADH_EUNIMPL;
+    P.x[t] = reinterpret_cast<const float *>(x_tiles[t]);
+    P.dy[t] = reinterpret_cast<const float *>(dy_tiles[t]);
+  }
+  P.part = reinterpret_cast<float *>(workspace);
+  P.N = N; P.C = Cin; P.M = Cout; P.HP = HP; P.WP = WP; P.OH = OH; P.OW = OW;
+  P.kh = kh; P.kw = kw; P.sh = sh; P.sw = sw; P.KK = Cin * kh * kw;
+  P.PRH = plan.PRH; P.PRW = plan.PRW; P.PP = plan.PRH * plan.PRW;
+  P.NRC = (OH + kThinWgRows - 1u) / kThinWgRows; P.NCC = (OW + kThinWgCols - 1u) / kThinWgCols;
+  P.MG = (Cout + kThinCo - 1u) / kThinCo;
+  P.chunks = plan.chunks; P.chunks_per_split = plan.chunks_per_split;
+  P.div_MG = FastDiv(P.MG); P.div_NCC = FastDiv(P.NCC); P.div_NRC = FastDiv(P.NRC); P.div_N = FastDiv(N);
+  P.div_PRW = FastDiv(P.PRW); P.div_PP = FastDiv(P.PP); P.div_kw = FastDiv(kw); P.div_khw = FastDiv(kh * kw);
+  const uint64_t blocks = (uint64_t)plan.nsplit * P.MG;
+  if (blocks >= (1ull << 31)) return ADH_EUNIMPL;
+  hipLaunchKernelGGL(conv_thin_wgrad_kernel, dim3((uint32_t)blocks), dim3(kThinThreads), plan.lds, st, P);
+  const int e = launch_status();
+  if (e) return e;
+  return split_sum_launch(P.part, dwt, Cout * P.KK, plan.nsplit, beta, st);
 }
 
 }  // namespace adh
