@@ -36,8 +36,9 @@ struct ThinParams {
 
 typedef float thin_floatx4 __attribute__((ext_vector_type(4)));
 
-// VEC: output rows are whole groups of four pixels at 16-byte aligned addresses
-template <bool VEC>
+// VEC: output rows are whole groups of four pixels at 16-byte aligned addresses.  PJ: patch elements per thread
+// (C * PP <= 256 PJ; 8 for a 7x7 window at stride 1, 17 at stride 2)
+template <bool VEC, int PJ>
 __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_fwd_kernel(const ThinParams P) {
   extern __shared__ __align__(16) float thin_lds[];
   float *wl = thin_lds;                             // [kThinK][kThinWPitch]
@@ -94,14 +95,14 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_fwd_kernel(const Th
   const float *b_base = wl + g * kThinWPitch + wm * 32u + l16;
 
   float *y = P.y[tile] + (size_t)n * P.M * P.OH * P.OW;
-  // a tile's patch: at most 8 elements per thread, loaded a tile ahead (in flight while the tile before is multiplied)
+  // a tile's patch: PJ elements per thread, loaded a tile ahead (in flight while the tile before is multiplied)
   const uint32_t total = P.C * P.PP;
-  float ptmp[8];
+  float ptmp[PJ];
   uint32_t pok = 0;
   auto load_patch = [&](uint32_t i0) {
     pok = 0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < PJ; ++j) {
       const uint32_t e = tid + (uint32_t)j * kThinThreads;
       uint32_t c, e2, pr, pc;
       P.div_PP.divmod(e, c, e2);
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_fwd_kernel(const Th
     if (i0 >= P.OH) break;
     if (tt > 0u) __syncthreads();  // every wave is done with the patch before
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < PJ; ++j) {
       const uint32_t e = tid + (uint32_t)j * kThinThreads;
       if (e < total) patch[e] = ((pok >> j) & 1u) ? ptmp[j] : 0.f;
     }
@@ -138,33 +139,17 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_fwd_kernel(const Th
 
     __syncthreads();  // the patch (and, the first time, the filter) is in place
     if (tt + 1u < kThinTiles && i0 + kThinBR < P.OH) load_patch(i0 + kThinBR);
-    // Two operand sets take turns: the reads of step q + 1 are issued, then the multiplications of step q (left
-    // to itself the compiler waits for every read right before the multiplication that uses it).
-    auto fetch = [&](int q, float (&a)[8], float (&b)[2]) {
+#pragma unroll
+    for (int q = 0; q < (int)kThinSteps; ++q) {
+      float a[8], b[2];
 #pragma unroll
       for (int pt = 0; pt < 8; ++pt) a[pt] = patch[koff[q] + pix_t[pt]];
 #pragma unroll
       for (int ct = 0; ct < 2; ++ct) b[ct] = b_base[(4 * q) * (int)kThinWPitch + 16 * ct];
-    };
-    auto multiply = [&](const float (&a)[8], const float (&b)[2]) {
 #pragma unroll
       for (int pt = 0; pt < 8; ++pt)
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) acc[pt][ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[pt], b[ct], acc[pt][ct], 0, 0, 0);
-    };
-    float a0[8], b0[2], a1[8], b1[2];
-    fetch(0, a0, b0);
-#pragma unroll
-    for (int q = 0; q < (int)kThinSteps; q += 2) {
-      fetch(q + 1 < (int)kThinSteps ? q + 1 : (int)kThinSteps - 1, a1, b1);
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(a0, b0);
-      __builtin_amdgcn_sched_barrier(0);
-      if (q + 1 >= (int)kThinSteps) break;
-      fetch(q + 2 < (int)kThinSteps ? q + 2 : (int)kThinSteps - 1, a0, b0);
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(a1, b1);
-      __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- the lane holds pixels 4 g .. 4 g + 3 of each tile for channel l16 of each channel tile
@@ -216,15 +201,19 @@ int conv_thin_fwd_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cou
   P.PRW = (kThinBC - 1u) * sw + kw;
   P.PP = P.PRH * P.PRW;
   const size_t lds = (size_t)(kThinK * kThinWPitch + Cin * P.PP) * sizeof(float);
-  if (lds > 64u * 1024u || Cin * P.PP > 8u * kThinThreads) return ADH_EUNIMPL;
+  if (lds > 64u * 1024u || Cin * P.PP > 17u * kThinThreads) return ADH_EUNIMPL;
+  const bool small = Cin * P.PP <= 8u * kThinThreads;
   P.NBR = (OH + kThinBR * kThinTiles - 1u) / (kThinBR * kThinTiles); P.NBC = (OW + kThinBC - 1u) / kThinBC; P.MG = (Cout + kThinCo - 1u) / kThinCo;
   P.beta = beta;
   P.div_NBC = FastDiv(P.NBC); P.div_NBR = FastDiv(P.NBR); P.div_MG = FastDiv(P.MG); P.div_N = FastDiv(N);
   P.div_PRW = FastDiv(P.PRW); P.div_PP = FastDiv(P.PP); P.div_kw = FastDiv(kw); P.div_khw = FastDiv(kh * kw);
   const uint64_t blocks = (uint64_t)num_tiles * N * P.MG * P.NBR * P.NBC;
   if (blocks == 0 || blocks >= (1ull << 31)) return ADH_EUNIMPL;
-  if (vec) hipLaunchKernelGGL((conv_thin_fwd_kernel<true>), dim3((uint32_t)blocks), dim3(kThinThreads), lds, st, P);
-  else hipLaunchKernelGGL((conv_thin_fwd_kernel<false>), dim3((uint32_t)blocks), dim3(kThinThreads), lds, st, P);
+  const dim3 grid((uint32_t)blocks), block(kThinThreads);
+  if (vec && small) hipLaunchKernelGGL((conv_thin_fwd_kernel<true, 8>), grid, block, lds, st, P);
+  else if (vec) hipLaunchKernelGGL((conv_thin_fwd_kernel<true, 17>), grid, block, lds, st, P);
+  else if (small) hipLaunchKernelGGL((conv_thin_fwd_kernel<false, 8>), grid, block, lds, st, P);
+  else hipLaunchKernelGGL((conv_thin_fwd_kernel<false, 17>), grid, block, lds, st, P);
   return launch_status();
 }
 
@@ -253,6 +242,8 @@ struct ThinWgradParams {
 
 int split_sum_launch(const float *part, float *dw, uint32_t elems, uint32_t nsplit, float beta, hipStream_t st);
 
+// PJ: patch elements per thread (C * PP <= 256 PJ)
+template <int PJ>
 __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_wgrad_kernel(const ThinWgradParams P) {
   extern __shared__ __align__(16) float thin_lds[];
   float *yl = thin_lds;                               // [64 co][kThinWgYPitch]
@@ -267,9 +258,9 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_wgrad_kernel(const 
 
   // what a thread stages of a chunk: pixel tid % 64 of dy for output channels tid / 64 + 4 j; patch elements tid + 256 j
   const uint32_t ypx = tid & 63u, yrow = ypx >> 5, ycol = ypx & 31u;
-  uint32_t p_rel[4], p_rc[4];  // offset in the image of the element for the chunk at (0, 0); patch row << 16 | column
+  uint32_t p_rel[PJ], p_rc[PJ];  // offset in the image of the element for the chunk at (0, 0); patch row << 16 | column
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < PJ; ++j) {
     const uint32_t e = tid + (uint32_t)j * kThinThreads;
     uint32_t c, e2, pr, pc;
     P.div_PP.divmod(e, c, e2);
@@ -278,7 +269,7 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_wgrad_kernel(const 
     p_rc[j] = pr << 16 | pc;
   }
 
-  float ypre[16], ppre[4];
+  float ypre[16], ppre[PJ];
   uint32_t y_ok = 0, p_ok = 0;
   auto load_chunk = [&](uint32_t ch) {
     uint32_t q1, q2, q3, cc, rc, n, tile;
@@ -298,7 +289,7 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_wgrad_kernel(const 
     const uint32_t base = i0 * P.sh * P.WP + j0 * P.sw;
     p_ok = 0;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < PJ; ++j) {
       const uint32_t e = tid + (uint32_t)j * kThinThreads;
       const bool ok = e < total && i0 * P.sh + (p_rc[j] >> 16) < P.HP && j0 * P.sw + (p_rc[j] & 0xffffu) < P.WP;
       p_ok |= ok ? 1u << j : 0u;
@@ -312,7 +303,7 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_wgrad_kernel(const 
       yl[cl * kThinWgYPitch + ypx] = y_ok && m0 + cl < P.M ? ypre[j] : 0.f;
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < PJ; ++j) {
       const uint32_t e = tid + (uint32_t)j * kThinThreads;
       if (e < total) patch[e] = ((p_ok >> j) & 1u) ? ppre[j] : 0.f;
     }
@@ -402,7 +393,7 @@ static bool thin_wgrad_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32
   plan->PRW = (kThinWgCols - 1u) * sw + kw;
   if (plan->PRH >= (1u << 16) || plan->PRW >= (1u << 16)) return false;
   const uint32_t total = Cin * plan->PRH * plan->PRW;
-  if (total > 4u * kThinThreads) return false;
+  if (total > 8u * kThinThreads) return false;
   plan->lds = (size_t)(kThinCo * kThinWgYPitch + total) * sizeof(float);
   if ((uint64_t)Cin * HP * WP >= (1ull << 31) || (uint64_t)Cout * Cin * kh * kw >= (1ull << 31)) return false;
   const uint64_t chunks = (uint64_t)num_tiles * N * ((OH + kThinWgRows - 1u) / kThinWgRows) * ((OW + kThinWgCols - 1u) / kThinWgCols);
@@ -449,7 +440,10 @@ int conv_thin_wgrad_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t C
   P.div_PRW = FastDiv(P.PRW); P.div_PP = FastDiv(P.PP); P.div_kw = FastDiv(kw); P.div_khw = FastDiv(kh * kw);
   const uint64_t blocks = (uint64_t)plan.nsplit * P.MG;
   if (blocks >= (1ull << 31)) return ADH_EUNIMPL;
-  hipLaunchKernelGGL(conv_thin_wgrad_kernel, dim3((uint32_t)blocks), dim3(kThinThreads), plan.lds, st, P);
+  if (Cin * P.PP <= 4u * kThinThreads)
+    hipLaunchKernelGGL((conv_thin_wgrad_kernel<4>), dim3((uint32_t)blocks), dim3(kThinThreads), plan.lds, st, P);
+  else
+    hipLaunchKernelGGL((conv_thin_wgrad_kernel<8>), dim3((uint32_t)blocks), dim3(kThinThreads), plan.lds, st, P);
   const int e = launch_status();
   if (e) return e;
   return split_sum_launch(P.part, dwt, Cout * P.KK, plan.nsplit, beta, st);
