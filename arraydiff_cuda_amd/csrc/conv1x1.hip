@@ -396,15 +396,26 @@ __global__ __launch_bounds__(kPwThreads, 2) void conv1x1_wgrad_kernel(const PwWg
     }
 }
 
-// dw[e] = beta dw[e] + part[0][e] + part[1][e] + ...: four waves take every fourth split each, then the four
-// sums are added in order
+// dw[e] = beta dw[e] + part[0][e] + part[1][e] + ...: four waves take every fourth split each (in four interleaved
+// chains), then the four sums are added in order: a fixed order, the same bits on every run
 __global__ __launch_bounds__(256) void conv1x1_wgrad_reduce_kernel(const float *part, float *dw, uint32_t elems,
                                                                    uint32_t nsplit, float beta) {
   __shared__ float sums[4][64];
   const uint32_t e = blockIdx.x * 64u + (threadIdx.x & 63u), sg = threadIdx.x >> 6;
   float s = 0.f;
-  if (e < elems)
-    for (uint32_t sp = sg; sp < nsplit; sp += 4u) s += part[(size_t)sp * elems + e];
+  if (e < elems) {
+    // four loads in flight per thread: with a few hundred splits a chain of single loads is all latency
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    uint32_t sp = sg;
+    for (; sp + 12u < nsplit; sp += 16u) {
+      s0 += part[(size_t)sp * elems + e];
+      s1 += part[(size_t)(sp + 4u) * elems + e];
+      s2 += part[(size_t)(sp + 8u) * elems + e];
+      s3 += part[(size_t)(sp + 12u) * elems + e];
+    }
+    for (; sp < nsplit; sp += 4u) s0 += part[(size_t)sp * elems + e];
+    s = (s0 + s1) + (s2 + s3);
+  }
   sums[sg][threadIdx.x & 63u] = s;
   __syncthreads();
   if (sg == 0u && e < elems) {
