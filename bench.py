@@ -445,16 +445,6 @@ def main():
                                                             ws5.data_ptr(), ws5_bytes, stream),
             "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
         del gu
-        # the clock under this kernel is set by power and the power by the data: the same launch on rectified
-        # activations (what a BN -> ReLU -> conv block feeds its convolution: half the values are zero)
-        xr = [t.clamp_min(0) for t in xu]
-        xr_tbl, _ku4 = capi.ptr_table([t.data_ptr() for t in xr])
-        add("conv fwd cfg5 over tiles without halo on rectified activations (bf16; the same launch, max(x, 0) as input)",
-            lambda: lib.adh_conv3x3_unpadded_fwd_tiles(1, K5, N5, C, C, Ht5, W5, xr_tbl, w5.data_ptr(), yu_tbl, 0.0,
-                                                       ws5.data_ptr(), ws5_bytes, stream),
-            "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s",
-            note="not the headline's data: shows how much of the distance to the peak is the clock the device picks for the data")
-        del xr
         add("conv bwd-filter cfg5 over tiles without halo (bf16 in, fp32 filter gradient, two kernels)",
             lambda: lib.adh_conv3x3_unpadded_bwd_filter_tiles(1, K5, N5, C, C, Ht5, W5, xu_tbl, y5_tbl, gw5.data_ptr(), 0.0,
                                                               ws5.data_ptr(), ws5_bytes, stream),
