@@ -687,9 +687,11 @@ def main():
             "hbm", 2 * (packed_b + packed_b) + packed_b, HBM_PEAK_GBS, "GB/s",
             note="x and the interior of dy read twice (sums, then gradient), dx written")
         del xb, dxb
-        # general slab conv (fp32 matrix cores): the 7x7 stride-2 stem over halo 3 (3 -> 64 channels, 224x224 in 4
-        # row-tiles) and a stride-2 3x3 (64 -> 128 channels) over cfg1's tiles
+        # slab conv of any window (fp32 matrix cores): the 7x7 stride-2 stem over halo 3 (3 -> 64 channels, 224x224 in 4
+        # row-tiles), the stride-1 stem of the spatially-parallel net (256x256 in 4 row-tiles; forward and backward-filter
+        # of both by the kernels for at most three input channels) and a stride-2 3x3 (64 -> 128 channels) over cfg1's tiles
         for label, Ci, Co, Hs, Ws, ph, geo in (("7x7 s2 stem 3->64, 4 tiles of 62x230", 3, 64, 56, 224, 3, (7, 7, 2, 2, 1, 1)),
+                                               ("7x7 s1 stem 3->64, 4 tiles of 70x262 (the parallel net's)", 3, 64, 64, 256, 3, (7, 7, 1, 1, 1, 1)),
                                                ("3x3 s2 64->128, 4 tiles of 16x58", 64, 128, 14, 56, 1, (3, 3, 2, 2, 1, 1))):
             HPs, WPs = Hs + 2 * ph, Ws + 2 * ph
             OHs = (HPs - ((geo[0] - 1) * geo[4] + 1)) // geo[2] + 1
