@@ -37,7 +37,7 @@ struct BnParams {
   float *o2[ADH_MAX_TILES];               // forward: saved mean
   float *o3[ADH_MAX_TILES];               // forward: saved 1/sqrt(var + eps)
   float *partial;                         // [tile][c][split][2]
-  uint32_t N, C, H, W, HW, p, split, n_per_split, tiles, groups_per_plane, slots_log2;
+  uint32_t N, C, H, W, HW, p, split, n_per_split, tiles, groups_per_plane, slots_log2, planes_per_pass;
   float eps, beta, beta_param;  // beta: input-gradient accumulation; beta_param: parameter-gradient accumulation
   int relu;
   FastDiv div_C, div_N, div_split, div_groups, div_cols;  // div_groups: the 16-byte groups of a plane; div_cols: row length of the index that a kernel splits into (row, column)
@@ -89,22 +89,25 @@ __global__ __launch_bounds__(kBnThreads) void bn_reduce_kernel(const BnParams P)
   const T *x = reinterpret_cast<const T *>(P.x[tile]);
   const uint32_t n0 = sp * P.n_per_split, n1 = min(P.N, n0 + P.n_per_split);
   const uint32_t groups = P.HW / (uint32_t)VEC;
-  const uint32_t items = n1 > n0 ? (n1 - n0) * groups : 0u;
   float s1 = 0.f, s2 = 0.f;
   if (!BWD) {
     const float K = bn_ld(x, (size_t)c * P.HW);
     // the groups of the split's planes are numbered through: a plane of a few groups (a late layer's 4 x 16 tile
     // is 16 of them) would otherwise leave most of the workgroup idle for one load latency per plane
-    for (uint32_t it = threadIdx.x; it < items; it += kBnThreads) {
-      uint32_t nr, i;
-      P.div_groups.divmod(it, nr, i);
-      const T *pl = x + ((size_t)(n0 + nr) * P.C + c) * P.HW;
-      const Vec xv = *reinterpret_cast<const Vec *>(pl + (size_t)i * VEC);
+    // (P.planes_per_pass planes at a time keep the running number below 2^31: one pass but for gigantic planes)
+    for (uint32_t nb = n0; nb < n1; nb += P.planes_per_pass) {
+      const uint32_t items = min(P.planes_per_pass, n1 - nb) * groups;
+      for (uint32_t it = threadIdx.x; it < items; it += kBnThreads) {
+        uint32_t nr, i;
+        P.div_groups.divmod(it, nr, i);
+        const T *pl = x + ((size_t)(nb + nr) * P.C + c) * P.HW;
+        const Vec xv = *reinterpret_cast<const Vec *>(pl + (size_t)i * VEC);
 #pragma unroll
-      for (int k = 0; k < VEC; ++k) {
-        const float v = bn_f(xv.v[k]) - K;
-        s1 += v;
-        s2 += v * v;
+        for (int k = 0; k < VEC; ++k) {
+          const float v = bn_f(xv.v[k]) - K;
+          s1 += v;
+          s2 += v * v;
+        }
       }
     }
   } else {
@@ -113,21 +116,24 @@ __global__ __launch_bounds__(kBnThreads) void bn_reduce_kernel(const BnParams P)
     const float a = P.relu ? P.scale[tile][c] * P.second_in[tile][c] : 0.f;
     const float mean = P.mean_in[tile][c];
     const float b = P.relu ? P.shift[tile][c] : 0.f;
-    for (uint32_t it = threadIdx.x; it < items; it += kBnThreads) {
-      uint32_t nr, i, h, w;
-      P.div_groups.divmod(it, nr, i);
-      P.div_cols.divmod(i, h, w);  // groups per row
-      const T *pl = x + ((size_t)(n0 + nr) * P.C + c) * P.HW;
-      const T *dl = dy + ((size_t)(n0 + nr) * P.C + c) * HPp * WP + (size_t)P.p * WP + P.p;
-      const Vec xv = *reinterpret_cast<const Vec *>(pl + (size_t)i * VEC);
-      const Vec dv = *reinterpret_cast<const Vec *>(dl + (size_t)h * WP + w * VEC);
+    for (uint32_t nb = n0; nb < n1; nb += P.planes_per_pass) {
+      const uint32_t items = min(P.planes_per_pass, n1 - nb) * groups;
+      for (uint32_t it = threadIdx.x; it < items; it += kBnThreads) {
+        uint32_t nr, i, h, w;
+        P.div_groups.divmod(it, nr, i);
+        P.div_cols.divmod(i, h, w);  // groups per row
+        const T *pl = x + ((size_t)(nb + nr) * P.C + c) * P.HW;
+        const T *dl = dy + ((size_t)(nb + nr) * P.C + c) * HPp * WP + (size_t)P.p * WP + P.p;
+        const Vec xv = *reinterpret_cast<const Vec *>(pl + (size_t)i * VEC);
+        const Vec dv = *reinterpret_cast<const Vec *>(dl + (size_t)h * WP + w * VEC);
 #pragma unroll
-      for (int k = 0; k < VEC; ++k) {
-        const float xc = bn_f(xv.v[k]) - mean;
-        float d = bn_f(dv.v[k]);
-        if (P.relu && !(a * xc + b > 0.f)) d = 0.f;
-        s1 += d;
-        s2 += d * xc;
+        for (int k = 0; k < VEC; ++k) {
+          const float xc = bn_f(xv.v[k]) - mean;
+          float d = bn_f(dv.v[k]);
+          if (P.relu && !(a * xc + b > 0.f)) d = 0.f;
+          s1 += d;
+          s2 += d * xc;
+        }
       }
     }
   }
@@ -452,6 +458,7 @@ int adh_batchnorm2d_fwd_tiles(int dtype, int training, uint32_t num_tiles, uint3
   const uint32_t vec = (uint32_t)(16 / dtype_size(dtype));
   const bool wide = (H * W) % vec == 0;  // the statistics pass reads whole 16-byte groups
   P.div_groups = FastDiv(wide ? H * W / vec : H * W);
+  P.planes_per_pass = std::max(1u, 0x7fffffffu / (wide ? H * W / vec : H * W));
   const uint32_t gpp = ((H + 2u * out_halo) * (W + 2u * out_halo) + vec - 1u) / vec;
   if ((gpp + kBnThreads - 1u) / kBnThreads > 65535u) return ADH_EINVAL;  // grid.y
   if (training) {
@@ -512,6 +519,7 @@ int adh_batchnorm2d_bwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_
   const bool wide = W % vec == 0;
   P.div_cols = FastDiv(wide ? W / vec : W);
   P.div_groups = FastDiv(wide ? H * W / vec : H * W);
+  P.planes_per_pass = std::max(1u, 0x7fffffffu / (wide ? H * W / vec : H * W));
   hipStream_t st = as_stream(stream);
   const uint32_t tc = num_tiles * C;
   if (((wide ? H * W / vec : H * W) + kBnThreads - 1u) / kBnThreads > 65535u) return ADH_EINVAL;  // grid.y
