@@ -52,7 +52,7 @@ __device__ __forceinline__ void st_f(float *p, size_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void st_f(uint16_t *p, size_t i, float v) { p[i] = f32_to_bf16_bits(v); }
 
 constexpr uint32_t kPoolThreads = 256;
-constexpr uint32_t kPoolBandBytes = 24u * 1024u;  // LDS aimed at per block (twice that for the max backward)
+constexpr uint32_t kPoolBandBytes = 24u * 1024u;  // LDS aimed at per block (the backward pass: bwd_band_aim)
 constexpr uint32_t kPoolMaxLds = 64u * 1024u;
 
 // Copies nrows rows of `items` vectors (vec: 16 bytes each) or elements into LDS rows of `pitch` elements, from
@@ -554,6 +554,16 @@ static uint32_t pick_band_rows(const PoolParams &P, uint32_t num_tiles, size_t a
   return rows;
 }
 
+// The LDS a band of the backward pass aims at.  A plane that fits 48 KB whole is one band (no window row is staged
+// twice: 4 tiles of 30 x 114, 0.052 ms against 0.064 in two bands); larger planes take bands of 24 KB, so that six
+// workgroups per CU in different phases keep loads in flight (the max backward over 64 x 256 tiles: 0.46 ms with
+// bands of 48 KB, 0.39 with 24 KB; 0.70 with 18 KB, whose bands stage too many window rows twice).
+template <typename P_>
+static size_t bwd_band_aim(const P_ &P, size_t es, bool is_max) {
+  if (is_max && bwd_band_lds(P, es, is_max, P.OH + P.up) <= 2u * kPoolBandBytes) return 2u * kPoolBandBytes;
+  return kPoolBandBytes;
+}
+
 static void set_bands(PoolParams *P, uint32_t rows) {
   P->band_rows = rows;
   P->bands = (P->OH + P->up + rows - 1u) / rows;  // (up: window rows of the tile above, backward over tiles without halo)
@@ -708,7 +718,7 @@ int adh_pool2d_slab_bwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t 
   P.beta = beta;
   const bool is_max = mode == ADH_POOL_MAX;
   const uint32_t band_rows =
-      wh * ww > 256u ? 0u : pick_band_rows(P, num_tiles, is_max ? 2u * kPoolBandBytes : kPoolBandBytes, [&](uint32_t r) { return bwd_band_lds(P, es, is_max, r); });
+      wh * ww > 256u ? 0u : pick_band_rows(P, num_tiles, bwd_band_aim(P, es, is_max), [&](uint32_t r) { return bwd_band_lds(P, es, is_max, r); });
   if (band_rows) {
     set_bands(&P, band_rows);
     launch_bwd_band(dtype, is_max, P, P.planes * num_tiles * P.bands, bwd_band_lds(P, es, is_max, band_rows),
@@ -787,7 +797,7 @@ int adh_pool2d_unpadded_bwd_tiles(int dtype, int mode, uint32_t num_tiles, uint3
   if (e) return e;
   pool_unpadded_vectors(&P, es, num_tiles, true);
   const uint32_t band_rows =
-      wh * ww > 256u ? 0u : pick_band_rows(P, num_tiles, is_max ? 2u * kPoolBandBytes : kPoolBandBytes, [&](uint32_t r) { return bwd_band_lds(P, es, is_max, r); });
+      wh * ww > 256u ? 0u : pick_band_rows(P, num_tiles, bwd_band_aim(P, es, is_max), [&](uint32_t r) { return bwd_band_lds(P, es, is_max, r); });
   if (!band_rows) return ADH_EUNIMPL;
   set_bands(&P, band_rows);
   launch_bwd_band_u<true>(dtype, is_max, P, P.planes * num_tiles * P.bands, bwd_band_lds(P, es, is_max, band_rows),
