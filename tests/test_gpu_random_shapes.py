@@ -391,6 +391,57 @@ def test_pointwise_and_strided_3x3_kernels_random(oracle, K, N, Cin, Cout, Ht, W
         assert rel_err(host(ga[r]), (g0 + g_want)[:, :, r * Ht:(r + 1) * Ht, :]) <= 1e-5
 
 
+def _thin_cases(seed, count):
+    """(K, N, Cin, Cout, HP, WP, kh, kw, sh, sw): at most three input channels and Cin kh kw <= 160, the shapes whose
+    forward and filter gradient over halo-padded tiles take the kernels for a network's stem."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        Cin, kh, kw = int(rng.integers(1, 4)), int(rng.integers(1, 8)), int(rng.integers(1, 8))
+        if (kh == 1 and kw == 1) or Cin * kh * kw > 160:
+            continue
+        sh, sw = int(rng.integers(1, 3)), int(rng.integers(1, 3))
+        HP, WP = kh + int(rng.integers(0, 40)), kw + int(rng.integers(0, 90))
+        K, N, Cout = int(rng.integers(1, 4)), int(rng.integers(1, 4)), int(rng.integers(1, 90))
+        if K * N * Cin * Cout * kh * kw * ((HP - kh) // sh + 1) * ((WP - kw) // sw + 1) > 4e7:
+            continue
+        out.append((K, N, Cin, Cout, HP, WP, kh, kw, sh, sw))
+    return out
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,HP,WP,kh,kw,sh,sw", _thin_cases(2034, 32))
+def test_few_input_channels_kernels_random(oracle, K, N, Cin, Cout, HP, WP, kh, kw, sh, sw):
+    """Forward and filter gradient (beta 0 and 1) over halo-padded tiles with one to three input channels against the
+    oracle (fp32, rel-err <= 1e-5)."""
+    rng = np.random.default_rng(HP * 101 + WP * 3 + Cout)
+    geo = (kh, kw, sh, sw, 1, 1)
+    OH, OW = (HP - kh) // sh + 1, (WP - kw) // sw + 1
+    xs = [rng.uniform(-1, 1, size=(N, Cin, HP, WP)).astype(np.float32) for _ in range(K)]
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * np.sqrt(2.0 / (Cin * kh * kw))).astype(np.float32)
+    dys = [rng.standard_normal((N, Cout, OH, OW)).astype(np.float32) for _ in range(K)]
+    y0 = [rng.standard_normal((N, Cout, OH, OW)).astype(np.float32) for _ in range(K)]
+    gw0 = rng.standard_normal(w.shape).astype(np.float32)
+    d_xs, d_dys, d_w = [dev(a) for a in xs], [dev(a) for a in dys], dev(w)
+    ws = torch.empty(max(capi.conv2d_workspace_bytes(wh, capi.ADH_F32, K, N, Cin, Cout, HP, WP, *geo) for wh in (0, 2)) // 4,
+                     device="cuda")
+    ys = [torch.full((N, Cout, OH, OW), float("nan"), device="cuda") for _ in range(K)]
+    ya = [dev(a) for a in y0]
+    gw, gwa = torch.full(w.shape, float("nan"), device="cuda"), dev(gw0)
+    capi.check(capi.conv2d_fwd_tiles(d_xs, d_w, ys, N, Cin, Cout, HP, WP, *geo, ws=ws), "fwd")
+    capi.check(capi.conv2d_fwd_tiles(d_xs, d_w, ya, N, Cin, Cout, HP, WP, *geo, beta=1.0, ws=ws), "fwd +")
+    capi.check(capi.conv2d_bwd_filter_tiles(d_xs, d_dys, gw, N, Cin, Cout, HP, WP, *geo, ws=ws), "bwd-filter")
+    capi.check(capi.conv2d_bwd_filter_tiles(d_xs, d_dys, gwa, N, Cin, Cout, HP, WP, *geo, beta=1.0, ws=ws), "bwd-filter +")
+    gw_want = np.zeros(w.shape, np.float32)
+    for r in range(K):
+        y = np.empty((N, Cout, OH, OW), np.float32)
+        oracle.conv2d_slab_fwd(xs[r], w, sh, sw, 1, 1, y)
+        assert rel_err(host(ys[r]), y) <= 1e-5
+        assert rel_err(host(ya[r]), y0[r] + y) <= 1e-5
+        oracle.conv2d_slab_bwd_filter(xs[r], dys[r], sh, sw, 1, 1, gw_want, beta=1.0)
+    assert rel_err(host(gw), gw_want) <= 1e-5
+    assert rel_err(host(gwa), gw0 + gw_want) <= 1e-5
+
+
 @pytest.mark.parametrize("K,Ht,W,wh,ww,sh,sw,dh,dw,pad_h,pad_w", _unpadded_geometries(2031, 24, 4))
 def test_pool_over_tiles_without_halo_random(oracle, K, Ht, W, wh, ww, sh, sw, dh, dw, pad_h, pad_w):
     """adh_pool2d_unpadded_*_tiles against the oracle's pooling of the unsplit zero-padded tensor (windows without
