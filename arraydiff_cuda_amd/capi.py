@@ -48,6 +48,7 @@ SIGNATURES = {
     "adh_conv3x3_slab_fwd_tiles_unexchanged": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_data_tiles_reduced": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_unpadded_fwd_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp, sz, vp]),
+    "adh_conv3x3_unpadded_fwd_residual_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, vpp, vp]),
     "adh_conv3x3_unpadded_bwd_data_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv3x3_unpadded_bwd_filter_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_fwd_tiles_static": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vp, vpp, f32, vp]),
@@ -280,6 +281,16 @@ def conv_unpadded_fwd_tiles(xs, w, ys, N, Cin, Cout, H, W, beta=0.0, ws=None):
     wp, wb = _ws(ws)
     return lib().adh_conv3x3_unpadded_fwd_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, xt, w.data_ptr(), yt, beta, wp,
                                                 wb, _stream())
+
+
+def conv_unpadded_fwd_residual_tiles(xs, w, res, ys, N, Cin, Cout, H, W):
+    """ys[t] = conv(xs, w)[t] + res[t] over tiles without halo (fp32)."""
+    _dev(w, *xs, *res, *ys)
+    xt, k1 = _tbl(xs)
+    rt, k2 = _tbl(res)
+    yt, k3 = _tbl(ys)
+    return lib().adh_conv3x3_unpadded_fwd_residual_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, xt, w.data_ptr(), rt, yt,
+                                                         _stream())
 
 
 def conv_unpadded_bwd_data_tiles(w, dys, dxs, N, Cin, Cout, H, W, beta=0.0, ws=None):

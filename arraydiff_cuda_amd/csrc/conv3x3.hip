@@ -62,6 +62,9 @@ struct ConvParams {
   // the interior of the gradient tile complete, as after a halo reduce.
   int32_t rows_from_neighbours, nb_lo, nb_hi, nb_above, nb_below;
   float beta;
+  // res[t] set (with beta = 1): the value added to the result is read from res[t], a tensor laid out like out[t],
+  // instead of from out[t] itself: out = conv(in) + res, the residual sum of a block in the convolution's stores
+  const float *res[ADH_MAX_TILES];
   FastDiv div_tiles_x, div_TW;
 };
 
@@ -123,6 +126,7 @@ __global__ __launch_bounds__(64 * WAVES, PROWS == kPatchRowsShort ? 2 : 1) void 
   const uint64_t out_plane = (uint64_t)P.OH * P.OW;
   const float *__restrict__ in = P.in[t] + (uint64_t)n * P.Cred * in_plane;
   float *__restrict__ out = P.out[t] + (uint64_t)n * P.Cout * out_plane;
+  const float *__restrict__ added = P.res[t] ? P.res[t] + (uint64_t)n * P.Cout * out_plane : out;
 
   const uint32_t rows_here = min(P.R, P.OH - oh0);
   const uint32_t cols_here = min(P.TW, P.OW - ow0);
@@ -312,12 +316,14 @@ __global__ __launch_bounds__(64 * WAVES, PROWS == kPatchRowsShort ? 2 : 1) void 
       uint32_t r_, c_;
       P.div_TW.divmod(q, r_, c_);
       if (q < npix && r_ < rows_here && c_ < cols_here) {
-        float *dst = out + (uint64_t)o_d * out_plane + (uint64_t)(oh0 + r_) * P.OW + ow0 + c_;
+        const uint64_t at = (uint64_t)o_d * out_plane + (uint64_t)(oh0 + r_) * P.OW + ow0 + c_;
+        float *dst = out + at;
+        const float *src = added + at;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           if (o_d + i < P.Cout) {
             float v = acc[j][i];
-            if (P.beta != 0.f) v += P.beta * dst[(uint64_t)i * out_plane];
+            if (P.beta != 0.f) v += P.beta * src[(uint64_t)i * out_plane];
             dst[(uint64_t)i * out_plane] = v;
           }
         }
@@ -423,7 +429,8 @@ int conv_bf16_via_f32(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, u
 // which: ADH_CONV_FWD or ADH_CONV_BWD_DATA.  H, W are the interior extents.
 static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                        uint32_t W, const void *const *in_tiles, const void *w, void *const *out_tiles, float beta,
-                       hipStream_t st, bool rows_from_neighbours = false, bool unpadded = false) {
+                       hipStream_t st, bool rows_from_neighbours = false, bool unpadded = false,
+                       const void *const *res_tiles = nullptr) {
   if (!dtype_ok(dtype)) return ADH_EINVAL;
   if (dtype != ADH_F32) return ADH_EUNIMPL;
   if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
@@ -442,11 +449,16 @@ static int conv_direct(int which, int dtype, uint32_t num_tiles, uint32_t N, uin
     if (!aligned_to(in_tiles[t], 4) || !aligned_to(out_tiles[t], 4)) return ADH_EALIGN;
     P.in[t] = reinterpret_cast<const float *>(in_tiles[t]);
     P.out[t] = reinterpret_cast<float *>(out_tiles[t]);
+    if (res_tiles) {
+      if (!res_tiles[t]) return ADH_ENULL;
+      if (!aligned_to(res_tiles[t], 4)) return ADH_EALIGN;
+      P.res[t] = reinterpret_cast<const float *>(res_tiles[t]);
+    }
   }
   P.w = reinterpret_cast<const float *>(w);
   P.num_tiles = num_tiles;
   P.N = N;
-  P.beta = beta;
+  P.beta = res_tiles ? 1.f : beta;
   P.rows_from_neighbours = rows_from_neighbours ? 1 : 0;
   if (which == ADH_CONV_FWD) {
     P.nb_lo = 0; P.nb_hi = (int32_t)H + 1; P.nb_above = (int32_t)H; P.nb_below = 1;
@@ -598,6 +610,16 @@ int adh_conv3x3_unpadded_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, ui
                        true, true);
   return conv_bf16_unpadded(ADH_CONV_FWD, dtype, num_tiles, N, Cin, Cout, H, W, x_tiles, w, y_tiles, beta, workspace,
                             workspace_bytes, as_stream(stream));
+}
+
+int adh_conv3x3_unpadded_fwd_residual_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                                            uint32_t W, const void *const *x_tiles, const void *w,
+                                            const void *const *res_tiles, void *const *y_tiles, void *stream) {
+  if (!dtype_ok(dtype)) return ADH_EINVAL;
+  if (dtype != ADH_F32) return ADH_EUNIMPL;
+  if (!res_tiles) return ADH_ENULL;
+  return conv_direct(ADH_CONV_FWD, dtype, num_tiles, N, Cin, Cout, H, W, x_tiles, w, y_tiles, 1.f, as_stream(stream), true,
+                     true, res_tiles);
 }
 
 int adh_conv3x3_unpadded_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,

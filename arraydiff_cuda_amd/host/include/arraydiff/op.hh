@@ -979,16 +979,24 @@ public:
   }
   // each rank holds its own copy of the filter in the reference; here kernels.at(r) may all be
   // the same variable, its gradient then accumulates over the tiles
+  // residuals (not in the reference; tiles without halo only): residuals.at(r) is added to rank r's result,
+  // y = conv(x, w) + residual, the sum that closes a residual block, in the convolution's own stores where the 3x3
+  // kernel serves the shape (else one pass that adds in place).  The residual's gradient is the output's gradient:
+  // its variable forwards to the output's, so the backward pass does nothing for it.  As with JoinOp's trunk_input,
+  // every other consumer of a residual must lie UPSTREAM of this node's input (the block input, whose other
+  // consumer is the first node of the path that ends here) or the residual must have no other consumer (the
+  // projection of a block that changes extents): those nodes then add to the shared buffer after this node has read it.
   static vector<shared_ptr<Var<V>>> MakeParallel(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs,
-                                                 vector<shared_ptr<Var<A>>> kernels, shared_ptr<Context> ctx) {
-    auto op = make_shared<SlabConv2DOp<V, A>>(shape, inputs, kernels, ctx);
+                                                 vector<shared_ptr<Var<A>>> kernels, shared_ptr<Context> ctx,
+                                                 vector<shared_ptr<Var<V>>> residuals = {}) {
+    auto op = make_shared<SlabConv2DOp<V, A>>(shape, inputs, kernels, ctx, residuals);
     vector<shared_ptr<Var<V>>> outputs;
     for (size_t r = 0; r < inputs.size(); ++r) outputs.push_back(make_shared<NoOp<V>>(op, op->ys_.at(r).clone()));
     return outputs;
   }
   SlabConv2DOp(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs, vector<shared_ptr<Var<A>>> kernels,
-               shared_ptr<Context> ctx)
-      : ctx_(ctx), shape_(shape), x_vars_(inputs), kernel_vars_(kernels) {
+               shared_ptr<Context> ctx, vector<shared_ptr<Var<V>>> residuals = {})
+      : ctx_(ctx), shape_(shape), x_vars_(inputs), kernel_vars_(kernels), res_vars_(residuals) {
     if (shape.kernel[0] == 0 || shape.kernel[1] == 0 || shape.stride[0] == 0 || shape.stride[1] == 0 ||
         shape.dilate[0] == 0 || shape.dilate[1] == 0)
       throw std::invalid_argument("SlabConv2DOp: empty window, stride or dilation");
@@ -1015,6 +1023,17 @@ public:
       kernels_.push_back(kernels[r]->data());
       ys_.push_back(VarData<V>(_get_output_shape(inputs[r]->shape(), inputs[r]->batch_shape()), inputs[r]->batch_shape()));
     }
+    if (!residuals.empty()) {
+      if (!shape.unpadded_tiles || residuals.size() != inputs.size())
+        throw std::invalid_argument("SlabConv2DOp: one residual per tile, over tiles without halo");
+      for (size_t r = 0; r < residuals.size(); ++r) {
+        if (residuals[r]->shape() != ys_[r].shape() || residuals[r]->batch_shape() != ys_[r].batch_shape() ||
+            !residuals[r]->offset().is_zero())
+          throw std::invalid_argument("SlabConv2DOp: a residual must be packed and of the output's shape");
+        res_.push_back(residuals[r]->data());
+        ys_[r].absorb_grad(res_[r]);
+      }
+    }
   }
   // out = floor((in + 2p - ((k-1)d+1)) / s) + 1 per axis (op.cc:1512-1523)
   Shape3D _get_output_shape(Shape3D in_shape, size_t) {
@@ -1038,6 +1057,7 @@ public:
   }
   virtual void _push(EpochId e, function<void(Op *)> apply) {
     if (1 == stack_.push(e)) {
+      for (auto &res : res_vars_) res->_push(e, apply);
       for (size_t r = 0; r < x_vars_.size(); ++r) {
         x_vars_[r]->_push(e, apply);
         kernel_vars_[r]->_push(e, apply);
@@ -1052,6 +1072,7 @@ public:
         kernel_vars_[r]->_pop(e, apply);
         x_vars_[r]->_pop(e, apply);
       }
+      for (size_t r = res_vars_.size(); r-- > 0;) res_vars_[r]->_pop(e, apply);
     }
   }
   virtual void _forward(TxnId txn);
@@ -1070,6 +1091,8 @@ private:
   vector<VarData<V>> xs_;
   vector<VarData<A>> kernels_;
   vector<VarData<V>> ys_;
+  vector<shared_ptr<Var<V>>> res_vars_;  // empty, or one per tile: added to the result
+  vector<VarData<V>> res_;
 };
 template <typename V, typename A, typename B = A>
 using CudnnConv2DOp = SlabConv2DOp<V, A>;

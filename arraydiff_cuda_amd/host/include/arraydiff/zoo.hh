@@ -53,7 +53,8 @@ inline void parallel_vars_insert_all(vector<VarIdSet> &dst, const vector<VarIdSe
 // into every rank.
 template <typename V, typename A = GPUArray4D<float>>
 ParallelParamOp<V> parallel_conv2d(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs,
-                                   typename ParamOp<A>::InitFn kernel_init, bool enable_bias, shared_ptr<Context> ctx) {
+                                   typename ParamOp<A>::InitFn kernel_init, bool enable_bias, shared_ptr<Context> ctx,
+                                   vector<shared_ptr<Var<V>>> residuals = {}) {
   if (enable_bias) throw std::invalid_argument("parallel_conv2d: bias is not implemented");
   // every rank's copy starts from rank 0's values (ParallelSGDOptimizer::reset) and receives the
   // same update: one launch serves all tiles
@@ -84,7 +85,7 @@ ParallelParamOp<V> parallel_conv2d(Conv2DShape shape, vector<shared_ptr<Var<V>>>
     out.params.push_back(VarIdSet::Singleton(kernel->vars().at(0)));
     out.grads.push_back(VarIdSet::Singleton(kernel->vars().at(1)));
   }
-  out.ops = CudnnConv2DOp<V, A, A>::MakeParallel(shape, inputs, kernels, ctx);
+  out.ops = CudnnConv2DOp<V, A, A>::MakeParallel(shape, inputs, kernels, ctx, residuals);
   return out;
 }
 
@@ -135,7 +136,8 @@ bool halo_free_conv(const Conv2DShape &shape, size_t stride, const vector<shared
 }
 template <typename V>
 vector<shared_ptr<Var<V>>> unpadded_conv(ParallelBatchNormParamOp<V> &block, Conv2DShape shape, size_t stride,
-                                         vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx) {
+                                         vector<shared_ptr<Var<V>>> inputs, shared_ptr<Context> ctx,
+                                         vector<shared_ptr<Var<V>>> residuals = {}) {
   typedef GPUArray4D<float> A;
   Conv2DShape cs = shape;
   cs.stride = {stride, stride};
@@ -143,7 +145,7 @@ vector<shared_ptr<Var<V>>> unpadded_conv(ParallelBatchNormParamOp<V> &block, Con
   cs.unpadded_tiles = true;
   const size_t cin = inputs.at(0)->shape().shape[2];
   auto conv = parallel_conv2d<V, A>(cs, inputs, kaiming_init_gen<A>(cin * shape.kernel[0] * shape.kernel[1], shape.filters),
-                                    false, ctx);
+                                    false, ctx, residuals);
   parallel_vars_insert_all(block.params, conv.params);
   parallel_vars_insert_all(block.grads, conv.grads);
   return conv.ops;
@@ -154,16 +156,22 @@ vector<shared_ptr<Var<V>>> unpadded_conv(ParallelBatchNormParamOp<V> &block, Con
 template <typename V>
 vector<shared_ptr<Var<V>>> bn_relu_pad_conv3x3(ParallelBatchNormParamOp<V> &block, Conv2DShape shape, size_t stride,
                                                shared_ptr<bool> switch_var, vector<shared_ptr<Var<V>>> inputs,
-                                               shared_ptr<Context> ctx) {
+                                               shared_ptr<Context> ctx, vector<shared_ptr<Var<V>>> residuals = {}) {
   const size_t cin = inputs.at(0)->shape().shape[2];
   if (halo_free_conv(shape, stride, inputs, ctx)) {
     auto bnorm = CudnnBatchNorm2DOp<bool, V, GPUArray1D<float>>::MakeParallel(cin, switch_var, inputs, ctx, true, 0);
     add_batch_norm(block, bnorm);
-    return unpadded_conv(block, shape, stride, bnorm.ops, ctx);
+    return unpadded_conv(block, shape, stride, bnorm.ops, ctx, residuals);
   }
   auto bnorm = CudnnBatchNorm2DOp<bool, V, GPUArray1D<float>>::MakeParallel(cin, switch_var, inputs, ctx, true, 1);
   add_batch_norm(block, bnorm);
-  return exchanged_conv3x3(block, shape, stride, bnorm.ops, ctx);
+  auto conv = exchanged_conv3x3(block, shape, stride, bnorm.ops, ctx);
+  if (residuals.empty()) return conv;
+  // the conv over exchanged tiles takes no residual: a sum node closes the block.  The conv feeds the sum only, and
+  // the residual's other consumers lie upstream of the conv: both gradients are the sum's output gradient, one
+  // buffer that the upstream nodes add to in place
+  vector<vector<shared_ptr<Var<V>>>> join_inputs{residuals, conv};
+  return parallel_sum<V>(join_inputs, ctx, 1, 0);
 }
 }  // namespace detail
 
@@ -175,11 +183,10 @@ ParallelBatchNormParamOp<V> spatial_parallel_residual_v2_conv2d(Conv2DShape shap
   if (shape.filters != cin) throw std::invalid_argument("spatial_parallel_residual_v2_conv2d: the block keeps the channel count");
   auto block = detail::empty_block<V>(inputs.size());
   auto conv1 = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, inputs, ctx);
-  auto conv2 = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, conv1, ctx);
-  vector<vector<shared_ptr<Var<V>>>> join_inputs{inputs, conv2};
-  // conv2 feeds the sum only, and the block input's other consumer (the first batch norm) lies upstream of conv2:
-  // both gradients are the sum's output gradient, one buffer that the batch norm's backward pass adds to in place
-  block.ops = parallel_sum<V>(join_inputs, ctx, 1, 0);
+  // the second conv adds the block input to its result.  The block input's other consumer (the first batch norm)
+  // lies upstream of that conv: the input's gradient is the output's gradient, one buffer that the batch norm's
+  // backward pass adds to in place
+  block.ops = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, conv1, ctx, inputs);
   return block;
 }
 
@@ -209,9 +216,9 @@ ParallelBatchNormParamOp<V> spatial_parallel_proj_residual_v2_conv2d(Conv2DShape
   auto conv1 = detail::halo_free_conv(shape, stride, relu0, ctx)
                    ? detail::unpadded_conv(block, shape, stride, relu0, ctx)
                    : detail::exchanged_conv3x3(block, shape, stride, HaloPad2DOp<V>::MakeParallel(1, relu0, ctx), ctx);
-  auto conv2 = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, conv1, ctx);
-  vector<vector<shared_ptr<Var<V>>>> join_inputs{proj.ops, conv2};
-  block.ops = parallel_sum<V>(join_inputs, ctx, 1, 0);  // both convs feed the sum only: their gradients are the sum's, one buffer
+  // the second conv adds the projection to its result; the projection feeds nothing else, so its gradient is the
+  // output's gradient, one buffer
+  block.ops = detail::bn_relu_pad_conv3x3(block, shape, 1, switch_var, conv1, ctx, proj.ops);
   return block;
 }
 

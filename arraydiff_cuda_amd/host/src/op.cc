@@ -482,8 +482,9 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
     const float *w0 = kernels_[replicated ? 0 : todo[0]].val().get(txn, id()).dptr();
     const void *xt[ADH_MAX_TILES];
     void *yt[ADH_MAX_TILES];
+    const void *rt[ADH_MAX_TILES];
     uint32_t n = 0;
-    TileDims d{};
+    TileDims d{}, yd{};
     vector<size_t> rest;
     for (size_t r : todo) {
       A4 &w = kernels_[r].val().get(txn, id());
@@ -499,6 +500,13 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
       check_filter(w, shape_, d.C);
       xt[n] = x.base_as_view().dptr();
       yt[n] = y.as_view().dptr();
+      yd = dims_of(y);
+      if (!res_.empty()) {
+        V3 &res = res_[r].val().get(txn, id());
+        check_packed(res, "SlabConv2DOp (residual)");
+        if (dims_of(res).N != d.N) throw HazardError("SlabConv2DOp: the residual's batch differs from the input's");
+        rt[n] = res.as_view().dptr();
+      }
       ++n;
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
@@ -506,15 +514,25 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
     if (shape_.unpadded_tiles) {
       if (n != K) throw HazardError("SlabConv2DOp: tiles without halo need every rank in one pass");
       if (unpadded_3x3_kernels(*this, d, n, shape_.filters)) {
-        adh_check(adh_conv3x3_unpadded_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt, 0.0f,
-                                                 nullptr, 0, conn.stream()),
-                  "SlabConv2DOp::_forward (tiles without halo)");
+        if (!res_.empty())
+          adh_check(adh_conv3x3_unpadded_fwd_residual_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, rt,
+                                                            yt, conn.stream()),
+                    "SlabConv2DOp::_forward (tiles without halo, residual)");
+        else
+          adh_check(adh_conv3x3_unpadded_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, d.H, d.W, xt, w0, yt, 0.0f,
+                                                   nullptr, 0, conn.stream()),
+                    "SlabConv2DOp::_forward (tiles without halo)");
       } else {
         size_t ws_bytes;
         void *ws = unpadded_conv_scratch(dc, ADH_CONV_FWD, n, d, shape_, &ws_bytes);
         adh_check(adh_conv2d_unpadded_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, ADH_UNPADDED_GEOMETRY(d, shape_),
                                                 xt, w0, yt, 0.0f, ws, ws_bytes, conn.stream()),
                   "SlabConv2DOp::_forward (tiles without halo, general)");
+        if (!res_.empty()) {
+          for (uint32_t t = 0; t < n; ++t)
+            adh_check(adh_add_f32((uint64_t)yd.W * yd.H * yd.C * yd.N, (const float *)rt[t], (float *)yt[t], conn.stream()),
+                      "SlabConv2DOp::_forward (residual)");
+        }
       }
       todo.swap(rest);
       continue;

@@ -217,6 +217,14 @@ int adh_conv3x3_unpadded_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, ui
                                    uint32_t H, uint32_t W, const void *const *x_tiles, const void *w,
                                    void *const *y_tiles, float beta, void *workspace, size_t workspace_bytes,
                                    void *stream);
+/* The sum that closes a residual block, JoinOp<SumJoin> after the block's second CudnnConv2DOp
+ * (src/zoo.cc:577-652: x + conv(...); src/op.cc:744-867), in the convolution's own stores:
+ * y = conv(x, w) + res over tiles without halo, res_tiles laid out like y_tiles (H x W x Cout x N each, packed;
+ * res_tiles[t] may be y_tiles[t] itself, but must not overlap another tile of y).  fp32 only (other dtypes:
+ * ADH_EUNIMPL), no workspace. */
+int adh_conv3x3_unpadded_fwd_residual_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                            uint32_t H, uint32_t W, const void *const *x_tiles, const void *w,
+                                            const void *const *res_tiles, void *const *y_tiles, void *stream);
 int adh_conv3x3_unpadded_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
                                         uint32_t H, uint32_t W, const void *w, const void *const *dy_tiles,
                                         void *const *dx_tiles, float beta, void *workspace,

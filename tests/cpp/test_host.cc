@@ -257,8 +257,10 @@ static void put_tile(std::vector<float> &full, const std::vector<float> &t, size
 // fused: batch norm + rectifier + halo pad as one node (SlabBatchNorm2DOp with relu and out_halo) instead of three
 // shared_grad: the sum's output gradient, the second conv's output gradient (JoinOp's sole_consumer_of) and the block
 // input's gradient (trunk_input: the first batch norm adds to it in place) are one buffer: the sum's backward pass copies nothing
+// sum_in_conv: both convs run over tiles without halo and the second adds the block input to its result (no pad,
+// exchange or sum node; the block input's gradient is the second conv's output gradient)
 static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, size_t W, bool fused = false,
-                                        bool shared_grad = false) {
+                                        bool shared_grad = false, bool sum_in_conv = false) {
   std::mt19937 gen(31337 + (unsigned)K);
   auto ctx = MultiGPUContext::Make(K);
   typedef GPUBatchArray3D<float> V;
@@ -281,16 +283,22 @@ static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, 
   Conv2DShape cs;
   cs.filters = C; cs.axes = {0, 1}; cs.kernel = {3, 3}; cs.dilate = {1, 1}; cs.stride = {1, 1}; cs.pad = {1, 1};
   cs.halo_padded_input = true; cs.enable_hmma = false;
-  auto bnorm0 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, inputs, ctx, fused, fused ? 1 : 0);
+  if (sum_in_conv) {
+    cs.halo_padded_input = false;
+    cs.unpadded_tiles = true;
+  }
+  const size_t halo = sum_in_conv ? 0 : 1;
+  auto bnorm0 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, inputs, ctx, fused, fused ? halo : 0);
   auto pad1 = fused ? bnorm0.ops : HaloPad2DOp<V>::MakeParallel(1, parallel_relu<V>(bnorm0.ops, ctx), ctx);
-  auto exch1 = HaloExch2DOp<V>::MakeParallel(1, pad1, ctx);
+  auto exch1 = sum_in_conv ? pad1 : HaloExch2DOp<V>::MakeParallel(1, pad1, ctx);
   auto conv1 = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch1, vector<shared_ptr<Var<A>>>(K, w1_src), ctx);
-  auto bnorm1 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, conv1, ctx, fused, fused ? 1 : 0);
+  auto bnorm1 = CudnnBatchNorm2DOp<bool, V, B>::MakeParallel(C, switch_var, conv1, ctx, fused, fused ? halo : 0);
   auto pad2 = fused ? bnorm1.ops : HaloPad2DOp<V>::MakeParallel(1, parallel_relu<V>(bnorm1.ops, ctx), ctx);
-  auto exch2 = HaloExch2DOp<V>::MakeParallel(1, pad2, ctx);
-  auto conv2 = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch2, vector<shared_ptr<Var<A>>>(K, w2_src), ctx);
+  auto exch2 = sum_in_conv ? pad2 : HaloExch2DOp<V>::MakeParallel(1, pad2, ctx);
+  auto conv2 = CudnnConv2DOp<V, A, A>::MakeParallel(cs, exch2, vector<shared_ptr<Var<A>>>(K, w2_src), ctx,
+                                                    sum_in_conv ? inputs : vector<shared_ptr<Var<V>>>());
   vector<vector<shared_ptr<Var<V>>>> join_inputs{inputs, conv2};
-  auto join = parallel_sum<V>(join_inputs, ctx, shared_grad ? 1 : -1, shared_grad ? 0 : -1);
+  auto join = sum_in_conv ? conv2 : parallel_sum<V>(join_inputs, ctx, shared_grad ? 1 : -1, shared_grad ? 0 : -1);
   auto y_full = SpatialJoinedGather2DOp<V>::Make(join, ctx);
   auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
   sink->set_host_grad(dY.data());
@@ -370,7 +378,8 @@ static void test_spatial_residual_block(size_t K, size_t N, size_t C, size_t H, 
     for (size_t i = 0; i < full; ++i) dXr[i] += dY[i];
     const double ey = rel_err(Y, Yr), ex = rel_err(dX, dXr), ew1 = rel_err(dW1, dW1r), ew2 = rel_err(dW2, dW2r);
     std::printf("residual block%s K=%zu N=%zu C=%zu %zux%zu rep %d: rel-err y %.2e dx %.2e dw1 %.2e dw2 %.2e bn params %.2e\n",
-                fused ? " (fused bn+relu+pad)" : "", K, N, C, H, W, rep, ey, ex, ew1, ew2, e_param);
+                sum_in_conv ? " (sum in the second conv)" : fused ? " (fused bn+relu+pad)" : "", K, N, C, H, W, rep, ey, ex, ew1,
+                ew2, e_param);
     CHECK(ey <= 1e-5 && ex <= 2e-5 && ew1 <= 2e-5 && ew2 <= 1e-5 && e_param <= 1e-4);
   }
 }
@@ -1037,6 +1046,8 @@ int main(int argc, char **argv) {
     test_spatial_residual_block(2, 4, 64, 28, 28, true);
     test_spatial_residual_block(4, 2, 8, 16, 12, true, true);
     test_spatial_residual_block(2, 4, 64, 28, 28, false, true);
+    test_spatial_residual_block(4, 2, 8, 16, 12, true, false, true);   // small tiles: the general kernel, then the sum
+    test_spatial_residual_block(2, 4, 64, 28, 28, true, false, true);  // the 3x3 kernel adds the block input itself
     test_spatial_pool_graph(kMaxPool, 4, 2, 8, 16, 12);
     test_spatial_pool_graph(kAveragePool, 2, 3, 5, 8, 10);
     test_spatial_pool_graph(kMaxPool, 4, 8, 64, 112, 112);

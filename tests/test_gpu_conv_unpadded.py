@@ -133,3 +133,50 @@ def test_unpadded_tiles_fp32_vs_unsplit_oracle(oracle, K, N, Cin, Cout, Ht, W):
         for r in range(K):
             assert rel_err(host(ys[r]), y_want[:, :, r * Ht:(r + 1) * Ht, :] + beta * host(y0[r])) <= 1e-5
             assert rel_err(host(gs[r]), gx_want[:, :, r * Ht:(r + 1) * Ht, :] + beta * host(g0[r])) <= 1e-5
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,Ht,W", [(1, 2, 8, 16, 5, 9), (2, 1, 19, 7, 6, 33), (4, 2, 9, 70, 1, 13), (3, 1, 24, 40, 23, 5),
+                                              (4, 32, 64, 64, 14, 56), (2, 8, 128, 128, 14, 28), (5, 1, 16, 8, 3, 150)])
+def test_unpadded_forward_with_residual(oracle, K, N, Cin, Cout, Ht, W):
+    """adh_conv3x3_unpadded_fwd_residual_tiles: y = conv(x, w) + res against the oracle's unsplit convolution plus the
+    same residual (rel-err <= 1e-5), and bit for bit against adh_conv3x3_unpadded_fwd_tiles with beta = 1 over a result
+    that holds the residual (the same kernel, the same order of additions) - with the residual in its own tensors and
+    with the result's tensors themselves as the residual."""
+    rng = np.random.default_rng(5300 + K * 13 + Cin)
+    H = K * Ht
+    x = rng.uniform(-1, 1, size=(N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))).astype(np.float32)
+    res = rng.standard_normal((N, Cout, H, W)).astype(np.float32)
+    xp = np.zeros((N, Cin, H + 2, W + 2), np.float32)
+    xp[:, :, 1:-1, 1:-1] = x
+    y_want = np.empty((N, Cout, H, W), np.float32)
+    oracle.conv_slab_fwd(xp, w, y_want)
+    y_want += res
+    xs = [dev(x[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    rs = [dev(res[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    kept = [t.clone() for t in rs]
+    ys = [torch.full_like(t, float("nan")) for t in rs]
+    capi.check(capi.conv_unpadded_fwd_residual_tiles(xs, dev(w), rs, ys, N, Cin, Cout, Ht, W), "fwd + residual")
+    by_beta = [t.clone() for t in rs]
+    capi.check(capi.conv_unpadded_fwd_tiles(xs, dev(w), by_beta, N, Cin, Cout, Ht, W, beta=1.0), "fwd, beta 1")
+    in_place = [t.clone() for t in rs]
+    capi.check(capi.conv_unpadded_fwd_residual_tiles(xs, dev(w), in_place, in_place, N, Cin, Cout, Ht, W), "fwd + residual, in place")
+    for r in range(K):
+        assert rel_err(host(ys[r]), y_want[:, :, r * Ht:(r + 1) * Ht, :]) <= 1e-5
+        assert torch.equal(ys[r], by_beta[r]) and torch.equal(ys[r], in_place[r])
+        assert torch.equal(rs[r], kept[r])  # the residual is read only
+
+
+def test_unpadded_forward_with_residual_rejects():
+    x = [torch.zeros(1, 8, 4, 16, device="cuda")]
+    y = [torch.zeros(1, 8, 4, 16, device="cuda")]
+    w = torch.zeros(8, 8, 3, 3, device="cuda")
+    xb, yb, wb = [t.bfloat16() for t in x], [t.bfloat16() for t in y], w.bfloat16()
+    assert capi.conv_unpadded_fwd_residual_tiles(xb, wb, yb, yb, 1, 8, 8, 4, 16) == capi.ADH_EUNIMPL  # fp32 only
+    from ctypes import c_void_p
+    tbl = (c_void_p * 1)(x[0].data_ptr())
+    nul = (c_void_p * 1)(None)
+    out = (c_void_p * 1)(y[0].data_ptr())
+    f = capi.lib().adh_conv3x3_unpadded_fwd_residual_tiles
+    assert f(capi.ADH_F32, 1, 1, 8, 8, 4, 16, tbl, w.data_ptr(), None, out, None) == capi.ADH_ENULL
+    assert f(capi.ADH_F32, 1, 1, 8, 8, 4, 16, tbl, w.data_ptr(), nul, out, None) == capi.ADH_ENULL
