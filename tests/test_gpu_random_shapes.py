@@ -478,3 +478,41 @@ def test_pool_over_tiles_without_halo_random(oracle, K, Ht, W, wh, ww, sh, sw, d
             else:
                 assert rel_err(host(ys[r]), want_y) <= 1e-5
             assert rel_err(host(gs[r]), g_want[:, :, r * Ht:(r + 1) * Ht, :]) <= 1e-5
+
+
+def _residual_cases(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        K = int(rng.integers(1, 6))
+        N = int(rng.integers(1, 5))
+        Cin, Cout = int(rng.integers(1, 97)), int(rng.integers(1, 97))
+        Ht, W = int(rng.integers(1, 20)), int(rng.integers(1, 70))
+        if N * (Cin + 2 * Cout) * K * Ht * W <= 3_000_000:
+            out.append((K, N, Cin, Cout, Ht, W))
+    return out
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,Ht,W", _residual_cases(2031, 24))
+def test_fp32_forward_with_residual_random(oracle, K, N, Cin, Cout, Ht, W):
+    """adh_conv3x3_unpadded_fwd_residual_tiles over random shapes: the unsplit convolution plus the residual (rel-err
+    <= 1e-5), and the same bits as beta = 1 over a result that holds the residual."""
+    rng = np.random.default_rng(Cin * 131 + Cout * 7 + K)
+    H = K * Ht
+    x = rng.uniform(-1, 1, size=(N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9))).astype(np.float32)
+    res = rng.standard_normal((N, Cout, H, W)).astype(np.float32)
+    xp = np.zeros((N, Cin, H + 2, W + 2), np.float32)
+    xp[:, :, 1:-1, 1:-1] = x
+    y_want = np.empty((N, Cout, H, W), np.float32)
+    oracle.conv_slab_fwd(xp, w, y_want)
+    y_want += res
+    xs = [dev(x[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    rs = [dev(res[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    ys = [torch.full_like(t, float("nan")) for t in rs]
+    capi.check(capi.conv_unpadded_fwd_residual_tiles(xs, dev(w), rs, ys, N, Cin, Cout, Ht, W), "fwd + residual")
+    by_beta = [t.clone() for t in rs]
+    capi.check(capi.conv_unpadded_fwd_tiles(xs, dev(w), by_beta, N, Cin, Cout, Ht, W, beta=1.0), "fwd, beta 1")
+    for r in range(K):
+        assert rel_err(host(ys[r]), y_want[:, :, r * Ht:(r + 1) * Ht, :]) <= 1e-5
+        assert torch.equal(ys[r], by_beta[r])
