@@ -38,6 +38,10 @@ CASES = [  # K, N, Cin, Cout, Ht, W, kh, kw, sh, sw, dh, dw, pad_h, pad_w
     (2, 2, 260, 16, 8, 32, 3, 3, 2, 2, 1, 1, 1, 1),   # 4x16 outputs, a last chunk of four input channels
     (3, 1, 256, 8, 16, 64, 3, 3, 2, 2, 1, 1, 1, 1),   # 8x32 outputs over three tiles: row -1 from the tile above
     (1, 1, 256, 8, 16, 16, 3, 3, 2, 2, 1, 1, 1, 1),   # 8x8 outputs on a single tile: zeros above
+    # many channels over few, full blocks of pixels: blocks of 64 output channels, the channel chunks dealt to 4 and 8 workgroups
+    (2, 16, 128, 64, 2, 8, 3, 3, 1, 1, 1, 1, 1, 1),   # 16 chunks of 8 channels in 4 parts
+    (2, 16, 256, 208, 2, 8, 3, 3, 1, 1, 1, 1, 1, 1),  # 32 chunks in 8 parts, 192 + 16 output channels; backward-data: 26 chunks in 4
+    (4, 4, 512, 64, 4, 16, 3, 3, 1, 1, 1, 1, 1, 1),   # 4x16 tiles, four images per block: 32 chunks of 16 channels in 8 parts
 ]
 
 
