@@ -272,7 +272,7 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_wgrad_kernel(const 
   float ypre[16], ppre[PJ];
   uint32_t y_ok = 0, p_ok = 0;
   auto load_chunk = [&](uint32_t ch) {
-    uint32_t q1, q2, q3, cc, rc, n, tile;
+    uint32_t q1, q2, cc, rc, n, tile;
     P.div_NCC.divmod(ch, q1, cc);
     P.div_NRC.divmod(q1, q2, rc);
     P.div_N.divmod(q2, tile, n);
