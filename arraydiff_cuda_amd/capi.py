@@ -58,6 +58,9 @@ SIGNATURES = {
     "adh_conv3x3_slab_bwd_filter_tiles": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp, f32, vp, sz, vp]),
     "adh_conv3x3_slab_bwd_filter_tiles_unexchanged": (i32, [i32, u32, u32, u32, u32, u32, u32, vpp, vpp, vp, f32, vp, sz,
                                                             vp]),
+    "adh_conv_bias_add_tiles": (i32, [i32, u32, u32, u32, u32, u32, vpp, vpp, vp]),
+    "adh_conv_bwd_bias_workspace_bytes": (sz, [u32, u32, u32]),
+    "adh_conv_bwd_bias_tiles": (i32, [i32, u32, u32, u32, u32, u32, vpp, vp, f32, vp, sz, vp]),
     "adh_conv2d_workspace_bytes": (sz, [i32, i32] + [u32] * 12),
     "adh_conv2d_slab_fwd_tiles": (i32, [i32] + [u32] * 12 + [vpp, vp, vpp, f32, vp, sz, vp]),
     "adh_conv2d_slab_bwd_data_tiles": (i32, [i32] + [u32] * 12 + [vp, vpp, vpp, f32, vp, sz, vp]),
@@ -309,6 +312,26 @@ def conv_unpadded_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, H, W, beta=0.0, ws
     wp, wb = _ws(ws)
     return lib().adh_conv3x3_unpadded_bwd_filter_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, H, W, xt, dt, dw.data_ptr(),
                                                        beta, wp, wb, _stream())
+
+
+def conv_bias_add_tiles(biases, ys, N, C, H, W):
+    """ys[t][n,c,h,w] += biases[t][c]; biases are fp32 vectors of C (entries may repeat)."""
+    _dev(*biases, *ys)
+    bt, k1 = _tbl(biases)
+    yt, k2 = _tbl(ys)
+    return lib().adh_conv_bias_add_tiles(_dt(ys[0]), len(ys), N, C, H, W, bt, yt, _stream())
+
+
+def conv_bwd_bias_workspace_bytes(K, N, C):
+    return lib().adh_conv_bwd_bias_workspace_bytes(K, N, C)
+
+
+def conv_bwd_bias_tiles(dys, db, N, C, H, W, beta=0.0, ws=None):
+    """db[c] = beta*db[c] + sum over tiles, n, h, w of dys[t][n,c,h,w]."""
+    _dev(db, *dys)
+    dt, k1 = _tbl(dys)
+    wp, wb = _ws(ws)
+    return lib().adh_conv_bwd_bias_tiles(_dt(dys[0]), len(dys), N, C, H, W, dt, db.data_ptr(), beta, wp, wb, _stream())
 
 
 def conv2d_workspace_bytes(which, dtype, K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw):

@@ -960,7 +960,9 @@ public:
 };
 
 // V = GPUBatchArray3D<float>, A = GPUArray4D<float> (filter, Shape4D(kw,kh,Cin,Cout) = KCRS).
-// Any window / stride / dilation, no bias.  With halo_padded_input the input's halo must equal the
+// Any window / stride / dilation; an optional bias per output channel (GPUArray1D<float>, one variable per rank
+// like the filter: y += bias after the conv, its gradient the sum of dy over images and pixels,
+// src/op.cc:1602-1610, 1632-1648).  With halo_padded_input the input's halo must equal the
 // conv pad (the padded tile is convolved with pad 0, src/op.cc:1392-1410); without it the input
 // must be packed and pad must be 0 (the 1x1 projections, src/zoo.cc:680-690).  Implicit zero
 // padding of an unpadded input is not part of this path and throws at construction.  3x3 /
@@ -972,10 +974,17 @@ public:
 template <typename V, typename A>
 class SlabConv2DOp : public virtual Op, public virtual Var<V> {
 public:
+  typedef GPUArray1D<float> Bias;
   static shared_ptr<Var<V>> Make(Conv2DShape shape, shared_ptr<Var<V>> input, shared_ptr<Var<A>> kernel,
                                  shared_ptr<Context> ctx) {
     return make_shared<SlabConv2DOp<V, A>>(shape, vector<shared_ptr<Var<V>>>{input},
                                            vector<shared_ptr<Var<A>>>{kernel}, ctx);
+  }
+  // the reference's constructor with a bias (op.hh:1828-1850): (shape, input, kernel, bias, ctx)
+  static shared_ptr<Var<V>> Make(Conv2DShape shape, shared_ptr<Var<V>> input, shared_ptr<Var<A>> kernel,
+                                 shared_ptr<Var<Bias>> bias, shared_ptr<Context> ctx) {
+    return make_shared<SlabConv2DOp<V, A>>(shape, vector<shared_ptr<Var<V>>>{input}, vector<shared_ptr<Var<A>>>{kernel},
+                                           ctx, vector<shared_ptr<Var<V>>>{}, vector<shared_ptr<Var<Bias>>>{bias});
   }
   // each rank holds its own copy of the filter in the reference; here kernels.at(r) may all be
   // the same variable, its gradient then accumulates over the tiles
@@ -986,17 +995,21 @@ public:
   // every other consumer of a residual must lie UPSTREAM of this node's input (the block input, whose other
   // consumer is the first node of the path that ends here) or the residual must have no other consumer (the
   // projection of a block that changes extents): those nodes then add to the shared buffer after this node has read it.
+  // biases: empty, or one variable of `filters` numbers per rank (with replicated_filters the ranks' biases are
+  // promised equal like their filters: rank 0's is added to every tile and receives every tile's gradient)
   static vector<shared_ptr<Var<V>>> MakeParallel(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs,
                                                  vector<shared_ptr<Var<A>>> kernels, shared_ptr<Context> ctx,
-                                                 vector<shared_ptr<Var<V>>> residuals = {}) {
-    auto op = make_shared<SlabConv2DOp<V, A>>(shape, inputs, kernels, ctx, residuals);
+                                                 vector<shared_ptr<Var<V>>> residuals = {},
+                                                 vector<shared_ptr<Var<Bias>>> biases = {}) {
+    auto op = make_shared<SlabConv2DOp<V, A>>(shape, inputs, kernels, ctx, residuals, biases);
     vector<shared_ptr<Var<V>>> outputs;
     for (size_t r = 0; r < inputs.size(); ++r) outputs.push_back(make_shared<NoOp<V>>(op, op->ys_.at(r).clone()));
     return outputs;
   }
   SlabConv2DOp(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs, vector<shared_ptr<Var<A>>> kernels,
-               shared_ptr<Context> ctx, vector<shared_ptr<Var<V>>> residuals = {})
-      : ctx_(ctx), shape_(shape), x_vars_(inputs), kernel_vars_(kernels), res_vars_(residuals) {
+               shared_ptr<Context> ctx, vector<shared_ptr<Var<V>>> residuals = {},
+               vector<shared_ptr<Var<Bias>>> biases = {})
+      : ctx_(ctx), shape_(shape), x_vars_(inputs), kernel_vars_(kernels), res_vars_(residuals), bias_vars_(biases) {
     if (shape.kernel[0] == 0 || shape.kernel[1] == 0 || shape.stride[0] == 0 || shape.stride[1] == 0 ||
         shape.dilate[0] == 0 || shape.dilate[1] == 0)
       throw std::invalid_argument("SlabConv2DOp: empty window, stride or dilation");
@@ -1022,6 +1035,14 @@ public:
       xs_.push_back(inputs[r]->data());
       kernels_.push_back(kernels[r]->data());
       ys_.push_back(VarData<V>(_get_output_shape(inputs[r]->shape(), inputs[r]->batch_shape()), inputs[r]->batch_shape()));
+    }
+    if (!biases.empty()) {
+      if (biases.size() != inputs.size()) throw std::invalid_argument("SlabConv2DOp: one bias variable per input");
+      for (size_t r = 0; r < biases.size(); ++r) {
+        if (biases[r]->shape() != Shape1D(shape.filters))
+          throw std::invalid_argument("SlabConv2DOp: a bias holds one number per filter");
+        biases_.push_back(biases[r]->data());
+      }
     }
     if (!residuals.empty()) {
       if (!shape.unpadded_tiles || residuals.size() != inputs.size())
@@ -1061,6 +1082,7 @@ public:
       for (size_t r = 0; r < x_vars_.size(); ++r) {
         x_vars_[r]->_push(e, apply);
         kernel_vars_[r]->_push(e, apply);
+        if (!bias_vars_.empty()) bias_vars_[r]->_push(e, apply);
       }
       apply(this);
     }
@@ -1069,6 +1091,7 @@ public:
     if (stack_.degree(e) == stack_.pop(e)) {
       apply(this);
       for (size_t r = x_vars_.size(); r-- > 0;) {
+        if (!bias_vars_.empty()) bias_vars_[r]->_pop(e, apply);
         kernel_vars_[r]->_pop(e, apply);
         x_vars_[r]->_pop(e, apply);
       }
@@ -1093,7 +1116,11 @@ private:
   vector<VarData<V>> ys_;
   vector<shared_ptr<Var<V>>> res_vars_;  // empty, or one per tile: added to the result
   vector<VarData<V>> res_;
+  vector<shared_ptr<Var<Bias>>> bias_vars_;  // empty, or one per rank
+  vector<VarData<Bias>> biases_;
+  void backward_bias(TxnId txn);
 };
+// the third parameter is the reference's bias array type; the bias here is always GPUArray1D<float>
 template <typename V, typename A, typename B = A>
 using CudnnConv2DOp = SlabConv2DOp<V, A>;
 

@@ -44,8 +44,9 @@ inline void parallel_vars_insert_all(vector<VarIdSet> &dst, const vector<VarIdSe
   for (size_t rank = 0; rank < dst.size(); ++rank) dst[rank].insert_all(src[rank]);
 }
 
-// One filter variable per rank, one node for all of them (src/zoo.cc:133-161).  The reference's
-// enable_bias is false wherever the spatial nets call this; a bias is not implemented.  The node is
+// One filter variable per rank, one node for all of them (src/zoo.cc:133-161).  enable_bias adds one bias
+// vector per rank, initialised to zeros, listed after the rank's filter in its parameter and gradient sets
+// (src/zoo.cc:111-120; the spatial nets enable it on their stem, src/zoo.cc:1548).  The node is
 // told that the copies are equal (Conv2DShape::replicated_filters), and they are from the start:
 // Op::init draws rank 0's values and hands every other rank a copy of them (the reference draws
 // each rank's own and the optimizer's first broadcast overwrites them, optimize.hh:283-300).
@@ -55,15 +56,16 @@ template <typename V, typename A = GPUArray4D<float>>
 ParallelParamOp<V> parallel_conv2d(Conv2DShape shape, vector<shared_ptr<Var<V>>> inputs,
                                    typename ParamOp<A>::InitFn kernel_init, bool enable_bias, shared_ptr<Context> ctx,
                                    vector<shared_ptr<Var<V>>> residuals = {}) {
-  if (enable_bias) throw std::invalid_argument("parallel_conv2d: bias is not implemented");
   // every rank's copy starts from rank 0's values (ParallelSGDOptimizer::reset) and receives the
   // same update: one launch serves all tiles
   shape.replicated_filters = true;
   MultiGPUContext *mgpu_ctx = mgpu_ctx_of(ctx);
   if (inputs.size() != mgpu_ctx->num_ranks()) throw std::invalid_argument("parallel_conv2d: one input per rank");
   const size_t cin = inputs.at(0)->shape().shape[2];
+  typedef GPUArray1D<float> B;
   ParallelParamOp<V> out;
   vector<shared_ptr<Var<A>>> kernels;
+  vector<shared_ptr<Var<B>>> biases;
   // the conv node visits rank 0's filter before the others (SlabConv2DOp::_push), so its values exist
   // when the copies are made
   auto drawn = make_shared<std::unique_ptr<A>>();
@@ -84,8 +86,15 @@ ParallelParamOp<V> parallel_conv2d(Conv2DShape shape, vector<shared_ptr<Var<V>>>
     kernels.push_back(kernel);
     out.params.push_back(VarIdSet::Singleton(kernel->vars().at(0)));
     out.grads.push_back(VarIdSet::Singleton(kernel->vars().at(1)));
+    if (enable_bias) {
+      // zeros on every rank: equal from the start, and the optimizer keeps them so
+      auto bias = ParamOp<B>::Make(Shape1D(shape.filters), zeros_init_gen<B>(), mgpu_ctx->device_context(rank));
+      biases.push_back(bias);
+      out.params.back().insert(bias->vars().at(0));
+      out.grads.back().insert(bias->vars().at(1));
+    }
   }
-  out.ops = CudnnConv2DOp<V, A, A>::MakeParallel(shape, inputs, kernels, ctx, residuals);
+  out.ops = CudnnConv2DOp<V, A, B>::MakeParallel(shape, inputs, kernels, ctx, residuals, biases);
   return out;
 }
 

@@ -483,6 +483,7 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
     const void *xt[ADH_MAX_TILES];
     void *yt[ADH_MAX_TILES];
     const void *rt[ADH_MAX_TILES];
+    const float *bt[ADH_MAX_TILES];
     uint32_t n = 0;
     TileDims d{}, yd{};
     vector<size_t> rest;
@@ -507,10 +508,16 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
         if (dims_of(res).N != d.N) throw HazardError("SlabConv2DOp: the residual's batch differs from the input's");
         rt[n] = res.as_view().dptr();
       }
+      if (!biases_.empty()) bt[n] = biases_[replicated ? 0 : r].val().get(txn, id()).dptr();
       ++n;
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
     GPUConn conn = dc->conn();
+    // y += bias once the convolution of this group is enqueued (cudnnAddTensor, op.cc:1602-1610)
+    auto add_bias = [&]() {
+      if (biases_.empty()) return;
+      adh_check(adh_conv_bias_add_tiles(ADH_F32, n, yd.N, yd.C, yd.H, yd.W, bt, yt, conn.stream()), "SlabConv2DOp::_forward (bias)");
+    };
     if (shape_.unpadded_tiles) {
       if (n != K) throw HazardError("SlabConv2DOp: tiles without halo need every rank in one pass");
       if (unpadded_3x3_kernels(*this, d, n, shape_.filters)) {
@@ -534,6 +541,7 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
                       "SlabConv2DOp::_forward (residual)");
         }
       }
+      add_bias();
       todo.swap(rest);
       continue;
     }
@@ -562,6 +570,73 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
                                           xt, w0, yt, 0.0f, ws, ws_bytes, conn.stream()),
                 "SlabConv2DOp::_forward (general)");
     }
+    add_bias();
+    todo.swap(rest);
+  }
+}
+
+// db += sum of dy over images and pixels (cudnnConvolutionBackwardBias, op.cc:1632-1648; zeroed on first touch and
+// accumulated with beta = 1 there, overwritten by the first toucher here).  Like the filter gradient: ranks that
+// share a gradient buffer are summed in one launch; with replicated parameters rank 0's variable receives every
+// tile's share and the other ranks' stay zero.
+template <>
+void SlabConv2DOp<V3, A4>::backward_bias(TxnId txn) {
+  const size_t K = xs_.size();
+  const bool replicated = shape_.replicated_filters;
+  vector<size_t> todo;
+  bool fresh[ADH_MAX_TILES] = {};
+  for (size_t r = 0; r < K; ++r) {
+    GPUContext *dc = rank_ctx(ctx_, r);
+    bool *fresh_r = &fresh[r];
+    const bool clear = replicated && r > 0 && !biases_[r].grad().known_zero();
+    if (biases_[r].grad().accumulate(txn, id(), dc, [dc, fresh_r, clear](Bias *g) {
+          *fresh_r = true;
+          if (clear) {
+            GPUConn conn = dc->conn();
+            g->set_constant(0.0f, conn);
+          }
+        })) {
+      todo.push_back(r);
+      if (replicated && r > 0 && fresh[r]) biases_[r].grad().declare_zero(txn, id());
+    }
+  }
+  for (size_t r = 0; r < K; ++r) {  // ranks whose variable was counted through a shared VarData still contribute
+    bool listed = false;
+    for (size_t q : todo) listed = listed || q == r;
+    if (!listed)
+      for (size_t q : todo)
+        if (biases_[q].grad().var() == biases_[r].grad().var()) {
+          todo.push_back(r);
+          break;
+        }
+  }
+  if (replicated && !todo.empty()) {
+    todo.clear();
+    for (size_t r = 0; r < K; ++r) todo.push_back(r);
+  }
+  while (!todo.empty()) {
+    float *db = biases_[replicated ? 0 : todo[0]].grad().get_mut(txn, id()).dptr();
+    const float beta = fresh[replicated ? 0 : todo[0]] ? 0.0f : 1.0f;
+    const void *dyt[ADH_MAX_TILES];
+    uint32_t n = 0;
+    TileDims yd{};
+    vector<size_t> rest;
+    for (size_t r : todo) {
+      if (!replicated && biases_[r].grad().get(txn, id()).dptr() != db) {
+        rest.push_back(r);
+        continue;
+      }
+      V3 &dy = ys_[r].grad().get(txn, id());
+      yd = dims_of(dy);
+      dyt[n++] = dy.as_view().dptr();
+    }
+    GPUContext *dc = rank_ctx(ctx_, todo[0]);
+    GPUConn conn = dc->conn();
+    dc->reserve_scratch(adh_conv_bwd_bias_workspace_bytes(n, yd.N, yd.C));
+    auto scratch = dc->get_scratch();
+    adh_check(adh_conv_bwd_bias_tiles(ADH_F32, n, yd.N, yd.C, yd.H, yd.W, dyt, db, beta, scratch->dptr(), scratch->size(),
+                                      conn.stream()),
+              "SlabConv2DOp::_backward (bias)");
     todo.swap(rest);
   }
 }
@@ -569,6 +644,7 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
 template <>
 void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
   const size_t K = xs_.size();
+  if (!biases_.empty()) backward_bias(txn);
   // filter gradient: dw += sum over the tiles that share the filter (zeroed on first touch,
   // op.cc:1651-1654; beta = 1, op.cc:1660-1671)
   // (the first toucher of a filter gradient overwrites it, beta = 0, instead of clearing it and adding; with
@@ -677,6 +753,9 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
   todo.clear();
   bool fresh[ADH_MAX_TILES] = {};
   bool reduce_after = false;  // unexchanged rows, but a kernel that cannot read across tiles: reduce once at the end
+  void *all_dx[ADH_MAX_TILES] = {};
+  size_t written = 0;
+  TileDims dx_dims{};
   for (size_t r = 0; r < K; ++r) {
     if (!x_vars_[r]->_requires_grad()) continue;  // e.g. the first layer: nobody wants the image's gradient
     GPUContext *dc = rank_ctx(ctx_, r);
@@ -707,6 +786,9 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
       d = dims_of(dx);
       dyt[n] = dy.as_view().dptr();
       dxt[n] = dx.base_as_view().dptr();
+      all_dx[r] = dxt[n];
+      dx_dims = d;
+      ++written;
       ++n;
     }
     GPUContext *dc = rank_ctx(ctx_, todo[0]);
@@ -732,7 +814,7 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
     const bool in_kernel_rows = n == K && reads_neighbour_rows(*this, shape_, d, n);
     if (shape_.unexchanged_rows && !in_kernel_rows) {
       // a halo reduce after this pass would add what the halo rows held before it a second time
-      if (!first || n != K) throw HazardError("SlabConv2DOp: unexchanged rows need the input gradient to themselves");
+      if (!first) throw HazardError("SlabConv2DOp: unexchanged rows need the input gradient to themselves");
       reduce_after = true;
     }
     if (in_kernel_rows) {
@@ -752,10 +834,16 @@ void SlabConv2DOp<V3, A4>::_backward(TxnId txn) {
                                                conn.stream()),
                 "SlabConv2DOp::_backward (data, general)");
     }
-    if (reduce_after)
-      adh_check(adh_halo_reduce_nchw(ADH_F32, 1, n, 1, d.W, d.H, d.C, d.N, dxt, conn.stream()),
-                "SlabConv2DOp::_backward (reduce)");
     todo.swap(rest);
+  }
+  if (reduce_after) {
+    // the mirror of the forward's single exchange: one reduce over all ranks' tiles once every group of ranks
+    // (one per distinct filter) has written its gradient tiles
+    if (written != K) throw HazardError("SlabConv2DOp: unexchanged rows need every rank's input gradient in one pass");
+    GPUConn conn = rank_ctx(ctx_, 0)->conn();
+    adh_check(adh_halo_reduce_nchw(ADH_F32, 1, (uint32_t)K, 1, dx_dims.W, dx_dims.H, dx_dims.C, dx_dims.N, all_dx,
+                                   conn.stream()),
+              "SlabConv2DOp::_backward (reduce)");
   }
 }
 

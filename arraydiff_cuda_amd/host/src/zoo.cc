@@ -49,7 +49,7 @@ ParallelCategoricalNLLBatchNormLoss<V1, F0> ResNet<float>::MakeParallelResNet18(
   Conv2DShape conv1_shape;
   conv1_shape.filters = 64; conv1_shape.axes = {0, 1}; conv1_shape.kernel = {7, 7}; conv1_shape.dilate = {1, 1};
   conv1_shape.stride = {1, 1}; conv1_shape.pad = {3, 3}; conv1_shape.halo_padded_input = true; conv1_shape.enable_hmma = false;
-  auto conv1 = parallel_conv2d<V3, A4>(conv1_shape, par_ys, xavier_init_gen<A4>(3 * 7 * 7, 64), false, parallel_ctx);
+  auto conv1 = parallel_conv2d<V3, A4>(conv1_shape, par_ys, xavier_init_gen<A4>(3 * 7 * 7, 64), true, parallel_ctx);  // with a bias, src/zoo.cc:1548
   parallel_vars_insert_all(net.dev_params, conv1.params);
   parallel_vars_insert_all(net.dev_grads, conv1.grads);
   par_ys = conv1.ops;

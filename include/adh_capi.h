@@ -257,6 +257,25 @@ int adh_conv3x3_slab_bwd_filter_tiles_unexchanged(int dtype, uint32_t num_tiles,
                                                   float *dw, float beta, void *workspace,
                                                   size_t workspace_bytes, void *stream);
 
+/* ---- convolution bias ------------------------------------------------------- */
+/* cudnnAddTensor(alpha = 1, bias_desc (1,C,1,1), beta = 1, y_desc) after the forward convolution of a
+ * CudnnConv2DOp built with a bias (src/op.cc:1602-1610; the stem of the spatial nets, src/zoo.cc:1548):
+ * y[n,c,h,w] += bias[c] over the K packed (N,C,H,W) result tiles in one launch.  Every rank of the
+ * reference holds its own bias vector: bias_tiles[t] is the fp32 vector of C added to y_tiles[t] (the
+ * entries may all be one pointer).  y is f32 or bf16 (sum in fp32, one rounding). */
+int adh_conv_bias_add_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H, uint32_t W,
+                            const float *const *bias_tiles, void *const *y_tiles, void *stream);
+/* cudnnConvolutionBackwardBias(alpha = 1, dy, beta, db) at src/op.cc:1632-1648:
+ * db[c] = beta*db[c] + sum_{tiles,n,h,w} dy[n,c,h,w], beta 0 or 1 (the reference zeroes db on first touch
+ * and passes 1); the sum over tiles is what ParallelSGDOptimizer's ncclReduce did across ranks
+ * (include/arraydiff/optimize.hh:443-451).  db is fp32.  The workspace (256-byte aligned,
+ * adh_conv_bwd_bias_workspace_bytes) holds partial sums that a second kernel adds in a fixed order:
+ * repeated calls give the same bits. */
+size_t adh_conv_bwd_bias_workspace_bytes(uint32_t num_tiles, uint32_t N, uint32_t C);
+int adh_conv_bwd_bias_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H, uint32_t W,
+                            const void *const *dy_tiles, float *db, float beta, void *workspace,
+                            size_t workspace_bytes, void *stream);
+
 /* ---- general window / stride / dilation over the halo-padded slab ------------ */
 /* The other consumers of halo-padded input (CudnnConv2DSize with halo_padded_input,
  * src/op.cc:1354-1410; the 7x7 stem src/zoo.cc:1528-1538, stride-2 3x3 src/zoo.cc:692-697, the

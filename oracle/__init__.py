@@ -286,6 +286,20 @@ def batchnorm2d_bwd(x, dy, scale, shift, save_mean, save_invstd, relu, p, dx, ds
                              ctypes.c_float(beta_param), _ptr(dx), _ptr(dscale), _ptr(dshift))
 
 
+def conv_bias_add(bias, y):
+    """y[n,c,h,w] += bias[c] in place; y is (N, C, H, W) float32."""
+    N, C, H, W = y.shape
+    assert bias.shape == (C,)
+    _lib.orc_conv_bias_add(_u32(N), _u32(C), _u32(H), _u32(W), _ptr(bias), _ptr(y))
+
+
+def conv_bwd_bias(dy, db, beta=0.0):
+    """db[c] = beta*db[c] + sum over n,h,w of dy[n,c,h,w]."""
+    N, C, H, W = dy.shape
+    assert db.shape == (C,)
+    _lib.orc_conv_bwd_bias(_u32(N), _u32(C), _u32(H), _u32(W), _ptr(dy), ctypes.c_float(beta), _ptr(db))
+
+
 def relu_fwd(x, y):
     _lib.orc_relu_fwd(ctypes.c_uint64(x.size), _ptr(x), _ptr(y))
 

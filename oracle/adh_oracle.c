@@ -28,6 +28,8 @@
  *   - general conv (any window / stride / dilation) : pinned against torch
  *     conv2d(stride, dilation) + autograd on the CPU and against the 3x3
  *     stride-1 functions above.
+ *   - convolution bias (add, backward-bias) : pinned against torch conv2d with a
+ *     bias + autograd on the CPU and numpy broadcasting / axis sums.
  *   - batch norm / rectifier / sum : pinned against torch batch_norm (training and
  *     evaluation) + relu + constant_pad + autograd on the CPU, and closed forms
  *     (normalised output has mean 0 / variance 1, dx sums to zero per channel).
@@ -552,6 +554,36 @@ void orc_conv2d_slab_bwd_filter(uint32_t N, uint32_t Cin, uint32_t Cout, uint32_
           size_t wi = ((co * (size_t)Cin + ci) * kh + a) * kw + b;
           dwt[wi] = (float)(acc + (beta != 0.0f ? (double)beta * dwt[wi] : 0.0));
         }
+}
+
+/* ------------------------------------------------------------------ */
+/* convolution bias                                                     */
+/* ------------------------------------------------------------------ */
+
+/* cudnnAddTensor(alpha = 1, bias_desc (1,C,1,1), beta = 1, y_desc) after the convolution
+ * (src/op.cc:1602-1610): y[n,c,h,w] += bias[c].  One rounding per element. */
+void orc_conv_bias_add(uint32_t N, uint32_t C, uint32_t H, uint32_t W, const float *bias, float *y) {
+  const size_t HW = (size_t)H * W;
+  for (uint32_t n = 0; n < N; ++n)
+    for (uint32_t c = 0; c < C; ++c) {
+      float *plane = y + ((size_t)n * C + c) * HW;
+      for (size_t i = 0; i < HW; ++i) plane[i] = plane[i] + bias[c];
+    }
+}
+
+/* cudnnConvolutionBackwardBias(alpha = 1, dy, beta, db) (src/op.cc:1632-1648; the reference
+ * zeroes db on first touch and passes beta = 1): db[c] = beta*db[c] + sum_{n,h,w} dy[n,c,h,w].
+ * Summed in double; cuDNN's order of additions is parity unpinned. */
+void orc_conv_bwd_bias(uint32_t N, uint32_t C, uint32_t H, uint32_t W, const float *dy, float beta, float *db) {
+  const size_t HW = (size_t)H * W;
+  for (uint32_t c = 0; c < C; ++c) {
+    double acc = 0.0;
+    for (uint32_t n = 0; n < N; ++n) {
+      const float *plane = dy + ((size_t)n * C + c) * HW;
+      for (size_t i = 0; i < HW; ++i) acc += plane[i];
+    }
+    db[c] = (float)(acc + (beta != 0.0f ? (double)beta * db[c] : 0.0));
+  }
 }
 
 /* ------------------------------------------------------------------ */

@@ -445,6 +445,102 @@ static void test_spatial_general_conv_graph(size_t K, size_t N, size_t C, size_t
   }
 }
 
+// The conv graph with what every rank of the reference owns for itself: a bias vector per rank (CudnnConv2DOp built
+// with a bias, src/op.cc:1602-1610, 1632-1648; distinct values per rank so that a tile given its neighbour's vector
+// shows) and, with rank_filters, a filter variable per rank (equal values, distinct buffers: one launch per rank, the
+// ranks' filter gradients add up to the unsplit one).  shared_bias: one bias variable for all ranks, whose gradient
+// is the sum over all tiles.  unexchanged: HaloExch2DOp copies nothing forward and the conv node exchanges (or reads
+// across tiles) itself; with rank_filters no single launch holds every tile, so it exchanges once before and reduces
+// once after the per-rank launches.
+static void test_spatial_conv_bias_graph(size_t K, size_t N, size_t C, size_t Co, size_t H, size_t W, size_t k, bool shared_bias,
+                                         bool rank_filters, bool unexchanged = false, bool halo_free = false) {
+  std::mt19937 gen(4321 + (unsigned)(K * 7 + k));
+  const size_t p = (k - 1) / 2, Ht = H / K;
+  auto ctx = MultiGPUContext::Make(K);
+  std::vector<float> X = uniform(gen, N * C * H * W, -1, 1);
+  std::vector<float> Wt = normal(gen, Co * C * k * k, std::sqrt(2.0f / (C * k * k)));
+  std::vector<float> dY = normal(gen, N * Co * H * W, 1.0f);
+  std::vector<std::vector<float>> Bv;
+  for (size_t r = 0; r < (shared_bias ? 1 : K); ++r) Bv.push_back(uniform(gen, Co, -1, 1));
+  typedef GPUBatchArray3D<float> V;
+  typedef GPUArray4D<float> A;
+  typedef GPUArray1D<float> B;
+  auto x_src = SrcOp<V>::Make(Shape3D(W, H, C), N, ctx->device_context(0));
+  vector<shared_ptr<ParamOp<A>>> w_srcs;
+  vector<shared_ptr<ParamOp<B>>> b_srcs;
+  vector<shared_ptr<Var<A>>> ws;
+  vector<shared_ptr<Var<B>>> bs;
+  for (size_t r = 0; r < K; ++r) {
+    if (r == 0 || rank_filters) w_srcs.push_back(ParamOp<A>::Make(Shape4D(k, k, C, Co), ctx->device_context(r)));
+    if (r == 0 || !shared_bias) b_srcs.push_back(ParamOp<B>::Make(Shape1D(Co), ctx->device_context(r)));
+    ws.push_back(w_srcs.back());
+    bs.push_back(b_srcs.back());
+  }
+  vector<shared_ptr<Var<V>>> xs(K, x_src);
+  auto tiles = SpatialScatter2DOp<V>::MakeParallel(xs, ctx);
+  vector<shared_ptr<Var<V>>> conv_in = tiles;
+  if (!halo_free) conv_in = HaloExch2DOp<V>::MakeParallel(p, HaloPad2DOp<V>::MakeParallel(p, tiles, ctx), ctx, unexchanged);
+  Conv2DShape cs;
+  cs.filters = Co;
+  cs.axes = {0, 1};
+  cs.kernel = {k, k};
+  cs.dilate = {1, 1};
+  cs.stride = {1, 1};
+  cs.pad = {p, p};
+  cs.halo_padded_input = !halo_free;
+  cs.unpadded_tiles = halo_free;
+  cs.unexchanged_rows = unexchanged;
+  cs.enable_hmma = false;
+  auto ys = CudnnConv2DOp<V, A, B>::MakeParallel(cs, conv_in, ws, ctx, {}, bs);
+  auto y_full = SpatialJoinedGather2DOp<V>::Make(ys, ctx);
+  auto sink = HostGradSinkOp<V>::Make(y_full, ctx->device_context(0));
+  sink->set_host_grad(dY.data());
+  for (int rep = 0; rep < 2; ++rep) {
+    TxnId txn;
+    x_src->load(txn, X.data());
+    for (auto &w : w_srcs) w->load(txn, Wt.data());
+    for (size_t r = 0; r < b_srcs.size(); ++r) b_srcs[r]->load(txn, Bv[r].data());
+    sink->gradient(txn);
+    ctx->sync();
+    std::vector<float> Y(dY.size()), dX(X.size()), dW(Wt.size(), 0.f), dWr_rank(Wt.size());
+    sink->store_val(txn, Y.data());
+    x_src->store_grad(txn, dX.data());
+    for (auto &w : w_srcs) {
+      w->store_grad(txn, dWr_rank.data());
+      for (size_t i = 0; i < dW.size(); ++i) dW[i] += dWr_rank[i];
+    }
+    const uint32_t HP = (uint32_t)(H + 2 * p), WP = (uint32_t)(W + 2 * p);
+    std::vector<float> Xp(N * C * HP * WP), Yr(Y.size()), dXp(Xp.size()), dXr(X.size()), dWr(Wt.size());
+    orc_halo_pad(0, (uint32_t)p, W, H, C, N, X.data(), Xp.data());
+    orc_conv2d_slab_fwd(N, C, Co, HP, WP, k, k, 1, 1, 1, 1, Xp.data(), Wt.data(), 0.f, Yr.data());
+    for (size_t n = 0; n < N; ++n)  // rows of tile r take rank r's bias
+      for (size_t c = 0; c < Co; ++c)
+        for (size_t h = 0; h < H; ++h)
+          for (size_t w = 0; w < W; ++w) Yr[((n * Co + c) * H + h) * W + w] += Bv[shared_bias ? 0 : h / Ht][c];
+    orc_conv2d_slab_bwd_data(N, C, Co, HP, WP, k, k, 1, 1, 1, 1, Wt.data(), dY.data(), 0.f, dXp.data());
+    orc_halo_unpad(0, (uint32_t)p, W, H, C, N, dXp.data(), dXr.data());
+    orc_conv2d_slab_bwd_filter(N, C, Co, HP, WP, k, k, 1, 1, 1, 1, Xp.data(), dY.data(), 0.f, dWr.data());
+    double eb = 0;
+    for (size_t r = 0; r < b_srcs.size(); ++r) {
+      std::vector<float> dB(Co), dBr(Co);
+      b_srcs[r]->store_grad(txn, dB.data());
+      for (size_t c = 0; c < Co; ++c) {
+        double a = 0;
+        for (size_t n = 0; n < N; ++n)
+          for (size_t h = shared_bias ? 0 : r * Ht; h < (shared_bias ? H : (r + 1) * Ht); ++h)
+            for (size_t w = 0; w < W; ++w) a += dY[((n * Co + c) * H + h) * W + w];
+        dBr[c] = (float)a;
+      }
+      eb = std::fmax(eb, rel_err(dB, dBr));
+    }
+    const double ey = rel_err(Y, Yr), ex = rel_err(dX, dXr), ew = rel_err(dW, dWr);
+    std::printf("conv + bias graph k=%zu K=%zu N=%zu C=%zu->%zu %zux%zu%s%s%s%s rep %d: rel-err y %.2e dx %.2e dw %.2e db %.2e\n", k,
+                K, N, C, Co, H, W, shared_bias ? " shared bias" : " bias per rank", rank_filters ? ", filter per rank" : "",
+                unexchanged ? ", unexchanged" : "", halo_free ? ", tiles without halo" : "", rep, ey, ex, ew, eb);
+    CHECK(ey <= 1e-5 && ex <= 1e-5 && ew <= 1e-5 && eb <= 1e-5);
+  }
+}
+
 // Scatter -> HaloPad(1) -> HaloExch(1) -> Pool(3x3, stride 2, pad 1, halo_padded_input) -> gather:
 // the stem pooling of src/zoo.cc:1562-1573 on K row-tiles of one GPU, against the oracle's pooling
 // of the zero-padded UNSPLIT tensor.
@@ -1040,6 +1136,13 @@ int main(int argc, char **argv) {
     test_spatial_general_conv_graph(4, 3, 3, 16, 32, 24, 7, 1, 1, true);   // the stem as the spatial net builds it (stride 1)
     test_spatial_general_conv_graph(4, 4, 24, 24, 16, 16, 3, 1, 1, true);  // 4x16 tiles: stride-1 3x3 through the general kernels
     test_spatial_general_conv_graph(4, 4, 16, 24, 8, 8, 3, 2, 1, true);    // 2x8 tiles at stride 2
+    test_spatial_conv_bias_graph(4, 3, 3, 16, 32, 24, 7, false, false);         // the stem's shape, a bias per rank
+    test_spatial_conv_bias_graph(4, 3, 3, 16, 32, 24, 7, true, false);          // one bias variable for all ranks
+    test_spatial_conv_bias_graph(2, 2, 8, 12, 40, 30, 3, false, true);          // 3x3, filter and bias per rank
+    test_spatial_conv_bias_graph(2, 2, 8, 12, 40, 30, 3, false, true, true);    // unexchanged rows + a filter per rank
+    test_spatial_conv_bias_graph(4, 2, 8, 16, 8, 12, 3, true, true, true);      // the same on small tiles (general kernels)
+    test_spatial_conv_bias_graph(4, 4, 64, 64, 56, 56, 3, true, false, true);   // one launch reads across tiles, then the bias
+    test_spatial_conv_bias_graph(4, 2, 8, 16, 32, 24, 3, false, false, false, true);  // tiles without halo
     test_spatial_residual_block(4, 2, 8, 16, 12);
     test_spatial_residual_block(2, 4, 64, 28, 28);
     test_spatial_residual_block(4, 2, 8, 16, 12, true);

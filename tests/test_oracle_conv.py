@@ -217,3 +217,41 @@ def test_general_conv_vs_torch(oracle, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh,
         dx3 = np.empty_like(dx)
         oracle.conv_slab_bwd_data(wt, dy, dx3)
         np.testing.assert_allclose(dx3, dx, rtol=0, atol=1e-6)
+
+
+@pytest.mark.parametrize("N,Cin,Cout,H,W,k", [(2, 3, 4, 5, 6, 3), (3, 2, 5, 4, 7, 1), (1, 3, 64, 6, 6, 7)])
+def test_conv_bias_vs_torch(oracle, N, Cin, Cout, H, W, k):
+    """cudnnAddTensor(bias) after the conv and cudnnConvolutionBackwardBias (src/op.cc:1602-1610,
+    1632-1648) against torch's conv2d with a bias and its autograd, and against numpy's
+    broadcasting / axis sums (neither reuses the oracle's loops)."""
+    rng = np.random.default_rng(12)
+    xp = rnd(rng, N, Cin, H + k - 1, W + k - 1)
+    wt = rnd(rng, Cout, Cin, k, k)
+    b = rnd(rng, Cout)
+    dy = rng.standard_normal((N, Cout, H, W)).astype(np.float32)
+    tb = torch.tensor(b, dtype=torch.float64, requires_grad=True)
+    ty = F.conv2d(torch.tensor(xp, dtype=torch.float64), torch.tensor(wt, dtype=torch.float64), bias=tb)
+    ty.backward(torch.tensor(dy, dtype=torch.float64))
+    y = np.empty((N, Cout, H, W), np.float32)
+    oracle.conv_slab_fwd(xp, wt, y)
+    y0 = y.copy()
+    oracle.conv_bias_add(b, y)
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=0, atol=3e-6)
+    assert np.array_equal(y, y0 + b[None, :, None, None])  # one rounding per element
+    db = np.full(Cout, np.nan, np.float32)
+    oracle.conv_bwd_bias(dy, db)
+    np.testing.assert_allclose(db, tb.grad.numpy(), rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(db, dy.astype(np.float64).sum(axis=(0, 2, 3)), rtol=1e-6, atol=1e-6)
+    db2 = db.copy()
+    oracle.conv_bwd_bias(dy, db2, beta=1.0)
+    np.testing.assert_allclose(db2, 2 * db, rtol=1e-6, atol=1e-6)
+    # a transposed (c, n) index or a dropped plane would change these closed forms
+    ones = np.ones((N, Cout, H, W), np.float32)
+    oracle.conv_bwd_bias(ones, db)
+    assert np.array_equal(db, np.full(Cout, N * H * W, np.float32))
+    hot = np.zeros((N, Cout, H, W), np.float32)
+    hot[N - 1, 1, H - 1, W - 1] = 3.0
+    oracle.conv_bwd_bias(hot, db)
+    want = np.zeros(Cout, np.float32)
+    want[1] = 3.0
+    assert np.array_equal(db, want)
