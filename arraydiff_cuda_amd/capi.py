@@ -81,6 +81,7 @@ SIGNATURES = {
     "adh_pool2d_slab_fwd": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, vp, vp, vp]),
     "adh_pool2d_slab_bwd_tiles": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, u32, vpp, vpp, vpp, vpp, f32, vp]),
     "adh_pool2d_slab_bwd": (i32, [i32, i32, u32, u32, u32, u32, u32, u32, u32, u32, vp, vp, vp, vp, f32, vp]),
+    "adh_pool2d_unpadded_supported": (i32, [i32, i32] + [u32] * 11),
     "adh_pool2d_unpadded_fwd_tiles": (i32, [i32, i32] + [u32] * 11 + [vpp, vpp, vp]),
     "adh_pool2d_unpadded_bwd_tiles": (i32, [i32, i32] + [u32] * 11 + [vpp, vpp, vpp, vpp, f32, vp]),
     "adh_softmax_fwd": (i32, [u32, u32, vp, vp, vp]),

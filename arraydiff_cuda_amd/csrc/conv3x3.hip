@@ -125,8 +125,10 @@ __global__ __launch_bounds__(64 * WAVES, PROWS == kPatchRowsShort ? 2 : 1) void 
   const uint64_t in_plane = (uint64_t)P.IH * P.IW;
   const uint64_t out_plane = (uint64_t)P.OH * P.OW;
   const float *__restrict__ in = P.in[t] + (uint64_t)n * P.Cred * in_plane;
-  float *__restrict__ out = P.out[t] + (uint64_t)n * P.Cout * out_plane;
-  const float *__restrict__ added = P.res[t] ? P.res[t] + (uint64_t)n * P.Cout * out_plane : out;
+  // `added` is `out` itself unless a residual is given, and a residual may be the result tensor: neither may be
+  // declared free of aliases (an element is read, then written, by the same lane)
+  float *out = P.out[t] + (uint64_t)n * P.Cout * out_plane;
+  const float *added = P.res[t] ? P.res[t] + (uint64_t)n * P.Cout * out_plane : out;
 
   const uint32_t rows_here = min(P.R, P.OH - oh0);
   const uint32_t cols_here = min(P.TW, P.OW - ow0);

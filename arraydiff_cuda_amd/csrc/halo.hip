@@ -259,16 +259,19 @@ __global__ __launch_bounds__(kBlock) void halo_strip_kernel(const StripParams P)
 }
 
 
-// Column strips through LDS, the measured alternative (built only with -DADH_HALO_COLUMNS_STAGED,
-// `make staged-columns`): a workgroup takes one plane of one neighbour pair, copies the source
+// Column strips through LDS: a workgroup takes one plane of one neighbour pair, copies the source
 // plane's interior rows into LDS as they lie in memory (contiguous 16-byte accesses instead of one
-// element per row and lane), and then moves the halo_pad columns out of LDS to their places.
+// element per row and lane), and then moves the halo_pad columns out of LDS to their places.  Only the
+// strip's own columns of the staged rows are used; what other workgroups write elsewhere in the
+// source plane meanwhile is staged but never used.
 // Measured against halo_strip_kernel<.., COLUMNS = true, 1> (N=32, C=64, fp32): 14-column tiles
 // 10.5 us against 9.7 (exchange) and 10.9 against 11.2 (reduce); 56-column tiles 31.0 against 19.0
-// and 38.8 against 27.1; halo 3 over 64 columns 15.8 against 12.6 and 16.3 against 19.7; and it
-// fetches 1.4 to 1.7 times the bytes, because a strip only needs the line of each row that holds
-// its column while the staging reads whole rows.  Every row of a column strip is its own line of
-// memory whatever the order it is asked for in, so the direct kernel is the default.
+// and 38.8 against 27.1; halo 3 over 64 columns 15.8 against 12.6 (exchange) and 16.3 against 19.7
+// (reduce).  It fetches 1.4 to 1.7 times the bytes, because a strip only needs the line of each row
+// that holds its column while the staging reads whole rows: every row of a column strip is its own
+// line of memory whatever the order it is asked for in.  It pays where several columns of a row are
+// read and written back (a reduce over a halo of two or more columns), and that is where halo_op
+// selects it; every other column strip takes the direct kernel.
 template <typename T, bool ADD>
 __global__ __launch_bounds__(kBlock) void halo_column_staged_kernel(const StripParams P) {
   extern __shared__ __attribute__((aligned(16))) uint8_t staged_rows[];
@@ -358,20 +361,13 @@ static int halo_op(bool reduce, int dtype, uint32_t grid_w, uint32_t grid_h, uin
   if (wide) P.run = W / vec;
   P.total = (uint32_t)(wide ? total / vec : total);
   P.div_run = FastDiv(P.run);
-#ifdef ADH_HALO_COLUMNS_STAGED
-  if (columns && (uint64_t)H * P.PW * dtype_size(dtype) <= 48u * 1024u && (uint64_t)C * N <= 0x7fffffffull) {
+  if (columns && reduce && p >= 2 && (uint64_t)H * P.PW * dtype_size(dtype) <= 48u * 1024u && (uint64_t)C * N <= 0x7fffffffull) {
     const dim3 sgrid(C * N, np, 1);
     const size_t lds_bytes = (size_t)H * P.PW * dtype_size(dtype);
-    if (dtype == ADH_F32) {
-      if (reduce) hipLaunchKernelGGL((halo_column_staged_kernel<float, true>), sgrid, dim3(kBlock), lds_bytes, st, P);
-      else hipLaunchKernelGGL((halo_column_staged_kernel<float, false>), sgrid, dim3(kBlock), lds_bytes, st, P);
-    } else {
-      if (reduce) hipLaunchKernelGGL((halo_column_staged_kernel<uint16_t, true>), sgrid, dim3(kBlock), lds_bytes, st, P);
-      else hipLaunchKernelGGL((halo_column_staged_kernel<uint16_t, false>), sgrid, dim3(kBlock), lds_bytes, st, P);
-    }
+    if (dtype == ADH_F32) hipLaunchKernelGGL((halo_column_staged_kernel<float, true>), sgrid, dim3(kBlock), lds_bytes, st, P);
+    else hipLaunchKernelGGL((halo_column_staged_kernel<uint16_t, true>), sgrid, dim3(kBlock), lds_bytes, st, P);
     return launch_status();
   }
-#endif
   dim3 grid((P.total + kBlock - 1) / kBlock, np * p, 1);
   if (grid.y > 65535u) return ADH_EINVAL;
 #define ADH_LAUNCH_STRIP(T, ADD, COL, V) \

@@ -743,6 +743,23 @@ int adh_pool2d_slab_bwd(int dtype, int mode, uint32_t N, uint32_t C, uint32_t HP
   return adh_pool2d_slab_bwd_tiles(dtype, mode, 1, N, C, HP, WP, wh, ww, sh, sw, xs, ys, dys, dxs, beta, stream);
 }
 
+int adh_pool2d_unpadded_supported(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H, uint32_t W,
+                                  uint32_t wh, uint32_t ww, uint32_t sh, uint32_t sw, uint32_t pad_h, uint32_t pad_w) {
+  PoolParams P = {};
+  int e = pool_check_unpadded(dtype, mode, num_tiles, N, C, H, W, wh, ww, sh, sw, pad_h, pad_w, &P);
+  if (e) return e;
+  if (N == 0 || C == 0) return ADH_OK;
+  const size_t es = dtype_size(dtype);
+  const bool is_max = mode == ADH_POOL_MAX;
+  if (!pick_band_rows(P, num_tiles, kPoolBandBytes, [&](uint32_t r) { return fwd_band_lds(P, es, r); })) return ADH_EUNIMPL;
+  e = pool_unpadded_bwd_rows(&P);
+  if (e) return e;
+  if (wh * ww > 256u ||
+      !pick_band_rows(P, num_tiles, bwd_band_aim(P, es, is_max), [&](uint32_t r) { return bwd_band_lds(P, es, is_max, r); }))
+    return ADH_EUNIMPL;
+  return ADH_OK;
+}
+
 int adh_pool2d_unpadded_fwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H, uint32_t W,
                                   uint32_t wh, uint32_t ww, uint32_t sh, uint32_t sw, uint32_t pad_h, uint32_t pad_w,
                                   const void *const *x_tiles, void *const *y_tiles, void *stream) {

@@ -58,7 +58,12 @@ ParallelCategoricalNLLBatchNormLoss<V1, F0> ResNet<float>::MakeParallelResNet18(
   Pool2DShape pool1_shape;
   pool1_shape.pooling = kMaxPool; pool1_shape.axes = {0, 1}; pool1_shape.window = {3, 3}; pool1_shape.stride = {2, 2};
   pool1_shape.pad = {1, 1}; pool1_shape.halo_padded_input = true;
-  if (mgpu_ctx->spatial_comm(0)->num_w_ranks == 1 && par_ys.at(0)->shape().shape[1] % 2 == 0) {
+  const auto stem_tile = par_ys.at(0)->shape();
+  // (very wide images: a band of window rows no longer fits LDS and the kernels over tiles without halo decline;
+  // the padded form below has direct kernels for such rows)
+  if (mgpu_ctx->spatial_comm(0)->num_w_ranks == 1 && stem_tile.shape[1] % 2 == 0 &&
+      adh_pool2d_unpadded_supported(ADH_F32, ADH_POOL_MAX, (uint32_t)num_ranks, (uint32_t)cfg.batch_size, (uint32_t)stem_tile.shape[2],
+                                    (uint32_t)stem_tile.shape[1], (uint32_t)stem_tile.shape[0], 3, 3, 2, 2, 1, 1) == ADH_OK) {
     // over row tiles the pooling reads its zero padding and its neighbours' rows itself: no pad, no exchange, and
     // the stem's output gradient comes out unpadded (two passes over the largest activation of the net fewer)
     pool1_shape.halo_padded_input = false;

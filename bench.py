@@ -29,13 +29,24 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# HBM bytes per conv-forward launch measured with rocprofv3 PMC (FETCH_SIZE and WRITE_SIZE, each
-# scaled by what the same counter reads for a 1 GiB plain copy); the summaries with the commands
-# are profiles/conv3x3_bf16_fwd_cfg5_hbm_traffic.txt and profiles/conv3x3_fwd_cfg2_hbm_traffic.txt.
-# Not re-measured by this script; each figure belongs to the kernel instance named beside it and is
-# left out (null) when the library routes the shape to another instance.
-CONV_FWD_CFG5_TRAFFIC = ("conv3x3_bf16_w8_kernel<false, false, false, false>", 1085.7e6)
-CONV_FWD_CFG2_TRAFFIC = ("conv3x3_f32_kernel<25, 8, false, 12>", 64.07e6)
+# HBM bytes per launch of a kernel instance, measured with rocprofv3 PMC (FETCH_SIZE and WRITE_SIZE, each scaled
+# by what the same counter reads for a 1 GiB plain copy).  Not re-measured by this script: the figures are read
+# from the committed summaries under profiles/ (lines `traffic_bytes_per_launch[<kernel instance>] = <bytes>`),
+# each belongs to the kernel instance named in its brackets, and an instance without such a line (the library
+# routes the shape elsewhere, or the kernel changed its name) reports null.
+def measured_traffic():
+    import glob
+    import re
+    found = {}
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*_hbm_traffic.txt"))):
+        with open(path) as f:
+            for line in f:
+                m = re.match(r"traffic_bytes_per_launch\[(.+)\] = ([0-9.eE+]+)", line.strip())
+                if m:
+                    found[m.group(1)] = (float(m.group(2)), os.path.relpath(path, ROOT))
+    return found
+
+
 CLOCK_RAMP_MS = 150.0
 HBM_PEAK_GBS = 8000.0
 MFMA_F32_PEAK_TFLOPS = 157.3
@@ -153,6 +164,27 @@ def main():
         else:
             print("bench.py: the graph-replay run of the trainer failed:\n" + g.stdout[-1000:] + g.stderr[-1000:], file=sys.stderr)
 
+    # The reference's own microbenchmarks (tools/microbench_spatial.cc, tools/microbench_spatial_conv.cc) as a C++
+    # binary over this library's Spatial2DComm and C ABI, also a child process: per rank group_start / halo_* /
+    # group_end with the reference's synchronisations, beside one launch for all ranks' tiles; wall-clock averages.
+    reference_microbench = None
+    micro = os.path.join(ROOT, "arraydiff_cuda_amd", "microbench_spatial")
+    if not args.no_secondary and not args.no_end_to_end and args.only is None:
+        import subprocess
+        if not os.path.exists(micro):
+            print("bench.py: %s is not built (run __graft_entry__.build())" % micro, file=sys.stderr)
+            sys.exit(3)
+        reference_microbench = []
+        for which, trials in (("spatial", "1000"), ("spatial_conv", "100")):
+            r = subprocess.run([micro, "--which", which, "--ranks", "4", "--trials", trials], capture_output=True, text=True,
+                               timeout=600)
+            if r.returncode != 0:
+                print("bench.py: microbench_spatial --which %s failed:\n" % which + r.stdout[-2000:] + r.stderr[-2000:],
+                      file=sys.stderr)
+                sys.exit(4)
+            lines = [json.loads(l) for l in r.stdout.strip().splitlines()]
+            reference_microbench += [l for l in lines if "name" in l]
+
     import numpy as np
     import torch
     from arraydiff_cuda_amd import capi
@@ -214,6 +246,7 @@ def main():
     value = flops5 / (ms_per_step * 1e-3) / 1e12
     achieved = flops5 / (kernel_ms * 1e-3) / 1e12
     name5 = capi.conv_kernel_name(capi.ADH_CONV_FWD, capi.ADH_BF16, K5, N5, C, C, Ht5, W5)
+    traffic = measured_traffic()
     in5_b = K5 * N5 * C * (Ht5 + 2) * (W5 + 2) * 2
     out5_b = N5 * C * H5 * W5 * 2
     ai5 = flops5 / (in5_b + out5_b + C * C * 9 * 2)
@@ -228,7 +261,7 @@ def main():
         "roofline": {"kernel": name5 + " (fwd; the only kernel of the call: it reads the filter as the caller holds it)", "bound": "mfma",
                      "achieved": round(achieved, 3), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": CONV_FWD_CFG5_TRAFFIC[1] if name5 == CONV_FWD_CFG5_TRAFFIC[0] else None,
+                     "traffic": traffic.get(name5, (None, None))[0], "traffic_source": traffic.get(name5, (None, None))[1],
                      "launch_ms": round(kernel_ms, 5),
                      "compulsory_bytes": in5_b + out5_b + C * C * 9 * 2,
                      "min_mfma_hbm_bound_TFLOPs": round(min(MFMA_BF16_PEAK_TFLOPS, HBM_PEAK_GBS * ai5 / 1e3), 1)},
@@ -324,7 +357,7 @@ def main():
             lambda: lib.adh_conv3x3_slab_fwd_tiles(capi.ADH_F32, K, N, C, C, Ht, W, tile_tbl, wt.data_ptr(), y_tbl, 0.0,
                                                    None, 0, stream),
             "mfma", flops_step, MFMA_F32_PEAK_TFLOPS, "TFLOP/s",
-            extra={"kernel": name2, "traffic": CONV_FWD_CFG2_TRAFFIC[1] if name2 == CONV_FWD_CFG2_TRAFFIC[0] else None})
+            extra={"kernel": name2, "traffic": traffic.get(name2, (None, None))[0]})
         reps, wu = 200, 20
         add("halo pack cfg1 (unsplit -> 4 padded tiles)",
             lambda: lib.adh_tiles_pack_nchw(0, K, p, W, H, C, N, X.data_ptr(), tile_tbl, stream),
@@ -753,7 +786,37 @@ def main():
             "hbm", (K + 2 + 3) * pdim * 4.0, HBM_PEAK_GBS, "GB/s", flushed=True,
             note="reads 4 gradient vectors + parameters + momentum, writes momentum + parameters + lagged copy")
         del p_arrays, flat_g, flush_scratch
+        if reference_microbench is not None:
+            # wall-clock milliseconds per trial of the reference's call sequence (synchronisations included), beside
+            # the same work as one launch for all tiles; the device-event figures of the one-launch forms are the
+            # "reference microbench_*" entries above
+            for m in reference_microbench:
+                m = dict(m)
+                m["name"] = "reference microbench_%s through Spatial2DComm (C++ binary, 4 ranks, wall clock): %s" % (
+                    m.pop("which"), m["name"])
+                sec.append(m)
         out["secondary"] = sec
+        # The halo half of the metric inside `roofline`: pack / unpack at the headline configuration (1.08 GB per
+        # launch, four times the on-package cache: the sustained HBM rate) and at cfg1 (56 MB: `warm` has its operands
+        # resident in the on-package cache, `flushed` reads 512 MB of something else before every launch).
+        by_name = {e["name"]: e for e in sec}
+
+        def halo_entry(name):
+            e = by_name.get(name)
+            if e is None:
+                return None
+            h = {"ms": e["ms"], "GBs": e["achieved"], "frac": e["frac"], "bytes": e["work"]}
+            if "ms_flushed" in e:
+                h = {"warm": h, "flushed": {"ms": e["ms_flushed"], "GBs": e["achieved_flushed"], "frac": e["frac_flushed"],
+                                            "bytes": e["work"]}}
+            return h
+
+        out["roofline"]["halo"] = {
+            "bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "pack_cfg5": halo_entry("halo pack cfg5 (bf16, 8 tiles of 128 rows)"),
+            "unpack_cfg5": halo_entry("halo unpack cfg5 (bf16)"),
+            "pack_cfg1": halo_entry("halo pack cfg1 (unsplit -> 4 padded tiles)"),
+            "unpack_cfg1": halo_entry("halo unpack cfg1 (4 padded tiles -> unsplit)")}
     if end_to_end is not None:
         out["end_to_end"] = end_to_end
 

@@ -19,7 +19,11 @@
  * include/arraydiff/array_gpu.hh:544-548).  Pointer tables (`void* const*`) are
  * HOST arrays of DEVICE pointers; they are read before the call returns.
  *
- * Re-entrant, no global state, callable from any host thread.
+ * Re-entrant and callable from any host thread: a call reads its arguments and enqueues work, and
+ * nothing a call leaves behind changes the result of another.  The library's only process-wide state
+ * is two caches filled on first use, the current device's compute-unit count (the persistent kernels'
+ * grid size) and the per-device address of the scratch array of adh_conv3x3_slab_fwd_tiles_static;
+ * that one entry point shares its scratch between calls and is the exception noted where it is declared.
  */
 #ifndef ADH_CAPI_H
 #define ADH_CAPI_H
@@ -437,6 +441,11 @@ int adh_pool2d_slab_bwd(int dtype, int mode, uint32_t N, uint32_t C, uint32_t HP
  * wh - 1 - pad_h <= H (windows, the neighbours' too, touch adjacent tiles only; ADH_EINVAL otherwise); a band
  * of window rows must fit in LDS (rows of up to a few thousand elements; ADH_EUNIMPL beyond: use the padded entry
  * points).  y_tiles of the backward call is not read (the maximum is recomputed) and may be NULL. */
+/* ADH_OK when both calls below take this shape, else the code they would return (ADH_EINVAL: the row split does
+ * not stitch; ADH_EUNIMPL: a band of window rows does not fit LDS), without launching anything: for callers that
+ * choose between this form and pad -> exchange -> pooling over padded tiles when they build a graph. */
+int adh_pool2d_unpadded_supported(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H, uint32_t W,
+                                  uint32_t wh, uint32_t ww, uint32_t sh, uint32_t sw, uint32_t pad_h, uint32_t pad_w);
 int adh_pool2d_unpadded_fwd_tiles(int dtype, int mode, uint32_t num_tiles, uint32_t N, uint32_t C, uint32_t H,
                                   uint32_t W, uint32_t wh, uint32_t ww, uint32_t sh, uint32_t sw, uint32_t pad_h,
                                   uint32_t pad_w, const void *const *x_tiles, void *const *y_tiles, void *stream);

@@ -51,3 +51,9 @@ def test_argument_errors_need_no_gpu():
     assert l.adh_softmax_fwd(10, 2, None, bogus, None) == capi.ADH_ENULL
     assert l.adh_fill_f32(0, 1.0, None, None) == capi.ADH_OK                                       # empty
     assert l.adh_softmax_fwd(0, 0, None, None, None) == capi.ADH_OK
+    # the shape query of the pooling over tiles without halo launches nothing
+    q = l.adh_pool2d_unpadded_supported
+    assert q(0, capi.ADH_POOL_MAX, 4, 32, 64, 64, 256, 3, 3, 2, 2, 1, 1) == capi.ADH_OK        # the stem's pooling
+    assert q(0, capi.ADH_POOL_MAX, 4, 32, 64, 64, 8192, 3, 3, 2, 2, 1, 1) == capi.ADH_EUNIMPL  # rows too wide for a band in LDS
+    assert q(0, capi.ADH_POOL_MAX, 4, 32, 64, 63, 256, 3, 3, 2, 2, 1, 1) == capi.ADH_EINVAL    # the row split does not stitch
+    assert l.adh_conv_bwd_bias_workspace_bytes(4, 32, 64) > 0

@@ -126,6 +126,13 @@ def test_conv_error_codes():
     assert capi.conv_bwd_filter_tiles([x], [y], dw, 1, 4, 4, 3, 3, ws=small) == capi.ADH_EWORKSPACE
 
 
+def assert_close_elementwise(got, ref):
+    """Every element on its own: the max-norm bar alone would pass a 1 % error on an output that is a thousandth
+    of the largest.  rtol 1e-4 with an absolute floor of 1e-5 of the largest reference value (sums of 576 and
+    more products that cancel towards zero keep the absolute error of their terms)."""
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5 * float(np.max(np.abs(ref))))
+
+
 def _config(rng, K=4, N=32, C=64, H=56, W=56):
     X = rng.uniform(-1, 1, size=(N, C, H, W)).astype(np.float32)
     w = he_normal(rng, C, C)
@@ -147,6 +154,7 @@ def test_config2_fwd_stitched_vs_unsplit(oracle):
     Y = torch.cat(ys, dim=2)
     ref = F.conv2d(torch.from_numpy(X).double(), torch.from_numpy(w).double(), padding=1).numpy()
     assert rel_err(host(Y), ref) <= TOL
+    assert_close_elementwise(host(Y), ref)
     # the oracle agrees on one full tile (scalar fp64 accumulate)
     want = np.empty((N, C, Ht, W), np.float32)
     oracle.conv_slab_fwd(host(tiles[1]), w, want)
@@ -178,10 +186,12 @@ def test_config3_fwd_bwd_vs_unsplit(oracle):
     gX = torch.empty_like(dX)
     capi.check(capi.tiles_unpack(K, p, W, H, C, N, gs, gX))
     assert rel_err(host(gX), tX.grad.numpy()) <= TOL
+    assert_close_elementwise(host(gX), tX.grad.numpy())
     ws = workspace(capi.ADH_CONV_BWD_FILTER, K, N, C, C, Ht, W)
     gw = torch.zeros_like(dw)
     capi.check(capi.conv_bwd_filter_tiles(tiles, dys, gw, N, C, C, Ht, W, beta=1.0, ws=ws))
     assert rel_err(host(gw), tw.grad.numpy()) <= TOL
+    assert_close_elementwise(host(gw), tw.grad.numpy())
     # oracle on one image of one tile (scalar fp64)
     want = np.zeros((1, C, Ht + 2, W + 2), np.float32)
     oracle.conv_slab_bwd_data(w, host(dys[1])[:1].copy(), want)

@@ -76,11 +76,15 @@ def test_halo_exchange_reduce_vs_oracle(oracle, K, p, Ht, W, C, N, dtype, which)
         np.testing.assert_array_equal(host(d2[r]), want[r])
 
 
+# a reduce over a halo of two or more columns runs the LDS-staged kernel (planes of up to 48 KB), every other
+# case the direct one: (2, 2, ...), (2, 3, ...) and (3, 2, ...) cover the former, the 200-row planes exceed 48 KB
+@pytest.mark.parametrize("dtype", [np.float32, np.uint16])
 @pytest.mark.parametrize("which", ["exch", "reduce"])
-@pytest.mark.parametrize("Kw,p,H,Wt,C,N", [(2, 1, 5, 4, 3, 2), (2, 2, 6, 7, 2, 2), (4, 1, 3, 5, 2, 1)])
-def test_column_halos_vs_oracle(oracle, Kw, p, H, Wt, C, N, which):
+@pytest.mark.parametrize("Kw,p,H,Wt,C,N", [(2, 1, 5, 4, 3, 2), (2, 2, 6, 7, 2, 2), (4, 1, 3, 5, 2, 1), (2, 3, 9, 64, 4, 2),
+                                           (3, 2, 33, 14, 5, 3), (2, 2, 200, 60, 2, 1)])
+def test_column_halos_vs_oracle(oracle, Kw, p, H, Wt, C, N, which, dtype):
     rng = np.random.default_rng(300)
-    tiles = rand_tiles(rng, Kw, N, C, H + 2 * p, Wt + 2 * p, np.float32)
+    tiles = rand_tiles(rng, Kw, N, C, H + 2 * p, Wt + 2 * p, dtype)
     want = [t.copy() for t in tiles]
     code = oracle.EXCH if which == "exch" else oracle.REDUCE
     assert oracle.halo_op(code, Kw, 1, p, Wt, H, C, N, want) == 0

@@ -32,11 +32,14 @@ def _run_pair(K, N, Cin, Cout, H, W, seed, beta=0.0):
     capi.check(lib.adh_conv3x3_slab_fwd_tiles(capi.ADH_BF16, K, N, Cin, Cout, H, W, x_tbl, w.data_ptr(), a_tbl, beta,
                                               ws.data_ptr(), ws_bytes, st), "fwd with workspace")
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # torch's own counter sees only torch's caching allocator; the driver's free-memory figure also sees what the
+    # library itself would take with hipMalloc and keep
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     capi.check(lib.adh_conv3x3_slab_fwd_tiles_static(capi.ADH_BF16, K, N, Cin, Cout, H, W, x_tbl, w.data_ptr(), b_tbl,
                                                      beta, st), "fwd, static scratch")
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     for r in range(K):
         a, b = ya[r].view(torch.int16).cpu().numpy(), yb[r].view(torch.int16).cpu().numpy()
         assert not np.array_equal(a, y0[r].view(torch.int16).cpu().numpy())  # something was computed
@@ -44,6 +47,10 @@ def _run_pair(K, N, Cin, Cout, H, W, seed, beta=0.0):
 
 
 def test_static_scratch_forward_matches_workspace_forward():
+    # fewer than 64 input channels: the filter is reordered into the scratch array (a 64-channel filter at an
+    # aligned address is read in place), and 256 output channels write and read all 294,912 bytes of it
+    print("static scratch: 2 tiles, N=2, 48->256 channels, 12x136", flush=True)
+    _run_pair(2, 2, 48, 256, 12, 136, seed=14)
     print("static scratch: 2 tiles, N=2, 64->200 channels, 12x136", flush=True)
     _run_pair(2, 2, 64, 200, 12, 136, seed=11)
     print("static scratch: second call, smaller: 1 tile, N=1, 24->40 channels, 5x24", flush=True)
