@@ -581,6 +581,6 @@ def softmax_xent_fwd_bwd(x, label, dloss, dloss_all, y, loss, beta, dx):
 
 def conv_kernel_name(which, dtype, K, N, Cin, Cout, H, W, beta=0.0):
     """Name of the kernel instance a 3x3 forward / backward-data call of this shape runs."""
-    buf = ctypes.create_string_buffer(128)
-    check(lib().adh_conv3x3_kernel_name(which, dtype, K, N, Cin, Cout, H, W, beta, buf, 128), "kernel name")
+    buf = ctypes.create_string_buffer(256)
+    check(lib().adh_conv3x3_kernel_name(which, dtype, K, N, Cin, Cout, H, W, beta, buf, 256), "kernel name")
     return buf.value.decode()

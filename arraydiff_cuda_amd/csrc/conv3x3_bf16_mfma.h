@@ -30,7 +30,10 @@ struct ConvBf16Params {
   // More than 64 reduction channels take one launch per 64 (a pass): the pass multiplies channels
   // chan0 .. chan0 + cred_pass - 1 and hands its sums to the next one as fp32 in `part`
   // ([image][output channel][row][column] per tile); the last pass rounds to bf16 into `out`.
-  uint32_t pass, passes, chan0, cred_pass;
+  // (`pass` counts in 64 channels, the unit of the transformed filter's layout; the kernel of
+  // conv3x3_bf16_k128.hip multiplies two such units per launch.  first_pass / last_pass: this launch reads no
+  // sums / rounds to bf16.)
+  uint32_t pass, passes, chan0, cred_pass, first_pass, last_pass;
   float *part[ADH_MAX_TILES];
   // the eight-wave kernel reads the filter as the caller holds it (no transformed copy): forward, a
   // multiple of 64 input channels, 16-byte aligned; else null
@@ -62,8 +65,13 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 
 // the eight-wave kernel: shapes it takes, and its launch (grid.x workgroups per output group)
 bool conv_bf16_w8_takes(const ConvBf16Params &P, uint32_t num_tiles);
-// launches pass P.pass of P.passes
+// launches the pass of up to 64 reduction channels from P.chan0 on
 int conv_bf16_w8_launch(const ConvBf16Params &P, uint32_t gx, uint32_t groups, hipStream_t st);
+// the kernel for more than 64 reduction channels (128 per pass, 128 output channels per workgroup, 32-column
+// strips): shapes it takes, and its launch (grid.x workgroups per group of 128 output channels)
+constexpr int kStripColsK128 = 32;
+bool conv_bf16_k128_takes(const ConvBf16Params &P, uint32_t num_tiles);
+int conv_bf16_k128_launch(const ConvBf16Params &P, uint32_t gx, uint32_t groups128, hipStream_t st);
 
 }  // namespace adh
 

@@ -509,11 +509,30 @@ bool conv_bf16_mfma_supported(int which, uint32_t Cin, uint32_t Cout, uint32_t H
 static uint32_t conv_bf16_passes(int which, uint32_t Cin, uint32_t Cout) {
   return ((which == ADH_CONV_FWD ? Cin : Cout) + 63u) / 64u;
 }
+// More than 64 reduction AND more than 64 output channels: launches of 128 reduction channels by the kernel of
+// conv3x3_bf16_k128.hip while more than 64 are left, then at most 64 by the eight-wave kernel.  Otherwise one
+// launch of the eight-wave kernel per 64.
+static bool conv_bf16_uses_k128(int which, uint32_t Cin, uint32_t Cout) { return Cin > 64u && Cout > 64u; }
+static uint32_t conv_bf16_launches(int which, uint32_t Cin, uint32_t Cout) {
+  const uint32_t cred = which == ADH_CONV_FWD ? Cin : Cout;
+  if (!conv_bf16_uses_k128(which, Cin, Cout)) return (cred + 63u) / 64u;
+  uint32_t n = 0, rem = cred;
+  while (rem > 64u) {
+    rem -= rem < 128u ? rem : 128u;
+    ++n;
+  }
+  return n + (rem ? 1u : 0u);
+}
 
 // name of the kernel a bf16 forward / backward-data call over padded tiles runs, for tiles aligned to 16 bytes
 // (template arguments: old output added, sums of earlier passes read, sums written for a later pass, tiles without halo)
 const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, float beta) {
   if (!conv_bf16_mfma_supported(which, Cin, Cout, H, W)) return "widen_bf16_kernel + conv3x3_f32_kernel + narrow_bf16_kernel";
+  if (conv_bf16_uses_k128(which, Cin, Cout)) {
+    if (conv_bf16_launches(which, Cin, Cout) == 1u)
+      return beta != 0.f ? "conv3x3_bf16_k128_kernel<true, false, false, false>" : "conv3x3_bf16_k128_kernel<false, false, false, false>";
+    return "conv3x3_bf16_k128_kernel per 128 reduction channels (fp32 sums between the launches) + conv3x3_bf16_w8_kernel for a rest of at most 64";
+  }
   if (conv_bf16_passes(which, Cin, Cout) > 1u)
     return beta != 0.f ? "conv3x3_bf16_w8_kernel<true, false, true, false> + <false, true, true, false> per middle pass + <false, true, false, false>"
                        : "conv3x3_bf16_w8_kernel<false, false, true, false> + <false, true, true, false> per middle pass + <false, true, false, false>";
@@ -535,7 +554,7 @@ static size_t part_region_bytes(int which, uint32_t N, uint32_t Cin, uint32_t Co
 size_t conv_bf16_mfma_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                                       uint32_t W) {
   size_t bytes = filter_region_bytes(which, Cin, Cout);
-  if (conv_bf16_passes(which, Cin, Cout) > 1u) bytes += (size_t)num_tiles * part_region_bytes(which, N, Cin, Cout, H, W);
+  if (conv_bf16_launches(which, Cin, Cout) > 1u) bytes += (size_t)num_tiles * part_region_bytes(which, N, Cin, Cout, H, W);
   return bytes;
 }
 
@@ -576,7 +595,9 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
   P.pass = 0;
   P.chan0 = 0;
   P.cred_pass = P.Cred < 64u ? P.Cred : 64u;
-  if (P.passes > 1u) {
+  P.first_pass = P.last_pass = 1;
+  const uint32_t launches = conv_bf16_launches(which, Cin, Cout);
+  if (launches > 1u) {
     uint8_t *part = reinterpret_cast<uint8_t *>(workspace) + filter_region_bytes(which, Cin, Cout);
     const size_t per_tile = part_region_bytes(which, N, Cin, Cout, H, W);
     for (uint32_t t = 0; t < num_tiles; ++t) P.part[t] = reinterpret_cast<float *>(part + t * per_tile);
@@ -595,33 +616,42 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
   }
 
   const uint32_t cus = (uint32_t)num_cus();
-  P.strips = (P.OW + kStripCols - 1) / kStripCols;
-  const uint64_t base_items = (uint64_t)N * num_tiles * P.strips;
-  if (base_items >= (1ull << 30)) return ADH_EINVAL;
-  P.items = (uint32_t)base_items;
-  P.steps_per_item = (P.OH + kStepRows - 1) / kStepRows;
-  uint32_t gx = cus / groups ? cus / groups : 1u;
-  if (gx > P.items * P.steps_per_item) gx = P.items * P.steps_per_item;
-  // whole items while they go round evenly; the rest in row segments of at least four steps
-  // (a segment re-reads two input rows and pays for filling the ring again)
-  P.whole_items = P.items / gx * gx;
-  const uint32_t rest = P.items - P.whole_items;
-  P.seg_steps = P.steps_per_item;
-  P.segs = 1;
-  if (rest) {
-    const uint32_t want_segs = gx / rest;  // >= 1
-    uint32_t seg_steps = (P.steps_per_item + want_segs - 1) / want_segs;
-    // the eight-wave kernel starts an item with one step without MFMAs; the four-wave one fills its ring first
-    const uint32_t min_steps = conv_bf16_w8_takes(P, num_tiles) ? 2u : 4u;
-    if (seg_steps < min_steps) seg_steps = P.steps_per_item < min_steps ? P.steps_per_item : min_steps;
-    P.seg_steps = seg_steps;
-    P.segs = (P.steps_per_item + seg_steps - 1) / seg_steps;
-  }
-  P.pieces = rest * P.segs;
-  P.div_strips = FastDiv(P.strips);
-  P.div_N = FastDiv(N);
-  P.div_rest = FastDiv(rest ? rest : 1u);
-  if (direct && conv_bf16_w8_takes(P, num_tiles)) {
+  // work items and their division among `gx` persistent workgroups per group of output channels, for strips of
+  // `strip_cols` columns
+  auto plan = [&](uint32_t strip_cols, uint32_t out_groups, uint32_t min_seg_steps, uint32_t *gx_out) -> int {
+    P.strips = (P.OW + strip_cols - 1) / strip_cols;
+    const uint64_t base_items = (uint64_t)N * num_tiles * P.strips;
+    if (base_items >= (1ull << 30)) return ADH_EINVAL;
+    P.items = (uint32_t)base_items;
+    P.steps_per_item = (P.OH + kStepRows - 1) / kStepRows;
+    uint32_t gx = cus / out_groups ? cus / out_groups : 1u;
+    if (gx > P.items * P.steps_per_item) gx = P.items * P.steps_per_item;
+    // whole items while they go round evenly; the rest in row segments of at least `min_seg_steps` steps
+    // (a segment re-reads two input rows and pays for filling the ring again)
+    P.whole_items = P.items / gx * gx;
+    const uint32_t rest = P.items - P.whole_items;
+    P.seg_steps = P.steps_per_item;
+    P.segs = 1;
+    if (rest) {
+      const uint32_t want_segs = gx / rest;  // >= 1
+      uint32_t seg_steps = (P.steps_per_item + want_segs - 1) / want_segs;
+      if (seg_steps < min_seg_steps) seg_steps = P.steps_per_item < min_seg_steps ? P.steps_per_item : min_seg_steps;
+      P.seg_steps = seg_steps;
+      P.segs = (P.steps_per_item + seg_steps - 1) / seg_steps;
+    }
+    P.pieces = rest * P.segs;
+    P.div_strips = FastDiv(P.strips);
+    P.div_N = FastDiv(N);
+    P.div_rest = FastDiv(rest ? rest : 1u);
+    *gx_out = gx;
+    return ADH_OK;
+  };
+  const bool w8 = conv_bf16_w8_takes(P, num_tiles);
+  uint32_t gx = 0;
+  // the eight-wave kernel starts an item with one step without MFMAs; the four-wave one fills its ring first
+  e = plan(kStripCols, groups, w8 ? 2u : 4u, &gx);
+  if (e) return e;
+  if (direct && w8) {
     P.w_direct = reinterpret_cast<const uint16_t *>(w);
   } else if (direct) {
     // the four-wave kernel takes this shape after all (tile alignment): it needs the transformed copy
@@ -634,12 +664,30 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
   }
   if (P.passes > 1u) {
     // conv_bf16_mfma_supported has checked widths and sizes; what is left is the tiles' alignment
-    if (!conv_bf16_w8_takes(P, num_tiles)) return ADH_EALIGN;
-    for (P.pass = 0; P.pass < P.passes; ++P.pass) {
-      P.chan0 = 64u * P.pass;
-      P.cred_pass = P.Cred - P.chan0 < 64u ? P.Cred - P.chan0 : 64u;
-      e = conv_bf16_w8_launch(P, gx, groups, st);
+    if (!w8) return ADH_EALIGN;
+    const bool k128 = conv_bf16_uses_k128(which, Cin, Cout) && conv_bf16_k128_takes(P, num_tiles);
+    uint32_t gx128 = 0;
+    const uint32_t groups128 = (P.Cout + 127u) / 128u;
+    const ConvBf16Params plan64 = P;  // the plan for 64-column strips, kept for a last launch of at most 64 channels
+    if (k128) {
+      e = plan(kStripColsK128, groups128, 2u, &gx128);
       if (e) return e;
+    }
+    ConvBf16Params plan128 = P;
+    uint32_t chan = 0, launch = 0;
+    while (chan < P.Cred) {
+      const uint32_t rem = P.Cred - chan;
+      const bool wide = k128 && rem > 64u;
+      ConvBf16Params Q = wide ? plan128 : plan64;
+      Q.chan0 = chan;
+      Q.pass = chan / 64u;
+      Q.cred_pass = wide ? (rem < 128u ? rem : 128u) : (rem < 64u ? rem : 64u);
+      Q.first_pass = launch == 0u ? 1u : 0u;
+      Q.last_pass = chan + Q.cred_pass >= P.Cred ? 1u : 0u;
+      e = wide ? conv_bf16_k128_launch(Q, gx128, groups128, st) : conv_bf16_w8_launch(Q, gx, groups, st);
+      if (e) return e;
+      chan += Q.cred_pass;
+      ++launch;
     }
     return ADH_OK;
   }

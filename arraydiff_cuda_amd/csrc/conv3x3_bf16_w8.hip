@@ -423,7 +423,8 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   // of the row group that has landed, the five copies of the next group, and for beta = 1 the
   // four loads of old values (buffer loads and stores: a row that does not exist gets an
   // out-of-range offset, so the sequence has no branches).
-  auto compute = [&](uint32_t sb, auto side_tag, auto bar_tag, auto nbr_tag, uint32_t row0, uint32_t nrows, bool barrier_owed) {
+  auto compute = [&](uint32_t sb, auto side_tag, auto bar_tag, auto nbr_tag, uint32_t row0, uint32_t nrows, bool barrier_owed,
+                     bool after_plain) {
     constexpr bool SIDE = decltype(side_tag)::value != 0;
     // 1: this phase's barrier comes between the rounds and the packing; 2: the previous phase's barrier, if still
     // owed, comes after the first operand fetches (row pair 0 only: they read rows that step shares with this one)
@@ -467,8 +468,14 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
     }
     // The copies of the group to transpose have landed: everything but the previous step's four
     // stores, which were issued after them (memory instructions complete in order).
-    // (eight stores when the sums go out as fp32)
-    if (SIDE) __builtin_amdgcn_s_waitcnt(POUT ? 0x0F78 : 0x0F74);  // vmcnt(8) : vmcnt(4)
+    // (eight stores when the sums go out as fp32).  After a phase without MFMAs nothing was issued after the
+    // copies, and the wait is for all of them.
+    if (SIDE) {
+      if (after_plain)
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      else
+        __builtin_amdgcn_s_waitcnt(POUT ? 0x0F78 : 0x0F74);  // vmcnt(8) : vmcnt(4)
+    }
     // packs tile i (row i / 2 of the pair, channel tile i % 2) back to store order through the
     // swap between lane rows and, in the interleaved form, stores it
     auto pack_tile = [&](auto tag) {
@@ -618,6 +625,7 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
   // with the one before it, which no wave overwrites meanwhile.  Its matrix pipe then starts the moment
   // the late waves arrive.  Row pair 1 passes the barrier between its rounds and its packing.
   bool barrier_owed = false;
+  bool after_plain = true;  // the last phase issued its copies last: no stores after them
   for (;;) {
     const bool fast = stepC >= 0 && wholeC;
     if (barrier_owed && !(fast && rp == 0u)) {
@@ -634,28 +642,31 @@ __global__ __launch_bounds__(kW8Threads, 1) void conv3x3_bf16_w8_kernel(ConvBf16
         if constexpr (HF) nbr = group_has_neighbour_row();
         if (rp == 0u) {
           if constexpr (HF) {
-            if (nbr) compute(sb, IntTag<1>(), IntTag<2>(), IntTag<1>(), row0, nrows, barrier_owed);
-            else compute(sb, IntTag<1>(), IntTag<2>(), IntTag<0>(), row0, nrows, barrier_owed);
+            if (nbr) compute(sb, IntTag<1>(), IntTag<2>(), IntTag<1>(), row0, nrows, barrier_owed, after_plain);
+            else compute(sb, IntTag<1>(), IntTag<2>(), IntTag<0>(), row0, nrows, barrier_owed, after_plain);
           } else {
-            compute(sb, IntTag<1>(), IntTag<2>(), IntTag<0>(), row0, nrows, barrier_owed);
+            compute(sb, IntTag<1>(), IntTag<2>(), IntTag<0>(), row0, nrows, barrier_owed, after_plain);
           }
           barrier_owed = false;
         } else {
           if constexpr (HF) {
-            if (nbr) compute(sb, IntTag<1>(), IntTag<1>(), IntTag<1>(), row0, nrows, false);
-            else compute(sb, IntTag<1>(), IntTag<1>(), IntTag<0>(), row0, nrows, false);
+            if (nbr) compute(sb, IntTag<1>(), IntTag<1>(), IntTag<1>(), row0, nrows, false, after_plain);
+            else compute(sb, IntTag<1>(), IntTag<1>(), IntTag<0>(), row0, nrows, false, after_plain);
           } else {
-            compute(sb, IntTag<1>(), IntTag<1>(), IntTag<0>(), row0, nrows, false);
+            compute(sb, IntTag<1>(), IntTag<1>(), IntTag<0>(), row0, nrows, false, after_plain);
           }
           barrier_done = true;
         }
+        after_plain = false;
       } else {
         if (BETA) load_old_guarded(row0, nrows);
         move_rows_plain();
-        compute(sb, IntTag<0>(), IntTag<0>(), IntTag<0>(), row0, nrows, false);
+        compute(sb, IntTag<0>(), IntTag<0>(), IntTag<0>(), row0, nrows, false, false);
+        after_plain = true;  // its stores are conditional: count on none
       }
     } else {
       move_rows_plain();
+      after_plain = true;
     }
     loader_advance();
     if (!barrier_done) {
@@ -699,35 +710,36 @@ bool conv_bf16_w8_takes(const ConvBf16Params &P, uint32_t num_tiles) {
 
 int conv_bf16_w8_launch(const ConvBf16Params &P, uint32_t gx, uint32_t groups, hipStream_t st) {
   const dim3 grid(gx, groups), block(kW8Threads);
+  const bool first = P.first_pass != 0u, last = P.last_pass != 0u;
   if (P.pad == 1) {  // no halo on either side
-    if (P.passes <= 1u) {
+    if (first && last) {
       if (P.beta != 0.f)
         hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<true, false, false, true>), grid, block, 0, st, P);
       else
         hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, false, false, true>), grid, block, 0, st, P);
-    } else if (P.pass == 0u) {
+    } else if (first) {
       if (P.beta != 0.f)
         hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<true, false, true, true>), grid, block, 0, st, P);
       else
         hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, false, true, true>), grid, block, 0, st, P);
-    } else if (P.pass + 1u < P.passes) {
+    } else if (!last) {
       hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, true, true, true>), grid, block, 0, st, P);
     } else {
       hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, true, false, true>), grid, block, 0, st, P);
     }
     return launch_status();
   }
-  if (P.passes <= 1u) {
+  if (first && last) {
     if (P.beta != 0.f)
       hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<true>), grid, block, 0, st, P);
     else
       hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false>), grid, block, 0, st, P);
-  } else if (P.pass == 0u) {
+  } else if (first) {
     if (P.beta != 0.f)
       hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<true, false, true>), grid, block, 0, st, P);
     else
       hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, false, true>), grid, block, 0, st, P);
-  } else if (P.pass + 1u < P.passes) {
+  } else if (!last) {
     hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, true, true>), grid, block, 0, st, P);
   } else {
     hipLaunchKernelGGL((conv3x3_bf16_w8_kernel<false, true, false>), grid, block, 0, st, P);

@@ -483,32 +483,48 @@ def main():
                                                               ws5.data_ptr(), ws5_bytes, stream),
             "mfma", flops5, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
         del Y5, xu, yu
-        # 128 channels on the bf16 matrix cores (two passes of 64 reduction channels with fp32 sums in between;
-        # the filter gradient as four 64 x 64 channel pairs): the high-resolution tiles at half the width
-        Cw, Ww = 128, W5 // 2
-        xw = [torch.rand((N5, Cw, Ht5 + 2, Ww + 2), device="cuda", generator=g).to(torch.bfloat16) for _ in range(K5)]
-        yw = [torch.rand((N5, Cw, Ht5, Ww), device="cuda", generator=g).to(torch.bfloat16) for _ in range(K5)]
-        ww = (torch.randn((Cw, Cw, 3, 3), device="cuda", generator=g) * 0.03).to(torch.bfloat16)
-        gww = torch.zeros((Cw, Cw, 3, 3), device="cuda")
-        xw_tbl, _kw1 = capi.ptr_table([t.data_ptr() for t in xw])
-        yw_tbl, _kw2 = capi.ptr_table([t.data_ptr() for t in yw])
-        wsw_bytes = max(capi.conv_workspace_bytes(wh, capi.ADH_BF16, K5, N5, Cw, Cw, Ht5, Ww)
-                        for wh in (capi.ADH_CONV_FWD, capi.ADH_CONV_BWD_DATA, capi.ADH_CONV_BWD_FILTER))
-        wsw = torch.empty(wsw_bytes // 4 + 64, device="cuda")
-        flopsw = 2.0 * K5 * N5 * Cw * Cw * 9 * Ht5 * Ww
-        add("conv fwd bf16 128->128 channels, 8 tiles of 128(+2)x1024(+2) (two passes)",
-            lambda: lib.adh_conv3x3_slab_fwd_tiles(1, K5, N5, Cw, Cw, Ht5, Ww, xw_tbl, ww.data_ptr(), yw_tbl, 0.0,
-                                                   wsw.data_ptr(), wsw_bytes, stream),
-            "mfma", flopsw, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
-        add("conv bwd-data bf16 128->128 channels, same tiles (two passes)",
-            lambda: lib.adh_conv3x3_slab_bwd_data_tiles(1, K5, N5, Cw, Cw, Ht5, Ww, ww.data_ptr(), yw_tbl, xw_tbl, 0.0,
-                                                        wsw.data_ptr(), wsw_bytes, stream),
-            "mfma", flopsw, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
-        add("conv bwd-filter bf16 128->128 channels, same tiles (four channel pairs in one launch + reduction)",
-            lambda: lib.adh_conv3x3_slab_bwd_filter_tiles(1, K5, N5, Cw, Cw, Ht5, Ww, xw_tbl, yw_tbl, gww.data_ptr(),
-                                                          0.0, wsw.data_ptr(), wsw_bytes, stream),
-            "mfma", flopsw, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
-        del xw, yw, wsw
+        # more than 64 channels on the bf16 matrix cores: 128 reduction channels per launch with the sums in registers
+        # (256: two launches with fp32 sums between them); the filter gradient as 64 x 64 channel pairs.  The
+        # high-resolution tiles at half (128 channels) and a quarter (256 channels) of the width.
+        for Cw, Ww, how in ((128, W5 // 2, "one launch"), (256, W5 // 4, "two launches of 128 reduction channels")):
+            xw = [torch.rand((N5, Cw, Ht5 + 2, Ww + 2), device="cuda", generator=g).to(torch.bfloat16) for _ in range(K5)]
+            yw = [torch.rand((N5, Cw, Ht5, Ww), device="cuda", generator=g).to(torch.bfloat16) for _ in range(K5)]
+            ww = (torch.randn((Cw, Cw, 3, 3), device="cuda", generator=g) * (2.0 / (Cw * 9)) ** 0.5).to(torch.bfloat16)
+            gww = torch.zeros((Cw, Cw, 3, 3), device="cuda")
+            xw_tbl, _kw1 = capi.ptr_table([t.data_ptr() for t in xw])
+            yw_tbl, _kw2 = capi.ptr_table([t.data_ptr() for t in yw])
+            wsw_bytes = max(capi.conv_workspace_bytes(wh, capi.ADH_BF16, K5, N5, Cw, Cw, Ht5, Ww)
+                            for wh in (capi.ADH_CONV_FWD, capi.ADH_CONV_BWD_DATA, capi.ADH_CONV_BWD_FILTER))
+            wsw = torch.empty(wsw_bytes // 4 + 64, device="cuda")
+            flopsw = 2.0 * K5 * N5 * Cw * Cw * 9 * Ht5 * Ww
+            shape_w = "%d->%d channels, 8 tiles of 128(+2)x%d(+2)" % (Cw, Cw, Ww)
+            kname = capi.conv_kernel_name(capi.ADH_CONV_FWD, capi.ADH_BF16, K5, N5, Cw, Cw, Ht5, Ww)
+            add("conv fwd bf16 %s (%s)" % (shape_w, how),
+                lambda: lib.adh_conv3x3_slab_fwd_tiles(1, K5, N5, Cw, Cw, Ht5, Ww, xw_tbl, ww.data_ptr(), yw_tbl, 0.0,
+                                                       wsw.data_ptr(), wsw_bytes, stream),
+                "mfma", flopsw, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s",
+                extra={"kernel": kname, "traffic": traffic.get(kname, (None, None))[0]})
+            add("conv bwd-data bf16 %s (%s)" % (shape_w, how),
+                lambda: lib.adh_conv3x3_slab_bwd_data_tiles(1, K5, N5, Cw, Cw, Ht5, Ww, ww.data_ptr(), yw_tbl, xw_tbl, 0.0,
+                                                            wsw.data_ptr(), wsw_bytes, stream),
+                "mfma", flopsw, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
+            add("conv bwd-filter bf16 %s (channel pairs of 64 x 64 in one launch + reduction)" % shape_w,
+                lambda: lib.adh_conv3x3_slab_bwd_filter_tiles(1, K5, N5, Cw, Cw, Ht5, Ww, xw_tbl, yw_tbl, gww.data_ptr(),
+                                                              0.0, wsw.data_ptr(), wsw_bytes, stream),
+                "mfma", flopsw, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
+            if Cw == 128:
+                xwu = [torch.rand((N5, Cw, Ht5, Ww), device="cuda", generator=g).to(torch.bfloat16) for _ in range(K5)]
+                xwu_tbl, _kw3 = capi.ptr_table([t.data_ptr() for t in xwu])
+                add("conv fwd bf16 %d->%d channels over tiles without halo, 8 tiles of 128x%d (one launch)" % (Cw, Cw, Ww),
+                    lambda: lib.adh_conv3x3_unpadded_fwd_tiles(1, K5, N5, Cw, Cw, Ht5, Ww, xwu_tbl, ww.data_ptr(), yw_tbl,
+                                                               0.0, wsw.data_ptr(), wsw_bytes, stream),
+                    "mfma", flopsw, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
+                add("conv bwd-data bf16 %d->%d channels into tiles without halo (beta=0, one launch)" % (Cw, Cw),
+                    lambda: lib.adh_conv3x3_unpadded_bwd_data_tiles(1, K5, N5, Cw, Cw, Ht5, Ww, ww.data_ptr(), yw_tbl, xwu_tbl,
+                                                                    0.0, wsw.data_ptr(), wsw_bytes, stream),
+                    "mfma", flopsw, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s")
+                del xwu
+            del xw, yw, wsw
         # ---- the shapes the reference's own microbenchmarks time, with its own figures of merit ----
         # tools/microbench_spatial.cc:23-28: halo exchange, fp32 N=32, C=64, W=256, H=256/ndev, p=1 (ndev = 4 tiles);
         # it prints p*W*C*N*4 / t (:100-103)

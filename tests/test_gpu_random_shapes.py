@@ -188,7 +188,14 @@ def _bf16_wide_cases(seed, count):
     return out
 
 
-@pytest.mark.parametrize("K,N,Cin,Cout,H,W", _bf16_wide_cases(2028, 16))
+# channel counts the 128-channel kernel takes in one launch (both sides above 64), in launches of 128 with fp32 sums
+# between them (192 = 128 + 64 by the 64-channel kernel, 256 = 128 + 128, 320 = 128 + 128 + 64, 200 = 128 + 72), with
+# output-channel remainders (130, 136, 200), strips off the 32-column step and several row segments
+_BF16_WIDE_FIXED = [(2, 1, 128, 128, 9, 72), (1, 2, 192, 136, 6, 40), (2, 1, 256, 256, 5, 64), (1, 1, 320, 130, 4, 24),
+                    (3, 1, 200, 200, 3, 8), (1, 1, 128, 256, 23, 104), (2, 2, 256, 128, 12, 32)]
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,H,W", _bf16_wide_cases(2028, 16) + _BF16_WIDE_FIXED)
 def test_bf16_conv_random_channel_counts(oracle, K, N, Cin, Cout, H, W):
     """bf16 forward, backward-data (beta 0 and 1) and filter gradient on the matrix cores for channel counts on
     both sides of 64 and 128 (passes of 64 reduction channels, 64 x 64 pairs for the filter gradient), widths that
@@ -227,7 +234,7 @@ def test_bf16_conv_random_channel_counts(oracle, K, N, Cin, Cout, H, W):
     assert rel_err(host(dw), dw_want) <= 1e-4
 
 
-@pytest.mark.parametrize("K,N,Cin,Cout,Ht,W", _bf16_wide_cases(2029, 16))
+@pytest.mark.parametrize("K,N,Cin,Cout,Ht,W", _bf16_wide_cases(2029, 16) + _BF16_WIDE_FIXED)
 def test_bf16_conv_over_tiles_without_halo_random(oracle, K, N, Cin, Cout, Ht, W):
     """adh_conv3x3_unpadded_{fwd,bwd_data,bwd_filter}_tiles against the UNSPLIT convolution with zero padding."""
     rng = np.random.default_rng(Cin * 311 + Cout + K)
