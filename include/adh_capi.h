@@ -134,11 +134,26 @@ int adh_tiles_unpack_nchw(int dtype, uint32_t K, uint32_t halo_pad, uint32_t W, 
 /* ---- C2/C3/C4: 3x3 convolution over the halo-padded slab ------------------ */
 /* All three: cross-correlation, stride 1, dilation 1, conv pad 0 over a slab padded by 1
  * (Conv2DShape.halo_padded_input, src/op.cc:1354-1410), filter KCRS (Cout,Cin,3,3),
- * no bias.  beta is 0 (overwrite) or 1 (accumulate), the two values the reference passes.
+ * no bias (adh_conv_bias_add_tiles / adh_conv_bwd_bias_tiles below).  beta is 0 (overwrite) or 1
+ * (accumulate), the two values the reference passes.
  * `*_tiles` variants run K slabs of identical shape in one launch.  Workspace may be NULL
  * when the matching *_workspace_bytes query returns 0; otherwise it must be 256-byte aligned.
  * ADH_BF16: x, w, y, dy, dx are bf16 in memory, sums are fp32, results rounded to nearest even;
- * dw stays fp32.  The bf16 entry needs a workspace for all three passes. */
+ * dw stays fp32.  The bf16 entry needs a workspace for all three passes.  Shapes and routes in bf16
+ * (forward / backward-data; "reduction channels" are Cin forward and Cout backward):
+ *   - up to 64 reduction channels: one launch on the bf16 matrix cores for any width and alignment;
+ *   - more than 64 reduction channels, even width (forward) or a width that is a multiple of 8
+ *     (backward-data), tiles aligned to 4 (16) bytes: the matrix cores, 128 reduction channels per launch
+ *     with the sums in registers when there are also more than 64 output channels (fp32 sums pass through
+ *     the workspace only between such launches: 256 channels are two), else 64 per launch;
+ *   - more than 64 reduction channels at any other width or alignment: the tensors are widened to fp32 in
+ *     the workspace and the fp32 kernels run, about ten times slower.  Callers that care pad the width.
+ * Backward-data into PADDED slabs is the form the reference's graph needs (cudnnConvolutionBackwardData
+ * writes the whole padded slab, src/op.cc:1701-1712) and the compatibility path here: rows of W + 2
+ * bf16 elements start 4 bytes further into a 64-byte sector with every row, so every store straddles
+ * two sectors and the launch moves 1.2-1.4 times its bytes (0.33 of the matrix peak at 64 channels
+ * where the forward reaches 0.45).  adh_conv3x3_unpadded_bwd_data_tiles, whose rows are aligned, is the
+ * fast form (0.44; 0.54 at 128 channels) and also replaces the halo reduce and the unpad pass. */
 #define ADH_CONV_FWD 0
 #define ADH_CONV_BWD_DATA 1
 #define ADH_CONV_BWD_FILTER 2
