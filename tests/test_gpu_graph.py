@@ -76,6 +76,52 @@ def test_graph_replays_match_eager():
             assert torch.equal(got, exp), "replay %d differs from the eager run" % rep
 
 
+def test_graph_replays_bf16_wide_channels_and_bias():
+    """The bf16 convolution with more than 64 reduction channels (a launch of 128 with the sums in registers, fp32 sums
+    through the workspace into a launch of 64), forward and backward-data, and the bias add and gradient, captured and
+    replayed: bit for bit the eager results on every replay."""
+    K, N, Cin, Cout, Ht, W = 2, 2, 192, 136, 12, 72
+    g = torch.Generator(device="cuda").manual_seed(8)
+    bf = lambda *s: torch.randn(s, device="cuda", generator=g).to(torch.bfloat16)
+    xs, dys = [bf(N, Cin, Ht + 2, W + 2) for _ in range(K)], [bf(N, Cout, Ht, W) for _ in range(K)]
+    w = (torch.randn((Cout, Cin, 3, 3), device="cuda", generator=g) * 0.05).to(torch.bfloat16)
+    bias = [torch.randn(Cout, device="cuda", generator=g) for _ in range(K)]
+    ys = [torch.empty((N, Cout, Ht, W), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
+    gs = [torch.empty((N, Cin, Ht + 2, W + 2), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
+    db = torch.empty(Cout, device="cuda")
+    ws = torch.empty(max(capi.conv_workspace_bytes(wh, capi.ADH_BF16, K, N, Cin, Cout, Ht, W)
+                         for wh in (capi.ADH_CONV_FWD, capi.ADH_CONV_BWD_DATA)) // 4 + 64, device="cuda")
+    bws = torch.empty(capi.conv_bwd_bias_workspace_bytes(K, N, Cout) // 4 + 64, device="cuda")
+
+    def sequence():
+        capi.check(capi.conv_fwd_tiles(xs, w, ys, N, Cin, Cout, Ht, W, ws=ws))
+        capi.check(capi.conv_bias_add_tiles(bias, ys, N, Cout, Ht, W))
+        capi.check(capi.conv_bwd_data_tiles(w, dys, gs, N, Cin, Cout, Ht, W, ws=ws))
+        capi.check(capi.conv_bwd_bias_tiles(dys, db, N, Cout, Ht, W, ws=bws))
+
+    outputs = lambda: [t.clone() for t in ys + gs] + [db.clone()]
+    sequence()
+    torch.cuda.synchronize()
+    want = outputs()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        sequence()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        sequence()
+    for rep in range(3):
+        for t in ys + gs + [db, ws, bws]:
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, exp in zip(outputs(), want):
+            assert torch.equal(got, exp), "replay %d differs from the eager run" % rep
+
+
 def test_filter_gradients_are_reproducible():
     g = torch.Generator(device="cuda").manual_seed(6)
     K, N, C, Ht, W = 2, 4, 64, 14, 56

@@ -264,9 +264,20 @@ def test_bf16_conv_over_tiles_without_halo_random(oracle, K, N, Cin, Cout, Ht, W
     capi.check(capi.conv_unpadded_fwd_tiles(xs, dev(w), ys, N, Cin, Cout, Ht, W, ws=ws_for(capi.ADH_CONV_FWD)))
     capi.check(capi.conv_unpadded_bwd_data_tiles(dev(w), dys, gs, N, Cin, Cout, Ht, W, ws=ws_for(capi.ADH_CONV_BWD_DATA)))
     capi.check(capi.conv_unpadded_bwd_filter_tiles(xs, dys, dw, N, Cin, Cout, Ht, W, ws=ws_for(capi.ADH_CONV_BWD_FILTER)))
+    # accumulating forms: prior contents are added to (beta 1)
+    y0 = bf(rng.standard_normal((N, Cout, H, W)))
+    g0 = bf(rng.standard_normal((N, Cin, H, W)))
+    ya = [dev(y0[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    ga = [dev(g0[:, :, r * Ht:(r + 1) * Ht, :].copy()) for r in range(K)]
+    capi.check(capi.conv_unpadded_fwd_tiles(xs, dev(w), ya, N, Cin, Cout, Ht, W, beta=1.0, ws=ws_for(capi.ADH_CONV_FWD)))
+    capi.check(capi.conv_unpadded_bwd_data_tiles(dev(w), dys, ga, N, Cin, Cout, Ht, W, beta=1.0, ws=ws_for(capi.ADH_CONV_BWD_DATA)))
     for r in range(K):
-        assert rel_err(oracle.bf16_to_f32(host(ys[r])), y_want[:, :, r * Ht:(r + 1) * Ht, :]) <= 5e-3
+        rows = slice(r * Ht, (r + 1) * Ht)
+        assert rel_err(oracle.bf16_to_f32(host(ys[r])), y_want[:, :, rows, :]) <= 5e-3
         assert rel_err(oracle.bf16_to_f32(host(gs[r])), gx_want[:, :, 1 + r * Ht:1 + (r + 1) * Ht, 1:-1]) <= 5e-3
+        assert rel_err(oracle.bf16_to_f32(host(ya[r])), y_want[:, :, rows, :] + oracle.bf16_to_f32(y0[:, :, rows, :])) <= 5e-3
+        assert rel_err(oracle.bf16_to_f32(host(ga[r])),
+                       gx_want[:, :, 1 + r * Ht:1 + (r + 1) * Ht, 1:-1] + oracle.bf16_to_f32(g0[:, :, rows, :])) <= 5e-3
     assert rel_err(host(dw), dw_want) <= 1e-4
 
 
