@@ -1,5 +1,5 @@
-// Declarations shared by the two bf16 matrix-core 3x3 slab convolution kernels
-// (conv3x3_bf16_mfma.hip: four waves, any shape; conv3x3_bf16_w8.hip: eight waves, even widths).
+// Declarations shared by the bf16 matrix-core 3x3 slab convolution kernels (conv3x3_bf16_mfma.hip: four waves,
+// any shape; conv3x3_bf16_w8.hip: eight waves, even widths; conv3x3_bf16_k128.hip: 128 reduction channels per launch).
 #ifndef ADH_CONV3X3_BF16_MFMA_H
 #define ADH_CONV3X3_BF16_MFMA_H
 
@@ -11,6 +11,7 @@ namespace adh {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef floatx4 floatx4_a4 __attribute__((aligned(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

@@ -1,5 +1,6 @@
 // 3x3 slab convolution on the bf16 matrix cores (v_mfma_f32_16x16x32_bf16), forward and
-// backward-data, for up to 64 reduction channels.
+// backward-data, for up to 64 reduction channels per launch (more: one launch per 64, fp32 sums
+// between them), any width and alignment.
 //
 // Shape of the computation.  A workgroup of four waves (one per SIMD, which leaves each wave the
 // whole register file) is persistent: it walks work items (image, 64-column strip, row segment)
@@ -62,7 +63,10 @@ __global__ __launch_bounds__(256) void conv3x3_bf16_filter_kernel(const uint16_t
   wt[i] = v;
 }
 
-template <bool BETA>
+// More than 64 reduction channels: one launch per 64 (P.pass), the sums travelling between the launches as fp32
+// in P.part (PIN: this launch adds the sums of the earlier ones, POUT: it leaves its sums there instead of
+// rounding them into the output).  BETA (old output added) belongs to the first launch.
+template <bool BETA, bool PIN, bool POUT>
 __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) {
   __shared__ __attribute__((aligned(16))) uint8_t ring[kRingBytes];
 
@@ -75,7 +79,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
   // this wave's filter share, in B-operand order: lane (n = l16, k-block = g)
   u32x4 wreg[9][2][2];
   {
-    const u32x4 *wt = reinterpret_cast<const u32x4 *>(P.wt + (size_t)grp * kWtGroupElems);
+    const u32x4 *wt = reinterpret_cast<const u32x4 *>(P.wt + ((size_t)grp * P.passes + P.pass) * kWtGroupElems);
 #pragma unroll
     for (int tap = 0; tap < 9; ++tap)
 #pragma unroll
@@ -92,8 +96,10 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
   const uint32_t image_bytes = P.Cred * plane_bytes;
   uint32_t chvalid = 0;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) chvalid |= (chg * 8u + j < P.Cred ? 1u : 0u) << j;
-  const uint32_t tkeep = tch < P.Cred ? 0xffffffffu : 0u;
+  for (int j = 0; j < 8; ++j) chvalid |= (chg * 8u + j < P.cred_pass ? 1u : 0u) << j;
+  const uint32_t tkeep = tch < P.cred_pass ? 0xffffffffu : 0u;
+  // the image's last channel, counted from this launch's first (beyond 63: it belongs to a later launch)
+  const uint32_t last_chan = P.Cred - 1u - P.chan0;
 
   // operand reads: pixel (32 cw + 16 cti + l16 + kw) of a ring row, channels 8 g .. 8 g + 7 of a half
   uint32_t read_lane_off[2][3];
@@ -144,8 +150,8 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
                         ((tcol0 + 1 >= 0 && tcol0 + 1 < (int32_t)P.IW) ? 0xffff0000u : 0u);
     const int32_t arow0 = (int32_t)r_begin - P.pad;  // input row of ring-relative row 0
     // byte offset of (channel chg*8, input row arow0 + lrow, column icol0); may be negative
-    const int32_t vbase = (int32_t)((chg * 8u * P.IH) * P.IW * 2u) + ((arow0 + (int32_t)lrow) * (int32_t)P.IW + icol0) * 2;
-    const int32_t tbase = (int32_t)((tch * P.IH) * P.IW * 2u) + ((arow0 + (int32_t)lrow) * (int32_t)P.IW + tcol0) * 2;
+    const int32_t vbase = (int32_t)(((P.chan0 + chg * 8u) * P.IH) * P.IW * 2u) + ((arow0 + (int32_t)lrow) * (int32_t)P.IW + icol0) * 2;
+    const int32_t tbase = (int32_t)(((P.chan0 + tch) * P.IH) * P.IW * 2u) + ((arow0 + (int32_t)lrow) * (int32_t)P.IW + tcol0) * 2;
 
     // per-channel load offsets and keep-masks (all ones for a channel that exists)
     uint32_t vch[8], vkeep[8];
@@ -195,20 +201,21 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
       const int32_t i = row0 + (int32_t)lrow;
       {
         const int32_t arow = arow0 + i;
-        // A load that starts left of the image's first element (first row of channel 0, left
-        // column halo) has a negative offset and is dropped as a whole: redo it dword by dword.
-        // icol0 is a multiple of two pixels below zero, so the in-range part starts on a dword.
-        if (arow == 0 && chg == 0 && icol0 < 0 && (chvalid & 1u)) {
-          const int32_t v = vbase + row0 * (int32_t)P.IW * 2;
+        // A load that starts left of the image's first element (channel 0, left column halo: the
+        // first row, and the second row of an image one column wide) has a negative offset and is
+        // dropped as a whole: redo it dword by dword.  icol0 is a multiple of two pixels below zero,
+        // so a dword that straddles the image's start holds no column of this row.
+        const int32_t voff = vbase + row0 * (int32_t)P.IW * 2;
+        if (arow >= 0 && chg == 0 && P.chan0 == 0u && voff < 0 && (chvalid & 1u)) {
 #pragma unroll
           for (int d = 0; d < 4; ++d)
-            L.ld[0][d] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, v + 4 * d >= 0 ? (uint32_t)(v + 4 * d) : kOutOfRange, 0, 0);
+            L.ld[0][d] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff + 4 * d >= 0 ? (uint32_t)(voff + 4 * d) : kOutOfRange, 0, 0);
         }
         // The range check drops a dword that straddles the end of the image even though its low
         // half is the image's last element: fetch that element on its own.
         if (arow == (int32_t)P.IH - 1) {
-          if (chg == (P.Cred - 1u) >> 3) {
-            const uint32_t j = (P.Cred - 1u) & 7u;
+          if (chg == last_chan >> 3) {
+            const uint32_t j = last_chan & 7u;
             const uint32_t v = (uint32_t)(vbase + row0 * (int32_t)P.IW * 2) + j * plane_bytes;
             const uint32_t gap = image_bytes - 2u - v;  // distance of the last element from the load start
             if (gap < 16u && (gap & 3u) == 0u) {
@@ -220,7 +227,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
                 for (int dd = 0; dd < 4; ++dd) L.ld[jj][dd] |= ((uint32_t)jj == j && (uint32_t)dd == d) ? e : 0u;
             }
           }
-          if (tch == P.Cred - 1u && (uint32_t)(tbase + row0 * (int32_t)P.IW * 2) == image_bytes - 2u)
+          if (tch == last_chan && (uint32_t)(tbase + row0 * (int32_t)P.IW * 2) == image_bytes - 2u)
             L.lt |= __builtin_amdgcn_raw_buffer_load_b16(rsrc, image_bytes - 2u, 0, 0) & 0xffffu;
         }
       }
@@ -275,6 +282,11 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
     const size_t ct_stride = (size_t)16u * P.OH * P.OW;
     uint16_t *const olane = out_img + (size_t)co0 * P.OH * P.OW + ocol;
     u32x4 pk[2][kStepRows], old[2][kStepRows];
+    // the fp32 sums between launches, [image][output channel][row][column] per tile: a lane's four columns of
+    // column tile cti start at pcol[cti], as the MFMA leaves them
+    float *const part_lane = (PIN || POUT) ? P.part[tile] + ((size_t)n * P.Cout + co0) * P.OH * P.OW : nullptr;
+    const uint32_t pcol[2] = {(uint32_t)c0 + 32u * cw + 4u * g, (uint32_t)c0 + 32u * cw + 16u + 4u * g};
+    floatx4 pin[kStepRows][2][2];
 
     // common case, decided per wave: all rows of a step, both channel tiles, eight whole columns
     const bool lanes_whole = __builtin_amdgcn_ballot_w64(!(full_cols && ok_ct[0] && ok_ct[1])) == 0ull;
@@ -322,6 +334,24 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
         }
     };
 
+    auto load_pin = [&](uint32_t row0, uint32_t nrows) {
+      if (!PIN) return;
+#pragma unroll
+      for (int r = 0; r < kStepRows; ++r)
+#pragma unroll
+        for (int cti = 0; cti < 2; ++cti)
+#pragma unroll
+          for (int ct = 0; ct < 2; ++ct) {
+            pin[r][cti][ct] = (floatx4){0.f, 0.f, 0.f, 0.f};
+            if ((uint32_t)r < nrows && ok_ct[ct]) {
+              const float *p = part_lane + ct * ct_stride + (size_t)(row0 + r) * P.OW + pcol[cti];
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                if (pcol[cti] + j < P.OW) pin[r][cti][ct][j] = p[j];
+            }
+          }
+    };
+
     uint32_t sb = 0;  // ring slot of this step's first input row
     uint32_t prev_row0 = 0, prev_nrows = 0;
 
@@ -330,7 +360,10 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
     // matrix pipe; then the results are packed to bf16.  kVm global-memory instructions and kLds
     // ring writes are spread over the rounds: issued in a burst they would fill the memory
     // pipeline's queue and hold every wave of the workgroup at the same point.
-    auto compute = [&](auto vm_tag, auto &&vm_op, auto lds_tag, auto &&lds_op, auto &&valu_op) {
+    // (row0, nrows, whole: where the sums of a POUT launch go; whole = every lane of the wave stores all of its
+    // columns, rows and channel tiles)
+    auto compute = [&](auto vm_tag, auto &&vm_op, auto lds_tag, auto &&lds_op, auto &&valu_op, uint32_t row0,
+                       uint32_t nrows, bool whole) {
       constexpr int kVm = decltype(vm_tag)::value;
       constexpr int kLds = decltype(lds_tag)::value;
       floatx4 acc[kStepRows][2][2];
@@ -355,6 +388,10 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) {
           floatx4 v0 = acc[r][0][ct], v1 = acc[r][1][ct];
+          if (PIN) {
+            v0 += pin[r][0][ct];
+            v1 += pin[r][1][ct];
+          }
           if (BETA) {
             // back to the MFMA's arrangement: the swap is its own inverse
             const u32x2 s0 = __builtin_amdgcn_permlane16_swap(old[ct][r][0], old[ct][r][2], false, false);
@@ -367,6 +404,21 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
             v1[1] += __uint_as_float(s0[1] & 0xffff0000u);
             v1[2] += __uint_as_float(s1[1] << 16);
             v1[3] += __uint_as_float(s1[1] & 0xffff0000u);
+          }
+          if constexpr (POUT) {
+            float *p0 = part_lane + ct * ct_stride + (size_t)(row0 + r) * P.OW + pcol[0];
+            float *p1 = part_lane + ct * ct_stride + (size_t)(row0 + r) * P.OW + pcol[1];
+            if (whole) {
+              *reinterpret_cast<floatx4_a4 *>(p0) = v0;
+              *reinterpret_cast<floatx4_a4 *>(p1) = v1;
+            } else if ((uint32_t)r < nrows && ok_ct[ct]) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                if (pcol[0] + j < P.OW) p0[j] = v0[j];
+                if (pcol[1] + j < P.OW) p1[j] = v1[j];
+              }
+            }
+            continue;
           }
           const u32x2 q0 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[0], v0[1]), pack_bf16x2(v1[0], v1[1]), false, false);
           const u32x2 q1 = __builtin_amdgcn_permlane16_swap(pack_bf16x2(v0[2], v0[3]), pack_bf16x2(v1[2], v1[3]), false, false);
@@ -452,25 +504,33 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
         // past the end of the segment are never used)
         uint16_t *const sbase = olane + (size_t)prev_row0 * P.OW;
         const uint16_t *const obase = olane + (size_t)row0 * P.OW;
-        compute(IntTag<BETA ? 25 : 17>(), [&](auto tag) {
+        const float *const pbase = part_lane + (size_t)row0 * P.OW;
+        // the memory instructions of a step, in issue order: the sums of the earlier launches and the old output
+        // (both needed when the rows are packed), the rows of the step after next, the previous step's stores
+        constexpr int kPinN = PIN ? 4 * kStepRows : 0, kOldN = BETA ? 2 * kStepRows : 0, kStoreN = POUT ? 0 : 2 * kStepRows;
+        compute(IntTag<kPinN + kOldN + 9 + kStoreN>(), [&](auto tag) {
           constexpr int t = decltype(tag)::value;
-          // beta = 1: the old values first, in the order the rows are packed
-          if constexpr (BETA && t < 8) {
-            constexpr int ct = t & 1, r = t >> 1;
+          if constexpr (t < kPinN) {
+            constexpr int ct = t & 1, cti = (t >> 1) & 1, r = t >> 2;
+            pin[r][cti][ct] = *reinterpret_cast<const floatx4_a4 *>(pbase + ct * ct_stride + (size_t)r * P.OW + pcol[cti]);
+          } else if constexpr (t < kPinN + kOldN) {
+            constexpr int u = t - kPinN;
+            constexpr int ct = u & 1, r = u >> 1;
             old[ct][r] = *reinterpret_cast<const u32x4_unaligned *>(obase + ct * ct_stride + (size_t)r * P.OW);
-          } else if constexpr (t < (BETA ? 17 : 9)) {
-            load_one(IntTag<t - (BETA ? 8 : 0)>(), next_row0 + kStepRows, L0);
+          } else if constexpr (t < kPinN + kOldN + 9) {
+            load_one(IntTag<t - kPinN - kOldN>(), next_row0 + kStepRows, L0);
           } else {
-            constexpr int u = t - (BETA ? 17 : 9);
+            constexpr int u = t - kPinN - kOldN - 9;
             constexpr int ct = u / kStepRows, r = u % kStepRows;
             *reinterpret_cast<u32x4_unaligned *>(sbase + ct * ct_stride + (size_t)r * P.OW) = pk[ct][r];
           }
-        }, IntTag<10>(), [&](auto tag) { ring_write(tag, T); }, [&](auto tag) { transpose_piece(tag, L0, T); });
+        }, IntTag<10>(), [&](auto tag) { ring_write(tag, T); }, [&](auto tag) { transpose_piece(tag, L0, T); }, row0, nrows, true);
       } else {
         if (more2) issue(next_row0 + kStepRows, L0);
-        if (s > 0) store_packed(prev_row0, prev_nrows);
+        if (!POUT && s > 0) store_packed(prev_row0, prev_nrows);
         load_old(row0, nrows);
-        compute(IntTag<0>(), [](auto) {}, IntTag<0>(), [](auto) {}, [](auto) {});
+        load_pin(row0, nrows);
+        compute(IntTag<0>(), [](auto) {}, IntTag<0>(), [](auto) {}, [](auto) {}, row0, nrows, false);
       }
       prev_row0 = row0;
       prev_nrows = nrows;
@@ -478,7 +538,7 @@ __global__ __launch_bounds__(256, 1) void conv3x3_bf16_kernel(ConvBf16Params P) 
       sb += kStepRows;
       sb = sb >= (uint32_t)kRingRows ? sb - (uint32_t)kRingRows : sb;
     }
-    store_packed(prev_row0, prev_nrows);
+    if (!POUT) store_packed(prev_row0, prev_nrows);
   }
 }
 
@@ -495,17 +555,20 @@ static int num_cus() {
   return g_num_cus;
 }
 
-// Up to 64 reduction channels: any shape.  More: one pass of the eight-wave kernel per 64, with fp32 sums between
-// the passes; that kernel needs rows on a 4-byte boundary (forward: even width) or whole 16-byte granules
-// (backward-data: a width that is a multiple of 8), and the sums of one image inside a 2 GiB buffer range.
+// Up to 64 reduction channels: any shape.  More: several launches with fp32 sums between them, which the
+// eight-wave kernels address through a buffer resource: the sums of one image have to lie inside 2 GiB.
+// (The eight-wave kernels need rows on a 4-byte boundary (forward: even width) or whole 16-byte granules
+// (backward-data: a width that is a multiple of 8) and aligned tiles; other shapes take the four-wave kernel
+// once per 64 reduction channels.)
 bool conv_bf16_mfma_supported(int which, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W) {
   const uint32_t cred = which == ADH_CONV_FWD ? Cin : Cout;
   if (cred <= 64u) return true;
   const uint32_t cout_k = which == ADH_CONV_FWD ? Cout : Cin;
   const uint64_t oh = which == ADH_CONV_FWD ? H : H + 2ull, ow = which == ADH_CONV_FWD ? W : W + 2ull;
-  if (cout_k * oh * ow * 4u >= (1ull << 31)) return false;
-  return which == ADH_CONV_FWD ? (W % 2u) == 0u : (W % 8u) == 0u;
+  return cout_k * oh * ow * 4u < (1ull << 31);
 }
+// widths whose rows the eight-wave kernels take
+static bool conv_bf16_w8_width(int which, uint32_t W) { return which == ADH_CONV_FWD ? (W % 2u) == 0u : (W % 8u) == 0u; }
 static uint32_t conv_bf16_passes(int which, uint32_t Cin, uint32_t Cout) {
   return ((which == ADH_CONV_FWD ? Cin : Cout) + 63u) / 64u;
 }
@@ -513,9 +576,10 @@ static uint32_t conv_bf16_passes(int which, uint32_t Cin, uint32_t Cout) {
 // conv3x3_bf16_k128.hip while more than 64 are left, then at most 64 by the eight-wave kernel.  Otherwise one
 // launch of the eight-wave kernel per 64.
 static bool conv_bf16_uses_k128(int which, uint32_t Cin, uint32_t Cout) { return Cin > 64u && Cout > 64u; }
-static uint32_t conv_bf16_launches(int which, uint32_t Cin, uint32_t Cout) {
+// (a width the eight-wave kernels do not take: one launch of the four-wave kernel per 64)
+static uint32_t conv_bf16_launches(int which, uint32_t Cin, uint32_t Cout, uint32_t W) {
   const uint32_t cred = which == ADH_CONV_FWD ? Cin : Cout;
-  if (!conv_bf16_uses_k128(which, Cin, Cout)) return (cred + 63u) / 64u;
+  if (!conv_bf16_uses_k128(which, Cin, Cout) || !conv_bf16_w8_width(which, W)) return (cred + 63u) / 64u;
   uint32_t n = 0, rem = cred;
   while (rem > 64u) {
     rem -= rem < 128u ? rem : 128u;
@@ -528,17 +592,40 @@ static uint32_t conv_bf16_launches(int which, uint32_t Cin, uint32_t Cout) {
 // (template arguments: old output added, sums of earlier passes read, sums written for a later pass, tiles without halo)
 const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, float beta) {
   if (!conv_bf16_mfma_supported(which, Cin, Cout, H, W)) return "widen_bf16_kernel + conv3x3_f32_kernel + narrow_bf16_kernel";
+  if (!conv_bf16_w8_width(which, W)) {
+    if (conv_bf16_passes(which, Cin, Cout) > 1u)
+      return beta != 0.f ? "conv3x3_bf16_kernel<true, false, true> + <false, true, true> per middle 64 reduction channels + <false, true, false>"
+                         : "conv3x3_bf16_kernel<false, false, true> + <false, true, true> per middle 64 reduction channels + <false, true, false>";
+    return beta != 0.f ? "conv3x3_bf16_kernel<true, false, false>" : "conv3x3_bf16_kernel<false, false, false>";
+  }
   if (conv_bf16_uses_k128(which, Cin, Cout)) {
-    if (conv_bf16_launches(which, Cin, Cout) == 1u)
+    if (conv_bf16_launches(which, Cin, Cout, W) == 1u)
       return beta != 0.f ? "conv3x3_bf16_k128_kernel<true, false, false, false>" : "conv3x3_bf16_k128_kernel<false, false, false, false>";
     return "conv3x3_bf16_k128_kernel per 128 reduction channels (fp32 sums between the launches) + conv3x3_bf16_w8_kernel for a rest of at most 64";
   }
   if (conv_bf16_passes(which, Cin, Cout) > 1u)
     return beta != 0.f ? "conv3x3_bf16_w8_kernel<true, false, true, false> + <false, true, true, false> per middle pass + <false, true, false, false>"
                        : "conv3x3_bf16_w8_kernel<false, false, true, false> + <false, true, true, false> per middle pass + <false, true, false, false>";
-  const bool w8 = which == ADH_CONV_FWD ? (W % 2u) == 0u : (W % 8u) == 0u;
-  if (w8) return beta != 0.f ? "conv3x3_bf16_w8_kernel<true, false, false, false>" : "conv3x3_bf16_w8_kernel<false, false, false, false>";
-  return beta != 0.f ? "conv3x3_bf16_kernel<true>" : "conv3x3_bf16_kernel<false>";
+  return beta != 0.f ? "conv3x3_bf16_w8_kernel<true, false, false, false>" : "conv3x3_bf16_w8_kernel<false, false, false, false>";
+}
+
+// the four-wave kernel over the reduction channels P.chan0 .. P.chan0 + P.cred_pass - 1
+static int conv_bf16_w4_launch(const ConvBf16Params &P, uint32_t gx, uint32_t groups, hipStream_t st) {
+  const dim3 grid(gx, groups), block(256);
+  const bool first = P.first_pass != 0u, last = P.last_pass != 0u, beta = P.beta != 0.f;
+  if (!(first && last) && !P.part[0]) return ADH_ENULL;  // sums between launches need their buffers
+  if (first && last) {
+    if (beta) hipLaunchKernelGGL((conv3x3_bf16_kernel<true, false, false>), grid, block, 0, st, P);
+    else hipLaunchKernelGGL((conv3x3_bf16_kernel<false, false, false>), grid, block, 0, st, P);
+  } else if (first) {
+    if (beta) hipLaunchKernelGGL((conv3x3_bf16_kernel<true, false, true>), grid, block, 0, st, P);
+    else hipLaunchKernelGGL((conv3x3_bf16_kernel<false, false, true>), grid, block, 0, st, P);
+  } else if (!last) {
+    hipLaunchKernelGGL((conv3x3_bf16_kernel<false, true, true>), grid, block, 0, st, P);
+  } else {
+    hipLaunchKernelGGL((conv3x3_bf16_kernel<false, true, false>), grid, block, 0, st, P);
+  }
+  return launch_status();
 }
 
 // the reordered filter, then (more than one pass) the fp32 sums of every tile, each region 256-byte aligned
@@ -554,7 +641,7 @@ static size_t part_region_bytes(int which, uint32_t N, uint32_t Cin, uint32_t Co
 size_t conv_bf16_mfma_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                                       uint32_t W) {
   size_t bytes = filter_region_bytes(which, Cin, Cout);
-  if (conv_bf16_launches(which, Cin, Cout) > 1u) bytes += (size_t)num_tiles * part_region_bytes(which, N, Cin, Cout, H, W);
+  if (conv_bf16_launches(which, Cin, Cout, W) > 1u) bytes += (size_t)num_tiles * part_region_bytes(which, N, Cin, Cout, H, W);
   return bytes;
 }
 
@@ -596,7 +683,7 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
   P.chan0 = 0;
   P.cred_pass = P.Cred < 64u ? P.Cred : 64u;
   P.first_pass = P.last_pass = 1;
-  const uint32_t launches = conv_bf16_launches(which, Cin, Cout);
+  const uint32_t launches = conv_bf16_launches(which, Cin, Cout, W);
   if (launches > 1u) {
     uint8_t *part = reinterpret_cast<uint8_t *>(workspace) + filter_region_bytes(which, Cin, Cout);
     const size_t per_tile = part_region_bytes(which, N, Cin, Cout, H, W);
@@ -663,8 +750,23 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
     if (e) return e;
   }
   if (P.passes > 1u) {
-    // conv_bf16_mfma_supported has checked widths and sizes; what is left is the tiles' alignment
-    if (!w8) return ADH_EALIGN;
+    if (!w8) {
+      // odd widths, tiles off the eight-wave kernels' alignment: the four-wave kernel once per 64 channels.  The
+      // workspace holds the sums between the launches unless the width promised one launch of 128 channels: then
+      // it is the tiles' alignment that keeps the eight-wave kernels away, and there is no room for the sums.
+      if (launches <= 1u) return ADH_EALIGN;
+      for (uint32_t pass = 0; pass < P.passes; ++pass) {
+        ConvBf16Params Q = P;
+        Q.pass = pass;
+        Q.chan0 = 64u * pass;
+        Q.cred_pass = P.Cred - Q.chan0 < 64u ? P.Cred - Q.chan0 : 64u;
+        Q.first_pass = pass == 0u ? 1u : 0u;
+        Q.last_pass = pass + 1u == P.passes ? 1u : 0u;
+        e = conv_bf16_w4_launch(Q, gx, groups, st);
+        if (e) return e;
+      }
+      return ADH_OK;
+    }
     const bool k128 = conv_bf16_uses_k128(which, Cin, Cout) && conv_bf16_k128_takes(P, num_tiles);
     uint32_t gx128 = 0;
     const uint32_t groups128 = (P.Cout + 127u) / 128u;
@@ -692,11 +794,7 @@ int conv_bf16_mfma(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
     return ADH_OK;
   }
   if (conv_bf16_w8_takes(P, num_tiles)) return conv_bf16_w8_launch(P, gx, groups, st);
-  if (beta != 0.f)
-    hipLaunchKernelGGL(conv3x3_bf16_kernel<true>, dim3(gx, groups), dim3(256), 0, st, P);
-  else
-    hipLaunchKernelGGL(conv3x3_bf16_kernel<false>, dim3(gx, groups), dim3(256), 0, st, P);
-  return launch_status();
+  return conv_bf16_w4_launch(P, gx, groups, st);
 }
 
 }  // namespace adh

@@ -146,8 +146,14 @@ int adh_tiles_unpack_nchw(int dtype, uint32_t K, uint32_t halo_pad, uint32_t W, 
  *     (backward-data), tiles aligned to 4 (16) bytes: the matrix cores, 128 reduction channels per launch
  *     with the sums in registers when there are also more than 64 output channels (fp32 sums pass through
  *     the workspace only between such launches: 256 channels are two), else 64 per launch;
- *   - more than 64 reduction channels at any other width or alignment: the tensors are widened to fp32 in
- *     the workspace and the fp32 kernels run, about ten times slower.  Callers that care pad the width.
+ *   - more than 64 reduction channels at any other width (odd; backward-data at a width that is no multiple
+ *     of 8): the four-wave matrix-core kernel once per 64 reduction channels with fp32 sums through the
+ *     workspace, 2.5-3.5 times slower than the route above (128 -> 128 channels on 64 x 255 tiles 340-430
+ *     TFLOP/s against 1020-1180 at 64 x 256; 512 -> 512 on 7 x 7 tiles 45-60).  Tiles off that alignment
+ *     take the same route when the reduction needs more than one launch anyway; where the width promises ONE
+ *     launch of 128 channels the workspace has no room for the sums and the call returns ADH_EALIGN;
+ *   - the sums of one image beyond 2 GiB (Cout * H * W * 4 bytes): the tensors are widened to fp32 in the
+ *     workspace and the fp32 kernels run, about ten times slower.
  * Backward-data into PADDED slabs is the form the reference's graph needs (cudnnConvolutionBackwardData
  * writes the whole padded slab, src/op.cc:1701-1712) and the compatibility path here: rows of W + 2
  * bf16 elements start 4 bytes further into a 64-byte sector with every row, so every store straddles

@@ -75,10 +75,11 @@ def test_bf16_conv_small_vs_oracle(oracle, K, N, Cin, Cout, H, W):
 
 def test_bf16_conv_odd_pointers_and_many_images(oracle):
     """Tile buffers that are only 2-byte aligned (views one element into an allocation), more work
-    items than workgroups, a one-row image and a single channel."""
+    items than workgroups, a one-row image, a single channel, and more than 64 channels on both sides
+    (several launches with fp32 sums between them)."""
     rng = np.random.default_rng(404)
     bf = lambda a: oracle.f32_to_bf16(a.astype(np.float32))
-    for (N, Cin, Cout, H, W) in ((300, 8, 8, 1, 8), (3, 1, 1, 5, 16), (2, 64, 64, 6, 64)):
+    for (N, Cin, Cout, H, W) in ((300, 8, 8, 1, 8), (3, 1, 1, 5, 16), (2, 64, 64, 6, 64), (2, 160, 136, 6, 64)):
         x = bf(rng.uniform(-1, 1, size=(N, Cin, H + 2, W + 2)))
         w = bf(rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9)))
         dy = bf(rng.standard_normal((N, Cout, H, W)))

@@ -195,17 +195,26 @@ _BF16_WIDE_FIXED = [(2, 1, 128, 128, 9, 72), (1, 2, 192, 136, 6, 40), (2, 1, 256
                     (3, 1, 200, 200, 3, 8), (1, 1, 128, 256, 23, 104), (2, 2, 256, 128, 12, 32)]
 
 
-@pytest.mark.parametrize("K,N,Cin,Cout,H,W", _bf16_wide_cases(2028, 16) + _BF16_WIDE_FIXED)
+# more than 64 reduction channels at widths the eight-wave kernels do not take (odd; even but no multiple of 8 for
+# backward-data): one launch of the four-wave kernel per 64 channels with fp32 sums between them; the last tiles of a
+# ResNet (7 x 7 at 512 channels), one column, channel remainders on both sides
+_BF16_WIDE_ANY_WIDTH = [(2, 1, 128, 128, 9, 7), (1, 2, 192, 136, 6, 13), (2, 1, 100, 70, 5, 66), (1, 1, 320, 130, 4, 27),
+                        (3, 1, 65, 65, 3, 1), (1, 1, 512, 512, 7, 7), (2, 2, 130, 40, 12, 33), (1, 1, 72, 200, 10, 70),
+                        (1, 2, 96, 96, 17, 131)]
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,H,W", _bf16_wide_cases(2028, 16) + _BF16_WIDE_FIXED + _BF16_WIDE_ANY_WIDTH)
 def test_bf16_conv_random_channel_counts(oracle, K, N, Cin, Cout, H, W):
-    """bf16 forward, backward-data (beta 0 and 1) and filter gradient on the matrix cores for channel counts on
-    both sides of 64 and 128 (passes of 64 reduction channels, 64 x 64 pairs for the filter gradient), widths that
-    are multiples of 8.  Tolerances as in test_gpu_conv_bf16.py."""
+    """bf16 forward and backward-data (beta 0 and 1 each) and filter gradient on the matrix cores for channel counts
+    on both sides of 64 and 128 (launches of 64 or 128 reduction channels, 64 x 64 pairs for the filter gradient).
+    Tolerances as in test_gpu_conv_bf16.py."""
     rng = np.random.default_rng(Cin * 211 + Cout)
     bf = lambda a: oracle.f32_to_bf16(a.astype(np.float32))
     xs = [bf(rng.uniform(-1, 1, size=(N, Cin, H + 2, W + 2))) for _ in range(K)]
     w = bf(rng.standard_normal((Cout, Cin, 3, 3)) * np.sqrt(2.0 / (Cin * 9)))
     dys = [bf(rng.standard_normal((N, Cout, H, W))) for _ in range(K)]
     g0 = [bf(rng.standard_normal((N, Cin, H + 2, W + 2))) for _ in range(K)]
+    y0 = [bf(rng.standard_normal((N, Cout, H, W))) for _ in range(K)]
     wf = oracle.bf16_to_f32(w)
 
     def ws_for(which):
@@ -215,8 +224,10 @@ def test_bf16_conv_random_channel_counts(oracle, K, N, Cin, Cout, H, W):
     ys = [torch.empty((N, Cout, H, W), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
     gs = [torch.empty((N, Cin, H + 2, W + 2), device="cuda", dtype=torch.bfloat16) for _ in range(K)]
     ga = [dev(a) for a in g0]
+    ya = [dev(a) for a in y0]
     dw = torch.full((Cout, Cin, 3, 3), float("nan"), device="cuda")
     capi.check(capi.conv_fwd_tiles(d_xs, d_w, ys, N, Cin, Cout, H, W, ws=ws_for(capi.ADH_CONV_FWD)))
+    capi.check(capi.conv_fwd_tiles(d_xs, d_w, ya, N, Cin, Cout, H, W, beta=1.0, ws=ws_for(capi.ADH_CONV_FWD)))
     capi.check(capi.conv_bwd_data_tiles(d_w, d_dys, gs, N, Cin, Cout, H, W, ws=ws_for(capi.ADH_CONV_BWD_DATA)))
     capi.check(capi.conv_bwd_data_tiles(d_w, d_dys, ga, N, Cin, Cout, H, W, beta=1.0, ws=ws_for(capi.ADH_CONV_BWD_DATA)))
     capi.check(capi.conv_bwd_filter_tiles(d_xs, d_dys, dw, N, Cin, Cout, H, W, ws=ws_for(capi.ADH_CONV_BWD_FILTER)))
@@ -226,6 +237,7 @@ def test_bf16_conv_random_channel_counts(oracle, K, N, Cin, Cout, H, W):
         y = np.empty((N, Cout, H, W), np.float32)
         oracle.conv_slab_fwd(xf, wf, y)
         assert rel_err(oracle.bf16_to_f32(host(ys[r])), y) <= 5e-3
+        assert rel_err(oracle.bf16_to_f32(host(ya[r])), y + oracle.bf16_to_f32(y0[r])) <= 5e-3
         g = np.empty((N, Cin, H + 2, W + 2), np.float32)
         oracle.conv_slab_bwd_data(wf, dyf, g)
         assert rel_err(oracle.bf16_to_f32(host(gs[r])), g) <= 5e-3
