@@ -1,10 +1,11 @@
 // bf16 entry of the 3x3 slab convolution: bf16 tensors in HBM, fp32 accumulation.
 //
-// Forward and backward-data with at most 64 reduction channels run on the bf16 matrix-core
-// kernel of conv3x3_bf16_mfma.hip.  Everything else (wider reductions, the filter gradient) takes
-// the route below: the bf16 slabs, filter and (for beta = 1) outputs are widened to fp32
-// in the caller's workspace, the fp32 MFMA kernels run on the copies, and the result is rounded
-// back to bf16 (round to nearest even).  Every product is therefore exact and every sum is in
+// Forward and backward-data run on the bf16 matrix-core kernels of conv3x3_bf16_mfma.hip, the filter
+// gradient on that of conv3x3_bf16_wgrad.hip (at a width that is no multiple of 8 over copies of the
+// tensors with wider rows, made here).  What those do not take (images or sums beyond the 2 GiB a
+// buffer resource addresses) goes the route below: the bf16 slabs, filter and (for beta = 1) outputs
+// are widened to fp32 in the caller's workspace, the fp32 MFMA kernels run on the copies, and the
+// result is rounded back to bf16 (round to nearest even).  Every product is therefore exact and every sum is in
 // fp32, i.e. the arithmetic of a bf16-input / fp32-accumulate matrix core, at the speed of the
 // fp32 path plus three streaming passes.  The filter gradient stays fp32.
 #include "adh_common.h"
@@ -51,6 +52,22 @@ __global__ __launch_bounds__(256) void narrow_bf16_kernel(uint64_t n, const floa
   }
 }
 
+// Rows of `w_src` bf16 elements copied into rows of `w_dst` >= w_src elements (w_dst even; dst 4-byte aligned),
+// zeros behind: one thread per dword of the destination.
+__global__ __launch_bounds__(256) void repitch_bf16_kernel(uint64_t rows, uint32_t w_src, uint32_t w_dst,
+                                                          const uint16_t *__restrict__ src, uint32_t *__restrict__ dst) {
+  const uint32_t row_dwords = w_dst >> 1;
+  const uint64_t n = rows * row_dwords;
+  const uint64_t stride = (uint64_t)gridDim.x * 256u;
+  for (uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x; i < n; i += stride) {
+    const uint64_t r = i / row_dwords;
+    const uint32_t c = (uint32_t)(i - r * row_dwords) * 2u;
+    const uint16_t *p = src + r * w_src + c;
+    const uint32_t lo = c < w_src ? p[0] : 0u, hi = c + 1u < w_src ? p[1] : 0u;
+    dst[i] = lo | (hi << 16);
+  }
+}
+
 static uint32_t cvt_grid(uint64_t n) {
   uint64_t b = (n + 2047) / 2048;
   if (b > 256ull * 32) b = 256ull * 32;
@@ -73,10 +90,28 @@ int conv_bf16_wgrad_mfma(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t 
                          const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta,
                          void *workspace, hipStream_t st, bool unpadded);
 
+// The filter gradient at a width that is no multiple of 8: the rows of x_pad and dy are copied into rows of the
+// next multiple of 8 (+ 2 for x_pad) with zeros behind, and the matrix-core kernel runs on the copies: a dy that
+// is zero in the added columns adds nothing to any tap.  (Not when the widened image passes the 2 GiB a buffer
+// resource addresses.)
+static uint32_t wgrad_wide_width(uint32_t W) { return (W + 7u) & ~7u; }
+static bool wgrad_repitch_route(uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W) {
+  if ((W % 8u) == 0u) return false;
+  const uint32_t Wd = wgrad_wide_width(W);
+  return conv_bf16_wgrad_mfma_supported(Cin, Cout, Wd) &&
+         (uint64_t)(Cin > Cout ? Cin : Cout) * (H + 2ull) * (Wd + 2ull) * 2u < (1ull << 31);
+}
+static size_t repitch_region(uint64_t elems) { return (size_t)((elems * 2u + 255u) / 256u * 256u); }
+
 size_t bf16_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
                             uint32_t W, size_t fp32_path_bytes) {
   if (which == ADH_CONV_BWD_FILTER && conv_bf16_wgrad_mfma_supported(Cin, Cout, W))
     return conv_bf16_wgrad_mfma_workspace_bytes(num_tiles, N, Cin, Cout, W);
+  if (which == ADH_CONV_BWD_FILTER && wgrad_repitch_route(Cin, Cout, H, W)) {
+    const uint32_t Wd = wgrad_wide_width(W);
+    return num_tiles * (repitch_region((uint64_t)N * Cin * (H + 2) * (Wd + 2)) + repitch_region((uint64_t)N * Cout * H * Wd)) +
+           conv_bf16_wgrad_mfma_workspace_bytes(num_tiles, N, Cin, Cout, Wd);
+  }
   if (which != ADH_CONV_BWD_FILTER && conv_bf16_mfma_supported(which, Cin, Cout, H, W))
     return conv_bf16_mfma_workspace_bytes(which, num_tiles, N, Cin, Cout, H, W);
   const uint64_t slab = (uint64_t)N * Cin * (H + 2) * (W + 2), out = (uint64_t)N * Cout * H * W;
@@ -183,6 +218,34 @@ int conv_bf16_filter_via_f32(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint3
       if (!aligned_to(x_tiles[t], 2) || !aligned_to(dy_tiles[t], 2)) return ADH_EALIGN;
     }
     return conv_bf16_wgrad_mfma(num_tiles, N, Cin, Cout, H, W, x_tiles, dy_tiles, dw, beta, workspace, st, false);
+  }
+  if (wgrad_repitch_route(Cin, Cout, H, W)) {
+    const uint32_t Wd = wgrad_wide_width(W);
+    if (!workspace) return ADH_ENULL;
+    if (!aligned_to(workspace, 256) || !aligned_to(dw, 4)) return ADH_EALIGN;
+    if (workspace_bytes < bf16_workspace_bytes(ADH_CONV_BWD_FILTER, num_tiles, N, Cin, Cout, H, W, 0)) return ADH_EWORKSPACE;
+    const uint64_t x_rows = (uint64_t)N * Cin * (H + 2), dy_rows = (uint64_t)N * Cout * H;
+    char *ws = reinterpret_cast<char *>(workspace);
+    const void *xw[ADH_MAX_TILES];
+    const void *dyw[ADH_MAX_TILES];
+    for (uint32_t t = 0; t < num_tiles; ++t) {
+      if (!x_tiles[t] || !dy_tiles[t]) return ADH_ENULL;
+      if (!aligned_to(x_tiles[t], 2) || !aligned_to(dy_tiles[t], 2)) return ADH_EALIGN;
+      uint32_t *a = reinterpret_cast<uint32_t *>(ws);
+      ws += repitch_region(x_rows * (Wd + 2));
+      uint32_t *b = reinterpret_cast<uint32_t *>(ws);
+      ws += repitch_region(dy_rows * Wd);
+      hipLaunchKernelGGL(repitch_bf16_kernel, dim3(cvt_grid(x_rows * (Wd + 2) * 4u)), dim3(256), 0, st, x_rows, W + 2u, Wd + 2u,
+                         reinterpret_cast<const uint16_t *>(x_tiles[t]), a);
+      int e = launch_status();
+      if (e) return e;
+      hipLaunchKernelGGL(repitch_bf16_kernel, dim3(cvt_grid(dy_rows * Wd * 4u)), dim3(256), 0, st, dy_rows, W, Wd,
+                         reinterpret_cast<const uint16_t *>(dy_tiles[t]), b);
+      if ((e = launch_status())) return e;
+      xw[t] = a;
+      dyw[t] = b;
+    }
+    return conv_bf16_wgrad_mfma(num_tiles, N, Cin, Cout, H, Wd, xw, dyw, dw, beta, ws, st, false);
   }
   const size_t f32_bytes = adh_conv3x3_workspace_bytes(ADH_CONV_BWD_FILTER, ADH_F32, num_tiles, N, Cin, Cout, H, W);
   if (f32_bytes == 0) return ADH_EUNIMPL;

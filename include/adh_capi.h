@@ -264,7 +264,10 @@ int adh_conv3x3_unpadded_bwd_filter_tiles(int dtype, uint32_t num_tiles, uint32_
 /* cudnnConvolutionBackwardFilter at src/op.cc:1660-1671:
  * dw[co,ci,kh,kw] = beta*dw + sum_{tiles,n,h,w} dy[n,co,h,w] * x_pad[n,ci,h+kh,w+kw]
  * (the sum over tiles is what ParallelSGDOptimizer's ncclReduce did across ranks,
- * include/arraydiff/optimize.hh:443-451).  dw is always fp32.  Deterministic. */
+ * include/arraydiff/optimize.hh:443-451).  dw is always fp32.  Deterministic.
+ * ADH_BF16: the matrix-core kernel reads rows of whole 16-byte granules; at a width that is no multiple
+ * of 8 the rows of x_pad and dy are first copied into the workspace at the next such width with zeros
+ * behind (a zero dy adds nothing to any tap), one more pass over both tensors. */
 int adh_conv3x3_slab_bwd_filter(int dtype, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
                                 const void *x_pad, const void *dy, float *dw, float beta,
                                 void *workspace, size_t workspace_bytes, void *stream);
