@@ -601,6 +601,19 @@ static bool gen_is_3x3s2_unpadded(int dtype, const GenShape &g, bool unpadded, u
          pad_h == 1u && pad_w == 1u;
 }
 
+// conv3x3.hip: the 3x3 window at stride 1 with dilation 3 over fp32 tiles padded by 3, forward and backward-data
+static bool gen_is_3x3_dilated(int dtype, const GenShape &g, bool unpadded) {
+  return dtype == ADH_F32 && !unpadded && g.kh == 3u && g.kw == 3u && g.sh == 1u && g.sw == 1u && g.dh == g.dw && g.dh > 1u;
+}
+int conv3x3_dilated_try(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                        uint32_t W, uint32_t dil, const void *const *in_tiles, const void *w, void *const *out_tiles,
+                        float beta, hipStream_t st);
+// conv3x3_wgrad.hip: its filter gradient
+size_t conv3x3_dilated_wgrad_workspace(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                                       uint32_t dil);
+int conv3x3_dilated_wgrad_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, uint32_t dil,
+                              const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta, void *workspace,
+                              hipStream_t st);
 // conv_thin.hip: forward over halo-padded fp32 tiles for at most three input channels (a network's stem)
 int conv_thin_fwd_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t OH,
                       uint32_t OW, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, const void *const *x_tiles,
@@ -1179,6 +1192,8 @@ size_t conv2d_workspace(int which, int dtype, uint32_t num_tiles, uint32_t N, ui
       bytes = std::max(bytes, conv3x3s2_wgrad_workspace(num_tiles, N, Cin, Cout, g.HP - 2u, g.WP - 2u));
     if (gen_is_thin(dtype, g, unpadded))
       bytes = std::max(bytes, conv_thin_wgrad_workspace(num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, kh, kw, sh, sw));
+    if (gen_is_3x3_dilated(dtype, g, unpadded))
+      bytes = std::max(bytes, conv3x3_dilated_wgrad_workspace(num_tiles, N, Cin, Cout, g.OH, g.OW, g.dh));
     return (bytes + 255u) & ~(size_t)255u;
   }
   GenPlan plan = {};
@@ -1229,6 +1244,13 @@ int conv2d_fwd(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t
                           as_stream(stream));
     if (e != ADH_EUNIMPL) return e;
   }
+  if (gen_is_3x3_dilated(dtype, g, unpadded)) {
+    e = gen_check_workspace(plan, workspace, workspace_bytes);
+    if (e) return e;
+    e = conv3x3_dilated_try(ADH_CONV_FWD, dtype, num_tiles, N, Cin, Cout, g.OH, g.OW, g.dh, x_tiles, w, y_tiles, beta,
+                            as_stream(stream));
+    if (e != ADH_EUNIMPL) return e;
+  }
   if (dtype == ADH_F32 && unpadded && kh == 3u && kw == 3u && sh == 2u && sw == 2u && dh == 1u && dw == 1u && pad_h == 1u &&
       pad_w == 1u) {
     e = gen_check_workspace(plan, workspace, workspace_bytes);
@@ -1269,6 +1291,13 @@ int conv2d_bwd_data(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uin
     e = gen_check_workspace(plan, workspace, workspace_bytes);
     if (e) return e;
     e = conv1x1_try(true, num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, g.sh, dy_tiles, w, dx_tiles, beta, as_stream(stream));
+    if (e != ADH_EUNIMPL) return e;
+  }
+  if (gen_is_3x3_dilated(dtype, g, unpadded)) {
+    e = gen_check_workspace(plan, workspace, workspace_bytes);
+    if (e) return e;
+    e = conv3x3_dilated_try(ADH_CONV_BWD_DATA, dtype, num_tiles, N, Cin, Cout, g.OH, g.OW, g.dh, dy_tiles, w, dx_tiles, beta,
+                            as_stream(stream));
     if (e != ADH_EUNIMPL) return e;
   }
   if (dtype == ADH_F32 && unpadded && kh == 3u && kw == 3u && sh == 2u && sw == 2u && dh == 1u && dw == 1u && pad_h == 1u &&
@@ -1327,6 +1356,14 @@ int conv2d_bwd_filter(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, u
       if (workspace_bytes < need) return ADH_EWORKSPACE;
       e = conv_thin_wgrad_try(num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, kh, kw, sh, sw, x_tiles, dy_tiles, dwt, beta,
                               workspace, st);
+      if (e != ADH_EUNIMPL) return e;
+    }
+  }
+  if (gen_is_3x3_dilated(dtype, g, unpadded)) {
+    const size_t need = conv3x3_dilated_wgrad_workspace(num_tiles, N, Cin, Cout, g.OH, g.OW, g.dh);
+    if (need != 0) {
+      if (workspace_bytes < need) return ADH_EWORKSPACE;
+      e = conv3x3_dilated_wgrad_try(num_tiles, N, Cin, Cout, g.OH, g.OW, g.dh, x_tiles, dy_tiles, dwt, beta, workspace, st);
       if (e != ADH_EUNIMPL) return e;
     }
   }

@@ -91,7 +91,10 @@ struct IntTag {
 //            other wave's MFMAs while every SIMD still carries exactly NT tile-MFMAs per k-step
 // FLIP  = false: forward (weights walked as w[o][k][tap]); true: backward-data
 //         (weights walked as w[k][o][8-tap]).
-template <int NT, int WAVES, bool FLIP, int PROWS>
+// DIL   = dilation of the window: tap (a, b) reads the input DIL * a rows and DIL * b columns on (pad counts input
+//         pixels: 0 forward over a slab padded by DIL, 2 * DIL backward-data); the staged patch is then
+//         (R + 2 DIL) x (TW + 2 DIL), which must fit PROWS rows of 64 floats.
+template <int NT, int WAVES, bool FLIP, int PROWS, int DIL = 1>
 __global__ __launch_bounds__(64 * WAVES, PROWS == kPatchRowsShort ? 2 : 1) void conv3x3_f32_kernel(const ConvParams P) {
   constexpr int kChanStride = PROWS * kLdsPitch + 16;  // == 16 (mod 64)
   constexpr int kPatchFloats = kChunk * kChanStride;
@@ -143,8 +146,8 @@ __global__ __launch_bounds__(64 * WAVES, PROWS == kPatchRowsShort ? 2 : 1) void 
   // address math and no branches: a lane whose element lies outside the input plane carries
   // an offset beyond the resource's size, for which the hardware writes ZERO into LDS. ----
   const int32_t iw = (int32_t)(ow0 + lane) - P.pad;
-  const bool col_ok = lane < P.TW + 2u && iw >= 0 && iw < (int32_t)P.IW;
-  const uint32_t patch_rows = P.R + 2u;
+  const bool col_ok = lane < P.TW + 2u * DIL && iw >= 0 && iw < (int32_t)P.IW;
+  const uint32_t patch_rows = P.R + 2u * DIL;
   uint32_t row_voff[RROWS];
   // a patch row is one wave's, so the image it is read from is a wave-uniform choice: one buffer
   // resource per patch row of this wave
@@ -238,7 +241,7 @@ __global__ __launch_bounds__(64 * WAVES, PROWS == kPatchRowsShort ? 2 : 1) void 
   };
   auto b_off = [](int s_) {
     const int kk = s_ / 9, tap = s_ % 9;
-    return kk * 4 * kChanStride + (tap / 3) * kLdsPitch + (tap % 3);
+    return kk * 4 * kChanStride + (tap / 3) * DIL * kLdsPitch + (tap % 3) * DIL;
   };
 
   // Everything that depends on the number of pixel tiles this wave owns.
@@ -516,6 +519,67 @@ static int conv_direct_kernel_name(int which, uint32_t num_tiles, uint32_t N, ui
   const int prows = patch_rows_for(tile.nt, tile.R);
   snprintf(name, name_bytes, "conv3x3_f32_kernel<%d, %d, %s, %d>", tile.nt, waves, which == ADH_CONV_FWD ? "false" : "true", prows);
   return ADH_OK;
+}
+
+// The 3x3 window at stride 1 with dilation 3 over fp32 tiles padded by 3 (the convolution of the reference's
+// tools/microbench_spatial_conv.cc:25-32), forward (x_pad tiles -> y tiles) and backward-data (dy tiles -> the
+// whole padded dx tiles): the kernel above with its taps three rows and columns apart, 25 pixel tiles per
+// workgroup over a patch of up to 20 rows.  H, W: the interior (= output) extents.  ADH_EUNIMPL (and nothing
+// launched) for another dilation or dtype and for launches of fewer workgroups than CUs, which the general
+// kernel spreads better.  Arguments are the caller's, already validated.
+int conv3x3_dilated_try(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,
+                        uint32_t W, uint32_t dil, const void *const *in_tiles, const void *w, void *const *out_tiles,
+                        float beta, hipStream_t st) {
+  constexpr uint32_t D = 3, NT = 25;
+  if (dtype != ADH_F32 || dil != D) return ADH_EUNIMPL;
+  const uint64_t HP = (uint64_t)H + 2u * D, WP = (uint64_t)W + 2u * D;
+  const uint64_t cmax = Cin > Cout ? Cin : Cout;
+  if ((uint64_t)N * num_tiles > 65535ull || cmax * HP * WP * 4u >= (1ull << 31) || (uint64_t)Cin * Cout * 36u >= (1ull << 31))
+    return ADH_EUNIMPL;
+  ConvParams P = {};
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    P.in[t] = reinterpret_cast<const float *>(in_tiles[t]);
+    P.out[t] = reinterpret_cast<float *>(out_tiles[t]);
+  }
+  P.w = reinterpret_cast<const float *>(w);
+  P.num_tiles = num_tiles;
+  P.N = N;
+  P.beta = beta;
+  if (which == ADH_CONV_FWD) {
+    P.Cred = Cin; P.Cout = Cout;
+    P.IH = (uint32_t)HP; P.IW = (uint32_t)WP; P.OH = H; P.OW = W;
+    P.pad = 0;
+    P.w_out_stride = Cin * 9u; P.w_red_stride = 9u; P.w_flip = 0;
+  } else {
+    P.Cred = Cout; P.Cout = Cin;
+    P.IH = H; P.IW = W; P.OH = (uint32_t)HP; P.OW = (uint32_t)WP;
+    P.pad = 2 * (int32_t)D;
+    P.w_out_stride = 9u; P.w_red_stride = Cin * 9u; P.w_flip = 1;
+  }
+  // R output rows x TW columns per workgroup: R + 2 D <= 20 patch rows, TW + 2 D <= 64 patch columns, R * TW <= 16 NT;
+  // the fewest workgroups win (every workgroup costs the same NT tile-MFMAs per k-step), then the fewest pixels
+  const uint32_t max_r = (uint32_t)kPatchRowsTall - 2u * D, max_tw = (uint32_t)kLdsPitch - 2u * D;
+  uint64_t best_blocks = ~0ull;
+  uint32_t best_r = 0, best_tw = 0;
+  for (uint32_t R = 1; R <= max_r && R <= P.OH; ++R)
+    for (uint32_t TW = 1; TW <= max_tw && TW <= P.OW && R * TW <= 16u * NT; ++TW) {
+      const uint64_t blocks = (uint64_t)((P.OH + R - 1) / R) * ((P.OW + TW - 1) / TW);
+      if (blocks < best_blocks || (blocks == best_blocks && R * TW < best_r * best_tw)) {
+        best_blocks = blocks; best_r = R; best_tw = TW;
+      }
+    }
+  const uint32_t o_groups = (P.Cout + 63u) / 64u;
+  if (best_r == 0 || best_blocks * N * num_tiles * o_groups < 256u || best_blocks >= (1ull << 31)) return ADH_EUNIMPL;
+  P.R = best_r; P.TW = best_tw;
+  P.tiles_x = (P.OW + P.TW - 1) / P.TW;
+  P.div_tiles_x = FastDiv(P.tiles_x);
+  P.div_TW = FastDiv(P.TW);
+  const dim3 grid((uint32_t)best_blocks, o_groups, N * num_tiles);
+  if (P.w_flip)
+    hipLaunchKernelGGL((conv3x3_f32_kernel<(int)NT, 8, true, kPatchRowsTall, (int)D>), grid, dim3(512), 0, st, P);
+  else
+    hipLaunchKernelGGL((conv3x3_f32_kernel<(int)NT, 8, false, kPatchRowsTall, (int)D>), grid, dim3(512), 0, st, P);
+  return launch_status();
 }
 
 const char *conv_bf16_kernel_name(int which, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, float beta);

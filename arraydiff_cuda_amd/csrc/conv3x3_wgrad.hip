@@ -269,6 +269,202 @@ __global__ __launch_bounds__(kWgThreads, PITCH == 44 ? 2 : 1) void conv3x3_wgrad
     }
 }
 
+
+// The same filter gradient for a window whose taps lie DIL rows and columns apart (stride 1, tiles padded by DIL):
+//   dw[co][ci][a][b] = beta*dw + sum dy[n][co][h][w] * x_pad[n][ci][h + DIL a][w + DIL b]
+// Output row r meets the slab rows r, r + DIL and r + 2 DIL, so the ring holds 2 DIL + 2 slab rows (the 2 DIL + 1
+// in use and the one arriving) and the row loop is unrolled once per slot; column tiles of at most 56 pixels at
+// pitch 68 (the last k-step reads column 8 * ceil(ceil(tw / 4) / 2) - 1 + 2 DIL).  Everything else as above.
+static constexpr int kMaxWDil = 56;
+
+template <int V>
+struct WgPhase {
+  static constexpr int value = V;
+};
+
+template <int DIL>
+__global__ __launch_bounds__(kWgThreads, 1) void conv3x3_wgrad_dil_f32_kernel(const WgradParams P) {
+  static_assert(DIL == 3, "eight ring slots are declared below");
+  constexpr int kRowPitch = 68, NS = 2 * DIL + 2;
+  constexpr int kXSlotFloats = 64 * kRowPitch, kDSlotFloats = 32 * kRowPitch;
+  __shared__ float xs0[kXSlotFloats];
+  __shared__ float xs1[kXSlotFloats];
+  __shared__ float xs2[kXSlotFloats];
+  __shared__ float xs3[kXSlotFloats];
+  __shared__ float xs4[kXSlotFloats];
+  __shared__ float xs5[kXSlotFloats];
+  __shared__ float xs6[kXSlotFloats];
+  __shared__ float xs7[kXSlotFloats];
+  __shared__ float dys0[kDSlotFloats];
+  __shared__ float dys1[kDSlotFloats];
+  float *const xs[NS] = {xs0, xs1, xs2, xs3, xs4, xs5, xs6, xs7};
+  float *const dys[2] = {dys0, dys1};
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & 63u, g = lane >> 4, l16 = lane & 15u;
+  const uint32_t wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t ot = wv & 1u;   // co tile inside the 32-channel half
+  const uint32_t ct = wv >> 1;   // ci tile
+
+  uint32_t rest, ctile, pgroup, chunk;
+  P.div_cols.divmod(blockIdx.x, rest, ctile);
+  P.div_chunks.divmod(rest, pgroup, chunk);
+  uint32_t coh, cig;
+  P.div_ci_groups.divmod(blockIdx.y, coh, cig);
+  const uint32_t r0 = chunk * P.rows_per_block;
+  const uint32_t r1 = min(r0 + P.rows_per_block, P.H);
+  const uint32_t WP = P.W + 2u * DIL, HP = P.H + 2u * DIL;
+  const uint32_t ci0 = cig * 64u, co0 = coh * 32u;
+
+  // columns 64..67 of every staged slab row are read by the last k-steps of wide rows but never written by the
+  // 64-lane loads: clear them once
+  for (uint32_t i = tid; i < 64u * 4u; i += kWgThreads) {
+    const uint32_t o = (i >> 2) * kRowPitch + 64u + (i & 3u);
+    xs0[o] = 0.f; xs1[o] = 0.f; xs2[o] = 0.f; xs3[o] = 0.f;
+    xs4[o] = 0.f; xs5[o] = 0.f; xs6[o] = 0.f; xs7[o] = 0.f;
+  }
+
+  const uint32_t w0 = ctile * P.cols_per_block;
+  const uint32_t tw = min(P.cols_per_block, P.W - w0);  // columns of this workgroup
+  const uint32_t x_voff = lane < tw + 2u * DIL ? (w0 + lane) * 4u : kWgOutOfRange;
+  const uint32_t d_voff = lane < tw ? (w0 + lane) * 4u : kWgOutOfRange;
+  const bool ragged_c = (ci0 + 64u > P.Cin) || (co0 + 32u > P.Cout);  // uniform
+  const int x_bytes = (int)(P.Cin * HP * WP * 4u), dy_bytes = (int)(P.Cout * P.H * P.W * 4u);
+  __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.x[0]), 0, 0, kWgBufferFlags);
+  __amdgpu_buffer_rsrc_t rsrc_dy = rsrc_x;
+  auto open_plane = [&](uint32_t plane) {
+    uint32_t n, t;
+    P.div_tiles.divmod(plane, n, t);
+    rsrc_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.x[t] + ((uint64_t)n * P.Cin) * HP * WP), 0, x_bytes,
+                                               kWgBufferFlags);
+    rsrc_dy = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P.dy[t] + ((uint64_t)n * P.Cout) * P.H * P.W), 0,
+                                                dy_bytes, kWgBufferFlags);
+  };
+  auto stage_x_row = [&](float *slot, uint32_t y) {  // slab row y of the 64 input channels; wave v loads channels [8v, 8v+8)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t cl = wv * 8u + i;
+      uint32_t voff = x_voff;
+      uint32_t ci = ci0 + cl;
+      if (ragged_c && ci >= P.Cin) {
+        voff = kWgOutOfRange;
+        ci = 0;
+      }
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, slot + cl * kRowPitch, 4, voff,
+                                               __builtin_amdgcn_readfirstlane((ci * HP + y) * WP * 4u), 0, 0);
+    }
+  };
+  auto stage_dy_row = [&](float *slot, uint32_t r) {  // output row r of the 32 output channels; wave v loads [4v, 4v+4)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t cl = wv * 4u + i;
+      uint32_t voff = d_voff;
+      uint32_t co = co0 + cl;
+      if (ragged_c && co >= P.Cout) {
+        voff = kWgOutOfRange;
+        co = 0;
+      }
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_dy, slot + cl * kRowPitch, 4, voff,
+                                               __builtin_amdgcn_readfirstlane((co * P.H + r) * P.W * 4u), 0, 0);
+    }
+  };
+
+  floatx4 acc[9];
+#pragma unroll
+  for (int tap = 0; tap < 9; ++tap) acc[tap] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const uint32_t ksteps = (tw + 3u) / 4u;
+  const uint32_t npairs = (ksteps + 1u) / 2u;   // an odd tail k-step multiplies the zero columns
+  const uint32_t a_lane = (16u * ot + l16) * kRowPitch + g;
+  const uint32_t b_lane = (16u * ct + l16) * kRowPitch + g;
+
+  // one output row: dyr = its dy slot, b0/b1/b2 = the slab rows r, r + DIL, r + 2 DIL
+  auto compute_row = [&](const float *dyr, const float *b0, const float *b1, const float *b2) {
+    float a[2], b[2][9];
+    auto read_operands = [&](int buf, uint32_t ks) {
+      const uint32_t col = 4u * ks;
+      a[buf] = dyr[a_lane + col];
+#pragma unroll
+      for (int kw = 0; kw < 3; ++kw) {
+        b[buf][0 + kw] = b0[b_lane + col + kw * DIL];
+        b[buf][3 + kw] = b1[b_lane + col + kw * DIL];
+        b[buf][6 + kw] = b2[b_lane + col + kw * DIL];
+      }
+    };
+    auto step = [&](int cur, uint32_t next_ks) {
+      read_operands(cur ^ 1, next_ks);
+#pragma unroll
+      for (int tap = 0; tap < 9; ++tap)
+        acc[tap] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[cur], b[cur][tap], acc[tap], 0, 0, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // the A read
+#pragma unroll
+      for (int tap = 0; tap < 9; ++tap) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    read_operands(0, 0);
+    const uint32_t last = 2u * npairs - 1u;
+    for (uint32_t kp = 0; kp < npairs; ++kp) {
+      step(0, 2u * kp + 1u);
+      step(1, min(2u * kp + 2u, last));  // the final prefetch is not used; keep it in range
+    }
+  };
+
+  // phase PH = (r - r0) mod NS: slab row y of the chunk lives in slot (y - r0) mod NS
+  auto phase = [&](auto tag, uint32_t r) {
+    constexpr int PH = decltype(tag)::value;
+    if (r + 1u < r1) {
+      stage_x_row(xs[(PH + 2 * DIL + 1) % NS], r + 2u * DIL + 1u);
+      stage_dy_row(dys[(PH + 1) & 1], r + 1u);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    compute_row(dys[PH & 1], xs[PH], xs[(PH + DIL) % NS], xs[(PH + 2 * DIL) % NS]);
+    __syncthreads();
+  };
+
+  const uint32_t plane0 = pgroup * P.planes_per_block;
+  const uint32_t plane1 = min(plane0 + P.planes_per_block, P.num_tiles * P.N);
+  for (uint32_t plane = plane0; plane < plane1; ++plane) {
+    open_plane(plane);
+    // prologue: slab rows r0 .. r0 + 2 DIL -> slots 0 .. 2 DIL and dy row r0 -> slot 0
+#pragma unroll
+    for (int y = 0; y <= 2 * DIL; ++y) stage_x_row(xs[y], r0 + (uint32_t)y);
+    stage_dy_row(dys0, r0);
+    __syncthreads();
+    for (uint32_t r = r0;;) {
+      phase(WgPhase<0>(), r);
+      if (++r == r1) break;
+      phase(WgPhase<1>(), r);
+      if (++r == r1) break;
+      phase(WgPhase<2>(), r);
+      if (++r == r1) break;
+      phase(WgPhase<3>(), r);
+      if (++r == r1) break;
+      phase(WgPhase<4>(), r);
+      if (++r == r1) break;
+      phase(WgPhase<5>(), r);
+      if (++r == r1) break;
+      phase(WgPhase<6>(), r);
+      if (++r == r1) break;
+      phase(WgPhase<7>(), r);
+      if (++r == r1) break;
+    }
+  }
+
+  // ---- epilogue: lane holds D[co = 4g+i][ci = l16] of each tap tile ----
+  const uint32_t block_lin = blockIdx.y * gridDim.x + blockIdx.x;
+  float *__restrict__ part = P.partial + (uint64_t)block_lin * kPartialFloats;
+#pragma unroll
+  for (int tap = 0; tap < 9; ++tap)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t co_l = 16u * ot + 4u * g + i, ci_l = 16u * ct + l16;
+      part[(co_l * 64u + ci_l) * 9u + tap] = acc[tap][i];
+    }
+}
+
 // dw[co][ci][tap] = beta*dw + sum over the pixel-chunk partials of its (co half, ci group), in
 // a fixed order (deterministic): 4 lanes-groups each sum a quarter of the partials, then the
 // quarters are combined through LDS in index order.
@@ -384,6 +580,78 @@ static bool wgrad_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Co
   plan->groups = groups;
   plan->workspace_bytes = (size_t)plan->blocks_x * groups * kPartialFloats * sizeof(float);
   return true;
+}
+
+
+// the plan of the dilated kernel: column tiles of at most kMaxWDil pixels, one workgroup per CU
+static bool wgrad_dil_plan(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, uint32_t dil,
+                           WgradPlan *plan) {
+  if (dil != 3u || num_tiles == 0 || N == 0 || Cin == 0 || Cout == 0 || H == 0 || W == 0) return false;
+  const uint64_t planes = (uint64_t)num_tiles * N;
+  const uint32_t groups = ((Cin + 63u) / 64u) * ((Cout + 31u) / 32u);
+  if (groups > 65535u) return false;
+  const uint32_t col_tiles = (W + kMaxWDil - 1) / kMaxWDil;
+  const uint32_t cols = (W + col_tiles - 1) / col_tiles;
+  uint32_t chunks = 1, ppb = 1;
+  wgrad_plan_rows(planes, (uint64_t)col_tiles * groups, H, cols, 1u, &chunks, &ppb);
+  const uint64_t blocks_x = ((planes + ppb - 1) / ppb) * chunks * col_tiles;
+  if (blocks_x > 0x7fffffffull) return false;
+  if ((uint64_t)Cin * (H + 2ull * dil) * (W + 2ull * dil) * 4u >= (1ull << 31) || (uint64_t)Cout * H * W * 4u >= (1ull << 31) ||
+      (uint64_t)Cin * Cout * 9u >= (1ull << 31))
+    return false;
+  plan->rows_per_block = (H + chunks - 1) / chunks;
+  plan->chunks_per_plane = chunks;
+  plan->planes_per_block = ppb;
+  plan->cols_per_block = cols;
+  plan->col_tiles = col_tiles;
+  plan->narrow = false;
+  plan->blocks_x = (uint32_t)blocks_x;
+  plan->groups = groups;
+  plan->workspace_bytes = (size_t)plan->blocks_x * groups * kPartialFloats * sizeof(float);
+  return true;
+}
+
+// The filter gradient of the 3x3 window at stride 1 with dilation 3 over fp32 tiles padded by 3 (the reference's
+// tools/microbench_spatial_conv.cc:25-32).  H, W: the interior (= dy) extents.  Workspace 0 / ADH_EUNIMPL (and
+// nothing launched) for another dilation and for images beyond a buffer resource's 2 GiB: the general kernel serves
+// those.  Arguments are the caller's, already validated.
+size_t conv3x3_dilated_wgrad_workspace(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W,
+                                       uint32_t dil) {
+  WgradPlan plan;
+  return wgrad_dil_plan(num_tiles, N, Cin, Cout, H, W, dil, &plan) ? plan.workspace_bytes : 0;
+}
+int conv3x3_dilated_wgrad_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H, uint32_t W, uint32_t dil,
+                              const void *const *x_tiles, const void *const *dy_tiles, float *dw, float beta, void *workspace,
+                              hipStream_t st) {
+  WgradPlan plan;
+  if (!wgrad_dil_plan(num_tiles, N, Cin, Cout, H, W, dil, &plan)) return ADH_EUNIMPL;
+  WgradParams P = {};
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    P.x[t] = reinterpret_cast<const float *>(x_tiles[t]);
+    P.dy[t] = reinterpret_cast<const float *>(dy_tiles[t]);
+  }
+  P.partial = reinterpret_cast<float *>(workspace);
+  P.num_tiles = num_tiles; P.N = N; P.Cin = Cin; P.Cout = Cout; P.H = H; P.W = W;
+  P.rows_per_block = plan.rows_per_block;
+  P.chunks_per_plane = plan.chunks_per_plane;
+  P.planes_per_block = plan.planes_per_block;
+  P.cols_per_block = plan.cols_per_block;
+  P.col_tiles = plan.col_tiles;
+  P.div_cols = FastDiv(plan.col_tiles);
+  P.ci_groups = (Cin + 63u) / 64u;
+  P.div_chunks = FastDiv(plan.chunks_per_plane);
+  P.div_tiles = FastDiv(num_tiles);
+  P.div_ci_groups = FastDiv(P.ci_groups);
+  hipLaunchKernelGGL(conv3x3_wgrad_dil_f32_kernel<3>, dim3(plan.blocks_x, plan.groups, 1), dim3(kWgThreads), 0, st, P);
+  int e = launch_status();
+  if (e) return e;
+  WgradReduceParams R = {};
+  R.partial = P.partial; R.dw = dw; R.Cin = Cin; R.Cout = Cout;
+  R.blocks_x = plan.blocks_x; R.ci_groups = P.ci_groups; R.beta = beta;
+  R.total = Cin * Cout * 9u;
+  R.div9 = FastDiv(9); R.div_cin = FastDiv(Cin);
+  hipLaunchKernelGGL(conv3x3_wgrad_reduce_kernel, dim3((R.total + 63u) / 64u), dim3(256), 0, st, R);
+  return launch_status();
 }
 
 size_t bf16_workspace_bytes(int which, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t H,

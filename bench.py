@@ -567,7 +567,7 @@ def main():
             "hbm", 3 * 2 * (Kd - 1) * strip_d, HBM_PEAK_GBS, "GB/s",
             extra=lambda ms: {"reference_figure_GBs": round(strip_d / (ms * 1e-3) / 1e9, 3)})
         reps, wu = 10, 3
-        add("reference microbench_spatial_conv: conv fwd 3x3 dilation 3 over halo 3 (fp32, 4 tiles, general kernel)",
+        add("reference microbench_spatial_conv: conv fwd 3x3 dilation 3 over halo 3 (fp32, 4 tiles; the 3x3 kernel with its taps three apart)",
             lambda: lib.adh_conv2d_slab_fwd_tiles(0, Kd, Nd, C, C, HPd, WPd, *geo_d, xd_tbl, wd.data_ptr(), yd_tbl, 0.0,
                                                   wsd.data_ptr(), wsd_bytes, stream),
             "mfma", fl_d, MFMA_F32_PEAK_TFLOPS, "TFLOP/s")

@@ -316,9 +316,10 @@ int adh_conv_bwd_bias_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t 
  * fp32 arithmetic on the matrix cores; ADH_BF16 tensors are widened on load and rounded on store.
  * The workspace (adh_conv2d_workspace_bytes, 256-byte aligned) holds the rewritten filter and, for thin
  * launches whose channel chunks are dealt to several workgroups, their fp32 partial sums (added in a
- * fixed order by a second kernel: results are reproducible).  In fp32, 1x1 windows at stride 1 or 2 and windows
- * over at most three input channels (a stem) are served by kernels of their own behind these entry points, chosen
- * by shape and alignment; arguments, workspace query and error codes are the same for every shape. */
+ * fixed order by a second kernel: results are reproducible).  In fp32, 1x1 windows at stride 1 or 2, windows
+ * over at most three input channels (a stem) and the 3x3 window at stride 1 with dilation 3 (the reference's
+ * microbenchmark) are served by kernels of their own behind these entry points, chosen by shape and alignment;
+ * arguments, workspace query and error codes are the same for every shape. */
 size_t adh_conv2d_workspace_bytes(int which, int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin,
                                   uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t kh, uint32_t kw,
                                   uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw);

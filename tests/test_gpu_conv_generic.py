@@ -43,6 +43,9 @@ CASES = [  # K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw
     (1, 2, 3, 64, 22, 70, 7, 7, 1, 1, 1, 1),     # the stem on 16x64 outputs: two row blocks and two column blocks, 16-byte stores
     (3, 2, 3, 70, 14, 45, 7, 7, 1, 1, 1, 1),     # 39 output columns (stores element by element), 64 + 6 output channels
     (2, 3, 1, 20, 19, 71, 3, 3, 2, 2, 1, 1),     # one input channel, stride 2
+    # 3x3 at dilation 3 over halo 3 on launches of at least 256 workgroups: the 3x3 kernels with their taps three apart
+    (2, 16, 20, 70, 40, 70, 3, 3, 1, 1, 3, 3),   # a ragged channel chunk, 64 + 6 output channels, two column tiles
+    (1, 130, 8, 64, 23, 37, 3, 3, 1, 1, 3, 3),   # one column tile narrower than the patch, a short last row tile
 ]
 
 
