@@ -517,7 +517,7 @@ static int conv_direct_kernel_name(int which, uint32_t num_tiles, uint32_t N, ui
   if (tile.nt == 0) return ADH_EINVAL;
   const int waves = tile.nt == 8 ? 4 : 8;
   const int prows = patch_rows_for(tile.nt, tile.R);
-  snprintf(name, name_bytes, "conv3x3_f32_kernel<%d, %d, %s, %d>", tile.nt, waves, which == ADH_CONV_FWD ? "false" : "true", prows);
+  snprintf(name, name_bytes, "conv3x3_f32_kernel<%d, %d, %s, %d, 1>", tile.nt, waves, which == ADH_CONV_FWD ? "false" : "true", prows);
   return ADH_OK;
 }
 
