@@ -63,6 +63,7 @@ SIGNATURES = {
     "adh_conv_bwd_bias_tiles": (i32, [i32, u32, u32, u32, u32, u32, vpp, vp, f32, vp, sz, vp]),
     "adh_conv2d_workspace_bytes": (sz, [i32, i32] + [u32] * 12),
     "adh_conv2d_slab_fwd_tiles": (i32, [i32] + [u32] * 12 + [vpp, vp, vpp, f32, vp, sz, vp]),
+    "adh_conv2d_slab_fwd_bias_tiles": (i32, [i32] + [u32] * 12 + [vpp, vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv2d_slab_bwd_data_tiles": (i32, [i32] + [u32] * 12 + [vp, vpp, vpp, f32, vp, sz, vp]),
     "adh_conv2d_slab_bwd_filter_tiles": (i32, [i32] + [u32] * 12 + [vpp, vpp, vp, f32, vp, sz, vp]),
     "adh_conv2d_unpadded_workspace_bytes": (sz, [i32, i32] + [u32] * 14),
@@ -346,6 +347,17 @@ def conv2d_fwd_tiles(xs, w, ys, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, be
     wp, wb = _ws(ws)
     return lib().adh_conv2d_slab_fwd_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, xt,
                                            w.data_ptr(), yt, beta, wp, wb, _stream())
+
+
+def conv2d_fwd_bias_tiles(xs, w, biases, ys, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, beta=0.0, ws=None):
+    """conv2d_fwd_tiles followed by ys[t] += biases[t] per channel, in the convolution's stores where its kernel can."""
+    _dev(*xs, w, *biases, *ys)
+    xt, k1 = _tbl(xs)
+    bt, k3 = _tbl(biases)
+    yt, k2 = _tbl(ys)
+    wp, wb = _ws(ws)
+    return lib().adh_conv2d_slab_fwd_bias_tiles(_dt(xs[0]), len(xs), N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, xt,
+                                                w.data_ptr(), bt, yt, beta, wp, wb, _stream())
 
 
 def conv2d_bwd_data_tiles(w, dys, dxs, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, beta=0.0, ws=None):

@@ -617,7 +617,7 @@ int conv3x3_dilated_wgrad_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint
 // conv_thin.hip: forward over halo-padded fp32 tiles for at most three input channels (a network's stem)
 int conv_thin_fwd_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t OH,
                       uint32_t OW, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, const void *const *x_tiles,
-                      const void *w, void *const *y_tiles, float beta, hipStream_t st);
+                      const void *w, void *const *y_tiles, float beta, hipStream_t st, const float *const *bias_tiles);
 
 size_t conv_thin_wgrad_workspace(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP,
                                  uint32_t OH, uint32_t OW, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw);
@@ -1208,7 +1208,8 @@ size_t conv2d_workspace(int which, int dtype, uint32_t num_tiles, uint32_t N, ui
 int conv2d_fwd(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP,
                uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw, bool unpadded, uint32_t pad_h,
                uint32_t pad_w, const void *const *x_tiles, const void *w, void *const *y_tiles, float beta, void *workspace,
-               size_t workspace_bytes, void *stream) {
+               size_t workspace_bytes, void *stream, const float *const *bias_tiles = nullptr, bool *bias_added = nullptr) {
+  // bias_tiles: added by the launch itself where the kernel that serves the shape can (*bias_added says so)
   if (!dtype_ok(dtype)) return ADH_EINVAL;
   GenShape g;
   int e = gen_check_shape(num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, &g);
@@ -1241,7 +1242,8 @@ int conv2d_fwd(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t
     e = gen_check_workspace(plan, workspace, workspace_bytes);
     if (e) return e;
     e = conv_thin_fwd_try(num_tiles, N, Cin, Cout, g.HP, g.WP, g.OH, g.OW, kh, kw, sh, sw, x_tiles, w, y_tiles, beta,
-                          as_stream(stream));
+                          as_stream(stream), bias_tiles);
+    if (e == ADH_OK && bias_tiles && bias_added) *bias_added = true;
     if (e != ADH_EUNIMPL) return e;
   }
   if (gen_is_3x3_dilated(dtype, g, unpadded)) {
@@ -1407,6 +1409,25 @@ int adh_conv2d_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_
                               void *workspace, size_t workspace_bytes, void *stream) {
   return conv2d_fwd(dtype, num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, false, 0, 0, x_pad_tiles, w, y_tiles, beta,
                     workspace, workspace_bytes, stream);
+}
+
+int adh_conv2d_slab_fwd_bias_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,
+                                   uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, uint32_t dh, uint32_t dw,
+                                   const void *const *x_pad_tiles, const void *w, const float *const *bias_tiles,
+                                   void *const *y_tiles, float beta, void *workspace, size_t workspace_bytes, void *stream) {
+  if (!bias_tiles) return ADH_ENULL;
+  if (num_tiles == 0 || num_tiles > ADH_MAX_TILES) return ADH_EINVAL;
+  for (uint32_t t = 0; t < num_tiles; ++t) {
+    if (!bias_tiles[t]) return ADH_ENULL;
+    if (!aligned_to(bias_tiles[t], 4)) return ADH_EALIGN;
+  }
+  bool added = false;
+  const int e = conv2d_fwd(dtype, num_tiles, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw, false, 0, 0, x_pad_tiles, w, y_tiles,
+                           beta, workspace, workspace_bytes, stream, bias_tiles, &added);
+  if (e != ADH_OK || added || N == 0 || Cout == 0) return e;
+  // the shape has been checked by the convolution: the output extents follow from it
+  const uint32_t OH = (HP - ((kh - 1u) * dh + 1u)) / sh + 1u, OW = (WP - ((kw - 1u) * dw + 1u)) / sw + 1u;
+  return adh_conv_bias_add_tiles(dtype, num_tiles, N, Cout, OH, OW, bias_tiles, y_tiles, stream);
 }
 
 int adh_conv2d_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP,

@@ -26,6 +26,7 @@ struct ThinParams {
   const float *x[ADH_MAX_TILES];
   float *y[ADH_MAX_TILES];
   const float *w;
+  const float *bias[ADH_MAX_TILES];  // forward: added to every pixel of its output channel after beta * y; null: none
   uint32_t N, C, M, HP, WP, OH, OW, kh, kw, sh, sw;
   uint32_t KK;            // C * kh * kw pairs
   uint32_t PRH, PRW, PP;  // patch rows, columns, floats per channel
@@ -95,6 +96,7 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_fwd_kernel(const Th
   const float *b_base = wl + g * kThinWPitch + wm * 32u + l16;
 
   float *y = P.y[tile] + (size_t)n * P.M * P.OH * P.OW;
+  const float *const bias_t = P.bias[tile];
   // a tile's patch: PJ elements per thread, loaded a tile ahead (in flight while the tile before is multiplied)
   const uint32_t total = P.C * P.PP;
   float ptmp[PJ];
@@ -163,13 +165,19 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_fwd_kernel(const Th
         if (m >= P.M) continue;
         float *o = y + ((size_t)m * P.OH + row) * P.OW + col;
         thin_floatx4 v = acc[pt][ct];
+        const float bias = bias_t ? bias_t[m] : 0.f;
         if (VEC) {
           if (P.beta != 0.f) v += *reinterpret_cast<const thin_floatx4 *>(o);
+          if (bias_t) v += bias;
           *reinterpret_cast<thin_floatx4 *>(o) = v;
         } else {
 #pragma unroll
           for (int k = 0; k < 4; ++k)
-            if (col + (uint32_t)k < P.OW) o[k] = P.beta != 0.f ? o[k] + v[k] : v[k];
+            if (col + (uint32_t)k < P.OW) {
+              float e = P.beta != 0.f ? o[k] + v[k] : v[k];
+              if (bias_t) e += bias;
+              o[k] = e;
+            }
         }
       }
     }
@@ -177,10 +185,12 @@ __global__ __launch_bounds__(kThinThreads, 2) void conv_thin_fwd_kernel(const Th
 }
 
 // Forward over halo-padded fp32 tiles of HP x WP for at most three input channels and Cin kh kw <= 148, any stride,
-// no dilation.  ADH_EUNIMPL: not a shape this kernel serves; nothing launched.
+// no dilation; bias_tiles (or null): one vector of Cout floats per tile, added in the stores (y = beta * y + conv +
+// bias, the order of a separate add after the convolution).  ADH_EUNIMPL: not a shape this kernel serves; nothing
+// launched.
 int conv_thin_fwd_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout, uint32_t HP, uint32_t WP, uint32_t OH,
                       uint32_t OW, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw, const void *const *x_tiles,
-                      const void *w, void *const *y_tiles, float beta, hipStream_t st) {
+                      const void *w, void *const *y_tiles, float beta, hipStream_t st, const float *const *bias_tiles) {
   if (Cin == 0 || Cin > 3u || Cin * kh * kw > kThinK) return ADH_EUNIMPL;
   if (!aligned_to(w, 4)) return ADH_EUNIMPL;
   bool vec = OW % 4u == 0u;
@@ -192,6 +202,7 @@ int conv_thin_fwd_try(uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cou
   for (uint32_t t = 0; t < num_tiles; ++t) {
     P.x[t] = reinterpret_cast<const float *>(x_tiles[t]);
     P.y[t] = reinterpret_cast<float *>(y_tiles[t]);
+    P.bias[t] = bias_tiles ? bias_tiles[t] : nullptr;
   }
   P.w = reinterpret_cast<const float *>(w);
   P.N = N; P.C = Cin; P.M = Cout; P.HP = HP; P.WP = WP; P.OH = OH; P.OW = OW;

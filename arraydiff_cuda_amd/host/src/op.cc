@@ -566,6 +566,14 @@ void SlabConv2DOp<V3, A4>::_forward(TxnId txn) {
     } else {
       size_t ws_bytes;
       void *ws = conv_scratch(dc, ADH_CONV_FWD, n, d, shape_, &ws_bytes);
+      if (!biases_.empty()) {
+        // the bias in the convolution's stores where its kernel can (the stem), else added after it by the library
+        adh_check(adh_conv2d_slab_fwd_bias_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, ADH_CONV_GEOMETRY(d, shape_),
+                                                 xt, w0, bt, yt, 0.0f, ws, ws_bytes, conn.stream()),
+                  "SlabConv2DOp::_forward (general, bias)");
+        todo.swap(rest);
+        continue;
+      }
       adh_check(adh_conv2d_slab_fwd_tiles(ADH_F32, n, d.N, d.C, (uint32_t)shape_.filters, ADH_CONV_GEOMETRY(d, shape_),
                                           xt, w0, yt, 0.0f, ws, ws_bytes, conn.stream()),
                 "SlabConv2DOp::_forward (general)");

@@ -330,6 +330,16 @@ int adh_conv2d_slab_fwd_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_
                               uint32_t dh, uint32_t dw, const void *const *x_pad_tiles, const void *w,
                               void *const *y_tiles, float beta, void *workspace, size_t workspace_bytes,
                               void *stream);
+/* The same followed by the bias (cudnnConvolutionForward + cudnnAddTensor, src/op.cc:1576-1610):
+ * y = beta*y + conv(x_pad, w) + bias[co], bias_tiles one fp32 vector of Cout per tile (entries may repeat).  Where the
+ * kernel that serves the shape can, the bias is added in its stores (windows over at most three input channels: a
+ * network's stem); elsewhere adh_conv_bias_add_tiles follows the convolution on the same stream.  Either way the
+ * result has the bits of the two separate calls. */
+int adh_conv2d_slab_fwd_bias_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,
+                                   uint32_t HP, uint32_t WP, uint32_t kh, uint32_t kw, uint32_t sh, uint32_t sw,
+                                   uint32_t dh, uint32_t dw, const void *const *x_pad_tiles, const void *w,
+                                   const float *const *bias_tiles, void *const *y_tiles, float beta,
+                                   void *workspace, size_t workspace_bytes, void *stream);
 /* cudnnConvolutionBackwardData at src/op.cc:1701-1712: the adjoint of the above, written over the
  * WHOLE padded tile (padded pixels that no window reads get beta*dx_pad) */
 int adh_conv2d_slab_bwd_data_tiles(int dtype, uint32_t num_tiles, uint32_t N, uint32_t Cin, uint32_t Cout,

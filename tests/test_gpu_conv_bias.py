@@ -90,3 +90,55 @@ def test_conv_bias_argument_errors():
     assert L.adh_conv_bwd_bias_tiles(capi.ADH_F32, 1, 1, 2, 2, 2, yt, db.data_ptr(), 0.0, small.data_ptr(), 4, None) == capi.ADH_EWORKSPACE
     assert L.adh_conv_bwd_bias_tiles(capi.ADH_F32, 1, 1, 2, 2, 2, nul, db.data_ptr(), 0.0, ws.data_ptr(), 4096, None) == capi.ADH_ENULL
     torch.cuda.synchronize()
+
+
+# K, N, Cin, Cout, HP, WP, kh, kw, sh, sw: the stem's shapes (at most three input channels: the bias goes into the
+# convolution's stores; 16-byte and element-wise stores, a channel remainder) and one the general kernel serves
+# (the add follows the convolution inside the library)
+FUSED_CASES = [(2, 2, 3, 64, 22, 70, 7, 7, 1, 1), (3, 2, 3, 70, 14, 45, 7, 7, 1, 1), (2, 3, 1, 20, 19, 71, 3, 3, 2, 2),
+               (2, 2, 3, 64, 20, 38, 7, 7, 2, 2), (2, 2, 16, 24, 10, 30, 3, 3, 2, 2)]
+
+
+@pytest.mark.parametrize("K,N,Cin,Cout,HP,WP,kh,kw,sh,sw", FUSED_CASES)
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+def test_conv_fwd_with_bias_equals_conv_then_bias(K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, beta):
+    """adh_conv2d_slab_fwd_bias_tiles has the bits of adh_conv2d_slab_fwd_tiles followed by adh_conv_bias_add_tiles
+    (which the tests above and tests/test_gpu_conv_generic.py hold against the oracle)."""
+    rng = np.random.default_rng(500 + Cout + WP)
+    OH, OW = (HP - kh) // sh + 1, (WP - kw) // sw + 1
+    xs = [dev(rng.uniform(-1, 1, (N, Cin, HP, WP)).astype(np.float32)) for _ in range(K)]
+    w = dev((rng.standard_normal((Cout, Cin, kh, kw)) * 0.1).astype(np.float32))
+    bs = [dev(rng.uniform(-1, 1, Cout).astype(np.float32)) for _ in range(K)]
+    y0 = [rng.standard_normal((N, Cout, OH, OW)).astype(np.float32) for _ in range(K)]
+    nbytes = capi.lib().adh_conv2d_workspace_bytes(capi.ADH_CONV_FWD, capi.ADH_F32, K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, 1, 1)
+    ws = torch.empty(nbytes // 4 + 64, device="cuda")
+    want = [dev(a) for a in y0]
+    capi.check(capi.conv2d_fwd_tiles(xs, w, want, N, Cin, Cout, HP, WP, kh, kw, sh, sw, 1, 1, beta=beta, ws=ws), "conv")
+    capi.check(capi.conv_bias_add_tiles(bs, want, N, Cout, OH, OW), "bias")
+    got = [dev(a) for a in y0]
+    capi.check(capi.conv2d_fwd_bias_tiles(xs, w, bs, got, N, Cin, Cout, HP, WP, kh, kw, sh, sw, 1, 1, beta=beta, ws=ws), "conv + bias")
+    for t in range(K):
+        assert np.array_equal(host(got[t]), host(want[t]))
+    # the bias took part: the result differs from the convolution alone wherever the bias is not zero
+    plain = [dev(a) for a in y0]
+    capi.check(capi.conv2d_fwd_tiles(xs, w, plain, N, Cin, Cout, HP, WP, kh, kw, sh, sw, 1, 1, beta=beta, ws=ws), "conv")
+    assert not np.array_equal(host(got[0]), host(plain[0]))
+
+
+def test_conv_fwd_with_bias_argument_errors():
+    x = torch.zeros((1, 3, 9, 9), device="cuda")
+    w = torch.zeros((4, 3, 3, 3), device="cuda")
+    y = torch.zeros((1, 4, 7, 7), device="cuda")
+    b = torch.zeros(4, device="cuda")
+    ws = torch.zeros(1 << 16, device="cuda")
+    L = capi.lib()
+    xt, k1 = capi.ptr_table([x.data_ptr()])
+    yt, k2 = capi.ptr_table([y.data_ptr()])
+    bt, k3 = capi.ptr_table([b.data_ptr()])
+    nul, k4 = capi.ptr_table([None])
+    args = (capi.ADH_F32, 1, 1, 3, 4, 9, 9, 3, 3, 1, 1, 1, 1, xt, w.data_ptr())
+    tail = (yt, 0.0, ws.data_ptr(), ws.numel() * 4, None)
+    assert L.adh_conv2d_slab_fwd_bias_tiles(*args, None, *tail) == capi.ADH_ENULL
+    assert L.adh_conv2d_slab_fwd_bias_tiles(*args, nul, *tail) == capi.ADH_ENULL
+    assert L.adh_conv2d_slab_fwd_bias_tiles(*args, bt, *tail) == capi.ADH_OK
+    torch.cuda.synchronize()
