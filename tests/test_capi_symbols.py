@@ -57,3 +57,28 @@ def test_argument_errors_need_no_gpu():
     assert q(0, capi.ADH_POOL_MAX, 4, 32, 64, 64, 8192, 3, 3, 2, 2, 1, 1) == capi.ADH_EUNIMPL  # rows too wide for a band in LDS
     assert q(0, capi.ADH_POOL_MAX, 4, 32, 64, 63, 256, 3, 3, 2, 2, 1, 1) == capi.ADH_EINVAL    # the row split does not stitch
     assert l.adh_conv_bwd_bias_workspace_bytes(4, 32, 64) > 0
+
+
+def test_bf16_conv_workspace_holds_the_sums_of_every_route_that_needs_them():
+    """More than 64 reduction channels at a width the eight-wave kernels do not take run one launch per 64 channels
+    with fp32 sums between them: the workspace query has to count those sums whatever one launch of 128 channels
+    would have needed at a friendlier width (host logic only, no GPU)."""
+    l = capi.lib()
+    group = 9 * 2 * 64 * 32 * 2  # bytes of the reordered filter per (64 outputs, 64 reduction channels)
+
+    def need(which, K, N, Cin, Cout, H, W):
+        cred, cout = (Cin, Cout) if which == capi.ADH_CONV_FWD else (Cout, Cin)
+        oh, ow = (H, W) if which == capi.ADH_CONV_FWD else (H + 2, W + 2)
+        filt = ((cout + 63) // 64) * ((cred + 63) // 64) * group
+        part = K * ((N * cout * oh * ow * 4 + 255) // 256 * 256)
+        return filt, part
+
+    for (K, N, Cin, Cout, H, W) in [(2, 1, 128, 128, 9, 7), (1, 2, 100, 70, 5, 13), (3, 1, 65, 65, 3, 1), (1, 1, 128, 96, 4, 27)]:
+        for which in (capi.ADH_CONV_FWD, capi.ADH_CONV_BWD_DATA):
+            filt, part = need(which, K, N, Cin, Cout, H, W)
+            got = l.adh_conv3x3_workspace_bytes(which, capi.ADH_BF16, K, N, Cin, Cout, H, W)
+            assert got >= filt + part, (which, K, N, Cin, Cout, H, W, got, filt, part)
+    # one launch of 128 channels (even width forward, a multiple of 8 backward): the filter alone
+    for which in (capi.ADH_CONV_FWD, capi.ADH_CONV_BWD_DATA):
+        filt, part = need(which, 2, 1, 128, 128, 9, 72)
+        assert l.adh_conv3x3_workspace_bytes(which, capi.ADH_BF16, 2, 1, 128, 128, 9, 72) == filt
