@@ -46,6 +46,8 @@ CASES = [  # K, N, Cin, Cout, HP, WP, kh, kw, sh, sw, dh, dw
     # 3x3 at dilation 3 over halo 3 on launches of at least 256 workgroups: the 3x3 kernels with their taps three apart
     (2, 16, 20, 70, 40, 70, 3, 3, 1, 1, 3, 3),   # a ragged channel chunk, 64 + 6 output channels, two column tiles
     (1, 130, 8, 64, 23, 37, 3, 3, 1, 1, 3, 3),   # one column tile narrower than the patch, a short last row tile
+    (1, 300, 8, 8, 7, 7, 3, 3, 1, 1, 3, 3),      # a single output pixel per image, 300 workgroups
+    (1, 140, 9, 130, 12, 20, 3, 3, 1, 1, 3, 3),  # three groups of output channels (the last holds 2), 9 input channels
 ]
 
 
