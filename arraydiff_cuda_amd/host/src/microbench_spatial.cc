@@ -12,6 +12,12 @@
 //                         backward-filter and one backward-data convolution per rank, sync, reduce sequence, sync
 //                         (:394-477); average wall-clock milliseconds per trial, as printed there
 //
+//   --which conv          tools/microbench_conv.cc:16-241: one device, N=32, 64 -> 64 channels, a 3x3 convolution
+//                         forward over a 64(+2) x 128(+2) halo-padded source, 1000 trials of (launch, stream
+//                         synchronise), average wall clock and "est flops" 2*N*Co*Ci*H*W*9 (:53, :180-240).  The
+//                         reference writes the result into the interior of a halo-padded destination through a
+//                         strided descriptor (:41-44); here it lands in a packed tensor.
+//
 // The reference's first two loops pass src_width = W + 2*halo as base_width (:246, :291), which indexes past
 // buf_size (:43); every loop here passes the interior width.  cuDNN's three convolution calls become the C ABI's
 // adh_conv2d_slab_{fwd,bwd_filter,bwd_data}_tiles with one tile per call.
@@ -21,7 +27,7 @@
 // synchronisation between exchange and convolution (one in-order stream is the barrier).  Each line printed is
 // one JSON object; the last line is the summary bench.py reads.
 //
-//   microbench_spatial --which spatial|spatial_conv [--ranks K] [--trials T] [--batch N]
+//   microbench_spatial --which spatial|spatial_conv|conv [--ranks K] [--trials T] [--batch N]
 #include <chrono>
 #include <cmath>
 #include <cstdio>
@@ -141,12 +147,13 @@ int main(int argc, char **argv) {
       return 2;
     }
   }
-  if ((which != "spatial" && which != "spatial_conv") || ranks == 0 || ranks > ADH_MAX_TILES || batch == 0 || argc % 2 == 0) {
-    std::fprintf(stderr, "usage: microbench_spatial --which spatial|spatial_conv [--ranks K] [--trials T] [--batch N]\n");
+  if ((which != "spatial" && which != "spatial_conv" && which != "conv") || ranks == 0 || ranks > ADH_MAX_TILES || batch == 0 ||
+      argc % 2 == 0) {
+    std::fprintf(stderr, "usage: microbench_spatial --which spatial|spatial_conv|conv [--ranks K] [--trials T] [--batch N]\n");
     return 2;
   }
   try {
-    const uint32_t K = (uint32_t)ranks, N = (uint32_t)batch, C = 64;
+    const uint32_t K = which == "conv" ? 1u : (uint32_t)ranks, N = (uint32_t)batch, C = 64;  // microbench_conv.cc:20: one device
     auto ctx = MultiGPUContext::Make(K);
     std::vector<Spatial2DComm> comms(K);
     check(Spatial2DComm::InitAll(comms.data(), 1, K), "InitAll");
@@ -176,6 +183,36 @@ int main(int argc, char **argv) {
       std::printf("{\"which\": \"spatial\", \"ranks\": %u, \"trials\": %d, \"halo\": %u, \"n\": %u, \"c\": %u, \"h\": %u, \"w\": %u, "
                   "\"exchange_per_rank_sequence_ms\": %.5f, \"exchange_one_launch_ms\": %.5f}\n",
                   K, trials, p, N, C, H, W, seq.avg_ms, one.avg_ms);
+      return 0;
+    }
+
+    if (which == "conv") {
+      // microbench_conv.cc:22-53
+      const uint32_t W = 128, H = 128 / 2;
+      if (trials < 0) trials = 1000;  // :180
+      const size_t src = (size_t)(W + 2) * (H + 2) * C * N, dst = (size_t)W * H * C * N, wsz = (size_t)9 * C * C;
+      GPUContext *dc = ctx->device_context(0).get();
+      GPUConn conn = dc->conn();
+      GPUMemory<float> x(src, dc), y(dst, dc), w(wsz, dc);
+      {
+        std::vector<float> host(src);
+        fill_uniform(host, 1);
+        x.load_sync(host.data(), 0, src, conn);
+        host.resize(wsz);
+        fill_uniform(host, 7);
+        const float scale = std::sqrt(2.0f / (C * 9));
+        for (auto &v : host) v *= scale;
+        w.load_sync(host.data(), 0, wsz, conn);
+      }
+      ctx->sync();
+      const double flops = 2.0 * N * C * C * (double)H * W * 9.0;  // :53
+      const Stat one = time_trials(ctx.get(), trials, [&] {
+        check(adh_conv3x3_slab_fwd(ADH_F32, N, C, C, H, W, x.dptr(), w.dptr(), y.dptr(), 0.0f, nullptr, 0, conn.stream()), "conv fwd");
+        dc->sync();  // :227-230
+      });
+      std::printf("{\"which\": \"conv\", \"name\": \"conv forward over a halo-padded source\", \"trials\": %d, \"n\": %u, \"c\": %u, "
+                  "\"h\": %u, \"w\": %u, \"avg_wallclock_ms\": %.5f, \"std_ms\": %.5f, \"est_gflop\": %.3f, \"tflops\": %.2f}\n",
+                  trials, N, C, H, W, one.avg_ms, one.std_ms, flops * 1e-9, flops * 1e-12 / (one.avg_ms * 1e-3));
       return 0;
     }
 

@@ -164,7 +164,7 @@ def main():
         else:
             print("bench.py: the graph-replay run of the trainer failed:\n" + g.stdout[-1000:] + g.stderr[-1000:], file=sys.stderr)
 
-    # The reference's own microbenchmarks (tools/microbench_spatial.cc, tools/microbench_spatial_conv.cc) as a C++
+    # The reference's own microbenchmarks (tools/microbench_spatial.cc, tools/microbench_spatial_conv.cc, tools/microbench_conv.cc) as a C++
     # binary over this library's Spatial2DComm and C ABI, also a child process: per rank group_start / halo_* /
     # group_end with the reference's synchronisations, beside one launch for all ranks' tiles; wall-clock averages.
     reference_microbench = None
@@ -175,7 +175,7 @@ def main():
             print("bench.py: %s is not built (run __graft_entry__.build())" % micro, file=sys.stderr)
             sys.exit(3)
         reference_microbench = []
-        for which, trials in (("spatial", "1000"), ("spatial_conv", "100")):
+        for which, trials in (("spatial", "1000"), ("spatial_conv", "100"), ("conv", "1000")):
             r = subprocess.run([micro, "--which", which, "--ranks", "4", "--trials", trials], capture_output=True, text=True,
                                timeout=600)
             if r.returncode != 0:
@@ -808,8 +808,11 @@ def main():
             # "reference microbench_*" entries above
             for m in reference_microbench:
                 m = dict(m)
-                m["name"] = "reference microbench_%s through Spatial2DComm (C++ binary, 4 ranks, wall clock): %s" % (
-                    m.pop("which"), m["name"])
+                which = m.pop("which")
+                if which == "conv":
+                    m["name"] = "reference microbench_conv (C++ binary, one device, wall clock of launch + synchronise): %s" % m["name"]
+                else:
+                    m["name"] = "reference microbench_%s through Spatial2DComm (C++ binary, 4 ranks, wall clock): %s" % (which, m["name"])
                 sec.append(m)
         out["secondary"] = sec
         # The halo half of the metric inside `roofline`: pack / unpack at the headline configuration (1.08 GB per
