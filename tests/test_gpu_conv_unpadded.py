@@ -67,7 +67,7 @@ def test_unpadded_tiles_vs_unsplit_oracle(oracle, K, N, Cin, Cout, Ht, W):
             assert rel_err(oracle.bf16_to_f32(host(gs[r])), want_g) <= 5e-3
 
 
-@pytest.mark.parametrize("K,N,C,Ht,W", [(4, 2, 64, 12, 128), (8, 2, 64, 128, 2048)])
+@pytest.mark.parametrize("K,N,C,Ht,W", [(4, 2, 64, 12, 128), (8, 2, 64, 128, 2048), (4, 2, 192, 12, 128), (8, 2, 128, 128, 1024)])
 def test_unpadded_forward_equals_the_padded_chain_bit_for_bit(K, N, C, Ht, W):
     """pack (pad) -> halo exchange -> conv over padded tiles multiplies the same values in the same order as the
     one launch over the tiles without halo: equal bits, at the full high-resolution configuration too."""
