@@ -203,3 +203,38 @@ def test_general_conv_error_codes():
     assert f(3, 3, 5, 5, 1, 1) == capi.ADH_EUNIMPL  # more than 16 residue classes
     assert capi.conv2d_fwd_tiles([x], w, [y], 1, 4, 4, 9, 9, 3, 3, 2, 2, 1, 1, beta=0.5, ws=ws) == capi.ADH_EINVAL
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("K,N,C,H,W,k,s,d", [(4, 32, 64, 128, 512, 3, 1, 3),   # tools/microbench_spatial_conv.cc:25-32 at full size
+                                             (4, 8, 64, 32, 128, 3, 2, 1)])    # a strided 3x3 over padded tiles
+def test_general_conv_three_passes_agree_on_one_number(K, N, C, H, W, k, s, d):
+    """<dy, conv(x, w)> = <x_pad, conv_bwd_data(w, dy)> = <w, conv_bwd_filter(x_pad, dy)> for the general entry points
+    at the reference's microbenchmark shape (3x3 at dilation 3 over halo 3: the 3x3 kernels with their taps three
+    apart), fp32: a size-independent check that ties the three kernels together where the oracle would take minutes.
+    Each stored output carries a relative rounding error of about 2^-20; the three numbers may differ by a few of
+    those times the random-walk size of the sum."""
+    g = torch.Generator(device="cuda").manual_seed(41)
+    p = d * (k - 1) // 2
+    HP, WP = H + 2 * p, W + 2 * p
+    OH, OW = (HP - ((k - 1) * d + 1)) // s + 1, (WP - ((k - 1) * d + 1)) // s + 1
+    xs = [torch.rand((N, C, HP, WP), device="cuda", generator=g) * 2 - 1 for _ in range(K)]
+    dys = [torch.randn((N, C, OH, OW), device="cuda", generator=g) for _ in range(K)]
+    w = torch.randn((C, C, k, k), device="cuda", generator=g) * (2.0 / (C * k * k)) ** 0.5
+    geo = (k, k, s, s, d, d)
+    nbytes = max(capi.lib().adh_conv2d_workspace_bytes(wh, capi.ADH_F32, K, N, C, C, HP, WP, *geo) for wh in (0, 1, 2))
+    ws = torch.empty(nbytes // 4 + 64, device="cuda")
+    ys = [torch.full((N, C, OH, OW), float("nan"), device="cuda") for _ in range(K)]
+    gs = [torch.full((N, C, HP, WP), float("nan"), device="cuda") for _ in range(K)]
+    gw = torch.full((C, C, k, k), float("nan"), device="cuda")
+    capi.check(capi.conv2d_fwd_tiles(xs, w, ys, N, C, C, HP, WP, *geo, ws=ws), "fwd")
+    capi.check(capi.conv2d_bwd_data_tiles(w, dys, gs, N, C, C, HP, WP, *geo, ws=ws), "bwd-data")
+    capi.check(capi.conv2d_bwd_filter_tiles(xs, dys, gw, N, C, C, HP, WP, *geo, ws=ws), "bwd-filter")
+    dot = lambda a, b: float((a.double() * b.double()).sum())
+    via_fwd = sum(dot(dy, y) for dy, y in zip(dys, ys))
+    via_data = sum(dot(x, gx) for x, gx in zip(xs, gs))
+    via_filter = dot(w, gw)
+    walk = sum(float(((dy.double() * y.double()) ** 2).sum()) for dy, y in zip(dys, ys)) ** 0.5
+    eps = 2.0 ** -20
+    assert np.isfinite(via_fwd) and abs(via_fwd) < 6.0 * walk
+    assert abs(via_fwd - via_data) <= 6.0 * eps * walk
+    assert abs(via_fwd - via_filter) <= 6.0 * eps * walk
